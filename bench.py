@@ -1,0 +1,206 @@
+#!/usr/bin/env python3
+"""Benchmark of fused quantized-KV decode attention on one MI355X.
+
+One "step" = one decode step (one new token per sequence) of the Qwen-style GQA configuration -- 32 query heads,
+8 kv heads, head_dim 128, ctx 8192, keys 3-bit, values 4-bit Lloyd-Max codes with an fp32 row scale -- over
+`--seqs` independent sequence caches held side by side (default 64 = 0.5 GB of packed cache, more than the 256 MB
+Infinity Cache, so the timed reads come from HBM).  Inputs are synthetic and already resident in HBM.
+
+Prints ONE JSON line: tokens/s (whole job), the HBM roofline of the dominant kernel measured with HIP events on the
+launch stream, and the CPU checker (a scalar restatement of the reference's path) timed on a bounded sample.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+
+def build_cache(capi, torch, wl, seed):
+    """Encode `wl.n_seq` sequences of synthetic K/V (N(0,1), 1 % of channels x10) generated on the device."""
+    d = wl.head_dim
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(seed)
+    rk = torch.zeros(d * d, device="cuda")
+    rv = torch.zeros(d * d, device="cuda")
+    capi.make_rotation(seed + 1, d, rk)
+    capi.make_rotation(seed + 2, d, rv)
+    cache = capi.KVCache(capi.KV_LLOYDMAX, wl.n_seq, wl.n_kv_heads, d, wl.max_len, wl.k_bits, wl.v_bits, wl.k_sign,
+                         wl.v_sign)
+    cache.set_rotations(rk, rv)
+    n_out = max(1, d // 100)
+    ch = torch.randperm(d, generator=gen, device="cuda")[:n_out]
+    for s, L in enumerate(wl.lens):
+        K = torch.randn((1, wl.n_kv_heads, L, d), generator=gen, device="cuda")
+        V = torch.randn((1, wl.n_kv_heads, L, d), generator=gen, device="cuda")
+        K[..., ch] *= 10.0
+        V[..., ch] *= 10.0
+        cache.encode_append(K, V, seq_begin=s, rotate=1)
+    q = torch.randn((wl.n_seq, wl.n_q_heads, d), generator=gen, device="cuda")
+    return cache, q, rk, rv
+
+
+def cpu_baseline(capi, torch, cache, wl, q, rk, rv, budget_s=12.0):
+    """Time the CPU checker (reference cost structure, one core) on one sequence of the same workload."""
+    from oracle import oracle as orc
+    d = wl.head_dim
+    L = wl.lens[0]
+    fields, scales = [], []
+    for which in (0, 1):
+        f = torch.empty((1, wl.n_kv_heads, L, d), dtype=torch.uint8, device="cuda")
+        a = torch.zeros((1, wl.n_kv_heads, L), device="cuda")
+        cache.export_fields(which, f, a)
+        fields.append(f.cpu().numpy())
+        scales.append(a.cpu().numpy())
+    specs = []
+    for which in (0, 1):
+        bounds, levels, recon = cache.get_tables(which)
+        specs.append(orc.CoderSpec(1, d, wl.v_bits if which else wl.k_bits, sign=wl.v_sign if which else wl.k_sign,
+                                   bounds=bounds, levels=levels, recon=recon))
+    qh = q[0:1].cpu().numpy()
+    rkh, rvh = rk.cpu().numpy(), rv.cpu().numpy()
+    steps, t0 = 0, time.perf_counter()
+    out = None
+    while True:
+        out = orc.decode_attn(specs[0], specs[1], fields[0], scales[0], fields[1], scales[1], qh, [L], gqa_weed=False,
+                              Rk=rkh, Rv=rvh)
+        steps += 1
+        elapsed = time.perf_counter() - t0
+        if elapsed >= budget_s or steps >= 200:
+            break
+    return steps / elapsed, steps, elapsed, out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--seqs", type=int, default=64, help="independent ctx-8192 sequence caches per launch")
+    ap.add_argument("--ctx", type=int, default=8192)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the path is sharded by (sequence, kv head) with no "
+              "exchange; see DESIGN.md); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from weed_amd import capi, workloads
+
+    lib = capi.load()  # raises if the HIP library is missing: there is no fallback path
+    capi.check(lib.weed_hip_init(0))
+    stream = torch.cuda.Stream()
+    capi.use_torch_stream(stream)
+    with torch.cuda.stream(stream):
+        wl = workloads.config(3, n_seq=args.seqs, scale=args.ctx / 8192.0)
+        cache, q, rk, rv = build_cache(capi, torch, wl, seed=1234)
+        out = torch.zeros_like(q)
+        flags = capi.ATTN_ROTATE_Q | capi.ATTN_UNROTATE_OUT
+
+        def step():
+            cache.decode_attn(q, out, capi.GQA_BLOCKED, flags)
+
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+        ms_per_step = 1e3 * elapsed / args.steps
+        tokens_per_s = wl.n_seq * args.steps / elapsed
+
+        # dominant kernel alone: HIP events recorded by the library around its launch, on the launch stream
+        capi.profile_reset()
+        capi.profile_enable(True)
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        k_ms, k_n = capi.profile_read("kv_decode_attn")
+        c_ms, c_n = capi.profile_read("kv_decode_combine")
+        capi.profile_enable(False)
+        kernel_ms = k_ms / max(1, k_n)
+        bytes_per_launch = wl.bytes_per_step(lloydmax=True)
+        achieved = bytes_per_launch / (kernel_ms * 1e-3) / 1e9
+
+        # batch = 1 latency of the same shape (one sequence per launch: launch-latency bound)
+        wl1 = workloads.config(3, n_seq=1, scale=args.ctx / 8192.0)
+        cache1, q1, _, _ = build_cache(capi, torch, wl1, seed=99)
+        out1 = torch.zeros_like(q1)
+        for _ in range(args.warmup):
+            cache1.decode_attn(q1, out1, capi.GQA_BLOCKED, flags)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            cache1.decode_attn(q1, out1, capi.GQA_BLOCKED, flags)
+        torch.cuda.synchronize()
+        single_ms = 1e3 * (time.perf_counter() - t0) / args.steps
+
+        traffic = None
+        traffic_file = os.path.join(ROOT, "profiles", "kv_decode_attn_traffic.json")
+        if os.path.exists(traffic_file):
+            with open(traffic_file) as f:
+                t = json.load(f)
+            if t.get("seqs") == args.seqs and t.get("ctx") == args.ctx:
+                traffic = t.get("hbm_bytes_per_launch")
+
+        result = {
+            "metric": "quantized-KV decode attn tokens/sec + HBM GB/s (% roofline) at ctx 8192",
+            "value": tokens_per_s,
+            "unit": "tokens/s",
+            "n_gpus": 1,
+            "steps": args.steps,
+            "warmup": args.warmup,
+            "ms_per_step": ms_per_step,
+            "higher_is_better": True,
+            "scaling": "weak",
+            "vs_baseline": None,
+            "dtype": "f32",
+            "data": "synthetic",
+            "config": {
+                "workload": "cfg3 Qwen-style GQA decode: 32 q / 8 kv heads, head_dim 128, ctx %d, K 3-bit + V 4-bit "
+                            "Lloyd-Max codes + fp32 row scale, %d independent sequence caches per launch "
+                            "(1 new token each), split-context" % (args.ctx, wl.n_seq),
+                "n_seq": wl.n_seq, "ctx": args.ctx, "n_q_heads": wl.n_q_heads, "n_kv_heads": wl.n_kv_heads,
+                "head_dim": wl.head_dim, "k_bits": wl.k_bits, "v_bits": wl.v_bits,
+                "packed_cache_bytes": bytes_per_launch,
+            },
+            "roofline": {
+                "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+                "kernel": "decode attention main kernel", "kernel_ms": kernel_ms,
+                "algorithmic_bytes_per_launch": bytes_per_launch,
+                "combine_kernel_ms": c_ms / max(1, c_n),
+            },
+            "whole_step_gbs": bytes_per_launch / (ms_per_step * 1e-3) / 1e9,
+            "single_sequence": {"ms_per_step": single_ms, "tokens_per_s": 1e3 / single_ms,
+                                "gbs": wl1.bytes_per_step(True) / (single_ms * 1e-3) / 1e9},
+        }
+        if not args.no_cpu_baseline:
+            tps, n, secs, cpu_out = cpu_baseline(capi, torch, cache, wl, q, rk, rv)
+            got = out[0:1].cpu().numpy()
+            err = float(np.abs(got - cpu_out).max())
+            result["cpu_baseline"] = {
+                "value": tps, "unit": "tokens/s", "cores": 1, "kind": "port",
+                "sample": "%d decode steps of ONE of the %d sequences (same shape, ctx %d) in %.1f s; scalar C "
+                          "restatement of the reference's path: full dequantise, GQA replicate, K^T copy, naive dots, "
+                          "divide, 3-pass softmax" % (n, wl.n_seq, args.ctx, secs),
+                "gbs": wl1.bytes_per_step(True) * tps / 1e9,
+                "max_abs_diff_vs_gpu": err,
+            }
+        cache.close()
+        cache1.close()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

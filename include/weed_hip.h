@@ -1,0 +1,198 @@
+/*
+ * weed_hip.h -- C ABI of the MI355X (gfx950) device layer for Weed's quantized-KV attention path.
+ *
+ * This is the seam a Weed build binds instead of its OpenCL device (include/devices/gpu_device.hpp,
+ * include/common/oclengine.hpp): plain C types only -- uint32_t for Weed's tcapint, int32_t for symint,
+ * float for real1 -- raw device pointers, explicit geometry in ELEMENTS exactly as Weed's ops pass it
+ * (offset + per-dimension stride, column-major by convention, see include/tensors/base_tensor.hpp:123-142).
+ *
+ * Conventions
+ *   - Every function returns an int status: WEED_HIP_OK (0) or a WEED_HIP_E* code, and never throws.
+ *     weed_hip_last_error() returns the message of the calling thread's last failure.  Weed's device layer
+ *     throws std::runtime_error / Weed::bad_alloc / std::invalid_argument instead
+ *     (include/devices/pool_item.hpp:32-40, src/devices/gpu_device.cpp:60-73,177, src/ops/matmul.cpp:96-109);
+ *     a host wrapper maps WEED_HIP_EINVAL -> std::invalid_argument, WEED_HIP_ENOMEM -> bad_alloc,
+ *     WEED_HIP_EDEVICE -> std::runtime_error.
+ *   - All launches are ordered on one HIP stream per process (weed_hip_set_stream / weed_hip_stream); an
+ *     asynchronous kernel fault surfaces at the next weed_hip_sync(), like Weed's callbackError latch
+ *     (include/devices/gpu_device.hpp:101-111).
+ *   - Entry points are not re-entrant per cache object; serialise callers per device as Weed serialises
+ *     enqueues under GpuDevice::queue_mutex (include/devices/gpu_device.hpp:41).
+ *   - Pointers named *_dev are device pointers; everything else is host memory.
+ */
+#ifndef WEED_HIP_H
+#define WEED_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+    WEED_HIP_OK = 0,
+    WEED_HIP_EINVAL = 1,   /* bad argument / shape mismatch (Weed: std::invalid_argument)      */
+    WEED_HIP_ENOMEM = 2,   /* device allocation failed (Weed: Weed::bad_alloc)                 */
+    WEED_HIP_EDEVICE = 3,  /* HIP runtime / kernel failure (Weed: std::runtime_error)          */
+    WEED_HIP_ECAPACITY = 4 /* append beyond max_tokens (Weed: unchecked std::vector overrun)   */
+};
+
+/* ------------------------------------------------------------------------------------------------ */
+/* device, stream, memory.  Replaces OCLEngine::GetWeedDevice (src/common/oclengine.cpp:186-194),      */
+/* GpuDevice::MakeBuffer (src/devices/gpu_device.cpp:34-76) and the blocking read/write helpers         */
+/* (src/devices/gpu_device.cpp:396-402, src/storage/gpu_real_storage.cpp:18-23).                        */
+/* ------------------------------------------------------------------------------------------------ */
+int weed_hip_init(int device_id);
+int weed_hip_device_count(int *count);
+int weed_hip_device_name(char *buf, size_t buf_len);
+/* Use an existing hipStream_t for all later launches (NULL restores the library's own stream). */
+int weed_hip_set_stream(void *hip_stream);
+void *weed_hip_stream(void);
+int weed_hip_sync(void);
+const char *weed_hip_last_error(void);
+const char *weed_hip_version(void);
+
+int weed_hip_malloc(void **ptr_dev, size_t bytes);
+int weed_hip_free(void *ptr_dev);
+int weed_hip_memset(void *ptr_dev, int byte_value, size_t bytes);
+int weed_hip_memcpy_h2d(void *dst_dev, const void *src, size_t bytes);
+int weed_hip_memcpy_d2h(void *dst, const void *src_dev, size_t bytes);
+int weed_hip_memcpy_d2d(void *dst_dev, const void *src_dev, size_t bytes);
+
+/* Per-kernel device timing (HIP events on the launch stream), off by default.  When enabled, each entry
+ * point brackets its dominant kernel with events; weed_hip_profile_read returns the accumulated time. */
+int weed_hip_profile_enable(int on);
+int weed_hip_profile_reset(void);
+/* name: "kv_decode_attn", "kv_decode_combine", "kv_encode", "kv_pack", "matmul", "softmax", "reduce" */
+int weed_hip_profile_read(const char *name, double *total_ms, uint64_t *launches);
+
+/* ------------------------------------------------------------------------------------------------ */
+/* dense ops on strided fp32 tensors                                                                  */
+/* ------------------------------------------------------------------------------------------------ */
+
+/* out[M,N] = a[M,K] . b[K,N].  Replaces Weed::matmul's real branch (src/ops/matmul.cpp:242-279; geometry as
+ * get_dim, matmul.cpp:95-122; OpenCL kernel matmul_real, src/common/qengine.cl:598-640).  Element (i,k) of a is
+ * a_dev[a_off + i*a_s0 + k*a_s1], and likewise for b and out. */
+int weed_hip_matmul_f32(uint32_t M, uint32_t N, uint32_t K, const float *a_dev, uint32_t a_off, uint32_t a_s0,
+                        uint32_t a_s1, const float *b_dev, uint32_t b_off, uint32_t b_s0, uint32_t b_s1, float *out_dev,
+                        uint32_t o_off, uint32_t o_s0, uint32_t o_s1);
+
+/* Numerically stable softmax along `axis`.  Replaces Weed::softmax (src/ops/softmax.cpp:276-287; OpenCL kernel
+ * softmax_forward, qengine.cl:1001-1033).  rank <= 8. */
+int weed_hip_softmax_f32(uint32_t rank, const uint32_t *shape, uint32_t axis, const float *a_dev, uint32_t a_off,
+                         const uint32_t *a_stride, float *out_dev, uint32_t o_off, const uint32_t *o_stride);
+
+/* Axis reductions.  Replace Weed::reduce / Weed::max / Weed::min (src/ops/reduce.cpp:342-386; OpenCL kernels
+ * reduce_real / axis_max / axis_min, qengine.cl:136-159,244-297).  out has the shape of a with `axis` removed;
+ * o_stride has `rank` entries and the one at `axis` is ignored. */
+enum { WEED_HIP_REDUCE_SUM = 0, WEED_HIP_REDUCE_MAX = 1, WEED_HIP_REDUCE_MIN = 2 };
+int weed_hip_reduce_f32(int op, uint32_t rank, const uint32_t *shape, uint32_t axis, const float *a_dev,
+                        uint32_t a_off, const uint32_t *a_stride, float *out_dev, uint32_t o_off,
+                        const uint32_t *o_stride);
+
+/* ------------------------------------------------------------------------------------------------ */
+/* rotation                                                                                            */
+/* ------------------------------------------------------------------------------------------------ */
+
+/* Seeded replacement of make_random_rotation (src/modules/multihead_attention.cpp:84-121): draws d*d N(0,1)
+ * values with std::mt19937(seed) + std::normal_distribution<float> on the host (column-major), uploads them and
+ * orthonormalises the columns on the device in the reference's order (normalise column j, remove its projection
+ * from every later column).  r_dev receives d*d floats, column-major. */
+int weed_hip_make_rotation(uint32_t seed, uint32_t d, float *r_dev);
+/* Device Gram-Schmidt only (input already in r_dev). */
+int weed_hip_orthonormalize_columns(uint32_t d, float *r_dev);
+
+/* ------------------------------------------------------------------------------------------------ */
+/* quantized KV cache: device twin of Weed::QuantizedKVCache (include/modules/multihead_attention.hpp:22-36)  */
+/* ------------------------------------------------------------------------------------------------ */
+
+enum {
+    WEED_HIP_KV_UNIFORM = 0, /* Weed's coder: 2^bits uniform cells on [-3s, 3s), one block_scale per tensor     */
+    WEED_HIP_KV_LLOYDMAX = 1 /* per-row scale, Lloyd-Max codes for N(0,1), optional residual sign bit           */
+};
+enum {
+    WEED_HIP_GQA_WEED = 0,    /* kv_head = q_head % n_kv_heads  (multihead_attention.cpp:301-306)               */
+    WEED_HIP_GQA_BLOCKED = 1  /* kv_head = q_head / (n_q_heads / n_kv_heads)                                    */
+};
+
+typedef struct {
+    int32_t mode;          /* WEED_HIP_KV_UNIFORM or WEED_HIP_KV_LLOYDMAX                                      */
+    int32_t n_seq;         /* B: sequences held side by side                                                  */
+    int32_t n_kv_heads;    /* Hkv                                                                             */
+    int32_t head_dim;      /* d, a multiple of 32, at most 256                                                 */
+    int32_t max_tokens;    /* capacity per sequence (Weed: max_seq_len)                                        */
+    int32_t k_bits;        /* code bits for keys, 1..4                                                         */
+    int32_t v_bits;        /* code bits for values, 1..4                                                       */
+    int32_t k_sign;        /* 1: keep a residual sign bit per key coordinate (LLOYDMAX only)                   */
+    int32_t v_sign;        /* 1: same for values                                                              */
+} weed_hip_kv_config;
+
+typedef struct weed_hip_kv_cache weed_hip_kv_cache;
+
+/* QuantizedKVCache::allocate for both K and V (multihead_attention.cpp:31-41,190-193). */
+int weed_hip_kv_cache_create(weed_hip_kv_cache **cache, const weed_hip_kv_config *cfg);
+int weed_hip_kv_cache_destroy(weed_hip_kv_cache *cache);
+/* MultiHeadAttention::reset_cache (include/modules/multihead_attention.hpp:140-149): lengths to 0; rotations,
+ * scales and tables are kept unless `drop_rotations` is non-zero. */
+int weed_hip_kv_cache_reset(weed_hip_kv_cache *cache, int drop_rotations);
+/* Bytes of device memory a decode step reads for the packed K and V fields and row scales of `n_tokens` tokens of
+ * one (sequence, kv head): the algorithmic bytes used for roofline accounting. */
+int weed_hip_kv_cache_row_bytes(const weed_hip_kv_cache *cache, uint32_t *k_row_bytes, uint32_t *v_row_bytes);
+int weed_hip_kv_cache_seq_lens(const weed_hip_kv_cache *cache, int32_t *lens /* [n_seq] host */);
+
+/* k_rotation / v_rotation (multihead_attention.cpp:177-178): column-major d x d, copied from device memory. */
+int weed_hip_kv_cache_set_rotations(weed_hip_kv_cache *cache, const float *rk_dev, const float *rv_dev);
+/* block_scale of the two caches (multihead_attention.cpp:240-241); UNIFORM mode only. */
+int weed_hip_kv_cache_set_scales(weed_hip_kv_cache *cache, float k_scale, float v_scale);
+int weed_hip_kv_cache_get_scales(const weed_hip_kv_cache *cache, float *k_scale, float *v_scale);
+/* Replace the built-in Lloyd-Max tables (host arrays): bounds[2^bits-1], levels[2^bits], recon[2^(bits+sign)].
+ * `which` 0 = keys, 1 = values.  Reconstruction levels are rounded to IEEE binary16 (the fused decode kernel keeps
+ * them in fp16 so that products with the split query are exact); recon_rounded receives the values in use. */
+int weed_hip_kv_cache_set_tables(weed_hip_kv_cache *cache, int which, const float *bounds, const float *levels,
+                                 const float *recon, float *recon_rounded);
+int weed_hip_kv_cache_get_tables(const weed_hip_kv_cache *cache, int which, float *bounds, float *levels, float *recon);
+
+/* sqrt(sum(x^2)/n + 1e-8) over a strided [n_seq, n_kv_heads, T, d] tensor (multihead_attention.cpp:226-241).
+ * `sequential` != 0 reproduces the reference's one-thread fp32 summation order (flat column-major order of the
+ * logical [rows, d] reshape of a CONTIGUOUS tensor) bit for bit; 0 uses a tree reduction. */
+int weed_hip_block_scale_f32(const float *x_dev, uint32_t off, const uint32_t shape[4], const uint32_t stride[4],
+                             int sequential, float *scale_out /* host */);
+
+/* Encode-and-append: apply_rotation + write_row for T_new tokens of every sequence in
+ * [seq_begin, seq_begin + seq_count) (multihead_attention.cpp:206-257).  k_dev / v_dev are logical
+ * [seq_count, n_kv_heads, T_new, d] tensors with strides in elements.  `rotate` = 0 means the inputs are already
+ * in the rotated basis.  Tokens are appended in logical order (token t of the call becomes token len+t). */
+int weed_hip_kv_encode_append(weed_hip_kv_cache *cache, int32_t seq_begin, int32_t seq_count, int32_t T_new,
+                              const float *k_dev, uint32_t k_off, const uint32_t k_stride[4], const float *v_dev,
+                              uint32_t v_off, const uint32_t v_stride[4], int rotate);
+
+/* read_row for a token range (multihead_attention.cpp:64-79,259-273): dense fp32 [seq_count, n_kv_heads, T, d]
+ * with caller strides, still in the rotated basis.  `which` 0 = keys, 1 = values. */
+int weed_hip_kv_dequant(const weed_hip_kv_cache *cache, int which, int32_t seq_begin, int32_t seq_count,
+                        int32_t tok_begin, int32_t T, float *out_dev, uint32_t o_off, const uint32_t o_stride[4]);
+
+/* Unpack for inspection: one field per byte, fields_dev[seq_count][n_kv_heads][T][d] (field = code, or
+ * (code<<1)|sign when a sign bit is kept), scales_dev[seq_count][n_kv_heads][T] (row scale alpha = |y|/sqrt(d);
+ * LLOYDMAX only, may be NULL). */
+int weed_hip_kv_export_fields(const weed_hip_kv_cache *cache, int which, int32_t seq_begin, int32_t seq_count,
+                              int32_t tok_begin, int32_t T, uint8_t *fields_dev, float *scales_dev);
+/* UNIFORM mode: the rows in Weed's own word packing, floor(32/bits) codes per int32
+ * (QuantizedKVCache::packed, multihead_attention.cpp:43-62); words_dev[seq_count][n_kv_heads][T][wpr]. */
+int weed_hip_kv_export_weed_words(const weed_hip_kv_cache *cache, int which, int32_t seq_begin, int32_t seq_count,
+                                  int32_t tok_begin, int32_t T, int32_t *words_dev);
+
+/* Fused single-query decode attention over the packed cache: everything MultiHeadAttention::forward does between
+ * the cache rebuild and the output projection for T = 1 (multihead_attention.cpp:259-348): un-pack, Q.K^T,
+ * /sqrt(d), softmax over each sequence's own length (split over the context and merged), P.V, un-rotate.
+ * q_dev / out_dev: logical [n_seq, n_q_heads, d] with strides in elements.
+ * flags: bit 0 rotate q by k_rotation first (cpp:276); bit 1 multiply the result by v_rotation^T (cpp:343-348). */
+enum { WEED_HIP_ATTN_ROTATE_Q = 1, WEED_HIP_ATTN_UNROTATE_OUT = 2 };
+int weed_hip_kv_decode_attn(weed_hip_kv_cache *cache, int32_t n_q_heads, int32_t gqa_mapping, const float *q_dev,
+                            uint32_t q_off, const uint32_t q_stride[3], float *out_dev, uint32_t o_off,
+                            const uint32_t o_stride[3], uint32_t flags);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

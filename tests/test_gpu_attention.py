@@ -1,0 +1,222 @@
+"""GPU parity of fused decode attention over the packed cache, through the C ABI.
+
+Bar (fp32): |gpu - checker| <= 1e-4 + 1e-3 * |checker| per output element, where the checker is the CPU restatement
+of the reference's path run on the same codes.  Full-size configurations that the scalar checker cannot finish in
+seconds are covered by size-independent properties.
+"""
+import numpy as np
+import pytest
+
+from gpu_helpers import assert_attn_close, col_major, coder_specs, dev, export
+from weed_amd import workloads
+
+pytestmark = pytest.mark.gpu
+
+
+def build_cache(gpu, wl, mode, K, V, rotations=None, scales=None, rotate=0):
+    cache = gpu.KVCache(mode, wl.n_seq, wl.n_kv_heads, wl.head_dim, wl.max_len, wl.k_bits, wl.v_bits,
+                        wl.k_sign if mode == gpu.KV_LLOYDMAX else 0, wl.v_sign if mode == gpu.KV_LLOYDMAX else 0)
+    if rotations is not None:
+        cache.set_rotations(dev(rotations[0]), dev(rotations[1]))
+    if scales is not None:
+        cache.set_scales(*scales)
+    Kd, Vd = dev(K), dev(V)
+    if len(set(wl.lens)) == 1:
+        cache.encode_append(Kd, Vd, rotate=rotate)
+    else:
+        for s, L in enumerate(wl.lens):
+            cache.encode_append(Kd[s:s + 1, :, :L], Vd[s:s + 1, :, :L], seq_begin=s, rotate=rotate)
+    return cache
+
+
+def checker_output(oracle, gpu, cache, wl, q, gqa_weed, Rk=None, Rv=None):
+    """Run the CPU checker on the fields the device cache actually holds."""
+    kspec, vspec = coder_specs(oracle, cache)
+    kf, ka = export(cache, 0, wl.max_len)
+    vf, va = export(cache, 1, wl.max_len)
+    lloyd = cache.cfg.mode == gpu.KV_LLOYDMAX
+    return oracle.decode_attn(kspec, vspec, kf, ka if lloyd else None, vf, va if lloyd else None, q, wl.lens,
+                              gqa_weed=gqa_weed, Rk=Rk, Rv=Rv)
+
+
+def run_decode(gpu, cache, q, gqa, flags, col_major_io=False):
+    import torch
+    qd = col_major(q) if col_major_io else dev(q)
+    out = torch.zeros_like(qd)
+    cache.decode_attn(qd, out, gqa_mapping=gqa, flags=flags)
+    gpu.sync()
+    return out.cpu().numpy()
+
+
+def rotations(oracle, d, seed):
+    rng = np.random.default_rng(seed)
+    return (oracle.orthonormalize_columns(rng.normal(size=d * d).astype(np.float32)),
+            oracle.orthonormalize_columns(rng.normal(size=d * d).astype(np.float32)))
+
+
+def test_cfg1_weed_uniform_end_to_end(gpu, oracle):
+    """Configuration 1 in Weed's own coder: rotation, global block scale, 4-bit uniform codes, one head, ctx 512.
+    The whole chain runs on the device (rotate = 2 keeps the reference's rounding order) and is compared with the
+    checker fed the raw inputs."""
+    wl = workloads.config(1)
+    K, V, q = wl.tensors()
+    d = wl.head_dim
+    Rk, Rv = rotations(oracle, d, 1)
+    Ky = oracle.apply_rotation(K.reshape(-1, d), Rk)
+    Vy = oracle.apply_rotation(V.reshape(-1, d), Rv)
+    scales = (oracle.block_scale(Ky), oracle.block_scale(Vy))
+    cache = build_cache(gpu, wl, gpu.KV_UNIFORM, K, V, (Rk, Rv), scales, rotate=2)
+    kspec, vspec = coder_specs(oracle, cache)
+    kf, _ = oracle.encode_rows(kspec, Ky)
+    vf, _ = oracle.encode_rows(vspec, Vy)
+    got_kf, _ = export(cache, 0, wl.max_len)
+    got_vf, _ = export(cache, 1, wl.max_len)
+    np.testing.assert_array_equal(got_kf.reshape(-1, d), kf)
+    np.testing.assert_array_equal(got_vf.reshape(-1, d), vf)
+    want = oracle.decode_attn(kspec, vspec, kf.reshape(1, 1, -1, d), None, vf.reshape(1, 1, -1, d), None, q, wl.lens,
+                              Rk=Rk, Rv=Rv)
+    got = run_decode(gpu, cache, q, gpu.GQA_WEED, gpu.ATTN_ROTATE_Q | gpu.ATTN_UNROTATE_OUT, col_major_io=True)
+    assert_attn_close(got, want, "cfg1 uniform")
+    cache.close()
+
+
+@pytest.mark.parametrize("index", [1, 2, 3])
+def test_configs_lloydmax(gpu, oracle, index):
+    """Configurations 1-3 at full size with the Lloyd-Max coder (config 3: 32 query / 8 kv heads, ctx 8192)."""
+    wl = workloads.config(index)
+    K, V, q = wl.tensors()
+    Rk, Rv = rotations(oracle, wl.head_dim, index)
+    cache = build_cache(gpu, wl, gpu.KV_LLOYDMAX, K, V, (Rk, Rv), rotate=1)
+    for gqa, weed in ((gpu.GQA_WEED, True), (gpu.GQA_BLOCKED, False)):
+        want = checker_output(oracle, gpu, cache, wl, q, weed, Rk, Rv)
+        got = run_decode(gpu, cache, q, gqa, gpu.ATTN_ROTATE_Q | gpu.ATTN_UNROTATE_OUT)
+        assert_attn_close(got, want, "cfg%d mapping %d" % (index, gqa))
+        if wl.n_q_heads == wl.n_kv_heads:
+            break
+    cache.close()
+
+
+def test_cfg4_ragged_batch_reduced(gpu, oracle):
+    """Configuration 4 (16 ragged sequences, 2-bit keys + sign, 3-bit values, split-context combine) with lengths
+    scaled down 16x so that the scalar checker finishes in seconds."""
+    wl = workloads.config(4, scale=1.0 / 16)
+    assert min(wl.lens) >= 128 and max(wl.lens) <= 2048 and len(set(wl.lens)) > 8
+    K, V, q = wl.tensors()
+    cache = build_cache(gpu, wl, gpu.KV_LLOYDMAX, K, V)
+    want = checker_output(oracle, gpu, cache, wl, q, True)
+    got = run_decode(gpu, cache, q, gpu.GQA_WEED, 0)
+    assert_attn_close(got, want, "cfg4 reduced")
+    # 32 query heads over the same 8 kv heads (the GQA variant of this configuration)
+    rng = np.random.default_rng(3)
+    q32 = rng.standard_normal((wl.n_seq, 32, wl.head_dim), dtype=np.float32)
+    want = checker_output(oracle, gpu, cache, wl, q32, False)
+    got = run_decode(gpu, cache, q32, gpu.GQA_BLOCKED, 0)
+    assert_attn_close(got, want, "cfg4 reduced, 32 query heads")
+    cache.close()
+
+
+def test_cfg4_full_size_properties(gpu, oracle):
+    """Configuration 4 at full size (lengths up to 32768): properties that do not need the scalar checker.
+      * identical V rows: the softmax weights sum to one, so every output equals that row's dequantised value;
+      * one sequence checked against the checker in full;
+      * permutation: swapping two sequences' queries and caches swaps the outputs."""
+    import torch
+    wl = workloads.config(4)
+    assert max(wl.lens) > 30000
+    d, Hkv, S = wl.head_dim, wl.n_kv_heads, wl.n_seq
+    rng = np.random.default_rng(11)
+    cache = gpu.KVCache(gpu.KV_LLOYDMAX, S, Hkv, d, wl.max_len, wl.k_bits, wl.v_bits, wl.k_sign, wl.v_sign)
+    v_row = rng.standard_normal((1, Hkv, 1, d), dtype=np.float32)
+    short = int(np.argmin(wl.lens))
+    K_short = None
+    for s, L in enumerate(wl.lens):
+        Ks = rng.standard_normal((1, Hkv, L, d), dtype=np.float32)
+        if s == short:
+            K_short = Ks
+        Kd = dev(Ks)
+        Vd = dev(v_row).expand(1, Hkv, L, d)  # stride 0 along tokens: every row is the same vector
+        cache.encode_append(Kd, Vd, seq_begin=s)
+        del Kd
+    assert cache.seq_lens() == wl.lens
+    q = rng.standard_normal((S, wl.n_q_heads, d), dtype=np.float32)
+    got = run_decode(gpu, cache, q, gpu.GQA_WEED, 0)
+    kspec, vspec = coder_specs(oracle, cache)
+    vf, va = oracle.encode_rows(vspec, v_row.reshape(-1, d))
+    v_hat = oracle.decode_rows(vspec, vf, va)  # [Hkv, d]
+    for s in range(S):
+        assert_attn_close(got[s], v_hat, "constant-V property, sequence %d" % s)
+    # the shortest sequence in full against the checker
+    L = wl.lens[short]
+    kf, ka = oracle.encode_rows(kspec, K_short.reshape(-1, d))
+    vf_full = np.broadcast_to(vf.reshape(1, Hkv, 1, d), (1, Hkv, L, d))
+    va_full = np.broadcast_to(va.reshape(1, Hkv, 1), (1, Hkv, L))
+    want = oracle.decode_attn(kspec, vspec, kf.reshape(1, Hkv, L, d), ka.reshape(1, Hkv, L), vf_full, va_full,
+                              q[short:short + 1], [L])
+    assert_attn_close(got[short:short + 1], want, "cfg4 full size, shortest sequence")
+    cache.close()
+
+
+def test_split_context_matches_single_pass(gpu, oracle):
+    """The split-context merge equals one pass over the whole context: a long single sequence (many splits) and the
+    same tokens as the tail of a batch (few splits) give the same answer as the checker's one-pass softmax, including
+    when one split holds a score far above all others."""
+    rng = np.random.default_rng(21)
+    d, Hkv, Hq, L = 64, 2, 4, 5000
+    K = rng.standard_normal((1, Hkv, L, d), dtype=np.float32)
+    V = rng.standard_normal((1, Hkv, L, d), dtype=np.float32)
+    q = rng.standard_normal((1, Hq, d), dtype=np.float32)
+    K[0, :, 4321] = 6.0 * q[0, :Hkv]  # a key aligned with the query: dominates the softmax
+    wl = workloads.Workload("split", 1, Hq, Hkv, d, [L], 4, 4, 0, 0, 0)
+    cache = build_cache(gpu, wl, gpu.KV_LLOYDMAX, K, V)
+    want = checker_output(oracle, gpu, cache, wl, q, True)
+    got = run_decode(gpu, cache, q, gpu.GQA_WEED, 0)
+    assert_attn_close(got, want, "split context")
+    cache.close()
+
+
+def test_edge_lengths(gpu, oracle):
+    """Empty sequences give zeros; lengths 1, 63, 64, 65 around the 64-token block; an appended token changes the
+    result exactly as the checker says."""
+    import torch
+    rng = np.random.default_rng(31)
+    d, Hkv, Hq = 128, 2, 8
+    lens = [0, 1, 63, 64, 65, 257]
+    S = len(lens)
+    wl = workloads.Workload("edges", S, Hq, Hkv, d, lens, 3, 4, 1, 0, 0)
+    K = rng.standard_normal((S, Hkv, max(lens) + 1, d), dtype=np.float32)
+    V = rng.standard_normal((S, Hkv, max(lens) + 1, d), dtype=np.float32)
+    q = rng.standard_normal((S, Hq, d), dtype=np.float32)
+    cache = gpu.KVCache(gpu.KV_LLOYDMAX, S, Hkv, d, max(lens) + 1, 3, 4, 1, 0)
+    Kd, Vd = dev(K), dev(V)
+    for s, L in enumerate(lens):
+        if L:
+            cache.encode_append(Kd[s:s + 1, :, :L], Vd[s:s + 1, :, :L], seq_begin=s)
+    want = checker_output(oracle, gpu, cache, wl, q, False)
+    got = run_decode(gpu, cache, q, gpu.GQA_BLOCKED, 0)
+    assert not got[0].any()
+    assert_attn_close(got, want, "edge lengths")
+    # decode step: append one token to every sequence and attend again
+    cache.encode_append(torch.stack([Kd[s, :, L:L + 1] for s, L in enumerate(lens)]),
+                        torch.stack([Vd[s, :, L:L + 1] for s, L in enumerate(lens)]))
+    wl2 = workloads.Workload("edges+1", S, Hq, Hkv, d, [L + 1 for L in lens], 3, 4, 1, 0, 0)
+    want2 = checker_output(oracle, gpu, cache, wl2, q, False)
+    got2 = run_decode(gpu, cache, q, gpu.GQA_BLOCKED, 0)
+    assert_attn_close(got2, want2, "edge lengths + 1")
+    assert np.abs(got2[1] - got[1]).max() > 1e-3
+    cache.close()
+
+
+def test_head_dims_and_wide_groups(gpu, oracle):
+    """head_dim 32 and 256, and 16 query heads per kv head (two passes of the 8-head inner loop)."""
+    rng = np.random.default_rng(41)
+    for d, Hkv, Hq, L in ((32, 2, 2, 300), (256, 1, 4, 200), (64, 1, 16, 333)):
+        wl = workloads.Workload("dims", 2, Hq, Hkv, d, [L, L // 2], 4, 2, 0, 1, 0)
+        K = rng.standard_normal((2, Hkv, L, d), dtype=np.float32)
+        V = rng.standard_normal((2, Hkv, L, d), dtype=np.float32)
+        q = rng.standard_normal((2, Hq, d), dtype=np.float32)
+        cache = build_cache(gpu, wl, gpu.KV_LLOYDMAX, K, V)
+        for gqa, weed in ((gpu.GQA_WEED, True), (gpu.GQA_BLOCKED, False)):
+            want = checker_output(oracle, gpu, cache, wl, q, weed)
+            got = run_decode(gpu, cache, q, gqa, 0)
+            assert_attn_close(got, want, "d=%d Hq=%d" % (d, Hq))
+        cache.close()

@@ -1,0 +1,158 @@
+"""GPU parity of the strided fp32 matmul, softmax and axis reductions, through the C ABI.
+
+The reference pins these ops with tiny known-answer tests (test/tests.cpp:177-228, 1020-1041, 1110-1171, 1206-1221);
+they are repeated here on the device, followed by strided / larger cases against the CPU checker.
+Tolerance: fp32 sums in a different order than the checker's sequential loop -> rtol 2e-5 (atol scaled to the data);
+max/min are exact.
+"""
+import numpy as np
+import pytest
+
+from gpu_helpers import col_major, dev
+from weed_amd import workloads
+
+pytestmark = pytest.mark.gpu
+
+
+def test_matmul_reference_cases(gpu):
+    import torch
+    # 1x2 . 2x1 = 23 and the 2x1 . 1x2 outer product (tests.cpp:1020-1040), column-major operands
+    x = col_major(np.array([[2, 3]], dtype=np.float32))
+    y = col_major(np.array([[4], [5]], dtype=np.float32))
+    z = col_major(np.zeros((1, 1), dtype=np.float32))
+    gpu.matmul(x, y, z)
+    assert z.cpu().item() == 23
+    x = col_major(np.array([[2], [3]], dtype=np.float32))
+    y = col_major(np.array([[4, 5]], dtype=np.float32))
+    z = col_major(np.zeros((2, 2), dtype=np.float32))
+    gpu.matmul(x, y, z)
+    np.testing.assert_array_equal(z.cpu().numpy(), [[8, 10], [12, 15]])
+    # tests.cpp:1327-1341
+    A = col_major(np.array([[1, 3, 5], [2, 4, 6]], dtype=np.float32))
+    B = col_major(np.array([[7, 10], [8, 11], [9, 12]], dtype=np.float32))
+    C = col_major(np.zeros((2, 2), dtype=np.float32))
+    gpu.matmul(A, B, C)
+    np.testing.assert_array_equal(C.cpu().numpy(), np.array([[1, 3, 5], [2, 4, 6]]) @ np.array([[7, 10], [8, 11],
+                                                                                                [9, 12]]))
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (7, 5, 11), (64, 64, 64), (130, 70, 33), (1, 300, 128), (257, 1, 1000),
+                                   (512, 384, 256)])
+def test_matmul_strided_against_checker(gpu, oracle, M, N, K):
+    import torch
+    rng = np.random.default_rng(M * 7 + N * 3 + K)
+    A = rng.standard_normal((M, K), dtype=np.float32)
+    B = rng.standard_normal((K, N), dtype=np.float32)
+    want = np.zeros(M * N, dtype=np.float32)
+    oracle.matmul(M, N, K, A.reshape(-1), (0, K, 1), B.reshape(-1), (0, N, 1), want, (0, N, 1))
+    tol = dict(rtol=2e-5, atol=2e-5 * np.sqrt(K))
+    # row-major, column-major, and views with offsets / non-unit strides
+    for mk in (dev, col_major):
+        C = mk(np.zeros((M, N), dtype=np.float32))
+        gpu.matmul(mk(A), mk(B), C)
+        np.testing.assert_allclose(C.cpu().numpy(), want.reshape(M, N), **tol)
+    big_a = torch.zeros((M + 3, 2 * K + 1), device="cuda")
+    big_a[2:2 + M, 1:1 + 2 * K:2] = dev(A)
+    big_c = torch.full((2 * M, N + 5), -1.0, device="cuda")
+    gpu.matmul(big_a[2:2 + M, 1:1 + 2 * K:2], dev(B).t().contiguous().t(), big_c[::2, 3:3 + N])
+    np.testing.assert_allclose(big_c[::2, 3:3 + N].cpu().numpy(), want.reshape(M, N), **tol)
+    assert torch.all(big_c[1::2] == -1.0) and torch.all(big_c[:, :3] == -1.0)  # nothing outside the view is written
+
+
+def test_matmul_cfg5_sampled(gpu):
+    """Configuration 5b at full size ([4096 x 1024] . [1024 x 4096], column-major): the scalar checker would need
+    minutes, so 4096 sampled outputs are compared with float64 dot products, plus the column sums identity
+    1^T (A W) = (1^T A) W."""
+    A, W = workloads.matmul_config()
+    M, K = A.shape
+    N = W.shape[1]
+    Ad, Wd = col_major(A), col_major(W)
+    C = col_major(np.zeros((M, N), dtype=np.float32))
+    gpu.matmul(Ad, Wd, C)
+    Ch = C.cpu().numpy()
+    rng = np.random.default_rng(0)
+    ii, jj = rng.integers(0, M, 4096), rng.integers(0, N, 4096)
+    want = np.einsum("ik,ki->i", A[ii].astype(np.float64), W[:, jj].astype(np.float64))
+    np.testing.assert_allclose(Ch[ii, jj], want, rtol=2e-5, atol=2e-5)
+    np.testing.assert_allclose(Ch.astype(np.float64).sum(axis=0), A.astype(np.float64).sum(axis=0) @ W.astype(np.float64),
+                               rtol=1e-4, atol=1e-3)
+
+
+def test_softmax_reference_cases(gpu):
+    import torch
+
+    def sm(v):
+        a = dev(np.array(v, dtype=np.float32))
+        out = torch.zeros_like(a)
+        gpu.softmax(a, out, 0)
+        return out.cpu().numpy()
+
+    assert abs(sm([1, 2, 3]).sum() - 1.0) < 1e-6
+    y = sm([1, 3, 2])
+    assert y[1] > y[2] > y[0]
+    y = sm([1000, 1001, 1002])
+    assert np.isfinite(y).all() and abs(y.sum() - 1.0) < 1e-6
+    np.testing.assert_allclose(sm([2, 2, 2]), 1.0 / 3.0, atol=1e-7)
+    denom = 1.0 + np.exp(1.0)
+    np.testing.assert_allclose(sm([0, 1]), [1.0 / denom, np.exp(1.0) / denom], atol=1e-7)
+    # axis 1 of the 2x3 column-major matrix (tests.cpp:1206-1221)
+    a = col_major(np.array([[1, 3, 5], [2, 4, 6]], dtype=np.float32))
+    out = torch.zeros_like(a)
+    gpu.softmax(a, out, 1)
+    e = np.exp(np.array([1.0, 3.0, 5.0]) - 5.0)
+    np.testing.assert_allclose(out.cpu().numpy(), np.stack([e / e.sum()] * 2), atol=1e-7)
+
+
+@pytest.mark.parametrize("shape", [(5,), (3, 1000), (1000, 3), (2, 3, 4, 5), (1, 32, 1, 2048), (4, 7, 33, 65)])
+def test_softmax_and_reduce_strided_against_checker(gpu, oracle, shape):
+    import torch
+    rng = np.random.default_rng(len(shape) * 100 + shape[-1])
+    x = (rng.standard_normal(shape, dtype=np.float32) * 3.0)
+    flat = np.transpose(x).reshape(-1).copy()  # column-major storage
+    stride = [int(np.prod(shape[:i])) for i in range(len(shape))]
+    for mk in (col_major, dev):
+        xd = mk(x)
+        for axis in range(len(shape)):
+            out = torch.zeros_like(xd)
+            gpu.softmax(xd, out, axis)
+            want = np.zeros_like(flat)
+            oracle.softmax(list(shape), axis, flat, 0, stride, want, 0, stride)
+            want = np.transpose(want.reshape(shape[::-1]))
+            np.testing.assert_allclose(out.cpu().numpy(), want, rtol=2e-5, atol=1e-7)
+            oshape = [s for i, s in enumerate(shape) if i != axis] or [1]
+            for op, fn in ((gpu.REDUCE_SUM, np.sum), (gpu.REDUCE_MAX, np.max), (gpu.REDUCE_MIN, np.min)):
+                r = torch.zeros(oshape, device="cuda")
+                if len(shape) == 1:
+                    gpu.check(gpu.load().weed_hip_reduce_f32(op, 1, gpu.u32(shape), 0, xd.data_ptr(), 0,
+                                                             gpu.u32(xd.stride()), r.data_ptr(), 0, gpu.u32([0])))
+                else:
+                    gpu.reduce(op, xd, r, axis)
+                ref = fn(x.astype(np.float64), axis=axis).reshape(oshape)
+                if op == gpu.REDUCE_SUM:
+                    np.testing.assert_allclose(r.cpu().numpy(), ref, rtol=2e-5, atol=2e-5 * np.sqrt(shape[axis]))
+                else:
+                    np.testing.assert_array_equal(r.cpu().numpy(), ref.astype(np.float32))
+
+
+def test_reduce_reference_cases(gpu):
+    import torch
+    # tests.cpp:177-228: sum([1,1]) = 2, max([0,1]) = 1, min([0,1]) = 0
+    for op, v, want in ((gpu.REDUCE_SUM, [1, 1], 2), (gpu.REDUCE_MAX, [0, 1], 1), (gpu.REDUCE_MIN, [0, 1], 0)):
+        a = dev(np.array(v, dtype=np.float32))
+        r = torch.zeros(1, device="cuda")
+        gpu.check(gpu.load().weed_hip_reduce_f32(op, 1, gpu.u32([2]), 0, a.data_ptr(), 0, gpu.u32([1]), r.data_ptr(), 0,
+                                                 gpu.u32([0])))
+        assert r.cpu().item() == want
+
+
+def test_softmax_on_a_view_with_offset(gpu, oracle):
+    import torch
+    rng = np.random.default_rng(8)
+    big = dev(rng.standard_normal((6, 40), dtype=np.float32))
+    view = big[1:5, 3:35:2]
+    out = torch.full((6, 40), 7.0, device="cuda")
+    gpu.softmax(view, out[1:5, 3:35:2], 1)
+    x = view.cpu().numpy().astype(np.float64)
+    e = np.exp(x - x.max(axis=1, keepdims=True))
+    np.testing.assert_allclose(out[1:5, 3:35:2].cpu().numpy(), e / e.sum(axis=1, keepdims=True), rtol=2e-5, atol=1e-7)
+    assert torch.all(out[0] == 7.0) and torch.all(out[:, 4::2] == 7.0)

@@ -1,0 +1,241 @@
+"""GPU parity of the KV encoder, the packed cache and its read-back, through the C ABI.
+
+Bar: codes, sign bits, Weed-packed words, row scales and dequantised values are BIT-EXACT against the CPU checker
+given the same rotated input; with the rotation done on the device in the reference's rounding order (rotate = 2)
+they are bit-exact end to end.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from gpu_helpers import col_major, coder_specs, dev, export
+
+pytestmark = pytest.mark.gpu
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def test_uniform_known_answers_on_device(gpu, oracle):
+    """The reference's recorded write_row / read_row answers (multihead_attention.cpp:43-79), padded to d = 32."""
+    import torch
+    with open(os.path.join(HERE, "golden", "weed_uniform_kat.json")) as f:
+        kat = json.load(f)
+    for case in kat["write_row"]:
+        n = len(case["vals"])
+        row = np.zeros((1, 1, 1, 32), dtype=np.float32)
+        row[0, 0, 0, :n] = case["vals"]
+        cache = gpu.KVCache(gpu.KV_UNIFORM, 1, 1, 32, 8, case["bits"], case["bits"])
+        cache.set_scales(case["block_scale"], case["block_scale"])
+        x = dev(row)
+        cache.encode_append(x, x, rotate=0)
+        fields, _ = export(cache, 0, 1)
+        np.testing.assert_array_equal(fields[0, 0, 0, :n], case["codes"])
+        # Weed's own word packing of the same row
+        wpr = oracle.words_per_row(32, case["bits"])
+        words = torch.zeros((1, 1, 1, wpr), dtype=torch.int32, device="cuda")
+        cache.export_weed_words(1, words)
+        np.testing.assert_array_equal(words.cpu().numpy()[0, 0, 0],
+                                      oracle.uniform_write_rows(row.reshape(1, 32), case["bits"],
+                                                                case["block_scale"])[0])
+        cache.close()
+    case = kat["read_row"][0]
+    row = np.zeros((1, 1, 1, 32), dtype=np.float32)
+    row[0, 0, 0, :4] = [0.5, -1.2, 2.0, -0.05]
+    cache = gpu.KVCache(gpu.KV_UNIFORM, 1, 1, 32, 8, 4, 4)
+    cache.set_scales(case["block_scale"], case["block_scale"])
+    x = dev(row)
+    cache.encode_append(x, x, rotate=0)
+    out = torch.zeros((1, 1, 1, 32), dtype=torch.float32, device="cuda")
+    cache.dequant(0, out)
+    np.testing.assert_allclose(out.cpu().numpy()[0, 0, 0, :4], np.array(case["vals"], dtype=np.float32), rtol=0,
+                               atol=6e-8)
+    cache.close()
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("d", [64, 128])
+def test_uniform_encode_bit_exact(gpu, oracle, bits, d):
+    import torch
+    rng = np.random.default_rng(100 * bits + d)
+    S, Hkv, T = 2, 3, 150
+    K = rng.normal(0, 1.2, size=(S, Hkv, T, d)).astype(np.float32)
+    V = rng.normal(0, 0.7, size=(S, Hkv, T, d)).astype(np.float32)
+    K[0, 0, 0, :4] = [np.inf, -np.inf, 1e30, -1e30]  # clamped, not faulted
+    ks, vs = oracle.block_scale(K[np.isfinite(K)]), oracle.block_scale(V)
+    cache = gpu.KVCache(gpu.KV_UNIFORM, S, Hkv, d, 200, bits, bits)
+    cache.set_scales(ks, vs)
+    # Weed's own layout: column-major [B, H, T, d] (dimension 0 fastest)
+    cache.encode_append(col_major(K), col_major(V), rotate=0)
+    assert cache.seq_lens() == [T, T]
+    kspec, vspec = coder_specs(oracle, cache)
+    for which, x, spec in ((0, K, kspec), (1, V, vspec)):
+        want_f, _ = oracle.encode_rows(spec, x.reshape(-1, d))
+        got_f, _ = export(cache, which, T)
+        np.testing.assert_array_equal(got_f.reshape(-1, d), want_f)
+        wpr = oracle.words_per_row(d, bits)
+        words = torch.zeros((S, Hkv, T, wpr), dtype=torch.int32, device="cuda")
+        cache.export_weed_words(which, words)
+        want_w = oracle.uniform_write_rows(x.reshape(-1, d), bits, spec.block_scale)
+        np.testing.assert_array_equal(words.cpu().numpy().reshape(-1, wpr), want_w)
+        # read_row: identical floats, not merely close
+        out = torch.zeros((S, Hkv, T, d), dtype=torch.float32, device="cuda")
+        cache.dequant(which, out)
+        want_d = oracle.uniform_read_rows(want_w, d, bits, spec.block_scale)
+        np.testing.assert_array_equal(out.cpu().numpy().reshape(-1, d), want_d)
+    cache.close()
+
+
+@pytest.mark.parametrize("k_bits,k_sign,v_bits,v_sign", [(4, 1, 4, 1), (3, 1, 4, 0), (3, 0, 4, 0), (2, 1, 3, 0),
+                                                         (1, 0, 2, 0)])
+@pytest.mark.parametrize("d", [64, 128])
+def test_lloydmax_encode_bit_exact(gpu, oracle, k_bits, k_sign, v_bits, v_sign, d):
+    import torch
+    rng = np.random.default_rng(k_bits * 1000 + v_bits * 100 + d)
+    S, Hkv, T = 2, 2, 133
+    K = (rng.normal(size=(S, Hkv, T, d)) * rng.uniform(0.2, 5, size=(S, Hkv, T, 1))).astype(np.float32)
+    V = rng.normal(size=(S, Hkv, T, d)).astype(np.float32)
+    V[1, 1, 7] = 0.0  # an all-zero row: scale 0, codes of u = 0
+    cache = gpu.KVCache(gpu.KV_LLOYDMAX, S, Hkv, d, 256, k_bits, v_bits, k_sign, v_sign)
+    cache.encode_append(dev(K), dev(V), rotate=0)
+    kspec, vspec = coder_specs(oracle, cache)
+    for which, x, spec in ((0, K, kspec), (1, V, vspec)):
+        want_f, want_a = oracle.encode_rows(spec, x.reshape(-1, d))
+        got_f, got_a = export(cache, which, T)
+        np.testing.assert_array_equal(got_f.reshape(-1, d), want_f)
+        np.testing.assert_array_equal(got_a.reshape(-1), want_a)  # row scales bit-exact
+        out = torch.zeros((S, Hkv, T, d), dtype=torch.float32, device="cuda")
+        cache.dequant(which, out)
+        np.testing.assert_array_equal(out.cpu().numpy().reshape(-1, d), oracle.decode_rows(spec, want_f, want_a))
+    assert cache.row_bytes() == (d * (k_bits + k_sign) // 8 + 4, d * (v_bits + v_sign) // 8 + 4)
+    cache.close()
+
+
+@pytest.mark.parametrize("mode", ["uniform", "lloydmax"])
+def test_device_rotation_modes(gpu, oracle, mode):
+    """rotate = 2 reproduces the reference's rounding (matmul.cpp:40-44), so codes stay bit-exact end to end;
+    rotate = 1 uses fused multiply-adds and may move values that sit on a cell edge."""
+    import torch
+    rng = np.random.default_rng(77)
+    S, Hkv, T, d = 1, 2, 96, 128
+    K = rng.normal(size=(S, Hkv, T, d)).astype(np.float32)
+    V = rng.normal(size=(S, Hkv, T, d)).astype(np.float32)
+    Rk = oracle.orthonormalize_columns(rng.normal(size=d * d).astype(np.float32))
+    Rv = oracle.orthonormalize_columns(rng.normal(size=d * d).astype(np.float32))
+    Ky = oracle.apply_rotation(K.reshape(-1, d), Rk)
+    Vy = oracle.apply_rotation(V.reshape(-1, d), Rv)
+    for rotate in (2, 1):
+        if mode == "uniform":
+            cache = gpu.KVCache(gpu.KV_UNIFORM, S, Hkv, d, 128, 4, 4)
+            cache.set_scales(oracle.block_scale(Ky), oracle.block_scale(Vy))
+        else:
+            cache = gpu.KVCache(gpu.KV_LLOYDMAX, S, Hkv, d, 128, 3, 4, 1, 0)
+        cache.set_rotations(dev(Rk), dev(Rv))
+        cache.encode_append(dev(K), dev(V), rotate=rotate)
+        kspec, vspec = coder_specs(oracle, cache)
+        for which, y, spec in ((0, Ky, kspec), (1, Vy, vspec)):
+            want_f, want_a = oracle.encode_rows(spec, y)
+            got_f, got_a = export(cache, which, T)
+            if rotate == 2:
+                np.testing.assert_array_equal(got_f.reshape(-1, d), want_f)
+                np.testing.assert_array_equal(got_a.reshape(-1), want_a)
+            else:
+                assert np.mean(got_f.reshape(-1, d) != want_f) < 2e-3
+                np.testing.assert_allclose(got_a.reshape(-1), want_a, rtol=1e-5)
+        cache.close()
+
+
+def test_incremental_and_ragged_append(gpu, oracle):
+    """Appending token by token, in uneven chunks and per sequence must give the cache a one-shot encode gives
+    (the reference's own incremental append re-reads old rows with the wrong strides)."""
+    rng = np.random.default_rng(5)
+    S, Hkv, d, cap = 3, 2, 64, 300
+    lens = [300, 71, 190]
+    K = rng.normal(size=(S, Hkv, cap, d)).astype(np.float32)
+    V = rng.normal(size=(S, Hkv, cap, d)).astype(np.float32)
+    cache = gpu.KVCache(gpu.KV_LLOYDMAX, S, Hkv, d, cap, 2, 3, 1, 0)
+    Kd, Vd = dev(K), dev(V)
+    # a shared prefill of 70 tokens for all sequences, then per-sequence continuations in odd chunk sizes
+    cache.encode_append(Kd[:, :, :70], Vd[:, :, :70])
+    for s, L in enumerate(lens):
+        pos = 70
+        for chunk in (1, 1, 1, 30, 64, 5, 1000):
+            n = min(chunk, L - pos)
+            if n <= 0:
+                break
+            cache.encode_append(Kd[s:s + 1, :, pos:pos + n], Vd[s:s + 1, :, pos:pos + n], seq_begin=s)
+            pos += n
+    assert cache.seq_lens() == lens
+    kspec, vspec = coder_specs(oracle, cache)
+    for which, x, spec in ((0, K, kspec), (1, V, vspec)):
+        got_f, got_a = export(cache, which, cap)
+        for s, L in enumerate(lens):
+            want_f, want_a = oracle.encode_rows(spec, x[s, :, :L].reshape(-1, d))
+            np.testing.assert_array_equal(got_f[s, :, :L].reshape(-1, d), want_f)
+            np.testing.assert_array_equal(got_a[s, :, :L].reshape(-1), want_a)
+    # capacity is checked on the host; nothing is written
+    with pytest.raises(gpu.WeedHipError) as e:
+        cache.encode_append(Kd[0:1, :, :1], Vd[0:1, :, :1], seq_begin=0)
+    assert e.value.code == gpu.ECAPACITY
+    # reset empties the cache and it can be refilled
+    cache.reset()
+    assert cache.seq_lens() == [0, 0, 0]
+    cache.encode_append(Kd[:, :, 5:15], Vd[:, :, 5:15])
+    got_f, _ = export(cache, 0, 10)
+    want_f, _ = oracle.encode_rows(kspec, K[:, :, 5:15].reshape(-1, d))
+    np.testing.assert_array_equal(got_f.reshape(-1, d), want_f)
+    cache.close()
+
+
+def test_block_scale(gpu, oracle):
+    rng = np.random.default_rng(9)
+    x = rng.normal(0, 1.7, size=(2, 3, 40, 64)).astype(np.float32)
+    # sequential: the reference's one-accumulator fp32 order over the storage of a contiguous tensor -> bit-exact
+    t = col_major(x)
+    flat = np.transpose(x).reshape(-1)  # storage order of the column-major tensor
+    assert gpu.block_scale(t, sequential=True) == np.float32(oracle.block_scale(flat))
+    want = np.sqrt(np.mean(x.astype(np.float64) ** 2) + 1e-8)
+    assert abs(gpu.block_scale(t) - want) < 1e-6 * want
+    assert abs(gpu.block_scale(dev(x)[:, 1:, ::2]) - np.sqrt(np.mean(x[:, 1:, ::2].astype(np.float64) ** 2) + 1e-8)) \
+        < 1e-6 * want
+
+
+def test_rotation_on_device(gpu, oracle):
+    import torch
+    for d in (64, 128):
+        R = torch.zeros(d * d, dtype=torch.float32, device="cuda")
+        gpu.make_rotation(1234 + d, d, R)
+        Rm = R.cpu().numpy().reshape(d, d).T.astype(np.float64)
+        np.testing.assert_allclose(Rm.T @ Rm, np.eye(d), atol=3e-4)
+        # same seed, same matrix; another seed, another matrix
+        R2 = torch.zeros_like(R)
+        gpu.make_rotation(1234 + d, d, R2)
+        assert torch.equal(R, R2)
+        gpu.make_rotation(99, d, R2)
+        assert not torch.equal(R, R2)
+        # device Gram-Schmidt against the CPU checker on the same Gaussian draws
+        g = np.random.default_rng(d).normal(size=d * d).astype(np.float32)
+        Rg = dev(g.copy())
+        gpu.orthonormalize_columns(d, Rg)
+        np.testing.assert_allclose(Rg.cpu().numpy(), oracle.orthonormalize_columns(g), atol=2e-4)
+
+
+def test_argument_errors_are_reported_not_faulted(gpu):
+    import torch
+    with pytest.raises(gpu.WeedHipError) as e:
+        gpu.KVCache(gpu.KV_LLOYDMAX, 1, 1, 48, 16, 3, 3)  # head_dim not a multiple of 32
+    assert e.value.code == gpu.EINVAL
+    with pytest.raises(gpu.WeedHipError):
+        gpu.KVCache(gpu.KV_UNIFORM, 1, 1, 64, 16, 3, 3, 1, 0)  # the uniform coder has no sign bit
+    with pytest.raises(gpu.WeedHipError):
+        gpu.KVCache(gpu.KV_LLOYDMAX, 1, 1, 64, 16, 5, 3)  # code width out of range
+    cache = gpu.KVCache(gpu.KV_LLOYDMAX, 2, 2, 64, 16, 3, 3)
+    x = torch.zeros((1, 2, 4, 64), device="cuda")
+    with pytest.raises(gpu.WeedHipError):
+        cache.encode_append(x, x, seq_begin=2)  # sequence range outside the cache
+    with pytest.raises(gpu.WeedHipError):
+        cache.encode_append(x, x, rotate=1)  # no rotations set
+    q = torch.zeros((2, 3, 64), device="cuda")
+    with pytest.raises(gpu.WeedHipError):
+        cache.decode_attn(q, torch.zeros_like(q))  # 3 query heads over 2 kv heads
+    cache.close()

@@ -1,0 +1,222 @@
+// Strided fp32 softmax and axis reductions (the standalone ops that feed attention in the reference:
+// src/ops/softmax.cpp:276-287, src/ops/reduce.cpp:342-386).
+//
+// Rows (all index combinations of the non-reduced dimensions) are enumerated with dimension 0 fastest, which is the
+// contiguous direction of Weed's column-major tensors; a workgroup takes RT neighbouring rows and spreads the
+// remaining threads along the reduced axis, so that loads are coalesced whether the axis is the contiguous
+// dimension (RT = 1) or a strided one (RT = 16).
+#include "common.h"
+
+#include <cmath>
+
+using namespace weedhip;
+
+namespace {
+
+constexpr int kMaxRank = 8;
+constexpr int kThreads = 256;
+
+struct AxisGeom {
+    uint32_t rank;
+    uint32_t axis;
+    uint32_t shape[kMaxRank];
+    uint32_t a_stride[kMaxRank];
+    uint32_t o_stride[kMaxRank];
+    uint32_t a_off, o_off;
+    uint32_t rows;
+    uint32_t axis_len;
+};
+
+__device__ __forceinline__ void row_bases(const AxisGeom &g, uint32_t row, uint64_t &a_base, uint64_t &o_base)
+{
+    a_base = g.a_off;
+    o_base = g.o_off;
+    uint32_t tmp = row;
+    for (uint32_t dd = 0; dd < g.rank; ++dd) {
+        if (dd == g.axis) {
+            continue;
+        }
+        const uint32_t dim = g.shape[dd];
+        const uint32_t i = tmp % dim;
+        tmp /= dim;
+        a_base += (uint64_t)i * g.a_stride[dd];
+        o_base += (uint64_t)i * g.o_stride[dd];
+    }
+}
+
+// op: 0 sum, 1 max, 2 min
+template <int OP> __device__ __forceinline__ float combine(float a, float b)
+{
+    if (OP == 0) {
+        return a + b;
+    }
+    if (OP == 1) {
+        return b > a ? b : a;
+    }
+    return b < a ? b : a;
+}
+
+template <int OP> __device__ __forceinline__ float identity()
+{
+    if (OP == 0) {
+        return 0.0f;
+    }
+    return OP == 1 ? -INFINITY : INFINITY;
+}
+
+// Reduce `v` over the NY threads that share threadIdx.x % RT; the result is valid in every thread.
+template <int OP, int RT> __device__ __forceinline__ float block_reduce(float v, float *red)
+{
+    constexpr int NY = kThreads / RT;
+    const uint32_t tx = threadIdx.x % RT, ty = threadIdx.x / RT;
+    red[ty * RT + tx] = v;
+    __syncthreads();
+    for (int s = NY / 2; s > 0; s >>= 1) {
+        if ((int)ty < s) {
+            red[ty * RT + tx] = combine<OP>(red[ty * RT + tx], red[(ty + s) * RT + tx]);
+        }
+        __syncthreads();
+    }
+    const float r = red[tx];
+    __syncthreads();
+    return r;
+}
+
+template <int RT> __global__ void __launch_bounds__(kThreads) softmax_kernel(const float *__restrict__ a,
+                                                                            float *__restrict__ out, AxisGeom g)
+{
+    __shared__ float red[kThreads];
+    constexpr int NY = kThreads / RT;
+    const uint32_t tx = threadIdx.x % RT, ty = threadIdx.x / RT;
+    const uint32_t row = blockIdx.x * RT + tx;
+    const bool valid = row < g.rows;
+    uint64_t a_base = 0, o_base = 0;
+    if (valid) {
+        row_bases(g, row, a_base, o_base);
+    }
+    const uint32_t as = g.a_stride[g.axis], os = g.o_stride[g.axis];
+    float mx = -INFINITY;
+    if (valid) {
+        for (uint32_t j = ty; j < g.axis_len; j += NY) {
+            mx = fmaxf(mx, a[a_base + (uint64_t)j * as]);
+        }
+    }
+    mx = block_reduce<1, RT>(mx, red);
+    float s = 0.0f;
+    if (valid) {
+        for (uint32_t j = ty; j < g.axis_len; j += NY) {
+            s += expf(a[a_base + (uint64_t)j * as] - mx);
+        }
+    }
+    s = block_reduce<0, RT>(s, red);
+    if (valid) {
+        for (uint32_t j = ty; j < g.axis_len; j += NY) {
+            out[o_base + (uint64_t)j * os] = expf(a[a_base + (uint64_t)j * as] - mx) / s;
+        }
+    }
+}
+
+template <int OP, int RT> __global__ void __launch_bounds__(kThreads) reduce_kernel(const float *__restrict__ a,
+                                                                                   float *__restrict__ out, AxisGeom g)
+{
+    __shared__ float red[kThreads];
+    constexpr int NY = kThreads / RT;
+    const uint32_t tx = threadIdx.x % RT, ty = threadIdx.x / RT;
+    const uint32_t row = blockIdx.x * RT + tx;
+    const bool valid = row < g.rows;
+    uint64_t a_base = 0, o_base = 0;
+    if (valid) {
+        row_bases(g, row, a_base, o_base);
+    }
+    const uint32_t as = g.a_stride[g.axis];
+    float v = identity<OP>();
+    if (valid) {
+        for (uint32_t j = ty; j < g.axis_len; j += NY) {
+            v = combine<OP>(v, a[a_base + (uint64_t)j * as]);
+        }
+    }
+    v = block_reduce<OP, RT>(v, red);
+    if (valid && ty == 0) {
+        out[o_base] = v;
+    }
+}
+
+int make_geom(const char *fn, uint32_t rank, const uint32_t *shape, uint32_t axis, uint32_t a_off,
+              const uint32_t *a_stride, uint32_t o_off, const uint32_t *o_stride, bool out_keeps_axis, AxisGeom &g)
+{
+    WEED_HIP_REQUIRE(shape && a_stride && o_stride, "%s: null pointer", fn);
+    WEED_HIP_REQUIRE(rank >= 1 && rank <= (uint32_t)kMaxRank, "%s: rank %u outside [1, %d]", fn, rank, kMaxRank);
+    WEED_HIP_REQUIRE(axis < rank, "%s: axis %u out of range for rank %u", fn, axis, rank);
+    g.rank = rank;
+    g.axis = axis;
+    g.a_off = a_off;
+    g.o_off = o_off;
+    uint64_t rows = 1;
+    for (uint32_t i = 0; i < rank; ++i) {
+        WEED_HIP_REQUIRE(shape[i] > 0, "%s: dimension %u is empty", fn, i);
+        g.shape[i] = shape[i];
+        g.a_stride[i] = a_stride[i];
+        g.o_stride[i] = (i == axis && !out_keeps_axis) ? 0 : o_stride[i];
+        if (i != axis) {
+            rows *= shape[i];
+        }
+    }
+    WEED_HIP_REQUIRE(rows < (1ull << 31), "%s: too many rows", fn);
+    g.rows = (uint32_t)rows;
+    g.axis_len = shape[axis];
+    return WEED_HIP_OK;
+}
+
+} // namespace
+
+extern "C" {
+
+int weed_hip_softmax_f32(uint32_t rank, const uint32_t *shape, uint32_t axis, const float *a_dev, uint32_t a_off,
+                         const uint32_t *a_stride, float *out_dev, uint32_t o_off, const uint32_t *o_stride)
+{
+    const char *fn = "weed_hip_softmax_f32";
+    WEED_HIP_REQUIRE(a_dev && out_dev, "%s: null pointer", fn);
+    WEED_HIP_TRY(ensure_init());
+    AxisGeom g;
+    WEED_HIP_TRY(make_geom(fn, rank, shape, axis, a_off, a_stride, o_off, o_stride, true, g));
+    ProfileScope prof("softmax");
+    if (g.a_stride[axis] <= 1 || g.rows < 16) {
+        softmax_kernel<1><<<g.rows, kThreads, 0, stream()>>>(a_dev, out_dev, g);
+    } else {
+        softmax_kernel<16><<<(g.rows + 15) / 16, kThreads, 0, stream()>>>(a_dev, out_dev, g);
+    }
+    WEED_HIP_LAUNCH_CHECK();
+    return WEED_HIP_OK;
+}
+
+int weed_hip_reduce_f32(int op, uint32_t rank, const uint32_t *shape, uint32_t axis, const float *a_dev, uint32_t a_off,
+                        const uint32_t *a_stride, float *out_dev, uint32_t o_off, const uint32_t *o_stride)
+{
+    const char *fn = "weed_hip_reduce_f32";
+    WEED_HIP_REQUIRE(a_dev && out_dev, "%s: null pointer", fn);
+    WEED_HIP_REQUIRE(op >= 0 && op <= 2, "%s: unknown op %d", fn, op);
+    WEED_HIP_TRY(ensure_init());
+    AxisGeom g;
+    WEED_HIP_TRY(make_geom(fn, rank, shape, axis, a_off, a_stride, o_off, o_stride, false, g));
+    ProfileScope prof("reduce");
+    const bool narrow = g.a_stride[axis] <= 1 || g.rows < 16;
+    const uint32_t blocks = narrow ? g.rows : (g.rows + 15) / 16;
+#define WEED_LAUNCH_REDUCE(OP)                                                                                         \
+    if (narrow) {                                                                                                      \
+        reduce_kernel<OP, 1><<<blocks, kThreads, 0, stream()>>>(a_dev, out_dev, g);                                    \
+    } else {                                                                                                           \
+        reduce_kernel<OP, 16><<<blocks, kThreads, 0, stream()>>>(a_dev, out_dev, g);                                   \
+    }
+    if (op == WEED_HIP_REDUCE_SUM) {
+        WEED_LAUNCH_REDUCE(0)
+    } else if (op == WEED_HIP_REDUCE_MAX) {
+        WEED_LAUNCH_REDUCE(1)
+    } else {
+        WEED_LAUNCH_REDUCE(2)
+    }
+#undef WEED_LAUNCH_REDUCE
+    WEED_HIP_LAUNCH_CHECK();
+    return WEED_HIP_OK;
+}
+
+} // extern "C"

@@ -1,0 +1,60 @@
+// Device twin of Weed::QuantizedKVCache (include/modules/multihead_attention.hpp:22-36) plus the state
+// MultiHeadAttention keeps beside it (k_rotation, v_rotation, v_rotation_trans, cache_len; hpp:56-68).
+#pragma once
+
+#include <vector>
+
+#include "common.h"
+#include "kv_layout.h"
+
+namespace weedhip {
+
+// What a kernel needs to turn one tensor's fields back into numbers: value = alpha * table[field] + beta,
+// with alpha the row scale (LLOYDMAX) or the cell width (UNIFORM, where table[c] = c + 0.5 and beta = -3s).
+struct SideParams {
+    const uint32_t *fields; // packed groups, one region per (sequence, kv head)
+    const float *alpha;     // [n_seq][n_kv_heads][padded_tokens] row scales, LLOYDMAX only
+    uint64_t region_dwords;
+    uint32_t w;             // field width
+    float alpha_const;      // UNIFORM: step
+    float beta;             // UNIFORM: lo
+    float table[32];        // reconstruction levels, 2^w entries
+};
+
+struct Side {
+    int bits = 0;
+    int sign = 0;
+    uint32_t w = 0;
+    uint32_t *fields = nullptr;
+    float *alpha = nullptr;
+    uint64_t region_dwords = 0;
+    float block_scale = 1.0f; // UNIFORM (Weed: QuantizedKVCache::block_scale)
+    float bounds[15] = {};
+    float levels[16] = {};
+    float recon[32] = {};
+    float *rot = nullptr;   // column-major d x d (k_rotation / v_rotation)
+    float *rot_t = nullptr; // its transpose (v_rotation_trans and the coalesced form of k_rotation)
+};
+
+} // namespace weedhip
+
+struct weed_hip_kv_cache {
+    weed_hip_kv_config cfg;
+    uint32_t padded_tokens = 0;
+    weedhip::Side k, v;
+    bool has_rotations = false;
+    std::vector<int32_t> lens; // host mirror of lens_dev
+    int32_t *lens_dev = nullptr;
+    // scratch for encode: one field per byte + row scales for the tokens being appended
+    uint8_t *enc_fields = nullptr;
+    float *enc_alpha = nullptr;
+    size_t enc_rows_cap = 0;
+    // scratch for decode: rotated queries and split partials
+    float *dec_ws = nullptr;
+    size_t dec_ws_bytes = 0;
+};
+
+namespace weedhip {
+// Builds the kernel-side view of one tensor of the cache.
+SideParams side_params(const weed_hip_kv_cache *c, int which);
+} // namespace weedhip

@@ -1,0 +1,979 @@
+// Quantized KV cache: allocation, encode-and-append, dequantise, export.
+//
+// Device twin of Weed::QuantizedKVCache (src/modules/multihead_attention.cpp:31-79) and of the encode half of
+// MultiHeadAttention::forward (cpp:206-257).  Compiled with -ffp-contract=off: every multiply-add that must round
+// twice (as the reference's x86-64 build does) is written as separate operations, every fused one as fmaf().
+#include "kv_cache.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <new>
+
+#include "lloyd_tables.inc"
+
+using namespace weedhip;
+using namespace weedkv;
+
+namespace {
+
+struct Geom4 {
+    uint32_t off;
+    uint32_t s[4];
+};
+
+struct BuiltinTable {
+    const float *levels, *bounds, *refined;
+};
+
+BuiltinTable builtin_table(int bits)
+{
+    switch (bits) {
+    case 1:
+        return { WEED_LM_LEVELS_1, WEED_LM_BOUNDS_1, WEED_LM_REFINED_1 };
+    case 2:
+        return { WEED_LM_LEVELS_2, WEED_LM_BOUNDS_2, WEED_LM_REFINED_2 };
+    case 3:
+        return { WEED_LM_LEVELS_3, WEED_LM_BOUNDS_3, WEED_LM_REFINED_3 };
+    default:
+        return { WEED_LM_LEVELS_4, WEED_LM_BOUNDS_4, WEED_LM_REFINED_4 };
+    }
+}
+
+// Round to the nearest IEEE binary16 value (ties to even), saturating at the largest finite one.
+float round_to_half(float x)
+{
+    if (!std::isfinite(x)) {
+        return x;
+    }
+    const float max_half = 65504.0f;
+    if (std::fabs(x) >= max_half) {
+        return std::copysign(max_half, x);
+    }
+    int e;
+    (void)std::frexp(x, &e); // x = m * 2^e, 0.5 <= |m| < 1
+    // binary16 keeps 11 significant bits for normal numbers (e >= -13), fewer below.
+    int quantum_exp = e - 11;
+    if (quantum_exp < -24) {
+        quantum_exp = -24;
+    }
+    const float q = std::ldexp(1.0f, quantum_exp);
+    return std::nearbyint(x / q) * q;
+}
+
+void load_builtin(Side &s)
+{
+    const BuiltinTable t = builtin_table(s.bits);
+    const int n = 1 << s.bits;
+    std::memcpy(s.levels, t.levels, sizeof(float) * n);
+    std::memcpy(s.bounds, t.bounds, sizeof(float) * (n - 1));
+    if (s.sign) {
+        std::memcpy(s.recon, t.refined, sizeof(float) * 2 * n);
+    } else {
+        std::memcpy(s.recon, t.levels, sizeof(float) * n);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// kernels
+// ------------------------------------------------------------------------------------------------
+
+__global__ void transpose_square_kernel(const float *__restrict__ r, float *__restrict__ rt, uint32_t d)
+{
+    const uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= d * d) {
+        return;
+    }
+    const uint32_t i = idx % d, j = idx / d;
+    rt[j + d * i] = r[i + d * j];
+}
+
+__global__ void bump_lens_kernel(int32_t *lens, int32_t seq_begin, int32_t seq_count, int32_t add)
+{
+    const int32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < seq_count) {
+        lens[seq_begin + i] += add;
+    }
+}
+
+__global__ void fill_i32_kernel(int32_t *p, int32_t v, uint32_t n)
+{
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        p[i] = v;
+    }
+}
+
+struct CoderParams {
+    int mode;
+    int bits;
+    int sign;
+    float block_scale;
+    float bounds[15];
+    float levels[16];
+};
+
+// The bucket arithmetic of QuantizedKVCache::write_row (multihead_attention.cpp:49-58), operation for operation.
+__device__ __forceinline__ uint32_t uniform_bucket(float v, float lo, float hi, float step, int levels)
+{
+    int bucket = 0;
+    if (step > 1e-8f) {
+        const float hs = hi - step;
+        const float m = (v < hs) ? v : hs;
+        const float clamped = (lo < m) ? m : lo;
+        bucket = (int)((clamped - lo) / step);
+        bucket = bucket > levels - 1 ? levels - 1 : bucket;
+        bucket = bucket < 0 ? 0 : bucket;
+    }
+    return (uint32_t)bucket;
+}
+
+constexpr int kEncRows = 32;     // rows per workgroup
+constexpr int kEncThreads = 256;
+
+// Rotate (optional) and quantise kEncRows rows of a strided [S, Hkv, T, d] tensor into one field per byte.
+//   rotate 0: y = x            1: y = x.R with fused multiply-adds         2: y = x.R with the reference's
+//   rounding (multiply, then add, i ascending: src/ops/matmul.cpp:40-44).
+// PARTS = number of row slices the 256 threads are split into (each thread owns one output column of its slice).
+template <int PARTS>
+__global__ void __launch_bounds__(kEncThreads)
+    encode_rows_kernel(const float *__restrict__ x, Geom4 g, uint32_t Hkv, uint32_t T, uint32_t d, uint32_t rows,
+                       const float *__restrict__ rot_t, int rotate, CoderParams cp, uint8_t *__restrict__ fields,
+                       float *__restrict__ alpha_out)
+{
+    extern __shared__ float smem[];
+    const uint32_t pitch = d + 1;
+    float *xs = smem;                   // [kEncRows][pitch]
+    float *ys = smem + kEncRows * pitch; // [kEncRows][pitch]
+    float *inv_s = ys + kEncRows * pitch; // [kEncRows]
+    const uint32_t tid = threadIdx.x;
+    const uint32_t row0 = blockIdx.x * kEncRows;
+
+    // gather the rows (logical row = (s*Hkv + h)*T + t)
+    for (uint32_t e = tid; e < kEncRows * d; e += kEncThreads) {
+        const uint32_t r = e / d, j = e % d;
+        const uint32_t row = row0 + r;
+        float val = 0.0f;
+        if (row < rows) {
+            const uint32_t t = row % T;
+            const uint32_t h = (row / T) % Hkv;
+            const uint32_t s = row / (T * Hkv);
+            const uint64_t idx = (uint64_t)g.off + (uint64_t)s * g.s[0] + (uint64_t)h * g.s[1] + (uint64_t)t * g.s[2] +
+                                 (uint64_t)j * g.s[3];
+            val = x[idx];
+        }
+        (rotate ? xs : ys)[r * pitch + j] = val;
+    }
+    __syncthreads();
+
+    if (rotate) {
+        constexpr int RPP = kEncRows / PARTS; // rows per part
+        const uint32_t j = tid % d;
+        const uint32_t part = tid / d;
+        if (part < PARTS) {
+            float acc[RPP];
+#pragma unroll
+            for (int r = 0; r < RPP; ++r) {
+                acc[r] = 0.0f;
+            }
+            const float *xrow = xs + part * RPP * pitch;
+            if (rotate == 2) {
+                for (uint32_t i = 0; i < d; ++i) {
+                    const float rv = rot_t[j + d * i];
+#pragma unroll
+                    for (int r = 0; r < RPP; ++r) {
+                        acc[r] = acc[r] + xrow[r * pitch + i] * rv;
+                    }
+                }
+            } else {
+                for (uint32_t i = 0; i < d; ++i) {
+                    const float rv = rot_t[j + d * i];
+#pragma unroll
+                    for (int r = 0; r < RPP; ++r) {
+                        acc[r] = fmaf(xrow[r * pitch + i], rv, acc[r]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < RPP; ++r) {
+                ys[(part * RPP + r) * pitch + j] = acc[r];
+            }
+        }
+        __syncthreads();
+    }
+
+    if (cp.mode == WEED_HIP_KV_UNIFORM) {
+        const int levels = 1 << cp.bits;
+        const float lo = -3.0f * cp.block_scale;
+        const float hi = 3.0f * cp.block_scale;
+        const float step = (hi - lo) / (float)levels;
+        for (uint32_t e = tid; e < kEncRows * d; e += kEncThreads) {
+            const uint32_t r = e / d, j = e % d;
+            if (row0 + r < rows) {
+                fields[(uint64_t)(row0 + r) * d + j] = (uint8_t)uniform_bucket(ys[r * pitch + j], lo, hi, step, levels);
+            }
+        }
+        return;
+    }
+
+    // LLOYDMAX: row scale from an fma-accumulated sum of squares, j ascending
+    if (tid < kEncRows) {
+        float n2 = 0.0f;
+        for (uint32_t j = 0; j < d; ++j) {
+            const float v = ys[tid * pitch + j];
+            n2 = fmaf(v, v, n2);
+        }
+        const float norm = sqrtf(n2);
+        const float sqrt_d = sqrtf((float)d);
+        float inv = 0.0f, a = 0.0f;
+        if (norm > 1e-30f) {
+            inv = sqrt_d / norm;
+            a = norm / sqrt_d;
+        }
+        inv_s[tid] = inv;
+        if (row0 + tid < rows) {
+            alpha_out[row0 + tid] = a;
+        }
+    }
+    __syncthreads();
+    const int nb = (1 << cp.bits) - 1;
+    for (uint32_t e = tid; e < kEncRows * d; e += kEncThreads) {
+        const uint32_t r = e / d, j = e % d;
+        if (row0 + r >= rows) {
+            continue;
+        }
+        const float u = ys[r * pitch + j] * inv_s[r];
+        int code = 0;
+        for (int k = 0; k < nb; ++k) {
+            code += (u >= cp.bounds[k]) ? 1 : 0;
+        }
+        uint32_t f = (uint32_t)code;
+        if (cp.sign) {
+            f = (f << 1) | ((u >= cp.levels[code]) ? 1u : 0u);
+        }
+        fields[(uint64_t)(row0 + r) * d + j] = (uint8_t)f;
+    }
+}
+
+// One thread per (new row, coordinate group): 32 bytes in, w dwords out.
+__global__ void pack_k_kernel(const uint8_t *__restrict__ fields, const float *__restrict__ alpha_in, uint32_t rows,
+                              uint32_t Hkv, uint32_t T, uint32_t d, uint32_t w, int32_t seq_begin,
+                              const int32_t *__restrict__ lens, uint32_t *__restrict__ out, uint64_t region_dwords,
+                              float *__restrict__ alpha_out, uint32_t padded)
+{
+    const uint32_t groups = d / 32;
+    const uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= rows * groups) {
+        return;
+    }
+    const uint32_t G = idx % groups, row = idx / groups;
+    const uint32_t t = row % T, h = (row / T) % Hkv, s = row / (T * Hkv);
+    const uint32_t n = (uint32_t)lens[seq_begin + s] + t;
+    uint32_t grp[5] = { 0, 0, 0, 0, 0 };
+    const uint8_t *src = fields + (uint64_t)row * d + G * 32;
+    for (uint32_t f = 0; f < 32; ++f) {
+        group_or(grp, f, w, src[f]);
+    }
+    const uint64_t region = (uint64_t)(seq_begin + s) * Hkv + h;
+    uint32_t *dst = out + region * region_dwords + k_group_index(n, G, d, w);
+    for (uint32_t m = 0; m < w; ++m) {
+        dst[m] = grp[m];
+    }
+    if (alpha_out && G == 0) {
+        alpha_out[region * padded + n] = alpha_in[row];
+    }
+}
+
+// One thread per (sequence, kv head, 32-token half block, coordinate): merges the new tokens' fields into the group.
+__global__ void pack_v_kernel(const uint8_t *__restrict__ fields, const float *__restrict__ alpha_in, uint32_t S,
+                              uint32_t Hkv, uint32_t T, uint32_t d, uint32_t w, int32_t seq_begin,
+                              const int32_t *__restrict__ lens, uint32_t halves, uint32_t *__restrict__ out,
+                              uint64_t region_dwords, float *__restrict__ alpha_out, uint32_t padded)
+{
+    const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const uint64_t total = (uint64_t)S * Hkv * halves * d;
+    if (idx >= total) {
+        return;
+    }
+    const uint32_t j = (uint32_t)(idx % d);
+    const uint32_t hf = (uint32_t)((idx / d) % halves);
+    const uint32_t h = (uint32_t)((idx / ((uint64_t)d * halves)) % Hkv);
+    const uint32_t s = (uint32_t)(idx / ((uint64_t)d * halves * Hkv));
+    const uint32_t old_len = (uint32_t)lens[seq_begin + s];
+    const uint32_t new_len = old_len + T;
+    const uint32_t half0 = old_len / 32; // first half block touched
+    const uint32_t half = half0 + hf;
+    const uint32_t block = half >> 1, u = half & 1;
+    const uint32_t tok0 = block * 64;
+    // tokens of this half: tiles 2u, 2u+1 -> [tok0 + 32u, tok0 + 32u + 32)
+    if (tok0 + 32 * u >= new_len) {
+        return;
+    }
+    const uint64_t region = (uint64_t)(seq_begin + s) * Hkv + h;
+    const VPos p = v_pos(tok0 + 32 * u, j, d, w);
+    uint32_t *dst = out + region * region_dwords + p.base;
+    uint32_t grp[5] = { 0, 0, 0, 0, 0 };
+    uint32_t keep[5] = { 0, 0, 0, 0, 0 };
+    for (uint32_t f = 0; f < 32; ++f) {
+        const uint32_t n = tok0 + v_field_token(u, f);
+        if (n < old_len) {
+            group_field_mask(keep, f, w);
+        } else if (n < new_len) {
+            const uint32_t row = (s * Hkv + h) * T + (n - old_len);
+            group_or(grp, f, w, fields[(uint64_t)row * d + j]);
+            if (alpha_out && j == 0) {
+                alpha_out[region * padded + n] = alpha_in[row];
+            }
+        }
+    }
+    for (uint32_t m = 0; m < w; ++m) {
+        uint32_t old = 0;
+        if (keep[m]) {
+            old = dst[(uint64_t)m * p.stride] & keep[m];
+        }
+        dst[(uint64_t)m * p.stride] = old | grp[m];
+    }
+}
+
+__device__ __forceinline__ uint32_t load_field(const SideParams &sp, int which, uint64_t region, uint32_t n, uint32_t j,
+                                               uint32_t d)
+{
+    const uint32_t *base = sp.fields + region * sp.region_dwords;
+    uint32_t grp[5];
+    if (which == 0) {
+        const uint32_t *g = base + k_group_index(n, j / 32, d, sp.w);
+        for (uint32_t m = 0; m < sp.w; ++m) {
+            grp[m] = g[m];
+        }
+        return group_get(grp, j % 32, sp.w);
+    }
+    const VPos p = v_pos(n, j, d, sp.w);
+    for (uint32_t m = 0; m < sp.w; ++m) {
+        grp[m] = base[p.base + (uint64_t)m * p.stride];
+    }
+    return group_get(grp, p.field, sp.w);
+}
+
+// mode 0: dense fp32 (read_row, multihead_attention.cpp:64-79: lo + (code + 0.5) * step, two roundings);
+// mode 1: one field per byte (+ row scales).
+__global__ void unpack_kernel(SideParams sp, int which, int kv_mode, uint32_t Hkv, uint32_t d, uint32_t padded,
+                              int32_t seq_begin, uint32_t S, uint32_t tok_begin, uint32_t T, int out_mode,
+                              float *__restrict__ out_f, Geom4 og, uint8_t *__restrict__ out_b,
+                              float *__restrict__ out_scale)
+{
+    const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const uint64_t total = (uint64_t)S * Hkv * T * d;
+    if (idx >= total) {
+        return;
+    }
+    const uint32_t j = (uint32_t)(idx % d);
+    const uint32_t t = (uint32_t)((idx / d) % T);
+    const uint32_t h = (uint32_t)((idx / ((uint64_t)d * T)) % Hkv);
+    const uint32_t s = (uint32_t)(idx / ((uint64_t)d * T * Hkv));
+    const uint64_t region = (uint64_t)(seq_begin + s) * Hkv + h;
+    const uint32_t n = tok_begin + t;
+    const uint32_t f = load_field(sp, which, region, n, j, d);
+    const float a = sp.alpha ? sp.alpha[region * padded + n] : 0.0f;
+    if (out_mode == 1) {
+        out_b[idx] = (uint8_t)f;
+        if (out_scale && j == 0) {
+            out_scale[(uint64_t)(s * Hkv + h) * T + t] = a;
+        }
+        return;
+    }
+    float val;
+    if (kv_mode == WEED_HIP_KV_UNIFORM) {
+        // sp.beta = lo, sp.alpha_const = step
+        val = sp.beta + ((float)f + 0.5f) * sp.alpha_const;
+    } else {
+        val = a * sp.table[f];
+    }
+    const uint64_t o = (uint64_t)og.off + (uint64_t)s * og.s[0] + (uint64_t)h * og.s[1] + (uint64_t)t * og.s[2] +
+                       (uint64_t)j * og.s[3];
+    out_f[o] = val;
+}
+
+// Rows in Weed's word packing: floor(32/bits) codes per int32 (multihead_attention.cpp:43-62).
+__global__ void weed_words_kernel(SideParams sp, int which, uint32_t Hkv, uint32_t d, int32_t seq_begin, uint32_t S,
+                                  uint32_t tok_begin, uint32_t T, uint32_t bits, int32_t *__restrict__ words)
+{
+    const uint32_t vpw = 32 / bits;
+    const uint32_t wpr = (d + vpw - 1) / vpw;
+    const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const uint64_t total = (uint64_t)S * Hkv * T * wpr;
+    if (idx >= total) {
+        return;
+    }
+    const uint32_t wi = (uint32_t)(idx % wpr);
+    const uint32_t t = (uint32_t)((idx / wpr) % T);
+    const uint32_t h = (uint32_t)((idx / ((uint64_t)wpr * T)) % Hkv);
+    const uint32_t s = (uint32_t)(idx / ((uint64_t)wpr * T * Hkv));
+    const uint64_t region = (uint64_t)(seq_begin + s) * Hkv + h;
+    uint32_t word = 0;
+    for (uint32_t k = 0; k < vpw; ++k) {
+        const uint32_t j = wi * vpw + k;
+        if (j < d) {
+            word |= load_field(sp, which, region, tok_begin + t, j, d) << (k * bits);
+        }
+    }
+    words[idx] = (int32_t)word;
+}
+
+// sum of squares: tree reduction (one partial per block, finished on the host in double)
+__global__ void sumsq_kernel(const float *__restrict__ x, Geom4 g, uint32_t n1, uint32_t n2, uint32_t n3, uint64_t total,
+                             double *__restrict__ partials)
+{
+    __shared__ double red[256];
+    double acc = 0.0;
+    for (uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (uint64_t)gridDim.x * blockDim.x) {
+        const uint32_t i3 = (uint32_t)(idx % n3);
+        const uint32_t i2 = (uint32_t)((idx / n3) % n2);
+        const uint32_t i1 = (uint32_t)((idx / ((uint64_t)n3 * n2)) % n1);
+        const uint32_t i0 = (uint32_t)(idx / ((uint64_t)n3 * n2 * n1));
+        const float v = x[(uint64_t)g.off + (uint64_t)i0 * g.s[0] + (uint64_t)i1 * g.s[1] + (uint64_t)i2 * g.s[2] +
+                          (uint64_t)i3 * g.s[3]];
+        acc += (double)v * (double)v;
+    }
+    red[threadIdx.x] = acc;
+    __syncthreads();
+    for (uint32_t s = blockDim.x / 2; s > 0; s >>= 1) {
+        if (threadIdx.x < s) {
+            red[threadIdx.x] += red[threadIdx.x + s];
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        partials[blockIdx.x] = red[0];
+    }
+}
+
+// The reference's order: one fp32 accumulator, storage order (multihead_attention.cpp:229-240).
+__global__ void sumsq_sequential_kernel(const float *__restrict__ x, uint64_t n, float *__restrict__ out)
+{
+    if (blockIdx.x || threadIdx.x) {
+        return;
+    }
+    float sum = 0.0f;
+    for (uint64_t i = 0; i < n; ++i) {
+        const float v = x[i];
+        sum = sum + v * v;
+    }
+    out[0] = sum;
+}
+
+int check_cache(const weed_hip_kv_cache *c, const char *fn)
+{
+    if (!c) {
+        return fail(WEED_HIP_EINVAL, "%s: null cache", fn);
+    }
+    return WEED_HIP_OK;
+}
+
+int check_range(const weed_hip_kv_cache *c, const char *fn, int32_t seq_begin, int32_t seq_count)
+{
+    if (seq_begin < 0 || seq_count < 0 || seq_begin + seq_count > c->cfg.n_seq) {
+        return fail(WEED_HIP_EINVAL, "%s: sequences [%d, %d) outside [0, %d)", fn, seq_begin, seq_begin + seq_count,
+                    c->cfg.n_seq);
+    }
+    return WEED_HIP_OK;
+}
+
+void free_side(Side &s)
+{
+    (void)hipFree(s.fields);
+    (void)hipFree(s.alpha);
+    (void)hipFree(s.rot);
+    (void)hipFree(s.rot_t);
+    s.fields = nullptr;
+    s.alpha = nullptr;
+    s.rot = nullptr;
+    s.rot_t = nullptr;
+}
+
+int encode_side(weed_hip_kv_cache *c, Side &side, int which, int32_t seq_begin, int32_t seq_count, int32_t T_new,
+                const float *x, uint32_t off, const uint32_t stride[4], int rotate)
+{
+    const uint32_t d = (uint32_t)c->cfg.head_dim;
+    const uint32_t Hkv = (uint32_t)c->cfg.n_kv_heads;
+    const uint32_t rows = (uint32_t)seq_count * Hkv * (uint32_t)T_new;
+    Geom4 g;
+    g.off = off;
+    for (int i = 0; i < 4; ++i) {
+        g.s[i] = stride[i];
+    }
+    CoderParams cp;
+    cp.mode = c->cfg.mode;
+    cp.bits = side.bits;
+    cp.sign = side.sign;
+    cp.block_scale = side.block_scale;
+    std::memcpy(cp.bounds, side.bounds, sizeof(cp.bounds));
+    std::memcpy(cp.levels, side.levels, sizeof(cp.levels));
+    const size_t smem = sizeof(float) * (2 * kEncRows * (d + 1) + kEncRows);
+    const uint32_t blocks = (rows + kEncRows - 1) / kEncRows;
+    int parts = 1;
+    while (parts * 2 * d <= (uint32_t)kEncThreads && parts < 8) {
+        parts *= 2;
+    }
+    if (smem > 48 * 1024) {
+        // more than the default dynamic LDS limit (head_dim 256): opt in per kernel instance
+        const void *fns[4] = { (const void *)encode_rows_kernel<1>, (const void *)encode_rows_kernel<2>,
+                               (const void *)encode_rows_kernel<4>, (const void *)encode_rows_kernel<8> };
+        for (const void *fn : fns) {
+            WEED_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        }
+    }
+    {
+        ProfileScope prof("kv_encode");
+        switch (parts) {
+        case 8:
+            encode_rows_kernel<8><<<blocks, kEncThreads, smem, stream()>>>(x, g, Hkv, (uint32_t)T_new, d, rows,
+                                                                           side.rot_t, rotate, cp, c->enc_fields,
+                                                                           c->enc_alpha);
+            break;
+        case 4:
+            encode_rows_kernel<4><<<blocks, kEncThreads, smem, stream()>>>(x, g, Hkv, (uint32_t)T_new, d, rows,
+                                                                           side.rot_t, rotate, cp, c->enc_fields,
+                                                                           c->enc_alpha);
+            break;
+        case 2:
+            encode_rows_kernel<2><<<blocks, kEncThreads, smem, stream()>>>(x, g, Hkv, (uint32_t)T_new, d, rows,
+                                                                           side.rot_t, rotate, cp, c->enc_fields,
+                                                                           c->enc_alpha);
+            break;
+        default:
+            encode_rows_kernel<1><<<blocks, kEncThreads, smem, stream()>>>(x, g, Hkv, (uint32_t)T_new, d, rows,
+                                                                           side.rot_t, rotate, cp, c->enc_fields,
+                                                                           c->enc_alpha);
+            break;
+        }
+        WEED_HIP_LAUNCH_CHECK();
+    }
+    ProfileScope prof("kv_pack");
+    float *alpha_out = (c->cfg.mode == WEED_HIP_KV_LLOYDMAX) ? side.alpha : nullptr;
+    if (which == 0) {
+        const uint32_t n = rows * (d / 32);
+        pack_k_kernel<<<(n + 255) / 256, 256, 0, stream()>>>(c->enc_fields, c->enc_alpha, rows, Hkv, (uint32_t)T_new, d,
+                                                             side.w, seq_begin, c->lens_dev, side.fields,
+                                                             side.region_dwords, alpha_out, c->padded_tokens);
+    } else {
+        // a run of T_new tokens starting anywhere touches at most (T_new + 30) / 32 + 1 half blocks
+        const uint32_t halves = ((uint32_t)T_new + 30) / 32 + 1;
+        const uint64_t n = (uint64_t)seq_count * Hkv * halves * d;
+        pack_v_kernel<<<(uint32_t)((n + 255) / 256), 256, 0, stream()>>>(
+            c->enc_fields, c->enc_alpha, (uint32_t)seq_count, Hkv, (uint32_t)T_new, d, side.w, seq_begin, c->lens_dev,
+            halves, side.fields, side.region_dwords, alpha_out, c->padded_tokens);
+    }
+    WEED_HIP_LAUNCH_CHECK();
+    return WEED_HIP_OK;
+}
+
+int launch_unpack(const weed_hip_kv_cache *c, int which, int32_t seq_begin, int32_t seq_count, int32_t tok_begin,
+                  int32_t T, int out_mode, float *out_f, uint32_t o_off, const uint32_t *o_stride, uint8_t *out_b,
+                  float *out_scale, const char *fn)
+{
+    WEED_HIP_TRY(check_cache(c, fn));
+    WEED_HIP_TRY(check_range(c, fn, seq_begin, seq_count));
+    WEED_HIP_REQUIRE(which == 0 || which == 1, "%s: which must be 0 (keys) or 1 (values)", fn);
+    WEED_HIP_REQUIRE(tok_begin >= 0 && T >= 0 && (uint32_t)(tok_begin + T) <= c->padded_tokens,
+                     "%s: tokens [%d, %d) outside the cache (capacity %d)", fn, tok_begin, tok_begin + T,
+                     c->cfg.max_tokens);
+    const uint64_t total = (uint64_t)seq_count * c->cfg.n_kv_heads * T * c->cfg.head_dim;
+    if (!total) {
+        return WEED_HIP_OK;
+    }
+    WEED_HIP_REQUIRE(total < (1ull << 40), "%s: request too large", fn);
+    Geom4 og = { 0, { 0, 0, 0, 0 } };
+    if (out_mode == 0) {
+        WEED_HIP_REQUIRE(out_f && o_stride, "%s: null output", fn);
+        og.off = o_off;
+        for (int i = 0; i < 4; ++i) {
+            og.s[i] = o_stride[i];
+        }
+    } else {
+        WEED_HIP_REQUIRE(out_b, "%s: null output", fn);
+    }
+    const SideParams sp = side_params(c, which);
+    unpack_kernel<<<(uint32_t)((total + 255) / 256), 256, 0, stream()>>>(
+        sp, which, c->cfg.mode, (uint32_t)c->cfg.n_kv_heads, (uint32_t)c->cfg.head_dim, c->padded_tokens, seq_begin,
+        (uint32_t)seq_count, (uint32_t)tok_begin, (uint32_t)T, out_mode, out_f, og, out_b, out_scale);
+    WEED_HIP_LAUNCH_CHECK();
+    return WEED_HIP_OK;
+}
+
+} // namespace
+
+namespace weedhip {
+
+SideParams side_params(const weed_hip_kv_cache *c, int which)
+{
+    const Side &s = which ? c->v : c->k;
+    SideParams sp;
+    sp.fields = s.fields;
+    sp.alpha = (c->cfg.mode == WEED_HIP_KV_LLOYDMAX) ? s.alpha : nullptr;
+    sp.region_dwords = s.region_dwords;
+    sp.w = s.w;
+    if (c->cfg.mode == WEED_HIP_KV_UNIFORM) {
+        // read_row (multihead_attention.cpp:71-78): lo = -3s, hi = 3s, step = (hi - lo) / levels
+        const float lo = -3.0f * s.block_scale;
+        const float hi = 3.0f * s.block_scale;
+        sp.alpha_const = (hi - lo) / (float)(1 << s.bits);
+        sp.beta = lo;
+        for (int i = 0; i < 32; ++i) {
+            sp.table[i] = (float)i + 0.5f;
+        }
+    } else {
+        sp.alpha_const = 0.0f;
+        sp.beta = 0.0f;
+        std::memcpy(sp.table, s.recon, sizeof(sp.table));
+    }
+    return sp;
+}
+
+} // namespace weedhip
+
+extern "C" {
+
+int weed_hip_kv_cache_create(weed_hip_kv_cache **cache, const weed_hip_kv_config *cfg)
+{
+    WEED_HIP_REQUIRE(cache && cfg, "weed_hip_kv_cache_create: null pointer");
+    *cache = nullptr;
+    WEED_HIP_TRY(ensure_init());
+    WEED_HIP_REQUIRE(cfg->mode == WEED_HIP_KV_UNIFORM || cfg->mode == WEED_HIP_KV_LLOYDMAX,
+                     "weed_hip_kv_cache_create: unknown mode %d", cfg->mode);
+    WEED_HIP_REQUIRE(cfg->n_seq > 0 && cfg->n_kv_heads > 0 && cfg->max_tokens > 0,
+                     "weed_hip_kv_cache_create: n_seq, n_kv_heads and max_tokens must be positive");
+    WEED_HIP_REQUIRE(cfg->head_dim >= 32 && cfg->head_dim <= 256 && cfg->head_dim % 32 == 0,
+                     "weed_hip_kv_cache_create: head_dim %d must be a multiple of 32 in [32, 256]", cfg->head_dim);
+    WEED_HIP_REQUIRE(cfg->k_bits >= 1 && cfg->k_bits <= 4 && cfg->v_bits >= 1 && cfg->v_bits <= 4,
+                     "weed_hip_kv_cache_create: code widths must be 1..4 bits (got K %d, V %d)", cfg->k_bits,
+                     cfg->v_bits);
+    WEED_HIP_REQUIRE((cfg->k_sign == 0 || cfg->k_sign == 1) && (cfg->v_sign == 0 || cfg->v_sign == 1),
+                     "weed_hip_kv_cache_create: sign flags must be 0 or 1");
+    WEED_HIP_REQUIRE(cfg->mode == WEED_HIP_KV_LLOYDMAX || (!cfg->k_sign && !cfg->v_sign),
+                     "weed_hip_kv_cache_create: the uniform coder keeps no residual sign bit");
+    weed_hip_kv_cache *c = new (std::nothrow) weed_hip_kv_cache();
+    if (!c) {
+        return fail(WEED_HIP_ENOMEM, "weed_hip_kv_cache_create: host allocation failed");
+    }
+    c->cfg = *cfg;
+    c->padded_tokens = padded_tokens((uint32_t)cfg->max_tokens);
+    c->lens.assign((size_t)cfg->n_seq, 0);
+    const uint64_t regions = (uint64_t)cfg->n_seq * cfg->n_kv_heads;
+    Side *sides[2] = { &c->k, &c->v };
+    for (int which = 0; which < 2; ++which) {
+        Side &s = *sides[which];
+        s.bits = which ? cfg->v_bits : cfg->k_bits;
+        s.sign = which ? cfg->v_sign : cfg->k_sign;
+        s.w = (uint32_t)(s.bits + s.sign);
+        s.region_dwords = region_dwords((uint32_t)cfg->max_tokens, (uint32_t)cfg->head_dim, s.w);
+        load_builtin(s);
+        const size_t fbytes = (size_t)(regions * s.region_dwords * sizeof(uint32_t));
+        hipError_t e = hipMalloc((void **)&s.fields, fbytes);
+        if (e == hipSuccess) {
+            e = hipMemsetAsync(s.fields, 0, fbytes, stream());
+        }
+        if (e == hipSuccess && cfg->mode == WEED_HIP_KV_LLOYDMAX) {
+            const size_t abytes = (size_t)(regions * c->padded_tokens * sizeof(float));
+            e = hipMalloc((void **)&s.alpha, abytes);
+            if (e == hipSuccess) {
+                e = hipMemsetAsync(s.alpha, 0, abytes, stream());
+            }
+        }
+        if (e != hipSuccess) {
+            weed_hip_kv_cache_destroy(c);
+            return fail(WEED_HIP_ENOMEM, "weed_hip_kv_cache_create: device allocation failed: %s",
+                        hipGetErrorString(e));
+        }
+    }
+    hipError_t e = hipMalloc((void **)&c->lens_dev, sizeof(int32_t) * (size_t)cfg->n_seq);
+    if (e == hipSuccess) {
+        e = hipMemsetAsync(c->lens_dev, 0, sizeof(int32_t) * (size_t)cfg->n_seq, stream());
+    }
+    if (e != hipSuccess) {
+        weed_hip_kv_cache_destroy(c);
+        return fail(WEED_HIP_ENOMEM, "weed_hip_kv_cache_create: device allocation failed: %s", hipGetErrorString(e));
+    }
+    *cache = c;
+    return WEED_HIP_OK;
+}
+
+int weed_hip_kv_cache_destroy(weed_hip_kv_cache *c)
+{
+    if (!c) {
+        return WEED_HIP_OK;
+    }
+    (void)hipStreamSynchronize(stream());
+    free_side(c->k);
+    free_side(c->v);
+    (void)hipFree(c->lens_dev);
+    (void)hipFree(c->enc_fields);
+    (void)hipFree(c->enc_alpha);
+    (void)hipFree(c->dec_ws);
+    delete c;
+    return WEED_HIP_OK;
+}
+
+int weed_hip_kv_cache_reset(weed_hip_kv_cache *c, int drop_rotations)
+{
+    WEED_HIP_TRY(check_cache(c, "weed_hip_kv_cache_reset"));
+    std::fill(c->lens.begin(), c->lens.end(), 0);
+    const uint32_t n = (uint32_t)c->cfg.n_seq;
+    fill_i32_kernel<<<(n + 255) / 256, 256, 0, stream()>>>(c->lens_dev, 0, n);
+    WEED_HIP_LAUNCH_CHECK();
+    if (drop_rotations) {
+        c->has_rotations = false;
+    }
+    return WEED_HIP_OK;
+}
+
+int weed_hip_kv_cache_row_bytes(const weed_hip_kv_cache *c, uint32_t *k_row_bytes, uint32_t *v_row_bytes)
+{
+    WEED_HIP_TRY(check_cache(c, "weed_hip_kv_cache_row_bytes"));
+    const uint32_t extra = (c->cfg.mode == WEED_HIP_KV_LLOYDMAX) ? 4u : 0u;
+    if (k_row_bytes) {
+        *k_row_bytes = (uint32_t)c->cfg.head_dim * c->k.w / 8 + extra;
+    }
+    if (v_row_bytes) {
+        *v_row_bytes = (uint32_t)c->cfg.head_dim * c->v.w / 8 + extra;
+    }
+    return WEED_HIP_OK;
+}
+
+int weed_hip_kv_cache_seq_lens(const weed_hip_kv_cache *c, int32_t *lens)
+{
+    WEED_HIP_TRY(check_cache(c, "weed_hip_kv_cache_seq_lens"));
+    WEED_HIP_REQUIRE(lens, "weed_hip_kv_cache_seq_lens: null pointer");
+    std::memcpy(lens, c->lens.data(), sizeof(int32_t) * c->lens.size());
+    return WEED_HIP_OK;
+}
+
+int weed_hip_kv_cache_set_rotations(weed_hip_kv_cache *c, const float *rk_dev, const float *rv_dev)
+{
+    WEED_HIP_TRY(check_cache(c, "weed_hip_kv_cache_set_rotations"));
+    WEED_HIP_REQUIRE(rk_dev && rv_dev, "weed_hip_kv_cache_set_rotations: null pointer");
+    const uint32_t d = (uint32_t)c->cfg.head_dim;
+    const size_t bytes = sizeof(float) * d * d;
+    Side *sides[2] = { &c->k, &c->v };
+    const float *src[2] = { rk_dev, rv_dev };
+    for (int which = 0; which < 2; ++which) {
+        Side &s = *sides[which];
+        if (!s.rot) {
+            if (hipMalloc((void **)&s.rot, bytes) != hipSuccess || hipMalloc((void **)&s.rot_t, bytes) != hipSuccess) {
+                return fail(WEED_HIP_ENOMEM, "weed_hip_kv_cache_set_rotations: device allocation failed");
+            }
+        }
+        WEED_HIP_CHECK(hipMemcpyAsync(s.rot, src[which], bytes, hipMemcpyDeviceToDevice, stream()));
+        transpose_square_kernel<<<(d * d + 255) / 256, 256, 0, stream()>>>(s.rot, s.rot_t, d);
+        WEED_HIP_LAUNCH_CHECK();
+    }
+    c->has_rotations = true;
+    return WEED_HIP_OK;
+}
+
+int weed_hip_kv_cache_set_scales(weed_hip_kv_cache *c, float k_scale, float v_scale)
+{
+    WEED_HIP_TRY(check_cache(c, "weed_hip_kv_cache_set_scales"));
+    WEED_HIP_REQUIRE(c->cfg.mode == WEED_HIP_KV_UNIFORM, "weed_hip_kv_cache_set_scales: only the uniform coder has a block scale");
+    c->k.block_scale = k_scale;
+    c->v.block_scale = v_scale;
+    return WEED_HIP_OK;
+}
+
+int weed_hip_kv_cache_get_scales(const weed_hip_kv_cache *c, float *k_scale, float *v_scale)
+{
+    WEED_HIP_TRY(check_cache(c, "weed_hip_kv_cache_get_scales"));
+    if (k_scale) {
+        *k_scale = c->k.block_scale;
+    }
+    if (v_scale) {
+        *v_scale = c->v.block_scale;
+    }
+    return WEED_HIP_OK;
+}
+
+int weed_hip_kv_cache_set_tables(weed_hip_kv_cache *c, int which, const float *bounds, const float *levels,
+                                 const float *recon, float *recon_rounded)
+{
+    WEED_HIP_TRY(check_cache(c, "weed_hip_kv_cache_set_tables"));
+    WEED_HIP_REQUIRE(which == 0 || which == 1, "weed_hip_kv_cache_set_tables: which must be 0 or 1");
+    WEED_HIP_REQUIRE(c->cfg.mode == WEED_HIP_KV_LLOYDMAX, "weed_hip_kv_cache_set_tables: only the Lloyd-Max coder uses tables");
+    WEED_HIP_REQUIRE(bounds && levels && recon, "weed_hip_kv_cache_set_tables: null pointer");
+    Side &s = which ? c->v : c->k;
+    const int n = 1 << s.bits;
+    for (int i = 0; i + 1 < n - 1; ++i) {
+        WEED_HIP_REQUIRE(bounds[i] <= bounds[i + 1], "weed_hip_kv_cache_set_tables: thresholds must ascend");
+    }
+    std::memcpy(s.bounds, bounds, sizeof(float) * (n - 1));
+    std::memcpy(s.levels, levels, sizeof(float) * n);
+    const int nr = n << s.sign;
+    for (int i = 0; i < nr; ++i) {
+        s.recon[i] = round_to_half(recon[i]);
+        if (recon_rounded) {
+            recon_rounded[i] = s.recon[i];
+        }
+    }
+    return WEED_HIP_OK;
+}
+
+int weed_hip_kv_cache_get_tables(const weed_hip_kv_cache *c, int which, float *bounds, float *levels, float *recon)
+{
+    WEED_HIP_TRY(check_cache(c, "weed_hip_kv_cache_get_tables"));
+    WEED_HIP_REQUIRE(which == 0 || which == 1, "weed_hip_kv_cache_get_tables: which must be 0 or 1");
+    const Side &s = which ? c->v : c->k;
+    const int n = 1 << s.bits;
+    if (bounds) {
+        std::memcpy(bounds, s.bounds, sizeof(float) * (n - 1));
+    }
+    if (levels) {
+        std::memcpy(levels, s.levels, sizeof(float) * n);
+    }
+    if (recon) {
+        std::memcpy(recon, s.recon, sizeof(float) * (n << s.sign));
+    }
+    return WEED_HIP_OK;
+}
+
+int weed_hip_block_scale_f32(const float *x_dev, uint32_t off, const uint32_t shape[4], const uint32_t stride[4],
+                             int sequential, float *scale_out)
+{
+    WEED_HIP_REQUIRE(x_dev && shape && stride && scale_out, "weed_hip_block_scale_f32: null pointer");
+    WEED_HIP_TRY(ensure_init());
+    const uint64_t total = (uint64_t)shape[0] * shape[1] * shape[2] * shape[3];
+    WEED_HIP_REQUIRE(total > 0, "weed_hip_block_scale_f32: empty tensor");
+    if (sequential) {
+        // the reference walks the flat buffer of a contiguous tensor, so the storage must be dense
+        uint64_t span = 1;
+        for (int i = 0; i < 4; ++i) {
+            span += (uint64_t)(shape[i] - 1) * stride[i];
+        }
+        WEED_HIP_REQUIRE(span == total, "weed_hip_block_scale_f32: sequential order needs a dense tensor");
+        float *sum_dev = nullptr;
+        if (hipMalloc((void **)&sum_dev, sizeof(float)) != hipSuccess) {
+            return fail(WEED_HIP_ENOMEM, "weed_hip_block_scale_f32: device allocation failed");
+        }
+        sumsq_sequential_kernel<<<1, 64, 0, stream()>>>(x_dev + off, total, sum_dev);
+        float sum = 0.0f;
+        hipError_t e = hipMemcpyAsync(&sum, sum_dev, sizeof(float), hipMemcpyDeviceToHost, stream());
+        if (e == hipSuccess) {
+            e = hipStreamSynchronize(stream());
+        }
+        (void)hipFree(sum_dev);
+        WEED_HIP_CHECK(e);
+        // multihead_attention.cpp:240: sqrt(sum / n + 1e-8) in fp32
+        *scale_out = std::sqrt(sum / (float)(uint32_t)total + 1e-8f);
+        return WEED_HIP_OK;
+    }
+    const uint32_t blocks = 1024;
+    double *partials_dev = nullptr;
+    if (hipMalloc((void **)&partials_dev, sizeof(double) * blocks) != hipSuccess) {
+        return fail(WEED_HIP_ENOMEM, "weed_hip_block_scale_f32: device allocation failed");
+    }
+    Geom4 g;
+    g.off = off;
+    for (int i = 0; i < 4; ++i) {
+        g.s[i] = stride[i];
+    }
+    sumsq_kernel<<<blocks, 256, 0, stream()>>>(x_dev, g, shape[1], shape[2], shape[3], total, partials_dev);
+    std::vector<double> partials(blocks);
+    hipError_t e = hipMemcpyAsync(partials.data(), partials_dev, sizeof(double) * blocks, hipMemcpyDeviceToHost, stream());
+    if (e == hipSuccess) {
+        e = hipStreamSynchronize(stream());
+    }
+    (void)hipFree(partials_dev);
+    WEED_HIP_CHECK(e);
+    double sum = 0.0;
+    for (double p : partials) {
+        sum += p;
+    }
+    *scale_out = (float)std::sqrt(sum / (double)total + 1e-8);
+    return WEED_HIP_OK;
+}
+
+int weed_hip_kv_encode_append(weed_hip_kv_cache *c, int32_t seq_begin, int32_t seq_count, int32_t T_new,
+                              const float *k_dev, uint32_t k_off, const uint32_t k_stride[4], const float *v_dev,
+                              uint32_t v_off, const uint32_t v_stride[4], int rotate)
+{
+    const char *fn = "weed_hip_kv_encode_append";
+    WEED_HIP_TRY(check_cache(c, fn));
+    WEED_HIP_TRY(check_range(c, fn, seq_begin, seq_count));
+    WEED_HIP_REQUIRE(T_new >= 0, "%s: negative token count", fn);
+    WEED_HIP_REQUIRE(rotate >= 0 && rotate <= 2, "%s: rotate must be 0, 1 or 2", fn);
+    if (!seq_count || !T_new) {
+        return WEED_HIP_OK;
+    }
+    WEED_HIP_REQUIRE(k_dev && v_dev && k_stride && v_stride, "%s: null pointer", fn);
+    WEED_HIP_REQUIRE(!rotate || c->has_rotations, "%s: rotation requested but no rotations are set", fn);
+    for (int32_t s = 0; s < seq_count; ++s) {
+        if (c->lens[(size_t)(seq_begin + s)] + T_new > c->cfg.max_tokens) {
+            return fail(WEED_HIP_ECAPACITY, "%s: sequence %d would hold %d tokens, capacity is %d", fn, seq_begin + s,
+                        c->lens[(size_t)(seq_begin + s)] + T_new, c->cfg.max_tokens);
+        }
+    }
+    const uint64_t rows64 = (uint64_t)seq_count * c->cfg.n_kv_heads * T_new;
+    WEED_HIP_REQUIRE(rows64 * c->cfg.head_dim < (1ull << 32), "%s: more than 2^32 elements in one call", fn);
+    const size_t rows = (size_t)rows64;
+    if (rows > c->enc_rows_cap) {
+        WEED_HIP_CHECK(hipStreamSynchronize(stream()));
+        (void)hipFree(c->enc_fields);
+        (void)hipFree(c->enc_alpha);
+        c->enc_fields = nullptr;
+        c->enc_alpha = nullptr;
+        c->enc_rows_cap = 0;
+        if (hipMalloc((void **)&c->enc_fields, rows * c->cfg.head_dim) != hipSuccess ||
+            hipMalloc((void **)&c->enc_alpha, rows * sizeof(float)) != hipSuccess) {
+            return fail(WEED_HIP_ENOMEM, "%s: scratch allocation failed", fn);
+        }
+        c->enc_rows_cap = rows;
+    }
+    WEED_HIP_TRY(encode_side(c, c->k, 0, seq_begin, seq_count, T_new, k_dev, k_off, k_stride, rotate));
+    WEED_HIP_TRY(encode_side(c, c->v, 1, seq_begin, seq_count, T_new, v_dev, v_off, v_stride, rotate));
+    bump_lens_kernel<<<((uint32_t)seq_count + 255) / 256, 256, 0, stream()>>>(c->lens_dev, seq_begin, seq_count, T_new);
+    WEED_HIP_LAUNCH_CHECK();
+    for (int32_t s = 0; s < seq_count; ++s) {
+        c->lens[(size_t)(seq_begin + s)] += T_new;
+    }
+    return WEED_HIP_OK;
+}
+
+int weed_hip_kv_dequant(const weed_hip_kv_cache *c, int which, int32_t seq_begin, int32_t seq_count, int32_t tok_begin,
+                        int32_t T, float *out_dev, uint32_t o_off, const uint32_t o_stride[4])
+{
+    return launch_unpack(c, which, seq_begin, seq_count, tok_begin, T, 0, out_dev, o_off, o_stride, nullptr, nullptr,
+                         "weed_hip_kv_dequant");
+}
+
+int weed_hip_kv_export_fields(const weed_hip_kv_cache *c, int which, int32_t seq_begin, int32_t seq_count,
+                              int32_t tok_begin, int32_t T, uint8_t *fields_dev, float *scales_dev)
+{
+    return launch_unpack(c, which, seq_begin, seq_count, tok_begin, T, 1, nullptr, 0, nullptr, fields_dev, scales_dev,
+                         "weed_hip_kv_export_fields");
+}
+
+int weed_hip_kv_export_weed_words(const weed_hip_kv_cache *c, int which, int32_t seq_begin, int32_t seq_count,
+                                  int32_t tok_begin, int32_t T, int32_t *words_dev)
+{
+    const char *fn = "weed_hip_kv_export_weed_words";
+    WEED_HIP_TRY(check_cache(c, fn));
+    WEED_HIP_TRY(check_range(c, fn, seq_begin, seq_count));
+    WEED_HIP_REQUIRE(which == 0 || which == 1, "%s: which must be 0 (keys) or 1 (values)", fn);
+    WEED_HIP_REQUIRE(c->cfg.mode == WEED_HIP_KV_UNIFORM, "%s: Weed's word packing exists for the uniform coder only", fn);
+    WEED_HIP_REQUIRE(tok_begin >= 0 && T >= 0 && (uint32_t)(tok_begin + T) <= c->padded_tokens,
+                     "%s: tokens [%d, %d) outside the cache", fn, tok_begin, tok_begin + T);
+    WEED_HIP_REQUIRE(words_dev, "%s: null output", fn);
+    const Side &s = which ? c->v : c->k;
+    const uint32_t vpw = 32 / (uint32_t)s.bits;
+    const uint32_t wpr = ((uint32_t)c->cfg.head_dim + vpw - 1) / vpw;
+    const uint64_t total = (uint64_t)seq_count * c->cfg.n_kv_heads * T * wpr;
+    if (!total) {
+        return WEED_HIP_OK;
+    }
+    const SideParams sp = side_params(c, which);
+    weed_words_kernel<<<(uint32_t)((total + 255) / 256), 256, 0, stream()>>>(
+        sp, which, (uint32_t)c->cfg.n_kv_heads, (uint32_t)c->cfg.head_dim, seq_begin, (uint32_t)seq_count,
+        (uint32_t)tok_begin, (uint32_t)T, (uint32_t)s.bits, words_dev);
+    WEED_HIP_LAUNCH_CHECK();
+    return WEED_HIP_OK;
+}
+
+} // extern "C"
