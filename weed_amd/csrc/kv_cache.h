@@ -12,9 +12,10 @@ namespace weedhip {
 // What a kernel needs to turn one tensor's fields back into numbers: value = alpha * table[field] + beta,
 // with alpha the row scale (LLOYDMAX) or the cell width (UNIFORM, where table[c] = c + 0.5 and beta = -3s).
 struct SideParams {
-    const uint32_t *fields; // packed groups, one region per (sequence, kv head)
+    const uint8_t *fields;  // packed items, one region per (sequence, kv head)
     const float *alpha;     // [n_seq][n_kv_heads][padded_tokens] row scales, LLOYDMAX only
-    uint64_t region_dwords;
+    const uint32_t *alpha_max; // [n_seq][n_kv_heads] bit pattern of the largest row scale seen, LLOYDMAX only
+    uint64_t region_bytes;
     uint32_t w;             // field width
     float alpha_const;      // UNIFORM: step
     float beta;             // UNIFORM: lo
@@ -25,9 +26,10 @@ struct Side {
     int bits = 0;
     int sign = 0;
     uint32_t w = 0;
-    uint32_t *fields = nullptr;
+    uint8_t *fields = nullptr;
     float *alpha = nullptr;
-    uint64_t region_dwords = 0;
+    uint32_t *alpha_max = nullptr;
+    uint64_t region_bytes = 0;
     float block_scale = 1.0f; // UNIFORM (Weed: QuantizedKVCache::block_scale)
     float bounds[15] = {};
     float levels[16] = {};

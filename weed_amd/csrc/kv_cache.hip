@@ -255,103 +255,97 @@ __global__ void __launch_bounds__(kEncThreads)
     }
 }
 
-// One thread per (new row, coordinate group): 32 bytes in, w dwords out.
+// One thread per (new row, item of 8 coordinates): 8 bytes in, w bytes out.
 __global__ void pack_k_kernel(const uint8_t *__restrict__ fields, const float *__restrict__ alpha_in, uint32_t rows,
                               uint32_t Hkv, uint32_t T, uint32_t d, uint32_t w, int32_t seq_begin,
-                              const int32_t *__restrict__ lens, uint32_t *__restrict__ out, uint64_t region_dwords,
+                              const int32_t *__restrict__ lens, uint8_t *__restrict__ out, uint64_t region_bytes,
                               float *__restrict__ alpha_out, uint32_t padded)
 {
-    const uint32_t groups = d / 32;
+    const uint32_t items = d / 8;
     const uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= rows * groups) {
+    if (idx >= rows * items) {
         return;
     }
-    const uint32_t G = idx % groups, row = idx / groups;
+    const uint32_t it = idx % items, row = idx / items;
     const uint32_t t = row % T, h = (row / T) % Hkv, s = row / (T * Hkv);
     const uint32_t n = (uint32_t)lens[seq_begin + s] + t;
-    uint32_t grp[5] = { 0, 0, 0, 0, 0 };
-    const uint8_t *src = fields + (uint64_t)row * d + G * 32;
-    for (uint32_t f = 0; f < 32; ++f) {
-        group_or(grp, f, w, src[f]);
-    }
+    uint8_t bytes[5];
+    item_build(fields + (uint64_t)row * d + it * 8, w, bytes);
     const uint64_t region = (uint64_t)(seq_begin + s) * Hkv + h;
-    uint32_t *dst = out + region * region_dwords + k_group_index(n, G, d, w);
-    for (uint32_t m = 0; m < w; ++m) {
-        dst[m] = grp[m];
+    uint8_t *dst = out + region * region_bytes + k_field_pos(n, it * 8, d, w).byte;
+    for (uint32_t b = 0; b < w; ++b) {
+        dst[b] = bytes[b];
     }
-    if (alpha_out && G == 0) {
+    if (alpha_out && it == 0) {
         alpha_out[region * padded + n] = alpha_in[row];
     }
 }
 
-// One thread per (sequence, kv head, 32-token half block, coordinate): merges the new tokens' fields into the group.
+// One thread per (sequence, kv head, 32-token half block, lane group, coordinate): rebuilds one item of 8 tokens,
+// keeping the fields of tokens that were already cached and zeroing those not yet written.
 __global__ void pack_v_kernel(const uint8_t *__restrict__ fields, const float *__restrict__ alpha_in, uint32_t S,
                               uint32_t Hkv, uint32_t T, uint32_t d, uint32_t w, int32_t seq_begin,
-                              const int32_t *__restrict__ lens, uint32_t halves, uint32_t *__restrict__ out,
-                              uint64_t region_dwords, float *__restrict__ alpha_out, uint32_t padded)
+                              const int32_t *__restrict__ lens, uint32_t halves, uint8_t *__restrict__ out,
+                              uint64_t region_bytes, float *__restrict__ alpha_out, uint32_t *__restrict__ alpha_max,
+                              uint32_t padded)
 {
     const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const uint64_t total = (uint64_t)S * Hkv * halves * d;
+    const uint64_t total = (uint64_t)S * Hkv * halves * 4 * d;
     if (idx >= total) {
         return;
     }
     const uint32_t j = (uint32_t)(idx % d);
-    const uint32_t hf = (uint32_t)((idx / d) % halves);
-    const uint32_t h = (uint32_t)((idx / ((uint64_t)d * halves)) % Hkv);
-    const uint32_t s = (uint32_t)(idx / ((uint64_t)d * halves * Hkv));
+    const uint32_t g = (uint32_t)((idx / d) % 4);
+    const uint32_t hf = (uint32_t)((idx / (4ull * d)) % halves);
+    const uint32_t h = (uint32_t)((idx / (4ull * d * halves)) % Hkv);
+    const uint32_t s = (uint32_t)(idx / (4ull * d * halves * Hkv));
     const uint32_t old_len = (uint32_t)lens[seq_begin + s];
     const uint32_t new_len = old_len + T;
-    const uint32_t half0 = old_len / 32; // first half block touched
-    const uint32_t half = half0 + hf;
+    const uint32_t half = old_len / 32 + hf; // halves are 32 consecutive tokens
     const uint32_t block = half >> 1, u = half & 1;
     const uint32_t tok0 = block * 64;
-    // tokens of this half: tiles 2u, 2u+1 -> [tok0 + 32u, tok0 + 32u + 32)
     if (tok0 + 32 * u >= new_len) {
         return;
     }
     const uint64_t region = (uint64_t)(seq_begin + s) * Hkv + h;
-    const VPos p = v_pos(tok0 + 32 * u, j, d, w);
-    uint32_t *dst = out + region * region_dwords + p.base;
-    uint32_t grp[5] = { 0, 0, 0, 0, 0 };
-    uint32_t keep[5] = { 0, 0, 0, 0, 0 };
-    for (uint32_t f = 0; f < 32; ++f) {
-        const uint32_t n = tok0 + v_field_token(u, f);
+    // all 8 tokens of the item share block, u, g and the coordinate, hence the item address
+    const FieldPos p0 = v_field_pos(tok0 + v_item_token(u, g, 0), j, d, w);
+    uint8_t *dst = out + region * region_bytes + p0.byte;
+    uint8_t f8[8];
+    bool touched = false;
+    for (uint32_t e = 0; e < 8; ++e) {
+        const uint32_t n = tok0 + v_item_token(u, g, e);
         if (n < old_len) {
-            group_field_mask(keep, f, w);
+            f8[e] = (uint8_t)item_get(dst, e * w, w);
         } else if (n < new_len) {
             const uint32_t row = (s * Hkv + h) * T + (n - old_len);
-            group_or(grp, f, w, fields[(uint64_t)row * d + j]);
+            f8[e] = fields[(uint64_t)row * d + j];
+            touched = true;
             if (alpha_out && j == 0) {
-                alpha_out[region * padded + n] = alpha_in[row];
+                const float a = alpha_in[row];
+                alpha_out[region * padded + n] = a;
+                atomicMax(alpha_max + region, __float_as_uint(fabsf(a)));
             }
+        } else {
+            f8[e] = 0;
         }
     }
-    for (uint32_t m = 0; m < w; ++m) {
-        uint32_t old = 0;
-        if (keep[m]) {
-            old = dst[(uint64_t)m * p.stride] & keep[m];
-        }
-        dst[(uint64_t)m * p.stride] = old | grp[m];
+    if (!touched) {
+        return;
+    }
+    uint8_t bytes[5];
+    item_build(f8, w, bytes);
+    for (uint32_t b = 0; b < w; ++b) {
+        dst[b] = bytes[b];
     }
 }
 
 __device__ __forceinline__ uint32_t load_field(const SideParams &sp, int which, uint64_t region, uint32_t n, uint32_t j,
                                                uint32_t d)
 {
-    const uint32_t *base = sp.fields + region * sp.region_dwords;
-    uint32_t grp[5];
-    if (which == 0) {
-        const uint32_t *g = base + k_group_index(n, j / 32, d, sp.w);
-        for (uint32_t m = 0; m < sp.w; ++m) {
-            grp[m] = g[m];
-        }
-        return group_get(grp, j % 32, sp.w);
-    }
-    const VPos p = v_pos(n, j, d, sp.w);
-    for (uint32_t m = 0; m < sp.w; ++m) {
-        grp[m] = base[p.base + (uint64_t)m * p.stride];
-    }
-    return group_get(grp, p.field, sp.w);
+    const uint8_t *base = sp.fields + region * sp.region_bytes;
+    const FieldPos p = which ? v_field_pos(n, j, d, sp.w) : k_field_pos(n, j, d, sp.w);
+    return item_get(base + p.byte, p.bit, sp.w);
 }
 
 // mode 0: dense fp32 (read_row, multihead_attention.cpp:64-79: lo + (code + 0.5) * step, two roundings);
@@ -483,10 +477,12 @@ void free_side(Side &s)
 {
     (void)hipFree(s.fields);
     (void)hipFree(s.alpha);
+    (void)hipFree(s.alpha_max);
     (void)hipFree(s.rot);
     (void)hipFree(s.rot_t);
     s.fields = nullptr;
     s.alpha = nullptr;
+    s.alpha_max = nullptr;
     s.rot = nullptr;
     s.rot_t = nullptr;
 }
@@ -552,17 +548,17 @@ int encode_side(weed_hip_kv_cache *c, Side &side, int which, int32_t seq_begin, 
     ProfileScope prof("kv_pack");
     float *alpha_out = (c->cfg.mode == WEED_HIP_KV_LLOYDMAX) ? side.alpha : nullptr;
     if (which == 0) {
-        const uint32_t n = rows * (d / 32);
+        const uint32_t n = rows * (d / 8);
         pack_k_kernel<<<(n + 255) / 256, 256, 0, stream()>>>(c->enc_fields, c->enc_alpha, rows, Hkv, (uint32_t)T_new, d,
                                                              side.w, seq_begin, c->lens_dev, side.fields,
-                                                             side.region_dwords, alpha_out, c->padded_tokens);
+                                                             side.region_bytes, alpha_out, c->padded_tokens);
     } else {
         // a run of T_new tokens starting anywhere touches at most (T_new + 30) / 32 + 1 half blocks
         const uint32_t halves = ((uint32_t)T_new + 30) / 32 + 1;
-        const uint64_t n = (uint64_t)seq_count * Hkv * halves * d;
+        const uint64_t n = (uint64_t)seq_count * Hkv * halves * 4 * d;
         pack_v_kernel<<<(uint32_t)((n + 255) / 256), 256, 0, stream()>>>(
             c->enc_fields, c->enc_alpha, (uint32_t)seq_count, Hkv, (uint32_t)T_new, d, side.w, seq_begin, c->lens_dev,
-            halves, side.fields, side.region_dwords, alpha_out, c->padded_tokens);
+            halves, side.fields, side.region_bytes, alpha_out, side.alpha_max, c->padded_tokens);
     }
     WEED_HIP_LAUNCH_CHECK();
     return WEED_HIP_OK;
@@ -611,7 +607,8 @@ SideParams side_params(const weed_hip_kv_cache *c, int which)
     SideParams sp;
     sp.fields = s.fields;
     sp.alpha = (c->cfg.mode == WEED_HIP_KV_LLOYDMAX) ? s.alpha : nullptr;
-    sp.region_dwords = s.region_dwords;
+    sp.alpha_max = (c->cfg.mode == WEED_HIP_KV_LLOYDMAX) ? s.alpha_max : nullptr;
+    sp.region_bytes = s.region_bytes;
     sp.w = s.w;
     if (c->cfg.mode == WEED_HIP_KV_UNIFORM) {
         // read_row (multihead_attention.cpp:71-78): lo = -3s, hi = 3s, step = (hi - lo) / levels
@@ -666,9 +663,9 @@ int weed_hip_kv_cache_create(weed_hip_kv_cache **cache, const weed_hip_kv_config
         s.bits = which ? cfg->v_bits : cfg->k_bits;
         s.sign = which ? cfg->v_sign : cfg->k_sign;
         s.w = (uint32_t)(s.bits + s.sign);
-        s.region_dwords = region_dwords((uint32_t)cfg->max_tokens, (uint32_t)cfg->head_dim, s.w);
+        s.region_bytes = region_bytes((uint32_t)cfg->max_tokens, (uint32_t)cfg->head_dim, s.w);
         load_builtin(s);
-        const size_t fbytes = (size_t)(regions * s.region_dwords * sizeof(uint32_t));
+        const size_t fbytes = (size_t)(regions * s.region_bytes);
         hipError_t e = hipMalloc((void **)&s.fields, fbytes);
         if (e == hipSuccess) {
             e = hipMemsetAsync(s.fields, 0, fbytes, stream());
@@ -678,6 +675,12 @@ int weed_hip_kv_cache_create(weed_hip_kv_cache **cache, const weed_hip_kv_config
             e = hipMalloc((void **)&s.alpha, abytes);
             if (e == hipSuccess) {
                 e = hipMemsetAsync(s.alpha, 0, abytes, stream());
+            }
+            if (e == hipSuccess) {
+                e = hipMalloc((void **)&s.alpha_max, regions * sizeof(uint32_t));
+            }
+            if (e == hipSuccess) {
+                e = hipMemsetAsync(s.alpha_max, 0, regions * sizeof(uint32_t), stream());
             }
         }
         if (e != hipSuccess) {
@@ -721,6 +724,12 @@ int weed_hip_kv_cache_reset(weed_hip_kv_cache *c, int drop_rotations)
     const uint32_t n = (uint32_t)c->cfg.n_seq;
     fill_i32_kernel<<<(n + 255) / 256, 256, 0, stream()>>>(c->lens_dev, 0, n);
     WEED_HIP_LAUNCH_CHECK();
+    if (c->v.alpha_max) {
+        const uint32_t regions = n * (uint32_t)c->cfg.n_kv_heads;
+        fill_i32_kernel<<<(regions + 255) / 256, 256, 0, stream()>>>((int32_t *)c->k.alpha_max, 0, regions);
+        fill_i32_kernel<<<(regions + 255) / 256, 256, 0, stream()>>>((int32_t *)c->v.alpha_max, 0, regions);
+        WEED_HIP_LAUNCH_CHECK();
+    }
     if (drop_rotations) {
         c->has_rotations = false;
     }

@@ -148,18 +148,14 @@ __global__ void __launch_bounds__(kThreads) decode_generic_kernel(DecodeParams p
                 acc[h] = 0.0f;
             }
             if (n < n1) {
-                const uint32_t *kbase = p.k.fields + region * p.k.region_dwords;
-                for (uint32_t G = 0; G < d / 32; ++G) {
-                    const uint32_t *gp = kbase + k_group_index(n, G, d, p.k.w);
-                    uint32_t grp[5];
-                    for (uint32_t m = 0; m < p.k.w; ++m) {
-                        grp[m] = gp[m];
-                    }
-                    for (uint32_t f = 0; f < 32; ++f) {
-                        const float kv = ktab[group_get(grp, f, p.k.w)];
+                const uint8_t *kbase = p.k.fields + region * p.k.region_bytes;
+                for (uint32_t j0 = 0; j0 < d; j0 += 8) {
+                    const uint8_t *item = kbase + k_field_pos(n, j0, d, p.k.w).byte;
+                    for (uint32_t e = 0; e < 8; ++e) {
+                        const float kv = ktab[item_get(item, e * p.k.w, p.k.w)];
 #pragma unroll
                         for (int h = 0; h < kGMax; ++h) {
-                            acc[h] = fmaf(q_s[h * 256 + G * 32 + f], kv, acc[h]);
+                            acc[h] = fmaf(q_s[h * 256 + j0 + e], kv, acc[h]);
                         }
                     }
                 }
@@ -214,16 +210,12 @@ __global__ void __launch_bounds__(kThreads) decode_generic_kernel(DecodeParams p
                     }
                 }
                 const uint32_t cnt = min((uint32_t)kChunk, n1 - c0);
-                const uint32_t *vbase = p.v.fields + region * p.v.region_dwords;
+                const uint8_t *vbase = p.v.fields + region * p.v.region_bytes;
                 for (uint32_t nl = part; nl < cnt; nl += parts) {
                     const uint32_t nn = c0 + nl;
-                    const VPos vp = v_pos(nn, jj, d, p.v.w);
-                    uint32_t grp[5];
-                    for (uint32_t m = 0; m < p.v.w; ++m) {
-                        grp[m] = vbase[vp.base + (uint64_t)m * vp.stride];
-                    }
+                    const FieldPos vp = v_field_pos(nn, jj, d, p.v.w);
                     const float a = p.v.alpha ? p.v.alpha[region * p.padded + nn] : p.v.alpha_const;
-                    const float vv = fmaf(a, vtab[group_get(grp, vp.field, p.v.w)], p.v.beta);
+                    const float vv = fmaf(a, vtab[item_get(vbase + vp.byte, vp.bit, p.v.w)], p.v.beta);
 #pragma unroll
                     for (int h = 0; h < kGMax; ++h) {
                         if ((uint32_t)h < gh) {
