@@ -9,6 +9,7 @@
 // un-normalised partial (running max m, running sum l, o[d]) per query head; (3) merge the partials of all splits,
 // normalise and un-rotate.
 #include "kv_cache.h"
+#include "kv_decode_mfma.h"
 
 #include <algorithm>
 #include <cmath>
@@ -45,29 +46,60 @@ __device__ __forceinline__ uint32_t q_head_of(const DecodeParams &p, uint32_t kv
 }
 
 // q_rot[s][h][:] = q[s][h][:] . Rk  (multihead_attention.cpp:276), or a plain gather when rotate == 0.
-__global__ void rotate_q_kernel(const float *__restrict__ q, Geom3 g, uint32_t Hq, uint32_t d,
-                                const float *__restrict__ rot_t, int rotate, float *__restrict__ q_rot)
+// For the matrix-core kernel the rotated query is also scaled by log2(e)/sqrt(d), divided by a power of two that
+// brings it into [-1, 1], and split into fp16 hi + lo halves.
+__global__ void __launch_bounds__(256) prep_q_kernel(const float *__restrict__ q, Geom3 g, uint32_t Hq, uint32_t d,
+                                                     const float *__restrict__ rot_t, int rotate,
+                                                     float *__restrict__ q_rot, uint16_t *__restrict__ q_hi,
+                                                     uint16_t *__restrict__ q_lo, float *__restrict__ q_scale,
+                                                     float *__restrict__ q_sum)
 {
     __shared__ float qs[256];
+    __shared__ float red_max[256];
+    __shared__ float red_sum[256];
     const uint32_t h = blockIdx.x, s = blockIdx.y;
     const uint32_t tid = threadIdx.x;
     if (tid < d) {
         qs[tid] = q[(uint64_t)g.off + (uint64_t)s * g.s[0] + (uint64_t)h * g.s[1] + (uint64_t)tid * g.s[2]];
     }
     __syncthreads();
-    if (tid >= d) {
-        return;
-    }
-    float acc;
-    if (rotate) {
-        acc = 0.0f;
-        for (uint32_t i = 0; i < d; ++i) {
-            acc = fmaf(qs[i], rot_t[tid + d * i], acc);
+    float acc = 0.0f;
+    if (tid < d) {
+        if (rotate) {
+            for (uint32_t i = 0; i < d; ++i) {
+                acc = fmaf(qs[i], rot_t[tid + d * i], acc);
+            }
+        } else {
+            acc = qs[tid];
         }
-    } else {
-        acc = qs[tid];
+        q_rot[((uint64_t)s * Hq + h) * d + tid] = acc;
     }
-    q_rot[((uint64_t)s * Hq + h) * d + tid] = acc;
+    const float qc = acc * (1.4426950408889634f / sqrtf((float)d));
+    red_max[tid] = fabsf(qc);
+    red_sum[tid] = qc;
+    __syncthreads();
+    for (uint32_t k = 128; k > 0; k >>= 1) {
+        if (tid < k) {
+            red_max[tid] = fmaxf(red_max[tid], red_max[tid + k]);
+            red_sum[tid] += red_sum[tid + k];
+        }
+        __syncthreads();
+    }
+    int e = 0;
+    (void)frexpf(red_max[0], &e); // max = f * 2^e with f in [0.5, 1), so 2^e exceeds every |qc|
+    e = e < -100 ? -100 : (e > 100 ? 100 : e);
+    const float inv = ldexpf(1.0f, -e);
+    if (tid < d) {
+        const float qn = qc * inv;
+        const _Float16 hi = (_Float16)qn;
+        const _Float16 lo = (_Float16)(qn - (float)hi);
+        q_hi[((uint64_t)s * Hq + h) * d + tid] = __builtin_bit_cast(uint16_t, hi);
+        q_lo[((uint64_t)s * Hq + h) * d + tid] = __builtin_bit_cast(uint16_t, lo);
+    }
+    if (tid == 0) {
+        q_scale[(uint64_t)s * Hq + h] = ldexpf(1.0f, e);
+        q_sum[(uint64_t)s * Hq + h] = red_sum[0];
+    }
 }
 
 __device__ __forceinline__ float wave_max(float v)
@@ -255,7 +287,8 @@ __global__ void __launch_bounds__(kThreads) decode_generic_kernel(DecodeParams p
 // Merge the partials of all splits: out = sum_s e^(m_s - M) o_s / sum_s e^(m_s - M) l_s, then multiply by
 // v_rotation^T (multihead_attention.cpp:343-348): out_i = sum_j O_j Rv[i + d*j].
 __global__ void combine_kernel(const float *__restrict__ partials, uint32_t Hq, uint32_t d, uint32_t n_splits,
-                               const float *__restrict__ rv, int unrotate, float *__restrict__ out, Geom3 og)
+                               const float *__restrict__ rv, int unrotate, int log2_domain, float *__restrict__ out,
+                               Geom3 og)
 {
     __shared__ float w_s[1024];
     __shared__ float o_sh[256];
@@ -272,7 +305,7 @@ __global__ void combine_kernel(const float *__restrict__ partials, uint32_t Hq, 
         float sum = 0.0f;
         for (uint32_t k = tid; k < n_splits; k += 64) {
             const float m = base[(uint64_t)k * (d + 2)];
-            const float w = (m == -INFINITY) ? 0.0f : expf(m - mx);
+            const float w = (m == -INFINITY) ? 0.0f : (log2_domain ? exp2f(m - mx) : expf(m - mx));
             w_s[k] = w;
             sum = fmaf(w, base[(uint64_t)k * (d + 2) + 1], sum);
         }
@@ -331,18 +364,34 @@ extern "C" int weed_hip_kv_decode_attn(weed_hip_kv_cache *c, int32_t n_q_heads, 
     for (int32_t l : c->lens) {
         max_len = std::max(max_len, (uint32_t)l);
     }
-    // split the context so that the launch has a few workgroups per compute unit
-    const uint32_t target_wgs = 2048;
-    uint32_t want = std::max(1u, target_wgs / (S * Hkv));
-    uint32_t n_splits = std::max(1u, std::min((max_len + kChunk - 1) / kChunk, want));
-    uint32_t split_tokens = (max_len + n_splits - 1) / n_splits;
-    split_tokens = std::max((uint32_t)kChunk, (split_tokens + kChunk - 1) / kChunk * kChunk);
-    n_splits = std::max(1u, (max_len + split_tokens - 1) / split_tokens);
+    const uint32_t G = Hq / Hkv;
+    const bool use_mfma = mfma_decode_supported(d, c->k.w, c->v.w, G);
+    uint32_t n_splits, split_tokens = 0, blocks_per_split = 0;
+    if (use_mfma) {
+        // a workgroup's four wavefronts interleave over its 64-token blocks; aim for ~6 workgroups per compute unit
+        const uint32_t nblk = std::max(1u, (max_len + 63) / 64);
+        const uint32_t want = std::max(1u, (1536u + S * Hkv - 1) / (S * Hkv));
+        blocks_per_split = std::max(4u, (nblk + want - 1) / want);
+        blocks_per_split = (blocks_per_split + 3) / 4 * 4;
+        n_splits = (nblk + blocks_per_split - 1) / blocks_per_split;
+    } else {
+        // split the context so that the launch has a few workgroups per compute unit
+        const uint32_t target_wgs = 2048;
+        uint32_t want = std::max(1u, target_wgs / (S * Hkv));
+        n_splits = std::max(1u, std::min((max_len + kChunk - 1) / kChunk, want));
+        split_tokens = (max_len + n_splits - 1) / n_splits;
+        split_tokens = std::max((uint32_t)kChunk, (split_tokens + kChunk - 1) / kChunk * kChunk);
+        n_splits = std::max(1u, (max_len + split_tokens - 1) / split_tokens);
+    }
     WEED_HIP_REQUIRE(n_splits <= 1024, "%s: internal split count %u too large", fn, n_splits);
 
-    const size_t q_bytes = sizeof(float) * (size_t)S * Hq * d;
+    // workspace: rotated q (fp32), its fp16 hi / lo halves, per-head scale and sum, split partials
+    const size_t n_q = (size_t)S * Hq * d;
+    const size_t q_bytes = sizeof(float) * n_q;
+    const size_t h_bytes = (sizeof(uint16_t) * n_q + 15) / 16 * 16;
+    const size_t s_bytes = (sizeof(float) * (size_t)S * Hq + 15) / 16 * 16;
     const size_t part_bytes = sizeof(float) * (size_t)S * Hq * n_splits * (d + 2);
-    const size_t need = q_bytes + part_bytes;
+    const size_t need = q_bytes + 2 * h_bytes + 2 * s_bytes + part_bytes;
     if (need > c->dec_ws_bytes) {
         WEED_HIP_CHECK(hipStreamSynchronize(stream()));
         (void)hipFree(c->dec_ws);
@@ -353,37 +402,62 @@ extern "C" int weed_hip_kv_decode_attn(weed_hip_kv_cache *c, int32_t n_q_heads, 
         }
         c->dec_ws_bytes = need;
     }
-    float *q_rot = c->dec_ws;
-    float *partials = c->dec_ws + (size_t)S * Hq * d;
+    uint8_t *wsp = reinterpret_cast<uint8_t *>(c->dec_ws);
+    float *q_rot = reinterpret_cast<float *>(wsp);
+    uint16_t *q_hi = reinterpret_cast<uint16_t *>(wsp + q_bytes);
+    uint16_t *q_lo = reinterpret_cast<uint16_t *>(wsp + q_bytes + h_bytes);
+    float *q_scale = reinterpret_cast<float *>(wsp + q_bytes + 2 * h_bytes);
+    float *q_sum = reinterpret_cast<float *>(wsp + q_bytes + 2 * h_bytes + s_bytes);
+    float *partials = reinterpret_cast<float *>(wsp + q_bytes + 2 * h_bytes + 2 * s_bytes);
 
     Geom3 qg = { q_off, { q_stride[0], q_stride[1], q_stride[2] } };
     Geom3 og = { o_off, { o_stride[0], o_stride[1], o_stride[2] } };
-    rotate_q_kernel<<<dim3(Hq, S), 256, 0, stream()>>>(q_dev, qg, Hq, d, c->k.rot_t, rot_q ? 1 : 0, q_rot);
+    prep_q_kernel<<<dim3(Hq, S), 256, 0, stream()>>>(q_dev, qg, Hq, d, c->k.rot_t, rot_q ? 1 : 0, q_rot, q_hi, q_lo,
+                                                     q_scale, q_sum);
     WEED_HIP_LAUNCH_CHECK();
 
-    DecodeParams p;
-    p.k = side_params(c, 0);
-    p.v = side_params(c, 1);
-    p.lens = c->lens_dev;
-    p.padded = c->padded_tokens;
-    p.d = d;
-    p.Hq = Hq;
-    p.Hkv = Hkv;
-    p.G = Hq / Hkv;
-    p.blocked = gqa_mapping == WEED_HIP_GQA_BLOCKED;
-    p.q_rot = q_rot;
-    p.partials = partials;
-    p.n_splits = n_splits;
-    p.split_tokens = split_tokens;
-    {
+    if (use_mfma) {
+        MfmaParams mp;
+        mp.k = side_params(c, 0);
+        mp.v = side_params(c, 1);
+        mp.lens = c->lens_dev;
+        mp.padded = c->padded_tokens;
+        mp.Hq = Hq;
+        mp.Hkv = Hkv;
+        mp.G = G;
+        mp.blocked = gqa_mapping == WEED_HIP_GQA_BLOCKED;
+        mp.q_hi = q_hi;
+        mp.q_lo = q_lo;
+        mp.q_scale = q_scale;
+        mp.q_sum = q_sum;
+        mp.partials = partials;
+        mp.n_splits = n_splits;
+        mp.blocks_per_split = blocks_per_split;
+        ProfileScope prof("kv_decode_attn");
+        WEED_HIP_TRY(launch_mfma_decode(mp, d, S, stream()));
+    } else {
+        DecodeParams p;
+        p.k = side_params(c, 0);
+        p.v = side_params(c, 1);
+        p.lens = c->lens_dev;
+        p.padded = c->padded_tokens;
+        p.d = d;
+        p.Hq = Hq;
+        p.Hkv = Hkv;
+        p.G = G;
+        p.blocked = gqa_mapping == WEED_HIP_GQA_BLOCKED;
+        p.q_rot = q_rot;
+        p.partials = partials;
+        p.n_splits = n_splits;
+        p.split_tokens = split_tokens;
         ProfileScope prof("kv_decode_attn");
         decode_generic_kernel<<<dim3(n_splits, Hkv, S), kThreads, 0, stream()>>>(p);
         WEED_HIP_LAUNCH_CHECK();
     }
     {
         ProfileScope prof("kv_decode_combine");
-        combine_kernel<<<dim3(Hq, S), 256, 0, stream()>>>(partials, Hq, d, n_splits, c->v.rot, unrot ? 1 : 0, out_dev,
-                                                          og);
+        combine_kernel<<<dim3(Hq, S), 256, 0, stream()>>>(partials, Hq, d, n_splits, c->v.rot, unrot ? 1 : 0,
+                                                          use_mfma ? 1 : 0, out_dev, og);
         WEED_HIP_LAUNCH_CHECK();
     }
     return WEED_HIP_OK;
