@@ -9,7 +9,8 @@ _HOST_LIB = os.path.join(_HERE, "lib", "libweed_host.so")
 
 
 def library_path():
-    return _LIB
+    """Path of libweed_hip.so; the environment variable WEED_HIP_LIBRARY overrides the in-tree build."""
+    return os.environ.get("WEED_HIP_LIBRARY", _LIB)
 
 
 def host_library_path():

@@ -1,0 +1,9 @@
+// Instantiates the matrix-core decode kernel for head_dim 128, uniform coder.
+#include "kv_decode_mfma_kernel.h"
+
+namespace weedhip {
+int launch_mfma_decode_d128_uniform(const MfmaParams &p, dim3 grid, hipStream_t s)
+{
+    return weedhip_mfma::launch_d<128, false>(p, grid, s);
+}
+} // namespace weedhip

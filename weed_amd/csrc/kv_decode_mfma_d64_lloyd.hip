@@ -1,0 +1,9 @@
+// Instantiates the matrix-core decode kernel for head_dim 64, Lloyd-Max coder.
+#include "kv_decode_mfma_kernel.h"
+
+namespace weedhip {
+int launch_mfma_decode_d64_lloyd(const MfmaParams &p, dim3 grid, hipStream_t s)
+{
+    return weedhip_mfma::launch_d<64, true>(p, grid, s);
+}
+} // namespace weedhip

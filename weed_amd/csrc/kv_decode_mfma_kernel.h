@@ -1,0 +1,543 @@
+#pragma once
+// Matrix-core decode attention over the packed cache (gfx950).
+//
+// One wavefront owns 64-token blocks of one (sequence, kv head).  Per block it
+//   1. streams its lane-major run of packed K items (coalesced 128-bit loads, every byte of the block read once),
+//   2. turns every pair of fields into two fp16 values with one conflict-free LDS lookup (the pair table is replicated
+//      over the 32 banks) and feeds them as the A operand of v_mfma_f32_16x16x32_f16 against the query, which sits in
+//      registers as fp16 hi + lo halves (products of fp16 values are exact in fp32, so the split keeps ~22 bits),
+//   3. runs an online softmax on the 16 tokens x 16 heads score tiles in registers (base-2 exponentials; 1/sqrt(d) and
+//      log2(e) are folded into the query),
+//   4. splits the probabilities (times the V row scales) into fp16 hi + lo, which are already in A-operand order,
+//      and multiplies them with the looked-up V items: out[head][coordinate] accumulates in 4*(d/16) registers.
+// The four wavefronts of a workgroup share the lookup tables, split the workgroup's blocks between them and merge
+// their partial results in LDS; one un-normalised partial (m, l, o[d]) per query head leaves the workgroup.
+//
+// Table values are exactly representable in fp16 (the Lloyd-Max tables are generated that way; the uniform coder's
+// table is code + 0.5), so de-quantisation itself is exact; the only roundings are those of the fp32 accumulators.
+#include "kv_decode_mfma.h"
+
+#include <type_traits>
+
+using namespace weedhip;
+using namespace weedkv;
+
+namespace weedhip_mfma {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
+
+constexpr int kWaves = 4;
+
+__device__ __forceinline__ uint32_t pack_half2(float a, float b)
+{
+    const _Float16 ha = (_Float16)a, hb = (_Float16)b;
+    return (uint32_t)__builtin_bit_cast(uint16_t, ha) | ((uint32_t)__builtin_bit_cast(uint16_t, hb) << 16);
+}
+
+// N dwords from a pointer aligned to 16 bytes when N % 4 == 0, else to 8 bytes (N is even for every supported shape).
+template <int N> __device__ __forceinline__ void load_dwords(const uint8_t *p, uint32_t (&x)[N])
+{
+    if constexpr (N % 4 == 0) {
+#pragma unroll
+        for (int i = 0; i < N / 4; ++i) {
+            const uint4v v = *reinterpret_cast<const uint4v *>(p + 16 * i);
+            x[4 * i] = v.x;
+            x[4 * i + 1] = v.y;
+            x[4 * i + 2] = v.z;
+            x[4 * i + 3] = v.w;
+        }
+    } else {
+        static_assert(N % 2 == 0, "lane runs are multiples of 8 bytes");
+#pragma unroll
+        for (int i = 0; i < N / 2; ++i) {
+            const uint2v v = *reinterpret_cast<const uint2v *>(p + 8 * i);
+            x[2 * i] = v.x;
+            x[2 * i + 1] = v.y;
+        }
+    }
+}
+
+// Pair `P` (2*W bits at bit 2*W*P of the lane's run) -> byte address of its table entry for this lane:
+// table base + entry * 128 + (lane % 32) * 4.  Two instructions per pair: extract the bit field, then shift-and-add
+// the lane's base
+// (written as inline assembly because the compiler's canonical form of the same expression takes three).
+template <int W, int N, int P> __device__ __forceinline__ uint32_t pair_addr(const uint32_t (&x)[N], uint32_t lane_off)
+{
+    constexpr int bit = 2 * W * P;
+    constexpr int dw = bit >> 5, sh = bit & 31;
+    uint32_t t, a;
+    if constexpr (sh + 2 * W <= 32) {
+        asm("v_bfe_u32 %0, %1, %2, %3" : "=v"(t) : "v"(x[dw]), "n"(sh), "n"(2 * W));
+    } else {
+        // the pair straddles two dwords: funnel-shift it down first
+        uint32_t f;
+        asm("v_alignbit_b32 %0, %1, %2, %3" : "=v"(f) : "v"(x[dw + 1 < N ? dw + 1 : dw]), "v"(x[dw]), "n"(sh));
+        asm("v_bfe_u32 %0, %1, 0, %2" : "=v"(t) : "v"(f), "n"(2 * W));
+    }
+    asm("v_lshl_add_u32 %0, %1, 7, %2" : "=v"(a) : "v"(t), "v"(lane_off));
+    return a;
+}
+
+// Item K (8 fields) of the lane's run -> 8 fp16 values in matrix-operand order.
+typedef const uint32_t __attribute__((address_space(3))) *lds_u32_ptr;
+
+__device__ __forceinline__ uint32_t lds_read(uint32_t byte_addr)
+{
+    return *reinterpret_cast<lds_u32_ptr>((uintptr_t)byte_addr);
+}
+
+// `lane_base` = LDS byte address of the table + (lane % 32) * 4.
+template <int W, int N, int K>
+__device__ __forceinline__ half8 dequant_item(const uint32_t (&x)[N], uint32_t lane_base)
+{
+    uint4v r;
+    r.x = lds_read(pair_addr<W, N, 4 * K>(x, lane_base));
+    r.y = lds_read(pair_addr<W, N, 4 * K + 1>(x, lane_base));
+    r.z = lds_read(pair_addr<W, N, 4 * K + 2>(x, lane_base));
+    r.w = lds_read(pair_addr<W, N, 4 * K + 3>(x, lane_base));
+    return __builtin_bit_cast(half8, r);
+}
+
+// Compile-time loop: f(std::integral_constant<int, I>) for I = 0..N-1.
+template <int I, int N, typename F> __device__ __forceinline__ void static_for(F &&f)
+{
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+__device__ __forceinline__ float4v mfma16(half8 a, half8 b, float4v c)
+{
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+
+// ---- cross-lane helpers.  A wavefront is 4 rows of 16 lanes; DPP moves data inside a row. ----
+template <int CTRL, int BANK_MASK> __device__ __forceinline__ uint32_t dpp_u32(uint32_t old, uint32_t src)
+{
+    return (uint32_t)__builtin_amdgcn_update_dpp((int)old, (int)src, CTRL, 0xf, BANK_MASK, false);
+}
+template <int CTRL, int BANK_MASK> __device__ __forceinline__ float dpp_f32(float old, float src)
+{
+    return __uint_as_float(dpp_u32<CTRL, BANK_MASK>(__float_as_uint(old), __float_as_uint(src)));
+}
+constexpr int kRowShl = 0x100, kRowShr = 0x110, kRowRor = 0x120;
+
+// Combine over the lanes that hold the same head: c % GP equal inside a row, then the 4 rows.
+template <int GP> __device__ __forceinline__ float head_max(float v)
+{
+    if constexpr (GP <= 4) {
+        v = fmaxf(v, dpp_f32<kRowRor + 4, 0xf>(v, v));
+    }
+    if constexpr (GP <= 8) {
+        v = fmaxf(v, dpp_f32<kRowRor + 8, 0xf>(v, v));
+    }
+    v = fmaxf(v, __shfl_xor(v, 16));
+    return fmaxf(v, __shfl_xor(v, 32));
+}
+template <int GP> __device__ __forceinline__ float head_sum(float v)
+{
+    if constexpr (GP <= 4) {
+        v += dpp_f32<kRowRor + 4, 0xf>(v, v);
+    }
+    if constexpr (GP <= 8) {
+        v += dpp_f32<kRowRor + 8, 0xf>(v, v);
+    }
+    v += __shfl_xor(v, 16);
+    return v + __shfl_xor(v, 32);
+}
+
+// Bank mask (4-lane banks of a row) of the lanes [GP*i, GP*i + GP).
+template <int GP, int I> constexpr int bank_mask_of() { return ((1 << (GP / 4)) - 1) << (I * GP / 4); }
+
+// GP = number of query-head columns kept per score tile (the group size rounded up to 4, 8 or 16).  The Q.K^T
+// instruction always produces 16 columns; with GP < 16 the useful columns of 16/GP tiles are merged into one register
+// set before the softmax, so the exponentials and the fp16 splitting run on full registers.
+template <int D, int WK, int WV, int GP, bool LLOYD>
+__global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_kernel(MfmaParams p)
+{
+    constexpr int KS = D / 32;       // Q.K^T k-steps (32 coordinates each); also K items per tile per lane
+    constexpr int JB = D / 16;       // 16-coordinate column blocks of the output
+    constexpr int NK = KS * WK;      // dwords of packed K per lane per block
+    constexpr int NV = D * WV / 32;  // dwords of packed V per lane per block
+    constexpr int TPS = 16 / GP;     // score tiles merged into one register set
+    constexpr int NSETS = 4 / TPS;   // register sets per 64-token block
+    constexpr uint32_t KT = (1u << (2 * WK)) * 32u; // dwords of the replicated K pair table
+    constexpr uint32_t VT = (1u << (2 * WV)) * 32u;
+
+    extern __shared__ uint32_t lds[];
+    uint32_t *ktab = lds;
+    uint32_t *vtab = lds + KT;
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t c = lane & 15, g = lane >> 4;
+    const uint32_t split = blockIdx.x, kvh = blockIdx.y, seq = blockIdx.z;
+    const uint32_t L = (uint32_t)p.lens[seq];
+    const uint32_t nblk = (L + 63) >> 6;
+    const uint32_t b0 = split * p.blocks_per_split;
+    const uint32_t b1 = min(nblk, b0 + p.blocks_per_split);
+    const uint64_t region = (uint64_t)seq * p.Hkv + kvh;
+    constexpr bool lloyd = LLOYD;
+
+    // ---- pair tables: entry e, replica i at dword e*32 + i; a lane always reads replica lane%32 ----
+    for (uint32_t i = tid; i < KT; i += 64 * kWaves) {
+        const uint32_t e = i >> 5;
+        ktab[i] = pack_half2(p.k.table[e & ((1u << WK) - 1u)], p.k.table[e >> WK]);
+    }
+    for (uint32_t i = tid; i < VT; i += 64 * kWaves) {
+        const uint32_t e = i >> 5;
+        vtab[i] = pack_half2(p.v.table[e & ((1u << WV) - 1u)], p.v.table[e >> WV]);
+    }
+    __syncthreads();
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint32_t *)lds;
+    const uint32_t kbase = lds_base + (lane & 31) * 4;
+    const uint32_t vbase = kbase + KT * 4;
+
+    // ---- query operand: column c of B is query head c of this kv head, rows are the lane group's coordinates ----
+    half8 qhi[KS], qlo[KS];
+    {
+        const bool col_ok = c < p.G;
+        const uint32_t qh = col_ok ? (p.blocked ? kvh * p.G + c : c * p.Hkv + kvh) : 0;
+        const uint64_t qbase = ((uint64_t)seq * p.Hq + qh) * D + g * (D / 4);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            uint4v hi = { 0, 0, 0, 0 }, lo = { 0, 0, 0, 0 };
+            if (col_ok) {
+                hi = *reinterpret_cast<const uint4v *>(p.q_hi + qbase + 8 * ks);
+                lo = *reinterpret_cast<const uint4v *>(p.q_lo + qbase + 8 * ks);
+            }
+            qhi[ks] = __builtin_bit_cast(half8, hi);
+            qlo[ks] = __builtin_bit_cast(half8, lo);
+        }
+    }
+    // after merging, this lane works on head c % GP of tile (set * TPS + c / GP)
+    const uint32_t hc = c % GP;
+    const uint32_t tile_in_set = c / GP;
+    const bool head_ok = hc < p.G;
+    const uint32_t qh_c = head_ok ? (p.blocked ? kvh * p.G + hc : hc * p.Hkv + kvh) : 0;
+    const float qscale = head_ok ? p.q_scale[(uint64_t)seq * p.Hq + qh_c] : 0.0f;
+    const float betaq = head_ok ? p.k.beta * p.q_sum[(uint64_t)seq * p.Hq + qh_c] : 0.0f;
+
+    // ---- exponent that keeps probability * V-row-scale inside fp16's normal range ----
+    int ep = 10;
+    if (lloyd) {
+        const uint32_t bits = p.v.alpha_max[region];
+        ep = bits ? 136 - (int)((bits >> 23) & 0xff) : 0;
+        ep = ep > 100 ? 100 : (ep < -100 ? -100 : ep);
+    }
+    const float unscale = __uint_as_float((uint32_t)(127 - ep) << 23); // 2^-ep
+
+    float m_run = -INFINITY; // running maximum of this lane's head (same value in every lane that shares the head)
+    float l_run = 0.0f;      // this lane's share of the running denominator, scaled by 2^ep
+    float4v O[JB];           // lane (c, g), register r: head slot 4g + r, coordinate 16*jb + c
+#pragma unroll
+    for (int jb = 0; jb < JB; ++jb) {
+        O[jb] = float4v{ 0.0f, 0.0f, 0.0f, 0.0f };
+    }
+
+    const uint8_t *kreg = p.k.fields + region * p.k.region_bytes + (uint64_t)lane * (4 * NK);
+    const uint8_t *vreg = p.v.fields + region * p.v.region_bytes + (uint64_t)lane * (4 * NV);
+    const float *ka = lloyd ? p.k.alpha + region * p.padded + 16 * tile_in_set + 4 * g : nullptr;
+    const float *va = lloyd ? p.v.alpha + region * p.padded + 16 * tile_in_set + 4 * g : nullptr;
+
+    // Single register buffers, refilled as soon as their last reader is done: K (and its row scales) right after the
+    // Q.K^T phase of a block, V right after its P.V phase -- so each load has about half a block of work to hide behind
+    // and the other wavefronts of the SIMD cover the rest.
+    uint32_t kraw[NK], vraw[NV];
+    float4v ak[NSETS], av[NSETS];
+
+    auto load_k = [&](uint32_t blk) {
+        load_dwords<NK>(kreg + (uint64_t)blk * (8u * D * WK), kraw);
+#pragma unroll
+        for (int s = 0; s < NSETS; ++s) {
+            if constexpr (lloyd) {
+                ak[s] = *reinterpret_cast<const float4v *>(ka + blk * 64 + 16 * TPS * s);
+            } else {
+                ak[s] = float4v{ p.k.alpha_const, p.k.alpha_const, p.k.alpha_const, p.k.alpha_const };
+            }
+        }
+    };
+    auto load_v = [&](uint32_t blk) {
+        load_dwords<NV>(vreg + (uint64_t)blk * (8u * D * WV), vraw);
+#pragma unroll
+        for (int s = 0; s < NSETS; ++s) {
+            if constexpr (lloyd) {
+                av[s] = *reinterpret_cast<const float4v *>(va + blk * 64 + 16 * TPS * s);
+            } else {
+                av[s] = float4v{ 1.0f, 1.0f, 1.0f, 1.0f };
+            }
+        }
+    };
+
+    auto process_block = [&](uint32_t blk, uint32_t next_blk) {
+        // ---- S[t] = K_tile . q: rows = tokens 16t + (lane%16), contraction over the lane groups' coordinates ----
+        // Lookups run one item ahead of the matrix instructions that consume them.
+        float4v S[4];
+        {
+            half8 cur = dequant_item<WK, NK, 0>(kraw, kbase);
+            static_for<0, 4 * KS>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                constexpr int ks = i / 4, t = i % 4;
+                half8 nxt = cur;
+                if constexpr (i + 1 < 4 * KS) {
+                    nxt = dequant_item<WK, NK, ((i + 1) % 4) * KS + (i + 1) / 4>(kraw, kbase);
+                }
+                if constexpr (ks == 0) {
+                    S[t] = mfma16(cur, qhi[0], float4v{ 0.0f, 0.0f, 0.0f, 0.0f });
+                } else {
+                    S[t] = mfma16(cur, qhi[ks], S[t]);
+                }
+                S[t] = mfma16(cur, qlo[ks], S[t]);
+                cur = nxt;
+            });
+        }
+
+        // ---- merge the useful columns: C[s][r] of lane (c, g) = token 16*(s*TPS + c/GP) + 4g + r, head c % GP ----
+        float C[NSETS][4];
+#pragma unroll
+        for (int s = 0; s < NSETS; ++s) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float v = S[s * TPS][r];
+                if constexpr (TPS >= 2) {
+                    v = dpp_f32<kRowShr + GP, bank_mask_of<GP, 1>()>(v, S[s * TPS + 1][r]);
+                }
+                if constexpr (TPS >= 4) {
+                    v = dpp_f32<kRowShr + 2 * GP, bank_mask_of<GP, 2>()>(v, S[s * TPS + 2][r]);
+                    v = dpp_f32<kRowShr + 3 * GP, bank_mask_of<GP, 3>()>(v, S[s * TPS + 3][r]);
+                }
+                // scores in log2 units
+                C[s][r] = fmaf(v, ak[s][r] * qscale, betaq);
+            }
+        }
+        load_k(next_blk); // the K buffer is free again
+        if (blk * 64 + 64 > L) {
+#pragma unroll
+            for (int s = 0; s < NSETS; ++s) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    if (blk * 64 + 16 * (s * TPS + tile_in_set) + 4 * g + r >= L) {
+                        C[s][r] = -INFINITY;
+                    }
+                }
+            }
+        }
+        float mloc = -INFINITY;
+#pragma unroll
+        for (int s = 0; s < NSETS; ++s) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                mloc = fmaxf(mloc, C[s][r]);
+            }
+        }
+        mloc = head_max<GP>(mloc);
+        const float m_new = fmaxf(m_run, mloc);
+        if (__any(m_new > m_run)) {
+            const float scale = (m_run == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(m_run - m_new);
+            l_run *= scale;
+            // output row 4g + r belongs to head slot 4g + r, whose scale lives in lane 4g + r (row 0)
+            float sr[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                sr[r] = __shfl(scale, (int)(4 * g + r));
+            }
+#pragma unroll
+            for (int jb = 0; jb < JB; ++jb) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    O[jb][r] *= sr[r];
+                }
+            }
+            m_run = m_new;
+        }
+        const float mm = m_run - (float)ep;
+
+        // ---- probabilities (times V row scale, times 2^ep), split into fp16 hi + lo pairs ----
+        uint32_t Phi[NSETS][2], Plo[NSETS][2];
+#pragma unroll
+        for (int s = 0; s < NSETS; ++s) {
+            float pv[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float e = __builtin_amdgcn_exp2f(C[s][r] - mm); // exp2(-inf) = 0 masks the tail
+                l_run += e;
+                pv[r] = e * av[s][r];
+            }
+#pragma unroll
+            for (int h2 = 0; h2 < 2; ++h2) {
+                // hi = top 11 significant bits (exact in fp16), lo = the rest
+                const float a0 = pv[2 * h2], a1 = pv[2 * h2 + 1];
+                const float h0 = __uint_as_float(__float_as_uint(a0) & 0xffffe000u);
+                const float h1 = __uint_as_float(__float_as_uint(a1) & 0xffffe000u);
+                Phi[s][h2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(h0, h1));
+                Plo[s][h2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(a0 - h0, a1 - h1));
+            }
+        }
+
+        // ---- O[head][coordinate] += P . V over the block's two 32-token halves.  The A operand of half u wants,
+        //      in lane (head, g), the tokens 4g..4g+3 of tile 2u (k-slots 0..3) and of tile 2u+1 (k-slots 4..7):
+        //      move each tile's pairs back from the lanes they were merged into. ----
+        half8 phi[2], plo[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            uint32_t ah[4], al[4];
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                const int t = 2 * u + half;
+                const int s = t / TPS;
+#pragma unroll
+                for (int h2 = 0; h2 < 2; ++h2) {
+                    uint32_t xh = Phi[s][h2], xl = Plo[s][h2];
+                    if (t % TPS == 1) {
+                        xh = dpp_u32<kRowShl + (TPS >= 2 ? GP : 1), bank_mask_of<GP, 0>()>(xh, xh);
+                        xl = dpp_u32<kRowShl + (TPS >= 2 ? GP : 1), bank_mask_of<GP, 0>()>(xl, xl);
+                    } else if (t % TPS == 2) {
+                        xh = dpp_u32<kRowShl + (TPS >= 4 ? 2 * GP : 1), bank_mask_of<GP, 0>()>(xh, xh);
+                        xl = dpp_u32<kRowShl + (TPS >= 4 ? 2 * GP : 1), bank_mask_of<GP, 0>()>(xl, xl);
+                    } else if (t % TPS == 3) {
+                        xh = dpp_u32<kRowShl + (TPS >= 4 ? 3 * GP : 1), bank_mask_of<GP, 0>()>(xh, xh);
+                        xl = dpp_u32<kRowShl + (TPS >= 4 ? 3 * GP : 1), bank_mask_of<GP, 0>()>(xl, xl);
+                    }
+                    ah[2 * half + h2] = xh;
+                    al[2 * half + h2] = xl;
+                }
+            }
+            phi[u] = __builtin_bit_cast(half8, uint4v{ ah[0], ah[1], ah[2], ah[3] });
+            plo[u] = __builtin_bit_cast(half8, uint4v{ al[0], al[1], al[2], al[3] });
+        }
+        {
+            half8 cur = dequant_item<WV, NV, 0>(vraw, vbase);
+            static_for<0, 2 * JB>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                constexpr int u = i / JB, jb = i % JB;
+                half8 nxt = cur;
+                if constexpr (i + 1 < 2 * JB) {
+                    nxt = dequant_item<WV, NV, i + 1>(vraw, vbase);
+                }
+                O[jb] = mfma16(phi[u], cur, O[jb]);
+                O[jb] = mfma16(plo[u], cur, O[jb]);
+                cur = nxt;
+            });
+        }
+        load_v(next_blk); // the V buffer is free again
+    };
+
+    // ---- main loop.  The refills are unconditional (the next block index is clamped to the last block of the split)
+    //      so that the loop body has no branch around loads and outstanding loads can be counted exactly. ----
+    {
+        uint32_t blk = b0 + wave;
+        if (blk < b1) {
+            const uint32_t last = b1 - 1;
+            load_k(blk);
+            load_v(blk);
+            for (; blk < b1; blk += kWaves) {
+                process_block(blk, min(blk + kWaves, last));
+            }
+        }
+    }
+
+    // ---- per-wave results -> LDS (the tables are no longer needed), then one merged partial per head ----
+    const float l_head = head_sum<GP>(l_run) * unscale; // every lane of a head now holds its denominator
+    float lrow[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        lrow[r] = __shfl(l_head, (int)(4 * g + r));
+    }
+    __syncthreads();
+    float *ws = reinterpret_cast<float *>(lds); // [wave][head slot 0..15][D + 2]
+    constexpr int PS = D + 2;
+    const float o_mul = unscale * (lloyd ? 1.0f : p.v.alpha_const);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const uint32_t hs = 4 * g + r;
+        if (hs < p.G) {
+            float *dst = ws + ((size_t)wave * 16 + hs) * PS;
+#pragma unroll
+            for (int jb = 0; jb < JB; ++jb) {
+                // uniform coder: value = step * (code + 0.5) + lo, so add lo * sum(p)
+                dst[2 + 16 * jb + c] = fmaf(O[jb][r], o_mul, p.v.beta * lrow[r]);
+            }
+        }
+    }
+    if (g == 0 && c < p.G) {
+        // lane c of row 0 holds head c (c < GP)
+        float *dst = ws + ((size_t)wave * 16 + c) * PS;
+        dst[0] = m_run;
+        dst[1] = l_head;
+    }
+    __syncthreads();
+    for (uint32_t idx = tid; idx < p.G * (uint32_t)PS; idx += 64 * kWaves) {
+        const uint32_t hs = idx / PS, j = idx % PS;
+        float mw[kWaves], mx = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            mw[w] = ws[((size_t)w * 16 + hs) * PS];
+            mx = fmaxf(mx, mw[w]);
+        }
+        float val;
+        if (j == 0) {
+            val = mx;
+        } else {
+            val = 0.0f;
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) {
+                const float f = (mw[w] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(mw[w] - mx);
+                val = fmaf(f, ws[((size_t)w * 16 + hs) * PS + j], val);
+            }
+        }
+        const uint32_t head = p.blocked ? kvh * p.G + hs : hs * p.Hkv + kvh;
+        p.partials[(((uint64_t)seq * p.Hq + head) * p.n_splits + split) * PS + j] = val;
+    }
+}
+
+template <int D, int WK, int WV, int GP, bool LLOYD> int launch_gp(const MfmaParams &p, dim3 grid, hipStream_t s)
+{
+    constexpr size_t tab_bytes = (((size_t)1 << (2 * WK)) + ((size_t)1 << (2 * WV))) * 32 * sizeof(uint32_t);
+    constexpr size_t merge_bytes = (size_t)kWaves * 16 * (D + 2) * sizeof(float);
+    constexpr size_t smem = tab_bytes > merge_bytes ? tab_bytes : merge_bytes;
+    static bool configured = false;
+    if (!configured) {
+        WEED_HIP_CHECK(hipFuncSetAttribute((const void *)decode_mfma_kernel<D, WK, WV, GP, LLOYD>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        configured = true;
+    }
+    decode_mfma_kernel<D, WK, WV, GP, LLOYD><<<grid, 64 * kWaves, smem, s>>>(p);
+    WEED_HIP_LAUNCH_CHECK();
+    return WEED_HIP_OK;
+}
+
+template <int D, int WK, int WV, bool LLOYD> int launch_one(const MfmaParams &p, dim3 grid, hipStream_t s)
+{
+    if (p.G <= 4) {
+        return launch_gp<D, WK, WV, 4, LLOYD>(p, grid, s);
+    }
+    if (p.G <= 8) {
+        return launch_gp<D, WK, WV, 8, LLOYD>(p, grid, s);
+    }
+    return launch_gp<D, WK, WV, 16, LLOYD>(p, grid, s);
+}
+
+template <int D, bool LLOYD> int launch_d(const MfmaParams &p, dim3 grid, hipStream_t s)
+{
+    const uint32_t wk = p.k.w, wv = p.v.w;
+#define WEED_CASE(K, V)                                                                                                \
+    if (wk == K && wv == V) {                                                                                          \
+        return launch_one<D, K, V, LLOYD>(p, grid, s);                                                                        \
+    }
+    WEED_CASE(2, 2)
+    WEED_CASE(2, 3)
+    WEED_CASE(2, 4)
+    WEED_CASE(3, 2)
+    WEED_CASE(3, 3)
+    WEED_CASE(3, 4)
+    WEED_CASE(4, 2)
+    WEED_CASE(4, 3)
+    WEED_CASE(4, 4)
+#undef WEED_CASE
+    return fail(WEED_HIP_EINVAL, "decode_mfma: unsupported field widths %u / %u", wk, wv);
+}
+
+} // namespace weedhip_mfma
