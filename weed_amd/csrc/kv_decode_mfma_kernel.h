@@ -196,11 +196,17 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_kernel(MfmaParams 
     const uint32_t kbase = lds_base + (lane & 31) * 4;
     const uint32_t vbase = kbase + KT * 4;
 
-    // ---- query operand: column c of B is query head c of this kv head, rows are the lane group's coordinates ----
-    half8 qhi[KS], qlo[KS];
+    // ---- query operand.  The score instruction has 16 columns.  With GP <= 8 the fp16 high halves of the GP heads sit
+    //      in columns [0, GP) and the low halves in [GP, 2GP), so ONE instruction per item yields both partial scores
+    //      (they are added with a lane shift afterwards); with GP = 16 the halves take two instructions. ----
+    constexpr bool PACKED = GP <= 8;
+    constexpr int NQ = PACKED ? 1 : 2;
+    half8 qop[NQ][KS];
     {
-        const bool col_ok = c < p.G;
-        const uint32_t qh = col_ok ? (p.blocked ? kvh * p.G + c : c * p.Hkv + kvh) : 0;
+        const uint32_t col_head = PACKED ? c % GP : c;
+        const uint32_t col_part = PACKED ? c / GP : 0; // 0: high half, 1: low half, above: unused column
+        const bool col_ok = col_head < p.G && col_part < 2;
+        const uint32_t qh = col_ok ? (p.blocked ? kvh * p.G + col_head : col_head * p.Hkv + kvh) : 0;
         const uint64_t qbase = ((uint64_t)seq * p.Hq + qh) * D + g * (D / 4);
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
@@ -209,8 +215,12 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_kernel(MfmaParams 
                 hi = *reinterpret_cast<const uint4v *>(p.q_hi + qbase + 8 * ks);
                 lo = *reinterpret_cast<const uint4v *>(p.q_lo + qbase + 8 * ks);
             }
-            qhi[ks] = __builtin_bit_cast(half8, hi);
-            qlo[ks] = __builtin_bit_cast(half8, lo);
+            if constexpr (PACKED) {
+                qop[0][ks] = __builtin_bit_cast(half8, col_part ? lo : hi);
+            } else {
+                qop[0][ks] = __builtin_bit_cast(half8, hi);
+                qop[NQ - 1][ks] = __builtin_bit_cast(half8, lo);
+            }
         }
     }
     // after merging, this lane works on head c % GP of tile (set * TPS + c / GP)
@@ -221,11 +231,14 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_kernel(MfmaParams 
     const float qscale = head_ok ? p.q_scale[(uint64_t)seq * p.Hq + qh_c] : 0.0f;
     const float betaq = head_ok ? p.k.beta * p.q_sum[(uint64_t)seq * p.Hq + qh_c] : 0.0f;
 
-    // ---- exponent that keeps probability * V-row-scale inside fp16's normal range ----
-    int ep = 10;
+    // ---- The running maximum is only raised when a block exceeds it by more than 2^kSlack, so most blocks skip the
+    //      rescaling of the output accumulators; probabilities may therefore reach 2^kSlack.  `ep` is the exponent
+    //      that keeps probability * V-row-scale * 2^ep below 2^15, inside fp16's range. ----
+    constexpr float kSlack = 8.0f;
+    int ep = 7;
     if (lloyd) {
         const uint32_t bits = p.v.alpha_max[region];
-        ep = bits ? 136 - (int)((bits >> 23) & 0xff) : 0;
+        ep = bits ? 133 - (int)((bits >> 23) & 0xff) : 0;
         ep = ep > 100 ? 100 : (ep < -100 ? -100 : ep);
     }
     const float unscale = __uint_as_float((uint32_t)(127 - ep) << 23); // 2^-ep
@@ -274,24 +287,31 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_kernel(MfmaParams 
 
     auto process_block = [&](uint32_t blk, uint32_t next_blk) {
         // ---- S[t] = K_tile . q: rows = tokens 16t + (lane%16), contraction over the lane groups' coordinates ----
-        // Lookups run one item ahead of the matrix instructions that consume them.
+        // Lookups run two items ahead of the matrix instructions that consume them.
         float4v S[4];
         {
-            half8 cur = dequant_item<WK, NK, 0>(kraw, kbase);
-            static_for<0, 4 * KS>([&](auto ic) {
+            constexpr int NI = 4 * KS;
+            half8 a0 = dequant_item<WK, NK, 0>(kraw, kbase);
+            half8 a1 = dequant_item<WK, NK, (1 % 4) * KS + 1 / 4>(kraw, kbase);
+            static_for<0, NI>([&](auto ic) {
                 constexpr int i = decltype(ic)::value;
                 constexpr int ks = i / 4, t = i % 4;
-                half8 nxt = cur;
-                if constexpr (i + 1 < 4 * KS) {
-                    nxt = dequant_item<WK, NK, ((i + 1) % 4) * KS + (i + 1) / 4>(kraw, kbase);
+                half8 a2 = a1;
+                if constexpr (i + 2 < NI) {
+                    a2 = dequant_item<WK, NK, ((i + 2) % 4) * KS + (i + 2) / 4>(kraw, kbase);
                 }
+                // keep the look-ahead lookups ahead of this item's matrix instruction
+                __builtin_amdgcn_sched_barrier(0);
                 if constexpr (ks == 0) {
-                    S[t] = mfma16(cur, qhi[0], float4v{ 0.0f, 0.0f, 0.0f, 0.0f });
+                    S[t] = mfma16(a0, qop[0][0], float4v{ 0.0f, 0.0f, 0.0f, 0.0f });
                 } else {
-                    S[t] = mfma16(cur, qhi[ks], S[t]);
+                    S[t] = mfma16(a0, qop[0][ks], S[t]);
                 }
-                S[t] = mfma16(cur, qlo[ks], S[t]);
-                cur = nxt;
+                if constexpr (!PACKED) {
+                    S[t] = mfma16(a0, qop[NQ - 1][ks], S[t]);
+                }
+                a0 = a1;
+                a1 = a2;
             });
         }
 
@@ -301,13 +321,22 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_kernel(MfmaParams 
         for (int s = 0; s < NSETS; ++s) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                float v = S[s * TPS][r];
+                // columns [0, GP) += columns [GP, 2GP): high-half score + low-half score
+                float part[TPS];
+#pragma unroll
+                for (int i = 0; i < TPS; ++i) {
+                    part[i] = S[s * TPS + i][r];
+                    if constexpr (PACKED) {
+                        part[i] += dpp_f32<kRowShl + (PACKED ? GP : 1), 0xf>(part[i], part[i]);
+                    }
+                }
+                float v = part[0];
                 if constexpr (TPS >= 2) {
-                    v = dpp_f32<kRowShr + GP, bank_mask_of<GP, 1>()>(v, S[s * TPS + 1][r]);
+                    v = dpp_f32<kRowShr + GP, bank_mask_of<GP, 1>()>(v, part[TPS >= 2 ? 1 : 0]);
                 }
                 if constexpr (TPS >= 4) {
-                    v = dpp_f32<kRowShr + 2 * GP, bank_mask_of<GP, 2>()>(v, S[s * TPS + 2][r]);
-                    v = dpp_f32<kRowShr + 3 * GP, bank_mask_of<GP, 3>()>(v, S[s * TPS + 3][r]);
+                    v = dpp_f32<kRowShr + 2 * GP, bank_mask_of<GP, 2>()>(v, part[TPS >= 4 ? 2 : 0]);
+                    v = dpp_f32<kRowShr + 3 * GP, bank_mask_of<GP, 3>()>(v, part[TPS >= 4 ? 3 : 0]);
                 }
                 // scores in log2 units
                 C[s][r] = fmaf(v, ak[s][r] * qscale, betaq);
@@ -335,14 +364,15 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_kernel(MfmaParams 
         }
         mloc = head_max<GP>(mloc);
         const float m_new = fmaxf(m_run, mloc);
-        if (__any(m_new > m_run)) {
+        if (__any(mloc > m_run + kSlack)) {
             const float scale = (m_run == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(m_run - m_new);
             l_run *= scale;
-            // output row 4g + r belongs to head slot 4g + r, whose scale lives in lane 4g + r (row 0)
+            // output row 4g + r belongs to head (4g + r) % GP (rows [GP, 2GP) hold the low-half products), whose scale
+            // lives in lane (4g + r) % GP of row 0
             float sr[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                sr[r] = __shfl(scale, (int)(4 * g + r));
+                sr[r] = __shfl(scale, (int)((4 * g + r) % GP));
             }
 #pragma unroll
             for (int jb = 0; jb < JB; ++jb) {
@@ -380,7 +410,10 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_kernel(MfmaParams 
         // ---- O[head][coordinate] += P . V over the block's two 32-token halves.  The A operand of half u wants,
         //      in lane (head, g), the tokens 4g..4g+3 of tile 2u (k-slots 0..3) and of tile 2u+1 (k-slots 4..7):
         //      move each tile's pairs back from the lanes they were merged into. ----
-        half8 phi[2], plo[2];
+        // A operand of half u, lane (row, g): rows [0, GP) carry the high halves of the probabilities of head `row`,
+        // rows [GP, 2GP) the low halves (GP <= 8); the tokens are 4g..4g+3 of tile 2u (k-slots 0..3) and of tile
+        // 2u+1 (k-slots 4..7).  Each tile's pairs are moved back from the lanes they were merged into.
+        half8 pa[2][NQ];
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             uint32_t ah[4], al[4];
@@ -388,38 +421,60 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_kernel(MfmaParams 
             for (int half = 0; half < 2; ++half) {
                 const int t = 2 * u + half;
                 const int s = t / TPS;
+                constexpr int kQuadId = 0xe4; // quad_perm [0,1,2,3]: no movement, used for bank-masked copies
 #pragma unroll
                 for (int h2 = 0; h2 < 2; ++h2) {
                     uint32_t xh = Phi[s][h2], xl = Plo[s][h2];
-                    if (t % TPS == 1) {
-                        xh = dpp_u32<kRowShl + (TPS >= 2 ? GP : 1), bank_mask_of<GP, 0>()>(xh, xh);
-                        xl = dpp_u32<kRowShl + (TPS >= 2 ? GP : 1), bank_mask_of<GP, 0>()>(xl, xl);
-                    } else if (t % TPS == 2) {
-                        xh = dpp_u32<kRowShl + (TPS >= 4 ? 2 * GP : 1), bank_mask_of<GP, 0>()>(xh, xh);
-                        xl = dpp_u32<kRowShl + (TPS >= 4 ? 2 * GP : 1), bank_mask_of<GP, 0>()>(xl, xl);
-                    } else if (t % TPS == 3) {
-                        xh = dpp_u32<kRowShl + (TPS >= 4 ? 3 * GP : 1), bank_mask_of<GP, 0>()>(xh, xh);
-                        xl = dpp_u32<kRowShl + (TPS >= 4 ? 3 * GP : 1), bank_mask_of<GP, 0>()>(xl, xl);
+                    const int i = t % TPS; // the tile sits in lanes [GP*i, GP*i + GP)
+                    if constexpr (PACKED) {
+                        // high halves -> lanes [0, GP), low halves -> lanes [GP, 2GP)
+                        uint32_t x = xh;
+                        if (i == 1) {
+                            x = dpp_u32<kRowShl + GP, bank_mask_of<GP, 0>()>(xh, xh);
+                        } else if (i == 2) {
+                            x = dpp_u32<kRowShl + (TPS >= 4 ? 2 * GP : 1), bank_mask_of<GP, 0>()>(xh, xh);
+                        } else if (i == 3) {
+                            x = dpp_u32<kRowShl + (TPS >= 4 ? 3 * GP : 1), bank_mask_of<GP, 0>()>(xh, xh);
+                        }
+                        if (i == 0) {
+                            x = dpp_u32<kRowShr + GP, bank_mask_of<GP, 1>()>(x, xl);
+                        } else if (i == 1) {
+                            x = dpp_u32<kQuadId, bank_mask_of<GP, 1>()>(x, xl);
+                        } else if (i == 2) {
+                            x = dpp_u32<kRowShl + GP, bank_mask_of<GP, 1>()>(x, xl);
+                        } else {
+                            x = dpp_u32<kRowShl + (TPS >= 4 ? 2 * GP : 1), bank_mask_of<GP, 1>()>(x, xl);
+                        }
+                        ah[2 * half + h2] = x;
+                    } else {
+                        ah[2 * half + h2] = xh;
+                        al[2 * half + h2] = xl;
                     }
-                    ah[2 * half + h2] = xh;
-                    al[2 * half + h2] = xl;
                 }
             }
-            phi[u] = __builtin_bit_cast(half8, uint4v{ ah[0], ah[1], ah[2], ah[3] });
-            plo[u] = __builtin_bit_cast(half8, uint4v{ al[0], al[1], al[2], al[3] });
+            pa[u][0] = __builtin_bit_cast(half8, uint4v{ ah[0], ah[1], ah[2], ah[3] });
+            if constexpr (!PACKED) {
+                pa[u][NQ - 1] = __builtin_bit_cast(half8, uint4v{ al[0], al[1], al[2], al[3] });
+            }
         }
         {
-            half8 cur = dequant_item<WV, NV, 0>(vraw, vbase);
-            static_for<0, 2 * JB>([&](auto ic) {
+            constexpr int NI = 2 * JB;
+            half8 b0v = dequant_item<WV, NV, 0>(vraw, vbase);
+            half8 b1v = dequant_item<WV, NV, 1>(vraw, vbase);
+            static_for<0, NI>([&](auto ic) {
                 constexpr int i = decltype(ic)::value;
                 constexpr int u = i / JB, jb = i % JB;
-                half8 nxt = cur;
-                if constexpr (i + 1 < 2 * JB) {
-                    nxt = dequant_item<WV, NV, i + 1>(vraw, vbase);
+                half8 b2v = b1v;
+                if constexpr (i + 2 < NI) {
+                    b2v = dequant_item<WV, NV, i + 2>(vraw, vbase);
                 }
-                O[jb] = mfma16(phi[u], cur, O[jb]);
-                O[jb] = mfma16(plo[u], cur, O[jb]);
-                cur = nxt;
+                __builtin_amdgcn_sched_barrier(0);
+                O[jb] = mfma16(pa[u][0], b0v, O[jb]);
+                if constexpr (!PACKED) {
+                    O[jb] = mfma16(pa[u][NQ - 1], b0v, O[jb]);
+                }
+                b0v = b1v;
+                b1v = b2v;
             });
         }
         load_v(next_blk); // the V buffer is free again
@@ -450,6 +505,16 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_kernel(MfmaParams 
     float *ws = reinterpret_cast<float *>(lds); // [wave][head slot 0..15][D + 2]
     constexpr int PS = D + 2;
     const float o_mul = unscale * (lloyd ? 1.0f : p.v.alpha_const);
+    if constexpr (PACKED) {
+        // rows [GP, 2GP) hold the low-half products of heads [0, GP): they sit GP/4 lane rows further up
+#pragma unroll
+        for (int jb = 0; jb < JB; ++jb) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                O[jb][r] += __shfl_down(O[jb][r], 4 * GP);
+            }
+        }
+    }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const uint32_t hs = 4 * g + r;
