@@ -13,6 +13,7 @@
 
 #include <algorithm>
 #include <cmath>
+#include <cstdlib>
 
 using namespace weedhip;
 using namespace weedkv;
@@ -370,7 +371,11 @@ extern "C" int weed_hip_kv_decode_attn(weed_hip_kv_cache *c, int32_t n_q_heads, 
     if (use_mfma) {
         // a workgroup's four wavefronts interleave over its 64-token blocks; aim for ~6 workgroups per compute unit
         const uint32_t nblk = std::max(1u, (max_len + 63) / 64);
-        const uint32_t want = std::max(1u, (1536u + S * Hkv - 1) / (S * Hkv));
+        uint32_t target_wgs = 1024u;
+        if (const char *env = std::getenv("WEED_HIP_DECODE_WGS")) {
+            target_wgs = (uint32_t)std::max(1, std::atoi(env)); // tuning knob
+        }
+        const uint32_t want = std::max(1u, (target_wgs + S * Hkv - 1) / (S * Hkv));
         blocks_per_split = std::max(4u, (nblk + want - 1) / want);
         blocks_per_split = (blocks_per_split + 3) / 4 * 4;
         n_splits = (nblk + blocks_per_split - 1) / blocks_per_split;

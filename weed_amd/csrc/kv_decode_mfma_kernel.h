@@ -182,14 +182,21 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_kernel(MfmaParams 
     const uint64_t region = (uint64_t)seq * p.Hkv + kvh;
     constexpr bool lloyd = LLOYD;
 
-    // ---- pair tables: entry e, replica i at dword e*32 + i; a lane always reads replica lane%32 ----
+    // ---- pair tables: entry e, replica i at dword e*32 + i; a lane always reads replica lane%32.  The 2^w fp16
+    //      levels are staged in LDS first so that building the pairs needs no global reads. ----
+    __shared__ uint16_t levels_h[2][32];
+    if (tid < 64) {
+        const float lv = (tid < 32) ? p.k.table[tid & 31] : p.v.table[tid & 31];
+        levels_h[tid >> 5][tid & 31] = __builtin_bit_cast(uint16_t, (_Float16)lv);
+    }
+    __syncthreads();
     for (uint32_t i = tid; i < KT; i += 64 * kWaves) {
         const uint32_t e = i >> 5;
-        ktab[i] = pack_half2(p.k.table[e & ((1u << WK) - 1u)], p.k.table[e >> WK]);
+        ktab[i] = (uint32_t)levels_h[0][e & ((1u << WK) - 1u)] | ((uint32_t)levels_h[0][e >> WK] << 16);
     }
     for (uint32_t i = tid; i < VT; i += 64 * kWaves) {
         const uint32_t e = i >> 5;
-        vtab[i] = pack_half2(p.v.table[e & ((1u << WV) - 1u)], p.v.table[e >> WV]);
+        vtab[i] = (uint32_t)levels_h[1][e & ((1u << WV) - 1u)] | ((uint32_t)levels_h[1][e >> WV] << 16);
     }
     __syncthreads();
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint32_t *)lds;
