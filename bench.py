@@ -77,6 +77,84 @@ def cpu_baseline(capi, torch, cache, wl, q, rk, rv, budget_s=12.0):
     return steps / elapsed, steps, elapsed, out
 
 
+def time_calls(torch, fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def extras(capi, torch, workloads, steps, warmup):
+    """The other configurations, measured the same way (reported beside the headline, not as `value`)."""
+    out = {}
+    # configuration 5b: [4096 x 1024] . [1024 x 4096] fp32, column-major operands as Weed passes them
+    A = torch.randn((1024, 4096), device="cuda").t()           # logical [4096, 1024], column-major
+    W = (torch.randn((4096, 1024), device="cuda") * 0.02).t()  # logical [1024, 4096], column-major
+    C = torch.empty((4096, 4096), device="cuda").t()
+    capi.profile_reset()
+    capi.profile_enable(True)
+    secs = time_calls(torch, lambda: capi.matmul(A, W, C), steps, warmup)
+    k_ms, k_n = capi.profile_read("matmul")
+    capi.profile_enable(False)
+    flops = 2.0 * 4096 * 1024 * 4096
+    kernel_s = 1e-3 * k_ms / max(1, k_n)
+    out["cfg5b_matmul_f32_4096x1024x4096"] = {
+        "tflops": flops / secs / 1e12, "kernel_ms": 1e3 * kernel_s, "kernel_tflops": flops / kernel_s / 1e12,
+        "roofline": {"bound": "mfma", "achieved": flops / kernel_s / 1e12, "peak": 157.3, "unit": "TFLOP/s",
+                     "frac": flops / kernel_s / 1e12 / 157.3}}
+    del A, W, C
+    # configuration 5a: encode-and-append 4096 tokens x 8 kv heads x 128, 3-bit codes (rotate, quantise, pack)
+    wl = workloads.config(5)
+    d = wl.head_dim
+    cache = capi.KVCache(capi.KV_LLOYDMAX, 1, wl.n_kv_heads, d, 4096, 3, 3)
+    rk = torch.zeros(d * d, device="cuda")
+    rv = torch.zeros(d * d, device="cuda")
+    capi.make_rotation(5, d, rk)
+    capi.make_rotation(6, d, rv)
+    cache.set_rotations(rk, rv)
+    K = torch.randn((1, wl.n_kv_heads, 4096, d), device="cuda")
+    V = torch.randn((1, wl.n_kv_heads, 4096, d), device="cuda")
+
+    def enc():
+        cache.reset()
+        cache.encode_append(K, V, rotate=1)
+
+    secs = time_calls(torch, enc, steps, warmup)
+    in_bytes = 2 * K.numel() * 4
+    out["cfg5a_encode_4096x8x128_3bit"] = {"tokens_per_s": 4096 / secs, "ms": 1e3 * secs,
+                                           "input_gbs": in_bytes / secs / 1e9,
+                                           "rotation_tflops": 2 * 2.0 * K.numel() * d / secs / 1e12}
+    cache.close()
+    # configuration 4: 16 ragged sequences in [2048, 32768], K 2-bit + sign, V 3-bit, split-context merge
+    wl4 = workloads.config(4)
+    cache4 = capi.KVCache(capi.KV_LLOYDMAX, wl4.n_seq, wl4.n_kv_heads, d, wl4.max_len, wl4.k_bits, wl4.v_bits,
+                          wl4.k_sign, wl4.v_sign)
+    for s, L in enumerate(wl4.lens):
+        Ks = torch.randn((1, wl4.n_kv_heads, L, d), device="cuda")
+        Vs = torch.randn((1, wl4.n_kv_heads, L, d), device="cuda")
+        cache4.encode_append(Ks, Vs, seq_begin=s)
+    for hq in (8, 32):
+        q = torch.randn((wl4.n_seq, hq, d), device="cuda")
+        o = torch.zeros_like(q)
+        capi.profile_reset()
+        capi.profile_enable(True)
+        secs = time_calls(torch, lambda: cache4.decode_attn(q, o, capi.GQA_BLOCKED, 0), steps, warmup)
+        k_ms, k_n = capi.profile_read("kv_decode_attn")
+        capi.profile_enable(False)
+        nbytes = wl4.bytes_per_step(True)
+        kernel_s = 1e-3 * k_ms / max(1, k_n)
+        out["cfg4_ragged16_hq%d" % hq] = {"tokens_per_s": wl4.n_seq / secs, "ms_per_step": 1e3 * secs,
+                                          "packed_cache_bytes": nbytes, "kernel_ms": 1e3 * kernel_s,
+                                          "kernel_gbs": nbytes / kernel_s / 1e9,
+                                          "frac_of_hbm_peak": nbytes / kernel_s / 1e9 / HBM_PEAK_GBS}
+    cache4.close()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -85,6 +163,7 @@ def main():
     ap.add_argument("--seqs", type=int, default=64, help="independent ctx-8192 sequence caches per launch")
     ap.add_argument("--ctx", type=int, default=8192)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true", help="skip the other configurations (4, 5a, 5b)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path is sharded by (sequence, kv head) with no "
@@ -199,6 +278,8 @@ def main():
             }
         cache.close()
         cache1.close()
+        if not args.no_extras:
+            result["other_configs"] = extras(capi, torch, workloads, min(args.steps, 20), min(args.warmup, 3))
     print(json.dumps(result))
 
 

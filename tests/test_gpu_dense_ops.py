@@ -59,6 +59,22 @@ def test_matmul_strided_against_checker(gpu, oracle, M, N, K):
     assert torch.all(big_c[1::2] == -1.0) and torch.all(big_c[:, :3] == -1.0)  # nothing outside the view is written
 
 
+@pytest.mark.parametrize("a_col,b_col,o_col", [(True, True, True), (True, False, False), (False, True, True),
+                                                 (False, False, False), (True, True, False)])
+def test_matmul_matrix_core_layouts(gpu, oracle, a_col, b_col, o_col):
+    """Full 128 x 128 x 16 tiles with every combination of contiguous dimension (the matrix-core kernel's four
+    instances) against the checker's sequential fp32 sums."""
+    M, N, K = 256, 384, 160
+    rng = np.random.default_rng(M + N + K + a_col * 4 + b_col * 2 + o_col)
+    A = rng.standard_normal((M, K), dtype=np.float32)
+    B = rng.standard_normal((K, N), dtype=np.float32)
+    want = np.zeros(M * N, dtype=np.float32)
+    oracle.matmul(M, N, K, A.reshape(-1), (0, K, 1), B.reshape(-1), (0, N, 1), want, (0, N, 1))
+    C = (col_major if o_col else dev)(np.zeros((M, N), dtype=np.float32))
+    gpu.matmul((col_major if a_col else dev)(A), (col_major if b_col else dev)(B), C)
+    np.testing.assert_allclose(C.cpu().numpy(), want.reshape(M, N), rtol=2e-5, atol=2e-5 * np.sqrt(K))
+
+
 def test_matmul_cfg5_sampled(gpu):
     """Configuration 5b at full size ([4096 x 1024] . [1024 x 4096], column-major): the scalar checker would need
     minutes, so 4096 sampled outputs are compared with float64 dot products, plus the column sums identity

@@ -73,6 +73,172 @@ __global__ void __launch_bounds__(256) matmul_tiled_kernel(const float *__restri
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Matrix-core kernel: v_mfma_f32_32x32x2_f32 (fp32 in, fp32 accumulate; products are exact to fp32 rounding).
+//   workgroup = 4 wavefronts, output tile 128 x 128, each wavefront a 64 x 64 quadrant = 2 x 2 instructions tiles;
+//   K is walked in slices of 16 staged through double-buffered LDS ([k][i] and [k][j], so a half-wavefront reads 32
+//   consecutive floats); the next slice is fetched from HBM into registers while the current one is multiplied.
+// Each operand must be contiguous along one of its two dimensions (Weed's column-major tensors and their transposes
+// are); the four combinations are template instances.  Shapes that are not multiples of the tile, and operands
+// strided in both dimensions, use the generic kernel above.
+// ------------------------------------------------------------------------------------------------
+typedef float float16v __attribute__((ext_vector_type(16)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+
+constexpr int TM = 128, TN = 128, TK = 16, PITCH = 132;
+
+template <bool A_ICONTIG, bool B_KCONTIG>
+__global__ void __launch_bounds__(256) matmul_mfma_kernel(const float *__restrict__ a, const float *__restrict__ b,
+                                                          float *__restrict__ out, MatGeom g)
+{
+    __shared__ __attribute__((aligned(16))) float As[2][TK][PITCH];
+    __shared__ __attribute__((aligned(16))) float Bs[2][TK][PITCH];
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t wi = wave >> 1, wj = wave & 1;
+    const uint32_t m0 = blockIdx.x * TM, n0 = blockIdx.y * TN;
+    const uint32_t l32 = lane & 31, lk = lane >> 5;
+
+    float16v acc[2][2];
+#pragma unroll
+    for (int x = 0; x < 2; ++x) {
+#pragma unroll
+        for (int y = 0; y < 2; ++y) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                acc[x][y][r] = 0.0f;
+            }
+        }
+    }
+
+    // two float4 per operand per thread and K slice
+    float4v ra[2], rb[2];
+    auto fetch = [&](uint32_t k0) {
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const uint32_t idx = tid + 256 * q;
+            if (A_ICONTIG) {
+                const uint32_t i4 = idx & 31, k = idx >> 5;
+                ra[q] = *reinterpret_cast<const float4v *>(a + (uint64_t)g.a_off + (m0 + 4 * i4) +
+                                                           (uint64_t)(k0 + k) * g.a_s1);
+            } else {
+                const uint32_t k4 = idx & 3, i = idx >> 2;
+                ra[q] = *reinterpret_cast<const float4v *>(a + (uint64_t)g.a_off + (uint64_t)(m0 + i) * g.a_s0 +
+                                                           (k0 + 4 * k4));
+            }
+            if (B_KCONTIG) {
+                const uint32_t k4 = idx & 3, j = idx >> 2;
+                rb[q] = *reinterpret_cast<const float4v *>(b + (uint64_t)g.b_off + (k0 + 4 * k4) +
+                                                           (uint64_t)(n0 + j) * g.b_s1);
+            } else {
+                const uint32_t j4 = idx & 31, k = idx >> 5;
+                rb[q] = *reinterpret_cast<const float4v *>(b + (uint64_t)g.b_off + (uint64_t)(k0 + k) * g.b_s0 +
+                                                           (n0 + 4 * j4));
+            }
+        }
+    };
+    auto stage = [&](int buf) {
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const uint32_t idx = tid + 256 * q;
+            if (A_ICONTIG) {
+                const uint32_t i4 = idx & 31, k = idx >> 5;
+                *reinterpret_cast<float4v *>(&As[buf][k][4 * i4]) = ra[q];
+            } else {
+                const uint32_t k4 = idx & 3, i = idx >> 2;
+#pragma unroll
+                for (int x = 0; x < 4; ++x) {
+                    As[buf][4 * k4 + x][i] = ra[q][x];
+                }
+            }
+            if (B_KCONTIG) {
+                const uint32_t k4 = idx & 3, j = idx >> 2;
+#pragma unroll
+                for (int x = 0; x < 4; ++x) {
+                    Bs[buf][4 * k4 + x][j] = rb[q][x];
+                }
+            } else {
+                const uint32_t j4 = idx & 31, k = idx >> 5;
+                *reinterpret_cast<float4v *>(&Bs[buf][k][4 * j4]) = rb[q];
+            }
+        }
+    };
+
+    const uint32_t n_slices = g.K / TK;
+    fetch(0);
+    stage(0);
+    __syncthreads();
+    for (uint32_t kt = 0; kt < n_slices; ++kt) {
+        const int buf = kt & 1;
+        if (kt + 1 < n_slices) {
+            fetch((kt + 1) * TK);
+        }
+#pragma unroll
+        for (int kk = 0; kk < TK; kk += 2) {
+            const float a0 = As[buf][kk + lk][64 * wi + l32];
+            const float a1 = As[buf][kk + lk][64 * wi + 32 + l32];
+            const float b0 = Bs[buf][kk + lk][64 * wj + l32];
+            const float b1 = Bs[buf][kk + lk][64 * wj + 32 + l32];
+            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
+            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
+            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
+            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+        }
+        if (kt + 1 < n_slices) {
+            stage(buf ^ 1);
+        }
+        __syncthreads();
+    }
+
+    // register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its 32 x 32 tile
+#pragma unroll
+    for (int x = 0; x < 2; ++x) {
+#pragma unroll
+        for (int y = 0; y < 2; ++y) {
+            const uint32_t col = n0 + 64 * wj + 32 * y + l32;
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                const uint32_t row = m0 + 64 * wi + 32 * x + 8 * r4 + 4 * lk;
+                float *dst = out + (uint64_t)g.o_off + (uint64_t)row * g.o_s0 + (uint64_t)col * g.o_s1;
+                if (g.o_s0 == 1) {
+                    *reinterpret_cast<float4v *>(dst) =
+                        float4v{ acc[x][y][4 * r4], acc[x][y][4 * r4 + 1], acc[x][y][4 * r4 + 2], acc[x][y][4 * r4 + 3] };
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        dst[(uint64_t)e * g.o_s0] = acc[x][y][4 * r4 + e];
+                    }
+                }
+            }
+        }
+    }
+}
+
+bool aligned16(const float *p, uint64_t elem_off) { return (((uintptr_t)p + 4 * elem_off) & 15) == 0; }
+
+// The matrix-core kernel needs full tiles, one contiguous dimension per operand and 16-byte aligned vector accesses.
+bool mfma_eligible(const MatGeom &g, const float *a, const float *b, const float *out)
+{
+    if (g.M % TM || g.N % TN || g.K % TK || !g.K) {
+        return false;
+    }
+    const bool a_i = g.a_s0 == 1, a_k = g.a_s1 == 1;
+    const bool b_k = g.b_s0 == 1, b_j = g.b_s1 == 1;
+    if (!(a_i || a_k) || !(b_k || b_j)) {
+        return false;
+    }
+    // vector loads step along the contiguous dimension in units of 4 floats; the other stride must keep alignment
+    if (!aligned16(a, g.a_off) || ((a_i ? g.a_s1 : g.a_s0) & 3)) {
+        return false;
+    }
+    if (!aligned16(b, g.b_off) || ((b_k ? g.b_s1 : g.b_s0) & 3)) {
+        return false;
+    }
+    if (g.o_s0 == 1 && (!aligned16(out, g.o_off) || (g.o_s1 & 3))) {
+        return false;
+    }
+    return true;
+}
+
 } // namespace
 
 extern "C" int weed_hip_matmul_f32(uint32_t M, uint32_t N, uint32_t K, const float *a_dev, uint32_t a_off,
@@ -86,9 +252,25 @@ extern "C" int weed_hip_matmul_f32(uint32_t M, uint32_t N, uint32_t K, const flo
         return WEED_HIP_OK;
     }
     MatGeom g = { M, N, K, a_off, a_s0, a_s1, b_off, b_s0, b_s1, o_off, o_s0, o_s1 };
+    ProfileScope prof("matmul");
+    if (mfma_eligible(g, a_dev, b_dev, out_dev)) {
+        const dim3 grid(M / TM, N / TN);
+        WEED_HIP_REQUIRE(grid.y <= 65535u, "%s: N = %u too large", fn, N);
+        const bool a_i = a_s0 == 1, b_k = b_s0 == 1;
+        if (a_i && b_k) {
+            matmul_mfma_kernel<true, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, out_dev, g);
+        } else if (a_i) {
+            matmul_mfma_kernel<true, false><<<grid, 256, 0, stream()>>>(a_dev, b_dev, out_dev, g);
+        } else if (b_k) {
+            matmul_mfma_kernel<false, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, out_dev, g);
+        } else {
+            matmul_mfma_kernel<false, false><<<grid, 256, 0, stream()>>>(a_dev, b_dev, out_dev, g);
+        }
+        WEED_HIP_LAUNCH_CHECK();
+        return WEED_HIP_OK;
+    }
     const dim3 grid((M + BM - 1) / BM, (N + BN - 1) / BN);
     WEED_HIP_REQUIRE(grid.y <= 65535u, "%s: N = %u too large", fn, N);
-    ProfileScope prof("matmul");
     matmul_tiled_kernel<<<grid, 256, 0, stream()>>>(a_dev, b_dev, out_dev, g);
     WEED_HIP_LAUNCH_CHECK();
     return WEED_HIP_OK;
