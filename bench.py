@@ -164,6 +164,9 @@ def main():
     ap.add_argument("--ctx", type=int, default=8192)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the other configurations (4, 5a, 5b)")
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
+                    help="only launch the library's plain copy kernel on MIB mebibytes (5 launches): the known-size "
+                         "reference against which rocprofv3's FETCH_SIZE / WRITE_SIZE readings are scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path is sharded by (sequence, kv head) with no "
@@ -178,6 +181,16 @@ def main():
     capi.check(lib.weed_hip_init(0))
     stream = torch.cuda.Stream()
     capi.use_torch_stream(stream)
+    if args.calibrate_copy:
+        with torch.cuda.stream(stream):
+            n = args.calibrate_copy * (1 << 20) // 4
+            src = torch.ones(n, device="cuda")
+            dst = torch.empty(n, device="cuda")
+            for _ in range(5):
+                capi.copy(src, dst)
+            torch.cuda.synchronize()
+        print(json.dumps({"calibrate_copy_bytes_read": 4 * n, "calibrate_copy_bytes_written": 4 * n, "launches": 5}))
+        return
     with torch.cuda.stream(stream):
         wl = workloads.config(3, n_seq=args.seqs, scale=args.ctx / 8192.0)
         cache, q, rk, rv = build_cache(capi, torch, wl, seed=1234)

@@ -78,6 +78,12 @@ int weed_hip_matmul_f32(uint32_t M, uint32_t N, uint32_t K, const float *a_dev, 
                         uint32_t a_s1, const float *b_dev, uint32_t b_off, uint32_t b_s0, uint32_t b_s1, float *out_dev,
                         uint32_t o_off, uint32_t o_s0, uint32_t o_s1);
 
+/* out[o_off + i*o_stride] = a[a_off + i*a_stride] for i < n.  Replaces the OpenCL kernel copy_real
+ * (src/common/qengine.cl:979, launched from src/ops/copy_broadcast.cpp:66); also the plain copy used to calibrate the
+ * HBM traffic counters. */
+int weed_hip_copy_f32(uint64_t n, const float *a_dev, uint32_t a_off, uint32_t a_stride, float *out_dev, uint32_t o_off,
+                      uint32_t o_stride);
+
 /* Numerically stable softmax along `axis`.  Replaces Weed::softmax (src/ops/softmax.cpp:276-287; OpenCL kernel
  * softmax_forward, qengine.cl:1001-1033).  rank <= 8. */
 int weed_hip_softmax_f32(uint32_t rank, const uint32_t *shape, uint32_t axis, const float *a_dev, uint32_t a_off,
@@ -191,6 +197,14 @@ enum { WEED_HIP_ATTN_ROTATE_Q = 1, WEED_HIP_ATTN_UNROTATE_OUT = 2 };
 int weed_hip_kv_decode_attn(weed_hip_kv_cache *cache, int32_t n_q_heads, int32_t gqa_mapping, const float *q_dev,
                             uint32_t q_off, const uint32_t q_stride[3], float *out_dev, uint32_t o_off,
                             const uint32_t o_stride[3], uint32_t flags);
+
+/* The same, attending only over the first lens_dev[s] tokens of sequence s (device array of n_seq lengths, each at
+ * most the cached length).  This is how a causal mask with a cache offset is expressed for one query position at a
+ * time: the reference adds a triangular mask to a dense score matrix instead (multihead_attention.cpp:322-328,
+ * src/ops/triu_fill.cpp:42-59). */
+int weed_hip_kv_decode_attn_prefix(weed_hip_kv_cache *cache, const int32_t *lens_dev, int32_t n_q_heads,
+                                   int32_t gqa_mapping, const float *q_dev, uint32_t q_off, const uint32_t q_stride[3],
+                                   float *out_dev, uint32_t o_off, const uint32_t o_stride[3], uint32_t flags);
 
 #ifdef __cplusplus
 }

@@ -220,3 +220,28 @@ def test_head_dims_and_wide_groups(gpu, oracle):
             got = run_decode(gpu, cache, q, gqa, 0)
             assert_attn_close(got, want, "d=%d Hq=%d" % (d, Hq))
         cache.close()
+
+
+def test_prefix_lengths_override(gpu, oracle):
+    """Attention over the first n tokens of each cached sequence (the per-position form of a causal mask) equals the
+    checker run with those lengths; the cache's own lengths are untouched."""
+    import torch
+    rng = np.random.default_rng(41)
+    d, Hkv, Hq = 64, 2, 4
+    lens = [300, 129, 64]
+    S = len(lens)
+    wl = workloads.Workload("prefix", S, Hq, Hkv, d, lens, 4, 4, 0, 0, 0)
+    K = rng.standard_normal((S, Hkv, max(lens), d), dtype=np.float32)
+    V = rng.standard_normal((S, Hkv, max(lens), d), dtype=np.float32)
+    q = rng.standard_normal((S, Hq, d), dtype=np.float32)
+    cache = build_cache(gpu, wl, gpu.KV_UNIFORM, K, V, scales=(1.0, 1.0))
+    for prefix in ([300, 129, 64], [1, 128, 63], [257, 0, 17]):
+        wl_p = workloads.Workload("prefix", S, Hq, Hkv, d, prefix, 4, 4, 0, 0, 0)
+        want = checker_output(oracle, gpu, cache, wl_p, q, True)
+        qd = dev(q)
+        out = torch.zeros_like(qd)
+        cache.decode_attn_prefix(torch.tensor(prefix, dtype=torch.int32, device="cuda"), qd, out)
+        gpu.sync()
+        assert_attn_close(out.cpu().numpy(), want, "prefix %s" % prefix)
+    assert list(cache.seq_lens()) == lens
+    cache.close()

@@ -52,6 +52,7 @@ SIGNATURES = {
     "weed_hip_profile_read": (c_int, [c_char_p, POINTER(c_double), POINTER(c_uint64)]),
     "weed_hip_matmul_f32": (c_int, [c_uint32, c_uint32, c_uint32, c_void_p, c_uint32, c_uint32, c_uint32, c_void_p,
                                     c_uint32, c_uint32, c_uint32, c_void_p, c_uint32, c_uint32, c_uint32]),
+    "weed_hip_copy_f32": (c_int, [c_uint64, c_void_p, c_uint32, c_uint32, c_void_p, c_uint32, c_uint32]),
     "weed_hip_softmax_f32": (c_int, [c_uint32, U32P, c_uint32, c_void_p, c_uint32, U32P, c_void_p, c_uint32, U32P]),
     "weed_hip_reduce_f32": (c_int, [c_int, c_uint32, U32P, c_uint32, c_void_p, c_uint32, U32P, c_void_p, c_uint32,
                                     U32P]),
@@ -76,6 +77,8 @@ SIGNATURES = {
     "weed_hip_kv_export_weed_words": (c_int, [c_void_p, c_int, c_int32, c_int32, c_int32, c_int32, c_void_p]),
     "weed_hip_kv_decode_attn": (c_int, [c_void_p, c_int32, c_int32, c_void_p, c_uint32, U32P, c_void_p, c_uint32, U32P,
                                         c_uint32]),
+    "weed_hip_kv_decode_attn_prefix": (c_int, [c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_uint32, U32P, c_void_p,
+                                               c_uint32, U32P, c_uint32]),
 }
 
 _lib = None
@@ -201,6 +204,15 @@ class KVCache:
         op, oo, os_ = _geom(out)
         check(self.lib.weed_hip_kv_decode_attn(self.handle, q.shape[1], gqa_mapping, qp, qo, qs, op, oo, os_, flags))
 
+    def decode_attn_prefix(self, lens, q, out, gqa_mapping=GQA_WEED, flags=0):
+        """As decode_attn, over the first lens[s] cached tokens only (lens: int32 torch tensor on the device)."""
+        assert q.dim() == 3 and q.shape == out.shape
+        assert lens.element_size() == 4 and lens.is_cuda and lens.is_contiguous() and lens.numel() == q.shape[0]
+        qp, qo, qs = _geom(q)
+        op, oo, os_ = _geom(out)
+        check(self.lib.weed_hip_kv_decode_attn_prefix(self.handle, c_void_p(lens.data_ptr()), q.shape[1], gqa_mapping,
+                                                      qp, qo, qs, op, oo, os_, flags))
+
 
 def use_torch_stream(stream):
     """Route every launch to a torch.cuda.Stream (so that torch events and allocations order with them)."""
@@ -219,6 +231,13 @@ def matmul(a, b, out):
     check(load().weed_hip_matmul_f32(M, N, K, c_void_p(a.data_ptr()), 0, a.stride(0), a.stride(1),
                                      c_void_p(b.data_ptr()), 0, b.stride(0), b.stride(1), c_void_p(out.data_ptr()), 0,
                                      out.stride(0), out.stride(1)))
+
+
+def copy(a, out):
+    """1-D torch views (any stride): out[i] = a[i]."""
+    assert a.dim() == 1 and a.shape == out.shape
+    check(load().weed_hip_copy_f32(a.numel(), c_void_p(a.data_ptr()), 0, a.stride(0), c_void_p(out.data_ptr()), 0,
+                                   out.stride(0)))
 
 
 def softmax(a, out, axis):

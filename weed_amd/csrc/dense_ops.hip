@@ -7,6 +7,7 @@
 // dimension (RT = 1) or a strided one (RT = 16).
 #include "common.h"
 
+#include <algorithm>
 #include <cmath>
 
 using namespace weedhip;
@@ -141,6 +142,16 @@ template <int OP, int RT> __global__ void __launch_bounds__(kThreads) reduce_ker
     }
 }
 
+// out[o_off + i*o_stride] = a[a_off + i*a_stride] (the reference's copy_real, src/common/qengine.cl:979)
+__global__ void __launch_bounds__(256) copy_kernel(const float *__restrict__ a, float *__restrict__ out, uint64_t n,
+                                                   uint32_t a_off, uint32_t a_stride, uint32_t o_off, uint32_t o_stride)
+{
+    const uint64_t step = (uint64_t)gridDim.x * blockDim.x;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += step) {
+        out[(uint64_t)o_off + i * o_stride] = a[(uint64_t)a_off + i * a_stride];
+    }
+}
+
 int make_geom(const char *fn, uint32_t rank, const uint32_t *shape, uint32_t axis, uint32_t a_off,
               const uint32_t *a_stride, uint32_t o_off, const uint32_t *o_stride, bool out_keeps_axis, AxisGeom &g)
 {
@@ -170,6 +181,21 @@ int make_geom(const char *fn, uint32_t rank, const uint32_t *shape, uint32_t axi
 } // namespace
 
 extern "C" {
+
+int weed_hip_copy_f32(uint64_t n, const float *a_dev, uint32_t a_off, uint32_t a_stride, float *out_dev,
+                      uint32_t o_off, uint32_t o_stride)
+{
+    WEED_HIP_REQUIRE(a_dev && out_dev, "weed_hip_copy_f32: null pointer");
+    WEED_HIP_TRY(ensure_init());
+    if (!n) {
+        return WEED_HIP_OK;
+    }
+    ProfileScope prof("copy");
+    const uint32_t blocks = (uint32_t)std::min<uint64_t>((n + 255) / 256, 256u * 64u);
+    copy_kernel<<<blocks, 256, 0, stream()>>>(a_dev, out_dev, n, a_off, a_stride, o_off, o_stride);
+    WEED_HIP_LAUNCH_CHECK();
+    return WEED_HIP_OK;
+}
 
 int weed_hip_softmax_f32(uint32_t rank, const uint32_t *shape, uint32_t axis, const float *a_dev, uint32_t a_off,
                          const uint32_t *a_stride, float *out_dev, uint32_t o_off, const uint32_t *o_stride)

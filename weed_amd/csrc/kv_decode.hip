@@ -343,13 +343,11 @@ __global__ void combine_kernel(const float *__restrict__ partials, uint32_t Hq, 
     out[(uint64_t)og.off + (uint64_t)s * og.s[0] + (uint64_t)h * og.s[1] + (uint64_t)tid * og.s[2]] = r;
 }
 
-} // namespace
-
-extern "C" int weed_hip_kv_decode_attn(weed_hip_kv_cache *c, int32_t n_q_heads, int32_t gqa_mapping, const float *q_dev,
-                                       uint32_t q_off, const uint32_t q_stride[3], float *out_dev, uint32_t o_off,
-                                       const uint32_t o_stride[3], uint32_t flags)
+// `lens_dev` (optional): attend over these per-sequence lengths instead of the cached ones.
+int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t gqa_mapping, const float *q_dev,
+                uint32_t q_off, const uint32_t q_stride[3], float *out_dev, uint32_t o_off, const uint32_t o_stride[3],
+                uint32_t flags, const int32_t *lens_dev)
 {
-    const char *fn = "weed_hip_kv_decode_attn";
     WEED_HIP_REQUIRE(c, "%s: null cache", fn);
     WEED_HIP_REQUIRE(q_dev && out_dev && q_stride && o_stride, "%s: null pointer", fn);
     const uint32_t Hkv = (uint32_t)c->cfg.n_kv_heads, d = (uint32_t)c->cfg.head_dim, S = (uint32_t)c->cfg.n_seq;
@@ -425,7 +423,7 @@ extern "C" int weed_hip_kv_decode_attn(weed_hip_kv_cache *c, int32_t n_q_heads, 
         MfmaParams mp;
         mp.k = side_params(c, 0);
         mp.v = side_params(c, 1);
-        mp.lens = c->lens_dev;
+        mp.lens = lens_dev ? lens_dev : c->lens_dev;
         mp.padded = c->padded_tokens;
         mp.Hq = Hq;
         mp.Hkv = Hkv;
@@ -444,7 +442,7 @@ extern "C" int weed_hip_kv_decode_attn(weed_hip_kv_cache *c, int32_t n_q_heads, 
         DecodeParams p;
         p.k = side_params(c, 0);
         p.v = side_params(c, 1);
-        p.lens = c->lens_dev;
+        p.lens = lens_dev ? lens_dev : c->lens_dev;
         p.padded = c->padded_tokens;
         p.d = d;
         p.Hq = Hq;
@@ -466,4 +464,24 @@ extern "C" int weed_hip_kv_decode_attn(weed_hip_kv_cache *c, int32_t n_q_heads, 
         WEED_HIP_LAUNCH_CHECK();
     }
     return WEED_HIP_OK;
+}
+
+} // namespace
+
+extern "C" int weed_hip_kv_decode_attn(weed_hip_kv_cache *c, int32_t n_q_heads, int32_t gqa_mapping, const float *q_dev,
+                                       uint32_t q_off, const uint32_t q_stride[3], float *out_dev, uint32_t o_off,
+                                       const uint32_t o_stride[3], uint32_t flags)
+{
+    return decode_impl("weed_hip_kv_decode_attn", c, n_q_heads, gqa_mapping, q_dev, q_off, q_stride, out_dev, o_off,
+                       o_stride, flags, nullptr);
+}
+
+extern "C" int weed_hip_kv_decode_attn_prefix(weed_hip_kv_cache *c, const int32_t *lens_dev, int32_t n_q_heads,
+                                              int32_t gqa_mapping, const float *q_dev, uint32_t q_off,
+                                              const uint32_t q_stride[3], float *out_dev, uint32_t o_off,
+                                              const uint32_t o_stride[3], uint32_t flags)
+{
+    const char *fn = "weed_hip_kv_decode_attn_prefix";
+    WEED_HIP_REQUIRE(lens_dev, "%s: null length array", fn);
+    return decode_impl(fn, c, n_q_heads, gqa_mapping, q_dev, q_off, q_stride, out_dev, o_off, o_stride, flags, lens_dev);
 }
