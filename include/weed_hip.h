@@ -84,6 +84,27 @@ int weed_hip_matmul_f32(uint32_t M, uint32_t N, uint32_t K, const float *a_dev, 
 int weed_hip_copy_f32(uint64_t n, const float *a_dev, uint32_t a_off, uint32_t a_stride, float *out_dev, uint32_t o_off,
                       uint32_t o_stride);
 
+/* Broadcasting elementwise ops on tensors of one logical shape (rank <= 8, strides in elements, stride 0 repeats a
+ * dimension): out = a (COPY; b may be NULL), a + b, a - b, a * b, a / b.  Replace Weed's add / mul
+ * (src/ops/commuting.cpp:17-25), sub (src/ops/sub.cpp), div with IEEE division (src/ops/div.cpp:17-20), add_in_place
+ * (src/ops/in_place.cpp:17-25, out aliasing a) and the strided gather behind Tensor::contiguous
+ * (include/tensors/tensor.hpp:319-331). */
+enum {
+    WEED_HIP_EW_COPY = 0,
+    WEED_HIP_EW_ADD = 1,
+    WEED_HIP_EW_SUB = 2,
+    WEED_HIP_EW_MUL = 3,
+    WEED_HIP_EW_DIV = 4
+};
+int weed_hip_elementwise_f32(int op, uint32_t rank, const uint32_t *shape, const float *a_dev, uint32_t a_off,
+                             const uint32_t *a_stride, const float *b_dev, uint32_t b_off, const uint32_t *b_stride,
+                             float *out_dev, uint32_t o_off, const uint32_t *o_stride);
+
+/* a[i,j] = val wherever i + diagonal <= j, on a rows x cols matrix.  Replaces Weed::triu_fill
+ * (src/ops/triu_fill.cpp:42-59), the causal mask builder of MultiHeadAttention::forward. */
+int weed_hip_triu_fill_f32(uint32_t rows, uint32_t cols, float val, uint32_t diagonal, float *a_dev, uint32_t a_off,
+                           uint32_t a_s0, uint32_t a_s1);
+
 /* Numerically stable softmax along `axis`.  Replaces Weed::softmax (src/ops/softmax.cpp:276-287; OpenCL kernel
  * softmax_forward, qengine.cl:1001-1033).  rank <= 8. */
 int weed_hip_softmax_f32(uint32_t rank, const uint32_t *shape, uint32_t axis, const float *a_dev, uint32_t a_off,
@@ -108,6 +129,14 @@ int weed_hip_reduce_f32(int op, uint32_t rank, const uint32_t *shape, uint32_t a
 int weed_hip_make_rotation(uint32_t seed, uint32_t d, float *r_dev);
 /* Device Gram-Schmidt only (input already in r_dev). */
 int weed_hip_orthonormalize_columns(uint32_t d, float *r_dev);
+
+/* apply_rotation (src/modules/multihead_attention.cpp:125-140): y = x . R over the last dimension (length d) of a
+ * strided tensor of rank <= 8; R is d x d column-major.  Products are added in ascending index order with separate
+ * multiplies and adds, the order of the reference's naive matmul (src/ops/matmul.cpp:40-44), so the rotated values
+ * match a BLAS-less reference build bit for bit.  x_dev and out_dev must not overlap. */
+int weed_hip_apply_rotation_f32(uint32_t d, const float *r_dev, uint32_t rank, const uint32_t *shape,
+                                const float *x_dev, uint32_t x_off, const uint32_t *x_stride, float *out_dev,
+                                uint32_t o_off, const uint32_t *o_stride);
 
 /* ------------------------------------------------------------------------------------------------ */
 /* quantized KV cache: device twin of Weed::QuantizedKVCache (include/modules/multihead_attention.hpp:22-36)  */

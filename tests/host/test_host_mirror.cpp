@@ -1,0 +1,666 @@
+// Tests of the host C++ mirror, written the way the reference writes its own (test/tests.cpp): tensors are built
+// with std::make_shared<Tensor>(values, shape, ...), ops are called through Tensor:: / operators, and results are
+// read back through storage.  Cases marked `needs_gpu = false` exercise host logic only and run anywhere; the rest
+// run every computation on the device and compare with the CPU checker (oracle/) or with closed forms.
+//
+// Usage: test_host_mirror [--no-gpu] [name-substring]
+#include "weed.hpp"
+
+#include "weed_oracle.h"
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <functional>
+#include <random>
+#include <string>
+#include <vector>
+
+using namespace Weed;
+
+namespace {
+
+struct Case {
+    const char *name;
+    bool needs_gpu;
+    std::function<void()> body;
+};
+std::vector<Case> &cases()
+{
+    static std::vector<Case> c;
+    return c;
+}
+struct Registrar {
+    Registrar(const char *n, bool g, std::function<void()> b) { cases().push_back({ n, g, std::move(b) }); }
+};
+int failures = 0;
+
+#define TEST_CASE(name, needs_gpu)                                                                                     \
+    static void name();                                                                                                \
+    static Registrar reg_##name(#name, needs_gpu, name);                                                               \
+    static void name()
+
+#define REQUIRE(cond)                                                                                                  \
+    do {                                                                                                               \
+        if (!(cond)) {                                                                                                 \
+            std::printf("    FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond);                                          \
+            ++failures;                                                                                                \
+        }                                                                                                              \
+    } while (0)
+
+#define EPSILON 0.01f // test/tests.cpp:30
+#define REQUIRE_FLOAT(A, B) REQUIRE(std::fabs((double)(A) - (double)(B)) < EPSILON)
+
+#define REQUIRE_THROWS_AS(expr, type)                                                                                  \
+    do {                                                                                                               \
+        bool caught = false;                                                                                           \
+        try {                                                                                                          \
+            (void)(expr);                                                                                              \
+        } catch (const type &) {                                                                                       \
+            caught = true;                                                                                             \
+        } catch (...) {                                                                                                \
+        }                                                                                                              \
+        if (!caught) {                                                                                                 \
+            std::printf("    FAILED %s:%d: %s did not throw %s\n", __FILE__, __LINE__, #expr, #type);                  \
+            ++failures;                                                                                                \
+        }                                                                                                              \
+    } while (0)
+
+#define R(v) real1(v)
+const DeviceTag TEST_DTAG = DeviceTag::GPU;
+
+real1 get_real(const TensorPtr &t) { return t->get_item(); }
+
+std::vector<real1> gaussian(size_t n, uint32_t seed, real1 scale = 1.0f)
+{
+    std::mt19937 rng(seed);
+    std::normal_distribution<real1> dist(0.0f, 1.0f);
+    std::vector<real1> v(n);
+    for (real1 &x : v) {
+        x = scale * dist(rng);
+    }
+    return v;
+}
+
+// The attention tolerance: |got - want| <= 1e-4 + 1e-3 |want|
+bool attn_close(const std::vector<real1> &got, const std::vector<double> &want, double *worst = nullptr)
+{
+    bool ok = got.size() == want.size();
+    double w = 0.0;
+    for (size_t i = 0; ok && i < got.size(); ++i) {
+        const double err = std::fabs((double)got[i] - want[i]);
+        w = std::max(w, err);
+        if (!(err <= 1e-4 + 1e-3 * std::fabs(want[i]))) {
+            ok = false;
+        }
+    }
+    if (worst) {
+        *worst = w;
+    }
+    return ok;
+}
+
+// --------------------------------------------------------------------------------------------------------------------
+// host logic (no device)
+// --------------------------------------------------------------------------------------------------------------------
+
+TEST_CASE(test_column_major_geometry, false)
+{
+    // test/tests.cpp:1214-1218: element [r, c] of a 2x3 tensor is at index r + c*nrows
+    TensorPtr x = std::make_shared<Tensor>(std::vector<real1>{ R(1), R(2), R(3), R(4), R(5), R(6) },
+        std::vector<tcapint>{ 2, 3 }, false, DeviceTag::CPU);
+    REQUIRE(x->stride == (std::vector<tcapint>{ 1U, 2U }));
+    REQUIRE(x->get_storage_index(3U) == 3U);
+    REQUIRE(get_real((*(*x)[2])[1]) == R(6)); // operator[] fixes the LAST index first
+    REQUIRE(get_real((*(*x)[0])[1]) == R(2));
+    TensorPtr t = Tensor::transpose(x);
+    REQUIRE(t->shape == (std::vector<tcapint>{ 3U, 2U }));
+    REQUIRE(t->stride == (std::vector<tcapint>{ 2U, 1U }));
+    REQUIRE(!t->is_contiguous());
+    REQUIRE(t->to_vector() == (std::vector<real1>{ 1, 3, 5, 2, 4, 6 }));
+    TensorPtr s = Tensor::slice(x, 1, 1U, 2U);
+    REQUIRE(s->offset == 2U);
+    REQUIRE(s->to_vector() == (std::vector<real1>{ 3, 4, 5, 6 }));
+    TensorPtr row = Tensor::slice(x, 1);
+    REQUIRE(row->to_vector() == (std::vector<real1>{ 2, 4, 6 }));
+    // size-1 dimensions carry stride 0 (include/tensors/base_tensor.hpp:282-292)
+    REQUIRE(Tensor::full_contiguous_stride({ 1U, 4U, 1U, 3U }) == (std::vector<tcapint>{ 0U, 1U, 0U, 4U }));
+    REQUIRE_THROWS_AS(x->get_storage_index(6U), std::invalid_argument);
+    REQUIRE_THROWS_AS((*x)[3], std::invalid_argument);
+}
+
+TEST_CASE(test_reshape_rules, false)
+{
+    TensorPtr x = std::make_shared<Tensor>(
+        std::vector<real1>{ 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11 }, std::vector<tcapint>{ 2, 6 }, false, DeviceTag::CPU);
+    TensorPtr y = Tensor::reshape(x, { 2, -1, 2 });
+    REQUIRE(y->shape == (std::vector<tcapint>{ 2U, 3U, 2U }));
+    REQUIRE(y->storage == x->storage); // a contiguous tensor is re-viewed, not copied
+    REQUIRE(y->to_vector() == x->to_vector());
+    REQUIRE_THROWS_AS(Tensor::reshape(x, { -1, -1 }), std::invalid_argument);
+    REQUIRE_THROWS_AS(Tensor::reshape(x, { 5, -1 }), std::invalid_argument);
+    REQUIRE_THROWS_AS(Tensor::reshape(x, { 5, 2 }), std::invalid_argument);
+    REQUIRE_THROWS_AS(std::make_shared<Tensor>(std::vector<real1>{ 1, 2, 3 }, std::vector<tcapint>{ 2, 2 }, false, DeviceTag::CPU),
+        std::invalid_argument);
+    REQUIRE_THROWS_AS(std::make_shared<CpuRealStorage>(0U), std::invalid_argument);
+}
+
+TEST_CASE(test_cpu_tensors_do_not_compute, false)
+{
+    // there is no CPU arithmetic in this build: an op handed host tensors must say so, never fall back
+    TensorPtr x = std::make_shared<Tensor>(std::vector<real1>{ R(2), R(3) }, std::vector<tcapint>{ 1, 2 }, false, DeviceTag::CPU);
+    TensorPtr y = std::make_shared<Tensor>(std::vector<real1>{ R(4), R(5) }, std::vector<tcapint>{ 2, 1 }, false, DeviceTag::CPU);
+    REQUIRE_THROWS_AS(x >> y, std::domain_error);
+    REQUIRE_THROWS_AS(Tensor::softmax(x, 1), std::domain_error);
+    REQUIRE_THROWS_AS(Tensor::sum(x, 1), std::domain_error);
+    REQUIRE_THROWS_AS(x + x, std::domain_error);
+    QuantizedKVCache qc;
+    real1 v[32] = { 0 };
+    REQUIRE_THROWS_AS(qc.write_row(0U, v), std::domain_error);
+    REQUIRE_THROWS_AS(qc.read_row(0U, v), std::domain_error);
+}
+
+// --------------------------------------------------------------------------------------------------------------------
+// the reference's op tests, on the device (forward values; there is no autograd here)
+// --------------------------------------------------------------------------------------------------------------------
+
+TEST_CASE(test_real_matmul, true)
+{
+    // test/tests.cpp:1020-1041
+    TensorPtr x = std::make_shared<Tensor>(std::vector<real1>{ R(2), R(3) }, std::vector<tcapint>{ 1, 2 }, false, TEST_DTAG);
+    TensorPtr y = std::make_shared<Tensor>(std::vector<real1>{ R(4), R(5) }, std::vector<tcapint>{ 2, 1 }, false, TEST_DTAG);
+    TensorPtr z = x >> y;
+    REQUIRE(get_real((*z)[0]) == R(23));
+
+    x = std::make_shared<Tensor>(std::vector<real1>{ R(2), R(3) }, std::vector<tcapint>{ 2, 1 }, false, TEST_DTAG);
+    y = std::make_shared<Tensor>(std::vector<real1>{ R(4), R(5) }, std::vector<tcapint>{ 1, 2 }, false, TEST_DTAG);
+    z = x >> y;
+    REQUIRE(get_real((*(*z)[0])[0]) == R(8));
+    REQUIRE(get_real((*(*z)[0])[1]) == R(12));
+    REQUIRE(get_real((*(*z)[1])[0]) == R(10));
+    REQUIRE(get_real((*(*z)[1])[1]) == R(15));
+    z = y << x; // same product, operands swapped
+    REQUIRE(get_real((*(*z)[1])[1]) == R(15));
+}
+
+TEST_CASE(test_matmul_2x3_3x2, true)
+{
+    // operands of test/tests.cpp:1327-1340 (column-major); C = A.B = [[76, 103], [100, 136]]
+    TensorPtr A = std::make_shared<Tensor>(
+        std::vector<real1>{ R(1), R(2), R(3), R(4), R(5), R(6) }, std::vector<tcapint>{ 2, 3 }, true, TEST_DTAG);
+    TensorPtr B = std::make_shared<Tensor>(
+        std::vector<real1>{ R(7), R(8), R(9), R(10), R(11), R(12) }, std::vector<tcapint>{ 3, 2 }, true, TEST_DTAG);
+    TensorPtr C = A >> B;
+    REQUIRE(C->to_vector() == (std::vector<real1>{ 76, 100, 103, 136 }));
+    // a transposed view is a valid operand: B^T.A^T = C^T
+    TensorPtr Ct = Tensor::transpose(B) >> Tensor::transpose(A);
+    REQUIRE(Ct->to_vector() == (std::vector<real1>{ 76, 103, 100, 136 }));
+    REQUIRE_THROWS_AS(A >> A, std::invalid_argument);
+    TensorPtr host = A->cast(DeviceTag::CPU);
+    REQUIRE_THROWS_AS(host >> B, std::invalid_argument); // device mismatch is reported before anything runs
+}
+
+TEST_CASE(test_softmax_forward, true)
+{
+    // test/tests.cpp:1110-1171
+    TensorPtr x = std::make_shared<Tensor>(std::vector<real1>{ R(1), R(2), R(3) }, std::vector<tcapint>{ 3 }, false, TEST_DTAG);
+    TensorPtr y = Tensor::softmax(x, 0);
+    RealStorage *ys = static_cast<RealStorage *>(y->storage.get());
+    REQUIRE_FLOAT((real1_f)(*ys)[0] + (real1_f)(*ys)[1] + (real1_f)(*ys)[2], 1.0f);
+
+    x = std::make_shared<Tensor>(std::vector<real1>{ R(1), R(3), R(2) }, std::vector<tcapint>{ 3 }, false, TEST_DTAG);
+    y = Tensor::softmax(x, 0);
+    ys = static_cast<RealStorage *>(y->storage.get());
+    REQUIRE((real1_f)(*ys)[1] > (real1_f)(*ys)[2]);
+    REQUIRE((real1_f)(*ys)[2] > (real1_f)(*ys)[0]);
+
+    x = std::make_shared<Tensor>(std::vector<real1>{ R(1000), R(1001), R(1002) }, std::vector<tcapint>{ 3 }, false, TEST_DTAG);
+    y = Tensor::softmax(x, 0);
+    ys = static_cast<RealStorage *>(y->storage.get());
+    const real1_f sum = (real1_f)(*ys)[0] + (real1_f)(*ys)[1] + (real1_f)(*ys)[2];
+    REQUIRE(std::isfinite(sum));
+    REQUIRE_FLOAT(sum, 1.0f);
+
+    x = std::make_shared<Tensor>(std::vector<real1>{ R(2), R(2), R(2) }, std::vector<tcapint>{ 3 }, false, TEST_DTAG);
+    y = Tensor::softmax(x, 0);
+    ys = static_cast<RealStorage *>(y->storage.get());
+    REQUIRE_FLOAT((real1_f)(*ys)[0], 1.0f / 3.0f);
+    REQUIRE_FLOAT((real1_f)(*ys)[2], 1.0f / 3.0f);
+
+    x = std::make_shared<Tensor>(std::vector<real1>{ R(0), R(1) }, std::vector<tcapint>{ 2 }, false, TEST_DTAG);
+    y = Tensor::softmax(x, 0);
+    ys = static_cast<RealStorage *>(y->storage.get());
+    const real1_f denom = 1.0f + std::exp(1.0f);
+    REQUIRE(std::fabs((*ys)[0] - 1.0f / denom) < 1e-6f);
+    REQUIRE(std::fabs((*ys)[1] - std::exp(1.0f) / denom) < 1e-6f);
+}
+
+TEST_CASE(test_softmax_axis1, true)
+{
+    // test/tests.cpp:1206-1221
+    TensorPtr x = std::make_shared<Tensor>(
+        std::vector<real1>{ R(1), R(2), R(3), R(4), R(5), R(6) }, std::vector<tcapint>{ 2, 3 }, false, TEST_DTAG);
+    TensorPtr y = Tensor::softmax(x, 1);
+    RealStorage *ys = static_cast<RealStorage *>(y->storage.get());
+    REQUIRE_FLOAT((real1_f)(*ys)[0] + (real1_f)(*ys)[2] + (real1_f)(*ys)[4], 1.0f);
+    REQUIRE_FLOAT((real1_f)(*ys)[1] + (real1_f)(*ys)[3] + (real1_f)(*ys)[5], 1.0f);
+    TensorPtr z = Tensor::softmax(x, -1); // negative axes count from the end
+    REQUIRE(z->to_vector() == y->to_vector());
+}
+
+TEST_CASE(test_axis_reductions, true)
+{
+    // test/tests.cpp:177-228
+    TensorPtr x = std::make_shared<Tensor>(std::vector<real1>{ R(1), R(1) }, std::vector<tcapint>{ 2 }, true, TEST_DTAG);
+    REQUIRE(get_real(Tensor::sum(x, 0U)) == R(2));
+    x = std::make_shared<Tensor>(std::vector<real1>{ R(0), R(1) }, std::vector<tcapint>{ 2 }, true, TEST_DTAG);
+    REQUIRE(get_real(Tensor::max(x, 0U)) == R(1));
+    REQUIRE(get_real(Tensor::min(x, 0U)) == R(0));
+    // a 2x3 matrix along both axes
+    x = std::make_shared<Tensor>(
+        std::vector<real1>{ R(1), R(2), R(3), R(4), R(5), R(6) }, std::vector<tcapint>{ 2, 3 }, false, TEST_DTAG);
+    REQUIRE(Tensor::sum(x, 0)->to_vector() == (std::vector<real1>{ 3, 7, 11 }));
+    REQUIRE(Tensor::sum(x, 1)->to_vector() == (std::vector<real1>{ 9, 12 }));
+    REQUIRE(Tensor::max(x, 1)->to_vector() == (std::vector<real1>{ 5, 6 }));
+    REQUIRE(Tensor::min(Tensor::transpose(x), 0)->to_vector() == (std::vector<real1>{ 1, 2 }));
+}
+
+TEST_CASE(test_elementwise_and_storage_round_trip, true)
+{
+    TensorPtr a = std::make_shared<Tensor>(
+        std::vector<real1>{ R(1), R(2), R(3), R(4), R(5), R(6) }, std::vector<tcapint>{ 2, 3 }, false, TEST_DTAG);
+    TensorPtr b = std::make_shared<Tensor>(std::vector<real1>{ R(10), R(20), R(30) }, std::vector<tcapint>{ 1, 3 }, false, TEST_DTAG);
+    REQUIRE((a + b)->to_vector() == (std::vector<real1>{ 11, 12, 23, 24, 35, 36 }));
+    REQUIRE((a - b)->to_vector() == (std::vector<real1>{ -9, -8, -17, -16, -25, -24 }));
+    REQUIRE((a * b)->to_vector() == (std::vector<real1>{ 10, 20, 60, 80, 150, 180 }));
+    REQUIRE((a / R(2))->to_vector() == (std::vector<real1>{ 0.5f, 1, 1.5f, 2, 2.5f, 3 }));
+    REQUIRE((R(2) * a)->to_vector() == (std::vector<real1>{ 2, 4, 6, 8, 10, 12 }));
+    REQUIRE(Tensor::contiguous(Tensor::transpose(a))->to_vector() == (std::vector<real1>{ 1, 3, 5, 2, 4, 6 }));
+    Weed::add_in_place(*a, *b);
+    REQUIRE(a->to_vector() == (std::vector<real1>{ 11, 12, 23, 24, 35, 36 }));
+    TensorPtr m = Tensor::zeros({ 3U, 4U }, false, false, DType::REAL, TEST_DTAG);
+    Weed::triu_fill(*m, R(-7));
+    REQUIRE(m->to_vector() == (std::vector<real1>{ 0, 0, 0, -7, 0, 0, -7, -7, 0, -7, -7, -7 }));
+    // storage: device -> host copy is a new object, host -> device likewise (src/storage/gpu_real_storage.cpp:18-23)
+    StoragePtr host = a->storage->cpu();
+    REQUIRE(host->device == DeviceTag::CPU);
+    REQUIRE(host != a->storage);
+    REQUIRE((*static_cast<RealStorage *>(host.get()))[5] == R(36));
+    StoragePtr back = host->gpu();
+    REQUIRE(back->device == DeviceTag::GPU);
+    REQUIRE((*static_cast<RealStorage *>(back.get()))[4] == R(35));
+    static_cast<RealStorage *>(back.get())->write(4U, R(-1));
+    REQUIRE((*static_cast<RealStorage *>(back.get()))[4] == R(-1));
+    REQUIRE_THROWS_AS((*static_cast<RealStorage *>(back.get()))[6], std::invalid_argument);
+    REQUIRE_THROWS_AS(a + Tensor::transpose(a), std::invalid_argument);
+}
+
+// --------------------------------------------------------------------------------------------------------------------
+// QuantizedKVCache
+// --------------------------------------------------------------------------------------------------------------------
+
+TEST_CASE(test_quantized_cache_known_answers, true)
+{
+    // write_row / read_row answers recorded from the reference's own coder, padded with zeros to d = 32
+    const std::vector<real1> vals = { -10, -3, -2.999f, -1e-4f, 0, .1874f, .1876f, 2.6249f, 2.625f, 2.99f, 3, 10 };
+    struct Kat {
+        int bits;
+        std::vector<uint32_t> words; // the words that hold the twelve codes
+    };
+    for (const Kat &k : { Kat{ 2, { 0x00ffea40u } }, Kat{ 3, { 0x3ff24600u, 0x0000003fu } }, Kat{ 4, { 0xe8887000u, 0x0000ffffu } } }) {
+        QuantizedKVCache qc;
+        qc.allocate(4U, 32U, k.bits);
+        qc.block_scale = ONE_R1;
+        std::vector<real1> row(32, -10.0f); // padding codes are 0, so the known words are not disturbed
+        std::copy(vals.begin(), vals.end(), row.begin());
+        qc.write_row(0U, row.data());
+        qc.sync_packed();
+        for (size_t w = 0; w < k.words.size(); ++w) {
+            REQUIRE((uint32_t)qc.packed[w] == k.words[w]);
+        }
+        // the whole row against the CPU checker, words and dequantised values
+        std::vector<int32_t> want_words((size_t)wo_words_per_row(32, k.bits), 0);
+        wo_uniform_write_row(want_words.data(), 0U, row.data(), 32, k.bits, 1.0f);
+        REQUIRE(qc.packed.size() == want_words.size());
+        REQUIRE(std::memcmp(qc.packed.data(), want_words.data(), want_words.size() * sizeof(int32_t)) == 0);
+        std::vector<real1> got(32), want(32);
+        qc.read_row(0U, got.data());
+        wo_uniform_read_row(want_words.data(), 0U, want.data(), 32, k.bits, 1.0f);
+        REQUIRE(got == want);
+        REQUIRE_THROWS_AS(qc.write_row(3U, row.data()), std::domain_error); // append-only
+    }
+    {
+        QuantizedKVCache qc;
+        qc.allocate(2U, 32U, 4);
+        qc.block_scale = 0.731f;
+        std::vector<real1> row(32, -10.0f);
+        const real1 in[4] = { 0.5f, -1.2f, 2.0f, -0.05f };
+        std::copy(in, in + 4, row.begin());
+        qc.write_row(0U, row.data());
+        qc.sync_packed();
+        REQUIRE(((uint32_t)qc.packed[0] & 0xffffu) == 0x7f39u);
+        std::vector<real1> got(32);
+        qc.read_row(0U, got.data());
+        REQUIRE(got[0] == 0.41118741f);
+        REQUIRE(got[1] == -1.23356247f);
+        REQUIRE(got[2] == 2.05593753f);
+        REQUIRE(got[3] == -0.13706255f);
+    }
+}
+
+// --------------------------------------------------------------------------------------------------------------------
+// MultiHeadAttention
+// --------------------------------------------------------------------------------------------------------------------
+
+struct HostLinear {
+    std::vector<real1> w, b; // w column-major (in, out)
+    tcapint in, out;
+};
+
+HostLinear install(const LinearPtr &l, uint32_t seed)
+{
+    HostLinear h;
+    h.in = l->in_features;
+    h.out = l->out_features;
+    h.w = gaussian((size_t)h.in * h.out, seed, 1.0f / std::sqrt((real1)h.in));
+    h.b = gaussian(h.out, seed + 1U, 0.1f);
+    l->weight = std::make_shared<Parameter>(h.w, std::vector<tcapint>{ h.in, h.out }, true, TEST_DTAG);
+    if (l->bias) {
+        l->bias = std::make_shared<Parameter>(h.b, std::vector<tcapint>{ 1U, h.out }, true, TEST_DTAG);
+    }
+    return h;
+}
+
+// y[r, o] = sum_i x[r, i] w[i, o] + b[o] in double; x is column-major (rows, in)
+std::vector<double> host_linear(const HostLinear &l, const std::vector<double> &x, size_t rows)
+{
+    std::vector<double> y(rows * l.out);
+    for (size_t r = 0; r < rows; ++r) {
+        for (tcapint o = 0; o < l.out; ++o) {
+            double acc = l.b[o];
+            for (tcapint i = 0; i < l.in; ++i) {
+                acc += x[r + rows * i] * (double)l.w[i + (size_t)l.in * o];
+            }
+            y[r + rows * o] = acc;
+        }
+    }
+    return y;
+}
+
+// Dense float64 attention over given K/V rows (already what the cache holds), as MultiHeadAttention::forward
+// defines it: element (b, t, h, j) of a (B, T, H, hd) column-major tensor is at b + B*(t + T*(h + H*j)).
+struct AttnCheck {
+    tcapint B, H, Hkv, hd;
+    bool blocked;
+    // kv(b, kvh, tok, j): cached row value
+    std::function<double(tcapint, tcapint, tcapint, tcapint)> kf, vf;
+};
+
+std::vector<double> host_attention(const AttnCheck &g, const std::vector<double> &Q, tcapint T, tcapint before)
+{
+    std::vector<double> out((size_t)g.B * T * g.H * g.hd, 0.0);
+    const tcapint groups = g.H / g.Hkv;
+    for (tcapint b = 0; b < g.B; ++b) {
+        for (tcapint t = 0; t < T; ++t) {
+            for (tcapint h = 0; h < g.H; ++h) {
+                const tcapint kvh = g.blocked ? h / groups : h % g.Hkv;
+                const tcapint n = before + t + 1U;
+                std::vector<double> s(n);
+                double mx = -1e300;
+                for (tcapint tok = 0; tok < n; ++tok) {
+                    double acc = 0.0;
+                    for (tcapint j = 0; j < g.hd; ++j) {
+                        acc += Q[b + (size_t)g.B * (t + (size_t)T * (h + (size_t)g.H * j))] * g.kf(b, kvh, tok, j);
+                    }
+                    s[tok] = acc / std::sqrt((double)g.hd);
+                    mx = std::max(mx, s[tok]);
+                }
+                double sum = 0.0;
+                for (double &v : s) {
+                    v = std::exp(v - mx);
+                    sum += v;
+                }
+                for (tcapint j = 0; j < g.hd; ++j) {
+                    double acc = 0.0;
+                    for (tcapint tok = 0; tok < n; ++tok) {
+                        acc += s[tok] * g.vf(b, kvh, tok, j);
+                    }
+                    out[b + (size_t)g.B * (t + (size_t)T * (h + (size_t)g.H * j))] = acc / sum;
+                }
+            }
+        }
+    }
+    return out;
+}
+
+// y = x.R over the last (slowest) dimension of a column-major (rows, hd) array
+std::vector<double> host_rotate(const std::vector<double> &x, size_t rows, tcapint hd, const std::vector<real1> &Rm)
+{
+    std::vector<double> y(rows * hd);
+    for (size_t r = 0; r < rows; ++r) {
+        for (tcapint j = 0; j < hd; ++j) {
+            double acc = 0.0;
+            for (tcapint i = 0; i < hd; ++i) {
+                acc += x[r + rows * i] * (double)Rm[i + (size_t)hd * j];
+            }
+            y[r + rows * j] = acc;
+        }
+    }
+    return y;
+}
+
+std::vector<double> to_double(const std::vector<real1> &v) { return std::vector<double>(v.begin(), v.end()); }
+
+void run_attention_case(KVCoder coder, int bits, bool blocked, uint32_t seed)
+{
+    const tcapint B = 2U, dm = 96U, H = 4U, Hkv = 2U, hd = 64U;
+    MultiHeadAttention mha(dm, H, Hkv, hd, TEST_DTAG, nullptr, ZERO_R1, -1, true, bits);
+    mha.kv_coder = coder;
+    mha.gqa_blocked = blocked;
+    mha.rotation_seed = seed;
+    if (coder == KV_LLOYDMAX) {
+        mha.k_bits = 3;
+        mha.k_sign = true;
+    }
+    mha.set_max_kv_seq_len(40U);
+    const HostLinear wq = install(mha.W_q, seed + 10U), wk = install(mha.W_k, seed + 20U);
+    const HostLinear wv = install(mha.W_v, seed + 30U), wo = install(mha.W_o, seed + 40U);
+    (void)wk;
+    (void)wv;
+
+    tcapint before = 0U;
+    for (const tcapint T : { 7U, 1U, 1U, 3U }) { // prefill, two decode steps, a chunk
+        const std::vector<real1> xv = gaussian((size_t)B * T * dm, seed + 100U + before);
+        TensorPtr x = std::make_shared<Tensor>(xv, std::vector<tcapint>{ B, T, dm }, false, TEST_DTAG);
+        TensorPtr y = mha.forward(x);
+        REQUIRE(y->shape == (std::vector<tcapint>{ B, T, dm }));
+        REQUIRE(mha.cache_len == before + T);
+        REQUIRE(mha.max_seq_len == 40U); // the reference overwrites this at the first call; here it sticks
+        REQUIRE(mha.k_rotation.size() == (size_t)hd * hd);
+
+        // check: float64 attention over the rows the device cache actually holds (rotated basis)
+        const size_t rows = (size_t)B * T;
+        std::vector<double> Qd = host_linear(wq, to_double(xv), rows); // (B, T, H*hd) = (B, T, H, hd)
+        Qd = host_rotate(Qd, rows * H, hd, mha.k_rotation);
+        const tcapint cap = mha.max_seq_len;
+        std::vector<real1> krows((size_t)B * Hkv * (before + T) * hd), vrows(krows.size());
+        for (tcapint p = 0; p < B * Hkv; ++p) {
+            for (tcapint tok = 0; tok < before + T; ++tok) {
+                mha.k_qcache.read_row(p * cap + tok, &krows[((size_t)p * (before + T) + tok) * hd]);
+                mha.v_qcache.read_row(p * cap + tok, &vrows[((size_t)p * (before + T) + tok) * hd]);
+            }
+        }
+        const tcapint n_tok = before + T;
+        AttnCheck g{ B, H, Hkv, hd, blocked,
+            [&](tcapint b, tcapint kvh, tcapint tok, tcapint j) { return (double)krows[(((size_t)(b * Hkv + kvh)) * n_tok + tok) * hd + j]; },
+            [&](tcapint b, tcapint kvh, tcapint tok, tcapint j) { return (double)vrows[(((size_t)(b * Hkv + kvh)) * n_tok + tok) * hd + j]; } };
+        std::vector<double> att = host_attention(g, Qd, T, before);
+        att = host_rotate(att, rows * H, hd, mha.v_rotation_trans);
+        const std::vector<double> want = host_linear(wo, att, rows);
+        double worst = 0.0;
+        const bool ok = attn_close(y->to_vector(), want, &worst);
+        if (!ok) {
+            std::printf("    coder %d bits %d T %u before %u: worst abs err %.3e\n", (int)coder, bits, T, before, worst);
+        }
+        REQUIRE(ok);
+        before += T;
+    }
+
+    // the cached rows are the coder's image of the rotated projections: compare one pair with the CPU checker
+    if (coder == KV_UNIFORM) {
+        mha.k_qcache.sync_packed();
+        REQUIRE(mha.k_qcache.packed.size() == (size_t)B * Hkv * before * (size_t)wo_words_per_row((int)hd, bits));
+        REQUIRE(mha.k_qcache.block_scale > 0.0f);
+        REQUIRE(mha.k_qcache.outer == B * Hkv * before);
+    }
+
+    // lifecycle (include/modules/multihead_attention.hpp:138-149)
+    const std::vector<real1> big = gaussian((size_t)B * 30U * dm, seed + 7U);
+    REQUIRE_THROWS_AS(mha.forward(std::make_shared<Tensor>(big, std::vector<tcapint>{ B, 30U, dm }, false, TEST_DTAG)),
+        std::out_of_range);
+    REQUIRE_THROWS_AS(mha.forward(std::make_shared<Tensor>(gaussian(3U * dm, 1U), std::vector<tcapint>{ 3U, 1U, dm }, false, TEST_DTAG)),
+        std::invalid_argument);
+    mha.reset_cache();
+    REQUIRE(mha.cache_len == 0U);
+    REQUIRE(mha.max_seq_len == 0U);
+    REQUIRE(mha.k_rotation.empty());
+    REQUIRE(mha.k_qcache.d == 0U);
+    TensorPtr y = mha.forward(std::make_shared<Tensor>(gaussian(3U * dm, 1U), std::vector<tcapint>{ 3U, 1U, dm }, false, TEST_DTAG));
+    REQUIRE(y->shape == (std::vector<tcapint>{ 3U, 1U, dm }));
+    REQUIRE(mha.max_seq_len == 2048U); // the reference's default capacity without RoPE (cpp:173)
+}
+
+TEST_CASE(test_attention_uniform_4bit, true) { run_attention_case(KV_UNIFORM, 4, false, 1234U); }
+TEST_CASE(test_attention_uniform_3bit_blocked_gqa, true) { run_attention_case(KV_UNIFORM, 3, true, 99U); }
+TEST_CASE(test_attention_lloydmax, true) { run_attention_case(KV_LLOYDMAX, 4, false, 4321U); }
+
+TEST_CASE(test_attention_uniform_codes_follow_reference_coder, true)
+{
+    // one call, B = 1, H = Hkv = 1, identity projections: the cached words must be exactly what the reference's
+    // write_row makes of x.R (rotation in ascending order, sequential block scale), i.e. the CPU checker's words
+    const tcapint T = 9U, hd = 64U;
+    MultiHeadAttention mha(hd, 1U, 1U, hd, TEST_DTAG, nullptr, ZERO_R1, -1, true, 4, false);
+    mha.rotation_seed = 5U;
+    std::vector<real1> eye((size_t)hd * hd, 0.0f);
+    for (tcapint i = 0; i < hd; ++i) {
+        eye[i + (size_t)hd * i] = 1.0f;
+    }
+    for (const LinearPtr &l : { mha.W_q, mha.W_k, mha.W_v, mha.W_o }) {
+        l->weight = std::make_shared<Parameter>(eye, std::vector<tcapint>{ hd, hd }, true, TEST_DTAG);
+    }
+    const std::vector<real1> xv = gaussian((size_t)T * hd, 77U); // (1, T, hd) column-major: row t is x[t + T*i]
+    mha.forward(std::make_shared<Tensor>(xv, std::vector<tcapint>{ 1U, T, hd }, false, TEST_DTAG));
+    std::vector<real1> rows((size_t)T * hd), rot((size_t)T * hd);
+    for (tcapint t = 0; t < T; ++t) {
+        for (tcapint i = 0; i < hd; ++i) {
+            rows[(size_t)t * hd + i] = xv[t + (size_t)T * i];
+        }
+    }
+    for (int which = 0; which < 2; ++which) {
+        QuantizedKVCache &qc = which ? mha.v_qcache : mha.k_qcache;
+        wo_apply_rotation(rows.data(), T, (int)hd, (which ? mha.v_rotation : mha.k_rotation).data(), rot.data());
+        // the module sums squares in the memory order of its (B, T, heads, hd) tensor: i-major, t-minor
+        std::vector<real1> flat((size_t)T * hd);
+        for (tcapint t = 0; t < T; ++t) {
+            for (tcapint i = 0; i < hd; ++i) {
+                flat[t + (size_t)T * i] = rot[(size_t)t * hd + i];
+            }
+        }
+        const real1 scale = wo_block_scale(flat.data(), flat.size());
+        REQUIRE(std::fabs(qc.block_scale - scale) <= 2e-7f * scale);
+        std::vector<int32_t> want((size_t)T * wo_words_per_row((int)hd, 4), 0);
+        wo_uniform_write_rows(want.data(), rot.data(), T, (int)hd, 4, qc.block_scale);
+        qc.sync_packed();
+        REQUIRE(qc.packed.size() == want.size());
+        REQUIRE(std::memcmp(qc.packed.data(), want.data(), want.size() * sizeof(int32_t)) == 0);
+    }
+}
+
+TEST_CASE(test_attention_dense_path_matches_quantized_at_fine_steps, true)
+{
+    // float cache (kv_quant_bits = 0) and no cache: the reference's own sequence of dense ops, on the device.
+    // Incremental calls must equal one call over the whole sequence, and both must equal float64 attention.
+    const tcapint B = 2U, dm = 48U, H = 4U, Hkv = 2U, hd = 16U, T = 6U;
+    MultiHeadAttention cached(dm, H, Hkv, hd, TEST_DTAG, nullptr, ZERO_R1, -1, true, 0);
+    MultiHeadAttention oneshot(dm, H, Hkv, hd, TEST_DTAG, nullptr, ZERO_R1, -1, false, 0);
+    cached.set_max_kv_seq_len(16U);
+    const HostLinear wq = install(cached.W_q, 1U), wk = install(cached.W_k, 2U), wv = install(cached.W_v, 3U),
+                     wo = install(cached.W_o, 4U);
+    install(oneshot.W_q, 1U);
+    install(oneshot.W_k, 2U);
+    install(oneshot.W_v, 3U);
+    install(oneshot.W_o, 4U);
+    const std::vector<real1> xv = gaussian((size_t)B * T * dm, 55U);
+    TensorPtr x = std::make_shared<Tensor>(xv, std::vector<tcapint>{ B, T, dm }, false, TEST_DTAG);
+    const std::vector<real1> whole = oneshot.forward(x)->to_vector();
+
+    const size_t rows = (size_t)B * T;
+    const std::vector<double> Qd = host_linear(wq, to_double(xv), rows), Kd = host_linear(wk, to_double(xv), rows),
+                              Vd = host_linear(wv, to_double(xv), rows);
+    AttnCheck g{ B, H, Hkv, hd, false,
+        [&](tcapint b, tcapint kvh, tcapint tok, tcapint j) { return Kd[b + (size_t)B * (tok + (size_t)T * (kvh + (size_t)Hkv * j))]; },
+        [&](tcapint b, tcapint kvh, tcapint tok, tcapint j) { return Vd[b + (size_t)B * (tok + (size_t)T * (kvh + (size_t)Hkv * j))]; } };
+    const std::vector<double> want = host_linear(wo, host_attention(g, Qd, T, 0U), rows);
+    REQUIRE(attn_close(whole, want));
+
+    // prefill 4 tokens, then 2 single-token steps, against the matching slices of the one-shot result
+    std::vector<real1> pieces(whole.size());
+    tcapint done = 0U;
+    for (const tcapint step : { 4U, 1U, 1U }) {
+        TensorPtr xs = Tensor::contiguous(Tensor::slice(x, 1, done, step));
+        const std::vector<real1> ys = cached.forward(xs)->to_vector(); // (B, step, dm)
+        for (tcapint f = 0; f < dm; ++f) {
+            for (tcapint t = 0; t < step; ++t) {
+                for (tcapint b = 0; b < B; ++b) {
+                    pieces[b + (size_t)B * ((done + t) + (size_t)T * f)] = ys[b + (size_t)B * (t + (size_t)step * f)];
+                }
+            }
+        }
+        done += step;
+    }
+    REQUIRE(attn_close(pieces, want));
+    REQUIRE(cached.cache_len == T);
+}
+
+} // namespace
+
+int main(int argc, char **argv)
+{
+    bool gpu = true;
+    const char *filter = nullptr;
+    for (int i = 1; i < argc; ++i) {
+        if (!std::strcmp(argv[i], "--no-gpu")) {
+            gpu = false;
+        } else {
+            filter = argv[i];
+        }
+    }
+    int ran = 0, failed_cases = 0;
+    for (const Case &c : cases()) {
+        if ((c.needs_gpu && !gpu) || (filter && !std::strstr(c.name, filter))) {
+            continue;
+        }
+        std::printf("[ RUN  ] %s\n", c.name);
+        std::fflush(stdout);
+        const int before = failures;
+        try {
+            c.body();
+        } catch (const std::exception &e) {
+            std::printf("    FAILED: unexpected exception: %s\n", e.what());
+            ++failures;
+        }
+        ++ran;
+        if (failures != before) {
+            ++failed_cases;
+            std::printf("[ FAIL ] %s\n", c.name);
+        } else {
+            std::printf("[  OK  ] %s\n", c.name);
+        }
+        std::fflush(stdout);
+    }
+    if (gpu) {
+        HipDevice::Instance().finish();
+    }
+    std::printf("%d case(s) run, %d failed\n", ran, failed_cases);
+    return failed_cases ? 1 : 0;
+}

@@ -172,3 +172,41 @@ def test_softmax_on_a_view_with_offset(gpu, oracle):
     e = np.exp(x - x.max(axis=1, keepdims=True))
     np.testing.assert_allclose(out[1:5, 3:35:2].cpu().numpy(), e / e.sum(axis=1, keepdims=True), rtol=2e-5, atol=1e-7)
     assert torch.all(out[0] == 7.0) and torch.all(out[:, 4::2] == 7.0)
+
+
+def test_elementwise_broadcast_and_gather(gpu):
+    """add / sub / mul / div are single IEEE operations, so they must equal numpy bit for bit, including with a
+    broadcast (stride 0) operand, transposed views and an output that aliases the first operand."""
+    import torch
+    rng = np.random.default_rng(9)
+    a = rng.standard_normal((5, 7, 3), dtype=np.float32)
+    b = rng.standard_normal((1, 7, 1), dtype=np.float32) + 3.0
+    ad, bd = col_major(a), dev(b)
+    for op, fn in ((gpu.EW_ADD, np.add), (gpu.EW_SUB, np.subtract), (gpu.EW_MUL, np.multiply), (gpu.EW_DIV, np.divide)):
+        out = torch.zeros((5, 7, 3), device="cuda")
+        gpu.elementwise(op, ad, bd, out)
+        np.testing.assert_array_equal(out.cpu().numpy(), fn(a, b))
+    # strided gather: a transposed view copied into a contiguous tensor (Tensor::contiguous)
+    out = torch.zeros((3, 5, 7), device="cuda")
+    gpu.elementwise(gpu.EW_COPY, ad.permute(2, 0, 1), None, out)
+    np.testing.assert_array_equal(out.cpu().numpy(), a.transpose(2, 0, 1))
+    # in place: a += b
+    acc = dev(a.copy())
+    gpu.elementwise(gpu.EW_ADD, acc, bd, acc)
+    np.testing.assert_array_equal(acc.cpu().numpy(), a + b)
+    # scalar division as attention uses it: scores / sqrt(d)
+    s = dev(np.array([np.sqrt(np.float32(128.0))], dtype=np.float32))
+    out = torch.zeros((5, 7, 3), device="cuda")
+    gpu.elementwise(gpu.EW_DIV, ad, s.reshape(1, 1, 1), out)
+    np.testing.assert_array_equal(out.cpu().numpy(), a / np.sqrt(np.float32(128.0)))
+
+
+@pytest.mark.parametrize("rows,cols,diag", [(1, 1, 1), (4, 4, 1), (5, 9, 1), (9, 5, 0), (6, 6, 3)])
+def test_triu_fill_against_checker(gpu, oracle, rows, cols, diag):
+    rng = np.random.default_rng(10)
+    a = rng.standard_normal((rows, cols), dtype=np.float32)
+    ad = col_major(a)
+    gpu.triu_fill(ad, -1.701411835e38, diag)
+    want = np.asfortranarray(a).ravel(order="F").copy()
+    oracle.triu_fill(want, 0, rows, cols, 1, rows, -1.701411835e38, diag)
+    np.testing.assert_array_equal(ad.cpu().numpy(), want.reshape((rows, cols), order="F"))

@@ -239,3 +239,18 @@ def test_argument_errors_are_reported_not_faulted(gpu):
     with pytest.raises(gpu.WeedHipError):
         cache.decode_attn(q, torch.zeros_like(q))  # 3 query heads over 2 kv heads
     cache.close()
+
+
+def test_apply_rotation_reference_order(gpu, oracle):
+    """y = x.R over the last dimension of a strided tensor, in the reference's summation order: bit-exact against the
+    checker's naive loop."""
+    import torch
+    rng = np.random.default_rng(77)
+    d = 64
+    R = oracle.orthonormalize_columns(rng.normal(size=d * d).astype(np.float32))
+    x = rng.standard_normal((3, 2, 5, d), dtype=np.float32)
+    xd = col_major(x)
+    out = torch.zeros_like(xd)
+    gpu.apply_rotation(xd, dev(R), out)
+    want = oracle.apply_rotation(x.reshape(-1, d), R).reshape(x.shape)
+    np.testing.assert_array_equal(out.cpu().numpy(), want)

@@ -30,3 +30,16 @@ def build_library(force=True, jobs=8, verbose=False):
     if not os.path.exists(_LIB):
         raise RuntimeError("make succeeded but %s is missing" % _LIB)
     return _LIB
+
+
+def build_host(force=True, verbose=False):
+    """Compile the host C++ mirror (weed_amd/host) into libweed_host.so; needs libweed_hip.so to link against."""
+    host = os.path.join(_HERE, "host")
+    if force:
+        subprocess.run(["make", "-C", host, "clean"], check=True, stdout=subprocess.DEVNULL)
+    proc = subprocess.run(["make", "-C", host, "all"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if verbose or proc.returncode:
+        print(proc.stdout)
+    if proc.returncode:
+        raise RuntimeError("building libweed_host.so failed (exit %d)" % proc.returncode)
+    return _HOST_LIB

@@ -53,11 +53,16 @@ SIGNATURES = {
     "weed_hip_matmul_f32": (c_int, [c_uint32, c_uint32, c_uint32, c_void_p, c_uint32, c_uint32, c_uint32, c_void_p,
                                     c_uint32, c_uint32, c_uint32, c_void_p, c_uint32, c_uint32, c_uint32]),
     "weed_hip_copy_f32": (c_int, [c_uint64, c_void_p, c_uint32, c_uint32, c_void_p, c_uint32, c_uint32]),
+    "weed_hip_elementwise_f32": (c_int, [c_int, c_uint32, U32P, c_void_p, c_uint32, U32P, c_void_p, c_uint32, U32P,
+                                         c_void_p, c_uint32, U32P]),
+    "weed_hip_triu_fill_f32": (c_int, [c_uint32, c_uint32, c_float, c_uint32, c_void_p, c_uint32, c_uint32, c_uint32]),
     "weed_hip_softmax_f32": (c_int, [c_uint32, U32P, c_uint32, c_void_p, c_uint32, U32P, c_void_p, c_uint32, U32P]),
     "weed_hip_reduce_f32": (c_int, [c_int, c_uint32, U32P, c_uint32, c_void_p, c_uint32, U32P, c_void_p, c_uint32,
                                     U32P]),
     "weed_hip_make_rotation": (c_int, [c_uint32, c_uint32, c_void_p]),
     "weed_hip_orthonormalize_columns": (c_int, [c_uint32, c_void_p]),
+    "weed_hip_apply_rotation_f32": (c_int, [c_uint32, c_void_p, c_uint32, U32P, c_void_p, c_uint32, U32P, c_void_p,
+                                            c_uint32, U32P]),
     "weed_hip_kv_cache_create": (c_int, [POINTER(c_void_p), POINTER(KVConfig)]),
     "weed_hip_kv_cache_destroy": (c_int, [c_void_p]),
     "weed_hip_kv_cache_reset": (c_int, [c_void_p, c_int]),
@@ -240,6 +245,26 @@ def copy(a, out):
                                    out.stride(0)))
 
 
+EW_COPY, EW_ADD, EW_SUB, EW_MUL, EW_DIV = range(5)
+
+
+def elementwise(op, a, b, out):
+    """out = a (op) b on torch views; a and b are expanded (stride 0) to out's shape."""
+    a = a.expand(out.shape)
+    bp, bs = None, u32(out.stride())
+    if b is not None:
+        b = b.expand(out.shape)
+        bp, bs = c_void_p(b.data_ptr()), u32(b.stride())
+    check(load().weed_hip_elementwise_f32(op, out.dim(), u32(out.shape), c_void_p(a.data_ptr()), 0, u32(a.stride()),
+                                          bp, 0, bs, c_void_p(out.data_ptr()), 0, u32(out.stride())))
+
+
+def triu_fill(a, val, diagonal=1):
+    rows, cols = a.shape
+    check(load().weed_hip_triu_fill_f32(rows, cols, val, diagonal, c_void_p(a.data_ptr()), 0, a.stride(0),
+                                        a.stride(1)))
+
+
 def softmax(a, out, axis):
     assert a.shape == out.shape
     check(load().weed_hip_softmax_f32(a.dim(), u32(a.shape), axis, c_void_p(a.data_ptr()), 0, u32(a.stride()),
@@ -256,6 +281,13 @@ def reduce(op, a, out, axis):
 
 def make_rotation(seed, d, out):
     check(load().weed_hip_make_rotation(seed, d, c_void_p(out.data_ptr())))
+
+
+def apply_rotation(x, r, out):
+    """out = x . r over the last dimension of torch views x / out (same shape); r is d x d column-major."""
+    d = x.shape[-1]
+    check(load().weed_hip_apply_rotation_f32(d, c_void_p(r.data_ptr()), x.dim(), u32(x.shape), c_void_p(x.data_ptr()),
+                                             0, u32(x.stride()), c_void_p(out.data_ptr()), 0, u32(out.stride())))
 
 
 def orthonormalize_columns(d, r):

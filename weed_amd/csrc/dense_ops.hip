@@ -152,6 +152,57 @@ __global__ void __launch_bounds__(256) copy_kernel(const float *__restrict__ a, 
     }
 }
 
+struct PointGeom {
+    uint32_t rank;
+    uint32_t shape[kMaxRank];
+    uint32_t a_stride[kMaxRank];
+    uint32_t b_stride[kMaxRank];
+    uint32_t o_stride[kMaxRank];
+    uint32_t a_off, b_off, o_off;
+    uint64_t n;
+};
+
+// One thread per logical element, dimension 0 fastest (the contiguous direction of column-major tensors).
+template <int OP> __global__ void __launch_bounds__(256) elementwise_kernel(const float *__restrict__ a,
+                                                                            const float *__restrict__ b, float *out,
+                                                                            PointGeom g)
+{
+    const uint64_t step = (uint64_t)gridDim.x * blockDim.x;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < g.n; i += step) {
+        uint64_t tmp = i, ai = g.a_off, bi = g.b_off, oi = g.o_off;
+        for (uint32_t dd = 0; dd < g.rank; ++dd) {
+            const uint32_t dim = g.shape[dd];
+            const uint32_t c = (uint32_t)(tmp % dim);
+            tmp /= dim;
+            ai += (uint64_t)c * g.a_stride[dd];
+            bi += (uint64_t)c * g.b_stride[dd];
+            oi += (uint64_t)c * g.o_stride[dd];
+        }
+        const float x = a[ai];
+        float r;
+        if (OP == 0) {
+            r = x;
+        } else {
+            const float y = b[bi];
+            r = OP == 1 ? x + y : OP == 2 ? x - y : OP == 3 ? x * y : x / y;
+        }
+        out[oi] = r;
+    }
+}
+
+__global__ void __launch_bounds__(256) triu_fill_kernel(float *a, uint32_t rows, uint32_t cols, float val,
+                                                        uint32_t diagonal, uint32_t a_off, uint32_t s0, uint32_t s1)
+{
+    const uint64_t n = (uint64_t)rows * cols;
+    const uint64_t step = (uint64_t)gridDim.x * blockDim.x;
+    for (uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n; idx += step) {
+        const uint32_t i = (uint32_t)(idx % rows), j = (uint32_t)(idx / rows);
+        if ((uint64_t)i + diagonal <= j) {
+            a[(uint64_t)a_off + (uint64_t)i * s0 + (uint64_t)j * s1] = val;
+        }
+    }
+}
+
 int make_geom(const char *fn, uint32_t rank, const uint32_t *shape, uint32_t axis, uint32_t a_off,
               const uint32_t *a_stride, uint32_t o_off, const uint32_t *o_stride, bool out_keeps_axis, AxisGeom &g)
 {
@@ -193,6 +244,70 @@ int weed_hip_copy_f32(uint64_t n, const float *a_dev, uint32_t a_off, uint32_t a
     ProfileScope prof("copy");
     const uint32_t blocks = (uint32_t)std::min<uint64_t>((n + 255) / 256, 256u * 64u);
     copy_kernel<<<blocks, 256, 0, stream()>>>(a_dev, out_dev, n, a_off, a_stride, o_off, o_stride);
+    WEED_HIP_LAUNCH_CHECK();
+    return WEED_HIP_OK;
+}
+
+int weed_hip_elementwise_f32(int op, uint32_t rank, const uint32_t *shape, const float *a_dev, uint32_t a_off,
+                             const uint32_t *a_stride, const float *b_dev, uint32_t b_off, const uint32_t *b_stride,
+                             float *out_dev, uint32_t o_off, const uint32_t *o_stride)
+{
+    const char *fn = "weed_hip_elementwise_f32";
+    WEED_HIP_REQUIRE(op >= WEED_HIP_EW_COPY && op <= WEED_HIP_EW_DIV, "%s: unknown op %d", fn, op);
+    WEED_HIP_REQUIRE(a_dev && out_dev && shape && a_stride && o_stride, "%s: null pointer", fn);
+    WEED_HIP_REQUIRE(op == WEED_HIP_EW_COPY || (b_dev && b_stride), "%s: null second operand", fn);
+    WEED_HIP_REQUIRE(rank >= 1 && rank <= (uint32_t)kMaxRank, "%s: rank %u outside [1, %d]", fn, rank, kMaxRank);
+    WEED_HIP_TRY(ensure_init());
+    PointGeom g;
+    g.rank = rank;
+    g.a_off = a_off;
+    g.b_off = b_off;
+    g.o_off = o_off;
+    g.n = 1;
+    for (uint32_t i = 0; i < rank; ++i) {
+        WEED_HIP_REQUIRE(shape[i] > 0, "%s: dimension %u is empty", fn, i);
+        g.shape[i] = shape[i];
+        g.a_stride[i] = a_stride[i];
+        g.b_stride[i] = op == WEED_HIP_EW_COPY ? 0 : b_stride[i];
+        g.o_stride[i] = o_stride[i];
+        g.n *= shape[i];
+    }
+    WEED_HIP_REQUIRE(g.n < (1ull << 32), "%s: more than 2^32 elements", fn);
+    ProfileScope prof("elementwise");
+    const uint32_t blocks = (uint32_t)std::min<uint64_t>((g.n + 255) / 256, 256u * 64u);
+    const float *b = op == WEED_HIP_EW_COPY ? a_dev : b_dev;
+    switch (op) {
+    case WEED_HIP_EW_COPY:
+        elementwise_kernel<0><<<blocks, 256, 0, stream()>>>(a_dev, b, out_dev, g);
+        break;
+    case WEED_HIP_EW_ADD:
+        elementwise_kernel<1><<<blocks, 256, 0, stream()>>>(a_dev, b, out_dev, g);
+        break;
+    case WEED_HIP_EW_SUB:
+        elementwise_kernel<2><<<blocks, 256, 0, stream()>>>(a_dev, b, out_dev, g);
+        break;
+    case WEED_HIP_EW_MUL:
+        elementwise_kernel<3><<<blocks, 256, 0, stream()>>>(a_dev, b, out_dev, g);
+        break;
+    default:
+        elementwise_kernel<4><<<blocks, 256, 0, stream()>>>(a_dev, b, out_dev, g);
+        break;
+    }
+    WEED_HIP_LAUNCH_CHECK();
+    return WEED_HIP_OK;
+}
+
+int weed_hip_triu_fill_f32(uint32_t rows, uint32_t cols, float val, uint32_t diagonal, float *a_dev, uint32_t a_off,
+                           uint32_t a_s0, uint32_t a_s1)
+{
+    WEED_HIP_REQUIRE(a_dev, "weed_hip_triu_fill_f32: null pointer");
+    WEED_HIP_TRY(ensure_init());
+    const uint64_t n = (uint64_t)rows * cols;
+    if (!n) {
+        return WEED_HIP_OK;
+    }
+    const uint32_t blocks = (uint32_t)std::min<uint64_t>((n + 255) / 256, 256u * 64u);
+    triu_fill_kernel<<<blocks, 256, 0, stream()>>>(a_dev, rows, cols, val, diagonal, a_off, a_s0, a_s1);
     WEED_HIP_LAUNCH_CHECK();
     return WEED_HIP_OK;
 }

@@ -63,6 +63,45 @@ __global__ void __launch_bounds__(256) gram_schmidt_kernel(float *r, uint32_t d)
     }
 }
 
+constexpr int kRotMaxRank = 8;
+struct RotGeom {
+    uint32_t rank; // the last dimension is the rotated one
+    uint32_t shape[kRotMaxRank];
+    uint32_t x_stride[kRotMaxRank];
+    uint32_t o_stride[kRotMaxRank];
+    uint32_t x_off, o_off;
+    uint32_t rows, d;
+};
+
+// y[row, j] = sum_i x[row, i] * R[i + d*j], products added in ascending i with separate multiply and add, the order
+// of the reference's naive matmul (src/ops/matmul.cpp:40-44).  Neighbouring threads take neighbouring rows (the
+// contiguous direction of a column-major tensor) and share one column of R, so x loads coalesce and R loads are
+// wave-uniform.
+__global__ void __launch_bounds__(256) apply_rotation_kernel(const float *__restrict__ x, const float *__restrict__ rot,
+                                                             float *__restrict__ out, RotGeom g)
+{
+    const uint32_t row = blockIdx.x * 256 + threadIdx.x;
+    const uint32_t j = blockIdx.y;
+    if (row >= g.rows) {
+        return;
+    }
+    uint64_t xb = g.x_off, ob = g.o_off;
+    uint32_t tmp = row;
+    for (uint32_t dd = 0; dd + 1 < g.rank; ++dd) {
+        const uint32_t c = tmp % g.shape[dd];
+        tmp /= g.shape[dd];
+        xb += (uint64_t)c * g.x_stride[dd];
+        ob += (uint64_t)c * g.o_stride[dd];
+    }
+    const uint32_t xs = g.x_stride[g.rank - 1];
+    const float *col = rot + (uint64_t)j * g.d;
+    float acc = 0.0f;
+    for (uint32_t i = 0; i < g.d; ++i) {
+        acc = acc + x[xb + (uint64_t)i * xs] * col[i];
+    }
+    out[ob + (uint64_t)j * g.o_stride[g.rank - 1]] = acc;
+}
+
 } // namespace
 
 extern "C" {
@@ -93,6 +132,38 @@ int weed_hip_make_rotation(uint32_t seed, uint32_t d, float *r_dev)
     WEED_HIP_CHECK(hipMemcpyAsync(r_dev, host.data(), sizeof(float) * host.size(), hipMemcpyHostToDevice, stream()));
     WEED_HIP_CHECK(hipStreamSynchronize(stream()));
     return weed_hip_orthonormalize_columns(d, r_dev);
+}
+
+int weed_hip_apply_rotation_f32(uint32_t d, const float *r_dev, uint32_t rank, const uint32_t *shape,
+                                const float *x_dev, uint32_t x_off, const uint32_t *x_stride, float *out_dev,
+                                uint32_t o_off, const uint32_t *o_stride)
+{
+    const char *fn = "weed_hip_apply_rotation_f32";
+    WEED_HIP_REQUIRE(r_dev && x_dev && out_dev && shape && x_stride && o_stride, "%s: null pointer", fn);
+    WEED_HIP_REQUIRE(x_dev != out_dev, "%s: cannot rotate in place", fn);
+    WEED_HIP_REQUIRE(rank >= 1 && rank <= (uint32_t)kRotMaxRank, "%s: rank %u outside [1, %d]", fn, rank, kRotMaxRank);
+    WEED_HIP_REQUIRE(d >= 1 && d <= 65535 && shape[rank - 1] == d, "%s: the last dimension must be d = %u", fn, d);
+    WEED_HIP_TRY(ensure_init());
+    RotGeom g;
+    g.rank = rank;
+    g.d = d;
+    g.x_off = x_off;
+    g.o_off = o_off;
+    uint64_t rows = 1;
+    for (uint32_t i = 0; i < rank; ++i) {
+        WEED_HIP_REQUIRE(shape[i] > 0, "%s: dimension %u is empty", fn, i);
+        g.shape[i] = shape[i];
+        g.x_stride[i] = x_stride[i];
+        g.o_stride[i] = o_stride[i];
+        if (i + 1 < rank) {
+            rows *= shape[i];
+        }
+    }
+    WEED_HIP_REQUIRE(rows * d < (1ull << 32), "%s: more than 2^32 elements", fn);
+    g.rows = (uint32_t)rows;
+    apply_rotation_kernel<<<dim3((g.rows + 255) / 256, d), 256, 0, stream()>>>(x_dev, r_dev, out_dev, g);
+    WEED_HIP_LAUNCH_CHECK();
+    return WEED_HIP_OK;
 }
 
 } // extern "C"

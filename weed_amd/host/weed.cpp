@@ -1,0 +1,1163 @@
+// Host-side mirror of Weed's tensor / op / module interface over the HIP device library (see weed.hpp).
+#include "weed.hpp"
+
+#include "weed_hip.h"
+
+#include <algorithm>
+#include <cmath>
+#include <random>
+
+namespace Weed {
+
+// ---------------------------------------------------------------------------------------------------------
+// device
+// ---------------------------------------------------------------------------------------------------------
+
+HipDevice::HipDevice()
+    : device_id(0)
+{
+    check(weed_hip_init(0));
+    char buf[256] = { 0 };
+    if (weed_hip_device_name(buf, sizeof(buf)) == WEED_HIP_OK) {
+        name = buf;
+    }
+}
+
+HipDevice &HipDevice::Instance()
+{
+    static HipDevice dev;
+    return dev;
+}
+
+void HipDevice::check(int status)
+{
+    if (status == WEED_HIP_OK) {
+        return;
+    }
+    const std::string msg = weed_hip_last_error();
+    switch (status) {
+    case WEED_HIP_EINVAL:
+        throw std::invalid_argument(msg);
+    case WEED_HIP_ENOMEM:
+        throw bad_alloc(msg);
+    case WEED_HIP_ECAPACITY:
+        throw std::out_of_range(msg);
+    default:
+        throw std::runtime_error(msg);
+    }
+}
+
+void HipDevice::finish()
+{
+    std::lock_guard<std::recursive_mutex> lock(mutex);
+    check(weed_hip_sync());
+}
+
+namespace {
+
+typedef std::lock_guard<std::recursive_mutex> DeviceLock;
+#define WEED_DEVICE_LOCK() DeviceLock device_lock(HipDevice::Instance().mutex)
+
+DeviceTag resolve(DeviceTag dtag) { return (dtag == CPU) ? CPU : GPU; }
+
+real1 *device_ptr(const Tensor &t, const char *who)
+{
+    if (!t.storage) {
+        throw std::invalid_argument(std::string(who) + ": tensor has no storage");
+    }
+    if (t.storage->dtype != DType::REAL) {
+        throw std::invalid_argument(std::string(who) + ": only real tensors are supported");
+    }
+    if (t.storage->device != GPU) {
+        throw std::domain_error(std::string(who) + ": this build computes on the GPU only; move the tensor with cast(GPU)");
+    }
+    return static_cast<GpuRealStorage *>(t.storage.get())->buffer;
+}
+
+void validate_all_same_device(std::initializer_list<const Tensor *> ts, const char *who)
+{
+    DeviceTag d = NONE_DEVICE;
+    for (const Tensor *t : ts) {
+        if (!t->storage) {
+            throw std::invalid_argument(std::string(who) + ": tensor has no storage");
+        }
+        if (d == NONE_DEVICE) {
+            d = t->storage->device;
+        } else if (d != t->storage->device) {
+            throw std::invalid_argument(std::string("Tensor device mismatch in ") + who + "!");
+        }
+    }
+}
+
+symint wrap_axis(symint axis, size_t rank, const char *who)
+{
+    if (axis < 0) {
+        axis += (symint)rank;
+    }
+    if (axis < 0 || (size_t)axis >= rank) {
+        throw std::invalid_argument(std::string(who) + ": axis out of range");
+    }
+    return axis;
+}
+
+TensorPtr allocate(const std::vector<tcapint> &shape, const Tensor &like)
+{
+    return std::make_shared<Tensor>(shape, Tensor::full_contiguous_stride(shape), false, false, DType::REAL,
+        like.storage->device, like.storage->get_device_id());
+}
+
+void elementwise(int op, const Tensor &a, const Tensor *b, Tensor &out, const char *who)
+{
+    // operands are right-aligned against out's shape; a dimension of size 1 repeats (stride 0)
+    const size_t rank = out.shape.size();
+    if (rank > 8U) {
+        throw std::invalid_argument(std::string(who) + ": rank above 8");
+    }
+    auto aligned = [&](const Tensor &t, std::vector<uint32_t> &str) {
+        if (t.shape.size() > rank) {
+            throw std::invalid_argument(std::string(who) + ": operand rank exceeds output rank");
+        }
+        const size_t pad = rank - t.shape.size();
+        str.assign(rank, 0U);
+        for (size_t i = 0; i < t.shape.size(); ++i) {
+            if (t.shape[i] == out.shape[pad + i]) {
+                str[pad + i] = (t.shape[i] == 1U) ? 0U : t.stride[i];
+            } else if (t.shape[i] != 1U) {
+                throw std::invalid_argument(std::string(who) + ": shapes cannot be broadcast together");
+            }
+        }
+    };
+    std::vector<uint32_t> as, bs, os(rank);
+    aligned(a, as);
+    if (b) {
+        aligned(*b, bs);
+    }
+    for (size_t i = 0; i < rank; ++i) {
+        os[i] = (out.shape[i] == 1U) ? 0U : out.stride[i];
+    }
+    real1 *ap = device_ptr(a, who), *op_ = device_ptr(out, who);
+    real1 *bp = b ? device_ptr(*b, who) : nullptr;
+    WEED_DEVICE_LOCK();
+    HipDevice::check(weed_hip_elementwise_f32(op, (uint32_t)rank, out.shape.data(), ap, a.offset, as.data(), bp,
+        b ? b->offset : 0U, b ? bs.data() : nullptr, op_, out.offset, os.data()));
+}
+
+std::vector<tcapint> broadcast_shape(const Tensor &a, const Tensor &b, const char *who)
+{
+    const size_t rank = std::max(a.shape.size(), b.shape.size());
+    std::vector<tcapint> shp(rank, 1U);
+    for (const Tensor *t : { &a, &b }) {
+        const size_t pad = rank - t->shape.size();
+        for (size_t i = 0; i < t->shape.size(); ++i) {
+            tcapint &o = shp[pad + i];
+            if (o == 1U) {
+                o = t->shape[i];
+            } else if (t->shape[i] != 1U && t->shape[i] != o) {
+                throw std::invalid_argument(std::string(who) + ": shapes cannot be broadcast together");
+            }
+        }
+    }
+    return shp;
+}
+
+TensorPtr binary(int op, const TensorPtr &a, const TensorPtr &b, const char *who)
+{
+    validate_all_same_device({ a.get(), b.get() }, who);
+    TensorPtr out = allocate(broadcast_shape(*a, *b, who), *a);
+    elementwise(op, *a, b.get(), *out, who);
+    return out;
+}
+
+} // namespace
+
+// ---------------------------------------------------------------------------------------------------------
+// storage
+// ---------------------------------------------------------------------------------------------------------
+
+Storage::Storage(StorageType stp, DeviceTag dtg, DType dtp, tcapint n)
+    : stype(stp)
+    , device(dtg)
+    , dtype(dtp)
+    , size(n)
+{
+    if (!size) {
+        throw std::invalid_argument("Storage must have size of at least 1!");
+    }
+}
+
+CpuRealStorage::CpuRealStorage(tcapint n)
+    : RealStorage(REAL_CPU_DENSE, CPU, DType::REAL, n)
+    , data(n)
+{
+}
+
+CpuRealStorage::CpuRealStorage(const std::vector<real1> &val)
+    : RealStorage(REAL_CPU_DENSE, CPU, DType::REAL, (tcapint)val.size())
+    , data(val)
+{
+}
+
+real1 CpuRealStorage::operator[](const tcapint &idx) const
+{
+    if (idx >= size) {
+        throw std::invalid_argument("CpuStorage::operator[] argument out-of-bounds!");
+    }
+    return data[idx];
+}
+
+void CpuRealStorage::write(const tcapint &idx, const real1 &val)
+{
+    if (idx >= size) {
+        throw std::invalid_argument("CpuStorage::write argument out-of-bounds!");
+    }
+    data[idx] = val;
+}
+
+void CpuRealStorage::add(const tcapint &idx, const real1 &val) { write(idx, (*this)[idx] + val); }
+void CpuRealStorage::FillZeros() { std::fill(data.begin(), data.end(), ZERO_R1); }
+void CpuRealStorage::FillOnes() { std::fill(data.begin(), data.end(), ONE_R1); }
+void CpuRealStorage::FillValue(const real1 &v) { std::fill(data.begin(), data.end(), v); }
+StoragePtr CpuRealStorage::gpu(int64_t did) { return std::make_shared<GpuRealStorage>(data, did); }
+
+GpuRealStorage::GpuRealStorage(tcapint n, int64_t did_)
+    : RealStorage(REAL_GPU_DENSE, GPU, DType::REAL, n)
+    , buffer(nullptr)
+    , did(did_ < 0 ? HipDevice::Instance().device_id : did_)
+{
+    WEED_DEVICE_LOCK();
+    void *p = nullptr;
+    HipDevice::check(weed_hip_malloc(&p, sizeof(real1) * (size_t)n));
+    buffer = static_cast<real1 *>(p);
+}
+
+GpuRealStorage::GpuRealStorage(const std::vector<real1> &val, int64_t did_)
+    : GpuRealStorage((tcapint)val.size(), did_)
+{
+    WEED_DEVICE_LOCK();
+    HipDevice::check(weed_hip_memcpy_h2d(buffer, val.data(), sizeof(real1) * val.size()));
+}
+
+GpuRealStorage::~GpuRealStorage()
+{
+    if (buffer) {
+        WEED_DEVICE_LOCK();
+        (void)weed_hip_free(buffer);
+    }
+}
+
+real1 GpuRealStorage::operator[](const tcapint &idx) const
+{
+    if (idx >= size) {
+        throw std::invalid_argument("GpuStorage::operator[] argument out-of-bounds!");
+    }
+    WEED_DEVICE_LOCK();
+    real1 v = ZERO_R1;
+    HipDevice::check(weed_hip_memcpy_d2h(&v, buffer + idx, sizeof(real1)));
+    return v;
+}
+
+void GpuRealStorage::write(const tcapint &idx, const real1 &val)
+{
+    if (idx >= size) {
+        throw std::invalid_argument("GpuStorage::write argument out-of-bounds!");
+    }
+    WEED_DEVICE_LOCK();
+    HipDevice::check(weed_hip_memcpy_h2d(buffer + idx, &val, sizeof(real1)));
+}
+
+void GpuRealStorage::add(const tcapint &idx, const real1 &val) { write(idx, (*this)[idx] + val); }
+
+void GpuRealStorage::FillZeros()
+{
+    WEED_DEVICE_LOCK();
+    HipDevice::check(weed_hip_memset(buffer, 0, sizeof(real1) * (size_t)size));
+}
+
+void GpuRealStorage::FillValue(const real1 &v)
+{
+    const std::vector<real1> host(size, v);
+    WEED_DEVICE_LOCK();
+    HipDevice::check(weed_hip_memcpy_h2d(buffer, host.data(), sizeof(real1) * host.size()));
+}
+
+void GpuRealStorage::FillOnes() { FillValue(ONE_R1); }
+
+StoragePtr GpuRealStorage::cpu()
+{
+    std::shared_ptr<CpuRealStorage> host = std::make_shared<CpuRealStorage>(size);
+    WEED_DEVICE_LOCK();
+    HipDevice::check(weed_hip_memcpy_d2h(host->data.data(), buffer, sizeof(real1) * (size_t)size));
+    return host;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// tensor
+// ---------------------------------------------------------------------------------------------------------
+
+bool Tensor::is_contiguous(const std::vector<tcapint> &shp, const std::vector<tcapint> &s)
+{
+    tcapint st = 1U;
+    for (size_t i = 0U; i < s.size(); ++i) {
+        if (shp[i] == 1U) {
+            continue; // any stride addresses the single element
+        }
+        if (s[i] != st) {
+            return false;
+        }
+        st *= shp[i];
+    }
+    return true;
+}
+
+std::vector<tcapint> Tensor::full_contiguous_stride(const std::vector<tcapint> &shp)
+{
+    std::vector<tcapint> str(shp.size());
+    tcapint run = 1U;
+    for (size_t i = 0U; i < shp.size(); ++i) {
+        str[i] = (shp[i] == 1U) ? 0U : run;
+        run *= shp[i];
+    }
+    return str;
+}
+
+Tensor::Tensor(const std::vector<tcapint> &shp, const std::vector<tcapint> &str, const bool &rg, const bool &,
+    const DType &dtype, const DeviceTag &dtag, const int64_t &did)
+    : shape(shp)
+    , stride(str)
+    , requires_grad(rg)
+{
+    if (shape.size() != stride.size()) {
+        throw std::invalid_argument("Tensor shape vector must have same length as stride vector!");
+    }
+    if (dtype != DType::REAL) {
+        throw std::invalid_argument("Tensor: only real tensors are supported");
+    }
+    if (!is_contiguous(shp, str)) {
+        throw std::invalid_argument("Initial tensor shape and stride must be contiguous!");
+    }
+    const tcapint n = get_size();
+    if (resolve(dtag) == GPU) {
+        storage = std::make_shared<GpuRealStorage>(n, did);
+    } else {
+        storage = std::make_shared<CpuRealStorage>(n);
+    }
+}
+
+Tensor::Tensor(const std::vector<real1> &val, const std::vector<tcapint> &shp, const bool &rg, const DeviceTag &dtag,
+    const int64_t &did)
+    : shape(shp)
+    , stride(full_contiguous_stride(shp))
+    , requires_grad(rg)
+{
+    if (get_size() != val.size()) {
+        throw std::invalid_argument("Tensor value vector must match the size implied by its shape!");
+    }
+    if (resolve(dtag) == GPU) {
+        storage = std::make_shared<GpuRealStorage>(val, did);
+    } else {
+        storage = std::make_shared<CpuRealStorage>(val);
+    }
+}
+
+Tensor::Tensor(const real1 &val, const bool &rg, const DeviceTag &dtag, const int64_t &did)
+    : Tensor(std::vector<real1>{ val }, std::vector<tcapint>{ 1U }, rg, dtag, did)
+{
+}
+
+tcapint Tensor::get_size() const
+{
+    tcapint n = 1U;
+    for (const tcapint &s : shape) {
+        n *= s;
+    }
+    return shape.empty() ? 0U : n;
+}
+
+bool Tensor::is_scalar() const { return get_size() == 1U; }
+
+tcapint Tensor::get_storage_index(const tcapint &idx) const
+{
+    tcapint curr = idx;
+    tcapint stor = offset;
+    for (size_t i = 0U; (i < shape.size()) && curr; ++i) {
+        stor += (curr % shape[i]) * stride[i];
+        curr /= shape[i];
+    }
+    if (curr) {
+        throw std::invalid_argument("Tensor index out-of-range!");
+    }
+    return stor;
+}
+
+real1 Tensor::get_item() const
+{
+    if (!is_scalar()) {
+        throw std::invalid_argument("Tensor::get_item(): not a one-element tensor");
+    }
+    return (*static_cast<RealStorage *>(storage.get()))[offset];
+}
+
+TensorPtr Tensor::operator[](const tcapint &idx) const
+{
+    if (idx >= shape.back()) {
+        throw std::invalid_argument("Tensor index out-of-range!");
+    }
+    TensorPtr v = std::make_shared<Tensor>(*this);
+    v->offset += idx * stride.back();
+    v->shape.pop_back();
+    v->stride.pop_back();
+    if (v->shape.empty()) {
+        v->shape = { 1U };
+        v->stride = { 0U };
+    }
+    return v;
+}
+
+std::vector<real1> Tensor::to_vector() const
+{
+    StoragePtr host = storage->cpu();
+    const RealStorage &rs = *static_cast<RealStorage *>(host.get());
+    const tcapint n = get_size();
+    std::vector<real1> out(n);
+    for (tcapint i = 0U; i < n; ++i) {
+        out[i] = rs[get_storage_index(i)];
+    }
+    return out;
+}
+
+TensorPtr Tensor::cast(const DeviceTag &dtag) const
+{
+    TensorPtr t = std::make_shared<Tensor>(*this);
+    t->storage = (resolve(dtag) == GPU) ? storage->gpu() : storage->cpu();
+    return t;
+}
+
+TensorPtr Tensor::zeros(const std::vector<tcapint> &shape, const bool &rg, const bool &s, const DType &dtype,
+    const DeviceTag &dtag, const int64_t &did)
+{
+    TensorPtr z = std::make_shared<Tensor>(shape, full_contiguous_stride(shape), rg, s, dtype, dtag, did);
+    z->storage->FillZeros();
+    return z;
+}
+
+TensorPtr Tensor::contiguous(const TensorPtr a)
+{
+    if (a->is_contiguous()) {
+        return a;
+    }
+    TensorPtr out = allocate(a->shape, *a);
+    elementwise(WEED_HIP_EW_COPY, *a, nullptr, *out, "Tensor::contiguous");
+    return out;
+}
+
+TensorPtr Tensor::reshape(const TensorPtr a, const std::vector<symint> &s)
+{
+    TensorPtr out = a->is_contiguous() ? std::make_shared<Tensor>(*a) : contiguous(a);
+    const tcapint total = out->get_size();
+    std::vector<tcapint> shp(s.size());
+    symint infer = -1;
+    tcapint known = 1U;
+    for (size_t i = 0U; i < s.size(); ++i) {
+        if (s[i] < 0) {
+            if (infer >= 0) {
+                throw std::invalid_argument("Tensor::reshape(): only one -1 dimension allowed");
+            }
+            infer = (symint)i;
+        } else {
+            shp[i] = (tcapint)s[i];
+            known *= (tcapint)s[i];
+        }
+    }
+    if (infer >= 0) {
+        if (!known || (total % known)) {
+            throw std::invalid_argument("Tensor::reshape(): cannot infer dimension size");
+        }
+        shp[(size_t)infer] = total / known;
+        known *= shp[(size_t)infer];
+    }
+    if (known != total || shp.empty()) {
+        throw std::invalid_argument("Tensor::reshape(): sizes do not match");
+    }
+    out->shape = shp;
+    out->stride = full_contiguous_stride(shp);
+    return out;
+}
+
+TensorPtr Tensor::transpose(const TensorPtr a)
+{
+    if (a->shape.size() != 2U) {
+        throw std::invalid_argument("Tensor::transpose is only for 2D tensors (and vectors and covectors)!");
+    }
+    return transpose(a, 0, 1);
+}
+
+TensorPtr Tensor::transpose(const TensorPtr a, symint i, symint j)
+{
+    i = wrap_axis(i, a->shape.size(), "Tensor::transpose");
+    j = wrap_axis(j, a->shape.size(), "Tensor::transpose");
+    TensorPtr out = std::make_shared<Tensor>(*a);
+    std::swap(out->shape[(size_t)i], out->shape[(size_t)j]);
+    std::swap(out->stride[(size_t)i], out->stride[(size_t)j]);
+    return out;
+}
+
+TensorPtr Tensor::slice(TensorPtr a, const int64_t &row)
+{
+    // fixes an index of dimension 0 and drops that dimension
+    if (row < 0 || (tcapint)row >= a->shape[0U]) {
+        throw std::invalid_argument("Tensor::slice(): row out of range");
+    }
+    TensorPtr out = std::make_shared<Tensor>(*a);
+    out->offset += (tcapint)row * a->stride[0U];
+    out->shape.erase(out->shape.begin());
+    out->stride.erase(out->stride.begin());
+    if (out->shape.empty()) {
+        out->shape = { 1U };
+        out->stride = { 0U };
+    }
+    return out;
+}
+
+TensorPtr Tensor::slice(TensorPtr a, int64_t axis, const tcapint &start, const tcapint &length)
+{
+    const size_t ax = (size_t)wrap_axis((symint)axis, a->shape.size(), "Tensor::slice");
+    if (!length || (start + length) > a->shape[ax]) {
+        throw std::invalid_argument("Tensor::slice(): range out of bounds");
+    }
+    TensorPtr out = std::make_shared<Tensor>(*a);
+    out->offset += start * a->stride[ax];
+    out->shape[ax] = length;
+    return out;
+}
+
+TensorPtr Tensor::softmax(const TensorPtr x, symint axis)
+{
+    axis = wrap_axis(axis, x->shape.size(), "Tensor::softmax");
+    TensorPtr out = allocate(x->shape, *x);
+    Weed::softmax((tcapint)axis, *x, *out);
+    return out;
+}
+
+namespace {
+TensorPtr axis_reduce(TensorPtr a, symint axis, void (*op)(const tcapint &, const Tensor &, Tensor &), const char *who)
+{
+    axis = wrap_axis(axis, a->shape.size(), who);
+    std::vector<tcapint> shp = a->shape;
+    shp.erase(shp.begin() + axis);
+    if (shp.empty()) {
+        shp = { 1U };
+    }
+    TensorPtr out = allocate(shp, *a);
+    op((tcapint)axis, *a, *out);
+    return out;
+}
+} // namespace
+
+TensorPtr Tensor::sum(TensorPtr a, symint axis) { return axis_reduce(a, axis, Weed::reduce, "Tensor::sum"); }
+TensorPtr Tensor::max(TensorPtr a, symint axis) { return axis_reduce(a, axis, Weed::max, "Tensor::max"); }
+TensorPtr Tensor::min(TensorPtr a, symint axis) { return axis_reduce(a, axis, Weed::min, "Tensor::min"); }
+TensorPtr Tensor::add(TensorPtr a, TensorPtr b) { return binary(WEED_HIP_EW_ADD, a, b, "Tensor::add"); }
+TensorPtr Tensor::sub(TensorPtr a, TensorPtr b) { return binary(WEED_HIP_EW_SUB, a, b, "Tensor::sub"); }
+TensorPtr Tensor::mul(TensorPtr a, TensorPtr b) { return binary(WEED_HIP_EW_MUL, a, b, "Tensor::mul"); }
+TensorPtr Tensor::div(TensorPtr a, TensorPtr b) { return binary(WEED_HIP_EW_DIV, a, b, "Tensor::div"); }
+
+TensorPtr Tensor::matmul(TensorPtr a, TensorPtr b)
+{
+    if (a->shape.size() < 2U) {
+        throw std::invalid_argument("Tensor::matmul requires a to have rank >= 2");
+    }
+    const size_t rank = a->shape.size();
+    if (rank > 2U && b->shape.size() > 2U) {
+        // one 2-D product per index of the leading (batch) dimensions (src/tensors/tensor.cpp:1213-1272)
+        if (rank != b->shape.size()) {
+            throw std::invalid_argument("batched matmul rank mismatch");
+        }
+        tcapint batch = 1U;
+        for (size_t i = 0; i < rank - 2U; ++i) {
+            if (a->shape[i] != b->shape[i]) {
+                throw std::invalid_argument("batched matmul batch mismatch");
+            }
+            batch *= a->shape[i];
+        }
+        const tcapint M = a->shape[rank - 2U], K = a->shape[rank - 1U], N = b->shape[rank - 1U];
+        if (K != b->shape[rank - 2U]) {
+            throw std::invalid_argument("batched matmul inner dim mismatch");
+        }
+        std::vector<tcapint> shp(a->shape.begin(), a->shape.end() - 2);
+        shp.push_back(M);
+        shp.push_back(N);
+        TensorPtr out = allocate(shp, *a);
+        for (tcapint i = 0U; i < batch; ++i) {
+            Tensor ai = *a, bi = *b, oi = *out;
+            tcapint rem = i;
+            for (size_t dd = 0; dd < rank - 2U; ++dd) {
+                const tcapint c = rem % a->shape[dd];
+                rem /= a->shape[dd];
+                ai.offset += c * a->stride[dd];
+                bi.offset += c * b->stride[dd];
+                oi.offset += c * out->stride[dd];
+            }
+            for (Tensor *t : { &ai, &bi, &oi }) {
+                t->shape.erase(t->shape.begin(), t->shape.end() - 2);
+                t->stride.erase(t->stride.begin(), t->stride.end() - 2);
+            }
+            Weed::matmul(ai, bi, oi);
+        }
+        return out;
+    }
+    if (b->shape.size() != 2U) {
+        throw std::invalid_argument("Tensor::matmul requires b to have rank 2 when a is flattened");
+    }
+    const tcapint K = a->shape.back(), N = b->shape[1U];
+    if (b->shape[0U] != K) {
+        throw std::invalid_argument("matmul dimension mismatch");
+    }
+    TensorPtr a2 = (rank > 2U) ? reshape(a, { -1, (symint)K }) : a;
+    TensorPtr out = allocate({ a2->shape[0U], N }, *a2);
+    Weed::matmul(*a2, *b, *out);
+    if (rank > 2U) {
+        std::vector<symint> shp(a->shape.begin(), a->shape.end() - 1);
+        shp.push_back((symint)N);
+        out = reshape(out, shp);
+    }
+    return out;
+}
+
+TensorPtr operator+(TensorPtr left, TensorPtr right) { return Tensor::add(left, right); }
+TensorPtr operator-(TensorPtr left, TensorPtr right) { return Tensor::sub(left, right); }
+TensorPtr operator*(TensorPtr left, TensorPtr right) { return Tensor::mul(left, right); }
+TensorPtr operator/(TensorPtr left, TensorPtr right) { return Tensor::div(left, right); }
+TensorPtr operator/(TensorPtr left, real1 right)
+{
+    // a scalar operand becomes a one-element tensor on the same device (include/tensors/tensor.hpp:622-624)
+    return Tensor::div(left, std::make_shared<Tensor>(right, false, left->storage->device, left->storage->get_device_id()));
+}
+TensorPtr operator*(real1 left, TensorPtr right)
+{
+    return Tensor::mul(std::make_shared<Tensor>(left, false, right->storage->device, right->storage->get_device_id()), right);
+}
+TensorPtr operator>>(TensorPtr left, TensorPtr right) { return Tensor::matmul(left, right); }
+TensorPtr operator<<(TensorPtr right, TensorPtr left) { return Tensor::matmul(left, right); }
+
+// ---------------------------------------------------------------------------------------------------------
+// ops
+// ---------------------------------------------------------------------------------------------------------
+
+void matmul(const Tensor &a, const Tensor &b, Tensor &out)
+{
+    validate_all_same_device({ &a, &b, &out }, "MatMulKernel::matmul");
+    if (a.shape.size() != 2U || b.shape.size() != 2U || out.shape.size() != 2U) {
+        throw std::invalid_argument("MatMul is only for matrices with 2 indices!");
+    }
+    const tcapint M = a.shape[0U], K = a.shape[1U], N = b.shape[1U];
+    if (K != b.shape[0U] || out.shape[0U] != M || out.shape[1U] != N) {
+        throw std::invalid_argument("MatMul operand dimensions aren't compatible!");
+    }
+    real1 *ap = device_ptr(a, "matmul"), *bp = device_ptr(b, "matmul"), *op = device_ptr(out, "matmul");
+    WEED_DEVICE_LOCK();
+    HipDevice::check(weed_hip_matmul_f32(M, N, K, ap, a.offset, a.stride[0U], a.stride[1U], bp, b.offset, b.stride[0U],
+        b.stride[1U], op, out.offset, out.stride[0U], out.stride[1U]));
+}
+
+void softmax(const tcapint &index, const Tensor &a, Tensor &out)
+{
+    validate_all_same_device({ &a, &out }, "SoftmaxKernel::softmax_forward");
+    if (a.shape != out.shape) {
+        throw std::invalid_argument("Tensor shape mismatch in softmax_forward!");
+    }
+    if (index >= a.shape.size()) {
+        throw std::invalid_argument("softmax axis out of range");
+    }
+    real1 *ap = device_ptr(a, "softmax"), *op = device_ptr(out, "softmax");
+    WEED_DEVICE_LOCK();
+    HipDevice::check(weed_hip_softmax_f32((uint32_t)a.shape.size(), a.shape.data(), index, ap, a.offset, a.stride.data(),
+        op, out.offset, out.stride.data()));
+}
+
+namespace {
+void axis_op(int op, const tcapint &index, const Tensor &a, Tensor &out, const char *who)
+{
+    validate_all_same_device({ &a, &out }, who);
+    if (index >= a.shape.size()) {
+        throw std::invalid_argument(std::string(who) + ": axis out of range");
+    }
+    std::vector<tcapint> want = a.shape;
+    want.erase(want.begin() + index);
+    if (want.empty()) {
+        want = { 1U };
+    }
+    if (want != out.shape) {
+        throw std::invalid_argument(std::string(who) + ": output shape mismatch");
+    }
+    std::vector<uint32_t> os(out.stride.begin(), out.stride.end());
+    if (a.shape.size() == 1U) {
+        os = { 0U };
+    } else {
+        os.insert(os.begin() + index, 0U);
+    }
+    real1 *ap = device_ptr(a, who), *op_ = device_ptr(out, who);
+    WEED_DEVICE_LOCK();
+    HipDevice::check(weed_hip_reduce_f32(op, (uint32_t)a.shape.size(), a.shape.data(), index, ap, a.offset,
+        a.stride.data(), op_, out.offset, os.data()));
+}
+} // namespace
+
+void reduce(const tcapint &index, const Tensor &a, Tensor &out) { axis_op(WEED_HIP_REDUCE_SUM, index, a, out, "ReduceKernel::reduce"); }
+void max(const tcapint &index, const Tensor &a, Tensor &out) { axis_op(WEED_HIP_REDUCE_MAX, index, a, out, "ReduceKernel::max"); }
+void min(const tcapint &index, const Tensor &a, Tensor &out) { axis_op(WEED_HIP_REDUCE_MIN, index, a, out, "ReduceKernel::min"); }
+
+void add(const Tensor &a, const Tensor &b, Tensor &out)
+{
+    validate_all_same_device({ &a, &b, &out }, "CommutingKernel::commuting");
+    elementwise(WEED_HIP_EW_ADD, a, &b, out, "add");
+}
+void mul(const Tensor &a, const Tensor &b, Tensor &out)
+{
+    validate_all_same_device({ &a, &b, &out }, "CommutingKernel::commuting");
+    elementwise(WEED_HIP_EW_MUL, a, &b, out, "mul");
+}
+void sub(const Tensor &a, const Tensor &b, Tensor &out)
+{
+    validate_all_same_device({ &a, &b, &out }, "SubKernel::sub");
+    elementwise(WEED_HIP_EW_SUB, a, &b, out, "sub");
+}
+void div(const Tensor &a, const Tensor &b, Tensor &out)
+{
+    validate_all_same_device({ &a, &b, &out }, "DivKernel::div");
+    elementwise(WEED_HIP_EW_DIV, a, &b, out, "div");
+}
+void add_in_place(Tensor &a, const Tensor &b)
+{
+    validate_all_same_device({ &a, &b }, "InPlaceKernel::in_place");
+    elementwise(WEED_HIP_EW_ADD, a, &b, a, "add_in_place");
+}
+
+void triu_fill(Tensor &a, const real1 &val, const tcapint diagonal)
+{
+    if (a.shape.size() != 2U) {
+        throw std::invalid_argument("triu_fill: tensor must be 2D [T, T]");
+    }
+    real1 *ap = device_ptr(a, "triu_fill");
+    WEED_DEVICE_LOCK();
+    HipDevice::check(
+        weed_hip_triu_fill_f32(a.shape[0U], a.shape[1U], val, diagonal, ap, a.offset, a.stride[0U], a.stride[1U]));
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Linear
+// ---------------------------------------------------------------------------------------------------------
+
+Linear::Linear(tcapint in_f, tcapint out_f, bool use_bias, bool init_rand, DType dtype, DeviceTag device, int64_t device_id)
+    : in_features(in_f)
+    , out_features(out_f)
+{
+    if (dtype != DType::REAL) {
+        throw std::invalid_argument("Linear: only real parameters are supported");
+    }
+    std::vector<real1> w((size_t)in_f * out_f, ZERO_R1);
+    if (init_rand) {
+        // uniform in +-1/sqrt(in_features)
+        std::mt19937 rng{ std::random_device{}() };
+        const real1 lim = ONE_R1 / std::sqrt((real1)in_f);
+        std::uniform_real_distribution<real1> dist(-lim, lim);
+        for (real1 &v : w) {
+            v = dist(rng);
+        }
+    }
+    weight = std::make_shared<Parameter>(w, std::vector<tcapint>{ in_f, out_f }, true, device, device_id);
+    if (use_bias) {
+        bias = std::make_shared<Parameter>(
+            std::vector<real1>(out_f, ZERO_R1), std::vector<tcapint>{ 1U, out_f }, true, device, device_id);
+    }
+}
+
+TensorPtr Linear::forward(const TensorPtr x)
+{
+    TensorPtr y = x >> weight;
+    if (bias) {
+        // unlike Tensor::add in the reference (src/tensors/tensor.cpp:1091), broadcasting never reshapes the bias
+        // itself, so the sequence length may change between calls
+        y = y + bias;
+    }
+    return y;
+}
+
+std::vector<ParameterPtr> Linear::parameters()
+{
+    std::vector<ParameterPtr> p{ weight };
+    if (bias) {
+        p.push_back(bias);
+    }
+    return p;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// quantized cache
+// ---------------------------------------------------------------------------------------------------------
+
+DeviceKVCache::DeviceKVCache(int mode, tcapint n_seq_, tcapint n_kv_heads_, tcapint head_dim_, tcapint max_tokens_,
+    int k_bits, int v_bits, int k_sign, int v_sign)
+    : n_seq(n_seq_)
+    , n_kv_heads(n_kv_heads_)
+    , head_dim(head_dim_)
+    , max_tokens(max_tokens_)
+{
+    weed_hip_kv_config cfg;
+    cfg.mode = mode;
+    cfg.n_seq = (int32_t)n_seq_;
+    cfg.n_kv_heads = (int32_t)n_kv_heads_;
+    cfg.head_dim = (int32_t)head_dim_;
+    cfg.max_tokens = (int32_t)max_tokens_;
+    cfg.k_bits = k_bits;
+    cfg.v_bits = v_bits;
+    cfg.k_sign = k_sign;
+    cfg.v_sign = v_sign;
+    WEED_DEVICE_LOCK();
+    HipDevice::check(weed_hip_kv_cache_create(&handle, &cfg));
+}
+
+DeviceKVCache::~DeviceKVCache()
+{
+    if (handle) {
+        WEED_DEVICE_LOCK();
+        (void)weed_hip_kv_cache_destroy(handle);
+    }
+}
+
+void QuantizedKVCache::allocate(const tcapint max_outer_, const tcapint d_, const int bits_)
+{
+    // a single (sequence, kv head) pair holding max_outer rows; both halves of the device object get the same rows
+    dev = std::make_shared<DeviceKVCache>(WEED_HIP_KV_UNIFORM, 1U, 1U, d_, max_outer_, bits_, bits_, 0, 0);
+    which = 0;
+    max_outer = max_outer_;
+    d = d_;
+    bits = bits_;
+    outer = 0U;
+    packed.clear();
+}
+
+void QuantizedKVCache::write_row(const tcapint row, const real1 *vals)
+{
+    if (!dev) {
+        throw std::domain_error("QuantizedKVCache::write_row(): allocate() first");
+    }
+    if (dev->n_seq != 1U || dev->n_kv_heads != 1U) {
+        throw std::domain_error("QuantizedKVCache::write_row(): rows of a module's cache are written by forward()");
+    }
+    if (row != outer) {
+        throw std::domain_error("QuantizedKVCache::write_row(): rows are append-only on the device");
+    }
+    GpuRealStorage staging(std::vector<real1>(vals, vals + d));
+    const uint32_t str[4] = { 0U, 0U, 0U, 1U };
+    WEED_DEVICE_LOCK();
+    HipDevice::check(weed_hip_kv_cache_set_scales(dev->handle, block_scale, block_scale));
+    HipDevice::check(
+        weed_hip_kv_encode_append(dev->handle, 0, 1, 1, staging.buffer, 0U, str, staging.buffer, 0U, str, 0));
+    HipDevice::check(weed_hip_sync());
+    ++outer;
+}
+
+void QuantizedKVCache::read_row(const tcapint row, real1 *vals) const
+{
+    if (!dev) {
+        throw std::domain_error("QuantizedKVCache::read_row(): allocate() first");
+    }
+    const tcapint pair = row / dev->max_tokens, tok = row % dev->max_tokens;
+    if (pair >= dev->n_seq * dev->n_kv_heads) {
+        throw std::invalid_argument("QuantizedKVCache::read_row(): row out of range");
+    }
+    // dequantise [1 sequence, all kv heads, 1 token, d] and keep the wanted head
+    const tcapint seq = pair / dev->n_kv_heads, head = pair % dev->n_kv_heads;
+    GpuRealStorage staging(dev->n_kv_heads * d);
+    const uint32_t str[4] = { 0U, d, 0U, 1U };
+    WEED_DEVICE_LOCK();
+    HipDevice::check(weed_hip_kv_dequant(dev->handle, which, (int32_t)seq, 1, (int32_t)tok, 1, staging.buffer, 0U, str));
+    HipDevice::check(weed_hip_memcpy_d2h(vals, staging.buffer + (size_t)head * d, sizeof(real1) * d));
+}
+
+void QuantizedKVCache::sync_packed()
+{
+    if (!dev) {
+        throw std::domain_error("QuantizedKVCache::sync_packed(): allocate() first");
+    }
+    const tcapint vpw = (tcapint)values_per_word(), wpr = (d + vpw - 1U) / vpw;
+    std::vector<int32_t> lens(dev->n_seq);
+    WEED_DEVICE_LOCK();
+    HipDevice::check(weed_hip_kv_cache_seq_lens(dev->handle, lens.data()));
+    const tcapint T = (tcapint)*std::max_element(lens.begin(), lens.end());
+    packed.assign((size_t)dev->n_seq * dev->n_kv_heads * T * wpr, 0);
+    if (!T) {
+        return;
+    }
+    void *words = nullptr;
+    HipDevice::check(weed_hip_malloc(&words, packed.size() * sizeof(int32_t)));
+    int st = weed_hip_kv_export_weed_words(dev->handle, which, 0, (int32_t)dev->n_seq, 0, (int32_t)T, (int32_t *)words);
+    if (st == WEED_HIP_OK) {
+        st = weed_hip_memcpy_d2h(packed.data(), words, packed.size() * sizeof(int32_t));
+    }
+    (void)weed_hip_free(words);
+    HipDevice::check(st);
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// attention
+// ---------------------------------------------------------------------------------------------------------
+
+MultiHeadAttention::MultiHeadAttention(tcapint d_model_, tcapint num_heads_, tcapint num_kv_heads_, tcapint head_dim_,
+    DeviceTag dtag, RoPEPtr r, real1_f mask_val_, const int64_t did, const bool _use_kv_cache, int kv_quant_bits_,
+    bool use_bias)
+    : d_model((symint)d_model_)
+    , num_heads((symint)num_heads_)
+    , num_kv_heads((symint)(num_kv_heads_ ? num_kv_heads_ : num_heads_))
+    , head_dim((symint)(!head_dim_ ? d_model_ / num_heads_ : head_dim_))
+    , mask_val(mask_val_)
+    , use_kv_cache(_use_kv_cache)
+    , kv_quant_bits(kv_quant_bits_)
+{
+    if (r) {
+        throw std::domain_error("MultiHeadAttention: rotary position embedding is not part of this build");
+    }
+    if (d_model % num_heads) {
+        throw std::invalid_argument("d_model must be divisible by num_heads");
+    }
+    if (num_heads % num_kv_heads) {
+        throw std::invalid_argument("num_heads must be divisible by num_kv_heads");
+    }
+    const tcapint q_dim = (tcapint)(num_heads * head_dim), kv_dim = (tcapint)(num_kv_heads * head_dim);
+    W_q = std::make_shared<Linear>(d_model_, q_dim, use_bias, true, DType::REAL, dtag, did);
+    W_k = std::make_shared<Linear>(d_model_, kv_dim, use_bias, true, DType::REAL, dtag, did);
+    W_v = std::make_shared<Linear>(d_model_, kv_dim, use_bias, true, DType::REAL, dtag, did);
+    W_o = std::make_shared<Linear>(q_dim, d_model_, use_bias, true, DType::REAL, dtag, did);
+    for (const LinearPtr &l : { W_q, W_k, W_v, W_o }) {
+        const std::vector<ParameterPtr> p = l->parameters();
+        param_vector.insert(param_vector.end(), p.begin(), p.end());
+    }
+    if (mask_val == ZERO_R1) {
+        mask_val = -1.701411835e38f; // -2^127 (multihead_attention.hpp:109-110 at fp32)
+    }
+}
+
+MultiHeadAttention::~MultiHeadAttention()
+{
+    if (lens_dev) {
+        WEED_DEVICE_LOCK();
+        (void)weed_hip_free(lens_dev);
+    }
+}
+
+void MultiHeadAttention::reset_cache()
+{
+    k_cache = nullptr;
+    v_cache = nullptr;
+    cache_len = 0U;
+    max_seq_len = 0U;
+    k_rotation.clear();
+    v_rotation.clear();
+    v_rotation_trans.clear();
+    k_rot_dev = nullptr;
+    v_rot_dev = nullptr;
+    k_qcache = QuantizedKVCache{};
+    v_qcache = QuantizedKVCache{};
+}
+
+TensorPtr MultiHeadAttention::forward(const TensorPtr x)
+{
+    // x: (B, T, d_model)
+    if (x->shape.size() != 3U || (symint)x->shape[2U] != d_model) {
+        throw std::invalid_argument("MultiHeadAttention::forward(): input must be (B, T, d_model)");
+    }
+    const symint B = (symint)x->shape[0U], T = (symint)x->shape[1U];
+
+    TensorPtr Q = W_q->forward(x);
+    TensorPtr K = W_k->forward(x);
+    TensorPtr V = W_v->forward(x);
+
+    Q = Tensor::reshape(Q, { B, T, num_heads, head_dim });
+    K = Tensor::reshape(K, { B, T, num_kv_heads, head_dim });
+    V = Tensor::reshape(V, { B, T, num_kv_heads, head_dim });
+
+    TensorPtr out = (use_kv_cache && kv_quant_bits > 0) ? forward_quantized(Q, K, V, B, T) : forward_dense(Q, K, V, B, T);
+
+    // (B, T, num_heads * head_dim)
+    out = Tensor::reshape(out, { B, T, num_heads * head_dim });
+    return W_o->forward(out);
+}
+
+// Quantized cache: rotate + encode + append the new tokens, then one fused kernel per query position over the
+// packed rows (multihead_attention.cpp:169-277, 291-348 collapse into these calls).  Q, K, V arrive as contiguous
+// (B, T, heads, head_dim) tensors; the (B, heads, T, head_dim) views the reference forms by transpose are expressed
+// through strides.  Returns (B, T, num_heads, head_dim), contiguous.
+TensorPtr MultiHeadAttention::forward_quantized(TensorPtr Q, TensorPtr K, TensorPtr V, symint B, symint T)
+{
+    const tcapint hd = (tcapint)head_dim, Hkv = (tcapint)num_kv_heads, Hq = (tcapint)num_heads;
+    const tcapint uB = (tcapint)B, uT = (tcapint)T;
+    device_ptr(*Q, "MultiHeadAttention::forward");
+    WEED_DEVICE_LOCK();
+
+    if (!k_qcache.dev) {
+        if (!max_seq_len) {
+            max_seq_len = 2048U;
+        }
+        cache_len = 0U;
+        const int kb = k_bits ? k_bits : kv_quant_bits, vb = v_bits ? v_bits : kv_quant_bits;
+        const bool lloyd = kv_coder == KV_LLOYDMAX;
+        DeviceKVCachePtr dev = std::make_shared<DeviceKVCache>(lloyd ? WEED_HIP_KV_LLOYDMAX : WEED_HIP_KV_UNIFORM, uB, Hkv,
+            hd, max_seq_len, kb, vb, (lloyd && k_sign) ? 1 : 0, (lloyd && v_sign) ? 1 : 0);
+        if (k_rotation.size() == (size_t)hd * hd && v_rotation.size() == (size_t)hd * hd) {
+            k_rot_dev = std::make_shared<GpuRealStorage>(k_rotation);
+            v_rot_dev = std::make_shared<GpuRealStorage>(v_rotation);
+        } else {
+            uint32_t seed = rotation_seed ? rotation_seed : (uint32_t)std::random_device{}();
+            k_rot_dev = std::make_shared<GpuRealStorage>(hd * hd);
+            v_rot_dev = std::make_shared<GpuRealStorage>(hd * hd);
+            HipDevice::check(weed_hip_make_rotation(seed, hd, k_rot_dev->buffer));
+            HipDevice::check(weed_hip_make_rotation(seed + 0x9e3779b9U, hd, v_rot_dev->buffer));
+            k_rotation = static_cast<CpuRealStorage *>(k_rot_dev->cpu().get())->data;
+            v_rotation = static_cast<CpuRealStorage *>(v_rot_dev->cpu().get())->data;
+        }
+        v_rotation_trans.resize((size_t)hd * hd);
+        for (tcapint i = 0U; i < hd; ++i) {
+            for (tcapint j = 0U; j < hd; ++j) {
+                v_rotation_trans[(size_t)i * hd + j] = v_rotation[(size_t)j * hd + i];
+            }
+        }
+        HipDevice::check(weed_hip_kv_cache_set_rotations(dev->handle, k_rot_dev->buffer, v_rot_dev->buffer));
+        for (QuantizedKVCache *qc : { &k_qcache, &v_qcache }) {
+            qc->dev = dev;
+            qc->which = (qc == &v_qcache) ? 1 : 0;
+            qc->d = hd;
+            qc->bits = qc->which ? vb : kb;
+            qc->max_outer = uB * Hkv * max_seq_len;
+            qc->outer = 0U;
+        }
+    }
+    weed_hip_kv_cache *cache = k_qcache.dev->handle;
+    if (k_qcache.dev->n_seq != uB) {
+        throw std::invalid_argument("MultiHeadAttention::forward(): batch size changed while the KV cache is live");
+    }
+
+    // element (b, h, t, j) of the logical (B, heads, T, head_dim) views
+    const uint32_t kv_str[4] = { 1U, uB * uT, uB, uB * uT * Hkv };
+    const uint32_t kv_shape[4] = { uB, Hkv, uT, hd };
+    real1 *kp = device_ptr(*K, "MultiHeadAttention::forward"), *vp = device_ptr(*V, "MultiHeadAttention::forward");
+    if (kv_coder == KV_UNIFORM) {
+        // rotate in the reference's rounding order, take the block scales from the first write, then code
+        TensorPtr Kr = allocate(K->shape, *K), Vr = allocate(V->shape, *V);
+        real1 *krp = device_ptr(*Kr, "forward"), *vrp = device_ptr(*Vr, "forward");
+        HipDevice::check(weed_hip_apply_rotation_f32(hd, k_rot_dev->buffer, 4U, kv_shape, kp, K->offset, kv_str, krp, 0U, kv_str));
+        HipDevice::check(weed_hip_apply_rotation_f32(hd, v_rot_dev->buffer, 4U, kv_shape, vp, V->offset, kv_str, vrp, 0U, kv_str));
+        if (cache_len == 0U) {
+            // sequential sums reproduce the reference bit for bit and are affordable for short first writes
+            const int sequential = ((uint64_t)uB * Hkv * uT * hd <= (1U << 16)) ? 1 : 0;
+            HipDevice::check(weed_hip_block_scale_f32(krp, 0U, kv_shape, kv_str, sequential, &k_qcache.block_scale));
+            HipDevice::check(weed_hip_block_scale_f32(vrp, 0U, kv_shape, kv_str, sequential, &v_qcache.block_scale));
+            HipDevice::check(weed_hip_kv_cache_set_scales(cache, k_qcache.block_scale, v_qcache.block_scale));
+        }
+        HipDevice::check(weed_hip_kv_encode_append(cache, 0, B, T, krp, 0U, kv_str, vrp, 0U, kv_str, 0));
+    } else {
+        HipDevice::check(weed_hip_kv_encode_append(cache, 0, B, T, kp, K->offset, kv_str, vp, V->offset, kv_str, 1));
+    }
+    const tcapint before = cache_len;
+    cache_len += uT;
+    k_qcache.outer = v_qcache.outer = uB * Hkv * cache_len;
+
+    TensorPtr out = allocate({ uB, uT, Hq, hd }, *Q);
+    real1 *qp = device_ptr(*Q, "forward"), *op = device_ptr(*out, "forward");
+    const uint32_t q_str[3] = { 1U, uB * uT, uB * uT * Hq }; // (b, h, j) at a fixed t
+    const int gqa = gqa_blocked ? WEED_HIP_GQA_BLOCKED : WEED_HIP_GQA_WEED;
+    const uint32_t flags = WEED_HIP_ATTN_ROTATE_Q | WEED_HIP_ATTN_UNROTATE_OUT;
+    if (T == 1) {
+        HipDevice::check(weed_hip_kv_decode_attn(cache, num_heads, gqa, qp, Q->offset, q_str, op, 0U, q_str, flags));
+        return out;
+    }
+    // causal attention: query position t sees the first before + t + 1 cached tokens of its sequence
+    const size_t need = sizeof(int32_t) * (size_t)uB * uT;
+    if (need > lens_cap) {
+        if (lens_dev) {
+            HipDevice::check(weed_hip_sync());
+            (void)weed_hip_free(lens_dev);
+            lens_dev = nullptr;
+            lens_cap = 0U;
+        }
+        HipDevice::check(weed_hip_malloc(&lens_dev, need));
+        lens_cap = need;
+    }
+    std::vector<int32_t> lens((size_t)uB * uT);
+    for (tcapint t = 0U; t < uT; ++t) {
+        std::fill(lens.begin() + (size_t)t * uB, lens.begin() + (size_t)(t + 1U) * uB, (int32_t)(before + t + 1U));
+    }
+    HipDevice::check(weed_hip_sync()); // earlier launches may still read the previous call's lengths
+    HipDevice::check(weed_hip_memcpy_h2d(lens_dev, lens.data(), need));
+    for (tcapint t = 0U; t < uT; ++t) {
+        HipDevice::check(weed_hip_kv_decode_attn_prefix(cache, static_cast<const int32_t *>(lens_dev) + (size_t)t * uB,
+            num_heads, gqa, qp, Q->offset + t * uB, q_str, op, t * uB, q_str, flags));
+    }
+    return out;
+}
+
+// Float cache or no cache: the reference's own sequence of dense ops (multihead_attention.cpp:279-340), each one a
+// device op.  Returns (B, T, num_heads, head_dim).
+TensorPtr MultiHeadAttention::forward_dense(TensorPtr Q, TensorPtr K, TensorPtr V, symint B, symint T)
+{
+    const tcapint hd = (tcapint)head_dim, Hkv = (tcapint)num_kv_heads, Hq = (tcapint)num_heads;
+    const tcapint uB = (tcapint)B, uT = (tcapint)T;
+    Q = Tensor::transpose(Q, 1, 2); // [B, num_heads, T, head_dim]
+    K = Tensor::transpose(K, 1, 2); // [B, kv_heads,  T, head_dim]
+    V = Tensor::transpose(V, 1, 2);
+
+    tcapint before = 0U;
+    if (use_kv_cache) {
+        if (!k_cache) {
+            if (!max_seq_len) {
+                max_seq_len = 2048U;
+            }
+            cache_len = 0U;
+            k_cache = Tensor::zeros({ uB, Hkv, max_seq_len, hd }, false, false, DType::REAL, Q->storage->device);
+            v_cache = Tensor::zeros({ uB, Hkv, max_seq_len, hd }, false, false, DType::REAL, Q->storage->device);
+        }
+        if (cache_len + uT > max_seq_len) {
+            throw std::out_of_range("MultiHeadAttention::forward(): KV cache is full");
+        }
+        TensorPtr k_slot = Tensor::slice(k_cache, 2, cache_len, uT);
+        TensorPtr v_slot = Tensor::slice(v_cache, 2, cache_len, uT);
+        Weed::add_in_place(*k_slot, *K);
+        Weed::add_in_place(*v_slot, *V);
+        before = cache_len;
+        cache_len += uT;
+        K = Tensor::slice(k_cache, 2, 0U, cache_len);
+        V = Tensor::slice(v_cache, 2, 0U, cache_len);
+    }
+
+    if (num_kv_heads < num_heads) {
+        const tcapint groups = Hq / Hkv, T_k = K->shape[2U];
+        TensorPtr K_rep = Tensor::zeros({ uB, Hq, T_k, hd }, false, false, DType::REAL, Q->storage->device);
+        TensorPtr V_rep = Tensor::zeros({ uB, Hq, T_k, hd }, false, false, DType::REAL, Q->storage->device);
+        if (gqa_blocked) {
+            for (tcapint h = 0U; h < Hkv; ++h) {
+                Weed::add_in_place(*Tensor::slice(K_rep, 1, h * groups, groups), *Tensor::slice(K, 1, h, 1U));
+                Weed::add_in_place(*Tensor::slice(V_rep, 1, h * groups, groups), *Tensor::slice(V, 1, h, 1U));
+            }
+        } else {
+            for (tcapint g = 0U; g < groups; ++g) {
+                Weed::add_in_place(*Tensor::slice(K_rep, 1, g * Hkv, Hkv), *K);
+                Weed::add_in_place(*Tensor::slice(V_rep, 1, g * Hkv, Hkv), *V);
+            }
+        }
+        K = K_rep;
+        V = V_rep;
+    }
+
+    TensorPtr scores = Q >> Tensor::transpose(K, -2, -1);
+    scores = scores / real1(std::sqrt((real1)head_dim));
+    if (T > 1) {
+        const tcapint T_k = K->shape[2U];
+        TensorPtr mask = Tensor::zeros({ uT, T_k }, false, false, DType::REAL, Q->storage->device);
+        Weed::triu_fill(*mask, (real1)mask_val, before + 1U);
+        scores = scores + mask;
+    }
+    TensorPtr weights = Tensor::softmax(scores, -1);
+    TensorPtr out = weights >> V;
+    return Tensor::transpose(out, 1, 2); // (B, T, H, head_dim)
+}
+
+} // namespace Weed

@@ -1,0 +1,347 @@
+// Host-side mirror of the part of Weed's C++ interface that sits on the quantized-KV attention path:
+// Storage / Tensor (real, dense, forward only), the op entry points with their device switch, Linear,
+// QuantizedKVCache and MultiHeadAttention.  Names, argument meaning and exception types follow the reference
+// (include/tensors/tensor.hpp, include/storage/*.hpp, include/ops/*.hpp, include/modules/linear.hpp,
+// include/modules/multihead_attention.hpp); every computation goes to the device library behind
+// include/weed_hip.h.  There is no CPU arithmetic here: a CPU-tagged tensor is a host container that can be filled,
+// read and moved to the device, and an op handed one throws std::domain_error.
+#pragma once
+
+#include <cstdint>
+#include <memory>
+#include <mutex>
+#include <new>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+struct weed_hip_kv_cache;
+
+namespace Weed {
+
+typedef uint32_t tcapint; // include/common/weed_types.hpp:48-66 at the default build width
+typedef int32_t symint;
+typedef float real1;
+typedef float real1_f;
+constexpr real1 ZERO_R1 = 0.0f;
+constexpr real1 ONE_R1 = 1.0f;
+
+enum DeviceTag { NONE_DEVICE = 0, DEFAULT_DEVICE = 1, CPU = 2, GPU = 3 }; // include/enums/device_tag.hpp
+enum DType { NONE_DTYPE = 0, REAL = 1, COMPLEX = 2, INT = 3, DEFAULT_DTYPE = REAL }; // include/enums/dtype.hpp
+enum StorageType { NONE_STORAGE_TYPE = 0, REAL_CPU_DENSE = 1, REAL_GPU_DENSE = 2 }; // include/enums/storage_type.hpp
+
+// include/devices/pool_item.hpp:32-40
+struct bad_alloc : public std::bad_alloc {
+    std::string m;
+    explicit bad_alloc(std::string message)
+        : m(std::move(message))
+    {
+    }
+    const char *what() const noexcept override { return m.c_str(); }
+};
+
+// The one device behind every GPU storage and op (stands where GpuDevice + OCLEngine stand in the reference,
+// include/devices/gpu_device.hpp, include/common/oclengine.hpp).  One HIP stream; entry points are serialised
+// by `mutex`, as the reference serialises its queue (src/devices/gpu_device.cpp:195-203).
+struct HipDevice {
+    static HipDevice &Instance();
+    std::recursive_mutex mutex;
+    int64_t device_id;
+    std::string name;
+    // Block until everything queued has finished; a kernel failure surfaces here as std::runtime_error.
+    void finish();
+    // Translate a status code of the C ABI into the exception the reference would throw.
+    static void check(int status);
+
+private:
+    HipDevice();
+};
+
+struct Storage;
+typedef std::shared_ptr<Storage> StoragePtr;
+
+// include/storage/storage.hpp:28-110
+struct Storage : public std::enable_shared_from_this<Storage> {
+    StorageType stype;
+    DeviceTag device;
+    DType dtype;
+    tcapint size;
+
+    Storage(StorageType stp, DeviceTag dtg, DType dtp, tcapint n);
+    virtual ~Storage() {}
+    virtual bool is_sparse() const { return false; }
+    virtual tcapint get_sparse_size() const { return size; }
+    virtual StoragePtr get_ptr() { return shared_from_this(); }
+    virtual int64_t get_device_id() const { return -1; }
+    virtual void FillZeros() = 0;
+    virtual void FillOnes() = 0;
+    virtual StoragePtr cpu() = 0;
+    virtual StoragePtr gpu(int64_t did = -1) = 0;
+};
+
+// include/storage/typed_storage.hpp:30-72 for T = real1
+struct RealStorage : public Storage {
+    using Storage::Storage;
+    virtual real1 operator[](const tcapint &idx) const = 0;
+    virtual void write(const tcapint &idx, const real1 &val) = 0;
+    virtual void add(const tcapint &idx, const real1 &val) = 0;
+    virtual void FillValue(const real1 &v) = 0;
+};
+typedef std::shared_ptr<RealStorage> RealStoragePtr;
+
+// include/storage/cpu_real_storage.hpp
+struct CpuRealStorage : public RealStorage {
+    std::vector<real1> data;
+    explicit CpuRealStorage(tcapint n);
+    explicit CpuRealStorage(const std::vector<real1> &val);
+    real1 operator[](const tcapint &idx) const override;
+    void write(const tcapint &idx, const real1 &val) override;
+    void add(const tcapint &idx, const real1 &val) override;
+    void FillZeros() override;
+    void FillOnes() override;
+    void FillValue(const real1 &v) override;
+    StoragePtr cpu() override { return get_ptr(); }
+    StoragePtr gpu(int64_t did = -1) override; // uploads a copy (src/storage/cpu_real_storage.cpp:19-34)
+};
+
+// include/storage/gpu_real_storage.hpp, include/storage/gpu_storage.hpp:25-60: owns its device buffer
+struct GpuRealStorage : public RealStorage {
+    real1 *buffer;
+    int64_t did;
+    GpuRealStorage(tcapint n, int64_t did = -1);
+    explicit GpuRealStorage(const std::vector<real1> &val, int64_t did = -1);
+    ~GpuRealStorage() override;
+    GpuRealStorage(const GpuRealStorage &) = delete;
+    GpuRealStorage &operator=(const GpuRealStorage &) = delete;
+    int64_t get_device_id() const override { return did; }
+    real1 operator[](const tcapint &idx) const override; // blocking one-element read, as GpuDevice::GetReal
+    void write(const tcapint &idx, const real1 &val) override;
+    void add(const tcapint &idx, const real1 &val) override;
+    void FillZeros() override;
+    void FillOnes() override;
+    void FillValue(const real1 &v) override;
+    StoragePtr cpu() override; // new CpuRealStorage filled by a blocking read (src/storage/gpu_real_storage.cpp:18-23)
+    StoragePtr gpu(int64_t = -1) override { return get_ptr(); }
+};
+
+struct Tensor;
+typedef std::shared_ptr<Tensor> TensorPtr;
+
+// include/tensors/base_tensor.hpp + include/tensors/tensor.hpp, real dense tensors only.  Column-major: dimension 0
+// is the contiguous one, dimensions of size 1 carry stride 0 (base_tensor.hpp:282-292).
+struct Tensor {
+    StoragePtr storage;
+    std::vector<tcapint> shape;
+    std::vector<tcapint> stride;
+    tcapint offset = 0U;
+    bool requires_grad = false; // kept for signature compatibility; there is no autograd on this path
+
+    Tensor() {}
+    Tensor(const std::vector<tcapint> &shp, const std::vector<tcapint> &str, const bool &rg = false,
+        const bool &s = true, const DType &dtype = DType::REAL, const DeviceTag &dtag = DeviceTag::DEFAULT_DEVICE,
+        const int64_t &did = -1);
+    Tensor(const std::vector<real1> &val, const std::vector<tcapint> &shp, const bool &rg = false,
+        const DeviceTag &dtag = DeviceTag::DEFAULT_DEVICE, const int64_t &did = -1);
+    Tensor(const real1 &val, const bool &rg = false, const DeviceTag &dtag = DeviceTag::DEFAULT_DEVICE,
+        const int64_t &did = -1);
+    virtual ~Tensor() {}
+
+    tcapint get_size() const;
+    bool is_scalar() const;
+    bool is_contiguous() const { return is_contiguous(shape, stride); }
+    tcapint get_storage_index(const tcapint &idx) const; // base_tensor.hpp:123-142
+    real1 get_item() const; // value of a one-element tensor (RealScalar::get_item)
+    TensorPtr operator[](const tcapint &idx) const; // view with the LAST dimension fixed (tensor.cpp:277-293)
+    std::vector<real1> to_vector() const; // logical elements in column-major order, read back from any device
+    TensorPtr cast(const DeviceTag &dtag) const; // copy of the storage on the other side, same geometry
+
+    static bool is_contiguous(const std::vector<tcapint> &shp, const std::vector<tcapint> &s);
+    static std::vector<tcapint> full_contiguous_stride(const std::vector<tcapint> &shp);
+
+    static TensorPtr zeros(const std::vector<tcapint> &shape, const bool &rg = false, const bool &s = true,
+        const DType &dtype = DType::REAL, const DeviceTag &dtag = DeviceTag::DEFAULT_DEVICE, const int64_t &did = -1);
+    static TensorPtr contiguous(const TensorPtr a);
+    static TensorPtr reshape(const TensorPtr a, const std::vector<symint> &s);
+    static TensorPtr transpose(const TensorPtr a);
+    static TensorPtr transpose(const TensorPtr a, symint i, symint j);
+    static TensorPtr slice(TensorPtr a, const int64_t &row);
+    static TensorPtr slice(TensorPtr a, int64_t axis, const tcapint &start, const tcapint &length);
+    static TensorPtr softmax(const TensorPtr x, symint axis);
+    static TensorPtr sum(TensorPtr a, symint axis);
+    static TensorPtr max(TensorPtr a, symint axis);
+    static TensorPtr min(TensorPtr a, symint axis);
+    static TensorPtr add(TensorPtr a, TensorPtr b);
+    static TensorPtr sub(TensorPtr a, TensorPtr b);
+    static TensorPtr mul(TensorPtr a, TensorPtr b);
+    static TensorPtr div(TensorPtr a, TensorPtr b);
+    static TensorPtr matmul(TensorPtr a, TensorPtr b);
+};
+
+TensorPtr operator+(TensorPtr left, TensorPtr right);
+TensorPtr operator-(TensorPtr left, TensorPtr right);
+TensorPtr operator*(TensorPtr left, TensorPtr right);
+TensorPtr operator/(TensorPtr left, TensorPtr right);
+TensorPtr operator/(TensorPtr left, real1 right);
+TensorPtr operator*(real1 left, TensorPtr right);
+TensorPtr operator>>(TensorPtr left, TensorPtr right); // matmul(left, right)
+TensorPtr operator<<(TensorPtr right, TensorPtr left); // matmul(left, right)
+
+// Op entry points (include/ops/*.hpp).  Each validates as the reference does and then switches on
+// out.storage->device (src/ops/matmul.cpp:76-84): GPU launches the HIP kernel, anything else throws std::domain_error.
+void matmul(const Tensor &a, const Tensor &b, Tensor &out); // src/ops/matmul.cpp:242-279
+void softmax(const tcapint &index, const Tensor &a, Tensor &out); // src/ops/softmax.cpp:276-287
+void reduce(const tcapint &index, const Tensor &a, Tensor &out); // src/ops/reduce.cpp:342-360
+void max(const tcapint &index, const Tensor &a, Tensor &out); // src/ops/reduce.cpp:362-373
+void min(const tcapint &index, const Tensor &a, Tensor &out); // src/ops/reduce.cpp:375-386
+void add(const Tensor &a, const Tensor &b, Tensor &out); // src/ops/commuting.cpp
+void mul(const Tensor &a, const Tensor &b, Tensor &out);
+void sub(const Tensor &a, const Tensor &b, Tensor &out); // src/ops/sub.cpp
+void div(const Tensor &a, const Tensor &b, Tensor &out); // src/ops/div.cpp:17-20
+void add_in_place(Tensor &a, const Tensor &b); // src/ops/in_place.cpp:17-25
+void triu_fill(Tensor &a, const real1 &val, const tcapint diagonal = 1); // src/ops/triu_fill.cpp:42-59
+
+struct Parameter : public Tensor { // include/tensors/parameter.hpp
+    using Tensor::Tensor;
+};
+typedef std::shared_ptr<Parameter> ParameterPtr;
+
+// include/modules/module.hpp, the members this path uses
+struct Module {
+    virtual ~Module() {}
+    virtual TensorPtr forward(const TensorPtr x) = 0;
+    virtual std::vector<ParameterPtr> parameters() { return {}; }
+    virtual void train() {}
+    virtual void eval() {}
+    virtual void set_max_kv_seq_len(tcapint) {}
+    virtual void reset_cache() {}
+};
+
+// include/modules/linear.hpp:20-41, src/modules/linear.cpp:86-100
+struct Linear : public Module {
+    tcapint in_features;
+    tcapint out_features;
+    ParameterPtr weight; // (in_features, out_features)
+    ParameterPtr bias; // (1, out_features) or null
+
+    Linear()
+        : in_features(0U)
+        , out_features(0U)
+    {
+    }
+    Linear(tcapint in_f, tcapint out_f, bool use_bias = true, bool init_rand = true, DType dtype = DType::REAL,
+        DeviceTag device = DeviceTag::DEFAULT_DEVICE, int64_t device_id = -1);
+    TensorPtr forward(const TensorPtr x) override;
+    std::vector<ParameterPtr> parameters() override;
+};
+typedef std::shared_ptr<Linear> LinearPtr;
+
+// The packed K and V rows of one attention module live in ONE device object (include/weed_hip.h); the two
+// QuantizedKVCache members of the module are views of its two halves.
+struct DeviceKVCache {
+    weed_hip_kv_cache *handle = nullptr;
+    tcapint n_seq = 0U, n_kv_heads = 0U, head_dim = 0U, max_tokens = 0U;
+    DeviceKVCache(int mode, tcapint n_seq_, tcapint n_kv_heads_, tcapint head_dim_, tcapint max_tokens_, int k_bits,
+        int v_bits, int k_sign, int v_sign);
+    ~DeviceKVCache();
+    DeviceKVCache(const DeviceKVCache &) = delete;
+    DeviceKVCache &operator=(const DeviceKVCache &) = delete;
+};
+typedef std::shared_ptr<DeviceKVCache> DeviceKVCachePtr;
+
+// include/modules/multihead_attention.hpp:22-36.  Rows live on the device.  Row r is token r % max_tokens of
+// (sequence, kv head) pair r / max_tokens; a stand-alone cache made with allocate() is a single pair, so its rows
+// are simply 0 .. max_outer-1.  Rows are append-only per pair: write_row(r) must name the next free row (the
+// reference ORs new codes into old bits, src/modules/multihead_attention.cpp:58, so it cannot rewrite a row
+// either).
+struct QuantizedKVCache {
+    std::vector<symint> packed; // Weed's int32 words of the rows written so far, refreshed by sync_packed()
+    real1 block_scale = ONE_R1;
+    tcapint outer = 0U; // rows written so far (stand-alone cache)
+    tcapint d = 0U;
+    tcapint max_outer = 0U;
+    int bits = 0;
+    DeviceKVCachePtr dev; // shared with the sibling cache inside a module
+    int which = 0; // 0: the K half of `dev`, 1: the V half
+
+    int values_per_word() const { return (int)(sizeof(symint) * 8) / bits; }
+    void allocate(const tcapint max_outer_, const tcapint d_, const int bits_);
+    void write_row(const tcapint row, const real1 *vals);
+    void read_row(const tcapint row, real1 *vals) const;
+    void sync_packed();
+};
+
+enum KVCoder { KV_UNIFORM = 0, KV_LLOYDMAX = 1 };
+
+// include/modules/rope.hpp: rotary embedding is not on this path; the type exists so that the attention constructor
+// keeps the reference's argument list, and only a null pointer is accepted.
+struct RoPE;
+typedef std::shared_ptr<RoPE> RoPEPtr;
+
+// include/modules/multihead_attention.hpp:41-173.  Differences, all deliberate:
+//  * W_k / W_v project to num_kv_heads * head_dim features, so grouped-query attention works with the stock
+//    constructor (the reference builds d_model x d_model and needs them swapped by hand);
+//  * tokens are appended in logical order, so prefill followed by decode steps is consistent (the reference's row
+//    order only works for a single call);
+//  * the causal mask honours the cache offset, and set_max_kv_seq_len() survives the first forward();
+//  * rotation_seed makes the rotations reproducible (0 = draw a seed from std::random_device like the reference);
+//    rotations already present in k_rotation / v_rotation at the first forward() are used as given;
+//  * kv_coder selects the reference's uniform coder (default) or the Lloyd-Max coder with k_bits / v_bits / sign
+//    bits; kv_quant_bits serves both K and V in uniform mode as in the reference.
+struct MultiHeadAttention : public Module {
+    symint d_model;
+    symint num_heads;
+    symint num_kv_heads;
+    symint head_dim;
+    real1_f mask_val;
+
+    LinearPtr W_q;
+    LinearPtr W_k;
+    LinearPtr W_v;
+    LinearPtr W_o;
+
+    RoPEPtr rope; // always null
+
+    bool use_kv_cache;
+    TensorPtr k_cache; // float cache (kv_quant_bits == 0)
+    TensorPtr v_cache;
+    tcapint cache_len = 0U;
+    tcapint max_seq_len = 0U;
+
+    int kv_quant_bits = 0;
+    std::vector<real1> k_rotation;
+    std::vector<real1> v_rotation;
+    QuantizedKVCache k_qcache;
+    QuantizedKVCache v_qcache;
+    std::vector<real1> v_rotation_trans;
+
+    // extensions (see above)
+    KVCoder kv_coder = KV_UNIFORM;
+    int k_bits = 0, v_bits = 0; // 0: use kv_quant_bits
+    bool k_sign = false, v_sign = false;
+    bool gqa_blocked = false; // false: kv head = q head % num_kv_heads, the reference's mapping (cpp:291-311)
+    uint32_t rotation_seed = 0U;
+
+    std::vector<ParameterPtr> param_vector;
+
+    MultiHeadAttention(tcapint d_model_, tcapint num_heads_, tcapint num_kv_heads_ = 0, tcapint head_dim_ = 0U,
+        DeviceTag dtag = DEFAULT_DEVICE, RoPEPtr r = nullptr, real1_f mask_val_ = ZERO_R1, const int64_t did = -1,
+        const bool _use_kv_cache = true, int kv_quant_bits_ = 4, bool use_bias = true);
+
+    std::vector<ParameterPtr> parameters() override { return param_vector; }
+    void set_max_kv_seq_len(tcapint m) override { max_seq_len = m; }
+    void reset_cache() override;
+    TensorPtr forward(const TensorPtr x) override;
+
+private:
+    TensorPtr forward_quantized(TensorPtr Q, TensorPtr K, TensorPtr V, symint B, symint T);
+    TensorPtr forward_dense(TensorPtr Q, TensorPtr K, TensorPtr V, symint B, symint T);
+    std::shared_ptr<GpuRealStorage> k_rot_dev, v_rot_dev; // device copies of the rotations
+    void *lens_dev = nullptr; // int32 prefix lengths for multi-token calls
+    size_t lens_cap = 0U;
+
+public:
+    ~MultiHeadAttention() override;
+};
+typedef std::shared_ptr<MultiHeadAttention> MultiHeadAttentionPtr;
+
+} // namespace Weed
