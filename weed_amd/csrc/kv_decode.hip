@@ -46,6 +46,37 @@ __device__ __forceinline__ uint32_t q_head_of(const DecodeParams &p, uint32_t kv
     return p.blocked ? (kvh * p.G + g) : (g * p.Hkv + kvh);
 }
 
+// blk_off[i] = number of 64-token blocks of the sequences before i, blk_off[n_seq] = all of them.  One workgroup of
+// 256 threads: every thread sums a chunk, the chunk sums are scanned in LDS.
+__device__ void block_offsets(const int32_t *__restrict__ lens, uint32_t n_seq, uint32_t *__restrict__ blk_off)
+{
+    __shared__ uint32_t chunk_sum[256];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t per = (n_seq + 255) / 256;
+    const uint32_t i0 = min(tid * per, n_seq), i1 = min(i0 + per, n_seq);
+    uint32_t mine = 0;
+    for (uint32_t i = i0; i < i1; ++i) {
+        mine += ((uint32_t)lens[i] + 63u) >> 6;
+    }
+    chunk_sum[tid] = mine;
+    __syncthreads();
+    for (uint32_t k = 1; k < 256; k <<= 1) {
+        const uint32_t add = tid >= k ? chunk_sum[tid - k] : 0;
+        __syncthreads();
+        chunk_sum[tid] += add;
+        __syncthreads();
+    }
+    uint32_t run = chunk_sum[tid] - mine; // exclusive prefix of this thread's chunk
+    for (uint32_t i = i0; i < i1; ++i) {
+        blk_off[i] = run;
+        run += ((uint32_t)lens[i] + 63u) >> 6;
+    }
+    if (tid == 255) {
+        blk_off[n_seq] = chunk_sum[255];
+    }
+    __syncthreads();
+}
+
 // q_rot[s][h][:] = q[s][h][:] . Rk  (multihead_attention.cpp:276), or a plain gather when rotate == 0.
 // For the matrix-core kernel the rotated query is also scaled by log2(e)/sqrt(d), divided by a power of two that
 // brings it into [-1, 1], and split into fp16 hi + lo halves.
@@ -53,13 +84,17 @@ __global__ void __launch_bounds__(256) prep_q_kernel(const float *__restrict__ q
                                                      const float *__restrict__ rot_t, int rotate,
                                                      float *__restrict__ q_rot, uint16_t *__restrict__ q_hi,
                                                      uint16_t *__restrict__ q_lo, float *__restrict__ q_scale,
-                                                     float *__restrict__ q_sum)
+                                                     float *__restrict__ q_sum, const int32_t *__restrict__ lens,
+                                                     uint32_t n_seq, uint32_t *__restrict__ blk_off)
 {
     __shared__ float qs[256];
     __shared__ float red_max[256];
     __shared__ float red_sum[256];
     const uint32_t h = blockIdx.x, s = blockIdx.y;
     const uint32_t tid = threadIdx.x;
+    if (blk_off && h == 0 && s == 0) {
+        block_offsets(lens, n_seq, blk_off);
+    }
     if (tid < d) {
         qs[tid] = q[(uint64_t)g.off + (uint64_t)s * g.s[0] + (uint64_t)h * g.s[1] + (uint64_t)tid * g.s[2]];
     }
@@ -117,6 +152,99 @@ __device__ __forceinline__ float wave_sum(float v)
         v += __shfl_xor(v, o);
     }
     return v;
+}
+
+constexpr int kRowsPerWg = 4;
+
+// The same as prep_q_kernel for kRowsPerWg (sequence, head) rows per workgroup: thread j owns output coordinate j of
+// every row, so each element of the rotation is read once per workgroup instead of once per row.  Used when there
+// are many rows (batched decode); results are identical (same order of fused multiply-adds).
+__global__ void __launch_bounds__(256) prep_q_rows_kernel(const float *__restrict__ q, Geom3 g, uint32_t Hq, uint32_t d,
+                                                          uint32_t n_rows, const float *__restrict__ rot_t, int rotate,
+                                                          float *__restrict__ q_rot, uint16_t *__restrict__ q_hi,
+                                                          uint16_t *__restrict__ q_lo, float *__restrict__ q_scale,
+                                                          float *__restrict__ q_sum, const int32_t *__restrict__ lens,
+                                                          uint32_t n_seq, uint32_t *__restrict__ blk_off)
+{
+    __shared__ float qs[kRowsPerWg][256];
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t row0 = blockIdx.x * kRowsPerWg;
+    if (blk_off && blockIdx.x == 0) {
+        block_offsets(lens, n_seq, blk_off);
+    }
+#pragma unroll
+    for (int r = 0; r < kRowsPerWg; ++r) {
+        const uint32_t row = row0 + r;
+        float v = 0.0f;
+        if (row < n_rows && tid < d) {
+            const uint32_t s = row / Hq, h = row % Hq;
+            v = q[(uint64_t)g.off + (uint64_t)s * g.s[0] + (uint64_t)h * g.s[1] + (uint64_t)tid * g.s[2]];
+        }
+        qs[r][tid] = v;
+    }
+    __syncthreads();
+    float acc[kRowsPerWg];
+#pragma unroll
+    for (int r = 0; r < kRowsPerWg; ++r) {
+        acc[r] = rotate ? 0.0f : qs[r][tid];
+    }
+    if (rotate && tid < d) {
+        // d is a multiple of 64 here (the host checks); sixty-four independent loads of the rotation are in flight at a time
+        for (uint32_t i0 = 0; i0 < d; i0 += 64) {
+            float x[64];
+#pragma unroll
+            for (int u = 0; u < 64; ++u) {
+                x[u] = rot_t[tid + d * (i0 + u)];
+            }
+#pragma unroll
+            for (int u = 0; u < 64; ++u) {
+#pragma unroll
+                for (int r = 0; r < kRowsPerWg; ++r) {
+                    acc[r] = fmaf(qs[r][i0 + u], x[u], acc[r]);
+                }
+            }
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < kRowsPerWg; ++r) {
+        qs[r][tid] = tid < d ? acc[r] : 0.0f;
+    }
+    __syncthreads();
+    // one wavefront per row from here on
+    for (uint32_t r = wave; r < (uint32_t)kRowsPerWg; r += 4) {
+        const uint32_t row = row0 + r;
+        if (row >= n_rows) {
+            break;
+        }
+        const float k = 1.4426950408889634f / sqrtf((float)d);
+        float mx = 0.0f, sum = 0.0f;
+        for (uint32_t j = lane; j < d; j += 64) {
+            const float qc = qs[r][j] * k;
+            mx = fmaxf(mx, fabsf(qc));
+            sum += qc;
+        }
+        mx = wave_max(mx);
+        // the single-row kernel adds the coordinates pairwise over 256 slots; keep its summation tree: fold 64 lanes
+        sum = wave_sum(sum);
+        int e = 0;
+        (void)frexpf(mx, &e);
+        e = e < -100 ? -100 : (e > 100 ? 100 : e);
+        const float inv = ldexpf(1.0f, -e);
+        for (uint32_t j = lane; j < d; j += 64) {
+            const float a = qs[r][j];
+            const float qn = a * k * inv;
+            const _Float16 hi = (_Float16)qn;
+            const _Float16 lo = (_Float16)(qn - (float)hi);
+            q_rot[(uint64_t)row * d + j] = a;
+            q_hi[(uint64_t)row * d + j] = __builtin_bit_cast(uint16_t, hi);
+            q_lo[(uint64_t)row * d + j] = __builtin_bit_cast(uint16_t, lo);
+        }
+        if (lane == 0) {
+            q_scale[row] = ldexpf(1.0f, e);
+            q_sum[row] = sum;
+        }
+    }
 }
 
 // Generic kernel: any head_dim that is a multiple of 32, any field width, any group size.
@@ -287,15 +415,30 @@ __global__ void __launch_bounds__(kThreads) decode_generic_kernel(DecodeParams p
 
 // Merge the partials of all splits: out = sum_s e^(m_s - M) o_s / sum_s e^(m_s - M) l_s, then multiply by
 // v_rotation^T (multihead_attention.cpp:343-348): out_i = sum_j O_j Rv[i + d*j].
-__global__ void combine_kernel(const float *__restrict__ partials, uint32_t Hq, uint32_t d, uint32_t n_splits,
-                               const float *__restrict__ rv, int unrotate, int log2_domain, float *__restrict__ out,
-                               Geom3 og)
+struct SlotGeom {
+    const uint32_t *blk_off; // null: every (sequence, head) has `max_slots` valid partials
+    uint32_t Hkv, G, unit_blocks;
+    int blocked;
+};
+
+__global__ void combine_kernel(const float *__restrict__ partials, uint32_t Hq, uint32_t d, uint32_t max_slots,
+                               SlotGeom sg, const float *__restrict__ rv, int unrotate, int log2_domain,
+                               float *__restrict__ out, Geom3 og)
 {
     __shared__ float w_s[1024];
     __shared__ float o_sh[256];
+    __shared__ float o_part[1024];
     __shared__ float red[2];
     const uint32_t h = blockIdx.x, s = blockIdx.y, tid = threadIdx.x;
-    const float *base = partials + ((uint64_t)s * Hq + h) * n_splits * (d + 2);
+    const float *base = partials + ((uint64_t)s * Hq + h) * max_slots * (d + 2);
+    uint32_t n_splits = max_slots;
+    if (sg.blk_off) {
+        // the wavefronts whose block runs intersect this head's region, in order
+        const uint32_t first_blk = sg.blk_off[s], nb = sg.blk_off[s + 1] - first_blk;
+        const uint32_t kvh = sg.blocked ? h / sg.G : h % sg.Hkv;
+        const uint32_t begin = first_blk * sg.Hkv + kvh * nb;
+        n_splits = nb ? (begin + nb - 1) / sg.unit_blocks - begin / sg.unit_blocks + 1 : 0;
+    }
     // n_splits <= 1024 is enforced by the host
     if (tid < 64) {
         float mx = -INFINITY;
@@ -317,15 +460,31 @@ __global__ void combine_kernel(const float *__restrict__ partials, uint32_t Hq, 
     }
     __syncthreads();
     const float denom = red[0];
-    if (tid < d) {
+    {
+        // thread groups of d2 (power of two >= d) threads take the partials in turn, then the groups are added up
+        uint32_t d2 = 32;
+        while (d2 < d) {
+            d2 <<= 1;
+        }
+        const uint32_t grp = tid / d2, ngrp = blockDim.x / d2, j = tid % d2;
         float acc = 0.0f;
-        for (uint32_t k = 0; k < n_splits; ++k) {
-            const float w = w_s[k];
-            if (w != 0.0f) {
-                acc = fmaf(w, base[(uint64_t)k * (d + 2) + 2 + tid], acc);
+        if (j < d) {
+            for (uint32_t k = grp; k < n_splits; k += ngrp) {
+                const float w = w_s[k];
+                if (w != 0.0f) {
+                    acc = fmaf(w, base[(uint64_t)k * (d + 2) + 2 + j], acc);
+                }
             }
         }
-        o_sh[tid] = (denom > 0.0f) ? acc / denom : 0.0f;
+        o_part[tid] = acc;
+        __syncthreads();
+        if (tid < d) {
+            float tot = 0.0f;
+            for (uint32_t gI = 0; gI < ngrp; ++gI) {
+                tot += o_part[gI * d2 + tid];
+            }
+            o_sh[tid] = (denom > 0.0f) ? tot / denom : 0.0f;
+        }
     }
     __syncthreads();
     if (tid >= d) {
@@ -341,6 +500,156 @@ __global__ void combine_kernel(const float *__restrict__ partials, uint32_t Hq, 
         r = o_sh[tid];
     }
     out[(uint64_t)og.off + (uint64_t)s * og.s[0] + (uint64_t)h * og.s[1] + (uint64_t)tid * og.s[2]] = r;
+}
+
+// The same as combine_kernel for kRowsPerWg (sequence, head) rows per workgroup and at most 64 partials per row:
+// thread j owns coordinate j of every row, so the rotation is read once per workgroup.
+__global__ void __launch_bounds__(256) combine_rows_kernel(const float *__restrict__ partials, uint32_t Hq, uint32_t d,
+                                                           uint32_t max_slots, uint32_t n_rows, SlotGeom sg,
+                                                           const float *__restrict__ rv, int unrotate, int log2_domain,
+                                                           float *__restrict__ out, Geom3 og)
+{
+    __shared__ float w_s[kRowsPerWg][64];
+    __shared__ float denom_s[kRowsPerWg];
+    __shared__ uint32_t n_s[kRowsPerWg];
+    __shared__ float o_sh[kRowsPerWg][256];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t row0 = blockIdx.x * kRowsPerWg;
+    const uint32_t PS = d + 2;
+    {
+        // one wavefront per row, one lane per partial: weights of the row's partials
+        static_assert(kRowsPerWg == 4, "one 64-lane wavefront per row");
+        const uint32_t r = tid >> 6, l = tid & 63;
+        const uint32_t row = row0 + r;
+        uint32_t n = 0;
+        if (row < n_rows) {
+            n = max_slots;
+            if (sg.blk_off) {
+                const uint32_t s = row / Hq, h = row % Hq;
+                const uint32_t first_blk = sg.blk_off[s], nb = sg.blk_off[s + 1] - first_blk;
+                const uint32_t kvh = sg.blocked ? h / sg.G : h % sg.Hkv;
+                const uint32_t begin = first_blk * sg.Hkv + kvh * nb;
+                n = nb ? (begin + nb - 1) / sg.unit_blocks - begin / sg.unit_blocks + 1 : 0;
+            }
+        }
+        const float *base = partials + (uint64_t)row * max_slots * PS;
+        float m0 = -INFINITY, l0 = 0.0f;
+        if (l < n) {
+            m0 = base[(uint64_t)l * PS];
+            l0 = base[(uint64_t)l * PS + 1];
+        }
+        const float mx = wave_max(m0);
+        const float w0 = (m0 == -INFINITY) ? 0.0f : (log2_domain ? exp2f(m0 - mx) : expf(m0 - mx));
+        const float sum = wave_sum(w0 * l0);
+        w_s[r][l] = w0;
+        if (l == 0) {
+            denom_s[r] = sum;
+            n_s[r] = n;
+        }
+    }
+    __syncthreads();
+    {
+        // Thread groups of d2 (power of two >= d) threads take the partials in turn.  The first four partials of
+        // every group and row are fetched without branches, so that all loads of all rows are in flight together.
+        uint32_t d2 = 32;
+        while (d2 < d) {
+            d2 <<= 1;
+        }
+        const uint32_t grp = tid / d2, ngrp = 256 / d2, j = tid % d2;
+        const bool col_ok = j < d;
+        float acc[kRowsPerWg];
+        float x[kRowsPerWg][4];
+#pragma unroll
+        for (int r = 0; r < kRowsPerWg; ++r) {
+            const float *base = partials + (uint64_t)(row0 + r) * max_slots * PS + 2 + j;
+            const uint32_t n = n_s[r];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const uint32_t k = grp + u * ngrp;
+                x[r][u] = (col_ok && k < n) ? base[(uint64_t)k * PS] : 0.0f;
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < kRowsPerWg; ++r) {
+            const float *base = partials + (uint64_t)(row0 + r) * max_slots * PS + 2 + j;
+            const uint32_t n = n_s[r];
+            float a = 0.0f;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const uint32_t k = grp + u * ngrp;
+                a = fmaf(k < n ? w_s[r][k] : 0.0f, x[r][u], a);
+            }
+            if (col_ok) {
+                for (uint32_t k = grp + 4 * ngrp; k < n; k += ngrp) {
+                    a = fmaf(w_s[r][k], base[(uint64_t)k * PS], a);
+                }
+            }
+            acc[r] = a;
+        }
+        // add the groups up through LDS (o_sh doubles as the staging area: [row][group * d2 + j])
+#pragma unroll
+        for (int r = 0; r < kRowsPerWg; ++r) {
+            o_sh[r][tid] = acc[r];
+        }
+        __syncthreads();
+        float tot[kRowsPerWg];
+#pragma unroll
+        for (int r = 0; r < kRowsPerWg; ++r) {
+            float t = 0.0f;
+            if (tid < d) {
+                for (uint32_t gI = 0; gI < ngrp; ++gI) {
+                    t += o_sh[r][gI * d2 + tid];
+                }
+                const float den = denom_s[r];
+                t = den > 0.0f ? t / den : 0.0f;
+            }
+            tot[r] = t;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < kRowsPerWg; ++r) {
+            o_sh[r][tid] = tot[r];
+        }
+    }
+    __syncthreads();
+    if (tid >= d) {
+        return;
+    }
+    float res[kRowsPerWg];
+    if (unrotate) {
+#pragma unroll
+        for (int r = 0; r < kRowsPerWg; ++r) {
+            res[r] = 0.0f;
+        }
+        // d is a multiple of 64 here (the host checks); sixty-four independent loads of the rotation are in flight at a time
+        for (uint32_t j0 = 0; j0 < d; j0 += 64) {
+            float x[64];
+#pragma unroll
+            for (int u = 0; u < 64; ++u) {
+                x[u] = rv[tid + d * (j0 + u)];
+            }
+#pragma unroll
+            for (int u = 0; u < 64; ++u) {
+#pragma unroll
+                for (int r = 0; r < kRowsPerWg; ++r) {
+                    res[r] = fmaf(o_sh[r][j0 + u], x[u], res[r]);
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < kRowsPerWg; ++r) {
+            res[r] = o_sh[r][tid];
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < kRowsPerWg; ++r) {
+        const uint32_t row = row0 + r;
+        if (row < n_rows) {
+            const uint32_t s = row / Hq, h = row % Hq;
+            out[(uint64_t)og.off + (uint64_t)s * og.s[0] + (uint64_t)h * og.s[1] + (uint64_t)tid * og.s[2]] = res[r];
+        }
+    }
 }
 
 // `lens_dev` (optional): attend over these per-sequence lengths instead of the cached ones.
@@ -365,18 +674,26 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
     }
     const uint32_t G = Hq / Hkv;
     const bool use_mfma = mfma_decode_supported(d, c->k.w, c->v.w, G);
-    uint32_t n_splits, split_tokens = 0, blocks_per_split = 0;
+    uint32_t n_splits, split_tokens = 0;
+    uint32_t total_blocks = 0, unit_blocks = 1;
     if (use_mfma) {
-        // a workgroup's four wavefronts interleave over its 64-token blocks; aim for ~6 workgroups per compute unit
-        const uint32_t nblk = std::max(1u, (max_len + 63) / 64);
-        uint32_t target_wgs = 1024u;
+        // every wavefront takes an equal run of 64-token blocks from the list of all regions' blocks; aim for three
+        // workgroups (twelve wavefronts) per compute unit, all resident at once
+        uint64_t blocks = 0;
+        for (int32_t l : c->lens) {
+            blocks += ((uint32_t)l + 63u) >> 6;
+        }
+        blocks *= Hkv;
+        WEED_HIP_REQUIRE(blocks < (1ull << 32), "%s: too many cached tokens for one launch", fn);
+        total_blocks = (uint32_t)blocks;
+        uint32_t target_wgs = 768u;
         if (const char *env = std::getenv("WEED_HIP_DECODE_WGS")) {
             target_wgs = (uint32_t)std::max(1, std::atoi(env)); // tuning knob
         }
-        const uint32_t want = std::max(1u, (target_wgs + S * Hkv - 1) / (S * Hkv));
-        blocks_per_split = std::max(4u, (nblk + want - 1) / want);
-        blocks_per_split = (blocks_per_split + 3) / 4 * 4;
-        n_splits = (nblk + blocks_per_split - 1) / blocks_per_split;
+        const uint32_t target_units = target_wgs * kMfmaDecodeWaves;
+        unit_blocks = std::max(1u, (total_blocks + target_units - 1) / target_units);
+        const uint32_t nblk = (max_len + 63) / 64;
+        n_splits = (nblk + unit_blocks - 1) / unit_blocks + 1; // partial slots per (sequence, head)
     } else {
         // split the context so that the launch has a few workgroups per compute unit
         const uint32_t target_wgs = 2048;
@@ -394,7 +711,8 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
     const size_t h_bytes = (sizeof(uint16_t) * n_q + 15) / 16 * 16;
     const size_t s_bytes = (sizeof(float) * (size_t)S * Hq + 15) / 16 * 16;
     const size_t part_bytes = sizeof(float) * (size_t)S * Hq * n_splits * (d + 2);
-    const size_t need = q_bytes + 2 * h_bytes + 2 * s_bytes + part_bytes;
+    const size_t off_bytes = (sizeof(uint32_t) * ((size_t)S + 1) + 15) / 16 * 16;
+    const size_t need = q_bytes + 2 * h_bytes + 2 * s_bytes + off_bytes + part_bytes;
     if (need > c->dec_ws_bytes) {
         WEED_HIP_CHECK(hipStreamSynchronize(stream()));
         (void)hipFree(c->dec_ws);
@@ -411,12 +729,22 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
     uint16_t *q_lo = reinterpret_cast<uint16_t *>(wsp + q_bytes + h_bytes);
     float *q_scale = reinterpret_cast<float *>(wsp + q_bytes + 2 * h_bytes);
     float *q_sum = reinterpret_cast<float *>(wsp + q_bytes + 2 * h_bytes + s_bytes);
-    float *partials = reinterpret_cast<float *>(wsp + q_bytes + 2 * h_bytes + 2 * s_bytes);
+    uint32_t *blk_off = reinterpret_cast<uint32_t *>(wsp + q_bytes + 2 * h_bytes + 2 * s_bytes);
+    float *partials = reinterpret_cast<float *>(wsp + q_bytes + 2 * h_bytes + 2 * s_bytes + off_bytes);
 
     Geom3 qg = { q_off, { q_stride[0], q_stride[1], q_stride[2] } };
     Geom3 og = { o_off, { o_stride[0], o_stride[1], o_stride[2] } };
-    prep_q_kernel<<<dim3(Hq, S), 256, 0, stream()>>>(q_dev, qg, Hq, d, c->k.rot_t, rot_q ? 1 : 0, q_rot, q_hi, q_lo,
-                                                     q_scale, q_sum);
+    const uint32_t n_rows = S * Hq;
+    // the multi-row kernels pay off with many (sequence, head) rows; their rotation loops step by 64
+    const bool many_rows = n_rows >= 512 && d % 64 == 0;
+    if (many_rows) {
+        prep_q_rows_kernel<<<(n_rows + kRowsPerWg - 1) / kRowsPerWg, 256, 0, stream()>>>(
+            q_dev, qg, Hq, d, n_rows, c->k.rot_t, rot_q ? 1 : 0, q_rot, q_hi, q_lo, q_scale, q_sum, c->lens_dev, S,
+            use_mfma ? blk_off : nullptr);
+    } else {
+        prep_q_kernel<<<dim3(Hq, S), 256, 0, stream()>>>(q_dev, qg, Hq, d, c->k.rot_t, rot_q ? 1 : 0, q_rot, q_hi, q_lo,
+                                                         q_scale, q_sum, c->lens_dev, S, use_mfma ? blk_off : nullptr);
+    }
     WEED_HIP_LAUNCH_CHECK();
 
     if (use_mfma) {
@@ -434,10 +762,15 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         mp.q_scale = q_scale;
         mp.q_sum = q_sum;
         mp.partials = partials;
-        mp.n_splits = n_splits;
-        mp.blocks_per_split = blocks_per_split;
+        mp.blk_off = blk_off;
+        mp.n_seq = S;
+        mp.total_blocks = total_blocks;
+        mp.unit_blocks = unit_blocks;
+        mp.max_slots = n_splits;
         ProfileScope prof("kv_decode_attn");
-        WEED_HIP_TRY(launch_mfma_decode(mp, d, S, stream()));
+        if (total_blocks) {
+            WEED_HIP_TRY(launch_mfma_decode(mp, d, stream()));
+        }
     } else {
         DecodeParams p;
         p.k = side_params(c, 0);
@@ -459,8 +792,15 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
     }
     {
         ProfileScope prof("kv_decode_combine");
-        combine_kernel<<<dim3(Hq, S), 256, 0, stream()>>>(partials, Hq, d, n_splits, c->v.rot, unrot ? 1 : 0,
-                                                          use_mfma ? 1 : 0, out_dev, og);
+        const SlotGeom sg = { use_mfma ? blk_off : nullptr, Hkv, G, unit_blocks,
+                              gqa_mapping == WEED_HIP_GQA_BLOCKED ? 1 : 0 };
+        if (many_rows && n_splits <= 64) {
+            combine_rows_kernel<<<(n_rows + kRowsPerWg - 1) / kRowsPerWg, 256, 0, stream()>>>(
+                partials, Hq, d, n_splits, n_rows, sg, c->v.rot, unrot ? 1 : 0, use_mfma ? 1 : 0, out_dev, og);
+        } else {
+            combine_kernel<<<dim3(Hq, S), n_splits > 16 ? 1024 : 256, 0, stream()>>>(
+                partials, Hq, d, n_splits, sg, c->v.rot, unrot ? 1 : 0, use_mfma ? 1 : 0, out_dev, og);
+        }
         WEED_HIP_LAUNCH_CHECK();
     }
     return WEED_HIP_OK;

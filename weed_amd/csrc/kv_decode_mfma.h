@@ -15,11 +15,18 @@ struct MfmaParams {
     const uint16_t *q_lo;   // [n_seq][Hq][d] fp16 bits: what the high half misses
     const float *q_scale;   // [n_seq][Hq] power of two the query was divided by
     const float *q_sum;     // [n_seq][Hq] sum of the scaled query (for the uniform coder's offset term)
-    float *partials;        // [n_seq][Hq][n_splits][d + 2]: m (log2 units), l, o[d]
-    uint32_t n_splits, blocks_per_split;
+    float *partials;        // [n_seq][Hq][max_slots][d + 2]: m (log2 units), l, o[d]
+    // Work partition: the 64-token blocks of all (sequence, kv head) regions form one list, region after region
+    // (sequence-major); wavefront u of the launch takes blocks [u * unit_blocks, (u + 1) * unit_blocks).
+    const uint32_t *blk_off; // [n_seq + 1] prefix sums of the sequences' block counts (cached lengths)
+    uint32_t n_seq;
+    uint32_t total_blocks;   // blk_off[n_seq] * Hkv
+    uint32_t unit_blocks;
+    uint32_t max_slots;      // partial slots per (sequence, head): most wavefronts that can touch one region
 };
 
 bool mfma_decode_supported(uint32_t d, uint32_t wk, uint32_t wv, uint32_t G);
-int launch_mfma_decode(const MfmaParams &p, uint32_t d, uint32_t n_seq, hipStream_t s);
+int launch_mfma_decode(const MfmaParams &p, uint32_t d, hipStream_t s);
+constexpr uint32_t kMfmaDecodeWaves = 4; // wavefronts per workgroup of the matrix-core kernel
 
 } // namespace weedhip

@@ -19,6 +19,16 @@
 
 #include <type_traits>
 
+#ifndef WEED_EXP_KORDER
+#define WEED_EXP_KORDER 1
+#endif
+#ifndef WEED_EXP_KROLL
+#define WEED_EXP_KROLL 0
+#endif
+#ifndef WEED_EXP_VROLL
+#define WEED_EXP_VROLL 0
+#endif
+
 using namespace weedhip;
 using namespace weedkv;
 
@@ -29,7 +39,7 @@ typedef float float4v __attribute__((ext_vector_type(4)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
 
-constexpr int kWaves = 4;
+constexpr int kWaves = (int)kMfmaDecodeWaves;
 
 __device__ __forceinline__ uint32_t pack_half2(float a, float b)
 {
@@ -43,7 +53,11 @@ template <int N> __device__ __forceinline__ void load_dwords(const uint8_t *p, u
     if constexpr (N % 4 == 0) {
 #pragma unroll
         for (int i = 0; i < N / 4; ++i) {
+#ifdef WEED_EXP_INTERLEAVE
+            const uint4v v = *reinterpret_cast<const uint4v *>(p + 1024 * i);
+#else
             const uint4v v = *reinterpret_cast<const uint4v *>(p + 16 * i);
+#endif
             x[4 * i] = v.x;
             x[4 * i + 1] = v.y;
             x[4 * i + 2] = v.z;
@@ -86,7 +100,11 @@ typedef const uint32_t __attribute__((address_space(3))) *lds_u32_ptr;
 
 __device__ __forceinline__ uint32_t lds_read(uint32_t byte_addr)
 {
+#ifdef WEED_EXP_NOLDS
+    return byte_addr;
+#else
     return *reinterpret_cast<lds_u32_ptr>((uintptr_t)byte_addr);
+#endif
 }
 
 // `lane_base` = LDS byte address of the table + (lane % 32) * 4.
@@ -108,6 +126,45 @@ template <int I, int N, typename F> __device__ __forceinline__ void static_for(F
         f(std::integral_constant<int, I>{});
         static_for<I + 1, N>(f);
     }
+}
+
+// The lane's run is loaded in chunks of 16 bytes (8 when N is not a multiple of 4).  chunk_last_item<N, W>(c) is the
+// last 8-field item (W bytes each) that reads chunk c; after its lookups the chunk's registers can be refilled.
+template <int N> constexpr int chunk_dwords() { return N % 4 == 0 ? 4 : 2; }
+template <int N> constexpr int chunk_count() { return N / chunk_dwords<N>(); }
+template <int N, int W> constexpr int chunk_last_item(int c)
+{
+    const int last_byte = 4 * chunk_dwords<N>() * (c + 1) - 1;
+    const int items = 4 * N / W;
+    return last_byte / W < items ? last_byte / W : items - 1;
+}
+template <int N, int C> __device__ __forceinline__ void load_chunk(const uint8_t *p, uint32_t (&x)[N])
+{
+    if constexpr (N % 4 == 0) {
+#ifdef WEED_EXP_INTERLEAVE
+        const uint4v v = *reinterpret_cast<const uint4v *>(p + 1024 * C);
+#else
+        const uint4v v = *reinterpret_cast<const uint4v *>(p + 16 * C);
+#endif
+        x[4 * C] = v.x;
+        x[4 * C + 1] = v.y;
+        x[4 * C + 2] = v.z;
+        x[4 * C + 3] = v.w;
+    } else {
+        const uint2v v = *reinterpret_cast<const uint2v *>(p + 8 * C);
+        x[2 * C] = v.x;
+        x[2 * C + 1] = v.y;
+    }
+}
+// Refill every chunk whose last reader is item I.
+template <int N, int W, int I> __device__ __forceinline__ void refill_after_item(const uint8_t *p, uint32_t (&x)[N])
+{
+    static_for<0, chunk_count<N>()>([&](auto cc) {
+        constexpr int c = decltype(cc)::value;
+        if constexpr (chunk_last_item<N, W>(c) == I) {
+            load_chunk<N, c>(p, x);
+        }
+    });
 }
 
 __device__ __forceinline__ float4v mfma16(half8 a, half8 b, float4v c)
@@ -174,12 +231,6 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_kernel(MfmaParams 
 
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t c = lane & 15, g = lane >> 4;
-    const uint32_t split = blockIdx.x, kvh = blockIdx.y, seq = blockIdx.z;
-    const uint32_t L = (uint32_t)p.lens[seq];
-    const uint32_t nblk = (L + 63) >> 6;
-    const uint32_t b0 = split * p.blocks_per_split;
-    const uint32_t b1 = min(nblk, b0 + p.blocks_per_split);
-    const uint64_t region = (uint64_t)seq * p.Hkv + kvh;
     constexpr bool lloyd = LLOYD;
 
     // ---- pair tables: entry e, replica i at dword e*32 + i; a lane always reads replica lane%32.  The 2^w fp16
@@ -202,6 +253,46 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_kernel(MfmaParams 
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint32_t *)lds;
     const uint32_t kbase = lds_base + (lane & 31) * 4;
     const uint32_t vbase = kbase + KT * 4;
+
+    // ---- this wavefront's share of the launch: a contiguous run of `unit_blocks` 64-token blocks of the global block
+    //      list (all blocks of (sequence 0, kv head 0), then (0, 1), ...).  A run is cut into segments at region
+    //      boundaries; every segment leaves one partial in the slot `unit - first unit of the region`. ----
+    const uint32_t unit = __builtin_amdgcn_readfirstlane(blockIdx.x * kWaves + wave);
+    uint32_t g0 = unit * p.unit_blocks;
+    const uint32_t g1 = min(g0 + p.unit_blocks, p.total_blocks);
+    if (g0 >= g1) {
+        return; // no barrier follows
+    }
+    uint32_t seq;
+    {
+        // largest s with blk_off[s] * Hkv <= g0 (sequences without tokens share their offset with the next one)
+        uint32_t lo = 0, hi = p.n_seq;
+        while (hi - lo > 1) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if (p.blk_off[mid] * p.Hkv <= g0) {
+                lo = mid;
+            } else {
+                hi = mid;
+            }
+        }
+        seq = __builtin_amdgcn_readfirstlane(lo);
+    }
+    while (g0 < g1) {
+    const uint32_t seq_first = p.blk_off[seq];
+    const uint32_t nb_cap = p.blk_off[seq + 1] - seq_first; // blocks the cached length of this sequence spans
+    if (nb_cap == 0) {
+        ++seq;
+        continue;
+    }
+    const uint32_t rel = g0 - seq_first * p.Hkv;
+    const uint32_t kvh = rel / nb_cap;
+    const uint32_t b0 = rel - kvh * nb_cap;
+    const uint32_t seg = min(nb_cap - b0, g1 - g0);
+    const uint32_t slot = unit - (seq_first * p.Hkv + kvh * nb_cap) / p.unit_blocks;
+    const uint32_t L = (uint32_t)p.lens[seq]; // may be shorter than the cached length (prefix attention)
+    const uint32_t b1 = min(b0 + seg, (L + 63) >> 6);
+    const uint64_t region = (uint64_t)seq * p.Hkv + kvh;
+    g0 += seg;
 
     // ---- query operand.  The score instruction has 16 columns.  With GP <= 8 the fp16 high halves of the GP heads sit
     //      in columns [0, GP) and the low halves in [GP, 2GP), so ONE instruction per item yields both partial scores
@@ -258,8 +349,13 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_kernel(MfmaParams 
         O[jb] = float4v{ 0.0f, 0.0f, 0.0f, 0.0f };
     }
 
+#ifdef WEED_EXP_INTERLEAVE
+    const uint8_t *kreg = p.k.fields + region * p.k.region_bytes + (uint64_t)lane * 16;
+    const uint8_t *vreg = p.v.fields + region * p.v.region_bytes + (uint64_t)lane * 16;
+#else
     const uint8_t *kreg = p.k.fields + region * p.k.region_bytes + (uint64_t)lane * (4 * NK);
     const uint8_t *vreg = p.v.fields + region * p.v.region_bytes + (uint64_t)lane * (4 * NV);
+#endif
     const float *ka = lloyd ? p.k.alpha + region * p.padded + 16 * tile_in_set + 4 * g : nullptr;
     const float *va = lloyd ? p.v.alpha + region * p.padded + 16 * tile_in_set + 4 * g : nullptr;
 
@@ -269,43 +365,121 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_kernel(MfmaParams 
     uint32_t kraw[NK], vraw[NV];
     float4v ak[NSETS], av[NSETS];
 
-    auto load_k = [&](uint32_t blk) {
-        load_dwords<NK>(kreg + (uint64_t)blk * (8u * D * WK), kraw);
+    auto load_k_scales = [&](uint32_t blk) {
 #pragma unroll
         for (int s = 0; s < NSETS; ++s) {
+#ifdef WEED_EXP_NOALPHA
+            if constexpr (false) {
+#else
             if constexpr (lloyd) {
+#endif
                 ak[s] = *reinterpret_cast<const float4v *>(ka + blk * 64 + 16 * TPS * s);
             } else {
                 ak[s] = float4v{ p.k.alpha_const, p.k.alpha_const, p.k.alpha_const, p.k.alpha_const };
             }
         }
     };
-    auto load_v = [&](uint32_t blk) {
-        load_dwords<NV>(vreg + (uint64_t)blk * (8u * D * WV), vraw);
+    auto load_v_scales = [&](uint32_t blk) {
 #pragma unroll
         for (int s = 0; s < NSETS; ++s) {
+#ifdef WEED_EXP_NOALPHA
+            if constexpr (false) {
+#else
             if constexpr (lloyd) {
+#endif
                 av[s] = *reinterpret_cast<const float4v *>(va + blk * 64 + 16 * TPS * s);
             } else {
                 av[s] = float4v{ 1.0f, 1.0f, 1.0f, 1.0f };
             }
         }
     };
+    bool first_load = true;
+    auto load_k = [&](uint32_t blk) {
+#ifdef WEED_EXP_NOLOAD
+        if (first_load)
+#endif
+        {
+            load_dwords<NK>(kreg + (uint64_t)blk * (8u * D * WK), kraw);
+            load_k_scales(blk);
+        }
+    };
+    auto load_v = [&](uint32_t blk) {
+#ifdef WEED_EXP_NOLOAD
+        if (first_load)
+#endif
+        {
+            load_dwords<NV>(vreg + (uint64_t)blk * (8u * D * WV), vraw);
+            load_v_scales(blk);
+        }
+        first_load = false;
+    };
 
+#ifdef WEED_EXP_MEMONLY
     auto process_block = [&](uint32_t blk, uint32_t next_blk) {
+        (void)blk;
+        const uint8_t *knext = kreg + (uint64_t)next_blk * (8u * D * WK);
+        const uint8_t *vnext = vreg + (uint64_t)next_blk * (8u * D * WV);
+        uint32_t acc = 0;
+        static_for<0, chunk_count<NK>()>([&](auto cc) {
+            constexpr int c = decltype(cc)::value;
+#pragma unroll
+            for (int k = 0; k < chunk_dwords<NK>(); ++k) {
+                acc ^= kraw[chunk_dwords<NK>() * c + k];
+            }
+            if constexpr (WEED_EXP_KROLL) {
+                load_chunk<NK, c>(knext, kraw);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        acc ^= __float_as_uint(ak[0][0]);
+        if constexpr (WEED_EXP_KROLL) {
+            load_k_scales(next_blk);
+        } else {
+            load_k(next_blk);
+        }
+        static_for<0, chunk_count<NV>()>([&](auto cc) {
+            constexpr int c = decltype(cc)::value;
+#pragma unroll
+            for (int k = 0; k < chunk_dwords<NV>(); ++k) {
+                acc ^= vraw[chunk_dwords<NV>() * c + k];
+            }
+            if constexpr (WEED_EXP_VROLL) {
+                load_chunk<NV, c>(vnext, vraw);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        acc ^= __float_as_uint(av[0][0]);
+        if constexpr (WEED_EXP_VROLL) {
+            load_v_scales(next_blk);
+        } else {
+            load_v(next_blk);
+        }
+        O[0][0] += (float)(acc & 1u);
+    };
+    auto process_block_unused = [&](uint32_t blk, uint32_t next_blk) {
+#else
+    auto process_block = [&](uint32_t blk, uint32_t next_blk) {
+#endif
         // ---- S[t] = K_tile . q: rows = tokens 16t + (lane%16), contraction over the lane groups' coordinates ----
         // Lookups run two items ahead of the matrix instructions that consume them.
         float4v S[4];
         {
+            // Items are taken in memory order (tile after tile), so the leading chunks of the lane's run retire early
+            // and are refilled with the next block's bytes while this block is still being worked on.
             constexpr int NI = 4 * KS;
-            half8 a0 = dequant_item<WK, NK, 0>(kraw, kbase);
-            half8 a1 = dequant_item<WK, NK, (1 % 4) * KS + 1 / 4>(kraw, kbase);
+            const uint8_t *knext = kreg + (uint64_t)next_blk * (8u * D * WK);
+            auto item_of = [](int i) constexpr { return WEED_EXP_KORDER ? i : (i % 4) * KS + i / 4; };
+            half8 a0 = dequant_item<WK, NK, item_of(0)>(kraw, kbase);
+            half8 a1 = dequant_item<WK, NK, item_of(1)>(kraw, kbase);
             static_for<0, NI>([&](auto ic) {
                 constexpr int i = decltype(ic)::value;
-                constexpr int ks = i / 4, t = i % 4;
+                constexpr int t = WEED_EXP_KORDER ? i / KS : i % 4, ks = WEED_EXP_KORDER ? i % KS : i / 4;
                 half8 a2 = a1;
                 if constexpr (i + 2 < NI) {
-                    a2 = dequant_item<WK, NK, ((i + 2) % 4) * KS + (i + 2) / 4>(kraw, kbase);
+                    a2 = dequant_item<WK, NK, item_of(i + 2)>(kraw, kbase);
+                    if constexpr (WEED_EXP_KORDER && WEED_EXP_KROLL) {
+                        refill_after_item<NK, WK, i + 2>(knext, kraw);
+                    }
                 }
                 // keep the look-ahead lookups ahead of this item's matrix instruction
                 __builtin_amdgcn_sched_barrier(0);
@@ -349,7 +523,11 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_kernel(MfmaParams 
                 C[s][r] = fmaf(v, ak[s][r] * qscale, betaq);
             }
         }
-        load_k(next_blk); // the K buffer is free again
+        if constexpr (WEED_EXP_KORDER && WEED_EXP_KROLL) {
+            load_k_scales(next_blk); // the row scales are free again (the packed fields were refilled on the way)
+        } else {
+            load_k(next_blk);
+        }
         if (blk * 64 + 64 > L) {
 #pragma unroll
             for (int s = 0; s < NSETS; ++s) {
@@ -466,6 +644,7 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_kernel(MfmaParams 
         }
         {
             constexpr int NI = 2 * JB;
+            const uint8_t *vnext = vreg + (uint64_t)next_blk * (8u * D * WV);
             half8 b0v = dequant_item<WV, NV, 0>(vraw, vbase);
             half8 b1v = dequant_item<WV, NV, 1>(vraw, vbase);
             static_for<0, NI>([&](auto ic) {
@@ -474,6 +653,9 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_kernel(MfmaParams 
                 half8 b2v = b1v;
                 if constexpr (i + 2 < NI) {
                     b2v = dequant_item<WV, NV, i + 2>(vraw, vbase);
+                    if constexpr (WEED_EXP_VROLL) {
+                        refill_after_item<NV, WV, i + 2>(vnext, vraw);
+                    }
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 O[jb] = mfma16(pa[u][0], b0v, O[jb]);
@@ -484,32 +666,34 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_kernel(MfmaParams 
                 b1v = b2v;
             });
         }
-        load_v(next_blk); // the V buffer is free again
+        if constexpr (WEED_EXP_VROLL) {
+            load_v_scales(next_blk);
+        } else {
+            load_v(next_blk);
+        }
     };
 
     // ---- main loop.  The refills are unconditional (the next block index is clamped to the last block of the split)
     //      so that the loop body has no branch around loads and outstanding loads can be counted exactly. ----
     {
-        uint32_t blk = b0 + wave;
+        uint32_t blk = b0;
         if (blk < b1) {
             const uint32_t last = b1 - 1;
             load_k(blk);
             load_v(blk);
-            for (; blk < b1; blk += kWaves) {
-                process_block(blk, min(blk + kWaves, last));
+            for (; blk < b1; ++blk) {
+                process_block(blk, min(blk + 1, last));
             }
         }
     }
 
-    // ---- per-wave results -> LDS (the tables are no longer needed), then one merged partial per head ----
+    // ---- this segment's un-normalised partial (m, l, o[d]) per query head, straight to global memory ----
     const float l_head = head_sum<GP>(l_run) * unscale; // every lane of a head now holds its denominator
     float lrow[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         lrow[r] = __shfl(l_head, (int)(4 * g + r));
     }
-    __syncthreads();
-    float *ws = reinterpret_cast<float *>(lds); // [wave][head slot 0..15][D + 2]
     constexpr int PS = D + 2;
     const float o_mul = unscale * (lloyd ? 1.0f : p.v.alpha_const);
     if constexpr (PACKED) {
@@ -526,7 +710,8 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_kernel(MfmaParams 
     for (int r = 0; r < 4; ++r) {
         const uint32_t hs = 4 * g + r;
         if (hs < p.G) {
-            float *dst = ws + ((size_t)wave * 16 + hs) * PS;
+            const uint32_t head = p.blocked ? kvh * p.G + hs : hs * p.Hkv + kvh;
+            float *dst = p.partials + (((uint64_t)seq * p.Hq + head) * p.max_slots + slot) * PS;
 #pragma unroll
             for (int jb = 0; jb < JB; ++jb) {
                 // uniform coder: value = step * (code + 0.5) + lo, so add lo * sum(p)
@@ -536,40 +721,20 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_kernel(MfmaParams 
     }
     if (g == 0 && c < p.G) {
         // lane c of row 0 holds head c (c < GP)
-        float *dst = ws + ((size_t)wave * 16 + c) * PS;
+        const uint32_t head = p.blocked ? kvh * p.G + c : c * p.Hkv + kvh;
+        float *dst = p.partials + (((uint64_t)seq * p.Hq + head) * p.max_slots + slot) * PS;
         dst[0] = m_run;
         dst[1] = l_head;
     }
-    __syncthreads();
-    for (uint32_t idx = tid; idx < p.G * (uint32_t)PS; idx += 64 * kWaves) {
-        const uint32_t hs = idx / PS, j = idx % PS;
-        float mw[kWaves], mx = -INFINITY;
-#pragma unroll
-        for (int w = 0; w < kWaves; ++w) {
-            mw[w] = ws[((size_t)w * 16 + hs) * PS];
-            mx = fmaxf(mx, mw[w]);
-        }
-        float val;
-        if (j == 0) {
-            val = mx;
-        } else {
-            val = 0.0f;
-#pragma unroll
-            for (int w = 0; w < kWaves; ++w) {
-                const float f = (mw[w] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(mw[w] - mx);
-                val = fmaf(f, ws[((size_t)w * 16 + hs) * PS + j], val);
-            }
-        }
-        const uint32_t head = p.blocked ? kvh * p.G + hs : hs * p.Hkv + kvh;
-        p.partials[(((uint64_t)seq * p.Hq + head) * p.n_splits + split) * PS + j] = val;
+    if (kvh + 1 == p.Hkv && b0 + seg == nb_cap) {
+        ++seq;
     }
+    } // segments
 }
 
 template <int D, int WK, int WV, int GP, bool LLOYD> int launch_gp(const MfmaParams &p, dim3 grid, hipStream_t s)
 {
-    constexpr size_t tab_bytes = (((size_t)1 << (2 * WK)) + ((size_t)1 << (2 * WV))) * 32 * sizeof(uint32_t);
-    constexpr size_t merge_bytes = (size_t)kWaves * 16 * (D + 2) * sizeof(float);
-    constexpr size_t smem = tab_bytes > merge_bytes ? tab_bytes : merge_bytes;
+    constexpr size_t smem = (((size_t)1 << (2 * WK)) + ((size_t)1 << (2 * WV))) * 32 * sizeof(uint32_t);
     static bool configured = false;
     if (!configured) {
         WEED_HIP_CHECK(hipFuncSetAttribute((const void *)decode_mfma_kernel<D, WK, WV, GP, LLOYD>,
