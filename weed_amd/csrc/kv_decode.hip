@@ -677,8 +677,8 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
     uint32_t n_splits, split_tokens = 0;
     uint32_t total_blocks = 0, unit_blocks = 1;
     if (use_mfma) {
-        // every wavefront takes an equal run of 64-token blocks from the list of all regions' blocks; aim for three
-        // workgroups (twelve wavefronts) per compute unit, all resident at once
+        // every wavefront takes an equal run of 64-token blocks from the list of all regions' blocks; as many
+        // wavefronts as the device holds at once
         uint64_t blocks = 0;
         for (int32_t l : c->lens) {
             blocks += ((uint32_t)l + 63u) >> 6;
@@ -686,11 +686,10 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         blocks *= Hkv;
         WEED_HIP_REQUIRE(blocks < (1ull << 32), "%s: too many cached tokens for one launch", fn);
         total_blocks = (uint32_t)blocks;
-        uint32_t target_wgs = 768u;
-        if (const char *env = std::getenv("WEED_HIP_DECODE_WGS")) {
-            target_wgs = (uint32_t)std::max(1, std::atoi(env)); // tuning knob
+        uint32_t target_units = mfma_decode_wavefronts(G);
+        if (const char *env = std::getenv("WEED_HIP_DECODE_WAVES")) {
+            target_units = (uint32_t)std::max(1, std::atoi(env)); // tuning knob
         }
-        const uint32_t target_units = target_wgs * kMfmaDecodeWaves;
         unit_blocks = std::max(1u, (total_blocks + target_units - 1) / target_units);
         const uint32_t nblk = (max_len + 63) / 64;
         n_splits = (nblk + unit_blocks - 1) / unit_blocks + 1; // partial slots per (sequence, head)

@@ -26,7 +26,8 @@ struct MfmaParams {
 };
 
 bool mfma_decode_supported(uint32_t d, uint32_t wk, uint32_t wv, uint32_t G);
+// Wavefronts that fill the device for group size G: the launch is cut into that many block runs.
+uint32_t mfma_decode_wavefronts(uint32_t G);
 int launch_mfma_decode(const MfmaParams &p, uint32_t d, hipStream_t s);
-constexpr uint32_t kMfmaDecodeWaves = 4; // wavefronts per workgroup of the matrix-core kernel
 
 } // namespace weedhip

@@ -3,25 +3,29 @@
 
 namespace weedhip {
 
-int launch_mfma_decode_d64_uniform(const MfmaParams &p, dim3 grid, hipStream_t s);
-int launch_mfma_decode_d64_lloyd(const MfmaParams &p, dim3 grid, hipStream_t s);
-int launch_mfma_decode_d128_uniform(const MfmaParams &p, dim3 grid, hipStream_t s);
-int launch_mfma_decode_d128_lloyd(const MfmaParams &p, dim3 grid, hipStream_t s);
+int launch_mfma_decode_d64_uniform(const MfmaParams &p, hipStream_t s);
+int launch_mfma_decode_d64_lloyd(const MfmaParams &p, hipStream_t s);
+int launch_mfma_decode_d128_uniform(const MfmaParams &p, hipStream_t s);
+int launch_mfma_decode_d128_lloyd(const MfmaParams &p, hipStream_t s);
 
 bool mfma_decode_supported(uint32_t d, uint32_t wk, uint32_t wv, uint32_t G)
 {
     return (d == 64 || d == 128) && wk >= 2 && wk <= 4 && wv >= 2 && wv <= 4 && G >= 1 && G <= 16;
 }
 
+uint32_t mfma_decode_wavefronts(uint32_t G)
+{
+    // every compute unit holds one workgroup: 12 wavefronts, or 8 for the 16-column variant (more registers)
+    return (G > 8 ? 8u : 12u) * 256u;
+}
+
 int launch_mfma_decode(const MfmaParams &p, uint32_t d, hipStream_t s)
 {
-    const uint32_t units = (p.total_blocks + p.unit_blocks - 1) / p.unit_blocks;
-    const dim3 grid((units + kMfmaDecodeWaves - 1) / kMfmaDecodeWaves);
     const bool lloyd = p.k.alpha != nullptr;
     if (d == 64) {
-        return lloyd ? launch_mfma_decode_d64_lloyd(p, grid, s) : launch_mfma_decode_d64_uniform(p, grid, s);
+        return lloyd ? launch_mfma_decode_d64_lloyd(p, s) : launch_mfma_decode_d64_uniform(p, s);
     }
-    return lloyd ? launch_mfma_decode_d128_lloyd(p, grid, s) : launch_mfma_decode_d128_uniform(p, grid, s);
+    return lloyd ? launch_mfma_decode_d128_lloyd(p, s) : launch_mfma_decode_d128_uniform(p, s);
 }
 
 } // namespace weedhip

@@ -2,8 +2,8 @@
 #include "kv_decode_mfma_kernel.h"
 
 namespace weedhip {
-int launch_mfma_decode_d64_lloyd(const MfmaParams &p, dim3 grid, hipStream_t s)
+int launch_mfma_decode_d64_lloyd(const MfmaParams &p, hipStream_t s)
 {
-    return weedhip_mfma::launch_d<64, true>(p, grid, s);
+    return weedhip_mfma::launch_d<64, true>(p, s);
 }
 } // namespace weedhip

@@ -2,8 +2,8 @@
 #include "kv_decode_mfma_kernel.h"
 
 namespace weedhip {
-int launch_mfma_decode_d64_uniform(const MfmaParams &p, dim3 grid, hipStream_t s)
+int launch_mfma_decode_d64_uniform(const MfmaParams &p, hipStream_t s)
 {
-    return weedhip_mfma::launch_d<64, false>(p, grid, s);
+    return weedhip_mfma::launch_d<64, false>(p, s);
 }
 } // namespace weedhip

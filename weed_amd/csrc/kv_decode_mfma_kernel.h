@@ -1,33 +1,24 @@
 #pragma once
 // Matrix-core decode attention over the packed cache (gfx950).
 //
-// One wavefront owns 64-token blocks of one (sequence, kv head).  Per block it
+// One wavefront owns a run of 64-token blocks of the launch's block list (region after region).  Per block it
 //   1. streams its lane-major run of packed K items (coalesced 128-bit loads, every byte of the block read once),
-//   2. turns every pair of fields into two fp16 values with one conflict-free LDS lookup (the pair table is replicated
-//      over the 32 banks) and feeds them as the A operand of v_mfma_f32_16x16x32_f16 against the query, which sits in
-//      registers as fp16 hi + lo halves (products of fp16 values are exact in fp32, so the split keeps ~22 bits),
+//   2. turns every pair of fields into two fp16 values with one conflict-free LDS lookup (each pair-table entry is
+//      replicated over the 32 banks) and feeds them as the A operand of v_mfma_f32_16x16x32_f16 against the query,
+//      which sits in registers as fp16 hi + lo halves (products of fp16 values are exact in fp32, so the split keeps
+//      ~22 bits),
 //   3. runs an online softmax on the 16 tokens x 16 heads score tiles in registers (base-2 exponentials; 1/sqrt(d) and
 //      log2(e) are folded into the query),
 //   4. splits the probabilities (times the V row scales) into fp16 hi + lo, which are already in A-operand order,
 //      and multiplies them with the looked-up V items: out[head][coordinate] accumulates in 4*(d/16) registers.
-// The four wavefronts of a workgroup share the lookup tables, split the workgroup's blocks between them and merge
-// their partial results in LDS; one un-normalised partial (m, l, o[d]) per query head leaves the workgroup.
+// The wavefronts of a workgroup share the lookup tables and nothing else; every wavefront writes one un-normalised
+// partial (m, l, o[d]) per query head and region segment, and a second kernel merges the partials.
 //
 // Table values are exactly representable in fp16 (the Lloyd-Max tables are generated that way; the uniform coder's
 // table is code + 0.5), so de-quantisation itself is exact; the only roundings are those of the fp32 accumulators.
 #include "kv_decode_mfma.h"
 
 #include <type_traits>
-
-#ifndef WEED_EXP_KORDER
-#define WEED_EXP_KORDER 1
-#endif
-#ifndef WEED_EXP_KROLL
-#define WEED_EXP_KROLL 0
-#endif
-#ifndef WEED_EXP_VROLL
-#define WEED_EXP_VROLL 0
-#endif
 
 using namespace weedhip;
 using namespace weedkv;
@@ -39,25 +30,13 @@ typedef float float4v __attribute__((ext_vector_type(4)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
 
-constexpr int kWaves = (int)kMfmaDecodeWaves;
-
-__device__ __forceinline__ uint32_t pack_half2(float a, float b)
-{
-    const _Float16 ha = (_Float16)a, hb = (_Float16)b;
-    return (uint32_t)__builtin_bit_cast(uint16_t, ha) | ((uint32_t)__builtin_bit_cast(uint16_t, hb) << 16);
-}
-
 // N dwords from a pointer aligned to 16 bytes when N % 4 == 0, else to 8 bytes (N is even for every supported shape).
 template <int N> __device__ __forceinline__ void load_dwords(const uint8_t *p, uint32_t (&x)[N])
 {
     if constexpr (N % 4 == 0) {
 #pragma unroll
         for (int i = 0; i < N / 4; ++i) {
-#ifdef WEED_EXP_INTERLEAVE
-            const uint4v v = *reinterpret_cast<const uint4v *>(p + 1024 * i);
-#else
             const uint4v v = *reinterpret_cast<const uint4v *>(p + 16 * i);
-#endif
             x[4 * i] = v.x;
             x[4 * i + 1] = v.y;
             x[4 * i + 2] = v.z;
@@ -74,48 +53,56 @@ template <int N> __device__ __forceinline__ void load_dwords(const uint8_t *p, u
     }
 }
 
-// Pair `P` (2*W bits at bit 2*W*P of the lane's run) -> byte address of its table entry for this lane:
-// table base + entry * 128 + (lane % 32) * 4.  Two instructions per pair: extract the bit field, then shift-and-add
-// the lane's base
-// (written as inline assembly because the compiler's canonical form of the same expression takes three).
-template <int W, int N, int P> __device__ __forceinline__ uint32_t pair_addr(const uint32_t (&x)[N], uint32_t lane_off)
+// ---- pair tables in LDS.  Entry e of a table is a row of 256 bytes starting at LDS byte e * 256; the V table uses
+//      the first 128 bytes of its rows (32 replicas of the entry, one per bank), the K table the second 128 bytes of
+//      rows [0, 2^(2 WK)).  The tables start at LDS address 0 (the kernel has no other LDS), so the byte address of
+//      a lookup is  (entry << 8) | lane byte,  lane byte = (lane % 32) * 4 (+ 128 for K): the entry index lands in
+//      byte 1 of the address.  When a pair is a whole byte of the packed run (4-bit fields), ONE byte-permute builds
+//      the address from the run's dword and the lane byte; otherwise a bit-field extract and a shift-add do. ----
+constexpr uint32_t kTableRowBytes = 256;
+template <int WK, int WV> constexpr uint32_t table_rows() { return 1u << (2 * (WK > WV ? WK : WV)); }
+
+template <int W, int N, int P> __device__ __forceinline__ uint32_t pair_addr(const uint32_t (&x)[N], uint32_t lane_byte)
 {
     constexpr int bit = 2 * W * P;
     constexpr int dw = bit >> 5, sh = bit & 31;
-    uint32_t t, a;
-    if constexpr (sh + 2 * W <= 32) {
-        asm("v_bfe_u32 %0, %1, %2, %3" : "=v"(t) : "v"(x[dw]), "n"(sh), "n"(2 * W));
+    uint32_t a;
+    if constexpr (W == 4) {
+        // result bytes (3..0) = (0, 0, byte sh/8 of the run's dword, lane byte); selector values 4..7 name the bytes of
+        // the first source, 0..3 those of the second, 0x0c a zero byte
+        constexpr uint32_t sel = 0x0c0c0000u | ((4u + sh / 8) << 8);
+        asm("v_perm_b32 %0, %1, %2, %3" : "=v"(a) : "v"(x[dw]), "v"(lane_byte), "s"(sel));
     } else {
-        // the pair straddles two dwords: funnel-shift it down first
-        uint32_t f;
-        asm("v_alignbit_b32 %0, %1, %2, %3" : "=v"(f) : "v"(x[dw + 1 < N ? dw + 1 : dw]), "v"(x[dw]), "n"(sh));
-        asm("v_bfe_u32 %0, %1, 0, %2" : "=v"(t) : "v"(f), "n"(2 * W));
+        uint32_t t;
+        if constexpr (sh + 2 * W <= 32) {
+            asm("v_bfe_u32 %0, %1, %2, %3" : "=v"(t) : "v"(x[dw]), "n"(sh), "n"(2 * W));
+        } else {
+            // the pair straddles two dwords: funnel-shift it down first
+            uint32_t f;
+            asm("v_alignbit_b32 %0, %1, %2, %3" : "=v"(f) : "v"(x[dw + 1 < N ? dw + 1 : dw]), "v"(x[dw]), "n"(sh));
+            asm("v_bfe_u32 %0, %1, 0, %2" : "=v"(t) : "v"(f), "n"(2 * W));
+        }
+        asm("v_lshl_add_u32 %0, %1, 8, %2" : "=v"(a) : "v"(t), "v"(lane_byte));
     }
-    asm("v_lshl_add_u32 %0, %1, 7, %2" : "=v"(a) : "v"(t), "v"(lane_off));
     return a;
 }
 
-// Item K (8 fields) of the lane's run -> 8 fp16 values in matrix-operand order.
 typedef const uint32_t __attribute__((address_space(3))) *lds_u32_ptr;
 
 __device__ __forceinline__ uint32_t lds_read(uint32_t byte_addr)
 {
-#ifdef WEED_EXP_NOLDS
-    return byte_addr;
-#else
     return *reinterpret_cast<lds_u32_ptr>((uintptr_t)byte_addr);
-#endif
 }
 
-// `lane_base` = LDS byte address of the table + (lane % 32) * 4.
+// Item K (8 fields) of the lane's run -> 8 fp16 values in matrix-operand order.
 template <int W, int N, int K>
-__device__ __forceinline__ half8 dequant_item(const uint32_t (&x)[N], uint32_t lane_base)
+__device__ __forceinline__ half8 dequant_item(const uint32_t (&x)[N], uint32_t lane_byte)
 {
     uint4v r;
-    r.x = lds_read(pair_addr<W, N, 4 * K>(x, lane_base));
-    r.y = lds_read(pair_addr<W, N, 4 * K + 1>(x, lane_base));
-    r.z = lds_read(pair_addr<W, N, 4 * K + 2>(x, lane_base));
-    r.w = lds_read(pair_addr<W, N, 4 * K + 3>(x, lane_base));
+    r.x = lds_read(pair_addr<W, N, 4 * K>(x, lane_byte));
+    r.y = lds_read(pair_addr<W, N, 4 * K + 1>(x, lane_byte));
+    r.z = lds_read(pair_addr<W, N, 4 * K + 2>(x, lane_byte));
+    r.w = lds_read(pair_addr<W, N, 4 * K + 3>(x, lane_byte));
     return __builtin_bit_cast(half8, r);
 }
 
@@ -126,45 +113,6 @@ template <int I, int N, typename F> __device__ __forceinline__ void static_for(F
         f(std::integral_constant<int, I>{});
         static_for<I + 1, N>(f);
     }
-}
-
-// The lane's run is loaded in chunks of 16 bytes (8 when N is not a multiple of 4).  chunk_last_item<N, W>(c) is the
-// last 8-field item (W bytes each) that reads chunk c; after its lookups the chunk's registers can be refilled.
-template <int N> constexpr int chunk_dwords() { return N % 4 == 0 ? 4 : 2; }
-template <int N> constexpr int chunk_count() { return N / chunk_dwords<N>(); }
-template <int N, int W> constexpr int chunk_last_item(int c)
-{
-    const int last_byte = 4 * chunk_dwords<N>() * (c + 1) - 1;
-    const int items = 4 * N / W;
-    return last_byte / W < items ? last_byte / W : items - 1;
-}
-template <int N, int C> __device__ __forceinline__ void load_chunk(const uint8_t *p, uint32_t (&x)[N])
-{
-    if constexpr (N % 4 == 0) {
-#ifdef WEED_EXP_INTERLEAVE
-        const uint4v v = *reinterpret_cast<const uint4v *>(p + 1024 * C);
-#else
-        const uint4v v = *reinterpret_cast<const uint4v *>(p + 16 * C);
-#endif
-        x[4 * C] = v.x;
-        x[4 * C + 1] = v.y;
-        x[4 * C + 2] = v.z;
-        x[4 * C + 3] = v.w;
-    } else {
-        const uint2v v = *reinterpret_cast<const uint2v *>(p + 8 * C);
-        x[2 * C] = v.x;
-        x[2 * C + 1] = v.y;
-    }
-}
-// Refill every chunk whose last reader is item I.
-template <int N, int W, int I> __device__ __forceinline__ void refill_after_item(const uint8_t *p, uint32_t (&x)[N])
-{
-    static_for<0, chunk_count<N>()>([&](auto cc) {
-        constexpr int c = decltype(cc)::value;
-        if constexpr (chunk_last_item<N, W>(c) == I) {
-            load_chunk<N, c>(p, x);
-        }
-    });
 }
 
 __device__ __forceinline__ float4v mfma16(half8 a, half8 b, float4v c)
@@ -210,49 +158,54 @@ template <int GP> __device__ __forceinline__ float head_sum(float v)
 // Bank mask (4-lane banks of a row) of the lanes [GP*i, GP*i + GP).
 template <int GP, int I> constexpr int bank_mask_of() { return ((1 << (GP / 4)) - 1) << (I * GP / 4); }
 
+// Wavefronts per workgroup: as many as fit a compute unit at the kernel's register budget (three per SIMD; two for the
+// 16-column variant, which needs more registers), so that one copy of the tables serves the whole compute unit.
+template <int GP> constexpr int waves_per_wg() { return GP == 16 ? 8 : 12; }
+
 // GP = number of query-head columns kept per score tile (the group size rounded up to 4, 8 or 16).  The Q.K^T
 // instruction always produces 16 columns; with GP < 16 the useful columns of 16/GP tiles are merged into one register
 // set before the softmax, so the exponentials and the fp16 splitting run on full registers.
 template <int D, int WK, int WV, int GP, bool LLOYD>
-__global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_kernel(MfmaParams p)
+__global__ void __launch_bounds__(64 * waves_per_wg<GP>()) decode_mfma_kernel(MfmaParams p)
 {
+    constexpr int kWaves = waves_per_wg<GP>();
     constexpr int KS = D / 32;       // Q.K^T k-steps (32 coordinates each); also K items per tile per lane
     constexpr int JB = D / 16;       // 16-coordinate column blocks of the output
     constexpr int NK = KS * WK;      // dwords of packed K per lane per block
     constexpr int NV = D * WV / 32;  // dwords of packed V per lane per block
     constexpr int TPS = 16 / GP;     // score tiles merged into one register set
     constexpr int NSETS = 4 / TPS;   // register sets per 64-token block
-    constexpr uint32_t KT = (1u << (2 * WK)) * 32u; // dwords of the replicated K pair table
-    constexpr uint32_t VT = (1u << (2 * WV)) * 32u;
+    constexpr uint32_t ROWS = table_rows<WK, WV>();
 
-    extern __shared__ uint32_t lds[];
-    uint32_t *ktab = lds;
-    uint32_t *vtab = lds + KT;
+    extern __shared__ uint32_t lds[]; // the tables, then 64 staged fp16 levels
 
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t c = lane & 15, g = lane >> 4;
     constexpr bool lloyd = LLOYD;
 
-    // ---- pair tables: entry e, replica i at dword e*32 + i; a lane always reads replica lane%32.  The 2^w fp16
-    //      levels are staged in LDS first so that building the pairs needs no global reads. ----
-    __shared__ uint16_t levels_h[2][32];
-    if (tid < 64) {
-        const float lv = (tid < 32) ? p.k.table[tid & 31] : p.v.table[tid & 31];
-        levels_h[tid >> 5][tid & 31] = __builtin_bit_cast(uint16_t, (_Float16)lv);
+    // ---- build the pair tables.  The 2^w fp16 levels are staged in LDS first so that building the pairs needs no
+    //      global reads. ----
+    {
+        uint16_t *levels_h = reinterpret_cast<uint16_t *>(lds + ROWS * (kTableRowBytes / 4)); // [2][32]
+        if (tid < 64) {
+            const float lv = (tid < 32) ? p.k.table[tid & 31] : p.v.table[tid & 31];
+            levels_h[tid] = __builtin_bit_cast(uint16_t, (_Float16)lv);
+        }
+        __syncthreads();
+        for (uint32_t i = tid; i < ROWS * 64; i += 64 * kWaves) {
+            const uint32_t e = i >> 6, half_row = (i >> 5) & 1; // 0: V table, 1: K table
+            uint32_t val = 0;
+            if (half_row == 0 && e < (1u << (2 * WV))) {
+                val = (uint32_t)levels_h[32 + (e & ((1u << WV) - 1u))] | ((uint32_t)levels_h[32 + (e >> WV)] << 16);
+            } else if (half_row == 1 && e < (1u << (2 * WK))) {
+                val = (uint32_t)levels_h[e & ((1u << WK) - 1u)] | ((uint32_t)levels_h[e >> WK] << 16);
+            }
+            lds[i] = val;
+        }
+        __syncthreads();
     }
-    __syncthreads();
-    for (uint32_t i = tid; i < KT; i += 64 * kWaves) {
-        const uint32_t e = i >> 5;
-        ktab[i] = (uint32_t)levels_h[0][e & ((1u << WK) - 1u)] | ((uint32_t)levels_h[0][e >> WK] << 16);
-    }
-    for (uint32_t i = tid; i < VT; i += 64 * kWaves) {
-        const uint32_t e = i >> 5;
-        vtab[i] = (uint32_t)levels_h[1][e & ((1u << WV) - 1u)] | ((uint32_t)levels_h[1][e >> WV] << 16);
-    }
-    __syncthreads();
-    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint32_t *)lds;
-    const uint32_t kbase = lds_base + (lane & 31) * 4;
-    const uint32_t vbase = kbase + KT * 4;
+    const uint32_t vbase = (lane & 31) * 4; // lane byte of a V lookup
+    const uint32_t kbase = vbase + 128;     // lane byte of a K lookup
 
     // ---- this wavefront's share of the launch: a contiguous run of `unit_blocks` 64-token blocks of the global block
     //      list (all blocks of (sequence 0, kv head 0), then (0, 1), ...).  A run is cut into segments at region
@@ -349,13 +302,8 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_kernel(MfmaParams 
         O[jb] = float4v{ 0.0f, 0.0f, 0.0f, 0.0f };
     }
 
-#ifdef WEED_EXP_INTERLEAVE
-    const uint8_t *kreg = p.k.fields + region * p.k.region_bytes + (uint64_t)lane * 16;
-    const uint8_t *vreg = p.v.fields + region * p.v.region_bytes + (uint64_t)lane * 16;
-#else
     const uint8_t *kreg = p.k.fields + region * p.k.region_bytes + (uint64_t)lane * (4 * NK);
     const uint8_t *vreg = p.v.fields + region * p.v.region_bytes + (uint64_t)lane * (4 * NV);
-#endif
     const float *ka = lloyd ? p.k.alpha + region * p.padded + 16 * tile_in_set + 4 * g : nullptr;
     const float *va = lloyd ? p.v.alpha + region * p.padded + 16 * tile_in_set + 4 * g : nullptr;
 
@@ -365,121 +313,44 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_kernel(MfmaParams 
     uint32_t kraw[NK], vraw[NV];
     float4v ak[NSETS], av[NSETS];
 
-    auto load_k_scales = [&](uint32_t blk) {
+    auto load_k = [&](uint32_t blk) {
+        load_dwords<NK>(kreg + (uint64_t)blk * (8u * D * WK), kraw);
 #pragma unroll
         for (int s = 0; s < NSETS; ++s) {
-#ifdef WEED_EXP_NOALPHA
-            if constexpr (false) {
-#else
             if constexpr (lloyd) {
-#endif
                 ak[s] = *reinterpret_cast<const float4v *>(ka + blk * 64 + 16 * TPS * s);
             } else {
                 ak[s] = float4v{ p.k.alpha_const, p.k.alpha_const, p.k.alpha_const, p.k.alpha_const };
             }
         }
     };
-    auto load_v_scales = [&](uint32_t blk) {
+    auto load_v = [&](uint32_t blk) {
+        load_dwords<NV>(vreg + (uint64_t)blk * (8u * D * WV), vraw);
 #pragma unroll
         for (int s = 0; s < NSETS; ++s) {
-#ifdef WEED_EXP_NOALPHA
-            if constexpr (false) {
-#else
             if constexpr (lloyd) {
-#endif
                 av[s] = *reinterpret_cast<const float4v *>(va + blk * 64 + 16 * TPS * s);
             } else {
                 av[s] = float4v{ 1.0f, 1.0f, 1.0f, 1.0f };
             }
         }
     };
-    bool first_load = true;
-    auto load_k = [&](uint32_t blk) {
-#ifdef WEED_EXP_NOLOAD
-        if (first_load)
-#endif
-        {
-            load_dwords<NK>(kreg + (uint64_t)blk * (8u * D * WK), kraw);
-            load_k_scales(blk);
-        }
-    };
-    auto load_v = [&](uint32_t blk) {
-#ifdef WEED_EXP_NOLOAD
-        if (first_load)
-#endif
-        {
-            load_dwords<NV>(vreg + (uint64_t)blk * (8u * D * WV), vraw);
-            load_v_scales(blk);
-        }
-        first_load = false;
-    };
 
-#ifdef WEED_EXP_MEMONLY
     auto process_block = [&](uint32_t blk, uint32_t next_blk) {
-        (void)blk;
-        const uint8_t *knext = kreg + (uint64_t)next_blk * (8u * D * WK);
-        const uint8_t *vnext = vreg + (uint64_t)next_blk * (8u * D * WV);
-        uint32_t acc = 0;
-        static_for<0, chunk_count<NK>()>([&](auto cc) {
-            constexpr int c = decltype(cc)::value;
-#pragma unroll
-            for (int k = 0; k < chunk_dwords<NK>(); ++k) {
-                acc ^= kraw[chunk_dwords<NK>() * c + k];
-            }
-            if constexpr (WEED_EXP_KROLL) {
-                load_chunk<NK, c>(knext, kraw);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        });
-        acc ^= __float_as_uint(ak[0][0]);
-        if constexpr (WEED_EXP_KROLL) {
-            load_k_scales(next_blk);
-        } else {
-            load_k(next_blk);
-        }
-        static_for<0, chunk_count<NV>()>([&](auto cc) {
-            constexpr int c = decltype(cc)::value;
-#pragma unroll
-            for (int k = 0; k < chunk_dwords<NV>(); ++k) {
-                acc ^= vraw[chunk_dwords<NV>() * c + k];
-            }
-            if constexpr (WEED_EXP_VROLL) {
-                load_chunk<NV, c>(vnext, vraw);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        });
-        acc ^= __float_as_uint(av[0][0]);
-        if constexpr (WEED_EXP_VROLL) {
-            load_v_scales(next_blk);
-        } else {
-            load_v(next_blk);
-        }
-        O[0][0] += (float)(acc & 1u);
-    };
-    auto process_block_unused = [&](uint32_t blk, uint32_t next_blk) {
-#else
-    auto process_block = [&](uint32_t blk, uint32_t next_blk) {
-#endif
-        // ---- S[t] = K_tile . q: rows = tokens 16t + (lane%16), contraction over the lane groups' coordinates ----
-        // Lookups run two items ahead of the matrix instructions that consume them.
+        // ---- S[t] = K_tile . q: rows = tokens 16t + (lane%16), contraction over the lane groups' coordinates.
+        //      Items are taken in memory order (tile after tile); lookups run two items ahead of the matrix
+        //      instructions that consume them. ----
         float4v S[4];
         {
-            // Items are taken in memory order (tile after tile), so the leading chunks of the lane's run retire early
-            // and are refilled with the next block's bytes while this block is still being worked on.
             constexpr int NI = 4 * KS;
-            const uint8_t *knext = kreg + (uint64_t)next_blk * (8u * D * WK);
-            auto item_of = [](int i) constexpr { return WEED_EXP_KORDER ? i : (i % 4) * KS + i / 4; };
-            half8 a0 = dequant_item<WK, NK, item_of(0)>(kraw, kbase);
-            half8 a1 = dequant_item<WK, NK, item_of(1)>(kraw, kbase);
+            half8 a0 = dequant_item<WK, NK, 0>(kraw, kbase);
+            half8 a1 = dequant_item<WK, NK, 1>(kraw, kbase);
             static_for<0, NI>([&](auto ic) {
                 constexpr int i = decltype(ic)::value;
-                constexpr int t = WEED_EXP_KORDER ? i / KS : i % 4, ks = WEED_EXP_KORDER ? i % KS : i / 4;
+                constexpr int t = i / KS, ks = i % KS;
                 half8 a2 = a1;
                 if constexpr (i + 2 < NI) {
-                    a2 = dequant_item<WK, NK, item_of(i + 2)>(kraw, kbase);
-                    if constexpr (WEED_EXP_KORDER && WEED_EXP_KROLL) {
-                        refill_after_item<NK, WK, i + 2>(knext, kraw);
-                    }
+                    a2 = dequant_item<WK, NK, i + 2>(kraw, kbase);
                 }
                 // keep the look-ahead lookups ahead of this item's matrix instruction
                 __builtin_amdgcn_sched_barrier(0);
@@ -523,11 +394,7 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_kernel(MfmaParams 
                 C[s][r] = fmaf(v, ak[s][r] * qscale, betaq);
             }
         }
-        if constexpr (WEED_EXP_KORDER && WEED_EXP_KROLL) {
-            load_k_scales(next_blk); // the row scales are free again (the packed fields were refilled on the way)
-        } else {
-            load_k(next_blk);
-        }
+        load_k(next_blk); // the K buffer is free again
         if (blk * 64 + 64 > L) {
 #pragma unroll
             for (int s = 0; s < NSETS; ++s) {
@@ -644,7 +511,6 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_kernel(MfmaParams 
         }
         {
             constexpr int NI = 2 * JB;
-            const uint8_t *vnext = vreg + (uint64_t)next_blk * (8u * D * WV);
             half8 b0v = dequant_item<WV, NV, 0>(vraw, vbase);
             half8 b1v = dequant_item<WV, NV, 1>(vraw, vbase);
             static_for<0, NI>([&](auto ic) {
@@ -653,9 +519,6 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_kernel(MfmaParams 
                 half8 b2v = b1v;
                 if constexpr (i + 2 < NI) {
                     b2v = dequant_item<WV, NV, i + 2>(vraw, vbase);
-                    if constexpr (WEED_EXP_VROLL) {
-                        refill_after_item<NV, WV, i + 2>(vnext, vraw);
-                    }
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 O[jb] = mfma16(pa[u][0], b0v, O[jb]);
@@ -666,15 +529,11 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_kernel(MfmaParams 
                 b1v = b2v;
             });
         }
-        if constexpr (WEED_EXP_VROLL) {
-            load_v_scales(next_blk);
-        } else {
-            load_v(next_blk);
-        }
+        load_v(next_blk); // the V buffer is free again
     };
 
-    // ---- main loop.  The refills are unconditional (the next block index is clamped to the last block of the split)
-    //      so that the loop body has no branch around loads and outstanding loads can be counted exactly. ----
+    // ---- main loop.  The refills are unconditional (the next block index is clamped to the last block of the
+    //      segment) so that the loop body has no branch around loads and outstanding loads can be counted exactly. ----
     {
         uint32_t blk = b0;
         if (blk < b1) {
@@ -732,37 +591,39 @@ __global__ void __launch_bounds__(64 * kWaves, 2) decode_mfma_kernel(MfmaParams 
     } // segments
 }
 
-template <int D, int WK, int WV, int GP, bool LLOYD> int launch_gp(const MfmaParams &p, dim3 grid, hipStream_t s)
+template <int D, int WK, int WV, int GP, bool LLOYD> int launch_gp(const MfmaParams &p, hipStream_t s)
 {
-    constexpr size_t smem = (((size_t)1 << (2 * WK)) + ((size_t)1 << (2 * WV))) * 32 * sizeof(uint32_t);
+    constexpr size_t smem = (size_t)table_rows<WK, WV>() * kTableRowBytes + 64 * sizeof(uint16_t);
+    constexpr uint32_t waves = (uint32_t)waves_per_wg<GP>();
     static bool configured = false;
     if (!configured) {
         WEED_HIP_CHECK(hipFuncSetAttribute((const void *)decode_mfma_kernel<D, WK, WV, GP, LLOYD>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         configured = true;
     }
-    decode_mfma_kernel<D, WK, WV, GP, LLOYD><<<grid, 64 * kWaves, smem, s>>>(p);
+    const uint32_t units = (p.total_blocks + p.unit_blocks - 1) / p.unit_blocks;
+    decode_mfma_kernel<D, WK, WV, GP, LLOYD><<<(units + waves - 1) / waves, 64 * waves, smem, s>>>(p);
     WEED_HIP_LAUNCH_CHECK();
     return WEED_HIP_OK;
 }
 
-template <int D, int WK, int WV, bool LLOYD> int launch_one(const MfmaParams &p, dim3 grid, hipStream_t s)
+template <int D, int WK, int WV, bool LLOYD> int launch_one(const MfmaParams &p, hipStream_t s)
 {
     if (p.G <= 4) {
-        return launch_gp<D, WK, WV, 4, LLOYD>(p, grid, s);
+        return launch_gp<D, WK, WV, 4, LLOYD>(p, s);
     }
     if (p.G <= 8) {
-        return launch_gp<D, WK, WV, 8, LLOYD>(p, grid, s);
+        return launch_gp<D, WK, WV, 8, LLOYD>(p, s);
     }
-    return launch_gp<D, WK, WV, 16, LLOYD>(p, grid, s);
+    return launch_gp<D, WK, WV, 16, LLOYD>(p, s);
 }
 
-template <int D, bool LLOYD> int launch_d(const MfmaParams &p, dim3 grid, hipStream_t s)
+template <int D, bool LLOYD> int launch_d(const MfmaParams &p, hipStream_t s)
 {
     const uint32_t wk = p.k.w, wv = p.v.w;
 #define WEED_CASE(K, V)                                                                                                \
     if (wk == K && wv == V) {                                                                                          \
-        return launch_one<D, K, V, LLOYD>(p, grid, s);                                                                        \
+        return launch_one<D, K, V, LLOYD>(p, s);                                                                       \
     }
     WEED_CASE(2, 2)
     WEED_CASE(2, 3)
