@@ -281,13 +281,44 @@ __global__ void pack_k_kernel(const uint8_t *__restrict__ fields, const float *_
     }
 }
 
+// Row scales of the new V rows: one thread per new row copies the scale to its token slot and the region's largest
+// scale is kept up to date (one atomic per wavefront and region, not one per row).
+__global__ void __launch_bounds__(256) scatter_v_scales_kernel(const float *__restrict__ alpha_in, uint32_t rows,
+                                                              uint32_t Hkv, uint32_t T, int32_t seq_begin,
+                                                              const int32_t *__restrict__ lens,
+                                                              float *__restrict__ alpha_out,
+                                                              uint32_t *__restrict__ alpha_max, uint32_t padded)
+{
+    const uint32_t row = blockIdx.x * blockDim.x + threadIdx.x;
+    const bool valid = row < rows;
+    uint32_t region = 0xffffffffu, bits = 0;
+    if (valid) {
+        const uint32_t t = row % T, h = (row / T) % Hkv, s = row / (T * Hkv);
+        const float a = alpha_in[row];
+        region = (uint32_t)(seq_begin + s) * Hkv + h;
+        alpha_out[(uint64_t)region * padded + (uint32_t)lens[seq_begin + s] + t] = a;
+        bits = __float_as_uint(fabsf(a));
+    }
+    // lanes of a wavefront that share the first valid lane's region fold their maximum into one atomic
+    const uint32_t lead = __builtin_amdgcn_readfirstlane(region);
+    uint32_t mine = (valid && region == lead) ? bits : 0u;
+    for (int o = 32; o > 0; o >>= 1) {
+        mine = max(mine, (uint32_t)__shfl_xor((int)mine, o));
+    }
+    if (valid) {
+        if (region != lead) {
+            atomicMax(alpha_max + region, bits);
+        } else if ((threadIdx.x & 63) == (uint32_t)__builtin_ctzll(__ballot(valid && region == lead))) {
+            atomicMax(alpha_max + region, mine);
+        }
+    }
+}
+
 // One thread per (sequence, kv head, 32-token half block, lane group, coordinate): rebuilds one item of 8 tokens,
 // keeping the fields of tokens that were already cached and zeroing those not yet written.
-__global__ void pack_v_kernel(const uint8_t *__restrict__ fields, const float *__restrict__ alpha_in, uint32_t S,
-                              uint32_t Hkv, uint32_t T, uint32_t d, uint32_t w, int32_t seq_begin,
-                              const int32_t *__restrict__ lens, uint32_t halves, uint8_t *__restrict__ out,
-                              uint64_t region_bytes, float *__restrict__ alpha_out, uint32_t *__restrict__ alpha_max,
-                              uint32_t padded)
+__global__ void pack_v_kernel(const uint8_t *__restrict__ fields, uint32_t S, uint32_t Hkv, uint32_t T, uint32_t d,
+                              uint32_t w, int32_t seq_begin, const int32_t *__restrict__ lens, uint32_t halves,
+                              uint8_t *__restrict__ out, uint64_t region_bytes)
 {
     const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const uint64_t total = (uint64_t)S * Hkv * halves * 4 * d;
@@ -321,11 +352,6 @@ __global__ void pack_v_kernel(const uint8_t *__restrict__ fields, const float *_
             const uint32_t row = (s * Hkv + h) * T + (n - old_len);
             f8[e] = fields[(uint64_t)row * d + j];
             touched = true;
-            if (alpha_out && j == 0) {
-                const float a = alpha_in[row];
-                alpha_out[region * padded + n] = a;
-                atomicMax(alpha_max + region, __float_as_uint(fabsf(a)));
-            }
         } else {
             f8[e] = 0;
         }
@@ -556,9 +582,16 @@ int encode_side(weed_hip_kv_cache *c, Side &side, int which, int32_t seq_begin, 
         // a run of T_new tokens starting anywhere touches at most (T_new + 30) / 32 + 1 half blocks
         const uint32_t halves = ((uint32_t)T_new + 30) / 32 + 1;
         const uint64_t n = (uint64_t)seq_count * Hkv * halves * 4 * d;
-        pack_v_kernel<<<(uint32_t)((n + 255) / 256), 256, 0, stream()>>>(
-            c->enc_fields, c->enc_alpha, (uint32_t)seq_count, Hkv, (uint32_t)T_new, d, side.w, seq_begin, c->lens_dev,
-            halves, side.fields, side.region_bytes, alpha_out, side.alpha_max, c->padded_tokens);
+        pack_v_kernel<<<(uint32_t)((n + 255) / 256), 256, 0, stream()>>>(c->enc_fields, (uint32_t)seq_count, Hkv,
+                                                                         (uint32_t)T_new, d, side.w, seq_begin,
+                                                                         c->lens_dev, halves, side.fields,
+                                                                         side.region_bytes);
+        if (alpha_out) {
+            WEED_HIP_LAUNCH_CHECK();
+            scatter_v_scales_kernel<<<(rows + 255) / 256, 256, 0, stream()>>>(c->enc_alpha, rows, Hkv, (uint32_t)T_new,
+                                                                              seq_begin, c->lens_dev, alpha_out,
+                                                                              side.alpha_max, c->padded_tokens);
+        }
     }
     WEED_HIP_LAUNCH_CHECK();
     return WEED_HIP_OK;
