@@ -196,8 +196,10 @@ int weed_hip_block_scale_f32(const float *x_dev, uint32_t off, const uint32_t sh
 
 /* Encode-and-append: apply_rotation + write_row for T_new tokens of every sequence in
  * [seq_begin, seq_begin + seq_count) (multihead_attention.cpp:206-257).  k_dev / v_dev are logical
- * [seq_count, n_kv_heads, T_new, d] tensors with strides in elements.  `rotate` = 0 means the inputs are already
- * in the rotated basis.  Tokens are appended in logical order (token t of the call becomes token len+t). */
+ * [seq_count, n_kv_heads, T_new, d] tensors with strides in elements.  `rotate` = 0: the inputs are already in the
+ * rotated basis; 1: rotate on the matrix cores (fp32, fastest; sums in a different order than the reference's loop);
+ * 2: rotate with the reference's order and rounding (src/ops/matmul.cpp:40-44), so that codes match a BLAS-less
+ * reference build bit for bit.  Tokens are appended in logical order (token t of the call becomes token len+t). */
 int weed_hip_kv_encode_append(weed_hip_kv_cache *cache, int32_t seq_begin, int32_t seq_count, int32_t T_new,
                               const float *k_dev, uint32_t k_off, const uint32_t k_stride[4], const float *v_dev,
                               uint32_t v_off, const uint32_t v_stride[4], int rotate);

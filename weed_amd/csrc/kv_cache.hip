@@ -132,7 +132,7 @@ constexpr int kEncRows = 32;     // rows per workgroup
 constexpr int kEncThreads = 256;
 
 // Rotate (optional) and quantise kEncRows rows of a strided [S, Hkv, T, d] tensor into one field per byte.
-//   rotate 0: y = x            1: y = x.R with fused multiply-adds         2: y = x.R with the reference's
+//   rotate 0: y = x            1: y = x.R on the matrix cores (fp32)        2: y = x.R with the reference's
 //   rounding (multiply, then add, i ascending: src/ops/matmul.cpp:40-44).
 // PARTS = number of row slices the 256 threads are split into (each thread owns one output column of its slice).
 template <int PARTS>
@@ -166,7 +166,42 @@ __global__ void __launch_bounds__(kEncThreads)
     }
     __syncthreads();
 
-    if (rotate) {
+    if (rotate == 1) {
+        // y = x . R on the matrix cores: each wavefront owns 32-column tiles of the 32 x d result and walks the
+        // contraction two coordinates at a time (v_mfma_f32_32x32x2f32: lane l feeds row/column l % 32 of step
+        // k = l / 32).  Sums are in a different order than the scalar loop below, as rotate = 1 allows.
+        typedef float float16v __attribute__((ext_vector_type(16)));
+        static_assert(kEncRows == 32, "one 32-row matrix tile per workgroup");
+        const uint32_t lane = tid & 63, wave = tid >> 6;
+        const uint32_t l32 = lane & 31, khalf = lane >> 5;
+        for (uint32_t tile = wave; tile < d / 32; tile += kEncThreads / 64) {
+            float16v acc;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                acc[i] = 0.0f;
+            }
+            const float *bcol = rot_t + 32 * tile + l32; // R[k][32*tile + l32] = rot_t[col + d*k]
+            // d is a multiple of 32: sixteen steps at a time, their operand loads issued together
+            for (uint32_t k0 = 0; k0 < d; k0 += 32) {
+                float a[16], b[16];
+#pragma unroll
+                for (int u = 0; u < 16; ++u) {
+                    a[u] = xs[l32 * pitch + k0 + 2 * u + khalf];
+                    b[u] = bcol[(uint64_t)d * (k0 + 2 * u + khalf)];
+                }
+#pragma unroll
+                for (int u = 0; u < 16; ++u) {
+                    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u], b[u], acc, 0, 0, 0);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const uint32_t r = 8 * (i / 4) + 4 * khalf + (i % 4);
+                ys[r * pitch + 32 * tile + l32] = acc[i];
+            }
+        }
+        __syncthreads();
+    } else if (rotate) {
         constexpr int RPP = kEncRows / PARTS; // rows per part
         const uint32_t j = tid % d;
         const uint32_t part = tid / d;
@@ -177,21 +212,12 @@ __global__ void __launch_bounds__(kEncThreads)
                 acc[r] = 0.0f;
             }
             const float *xrow = xs + part * RPP * pitch;
-            if (rotate == 2) {
-                for (uint32_t i = 0; i < d; ++i) {
-                    const float rv = rot_t[j + d * i];
+            // the reference's order and rounding: multiply, then add, i ascending
+            for (uint32_t i = 0; i < d; ++i) {
+                const float rv = rot_t[j + d * i];
 #pragma unroll
-                    for (int r = 0; r < RPP; ++r) {
-                        acc[r] = acc[r] + xrow[r * pitch + i] * rv;
-                    }
-                }
-            } else {
-                for (uint32_t i = 0; i < d; ++i) {
-                    const float rv = rot_t[j + d * i];
-#pragma unroll
-                    for (int r = 0; r < RPP; ++r) {
-                        acc[r] = fmaf(xrow[r * pitch + i], rv, acc[r]);
-                    }
+                for (int r = 0; r < RPP; ++r) {
+                    acc[r] = acc[r] + xrow[r * pitch + i] * rv;
                 }
             }
 #pragma unroll
