@@ -254,3 +254,51 @@ def test_apply_rotation_reference_order(gpu, oracle):
     gpu.apply_rotation(xd, dev(R), out)
     want = oracle.apply_rotation(x.reshape(-1, d), R).reshape(x.shape)
     np.testing.assert_array_equal(out.cpu().numpy(), want)
+
+
+def test_cfg5a_encode_full_size(gpu, oracle):
+    """Configuration 5's encode half at full size (4096 tokens x 8 kv heads x head_dim 128, 3-bit Lloyd-Max codes):
+    with the reference-order rotation every field and row scale of both caches equals the CPU checker's, and the
+    matrix-core rotation moves only values that sit on a cell edge; appending the same tokens in four chunks gives
+    the same packed cache as one call (idempotence of the layout under incremental writes)."""
+    import torch
+    from weed_amd import workloads
+    wl = workloads.config(5)
+    d, T, Hkv = wl.head_dim, wl.max_len, wl.n_kv_heads
+    assert (T, Hkv, d) == (4096, 8, 128)
+    K, V, _ = wl.tensors()
+    rng = np.random.default_rng(5)
+    Rk = oracle.orthonormalize_columns(rng.normal(size=d * d).astype(np.float32))
+    Rv = oracle.orthonormalize_columns(rng.normal(size=d * d).astype(np.float32))
+    Ky = oracle.apply_rotation(K.reshape(-1, d), Rk)
+    Vy = oracle.apply_rotation(V.reshape(-1, d), Rv)
+    Kd, Vd = dev(K), dev(V)
+    exported = {}
+    for rotate in (2, 1):
+        cache = gpu.KVCache(gpu.KV_LLOYDMAX, 1, Hkv, d, T, wl.k_bits, wl.v_bits, wl.k_sign, wl.v_sign)
+        cache.set_rotations(dev(Rk), dev(Rv))
+        cache.encode_append(Kd, Vd, rotate=rotate)
+        kspec, vspec = coder_specs(oracle, cache)
+        for which, y, spec in ((0, Ky, kspec), (1, Vy, vspec)):
+            want_f, want_a = oracle.encode_rows(spec, y)
+            got_f, got_a = export(cache, which, T)
+            if rotate == 2:
+                np.testing.assert_array_equal(got_f.reshape(-1, d), want_f)
+                np.testing.assert_array_equal(got_a.reshape(-1), want_a)
+                exported[which] = (got_f, got_a)
+            else:
+                assert np.mean(got_f.reshape(-1, d) != want_f) < 2e-3
+                np.testing.assert_allclose(got_a.reshape(-1), want_a, rtol=1e-5)
+        cache.close()
+    # the same tokens in uneven chunks (the V items are rebuilt read-modify-write across calls)
+    cache = gpu.KVCache(gpu.KV_LLOYDMAX, 1, Hkv, d, T, wl.k_bits, wl.v_bits, wl.k_sign, wl.v_sign)
+    cache.set_rotations(dev(Rk), dev(Rv))
+    edges = [0, 1, 1000, 1031, 4096]
+    for a, b in zip(edges[:-1], edges[1:]):
+        cache.encode_append(Kd[:, :, a:b], Vd[:, :, a:b], rotate=2)
+    for which in (0, 1):
+        got_f, got_a = export(cache, which, T)
+        np.testing.assert_array_equal(got_f, exported[which][0])
+        np.testing.assert_array_equal(got_a, exported[which][1])
+    assert cache.seq_lens() == [T]
+    cache.close()
