@@ -105,6 +105,15 @@ int weed_hip_elementwise_f32(int op, uint32_t rank, const uint32_t *shape, const
 int weed_hip_triu_fill_f32(uint32_t rows, uint32_t cols, float val, uint32_t diagonal, float *a_dev, uint32_t a_off,
                            uint32_t a_s0, uint32_t a_s1);
 
+/* Rotary position embedding: out = x * cos + rotate_half(x) * sin over the last dimension of a strided
+ * [B, H, T, head_dim] tensor, rotate_half(x) = [-x[half:], x[:half]].  Replaces RoPE::forward
+ * (src/modules/rope.cpp:77-98) and its helper _rotate_half (53-75).  cos_dev / sin_dev are the module's tables,
+ * column-major [table_rows, head_dim] as RoPE::_build_tables lays them out (rope.cpp:18-51).  Token t of the call
+ * uses table row pos0 + t; the reference always uses pos0 = 0, a decode step with a cache passes the cache length. */
+int weed_hip_rope_f32(const uint32_t shape[4], const float *x_dev, uint32_t x_off, const uint32_t x_stride[4],
+                      const float *cos_dev, const float *sin_dev, uint32_t table_rows, uint32_t pos0, float *out_dev,
+                      uint32_t o_off, const uint32_t o_stride[4]);
+
 /* Numerically stable softmax along `axis`.  Replaces Weed::softmax (src/ops/softmax.cpp:276-287; OpenCL kernel
  * softmax_forward, qengine.cl:1001-1033).  rank <= 8. */
 int weed_hip_softmax_f32(uint32_t rank, const uint32_t *shape, uint32_t axis, const float *a_dev, uint32_t a_off,

@@ -185,6 +185,27 @@ def triu_fill(a, off, rows, cols, s0, s1, val, diagonal):
     return a
 
 
+def rope_tables(head_dim, max_seq_len, base=10000.0):
+    """(cos, sin) float32 [max_seq_len, head_dim] (logical view of the column-major tables)."""
+    cos_t = np.empty(max_seq_len * head_dim, dtype=np.float32)
+    sin_t = np.empty_like(cos_t)
+    fn = lib().wo_rope_tables
+    fn.argtypes = [c_uint32, c_uint32, c_float, c_void_p, c_void_p]
+    fn(head_dim, max_seq_len, c_float(base), _p(cos_t), _p(sin_t))
+    return cos_t, sin_t
+
+
+def rope_forward(x, cos_t, sin_t, max_seq_len, pos0=0):
+    """x: [B, H, T, head_dim]; cos_t / sin_t: flat column-major tables from rope_tables."""
+    x = _f32(x)
+    B, H, T, d = x.shape
+    out = np.empty_like(x)
+    fn = lib().wo_rope_forward
+    fn.argtypes = [c_void_p, c_uint32, c_uint32, c_uint32, c_uint32, c_void_p, c_void_p, c_uint32, c_uint32, c_void_p]
+    fn(_p(x), B, H, T, d, _p(cos_t), _p(sin_t), max_seq_len, pos0, _p(out))
+    return out
+
+
 # ---- decode attention ----------------------------------------------------------------------------
 
 def decode_attn(kspec, vspec, kf, ka, vf, va, q, seq_lens, gqa_weed=True, Rk=None, Rv=None, want_scores=False):

@@ -12,6 +12,9 @@
  *   wo_matmul, wo_softmax, wo_reduce        : the reference's unit tests (test/tests.cpp:177-228,
  *       1020-1041, 1110-1171, 1206-1221) and float64 numpy closed forms.
  *   wo_triu_fill                            : brute force against the rule i + diag <= j.
+ *   wo_rope_tables / wo_rope_forward        : the reference has no test of RoPE -- PARITY UNPINNED against
+ *       the reference; pinned by float64 closed forms of the tables, the identity at position 0 and the
+ *       per-coordinate formula evaluated independently in numpy.
  *   wo_block_scale                          : float64 closed form (order-dependent in the last ulps).
  *   wo_orthonormalize_columns, wo_apply_rotation : invariants only (R^T R = I, y = x R, R R^T = I);
  *       the reference draws its Gaussian matrix from std::random_device, so no vector exists.
@@ -376,6 +379,53 @@ void wo_triu_fill(float *a, uint32_t off, uint32_t rows, uint32_t cols, uint32_t
         const uint32_t j = idx / rows;
         if ((i + diagonal) <= j) {
             a[off + i * s0 + j * s1] = val;
+        }
+    }
+}
+
+/* ------------------------------------------------------------------------------------------ */
+/* rotary position embedding                                                                   */
+/* ------------------------------------------------------------------------------------------ */
+
+/* src/modules/rope.cpp:18-51 (RoPE::_build_tables): theta_i = base^(-2i/head_dim) in fp32 (std::pow on floats),
+ * angle = pos * theta_i, the cosine / sine stored for BOTH coordinates 2i and 2i+1; tables are column-major
+ * [max_seq_len, head_dim]: entry (pos, j) at pos + j * max_seq_len. */
+void wo_rope_tables(uint32_t head_dim, uint32_t max_seq_len, float base, float *cos_t, float *sin_t)
+{
+    const uint32_t half = head_dim >> 1;
+    for (uint32_t pos = 0; pos < max_seq_len; ++pos) {
+        for (uint32_t i = 0; i < half; ++i) {
+            const float theta = powf(base, -2.0f * (float)i / (float)head_dim);
+            const float angle = (float)pos * theta;
+            const float c = cosf(angle), sn = sinf(angle);
+            cos_t[pos + (size_t)(2 * i) * max_seq_len] = c;
+            cos_t[pos + (size_t)(2 * i + 1) * max_seq_len] = c;
+            sin_t[pos + (size_t)(2 * i) * max_seq_len] = sn;
+            sin_t[pos + (size_t)(2 * i + 1) * max_seq_len] = sn;
+        }
+    }
+}
+
+/* src/modules/rope.cpp:53-98 (RoPE::_rotate_half + RoPE::forward): out = x * cos + rotate_half(x) * sin with
+ * rotate_half(x) = [-x[half:], x[:half]] along the last dimension, each product rounded before the add.  x, out:
+ * dense [B, H, T, head_dim] in C order here (the strides are the caller's business on the device).  The reference
+ * always uses positions 0..T-1; `pos0` shifts them (0 = reference behaviour). */
+void wo_rope_forward(const float *x, uint32_t B, uint32_t H, uint32_t T, uint32_t head_dim, const float *cos_t,
+                     const float *sin_t, uint32_t max_seq_len, uint32_t pos0, float *out)
+{
+    const uint32_t half = head_dim >> 1;
+    for (size_t bh = 0; bh < (size_t)B * H; ++bh) {
+        for (uint32_t t = 0; t < T; ++t) {
+            const float *row = x + (bh * T + t) * head_dim;
+            float *dst = out + (bh * T + t) * head_dim;
+            for (uint32_t j = 0; j < head_dim; ++j) {
+                const float rot = (j < half) ? -row[j + half] : row[j - half];
+                const float c = cos_t[(pos0 + t) + (size_t)j * max_seq_len];
+                const float sn = sin_t[(pos0 + t) + (size_t)j * max_seq_len];
+                const float a = row[j] * c;
+                const float b = rot * sn;
+                dst[j] = a + b;
+            }
         }
     }
 }

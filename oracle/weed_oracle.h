@@ -77,6 +77,12 @@ void wo_triu_fill(float *a, uint32_t off, uint32_t rows, uint32_t cols, uint32_t
 /* ---- single-query decode attention over a quantized cache, in the reference's cost structure
  * (multihead_attention.cpp:259-348): dequantise the whole cache to dense fp32, replicate KV heads,
  * materialise K^T, naive dots, divide by sqrt(d), three-pass softmax, naive P.V, un-rotate. ---- */
+/* RoPE::_build_tables and RoPE::forward (src/modules/rope.cpp:18-98); tables column-major [max_seq_len, head_dim];
+ * x, out dense [B, H, T, head_dim] in C order; pos0 = position of token 0 (the reference always uses 0). */
+void wo_rope_tables(uint32_t head_dim, uint32_t max_seq_len, float base, float *cos_t, float *sin_t);
+void wo_rope_forward(const float *x, uint32_t B, uint32_t H, uint32_t T, uint32_t head_dim, const float *cos_t,
+                     const float *sin_t, uint32_t max_seq_len, uint32_t pos0, float *out);
+
 typedef struct {
     int n_seq, n_q_heads, n_kv_heads, d;
     int max_tokens;          /* row pitch of the field/alpha arrays */

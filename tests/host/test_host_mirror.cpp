@@ -451,10 +451,67 @@ std::vector<double> host_rotate(const std::vector<double> &x, size_t rows, tcapi
 
 std::vector<double> to_double(const std::vector<real1> &v) { return std::vector<double>(v.begin(), v.end()); }
 
-void run_attention_case(KVCoder coder, int bits, bool blocked, uint32_t seed)
+// RoPE on a (B, T, H, hd) column-major array in double, positions pos0 + t, with the module's own tables
+std::vector<double> host_rope(const std::vector<double> &x, tcapint B, tcapint T, tcapint H, tcapint hd, const RoPE &rope,
+    tcapint pos0)
+{
+    const std::vector<real1> ct = rope.cos_table->to_vector(), st = rope.sin_table->to_vector();
+    std::vector<double> y(x.size());
+    const tcapint half = hd / 2U, L = rope.max_seq_len;
+    for (tcapint b = 0; b < B; ++b) {
+        for (tcapint t = 0; t < T; ++t) {
+            for (tcapint h = 0; h < H; ++h) {
+                for (tcapint j = 0; j < hd; ++j) {
+                    auto at = [&](tcapint jj) { return x[b + (size_t)B * (t + (size_t)T * (h + (size_t)H * jj))]; };
+                    const double partner = j < half ? -at(j + half) : at(j - half);
+                    const size_t ti = (pos0 + t) + (size_t)j * L;
+                    y[b + (size_t)B * (t + (size_t)T * (h + (size_t)H * j))] = at(j) * (double)ct[ti] + partner * (double)st[ti];
+                }
+            }
+        }
+    }
+    return y;
+}
+
+TEST_CASE(test_rope_matches_checker, true)
+{
+    // tables and forward pass against the CPU checker's restatement of src/modules/rope.cpp, bit for bit
+    const tcapint B = 2U, H = 3U, T = 5U, hd = 32U, L = 24U;
+    RoPE rope(hd, L, 10000.0f, TEST_DTAG);
+    std::vector<real1> ct((size_t)L * hd), st((size_t)L * hd);
+    wo_rope_tables(hd, L, 10000.0f, ct.data(), st.data());
+    REQUIRE(rope.cos_table->to_vector() == ct);
+    REQUIRE(rope.sin_table->to_vector() == st);
+    const std::vector<real1> xc = gaussian((size_t)B * H * T * hd, 8U); // C order [B][H][T][hd] for the checker
+    std::vector<real1> xcm(xc.size());                                   // column-major for the tensor
+    for (tcapint b = 0; b < B; ++b)
+        for (tcapint h = 0; h < H; ++h)
+            for (tcapint t = 0; t < T; ++t)
+                for (tcapint j = 0; j < hd; ++j)
+                    xcm[b + (size_t)B * (h + (size_t)H * (t + (size_t)T * j))] = xc[(((size_t)b * H + h) * T + t) * hd + j];
+    TensorPtr x = std::make_shared<Tensor>(xcm, std::vector<tcapint>{ B, H, T, hd }, false, TEST_DTAG);
+    for (const tcapint pos0 : { 0U, 7U }) {
+        std::vector<real1> want(xc.size());
+        wo_rope_forward(xc.data(), B, H, T, hd, ct.data(), st.data(), L, pos0, want.data());
+        const std::vector<real1> got = rope.forward(x, pos0)->to_vector();
+        bool same = true;
+        for (tcapint b = 0; b < B && same; ++b)
+            for (tcapint h = 0; h < H && same; ++h)
+                for (tcapint t = 0; t < T && same; ++t)
+                    for (tcapint j = 0; j < hd && same; ++j)
+                        same = got[b + (size_t)B * (h + (size_t)H * (t + (size_t)T * j))] == want[(((size_t)b * H + h) * T + t) * hd + j];
+        REQUIRE(same);
+    }
+    REQUIRE(rope.forward(x)->to_vector() == rope.forward(x, 0U)->to_vector());
+    REQUIRE_THROWS_AS(rope.forward(x, L - T + 1U), std::out_of_range);
+    REQUIRE_THROWS_AS(std::make_shared<RoPE>(31U, L), std::invalid_argument);
+}
+
+void run_attention_case(KVCoder coder, int bits, bool blocked, uint32_t seed, bool with_rope = false)
 {
     const tcapint B = 2U, dm = 96U, H = 4U, Hkv = 2U, hd = 64U;
-    MultiHeadAttention mha(dm, H, Hkv, hd, TEST_DTAG, nullptr, ZERO_R1, -1, true, bits);
+    RoPEPtr rope = with_rope ? std::make_shared<RoPE>(hd, 40U, 10000.0f, TEST_DTAG) : nullptr;
+    MultiHeadAttention mha(dm, H, Hkv, hd, TEST_DTAG, rope, ZERO_R1, -1, true, bits);
     mha.kv_coder = coder;
     mha.gqa_blocked = blocked;
     mha.rotation_seed = seed;
@@ -481,6 +538,9 @@ void run_attention_case(KVCoder coder, int bits, bool blocked, uint32_t seed)
         // check: float64 attention over the rows the device cache actually holds (rotated basis)
         const size_t rows = (size_t)B * T;
         std::vector<double> Qd = host_linear(wq, to_double(xv), rows); // (B, T, H*hd) = (B, T, H, hd)
+        if (with_rope) {
+            Qd = host_rope(Qd, B, T, H, hd, *rope, before); // the query sits at positions before .. before + T - 1
+        }
         Qd = host_rotate(Qd, rows * H, hd, mha.k_rotation);
         const tcapint cap = mha.max_seq_len;
         std::vector<real1> krows((size_t)B * Hkv * (before + T) * hd), vrows(krows.size());
@@ -527,12 +587,13 @@ void run_attention_case(KVCoder coder, int bits, bool blocked, uint32_t seed)
     REQUIRE(mha.k_qcache.d == 0U);
     TensorPtr y = mha.forward(std::make_shared<Tensor>(gaussian(3U * dm, 1U), std::vector<tcapint>{ 3U, 1U, dm }, false, TEST_DTAG));
     REQUIRE(y->shape == (std::vector<tcapint>{ 3U, 1U, dm }));
-    REQUIRE(mha.max_seq_len == 2048U); // the reference's default capacity without RoPE (cpp:173)
+    REQUIRE(mha.max_seq_len == (with_rope ? 40U : 2048U)); // the reference's default capacity (cpp:173)
 }
 
 TEST_CASE(test_attention_uniform_4bit, true) { run_attention_case(KV_UNIFORM, 4, false, 1234U); }
 TEST_CASE(test_attention_uniform_3bit_blocked_gqa, true) { run_attention_case(KV_UNIFORM, 3, true, 99U); }
 TEST_CASE(test_attention_lloydmax, true) { run_attention_case(KV_LLOYDMAX, 4, false, 4321U); }
+TEST_CASE(test_attention_with_rope, true) { run_attention_case(KV_LLOYDMAX, 4, false, 777U, true); }
 
 TEST_CASE(test_attention_uniform_codes_follow_reference_coder, true)
 {

@@ -210,3 +210,21 @@ def test_triu_fill_against_checker(gpu, oracle, rows, cols, diag):
     want = np.asfortranarray(a).ravel(order="F").copy()
     oracle.triu_fill(want, 0, rows, cols, 1, rows, -1.701411835e38, diag)
     np.testing.assert_array_equal(ad.cpu().numpy(), want.reshape((rows, cols), order="F"))
+
+
+@pytest.mark.parametrize("pos0", [0, 11])
+def test_rope_bit_exact_against_checker(gpu, oracle, pos0):
+    """x * cos + rotate_half(x) * sin is two rounded products and one add: bit-exact against the checker, on the
+    (B, heads, T, head_dim) view of a column-major (B, T, heads, head_dim) tensor as the attention module forms it."""
+    import torch
+    rng = np.random.default_rng(12)
+    B, H, T, d, L = 2, 3, 5, 64, 32
+    x = rng.standard_normal((B, H, T, d)).astype(np.float32)
+    cos_t, sin_t = oracle.rope_tables(d, L)
+    want = oracle.rope_forward(x, cos_t, sin_t, L, pos0=pos0)
+    xd = col_major(np.ascontiguousarray(x.transpose(0, 2, 1, 3))).permute(0, 2, 1, 3)  # logical [B, H, T, d]
+    out = torch.zeros((B, H, T, d), device="cuda")
+    gpu.rope(xd, dev(cos_t), dev(sin_t), L, out, pos0=pos0)
+    np.testing.assert_array_equal(out.cpu().numpy(), want)
+    with pytest.raises(gpu.WeedHipError):
+        gpu.rope(xd, dev(cos_t), dev(sin_t), L, out, pos0=L - T + 1)  # positions past the table

@@ -56,6 +56,8 @@ SIGNATURES = {
     "weed_hip_elementwise_f32": (c_int, [c_int, c_uint32, U32P, c_void_p, c_uint32, U32P, c_void_p, c_uint32, U32P,
                                          c_void_p, c_uint32, U32P]),
     "weed_hip_triu_fill_f32": (c_int, [c_uint32, c_uint32, c_float, c_uint32, c_void_p, c_uint32, c_uint32, c_uint32]),
+    "weed_hip_rope_f32": (c_int, [U32P, c_void_p, c_uint32, U32P, c_void_p, c_void_p, c_uint32, c_uint32, c_void_p,
+                                  c_uint32, U32P]),
     "weed_hip_softmax_f32": (c_int, [c_uint32, U32P, c_uint32, c_void_p, c_uint32, U32P, c_void_p, c_uint32, U32P]),
     "weed_hip_reduce_f32": (c_int, [c_int, c_uint32, U32P, c_uint32, c_void_p, c_uint32, U32P, c_void_p, c_uint32,
                                     U32P]),
@@ -263,6 +265,13 @@ def triu_fill(a, val, diagonal=1):
     rows, cols = a.shape
     check(load().weed_hip_triu_fill_f32(rows, cols, val, diagonal, c_void_p(a.data_ptr()), 0, a.stride(0),
                                         a.stride(1)))
+
+
+def rope(x, cos_t, sin_t, table_rows, out, pos0=0):
+    """x, out: torch views [B, H, T, head_dim]; cos_t / sin_t: flat column-major [table_rows, head_dim] tables."""
+    check(load().weed_hip_rope_f32(u32(x.shape), c_void_p(x.data_ptr()), 0, u32(x.stride()), c_void_p(cos_t.data_ptr()),
+                                   c_void_p(sin_t.data_ptr()), table_rows, pos0, c_void_p(out.data_ptr()), 0,
+                                   u32(out.stride())))
 
 
 def softmax(a, out, axis):

@@ -203,6 +203,44 @@ __global__ void __launch_bounds__(256) triu_fill_kernel(float *a, uint32_t rows,
     }
 }
 
+struct RopeGeom {
+    uint32_t shape[4]; // B, H, T, head_dim
+    uint32_t x_stride[4], o_stride[4];
+    uint32_t x_off, o_off;
+    uint32_t table_rows, pos0;
+    uint64_t n;
+};
+
+// out = x * cos + rotate_half(x) * sin (src/modules/rope.cpp:53-98): two rounded products, then the add.
+// One thread per element, dimension 0 fastest.
+__global__ void __launch_bounds__(256) rope_kernel(const float *__restrict__ x, const float *__restrict__ cos_t,
+                                                   const float *__restrict__ sin_t, float *__restrict__ out, RopeGeom g)
+{
+    const uint64_t step = (uint64_t)gridDim.x * blockDim.x;
+    const uint32_t half = g.shape[3] >> 1;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < g.n; i += step) {
+        uint64_t tmp = i;
+        uint32_t c[4];
+        uint64_t xi = g.x_off, oi = g.o_off;
+        for (int dd = 0; dd < 4; ++dd) {
+            c[dd] = (uint32_t)(tmp % g.shape[dd]);
+            tmp /= g.shape[dd];
+            oi += (uint64_t)c[dd] * g.o_stride[dd];
+            if (dd < 3) {
+                xi += (uint64_t)c[dd] * g.x_stride[dd];
+            }
+        }
+        const uint32_t j = c[3];
+        const float xv = x[xi + (uint64_t)j * g.x_stride[3]];
+        const float partner = (j < half) ? -x[xi + (uint64_t)(j + half) * g.x_stride[3]]
+                                         : x[xi + (uint64_t)(j - half) * g.x_stride[3]];
+        const uint64_t ti = (uint64_t)(g.pos0 + c[2]) + (uint64_t)j * g.table_rows;
+        const float a = xv * cos_t[ti];
+        const float b = partner * sin_t[ti];
+        out[oi] = a + b;
+    }
+}
+
 int make_geom(const char *fn, uint32_t rank, const uint32_t *shape, uint32_t axis, uint32_t a_off,
               const uint32_t *a_stride, uint32_t o_off, const uint32_t *o_stride, bool out_keeps_axis, AxisGeom &g)
 {
@@ -308,6 +346,38 @@ int weed_hip_triu_fill_f32(uint32_t rows, uint32_t cols, float val, uint32_t dia
     }
     const uint32_t blocks = (uint32_t)std::min<uint64_t>((n + 255) / 256, 256u * 64u);
     triu_fill_kernel<<<blocks, 256, 0, stream()>>>(a_dev, rows, cols, val, diagonal, a_off, a_s0, a_s1);
+    WEED_HIP_LAUNCH_CHECK();
+    return WEED_HIP_OK;
+}
+
+int weed_hip_rope_f32(const uint32_t shape[4], const float *x_dev, uint32_t x_off, const uint32_t x_stride[4],
+                      const float *cos_dev, const float *sin_dev, uint32_t table_rows, uint32_t pos0, float *out_dev,
+                      uint32_t o_off, const uint32_t o_stride[4])
+{
+    const char *fn = "weed_hip_rope_f32";
+    WEED_HIP_REQUIRE(shape && x_dev && x_stride && cos_dev && sin_dev && out_dev && o_stride, "%s: null pointer", fn);
+    WEED_HIP_REQUIRE(x_dev != out_dev, "%s: cannot run in place", fn);
+    WEED_HIP_TRY(ensure_init());
+    RopeGeom g;
+    g.n = 1;
+    for (int i = 0; i < 4; ++i) {
+        WEED_HIP_REQUIRE(shape[i] > 0, "%s: dimension %d is empty", fn, i);
+        g.shape[i] = shape[i];
+        g.x_stride[i] = x_stride[i];
+        g.o_stride[i] = o_stride[i];
+        g.n *= shape[i];
+    }
+    WEED_HIP_REQUIRE(shape[3] % 2 == 0, "%s: head_dim %u must be even", fn, shape[3]);
+    WEED_HIP_REQUIRE((uint64_t)pos0 + shape[2] <= table_rows, "%s: positions [%u, %u) exceed the table's %u rows", fn,
+                     pos0, pos0 + shape[2], table_rows);
+    WEED_HIP_REQUIRE(g.n < (1ull << 32), "%s: more than 2^32 elements", fn);
+    g.x_off = x_off;
+    g.o_off = o_off;
+    g.table_rows = table_rows;
+    g.pos0 = pos0;
+    ProfileScope prof("rope");
+    const uint32_t blocks = (uint32_t)std::min<uint64_t>((g.n + 255) / 256, 256u * 64u);
+    rope_kernel<<<blocks, 256, 0, stream()>>>(x_dev, cos_dev, sin_dev, out_dev, g);
     WEED_HIP_LAUNCH_CHECK();
     return WEED_HIP_OK;
 }

@@ -16,7 +16,12 @@ bool mfma_decode_supported(uint32_t d, uint32_t wk, uint32_t wv, uint32_t G)
 uint32_t mfma_decode_wavefronts(uint32_t G)
 {
     // every compute unit holds one workgroup: 12 wavefronts, or 8 for the 16-column variant (more registers)
+#ifdef WEED_EXP_DB
+    (void)G;
+    return 8u * 256u;
+#else
     return (G > 8 ? 8u : 12u) * 256u;
+#endif
 }
 
 int launch_mfma_decode(const MfmaParams &p, uint32_t d, hipStream_t s)

@@ -160,7 +160,11 @@ template <int GP, int I> constexpr int bank_mask_of() { return ((1 << (GP / 4)) 
 
 // Wavefronts per workgroup: as many as fit a compute unit at the kernel's register budget (three per SIMD; two for the
 // 16-column variant, which needs more registers), so that one copy of the tables serves the whole compute unit.
+#ifdef WEED_EXP_DB
+template <int GP> constexpr int waves_per_wg() { return 8; }
+#else
 template <int GP> constexpr int waves_per_wg() { return GP == 16 ? 8 : 12; }
+#endif
 
 // GP = number of query-head columns kept per score tile (the group size rounded up to 4, 8 or 16).  The Q.K^T
 // instruction always produces 16 columns; with GP < 16 the useful columns of 16/GP tiles are merged into one register
@@ -310,33 +314,51 @@ __global__ void __launch_bounds__(64 * waves_per_wg<GP>()) decode_mfma_kernel(Mf
     // Single register buffers, refilled as soon as their last reader is done: K (and its row scales) right after the
     // Q.K^T phase of a block, V right after its P.V phase -- so each load has about half a block of work to hide behind
     // and the other wavefronts of the SIMD cover the rest.
-    uint32_t kraw[NK], vraw[NV];
-    float4v ak[NSETS], av[NSETS];
+#ifdef WEED_EXP_DB
+    constexpr int NB = 2;
+#else
+    constexpr int NB = 1;
+#endif
+    uint32_t kraw_[NB][NK], vraw_[NB][NV];
+    float4v ak_[NB][NSETS], av_[NB][NSETS];
 
-    auto load_k = [&](uint32_t blk) {
-        load_dwords<NK>(kreg + (uint64_t)blk * (8u * D * WK), kraw);
+    auto load_k = [&](auto pc, uint32_t blk) {
+        constexpr int P = decltype(pc)::value;
+        load_dwords<NK>(kreg + (uint64_t)blk * (8u * D * WK), kraw_[P]);
 #pragma unroll
         for (int s = 0; s < NSETS; ++s) {
             if constexpr (lloyd) {
-                ak[s] = *reinterpret_cast<const float4v *>(ka + blk * 64 + 16 * TPS * s);
+                ak_[P][s] = *reinterpret_cast<const float4v *>(ka + blk * 64 + 16 * TPS * s);
             } else {
-                ak[s] = float4v{ p.k.alpha_const, p.k.alpha_const, p.k.alpha_const, p.k.alpha_const };
+                ak_[P][s] = float4v{ p.k.alpha_const, p.k.alpha_const, p.k.alpha_const, p.k.alpha_const };
             }
         }
     };
-    auto load_v = [&](uint32_t blk) {
-        load_dwords<NV>(vreg + (uint64_t)blk * (8u * D * WV), vraw);
+    auto load_v = [&](auto pc, uint32_t blk) {
+        constexpr int P = decltype(pc)::value;
+        load_dwords<NV>(vreg + (uint64_t)blk * (8u * D * WV), vraw_[P]);
 #pragma unroll
         for (int s = 0; s < NSETS; ++s) {
             if constexpr (lloyd) {
-                av[s] = *reinterpret_cast<const float4v *>(va + blk * 64 + 16 * TPS * s);
+                av_[P][s] = *reinterpret_cast<const float4v *>(va + blk * 64 + 16 * TPS * s);
             } else {
-                av[s] = float4v{ 1.0f, 1.0f, 1.0f, 1.0f };
+                av_[P][s] = float4v{ 1.0f, 1.0f, 1.0f, 1.0f };
             }
         }
     };
 
-    auto process_block = [&](uint32_t blk, uint32_t next_blk) {
+    auto process_block = [&](auto pc, uint32_t blk, uint32_t next_blk) {
+        constexpr int P = decltype(pc)::value;
+        constexpr std::integral_constant<int, (NB == 2 ? 1 - P : 0)> other{};
+        auto &kraw = kraw_[P];
+        auto &vraw = vraw_[P];
+        auto &ak = ak_[P];
+        auto &av = av_[P];
+        if constexpr (NB == 2) {
+            // double buffering: the whole next block is requested before this one is touched
+            load_k(other, next_blk);
+            load_v(other, next_blk);
+        }
         // ---- S[t] = K_tile . q: rows = tokens 16t + (lane%16), contraction over the lane groups' coordinates.
         //      Items are taken in memory order (tile after tile); lookups run two items ahead of the matrix
         //      instructions that consume them. ----
@@ -394,7 +416,9 @@ __global__ void __launch_bounds__(64 * waves_per_wg<GP>()) decode_mfma_kernel(Mf
                 C[s][r] = fmaf(v, ak[s][r] * qscale, betaq);
             }
         }
-        load_k(next_blk); // the K buffer is free again
+        if constexpr (NB == 1) {
+            load_k(other, next_blk); // the K buffer is free again
+        }
         if (blk * 64 + 64 > L) {
 #pragma unroll
             for (int s = 0; s < NSETS; ++s) {
@@ -529,7 +553,9 @@ __global__ void __launch_bounds__(64 * waves_per_wg<GP>()) decode_mfma_kernel(Mf
                 b1v = b2v;
             });
         }
-        load_v(next_blk); // the V buffer is free again
+        if constexpr (NB == 1) {
+            load_v(other, next_blk); // the V buffer is free again
+        }
     };
 
     // ---- main loop.  The refills are unconditional (the next block index is clamped to the last block of the
@@ -538,10 +564,22 @@ __global__ void __launch_bounds__(64 * waves_per_wg<GP>()) decode_mfma_kernel(Mf
         uint32_t blk = b0;
         if (blk < b1) {
             const uint32_t last = b1 - 1;
-            load_k(blk);
-            load_v(blk);
-            for (; blk < b1; ++blk) {
-                process_block(blk, min(blk + 1, last));
+            constexpr std::integral_constant<int, 0> p0{};
+            load_k(p0, blk);
+            load_v(p0, blk);
+            if constexpr (NB == 2) {
+                constexpr std::integral_constant<int, 1> p1{};
+                for (; blk + 1 < b1; blk += 2) {
+                    process_block(p0, blk, blk + 1);
+                    process_block(p1, blk + 1, min(blk + 2, last));
+                }
+                if (blk < b1) {
+                    process_block(p0, blk, last);
+                }
+            } else {
+                for (; blk < b1; ++blk) {
+                    process_block(p0, blk, min(blk + 1, last));
+                }
             }
         }
     }

@@ -792,6 +792,67 @@ std::vector<ParameterPtr> Linear::parameters()
 }
 
 // ---------------------------------------------------------------------------------------------------------
+// RoPE
+// ---------------------------------------------------------------------------------------------------------
+
+RoPE::RoPE(const tcapint &head_dim_, const tcapint &max_seq_len_, const real1_f &base_, DeviceTag dtag)
+    : head_dim(head_dim_)
+    , max_seq_len(max_seq_len_)
+    , base(base_)
+{
+    if (!head_dim || (head_dim & 1U) || !max_seq_len) {
+        throw std::invalid_argument("RoPE: head_dim must be even and max_seq_len positive");
+    }
+    _build_tables(dtag);
+}
+
+void RoPE::_build_tables(DeviceTag dtag)
+{
+    // theta_i = base^(-2i/head_dim); entry (pos, 2i) = (pos, 2i+1) = cos / sin (pos * theta_i); column-major
+    const tcapint half = head_dim >> 1U;
+    std::vector<real1> cos_data((size_t)max_seq_len * head_dim), sin_data((size_t)max_seq_len * head_dim);
+    for (tcapint pos = 0U; pos < max_seq_len; ++pos) {
+        for (tcapint i = 0U; i < half; ++i) {
+            const real1_f theta = (real1_f)std::pow(base, -2.0f * (real1_f)i / (real1_f)head_dim);
+            const real1_f angle = (real1_f)pos * theta;
+            const real1 c = (real1)std::cos(angle), sn = (real1)std::sin(angle);
+            for (tcapint e = 0U; e < 2U; ++e) {
+                cos_data[pos + (size_t)(2U * i + e) * max_seq_len] = c;
+                sin_data[pos + (size_t)(2U * i + e) * max_seq_len] = sn;
+            }
+        }
+    }
+    cos_table = std::make_shared<Tensor>(cos_data, std::vector<tcapint>{ max_seq_len, head_dim }, false, dtag);
+    sin_table = std::make_shared<Tensor>(sin_data, std::vector<tcapint>{ max_seq_len, head_dim }, false, dtag);
+}
+
+void RoPE::apply(const Tensor &x, Tensor &out, tcapint pos0)
+{
+    if (x.shape.size() != 4U || x.shape[3U] != head_dim || out.shape != x.shape) {
+        throw std::invalid_argument("RoPE: input and output must be (B, H, T, head_dim)");
+    }
+    validate_all_same_device({ &x, &out, cos_table.get(), sin_table.get() }, "RoPE::forward");
+    if ((uint64_t)pos0 + x.shape[2U] > max_seq_len) {
+        throw std::out_of_range("RoPE: positions beyond max_seq_len");
+    }
+    real1 *xp = device_ptr(x, "RoPE::forward"), *op = device_ptr(out, "RoPE::forward");
+    real1 *cp = device_ptr(*cos_table, "RoPE::forward"), *sp = device_ptr(*sin_table, "RoPE::forward");
+    WEED_DEVICE_LOCK();
+    HipDevice::check(weed_hip_rope_f32(x.shape.data(), xp, x.offset, x.stride.data(), cp + cos_table->offset,
+        sp + sin_table->offset, max_seq_len, pos0, op, out.offset, out.stride.data()));
+}
+
+TensorPtr RoPE::forward(const TensorPtr x, tcapint pos0)
+{
+    if (x->shape.size() != 4U) {
+        throw std::invalid_argument("RoPE::forward(): input must be (B, H, T, head_dim)");
+    }
+    TensorPtr out = allocate(x->shape, *x);
+    apply(*x, *out, pos0);
+    return out;
+}
+
+// ---------------------------------------------------------------------------------------------------------
 // quantized cache
 // ---------------------------------------------------------------------------------------------------------
 
@@ -914,8 +975,9 @@ MultiHeadAttention::MultiHeadAttention(tcapint d_model_, tcapint num_heads_, tca
     , use_kv_cache(_use_kv_cache)
     , kv_quant_bits(kv_quant_bits_)
 {
-    if (r) {
-        throw std::domain_error("MultiHeadAttention: rotary position embedding is not part of this build");
+    rope = r;
+    if (rope && (symint)rope->head_dim != head_dim) {
+        throw std::invalid_argument("MultiHeadAttention: RoPE head_dim does not match");
     }
     if (d_model % num_heads) {
         throw std::invalid_argument("d_model must be divisible by num_heads");
@@ -975,6 +1037,21 @@ TensorPtr MultiHeadAttention::forward(const TensorPtr x)
     Q = Tensor::reshape(Q, { B, T, num_heads, head_dim });
     K = Tensor::reshape(K, { B, T, num_kv_heads, head_dim });
     V = Tensor::reshape(V, { B, T, num_kv_heads, head_dim });
+
+    if (rope) {
+        // optional RoPE on the (B, heads, T, head_dim) views, at the tokens' positions in the sequence
+        const tcapint pos0 = use_kv_cache ? cache_len : 0U;
+        if (use_kv_cache && !max_seq_len) {
+            max_seq_len = rope->max_seq_len; // the reference's default capacity with RoPE (cpp:173)
+        }
+        // written straight into fresh contiguous (B, T, heads, head_dim) tensors through transposed views
+        for (TensorPtr *t : { &Q, &K }) {
+            TensorPtr fresh = allocate((*t)->shape, **t);
+            TensorPtr fresh_view = Tensor::transpose(fresh, 1, 2);
+            rope->apply(*Tensor::transpose(*t, 1, 2), *fresh_view, pos0);
+            *t = fresh;
+        }
+    }
 
     TensorPtr out = (use_kv_cache && kv_quant_bits > 0) ? forward_quantized(Q, K, V, B, T) : forward_dense(Q, K, V, B, T);
 

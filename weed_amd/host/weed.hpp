@@ -272,9 +272,24 @@ struct QuantizedKVCache {
 
 enum KVCoder { KV_UNIFORM = 0, KV_LLOYDMAX = 1 };
 
-// include/modules/rope.hpp: rotary embedding is not on this path; the type exists so that the attention constructor
-// keeps the reference's argument list, and only a null pointer is accepted.
-struct RoPE;
+// include/modules/rope.hpp, src/modules/rope.cpp: rotary position embedding.  The tables are built on the host with
+// the reference's fp32 arithmetic (rope.cpp:18-51) and live on the device; forward() is one fused kernel.
+// forward(x, pos0) is an extension: token t of x uses position pos0 + t (the reference always starts at 0, which is
+// only right for a call that begins a sequence).
+struct RoPE : public Module {
+    tcapint head_dim;
+    tcapint max_seq_len;
+    real1_f base;
+    TensorPtr cos_table; // [max_seq_len, head_dim]
+    TensorPtr sin_table; // [max_seq_len, head_dim]
+
+    RoPE(const tcapint &head_dim_, const tcapint &max_seq_len_ = 2048U, const real1_f &base_ = 10000.0f,
+        DeviceTag dtag = DEFAULT_DEVICE);
+    void _build_tables(DeviceTag dtag);
+    TensorPtr forward(const TensorPtr x) override { return forward(x, 0U); }
+    TensorPtr forward(const TensorPtr x, tcapint pos0); // x: [B, H, T, head_dim], any strides
+    void apply(const Tensor &x, Tensor &out, tcapint pos0); // the same into a given (possibly strided) output
+};
 typedef std::shared_ptr<RoPE> RoPEPtr;
 
 // include/modules/multihead_attention.hpp:41-173.  Differences, all deliberate:
@@ -283,6 +298,8 @@ typedef std::shared_ptr<RoPE> RoPEPtr;
 //  * tokens are appended in logical order, so prefill followed by decode steps is consistent (the reference's row
 //    order only works for a single call);
 //  * the causal mask honours the cache offset, and set_max_kv_seq_len() survives the first forward();
+//  * RoPE, when present, is applied at the tokens' true positions (cache_len onwards), and max_seq_len defaults to
+//    the RoPE table length as in the reference (cpp:173);
 //  * rotation_seed makes the rotations reproducible (0 = draw a seed from std::random_device like the reference);
 //    rotations already present in k_rotation / v_rotation at the first forward() are used as given;
 //  * kv_coder selects the reference's uniform coder (default) or the Lloyd-Max coder with k_bits / v_bits / sign
@@ -299,7 +316,7 @@ struct MultiHeadAttention : public Module {
     LinearPtr W_v;
     LinearPtr W_o;
 
-    RoPEPtr rope; // always null
+    RoPEPtr rope; // applied to Q and K before the cache, at position cache_len (the reference: always position 0)
 
     bool use_kv_cache;
     TensorPtr k_cache; // float cache (kv_quant_bits == 0)
