@@ -170,7 +170,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path is sharded by (sequence, kv head) with no "
-              "exchange; see DESIGN.md); run with --gpus 1", file=sys.stderr)
+              "exchange between GPUs); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
 
     import numpy as np

@@ -147,7 +147,7 @@ def test_device_rotation_modes(gpu, oracle, mode):
 
 def test_incremental_and_ragged_append(gpu, oracle):
     """Appending token by token, in uneven chunks and per sequence must give the cache a one-shot encode gives
-    (the reference's own incremental append re-reads old rows with the wrong strides)."""
+    (the reference's own incremental append re-reads old rows with the wrong strides, multihead_attention.cpp:247-273)."""
     rng = np.random.default_rng(5)
     S, Hkv, d, cap = 3, 2, 64, 300
     lens = [300, 71, 190]
