@@ -686,7 +686,7 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         blocks *= Hkv;
         WEED_HIP_REQUIRE(blocks < (1ull << 32), "%s: too many cached tokens for one launch", fn);
         total_blocks = (uint32_t)blocks;
-        uint32_t target_units = mfma_decode_wavefronts(G);
+        uint32_t target_units = mfma_decode_wavefronts(G, d, c->k.w, c->v.w);
         if (const char *env = std::getenv("WEED_HIP_DECODE_WAVES")) {
             target_units = (uint32_t)std::max(1, std::atoi(env)); // tuning knob
         }

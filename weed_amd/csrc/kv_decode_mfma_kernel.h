@@ -158,21 +158,13 @@ template <int GP> __device__ __forceinline__ float head_sum(float v)
 // Bank mask (4-lane banks of a row) of the lanes [GP*i, GP*i + GP).
 template <int GP, int I> constexpr int bank_mask_of() { return ((1 << (GP / 4)) - 1) << (I * GP / 4); }
 
-// Wavefronts per workgroup: as many as fit a compute unit at the kernel's register budget (three per SIMD; two for the
-// 16-column variant, which needs more registers), so that one copy of the tables serves the whole compute unit.
-#ifdef WEED_EXP_DB
-template <int GP> constexpr int waves_per_wg() { return 8; }
-#else
-template <int GP> constexpr int waves_per_wg() { return GP == 16 ? 8 : 12; }
-#endif
-
 // GP = number of query-head columns kept per score tile (the group size rounded up to 4, 8 or 16).  The Q.K^T
 // instruction always produces 16 columns; with GP < 16 the useful columns of 16/GP tiles are merged into one register
 // set before the softmax, so the exponentials and the fp16 splitting run on full registers.
 template <int D, int WK, int WV, int GP, bool LLOYD>
-__global__ void __launch_bounds__(64 * waves_per_wg<GP>()) decode_mfma_kernel(MfmaParams p)
+__global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) decode_mfma_kernel(MfmaParams p)
 {
-    constexpr int kWaves = waves_per_wg<GP>();
+    constexpr int kWaves = (int)mfma_decode_waves_per_wg(GP, D, WK, WV);
     constexpr int KS = D / 32;       // Q.K^T k-steps (32 coordinates each); also K items per tile per lane
     constexpr int JB = D / 16;       // 16-coordinate column blocks of the output
     constexpr int NK = KS * WK;      // dwords of packed K per lane per block
@@ -314,11 +306,10 @@ __global__ void __launch_bounds__(64 * waves_per_wg<GP>()) decode_mfma_kernel(Mf
     // Single register buffers, refilled as soon as their last reader is done: K (and its row scales) right after the
     // Q.K^T phase of a block, V right after its P.V phase -- so each load has about half a block of work to hide behind
     // and the other wavefronts of the SIMD cover the rest.
-#ifdef WEED_EXP_DB
-    constexpr int NB = 2;
-#else
-    constexpr int NB = 1;
-#endif
+    // Register buffers for the packed block: one (refilled as soon as its last reader is done: K right after the
+    // Q.K^T phase, V right after the P.V phase), or two when the shape is double-buffered (the whole next block is
+    // requested before the current one is touched).
+    constexpr int NB = mfma_decode_double_buffered(GP, D, WK, WV) ? 2 : 1;
     uint32_t kraw_[NB][NK], vraw_[NB][NV];
     float4v ak_[NB][NSETS], av_[NB][NSETS];
 
@@ -632,7 +623,7 @@ __global__ void __launch_bounds__(64 * waves_per_wg<GP>()) decode_mfma_kernel(Mf
 template <int D, int WK, int WV, int GP, bool LLOYD> int launch_gp(const MfmaParams &p, hipStream_t s)
 {
     constexpr size_t smem = (size_t)table_rows<WK, WV>() * kTableRowBytes + 64 * sizeof(uint16_t);
-    constexpr uint32_t waves = (uint32_t)waves_per_wg<GP>();
+    constexpr uint32_t waves = mfma_decode_waves_per_wg(GP, D, WK, WV);
     static bool configured = false;
     if (!configured) {
         WEED_HIP_CHECK(hipFuncSetAttribute((const void *)decode_mfma_kernel<D, WK, WV, GP, LLOYD>,
