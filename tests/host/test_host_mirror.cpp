@@ -526,7 +526,7 @@ void run_attention_case(KVCoder coder, int bits, bool blocked, uint32_t seed, bo
     (void)wv;
 
     tcapint before = 0U;
-    for (const tcapint T : { 7U, 1U, 1U, 3U }) { // prefill, two decode steps, a chunk
+    for (const tcapint T : { 7U, 1U, 1U, 3U, 12U }) { // prefill, two decode steps, a chunk, a long chunk (dense path)
         const std::vector<real1> xv = gaussian((size_t)B * T * dm, seed + 100U + before);
         TensorPtr x = std::make_shared<Tensor>(xv, std::vector<tcapint>{ B, T, dm }, false, TEST_DTAG);
         TensorPtr y = mha.forward(x);

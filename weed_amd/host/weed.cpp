@@ -1018,6 +1018,7 @@ void MultiHeadAttention::reset_cache()
     v_rotation_trans.clear();
     k_rot_dev = nullptr;
     v_rot_dev = nullptr;
+    v_rot_t_dev = nullptr;
     k_qcache = QuantizedKVCache{};
     v_qcache = QuantizedKVCache{};
 }
@@ -1147,6 +1148,28 @@ TensorPtr MultiHeadAttention::forward_quantized(TensorPtr Q, TensorPtr K, Tensor
         HipDevice::check(weed_hip_kv_decode_attn(cache, num_heads, gqa, qp, Q->offset, q_str, op, 0U, q_str, flags));
         return out;
     }
+    if (uT > kFusedQueryLimit) {
+        // Long multi-token calls (prefill): the fused kernel serves one query position per launch, so beyond a few
+        // positions it is cheaper to do what the reference does -- dequantise the cache once (still in the rotated
+        // basis) and run dense matrix products: rotate Q, attend, un-rotate.
+        TensorPtr K_deq = allocate({ uB, Hkv, cache_len, hd }, *Q), V_deq = allocate({ uB, Hkv, cache_len, hd }, *Q);
+        HipDevice::check(weed_hip_kv_dequant(cache, 0, 0, B, 0, (int32_t)cache_len, device_ptr(*K_deq, "forward"), 0U,
+            K_deq->stride.data()));
+        HipDevice::check(weed_hip_kv_dequant(cache, 1, 0, B, 0, (int32_t)cache_len, device_ptr(*V_deq, "forward"), 0U,
+            V_deq->stride.data()));
+        TensorPtr Qv = Tensor::transpose(Q, 1, 2); // (B, H, T, hd) view
+        TensorPtr Q_rot = allocate(Qv->shape, *Q);
+        HipDevice::check(weed_hip_apply_rotation_f32(hd, k_rot_dev->buffer, 4U, Qv->shape.data(), qp, Qv->offset,
+            Qv->stride.data(), device_ptr(*Q_rot, "forward"), 0U, Q_rot->stride.data()));
+        TensorPtr att = attend_dense(Q_rot, K_deq, V_deq, before); // (B, H, T, hd), rotated basis
+        if (!v_rot_t_dev) {
+            v_rot_t_dev = std::make_shared<GpuRealStorage>(v_rotation_trans);
+        }
+        TensorPtr outv = Tensor::transpose(out, 1, 2); // (B, H, T, hd) view of the (B, T, H, hd) result
+        HipDevice::check(weed_hip_apply_rotation_f32(hd, v_rot_t_dev->buffer, 4U, att->shape.data(),
+            device_ptr(*att, "forward"), att->offset, att->stride.data(), op, 0U, outv->stride.data()));
+        return out;
+    }
     // causal attention: query position t sees the first before + t + 1 cached tokens of its sequence
     const size_t need = sizeof(int32_t) * (size_t)uB * uT;
     if (need > lens_cap) {
@@ -1176,7 +1199,7 @@ TensorPtr MultiHeadAttention::forward_quantized(TensorPtr Q, TensorPtr K, Tensor
 // device op.  Returns (B, T, num_heads, head_dim).
 TensorPtr MultiHeadAttention::forward_dense(TensorPtr Q, TensorPtr K, TensorPtr V, symint B, symint T)
 {
-    const tcapint hd = (tcapint)head_dim, Hkv = (tcapint)num_kv_heads, Hq = (tcapint)num_heads;
+    const tcapint hd = (tcapint)head_dim, Hkv = (tcapint)num_kv_heads;
     const tcapint uB = (tcapint)B, uT = (tcapint)T;
     Q = Tensor::transpose(Q, 1, 2); // [B, num_heads, T, head_dim]
     K = Tensor::transpose(K, 1, 2); // [B, kv_heads,  T, head_dim]
@@ -1205,6 +1228,15 @@ TensorPtr MultiHeadAttention::forward_dense(TensorPtr Q, TensorPtr K, TensorPtr 
         V = Tensor::slice(v_cache, 2, 0U, cache_len);
     }
 
+    return Tensor::transpose(attend_dense(Q, K, V, before), 1, 2); // (B, T, H, head_dim)
+}
+
+// Dense causal attention as the reference spells it (multihead_attention.cpp:291-337): Q (B, H, T, hd), K and V
+// (B, Hkv, T_k, hd) with the T new tokens last; query t sees keys 0 .. before + t.  Returns (B, H, T, hd).
+TensorPtr MultiHeadAttention::attend_dense(TensorPtr Q, TensorPtr K, TensorPtr V, tcapint before)
+{
+    const tcapint hd = (tcapint)head_dim, Hkv = (tcapint)num_kv_heads, Hq = (tcapint)num_heads;
+    const tcapint uB = Q->shape[0U], uT = Q->shape[2U];
     if (num_kv_heads < num_heads) {
         const tcapint groups = Hq / Hkv, T_k = K->shape[2U];
         TensorPtr K_rep = Tensor::zeros({ uB, Hq, T_k, hd }, false, false, DType::REAL, Q->storage->device);
@@ -1226,15 +1258,14 @@ TensorPtr MultiHeadAttention::forward_dense(TensorPtr Q, TensorPtr K, TensorPtr 
 
     TensorPtr scores = Q >> Tensor::transpose(K, -2, -1);
     scores = scores / real1(std::sqrt((real1)head_dim));
-    if (T > 1) {
+    if (uT > 1U) {
         const tcapint T_k = K->shape[2U];
         TensorPtr mask = Tensor::zeros({ uT, T_k }, false, false, DType::REAL, Q->storage->device);
         Weed::triu_fill(*mask, (real1)mask_val, before + 1U);
         scores = scores + mask;
     }
     TensorPtr weights = Tensor::softmax(scores, -1);
-    TensorPtr out = weights >> V;
-    return Tensor::transpose(out, 1, 2); // (B, T, H, head_dim)
+    return weights >> V;
 }
 
 } // namespace Weed

@@ -352,7 +352,9 @@ struct MultiHeadAttention : public Module {
 private:
     TensorPtr forward_quantized(TensorPtr Q, TensorPtr K, TensorPtr V, symint B, symint T);
     TensorPtr forward_dense(TensorPtr Q, TensorPtr K, TensorPtr V, symint B, symint T);
-    std::shared_ptr<GpuRealStorage> k_rot_dev, v_rot_dev; // device copies of the rotations
+    TensorPtr attend_dense(TensorPtr Q, TensorPtr K, TensorPtr V, tcapint before);
+    std::shared_ptr<GpuRealStorage> k_rot_dev, v_rot_dev, v_rot_t_dev; // device copies of the rotations
+    static constexpr tcapint kFusedQueryLimit = 8U; // multi-token calls up to this many positions use the fused kernel
     void *lens_dev = nullptr; // int32 prefix lengths for multi-token calls
     size_t lens_cap = 0U;
 
