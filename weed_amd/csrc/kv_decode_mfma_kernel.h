@@ -31,8 +31,11 @@ typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
 
 // N dwords from a pointer aligned to 16 bytes when N % 4 == 0, else to 8 bytes (N is even for every supported shape).
-template <int N> __device__ __forceinline__ void load_dwords(const uint8_t *p, uint32_t (&x)[N])
+// `base` is the same in every lane and `lane_off` a 32-bit byte offset, so the loads take the scalar-base form (one
+// offset register per lane instead of a 64-bit address).
+template <int N> __device__ __forceinline__ void load_dwords(const uint8_t *base, uint32_t lane_off, uint32_t (&x)[N])
 {
+    const uint8_t *p = base + lane_off;
     if constexpr (N % 4 == 0) {
 #pragma unroll
         for (int i = 0; i < N / 4; ++i) {
@@ -179,9 +182,10 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     const uint32_t c = lane & 15, g = lane >> 4;
     constexpr bool lloyd = LLOYD;
 
-    // ---- build the pair tables.  The 2^w fp16 levels are staged in LDS first so that building the pairs needs no
-    //      global reads. ----
-    {
+    // ---- the pair tables.  The 2^w fp16 levels are staged in LDS first so that building the pairs needs no global
+    //      reads.  Every wavefront of the workgroup calls this exactly once (it contains barriers): wavefronts with
+    //      work after they have requested their first block and query, so that those loads travel meanwhile. ----
+    auto build_tables = [&]() {
         uint16_t *levels_h = reinterpret_cast<uint16_t *>(lds + ROWS * (kTableRowBytes / 4)); // [2][32]
         if (tid < 64) {
             const float lv = (tid < 32) ? p.k.table[tid & 31] : p.v.table[tid & 31];
@@ -199,7 +203,8 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
             lds[i] = val;
         }
         __syncthreads();
-    }
+    };
+    bool tables_ready = false;
     const uint32_t vbase = (lane & 31) * 4; // lane byte of a V lookup
     const uint32_t kbase = vbase + 128;     // lane byte of a K lookup
 
@@ -210,19 +215,21 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     uint32_t g0 = unit * p.unit_blocks;
     const uint32_t g1 = min(g0 + p.unit_blocks, p.total_blocks);
     if (g0 >= g1) {
-        return; // no barrier follows
+        build_tables();
+        return;
     }
     uint32_t seq;
     {
-        // largest s with blk_off[s] * Hkv <= g0 (sequences without tokens share their offset with the next one)
+        // largest s with blk_off[s] * Hkv <= g0 (sequences without tokens share their offset with the next one):
+        // a 64-way search, one probe per lane and step
         uint32_t lo = 0, hi = p.n_seq;
         while (hi - lo > 1) {
-            const uint32_t mid = (lo + hi) >> 1;
-            if (p.blk_off[mid] * p.Hkv <= g0) {
-                lo = mid;
-            } else {
-                hi = mid;
-            }
+            const uint32_t stride = (hi - lo + 63) >> 6;
+            const uint32_t idx = lo + lane * stride;
+            const bool le = idx < hi && p.blk_off[idx] * p.Hkv <= g0; // true for a prefix of the lanes, lane 0 included
+            const uint32_t n_le = (uint32_t)__builtin_popcountll(__ballot(le));
+            lo += (n_le - 1) * stride;
+            hi = min(lo + stride, hi);
         }
         seq = __builtin_amdgcn_readfirstlane(lo);
     }
@@ -298,10 +305,13 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
         O[jb] = float4v{ 0.0f, 0.0f, 0.0f, 0.0f };
     }
 
-    const uint8_t *kreg = p.k.fields + region * p.k.region_bytes + (uint64_t)lane * (4 * NK);
-    const uint8_t *vreg = p.v.fields + region * p.v.region_bytes + (uint64_t)lane * (4 * NV);
-    const float *ka = lloyd ? p.k.alpha + region * p.padded + 16 * tile_in_set + 4 * g : nullptr;
-    const float *va = lloyd ? p.v.alpha + region * p.padded + 16 * tile_in_set + 4 * g : nullptr;
+    // region bases are the same in every lane; the lane's share is a 32-bit offset
+    const uint8_t *kreg = p.k.fields + region * p.k.region_bytes;
+    const uint8_t *vreg = p.v.fields + region * p.v.region_bytes;
+    const uint32_t klane = lane * (4 * NK), vlane = lane * (4 * NV);
+    const float *ka = lloyd ? p.k.alpha + region * p.padded : nullptr;
+    const float *va = lloyd ? p.v.alpha + region * p.padded : nullptr;
+    const uint32_t alane = 16 * tile_in_set + 4 * g;
 
     // Single register buffers, refilled as soon as their last reader is done: K (and its row scales) right after the
     // Q.K^T phase of a block, V right after its P.V phase -- so each load has about half a block of work to hide behind
@@ -315,11 +325,11 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
 
     auto load_k = [&](auto pc, uint32_t blk) {
         constexpr int P = decltype(pc)::value;
-        load_dwords<NK>(kreg + (uint64_t)blk * (8u * D * WK), kraw_[P]);
+        load_dwords<NK>(kreg + (uint64_t)blk * (8u * D * WK), klane, kraw_[P]);
 #pragma unroll
         for (int s = 0; s < NSETS; ++s) {
             if constexpr (lloyd) {
-                ak_[P][s] = *reinterpret_cast<const float4v *>(ka + blk * 64 + 16 * TPS * s);
+                ak_[P][s] = *reinterpret_cast<const float4v *>(ka + blk * 64 + 16 * TPS * s + alane);
             } else {
                 ak_[P][s] = float4v{ p.k.alpha_const, p.k.alpha_const, p.k.alpha_const, p.k.alpha_const };
             }
@@ -327,11 +337,11 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     };
     auto load_v = [&](auto pc, uint32_t blk) {
         constexpr int P = decltype(pc)::value;
-        load_dwords<NV>(vreg + (uint64_t)blk * (8u * D * WV), vraw_[P]);
+        load_dwords<NV>(vreg + (uint64_t)blk * (8u * D * WV), vlane, vraw_[P]);
 #pragma unroll
         for (int s = 0; s < NSETS; ++s) {
             if constexpr (lloyd) {
-                av_[P][s] = *reinterpret_cast<const float4v *>(va + blk * 64 + 16 * TPS * s);
+                av_[P][s] = *reinterpret_cast<const float4v *>(va + blk * 64 + 16 * TPS * s + alane);
             } else {
                 av_[P][s] = float4v{ 1.0f, 1.0f, 1.0f, 1.0f };
             }
@@ -553,11 +563,17 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     //      segment) so that the loop body has no branch around loads and outstanding loads can be counted exactly. ----
     {
         uint32_t blk = b0;
+        constexpr std::integral_constant<int, 0> p0{};
         if (blk < b1) {
-            const uint32_t last = b1 - 1;
-            constexpr std::integral_constant<int, 0> p0{};
             load_k(p0, blk);
             load_v(p0, blk);
+        }
+        if (!tables_ready) {
+            build_tables(); // while the first block and the query are on their way
+            tables_ready = true;
+        }
+        if (blk < b1) {
+            const uint32_t last = b1 - 1;
             if constexpr (NB == 2) {
                 constexpr std::integral_constant<int, 1> p1{};
                 for (; blk + 1 < b1; blk += 2) {
