@@ -415,11 +415,27 @@ __global__ void __launch_bounds__(kThreads) decode_generic_kernel(DecodeParams p
 
 // Merge the partials of all splits: out = sum_s e^(m_s - M) o_s / sum_s e^(m_s - M) l_s, then multiply by
 // v_rotation^T (multihead_attention.cpp:343-348): out_i = sum_j O_j Rv[i + d*j].
+// Run-length skew between the wavefront age classes of a workgroup, in percent of the mean run (see RunGeom).
+constexpr uint32_t kRunSkewPercent = 8;
+
 struct SlotGeom {
     const uint32_t *blk_off; // null: every (sequence, head) has `max_slots` valid partials
-    uint32_t Hkv, G, unit_blocks;
+    uint32_t Hkv, G;
+    RunGeom runs; // matrix-core kernel: how the block list was cut into per-wavefront runs
     int blocked;
 };
+
+// Partial slots of head h of sequence s: the wavefronts whose runs intersect the head's region, in order.
+__device__ __forceinline__ uint32_t slots_of_row(const SlotGeom &sg, uint32_t s, uint32_t h)
+{
+    const uint32_t first_blk = sg.blk_off[s], nb = sg.blk_off[s + 1] - first_blk;
+    if (nb == 0) {
+        return 0;
+    }
+    const uint32_t kvh = sg.blocked ? h / sg.G : h % sg.Hkv;
+    const uint32_t begin = first_blk * sg.Hkv + kvh * nb;
+    return run_of_block(sg.runs, begin + nb - 1) - run_of_block(sg.runs, begin) + 1;
+}
 
 __global__ void combine_kernel(const float *__restrict__ partials, uint32_t Hq, uint32_t d, uint32_t max_slots,
                                SlotGeom sg, const float *__restrict__ rv, int unrotate, int log2_domain,
@@ -433,11 +449,7 @@ __global__ void combine_kernel(const float *__restrict__ partials, uint32_t Hq, 
     const float *base = partials + ((uint64_t)s * Hq + h) * max_slots * (d + 2);
     uint32_t n_splits = max_slots;
     if (sg.blk_off) {
-        // the wavefronts whose block runs intersect this head's region, in order
-        const uint32_t first_blk = sg.blk_off[s], nb = sg.blk_off[s + 1] - first_blk;
-        const uint32_t kvh = sg.blocked ? h / sg.G : h % sg.Hkv;
-        const uint32_t begin = first_blk * sg.Hkv + kvh * nb;
-        n_splits = nb ? (begin + nb - 1) / sg.unit_blocks - begin / sg.unit_blocks + 1 : 0;
+        n_splits = slots_of_row(sg, s, h);
     }
     // n_splits <= 1024 is enforced by the host
     if (tid < 64) {
@@ -525,11 +537,7 @@ __global__ void __launch_bounds__(256) combine_rows_kernel(const float *__restri
         if (row < n_rows) {
             n = max_slots;
             if (sg.blk_off) {
-                const uint32_t s = row / Hq, h = row % Hq;
-                const uint32_t first_blk = sg.blk_off[s], nb = sg.blk_off[s + 1] - first_blk;
-                const uint32_t kvh = sg.blocked ? h / sg.G : h % sg.Hkv;
-                const uint32_t begin = first_blk * sg.Hkv + kvh * nb;
-                n = nb ? (begin + nb - 1) / sg.unit_blocks - begin / sg.unit_blocks + 1 : 0;
+                n = slots_of_row(sg, row / Hq, row % Hq);
             }
         }
         const float *base = partials + (uint64_t)row * max_slots * PS;
@@ -675,7 +683,8 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
     const uint32_t G = Hq / Hkv;
     const bool use_mfma = mfma_decode_supported(d, c->k.w, c->v.w, G);
     uint32_t n_splits, split_tokens = 0;
-    uint32_t total_blocks = 0, unit_blocks = 1;
+    uint32_t total_blocks = 0;
+    RunGeom runs = { 1, 0, 8 };
     if (use_mfma) {
         // every wavefront takes an equal run of 64-token blocks from the list of all regions' blocks; as many
         // wavefronts as the device holds at once
@@ -686,13 +695,20 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         blocks *= Hkv;
         WEED_HIP_REQUIRE(blocks < (1ull << 32), "%s: too many cached tokens for one launch", fn);
         total_blocks = (uint32_t)blocks;
-        uint32_t target_units = mfma_decode_wavefronts(G, d, c->k.w, c->v.w);
+        runs.waves = mfma_decode_workgroup_waves(G, d, c->k.w, c->v.w);
+        uint32_t target_units = runs.waves * 256u; // one workgroup per compute unit
         if (const char *env = std::getenv("WEED_HIP_DECODE_WAVES")) {
             target_units = (uint32_t)std::max(1, std::atoi(env)); // tuning knob
         }
-        unit_blocks = std::max(1u, (total_blocks + target_units - 1) / target_units);
+        runs.unit_blocks = std::max(1u, (total_blocks + target_units - 1) / target_units);
+        uint32_t skew_pct = kRunSkewPercent;
+        if (const char *env = std::getenv("WEED_HIP_DECODE_SKEW")) {
+            skew_pct = (uint32_t)std::min(90, std::max(0, std::atoi(env))); // tuning knob
+        }
+        runs.skew = std::min(runs.unit_blocks - 1, (runs.unit_blocks * skew_pct + 50) / 100);
         const uint32_t nblk = (max_len + 63) / 64;
-        n_splits = (nblk + unit_blocks - 1) / unit_blocks + 1; // partial slots per (sequence, head)
+        const uint32_t shortest = runs.unit_blocks - runs.skew;
+        n_splits = (nblk + shortest - 1) / shortest + 1; // partial slots per (sequence, head)
     } else {
         // split the context so that the launch has a few workgroups per compute unit
         const uint32_t target_wgs = 2048;
@@ -764,7 +780,7 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         mp.blk_off = blk_off;
         mp.n_seq = S;
         mp.total_blocks = total_blocks;
-        mp.unit_blocks = unit_blocks;
+        mp.runs = runs;
         mp.max_slots = n_splits;
         ProfileScope prof("kv_decode_attn");
         if (total_blocks) {
@@ -791,7 +807,7 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
     }
     {
         ProfileScope prof("kv_decode_combine");
-        const SlotGeom sg = { use_mfma ? blk_off : nullptr, Hkv, G, unit_blocks,
+        const SlotGeom sg = { use_mfma ? blk_off : nullptr, Hkv, G, runs,
                               gqa_mapping == WEED_HIP_GQA_BLOCKED ? 1 : 0 };
         if (many_rows && n_splits <= 64) {
             combine_rows_kernel<<<(n_rows + kRowsPerWg - 1) / kRowsPerWg, 256, 0, stream()>>>(

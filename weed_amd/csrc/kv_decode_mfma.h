@@ -5,6 +5,48 @@
 
 namespace weedhip {
 
+// How the launch's list of 64-token blocks is cut into one run per wavefront.  Workgroup j owns blocks
+// [j * waves * unit_blocks, (j + 1) * waves * unit_blocks); inside it the runs follow each other in wavefront order.
+// The hardware serves the wavefronts of a SIMD by age (the first four wavefronts of a workgroup are the oldest of
+// their SIMDs, the next four the second oldest, ...), so the runs of the oldest class are `skew` blocks longer than
+// the mean and those of the youngest `skew` shorter: all classes then finish at about the same time.
+struct RunGeom {
+    uint32_t unit_blocks; // mean run length
+    uint32_t skew;        // < unit_blocks
+    uint32_t waves;       // wavefronts per workgroup: 8 or 12
+};
+__host__ __device__ inline uint32_t run_len(const RunGeom &rg, uint32_t age_class)
+{
+    const int classes = (int)rg.waves / 4; // 2 or 3
+    return (uint32_t)((int)rg.unit_blocks + (int)rg.skew * (classes - 1 - 2 * (int)age_class) / (classes - 1));
+}
+// First block of the run of wavefront `unit` (= workgroup * waves + wavefront in workgroup).
+__host__ __device__ inline uint32_t run_begin(const RunGeom &rg, uint32_t unit)
+{
+    const uint32_t wg = unit / rg.waves, w = unit % rg.waves;
+    uint32_t b = wg * rg.waves * rg.unit_blocks;
+    for (uint32_t t = 0; t < (w >> 2); ++t) {
+        b += 4 * run_len(rg, t);
+    }
+    return b + (w & 3) * run_len(rg, w >> 2);
+}
+// The wavefront whose run holds block b.
+__host__ __device__ inline uint32_t run_of_block(const RunGeom &rg, uint32_t b)
+{
+    const uint32_t wg_blocks = rg.waves * rg.unit_blocks;
+    const uint32_t wg = b / wg_blocks;
+    uint32_t r = b - wg * wg_blocks;
+    uint32_t t = 0;
+    for (; t + 1 < rg.waves / 4; ++t) {
+        const uint32_t span = 4 * run_len(rg, t);
+        if (r < span) {
+            break;
+        }
+        r -= span;
+    }
+    return wg * rg.waves + 4 * t + r / run_len(rg, t);
+}
+
 struct MfmaParams {
     SideParams k, v;
     const int32_t *lens;
@@ -17,11 +59,11 @@ struct MfmaParams {
     const float *q_sum;     // [n_seq][Hq] sum of the scaled query (for the uniform coder's offset term)
     float *partials;        // [n_seq][Hq][max_slots][d + 2]: m (log2 units), l, o[d]
     // Work partition: the 64-token blocks of all (sequence, kv head) regions form one list, region after region
-    // (sequence-major); wavefront u of the launch takes blocks [u * unit_blocks, (u + 1) * unit_blocks).
+    // (sequence-major), cut into one run per wavefront (`runs`).
     const uint32_t *blk_off; // [n_seq + 1] prefix sums of the sequences' block counts (cached lengths)
     uint32_t n_seq;
     uint32_t total_blocks;   // blk_off[n_seq] * Hkv
-    uint32_t unit_blocks;
+    RunGeom runs;
     uint32_t max_slots;      // partial slots per (sequence, head): most wavefronts that can touch one region
 };
 
@@ -39,8 +81,8 @@ constexpr uint32_t mfma_decode_waves_per_wg(uint32_t gp, uint32_t d, uint32_t wk
 {
     return (gp > 8 || mfma_decode_double_buffered(gp, d, wk, wv)) ? 8u : 12u;
 }
-// Wavefronts that fill the device: the launch is cut into that many block runs.
-uint32_t mfma_decode_wavefronts(uint32_t G, uint32_t d, uint32_t wk, uint32_t wv);
+// Wavefronts per workgroup of the kernel instance that serves this shape (one workgroup fills a compute unit).
+uint32_t mfma_decode_workgroup_waves(uint32_t G, uint32_t d, uint32_t wk, uint32_t wv);
 int launch_mfma_decode(const MfmaParams &p, uint32_t d, hipStream_t s);
 
 } // namespace weedhip

@@ -13,10 +13,10 @@ bool mfma_decode_supported(uint32_t d, uint32_t wk, uint32_t wv, uint32_t G)
     return (d == 64 || d == 128) && wk >= 2 && wk <= 4 && wv >= 2 && wv <= 4 && G >= 1 && G <= 16;
 }
 
-uint32_t mfma_decode_wavefronts(uint32_t G, uint32_t d, uint32_t wk, uint32_t wv)
+uint32_t mfma_decode_workgroup_waves(uint32_t G, uint32_t d, uint32_t wk, uint32_t wv)
 {
     const uint32_t gp = G <= 4 ? 4u : (G <= 8 ? 8u : 16u);
-    return mfma_decode_waves_per_wg(gp, d, wk, wv) * 256u; // one workgroup per compute unit
+    return mfma_decode_waves_per_wg(gp, d, wk, wv);
 }
 
 int launch_mfma_decode(const MfmaParams &p, uint32_t d, hipStream_t s)

@@ -208,12 +208,12 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     const uint32_t vbase = (lane & 31) * 4; // lane byte of a V lookup
     const uint32_t kbase = vbase + 128;     // lane byte of a K lookup
 
-    // ---- this wavefront's share of the launch: a contiguous run of `unit_blocks` 64-token blocks of the global block
+    // ---- this wavefront's share of the launch: a contiguous run (see RunGeom) of 64-token blocks of the global block
     //      list (all blocks of (sequence 0, kv head 0), then (0, 1), ...).  A run is cut into segments at region
     //      boundaries; every segment leaves one partial in the slot `unit - first unit of the region`. ----
     const uint32_t unit = __builtin_amdgcn_readfirstlane(blockIdx.x * kWaves + wave);
-    uint32_t g0 = unit * p.unit_blocks;
-    const uint32_t g1 = min(g0 + p.unit_blocks, p.total_blocks);
+    uint32_t g0 = __builtin_amdgcn_readfirstlane(run_begin(p.runs, unit));
+    const uint32_t g1 = min(g0 + run_len(p.runs, wave >> 2), p.total_blocks);
     if (g0 >= g1) {
         build_tables();
         return;
@@ -244,7 +244,7 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     const uint32_t kvh = rel / nb_cap;
     const uint32_t b0 = rel - kvh * nb_cap;
     const uint32_t seg = min(nb_cap - b0, g1 - g0);
-    const uint32_t slot = unit - (seq_first * p.Hkv + kvh * nb_cap) / p.unit_blocks;
+    const uint32_t slot = unit - run_of_block(p.runs, seq_first * p.Hkv + kvh * nb_cap);
     const uint32_t L = (uint32_t)p.lens[seq]; // may be shorter than the cached length (prefix attention)
     const uint32_t b1 = min(b0 + seg, (L + 63) >> 6);
     const uint64_t region = (uint64_t)seq * p.Hkv + kvh;
@@ -646,8 +646,12 @@ template <int D, int WK, int WV, int GP, bool LLOYD> int launch_gp(const MfmaPar
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         configured = true;
     }
-    const uint32_t units = (p.total_blocks + p.unit_blocks - 1) / p.unit_blocks;
-    decode_mfma_kernel<D, WK, WV, GP, LLOYD><<<(units + waves - 1) / waves, 64 * waves, smem, s>>>(p);
+    if (p.runs.waves != waves) {
+        return fail(WEED_HIP_EDEVICE, "decode_mfma: runs were cut for %u wavefronts per workgroup, the kernel has %u",
+                    p.runs.waves, waves);
+    }
+    const uint32_t wg_blocks = waves * p.runs.unit_blocks;
+    decode_mfma_kernel<D, WK, WV, GP, LLOYD><<<(p.total_blocks + wg_blocks - 1) / wg_blocks, 64 * waves, smem, s>>>(p);
     WEED_HIP_LAUNCH_CHECK();
     return WEED_HIP_OK;
 }
