@@ -14,6 +14,7 @@
 #include <functional>
 #include <random>
 #include <string>
+#include <sstream>
 #include <vector>
 
 using namespace Weed;
@@ -681,6 +682,168 @@ TEST_CASE(test_attention_dense_path_matches_quantized_at_fine_steps, true)
     }
     REQUIRE(attn_close(pieces, want));
     REQUIRE(cached.cache_len == T);
+}
+
+
+// ---- checkpoint streams (weed_amd/host/serialize.cpp).  The reference has no test or fixture of its streams; the
+//      expected bytes below are assembled by hand from its writer code (serializer.hpp, storage.cpp:25-30,
+//      parameter.cpp:16-31, linear.cpp:109-118, rope.cpp:100-106, multihead_attention.cpp:358-375). ----
+struct Bytes {
+    std::string b;
+    Bytes &u8(uint8_t v)
+    {
+        b.push_back((char)v);
+        return *this;
+    }
+    Bytes &u32(uint32_t v)
+    {
+        for (int i = 0; i < 4; ++i) {
+            b.push_back((char)((v >> (8 * i)) & 0xff));
+        }
+        return *this;
+    }
+    Bytes &f32(float v)
+    {
+        uint32_t w;
+        std::memcpy(&w, &v, 4);
+        return u32(w);
+    }
+};
+
+TEST_CASE(test_checkpoint_linear_known_bytes, false)
+{
+    // host-side storage: serialization needs no device
+    Linear l(2U, 3U, true, false, DType::REAL, DeviceTag::CPU);
+    const std::vector<real1> w{ 1.0f, 2.0f, 3.0f, 4.0f, 5.0f, 6.0f }, b{ 0.5f, -1.0f, 2.0f };
+    for (tcapint i = 0; i < 6U; ++i) {
+        std::dynamic_pointer_cast<RealStorage>(l.weight->storage)->write(i, w[i]);
+    }
+    for (tcapint i = 0; i < 3U; ++i) {
+        std::dynamic_pointer_cast<RealStorage>(l.bias->storage)->write(i, b[i]);
+    }
+    std::ostringstream os;
+    l.save(os);
+
+    Bytes e;
+    e.u32(2U);                                  // LINEAR_T
+    e.u32(2U).u32(3U);                          // in_features, out_features
+    e.u32(0xffffffffU).u32(0U).u32(2U);         // weight: device id -1, offset 0, rank 2
+    e.u32(2U).u32(1U).u32(3U).u32(2U);          // (shape, stride) of the column-major 2 x 3 matrix
+    e.u32(1U).u32(0xffffffffU).u32(0xffffffffU).u32(6U); // storage: REAL_CPU_DENSE, 8-byte device id -1, 6 elements
+    for (float v : w) {
+        e.f32(v);
+    }
+    e.u8(1U);                                   // has bias
+    e.u32(0xffffffffU).u32(0U).u32(2U);         // bias: device id -1, offset 0, rank 2
+    e.u32(1U).u32(0U).u32(3U).u32(1U);          // (1, 3): the size-1 dimension has stride 0
+    e.u32(1U).u32(0xffffffffU).u32(0xffffffffU).u32(3U);
+    for (float v : b) {
+        e.f32(v);
+    }
+    REQUIRE(os.str() == e.b);
+
+    // reading the hand-assembled bytes gives the module back; the upper half of the 8-byte device id is ignored
+    std::string junk = e.b;
+    junk[4 * 11 + 4] = (char)0x5a; // first byte of the undefined upper half in the weight's storage record
+    for (const std::string &src : { e.b, junk }) {
+        std::istringstream is(src);
+        LinearPtr r = std::dynamic_pointer_cast<Linear>(Module::load(is));
+        REQUIRE(r && r->in_features == 2U && r->out_features == 3U && r->bias);
+        if (r && r->bias) {
+            REQUIRE(r->weight->shape == (std::vector<tcapint>{ 2U, 3U }) && r->weight->stride == (std::vector<tcapint>{ 1U, 2U }));
+            REQUIRE(r->bias->shape == (std::vector<tcapint>{ 1U, 3U }) && r->bias->stride == (std::vector<tcapint>{ 0U, 1U }));
+            REQUIRE(r->weight->to_vector() == w && r->bias->to_vector() == b);
+            REQUIRE(r->weight->storage->device == DeviceTag::CPU);
+        }
+        REQUIRE(is.peek() == std::char_traits<char>::eof()); // the record was consumed exactly
+    }
+
+    // error paths: truncated stream, foreign module tag, foreign storage tag
+    {
+        std::istringstream is(e.b.substr(0, e.b.size() - 3));
+        REQUIRE_THROWS_AS(Module::load(is), std::runtime_error);
+    }
+    {
+        std::istringstream is(Bytes().u32(7U).b); // LAYERNORM_T in the reference
+        REQUIRE_THROWS_AS(Module::load(is), std::domain_error);
+    }
+    {
+        std::string bad = e.b;
+        bad[4 * 10] = 3; // COMPLEX_CPU_DENSE
+        std::istringstream is(bad);
+        REQUIRE_THROWS_AS(Module::load(is), std::domain_error);
+    }
+}
+
+TEST_CASE(test_checkpoint_attention_header_bytes, false)
+{
+    // the fixed-size part of an attention record: tag, mask value, four sizes, cache flag, bit width
+    MultiHeadAttention m(8U, 2U, 1U, 4U, DeviceTag::CPU, nullptr, -5.0f, -1, true, 3, false);
+    std::ostringstream os;
+    m.save(os);
+    Bytes e;
+    e.u32(17U).f32(-5.0f).u32(8U).u32(2U).u32(1U).u32(4U).u8(1U).u32(3U);
+    REQUIRE(os.str().size() > e.b.size() && os.str().compare(0, e.b.size(), e.b) == 0);
+    // ... four bias-free projections follow: W_q 8x8, W_k 8x4, W_v 8x4, W_o 8x8, then "no RoPE"
+    const size_t lin = 4U * 3U + 4U * 7U + 4U * 4U + 1U; // tag + sizes, parameter header (rank 2), storage header, bias flag
+    const size_t want = e.b.size() + 4U * lin + 4U * (64U + 32U + 32U + 64U) + 1U;
+    REQUIRE(os.str().size() == want);
+    REQUIRE(os.str().back() == '\0');
+    // a RoPE record: tag 31, head_dim, max_seq_len, base
+    std::ostringstream ro;
+    RoPE(4U, 16U, 10000.0f, DeviceTag::CPU).save(ro);
+    REQUIRE(ro.str() == Bytes().u32(31U).u32(4U).u32(16U).f32(10000.0f).b);
+}
+
+TEST_CASE(test_checkpoint_attention_round_trip, true)
+{
+    // save -> load -> the same outputs, prefill and decode, with RoPE and the Lloyd-Max coder; the quantizer record
+    // carries the coder settings and the rotations, so the reloaded module also produces the same cache words
+    const tcapint B = 2U, dm = 64U, H = 4U, Hkv = 2U, hd = 32U;
+    RoPEPtr rope = std::make_shared<RoPE>(hd, 32U, 10000.0f, TEST_DTAG);
+    MultiHeadAttention a(dm, H, Hkv, hd, TEST_DTAG, rope, ZERO_R1, -1, true, 4);
+    a.kv_coder = KV_LLOYDMAX;
+    a.k_bits = 3;
+    a.v_bits = 4;
+    a.rotation_seed = 4242U;
+    a.set_max_kv_seq_len(32U);
+    const std::vector<real1> x0 = gaussian((size_t)B * 5U * dm, 11U), x1 = gaussian((size_t)B * dm, 12U);
+    TensorPtr t0 = std::make_shared<Tensor>(x0, std::vector<tcapint>{ B, 5U, dm }, false, TEST_DTAG);
+    TensorPtr t1 = std::make_shared<Tensor>(x1, std::vector<tcapint>{ B, 1U, dm }, false, TEST_DTAG);
+    const std::vector<real1> y0 = a.forward(t0)->to_vector(), y1 = a.forward(t1)->to_vector();
+
+    std::stringstream ss;
+    a.save(ss);
+    a.save_quantizer(ss);
+    MultiHeadAttentionPtr b = std::dynamic_pointer_cast<MultiHeadAttention>(Module::load(ss));
+    REQUIRE((bool)b);
+    if (!b) {
+        return;
+    }
+    b->load_quantizer(ss);
+    REQUIRE(ss.peek() == std::char_traits<char>::eof());
+    REQUIRE(b->d_model == a.d_model && b->num_heads == a.num_heads && b->num_kv_heads == a.num_kv_heads &&
+        b->head_dim == a.head_dim && b->kv_quant_bits == a.kv_quant_bits && b->use_kv_cache == a.use_kv_cache &&
+        b->mask_val == a.mask_val);
+    REQUIRE(b->rope && b->rope->head_dim == hd && b->rope->max_seq_len == 32U && b->rope->base == 10000.0f);
+    REQUIRE(b->kv_coder == KV_LLOYDMAX && b->k_bits == 3 && b->v_bits == 4 && b->rotation_seed == 4242U &&
+        b->max_seq_len == 32U);
+    REQUIRE(b->k_rotation == a.k_rotation && b->v_rotation == a.v_rotation && b->k_rotation.size() == (size_t)hd * hd);
+    REQUIRE(b->parameters().size() == a.parameters().size());
+    for (size_t i = 0; i < a.parameters().size() && i < b->parameters().size(); ++i) {
+        REQUIRE(b->parameters()[i]->to_vector() == a.parameters()[i]->to_vector());
+        REQUIRE(b->parameters()[i]->storage->device == DeviceTag::GPU);
+    }
+    // bit-identical replay: same weights, same rotations, same kernels
+    REQUIRE(b->forward(t0)->to_vector() == y0);
+    REQUIRE(b->forward(t1)->to_vector() == y1);
+    // a record that is not a quantizer record is refused, and so is loading one into a cache that holds tokens
+    std::stringstream again;
+    a.save_quantizer(again);
+    REQUIRE_THROWS_AS(b->load_quantizer(again), std::logic_error);
+    std::istringstream wrong(std::string(64, 'x'));
+    b->reset_cache();
+    REQUIRE_THROWS_AS(b->load_quantizer(wrong), std::runtime_error);
 }
 
 } // namespace

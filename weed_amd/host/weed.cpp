@@ -748,7 +748,8 @@ void triu_fill(Tensor &a, const real1 &val, const tcapint diagonal)
 // ---------------------------------------------------------------------------------------------------------
 
 Linear::Linear(tcapint in_f, tcapint out_f, bool use_bias, bool init_rand, DType dtype, DeviceTag device, int64_t device_id)
-    : in_features(in_f)
+    : Module(LINEAR_T)
+    , in_features(in_f)
     , out_features(out_f)
 {
     if (dtype != DType::REAL) {
@@ -796,7 +797,8 @@ std::vector<ParameterPtr> Linear::parameters()
 // ---------------------------------------------------------------------------------------------------------
 
 RoPE::RoPE(const tcapint &head_dim_, const tcapint &max_seq_len_, const real1_f &base_, DeviceTag dtag)
-    : head_dim(head_dim_)
+    : Module(ROPE_T)
+    , head_dim(head_dim_)
     , max_seq_len(max_seq_len_)
     , base(base_)
 {
@@ -967,7 +969,8 @@ void QuantizedKVCache::sync_packed()
 MultiHeadAttention::MultiHeadAttention(tcapint d_model_, tcapint num_heads_, tcapint num_kv_heads_, tcapint head_dim_,
     DeviceTag dtag, RoPEPtr r, real1_f mask_val_, const int64_t did, const bool _use_kv_cache, int kv_quant_bits_,
     bool use_bias)
-    : d_model((symint)d_model_)
+    : Module(MULTIHEAD_ATTENTION_T)
+    , d_model((symint)d_model_)
     , num_heads((symint)num_heads_)
     , num_kv_heads((symint)(num_kv_heads_ ? num_kv_heads_ : num_heads_))
     , head_dim((symint)(!head_dim_ ? d_model_ / num_heads_ : head_dim_))
@@ -997,6 +1000,17 @@ MultiHeadAttention::MultiHeadAttention(tcapint d_model_, tcapint num_heads_, tca
     if (mask_val == ZERO_R1) {
         mask_val = -1.701411835e38f; // -2^127 (multihead_attention.hpp:109-110 at fp32)
     }
+}
+
+MultiHeadAttention::MultiHeadAttention()
+    : Module(MULTIHEAD_ATTENTION_T)
+    , d_model(0)
+    , num_heads(0)
+    , num_kv_heads(0)
+    , head_dim(0)
+    , mask_val(ZERO_R1)
+    , use_kv_cache(true)
+{
 }
 
 MultiHeadAttention::~MultiHeadAttention()

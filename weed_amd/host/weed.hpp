@@ -8,6 +8,7 @@
 #pragma once
 
 #include <cstdint>
+#include <iosfwd>
 #include <memory>
 #include <mutex>
 #include <new>
@@ -29,6 +30,33 @@ constexpr real1 ONE_R1 = 1.0f;
 enum DeviceTag { NONE_DEVICE = 0, DEFAULT_DEVICE = 1, CPU = 2, GPU = 3 }; // include/enums/device_tag.hpp
 enum DType { NONE_DTYPE = 0, REAL = 1, COMPLEX = 2, INT = 3, DEFAULT_DTYPE = REAL }; // include/enums/dtype.hpp
 enum StorageType { NONE_STORAGE_TYPE = 0, REAL_CPU_DENSE = 1, REAL_GPU_DENSE = 2 }; // include/enums/storage_type.hpp
+// include/enums/module_type.hpp: the tags a serialized module starts with.  Only the three modules of this path can
+// be written or read here; the other values are listed so that a foreign tag is reported by name of its number.
+enum ModuleType {
+    NONE_MODULE_TYPE = 0,
+    LINEAR_T = 2,
+    MULTIHEAD_ATTENTION_T = 17,
+    ROPE_T = 31,
+};
+
+// include/common/serializer.hpp: fixed-width little-endian fields, written as the reference's default build writes
+// them (tcapint and symint 32 bits, real1 and real1_f IEEE single, bool one byte, enums 32 bits).
+struct Serializer {
+    static void write_bool(std::ostream &out, const bool &x);
+    static void read_bool(std::istream &in, bool &x);
+    static void write_tcapint(std::ostream &out, const tcapint &x);
+    static void read_tcapint(std::istream &in, tcapint &x);
+    static void write_symint(std::ostream &out, const symint &x);
+    static void read_symint(std::istream &in, symint &x);
+    // Eight bytes.  The reference passes a 32-bit value by reference and writes eight bytes from its address
+    // (serializer.hpp:51-56), so only the low four are defined: this writer sign-extends, the reader keeps the low four.
+    static void write_int64(std::ostream &out, const symint &x);
+    static void read_int64(std::istream &in, symint &x);
+    static void write_real(std::ostream &out, const real1 &x);
+    static void read_real(std::istream &in, real1 &x);
+    static void write_real1_f(std::ostream &out, const real1_f &x);
+    static void read_real1_f(std::istream &in, real1_f &x);
+};
 
 // include/devices/pool_item.hpp:32-40
 struct bad_alloc : public std::bad_alloc {
@@ -77,6 +105,11 @@ struct Storage : public std::enable_shared_from_this<Storage> {
     virtual void FillOnes() = 0;
     virtual StoragePtr cpu() = 0;
     virtual StoragePtr gpu(int64_t did = -1) = 0;
+    // src/storage/storage.cpp:25-30 plus the element loop of the real storages (cpu_real_storage.cpp:46-51,
+    // gpu_real_storage.cpp:35-50): type tag, device id (8 bytes), size, then the elements.
+    virtual void save(std::ostream &os) const;
+    // src/storage/storage.cpp:32-119 for the two real dense types; a GPU storage is uploaded on load.
+    static StoragePtr load(std::istream &is);
 };
 
 // include/storage/typed_storage.hpp:30-72 for T = real1
@@ -202,12 +235,26 @@ void triu_fill(Tensor &a, const real1 &val, const tcapint diagonal = 1); // src/
 
 struct Parameter : public Tensor { // include/tensors/parameter.hpp
     using Tensor::Tensor;
+    // src/tensors/parameter.cpp:16-56: device id, offset, rank, (shape, stride) pairs, storage.  As in the reference,
+    // save() first sets the extent of every stride-0 dimension to 1.
+    void save(std::ostream &out);
+    static std::shared_ptr<Parameter> load(std::istream &in);
 };
 typedef std::shared_ptr<Parameter> ParameterPtr;
 
 // include/modules/module.hpp, the members this path uses
 struct Module {
+    ModuleType mtype;
+    explicit Module(ModuleType t = NONE_MODULE_TYPE)
+        : mtype(t)
+    {
+    }
     virtual ~Module() {}
+    // src/modules/module.cpp:53-56: the type tag; the inheriting struct writes the rest.
+    virtual void save(std::ostream &os) const;
+    // src/modules/module.cpp:58-260 for LINEAR_T, ROPE_T and MULTIHEAD_ATTENTION_T; any other tag throws
+    // std::domain_error.
+    static std::shared_ptr<Module> load(std::istream &is);
     virtual TensorPtr forward(const TensorPtr x) = 0;
     virtual std::vector<ParameterPtr> parameters() { return {}; }
     virtual void train() {}
@@ -224,7 +271,8 @@ struct Linear : public Module {
     ParameterPtr bias; // (1, out_features) or null
 
     Linear()
-        : in_features(0U)
+        : Module(LINEAR_T)
+        , in_features(0U)
         , out_features(0U)
     {
     }
@@ -232,6 +280,7 @@ struct Linear : public Module {
         DeviceTag device = DeviceTag::DEFAULT_DEVICE, int64_t device_id = -1);
     TensorPtr forward(const TensorPtr x) override;
     std::vector<ParameterPtr> parameters() override;
+    void save(std::ostream &os) const override; // src/modules/linear.cpp:109-118
 };
 typedef std::shared_ptr<Linear> LinearPtr;
 
@@ -289,6 +338,7 @@ struct RoPE : public Module {
     TensorPtr forward(const TensorPtr x) override { return forward(x, 0U); }
     TensorPtr forward(const TensorPtr x, tcapint pos0); // x: [B, H, T, head_dim], any strides
     void apply(const Tensor &x, Tensor &out, tcapint pos0); // the same into a given (possibly strided) output
+    void save(std::ostream &os) const override; // src/modules/rope.cpp:100-106: the tables are rebuilt on load
 };
 typedef std::shared_ptr<RoPE> RoPEPtr;
 
@@ -343,6 +393,18 @@ struct MultiHeadAttention : public Module {
     MultiHeadAttention(tcapint d_model_, tcapint num_heads_, tcapint num_kv_heads_ = 0, tcapint head_dim_ = 0U,
         DeviceTag dtag = DEFAULT_DEVICE, RoPEPtr r = nullptr, real1_f mask_val_ = ZERO_R1, const int64_t did = -1,
         const bool _use_kv_cache = true, int kv_quant_bits_ = 4, bool use_bias = true);
+
+    // What Module::load builds on (multihead_attention.hpp: the reference's default constructor): no projections yet.
+    MultiHeadAttention();
+    // src/modules/multihead_attention.cpp:358-375, byte for byte the reference's stream: mask value, the four sizes,
+    // use_kv_cache, kv_quant_bits, the four projections, the RoPE flag and module.  Neither the reference nor this
+    // stream holds the cached tokens.
+    void save(std::ostream &os) const override;
+    // Extension, a separate record that a caller may write after save(): what the stream above lacks to make a
+    // reloaded module encode and decode identically -- coder, bit widths, sign bits, head mapping, rotation seed,
+    // max_seq_len, the two block scales and the two rotations (empty before the first forward()).
+    void save_quantizer(std::ostream &os) const;
+    void load_quantizer(std::istream &is);
 
     std::vector<ParameterPtr> parameters() override { return param_vector; }
     void set_max_kv_seq_len(tcapint m) override { max_seq_len = m; }
