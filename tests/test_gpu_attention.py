@@ -174,6 +174,22 @@ def test_split_context_matches_single_pass(gpu, oracle):
     cache.close()
 
 
+def test_one_long_region_keeps_within_the_slot_limit(gpu, oracle):
+    """A single sequence with one kv head and more 64-token blocks (1032) than the merge kernel has partial slots per
+    head: the launch must lengthen its runs instead of failing, and still match the checker."""
+    rng = np.random.default_rng(23)
+    d, Hkv, Hq, L = 64, 1, 2, 66000
+    K = rng.standard_normal((1, Hkv, L, d), dtype=np.float32)
+    V = rng.standard_normal((1, Hkv, L, d), dtype=np.float32)
+    q = rng.standard_normal((1, Hq, d), dtype=np.float32)
+    wl = workloads.Workload("long", 1, Hq, Hkv, d, [L], 2, 2, 0, 0, 0)
+    cache = build_cache(gpu, wl, gpu.KV_LLOYDMAX, K, V)
+    want = checker_output(oracle, gpu, cache, wl, q, True)
+    got = run_decode(gpu, cache, q, gpu.GQA_WEED, 0)
+    assert_attn_close(got, want, "one long region")
+    cache.close()
+
+
 def test_edge_lengths(gpu, oracle):
     """Empty sequences give zeros; lengths 1, 63, 64, 65 around the 64-token block; an appended token changes the
     result exactly as the checker says."""

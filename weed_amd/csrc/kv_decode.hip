@@ -415,6 +415,8 @@ __global__ void __launch_bounds__(kThreads) decode_generic_kernel(DecodeParams p
 
 // Merge the partials of all splits: out = sum_s e^(m_s - M) o_s / sum_s e^(m_s - M) l_s, then multiply by
 // v_rotation^T (multihead_attention.cpp:343-348): out_i = sum_j O_j Rv[i + d*j].
+constexpr uint32_t kMaxSlots = 1024; // partials per (sequence, head) that combine_kernel can weigh in one pass
+
 // Run-length skew between the wavefront age classes of a workgroup, in percent of the mean run (see RunGeom).
 constexpr uint32_t kRunSkewPercent = 8;
 
@@ -705,10 +707,17 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         if (const char *env = std::getenv("WEED_HIP_DECODE_SKEW")) {
             skew_pct = (uint32_t)std::min(90, std::max(0, std::atoi(env))); // tuning knob
         }
-        runs.skew = std::min(runs.unit_blocks - 1, (runs.unit_blocks * skew_pct + 50) / 100);
         const uint32_t nblk = (max_len + 63) / 64;
-        const uint32_t shortest = runs.unit_blocks - runs.skew;
-        n_splits = (nblk + shortest - 1) / shortest + 1; // partial slots per (sequence, head)
+        for (;;) {
+            runs.skew = std::min(runs.unit_blocks - 1, (runs.unit_blocks * skew_pct + 50) / 100);
+            const uint32_t shortest = runs.unit_blocks - runs.skew;
+            n_splits = (nblk + shortest - 1) / shortest + 1; // partial slots per (sequence, head)
+            if (n_splits <= kMaxSlots) {
+                break;
+            }
+            // one very long region and few of them: longer runs (fewer wavefronts) keep the merge within its limit
+            runs.unit_blocks += std::max(1u, runs.unit_blocks / 8);
+        }
     } else {
         // split the context so that the launch has a few workgroups per compute unit
         const uint32_t target_wgs = 2048;
@@ -718,7 +727,7 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         split_tokens = std::max((uint32_t)kChunk, (split_tokens + kChunk - 1) / kChunk * kChunk);
         n_splits = std::max(1u, (max_len + split_tokens - 1) / split_tokens);
     }
-    WEED_HIP_REQUIRE(n_splits <= 1024, "%s: internal split count %u too large", fn, n_splits);
+    WEED_HIP_REQUIRE(n_splits <= kMaxSlots, "%s: internal split count %u too large", fn, n_splits);
 
     // workspace: rotated q (fp32), its fp16 hi / lo halves, per-head scale and sum, split partials
     const size_t n_q = (size_t)S * Hq * d;
