@@ -152,6 +152,24 @@ def extras(capi, torch, workloads, steps, warmup):
                                           "kernel_gbs": nbytes / kernel_s / 1e9,
                                           "frac_of_hbm_peak": nbytes / kernel_s / 1e9 / HBM_PEAK_GBS}
     cache4.close()
+    # configuration 3 again with 256 sequence caches per launch (2 GB of packed rows): what the per-launch fixed cost
+    # (launch, table build, first-block latency, uneven finish) amortises to with four times the bytes
+    wl3 = workloads.config(3, n_seq=256)
+    cache3, q3, _, _ = build_cache(capi, torch, wl3, seed=77)
+    o3 = torch.zeros_like(q3)
+    flags = capi.ATTN_ROTATE_Q | capi.ATTN_UNROTATE_OUT
+    capi.profile_reset()
+    capi.profile_enable(True)
+    secs = time_calls(torch, lambda: cache3.decode_attn(q3, o3, capi.GQA_BLOCKED, flags), steps, warmup)
+    k_ms, k_n = capi.profile_read("kv_decode_attn")
+    capi.profile_enable(False)
+    nbytes = wl3.bytes_per_step(lloydmax=True)
+    kernel_s = 1e-3 * k_ms / max(1, k_n)
+    out["cfg3_256_sequences"] = {"tokens_per_s": wl3.n_seq / secs, "ms_per_step": 1e3 * secs,
+                                 "packed_cache_bytes": nbytes, "kernel_ms": 1e3 * kernel_s,
+                                 "kernel_gbs": nbytes / kernel_s / 1e9,
+                                 "frac_of_hbm_peak": nbytes / kernel_s / 1e9 / HBM_PEAK_GBS}
+    cache3.close()
     return out
 
 
