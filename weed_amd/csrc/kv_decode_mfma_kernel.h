@@ -185,22 +185,38 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     // ---- the pair tables.  The 2^w fp16 levels are staged in LDS first so that building the pairs needs no global
     //      reads.  Every wavefront of the workgroup calls this exactly once (it contains barriers): wavefronts with
     //      work after they have requested their first block and query, so that those loads travel meanwhile. ----
+    // the levels are requested first thing, so that they have arrived when the tables are built
+    float level_of_lane = 0.0f;
+    if (tid < 64) {
+        level_of_lane = (tid < 32) ? p.k.table[tid & 31] : p.v.table[tid & 31];
+    }
     auto build_tables = [&]() {
         uint16_t *levels_h = reinterpret_cast<uint16_t *>(lds + ROWS * (kTableRowBytes / 4)); // [2][32]
         if (tid < 64) {
-            const float lv = (tid < 32) ? p.k.table[tid & 31] : p.v.table[tid & 31];
-            levels_h[tid] = __builtin_bit_cast(uint16_t, (_Float16)lv);
+            levels_h[tid] = __builtin_bit_cast(uint16_t, (_Float16)level_of_lane);
         }
         __syncthreads();
-        for (uint32_t i = tid; i < ROWS * 64; i += 64 * kWaves) {
-            const uint32_t e = i >> 6, half_row = (i >> 5) & 1; // 0: V table, 1: K table
-            uint32_t val = 0;
-            if (half_row == 0 && e < (1u << (2 * WV))) {
-                val = (uint32_t)levels_h[32 + (e & ((1u << WV) - 1u))] | ((uint32_t)levels_h[32 + (e >> WV)] << 16);
-            } else if (half_row == 1 && e < (1u << (2 * WK))) {
-                val = (uint32_t)levels_h[e & ((1u << WK) - 1u)] | ((uint32_t)levels_h[e >> WK] << 16);
+        // eight table words per thread and pass: the reads of a pass are independent, so their latencies overlap
+        constexpr uint32_t kWords = ROWS * 64, kStep = 64 * kWaves, kBatch = 8;
+        for (uint32_t i0 = tid; i0 < kWords; i0 += kBatch * kStep) {
+            uint32_t val[kBatch];
+#pragma unroll
+            for (uint32_t u = 0; u < kBatch; ++u) {
+                const uint32_t i = min(i0 + u * kStep, kWords - 1);
+                const uint32_t e = i >> 6, half_row = (i >> 5) & 1; // 0: V table, 1: K table
+                const uint32_t w = half_row ? WK : WV;
+                const uint32_t base = half_row ? 0u : 32u;
+                const uint32_t lo = levels_h[base + (e & ((1u << w) - 1u))];
+                const uint32_t hi = levels_h[base + ((e >> w) & ((1u << w) - 1u))];
+                val[u] = (e < (1u << (2 * w))) ? (lo | (hi << 16)) : 0u;
             }
-            lds[i] = val;
+#pragma unroll
+            for (uint32_t u = 0; u < kBatch; ++u) {
+                const uint32_t i = i0 + u * kStep;
+                if (i < kWords) {
+                    lds[i] = val[u];
+                }
+            }
         }
         __syncthreads();
     };
@@ -213,7 +229,7 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     //      boundaries; every segment leaves one partial in the slot `unit - first unit of the region`. ----
     const uint32_t unit = __builtin_amdgcn_readfirstlane(blockIdx.x * kWaves + wave);
     uint32_t g0 = __builtin_amdgcn_readfirstlane(run_begin(p.runs, unit));
-    const uint32_t g1 = min(g0 + run_len(p.runs, wave >> 2), p.total_blocks);
+    const uint32_t g1 = min(g0 + run_len(p.runs, (unit % kWaves) >> 2), p.total_blocks);
     if (g0 >= g1) {
         build_tables();
         return;
@@ -249,61 +265,9 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     const uint32_t b1 = min(b0 + seg, (L + 63) >> 6);
     const uint64_t region = (uint64_t)seq * p.Hkv + kvh;
     g0 += seg;
-
-    // ---- query operand.  The score instruction has 16 columns.  With GP <= 8 the fp16 high halves of the GP heads sit
-    //      in columns [0, GP) and the low halves in [GP, 2GP), so ONE instruction per item yields both partial scores
-    //      (they are added with a lane shift afterwards); with GP = 16 the halves take two instructions. ----
-    constexpr bool PACKED = GP <= 8;
-    constexpr int NQ = PACKED ? 1 : 2;
-    half8 qop[NQ][KS];
-    {
-        const uint32_t col_head = PACKED ? c % GP : c;
-        const uint32_t col_part = PACKED ? c / GP : 0; // 0: high half, 1: low half, above: unused column
-        const bool col_ok = col_head < p.G && col_part < 2;
-        const uint32_t qh = col_ok ? (p.blocked ? kvh * p.G + col_head : col_head * p.Hkv + kvh) : 0;
-        const uint64_t qbase = ((uint64_t)seq * p.Hq + qh) * D + g * (D / 4);
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            uint4v hi = { 0, 0, 0, 0 }, lo = { 0, 0, 0, 0 };
-            if (col_ok) {
-                hi = *reinterpret_cast<const uint4v *>(p.q_hi + qbase + 8 * ks);
-                lo = *reinterpret_cast<const uint4v *>(p.q_lo + qbase + 8 * ks);
-            }
-            if constexpr (PACKED) {
-                qop[0][ks] = __builtin_bit_cast(half8, col_part ? lo : hi);
-            } else {
-                qop[0][ks] = __builtin_bit_cast(half8, hi);
-                qop[NQ - 1][ks] = __builtin_bit_cast(half8, lo);
-            }
-        }
-    }
     // after merging, this lane works on head c % GP of tile (set * TPS + c / GP)
     const uint32_t hc = c % GP;
     const uint32_t tile_in_set = c / GP;
-    const bool head_ok = hc < p.G;
-    const uint32_t qh_c = head_ok ? (p.blocked ? kvh * p.G + hc : hc * p.Hkv + kvh) : 0;
-    const float qscale = head_ok ? p.q_scale[(uint64_t)seq * p.Hq + qh_c] : 0.0f;
-    const float betaq = head_ok ? p.k.beta * p.q_sum[(uint64_t)seq * p.Hq + qh_c] : 0.0f;
-
-    // ---- The running maximum is only raised when a block exceeds it by more than 2^kSlack, so most blocks skip the
-    //      rescaling of the output accumulators; probabilities may therefore reach 2^kSlack.  `ep` is the exponent
-    //      that keeps probability * V-row-scale * 2^ep below 2^15, inside fp16's range. ----
-    constexpr float kSlack = 8.0f;
-    int ep = 7;
-    if (lloyd) {
-        const uint32_t bits = p.v.alpha_max[region];
-        ep = bits ? 133 - (int)((bits >> 23) & 0xff) : 0;
-        ep = ep > 100 ? 100 : (ep < -100 ? -100 : ep);
-    }
-    const float unscale = __uint_as_float((uint32_t)(127 - ep) << 23); // 2^-ep
-
-    float m_run = -INFINITY; // running maximum of this lane's head (same value in every lane that shares the head)
-    float l_run = 0.0f;      // this lane's share of the running denominator, scaled by 2^ep
-    float4v O[JB];           // lane (c, g), register r: head slot 4g + r, coordinate 16*jb + c
-#pragma unroll
-    for (int jb = 0; jb < JB; ++jb) {
-        O[jb] = float4v{ 0.0f, 0.0f, 0.0f, 0.0f };
-    }
 
     // region bases are the same in every lane; the lane's share is a 32-bit offset
     const uint8_t *kreg = p.k.fields + region * p.k.region_bytes;
@@ -313,9 +277,6 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     const float *va = lloyd ? p.v.alpha + region * p.padded : nullptr;
     const uint32_t alane = 16 * tile_in_set + 4 * g;
 
-    // Single register buffers, refilled as soon as their last reader is done: K (and its row scales) right after the
-    // Q.K^T phase of a block, V right after its P.V phase -- so each load has about half a block of work to hide behind
-    // and the other wavefronts of the SIMD cover the rest.
     // Register buffers for the packed block: one (refilled as soon as its last reader is done: K right after the
     // Q.K^T phase, V right after the P.V phase), or two when the shape is double-buffered (the whole next block is
     // requested before the current one is touched).
@@ -347,6 +308,69 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
             }
         }
     };
+
+    // The first block of the segment is requested before anything else of the segment is read (the sequence's
+    // attended length, the query): it exists whatever that length is, and its latency is the longest of the prologue.
+    constexpr std::integral_constant<int, 0> p0{};
+    load_k(p0, b0);
+    load_v(p0, b0);
+
+    // ---- query operand.  The score instruction has 16 columns.  With GP <= 8 the fp16 high halves of the GP heads sit
+    //      in columns [0, GP) and the low halves in [GP, 2GP), so ONE instruction per item yields both partial scores
+    //      (they are added with a lane shift afterwards); with GP = 16 the halves take two instructions. ----
+    constexpr bool PACKED = GP <= 8;
+    constexpr int NQ = PACKED ? 1 : 2;
+    half8 qop[NQ][KS];
+    {
+        const uint32_t col_head = PACKED ? c % GP : c;
+        const uint32_t col_part = PACKED ? c / GP : 0; // 0: high half, 1: low half, above: unused column
+        const bool col_ok = col_head < p.G && col_part < 2;
+        const uint32_t qh = col_ok ? (p.blocked ? kvh * p.G + col_head : col_head * p.Hkv + kvh) : 0;
+        const uint64_t qbase = ((uint64_t)seq * p.Hq + qh) * D + g * (D / 4);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            uint4v hi = { 0, 0, 0, 0 }, lo = { 0, 0, 0, 0 };
+            if (col_ok) {
+                hi = *reinterpret_cast<const uint4v *>(p.q_hi + qbase + 8 * ks);
+                lo = *reinterpret_cast<const uint4v *>(p.q_lo + qbase + 8 * ks);
+            }
+            if constexpr (PACKED) {
+                qop[0][ks] = __builtin_bit_cast(half8, col_part ? lo : hi);
+            } else {
+                qop[0][ks] = __builtin_bit_cast(half8, hi);
+                qop[NQ - 1][ks] = __builtin_bit_cast(half8, lo);
+            }
+        }
+    }
+    const bool head_ok = hc < p.G;
+    const uint32_t qh_c = head_ok ? (p.blocked ? kvh * p.G + hc : hc * p.Hkv + kvh) : 0;
+    const float qscale = head_ok ? p.q_scale[(uint64_t)seq * p.Hq + qh_c] : 0.0f;
+    const float betaq = head_ok ? p.k.beta * p.q_sum[(uint64_t)seq * p.Hq + qh_c] : 0.0f;
+
+    // ---- The running maximum is only raised when a block exceeds it by more than 2^kSlack, so most blocks skip the
+    //      rescaling of the output accumulators; probabilities may therefore reach 2^kSlack.  `ep` is the exponent
+    //      that keeps probability * V-row-scale * 2^ep below 2^15, inside fp16's range. ----
+    constexpr float kSlack = 8.0f;
+    int ep = 7;
+    if (lloyd) {
+        const uint32_t bits = p.v.alpha_max[region];
+        ep = bits ? 133 - (int)((bits >> 23) & 0xff) : 0;
+        ep = ep > 100 ? 100 : (ep < -100 ? -100 : ep);
+    }
+    const float unscale = __uint_as_float((uint32_t)(127 - ep) << 23); // 2^-ep
+
+    if (!tables_ready) {
+        build_tables(); // while the first block and the query are on their way, and before the accumulators exist
+        tables_ready = true;
+    }
+
+    float m_run = -INFINITY; // running maximum of this lane's head (same value in every lane that shares the head)
+    float l_run = 0.0f;      // this lane's share of the running denominator, scaled by 2^ep
+    float4v O[JB];           // lane (c, g), register r: head slot 4g + r, coordinate 16*jb + c
+#pragma unroll
+    for (int jb = 0; jb < JB; ++jb) {
+        O[jb] = float4v{ 0.0f, 0.0f, 0.0f, 0.0f };
+    }
 
     auto process_block = [&](auto pc, uint32_t blk, uint32_t next_blk) {
         constexpr int P = decltype(pc)::value;
@@ -563,15 +587,6 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     //      segment) so that the loop body has no branch around loads and outstanding loads can be counted exactly. ----
     {
         uint32_t blk = b0;
-        constexpr std::integral_constant<int, 0> p0{};
-        if (blk < b1) {
-            load_k(p0, blk);
-            load_v(p0, blk);
-        }
-        if (!tables_ready) {
-            build_tables(); // while the first block and the query are on their way
-            tables_ready = true;
-        }
         if (blk < b1) {
             const uint32_t last = b1 - 1;
             if constexpr (NB == 2) {
