@@ -418,7 +418,7 @@ __global__ void __launch_bounds__(kThreads) decode_generic_kernel(DecodeParams p
 constexpr uint32_t kMaxSlots = 1024; // partials per (sequence, head) that combine_kernel can weigh in one pass
 
 // Run-length skew between the wavefront age classes of a workgroup, in percent of the mean run (see RunGeom).
-constexpr uint32_t kRunSkewPercent = 8;
+constexpr uint32_t kRunSkewPercent = 16;
 
 struct SlotGeom {
     const uint32_t *blk_off; // null: every (sequence, head) has `max_slots` valid partials

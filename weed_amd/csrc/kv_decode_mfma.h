@@ -6,45 +6,58 @@
 namespace weedhip {
 
 // How the launch's list of 64-token blocks is cut into one run per wavefront.  Workgroup j owns blocks
-// [j * waves * unit_blocks, (j + 1) * waves * unit_blocks); inside it the runs follow each other in wavefront order.
-// The hardware serves the wavefronts of a SIMD by age (the first four wavefronts of a workgroup are the oldest of
-// their SIMDs, the next four the second oldest, ...), so the runs of the oldest class are `skew` blocks longer than
-// the mean and those of the youngest `skew` shorter: all classes then finish at about the same time.
+// [j * waves * unit_blocks, (j + 1) * waves * unit_blocks); inside it the runs follow each other by POSITION
+// 0 .. waves-1.  The hardware serves the wavefronts of a SIMD by age (the first four wavefronts of a workgroup are the
+// oldest of their SIMDs, the next four the second oldest, ...), so the age classes get runs of different length: the
+// oldest `skew` blocks more than the mean, the youngest `skew` fewer, and all classes finish at about the same time.
+// Positions cycle through the classes (position p belongs to class p % classes, and is worked on by wavefront
+// (p % classes) * 4 + p / classes), so every group of `classes` consecutive runs spans classes * unit_blocks blocks:
+// regions whose boundaries fall on multiples of that (equal sequences, the common case) are never straddled by a run.
 struct RunGeom {
     uint32_t unit_blocks; // mean run length
     uint32_t skew;        // < unit_blocks
     uint32_t waves;       // wavefronts per workgroup: 8 or 12
 };
+__host__ __device__ inline uint32_t run_classes(const RunGeom &rg) { return rg.waves / 4; } // 2 or 3
 __host__ __device__ inline uint32_t run_len(const RunGeom &rg, uint32_t age_class)
 {
-    const int classes = (int)rg.waves / 4; // 2 or 3
+    const int classes = (int)run_classes(rg);
     return (uint32_t)((int)rg.unit_blocks + (int)rg.skew * (classes - 1 - 2 * (int)age_class) / (classes - 1));
 }
-// First block of the run of wavefront `unit` (= workgroup * waves + wavefront in workgroup).
-__host__ __device__ inline uint32_t run_begin(const RunGeom &rg, uint32_t unit)
+// Position in the workgroup of its wavefront w, and back.
+__host__ __device__ inline uint32_t run_position_of_wave(const RunGeom &rg, uint32_t w)
 {
-    const uint32_t wg = unit / rg.waves, w = unit % rg.waves;
-    uint32_t b = wg * rg.waves * rg.unit_blocks;
-    for (uint32_t t = 0; t < (w >> 2); ++t) {
-        b += 4 * run_len(rg, t);
-    }
-    return b + (w & 3) * run_len(rg, w >> 2);
+    return (w & 3) * run_classes(rg) + (w >> 2);
 }
-// The wavefront whose run holds block b.
+// First block of the run at position index P (= workgroup * waves + position in workgroup).
+__host__ __device__ inline uint32_t run_begin(const RunGeom &rg, uint32_t P)
+{
+    const uint32_t classes = run_classes(rg);
+    const uint32_t wg = P / rg.waves, pos = P % rg.waves;
+    uint32_t b = wg * rg.waves * rg.unit_blocks + (pos / classes) * classes * rg.unit_blocks;
+    for (uint32_t t = 0; t < pos % classes; ++t) {
+        b += run_len(rg, t);
+    }
+    return b;
+}
+// Position index of the run that holds block b.
 __host__ __device__ inline uint32_t run_of_block(const RunGeom &rg, uint32_t b)
 {
-    const uint32_t wg_blocks = rg.waves * rg.unit_blocks;
+    const uint32_t classes = run_classes(rg);
+    const uint32_t wg_blocks = rg.waves * rg.unit_blocks, cycle = classes * rg.unit_blocks;
     const uint32_t wg = b / wg_blocks;
     uint32_t r = b - wg * wg_blocks;
+    const uint32_t group = r / cycle;
+    r -= group * cycle;
     uint32_t t = 0;
-    for (; t + 1 < rg.waves / 4; ++t) {
-        const uint32_t span = 4 * run_len(rg, t);
-        if (r < span) {
+    for (; t + 1 < classes; ++t) {
+        const uint32_t len = run_len(rg, t);
+        if (r < len) {
             break;
         }
-        r -= span;
+        r -= len;
     }
-    return wg * rg.waves + 4 * t + r / run_len(rg, t);
+    return wg * rg.waves + group * classes + t;
 }
 
 struct MfmaParams {

@@ -227,9 +227,11 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     // ---- this wavefront's share of the launch: a contiguous run (see RunGeom) of 64-token blocks of the global block
     //      list (all blocks of (sequence 0, kv head 0), then (0, 1), ...).  A run is cut into segments at region
     //      boundaries; every segment leaves one partial in the slot `unit - first unit of the region`. ----
-    const uint32_t unit = __builtin_amdgcn_readfirstlane(blockIdx.x * kWaves + wave);
+    // `unit`: position index of this wavefront's run (runs are numbered along the block list)
+    const uint32_t unit =
+        __builtin_amdgcn_readfirstlane(blockIdx.x * kWaves + run_position_of_wave(p.runs, wave));
     uint32_t g0 = __builtin_amdgcn_readfirstlane(run_begin(p.runs, unit));
-    const uint32_t g1 = min(g0 + run_len(p.runs, (unit % kWaves) >> 2), p.total_blocks);
+    const uint32_t g1 = min(g0 + run_len(p.runs, (unit % kWaves) % run_classes(p.runs)), p.total_blocks);
     if (g0 >= g1) {
         build_tables();
         return;
