@@ -190,6 +190,29 @@ def test_one_long_region_keeps_within_the_slot_limit(gpu, oracle):
     cache.close()
 
 
+def test_run_geometry_knobs_do_not_change_the_answer(gpu, oracle, monkeypatch):
+    """The launch cuts the block list into per-wavefront runs whose lengths are skewed by wavefront age; whatever
+    the skew and the number of runs, every block must be attended exactly once: ragged batch (runs straddle regions,
+    empty sequence in the middle) against the checker under several settings of the two tuning variables."""
+    rng = np.random.default_rng(29)
+    d, Hkv, Hq = 128, 2, 8
+    lens = [700, 0, 64, 3000, 129, 1]
+    S = len(lens)
+    wl = workloads.Workload("knobs", S, Hq, Hkv, d, lens, 3, 4, 0, 0, 0)
+    K = rng.standard_normal((S, Hkv, max(lens), d), dtype=np.float32)
+    V = rng.standard_normal((S, Hkv, max(lens), d), dtype=np.float32)
+    q = rng.standard_normal((S, Hq, d), dtype=np.float32)
+    cache = build_cache(gpu, wl, gpu.KV_LLOYDMAX, K, V)
+    want = checker_output(oracle, gpu, cache, wl, q, False)
+    for waves, skew in (("", ""), ("16", "0"), ("16", "45"), ("7", "90"), ("40", "30"), ("100000", "16")):
+        if waves:
+            monkeypatch.setenv("WEED_HIP_DECODE_WAVES", waves)
+            monkeypatch.setenv("WEED_HIP_DECODE_SKEW", skew)
+        got = run_decode(gpu, cache, q, gpu.GQA_BLOCKED, 0)
+        assert_attn_close(got, want, "waves=%s skew=%s" % (waves or "default", skew or "default"))
+    cache.close()
+
+
 def test_edge_lengths(gpu, oracle):
     """Empty sequences give zeros; lengths 1, 63, 64, 65 around the 64-token block; an appended token changes the
     result exactly as the checker says."""
