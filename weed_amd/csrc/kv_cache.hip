@@ -149,20 +149,30 @@ __global__ void __launch_bounds__(kEncThreads)
     const uint32_t tid = threadIdx.x;
     const uint32_t row0 = blockIdx.x * kEncRows;
 
-    // gather the rows (logical row = (s*Hkv + h)*T + t)
-    for (uint32_t e = tid; e < kEncRows * d; e += kEncThreads) {
-        const uint32_t r = e / d, j = e % d;
-        const uint32_t row = row0 + r;
-        float val = 0.0f;
+    // gather the rows (logical row = (s*Hkv + h)*T + t): the first 32 threads work out where their row starts, then
+    // thread (tid / 32, tid % 32) walks rows tid / 32, +8, ... and columns tid % 32, +32, ... (no divisions per element)
+    unsigned long long *row_base = reinterpret_cast<unsigned long long *>(inv_s + kEncRows); // [kEncRows], 8-byte aligned
+    if (tid < kEncRows) {
+        const uint32_t row = row0 + tid;
+        unsigned long long base = ~0ull;
         if (row < rows) {
             const uint32_t t = row % T;
             const uint32_t h = (row / T) % Hkv;
             const uint32_t s = row / (T * Hkv);
-            const uint64_t idx = (uint64_t)g.off + (uint64_t)s * g.s[0] + (uint64_t)h * g.s[1] + (uint64_t)t * g.s[2] +
-                                 (uint64_t)j * g.s[3];
-            val = x[idx];
+            base = (uint64_t)g.off + (uint64_t)s * g.s[0] + (uint64_t)h * g.s[1] + (uint64_t)t * g.s[2];
         }
-        (rotate ? xs : ys)[r * pitch + j] = val;
+        row_base[tid] = base;
+    }
+    __syncthreads();
+    {
+        float *dst = rotate ? xs : ys;
+        const uint32_t jl = tid & 31;
+        for (uint32_t r = tid >> 5; r < kEncRows; r += kEncThreads / 32) {
+            const unsigned long long base = row_base[r];
+            for (uint32_t j = jl; j < d; j += 32) {
+                dst[r * pitch + j] = (base != ~0ull) ? x[base + (uint64_t)j * g.s[3]] : 0.0f;
+            }
+        }
     }
     __syncthreads();
 
@@ -181,8 +191,21 @@ __global__ void __launch_bounds__(kEncThreads)
                 acc[i] = 0.0f;
             }
             const float *bcol = rot_t + 32 * tile + l32; // R[k][32*tile + l32] = rot_t[col + d*k]
-            // d is a multiple of 32: sixteen steps at a time, their operand loads issued together
-            for (uint32_t k0 = 0; k0 < d; k0 += 32) {
+            // d is a multiple of 32: sixty-four steps at a time where d allows (the loads of the rotation come from
+            // L2 and are the long pole: as many as possible are issued together), else sixteen
+            uint32_t k0 = 0;
+            for (; k0 + 128 <= d; k0 += 128) {
+                float b[64];
+#pragma unroll
+                for (int u = 0; u < 64; ++u) {
+                    b[u] = bcol[(uint64_t)d * (k0 + 2 * u + khalf)];
+                }
+#pragma unroll
+                for (int u = 0; u < 64; ++u) {
+                    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xs[l32 * pitch + k0 + 2 * u + khalf], b[u], acc, 0, 0, 0);
+                }
+            }
+            for (; k0 < d; k0 += 32) {
                 float a[16], b[16];
 #pragma unroll
                 for (int u = 0; u < 16; ++u) {
@@ -233,9 +256,9 @@ __global__ void __launch_bounds__(kEncThreads)
         const float lo = -3.0f * cp.block_scale;
         const float hi = 3.0f * cp.block_scale;
         const float step = (hi - lo) / (float)levels;
-        for (uint32_t e = tid; e < kEncRows * d; e += kEncThreads) {
-            const uint32_t r = e / d, j = e % d;
-            if (row0 + r < rows) {
+        const uint32_t jl = tid & 31;
+        for (uint32_t r = tid >> 5; r < kEncRows && row0 + r < rows; r += kEncThreads / 32) {
+            for (uint32_t j = jl; j < d; j += 32) {
                 fields[(uint64_t)(row0 + r) * d + j] = (uint8_t)uniform_bucket(ys[r * pitch + j], lo, hi, step, levels);
             }
         }
@@ -245,9 +268,16 @@ __global__ void __launch_bounds__(kEncThreads)
     // LLOYDMAX: row scale from an fma-accumulated sum of squares, j ascending
     if (tid < kEncRows) {
         float n2 = 0.0f;
-        for (uint32_t j = 0; j < d; ++j) {
-            const float v = ys[tid * pitch + j];
-            n2 = fmaf(v, v, n2);
+        for (uint32_t j0 = 0; j0 < d; j0 += 16) { // d is a multiple of 32
+            float v[16];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) {
+                v[u] = ys[tid * pitch + j0 + u];
+            }
+#pragma unroll
+            for (int u = 0; u < 16; ++u) {
+                n2 = fmaf(v[u], v[u], n2);
+            }
         }
         const float norm = sqrtf(n2);
         const float sqrt_d = sqrtf((float)d);
@@ -263,21 +293,36 @@ __global__ void __launch_bounds__(kEncThreads)
     }
     __syncthreads();
     const int nb = (1 << cp.bits) - 1;
-    for (uint32_t e = tid; e < kEncRows * d; e += kEncThreads) {
-        const uint32_t r = e / d, j = e % d;
-        if (row0 + r >= rows) {
-            continue;
+    // all fifteen possible thresholds in registers (unused ones at +inf), so that the count below is branch- and
+    // load-free
+    float bound[15];
+#pragma unroll
+    for (int k = 0; k < 15; ++k) {
+        bound[k] = k < nb ? cp.bounds[k] : INFINITY;
+    }
+    // four consecutive coordinates per thread, stored as one 32-bit word (d is a multiple of 32, the field array is
+    // 4-byte aligned and rows are d bytes long)
+    const uint32_t jl = tid & 31;
+    for (uint32_t r = tid >> 5; r < kEncRows && row0 + r < rows; r += kEncThreads / 32) {
+        const float inv = inv_s[r];
+        for (uint32_t j = 4 * jl; j < d; j += 128) {
+            uint32_t word = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float u = ys[r * pitch + j + i] * inv;
+                int code = 0;
+#pragma unroll
+                for (int k = 0; k < 15; ++k) {
+                    code += (u >= bound[k]) ? 1 : 0;
+                }
+                uint32_t f = (uint32_t)code;
+                if (cp.sign) {
+                    f = (f << 1) | ((u >= cp.levels[code]) ? 1u : 0u);
+                }
+                word |= f << (8 * i);
+            }
+            *reinterpret_cast<uint32_t *>(fields + (uint64_t)(row0 + r) * d + j) = word;
         }
-        const float u = ys[r * pitch + j] * inv_s[r];
-        int code = 0;
-        for (int k = 0; k < nb; ++k) {
-            code += (u >= cp.bounds[k]) ? 1 : 0;
-        }
-        uint32_t f = (uint32_t)code;
-        if (cp.sign) {
-            f = (f << 1) | ((u >= cp.levels[code]) ? 1u : 0u);
-        }
-        fields[(uint64_t)(row0 + r) * d + j] = (uint8_t)f;
     }
 }
 
@@ -557,7 +602,7 @@ int encode_side(weed_hip_kv_cache *c, Side &side, int which, int32_t seq_begin, 
     cp.block_scale = side.block_scale;
     std::memcpy(cp.bounds, side.bounds, sizeof(cp.bounds));
     std::memcpy(cp.levels, side.levels, sizeof(cp.levels));
-    const size_t smem = sizeof(float) * (2 * kEncRows * (d + 1) + kEncRows);
+    const size_t smem = sizeof(float) * (2 * kEncRows * (d + 1) + kEncRows) + sizeof(unsigned long long) * kEncRows;
     const uint32_t blocks = (rows + kEncRows - 1) / kEncRows;
     int parts = 1;
     while (parts * 2 * d <= (uint32_t)kEncThreads && parts < 8) {
