@@ -107,6 +107,22 @@ def extras(capi, torch, workloads, steps, warmup):
         "roofline": {"bound": "mfma", "achieved": flops / kernel_s / 1e12, "peak": 157.3, "unit": "TFLOP/s",
                      "frac": flops / kernel_s / 1e12 / 157.3}}
     del A, W, C
+    # decode-time projection y = x.W: 8 rows against a [4096 x 4096] column-major weight (64 MiB streamed per call)
+    X = torch.randn((4096, 8), device="cuda").t()               # logical [8, 4096], column-major
+    Wp = (torch.randn((4096, 4096), device="cuda") * 0.02).t()  # logical [4096, 4096], column-major
+    Y = torch.empty((4096, 8), device="cuda").t()
+    capi.profile_reset()
+    capi.profile_enable(True)
+    secs = time_calls(torch, lambda: capi.matmul(X, Wp, Y), steps, warmup)
+    k_ms, k_n = capi.profile_read("matmul")
+    capi.profile_enable(False)
+    kernel_s = 1e-3 * k_ms / max(1, k_n)
+    wbytes = 4096 * 4096 * 4
+    out["projection_8x4096x4096"] = {
+        "ms": 1e3 * secs, "kernel_ms": 1e3 * kernel_s,
+        "roofline": {"bound": "hbm", "achieved": wbytes / kernel_s / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": wbytes / kernel_s / 1e9 / HBM_PEAK_GBS}}
+    del X, Wp, Y
     # configuration 5a: encode-and-append 4096 tokens x 8 kv heads x 128, 3-bit codes (rotate, quantise, pack)
     wl = workloads.config(5)
     d = wl.head_dim

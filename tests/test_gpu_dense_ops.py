@@ -75,6 +75,36 @@ def test_matmul_matrix_core_layouts(gpu, oracle, a_col, b_col, o_col):
     np.testing.assert_allclose(C.cpu().numpy(), want.reshape(M, N), rtol=2e-5, atol=2e-5 * np.sqrt(K))
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (1, 100, 260), (5, 33, 1000), (16, 48, 256), (17, 16, 4100),
+                                   (33, 250, 516), (64, 512, 1024)])
+def test_matmul_decode_projections(gpu, oracle, M, N, K):
+    """Few rows against a tall column-major weight (y = x.W at decode time, the matrix-core streaming kernel):
+    row counts on both sides of the 16-row tiles, column counts that are not multiples of 16, k ranges that do not
+    fill the last 64-step, activations column-major, row-major and as a strided view; nothing outside the output
+    view may be written."""
+    import torch
+    rng = np.random.default_rng(M * 11 + N * 5 + K)
+    A = rng.standard_normal((M, K), dtype=np.float32)
+    W = (rng.standard_normal((K, N), dtype=np.float32) * 0.05).astype(np.float32)
+    want = (A.astype(np.float64) @ W.astype(np.float64))
+    if M * N * K <= 5_000_000:
+        chk = np.zeros(M * N, dtype=np.float32)
+        oracle.matmul(M, N, K, A.reshape(-1), (0, K, 1), W.reshape(-1), (0, N, 1), chk, (0, N, 1))
+        np.testing.assert_allclose(chk.reshape(M, N), want, rtol=2e-5, atol=2e-5 * np.sqrt(K))
+    tol = dict(rtol=2e-5, atol=2e-6 * np.sqrt(K))
+    Wd = col_major(W)
+    for mk in (col_major, dev):
+        C = mk(np.zeros((M, N), dtype=np.float32))
+        gpu.matmul(mk(A), Wd, C)
+        np.testing.assert_allclose(C.cpu().numpy(), want, **tol)
+    big_a = torch.zeros((M + 2, 3 * K + 2), device="cuda")
+    big_a[1:1 + M, 2:2 + 3 * K:3] = dev(A)
+    big_c = torch.full((M + 4, 2 * N + 3), -7.0, device="cuda")
+    gpu.matmul(big_a[1:1 + M, 2:2 + 3 * K:3], Wd, big_c[2:2 + M, 1:1 + 2 * N:2])
+    np.testing.assert_allclose(big_c[2:2 + M, 1:1 + 2 * N:2].cpu().numpy(), want, **tol)
+    assert torch.all(big_c[:2] == -7.0) and torch.all(big_c[2 + M:] == -7.0) and torch.all(big_c[:, 0::2] == -7.0)
+
+
 def test_matmul_cfg5_sampled(gpu):
     """Configuration 5b at full size ([4096 x 1024] . [1024 x 4096], column-major): the scalar checker would need
     minutes, so 4096 sampled outputs are compared with float64 dot products, plus the column sums identity

@@ -2,6 +2,8 @@
 // src/ops/matmul.cpp:95-122).  Replaces the OpenCL kernel matmul_real (src/common/qengine.cl:598-640).
 #include "common.h"
 
+#include <type_traits>
+
 using namespace weedhip;
 
 namespace {
@@ -213,6 +215,153 @@ __global__ void __launch_bounds__(256) matmul_mfma_kernel(const float *__restric
     }
 }
 
+
+// ---- "Skinny" products: few rows (M <= 64) against a tall weight matrix whose columns are contiguous along k -- the
+//      decode-time projections y = x.W of the attention module (src/modules/linear.cpp:86-100 with x = [B, d_model]).
+//      The time is the time to stream W once from HBM, so W is read with 16-byte loads along k, every element once.
+//
+//      A workgroup of 8 wavefronts owns 16 output columns; wavefront w takes the k range [w*k_per_wave, (w+1)*...).
+//      The products run on v_mfma_f32_16x16x4f32 (16 rows x 16 columns x 4 k per instruction).  The contraction
+//      index of an instruction may be any four k as long as both operands agree, so lane (column c = l % 16,
+//      group g = l / 16) keeps the sixteen consecutive k  kb + 16 g .. kb + 16 g + 15  of its column (four 16-byte
+//      loads) and instruction j of an iteration contracts over  { kb + 16 g + j : g = 0..3 }.  The few rows of `a`
+//      come from L2 (every workgroup reads all of them).  The eight partial tiles of a workgroup are added in LDS.
+constexpr int kSkinnyWaves = 8;
+
+template <int I, int N, typename F> __device__ __forceinline__ void static_for_sets(F &&f)
+{
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for_sets<I + 1, N>(f);
+    }
+}
+
+template <int MT> // 16-row tiles of a: M <= 16 * MT
+__global__ void __launch_bounds__(64 * kSkinnyWaves)
+    matmul_skinny_kernel(const float *__restrict__ a, const float *__restrict__ b, float *__restrict__ out, MatGeom g,
+                         uint32_t k_per_wave)
+{
+    typedef float float4v __attribute__((ext_vector_type(4)));
+    __shared__ float red[kSkinnyWaves][MT][256];
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t c = lane & 15, grp = lane >> 4;
+    const uint32_t n = blockIdx.x * 16 + c;
+    const bool n_ok = n < g.N;
+    const float *wcol = b + (uint64_t)g.b_off + (uint64_t)(n_ok ? n : 0) * g.b_s1; // b_s0 == 1: k contiguous
+    const uint32_t kb0 = wave * k_per_wave;
+    const uint32_t kb1 = min(kb0 + k_per_wave, g.K);
+    float4v acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        acc[mt] = float4v{ 0.0f, 0.0f, 0.0f, 0.0f };
+    }
+    // sixteen consecutive k of this lane's column, zero beyond the range (K is a multiple of 4: whole 16-byte loads)
+    auto load_w = [&](uint32_t kb, float4v (&w)[4]) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const uint32_t k = kb + 16 * grp + 4 * q;
+            w[q] = (n_ok && k < kb1) ? *reinterpret_cast<const float4v *>(wcol + k) : float4v{ 0.0f, 0.0f, 0.0f, 0.0f };
+        }
+    };
+    // the rows of a that go with them, for row tiles mt0 and mt0 + 1 (or mt0 alone): a[16 mt + c][kb + 16 grp + j]
+    constexpr int TA = MT >= 2 ? 2 : 1; // row tiles fetched and multiplied together
+    auto load_a = [&](uint32_t kb, int mt0, float (&av)[TA][16]) {
+#pragma unroll
+        for (int t = 0; t < TA; ++t) {
+            const uint32_t m = 16 * (mt0 + t) + c;
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const uint32_t k = kb + 16 * grp + j;
+                av[t][j] = (m < g.M && k < kb1)
+                    ? a[(uint64_t)g.a_off + (uint64_t)m * g.a_s0 + (uint64_t)k * g.a_s1] : 0.0f;
+            }
+        }
+    };
+    // Register sets in a ring: the operands of the next kAhead iterations travel while this one is multiplied.  With
+    // one or two row tiles both operands are fetched ahead; with four only the columns of b are, and the rows of a
+    // (which come from L2) are fetched pair by pair when needed.
+    constexpr bool kPrefetchA = MT <= 2;
+    constexpr int kAhead = 1; // more sets did not pay: a wavefront only runs a handful of iterations
+    constexpr int kSets = kAhead + 1;
+    float4v w[kSets][4];
+    float av[kPrefetchA ? kSets : 1][TA][16];
+    auto iterate = [&](auto pc, uint32_t kb) {
+        constexpr int P = decltype(pc)::value;
+        constexpr int Q = (P + kAhead) % kSets; // the set that was used last iteration is free again
+        load_w(kb + 64 * kAhead, w[Q]);
+        if constexpr (kPrefetchA) {
+            load_a(kb + 64 * kAhead, 0, av[Q]);
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+#pragma unroll
+                for (int t = 0; t < TA; ++t) {
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[P][t][j], w[P][j / 4][j % 4], acc[t], 0, 0, 0);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int mt0 = 0; mt0 < MT; mt0 += TA) {
+                load_a(kb, mt0, av[0]);
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+#pragma unroll
+                    for (int t = 0; t < TA; ++t) {
+                        acc[mt0 + t] =
+                            __builtin_amdgcn_mfma_f32_16x16x4f32(av[0][t][j], w[P][j / 4][j % 4], acc[mt0 + t], 0, 0, 0);
+                    }
+                }
+            }
+        }
+    };
+    if (kb0 < kb1) {
+        static_for_sets<0, kAhead>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            load_w(kb0 + 64 * i, w[i]);
+            if constexpr (kPrefetchA) {
+                load_a(kb0 + 64 * i, 0, av[i]);
+            }
+        });
+        uint32_t kb = kb0;
+        while (kb < kb1) {
+            // kSets iterations per round so that the set indices are compile-time constants
+            static_for_sets<0, kSets>([&](auto ic) {
+                if (kb < kb1) {
+                    iterate(ic, kb);
+                    kb += 64;
+                }
+            });
+        }
+    }
+    // lane (c, grp), register v of a tile: row 4 * grp + v, column c
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            red[wave][mt][(4 * grp + v) * 16 + c] = acc[mt][v];
+        }
+    }
+    __syncthreads();
+    for (uint32_t e = tid; e < (uint32_t)MT * 256; e += 64 * kSkinnyWaves) {
+        const uint32_t mt = e >> 8, r = (e >> 4) & 15, cc = e & 15;
+        float sum = 0.0f;
+#pragma unroll
+        for (int wv = 0; wv < kSkinnyWaves; ++wv) {
+            sum += red[wv][mt][r * 16 + cc];
+        }
+        const uint32_t m = 16 * mt + r, nn = blockIdx.x * 16 + cc;
+        if (m < g.M && nn < g.N) {
+            out[(uint64_t)g.o_off + (uint64_t)m * g.o_s0 + (uint64_t)nn * g.o_s1] = sum;
+        }
+    }
+}
+
+// Few rows, columns of b contiguous along k and 16-byte aligned, enough k to be worth streaming.
+bool skinny_eligible(const MatGeom &g, const float *b)
+{
+    return g.M <= 64 && g.K >= 256 && g.K % 4 == 0 && g.b_s0 == 1 && (g.b_s1 & 3) == 0 &&
+        (((uintptr_t)b + 4 * (uint64_t)g.b_off) & 15) == 0;
+}
+
 bool aligned16(const float *p, uint64_t elem_off) { return (((uintptr_t)p + 4 * elem_off) & 15) == 0; }
 
 // The matrix-core kernel needs full tiles, one contiguous dimension per operand and 16-byte aligned vector accesses.
@@ -265,6 +414,20 @@ extern "C" int weed_hip_matmul_f32(uint32_t M, uint32_t N, uint32_t K, const flo
             matmul_mfma_kernel<false, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, out_dev, g);
         } else {
             matmul_mfma_kernel<false, false><<<grid, 256, 0, stream()>>>(a_dev, b_dev, out_dev, g);
+        }
+        WEED_HIP_LAUNCH_CHECK();
+        return WEED_HIP_OK;
+    }
+    if (skinny_eligible(g, b_dev)) {
+        // every wavefront of a workgroup takes a whole number of 64-k iterations
+        const uint32_t k_per_wave = ((K + kSkinnyWaves - 1) / kSkinnyWaves + 63) / 64 * 64;
+        const uint32_t wgs = (N + 15) / 16;
+        if (M <= 16) {
+            matmul_skinny_kernel<1><<<wgs, 64 * kSkinnyWaves, 0, stream()>>>(a_dev, b_dev, out_dev, g, k_per_wave);
+        } else if (M <= 32) {
+            matmul_skinny_kernel<2><<<wgs, 64 * kSkinnyWaves, 0, stream()>>>(a_dev, b_dev, out_dev, g, k_per_wave);
+        } else {
+            matmul_skinny_kernel<4><<<wgs, 64 * kSkinnyWaves, 0, stream()>>>(a_dev, b_dev, out_dev, g, k_per_wave);
         }
         WEED_HIP_LAUNCH_CHECK();
         return WEED_HIP_OK;
