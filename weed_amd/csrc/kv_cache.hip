@@ -135,11 +135,12 @@ constexpr int kEncThreads = 256;
 //   rotate 0: y = x            1: y = x.R on the matrix cores (fp32)        2: y = x.R with the reference's
 //   rounding (multiply, then add, i ascending: src/ops/matmul.cpp:40-44).
 // PARTS = number of row slices the 256 threads are split into (each thread owns one output column of its slice).
+// `block` = index of the workgroup among those that work on this tensor.
 template <int PARTS>
-__global__ void __launch_bounds__(kEncThreads)
-    encode_rows_kernel(const float *__restrict__ x, Geom4 g, uint32_t Hkv, uint32_t T, uint32_t d, uint32_t rows,
-                       const float *__restrict__ rot_t, int rotate, CoderParams cp, uint8_t *__restrict__ fields,
-                       float *__restrict__ alpha_out)
+__device__ __forceinline__ void encode_rows_body(const float *__restrict__ x, const Geom4 &g, uint32_t Hkv, uint32_t T,
+                                                 uint32_t d, uint32_t rows, const float *__restrict__ rot_t, int rotate,
+                                                 const CoderParams &cp, uint8_t *__restrict__ fields,
+                                                 float *__restrict__ alpha_out, uint32_t block)
 {
     extern __shared__ float smem[];
     const uint32_t pitch = d + 1;
@@ -147,7 +148,7 @@ __global__ void __launch_bounds__(kEncThreads)
     float *ys = smem + kEncRows * pitch; // [kEncRows][pitch]
     float *inv_s = ys + kEncRows * pitch; // [kEncRows]
     const uint32_t tid = threadIdx.x;
-    const uint32_t row0 = blockIdx.x * kEncRows;
+    const uint32_t row0 = block * kEncRows;
 
     // gather the rows (logical row = (s*Hkv + h)*T + t): the first 32 threads work out where their row starts, then
     // thread (tid / 32, tid % 32) walks rows tid / 32, +8, ... and columns tid % 32, +32, ... (no divisions per element)
@@ -326,14 +327,38 @@ __global__ void __launch_bounds__(kEncThreads)
     }
 }
 
+// K and V of an append in ONE launch (the first `blocks_per_side` workgroups take K, the rest V): the appends of a
+// decode step are a chain of small kernels whose launches cost more than their work.
+struct EncSide {
+    const float *x;
+    Geom4 g;
+    const float *rot_t;
+    CoderParams cp;
+    uint8_t *fields;
+    float *alpha_out;
+};
+template <int PARTS>
+__global__ void __launch_bounds__(kEncThreads)
+    encode_rows_pair_kernel(EncSide k, EncSide v, uint32_t blocks_per_side, uint32_t Hkv, uint32_t T, uint32_t d,
+                            uint32_t rows, int rotate)
+{
+    if (blockIdx.x < blocks_per_side) {
+        encode_rows_body<PARTS>(k.x, k.g, Hkv, T, d, rows, k.rot_t, rotate, k.cp, k.fields, k.alpha_out, blockIdx.x);
+    } else {
+        encode_rows_body<PARTS>(v.x, v.g, Hkv, T, d, rows, v.rot_t, rotate, v.cp, v.fields, v.alpha_out,
+                                blockIdx.x - blocks_per_side);
+    }
+}
+
 // One thread per (new row, item of 8 coordinates): 8 bytes in, w bytes out.
-__global__ void pack_k_kernel(const uint8_t *__restrict__ fields, const float *__restrict__ alpha_in, uint32_t rows,
-                              uint32_t Hkv, uint32_t T, uint32_t d, uint32_t w, int32_t seq_begin,
-                              const int32_t *__restrict__ lens, uint8_t *__restrict__ out, uint64_t region_bytes,
-                              float *__restrict__ alpha_out, uint32_t padded)
+__device__ __forceinline__ void pack_k_body(const uint8_t *__restrict__ fields, const float *__restrict__ alpha_in,
+                                            uint32_t rows, uint32_t Hkv, uint32_t T, uint32_t d, uint32_t w,
+                                            int32_t seq_begin, const int32_t *__restrict__ lens,
+                                            uint8_t *__restrict__ out, uint64_t region_bytes,
+                                            float *__restrict__ alpha_out, uint32_t padded, uint32_t block)
 {
     const uint32_t items = d / 8;
-    const uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t idx = block * blockDim.x + threadIdx.x;
     if (idx >= rows * items) {
         return;
     }
@@ -354,13 +379,12 @@ __global__ void pack_k_kernel(const uint8_t *__restrict__ fields, const float *_
 
 // Row scales of the new V rows: one thread per new row copies the scale to its token slot and the region's largest
 // scale is kept up to date (one atomic per wavefront and region, not one per row).
-__global__ void __launch_bounds__(256) scatter_v_scales_kernel(const float *__restrict__ alpha_in, uint32_t rows,
-                                                              uint32_t Hkv, uint32_t T, int32_t seq_begin,
-                                                              const int32_t *__restrict__ lens,
-                                                              float *__restrict__ alpha_out,
-                                                              uint32_t *__restrict__ alpha_max, uint32_t padded)
+__device__ __forceinline__ void scatter_v_scales_body(const float *__restrict__ alpha_in, uint32_t rows, uint32_t Hkv,
+                                                      uint32_t T, int32_t seq_begin, const int32_t *__restrict__ lens,
+                                                      float *__restrict__ alpha_out, uint32_t *__restrict__ alpha_max,
+                                                      uint32_t padded, uint32_t block)
 {
-    const uint32_t row = blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t row = block * blockDim.x + threadIdx.x;
     const bool valid = row < rows;
     uint32_t region = 0xffffffffu, bits = 0;
     if (valid) {
@@ -387,11 +411,12 @@ __global__ void __launch_bounds__(256) scatter_v_scales_kernel(const float *__re
 
 // One thread per (sequence, kv head, 32-token half block, lane group, coordinate): rebuilds one item of 8 tokens,
 // keeping the fields of tokens that were already cached and zeroing those not yet written.
-__global__ void pack_v_kernel(const uint8_t *__restrict__ fields, uint32_t S, uint32_t Hkv, uint32_t T, uint32_t d,
-                              uint32_t w, int32_t seq_begin, const int32_t *__restrict__ lens, uint32_t halves,
-                              uint8_t *__restrict__ out, uint64_t region_bytes)
+__device__ __forceinline__ void pack_v_body(const uint8_t *__restrict__ fields, uint32_t S, uint32_t Hkv, uint32_t T,
+                                            uint32_t d, uint32_t w, int32_t seq_begin, const int32_t *__restrict__ lens,
+                                            uint32_t halves, uint8_t *__restrict__ out, uint64_t region_bytes,
+                                            uint32_t wg)
 {
-    const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const uint64_t idx = (uint64_t)wg * blockDim.x + threadIdx.x;
     const uint64_t total = (uint64_t)S * Hkv * halves * 4 * d;
     if (idx >= total) {
         return;
@@ -434,6 +459,34 @@ __global__ void pack_v_kernel(const uint8_t *__restrict__ fields, uint32_t S, ui
     item_build(f8, w, bytes);
     for (uint32_t b = 0; b < w; ++b) {
         dst[b] = bytes[b];
+    }
+}
+
+// The three packing steps of an append in ONE launch: workgroups [0, bk) pack the K items, [bk, bk + bv) rebuild the
+// V items, the rest store the V row scales.  All of them read the sequence lengths as they were before the append.
+struct PackArgs {
+    const uint8_t *k_fields, *v_fields; // one field per byte, as the encoder left them
+    const float *k_alpha_in, *v_alpha_in;
+    uint32_t rows, S, Hkv, T, d, wk, wv, halves, padded;
+    int32_t seq_begin;
+    const int32_t *lens;
+    uint8_t *k_out, *v_out;
+    uint64_t k_region_bytes, v_region_bytes;
+    float *k_alpha_out, *v_alpha_out; // null: the coder has no row scales
+    uint32_t *v_alpha_max;
+    uint32_t blocks_k, blocks_v;
+};
+__global__ void __launch_bounds__(256) pack_all_kernel(PackArgs a)
+{
+    if (blockIdx.x < a.blocks_k) {
+        pack_k_body(a.k_fields, a.k_alpha_in, a.rows, a.Hkv, a.T, a.d, a.wk, a.seq_begin, a.lens, a.k_out,
+                    a.k_region_bytes, a.k_alpha_out, a.padded, blockIdx.x);
+    } else if (blockIdx.x < a.blocks_k + a.blocks_v) {
+        pack_v_body(a.v_fields, a.S, a.Hkv, a.T, a.d, a.wv, a.seq_begin, a.lens, a.halves, a.v_out, a.v_region_bytes,
+                    blockIdx.x - a.blocks_k);
+    } else {
+        scatter_v_scales_body(a.v_alpha_in, a.rows, a.Hkv, a.T, a.seq_begin, a.lens, a.v_alpha_out, a.v_alpha_max,
+                              a.padded, blockIdx.x - a.blocks_k - a.blocks_v);
     }
 }
 
@@ -584,24 +637,40 @@ void free_side(Side &s)
     s.rot_t = nullptr;
 }
 
-int encode_side(weed_hip_kv_cache *c, Side &side, int which, int32_t seq_begin, int32_t seq_count, int32_t T_new,
-                const float *x, uint32_t off, const uint32_t stride[4], int rotate)
+EncSide enc_side_args(const weed_hip_kv_cache *c, const Side &side, const float *x, uint32_t off,
+                      const uint32_t stride[4], uint8_t *fields, float *alpha)
+{
+    EncSide e;
+    e.x = x;
+    e.g.off = off;
+    for (int i = 0; i < 4; ++i) {
+        e.g.s[i] = stride[i];
+    }
+    e.rot_t = side.rot_t;
+    e.cp.mode = c->cfg.mode;
+    e.cp.bits = side.bits;
+    e.cp.sign = side.sign;
+    e.cp.block_scale = side.block_scale;
+    std::memcpy(e.cp.bounds, side.bounds, sizeof(e.cp.bounds));
+    std::memcpy(e.cp.levels, side.levels, sizeof(e.cp.levels));
+    e.fields = fields;
+    e.alpha_out = alpha;
+    return e;
+}
+
+// Rotate, quantise and pack the new K and V rows: one launch for the two encoders, one for the three packing steps.
+// The scratch holds the K rows first, then the V rows.
+int encode_both(weed_hip_kv_cache *c, int32_t seq_begin, int32_t seq_count, int32_t T_new, const float *k_dev,
+                uint32_t k_off, const uint32_t k_stride[4], const float *v_dev, uint32_t v_off,
+                const uint32_t v_stride[4], int rotate)
 {
     const uint32_t d = (uint32_t)c->cfg.head_dim;
     const uint32_t Hkv = (uint32_t)c->cfg.n_kv_heads;
     const uint32_t rows = (uint32_t)seq_count * Hkv * (uint32_t)T_new;
-    Geom4 g;
-    g.off = off;
-    for (int i = 0; i < 4; ++i) {
-        g.s[i] = stride[i];
-    }
-    CoderParams cp;
-    cp.mode = c->cfg.mode;
-    cp.bits = side.bits;
-    cp.sign = side.sign;
-    cp.block_scale = side.block_scale;
-    std::memcpy(cp.bounds, side.bounds, sizeof(cp.bounds));
-    std::memcpy(cp.levels, side.levels, sizeof(cp.levels));
+    uint8_t *k_fields = c->enc_fields, *v_fields = c->enc_fields + (size_t)rows * d;
+    float *k_alpha = c->enc_alpha, *v_alpha = c->enc_alpha + rows;
+    const EncSide ek = enc_side_args(c, c->k, k_dev, k_off, k_stride, k_fields, k_alpha);
+    const EncSide ev = enc_side_args(c, c->v, v_dev, v_off, v_stride, v_fields, v_alpha);
     const size_t smem = sizeof(float) * (2 * kEncRows * (d + 1) + kEncRows) + sizeof(unsigned long long) * kEncRows;
     const uint32_t blocks = (rows + kEncRows - 1) / kEncRows;
     int parts = 1;
@@ -610,60 +679,63 @@ int encode_side(weed_hip_kv_cache *c, Side &side, int which, int32_t seq_begin, 
     }
     if (smem > 48 * 1024) {
         // more than the default dynamic LDS limit (head_dim 256): opt in per kernel instance
-        const void *fns[4] = { (const void *)encode_rows_kernel<1>, (const void *)encode_rows_kernel<2>,
-                               (const void *)encode_rows_kernel<4>, (const void *)encode_rows_kernel<8> };
+        const void *fns[4] = { (const void *)encode_rows_pair_kernel<1>, (const void *)encode_rows_pair_kernel<2>,
+                               (const void *)encode_rows_pair_kernel<4>, (const void *)encode_rows_pair_kernel<8> };
         for (const void *fn : fns) {
             WEED_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         }
     }
     {
         ProfileScope prof("kv_encode");
+        const uint32_t T = (uint32_t)T_new;
         switch (parts) {
         case 8:
-            encode_rows_kernel<8><<<blocks, kEncThreads, smem, stream()>>>(x, g, Hkv, (uint32_t)T_new, d, rows,
-                                                                           side.rot_t, rotate, cp, c->enc_fields,
-                                                                           c->enc_alpha);
+            encode_rows_pair_kernel<8><<<2 * blocks, kEncThreads, smem, stream()>>>(ek, ev, blocks, Hkv, T, d, rows, rotate);
             break;
         case 4:
-            encode_rows_kernel<4><<<blocks, kEncThreads, smem, stream()>>>(x, g, Hkv, (uint32_t)T_new, d, rows,
-                                                                           side.rot_t, rotate, cp, c->enc_fields,
-                                                                           c->enc_alpha);
+            encode_rows_pair_kernel<4><<<2 * blocks, kEncThreads, smem, stream()>>>(ek, ev, blocks, Hkv, T, d, rows, rotate);
             break;
         case 2:
-            encode_rows_kernel<2><<<blocks, kEncThreads, smem, stream()>>>(x, g, Hkv, (uint32_t)T_new, d, rows,
-                                                                           side.rot_t, rotate, cp, c->enc_fields,
-                                                                           c->enc_alpha);
+            encode_rows_pair_kernel<2><<<2 * blocks, kEncThreads, smem, stream()>>>(ek, ev, blocks, Hkv, T, d, rows, rotate);
             break;
         default:
-            encode_rows_kernel<1><<<blocks, kEncThreads, smem, stream()>>>(x, g, Hkv, (uint32_t)T_new, d, rows,
-                                                                           side.rot_t, rotate, cp, c->enc_fields,
-                                                                           c->enc_alpha);
+            encode_rows_pair_kernel<1><<<2 * blocks, kEncThreads, smem, stream()>>>(ek, ev, blocks, Hkv, T, d, rows, rotate);
             break;
         }
         WEED_HIP_LAUNCH_CHECK();
     }
     ProfileScope prof("kv_pack");
-    float *alpha_out = (c->cfg.mode == WEED_HIP_KV_LLOYDMAX) ? side.alpha : nullptr;
-    if (which == 0) {
-        const uint32_t n = rows * (d / 8);
-        pack_k_kernel<<<(n + 255) / 256, 256, 0, stream()>>>(c->enc_fields, c->enc_alpha, rows, Hkv, (uint32_t)T_new, d,
-                                                             side.w, seq_begin, c->lens_dev, side.fields,
-                                                             side.region_bytes, alpha_out, c->padded_tokens);
-    } else {
-        // a run of T_new tokens starting anywhere touches at most (T_new + 30) / 32 + 1 half blocks
-        const uint32_t halves = ((uint32_t)T_new + 30) / 32 + 1;
-        const uint64_t n = (uint64_t)seq_count * Hkv * halves * 4 * d;
-        pack_v_kernel<<<(uint32_t)((n + 255) / 256), 256, 0, stream()>>>(c->enc_fields, (uint32_t)seq_count, Hkv,
-                                                                         (uint32_t)T_new, d, side.w, seq_begin,
-                                                                         c->lens_dev, halves, side.fields,
-                                                                         side.region_bytes);
-        if (alpha_out) {
-            WEED_HIP_LAUNCH_CHECK();
-            scatter_v_scales_kernel<<<(rows + 255) / 256, 256, 0, stream()>>>(c->enc_alpha, rows, Hkv, (uint32_t)T_new,
-                                                                              seq_begin, c->lens_dev, alpha_out,
-                                                                              side.alpha_max, c->padded_tokens);
-        }
-    }
+    const bool scales = c->cfg.mode == WEED_HIP_KV_LLOYDMAX;
+    PackArgs a;
+    a.k_fields = k_fields;
+    a.v_fields = v_fields;
+    a.k_alpha_in = k_alpha;
+    a.v_alpha_in = v_alpha;
+    a.rows = rows;
+    a.S = (uint32_t)seq_count;
+    a.Hkv = Hkv;
+    a.T = (uint32_t)T_new;
+    a.d = d;
+    a.wk = c->k.w;
+    a.wv = c->v.w;
+    // a run of T_new tokens starting anywhere touches at most (T_new + 30) / 32 + 1 half blocks
+    a.halves = ((uint32_t)T_new + 30) / 32 + 1;
+    a.padded = c->padded_tokens;
+    a.seq_begin = seq_begin;
+    a.lens = c->lens_dev;
+    a.k_out = c->k.fields;
+    a.v_out = c->v.fields;
+    a.k_region_bytes = c->k.region_bytes;
+    a.v_region_bytes = c->v.region_bytes;
+    a.k_alpha_out = scales ? c->k.alpha : nullptr;
+    a.v_alpha_out = scales ? c->v.alpha : nullptr;
+    a.v_alpha_max = c->v.alpha_max;
+    const uint64_t nk = (uint64_t)rows * (d / 8);
+    const uint64_t nv = (uint64_t)seq_count * Hkv * a.halves * 4 * d;
+    a.blocks_k = (uint32_t)((nk + 255) / 256);
+    a.blocks_v = (uint32_t)((nv + 255) / 256);
+    const uint32_t blocks_s = scales ? (rows + 255) / 256 : 0;
+    pack_all_kernel<<<a.blocks_k + a.blocks_v + blocks_s, 256, 0, stream()>>>(a);
     WEED_HIP_LAUNCH_CHECK();
     return WEED_HIP_OK;
 }
@@ -1033,14 +1105,14 @@ int weed_hip_kv_encode_append(weed_hip_kv_cache *c, int32_t seq_begin, int32_t s
         c->enc_fields = nullptr;
         c->enc_alpha = nullptr;
         c->enc_rows_cap = 0;
-        if (hipMalloc((void **)&c->enc_fields, rows * c->cfg.head_dim) != hipSuccess ||
-            hipMalloc((void **)&c->enc_alpha, rows * sizeof(float)) != hipSuccess) {
+        // K rows, then V rows
+        if (hipMalloc((void **)&c->enc_fields, 2 * rows * c->cfg.head_dim) != hipSuccess ||
+            hipMalloc((void **)&c->enc_alpha, 2 * rows * sizeof(float)) != hipSuccess) {
             return fail(WEED_HIP_ENOMEM, "%s: scratch allocation failed", fn);
         }
         c->enc_rows_cap = rows;
     }
-    WEED_HIP_TRY(encode_side(c, c->k, 0, seq_begin, seq_count, T_new, k_dev, k_off, k_stride, rotate));
-    WEED_HIP_TRY(encode_side(c, c->v, 1, seq_begin, seq_count, T_new, v_dev, v_off, v_stride, rotate));
+    WEED_HIP_TRY(encode_both(c, seq_begin, seq_count, T_new, k_dev, k_off, k_stride, v_dev, v_off, v_stride, rotate));
     bump_lens_kernel<<<((uint32_t)seq_count + 255) / 256, 256, 0, stream()>>>(c->lens_dev, seq_begin, seq_count, T_new);
     WEED_HIP_LAUNCH_CHECK();
     for (int32_t s = 0; s < seq_count; ++s) {
