@@ -78,6 +78,16 @@ int weed_hip_matmul_f32(uint32_t M, uint32_t N, uint32_t K, const float *a_dev, 
                         uint32_t a_s1, const float *b_dev, uint32_t b_off, uint32_t b_s0, uint32_t b_s1, float *out_dev,
                         uint32_t o_off, uint32_t o_s0, uint32_t o_s1);
 
+/* batch[0] * batch[1] independent products in one launch: product (c0, c1) uses the offsets
+ * off + c0 * bs[0] + c1 * bs[1] of each operand.  The reference has no device entry for this: Tensor::matmul loops
+ * over the leading dimensions on the host and calls the 2-D product once per index (src/tensors/tensor.cpp:1213-1272);
+ * the attention scores and weights of a prefill are (batch x heads) such products.  At most 65535 products. */
+int weed_hip_matmul_batched_f32(const uint32_t batch[2], uint32_t M, uint32_t N, uint32_t K, const float *a_dev,
+                                uint32_t a_off, uint32_t a_s0, uint32_t a_s1, const uint32_t a_bs[2],
+                                const float *b_dev, uint32_t b_off, uint32_t b_s0, uint32_t b_s1,
+                                const uint32_t b_bs[2], float *out_dev, uint32_t o_off, uint32_t o_s0, uint32_t o_s1,
+                                const uint32_t o_bs[2]);
+
 /* out[o_off + i*o_stride] = a[a_off + i*a_stride] for i < n.  Replaces the OpenCL kernel copy_real
  * (src/common/qengine.cl:979, launched from src/ops/copy_broadcast.cpp:66); also the plain copy used to calibrate the
  * HBM traffic counters. */

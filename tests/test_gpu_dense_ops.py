@@ -105,6 +105,33 @@ def test_matmul_decode_projections(gpu, oracle, M, N, K):
     assert torch.all(big_c[:2] == -7.0) and torch.all(big_c[2 + M:] == -7.0) and torch.all(big_c[:, 0::2] == -7.0)
 
 
+@pytest.mark.parametrize("M,N,K", [(7, 5, 11), (64, 300, 128), (128, 256, 64), (4, 32, 512)])
+def test_matmul_batched_equals_the_loop(gpu, M, N, K):
+    """(batch x heads) products in one launch give what the 2-D entry point gives product by product (bit for bit:
+    the same kernel instance runs either way), for contiguous batches and for permuted / strided views, on the
+    generic, the matrix-core and the streaming kernel."""
+    import torch
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(M + N + K)
+    B0, B1 = 3, 4
+    a = torch.randn((B0, B1, M, K), generator=gen, device="cuda")
+    b = torch.randn((B0, B1, K, N), generator=gen, device="cuda")
+    views = [(a, b, torch.zeros((B0, B1, M, N), device="cuda")),
+             # [B0, M, B1, K] storage seen as [B0, B1, M, K]; b column-major per product; out with padding
+             (a.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3),
+              b.transpose(2, 3).contiguous().transpose(2, 3),
+              torch.zeros((B0, B1, M, N + 4), device="cuda")[..., :N])]
+    for av, bv, out in views:
+        gpu.matmul_batched(av, bv, out)
+        for i in range(B0):
+            for j in range(B1):
+                one = torch.zeros_like(out[i, j])
+                gpu.matmul(av[i, j], bv[i, j], one)
+                assert torch.equal(out[i, j], one)
+        ref = (a.double() @ b.double()).float()
+        torch.testing.assert_close(out, ref, rtol=2e-5, atol=2e-5 * K ** 0.5)
+
+
 def test_matmul_cfg5_sampled(gpu):
     """Configuration 5b at full size ([4096 x 1024] . [1024 x 4096], column-major): the scalar checker would need
     minutes, so 4096 sampled outputs are compared with float64 dot products, plus the column sums identity

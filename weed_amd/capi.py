@@ -52,6 +52,9 @@ SIGNATURES = {
     "weed_hip_profile_read": (c_int, [c_char_p, POINTER(c_double), POINTER(c_uint64)]),
     "weed_hip_matmul_f32": (c_int, [c_uint32, c_uint32, c_uint32, c_void_p, c_uint32, c_uint32, c_uint32, c_void_p,
                                     c_uint32, c_uint32, c_uint32, c_void_p, c_uint32, c_uint32, c_uint32]),
+    "weed_hip_matmul_batched_f32": (c_int, [U32P, c_uint32, c_uint32, c_uint32, c_void_p, c_uint32, c_uint32, c_uint32,
+                                            U32P, c_void_p, c_uint32, c_uint32, c_uint32, U32P, c_void_p, c_uint32,
+                                            c_uint32, c_uint32, U32P]),
     "weed_hip_copy_f32": (c_int, [c_uint64, c_void_p, c_uint32, c_uint32, c_void_p, c_uint32, c_uint32]),
     "weed_hip_elementwise_f32": (c_int, [c_int, c_uint32, U32P, c_void_p, c_uint32, U32P, c_void_p, c_uint32, U32P,
                                          c_void_p, c_uint32, U32P]),
@@ -238,6 +241,17 @@ def matmul(a, b, out):
     check(load().weed_hip_matmul_f32(M, N, K, c_void_p(a.data_ptr()), 0, a.stride(0), a.stride(1),
                                      c_void_p(b.data_ptr()), 0, b.stride(0), b.stride(1), c_void_p(out.data_ptr()), 0,
                                      out.stride(0), out.stride(1)))
+
+
+def matmul_batched(a, b, out):
+    """4-D torch views [B0, B1, ., .] (any strides): out[i, j] = a[i, j] @ b[i, j], one launch."""
+    B0, B1, M, K = a.shape
+    N = b.shape[3]
+    assert tuple(b.shape) == (B0, B1, K, N) and tuple(out.shape) == (B0, B1, M, N)
+    check(load().weed_hip_matmul_batched_f32(
+        u32([B0, B1]), M, N, K, c_void_p(a.data_ptr()), 0, a.stride(2), a.stride(3), u32([a.stride(0), a.stride(1)]),
+        c_void_p(b.data_ptr()), 0, b.stride(2), b.stride(3), u32([b.stride(0), b.stride(1)]),
+        c_void_p(out.data_ptr()), 0, out.stride(2), out.stride(3), u32([out.stride(0), out.stride(1)])))
 
 
 def copy(a, out):

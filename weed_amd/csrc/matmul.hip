@@ -13,14 +13,28 @@ struct MatGeom {
     uint32_t a_off, a_s0, a_s1;
     uint32_t b_off, b_s0, b_s1;
     uint32_t o_off, o_s0, o_s1;
+    // batched products: grid.z = nb0 * nb1 independent products, product (c0, c1) starts at off + c0*bs[0] + c1*bs[1]
+    uint32_t nb0;
+    uint32_t a_bs[2], b_bs[2], o_bs[2];
 };
+
+// The geometry of the product this workgroup belongs to (blockIdx.z selects it).
+__device__ __forceinline__ MatGeom batch_geom(MatGeom g)
+{
+    const uint32_t c0 = blockIdx.z % g.nb0, c1 = blockIdx.z / g.nb0;
+    g.a_off += c0 * g.a_bs[0] + c1 * g.a_bs[1];
+    g.b_off += c0 * g.b_bs[0] + c1 * g.b_bs[1];
+    g.o_off += c0 * g.o_bs[0] + c1 * g.o_bs[1];
+    return g;
+}
 
 constexpr int BM = 64, BN = 64, BK = 16;
 
 // Generic tiled kernel on the vector ALU: any shape, any strides.
 __global__ void __launch_bounds__(256) matmul_tiled_kernel(const float *__restrict__ a, const float *__restrict__ b,
-                                                          float *__restrict__ out, MatGeom g)
+                                                          float *__restrict__ out, MatGeom g_launch)
 {
+    const MatGeom g = batch_geom(g_launch);
     __shared__ float As[BK][BM + 4];
     __shared__ float Bs[BK][BN + 4];
     const uint32_t tid = threadIdx.x;
@@ -91,8 +105,9 @@ constexpr int TM = 128, TN = 128, TK = 16, PITCH = 132;
 
 template <bool A_ICONTIG, bool B_KCONTIG>
 __global__ void __launch_bounds__(256) matmul_mfma_kernel(const float *__restrict__ a, const float *__restrict__ b,
-                                                          float *__restrict__ out, MatGeom g)
+                                                          float *__restrict__ out, MatGeom g_launch)
 {
+    const MatGeom g = batch_geom(g_launch);
     __shared__ __attribute__((aligned(16))) float As[2][TK][PITCH];
     __shared__ __attribute__((aligned(16))) float Bs[2][TK][PITCH];
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -238,9 +253,10 @@ template <int I, int N, typename F> __device__ __forceinline__ void static_for_s
 
 template <int MT> // 16-row tiles of a: M <= 16 * MT
 __global__ void __launch_bounds__(64 * kSkinnyWaves)
-    matmul_skinny_kernel(const float *__restrict__ a, const float *__restrict__ b, float *__restrict__ out, MatGeom g,
-                         uint32_t k_per_wave)
+    matmul_skinny_kernel(const float *__restrict__ a, const float *__restrict__ b, float *__restrict__ out,
+                         MatGeom g_launch, uint32_t k_per_wave)
 {
+    const MatGeom g = batch_geom(g_launch);
     typedef float float4v __attribute__((ext_vector_type(4)));
     __shared__ float red[kSkinnyWaves][MT][256];
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -359,7 +375,7 @@ __global__ void __launch_bounds__(64 * kSkinnyWaves)
 bool skinny_eligible(const MatGeom &g, const float *b)
 {
     return g.M <= 64 && g.K >= 256 && g.K % 4 == 0 && g.b_s0 == 1 && (g.b_s1 & 3) == 0 &&
-        (((uintptr_t)b + 4 * (uint64_t)g.b_off) & 15) == 0;
+        ((g.b_bs[0] | g.b_bs[1]) & 3) == 0 && (((uintptr_t)b + 4 * (uint64_t)g.b_off) & 15) == 0;
 }
 
 bool aligned16(const float *p, uint64_t elem_off) { return (((uintptr_t)p + 4 * elem_off) & 15) == 0; }
@@ -385,27 +401,28 @@ bool mfma_eligible(const MatGeom &g, const float *a, const float *b, const float
     if (g.o_s0 == 1 && (!aligned16(out, g.o_off) || (g.o_s1 & 3))) {
         return false;
     }
-    return true;
+    // every product of a batch keeps the alignment
+    return !((g.a_bs[0] | g.a_bs[1] | g.b_bs[0] | g.b_bs[1] | g.o_bs[0] | g.o_bs[1]) & 3);
 }
 
 } // namespace
 
-extern "C" int weed_hip_matmul_f32(uint32_t M, uint32_t N, uint32_t K, const float *a_dev, uint32_t a_off,
-                                   uint32_t a_s0, uint32_t a_s1, const float *b_dev, uint32_t b_off, uint32_t b_s0,
-                                   uint32_t b_s1, float *out_dev, uint32_t o_off, uint32_t o_s0, uint32_t o_s1)
+namespace {
+
+int launch_matmul(const char *fn, const MatGeom &g, uint32_t batch, const float *a_dev, const float *b_dev, float *out_dev)
 {
-    const char *fn = "weed_hip_matmul_f32";
     WEED_HIP_REQUIRE(a_dev && b_dev && out_dev, "%s: null pointer", fn);
     WEED_HIP_TRY(ensure_init());
-    if (!M || !N) {
+    if (!g.M || !g.N || !batch) {
         return WEED_HIP_OK;
     }
-    MatGeom g = { M, N, K, a_off, a_s0, a_s1, b_off, b_s0, b_s1, o_off, o_s0, o_s1 };
+    WEED_HIP_REQUIRE(batch <= 65535u, "%s: %u products in one call (at most 65535)", fn, batch);
+    const uint32_t M = g.M, N = g.N, K = g.K;
     ProfileScope prof("matmul");
     if (mfma_eligible(g, a_dev, b_dev, out_dev)) {
-        const dim3 grid(M / TM, N / TN);
+        const dim3 grid(M / TM, N / TN, batch);
         WEED_HIP_REQUIRE(grid.y <= 65535u, "%s: N = %u too large", fn, N);
-        const bool a_i = a_s0 == 1, b_k = b_s0 == 1;
+        const bool a_i = g.a_s0 == 1, b_k = g.b_s0 == 1;
         if (a_i && b_k) {
             matmul_mfma_kernel<true, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, out_dev, g);
         } else if (a_i) {
@@ -421,7 +438,7 @@ extern "C" int weed_hip_matmul_f32(uint32_t M, uint32_t N, uint32_t K, const flo
     if (skinny_eligible(g, b_dev)) {
         // every wavefront of a workgroup takes a whole number of 64-k iterations
         const uint32_t k_per_wave = ((K + kSkinnyWaves - 1) / kSkinnyWaves + 63) / 64 * 64;
-        const uint32_t wgs = (N + 15) / 16;
+        const dim3 wgs((N + 15) / 16, 1, batch);
         if (M <= 16) {
             matmul_skinny_kernel<1><<<wgs, 64 * kSkinnyWaves, 0, stream()>>>(a_dev, b_dev, out_dev, g, k_per_wave);
         } else if (M <= 32) {
@@ -432,9 +449,34 @@ extern "C" int weed_hip_matmul_f32(uint32_t M, uint32_t N, uint32_t K, const flo
         WEED_HIP_LAUNCH_CHECK();
         return WEED_HIP_OK;
     }
-    const dim3 grid((M + BM - 1) / BM, (N + BN - 1) / BN);
+    const dim3 grid((M + BM - 1) / BM, (N + BN - 1) / BN, batch);
     WEED_HIP_REQUIRE(grid.y <= 65535u, "%s: N = %u too large", fn, N);
     matmul_tiled_kernel<<<grid, 256, 0, stream()>>>(a_dev, b_dev, out_dev, g);
     WEED_HIP_LAUNCH_CHECK();
     return WEED_HIP_OK;
+}
+
+} // namespace
+
+extern "C" int weed_hip_matmul_f32(uint32_t M, uint32_t N, uint32_t K, const float *a_dev, uint32_t a_off,
+                                   uint32_t a_s0, uint32_t a_s1, const float *b_dev, uint32_t b_off, uint32_t b_s0,
+                                   uint32_t b_s1, float *out_dev, uint32_t o_off, uint32_t o_s0, uint32_t o_s1)
+{
+    const MatGeom g = { M, N, K, a_off, a_s0, a_s1, b_off, b_s0, b_s1, o_off, o_s0, o_s1, 1, { 0, 0 }, { 0, 0 }, { 0, 0 } };
+    return launch_matmul("weed_hip_matmul_f32", g, 1, a_dev, b_dev, out_dev);
+}
+
+extern "C" int weed_hip_matmul_batched_f32(const uint32_t batch[2], uint32_t M, uint32_t N, uint32_t K,
+                                           const float *a_dev, uint32_t a_off, uint32_t a_s0, uint32_t a_s1,
+                                           const uint32_t a_bs[2], const float *b_dev, uint32_t b_off, uint32_t b_s0,
+                                           uint32_t b_s1, const uint32_t b_bs[2], float *out_dev, uint32_t o_off,
+                                           uint32_t o_s0, uint32_t o_s1, const uint32_t o_bs[2])
+{
+    const char *fn = "weed_hip_matmul_batched_f32";
+    WEED_HIP_REQUIRE(batch && a_bs && b_bs && o_bs, "%s: null pointer", fn);
+    const uint64_t n = (uint64_t)batch[0] * batch[1];
+    WEED_HIP_REQUIRE(n <= 65535u, "%s: %llu products in one call (at most 65535)", fn, (unsigned long long)n);
+    const MatGeom g = { M, N, K, a_off, a_s0, a_s1, b_off, b_s0, b_s1, o_off, o_s0, o_s1, batch[0] ? batch[0] : 1u,
+                        { a_bs[0], a_bs[1] }, { b_bs[0], b_bs[1] }, { o_bs[0], o_bs[1] } };
+    return launch_matmul(fn, g, (uint32_t)n, a_dev, b_dev, out_dev);
 }

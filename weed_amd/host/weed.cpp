@@ -587,21 +587,46 @@ TensorPtr Tensor::matmul(TensorPtr a, TensorPtr b)
         shp.push_back(M);
         shp.push_back(N);
         TensorPtr out = allocate(shp, *a);
-        for (tcapint i = 0U; i < batch; ++i) {
-            Tensor ai = *a, bi = *b, oi = *out;
-            tcapint rem = i;
-            for (size_t dd = 0; dd < rank - 2U; ++dd) {
+        // The reference calls the 2-D product once per index of the leading dimensions; here the two innermost
+        // leading dimensions go to the device as ONE batched launch and only what lies beyond them is looped over.
+        validate_all_same_device({ a.get(), b.get(), out.get() }, "MatMulKernel::matmul");
+        real1 *ap = device_ptr(*a, "matmul"), *bp = device_ptr(*b, "matmul"), *op = device_ptr(*out, "matmul");
+        const size_t lead = rank - 2U;          // leading dimensions
+        const size_t inner = lead >= 2U ? 2U : lead; // handled by the device: dimensions [0, inner)
+        tcapint nb[2] = { 1U, 1U }, abs_[2] = { 0U, 0U }, bbs[2] = { 0U, 0U }, obs[2] = { 0U, 0U };
+        for (size_t dd = 0; dd < inner; ++dd) {
+            nb[dd] = a->shape[dd];
+            abs_[dd] = a->stride[dd];
+            bbs[dd] = b->stride[dd];
+            obs[dd] = out->stride[dd];
+        }
+        tcapint outer = 1U;
+        for (size_t dd = inner; dd < lead; ++dd) {
+            outer *= a->shape[dd];
+        }
+        (void)batch;
+        WEED_DEVICE_LOCK();
+        for (tcapint i = 0U; i < outer; ++i) {
+            tcapint aoff = a->offset, boff = b->offset, ooff = out->offset, rem = i;
+            for (size_t dd = inner; dd < lead; ++dd) {
                 const tcapint c = rem % a->shape[dd];
                 rem /= a->shape[dd];
-                ai.offset += c * a->stride[dd];
-                bi.offset += c * b->stride[dd];
-                oi.offset += c * out->stride[dd];
+                aoff += c * a->stride[dd];
+                boff += c * b->stride[dd];
+                ooff += c * out->stride[dd];
             }
-            for (Tensor *t : { &ai, &bi, &oi }) {
-                t->shape.erase(t->shape.begin(), t->shape.end() - 2);
-                t->stride.erase(t->stride.begin(), t->stride.end() - 2);
+            // at most 65535 products per launch: split the second batch dimension if need be
+            const tcapint per = nb[0] ? std::max<tcapint>(1U, std::min<tcapint>(nb[1], 65535U / std::max<tcapint>(nb[0], 1U))) : 1U;
+            if (nb[0] > 65535U) {
+                throw std::invalid_argument("batched matmul: more than 65535 products along one dimension");
             }
-            Weed::matmul(ai, bi, oi);
+            for (tcapint c1 = 0U; c1 < nb[1]; c1 += per) {
+                const tcapint n1 = std::min<tcapint>(per, nb[1] - c1);
+                const tcapint bshape[2] = { nb[0], n1 };
+                HipDevice::check(weed_hip_matmul_batched_f32(bshape, M, N, K, ap, aoff + c1 * abs_[1], a->stride[rank - 2U],
+                    a->stride[rank - 1U], abs_, bp, boff + c1 * bbs[1], b->stride[rank - 2U], b->stride[rank - 1U], bbs, op,
+                    ooff + c1 * obs[1], out->stride[rank - 2U], out->stride[rank - 1U], obs));
+            }
         }
         return out;
     }
