@@ -169,14 +169,29 @@ template <int OP> __global__ void __launch_bounds__(256) elementwise_kernel(cons
 {
     const uint64_t step = (uint64_t)gridDim.x * blockDim.x;
     for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < g.n; i += step) {
-        uint64_t tmp = i, ai = g.a_off, bi = g.b_off, oi = g.o_off;
-        for (uint32_t dd = 0; dd < g.rank; ++dd) {
-            const uint32_t dim = g.shape[dd];
-            const uint32_t c = (uint32_t)(tmp % dim);
-            tmp /= dim;
-            ai += (uint64_t)c * g.a_stride[dd];
-            bi += (uint64_t)c * g.b_stride[dd];
-            oi += (uint64_t)c * g.o_stride[dd];
+        uint64_t ai = g.a_off, bi = g.b_off, oi = g.o_off;
+        if (g.n <= 0xffffffffull) {
+            // the usual case: 32-bit index arithmetic (a 64-bit division costs several times as much)
+            uint32_t tmp = (uint32_t)i;
+            for (uint32_t dd = 0; dd < g.rank; ++dd) {
+                const uint32_t dim = g.shape[dd];
+                const uint32_t q = tmp / dim;
+                const uint32_t c = tmp - q * dim;
+                tmp = q;
+                ai += (uint64_t)c * g.a_stride[dd];
+                bi += (uint64_t)c * g.b_stride[dd];
+                oi += (uint64_t)c * g.o_stride[dd];
+            }
+        } else {
+            uint64_t tmp = i;
+            for (uint32_t dd = 0; dd < g.rank; ++dd) {
+                const uint32_t dim = g.shape[dd];
+                const uint32_t c = (uint32_t)(tmp % dim);
+                tmp /= dim;
+                ai += (uint64_t)c * g.a_stride[dd];
+                bi += (uint64_t)c * g.b_stride[dd];
+                oi += (uint64_t)c * g.o_stride[dd];
+            }
         }
         const float x = a[ai];
         float r;
