@@ -2,6 +2,7 @@
 // src/ops/matmul.cpp:95-122).  Replaces the OpenCL kernel matmul_real (src/common/qengine.cl:598-640).
 #include "common.h"
 
+#include <algorithm>
 #include <type_traits>
 
 using namespace weedhip;
@@ -371,6 +372,123 @@ __global__ void __launch_bounds__(64 * kSkinnyWaves)
     }
 }
 
+
+// ---- Seventeen to 64 rows: the same streaming of b, but the rows of a no longer come cheaply from L2 if every
+//      16-column workgroup reads all of them (64 rows x K floats per workgroup, four times the bytes of b in total).
+//      Here a workgroup owns 128 columns (16 per wavefront), all its wavefronts walk the same k range and share the
+//      rows of a through LDS ([k][row], two buffers, one barrier per 64-k step), and the k ranges are split over
+//      gridDim.y workgroups whose partial results a small second kernel adds up in a fixed order.
+constexpr int kWideWaves = 8;
+constexpr int kWidePitch = 65; // floats per k row of the staged block of a: two-way bank conflicts at worst
+
+template <int MT>
+__global__ void __launch_bounds__(64 * kWideWaves)
+    matmul_skinny_wide_kernel(const float *__restrict__ a, const float *__restrict__ b, float *__restrict__ part,
+                              MatGeom g_launch, uint32_t k_per_split)
+{
+    typedef float float4v __attribute__((ext_vector_type(4)));
+    const MatGeom g = batch_geom(g_launch);
+    __shared__ float As[2][64][kWidePitch];
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t c = lane & 15, grp = lane >> 4;
+    const uint32_t n = blockIdx.x * 128 + wave * 16 + c;
+    const bool n_ok = n < g.N;
+    const float *wcol = b + (uint64_t)g.b_off + (uint64_t)(n_ok ? n : 0) * g.b_s1;
+    const uint32_t kb0 = blockIdx.y * k_per_split;
+    const uint32_t kb1 = min(kb0 + k_per_split, g.K);
+    float4v acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        acc[mt] = float4v{ 0.0f, 0.0f, 0.0f, 0.0f };
+    }
+    auto load_w = [&](uint32_t kb, float4v (&w)[4]) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const uint32_t k = kb + 16 * grp + 4 * q;
+            w[q] = (n_ok && k < kb1) ? *reinterpret_cast<const float4v *>(wcol + k) : float4v{ 0.0f, 0.0f, 0.0f, 0.0f };
+        }
+    };
+    // the 16*MT x 64 block of a for one step: thread t fetches rows (t % 16) + 16 i of k column t / 16 + 32 j
+    constexpr int kStage = MT * 2; // elements per thread: 16*MT rows x 64 k over 512 threads
+    auto fetch_a = [&](uint32_t kb, float (&v)[kStage]) {
+#pragma unroll
+        for (int e = 0; e < kStage; ++e) {
+            const uint32_t m = (tid & 15) + 16 * (e % MT);
+            const uint32_t k = kb + (tid >> 4) + 32 * (e / MT);
+            v[e] = (m < g.M && k < kb1) ? a[(uint64_t)g.a_off + (uint64_t)m * g.a_s0 + (uint64_t)k * g.a_s1] : 0.0f;
+        }
+    };
+    auto store_a = [&](int buf, const float (&v)[kStage]) {
+#pragma unroll
+        for (int e = 0; e < kStage; ++e) {
+            As[buf][(tid >> 4) + 32 * (e / MT)][(tid & 15) + 16 * (e % MT)] = v[e];
+        }
+    };
+    float4v w[2][4];
+    float stage[kStage];
+    if (kb0 < kb1) {
+        load_w(kb0, w[0]);
+        fetch_a(kb0, stage);
+        store_a(0, stage);
+    }
+    __syncthreads();
+    auto iterate = [&](auto pc, uint32_t kb) {
+        constexpr int P = decltype(pc)::value;
+        load_w(kb + 64, w[1 - P]);
+        fetch_a(kb + 64, stage); // lands in registers while this step is multiplied
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(As[P][16 * grp + j][16 * mt + c], w[P][j / 4][j % 4],
+                                                               acc[mt], 0, 0, 0);
+            }
+        }
+        store_a(1 - P, stage);
+        __syncthreads(); // the other buffer is complete, and nobody reads this one any more
+    };
+    for (uint32_t kb = kb0; kb < kb1; kb += 128) {
+        iterate(std::integral_constant<int, 0>{}, kb);
+        if (kb + 64 < kb1) {
+            iterate(std::integral_constant<int, 1>{}, kb + 64);
+        }
+    }
+    // partial result of this k range: part[split][row][column] (dense, row-major in columns)
+    float *dst = part + ((uint64_t)blockIdx.z * gridDim.y + blockIdx.y) * g.M * g.N;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const uint32_t m = 16 * mt + 4 * grp + v;
+            if (m < g.M && n_ok) {
+                dst[(uint64_t)m * g.N + n] = acc[mt][v];
+            }
+        }
+    }
+}
+
+// out = sum over the k splits, in rising split order.
+__global__ void __launch_bounds__(256) matmul_split_sum_kernel(const float *__restrict__ part, float *__restrict__ out,
+                                                              MatGeom g_launch, uint32_t splits)
+{
+    const MatGeom g = batch_geom(g_launch);
+    const uint32_t idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= g.M * g.N) {
+        return;
+    }
+    const uint32_t m = idx / g.N, n = idx - m * g.N;
+    const float *src = part + (uint64_t)blockIdx.z * splits * g.M * g.N + idx;
+    float sum = 0.0f;
+    for (uint32_t s = 0; s < splits; ++s) {
+        sum += src[(uint64_t)s * g.M * g.N];
+    }
+    out[(uint64_t)g.o_off + (uint64_t)m * g.o_s0 + (uint64_t)n * g.o_s1] = sum;
+}
+
+// Scratch for the partial results of split products: grows as needed, kept for the life of the process.
+float *g_split_ws = nullptr;
+size_t g_split_ws_bytes = 0;
+
 // Few rows, columns of b contiguous along k and 16-byte aligned, enough k to be worth streaming.
 bool skinny_eligible(const MatGeom &g, const float *b)
 {
@@ -439,6 +557,37 @@ int launch_matmul(const char *fn, const MatGeom &g, uint32_t batch, const float 
         // every wavefront of a workgroup takes a whole number of 64-k iterations
         const uint32_t k_per_wave = ((K + kSkinnyWaves - 1) / kSkinnyWaves + 63) / 64 * 64;
         const dim3 wgs((N + 15) / 16, 1, batch);
+        if (M > 16 && N >= 512) {
+            // shared rows, k split over workgroups (about one workgroup per compute unit), second pass adds the splits
+            const uint32_t col_wgs = (N + 127) / 128;
+            uint32_t splits = std::max(1u, std::min((256u + col_wgs - 1) / col_wgs, K / 256u));
+            const uint32_t k_per_split = ((K + splits - 1) / splits + 63) / 64 * 64;
+            splits = (K + k_per_split - 1) / k_per_split;
+            const size_t need = sizeof(float) * (size_t)batch * splits * M * N;
+            if (need > g_split_ws_bytes) {
+                WEED_HIP_CHECK(hipStreamSynchronize(stream()));
+                (void)hipFree(g_split_ws);
+                g_split_ws = nullptr;
+                g_split_ws_bytes = 0;
+                if (hipMalloc((void **)&g_split_ws, need) != hipSuccess) {
+                    return fail(WEED_HIP_ENOMEM, "%s: scratch allocation of %zu bytes failed", fn, need);
+                }
+                g_split_ws_bytes = need;
+            }
+            const dim3 wide(col_wgs, splits, batch);
+            if (M <= 32) {
+                matmul_skinny_wide_kernel<2><<<wide, 64 * kWideWaves, 0, stream()>>>(a_dev, b_dev, g_split_ws, g,
+                                                                                   k_per_split);
+            } else {
+                matmul_skinny_wide_kernel<4><<<wide, 64 * kWideWaves, 0, stream()>>>(a_dev, b_dev, g_split_ws, g,
+                                                                                   k_per_split);
+            }
+            WEED_HIP_LAUNCH_CHECK();
+            matmul_split_sum_kernel<<<dim3((M * N + 255) / 256, 1, batch), 256, 0, stream()>>>(g_split_ws, out_dev, g,
+                                                                                             splits);
+            WEED_HIP_LAUNCH_CHECK();
+            return WEED_HIP_OK;
+        }
         if (M <= 16) {
             matmul_skinny_kernel<1><<<wgs, 64 * kSkinnyWaves, 0, stream()>>>(a_dev, b_dev, out_dev, g, k_per_wave);
         } else if (M <= 32) {
