@@ -207,6 +207,41 @@ def test_softmax_and_reduce_strided_against_checker(gpu, oracle, shape):
                     np.testing.assert_array_equal(r.cpu().numpy(), ref.astype(np.float32))
 
 
+@pytest.mark.parametrize("shape,axis", [((9004, 40), 0), ((40000, 24), 1), ((64, 8, 1, 700), 3), ((260, 3, 5), 0)])
+def test_softmax_and_reduce_launch_shapes(gpu, shape, axis):
+    """One case per way the threads are spread: a contiguous row longer than what the registers keep between the
+    passes, enough rows for 32 per workgroup, few long strided rows (decode-time scores), a short aligned row.
+    Some positions are masked with -inf, one row of the decode case entirely (its softmax is NaN, as in numpy)."""
+    import torch
+    rng = np.random.default_rng(shape[0] + axis)
+    x = rng.standard_normal(shape, dtype=np.float32) * 4.0
+    x[rng.random(shape) < 0.1] = -np.inf
+    if len(shape) == 4:
+        x[3, 2, 0, :] = -np.inf
+    xd = col_major(x)
+    out = torch.zeros_like(xd)
+    gpu.softmax(xd, out, axis)
+    x64 = x.astype(np.float64)
+    with np.errstate(invalid="ignore"):
+        e = np.exp(x64 - x64.max(axis=axis, keepdims=True))
+        want = e / e.sum(axis=axis, keepdims=True)
+    got = out.cpu().numpy()
+    np.testing.assert_array_equal(np.isnan(got), np.isnan(want))
+    np.testing.assert_allclose(np.nan_to_num(got), np.nan_to_num(want), rtol=2e-5, atol=1e-7)
+    oshape = [s for i, s in enumerate(shape) if i != axis]
+    finite = np.where(np.isinf(x), 0.0, x).astype(np.float32)
+    fd = col_major(finite)
+    for op, fn, src, srcd in ((gpu.REDUCE_SUM, np.sum, finite, fd), (gpu.REDUCE_MAX, np.max, x, xd),
+                              (gpu.REDUCE_MIN, np.min, finite, fd)):
+        r = col_major(np.zeros(oshape, dtype=np.float32))
+        gpu.reduce(op, srcd, r, axis)
+        ref = fn(src.astype(np.float64), axis=axis)
+        if op == gpu.REDUCE_SUM:
+            np.testing.assert_allclose(r.cpu().numpy(), ref, rtol=2e-5, atol=2e-5 * np.sqrt(shape[axis]))
+        else:
+            np.testing.assert_array_equal(r.cpu().numpy(), ref.astype(np.float32))
+
+
 def test_reduce_reference_cases(gpu):
     import torch
     # tests.cpp:177-228: sum([1,1]) = 2, max([0,1]) = 1, min([0,1]) = 0
@@ -229,6 +264,27 @@ def test_softmax_on_a_view_with_offset(gpu, oracle):
     e = np.exp(x - x.max(axis=1, keepdims=True))
     np.testing.assert_allclose(out[1:5, 3:35:2].cpu().numpy(), e / e.sum(axis=1, keepdims=True), rtol=2e-5, atol=1e-7)
     assert torch.all(out[0] == 7.0) and torch.all(out[:, 4::2] == 7.0)
+
+
+@pytest.mark.parametrize("shape,perm", [((130, 67), (1, 0)), ((5, 33, 70), (2, 1, 0)), ((5, 33, 70), (1, 0, 2)),
+                                        ((3, 17, 4, 32), (0, 2, 1, 3)), ((3, 17, 4, 32), (3, 1, 2, 0)),
+                                        ((64, 200), (1, 0)), ((16, 16), (1, 0))])
+def test_copy_of_permuted_views(gpu, shape, perm):
+    """A permuted view made contiguous (what follows every transpose in the attention module): exact copies, with
+    ragged tiles, extra dimensions on either side and a destination that is itself a slice of a larger tensor."""
+    import torch
+    rng = np.random.default_rng(sum(shape))
+    x = rng.standard_normal(shape, dtype=np.float32)
+    view = col_major(x).permute(*perm)
+    want = np.transpose(x, perm)
+    out = col_major(np.zeros(want.shape, dtype=np.float32))
+    gpu.elementwise(gpu.EW_COPY, view, None, out)
+    np.testing.assert_array_equal(out.cpu().numpy(), want)
+    big = col_major(np.full((want.shape[0] + 3,) + want.shape[1:], 7.0, dtype=np.float32))
+    gpu.elementwise(gpu.EW_COPY, view, None, big[2:-1])
+    got = big.cpu().numpy()
+    np.testing.assert_array_equal(got[2:-1], want)
+    assert (got[:2] == 7.0).all() and (got[-1:] == 7.0).all()
 
 
 def test_elementwise_broadcast_and_gather(gpu):

@@ -4,7 +4,8 @@
 // Rows (all index combinations of the non-reduced dimensions) are enumerated with dimension 0 fastest, which is the
 // contiguous direction of Weed's column-major tensors; a workgroup takes RT neighbouring rows and spreads the
 // remaining threads along the reduced axis, so that loads are coalesced whether the axis is the contiguous
-// dimension (RT = 1) or a strided one (RT = 16).
+// dimension (RT = 1, float4 accesses where alignment allows) or a strided one (RT = 32 or 16).  Softmax keeps a
+// running (max, sum) per thread, so the data is read twice, or once when a contiguous row fits the registers.
 #include "common.h"
 
 #include <algorithm>
@@ -66,9 +67,9 @@ template <int OP> __device__ __forceinline__ float identity()
 }
 
 // Reduce `v` over the NY threads that share threadIdx.x % RT; the result is valid in every thread.
-template <int OP, int RT> __device__ __forceinline__ float block_reduce(float v, float *red)
+template <int OP, int RT, int THREADS> __device__ __forceinline__ float block_reduce(float v, float *red)
 {
-    constexpr int NY = kThreads / RT;
+    constexpr int NY = THREADS / RT;
     const uint32_t tx = threadIdx.x % RT, ty = threadIdx.x / RT;
     red[ty * RT + tx] = v;
     __syncthreads();
@@ -83,11 +84,38 @@ template <int OP, int RT> __device__ __forceinline__ float block_reduce(float v,
     return r;
 }
 
-template <int RT> __global__ void __launch_bounds__(kThreads) softmax_kernel(const float *__restrict__ a,
-                                                                            float *__restrict__ out, AxisGeom g)
+// Running (max, sum of exp(x - max)) of a softmax row: one exponential per element, one pass over the data.
+// -inf elements (masked positions) add nothing, also while the running maximum is still -inf.
+__device__ __forceinline__ void softmax_accumulate(float &m, float &s, float x)
 {
-    __shared__ float red[kThreads];
-    constexpr int NY = kThreads / RT;
+    if (x > m) {
+        s = s * expf(m - x) + 1.0f;
+        m = x;
+    } else if (x > -INFINITY) {
+        s += expf(x - m);
+    }
+}
+
+// Merge the per-thread (m, s) pairs of the threads that share a row; returns the row's (max, sum) in every thread.
+template <int RT, int THREADS> __device__ __forceinline__ void softmax_merge(float &m, float &s, float *red)
+{
+    const float row_max = block_reduce<1, RT, THREADS>(m, red);
+    const float scaled = (m > -INFINITY) ? s * expf(m - row_max) : 0.0f;
+    s = block_reduce<0, RT, THREADS>(scaled, red);
+    m = row_max;
+}
+
+constexpr int kAxisUnroll = 8; // independent loads in flight per thread
+
+// Softmax along any axis.  First pass: running (max, sum) with kAxisUnroll loads in flight per thread; second pass:
+// exp(x - max) / sum.  Two reads and one write per element.
+template <int RT, int THREADS> __global__ void __launch_bounds__(THREADS) softmax_kernel(const float *__restrict__ a,
+                                                                                        float *__restrict__ out,
+                                                                                        AxisGeom g)
+{
+    __shared__ float red[THREADS];
+    constexpr int NY = THREADS / RT;
+    constexpr int U = kAxisUnroll;
     const uint32_t tx = threadIdx.x % RT, ty = threadIdx.x / RT;
     const uint32_t row = blockIdx.x * RT + tx;
     const bool valid = row < g.rows;
@@ -96,32 +124,96 @@ template <int RT> __global__ void __launch_bounds__(kThreads) softmax_kernel(con
         row_bases(g, row, a_base, o_base);
     }
     const uint32_t as = g.a_stride[g.axis], os = g.o_stride[g.axis];
-    float mx = -INFINITY;
-    if (valid) {
-        for (uint32_t j = ty; j < g.axis_len; j += NY) {
-            mx = fmaxf(mx, a[a_base + (uint64_t)j * as]);
+    const uint32_t len = valid ? g.axis_len : 0U;
+    const float *ap = a + a_base;
+    float *op = out + o_base;
+    float m = -INFINITY, s = 0.0f;
+    for (uint32_t j0 = ty; j0 < len; j0 += NY * U) {
+        float x[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint32_t j = j0 + u * NY;
+            x[u] = j < len ? ap[(uint64_t)j * as] : -INFINITY;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            softmax_accumulate(m, s, x[u]);
         }
     }
-    mx = block_reduce<1, RT>(mx, red);
-    float s = 0.0f;
-    if (valid) {
-        for (uint32_t j = ty; j < g.axis_len; j += NY) {
-            s += expf(a[a_base + (uint64_t)j * as] - mx);
+    softmax_merge<RT, THREADS>(m, s, red);
+    for (uint32_t j0 = ty; j0 < len; j0 += NY * U) {
+        float x[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint32_t j = j0 + u * NY;
+            x[u] = j < len ? ap[(uint64_t)j * as] : 0.0f;
         }
-    }
-    s = block_reduce<0, RT>(s, red);
-    if (valid) {
-        for (uint32_t j = ty; j < g.axis_len; j += NY) {
-            out[o_base + (uint64_t)j * os] = expf(a[a_base + (uint64_t)j * as] - mx) / s;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint32_t j = j0 + u * NY;
+            if (j < len) {
+                op[(uint64_t)j * os] = expf(x[u] - m) / s;
+            }
         }
     }
 }
 
-template <int OP, int RT> __global__ void __launch_bounds__(kThreads) reduce_kernel(const float *__restrict__ a,
-                                                                                   float *__restrict__ out, AxisGeom g)
+// Softmax along a contiguous, 16-byte aligned axis: one workgroup per row, float4 accesses, and the first
+// CACHED * 4 * THREADS elements of the row stay in registers between the two passes (rows up to that length are
+// read once).
+template <int CACHED, int THREADS>
+__global__ void __launch_bounds__(THREADS) softmax_contiguous_kernel(const float *__restrict__ a,
+                                                                    float *__restrict__ out, AxisGeom g)
 {
-    __shared__ float red[kThreads];
-    constexpr int NY = kThreads / RT;
+    __shared__ float red[THREADS];
+    uint64_t a_base, o_base;
+    row_bases(g, blockIdx.x, a_base, o_base);
+    const float4 *ap = reinterpret_cast<const float4 *>(a + a_base);
+    float4 *op = reinterpret_cast<float4 *>(out + o_base);
+    const uint32_t n4 = g.axis_len / 4U;
+    float4 cache[CACHED];
+    float m = -INFINITY, s = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CACHED; ++c) {
+        const uint32_t idx = threadIdx.x + c * THREADS;
+        cache[c] = idx < n4 ? ap[idx] : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+    }
+#pragma unroll
+    for (int c = 0; c < CACHED; ++c) {
+        softmax_accumulate(m, s, cache[c].x);
+        softmax_accumulate(m, s, cache[c].y);
+        softmax_accumulate(m, s, cache[c].z);
+        softmax_accumulate(m, s, cache[c].w);
+    }
+    for (uint32_t idx = threadIdx.x + CACHED * THREADS; idx < n4; idx += THREADS) {
+        const float4 v = ap[idx];
+        softmax_accumulate(m, s, v.x);
+        softmax_accumulate(m, s, v.y);
+        softmax_accumulate(m, s, v.z);
+        softmax_accumulate(m, s, v.w);
+    }
+    softmax_merge<1, THREADS>(m, s, red);
+#pragma unroll
+    for (int c = 0; c < CACHED; ++c) {
+        const uint32_t idx = threadIdx.x + c * THREADS;
+        if (idx < n4) {
+            const float4 v = cache[c];
+            op[idx] = make_float4(expf(v.x - m) / s, expf(v.y - m) / s, expf(v.z - m) / s, expf(v.w - m) / s);
+        }
+    }
+    for (uint32_t idx = threadIdx.x + CACHED * THREADS; idx < n4; idx += THREADS) {
+        const float4 v = ap[idx];
+        op[idx] = make_float4(expf(v.x - m) / s, expf(v.y - m) / s, expf(v.z - m) / s, expf(v.w - m) / s);
+    }
+}
+
+template <int OP, int RT, int THREADS>
+__global__ void __launch_bounds__(THREADS) reduce_kernel(const float *__restrict__ a, float *__restrict__ out,
+                                                         AxisGeom g)
+{
+    __shared__ float red[THREADS];
+    constexpr int NY = THREADS / RT;
+    constexpr int U = kAxisUnroll;
     const uint32_t tx = threadIdx.x % RT, ty = threadIdx.x / RT;
     const uint32_t row = blockIdx.x * RT + tx;
     const bool valid = row < g.rows;
@@ -130,14 +222,53 @@ template <int OP, int RT> __global__ void __launch_bounds__(kThreads) reduce_ker
         row_bases(g, row, a_base, o_base);
     }
     const uint32_t as = g.a_stride[g.axis];
+    const uint32_t len = valid ? g.axis_len : 0U;
+    const float *ap = a + a_base;
     float v = identity<OP>();
-    if (valid) {
-        for (uint32_t j = ty; j < g.axis_len; j += NY) {
-            v = combine<OP>(v, a[a_base + (uint64_t)j * as]);
+    for (uint32_t j0 = ty; j0 < len; j0 += NY * U) {
+        float x[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint32_t j = j0 + u * NY;
+            x[u] = j < len ? ap[(uint64_t)j * as] : identity<OP>();
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            v = combine<OP>(v, x[u]);
         }
     }
-    v = block_reduce<OP, RT>(v, red);
+    v = block_reduce<OP, RT, THREADS>(v, red);
     if (valid && ty == 0) {
+        out[o_base] = v;
+    }
+}
+
+// Reduction along a contiguous, 16-byte aligned axis: one workgroup per row, four float4 loads in flight per thread.
+template <int OP, int THREADS>
+__global__ void __launch_bounds__(THREADS) reduce_contiguous_kernel(const float *__restrict__ a,
+                                                                   float *__restrict__ out, AxisGeom g)
+{
+    __shared__ float red[THREADS];
+    constexpr int U = 4;
+    uint64_t a_base, o_base;
+    row_bases(g, blockIdx.x, a_base, o_base);
+    const float4 *ap = reinterpret_cast<const float4 *>(a + a_base);
+    const uint32_t n4 = g.axis_len / 4U;
+    float v = identity<OP>();
+    for (uint32_t i0 = threadIdx.x; i0 < n4; i0 += THREADS * U) {
+        float4 x[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint32_t idx = i0 + u * THREADS;
+            x[u] = idx < n4 ? ap[idx] : make_float4(identity<OP>(), identity<OP>(), identity<OP>(), identity<OP>());
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            v = combine<OP>(v, combine<OP>(combine<OP>(x[u].x, x[u].y), combine<OP>(x[u].z, x[u].w)));
+        }
+    }
+    v = block_reduce<OP, 1, THREADS>(v, red);
+    if (threadIdx.x == 0) {
         out[o_base] = v;
     }
 }
@@ -202,6 +333,53 @@ template <int OP> __global__ void __launch_bounds__(256) elementwise_kernel(cons
             r = OP == 1 ? x + y : OP == 2 ? x - y : OP == 3 ? x * y : x / y;
         }
         out[oi] = r;
+    }
+}
+
+// Copy between layouts whose contiguous dimensions differ (a transposed view made contiguous): 64 x 64 tiles of
+// dimensions (0, k) go through LDS, read along k, where `a` is contiguous, and written along dimension 0, where `out`
+// is.  One workgroup per tile; the other dimensions are enumerated by the workgroup index, dimension order kept.
+__global__ void __launch_bounds__(256) transpose_copy_kernel(const float *__restrict__ a, float *__restrict__ out,
+                                                             PointGeom g, uint32_t k, uint32_t tiles0, uint32_t tilesk)
+{
+    __shared__ float tile[64][65];
+    uint32_t b = blockIdx.x;
+    const uint32_t t0 = b % tiles0;
+    b /= tiles0;
+    const uint32_t tk = b % tilesk;
+    uint32_t rest = b / tilesk;
+    uint64_t ai = g.a_off, oi = g.o_off;
+    for (uint32_t dd = 1; dd < g.rank; ++dd) {
+        if (dd == k) {
+            continue;
+        }
+        const uint32_t c = rest % g.shape[dd];
+        rest /= g.shape[dd];
+        ai += (uint64_t)c * g.a_stride[dd];
+        oi += (uint64_t)c * g.o_stride[dd];
+    }
+    const uint32_t lx = threadIdx.x % 64U, ly = threadIdx.x / 64U;
+    const uint32_t n0 = g.shape[0], nk = g.shape[k];
+    {
+        const uint32_t ik = tk * 64U + lx;
+#pragma unroll 4
+        for (uint32_t r = ly; r < 64U; r += 4U) {
+            const uint32_t i0 = t0 * 64U + r;
+            if (i0 < n0 && ik < nk) {
+                tile[r][lx] = a[ai + (uint64_t)i0 * g.a_stride[0] + (uint64_t)ik * g.a_stride[k]];
+            }
+        }
+    }
+    __syncthreads();
+    {
+        const uint32_t i0 = t0 * 64U + lx;
+#pragma unroll 4
+        for (uint32_t r = ly; r < 64U; r += 4U) {
+            const uint32_t ik = tk * 64U + r;
+            if (i0 < n0 && ik < nk) {
+                out[oi + (uint64_t)i0 * g.o_stride[0] + (uint64_t)ik * g.o_stride[k]] = tile[lx][r];
+            }
+        }
     }
 }
 
@@ -282,6 +460,32 @@ int make_geom(const char *fn, uint32_t rank, const uint32_t *shape, uint32_t axi
     return WEED_HIP_OK;
 }
 
+enum AxisLaunch { AXIS_CONTIGUOUS, AXIS_ROW, AXIS_ROWS32, AXIS_ROWS32_WIDE, AXIS_ROWS16 };
+
+// How a softmax or reduction spreads its threads.  A contiguous axis gets one workgroup per row (float4 accesses
+// where every row starts on a 16-byte boundary); a strided axis gets 32 neighbouring rows per workgroup (128-byte
+// segments; 256 threads when that still makes a thousand workgroups, else 1024), and 16 rows with 1024 threads when
+// rows are few and long (decode-time scores, [B * heads] rows of the context's length), so that enough loads stay
+// in flight.
+AxisLaunch choose_axis_launch(const AxisGeom &g, const float *a_dev, const float *out_dev, bool out_keeps_axis)
+{
+    const uint32_t as = g.a_stride[g.axis];
+    if (as <= 1U || g.rows < 16U) {
+        bool vec = as == 1U && g.axis_len % 4U == 0U && g.axis_len >= 256U && g.a_off % 4U == 0U &&
+            reinterpret_cast<uintptr_t>(a_dev) % 16U == 0U;
+        if (out_keeps_axis) {
+            vec = vec && g.o_stride[g.axis] == 1U && g.o_off % 4U == 0U && reinterpret_cast<uintptr_t>(out_dev) % 16U == 0U;
+        }
+        for (uint32_t i = 0; vec && i < g.rank; ++i) {
+            if (i != g.axis && g.shape[i] > 1U) {
+                vec = g.a_stride[i] % 4U == 0U && (!out_keeps_axis || g.o_stride[i] % 4U == 0U);
+            }
+        }
+        return vec ? AXIS_CONTIGUOUS : AXIS_ROW;
+    }
+    return g.rows >= 32U * 1024U ? AXIS_ROWS32 : g.rows >= 32U * 128U ? AXIS_ROWS32_WIDE : AXIS_ROWS16;
+}
+
 } // namespace
 
 extern "C" {
@@ -327,6 +531,27 @@ int weed_hip_elementwise_f32(int op, uint32_t rank, const uint32_t *shape, const
     }
     WEED_HIP_REQUIRE(g.n < (1ull << 32), "%s: more than 2^32 elements", fn);
     ProfileScope prof("elementwise");
+    if (op == WEED_HIP_EW_COPY && g.rank >= 2 && g.o_stride[0] == 1U && g.a_stride[0] > 1U && g.shape[0] >= 16U) {
+        // a transposed view: find the dimension along which `a` is contiguous
+        uint32_t k = 0;
+        for (uint32_t dd = 1; dd < g.rank && !k; ++dd) {
+            if (g.a_stride[dd] == 1U && g.shape[dd] >= 16U) {
+                k = dd;
+            }
+        }
+        const uint32_t tiles0 = (g.shape[0] + 63U) / 64U, tilesk = k ? (g.shape[k] + 63U) / 64U : 0U;
+        uint64_t tiles = (uint64_t)tiles0 * tilesk;
+        for (uint32_t dd = 1; dd < g.rank; ++dd) {
+            if (dd != k) {
+                tiles *= g.shape[dd];
+            }
+        }
+        if (k && tiles < (1ull << 31)) {
+            transpose_copy_kernel<<<(uint32_t)tiles, 256, 0, stream()>>>(a_dev, out_dev, g, k, tiles0, tilesk);
+            WEED_HIP_LAUNCH_CHECK();
+            return WEED_HIP_OK;
+        }
+    }
     const uint32_t blocks = (uint32_t)std::min<uint64_t>((g.n + 255) / 256, 256u * 64u);
     const float *b = op == WEED_HIP_EW_COPY ? a_dev : b_dev;
     switch (op) {
@@ -406,10 +631,17 @@ int weed_hip_softmax_f32(uint32_t rank, const uint32_t *shape, uint32_t axis, co
     AxisGeom g;
     WEED_HIP_TRY(make_geom(fn, rank, shape, axis, a_off, a_stride, o_off, o_stride, true, g));
     ProfileScope prof("softmax");
-    if (g.a_stride[axis] <= 1 || g.rows < 16) {
-        softmax_kernel<1><<<g.rows, kThreads, 0, stream()>>>(a_dev, out_dev, g);
+    const AxisLaunch how = choose_axis_launch(g, a_dev, out_dev, true);
+    if (how == AXIS_CONTIGUOUS) {
+        softmax_contiguous_kernel<8, 256><<<g.rows, 256, 0, stream()>>>(a_dev, out_dev, g);
+    } else if (how == AXIS_ROW) {
+        softmax_kernel<1, 256><<<g.rows, 256, 0, stream()>>>(a_dev, out_dev, g);
+    } else if (how == AXIS_ROWS32) {
+        softmax_kernel<32, 256><<<(g.rows + 31) / 32, 256, 0, stream()>>>(a_dev, out_dev, g);
+    } else if (how == AXIS_ROWS32_WIDE) {
+        softmax_kernel<32, 1024><<<(g.rows + 31) / 32, 1024, 0, stream()>>>(a_dev, out_dev, g);
     } else {
-        softmax_kernel<16><<<(g.rows + 15) / 16, kThreads, 0, stream()>>>(a_dev, out_dev, g);
+        softmax_kernel<16, 1024><<<(g.rows + 15) / 16, 1024, 0, stream()>>>(a_dev, out_dev, g);
     }
     WEED_HIP_LAUNCH_CHECK();
     return WEED_HIP_OK;
@@ -425,13 +657,18 @@ int weed_hip_reduce_f32(int op, uint32_t rank, const uint32_t *shape, uint32_t a
     AxisGeom g;
     WEED_HIP_TRY(make_geom(fn, rank, shape, axis, a_off, a_stride, o_off, o_stride, false, g));
     ProfileScope prof("reduce");
-    const bool narrow = g.a_stride[axis] <= 1 || g.rows < 16;
-    const uint32_t blocks = narrow ? g.rows : (g.rows + 15) / 16;
+    const AxisLaunch how = choose_axis_launch(g, a_dev, out_dev, false);
 #define WEED_LAUNCH_REDUCE(OP)                                                                                         \
-    if (narrow) {                                                                                                      \
-        reduce_kernel<OP, 1><<<blocks, kThreads, 0, stream()>>>(a_dev, out_dev, g);                                    \
+    if (how == AXIS_CONTIGUOUS) {                                                                                      \
+        reduce_contiguous_kernel<OP, 256><<<g.rows, 256, 0, stream()>>>(a_dev, out_dev, g);                            \
+    } else if (how == AXIS_ROW) {                                                                                      \
+        reduce_kernel<OP, 1, 256><<<g.rows, 256, 0, stream()>>>(a_dev, out_dev, g);                                    \
+    } else if (how == AXIS_ROWS32) {                                                                                   \
+        reduce_kernel<OP, 32, 256><<<(g.rows + 31) / 32, 256, 0, stream()>>>(a_dev, out_dev, g);                       \
+    } else if (how == AXIS_ROWS32_WIDE) {                                                                              \
+        reduce_kernel<OP, 32, 1024><<<(g.rows + 31) / 32, 1024, 0, stream()>>>(a_dev, out_dev, g);                     \
     } else {                                                                                                           \
-        reduce_kernel<OP, 16><<<blocks, kThreads, 0, stream()>>>(a_dev, out_dev, g);                                   \
+        reduce_kernel<OP, 16, 1024><<<(g.rows + 15) / 16, 1024, 0, stream()>>>(a_dev, out_dev, g);                     \
     }
     if (op == WEED_HIP_REDUCE_SUM) {
         WEED_LAUNCH_REDUCE(0)

@@ -73,15 +73,18 @@ struct RotGeom {
     uint32_t rows, d;
 };
 
+constexpr int kRotOutputs = 16; // outputs per thread: one pass over a row of x serves this many columns of R
+constexpr int kRotBatch = 4; // contraction steps per batch of loads
+
 // y[row, j] = sum_i x[row, i] * R[i + d*j], products added in ascending i with separate multiply and add, the order
 // of the reference's naive matmul (src/ops/matmul.cpp:40-44).  Neighbouring threads take neighbouring rows (the
-// contiguous direction of a column-major tensor) and share one column of R, so x loads coalesce and R loads are
-// wave-uniform.
+// contiguous direction of a column-major tensor) and share kRotOutputs columns of R, so x loads coalesce, R loads
+// are wave-uniform and x is read d / kRotOutputs times instead of d times.
 __global__ void __launch_bounds__(256) apply_rotation_kernel(const float *__restrict__ x, const float *__restrict__ rot,
                                                              float *__restrict__ out, RotGeom g)
 {
     const uint32_t row = blockIdx.x * 256 + threadIdx.x;
-    const uint32_t j = blockIdx.y;
+    const uint32_t j0 = blockIdx.y * kRotOutputs;
     if (row >= g.rows) {
         return;
     }
@@ -93,13 +96,48 @@ __global__ void __launch_bounds__(256) apply_rotation_kernel(const float *__rest
         xb += (uint64_t)c * g.x_stride[dd];
         ob += (uint64_t)c * g.o_stride[dd];
     }
+    const uint32_t d = g.d;
     const uint32_t xs = g.x_stride[g.rank - 1];
-    const float *col = rot + (uint64_t)j * g.d;
-    float acc = 0.0f;
-    for (uint32_t i = 0; i < g.d; ++i) {
-        acc = acc + x[xb + (uint64_t)i * xs] * col[i];
+    const float *xp = x + xb;
+    // every accumulator adds its products in the order i = 0, 1, ..., d - 1 with separately rounded products; the
+    // columns of R are addressed by workgroup-wide values, so they travel through the scalar data path
+    float acc[kRotOutputs];
+#pragma unroll
+    for (int jj = 0; jj < kRotOutputs; ++jj) {
+        acc[jj] = 0.0f;
     }
-    out[ob + (uint64_t)j * g.o_stride[g.rank - 1]] = acc;
+    uint32_t i = 0;
+    for (; i + kRotBatch <= d; i += kRotBatch) {
+        float xv[kRotBatch];
+#pragma unroll
+        for (int u = 0; u < kRotBatch; ++u) {
+            xv[u] = xp[(uint64_t)(i + u) * xs];
+        }
+#pragma unroll
+        for (int jj = 0; jj < kRotOutputs; ++jj) {
+            const uint32_t j = min(j0 + (uint32_t)jj, d - 1U);
+            const float *col = rot + (uint64_t)j * d + i;
+#pragma unroll
+            for (int u = 0; u < kRotBatch; ++u) {
+                acc[jj] = acc[jj] + xv[u] * col[u];
+            }
+        }
+    }
+    for (; i < d; ++i) {
+        const float xv = xp[(uint64_t)i * xs];
+#pragma unroll
+        for (int jj = 0; jj < kRotOutputs; ++jj) {
+            const uint32_t j = min(j0 + (uint32_t)jj, d - 1U);
+            acc[jj] = acc[jj] + xv * rot[(uint64_t)j * d + i];
+        }
+    }
+    const uint32_t os = g.o_stride[g.rank - 1];
+#pragma unroll
+    for (int jj = 0; jj < kRotOutputs; ++jj) {
+        if (j0 + jj < d) {
+            out[ob + (uint64_t)(j0 + jj) * os] = acc[jj];
+        }
+    }
 }
 
 } // namespace
@@ -161,7 +199,7 @@ int weed_hip_apply_rotation_f32(uint32_t d, const float *r_dev, uint32_t rank, c
     }
     WEED_HIP_REQUIRE(rows * d < (1ull << 32), "%s: more than 2^32 elements", fn);
     g.rows = (uint32_t)rows;
-    apply_rotation_kernel<<<dim3((g.rows + 255) / 256, d), 256, 0, stream()>>>(x_dev, r_dev, out_dev, g);
+    apply_rotation_kernel<<<dim3((g.rows + 255) / 256, (d + kRotOutputs - 1) / kRotOutputs), 256, 0, stream()>>>(x_dev, r_dev, out_dev, g);
     WEED_HIP_LAUNCH_CHECK();
     return WEED_HIP_OK;
 }
