@@ -88,6 +88,15 @@ int weed_hip_matmul_batched_f32(const uint32_t batch[2], uint32_t M, uint32_t N,
                                 const uint32_t b_bs[2], float *out_dev, uint32_t o_off, uint32_t o_s0, uint32_t o_s1,
                                 const uint32_t o_bs[2]);
 
+/* out[M,N] = a[M,K] . w[K,N] + bias[N]: Linear::forward (src/modules/linear.cpp:86-100: `x >> weight`, then
+ * `+ bias` broadcast over the rows) as one launch.  The bias (element n at bias_dev[bias_off + n*bias_stride]) is added
+ * to the rounded sum, so the result is bit-identical to weed_hip_matmul_f32 followed by the broadcast add of
+ * weed_hip_elementwise_f32; bias_dev may be null (no bias). */
+int weed_hip_linear_f32(uint32_t M, uint32_t N, uint32_t K, const float *a_dev, uint32_t a_off, uint32_t a_s0,
+                        uint32_t a_s1, const float *w_dev, uint32_t w_off, uint32_t w_s0, uint32_t w_s1,
+                        const float *bias_dev, uint32_t bias_off, uint32_t bias_stride, float *out_dev, uint32_t o_off,
+                        uint32_t o_s0, uint32_t o_s1);
+
 /* out[o_off + i*o_stride] = a[a_off + i*a_stride] for i < n.  Replaces the OpenCL kernel copy_real
  * (src/common/qengine.cl:979, launched from src/ops/copy_broadcast.cpp:66); also the plain copy used to calibrate the
  * HBM traffic counters. */

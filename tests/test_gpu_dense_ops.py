@@ -105,6 +105,60 @@ def test_matmul_decode_projections(gpu, oracle, M, N, K):
     assert torch.all(big_c[:2] == -7.0) and torch.all(big_c[2 + M:] == -7.0) and torch.all(big_c[:, 0::2] == -7.0)
 
 
+@pytest.mark.parametrize("M,N,K", [(200, 300, 4096), (128, 128, 2048), (130, 70, 1030), (17, 17, 8), (257, 129, 33),
+                                   (1000, 1000, 100)])
+def test_matmul_matrix_core_edges(gpu, M, N, K):
+    """Shapes that are not multiples of the 128 x 128 x 16 tiles, unaligned and doubly strided views, and few tiles with
+    a long k (split over workgroups, summed by a second kernel): against float64, and nothing outside the output view
+    may be written."""
+    import torch
+    rng = np.random.default_rng(M + 2 * N + 3 * K)
+    A = rng.standard_normal((M, K), dtype=np.float32)
+    B = rng.standard_normal((K, N), dtype=np.float32)
+    want = A.astype(np.float64) @ B.astype(np.float64)
+    tol = dict(rtol=2e-5, atol=4e-6 * np.sqrt(K) * 3)
+    for mk_a, mk_b in ((col_major, col_major), (dev, dev), (col_major, dev), (dev, col_major)):
+        C = col_major(np.zeros((M, N), dtype=np.float32))
+        gpu.matmul(mk_a(A), mk_b(B), C)
+        np.testing.assert_allclose(C.cpu().numpy(), want, **tol)
+    # views strided in both dimensions, with odd offsets; the output is a padded slice
+    big_a = torch.zeros((2 * M + 1, 3 * K + 1), device="cuda")
+    big_a[1::2, 1::3] = dev(A)
+    big_b = torch.zeros((2 * K + 3, 2 * N + 1), device="cuda")
+    big_b[3::2, 1::2] = dev(B)
+    big_c = torch.full((M + 3, N + 5), -7.0, device="cuda")
+    gpu.matmul(big_a[1::2, 1::3], big_b[3::2, 1::2], big_c[1:1 + M, 2:2 + N])
+    got = big_c.cpu().numpy()
+    np.testing.assert_allclose(got[1:1 + M, 2:2 + N], want, **tol)
+    inner = np.zeros_like(got, dtype=bool)
+    inner[1:1 + M, 2:2 + N] = True
+    assert (got[~inner] == -7.0).all()
+
+
+@pytest.mark.parametrize("M,N,K", [(3, 5, 7), (8, 4096, 1024), (16, 100, 260), (40, 640, 1024), (64, 250, 516),
+                                   (128, 256, 64), (70, 33, 19)])
+def test_linear_equals_product_then_broadcast_add(gpu, M, N, K):
+    """The bias added in the product's last step gives the bits of the two separate ops of Linear::forward
+    (matmul, then the broadcast add), on every product kernel (generic, matrix-core tiles, both streaming kernels);
+    the bias may be a strided view, and a null bias gives the plain product."""
+    import torch
+    rng = np.random.default_rng(M + 3 * N + 7 * K)
+    A = col_major(rng.standard_normal((M, K), dtype=np.float32))
+    W = col_major(rng.standard_normal((K, N), dtype=np.float32) * 0.05)
+    bias_store = dev(rng.standard_normal(2 * N + 1, dtype=np.float32))
+    bias = bias_store[1:1 + 2 * N:2]
+    plain = col_major(np.zeros((M, N), dtype=np.float32))
+    gpu.matmul(A, W, plain)
+    want = col_major(np.zeros((M, N), dtype=np.float32))
+    gpu.elementwise(gpu.EW_ADD, plain, bias.reshape(1, N), want)
+    got = col_major(np.full((M, N), 9.0, dtype=np.float32))
+    gpu.linear(A, W, bias, got)
+    assert torch.equal(got, want)
+    assert torch.equal(want, plain + bias.reshape(1, N))
+    gpu.linear(A, W, None, got)
+    assert torch.equal(got, plain)
+
+
 @pytest.mark.parametrize("M,N,K", [(7, 5, 11), (64, 300, 128), (128, 256, 64), (4, 32, 512)])
 def test_matmul_batched_equals_the_loop(gpu, M, N, K):
     """(batch x heads) products in one launch give what the 2-D entry point gives product by product (bit for bit:
@@ -207,10 +261,12 @@ def test_softmax_and_reduce_strided_against_checker(gpu, oracle, shape):
                     np.testing.assert_array_equal(r.cpu().numpy(), ref.astype(np.float32))
 
 
-@pytest.mark.parametrize("shape,axis", [((9004, 40), 0), ((40000, 24), 1), ((64, 8, 1, 700), 3), ((260, 3, 5), 0)])
+@pytest.mark.parametrize("shape,axis", [((9004, 40), 0), ((40000, 24), 1), ((64, 8, 1, 700), 3), ((260, 3, 5), 0),
+                                        ((192, 1100), 0), ((2044, 1030), 0), ((67, 1500), 0), ((1101, 1200), 0)])
 def test_softmax_and_reduce_launch_shapes(gpu, shape, axis):
     """One case per way the threads are spread: a contiguous row longer than what the registers keep between the
-    passes, enough rows for 32 per workgroup, few long strided rows (decode-time scores), a short aligned row.
+    passes, enough rows for 32 per workgroup, few long strided rows (decode-time scores), a short aligned row, and
+    many short contiguous rows (one wavefront each: aligned, longer than a wavefront's registers, unaligned lengths).
     Some positions are masked with -inf, one row of the decode case entirely (its softmax is NaN, as in numpy)."""
     import torch
     rng = np.random.default_rng(shape[0] + axis)

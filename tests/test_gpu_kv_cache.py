@@ -241,19 +241,28 @@ def test_argument_errors_are_reported_not_faulted(gpu):
     cache.close()
 
 
-def test_apply_rotation_reference_order(gpu, oracle):
+@pytest.mark.parametrize("shape", [(3, 2, 5, 64), (7, 19, 128), (70, 20), (5, 3, 130), (130, 1, 2, 32)])
+def test_apply_rotation_reference_order(gpu, oracle, shape):
     """y = x.R over the last dimension of a strided tensor, in the reference's summation order: bit-exact against the
-    checker's naive loop."""
+    checker's naive loop, for column-major and row-major operands in every combination (the kernel walks each side
+    along its contiguous direction), ragged row tiles, widths that are not multiples of the column chunks, a width
+    beyond the LDS-tiled kernel, and an output that is a slice of a larger tensor."""
     import torch
-    rng = np.random.default_rng(77)
-    d = 64
+    rng = np.random.default_rng(77 + len(shape))
+    d = shape[-1]
     R = oracle.orthonormalize_columns(rng.normal(size=d * d).astype(np.float32))
-    x = rng.standard_normal((3, 2, 5, d), dtype=np.float32)
-    xd = col_major(x)
-    out = torch.zeros_like(xd)
-    gpu.apply_rotation(xd, dev(R), out)
+    x = rng.standard_normal(shape, dtype=np.float32)
     want = oracle.apply_rotation(x.reshape(-1, d), R).reshape(x.shape)
-    np.testing.assert_array_equal(out.cpu().numpy(), want)
+    for mk_x in (col_major, dev):
+        for mk_o in (col_major, dev):
+            out = mk_o(np.zeros(shape, dtype=np.float32))
+            gpu.apply_rotation(mk_x(x), dev(R), out)
+            np.testing.assert_array_equal(out.cpu().numpy(), want)
+    big = torch.full((shape[0] + 2,) + tuple(shape[1:-1]) + (d + 3,), 5.0, device="cuda")
+    gpu.apply_rotation(col_major(x), dev(R), big[1:-1, ..., 2:2 + d])
+    got = big.cpu().numpy()
+    np.testing.assert_array_equal(got[1:-1, ..., 2:2 + d], want)
+    assert (got[0] == 5.0).all() and (got[-1] == 5.0).all() and (got[..., :2] == 5.0).all() and (got[..., 2 + d:] == 5.0).all()
 
 
 def test_cfg5a_encode_full_size(gpu, oracle):

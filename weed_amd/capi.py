@@ -55,6 +55,9 @@ SIGNATURES = {
     "weed_hip_matmul_batched_f32": (c_int, [U32P, c_uint32, c_uint32, c_uint32, c_void_p, c_uint32, c_uint32, c_uint32,
                                             U32P, c_void_p, c_uint32, c_uint32, c_uint32, U32P, c_void_p, c_uint32,
                                             c_uint32, c_uint32, U32P]),
+    "weed_hip_linear_f32": (c_int, [c_uint32, c_uint32, c_uint32, c_void_p, c_uint32, c_uint32, c_uint32, c_void_p,
+                                    c_uint32, c_uint32, c_uint32, c_void_p, c_uint32, c_uint32, c_void_p, c_uint32,
+                                    c_uint32, c_uint32]),
     "weed_hip_copy_f32": (c_int, [c_uint64, c_void_p, c_uint32, c_uint32, c_void_p, c_uint32, c_uint32]),
     "weed_hip_elementwise_f32": (c_int, [c_int, c_uint32, U32P, c_void_p, c_uint32, U32P, c_void_p, c_uint32, U32P,
                                          c_void_p, c_uint32, U32P]),
@@ -252,6 +255,18 @@ def matmul_batched(a, b, out):
         u32([B0, B1]), M, N, K, c_void_p(a.data_ptr()), 0, a.stride(2), a.stride(3), u32([a.stride(0), a.stride(1)]),
         c_void_p(b.data_ptr()), 0, b.stride(2), b.stride(3), u32([b.stride(0), b.stride(1)]),
         c_void_p(out.data_ptr()), 0, out.stride(2), out.stride(3), u32([out.stride(0), out.stride(1)])))
+
+
+def linear(a, w, bias, out):
+    """2-D torch views: out = a @ w + bias (bias: 1-D view of length N, or None), one launch."""
+    M, K = a.shape
+    K2, N = w.shape
+    assert K == K2 and tuple(out.shape) == (M, N) and (bias is None or tuple(bias.shape) == (N,))
+    check(load().weed_hip_linear_f32(M, N, K, c_void_p(a.data_ptr()), 0, a.stride(0), a.stride(1),
+                                     c_void_p(w.data_ptr()), 0, w.stride(0), w.stride(1),
+                                     c_void_p(bias.data_ptr()) if bias is not None else None, 0,
+                                     bias.stride(0) if bias is not None else 0, c_void_p(out.data_ptr()), 0,
+                                     out.stride(0), out.stride(1)))
 
 
 def copy(a, out):

@@ -207,6 +207,112 @@ __global__ void __launch_bounds__(THREADS) softmax_contiguous_kernel(const float
     }
 }
 
+template <int OP> __device__ __forceinline__ float wave_reduce(float v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        v = combine<OP>(v, __shfl_xor(v, off, 64));
+    }
+    return v;
+}
+
+// Short contiguous rows (a causal prefill's scores: [B * heads * T] rows of at most a few thousand key positions):
+// one WAVEFRONT per row, four rows per workgroup, so no lane idles on a 64..2048-element row and nothing goes
+// through LDS.  V = 4: float4 accesses (every row 16-byte aligned, length a multiple of 4), V = 1: scalar.  The first
+// CACHED * 64 * V elements of a row stay in registers between the two passes.
+template <int V, int CACHED>
+__global__ void __launch_bounds__(256) softmax_wave_rows_kernel(const float *__restrict__ a, float *__restrict__ out,
+                                                                AxisGeom g)
+{
+    const uint32_t lane = threadIdx.x & 63U;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t nvec = g.axis_len / V;
+    for (uint32_t row = blockIdx.x * 4U + wave; row < g.rows; row += gridDim.x * 4U) {
+        uint64_t a_base, o_base;
+        row_bases(g, row, a_base, o_base);
+        const float *ap = a + a_base;
+        float *op = out + o_base;
+        float cache[CACHED][V];
+        float m = -INFINITY, s = 0.0f;
+#pragma unroll
+        for (int c = 0; c < CACHED; ++c) {
+            const uint32_t idx = lane + 64U * c;
+            if (V == 4) {
+                const float4 v = idx < nvec ? reinterpret_cast<const float4 *>(ap)[idx]
+                                            : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+                cache[c][0] = v.x;
+                cache[c][V > 1 ? 1 : 0] = v.y;
+                cache[c][V > 2 ? 2 : 0] = v.z;
+                cache[c][V > 3 ? 3 : 0] = v.w;
+            } else {
+                cache[c][0] = idx < nvec ? ap[idx] : -INFINITY;
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < CACHED; ++c) {
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                softmax_accumulate(m, s, cache[c][e]);
+            }
+        }
+        for (uint32_t idx = lane + 64U * CACHED; idx < nvec; idx += 64U) {
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                softmax_accumulate(m, s, ap[(uint64_t)idx * V + e]);
+            }
+        }
+        const float row_max = wave_reduce<1>(m);
+        const float total = wave_reduce<0>((m > -INFINITY) ? s * expf(m - row_max) : 0.0f);
+#pragma unroll
+        for (int c = 0; c < CACHED; ++c) {
+            const uint32_t idx = lane + 64U * c;
+            if (idx < nvec) {
+                if (V == 4) {
+                    reinterpret_cast<float4 *>(op)[idx] =
+                        make_float4(expf(cache[c][0] - row_max) / total, expf(cache[c][V > 1 ? 1 : 0] - row_max) / total,
+                                    expf(cache[c][V > 2 ? 2 : 0] - row_max) / total,
+                                    expf(cache[c][V > 3 ? 3 : 0] - row_max) / total);
+                } else {
+                    op[idx] = expf(cache[c][0] - row_max) / total;
+                }
+            }
+        }
+        for (uint32_t idx = lane + 64U * CACHED; idx < nvec; idx += 64U) {
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                op[(uint64_t)idx * V + e] = expf(ap[(uint64_t)idx * V + e] - row_max) / total;
+            }
+        }
+    }
+}
+
+template <int OP, int V>
+__global__ void __launch_bounds__(256) reduce_wave_rows_kernel(const float *__restrict__ a, float *__restrict__ out,
+                                                               AxisGeom g)
+{
+    const uint32_t lane = threadIdx.x & 63U;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t nvec = g.axis_len / V;
+    for (uint32_t row = blockIdx.x * 4U + wave; row < g.rows; row += gridDim.x * 4U) {
+        uint64_t a_base, o_base;
+        row_bases(g, row, a_base, o_base);
+        const float *ap = a + a_base;
+        float v = identity<OP>();
+        for (uint32_t idx = lane; idx < nvec; idx += 64U) {
+            if (V == 4) {
+                const float4 x = reinterpret_cast<const float4 *>(ap)[idx];
+                v = combine<OP>(v, combine<OP>(combine<OP>(x.x, x.y), combine<OP>(x.z, x.w)));
+            } else {
+                v = combine<OP>(v, ap[idx]);
+            }
+        }
+        v = wave_reduce<OP>(v);
+        if (lane == 0U) {
+            out[o_base] = v;
+        }
+    }
+}
+
 template <int OP, int RT, int THREADS>
 __global__ void __launch_bounds__(THREADS) reduce_kernel(const float *__restrict__ a, float *__restrict__ out,
                                                          AxisGeom g)
@@ -293,7 +399,8 @@ struct PointGeom {
     uint64_t n;
 };
 
-// One thread per logical element, dimension 0 fastest (the contiguous direction of column-major tensors).
+// One thread per logical element, dimension 0 fastest (the host orders the dimensions so that this is the direction
+// in which the output is most contiguous).
 template <int OP> __global__ void __launch_bounds__(256) elementwise_kernel(const float *__restrict__ a,
                                                                             const float *__restrict__ b, float *out,
                                                                             PointGeom g)
@@ -460,10 +567,12 @@ int make_geom(const char *fn, uint32_t rank, const uint32_t *shape, uint32_t axi
     return WEED_HIP_OK;
 }
 
-enum AxisLaunch { AXIS_CONTIGUOUS, AXIS_ROW, AXIS_ROWS32, AXIS_ROWS32_WIDE, AXIS_ROWS16 };
+enum AxisLaunch { AXIS_CONTIGUOUS, AXIS_ROW, AXIS_WAVE_VEC, AXIS_WAVE, AXIS_ROWS32, AXIS_ROWS32_WIDE, AXIS_ROWS16 };
+constexpr uint32_t kWaveRowMax = 2048; // longest contiguous row that one wavefront takes
 
-// How a softmax or reduction spreads its threads.  A contiguous axis gets one workgroup per row (float4 accesses
-// where every row starts on a 16-byte boundary); a strided axis gets 32 neighbouring rows per workgroup (128-byte
+// How a softmax or reduction spreads its threads.  A contiguous axis gets one workgroup per row, or one wavefront
+// per row when there are many rows of at most kWaveRowMax elements (float4 accesses where every row starts on a
+// 16-byte boundary); a strided axis gets 32 neighbouring rows per workgroup (128-byte
 // segments; 256 threads when that still makes a thousand workgroups, else 1024), and 16 rows with 1024 threads when
 // rows are few and long (decode-time scores, [B * heads] rows of the context's length), so that enough loads stay
 // in flight.
@@ -471,7 +580,7 @@ AxisLaunch choose_axis_launch(const AxisGeom &g, const float *a_dev, const float
 {
     const uint32_t as = g.a_stride[g.axis];
     if (as <= 1U || g.rows < 16U) {
-        bool vec = as == 1U && g.axis_len % 4U == 0U && g.axis_len >= 256U && g.a_off % 4U == 0U &&
+        bool vec = as == 1U && g.axis_len % 4U == 0U && g.a_off % 4U == 0U &&
             reinterpret_cast<uintptr_t>(a_dev) % 16U == 0U;
         if (out_keeps_axis) {
             vec = vec && g.o_stride[g.axis] == 1U && g.o_off % 4U == 0U && reinterpret_cast<uintptr_t>(out_dev) % 16U == 0U;
@@ -481,10 +590,17 @@ AxisLaunch choose_axis_launch(const AxisGeom &g, const float *a_dev, const float
                 vec = g.a_stride[i] % 4U == 0U && (!out_keeps_axis || g.o_stride[i] % 4U == 0U);
             }
         }
-        return vec ? AXIS_CONTIGUOUS : AXIS_ROW;
+        const bool unit_strides = as == 1U && (!out_keeps_axis || g.o_stride[g.axis] == 1U);
+        if (unit_strides && g.axis_len <= kWaveRowMax && g.rows >= 1024U) {
+            return vec ? AXIS_WAVE_VEC : AXIS_WAVE;
+        }
+        return (vec && g.axis_len >= 256U) ? AXIS_CONTIGUOUS : AXIS_ROW;
     }
     return g.rows >= 32U * 1024U ? AXIS_ROWS32 : g.rows >= 32U * 128U ? AXIS_ROWS32_WIDE : AXIS_ROWS16;
 }
+
+// Four rows per workgroup; beyond 16 workgroups per compute unit the wavefronts loop over rows.
+uint32_t wave_row_blocks(uint32_t rows) { return std::min<uint32_t>((rows + 3U) / 4U, 256U * 16U); }
 
 } // namespace
 
@@ -530,6 +646,22 @@ int weed_hip_elementwise_f32(int op, uint32_t rank, const uint32_t *shape, const
         g.n *= shape[i];
     }
     WEED_HIP_REQUIRE(g.n < (1ull << 32), "%s: more than 2^32 elements", fn);
+    // The order in which the dimensions are enumerated does not change an elementwise result, so they are walked in
+    // rising order of the output's strides (size-1 dimensions last): neighbouring threads then write neighbouring
+    // addresses whatever the layout (column-major, row-major views, permuted outputs).
+    for (uint32_t i = 1; i < rank; ++i) {
+        for (uint32_t j = i; j > 0; --j) {
+            const bool prev_last = g.shape[j - 1] == 1U, cur_last = g.shape[j] == 1U;
+            const bool swap = prev_last != cur_last ? prev_last : (!cur_last && g.o_stride[j] < g.o_stride[j - 1]);
+            if (!swap) {
+                break;
+            }
+            std::swap(g.shape[j], g.shape[j - 1]);
+            std::swap(g.a_stride[j], g.a_stride[j - 1]);
+            std::swap(g.b_stride[j], g.b_stride[j - 1]);
+            std::swap(g.o_stride[j], g.o_stride[j - 1]);
+        }
+    }
     ProfileScope prof("elementwise");
     if (op == WEED_HIP_EW_COPY && g.rank >= 2 && g.o_stride[0] == 1U && g.a_stride[0] > 1U && g.shape[0] >= 16U) {
         // a transposed view: find the dimension along which `a` is contiguous
@@ -634,6 +766,10 @@ int weed_hip_softmax_f32(uint32_t rank, const uint32_t *shape, uint32_t axis, co
     const AxisLaunch how = choose_axis_launch(g, a_dev, out_dev, true);
     if (how == AXIS_CONTIGUOUS) {
         softmax_contiguous_kernel<8, 256><<<g.rows, 256, 0, stream()>>>(a_dev, out_dev, g);
+    } else if (how == AXIS_WAVE_VEC) {
+        softmax_wave_rows_kernel<4, 8><<<wave_row_blocks(g.rows), 256, 0, stream()>>>(a_dev, out_dev, g);
+    } else if (how == AXIS_WAVE) {
+        softmax_wave_rows_kernel<1, 16><<<wave_row_blocks(g.rows), 256, 0, stream()>>>(a_dev, out_dev, g);
     } else if (how == AXIS_ROW) {
         softmax_kernel<1, 256><<<g.rows, 256, 0, stream()>>>(a_dev, out_dev, g);
     } else if (how == AXIS_ROWS32) {
@@ -661,6 +797,10 @@ int weed_hip_reduce_f32(int op, uint32_t rank, const uint32_t *shape, uint32_t a
 #define WEED_LAUNCH_REDUCE(OP)                                                                                         \
     if (how == AXIS_CONTIGUOUS) {                                                                                      \
         reduce_contiguous_kernel<OP, 256><<<g.rows, 256, 0, stream()>>>(a_dev, out_dev, g);                            \
+    } else if (how == AXIS_WAVE_VEC) {                                                                                 \
+        reduce_wave_rows_kernel<OP, 4><<<wave_row_blocks(g.rows), 256, 0, stream()>>>(a_dev, out_dev, g);              \
+    } else if (how == AXIS_WAVE) {                                                                                     \
+        reduce_wave_rows_kernel<OP, 1><<<wave_row_blocks(g.rows), 256, 0, stream()>>>(a_dev, out_dev, g);              \
     } else if (how == AXIS_ROW) {                                                                                      \
         reduce_kernel<OP, 1, 256><<<g.rows, 256, 0, stream()>>>(a_dev, out_dev, g);                                    \
     } else if (how == AXIS_ROWS32) {                                                                                   \

@@ -17,7 +17,16 @@ struct MatGeom {
     // batched products: grid.z = nb0 * nb1 independent products, product (c0, c1) starts at off + c0*bs[0] + c1*bs[1]
     uint32_t nb0;
     uint32_t a_bs[2], b_bs[2], o_bs[2];
+    // optional row vector added to every row of the product after the sum is rounded (null: none), so the result
+    // equals a product followed by a broadcast add, bit for bit
+    const float *bias;
+    uint32_t bias_off, bias_s;
 };
+
+__device__ __forceinline__ float with_bias(const MatGeom &g, float v, uint32_t col)
+{
+    return g.bias ? v + g.bias[(uint64_t)g.bias_off + (uint64_t)col * g.bias_s] : v;
+}
 
 // The geometry of the product this workgroup belongs to (blockIdx.z selects it).
 __device__ __forceinline__ MatGeom batch_geom(MatGeom g)
@@ -84,7 +93,7 @@ __global__ void __launch_bounds__(256) matmul_tiled_kernel(const float *__restri
         for (int c = 0; c < 4; ++c) {
             const uint32_t i = m0 + ty * 4 + r, j = n0 + tx * 4 + c;
             if (i < g.M && j < g.N) {
-                out[(uint64_t)g.o_off + (uint64_t)i * g.o_s0 + (uint64_t)j * g.o_s1] = acc[r][c];
+                out[(uint64_t)g.o_off + (uint64_t)i * g.o_s0 + (uint64_t)j * g.o_s1] = with_bias(g, acc[r][c], j);
             }
         }
     }
@@ -96,19 +105,28 @@ __global__ void __launch_bounds__(256) matmul_tiled_kernel(const float *__restri
 //   K is walked in slices of 16 staged through double-buffered LDS ([k][i] and [k][j], so a half-wavefront reads 32
 //   consecutive floats); the next slice is fetched from HBM into registers while the current one is multiplied.
 // Each operand must be contiguous along one of its two dimensions (Weed's column-major tensors and their transposes
-// are); the four combinations are template instances.  Shapes that are not multiples of the tile, and operands
-// strided in both dimensions, use the generic kernel above.
+// are); the four combinations are template instances.  Shapes that are not multiples of the tile, operands strided
+// in both dimensions and unaligned views use the EDGE instances: the same tiles and instructions, with element-wise
+// guarded loads (zeros beyond the edges) and guarded stores; there the two flags only choose which way the threads
+// walk an operand.  Products with fewer than 17 rows or columns use the generic kernel above.
 // ------------------------------------------------------------------------------------------------
 typedef float float16v __attribute__((ext_vector_type(16)));
 typedef float float4v __attribute__((ext_vector_type(4)));
 
 constexpr int TM = 128, TN = 128, TK = 16, PITCH = 132;
 
-template <bool A_ICONTIG, bool B_KCONTIG>
+template <bool A_ICONTIG, bool B_KCONTIG, bool EDGE = false>
 __global__ void __launch_bounds__(256) matmul_mfma_kernel(const float *__restrict__ a, const float *__restrict__ b,
-                                                          float *__restrict__ out, MatGeom g_launch)
+                                                          float *__restrict__ out, MatGeom g_launch,
+                                                          uint32_t k_per_split = 0)
 {
-    const MatGeom g = batch_geom(g_launch);
+    // EDGE instances may split k over blockIdx.z (unbatched products only, so batch_geom adds nothing then):
+    // k_per_split != 0 means `out` is the dense scratch part[split][row][column] and a second kernel adds the splits
+    MatGeom g = batch_geom(g_launch);
+    const uint32_t k_first = (EDGE && k_per_split) ? blockIdx.z * k_per_split : 0U;
+    if (EDGE && k_per_split) {
+        g.K = min(g.K, k_first + k_per_split);
+    }
     __shared__ __attribute__((aligned(16))) float As[2][TK][PITCH];
     __shared__ __attribute__((aligned(16))) float Bs[2][TK][PITCH];
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -134,6 +152,23 @@ __global__ void __launch_bounds__(256) matmul_mfma_kernel(const float *__restric
 #pragma unroll
         for (int q = 0; q < 2; ++q) {
             const uint32_t idx = tid + 256 * q;
+            if (EDGE) {
+                // any shape, any strides: element-wise loads, zeros beyond the edges (they add nothing to the sums)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const uint32_t ai = A_ICONTIG ? m0 + 4 * (idx & 31) + e : m0 + (idx >> 2);
+                    const uint32_t ak = A_ICONTIG ? k0 + (idx >> 5) : k0 + 4 * (idx & 3) + e;
+                    ra[q][e] = (ai < g.M && ak < g.K)
+                        ? a[(uint64_t)g.a_off + (uint64_t)ai * g.a_s0 + (uint64_t)ak * g.a_s1]
+                        : 0.0f;
+                    const uint32_t bj = B_KCONTIG ? n0 + (idx >> 2) : n0 + 4 * (idx & 31) + e;
+                    const uint32_t bk = B_KCONTIG ? k0 + 4 * (idx & 3) + e : k0 + (idx >> 5);
+                    rb[q][e] = (bj < g.N && bk < g.K)
+                        ? b[(uint64_t)g.b_off + (uint64_t)bk * g.b_s0 + (uint64_t)bj * g.b_s1]
+                        : 0.0f;
+                }
+                continue;
+            }
             if (A_ICONTIG) {
                 const uint32_t i4 = idx & 31, k = idx >> 5;
                 ra[q] = *reinterpret_cast<const float4v *>(a + (uint64_t)g.a_off + (m0 + 4 * i4) +
@@ -181,14 +216,14 @@ __global__ void __launch_bounds__(256) matmul_mfma_kernel(const float *__restric
         }
     };
 
-    const uint32_t n_slices = g.K / TK;
-    fetch(0);
+    const uint32_t n_slices = (g.K - k_first + TK - 1) / TK;
+    fetch(k_first);
     stage(0);
     __syncthreads();
     for (uint32_t kt = 0; kt < n_slices; ++kt) {
         const int buf = kt & 1;
         if (kt + 1 < n_slices) {
-            fetch((kt + 1) * TK);
+            fetch(k_first + (kt + 1) * TK);
         }
 #pragma unroll
         for (int kk = 0; kk < TK; kk += 2) {
@@ -217,13 +252,32 @@ __global__ void __launch_bounds__(256) matmul_mfma_kernel(const float *__restric
             for (int r4 = 0; r4 < 4; ++r4) {
                 const uint32_t row = m0 + 64 * wi + 32 * x + 8 * r4 + 4 * lk;
                 float *dst = out + (uint64_t)g.o_off + (uint64_t)row * g.o_s0 + (uint64_t)col * g.o_s1;
-                if (g.o_s0 == 1) {
-                    *reinterpret_cast<float4v *>(dst) =
-                        float4v{ acc[x][y][4 * r4], acc[x][y][4 * r4 + 1], acc[x][y][4 * r4 + 2], acc[x][y][4 * r4 + 3] };
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    v[e] = (!EDGE || col < g.N) ? with_bias(g, acc[x][y][4 * r4 + e], col) : 0.0f;
+                }
+                if (EDGE && k_per_split) {
+                    float *part = out + ((uint64_t)blockIdx.z * g.M + row) * g.N + col;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if (row + e < g.M && col < g.N) {
+                            part[(uint64_t)e * g.N] = acc[x][y][4 * r4 + e];
+                        }
+                    }
+                } else if (EDGE) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if (row + e < g.M && col < g.N) {
+                            dst[(uint64_t)e * g.o_s0] = v[e];
+                        }
+                    }
+                } else if (g.o_s0 == 1) {
+                    *reinterpret_cast<float4v *>(dst) = float4v{ v[0], v[1], v[2], v[3] };
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        dst[(uint64_t)e * g.o_s0] = acc[x][y][4 * r4 + e];
+                        dst[(uint64_t)e * g.o_s0] = v[e];
                     }
                 }
             }
@@ -367,7 +421,7 @@ __global__ void __launch_bounds__(64 * kSkinnyWaves)
         }
         const uint32_t m = 16 * mt + r, nn = blockIdx.x * 16 + cc;
         if (m < g.M && nn < g.N) {
-            out[(uint64_t)g.o_off + (uint64_t)m * g.o_s0 + (uint64_t)nn * g.o_s1] = sum;
+            out[(uint64_t)g.o_off + (uint64_t)m * g.o_s0 + (uint64_t)nn * g.o_s1] = with_bias(g, sum, nn);
         }
     }
 }
@@ -482,12 +536,27 @@ __global__ void __launch_bounds__(256) matmul_split_sum_kernel(const float *__re
     for (uint32_t s = 0; s < splits; ++s) {
         sum += src[(uint64_t)s * g.M * g.N];
     }
-    out[(uint64_t)g.o_off + (uint64_t)m * g.o_s0 + (uint64_t)n * g.o_s1] = sum;
+    out[(uint64_t)g.o_off + (uint64_t)m * g.o_s0 + (uint64_t)n * g.o_s1] = with_bias(g, sum, n);
 }
 
 // Scratch for the partial results of split products: grows as needed, kept for the life of the process.
 float *g_split_ws = nullptr;
 size_t g_split_ws_bytes = 0;
+
+int grow_split_scratch(const char *fn, size_t need)
+{
+    if (need > g_split_ws_bytes) {
+        WEED_HIP_CHECK(hipStreamSynchronize(stream()));
+        (void)hipFree(g_split_ws);
+        g_split_ws = nullptr;
+        g_split_ws_bytes = 0;
+        if (hipMalloc((void **)&g_split_ws, need) != hipSuccess) {
+            return fail(WEED_HIP_ENOMEM, "%s: scratch allocation of %zu bytes failed", fn, need);
+        }
+        g_split_ws_bytes = need;
+    }
+    return WEED_HIP_OK;
+}
 
 // Few rows, columns of b contiguous along k and 16-byte aligned, enough k to be worth streaming.
 bool skinny_eligible(const MatGeom &g, const float *b)
@@ -537,7 +606,10 @@ int launch_matmul(const char *fn, const MatGeom &g, uint32_t batch, const float 
     WEED_HIP_REQUIRE(batch <= 65535u, "%s: %u products in one call (at most 65535)", fn, batch);
     const uint32_t M = g.M, N = g.N, K = g.K;
     ProfileScope prof("matmul");
-    if (mfma_eligible(g, a_dev, b_dev, out_dev)) {
+    // few output tiles and a long k: the tiles' k ranges are split over more workgroups (guarded instances below)
+    const uint64_t out_tiles = (uint64_t)((M + TM - 1) / TM) * ((N + TN - 1) / TN) * batch;
+    const bool split_k = batch == 1 && M > 16 && N > 16 && out_tiles < 128 && K >= 1024;
+    if (!split_k && mfma_eligible(g, a_dev, b_dev, out_dev)) {
         const dim3 grid(M / TM, N / TN, batch);
         WEED_HIP_REQUIRE(grid.y <= 65535u, "%s: N = %u too large", fn, N);
         const bool a_i = g.a_s0 == 1, b_k = g.b_s0 == 1;
@@ -553,7 +625,7 @@ int launch_matmul(const char *fn, const MatGeom &g, uint32_t batch, const float 
         WEED_HIP_LAUNCH_CHECK();
         return WEED_HIP_OK;
     }
-    if (skinny_eligible(g, b_dev)) {
+    if (skinny_eligible(g, b_dev)) { // (few rows: this streaming kernel splits k by itself)
         // every wavefront of a workgroup takes a whole number of 64-k iterations
         const uint32_t k_per_wave = ((K + kSkinnyWaves - 1) / kSkinnyWaves + 63) / 64 * 64;
         const dim3 wgs((N + 15) / 16, 1, batch);
@@ -564,16 +636,7 @@ int launch_matmul(const char *fn, const MatGeom &g, uint32_t batch, const float 
             const uint32_t k_per_split = ((K + splits - 1) / splits + 63) / 64 * 64;
             splits = (K + k_per_split - 1) / k_per_split;
             const size_t need = sizeof(float) * (size_t)batch * splits * M * N;
-            if (need > g_split_ws_bytes) {
-                WEED_HIP_CHECK(hipStreamSynchronize(stream()));
-                (void)hipFree(g_split_ws);
-                g_split_ws = nullptr;
-                g_split_ws_bytes = 0;
-                if (hipMalloc((void **)&g_split_ws, need) != hipSuccess) {
-                    return fail(WEED_HIP_ENOMEM, "%s: scratch allocation of %zu bytes failed", fn, need);
-                }
-                g_split_ws_bytes = need;
-            }
+            WEED_HIP_TRY(grow_split_scratch(fn, need));
             const dim3 wide(col_wgs, splits, batch);
             if (M <= 32) {
                 matmul_skinny_wide_kernel<2><<<wide, 64 * kWideWaves, 0, stream()>>>(a_dev, b_dev, g_split_ws, g,
@@ -598,6 +661,41 @@ int launch_matmul(const char *fn, const MatGeom &g, uint32_t batch, const float 
         WEED_HIP_LAUNCH_CHECK();
         return WEED_HIP_OK;
     }
+    if (M > 16 && N > 16 && K >= 8) {
+        // ragged, unaligned or doubly strided: matrix-core tiles with guarded loads and stores
+        uint32_t splits = 1, k_per_split = 0;
+        if (split_k) {
+            splits = std::min<uint32_t>((uint32_t)(256 / out_tiles), K / 256);
+            k_per_split = ((K + splits - 1) / splits + TK - 1) / TK * TK;
+            splits = (K + k_per_split - 1) / k_per_split;
+            if (splits < 2) {
+                k_per_split = 0;
+            }
+        }
+        float *dst = out_dev;
+        if (k_per_split) {
+            WEED_HIP_TRY(grow_split_scratch(fn, sizeof(float) * (size_t)splits * M * N));
+            dst = g_split_ws;
+        }
+        const dim3 grid((M + TM - 1) / TM, (N + TN - 1) / TN, k_per_split ? splits : batch);
+        WEED_HIP_REQUIRE(grid.y <= 65535u, "%s: N = %u too large", fn, N);
+        const bool a_i = g.a_s0 <= g.a_s1, b_k = g.b_s0 <= g.b_s1;
+        if (a_i && b_k) {
+            matmul_mfma_kernel<true, true, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, dst, g, k_per_split);
+        } else if (a_i) {
+            matmul_mfma_kernel<true, false, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, dst, g, k_per_split);
+        } else if (b_k) {
+            matmul_mfma_kernel<false, true, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, dst, g, k_per_split);
+        } else {
+            matmul_mfma_kernel<false, false, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, dst, g, k_per_split);
+        }
+        WEED_HIP_LAUNCH_CHECK();
+        if (k_per_split) {
+            matmul_split_sum_kernel<<<dim3((M * N + 255) / 256, 1, 1), 256, 0, stream()>>>(g_split_ws, out_dev, g, splits);
+            WEED_HIP_LAUNCH_CHECK();
+        }
+        return WEED_HIP_OK;
+    }
     const dim3 grid((M + BM - 1) / BM, (N + BN - 1) / BN, batch);
     WEED_HIP_REQUIRE(grid.y <= 65535u, "%s: N = %u too large", fn, N);
     matmul_tiled_kernel<<<grid, 256, 0, stream()>>>(a_dev, b_dev, out_dev, g);
@@ -611,8 +709,19 @@ extern "C" int weed_hip_matmul_f32(uint32_t M, uint32_t N, uint32_t K, const flo
                                    uint32_t a_s0, uint32_t a_s1, const float *b_dev, uint32_t b_off, uint32_t b_s0,
                                    uint32_t b_s1, float *out_dev, uint32_t o_off, uint32_t o_s0, uint32_t o_s1)
 {
-    const MatGeom g = { M, N, K, a_off, a_s0, a_s1, b_off, b_s0, b_s1, o_off, o_s0, o_s1, 1, { 0, 0 }, { 0, 0 }, { 0, 0 } };
+    const MatGeom g = { M, N, K, a_off, a_s0, a_s1, b_off, b_s0, b_s1, o_off, o_s0, o_s1, 1, { 0, 0 }, { 0, 0 }, { 0, 0 },
+                        nullptr, 0, 0 };
     return launch_matmul("weed_hip_matmul_f32", g, 1, a_dev, b_dev, out_dev);
+}
+
+extern "C" int weed_hip_linear_f32(uint32_t M, uint32_t N, uint32_t K, const float *a_dev, uint32_t a_off, uint32_t a_s0,
+                                   uint32_t a_s1, const float *w_dev, uint32_t w_off, uint32_t w_s0, uint32_t w_s1,
+                                   const float *bias_dev, uint32_t bias_off, uint32_t bias_stride, float *out_dev,
+                                   uint32_t o_off, uint32_t o_s0, uint32_t o_s1)
+{
+    const MatGeom g = { M, N, K, a_off, a_s0, a_s1, w_off, w_s0, w_s1, o_off, o_s0, o_s1, 1, { 0, 0 }, { 0, 0 }, { 0, 0 },
+                        bias_dev, bias_off, bias_stride };
+    return launch_matmul("weed_hip_linear_f32", g, 1, a_dev, w_dev, out_dev);
 }
 
 extern "C" int weed_hip_matmul_batched_f32(const uint32_t batch[2], uint32_t M, uint32_t N, uint32_t K,
@@ -626,6 +735,6 @@ extern "C" int weed_hip_matmul_batched_f32(const uint32_t batch[2], uint32_t M, 
     const uint64_t n = (uint64_t)batch[0] * batch[1];
     WEED_HIP_REQUIRE(n <= 65535u, "%s: %llu products in one call (at most 65535)", fn, (unsigned long long)n);
     const MatGeom g = { M, N, K, a_off, a_s0, a_s1, b_off, b_s0, b_s1, o_off, o_s0, o_s1, batch[0] ? batch[0] : 1u,
-                        { a_bs[0], a_bs[1] }, { b_bs[0], b_bs[1] }, { o_bs[0], o_bs[1] } };
+                        { a_bs[0], a_bs[1] }, { b_bs[0], b_bs[1] }, { o_bs[0], o_bs[1] }, nullptr, 0, 0 };
     return launch_matmul(fn, g, (uint32_t)n, a_dev, b_dev, out_dev);
 }

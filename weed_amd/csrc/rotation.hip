@@ -140,6 +140,119 @@ __global__ void __launch_bounds__(256) apply_rotation_kernel(const float *__rest
     }
 }
 
+// The same sums for head-sized d (d <= kRotTiledMaxD) with every global access coalesced whatever the two layouts:
+// a workgroup stages 64 rows of x in LDS (walking x along whichever of its directions is contiguous), wavefront w
+// computes the column chunks w, w + 4, ... for all 64 rows (x from LDS, R through the scalar path, every sum in
+// ascending i with separately rounded products, as above) and writes them along the contiguous direction of `out`
+// (through a per-wavefront LDS patch when that is the rotated dimension itself).
+constexpr int kRotTileRows = 64;
+constexpr int kRotTiledMaxD = 128;
+constexpr int kRotPitch = kRotTileRows + 1;
+
+__global__ void __launch_bounds__(256) apply_rotation_tiled_kernel(const float *__restrict__ x,
+                                                                   const float *__restrict__ rot,
+                                                                   float *__restrict__ out, RotGeom g)
+{
+    __shared__ float tile[kRotTiledMaxD * kRotPitch];
+    __shared__ float patch[4][kRotOutputs * kRotPitch];
+    __shared__ uint64_t xbase[kRotTileRows], obase[kRotTileRows];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t row0 = blockIdx.x * kRotTileRows;
+    const uint32_t nrows = min((uint32_t)kRotTileRows, g.rows - row0);
+    if (tid < nrows) {
+        uint64_t xb = g.x_off, ob = g.o_off;
+        uint32_t tmp = row0 + tid;
+        for (uint32_t dd = 0; dd + 1 < g.rank; ++dd) {
+            const uint32_t c = tmp % g.shape[dd];
+            tmp /= g.shape[dd];
+            xb += (uint64_t)c * g.x_stride[dd];
+            ob += (uint64_t)c * g.o_stride[dd];
+        }
+        xbase[tid] = xb;
+        obase[tid] = ob;
+    }
+    __syncthreads();
+    const uint32_t d = g.d;
+    const uint32_t xs = g.x_stride[g.rank - 1], os = g.o_stride[g.rank - 1];
+    if (xs == 1U) {
+        // rows of x are contiguous: neighbouring threads take neighbouring i
+#pragma unroll 4
+        for (uint32_t e = tid; e < kRotTileRows * d; e += 256) {
+            const uint32_t r = e / d, i = e - r * d;
+            if (r < nrows) {
+                tile[i * kRotPitch + r] = x[xbase[r] + i];
+            }
+        }
+    } else {
+#pragma unroll 4
+        for (uint32_t e = tid; e < kRotTileRows * d; e += 256) {
+            const uint32_t r = e % kRotTileRows, i = e / kRotTileRows;
+            if (r < nrows) {
+                tile[i * kRotPitch + r] = x[xbase[r] + (uint64_t)i * xs];
+            }
+        }
+    }
+    __syncthreads();
+    const uint32_t r = tid % kRotTileRows;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / kRotTileRows);
+    for (uint32_t j0 = wave * kRotOutputs; j0 < d; j0 += 4 * kRotOutputs) {
+        float acc[kRotOutputs];
+#pragma unroll
+        for (int jj = 0; jj < kRotOutputs; ++jj) {
+            acc[jj] = 0.0f;
+        }
+        uint32_t i = 0;
+        for (; i + kRotBatch <= d; i += kRotBatch) {
+            float xv[kRotBatch];
+#pragma unroll
+            for (int u = 0; u < kRotBatch; ++u) {
+                xv[u] = tile[(i + u) * kRotPitch + r];
+            }
+#pragma unroll
+            for (int jj = 0; jj < kRotOutputs; ++jj) {
+                const uint32_t j = min(j0 + (uint32_t)jj, d - 1U);
+                const float *col = rot + (uint64_t)j * d + i;
+#pragma unroll
+                for (int u = 0; u < kRotBatch; ++u) {
+                    acc[jj] = acc[jj] + xv[u] * col[u];
+                }
+            }
+        }
+        for (; i < d; ++i) {
+            const float xv = tile[i * kRotPitch + r];
+#pragma unroll
+            for (int jj = 0; jj < kRotOutputs; ++jj) {
+                const uint32_t j = min(j0 + (uint32_t)jj, d - 1U);
+                acc[jj] = acc[jj] + xv * rot[(uint64_t)j * d + i];
+            }
+        }
+        if (os == 1U) {
+            // rows of out are contiguous: turn the 64 x 16 patch so that neighbouring lanes write neighbouring j
+            float *mine = patch[wave];
+#pragma unroll
+            for (int jj = 0; jj < kRotOutputs; ++jj) {
+                mine[jj * kRotPitch + r] = acc[jj];
+            }
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll 4
+            for (uint32_t e = r; e < kRotTileRows * kRotOutputs; e += kRotTileRows) {
+                const uint32_t jj = e % kRotOutputs, rr = e / kRotOutputs;
+                if (rr < nrows && j0 + jj < d) {
+                    out[obase[rr] + j0 + jj] = mine[jj * kRotPitch + rr];
+                }
+            }
+            __builtin_amdgcn_wave_barrier();
+        } else if (r < nrows) {
+#pragma unroll
+            for (int jj = 0; jj < kRotOutputs; ++jj) {
+                if (j0 + jj < d) {
+                    out[obase[r] + (uint64_t)(j0 + jj) * os] = acc[jj];
+                }
+            }
+        }
+    }
+}
+
 } // namespace
 
 extern "C" {
@@ -199,6 +312,15 @@ int weed_hip_apply_rotation_f32(uint32_t d, const float *r_dev, uint32_t rank, c
     }
     WEED_HIP_REQUIRE(rows * d < (1ull << 32), "%s: more than 2^32 elements", fn);
     g.rows = (uint32_t)rows;
+    // the LDS-tiled kernel pays off when the rotated dimension is the contiguous one on either side; with both sides
+    // contiguous along the rows (Weed's column-major tensors) the register-only kernel is already coalesced and faster
+    const bool rows_contiguous = g.x_stride[rank - 1] != 1U && g.o_stride[rank - 1] != 1U;
+    if (d <= (uint32_t)kRotTiledMaxD && !rows_contiguous) {
+        apply_rotation_tiled_kernel<<<(g.rows + kRotTileRows - 1) / kRotTileRows, 256, 0, stream()>>>(x_dev, r_dev, out_dev,
+                                                                                                     g);
+        WEED_HIP_LAUNCH_CHECK();
+        return WEED_HIP_OK;
+    }
     apply_rotation_kernel<<<dim3((g.rows + 255) / 256, (d + kRotOutputs - 1) / kRotOutputs), 256, 0, stream()>>>(x_dev, r_dev, out_dev, g);
     WEED_HIP_LAUNCH_CHECK();
     return WEED_HIP_OK;

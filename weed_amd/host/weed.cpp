@@ -106,6 +106,16 @@ TensorPtr allocate(const std::vector<tcapint> &shape, const Tensor &like)
         like.storage->device, like.storage->get_device_id());
 }
 
+// A tensor whose LAST dimension is the contiguous one (the reversed view of a column-major allocation): for
+// intermediates that only device kernels see.
+TensorPtr allocate_last_fastest(const std::vector<tcapint> &shape, const Tensor &like)
+{
+    TensorPtr t = allocate(std::vector<tcapint>(shape.rbegin(), shape.rend()), like);
+    std::reverse(t->shape.begin(), t->shape.end());
+    std::reverse(t->stride.begin(), t->stride.end());
+    return t;
+}
+
 void elementwise(int op, const Tensor &a, const Tensor *b, Tensor &out, const char *who)
 {
     // operands are right-aligned against out's shape; a dimension of size 1 repeats (stride 0)
@@ -799,13 +809,40 @@ Linear::Linear(tcapint in_f, tcapint out_f, bool use_bias, bool init_rand, DType
 
 TensorPtr Linear::forward(const TensorPtr x)
 {
-    TensorPtr y = x >> weight;
-    if (bias) {
-        // unlike Tensor::add in the reference (src/tensors/tensor.cpp:1091), broadcasting never reshapes the bias
-        // itself, so the sequence length may change between calls
-        y = y + bias;
+    const bool plain_bias = bias && bias->shape.size() == 2U && bias->shape[0U] == 1U && bias->shape[1U] == out_features;
+    if (!plain_bias || x->shape.size() < 2U || weight->shape.size() != 2U) {
+        TensorPtr y = x >> weight;
+        if (bias) {
+            // unlike Tensor::add in the reference (src/tensors/tensor.cpp:1091), broadcasting never reshapes the bias
+            // itself, so the sequence length may change between calls
+            y = y + bias;
+        }
+        return y;
     }
-    return y;
+    // `x >> weight` then `+ bias` (src/modules/linear.cpp:86-100) as one launch: the product's epilogue adds the bias
+    // to the rounded sum, which gives the same bits as the two separate ops
+    const size_t rank = x->shape.size();
+    const tcapint K = x->shape.back(), N = weight->shape[1U];
+    if (weight->shape[0U] != K) {
+        throw std::invalid_argument("matmul dimension mismatch");
+    }
+    TensorPtr a2 = (rank > 2U) ? Tensor::reshape(x, { -1, (symint)K }) : x;
+    TensorPtr out = allocate({ a2->shape[0U], N }, *a2);
+    validate_all_same_device({ a2.get(), weight.get(), bias.get(), out.get() }, "Linear::forward");
+    real1 *ap = device_ptr(*a2, "Linear::forward"), *wp = device_ptr(*weight, "Linear::forward");
+    real1 *bp = device_ptr(*bias, "Linear::forward"), *op = device_ptr(*out, "Linear::forward");
+    {
+        WEED_DEVICE_LOCK();
+        HipDevice::check(weed_hip_linear_f32(a2->shape[0U], N, K, ap, a2->offset, a2->stride[0U], a2->stride[1U], wp,
+            weight->offset, weight->stride[0U], weight->stride[1U], bp, bias->offset, bias->stride[1U], op, out->offset,
+            out->stride[0U], out->stride[1U]));
+    }
+    if (rank > 2U) {
+        std::vector<symint> shp(x->shape.begin(), x->shape.end() - 1);
+        shp.push_back((symint)N);
+        out = Tensor::reshape(out, shp);
+    }
+    return out;
 }
 
 std::vector<ParameterPtr> Linear::parameters()
@@ -1190,23 +1227,54 @@ TensorPtr MultiHeadAttention::forward_quantized(TensorPtr Q, TensorPtr K, Tensor
     if (uT > kFusedQueryLimit) {
         // Long multi-token calls (prefill): the fused kernel serves one query position per launch, so beyond a few
         // positions it is cheaper to do what the reference does -- dequantise the cache once (still in the rotated
-        // basis) and run dense matrix products: rotate Q, attend, un-rotate.
-        TensorPtr K_deq = allocate({ uB, Hkv, cache_len, hd }, *Q), V_deq = allocate({ uB, Hkv, cache_len, hd }, *Q);
-        HipDevice::check(weed_hip_kv_dequant(cache, 0, 0, B, 0, (int32_t)cache_len, device_ptr(*K_deq, "forward"), 0U,
-            K_deq->stride.data()));
-        HipDevice::check(weed_hip_kv_dequant(cache, 1, 0, B, 0, (int32_t)cache_len, device_ptr(*V_deq, "forward"), 0U,
-            V_deq->stride.data()));
-        TensorPtr Qv = Tensor::transpose(Q, 1, 2); // (B, H, T, hd) view
-        TensorPtr Q_rot = allocate(Qv->shape, *Q);
-        HipDevice::check(weed_hip_apply_rotation_f32(hd, k_rot_dev->buffer, 4U, Qv->shape.data(), qp, Qv->offset,
-            Qv->stride.data(), device_ptr(*Q_rot, "forward"), 0U, Q_rot->stride.data()));
-        TensorPtr att = attend_dense(Q_rot, K_deq, V_deq, before); // (B, H, T, hd), rotated basis
+        // basis) and run dense ops: rotate Q, product, / sqrt(d), + mask, softmax, product, un-rotate
+        // (multihead_attention.cpp:279-340).  The intermediates are private to this call, so they are laid out for
+        // the device instead of column-major: head_dim (or the key position) is the contiguous dimension, the query
+        // heads that share a KV head sit next to each other, and one batched product per (sequence, KV head) covers
+        // the whole group without replicating K and V.
+        const tcapint G = Hq / Hkv, L = cache_len, GT = G * uT;
+        if ((uint64_t)uB * Hkv > 65535U) {
+            throw std::invalid_argument("MultiHeadAttention::forward(): more than 65535 (sequence, KV head) pairs in a prefill");
+        }
+        TensorPtr K_deq = allocate_last_fastest({ uB, Hkv, L, hd }, *Q), V_deq = allocate_last_fastest({ uB, Hkv, L, hd }, *Q);
+        HipDevice::check(weed_hip_kv_dequant(cache, 0, 0, B, 0, (int32_t)L, device_ptr(*K_deq, "forward"), 0U, K_deq->stride.data()));
+        HipDevice::check(weed_hip_kv_dequant(cache, 1, 0, B, 0, (int32_t)L, device_ptr(*V_deq, "forward"), 0U, V_deq->stride.data()));
+        // logical (B, Hkv, G, T, head_dim) views of Q and of the result: query head h = kv * G + g (blocked) or
+        // g * Hkv + kv (Weed's kv = h % Hkv)
+        const tcapint sH = Q->stride[2U];
+        const tcapint shape5[5] = { uB, Hkv, G, uT, hd };
+        const tcapint q5_str[5] = { Q->stride[0U], gqa_blocked ? G * sH : sH, gqa_blocked ? sH : Hkv * sH, Q->stride[1U],
+            Q->stride[3U] };
+        TensorPtr Q_rot = allocate_last_fastest({ uB, Hkv, G, uT, hd }, *Q);
+        HipDevice::check(weed_hip_apply_rotation_f32(hd, k_rot_dev->buffer, 5U, shape5, qp, Q->offset, q5_str,
+            device_ptr(*Q_rot, "forward"), 0U, Q_rot->stride.data()));
+        // scores[b, kv, g*T + t, l] = q . k
+        TensorPtr scores = allocate_last_fastest({ uB, Hkv, G, uT, L }, *Q);
+        const tcapint pairs[2] = { uB, Hkv };
+        const tcapint q_bs[2] = { Hkv * GT * hd, GT * hd }, kv_bs[2] = { Hkv * L * hd, L * hd }, s_bs[2] = { Hkv * GT * L, GT * L };
+        HipDevice::check(weed_hip_matmul_batched_f32(pairs, GT, L, hd, device_ptr(*Q_rot, "forward"), 0U, hd, 1U, q_bs,
+            device_ptr(*K_deq, "forward"), 0U, 1U, hd, kv_bs, device_ptr(*scores, "forward"), 0U, L, 1U, s_bs));
+        TensorPtr inv = std::make_shared<Tensor>(real1(std::sqrt((real1)head_dim)), false, Q->storage->device,
+            Q->storage->get_device_id());
+        elementwise(WEED_HIP_EW_DIV, *scores, inv.get(), *scores, "MultiHeadAttention::forward");
+        TensorPtr mask = Tensor::zeros({ uT, L }, false, false, DType::REAL, Q->storage->device);
+        Weed::triu_fill(*mask, (real1)mask_val, before + 1U);
+        elementwise(WEED_HIP_EW_ADD, *scores, mask.get(), *scores, "MultiHeadAttention::forward");
+        TensorPtr weights = allocate_last_fastest({ uB, Hkv, G, uT, L }, *Q);
+        HipDevice::check(weed_hip_softmax_f32(5U, scores->shape.data(), 4U, device_ptr(*scores, "forward"), 0U,
+            scores->stride.data(), device_ptr(*weights, "forward"), 0U, weights->stride.data()));
+        TensorPtr att = allocate_last_fastest({ uB, Hkv, G, uT, hd }, *Q);
+        HipDevice::check(weed_hip_matmul_batched_f32(pairs, GT, hd, L, device_ptr(*weights, "forward"), 0U, L, 1U, s_bs,
+            device_ptr(*V_deq, "forward"), 0U, hd, 1U, kv_bs, device_ptr(*att, "forward"), 0U, hd, 1U, q_bs));
         if (!v_rot_t_dev) {
             v_rot_t_dev = std::make_shared<GpuRealStorage>(v_rotation_trans);
         }
-        TensorPtr outv = Tensor::transpose(out, 1, 2); // (B, H, T, hd) view of the (B, T, H, hd) result
-        HipDevice::check(weed_hip_apply_rotation_f32(hd, v_rot_t_dev->buffer, 4U, att->shape.data(),
-            device_ptr(*att, "forward"), att->offset, att->stride.data(), op, 0U, outv->stride.data()));
+        // out is (B, T, H, head_dim) column-major like Q
+        const tcapint oH = out->stride[2U];
+        const tcapint o5_str[5] = { out->stride[0U], gqa_blocked ? G * oH : oH, gqa_blocked ? oH : Hkv * oH, out->stride[1U],
+            out->stride[3U] };
+        HipDevice::check(weed_hip_apply_rotation_f32(hd, v_rot_t_dev->buffer, 5U, shape5, device_ptr(*att, "forward"), 0U,
+            att->stride.data(), op, 0U, o5_str));
         return out;
     }
     // causal attention: query position t sees the first before + t + 1 cached tokens of its sequence
