@@ -53,8 +53,12 @@ int weed_hip_sync(void);
 const char *weed_hip_last_error(void);
 const char *weed_hip_version(void);
 
+/* Device memory for tensors.  Freed blocks are kept and handed out again in stream order (no wait, no driver call)
+ * while the working set repeats, as the intermediates of a module's forward do; weed_hip_release_cached drains the
+ * stream and returns them to the driver.  WEED_HIP_POOL_MAX_MB caps the cached bytes (default 64 GiB, 0 = no cache). */
 int weed_hip_malloc(void **ptr_dev, size_t bytes);
 int weed_hip_free(void *ptr_dev);
+int weed_hip_release_cached(void);
 int weed_hip_memset(void *ptr_dev, int byte_value, size_t bytes);
 int weed_hip_memcpy_h2d(void *dst_dev, const void *src, size_t bytes);
 int weed_hip_memcpy_d2h(void *dst, const void *src_dev, size_t bytes);

@@ -397,3 +397,47 @@ def test_rope_bit_exact_against_checker(gpu, oracle, pos0):
     np.testing.assert_array_equal(out.cpu().numpy(), want)
     with pytest.raises(gpu.WeedHipError):
         gpu.rope(xd, dev(cos_t), dev(sin_t), L, out, pos0=L - T + 1)  # positions past the table
+
+
+def test_device_memory_blocks_are_reused_in_stream_order(gpu):
+    """weed_hip_free keeps a block, weed_hip_malloc hands it out again for a request of about the same size (no driver
+    call, no wait), a much smaller or larger request gets its own block, and weed_hip_release_cached empties the
+    cache.  Reuse is safe without a wait because all work goes to one stream: a copy queued before the free is still
+    read back intact after the block's next owner overwrote it later in the stream."""
+    from ctypes import byref, c_void_p
+    lib = gpu.load()
+
+    def malloc(n):
+        p = c_void_p()
+        gpu.check(lib.weed_hip_malloc(byref(p), n))
+        return p.value
+
+    gpu.check(lib.weed_hip_release_cached())
+    a = malloc(3 << 20)
+    gpu.check(lib.weed_hip_free(c_void_p(a)))
+    b = malloc((3 << 20) - 4096)
+    assert b == a
+    c = malloc(3 << 20)
+    assert c != a
+    small = malloc(1000)
+    assert small not in (a, c)
+    big = malloc(64 << 20)
+    assert big not in (a, c)
+    # stream order: fill b, copy it out, free it, let the next owner overwrite it, then look at the copy
+    src = np.arange(1 << 18, dtype=np.float32)
+    keep = malloc(src.nbytes)
+    gpu.check(lib.weed_hip_memcpy_h2d(c_void_p(b), src.ctypes.data_as(c_void_p), src.nbytes))
+    gpu.check(lib.weed_hip_memcpy_d2d(c_void_p(keep), c_void_p(b), src.nbytes))
+    gpu.check(lib.weed_hip_free(c_void_p(b)))
+    again = malloc(3 << 20)
+    assert again == a
+    gpu.check(lib.weed_hip_memset(c_void_p(again), 0, 3 << 20))
+    back = np.empty_like(src)
+    gpu.check(lib.weed_hip_memcpy_d2h(back.ctypes.data_as(c_void_p), c_void_p(keep), src.nbytes))
+    np.testing.assert_array_equal(back, src)
+    for p in (again, c, small, big, keep):
+        gpu.check(lib.weed_hip_free(c_void_p(p)))
+    gpu.check(lib.weed_hip_release_cached())
+    fresh = malloc(3 << 20)
+    gpu.check(lib.weed_hip_free(c_void_p(fresh)))
+    gpu.check(lib.weed_hip_release_cached())

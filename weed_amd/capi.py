@@ -43,6 +43,7 @@ SIGNATURES = {
     "weed_hip_version": (c_char_p, []),
     "weed_hip_malloc": (c_int, [POINTER(c_void_p), c_size_t]),
     "weed_hip_free": (c_int, [c_void_p]),
+    "weed_hip_release_cached": (c_int, []),
     "weed_hip_memset": (c_int, [c_void_p, c_int, c_size_t]),
     "weed_hip_memcpy_h2d": (c_int, [c_void_p, c_void_p, c_size_t]),
     "weed_hip_memcpy_d2h": (c_int, [c_void_p, c_void_p, c_size_t]),

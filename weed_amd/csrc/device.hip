@@ -4,6 +4,7 @@
 // include/devices/gpu_device.hpp): one HIP stream, stream-ordered launches, no callbacks, no JIT.
 #include "common.h"
 
+#include <cstdlib>
 #include <map>
 #include <mutex>
 #include <string>
@@ -26,6 +27,44 @@ struct ProfileEntry {
     uint64_t launches = 0;
 };
 std::map<std::string, ProfileEntry> g_profiles;
+
+// Stream-ordered block cache behind weed_hip_malloc / weed_hip_free.  Every launch of the library goes to ONE stream,
+// so a freed block may be handed out again without waiting: whatever still reads it was enqueued before whatever
+// will write it.  hipMalloc and hipFree (which waits for the device) then only run while the working set grows, not
+// once per intermediate tensor of every module call.  Sizes are rounded up (512 B, 2 MiB above 1 MiB); a request takes
+// the smallest cached block that is large enough and at most half again as large.  When the stream is replaced the old
+// one is drained first.  Cached bytes are capped (kPoolCapBytes, or WEED_HIP_POOL_MAX_MB; 0 turns the cache off).
+std::mutex g_pool_mutex;
+std::map<void *, size_t> g_pool_sizes;       // every live or cached block of the pool -> rounded size
+std::multimap<size_t, void *> g_pool_free;   // cached blocks by size
+size_t g_pool_cached = 0;
+constexpr size_t kPoolCapBytes = 64ull << 30;
+
+size_t pool_cap()
+{
+    static const size_t cap = [] {
+        const char *env = std::getenv("WEED_HIP_POOL_MAX_MB");
+        return env ? (size_t)std::strtoull(env, nullptr, 10) << 20 : kPoolCapBytes;
+    }();
+    return cap;
+}
+
+size_t pool_round(size_t bytes)
+{
+    const size_t unit = bytes > (1u << 20) ? (2u << 20) : 512u;
+    return (bytes + unit - 1) / unit * unit;
+}
+
+// Give every cached block back to the driver (the caller holds g_pool_mutex and has drained the stream).
+void pool_release_locked()
+{
+    for (auto &kv : g_pool_free) {
+        (void)hipFree(kv.second);
+        g_pool_sizes.erase(kv.second);
+    }
+    g_pool_free.clear();
+    g_pool_cached = 0;
+}
 
 void resolve_pending(ProfileEntry &e)
 {
@@ -155,7 +194,12 @@ int weed_hip_device_name(char *buf, size_t buf_len)
 int weed_hip_set_stream(void *hip_stream)
 {
     WEED_HIP_TRY(ensure_init());
-    g_stream = hip_stream ? (hipStream_t)hip_stream : g_own_stream;
+    hipStream_t next = hip_stream ? (hipStream_t)hip_stream : g_own_stream;
+    if (next != g_stream) {
+        // cached blocks are reused without waiting, which is only in order on one stream
+        WEED_HIP_CHECK(hipStreamSynchronize(g_stream));
+        g_stream = next;
+    }
     return WEED_HIP_OK;
 }
 
@@ -180,11 +224,29 @@ int weed_hip_malloc(void **ptr_dev, size_t bytes)
     if (!bytes) {
         return WEED_HIP_OK;
     }
-    hipError_t e = hipMalloc(ptr_dev, bytes);
+    const size_t want = pool_round(bytes);
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    auto it = g_pool_free.lower_bound(want);
+    if (it != g_pool_free.end() && it->first <= want + want / 2) {
+        *ptr_dev = it->second;
+        g_pool_cached -= it->first;
+        g_pool_free.erase(it);
+        return WEED_HIP_OK;
+    }
+    hipError_t e = hipMalloc(ptr_dev, want);
+    if (e != hipSuccess && !g_pool_free.empty()) {
+        // out of memory with blocks in the cache: drain, give them back, try once more
+        (void)hipGetLastError();
+        WEED_HIP_CHECK(hipStreamSynchronize(g_stream));
+        pool_release_locked();
+        e = hipMalloc(ptr_dev, want);
+    }
     if (e != hipSuccess) {
+        (void)hipGetLastError();
         *ptr_dev = nullptr;
         return fail(WEED_HIP_ENOMEM, "weed_hip_malloc: %zu bytes: %s", bytes, hipGetErrorString(e));
     }
+    g_pool_sizes[*ptr_dev] = want;
     return WEED_HIP_OK;
 }
 
@@ -194,8 +256,28 @@ int weed_hip_free(void *ptr_dev)
         return WEED_HIP_OK;
     }
     WEED_HIP_TRY(ensure_init());
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    auto it = g_pool_sizes.find(ptr_dev);
+    if (it != g_pool_sizes.end() && g_pool_cached + it->second <= pool_cap()) {
+        g_pool_free.emplace(it->second, ptr_dev);
+        g_pool_cached += it->second;
+        return WEED_HIP_OK;
+    }
+    // not one of the pool's blocks, or the cache is full: wait for whatever still uses it, then give it back
+    if (it != g_pool_sizes.end()) {
+        g_pool_sizes.erase(it);
+    }
     WEED_HIP_CHECK(hipStreamSynchronize(g_stream));
     WEED_HIP_CHECK(hipFree(ptr_dev));
+    return WEED_HIP_OK;
+}
+
+int weed_hip_release_cached(void)
+{
+    WEED_HIP_TRY(ensure_init());
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    WEED_HIP_CHECK(hipStreamSynchronize(g_stream));
+    pool_release_locked();
     return WEED_HIP_OK;
 }
 
