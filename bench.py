@@ -123,6 +123,27 @@ def extras(capi, torch, workloads, steps, warmup):
         "roofline": {"bound": "hbm", "achieved": wbytes / kernel_s / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": wbytes / kernel_s / 1e9 / HBM_PEAK_GBS}}
     del X, Wp, Y
+    # standalone softmax and sum over an [8192 x 8192] column-major matrix (256 MiB), along the contiguous axis and
+    # along the strided one: 8 B per element (softmax) and 4 B per element (sum) of algorithmic traffic
+    S = torch.randn((8192, 8192), device="cuda").t()
+    So = torch.empty((8192, 8192), device="cuda").t()
+    Sr = torch.empty(8192, device="cuda")
+    dense = {}
+    for axis, name in ((0, "contiguous_axis"), (1, "strided_axis")):
+        for op, fn, bytes_per in (("softmax", lambda: capi.softmax(S, So, axis), 8),
+                                  ("reduce", lambda: capi.reduce(capi.REDUCE_SUM, S, Sr, axis), 4)):
+            capi.profile_reset()
+            capi.profile_enable(True)
+            time_calls(torch, fn, steps, warmup)
+            k_ms, k_n = capi.profile_read(op)
+            capi.profile_enable(False)
+            kernel_s = 1e-3 * k_ms / max(1, k_n)
+            gbs = S.numel() * bytes_per / kernel_s / 1e9
+            dense["%s_%s" % (op, name)] = {"kernel_ms": 1e3 * kernel_s,
+                                           "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS,
+                                                        "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS}}
+    out["softmax_sum_f32_8192x8192"] = dense
+    del S, So, Sr
     # configuration 5a: encode-and-append 4096 tokens x 8 kv heads x 128, 3-bit codes (rotate, quantise, pack)
     wl = workloads.config(5)
     d = wl.head_dim

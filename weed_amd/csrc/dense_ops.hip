@@ -159,9 +159,9 @@ template <int RT, int THREADS> __global__ void __launch_bounds__(THREADS) softma
 }
 
 // Softmax along a contiguous, 16-byte aligned axis: one workgroup per row, float4 accesses, and the first
-// CACHED * 4 * THREADS elements of the row stay in registers between the two passes (rows up to that length are
-// read once).
-template <int CACHED, int THREADS>
+// CACHED * 4 * THREADS elements of the row stay in registers between the passes.  Rows up to that length (FITS) are
+// read once and cost one exponential per element; longer rows keep a running (max, sum) and are read twice.
+template <int CACHED, int THREADS, bool FITS>
 __global__ void __launch_bounds__(THREADS) softmax_contiguous_kernel(const float *__restrict__ a,
                                                                     float *__restrict__ out, AxisGeom g)
 {
@@ -177,6 +177,29 @@ __global__ void __launch_bounds__(THREADS) softmax_contiguous_kernel(const float
     for (int c = 0; c < CACHED; ++c) {
         const uint32_t idx = threadIdx.x + c * THREADS;
         cache[c] = idx < n4 ? ap[idx] : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+    }
+    if (FITS) {
+        // the whole row is in registers: maximum, then ONE exponential per element (kept), then the division -- the
+        // reference's three passes (src/ops/softmax.cpp:276-287) without touching memory again
+#pragma unroll
+        for (int c = 0; c < CACHED; ++c) {
+            m = fmaxf(fmaxf(m, fmaxf(cache[c].x, cache[c].y)), fmaxf(cache[c].z, cache[c].w));
+        }
+        m = block_reduce<1, 1, THREADS>(m, red);
+#pragma unroll
+        for (int c = 0; c < CACHED; ++c) {
+            cache[c] = make_float4(expf(cache[c].x - m), expf(cache[c].y - m), expf(cache[c].z - m), expf(cache[c].w - m));
+            s += (cache[c].x + cache[c].y) + (cache[c].z + cache[c].w);
+        }
+        s = block_reduce<0, 1, THREADS>(s, red);
+#pragma unroll
+        for (int c = 0; c < CACHED; ++c) {
+            const uint32_t idx = threadIdx.x + c * THREADS;
+            if (idx < n4) {
+                op[idx] = make_float4(cache[c].x / s, cache[c].y / s, cache[c].z / s, cache[c].w / s);
+            }
+        }
+        return;
     }
 #pragma unroll
     for (int c = 0; c < CACHED; ++c) {
@@ -220,7 +243,7 @@ template <int OP> __device__ __forceinline__ float wave_reduce(float v)
 // one WAVEFRONT per row, four rows per workgroup, so no lane idles on a 64..2048-element row and nothing goes
 // through LDS.  V = 4: float4 accesses (every row 16-byte aligned, length a multiple of 4), V = 1: scalar.  The first
 // CACHED * 64 * V elements of a row stay in registers between the two passes.
-template <int V, int CACHED>
+template <int V, int CACHED, bool FITS>
 __global__ void __launch_bounds__(256) softmax_wave_rows_kernel(const float *__restrict__ a, float *__restrict__ out,
                                                                 AxisGeom g)
 {
@@ -247,6 +270,40 @@ __global__ void __launch_bounds__(256) softmax_wave_rows_kernel(const float *__r
             } else {
                 cache[c][0] = idx < nvec ? ap[idx] : -INFINITY;
             }
+        }
+        if (FITS) {
+            // the row is in registers: maximum, one exponential per element (kept), division
+#pragma unroll
+            for (int c = 0; c < CACHED; ++c) {
+#pragma unroll
+                for (int e = 0; e < V; ++e) {
+                    m = fmaxf(m, cache[c][e]);
+                }
+            }
+            m = wave_reduce<1>(m);
+#pragma unroll
+            for (int c = 0; c < CACHED; ++c) {
+#pragma unroll
+                for (int e = 0; e < V; ++e) {
+                    cache[c][e] = expf(cache[c][e] - m);
+                    s += cache[c][e];
+                }
+            }
+            s = wave_reduce<0>(s);
+#pragma unroll
+            for (int c = 0; c < CACHED; ++c) {
+                const uint32_t idx = lane + 64U * c;
+                if (idx < nvec) {
+                    if (V == 4) {
+                        reinterpret_cast<float4 *>(op)[idx] = make_float4(cache[c][0] / s, cache[c][V > 1 ? 1 : 0] / s,
+                                                                          cache[c][V > 2 ? 2 : 0] / s,
+                                                                          cache[c][V > 3 ? 3 : 0] / s);
+                    } else {
+                        op[idx] = cache[c][0] / s;
+                    }
+                }
+            }
+            continue;
         }
 #pragma unroll
         for (int c = 0; c < CACHED; ++c) {
@@ -765,11 +822,20 @@ int weed_hip_softmax_f32(uint32_t rank, const uint32_t *shape, uint32_t axis, co
     ProfileScope prof("softmax");
     const AxisLaunch how = choose_axis_launch(g, a_dev, out_dev, true);
     if (how == AXIS_CONTIGUOUS) {
-        softmax_contiguous_kernel<8, 256><<<g.rows, 256, 0, stream()>>>(a_dev, out_dev, g);
+        if (g.axis_len <= 8U * 4U * 256U) {
+            softmax_contiguous_kernel<8, 256, true><<<g.rows, 256, 0, stream()>>>(a_dev, out_dev, g);
+        } else {
+            softmax_contiguous_kernel<8, 256, false><<<g.rows, 256, 0, stream()>>>(a_dev, out_dev, g);
+        }
     } else if (how == AXIS_WAVE_VEC) {
-        softmax_wave_rows_kernel<4, 8><<<wave_row_blocks(g.rows), 256, 0, stream()>>>(a_dev, out_dev, g);
+        // (kWaveRowMax = 8 * 4 * 64: such a row always fits a wavefront's registers)
+        softmax_wave_rows_kernel<4, 8, true><<<wave_row_blocks(g.rows), 256, 0, stream()>>>(a_dev, out_dev, g);
     } else if (how == AXIS_WAVE) {
-        softmax_wave_rows_kernel<1, 16><<<wave_row_blocks(g.rows), 256, 0, stream()>>>(a_dev, out_dev, g);
+        if (g.axis_len <= 16U * 64U) {
+            softmax_wave_rows_kernel<1, 16, true><<<wave_row_blocks(g.rows), 256, 0, stream()>>>(a_dev, out_dev, g);
+        } else {
+            softmax_wave_rows_kernel<1, 16, false><<<wave_row_blocks(g.rows), 256, 0, stream()>>>(a_dev, out_dev, g);
+        }
     } else if (how == AXIS_ROW) {
         softmax_kernel<1, 256><<<g.rows, 256, 0, stream()>>>(a_dev, out_dev, g);
     } else if (how == AXIS_ROWS32) {
