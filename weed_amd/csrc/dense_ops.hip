@@ -158,6 +158,64 @@ template <int RT, int THREADS> __global__ void __launch_bounds__(THREADS) softma
     }
 }
 
+// Softmax along a strided axis of at most kStridedCached * (kStridedThreads / RT) elements: RT neighbouring rows per
+// workgroup, every thread keeps its share of a row in registers (all loads in flight at once), so the data is read
+// once and each element costs one exponential.
+constexpr int kStridedCached = 64;
+constexpr int kStridedThreads = 512;
+
+template <int RT>
+__global__ void __launch_bounds__(kStridedThreads) softmax_strided_cached_kernel(const float *__restrict__ a,
+                                                                      float *__restrict__ out, AxisGeom g)
+{
+    __shared__ float red[kStridedThreads];
+    constexpr int NY = kStridedThreads / RT;
+    const uint32_t tx = threadIdx.x % RT, ty = threadIdx.x / RT;
+    const uint32_t row = blockIdx.x * RT + tx;
+    const bool valid = row < g.rows;
+    uint64_t a_base = 0, o_base = 0;
+    if (valid) {
+        row_bases(g, row, a_base, o_base);
+    }
+    const uint32_t as = g.a_stride[g.axis], os = g.o_stride[g.axis];
+    const uint32_t len = valid ? g.axis_len : 0U;
+    // rows past the end read row 0's first element (any readable address) and are discarded
+    const float *ap = a + (valid ? a_base : (uint64_t)g.a_off);
+    float *op = out + o_base;
+    float x[kStridedCached];
+    // unconditional loads of clamped positions (the host checks that the row's span fits 32 bits), then the select
+    const uint32_t last = len ? len - 1U : 0U;
+#pragma unroll
+    for (int c = 0; c < kStridedCached; ++c) {
+        const uint32_t j = ty + c * NY;
+        x[c] = ap[min(j, last) * as];
+    }
+#pragma unroll
+    for (int c = 0; c < kStridedCached; ++c) {
+        const uint32_t j = ty + c * NY;
+        x[c] = j < len ? x[c] : -INFINITY;
+    }
+    float m = -INFINITY, s = 0.0f;
+#pragma unroll
+    for (int c = 0; c < kStridedCached; ++c) {
+        m = fmaxf(m, x[c]);
+    }
+    m = block_reduce<1, RT, kStridedThreads>(m, red);
+#pragma unroll
+    for (int c = 0; c < kStridedCached; ++c) {
+        x[c] = expf(x[c] - m);
+        s += x[c];
+    }
+    s = block_reduce<0, RT, kStridedThreads>(s, red);
+#pragma unroll
+    for (int c = 0; c < kStridedCached; ++c) {
+        const uint32_t j = ty + c * NY;
+        if (j < len) {
+            op[(uint64_t)j * os] = x[c] / s;
+        }
+    }
+}
+
 // Softmax along a contiguous, 16-byte aligned axis: one workgroup per row, float4 accesses, and the first
 // CACHED * 4 * THREADS elements of the row stay in registers between the passes.  Rows up to that length (FITS) are
 // read once and cost one exponential per element; longer rows keep a running (max, sum) and are read twice.
@@ -838,6 +896,12 @@ int weed_hip_softmax_f32(uint32_t rank, const uint32_t *shape, uint32_t axis, co
         }
     } else if (how == AXIS_ROW) {
         softmax_kernel<1, 256><<<g.rows, 256, 0, stream()>>>(a_dev, out_dev, g);
+    } else if ((uint64_t)g.axis_len * g.a_stride[axis] >= (1ull << 32)) {
+        softmax_kernel<16, 1024><<<(g.rows + 15) / 16, 1024, 0, stream()>>>(a_dev, out_dev, g);
+    } else if (g.axis_len <= (uint32_t)(kStridedCached * kStridedThreads / 32) && g.rows >= 32U * 256U) {
+        softmax_strided_cached_kernel<32><<<(g.rows + 31) / 32, kStridedThreads, 0, stream()>>>(a_dev, out_dev, g);
+    } else if (g.axis_len <= (uint32_t)(kStridedCached * kStridedThreads / 16)) {
+        softmax_strided_cached_kernel<16><<<(g.rows + 15) / 16, kStridedThreads, 0, stream()>>>(a_dev, out_dev, g);
     } else if (how == AXIS_ROWS32) {
         softmax_kernel<32, 256><<<(g.rows + 31) / 32, 256, 0, stream()>>>(a_dev, out_dev, g);
     } else if (how == AXIS_ROWS32_WIDE) {
