@@ -441,3 +441,42 @@ def test_device_memory_blocks_are_reused_in_stream_order(gpu):
     fresh = malloc(3 << 20)
     gpu.check(lib.weed_hip_free(c_void_p(fresh)))
     gpu.check(lib.weed_hip_release_cached())
+
+
+def test_degenerate_shapes(gpu):
+    """Axes of length one, single rows, one very long row (contiguous and strided), rank-8 broadcasting with size-1
+    dimensions everywhere, transposed copies smaller than a tile, rotations of width 1, 2, 3 and 129."""
+    import torch
+    rng = np.random.default_rng(123)
+    for shape, axis in [((1,), 0), ((5, 1), 1), ((1, 5), 0), ((1, 1, 1), 1), ((3000, 1), 1), ((1, 3000), 0),
+                        ((1, 300000), 1), ((300000, 1), 0)]:
+        x = rng.standard_normal(shape, dtype=np.float32)
+        for mk in (col_major, dev):
+            xd = mk(x)
+            out = torch.zeros_like(xd)
+            gpu.softmax(xd, out, axis)
+            x64 = x.astype(np.float64)
+            e = np.exp(x64 - x64.max(axis=axis, keepdims=True))
+            np.testing.assert_allclose(out.cpu().numpy(), e / e.sum(axis=axis, keepdims=True), rtol=3e-5, atol=1e-12)
+            if len(shape) > 1:
+                r = mk(np.zeros([n for i, n in enumerate(shape) if i != axis], dtype=np.float32))
+                gpu.reduce(gpu.REDUCE_MAX, xd, r, axis)
+                np.testing.assert_array_equal(r.cpu().numpy(), x.max(axis=axis))
+                gpu.reduce(gpu.REDUCE_SUM, xd, r, axis)
+                np.testing.assert_allclose(r.cpu().numpy(), x64.sum(axis=axis), rtol=2e-5, atol=2e-5 * np.sqrt(shape[axis]))
+    x = rng.standard_normal((2, 1, 3, 1, 4, 1, 5, 2), dtype=np.float32)
+    y = rng.standard_normal((1, 1, 3, 1, 1, 1, 5, 1), dtype=np.float32)
+    out = col_major(np.zeros(x.shape, dtype=np.float32))
+    gpu.elementwise(gpu.EW_MUL, col_major(x), dev(y), out)
+    np.testing.assert_array_equal(out.cpu().numpy(), x * y)
+    for shape in [(16, 16), (17, 33), (1, 64), (64, 1), (15, 100)]:
+        x = rng.standard_normal(shape, dtype=np.float32)
+        out = col_major(np.zeros(shape[::-1], dtype=np.float32))
+        gpu.elementwise(gpu.EW_COPY, col_major(x).t(), None, out)
+        np.testing.assert_array_equal(out.cpu().numpy(), x.T)
+    for d in (1, 2, 3, 129):
+        x = rng.standard_normal((7, d), dtype=np.float32)
+        r = rng.standard_normal((d, d), dtype=np.float32)  # element (i, j) of the column-major matrix: r.T.flat[i + d*j]
+        out = dev(np.zeros((7, d), dtype=np.float32))
+        gpu.apply_rotation(dev(x), col_major(r), out)
+        np.testing.assert_allclose(out.cpu().numpy(), x.astype(np.float64) @ r.astype(np.float64), rtol=1e-5, atol=1e-5)
