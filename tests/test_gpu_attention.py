@@ -284,3 +284,55 @@ def test_prefix_lengths_override(gpu, oracle):
         assert_attn_close(out.cpu().numpy(), want, "prefix %s" % prefix)
     assert list(cache.seq_lens()) == lens
     cache.close()
+
+
+@pytest.mark.parametrize("lloyd,d,Hkv,Hq,T,gqa_weed", [(False, 64, 2, 4, 3, True), (True, 128, 2, 8, 2, False),
+                                                       (True, 128, 1, 4, 4, True), (False, 128, 2, 2, 5, False),
+                                                       (True, 64, 2, 16, 2, True), (True, 128, 2, 8, 4, False)])
+def test_chunk_of_query_positions(gpu, oracle, lloyd, d, Hkv, Hq, T, gqa_weed):
+    """Several query positions per sequence in one pass over the cache: position t must equal the checker run over
+    all but the last T - 1 - t tokens.  The lengths put the chunk across a block boundary (a block whose tokens are
+    all hidden from the early positions), inside one block, and far from any edge; both GQA mappings; column-major
+    operands; rotations on; and the same with the attended lengths given explicitly."""
+    import torch
+    rng = np.random.default_rng(1000 * T + Hq + d)
+    lens = [64 + 1, 300, 129, 64 + T, 5 * 64]
+    S = len(lens)
+    kb, vb, ks = (3, 4, 1) if lloyd else (4, 3, 0)
+    mode = gpu.KV_LLOYDMAX if lloyd else gpu.KV_UNIFORM
+    wl = workloads.Workload("chunk", S, Hq, Hkv, d, lens, kb, vb, ks, 0, 0)
+    K = rng.standard_normal((S, Hkv, max(lens), d), dtype=np.float32)
+    V = rng.standard_normal((S, Hkv, max(lens), d), dtype=np.float32)
+    q = rng.standard_normal((S, T, Hq, d), dtype=np.float32)
+    Rk, Rv = rotations(oracle, d, 5)
+    cache = build_cache(gpu, wl, mode, K, V, (Rk, Rv), None if lloyd else (1.0, 1.0))
+    gqa = gpu.GQA_WEED if gqa_weed else gpu.GQA_BLOCKED
+    flags = gpu.ATTN_ROTATE_Q | gpu.ATTN_UNROTATE_OUT
+
+    def check(seen, lens_dev, what):
+        for mk in (dev, col_major):
+            qd = mk(q)
+            out = torch.zeros_like(qd)
+            cache.decode_attn_chunk(qd, out, lens=lens_dev, gqa_mapping=gqa, flags=flags)
+            gpu.sync()
+            got = out.cpu().numpy()
+            for t in range(T):
+                wl_t = workloads.Workload("chunk", S, Hq, Hkv, d, [n - (T - 1 - t) for n in seen], kb, vb, ks, 0, 0)
+                want = checker_output(oracle, gpu, cache, wl_t, np.ascontiguousarray(q[:, t]), gqa_weed, Rk, Rv)
+                assert_attn_close(got[:, t], want, "%s position %d" % (what, t))
+
+    check(lens, None, "cached lengths")
+    shorter = [max(T, n - 37) for n in lens]
+    check(shorter, torch.tensor(shorter, dtype=torch.int32, device="cuda"), "explicit lengths")
+    # a chunk of one position is the single-query call
+    q1 = dev(np.ascontiguousarray(q[:, :1]))
+    out1 = torch.zeros_like(q1)
+    cache.decode_attn_chunk(q1, out1, gqa_mapping=gqa, flags=flags)
+    ref1 = torch.zeros_like(q1[:, 0])
+    cache.decode_attn(q1[:, 0], ref1, gqa_mapping=gqa, flags=flags)
+    assert torch.equal(out1[:, 0], ref1)
+    # more (position, head) pairs per KV head than a tile has rows
+    too_many = dev(np.zeros((S, 17, Hq, d), dtype=np.float32))
+    with pytest.raises(gpu.WeedHipError):
+        cache.decode_attn_chunk(too_many, torch.zeros_like(too_many), gqa_mapping=gqa)
+    cache.close()

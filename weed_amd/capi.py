@@ -93,6 +93,8 @@ SIGNATURES = {
                                         c_uint32]),
     "weed_hip_kv_decode_attn_prefix": (c_int, [c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_uint32, U32P, c_void_p,
                                                c_uint32, U32P, c_uint32]),
+    "weed_hip_kv_decode_attn_chunk": (c_int, [c_void_p, c_void_p, c_int32, c_int32, c_int32, c_void_p, c_uint32, U32P,
+                                              c_void_p, c_uint32, U32P, c_uint32]),
 }
 
 _lib = None
@@ -226,6 +228,20 @@ class KVCache:
         op, oo, os_ = _geom(out)
         check(self.lib.weed_hip_kv_decode_attn_prefix(self.handle, c_void_p(lens.data_ptr()), q.shape[1], gqa_mapping,
                                                       qp, qo, qs, op, oo, os_, flags))
+
+
+    def decode_attn_chunk(self, q, out, lens=None, gqa_mapping=GQA_WEED, flags=0):
+        """q, out: torch views of logical shape [n_seq, n_tokens, n_q_heads, d]; the last n_tokens of the attended
+        tokens (lens, or the cached lengths) are the chunk's own and are masked causally."""
+        assert q.dim() == 4 and q.shape == out.shape
+        qp, qo, qs = _geom(q)
+        op, oo, os_ = _geom(out)
+        lp = None
+        if lens is not None:
+            assert lens.element_size() == 4 and lens.is_cuda and lens.is_contiguous() and lens.numel() == q.shape[0]
+            lp = c_void_p(lens.data_ptr())
+        check(self.lib.weed_hip_kv_decode_attn_chunk(self.handle, lp, q.shape[1], q.shape[2], gqa_mapping, qp, qo, qs,
+                                                     op, oo, os_, flags))
 
 
 def use_torch_stream(stream):

@@ -24,10 +24,26 @@ constexpr int kGMax = 8;        // query heads of one kv head handled per pass
 constexpr int kThreads = 256;
 constexpr int kChunk = 256;     // tokens per inner iteration of the generic kernel
 
+// Strides of a (sequence, head, coordinate) tensor.  With `tokens` > 1 the "heads" the kernels see are (query
+// position, head) pairs of a multi-token chunk: virtual head hv stands for head hv / tokens at position hv % tokens
+// (blocked GQA: the pairs of one KV head stay together) or for head hv % heads at position hv / heads (Weed's
+// kv = h % Hkv, which the pairs then follow without change); `ts` is the stride between query positions.
 struct Geom3 {
     uint32_t off;
     uint32_t s[3];
+    uint32_t tokens, heads, ts;
+    int blocked;
 };
+
+__device__ __forceinline__ uint64_t head_offset(const Geom3 &g, uint32_t hv)
+{
+    if (g.tokens <= 1U) {
+        return (uint64_t)hv * g.s[1];
+    }
+    const uint32_t h = g.blocked ? hv / g.tokens : hv % g.heads;
+    const uint32_t t = g.blocked ? hv % g.tokens : hv / g.heads;
+    return (uint64_t)h * g.s[1] + (uint64_t)t * g.ts;
+}
 
 struct DecodeParams {
     SideParams k, v;
@@ -96,7 +112,7 @@ __global__ void __launch_bounds__(256) prep_q_kernel(const float *__restrict__ q
         block_offsets(lens, n_seq, blk_off);
     }
     if (tid < d) {
-        qs[tid] = q[(uint64_t)g.off + (uint64_t)s * g.s[0] + (uint64_t)h * g.s[1] + (uint64_t)tid * g.s[2]];
+        qs[tid] = q[(uint64_t)g.off + (uint64_t)s * g.s[0] + head_offset(g, h) + (uint64_t)tid * g.s[2]];
     }
     __syncthreads();
     float acc = 0.0f;
@@ -178,7 +194,7 @@ __global__ void __launch_bounds__(256) prep_q_rows_kernel(const float *__restric
         float v = 0.0f;
         if (row < n_rows && tid < d) {
             const uint32_t s = row / Hq, h = row % Hq;
-            v = q[(uint64_t)g.off + (uint64_t)s * g.s[0] + (uint64_t)h * g.s[1] + (uint64_t)tid * g.s[2]];
+            v = q[(uint64_t)g.off + (uint64_t)s * g.s[0] + head_offset(g, h) + (uint64_t)tid * g.s[2]];
         }
         qs[r][tid] = v;
     }
@@ -513,7 +529,7 @@ __global__ void combine_kernel(const float *__restrict__ partials, uint32_t Hq, 
     } else {
         r = o_sh[tid];
     }
-    out[(uint64_t)og.off + (uint64_t)s * og.s[0] + (uint64_t)h * og.s[1] + (uint64_t)tid * og.s[2]] = r;
+    out[(uint64_t)og.off + (uint64_t)s * og.s[0] + head_offset(og, h) + (uint64_t)tid * og.s[2]] = r;
 }
 
 // The same as combine_kernel for kRowsPerWg (sequence, head) rows per workgroup and at most 64 partials per row:
@@ -657,15 +673,18 @@ __global__ void __launch_bounds__(256) combine_rows_kernel(const float *__restri
         const uint32_t row = row0 + r;
         if (row < n_rows) {
             const uint32_t s = row / Hq, h = row % Hq;
-            out[(uint64_t)og.off + (uint64_t)s * og.s[0] + (uint64_t)h * og.s[1] + (uint64_t)tid * og.s[2]] = res[r];
+            out[(uint64_t)og.off + (uint64_t)s * og.s[0] + head_offset(og, h) + (uint64_t)tid * og.s[2]] = res[r];
         }
     }
 }
 
 // `lens_dev` (optional): attend over these per-sequence lengths instead of the cached ones.
+// `n_tokens` > 1: a chunk of query positions per sequence, the last `n_tokens` of the attended tokens being the
+// chunk's own (position t sees all but the last n_tokens - 1 - t); q_tstride / o_tstride step between positions.
 int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t gqa_mapping, const float *q_dev,
                 uint32_t q_off, const uint32_t q_stride[3], float *out_dev, uint32_t o_off, const uint32_t o_stride[3],
-                uint32_t flags, const int32_t *lens_dev)
+                uint32_t flags, const int32_t *lens_dev, uint32_t n_tokens = 1, uint32_t q_tstride = 0,
+                uint32_t o_tstride = 0)
 {
     WEED_HIP_REQUIRE(c, "%s: null cache", fn);
     WEED_HIP_REQUIRE(q_dev && out_dev && q_stride && o_stride, "%s: null pointer", fn);
@@ -676,7 +695,9 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
                      "%s: unknown GQA mapping %d", fn, gqa_mapping);
     const bool rot_q = flags & WEED_HIP_ATTN_ROTATE_Q, unrot = flags & WEED_HIP_ATTN_UNROTATE_OUT;
     WEED_HIP_REQUIRE(!(rot_q || unrot) || c->has_rotations, "%s: rotation requested but no rotations are set", fn);
-    const uint32_t Hq = (uint32_t)n_q_heads;
+    // the kernels see (position, head) pairs as heads
+    const uint32_t real_heads = (uint32_t)n_q_heads;
+    const uint32_t Hq = real_heads * n_tokens;
 
     uint32_t max_len = 0;
     for (int32_t l : c->lens) {
@@ -684,6 +705,9 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
     }
     const uint32_t G = Hq / Hkv;
     const bool use_mfma = mfma_decode_supported(d, c->k.w, c->v.w, G);
+    WEED_HIP_REQUIRE(n_tokens == 1 || use_mfma,
+                     "%s: %u positions x %u heads per KV head (at most 16 rows), head_dim %u: not served by the chunk kernel",
+                     fn, n_tokens, real_heads / Hkv, d);
     uint32_t n_splits, split_tokens = 0;
     uint32_t total_blocks = 0;
     RunGeom runs = { 1, 0, 8 };
@@ -756,8 +780,9 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
     uint32_t *blk_off = reinterpret_cast<uint32_t *>(wsp + q_bytes + 2 * h_bytes + 2 * s_bytes);
     float *partials = reinterpret_cast<float *>(wsp + q_bytes + 2 * h_bytes + 2 * s_bytes + off_bytes);
 
-    Geom3 qg = { q_off, { q_stride[0], q_stride[1], q_stride[2] } };
-    Geom3 og = { o_off, { o_stride[0], o_stride[1], o_stride[2] } };
+    const int blocked = gqa_mapping == WEED_HIP_GQA_BLOCKED ? 1 : 0;
+    Geom3 qg = { q_off, { q_stride[0], q_stride[1], q_stride[2] }, n_tokens, real_heads, q_tstride, blocked };
+    Geom3 og = { o_off, { o_stride[0], o_stride[1], o_stride[2] }, n_tokens, real_heads, o_tstride, blocked };
     const uint32_t n_rows = S * Hq;
     // the multi-row kernels pay off with many (sequence, head) rows; their rotation loops step by 64
     const bool many_rows = n_rows >= 512 && d % 64 == 0;
@@ -781,6 +806,8 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         mp.Hkv = Hkv;
         mp.G = G;
         mp.blocked = gqa_mapping == WEED_HIP_GQA_BLOCKED;
+        mp.q_tokens = n_tokens;
+        mp.real_group = real_heads / Hkv;
         mp.q_hi = q_hi;
         mp.q_lo = q_lo;
         mp.q_scale = q_scale;
@@ -848,4 +875,22 @@ extern "C" int weed_hip_kv_decode_attn_prefix(weed_hip_kv_cache *c, const int32_
     const char *fn = "weed_hip_kv_decode_attn_prefix";
     WEED_HIP_REQUIRE(lens_dev, "%s: null length array", fn);
     return decode_impl(fn, c, n_q_heads, gqa_mapping, q_dev, q_off, q_stride, out_dev, o_off, o_stride, flags, lens_dev);
+}
+
+extern "C" int weed_hip_kv_decode_attn_chunk(weed_hip_kv_cache *c, const int32_t *lens_dev, int32_t n_tokens,
+                                             int32_t n_q_heads, int32_t gqa_mapping, const float *q_dev, uint32_t q_off,
+                                             const uint32_t q_stride[4], float *out_dev, uint32_t o_off,
+                                             const uint32_t o_stride[4], uint32_t flags)
+{
+    const char *fn = "weed_hip_kv_decode_attn_chunk";
+    WEED_HIP_REQUIRE(q_stride && o_stride, "%s: null pointer", fn);
+    WEED_HIP_REQUIRE(n_tokens >= 1 && n_tokens <= 16, "%s: %d positions outside [1, 16]", fn, n_tokens);
+    if (c && !lens_dev) {
+        for (int32_t l : c->lens) {
+            WEED_HIP_REQUIRE(l >= n_tokens, "%s: a sequence holds %d tokens, fewer than the chunk's %d", fn, l, n_tokens);
+        }
+    }
+    const uint32_t qs3[3] = { q_stride[0], q_stride[2], q_stride[3] }, os3[3] = { o_stride[0], o_stride[2], o_stride[3] };
+    return decode_impl(fn, c, n_q_heads, gqa_mapping, q_dev, q_off, qs3, out_dev, o_off, os3, flags, lens_dev,
+                       (uint32_t)n_tokens, q_stride[1], o_stride[1]);
 }

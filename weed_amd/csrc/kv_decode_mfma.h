@@ -66,6 +66,10 @@ struct MfmaParams {
     uint32_t padded;
     uint32_t Hq, Hkv, G;
     int blocked;            // 1: kv = h / G, 0: kv = h % Hkv (Weed)
+    // multi-token chunks: the G "heads" of a KV head are (position, head) pairs, q_tokens positions x real_group
+    // heads; pair hc stands for position hc % q_tokens (blocked) or hc / real_group (Weed mapping), and position t
+    // does not see the last q_tokens - 1 - t tokens
+    uint32_t q_tokens, real_group;
     const uint16_t *q_hi;   // [n_seq][Hq][d] fp16 bits: high half of the scaled, normalised query
     const uint16_t *q_lo;   // [n_seq][Hq][d] fp16 bits: what the high half misses
     const float *q_scale;   // [n_seq][Hq] power of two the query was divided by

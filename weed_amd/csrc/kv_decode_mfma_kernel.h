@@ -345,6 +345,10 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
         }
     }
     const bool head_ok = hc < p.G;
+    // tokens at the end of the region that this lane's (position, head) pair does not see (0 unless the call is a
+    // multi-token chunk), and the largest such count over the pairs
+    const uint32_t hidden_max = p.q_tokens - 1U;
+    const uint32_t hidden = (hidden_max && head_ok) ? hidden_max - (p.blocked ? hc % p.q_tokens : hc / p.real_group) : 0U;
     const uint32_t qh_c = head_ok ? (p.blocked ? kvh * p.G + hc : hc * p.Hkv + kvh) : 0;
     const float qscale = head_ok ? p.q_scale[(uint64_t)seq * p.Hq + qh_c] : 0.0f;
     const float betaq = head_ok ? p.k.beta * p.q_sum[(uint64_t)seq * p.Hq + qh_c] : 0.0f;
@@ -446,12 +450,12 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
         if constexpr (NB == 1) {
             load_k(other, next_blk); // the K buffer is free again
         }
-        if (blk * 64 + 64 > L) {
+        if (blk * 64 + 64 + hidden_max > L) {
 #pragma unroll
             for (int s = 0; s < NSETS; ++s) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    if (blk * 64 + 16 * (s * TPS + tile_in_set) + 4 * g + r >= L) {
+                    if (blk * 64 + 16 * (s * TPS + tile_in_set) + 4 * g + r + hidden >= L) {
                         C[s][r] = -INFINITY;
                     }
                 }
@@ -486,7 +490,8 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
             }
             m_run = m_new;
         }
-        const float mm = m_run - (float)ep;
+        // (a chunk's early positions can have a whole block hidden before anything was seen: m_run is still -inf)
+        const float mm = (m_run == -INFINITY ? 0.0f : m_run) - (float)ep;
 
         // ---- probabilities (times V row scale, times 2^ep), split into fp16 hi + lo pairs ----
         uint32_t Phi[NSETS][2], Plo[NSETS][2];

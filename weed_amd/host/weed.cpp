@@ -1295,9 +1295,23 @@ TensorPtr MultiHeadAttention::forward_quantized(TensorPtr Q, TensorPtr K, Tensor
     }
     HipDevice::check(weed_hip_sync()); // earlier launches may still read the previous call's lengths
     HipDevice::check(weed_hip_memcpy_h2d(lens_dev, lens.data(), need));
-    for (tcapint t = 0U; t < uT; ++t) {
-        HipDevice::check(weed_hip_kv_decode_attn_prefix(cache, static_cast<const int32_t *>(lens_dev) + (size_t)t * uB,
-            num_heads, gqa, qp, Q->offset + t * uB, q_str, op, t * uB, q_str, flags));
+    // The (position, head) pairs of a KV head are the rows of one tile of the fused kernel (16 at most), so a few
+    // positions go through the cache together: position t0 + i of a group attends to before + t0 + i + 1 tokens, which
+    // is "the group's last length minus the positions after it".
+    const tcapint G = Hq / Hkv;
+    const tcapint per_call = (G <= 16U && (hd == 64U || hd == 128U)) ? std::max<tcapint>(1U, 16U / G) : 1U;
+    const uint32_t q_str4[4] = { Q->stride[0U], Q->stride[1U], Q->stride[2U], Q->stride[3U] };
+    const uint32_t o_str4[4] = { out->stride[0U], out->stride[1U], out->stride[2U], out->stride[3U] };
+    for (tcapint t = 0U; t < uT; t += per_call) {
+        const tcapint n = std::min(per_call, uT - t);
+        const int32_t *lens_t = static_cast<const int32_t *>(lens_dev) + (size_t)(t + n - 1U) * uB;
+        if (n == 1U) {
+            HipDevice::check(weed_hip_kv_decode_attn_prefix(cache, lens_t, num_heads, gqa, qp, Q->offset + t * Q->stride[1U],
+                q_str, op, t * out->stride[1U], q_str, flags));
+        } else {
+            HipDevice::check(weed_hip_kv_decode_attn_chunk(cache, lens_t, (int32_t)n, num_heads, gqa, qp,
+                Q->offset + t * Q->stride[1U], q_str4, op, t * out->stride[1U], o_str4, flags));
+        }
     }
     return out;
 }
