@@ -340,6 +340,16 @@ def main():
             },
             "whole_step_gbs": bytes_per_launch / (ms_per_step * 1e-3) / 1e9,
         }
+        if not args.no_extras:
+            # a chunk of 4 query positions per sequence in one pass over the same caches (speculative decoding)
+            S_, Hq_, d_ = q.shape
+            qc = torch.randn((S_, 4, Hq_, d_), device="cuda")
+            oc = torch.zeros_like(qc)
+            chunk_s = time_calls(torch, lambda: cache.decode_attn_chunk(qc, oc, None, capi.GQA_BLOCKED, flags),
+                                 min(args.steps, 20), min(args.warmup, 3))
+            result["chunk_of_4_positions"] = {"ms_per_call": 1e3 * chunk_s, "positions_per_s": 4 * wl.n_seq / chunk_s,
+                                              "vs_4_single_position_calls": 4 * ms_per_step * 1e-3 / chunk_s}
+            del qc, oc
         if single_ms is not None:
             result["single_sequence"] = {"ms_per_step": single_ms, "tokens_per_s": 1e3 / single_ms,
                                          "gbs": wl1.bytes_per_step(True) / (single_ms * 1e-3) / 1e9}
