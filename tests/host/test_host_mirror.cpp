@@ -527,7 +527,14 @@ void run_attention_case(KVCoder coder, int bits, bool blocked, uint32_t seed, bo
     (void)wv;
 
     tcapint before = 0U;
-    for (const tcapint T : { 7U, 1U, 1U, 3U, 12U }) { // prefill, two decode steps, a chunk, a long chunk (dense path)
+    // prefill, two decode steps, a chunk, a long chunk on the dense path, a long chunk in groups through the fused kernel
+    const std::pair<tcapint, MultiHeadAttention::PrefillPath> calls[] = { { 7U, MultiHeadAttention::PREFILL_AUTO },
+        { 1U, MultiHeadAttention::PREFILL_AUTO }, { 1U, MultiHeadAttention::PREFILL_AUTO },
+        { 3U, MultiHeadAttention::PREFILL_AUTO }, { 12U, MultiHeadAttention::PREFILL_DENSE },
+        { 9U, MultiHeadAttention::PREFILL_FUSED } };
+    for (const auto &call : calls) {
+        const tcapint T = call.first;
+        mha.prefill_path = call.second;
         const std::vector<real1> xv = gaussian((size_t)B * T * dm, seed + 100U + before);
         TensorPtr x = std::make_shared<Tensor>(xv, std::vector<tcapint>{ B, T, dm }, false, TEST_DTAG);
         TensorPtr y = mha.forward(x);
@@ -589,6 +596,20 @@ void run_attention_case(KVCoder coder, int bits, bool blocked, uint32_t seed, bo
     TensorPtr y = mha.forward(std::make_shared<Tensor>(gaussian(3U * dm, 1U), std::vector<tcapint>{ 3U, 1U, dm }, false, TEST_DTAG));
     REQUIRE(y->shape == (std::vector<tcapint>{ 3U, 1U, dm }));
     REQUIRE(mha.max_seq_len == (with_rope ? 40U : 2048U)); // the reference's default capacity (cpp:173)
+}
+
+TEST_CASE(test_prefill_path_estimate, true)
+{
+    // Llama-like shape, 3 + 4 bit rows: a few new tokens against long contexts stay on the packed cache, a long
+    // prefill of one sequence is dequantised once; forcing either path is covered by run_attention_case
+    MultiHeadAttention mha(4096U, 32U, 8U, 128U, TEST_DTAG, nullptr, ZERO_R1, -1, true, 4);
+    mha.kv_coder = KV_LLOYDMAX;
+    mha.k_bits = 3;
+    REQUIRE(!mha.dense_is_cheaper(64U, 4U, 8192U));
+    REQUIRE(!mha.dense_is_cheaper(64U, 64U, 8192U));
+    REQUIRE(!mha.dense_is_cheaper(1U, 8U, 300U));
+    REQUIRE(mha.dense_is_cheaper(1U, 4096U, 4096U));
+    REQUIRE(mha.dense_is_cheaper(8U, 2048U, 2048U));
 }
 
 TEST_CASE(test_attention_uniform_4bit, true) { run_attention_case(KV_UNIFORM, 4, false, 1234U); }

@@ -1224,7 +1224,9 @@ TensorPtr MultiHeadAttention::forward_quantized(TensorPtr Q, TensorPtr K, Tensor
         HipDevice::check(weed_hip_kv_decode_attn(cache, num_heads, gqa, qp, Q->offset, q_str, op, 0U, q_str, flags));
         return out;
     }
-    if (uT > kFusedQueryLimit) {
+    const bool fused_possible = (Hq / Hkv) <= 16U && (hd == 64U || hd == 128U);
+    if (prefill_path == PREFILL_DENSE || !fused_possible ||
+        (prefill_path == PREFILL_AUTO && dense_is_cheaper(uB, uT, cache_len))) {
         // Long multi-token calls (prefill): the fused kernel serves one query position per launch, so beyond a few
         // positions it is cheaper to do what the reference does -- dequantise the cache once (still in the rotated
         // basis) and run dense ops: rotate Q, product, / sqrt(d), + mask, softmax, product, un-rotate
@@ -1299,7 +1301,7 @@ TensorPtr MultiHeadAttention::forward_quantized(TensorPtr Q, TensorPtr K, Tensor
     // positions go through the cache together: position t0 + i of a group attends to before + t0 + i + 1 tokens, which
     // is "the group's last length minus the positions after it".
     const tcapint G = Hq / Hkv;
-    const tcapint per_call = (G <= 16U && (hd == 64U || hd == 128U)) ? std::max<tcapint>(1U, 16U / G) : 1U;
+    const tcapint per_call = std::max<tcapint>(1U, 16U / G);
     const uint32_t q_str4[4] = { Q->stride[0U], Q->stride[1U], Q->stride[2U], Q->stride[3U] };
     const uint32_t o_str4[4] = { out->stride[0U], out->stride[1U], out->stride[2U], out->stride[3U] };
     for (tcapint t = 0U; t < uT; t += per_call) {
@@ -1314,6 +1316,26 @@ TensorPtr MultiHeadAttention::forward_quantized(TensorPtr Q, TensorPtr K, Tensor
         }
     }
     return out;
+}
+
+// Rough device times of the two ways to serve T new tokens against L cached ones (measured on MI355X: a pass of the
+// fused kernel costs about 55 us plus the packed bytes at 5 TB/s; the dense path is a dozen launches (200 us), writes
+// and re-reads fp32 K and V, runs two batched fp32 products at 60 TFLOP/s and walks the [B, heads, T, L] scores seven
+// times at 4 TB/s).
+bool MultiHeadAttention::dense_is_cheaper(tcapint B, tcapint T, tcapint L) const
+{
+    const double Hkv = (double)num_kv_heads, Hq = (double)num_heads, hd = (double)head_dim;
+    const double kb = (double)(k_bits ? k_bits : kv_quant_bits) + (k_sign ? 1.0 : 0.0);
+    const double vb = (double)(v_bits ? v_bits : kv_quant_bits) + (v_sign ? 1.0 : 0.0);
+    const double packed = (double)B * Hkv * (double)L * (hd * (kb + vb) / 8.0 + 8.0);
+    const double per_call = std::max(1.0, std::floor(16.0 / (Hq / Hkv)));
+    const double passes = std::ceil((double)T / per_call);
+    const double fused_us = passes * (55.0 + packed / 5.0e6);
+    const double deq_bytes = (double)B * Hkv * (double)L * hd * 4.0 * 2.0;
+    const double flops = 2.0 * 2.0 * (double)B * Hq * (double)T * (double)L * hd;
+    const double score_bytes = (double)B * Hq * (double)T * (double)L * 4.0 * 7.0;
+    const double dense_us = 200.0 + deq_bytes / 3.0e6 + flops / 60.0e6 + score_bytes / 4.0e6;
+    return dense_us < fused_us;
 }
 
 // Float cache or no cache: the reference's own sequence of dense ops (multihead_attention.cpp:279-340), each one a

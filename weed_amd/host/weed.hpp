@@ -386,6 +386,12 @@ struct MultiHeadAttention : public Module {
     int k_bits = 0, v_bits = 0; // 0: use kv_quant_bits
     bool k_sign = false, v_sign = false;
     bool gqa_blocked = false; // false: kv head = q head % num_kv_heads, the reference's mapping (cpp:291-311)
+    // How a call with several new tokens attends over the quantised cache.  FUSED: groups of up to 16 / (heads per KV
+    // head) positions per pass of the fused kernel over the packed rows.  DENSE: what the reference does -- dequantise
+    // the cache once, then dense products, mask, softmax (multihead_attention.cpp:259-340).  AUTO picks by estimated
+    // cost: short chunks against a long context go FUSED, a long prefill goes DENSE.
+    enum PrefillPath { PREFILL_AUTO = 0, PREFILL_FUSED = 1, PREFILL_DENSE = 2 };
+    PrefillPath prefill_path = PREFILL_AUTO;
     uint32_t rotation_seed = 0U;
 
     std::vector<ParameterPtr> param_vector;
@@ -410,13 +416,15 @@ struct MultiHeadAttention : public Module {
     void set_max_kv_seq_len(tcapint m) override { max_seq_len = m; }
     void reset_cache() override;
     TensorPtr forward(const TensorPtr x) override;
+    // PREFILL_AUTO's rule for B sequences, T new tokens and L cached ones (the new ones included): true when
+    // dequantising once and attending densely is estimated cheaper than the passes of the fused kernel
+    bool dense_is_cheaper(tcapint B, tcapint T, tcapint L) const;
 
 private:
     TensorPtr forward_quantized(TensorPtr Q, TensorPtr K, TensorPtr V, symint B, symint T);
     TensorPtr forward_dense(TensorPtr Q, TensorPtr K, TensorPtr V, symint B, symint T);
     TensorPtr attend_dense(TensorPtr Q, TensorPtr K, TensorPtr V, tcapint before);
     std::shared_ptr<GpuRealStorage> k_rot_dev, v_rot_dev, v_rot_t_dev; // device copies of the rotations
-    static constexpr tcapint kFusedQueryLimit = 8U; // multi-token calls up to this many positions use the fused kernel
     void *lens_dev = nullptr; // int32 prefix lengths for multi-token calls
     size_t lens_cap = 0U;
 
