@@ -251,6 +251,14 @@ int weed_hip_kv_export_fields(const weed_hip_kv_cache *cache, int which, int32_t
 int weed_hip_kv_export_weed_words(const weed_hip_kv_cache *cache, int which, int32_t seq_begin, int32_t seq_count,
                                   int32_t tok_begin, int32_t T, int32_t *words_dev);
 
+/* The reverse of weed_hip_kv_export_weed_words: append T_new tokens per sequence whose rows arrive already coded in
+ * Weed's word packing (QuantizedKVCache::packed as write_row leaves it, multihead_attention.cpp:43-62; both arrays
+ * [seq_count][n_kv_heads][T_new][words per row], on the device).  A cache built by the reference on another device is
+ * moved over this way without a round trip through floats; set the two block scales with
+ * weed_hip_kv_cache_set_scales first.  UNIFORM mode only. */
+int weed_hip_kv_append_weed_words(weed_hip_kv_cache *cache, int32_t seq_begin, int32_t seq_count, int32_t T_new,
+                                  const int32_t *k_words_dev, const int32_t *v_words_dev);
+
 /* Fused single-query decode attention over the packed cache: everything MultiHeadAttention::forward does between
  * the cache rebuild and the output projection for T = 1 (multihead_attention.cpp:259-348): un-pack, Q.K^T,
  * /sqrt(d), softmax over each sequence's own length (split over the context and merged), P.V, un-rotate.

@@ -53,6 +53,70 @@ def test_uniform_known_answers_on_device(gpu, oracle):
     cache.close()
 
 
+@pytest.mark.parametrize("kbits,vbits,d", [(4, 4, 64), (3, 2, 128), (2, 3, 32)])
+def test_rows_in_weeds_word_packing_are_appended_as_they_are(gpu, oracle, kbits, vbits, d):
+    """Rows that arrive already coded in Weed's word packing (what the reference's write_row leaves in
+    QuantizedKVCache::packed; the words here come from the checker's write_row, which the recorded answers pin) are
+    appended without a round trip through floats: in one call and token by token, the cache then holds exactly the
+    codes of the float path, exports the same words, dequantises to read_row's floats and attends identically."""
+    import torch
+    rng = np.random.default_rng(kbits * 10 + vbits + d)
+    S, Hkv, T = 2, 3, 70
+    K = rng.normal(0, 1.1, size=(S, Hkv, T, d)).astype(np.float32)
+    V = rng.normal(0, 0.8, size=(S, Hkv, T, d)).astype(np.float32)
+    ks, vs = oracle.block_scale(K), oracle.block_scale(V)
+    k_words = oracle.uniform_write_rows(K.reshape(-1, d), kbits, ks).reshape(S, Hkv, T, -1)
+    v_words = oracle.uniform_write_rows(V.reshape(-1, d), vbits, vs).reshape(S, Hkv, T, -1)
+
+    ref = gpu.KVCache(gpu.KV_UNIFORM, S, Hkv, d, 100, kbits, vbits)
+    ref.set_scales(ks, vs)
+    ref.encode_append(dev(K), dev(V), rotate=0)
+    want = [export(ref, which, T)[0] for which in (0, 1)]
+    q = dev(rng.standard_normal((S, 2 * Hkv, d), dtype=np.float32))
+    want_out = torch.zeros_like(q)
+    ref.decode_attn(q, want_out)
+
+    for pieces in ([T], [1] * 5 + [64, 1]):
+        cache = gpu.KVCache(gpu.KV_UNIFORM, S, Hkv, d, 100, kbits, vbits)
+        cache.set_scales(ks, vs)
+        t0 = 0
+        for n in pieces:
+            kw = torch.from_numpy(np.ascontiguousarray(k_words[:, :, t0:t0 + n])).cuda()
+            vw = torch.from_numpy(np.ascontiguousarray(v_words[:, :, t0:t0 + n])).cuda()
+            cache.append_weed_words(kw, vw)
+            t0 += n
+        assert cache.seq_lens() == [T] * S
+        for which, words in ((0, k_words), (1, v_words)):
+            np.testing.assert_array_equal(export(cache, which, T)[0], want[which])
+            back = torch.zeros(words.shape, dtype=torch.int32, device="cuda")
+            cache.export_weed_words(which, back)
+            np.testing.assert_array_equal(back.cpu().numpy(), words)
+        deq = torch.zeros((S, Hkv, T, d), device="cuda")
+        cache.dequant(0, deq)
+        np.testing.assert_array_equal(deq.cpu().numpy().reshape(-1, d),
+                                      oracle.uniform_read_rows(k_words.reshape(-1, k_words.shape[-1]), d, kbits, ks))
+        out = torch.zeros_like(q)
+        cache.decode_attn(q, out)
+        assert torch.equal(out, want_out)
+        # one sequence only, and the error paths
+        cache.reset()
+        cache.set_scales(ks, vs)
+        kw1 = torch.from_numpy(np.ascontiguousarray(k_words[1:2])).cuda()
+        vw1 = torch.from_numpy(np.ascontiguousarray(v_words[1:2])).cuda()
+        cache.append_weed_words(kw1, vw1, seq_begin=1)
+        assert cache.seq_lens() == [0, T]
+        np.testing.assert_array_equal(export(cache, 0, T)[0][1], want[0][1])
+        with pytest.raises(gpu.WeedHipError):
+            cache.append_weed_words(kw1, vw1, seq_begin=1)  # 140 tokens > capacity 100
+        cache.close()
+    lm = gpu.KVCache(gpu.KV_LLOYDMAX, S, Hkv, max(d, 32), 100, 3, 3)
+    with pytest.raises(gpu.WeedHipError):
+        lm.append_weed_words(torch.zeros((S, Hkv, 1, 16), dtype=torch.int32, device="cuda"),
+                             torch.zeros((S, Hkv, 1, 16), dtype=torch.int32, device="cuda"))
+    lm.close()
+    ref.close()
+
+
 @pytest.mark.parametrize("bits", [2, 3, 4])
 @pytest.mark.parametrize("d", [64, 128])
 def test_uniform_encode_bit_exact(gpu, oracle, bits, d):

@@ -89,6 +89,7 @@ SIGNATURES = {
     "weed_hip_kv_dequant": (c_int, [c_void_p, c_int, c_int32, c_int32, c_int32, c_int32, c_void_p, c_uint32, U32P]),
     "weed_hip_kv_export_fields": (c_int, [c_void_p, c_int, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
     "weed_hip_kv_export_weed_words": (c_int, [c_void_p, c_int, c_int32, c_int32, c_int32, c_int32, c_void_p]),
+    "weed_hip_kv_append_weed_words": (c_int, [c_void_p, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
     "weed_hip_kv_decode_attn": (c_int, [c_void_p, c_int32, c_int32, c_void_p, c_uint32, U32P, c_void_p, c_uint32, U32P,
                                         c_uint32]),
     "weed_hip_kv_decode_attn_prefix": (c_int, [c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_uint32, U32P, c_void_p,
@@ -212,6 +213,12 @@ class KVCache:
         assert words.is_contiguous()
         check(self.lib.weed_hip_kv_export_weed_words(self.handle, which, seq_begin, words.shape[0], tok_begin,
                                                      words.shape[2], c_void_p(words.data_ptr())))
+
+    def append_weed_words(self, k_words, v_words, seq_begin=0):
+        """k_words, v_words: contiguous int32 torch tensors [seq_count, n_kv_heads, T_new, words per row]."""
+        assert k_words.is_contiguous() and v_words.is_contiguous() and k_words.shape[:3] == v_words.shape[:3]
+        check(self.lib.weed_hip_kv_append_weed_words(self.handle, seq_begin, k_words.shape[0], k_words.shape[2],
+                                                     c_void_p(k_words.data_ptr()), c_void_p(v_words.data_ptr())))
 
     def decode_attn(self, q, out, gqa_mapping=GQA_WEED, flags=0):
         """q, out: torch views of logical shape [n_seq, n_q_heads, d]."""

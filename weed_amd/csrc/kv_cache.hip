@@ -563,6 +563,22 @@ __global__ void weed_words_kernel(SideParams sp, int which, uint32_t Hkv, uint32
     words[idx] = (int32_t)word;
 }
 
+// The reverse: rows in Weed's word packing become one code per byte, rows in (sequence, head, token) order.
+__global__ void fields_from_words_kernel(const int32_t *__restrict__ words, uint64_t rows, uint32_t d, uint32_t bits,
+                                         uint8_t *__restrict__ fields)
+{
+    const uint32_t vpw = 32 / bits;
+    const uint32_t wpr = (d + vpw - 1) / vpw;
+    const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= rows * d) {
+        return;
+    }
+    const uint64_t row = idx / d;
+    const uint32_t j = (uint32_t)(idx - row * d);
+    const uint32_t word = (uint32_t)words[row * wpr + j / vpw];
+    fields[idx] = (uint8_t)((word >> ((j % vpw) * bits)) & ((1u << bits) - 1u));
+}
+
 // sum of squares: tree reduction (one partial per block, finished on the host in double)
 __global__ void sumsq_kernel(const float *__restrict__ x, Geom4 g, uint32_t n1, uint32_t n2, uint32_t n3, uint64_t total,
                              double *__restrict__ partials)
@@ -660,6 +676,8 @@ EncSide enc_side_args(const weed_hip_kv_cache *c, const Side &side, const float 
 
 // Rotate, quantise and pack the new K and V rows: one launch for the two encoders, one for the three packing steps.
 // The scratch holds the K rows first, then the V rows.
+int pack_rows(weed_hip_kv_cache *c, int32_t seq_begin, int32_t seq_count, int32_t T_new);
+
 int encode_both(weed_hip_kv_cache *c, int32_t seq_begin, int32_t seq_count, int32_t T_new, const float *k_dev,
                 uint32_t k_off, const uint32_t k_stride[4], const float *v_dev, uint32_t v_off,
                 const uint32_t v_stride[4], int rotate)
@@ -704,6 +722,18 @@ int encode_both(weed_hip_kv_cache *c, int32_t seq_begin, int32_t seq_count, int3
         }
         WEED_HIP_LAUNCH_CHECK();
     }
+    return pack_rows(c, seq_begin, seq_count, T_new);
+}
+
+// Second stage of an append: the one-field-per-byte rows in the scratch buffers (K rows, then V rows, each in
+// (sequence, head, token) order) go into the block layout behind the tokens already cached.
+int pack_rows(weed_hip_kv_cache *c, int32_t seq_begin, int32_t seq_count, int32_t T_new)
+{
+    const uint32_t d = (uint32_t)c->cfg.head_dim;
+    const uint32_t Hkv = (uint32_t)c->cfg.n_kv_heads;
+    const uint32_t rows = (uint32_t)seq_count * Hkv * (uint32_t)T_new;
+    uint8_t *k_fields = c->enc_fields, *v_fields = c->enc_fields + (size_t)rows * d;
+    float *k_alpha = c->enc_alpha, *v_alpha = c->enc_alpha + rows;
     ProfileScope prof("kv_pack");
     const bool scales = c->cfg.mode == WEED_HIP_KV_LLOYDMAX;
     PackArgs a;
@@ -737,6 +767,39 @@ int encode_both(weed_hip_kv_cache *c, int32_t seq_begin, int32_t seq_count, int3
     const uint32_t blocks_s = scales ? (rows + 255) / 256 : 0;
     pack_all_kernel<<<a.blocks_k + a.blocks_v + blocks_s, 256, 0, stream()>>>(a);
     WEED_HIP_LAUNCH_CHECK();
+    return WEED_HIP_OK;
+}
+
+// Scratch for the rows of one append (K rows, then V rows): grows as needed.
+int reserve_append_scratch(weed_hip_kv_cache *c, const char *fn, int32_t seq_count, int32_t T_new)
+{
+    const uint64_t rows64 = (uint64_t)seq_count * c->cfg.n_kv_heads * T_new;
+    WEED_HIP_REQUIRE(rows64 * c->cfg.head_dim < (1ull << 32), "%s: more than 2^32 elements in one call", fn);
+    const size_t rows = (size_t)rows64;
+    if (rows > c->enc_rows_cap) {
+        WEED_HIP_CHECK(hipStreamSynchronize(stream()));
+        (void)hipFree(c->enc_fields);
+        (void)hipFree(c->enc_alpha);
+        c->enc_fields = nullptr;
+        c->enc_alpha = nullptr;
+        c->enc_rows_cap = 0;
+        if (hipMalloc((void **)&c->enc_fields, 2 * rows * c->cfg.head_dim) != hipSuccess ||
+            hipMalloc((void **)&c->enc_alpha, 2 * rows * sizeof(float)) != hipSuccess) {
+            return fail(WEED_HIP_ENOMEM, "%s: scratch allocation failed", fn);
+        }
+        c->enc_rows_cap = rows;
+    }
+    return WEED_HIP_OK;
+}
+
+// The appended tokens become visible: device and host copies of the lengths move on.
+int finish_append(weed_hip_kv_cache *c, int32_t seq_begin, int32_t seq_count, int32_t T_new)
+{
+    bump_lens_kernel<<<((uint32_t)seq_count + 255) / 256, 256, 0, stream()>>>(c->lens_dev, seq_begin, seq_count, T_new);
+    WEED_HIP_LAUNCH_CHECK();
+    for (int32_t s = 0; s < seq_count; ++s) {
+        c->lens[(size_t)(seq_begin + s)] += T_new;
+    }
     return WEED_HIP_OK;
 }
 
@@ -1095,30 +1158,40 @@ int weed_hip_kv_encode_append(weed_hip_kv_cache *c, int32_t seq_begin, int32_t s
                         c->lens[(size_t)(seq_begin + s)] + T_new, c->cfg.max_tokens);
         }
     }
-    const uint64_t rows64 = (uint64_t)seq_count * c->cfg.n_kv_heads * T_new;
-    WEED_HIP_REQUIRE(rows64 * c->cfg.head_dim < (1ull << 32), "%s: more than 2^32 elements in one call", fn);
-    const size_t rows = (size_t)rows64;
-    if (rows > c->enc_rows_cap) {
-        WEED_HIP_CHECK(hipStreamSynchronize(stream()));
-        (void)hipFree(c->enc_fields);
-        (void)hipFree(c->enc_alpha);
-        c->enc_fields = nullptr;
-        c->enc_alpha = nullptr;
-        c->enc_rows_cap = 0;
-        // K rows, then V rows
-        if (hipMalloc((void **)&c->enc_fields, 2 * rows * c->cfg.head_dim) != hipSuccess ||
-            hipMalloc((void **)&c->enc_alpha, 2 * rows * sizeof(float)) != hipSuccess) {
-            return fail(WEED_HIP_ENOMEM, "%s: scratch allocation failed", fn);
-        }
-        c->enc_rows_cap = rows;
-    }
+    WEED_HIP_TRY(reserve_append_scratch(c, fn, seq_count, T_new));
     WEED_HIP_TRY(encode_both(c, seq_begin, seq_count, T_new, k_dev, k_off, k_stride, v_dev, v_off, v_stride, rotate));
-    bump_lens_kernel<<<((uint32_t)seq_count + 255) / 256, 256, 0, stream()>>>(c->lens_dev, seq_begin, seq_count, T_new);
-    WEED_HIP_LAUNCH_CHECK();
-    for (int32_t s = 0; s < seq_count; ++s) {
-        c->lens[(size_t)(seq_begin + s)] += T_new;
+    return finish_append(c, seq_begin, seq_count, T_new);
+}
+
+int weed_hip_kv_append_weed_words(weed_hip_kv_cache *c, int32_t seq_begin, int32_t seq_count, int32_t T_new,
+                                  const int32_t *k_words_dev, const int32_t *v_words_dev)
+{
+    const char *fn = "weed_hip_kv_append_weed_words";
+    WEED_HIP_TRY(check_cache(c, fn));
+    WEED_HIP_TRY(check_range(c, fn, seq_begin, seq_count));
+    WEED_HIP_REQUIRE(c->cfg.mode == WEED_HIP_KV_UNIFORM, "%s: Weed's word packing exists for the uniform coder only", fn);
+    WEED_HIP_REQUIRE(T_new >= 0, "%s: negative token count", fn);
+    if (!seq_count || !T_new) {
+        return WEED_HIP_OK;
     }
-    return WEED_HIP_OK;
+    WEED_HIP_REQUIRE(k_words_dev && v_words_dev, "%s: null pointer", fn);
+    for (int32_t s = 0; s < seq_count; ++s) {
+        if (c->lens[(size_t)(seq_begin + s)] + T_new > c->cfg.max_tokens) {
+            return fail(WEED_HIP_ECAPACITY, "%s: sequence %d would hold %d tokens, capacity is %d", fn, seq_begin + s,
+                        c->lens[(size_t)(seq_begin + s)] + T_new, c->cfg.max_tokens);
+        }
+    }
+    WEED_HIP_TRY(reserve_append_scratch(c, fn, seq_count, T_new));
+    const uint32_t d = (uint32_t)c->cfg.head_dim;
+    const uint64_t rows = (uint64_t)seq_count * c->cfg.n_kv_heads * T_new;
+    const uint32_t blocks = (uint32_t)((rows * d + 255) / 256);
+    fields_from_words_kernel<<<blocks, 256, 0, stream()>>>(k_words_dev, rows, d, (uint32_t)c->k.bits, c->enc_fields);
+    WEED_HIP_LAUNCH_CHECK();
+    fields_from_words_kernel<<<blocks, 256, 0, stream()>>>(v_words_dev, rows, d, (uint32_t)c->v.bits,
+                                                           c->enc_fields + rows * d);
+    WEED_HIP_LAUNCH_CHECK();
+    WEED_HIP_TRY(pack_rows(c, seq_begin, seq_count, T_new));
+    return finish_append(c, seq_begin, seq_count, T_new);
 }
 
 int weed_hip_kv_dequant(const weed_hip_kv_cache *c, int which, int32_t seq_begin, int32_t seq_count, int32_t tok_begin,
