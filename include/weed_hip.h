@@ -189,8 +189,8 @@ typedef struct {
     int32_t n_kv_heads;    /* Hkv                                                                             */
     int32_t head_dim;      /* d, a multiple of 32, at most 256                                                 */
     int32_t max_tokens;    /* capacity per sequence (Weed: max_seq_len)                                        */
-    int32_t k_bits;        /* code bits for keys, 1..4                                                         */
-    int32_t v_bits;        /* code bits for values, 1..4                                                       */
+    int32_t k_bits;        /* code bits for keys: 1..8 (UNIFORM, any kv_quant_bits of the reference), 1..4 (LLOYDMAX) */
+    int32_t v_bits;        /* code bits for values, likewise                                                   */
     int32_t k_sign;        /* 1: keep a residual sign bit per key coordinate (LLOYDMAX only)                   */
     int32_t v_sign;        /* 1: same for values                                                              */
 } weed_hip_kv_config;

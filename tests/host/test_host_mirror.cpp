@@ -616,6 +616,9 @@ TEST_CASE(test_attention_uniform_4bit, true) { run_attention_case(KV_UNIFORM, 4,
 TEST_CASE(test_attention_uniform_3bit_blocked_gqa, true) { run_attention_case(KV_UNIFORM, 3, true, 99U); }
 TEST_CASE(test_attention_lloydmax, true) { run_attention_case(KV_LLOYDMAX, 4, false, 4321U); }
 TEST_CASE(test_attention_with_rope, true) { run_attention_case(KV_LLOYDMAX, 4, false, 777U, true); }
+// 8-bit codes (any kv_quant_bits the reference takes): no matrix-core tiles for such fields, every call goes through
+// the generic kernel position by position, or densely
+TEST_CASE(test_attention_uniform_8bit, true) { run_attention_case(KV_UNIFORM, 8, true, 31U); }
 
 TEST_CASE(test_attention_uniform_codes_follow_reference_coder, true)
 {

@@ -21,10 +21,10 @@ using namespace weedkv;
 int main()
 {
     // items: 8 fields of w bits in w bytes
-    for (uint32_t w = 1; w <= 5; ++w) {
+    for (uint32_t w = 1; w <= 8; ++w) {
         std::srand(w);
         for (int trial = 0; trial < 200; ++trial) {
-            uint8_t f8[8], bytes[8] = { 0 };
+            uint8_t f8[8], bytes[9] = { 0 };
             for (uint32_t e = 0; e < 8; ++e) {
                 f8[e] = (uint8_t)(std::rand() & ((1 << w) - 1));
             }
@@ -44,7 +44,7 @@ int main()
     // tokens, no byte of a region is wasted
     const uint32_t dims[] = { 32, 64, 96, 128, 256 };
     for (uint32_t d : dims) {
-        for (uint32_t w = 1; w <= 5; ++w) {
+        for (uint32_t w = 1; w <= 8; ++w) {
             const uint32_t max_tokens = 200; // 4 blocks after padding
             const uint64_t region = region_bytes(max_tokens, d, w);
             CHECK(padded_tokens(max_tokens) == 256);

@@ -261,6 +261,31 @@ def test_head_dims_and_wide_groups(gpu, oracle):
         cache.close()
 
 
+@pytest.mark.parametrize("kb,vb,d", [(8, 8, 128), (5, 6, 64), (8, 4, 128), (1, 7, 32)])
+def test_uniform_widths_beyond_four_bits(gpu, oracle, kb, vb, d):
+    """Weed's uniform coder at any width the reference's `kv_quant_bits` may take (an 8-bit cache is the common
+    request): attention equals the checker on the same codes, with rotations, both GQA mappings and an append."""
+    import torch
+    rng = np.random.default_rng(kb * 16 + vb + d)
+    Hkv, Hq, lens = 2, 8, [300, 77, 64]
+    S = len(lens)
+    wl = workloads.Workload("wide", S, Hq, Hkv, d, lens, kb, vb, 0, 0, 0)
+    K = rng.standard_normal((S, Hkv, max(lens), d), dtype=np.float32)
+    V = rng.standard_normal((S, Hkv, max(lens), d), dtype=np.float32)
+    q = rng.standard_normal((S, Hq, d), dtype=np.float32)
+    Rk, Rv = rotations(oracle, d, kb)
+    cache = build_cache(gpu, wl, gpu.KV_UNIFORM, K, V, (Rk, Rv), (1.1, 0.9), rotate=2)
+    flags = gpu.ATTN_ROTATE_Q | gpu.ATTN_UNROTATE_OUT
+    for gqa, weed in ((gpu.GQA_WEED, True), (gpu.GQA_BLOCKED, False)):
+        want = checker_output(oracle, gpu, cache, wl, q, weed, Rk, Rv)
+        got = run_decode(gpu, cache, q, gqa, flags)
+        assert_attn_close(got, want, "K %d-bit V %d-bit" % (kb, vb))
+    # the codes really use the whole range
+    kf, _ = export(cache, 0, 64)
+    assert kf.max() == (1 << kb) - 1 and kf.min() == 0
+    cache.close()
+
+
 def test_prefix_lengths_override(gpu, oracle):
     """Attention over the first n tokens of each cached sequence (the per-position form of a causal mask) equals the
     checker run with those lengths; the cache's own lengths are untouched."""

@@ -53,7 +53,7 @@ def test_uniform_known_answers_on_device(gpu, oracle):
     cache.close()
 
 
-@pytest.mark.parametrize("kbits,vbits,d", [(4, 4, 64), (3, 2, 128), (2, 3, 32)])
+@pytest.mark.parametrize("kbits,vbits,d", [(4, 4, 64), (3, 2, 128), (2, 3, 32), (8, 8, 64), (5, 7, 128)])
 def test_rows_in_weeds_word_packing_are_appended_as_they_are(gpu, oracle, kbits, vbits, d):
     """Rows that arrive already coded in Weed's word packing (what the reference's write_row leaves in
     QuantizedKVCache::packed; the words here come from the checker's write_row, which the recorded answers pin) are
@@ -117,7 +117,7 @@ def test_rows_in_weeds_word_packing_are_appended_as_they_are(gpu, oracle, kbits,
     ref.close()
 
 
-@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("bits", [1, 2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("d", [64, 128])
 def test_uniform_encode_bit_exact(gpu, oracle, bits, d):
     import torch

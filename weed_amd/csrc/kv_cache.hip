@@ -63,6 +63,9 @@ float round_to_half(float x)
 
 void load_builtin(Side &s)
 {
+    if (s.bits > 4) {
+        return; // uniform coder only: its cells are arithmetic, no table
+    }
     const BuiltinTable t = builtin_table(s.bits);
     const int n = 1 << s.bits;
     std::memcpy(s.levels, t.levels, sizeof(float) * n);
@@ -365,7 +368,7 @@ __device__ __forceinline__ void pack_k_body(const uint8_t *__restrict__ fields, 
     const uint32_t it = idx % items, row = idx / items;
     const uint32_t t = row % T, h = (row / T) % Hkv, s = row / (T * Hkv);
     const uint32_t n = (uint32_t)lens[seq_begin + s] + t;
-    uint8_t bytes[5];
+    uint8_t bytes[8];
     item_build(fields + (uint64_t)row * d + it * 8, w, bytes);
     const uint64_t region = (uint64_t)(seq_begin + s) * Hkv + h;
     uint8_t *dst = out + region * region_bytes + k_field_pos(n, it * 8, d, w).byte;
@@ -455,7 +458,7 @@ __device__ __forceinline__ void pack_v_body(const uint8_t *__restrict__ fields, 
     if (!touched) {
         return;
     }
-    uint8_t bytes[5];
+    uint8_t bytes[8];
     item_build(f8, w, bytes);
     for (uint32_t b = 0; b < w; ++b) {
         dst[b] = bytes[b];
@@ -881,9 +884,12 @@ int weed_hip_kv_cache_create(weed_hip_kv_cache **cache, const weed_hip_kv_config
                      "weed_hip_kv_cache_create: n_seq, n_kv_heads and max_tokens must be positive");
     WEED_HIP_REQUIRE(cfg->head_dim >= 32 && cfg->head_dim <= 256 && cfg->head_dim % 32 == 0,
                      "weed_hip_kv_cache_create: head_dim %d must be a multiple of 32 in [32, 256]", cfg->head_dim);
-    WEED_HIP_REQUIRE(cfg->k_bits >= 1 && cfg->k_bits <= 4 && cfg->v_bits >= 1 && cfg->v_bits <= 4,
-                     "weed_hip_kv_cache_create: code widths must be 1..4 bits (got K %d, V %d)", cfg->k_bits,
-                     cfg->v_bits);
+    // Weed's uniform coder takes any width that divides into its 32-bit words sensibly; the Lloyd-Max tables exist
+    // for 1..4 bits
+    const int max_bits = cfg->mode == WEED_HIP_KV_UNIFORM ? 8 : 4;
+    WEED_HIP_REQUIRE(cfg->k_bits >= 1 && cfg->k_bits <= max_bits && cfg->v_bits >= 1 && cfg->v_bits <= max_bits,
+                     "weed_hip_kv_cache_create: code widths must be 1..%d bits in this mode (got K %d, V %d)", max_bits,
+                     cfg->k_bits, cfg->v_bits);
     WEED_HIP_REQUIRE((cfg->k_sign == 0 || cfg->k_sign == 1) && (cfg->v_sign == 0 || cfg->v_sign == 1),
                      "weed_hip_kv_cache_create: sign flags must be 0 or 1");
     WEED_HIP_REQUIRE(cfg->mode == WEED_HIP_KV_LLOYDMAX || (!cfg->k_sign && !cfg->v_sign),
@@ -1069,6 +1075,7 @@ int weed_hip_kv_cache_get_tables(const weed_hip_kv_cache *c, int which, float *b
     WEED_HIP_TRY(check_cache(c, "weed_hip_kv_cache_get_tables"));
     WEED_HIP_REQUIRE(which == 0 || which == 1, "weed_hip_kv_cache_get_tables: which must be 0 or 1");
     const Side &s = which ? c->v : c->k;
+    WEED_HIP_REQUIRE(s.bits <= 4, "weed_hip_kv_cache_get_tables: there are no tables for %d-bit codes", s.bits);
     const int n = 1 << s.bits;
     if (bounds) {
         std::memcpy(bounds, s.bounds, sizeof(float) * (n - 1));

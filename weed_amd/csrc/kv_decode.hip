@@ -271,7 +271,7 @@ __global__ void __launch_bounds__(kThreads) decode_generic_kernel(DecodeParams p
     __shared__ float sc[kGMax * kChunk];
     __shared__ float m_s[kGMax], l_s[kGMax], scale_s[kGMax];
     __shared__ float o_s[kGMax * 256];
-    __shared__ float ktab[32], vtab[32];
+    __shared__ float ktab[256], vtab[256];
 
     const uint32_t split = blockIdx.x, kvh = blockIdx.y, seq = blockIdx.z;
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -285,10 +285,10 @@ __global__ void __launch_bounds__(kThreads) decode_generic_kernel(DecodeParams p
     const uint32_t part = tid / d, jj = tid % d;
     const bool pv_active = part < parts;
 
-    if (tid < 32) {
-        ktab[tid] = p.k.table[tid];
-        vtab[tid] = p.v.table[tid];
-    }
+    // fields wider than 5 bits exist in the uniform coder only, whose table is code + 0.5
+    static_assert(kThreads == 256, "one table entry per thread");
+    ktab[tid] = p.k.w > 5U ? (float)tid + 0.5f : p.k.table[tid & 31U];
+    vtab[tid] = p.v.w > 5U ? (float)tid + 0.5f : p.v.table[tid & 31U];
 
     for (uint32_t hc = 0; hc < p.G; hc += kGMax) {
         const uint32_t gh = min((uint32_t)kGMax, p.G - hc);

@@ -1,7 +1,7 @@
 // Packed-cache layout of libweed_hip, shared by host code, every kernel and the CPU layout test.
 //
 // A *field* is what one coordinate of one cached row stores: the scalar code, or (code << 1) | sign when a
-// residual sign bit is kept.  Field width w = bits + sign, 1..5.
+// residual sign bit is kept.  Field width w = bits + sign: 1..5 with Lloyd-Max codes, 1..8 with Weed's uniform coder.
 //
 // Fields are stored in *items*: 8 fields in exactly w bytes, field e at bits [e*w, (e+1)*w) of the item
 // (little-endian bit string).  Consecutive fields (2p, 2p+1) form *pair* p of the item: the decode kernel turns one
@@ -75,7 +75,7 @@ WK_HD FieldPos v_field_pos(uint32_t n, uint32_t j, uint32_t d, uint32_t w)
 // Token (inside its 64-block) stored in field e of a V item of lane group g, half u.
 WK_HD uint32_t v_item_token(uint32_t u, uint32_t g, uint32_t e) { return 16 * (2 * u + (e >> 2)) + 4 * g + (e & 3); }
 
-// Read / write one field of an item through byte accesses (w <= 5, so a field spans at most two bytes).
+// Read / write one field of an item through byte accesses (w <= 8, so a field spans at most two bytes).
 WK_HD uint32_t item_get(const uint8_t *item, uint32_t bit, uint32_t w)
 {
     const uint32_t b = bit >> 3, s = bit & 7;

@@ -1224,9 +1224,7 @@ TensorPtr MultiHeadAttention::forward_quantized(TensorPtr Q, TensorPtr K, Tensor
         HipDevice::check(weed_hip_kv_decode_attn(cache, num_heads, gqa, qp, Q->offset, q_str, op, 0U, q_str, flags));
         return out;
     }
-    const bool fused_possible = (Hq / Hkv) <= 16U && (hd == 64U || hd == 128U);
-    if (prefill_path == PREFILL_DENSE || !fused_possible ||
-        (prefill_path == PREFILL_AUTO && dense_is_cheaper(uB, uT, cache_len))) {
+    if (prefill_path == PREFILL_DENSE || (prefill_path == PREFILL_AUTO && dense_is_cheaper(uB, uT, cache_len))) {
         // Long multi-token calls (prefill): the fused kernel serves one query position per launch, so beyond a few
         // positions it is cheaper to do what the reference does -- dequantise the cache once (still in the rotated
         // basis) and run dense ops: rotate Q, product, / sqrt(d), + mask, softmax, product, un-rotate
@@ -1300,8 +1298,7 @@ TensorPtr MultiHeadAttention::forward_quantized(TensorPtr Q, TensorPtr K, Tensor
     // The (position, head) pairs of a KV head are the rows of one tile of the fused kernel (16 at most), so a few
     // positions go through the cache together: position t0 + i of a group attends to before + t0 + i + 1 tokens, which
     // is "the group's last length minus the positions after it".
-    const tcapint G = Hq / Hkv;
-    const tcapint per_call = std::max<tcapint>(1U, 16U / G);
+    const tcapint per_call = positions_per_pass();
     const uint32_t q_str4[4] = { Q->stride[0U], Q->stride[1U], Q->stride[2U], Q->stride[3U] };
     const uint32_t o_str4[4] = { out->stride[0U], out->stride[1U], out->stride[2U], out->stride[3U] };
     for (tcapint t = 0U; t < uT; t += per_call) {
@@ -1318,6 +1315,18 @@ TensorPtr MultiHeadAttention::forward_quantized(TensorPtr Q, TensorPtr K, Tensor
     return out;
 }
 
+// Query positions that one pass of the fused kernel serves: the (position, head) pairs of a KV head are the rows of
+// one matrix tile (16), which exists for head_dim 64 / 128 and fields of 2..4 bits; any other shape goes through the
+// generic kernel one position at a time.
+tcapint MultiHeadAttention::positions_per_pass() const
+{
+    const tcapint G = num_heads / num_kv_heads;
+    const int wk = (k_bits ? k_bits : kv_quant_bits) + ((kv_coder == KV_LLOYDMAX && k_sign) ? 1 : 0);
+    const int wv = (v_bits ? v_bits : kv_quant_bits) + ((kv_coder == KV_LLOYDMAX && v_sign) ? 1 : 0);
+    const bool tiles = G <= 16U && (head_dim == 64U || head_dim == 128U) && wk >= 2 && wk <= 4 && wv >= 2 && wv <= 4;
+    return tiles ? std::max<tcapint>(1U, 16U / G) : 1U;
+}
+
 // Rough device times of the two ways to serve T new tokens against L cached ones (measured on MI355X: a pass of the
 // fused kernel costs about 55 us plus the packed bytes at 5 TB/s; the dense path is a dozen launches (200 us), writes
 // and re-reads fp32 K and V, runs two batched fp32 products at 60 TFLOP/s and walks the [B, heads, T, L] scores seven
@@ -1328,7 +1337,7 @@ bool MultiHeadAttention::dense_is_cheaper(tcapint B, tcapint T, tcapint L) const
     const double kb = (double)(k_bits ? k_bits : kv_quant_bits) + (k_sign ? 1.0 : 0.0);
     const double vb = (double)(v_bits ? v_bits : kv_quant_bits) + (v_sign ? 1.0 : 0.0);
     const double packed = (double)B * Hkv * (double)L * (hd * (kb + vb) / 8.0 + 8.0);
-    const double per_call = std::max(1.0, std::floor(16.0 / (Hq / Hkv)));
+    const double per_call = (double)positions_per_pass();
     const double passes = std::ceil((double)T / per_call);
     const double fused_us = passes * (55.0 + packed / 5.0e6);
     const double deq_bytes = (double)B * Hkv * (double)L * hd * 4.0 * 2.0;
