@@ -261,10 +261,12 @@ def test_head_dims_and_wide_groups(gpu, oracle):
         cache.close()
 
 
-@pytest.mark.parametrize("kb,vb,d", [(8, 8, 128), (5, 6, 64), (8, 4, 128), (1, 7, 32)])
+@pytest.mark.parametrize("kb,vb,d", [(8, 8, 128), (8, 8, 64), (5, 6, 64), (8, 4, 128), (1, 7, 32)])
 def test_uniform_widths_beyond_four_bits(gpu, oracle, kb, vb, d):
-    """Weed's uniform coder at any width the reference's `kv_quant_bits` may take (an 8-bit cache is the common
-    request): attention equals the checker on the same codes, with rotations, both GQA mappings and an append."""
+    """Weed's uniform coder at any width the reference's `kv_quant_bits` may take: attention equals the checker on the
+    same codes, with rotations and both GQA mappings.  8 + 8 bits (the common request) runs on the matrix cores, its
+    codes turned into fp16 arithmetically, also for a chunk of query positions and for 16 heads per KV head; the
+    other widths go through the generic kernel."""
     import torch
     rng = np.random.default_rng(kb * 16 + vb + d)
     Hkv, Hq, lens = 2, 8, [300, 77, 64]
@@ -283,6 +285,20 @@ def test_uniform_widths_beyond_four_bits(gpu, oracle, kb, vb, d):
     # the codes really use the whole range
     kf, _ = export(cache, 0, 64)
     assert kf.max() == (1 << kb) - 1 and kf.min() == 0
+    if kb == 8 and vb == 8:
+        T = 2
+        qc = rng.standard_normal((S, T, Hq, d), dtype=np.float32)
+        out = torch.zeros((S, T, Hq, d), device="cuda")
+        cache.decode_attn_chunk(dev(qc), out, gqa_mapping=gpu.GQA_BLOCKED, flags=flags)
+        for t in range(T):
+            wl_t = workloads.Workload("wide", S, Hq, Hkv, d, [n - (T - 1 - t) for n in lens], kb, vb, 0, 0, 0)
+            want = checker_output(oracle, gpu, cache, wl_t, np.ascontiguousarray(qc[:, t]), False, Rk, Rv)
+            assert_attn_close(out[:, t].cpu().numpy(), want, "chunk position %d" % t)
+        # sixteen heads per KV head (the 16-column instance)
+        q16 = rng.standard_normal((S, 16 * Hkv, d), dtype=np.float32)
+        wl16 = workloads.Workload("wide", S, 16 * Hkv, Hkv, d, lens, kb, vb, 0, 0, 0)
+        want = checker_output(oracle, gpu, cache, wl16, q16, True, Rk, Rv)
+        assert_attn_close(run_decode(gpu, cache, q16, gpu.GQA_WEED, flags), want, "16 heads per KV head")
     cache.close()
 
 

@@ -63,7 +63,8 @@ template <int N> __device__ __forceinline__ void load_dwords(const uint8_t *base
 //      byte 1 of the address.  When a pair is a whole byte of the packed run (4-bit fields), ONE byte-permute builds
 //      the address from the run's dword and the lane byte; otherwise a bit-field extract and a shift-add do. ----
 constexpr uint32_t kTableRowBytes = 256;
-template <int WK, int WV> constexpr uint32_t table_rows() { return 1u << (2 * (WK > WV ? WK : WV)); }
+// (8-bit fields are turned into fp16 values arithmetically and need no table)
+template <int WK, int WV> constexpr uint32_t table_rows() { return WK == 8 ? 0u : 1u << (2 * (WK > WV ? WK : WV)); }
 
 template <int W, int N, int P> __device__ __forceinline__ uint32_t pair_addr(const uint32_t (&x)[N], uint32_t lane_byte)
 {
@@ -97,11 +98,34 @@ __device__ __forceinline__ uint32_t lds_read(uint32_t byte_addr)
     return *reinterpret_cast<lds_u32_ptr>((uintptr_t)byte_addr);
 }
 
+// 8-bit fields (uniform coder only, value = code + 0.5): pair P of the run is two bytes of one dword.  A byte-permute
+// puts each code under the byte 0x64 -- the fp16 number 1024 + code, exactly -- and one packed fp16 add of -1023.5
+// leaves code + 0.5, also exact.
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+template <int N, int P> __device__ __forceinline__ uint32_t pair_from_bytes(const uint32_t (&x)[N])
+{
+    constexpr int dw = P >> 1, hi = P & 1;
+    // result bytes (3..0) = (0x64, code 2P + 1, 0x64, code 2P): selector values 4..7 name the bytes of the first
+    // source, 0..3 those of the second
+    constexpr uint32_t sel = hi ? 0x00070006u : 0x00050004u;
+    uint32_t a;
+    asm("v_perm_b32 %0, %1, %2, %3" : "=v"(a) : "v"(x[dw]), "v"(0x64646464u), "s"(sel));
+    const half2v h = __builtin_bit_cast(half2v, a) + half2v{ (_Float16)-1023.5f, (_Float16)-1023.5f };
+    return __builtin_bit_cast(uint32_t, h);
+}
+
 // Item K (8 fields) of the lane's run -> 8 fp16 values in matrix-operand order.
 template <int W, int N, int K>
 __device__ __forceinline__ half8 dequant_item(const uint32_t (&x)[N], uint32_t lane_byte)
 {
     uint4v r;
+    if constexpr (W == 8) {
+        r.x = pair_from_bytes<N, 4 * K>(x);
+        r.y = pair_from_bytes<N, 4 * K + 1>(x);
+        r.z = pair_from_bytes<N, 4 * K + 2>(x);
+        r.w = pair_from_bytes<N, 4 * K + 3>(x);
+        return __builtin_bit_cast(half8, r);
+    }
     r.x = lds_read(pair_addr<W, N, 4 * K>(x, lane_byte));
     r.y = lds_read(pair_addr<W, N, 4 * K + 1>(x, lane_byte));
     r.z = lds_read(pair_addr<W, N, 4 * K + 2>(x, lane_byte));
@@ -191,6 +215,9 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
         level_of_lane = (tid < 32) ? p.k.table[tid & 31] : p.v.table[tid & 31];
     }
     auto build_tables = [&]() {
+        if constexpr (ROWS == 0) {
+            return; // no tables, hence no barriers either
+        }
         uint16_t *levels_h = reinterpret_cast<uint16_t *>(lds + ROWS * (kTableRowBytes / 4)); // [2][32]
         if (tid < 64) {
             levels_h[tid] = __builtin_bit_cast(uint16_t, (_Float16)level_of_lane);
@@ -705,6 +732,9 @@ template <int D, bool LLOYD> int launch_d(const MfmaParams &p, hipStream_t s)
     WEED_CASE(4, 2)
     WEED_CASE(4, 3)
     WEED_CASE(4, 4)
+    if constexpr (!LLOYD) {
+        WEED_CASE(8, 8) // kv_quant_bits = 8 of the reference's uniform coder
+    }
 #undef WEED_CASE
     return fail(WEED_HIP_EINVAL, "decode_mfma: unsupported field widths %u / %u", wk, wv);
 }
