@@ -88,6 +88,19 @@ def time_calls(torch, fn, steps, warmup):
     return (time.perf_counter() - t0) / steps
 
 
+def time_kernel(capi, torch, fn, name, steps, warmup):
+    """(seconds per call, seconds per launch of the kernel recorded under `name`): one untimed call first, so that
+    one-off work of a shape's first launch (workspace growth, kernel attributes) stays out of both figures."""
+    fn()
+    torch.cuda.synchronize()
+    capi.profile_reset()
+    capi.profile_enable(True)
+    secs = time_calls(torch, fn, steps, warmup)
+    k_ms, k_n = capi.profile_read(name)
+    capi.profile_enable(False)
+    return secs, 1e-3 * k_ms / max(1, k_n)
+
+
 def extras(capi, torch, workloads, steps, warmup):
     """The other configurations, measured the same way (reported beside the headline, not as `value`)."""
     out = {}
@@ -95,13 +108,8 @@ def extras(capi, torch, workloads, steps, warmup):
     A = torch.randn((1024, 4096), device="cuda").t()           # logical [4096, 1024], column-major
     W = (torch.randn((4096, 1024), device="cuda") * 0.02).t()  # logical [1024, 4096], column-major
     C = torch.empty((4096, 4096), device="cuda").t()
-    capi.profile_reset()
-    capi.profile_enable(True)
-    secs = time_calls(torch, lambda: capi.matmul(A, W, C), steps, warmup)
-    k_ms, k_n = capi.profile_read("matmul")
-    capi.profile_enable(False)
+    secs, kernel_s = time_kernel(capi, torch, lambda: capi.matmul(A, W, C), "matmul", steps, warmup)
     flops = 2.0 * 4096 * 1024 * 4096
-    kernel_s = 1e-3 * k_ms / max(1, k_n)
     out["cfg5b_matmul_f32_4096x1024x4096"] = {
         "tflops": flops / secs / 1e12, "kernel_ms": 1e3 * kernel_s, "kernel_tflops": flops / kernel_s / 1e12,
         "roofline": {"bound": "mfma", "achieved": flops / kernel_s / 1e12, "peak": 157.3, "unit": "TFLOP/s",
@@ -111,12 +119,7 @@ def extras(capi, torch, workloads, steps, warmup):
     X = torch.randn((4096, 8), device="cuda").t()               # logical [8, 4096], column-major
     Wp = (torch.randn((4096, 4096), device="cuda") * 0.02).t()  # logical [4096, 4096], column-major
     Y = torch.empty((4096, 8), device="cuda").t()
-    capi.profile_reset()
-    capi.profile_enable(True)
-    secs = time_calls(torch, lambda: capi.matmul(X, Wp, Y), steps, warmup)
-    k_ms, k_n = capi.profile_read("matmul")
-    capi.profile_enable(False)
-    kernel_s = 1e-3 * k_ms / max(1, k_n)
+    secs, kernel_s = time_kernel(capi, torch, lambda: capi.matmul(X, Wp, Y), "matmul", steps, warmup)
     wbytes = 4096 * 4096 * 4
     out["projection_8x4096x4096"] = {
         "ms": 1e3 * secs, "kernel_ms": 1e3 * kernel_s,
@@ -132,12 +135,7 @@ def extras(capi, torch, workloads, steps, warmup):
     for axis, name in ((0, "contiguous_axis"), (1, "strided_axis")):
         for op, fn, bytes_per in (("softmax", lambda: capi.softmax(S, So, axis), 8),
                                   ("reduce", lambda: capi.reduce(capi.REDUCE_SUM, S, Sr, axis), 4)):
-            capi.profile_reset()
-            capi.profile_enable(True)
-            time_calls(torch, fn, steps, warmup)
-            k_ms, k_n = capi.profile_read(op)
-            capi.profile_enable(False)
-            kernel_s = 1e-3 * k_ms / max(1, k_n)
+            _, kernel_s = time_kernel(capi, torch, fn, op, steps, warmup)
             gbs = S.numel() * bytes_per / kernel_s / 1e9
             dense["%s_%s" % (op, name)] = {"kernel_ms": 1e3 * kernel_s,
                                            "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS,
@@ -177,31 +175,44 @@ def extras(capi, torch, workloads, steps, warmup):
     for hq in (8, 32):
         q = torch.randn((wl4.n_seq, hq, d), device="cuda")
         o = torch.zeros_like(q)
-        capi.profile_reset()
-        capi.profile_enable(True)
-        secs = time_calls(torch, lambda: cache4.decode_attn(q, o, capi.GQA_BLOCKED, 0), steps, warmup)
-        k_ms, k_n = capi.profile_read("kv_decode_attn")
-        capi.profile_enable(False)
+        secs, kernel_s = time_kernel(capi, torch, lambda: cache4.decode_attn(q, o, capi.GQA_BLOCKED, 0),
+                                     "kv_decode_attn", steps, warmup)
         nbytes = wl4.bytes_per_step(True)
-        kernel_s = 1e-3 * k_ms / max(1, k_n)
         out["cfg4_ragged16_hq%d" % hq] = {"tokens_per_s": wl4.n_seq / secs, "ms_per_step": 1e3 * secs,
                                           "packed_cache_bytes": nbytes, "kernel_ms": 1e3 * kernel_s,
                                           "kernel_gbs": nbytes / kernel_s / 1e9,
                                           "frac_of_hbm_peak": nbytes / kernel_s / 1e9 / HBM_PEAK_GBS}
     cache4.close()
+    # Weed's own uniform coder at kv_quant_bits = 8 on the headline shape (64 x 8192 tokens x 8 heads, 256 B per token
+    # and head): the matrix-core kernel with arithmetic de-quantisation instead of tables
+    wl8 = workloads.config(3, n_seq=64)
+    cache8 = capi.KVCache(capi.KV_UNIFORM, wl8.n_seq, wl8.n_kv_heads, d, wl8.max_len, 8, 8)
+    cache8.set_scales(1.0, 1.0)
+    for s0 in range(0, wl8.n_seq, 8):
+        Ks = torch.randn((8, wl8.n_kv_heads, wl8.max_len, d), device="cuda")
+        Vs = torch.randn((8, wl8.n_kv_heads, wl8.max_len, d), device="cuda")
+        cache8.encode_append(Ks, Vs, seq_begin=s0)
+    del Ks, Vs
+    q8 = torch.randn((wl8.n_seq, wl8.n_q_heads, d), device="cuda")
+    o8 = torch.zeros_like(q8)
+    secs, kernel_s = time_kernel(capi, torch, lambda: cache8.decode_attn(q8, o8, capi.GQA_BLOCKED, 0),
+                                 "kv_decode_attn", steps, warmup)
+    nbytes = sum(wl8.lens) * wl8.n_kv_heads * 2 * d
+    out["uniform_8bit_64_sequences"] = {"tokens_per_s": wl8.n_seq / secs, "ms_per_step": 1e3 * secs,
+                                        "packed_cache_bytes": nbytes, "kernel_ms": 1e3 * kernel_s,
+                                        "kernel_gbs": nbytes / kernel_s / 1e9,
+                                        "frac_of_hbm_peak": nbytes / kernel_s / 1e9 / HBM_PEAK_GBS}
+    cache8.close()
+    del q8, o8
     # configuration 3 again with 256 sequence caches per launch (2 GB of packed rows): what the per-launch fixed cost
     # (launch, table build, first-block latency, uneven finish) amortises to with four times the bytes
     wl3 = workloads.config(3, n_seq=256)
     cache3, q3, _, _ = build_cache(capi, torch, wl3, seed=77)
     o3 = torch.zeros_like(q3)
     flags = capi.ATTN_ROTATE_Q | capi.ATTN_UNROTATE_OUT
-    capi.profile_reset()
-    capi.profile_enable(True)
-    secs = time_calls(torch, lambda: cache3.decode_attn(q3, o3, capi.GQA_BLOCKED, flags), steps, warmup)
-    k_ms, k_n = capi.profile_read("kv_decode_attn")
-    capi.profile_enable(False)
+    secs, kernel_s = time_kernel(capi, torch, lambda: cache3.decode_attn(q3, o3, capi.GQA_BLOCKED, flags),
+                                 "kv_decode_attn", steps, warmup)
     nbytes = wl3.bytes_per_step(lloydmax=True)
-    kernel_s = 1e-3 * k_ms / max(1, k_n)
     out["cfg3_256_sequences"] = {"tokens_per_s": wl3.n_seq / secs, "ms_per_step": 1e3 * secs,
                                  "packed_cache_bytes": nbytes, "kernel_ms": 1e3 * kernel_s,
                                  "kernel_gbs": nbytes / kernel_s / 1e9,
