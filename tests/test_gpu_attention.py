@@ -261,6 +261,32 @@ def test_head_dims_and_wide_groups(gpu, oracle):
         cache.close()
 
 
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("wk", [2, 3, 4, 5])
+@pytest.mark.parametrize("wv", [2, 3, 4, 5])
+def test_every_pair_of_field_widths(gpu, oracle, d, wk, wv):
+    """Lloyd-Max fields of 2 to 5 bits on either side (a width is code bits plus the optional sign bit; both ways of
+    making 3 and 4 occur): every pair has its own instance of the matrix-core kernel, the 5-bit ones with single-value
+    tables.  Ragged lengths across block edges, groups of 4 and of 16 heads per KV head, both GQA mappings."""
+    rng = np.random.default_rng(100 * wk + 10 * wv + d)
+    with_sign = (wk + wv) % 2 == 0
+    split = {2: (2, 0), 3: (2, 1) if with_sign else (3, 0), 4: (3, 1) if with_sign else (4, 0), 5: (4, 1)}
+    (kb, ks), (vb, vs) = split[wk], split[wv]
+    Hkv, lens = 2, [200, 65, 64]
+    S = len(lens)
+    K = rng.standard_normal((S, Hkv, max(lens), d), dtype=np.float32) * rng.uniform(0.3, 3.0, size=(S, Hkv, max(lens), 1)).astype(np.float32)
+    V = rng.standard_normal((S, Hkv, max(lens), d), dtype=np.float32)
+    wl = workloads.Workload("widths", S, 4 * Hkv, Hkv, d, lens, kb, vb, ks, vs, 0)
+    cache = build_cache(gpu, wl, gpu.KV_LLOYDMAX, K, V)
+    assert cache.row_bytes() == (d * wk // 8 + 4, d * wv // 8 + 4)
+    for Hq, gqa, weed in ((4 * Hkv, gpu.GQA_BLOCKED, False), (16 * Hkv, gpu.GQA_WEED, True)):
+        q = rng.standard_normal((S, Hq, d), dtype=np.float32)
+        wl_q = workloads.Workload("widths", S, Hq, Hkv, d, lens, kb, vb, ks, vs, 0)
+        want = checker_output(oracle, gpu, cache, wl_q, q, weed)
+        assert_attn_close(run_decode(gpu, cache, q, gqa, 0), want, "K %d+%d V %d+%d, %d heads" % (kb, ks, vb, vs, Hq))
+    cache.close()
+
+
 @pytest.mark.parametrize("kb,vb,d", [(8, 8, 128), (8, 8, 64), (5, 6, 64), (8, 4, 128), (1, 7, 32)])
 def test_uniform_widths_beyond_four_bits(gpu, oracle, kb, vb, d):
     """Weed's uniform coder at any width the reference's `kv_quant_bits` may take: attention equals the checker on the
@@ -340,8 +366,11 @@ def test_chunk_of_query_positions(gpu, oracle, lloyd, d, Hkv, Hq, T, gqa_weed):
     lens = [64 + 1, 300, 129, 64 + T, 5 * 64]
     S = len(lens)
     kb, vb, ks = (3, 4, 1) if lloyd else (4, 3, 0)
+    vs = 0
+    if lloyd and d == 64:
+        kb, vb, ks, vs = 4, 4, 1, 1  # 5-bit fields on both sides
     mode = gpu.KV_LLOYDMAX if lloyd else gpu.KV_UNIFORM
-    wl = workloads.Workload("chunk", S, Hq, Hkv, d, lens, kb, vb, ks, 0, 0)
+    wl = workloads.Workload("chunk", S, Hq, Hkv, d, lens, kb, vb, ks, vs, 0)
     K = rng.standard_normal((S, Hkv, max(lens), d), dtype=np.float32)
     V = rng.standard_normal((S, Hkv, max(lens), d), dtype=np.float32)
     q = rng.standard_normal((S, T, Hq, d), dtype=np.float32)
@@ -358,7 +387,7 @@ def test_chunk_of_query_positions(gpu, oracle, lloyd, d, Hkv, Hq, T, gqa_weed):
             gpu.sync()
             got = out.cpu().numpy()
             for t in range(T):
-                wl_t = workloads.Workload("chunk", S, Hq, Hkv, d, [n - (T - 1 - t) for n in seen], kb, vb, ks, 0, 0)
+                wl_t = workloads.Workload("chunk", S, Hq, Hkv, d, [n - (T - 1 - t) for n in seen], kb, vb, ks, vs, 0)
                 want = checker_output(oracle, gpu, cache, wl_t, np.ascontiguousarray(q[:, t]), gqa_weed, Rk, Rv)
                 assert_attn_close(got[:, t], want, "%s position %d" % (what, t))
 

@@ -10,8 +10,8 @@ int launch_mfma_decode_d128_lloyd(const MfmaParams &p, hipStream_t s);
 
 bool mfma_decode_supported(uint32_t d, uint32_t wk, uint32_t wv, uint32_t G)
 {
-    // fields of 2..4 bits through pair tables, or the uniform coder's 8-bit codes on both sides
-    const bool widths = (wk >= 2 && wk <= 4 && wv >= 2 && wv <= 4) || (wk == 8 && wv == 8);
+    // fields of 2..5 bits through lookup tables, or the uniform coder's 8-bit codes on both sides
+    const bool widths = (wk >= 2 && wk <= 5 && wv >= 2 && wv <= 5) || (wk == 8 && wv == 8);
     return (d == 64 || d == 128) && widths && G >= 1 && G <= 16;
 }
 

@@ -63,8 +63,15 @@ template <int N> __device__ __forceinline__ void load_dwords(const uint8_t *base
 //      byte 1 of the address.  When a pair is a whole byte of the packed run (4-bit fields), ONE byte-permute builds
 //      the address from the run's dword and the lane byte; otherwise a bit-field extract and a shift-add do. ----
 constexpr uint32_t kTableRowBytes = 256;
-// (8-bit fields are turned into fp16 values arithmetically and need no table)
-template <int WK, int WV> constexpr uint32_t table_rows() { return WK == 8 ? 0u : 1u << (2 * (WK > WV ? WK : WV)); }
+// Rows of one side's table: pair tables (2^(2W) entries) for fields of up to 4 bits; 5-bit fields (4-bit codes with
+// the residual sign) would need 1024 pairs, so they use a table of the 32 single values, each stored twice (both
+// halves of the word), and a pair is assembled from two lookups; 8-bit fields are turned into fp16 values
+// arithmetically and need no table.
+template <int W> constexpr uint32_t side_rows() { return W == 8 ? 0u : (W == 5 ? 32u : 1u << (2 * W)); }
+template <int WK, int WV> constexpr uint32_t table_rows()
+{
+    return side_rows<WK>() > side_rows<WV>() ? side_rows<WK>() : side_rows<WV>();
+}
 
 template <int W, int N, int P> __device__ __forceinline__ uint32_t pair_addr(const uint32_t (&x)[N], uint32_t lane_byte)
 {
@@ -91,11 +98,36 @@ template <int W, int N, int P> __device__ __forceinline__ uint32_t pair_addr(con
     return a;
 }
 
+// LDS byte address of the single-value entry of field F (5-bit fields): (field << 8) | lane byte.
+template <int W, int N, int F> __device__ __forceinline__ uint32_t field_addr(const uint32_t (&x)[N], uint32_t lane_byte)
+{
+    constexpr int bit = W * F;
+    constexpr int dw = bit >> 5, sh = bit & 31;
+    uint32_t t, a;
+    if constexpr (sh + W <= 32) {
+        asm("v_bfe_u32 %0, %1, %2, %3" : "=v"(t) : "v"(x[dw]), "n"(sh), "n"(W));
+    } else {
+        uint32_t f;
+        asm("v_alignbit_b32 %0, %1, %2, %3" : "=v"(f) : "v"(x[dw + 1 < N ? dw + 1 : dw]), "v"(x[dw]), "n"(sh));
+        asm("v_bfe_u32 %0, %1, 0, %2" : "=v"(t) : "v"(f), "n"(W));
+    }
+    asm("v_lshl_add_u32 %0, %1, 8, %2" : "=v"(a) : "v"(t), "v"(lane_byte));
+    return a;
+}
+
 typedef const uint32_t __attribute__((address_space(3))) *lds_u32_ptr;
 
 __device__ __forceinline__ uint32_t lds_read(uint32_t byte_addr)
 {
     return *reinterpret_cast<lds_u32_ptr>((uintptr_t)byte_addr);
+}
+
+template <int I, int N, typename F> __device__ __forceinline__ void static_for_fields(F &&f)
+{
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for_fields<I + 1, N>(f);
+    }
 }
 
 // 8-bit fields (uniform coder only, value = code + 0.5): pair P of the run is two bytes of one dword.  A byte-permute
@@ -124,6 +156,19 @@ __device__ __forceinline__ half8 dequant_item(const uint32_t (&x)[N], uint32_t l
         r.y = pair_from_bytes<N, 4 * K + 1>(x);
         r.z = pair_from_bytes<N, 4 * K + 2>(x);
         r.w = pair_from_bytes<N, 4 * K + 3>(x);
+        return __builtin_bit_cast(half8, r);
+    }
+    if constexpr (W == 5) {
+        // every entry holds its value in both halves: low half from the even field, high half from the odd one
+        uint32_t v[8];
+        static_for_fields<0, 8>([&](auto fc) {
+            constexpr int f = decltype(fc)::value;
+            v[f] = lds_read(field_addr<W, N, 8 * K + f>(x, lane_byte));
+        });
+        r.x = (v[0] & 0xffffu) | (v[1] & 0xffff0000u);
+        r.y = (v[2] & 0xffffu) | (v[3] & 0xffff0000u);
+        r.z = (v[4] & 0xffffu) | (v[5] & 0xffff0000u);
+        r.w = (v[6] & 0xffffu) | (v[7] & 0xffff0000u);
         return __builtin_bit_cast(half8, r);
     }
     r.x = lds_read(pair_addr<W, N, 4 * K>(x, lane_byte));
@@ -233,6 +278,12 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
                 const uint32_t e = i >> 6, half_row = (i >> 5) & 1; // 0: V table, 1: K table
                 const uint32_t w = half_row ? WK : WV;
                 const uint32_t base = half_row ? 0u : 32u;
+                if (w == 5u) {
+                    // the 32 single values, in both halves of the word
+                    const uint32_t lv = levels_h[base + (e & 31u)];
+                    val[u] = e < 32u ? (lv | (lv << 16)) : 0u;
+                    continue;
+                }
                 const uint32_t lo = levels_h[base + (e & ((1u << w) - 1u))];
                 const uint32_t hi = levels_h[base + ((e >> w) & ((1u << w) - 1u))];
                 val[u] = (e < (1u << (2 * w))) ? (lo | (hi << 16)) : 0u;
@@ -732,6 +783,14 @@ template <int D, bool LLOYD> int launch_d(const MfmaParams &p, hipStream_t s)
     WEED_CASE(4, 2)
     WEED_CASE(4, 3)
     WEED_CASE(4, 4)
+    // 5-bit fields: 4-bit codes with the residual sign (or 5-bit uniform codes)
+    WEED_CASE(5, 2)
+    WEED_CASE(5, 3)
+    WEED_CASE(5, 4)
+    WEED_CASE(5, 5)
+    WEED_CASE(2, 5)
+    WEED_CASE(3, 5)
+    WEED_CASE(4, 5)
     if constexpr (!LLOYD) {
         WEED_CASE(8, 8) // kv_quant_bits = 8 of the reference's uniform coder
     }
