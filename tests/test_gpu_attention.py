@@ -287,12 +287,13 @@ def test_every_pair_of_field_widths(gpu, oracle, d, wk, wv):
     cache.close()
 
 
-@pytest.mark.parametrize("kb,vb,d", [(8, 8, 128), (8, 8, 64), (5, 6, 64), (8, 4, 128), (1, 7, 32)])
+@pytest.mark.parametrize("kb,vb,d", [(8, 8, 128), (8, 8, 64), (5, 5, 128), (5, 4, 64), (5, 6, 64), (8, 4, 128),
+                                     (1, 7, 32)])
 def test_uniform_widths_beyond_four_bits(gpu, oracle, kb, vb, d):
     """Weed's uniform coder at any width the reference's `kv_quant_bits` may take: attention equals the checker on the
     same codes, with rotations and both GQA mappings.  8 + 8 bits (the common request) runs on the matrix cores, its
-    codes turned into fp16 arithmetically, also for a chunk of query positions and for 16 heads per KV head; the
-    other widths go through the generic kernel."""
+    codes turned into fp16 arithmetically, also for a chunk of query positions and for 16 heads per KV head; 5-bit
+    codes use the single-value tables; the other widths go through the generic kernel."""
     import torch
     rng = np.random.default_rng(kb * 16 + vb + d)
     Hkv, Hq, lens = 2, 8, [300, 77, 64]
