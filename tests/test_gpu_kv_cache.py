@@ -10,7 +10,7 @@ import os
 import numpy as np
 import pytest
 
-from gpu_helpers import col_major, coder_specs, dev, export
+from gpu_helpers import assert_attn_close, col_major, coder_specs, dev, export
 
 pytestmark = pytest.mark.gpu
 HERE = os.path.dirname(os.path.abspath(__file__))
@@ -207,6 +207,52 @@ def test_device_rotation_modes(gpu, oracle, mode):
                 assert np.mean(got_f.reshape(-1, d) != want_f) < 2e-3
                 np.testing.assert_allclose(got_a.reshape(-1), want_a, rtol=1e-5)
         cache.close()
+
+
+@pytest.mark.parametrize("lloyd,kw,vw,d", [(True, (4, 1), (4, 0), 128), (True, (2, 1), (3, 0), 64),
+                                           (False, (4, 0), (8, 0), 128), (False, (3, 0), (2, 0), 32)])
+def test_half_block_appends_mix_with_packed_ones(gpu, oracle, lloyd, kw, vw, d):
+    """Appends that add whole 32-token half blocks behind whole half blocks are written by the encoder itself, any
+    other append goes through the packing kernel; a cache may see both in any order and per sequence.  After every
+    step the fields, the row scales and the attention over the cache equal the checker's on the rows appended so far."""
+    import torch
+    rng = np.random.default_rng(d + kw[0] * 7 + vw[0])
+    S, Hkv, cap = 3, 2, 256
+    mode = gpu.KV_LLOYDMAX if lloyd else gpu.KV_UNIFORM
+    cache = gpu.KVCache(mode, S, Hkv, d, cap, kw[0], vw[0], kw[1], vw[1])
+    if not lloyd:
+        cache.set_scales(1.2, 0.8)
+    K = (rng.normal(size=(S, Hkv, cap, d)) * rng.uniform(0.3, 4, size=(S, Hkv, cap, 1))).astype(np.float32)
+    V = rng.normal(size=(S, Hkv, cap, d)).astype(np.float32)
+    Kd, Vd = dev(K), dev(V)
+    lens = [0] * S
+    q = rng.standard_normal((S, 2 * Hkv, d), dtype=np.float32)
+    # (first sequence, sequence count, tokens): direct, direct for one sequence, packed, packed (unaligned start),
+    # direct again for the one sequence that is still aligned, packed single tokens
+    steps = [(0, 3, 64), (1, 1, 32), (0, 1, 5), (0, 3, 32), (2, 1, 32), (0, 3, 1), (1, 2, 1)]
+    for s0, n, T in steps:
+        k_new = torch.stack([Kd[s, :, lens[s]:lens[s] + T] for s in range(s0, s0 + n)])
+        v_new = torch.stack([Vd[s, :, lens[s]:lens[s] + T] for s in range(s0, s0 + n)])
+        cache.encode_append(k_new, v_new, seq_begin=s0)
+        for s in range(s0, s0 + n):
+            lens[s] += T
+        assert cache.seq_lens() == lens
+        kspec, vspec = coder_specs(oracle, cache)
+        for which, x, spec in ((0, K, kspec), (1, V, vspec)):
+            got_f, got_a = export(cache, which, max(lens))
+            for s in range(S):
+                want_f, want_a = oracle.encode_rows(spec, x[s, :, :lens[s]].reshape(-1, d))
+                np.testing.assert_array_equal(got_f[s, :, :lens[s]].reshape(-1, d), want_f)
+                if lloyd:
+                    np.testing.assert_array_equal(got_a[s, :, :lens[s]].reshape(-1), want_a)
+        kf, ka = export(cache, 0, max(lens))
+        vf, va = export(cache, 1, max(lens))
+        want = oracle.decode_attn(kspec, vspec, kf, ka if lloyd else None, vf, va if lloyd else None, q, lens,
+                                  gqa_weed=True)
+        out = torch.zeros((S, 2 * Hkv, d), device="cuda")
+        cache.decode_attn(dev(q), out)
+        assert_attn_close(out.cpu().numpy(), want, "after %s" % ((s0, n, T),))
+    cache.close()
 
 
 def test_incremental_and_ragged_append(gpu, oracle):

@@ -139,11 +139,65 @@ constexpr int kEncThreads = 256;
 //   rounding (multiply, then add, i ascending: src/ops/matmul.cpp:40-44).
 // PARTS = number of row slices the 256 threads are split into (each thread owns one output column of its slice).
 // `block` = index of the workgroup among those that work on this tensor.
+// Where an append whose rows fill whole 32-token half blocks goes directly (see encode_rows_body): the cache side's
+// own arrays.  `out` null: the rows go to the scratch arrays and a second kernel packs them.
+struct DirectOut {
+    uint8_t *out;        // packed fields of the side
+    uint64_t region_bytes;
+    float *alpha;        // [region][padded] row scales, null for the uniform coder
+    uint32_t *alpha_max; // [region] largest row scale (V side), or null
+    const int32_t *lens; // cached lengths BEFORE this append
+    int32_t seq_begin;
+    uint32_t padded, w;
+    int is_v;
+};
+
+// The kEncRows = 32 staged rows are tokens [n0, n0 + 32) of one (sequence, head), n0 a multiple of 32: one half of a
+// 64-token block.  Every K item (8 coordinates of a token) and every V item (8 tokens of a coordinate, all inside
+// this half) is assembled from LDS and written to its place; nothing already cached shares an item with them.
+__device__ __forceinline__ void write_half_block(const uint8_t *staged, const DirectOut &o, uint32_t Hkv, uint32_t T,
+                                                 uint32_t d, uint32_t row0)
+{
+    const uint32_t h = (row0 / T) % Hkv, sq = row0 / (T * Hkv);
+    const uint64_t region = (uint64_t)(o.seq_begin + (int32_t)sq) * Hkv + h;
+    const uint32_t n0 = (uint32_t)o.lens[o.seq_begin + (int32_t)sq] + row0 % T;
+    uint8_t *base = o.out + region * o.region_bytes;
+    const uint32_t w = o.w;
+    uint8_t bytes[8];
+    if (!o.is_v) {
+        const uint32_t items = d / 8;
+        for (uint32_t idx = threadIdx.x; idx < kEncRows * items; idx += kEncThreads) {
+            const uint32_t r = idx / items, it = idx - r * items;
+            item_build(staged + (uint64_t)r * d + it * 8, w, bytes);
+            uint8_t *dst = base + k_field_pos(n0 + r, it * 8, d, w).byte;
+            for (uint32_t b = 0; b < w; ++b) {
+                dst[b] = bytes[b];
+            }
+        }
+        return;
+    }
+    const uint32_t u = (n0 >> 5) & 1U, tok0 = n0 & ~63U;
+    for (uint32_t idx = threadIdx.x; idx < 4 * d; idx += kEncThreads) {
+        const uint32_t j = idx % d, gq = idx / d;
+        uint8_t f8[8];
+#pragma unroll
+        for (uint32_t e = 0; e < 8; ++e) {
+            // token of field e inside this half: rows 4g .. 4g+3 of its first tile, then of its second
+            f8[e] = staged[(uint64_t)(16 * (e >> 2) + 4 * gq + (e & 3)) * d + j];
+        }
+        item_build(f8, w, bytes);
+        uint8_t *dst = base + v_field_pos(tok0 + v_item_token(u, gq, 0), j, d, w).byte;
+        for (uint32_t b = 0; b < w; ++b) {
+            dst[b] = bytes[b];
+        }
+    }
+}
+
 template <int PARTS>
 __device__ __forceinline__ void encode_rows_body(const float *__restrict__ x, const Geom4 &g, uint32_t Hkv, uint32_t T,
                                                  uint32_t d, uint32_t rows, const float *__restrict__ rot_t, int rotate,
                                                  const CoderParams &cp, uint8_t *__restrict__ fields,
-                                                 float *__restrict__ alpha_out, uint32_t block)
+                                                 float *__restrict__ alpha_out, const DirectOut &direct, uint32_t block)
 {
     extern __shared__ float smem[];
     const uint32_t pitch = d + 1;
@@ -255,6 +309,10 @@ __device__ __forceinline__ void encode_rows_body(const float *__restrict__ x, co
         __syncthreads();
     }
 
+    // one field per byte: into the scratch array, or (direct append) into LDS where xs was, [kEncRows][d]
+    uint8_t *staged = reinterpret_cast<uint8_t *>(xs);
+    uint8_t *fdst = direct.out ? staged : fields + (uint64_t)row0 * d;
+
     if (cp.mode == WEED_HIP_KV_UNIFORM) {
         const int levels = 1 << cp.bits;
         const float lo = -3.0f * cp.block_scale;
@@ -263,8 +321,12 @@ __device__ __forceinline__ void encode_rows_body(const float *__restrict__ x, co
         const uint32_t jl = tid & 31;
         for (uint32_t r = tid >> 5; r < kEncRows && row0 + r < rows; r += kEncThreads / 32) {
             for (uint32_t j = jl; j < d; j += 32) {
-                fields[(uint64_t)(row0 + r) * d + j] = (uint8_t)uniform_bucket(ys[r * pitch + j], lo, hi, step, levels);
+                fdst[(uint64_t)r * d + j] = (uint8_t)uniform_bucket(ys[r * pitch + j], lo, hi, step, levels);
             }
+        }
+        if (direct.out) {
+            __syncthreads();
+            write_half_block(staged, direct, Hkv, T, d, row0);
         }
         return;
     }
@@ -291,7 +353,22 @@ __device__ __forceinline__ void encode_rows_body(const float *__restrict__ x, co
             a = norm / sqrt_d;
         }
         inv_s[tid] = inv;
-        if (row0 + tid < rows) {
+        if (direct.out) {
+            // all kEncRows rows belong to one (sequence, head): scale to its token slot, largest scale to the region
+            const uint32_t h = (row0 / T) % Hkv, sq = row0 / (T * Hkv);
+            const uint32_t region = (uint32_t)(direct.seq_begin + (int32_t)sq) * Hkv + h;
+            const uint32_t n = (uint32_t)direct.lens[direct.seq_begin + (int32_t)sq] + row0 % T + tid;
+            direct.alpha[(uint64_t)region * direct.padded + n] = a;
+            if (direct.alpha_max) {
+                uint32_t bits = __float_as_uint(fabsf(a));
+                for (int o = 16; o > 0; o >>= 1) {
+                    bits = max(bits, (uint32_t)__shfl_xor((int)bits, o));
+                }
+                if (tid == 0) {
+                    atomicMax(direct.alpha_max + region, bits);
+                }
+            }
+        } else if (row0 + tid < rows) {
             alpha_out[row0 + tid] = a;
         }
     }
@@ -325,8 +402,12 @@ __device__ __forceinline__ void encode_rows_body(const float *__restrict__ x, co
                 }
                 word |= f << (8 * i);
             }
-            *reinterpret_cast<uint32_t *>(fields + (uint64_t)(row0 + r) * d + j) = word;
+            *reinterpret_cast<uint32_t *>(fdst + (uint64_t)r * d + j) = word;
         }
+    }
+    if (direct.out) {
+        __syncthreads();
+        write_half_block(staged, direct, Hkv, T, d, row0);
     }
 }
 
@@ -339,6 +420,7 @@ struct EncSide {
     CoderParams cp;
     uint8_t *fields;
     float *alpha_out;
+    DirectOut direct;
 };
 template <int PARTS>
 __global__ void __launch_bounds__(kEncThreads)
@@ -346,9 +428,10 @@ __global__ void __launch_bounds__(kEncThreads)
                             uint32_t rows, int rotate)
 {
     if (blockIdx.x < blocks_per_side) {
-        encode_rows_body<PARTS>(k.x, k.g, Hkv, T, d, rows, k.rot_t, rotate, k.cp, k.fields, k.alpha_out, blockIdx.x);
+        encode_rows_body<PARTS>(k.x, k.g, Hkv, T, d, rows, k.rot_t, rotate, k.cp, k.fields, k.alpha_out, k.direct,
+                                blockIdx.x);
     } else {
-        encode_rows_body<PARTS>(v.x, v.g, Hkv, T, d, rows, v.rot_t, rotate, v.cp, v.fields, v.alpha_out,
+        encode_rows_body<PARTS>(v.x, v.g, Hkv, T, d, rows, v.rot_t, rotate, v.cp, v.fields, v.alpha_out, v.direct,
                                 blockIdx.x - blocks_per_side);
     }
 }
@@ -674,6 +757,7 @@ EncSide enc_side_args(const weed_hip_kv_cache *c, const Side &side, const float 
     std::memcpy(e.cp.levels, side.levels, sizeof(e.cp.levels));
     e.fields = fields;
     e.alpha_out = alpha;
+    e.direct = DirectOut{ nullptr, 0, nullptr, nullptr, nullptr, 0, 0, 0, 0 };
     return e;
 }
 
@@ -690,8 +774,22 @@ int encode_both(weed_hip_kv_cache *c, int32_t seq_begin, int32_t seq_count, int3
     const uint32_t rows = (uint32_t)seq_count * Hkv * (uint32_t)T_new;
     uint8_t *k_fields = c->enc_fields, *v_fields = c->enc_fields + (size_t)rows * d;
     float *k_alpha = c->enc_alpha, *v_alpha = c->enc_alpha + rows;
-    const EncSide ek = enc_side_args(c, c->k, k_dev, k_off, k_stride, k_fields, k_alpha);
-    const EncSide ev = enc_side_args(c, c->v, v_dev, v_off, v_stride, v_fields, v_alpha);
+    EncSide ek = enc_side_args(c, c->k, k_dev, k_off, k_stride, k_fields, k_alpha);
+    EncSide ev = enc_side_args(c, c->v, v_dev, v_off, v_stride, v_fields, v_alpha);
+    // An append that adds whole 32-token half blocks behind whole half blocks (a prefill, in chunks or not) needs no
+    // packing pass: every workgroup of the encoder holds one half block of one (sequence, head) and writes its items
+    // itself.
+    bool direct = T_new % 32 == 0;
+    for (int32_t sq = 0; direct && sq < seq_count; ++sq) {
+        direct = c->lens[(size_t)(seq_begin + sq)] % 32 == 0;
+    }
+    if (direct) {
+        const bool scales = c->cfg.mode == WEED_HIP_KV_LLOYDMAX;
+        ek.direct = DirectOut{ c->k.fields, c->k.region_bytes, scales ? c->k.alpha : nullptr, nullptr, c->lens_dev,
+                               seq_begin, c->padded_tokens, c->k.w, 0 };
+        ev.direct = DirectOut{ c->v.fields, c->v.region_bytes, scales ? c->v.alpha : nullptr,
+                               scales ? c->v.alpha_max : nullptr, c->lens_dev, seq_begin, c->padded_tokens, c->v.w, 1 };
+    }
     const size_t smem = sizeof(float) * (2 * kEncRows * (d + 1) + kEncRows) + sizeof(unsigned long long) * kEncRows;
     const uint32_t blocks = (rows + kEncRows - 1) / kEncRows;
     int parts = 1;
@@ -725,7 +823,7 @@ int encode_both(weed_hip_kv_cache *c, int32_t seq_begin, int32_t seq_count, int3
         }
         WEED_HIP_LAUNCH_CHECK();
     }
-    return pack_rows(c, seq_begin, seq_count, T_new);
+    return direct ? WEED_HIP_OK : pack_rows(c, seq_begin, seq_count, T_new);
 }
 
 // Second stage of an append: the one-field-per-byte rows in the scratch buffers (K rows, then V rows, each in
