@@ -287,6 +287,39 @@ def test_every_pair_of_field_widths(gpu, oracle, d, wk, wv):
     cache.close()
 
 
+@pytest.mark.parametrize("wk,wv,Hq", [(2, 2, 2), (3, 4, 8), (4, 4, 16), (4, 3, 4), (4, 2, 32)])
+def test_head_dim_256(gpu, oracle, wk, wv, Hq):
+    """head_dim 256 on the matrix cores (fields of 2 to 4 bits, up to 8 heads per KV head; 16 heads per KV head fall
+    back to the generic kernel): ragged lengths, both coders, rotations, a chunk of two positions."""
+    import torch
+    rng = np.random.default_rng(wk * 10 + wv + Hq)
+    d, Hkv, lens = 256, 2, [130, 64, 257]
+    S = len(lens)
+    K = rng.standard_normal((S, Hkv, max(lens), d), dtype=np.float32)
+    V = rng.standard_normal((S, Hkv, max(lens), d), dtype=np.float32)
+    q = rng.standard_normal((S, Hq, d), dtype=np.float32)
+    Rk, Rv = rotations(oracle, d, wk)
+    flags = gpu.ATTN_ROTATE_Q | gpu.ATTN_UNROTATE_OUT
+    for lloyd in (True, False):
+        (kb, ks), (vb, vs) = ((wk - 1, 1), (wv, 0)) if lloyd else ((wk, 0), (wv, 0))
+        wl = workloads.Workload("d256", S, Hq, Hkv, d, lens, kb, vb, ks, vs, 0)
+        cache = build_cache(gpu, wl, gpu.KV_LLOYDMAX if lloyd else gpu.KV_UNIFORM, K, V, (Rk, Rv),
+                            None if lloyd else (1.0, 1.1), rotate=2)
+        for gqa, weed in ((gpu.GQA_WEED, True), (gpu.GQA_BLOCKED, False)):
+            want = checker_output(oracle, gpu, cache, wl, q, weed, Rk, Rv)
+            assert_attn_close(run_decode(gpu, cache, q, gqa, flags), want, "d 256, %d + %d bits" % (wk, wv))
+        if Hq // Hkv <= 4:
+            T = 2
+            qc = rng.standard_normal((S, T, Hq, d), dtype=np.float32)
+            out = torch.zeros((S, T, Hq, d), device="cuda")
+            cache.decode_attn_chunk(dev(qc), out, gqa_mapping=gpu.GQA_WEED, flags=flags)
+            for t in range(T):
+                wl_t = workloads.Workload("d256", S, Hq, Hkv, d, [n - (T - 1 - t) for n in lens], kb, vb, ks, vs, 0)
+                want = checker_output(oracle, gpu, cache, wl_t, np.ascontiguousarray(qc[:, t]), True, Rk, Rv)
+                assert_attn_close(out[:, t].cpu().numpy(), want, "chunk position %d" % t)
+        cache.close()
+
+
 @pytest.mark.parametrize("kb,vb,d", [(8, 8, 128), (8, 8, 64), (5, 5, 128), (5, 4, 64), (5, 6, 64), (8, 4, 128),
                                      (1, 7, 32)])
 def test_uniform_widths_beyond_four_bits(gpu, oracle, kb, vb, d):

@@ -7,9 +7,15 @@ int launch_mfma_decode_d64_uniform(const MfmaParams &p, hipStream_t s);
 int launch_mfma_decode_d64_lloyd(const MfmaParams &p, hipStream_t s);
 int launch_mfma_decode_d128_uniform(const MfmaParams &p, hipStream_t s);
 int launch_mfma_decode_d128_lloyd(const MfmaParams &p, hipStream_t s);
+int launch_mfma_decode_d256_uniform(const MfmaParams &p, hipStream_t s);
+int launch_mfma_decode_d256_lloyd(const MfmaParams &p, hipStream_t s);
 
 bool mfma_decode_supported(uint32_t d, uint32_t wk, uint32_t wv, uint32_t G)
 {
+    if (d == 256) {
+        // 64 output registers per lane: fields of 2..4 bits and groups up to 8 only
+        return wk >= 2 && wk <= 4 && wv >= 2 && wv <= 4 && G >= 1 && G <= 8;
+    }
     // fields of 2..5 bits through lookup tables, or the uniform coder's 8-bit codes on both sides
     const bool widths = (wk >= 2 && wk <= 5 && wv >= 2 && wv <= 5) || (wk == 8 && wv == 8);
     return (d == 64 || d == 128) && widths && G >= 1 && G <= 16;
@@ -26,6 +32,9 @@ int launch_mfma_decode(const MfmaParams &p, uint32_t d, hipStream_t s)
     const bool lloyd = p.k.alpha != nullptr;
     if (d == 64) {
         return lloyd ? launch_mfma_decode_d64_lloyd(p, s) : launch_mfma_decode_d64_uniform(p, s);
+    }
+    if (d == 256) {
+        return lloyd ? launch_mfma_decode_d256_lloyd(p, s) : launch_mfma_decode_d256_uniform(p, s);
     }
     return lloyd ? launch_mfma_decode_d128_lloyd(p, s) : launch_mfma_decode_d128_uniform(p, s);
 }

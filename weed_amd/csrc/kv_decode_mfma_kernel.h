@@ -764,7 +764,12 @@ template <int D, int WK, int WV, bool LLOYD> int launch_one(const MfmaParams &p,
     if (p.G <= 8) {
         return launch_gp<D, WK, WV, 8, LLOYD>(p, s);
     }
-    return launch_gp<D, WK, WV, 16, LLOYD>(p, s);
+    if constexpr (D <= 128) {
+        return launch_gp<D, WK, WV, 16, LLOYD>(p, s);
+    } else {
+        // (64 output registers per lane at head_dim 256 leave no room for the 16-column variant)
+        return fail(WEED_HIP_EINVAL, "decode_mfma: groups above 8 are not served at head_dim %d", D);
+    }
 }
 
 template <int D, bool LLOYD> int launch_d(const MfmaParams &p, hipStream_t s)
@@ -783,6 +788,7 @@ template <int D, bool LLOYD> int launch_d(const MfmaParams &p, hipStream_t s)
     WEED_CASE(4, 2)
     WEED_CASE(4, 3)
     WEED_CASE(4, 4)
+    if constexpr (D <= 128) {
     // 5-bit fields: 4-bit codes with the residual sign (or 5-bit uniform codes)
     WEED_CASE(5, 2)
     WEED_CASE(5, 3)
@@ -793,6 +799,7 @@ template <int D, bool LLOYD> int launch_d(const MfmaParams &p, hipStream_t s)
     WEED_CASE(4, 5)
     if constexpr (!LLOYD) {
         WEED_CASE(8, 8) // kv_quant_bits = 8 of the reference's uniform coder
+    }
     }
 #undef WEED_CASE
     return fail(WEED_HIP_EINVAL, "decode_mfma: unsupported field widths %u / %u", wk, wv);

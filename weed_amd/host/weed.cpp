@@ -1323,6 +1323,11 @@ tcapint MultiHeadAttention::positions_per_pass() const
     const tcapint G = num_heads / num_kv_heads;
     const int wk = (k_bits ? k_bits : kv_quant_bits) + ((kv_coder == KV_LLOYDMAX && k_sign) ? 1 : 0);
     const int wv = (v_bits ? v_bits : kv_quant_bits) + ((kv_coder == KV_LLOYDMAX && v_sign) ? 1 : 0);
+    if (head_dim == 256U) {
+        // half the rows there: fields of 2..4 bits, at most 8 (position, head) pairs
+        const bool narrow = wk >= 2 && wk <= 4 && wv >= 2 && wv <= 4;
+        return (narrow && G <= 8U) ? std::max<tcapint>(1U, 8U / G) : 1U;
+    }
     const bool widths = (wk >= 2 && wk <= 5 && wv >= 2 && wv <= 5) || (wk == 8 && wv == 8);
     const bool tiles = G <= 16U && (head_dim == 64U || head_dim == 128U) && widths;
     return tiles ? std::max<tcapint>(1U, 16U / G) : 1U;
