@@ -287,6 +287,25 @@ def test_every_pair_of_field_widths(gpu, oracle, d, wk, wv):
     cache.close()
 
 
+@pytest.mark.parametrize("d,Hkv,G", [(128, 1, 32), (64, 2, 24), (128, 2, 40), (256, 1, 12), (64, 1, 71)])
+def test_groups_larger_than_a_tile(gpu, oracle, d, Hkv, G):
+    """Multi-query shapes (one or two KV heads for dozens of query heads): the group goes through the cache in several
+    passes of the matrix-core kernel, 16 heads (8 at head_dim 256) at most per pass, one merge for all of them; both
+    GQA mappings, ragged lengths, group sizes that do not split evenly."""
+    rng = np.random.default_rng(d + Hkv + G)
+    lens = [190, 64, 3]
+    S, Hq = len(lens), Hkv * G
+    K = rng.standard_normal((S, Hkv, max(lens), d), dtype=np.float32)
+    V = rng.standard_normal((S, Hkv, max(lens), d), dtype=np.float32)
+    q = rng.standard_normal((S, Hq, d), dtype=np.float32)
+    wl = workloads.Workload("mqa", S, Hq, Hkv, d, lens, 3, 4, 1, 0, 0)
+    cache = build_cache(gpu, wl, gpu.KV_LLOYDMAX, K, V)
+    for gqa, weed in ((gpu.GQA_WEED, True), (gpu.GQA_BLOCKED, False)):
+        want = checker_output(oracle, gpu, cache, wl, q, weed)
+        assert_attn_close(run_decode(gpu, cache, q, gqa, 0), want, "group of %d" % G)
+    cache.close()
+
+
 @pytest.mark.parametrize("wk,wv,Hq", [(2, 2, 2), (3, 4, 8), (4, 4, 16), (4, 3, 4), (4, 2, 32)])
 def test_head_dim_256(gpu, oracle, wk, wv, Hq):
     """head_dim 256 on the matrix cores (fields of 2 to 4 bits, up to 8 heads per KV head; 16 heads per KV head fall

@@ -704,7 +704,11 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         max_len = std::max(max_len, (uint32_t)l);
     }
     const uint32_t G = Hq / Hkv;
-    const bool use_mfma = mfma_decode_supported(d, c->k.w, c->v.w, G);
+    // groups beyond a tile's rows take several passes of the matrix-core kernel (a chunk of positions must fit one)
+    const uint32_t tile_rows = mfma_decode_tile_rows(d);
+    const uint32_t passes = n_tokens == 1 ? (G + tile_rows - 1) / tile_rows : 1;
+    const uint32_t pass_heads = (G + passes - 1) / passes;
+    const bool use_mfma = mfma_decode_supported(d, c->k.w, c->v.w, pass_heads);
     WEED_HIP_REQUIRE(n_tokens == 1 || use_mfma,
                      "%s: %u positions x %u heads per KV head (at most 16 rows), head_dim %u: not served by the chunk kernel",
                      fn, n_tokens, real_heads / Hkv, d);
@@ -721,7 +725,7 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         blocks *= Hkv;
         WEED_HIP_REQUIRE(blocks < (1ull << 32), "%s: too many cached tokens for one launch", fn);
         total_blocks = (uint32_t)blocks;
-        runs.waves = mfma_decode_workgroup_waves(G, d, c->k.w, c->v.w);
+        runs.waves = mfma_decode_workgroup_waves(pass_heads, d, c->k.w, c->v.w);
         uint32_t target_units = runs.waves * 256u; // one workgroup per compute unit
         if (const char *env = std::getenv("WEED_HIP_DECODE_WAVES")) {
             target_units = (uint32_t)std::max(1, std::atoi(env)); // tuning knob
@@ -818,8 +822,12 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         mp.total_blocks = total_blocks;
         mp.runs = runs;
         mp.max_slots = n_splits;
+        mp.group_total = G;
+        mp.tile_rows = pass_heads;
         ProfileScope prof("kv_decode_attn");
-        if (total_blocks) {
+        for (uint32_t first = 0; total_blocks && first < G; first += pass_heads) {
+            mp.head_first = first;
+            mp.G = std::min(pass_heads, G - first);
             WEED_HIP_TRY(launch_mfma_decode(mp, d, stream()));
         }
     } else {

@@ -70,6 +70,9 @@ struct MfmaParams {
     // heads; pair hc stands for position hc % q_tokens (blocked) or hc / real_group (Weed mapping), and position t
     // does not see the last q_tokens - 1 - t tokens
     uint32_t q_tokens, real_group;
+    // groups larger than a tile has rows go through the cache in several launches: this one serves the heads
+    // [head_first, head_first + G) of the group_total that share a KV head; tile_rows (0: G) picks the kernel instance
+    uint32_t head_first, group_total, tile_rows;
     const uint16_t *q_hi;   // [n_seq][Hq][d] fp16 bits: high half of the scaled, normalised query
     const uint16_t *q_lo;   // [n_seq][Hq][d] fp16 bits: what the high half misses
     const float *q_scale;   // [n_seq][Hq] power of two the query was divided by
@@ -85,6 +88,8 @@ struct MfmaParams {
 };
 
 bool mfma_decode_supported(uint32_t d, uint32_t wk, uint32_t wv, uint32_t G);
+// Heads of a group that one launch can take (rows of its tile): 16, or 8 at head_dim 256.
+uint32_t mfma_decode_tile_rows(uint32_t d);
 // Shapes whose 64-token block is large (7 KB or more of packed K + V per wavefront) run with two register buffers
 // per wavefront and two wavefronts per SIMD: the deeper prefetch is worth more than the third wavefront there.  Smaller
 // blocks run single-buffered with three wavefronts per SIMD.  The 16-column variant (groups above 8) and head_dim 256

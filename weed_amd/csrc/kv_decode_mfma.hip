@@ -10,15 +10,21 @@ int launch_mfma_decode_d128_lloyd(const MfmaParams &p, hipStream_t s);
 int launch_mfma_decode_d256_uniform(const MfmaParams &p, hipStream_t s);
 int launch_mfma_decode_d256_lloyd(const MfmaParams &p, hipStream_t s);
 
+uint32_t mfma_decode_tile_rows(uint32_t d) { return d == 256 ? 8u : 16u; }
+
+// `G` heads per KV head in ONE launch; larger groups are split by the caller.
 bool mfma_decode_supported(uint32_t d, uint32_t wk, uint32_t wv, uint32_t G)
 {
+    if (G < 1 || G > mfma_decode_tile_rows(d)) {
+        return false;
+    }
     if (d == 256) {
-        // 64 output registers per lane: fields of 2..4 bits and groups up to 8 only
-        return wk >= 2 && wk <= 4 && wv >= 2 && wv <= 4 && G >= 1 && G <= 8;
+        // 64 output registers per lane: fields of 2..4 bits only
+        return wk >= 2 && wk <= 4 && wv >= 2 && wv <= 4;
     }
     // fields of 2..5 bits through lookup tables, or the uniform coder's 8-bit codes on both sides
     const bool widths = (wk >= 2 && wk <= 5 && wv >= 2 && wv <= 5) || (wk == 8 && wv == 8);
-    return (d == 64 || d == 128) && widths && G >= 1 && G <= 16;
+    return (d == 64 || d == 128) && widths;
 }
 
 uint32_t mfma_decode_workgroup_waves(uint32_t G, uint32_t d, uint32_t wk, uint32_t wv)

@@ -227,6 +227,13 @@ template <int GP> __device__ __forceinline__ float head_sum(float v)
     return v + __shfl_xor(v, 32);
 }
 
+// Query head that row `x` of this launch's tile stands for under KV head `kvh`: the launch covers the rows
+// [head_first, head_first + G) of the group_total heads that share the KV head.
+__device__ __forceinline__ uint32_t q_head_of(const MfmaParams &p, uint32_t kvh, uint32_t x)
+{
+    return p.blocked ? kvh * p.group_total + p.head_first + x : (p.head_first + x) * p.Hkv + kvh;
+}
+
 // Bank mask (4-lane banks of a row) of the lanes [GP*i, GP*i + GP).
 template <int GP, int I> constexpr int bank_mask_of() { return ((1 << (GP / 4)) - 1) << (I * GP / 4); }
 
@@ -405,7 +412,7 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
         const uint32_t col_head = PACKED ? c % GP : c;
         const uint32_t col_part = PACKED ? c / GP : 0; // 0: high half, 1: low half, above: unused column
         const bool col_ok = col_head < p.G && col_part < 2;
-        const uint32_t qh = col_ok ? (p.blocked ? kvh * p.G + col_head : col_head * p.Hkv + kvh) : 0;
+        const uint32_t qh = col_ok ? q_head_of(p, kvh, col_head) : 0;
         const uint64_t qbase = ((uint64_t)seq * p.Hq + qh) * D + g * (D / 4);
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
@@ -427,7 +434,7 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     // multi-token chunk), and the largest such count over the pairs
     const uint32_t hidden_max = p.q_tokens - 1U;
     const uint32_t hidden = (hidden_max && head_ok) ? hidden_max - (p.blocked ? hc % p.q_tokens : hc / p.real_group) : 0U;
-    const uint32_t qh_c = head_ok ? (p.blocked ? kvh * p.G + hc : hc * p.Hkv + kvh) : 0;
+    const uint32_t qh_c = head_ok ? q_head_of(p, kvh, hc) : 0;
     const float qscale = head_ok ? p.q_scale[(uint64_t)seq * p.Hq + qh_c] : 0.0f;
     const float betaq = head_ok ? p.k.beta * p.q_sum[(uint64_t)seq * p.Hq + qh_c] : 0.0f;
 
@@ -714,7 +721,7 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     for (int r = 0; r < 4; ++r) {
         const uint32_t hs = 4 * g + r;
         if (hs < p.G) {
-            const uint32_t head = p.blocked ? kvh * p.G + hs : hs * p.Hkv + kvh;
+            const uint32_t head = q_head_of(p, kvh, hs);
             float *dst = p.partials + (((uint64_t)seq * p.Hq + head) * p.max_slots + slot) * PS;
 #pragma unroll
             for (int jb = 0; jb < JB; ++jb) {
@@ -725,7 +732,7 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     }
     if (g == 0 && c < p.G) {
         // lane c of row 0 holds head c (c < GP)
-        const uint32_t head = p.blocked ? kvh * p.G + c : c * p.Hkv + kvh;
+        const uint32_t head = q_head_of(p, kvh, c);
         float *dst = p.partials + (((uint64_t)seq * p.Hq + head) * p.max_slots + slot) * PS;
         dst[0] = m_run;
         dst[1] = l_head;
@@ -758,10 +765,12 @@ template <int D, int WK, int WV, int GP, bool LLOYD> int launch_gp(const MfmaPar
 
 template <int D, int WK, int WV, bool LLOYD> int launch_one(const MfmaParams &p, hipStream_t s)
 {
-    if (p.G <= 4) {
+    // (all launches of a call use the instance of the call's largest pass, for which the runs were cut)
+    const uint32_t rows = p.tile_rows ? p.tile_rows : p.G;
+    if (rows <= 4) {
         return launch_gp<D, WK, WV, 4, LLOYD>(p, s);
     }
-    if (p.G <= 8) {
+    if (rows <= 8) {
         return launch_gp<D, WK, WV, 8, LLOYD>(p, s);
     }
     if constexpr (D <= 128) {
