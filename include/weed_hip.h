@@ -282,8 +282,8 @@ int weed_hip_kv_decode_attn_prefix(weed_hip_kv_cache *cache, const int32_t *lens
  * 322-328).  The last n_tokens of the attended tokens (lens_dev[s], or the cached length when lens_dev is NULL) are
  * the chunk's own: position t attends to all but the last n_tokens - 1 - t of them.  q_dev / out_dev: logical
  * [n_seq, n_tokens, n_q_heads, d] with strides in elements.  The (position, head) pairs of a KV head are the rows of
- * one matrix tile, so n_tokens * (n_q_heads / n_kv_heads) may not exceed 16, head_dim must be 64 or 128 and the
- * fields 2..5 bits wide (or 8 + 8 bits, uniform coder); head_dim 256 allows 8 pairs and fields of 2..4 bits; callers
+ * one matrix tile, so n_tokens * (n_q_heads / n_kv_heads) may not exceed 16 and the fields must be 2..5 bits wide
+ * (or 8 + 8 bits, uniform coder); head_dim above 128 allows 8 pairs and fields of 2..4 bits; callers
  * with longer chunks split them (each part with its own lens_dev) or dequantise once and attend densely. */
 int weed_hip_kv_decode_attn_chunk(weed_hip_kv_cache *cache, const int32_t *lens_dev, int32_t n_tokens,
                                   int32_t n_q_heads, int32_t gqa_mapping, const float *q_dev, uint32_t q_off,

@@ -261,7 +261,7 @@ def test_head_dims_and_wide_groups(gpu, oracle):
         cache.close()
 
 
-@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("d", [32, 64, 96, 128])
 @pytest.mark.parametrize("wk", [2, 3, 4, 5])
 @pytest.mark.parametrize("wv", [2, 3, 4, 5])
 def test_every_pair_of_field_widths(gpu, oracle, d, wk, wv):
@@ -287,7 +287,8 @@ def test_every_pair_of_field_widths(gpu, oracle, d, wk, wv):
     cache.close()
 
 
-@pytest.mark.parametrize("d,Hkv,G", [(128, 1, 32), (64, 2, 24), (128, 2, 40), (256, 1, 12), (64, 1, 71)])
+@pytest.mark.parametrize("d,Hkv,G", [(128, 1, 32), (64, 2, 24), (128, 2, 40), (256, 1, 12), (64, 1, 71), (96, 1, 32),
+                                     (32, 2, 20)])
 def test_groups_larger_than_a_tile(gpu, oracle, d, Hkv, G):
     """Multi-query shapes (one or two KV heads for dozens of query heads): the group goes through the cache in several
     passes of the matrix-core kernel, 16 heads (8 at head_dim 256) at most per pass, one merge for all of them; both
@@ -306,13 +307,14 @@ def test_groups_larger_than_a_tile(gpu, oracle, d, Hkv, G):
     cache.close()
 
 
+@pytest.mark.parametrize("d", [160, 192, 224, 256])
 @pytest.mark.parametrize("wk,wv,Hq", [(2, 2, 2), (3, 4, 8), (4, 4, 16), (4, 3, 4), (4, 2, 32)])
-def test_head_dim_256(gpu, oracle, wk, wv, Hq):
-    """head_dim 256 on the matrix cores (fields of 2 to 4 bits, up to 8 heads per KV head; 16 heads per KV head fall
-    back to the generic kernel): ragged lengths, both coders, rotations, a chunk of two positions."""
+def test_head_dims_above_128(gpu, oracle, d, wk, wv, Hq):
+    """head_dim 160 to 256 on the matrix cores (fields of 2 to 4 bits, up to 8 heads per KV head and pass; 16 heads
+    per KV head take two passes): ragged lengths, both coders, rotations, a chunk of two positions."""
     import torch
-    rng = np.random.default_rng(wk * 10 + wv + Hq)
-    d, Hkv, lens = 256, 2, [130, 64, 257]
+    rng = np.random.default_rng(wk * 10 + wv + Hq + d)
+    Hkv, lens = 2, [130, 64, 257]
     S = len(lens)
     K = rng.standard_normal((S, Hkv, max(lens), d), dtype=np.float32)
     V = rng.standard_normal((S, Hkv, max(lens), d), dtype=np.float32)
@@ -321,26 +323,26 @@ def test_head_dim_256(gpu, oracle, wk, wv, Hq):
     flags = gpu.ATTN_ROTATE_Q | gpu.ATTN_UNROTATE_OUT
     for lloyd in (True, False):
         (kb, ks), (vb, vs) = ((wk - 1, 1), (wv, 0)) if lloyd else ((wk, 0), (wv, 0))
-        wl = workloads.Workload("d256", S, Hq, Hkv, d, lens, kb, vb, ks, vs, 0)
+        wl = workloads.Workload("wide_heads", S, Hq, Hkv, d, lens, kb, vb, ks, vs, 0)
         cache = build_cache(gpu, wl, gpu.KV_LLOYDMAX if lloyd else gpu.KV_UNIFORM, K, V, (Rk, Rv),
                             None if lloyd else (1.0, 1.1), rotate=2)
         for gqa, weed in ((gpu.GQA_WEED, True), (gpu.GQA_BLOCKED, False)):
             want = checker_output(oracle, gpu, cache, wl, q, weed, Rk, Rv)
-            assert_attn_close(run_decode(gpu, cache, q, gqa, flags), want, "d 256, %d + %d bits" % (wk, wv))
+            assert_attn_close(run_decode(gpu, cache, q, gqa, flags), want, "d %d, %d + %d bits" % (d, wk, wv))
         if Hq // Hkv <= 4:
             T = 2
             qc = rng.standard_normal((S, T, Hq, d), dtype=np.float32)
             out = torch.zeros((S, T, Hq, d), device="cuda")
             cache.decode_attn_chunk(dev(qc), out, gqa_mapping=gpu.GQA_WEED, flags=flags)
             for t in range(T):
-                wl_t = workloads.Workload("d256", S, Hq, Hkv, d, [n - (T - 1 - t) for n in lens], kb, vb, ks, vs, 0)
+                wl_t = workloads.Workload("wide_heads", S, Hq, Hkv, d, [n - (T - 1 - t) for n in lens], kb, vb, ks, vs, 0)
                 want = checker_output(oracle, gpu, cache, wl_t, np.ascontiguousarray(qc[:, t]), True, Rk, Rv)
                 assert_attn_close(out[:, t].cpu().numpy(), want, "chunk position %d" % t)
         cache.close()
 
 
-@pytest.mark.parametrize("kb,vb,d", [(8, 8, 128), (8, 8, 64), (5, 5, 128), (5, 4, 64), (5, 6, 64), (8, 4, 128),
-                                     (1, 7, 32)])
+@pytest.mark.parametrize("kb,vb,d", [(8, 8, 128), (8, 8, 64), (8, 8, 96), (8, 8, 32), (5, 5, 128), (5, 4, 64),
+                                     (5, 6, 64), (8, 4, 128), (1, 7, 32)])
 def test_uniform_widths_beyond_four_bits(gpu, oracle, kb, vb, d):
     """Weed's uniform coder at any width the reference's `kv_quant_bits` may take: attention equals the checker on the
     same codes, with rotations and both GQA mappings.  8 + 8 bits (the common request) runs on the matrix cores, its
@@ -408,7 +410,8 @@ def test_prefix_lengths_override(gpu, oracle):
 
 @pytest.mark.parametrize("lloyd,d,Hkv,Hq,T,gqa_weed", [(False, 64, 2, 4, 3, True), (True, 128, 2, 8, 2, False),
                                                        (True, 128, 1, 4, 4, True), (False, 128, 2, 2, 5, False),
-                                                       (True, 64, 2, 16, 2, True), (True, 128, 2, 8, 4, False)])
+                                                       (True, 64, 2, 16, 2, True), (True, 128, 2, 8, 4, False),
+                                                       (True, 96, 2, 8, 3, True), (False, 32, 1, 4, 4, False)])
 def test_chunk_of_query_positions(gpu, oracle, lloyd, d, Hkv, Hq, T, gqa_weed):
     """Several query positions per sequence in one pass over the cache: position t must equal the checker run over
     all but the last T - 1 - t tokens.  The lengths put the chunk across a block boundary (a block whose tokens are

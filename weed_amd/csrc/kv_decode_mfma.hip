@@ -3,14 +3,24 @@
 
 namespace weedhip {
 
+int launch_mfma_decode_d32_uniform(const MfmaParams &p, hipStream_t s);
+int launch_mfma_decode_d32_lloyd(const MfmaParams &p, hipStream_t s);
+int launch_mfma_decode_d96_uniform(const MfmaParams &p, hipStream_t s);
+int launch_mfma_decode_d96_lloyd(const MfmaParams &p, hipStream_t s);
 int launch_mfma_decode_d64_uniform(const MfmaParams &p, hipStream_t s);
 int launch_mfma_decode_d64_lloyd(const MfmaParams &p, hipStream_t s);
 int launch_mfma_decode_d128_uniform(const MfmaParams &p, hipStream_t s);
 int launch_mfma_decode_d128_lloyd(const MfmaParams &p, hipStream_t s);
+int launch_mfma_decode_d160_uniform(const MfmaParams &p, hipStream_t s);
+int launch_mfma_decode_d160_lloyd(const MfmaParams &p, hipStream_t s);
+int launch_mfma_decode_d192_uniform(const MfmaParams &p, hipStream_t s);
+int launch_mfma_decode_d192_lloyd(const MfmaParams &p, hipStream_t s);
+int launch_mfma_decode_d224_uniform(const MfmaParams &p, hipStream_t s);
+int launch_mfma_decode_d224_lloyd(const MfmaParams &p, hipStream_t s);
 int launch_mfma_decode_d256_uniform(const MfmaParams &p, hipStream_t s);
 int launch_mfma_decode_d256_lloyd(const MfmaParams &p, hipStream_t s);
 
-uint32_t mfma_decode_tile_rows(uint32_t d) { return d == 256 ? 8u : 16u; }
+uint32_t mfma_decode_tile_rows(uint32_t d) { return d > 128 ? 8u : 16u; }
 
 // `G` heads per KV head in ONE launch; larger groups are split by the caller.
 bool mfma_decode_supported(uint32_t d, uint32_t wk, uint32_t wv, uint32_t G)
@@ -18,13 +28,13 @@ bool mfma_decode_supported(uint32_t d, uint32_t wk, uint32_t wv, uint32_t G)
     if (G < 1 || G > mfma_decode_tile_rows(d)) {
         return false;
     }
-    if (d == 256) {
-        // 64 output registers per lane: fields of 2..4 bits only
+    if (d == 160 || d == 192 || d == 224 || d == 256) {
+        // up to 64 output registers per lane: fields of 2..4 bits only
         return wk >= 2 && wk <= 4 && wv >= 2 && wv <= 4;
     }
     // fields of 2..5 bits through lookup tables, or the uniform coder's 8-bit codes on both sides
     const bool widths = (wk >= 2 && wk <= 5 && wv >= 2 && wv <= 5) || (wk == 8 && wv == 8);
-    return (d == 64 || d == 128) && widths;
+    return (d == 32 || d == 64 || d == 96 || d == 128) && widths;
 }
 
 uint32_t mfma_decode_workgroup_waves(uint32_t G, uint32_t d, uint32_t wk, uint32_t wv)
@@ -36,8 +46,23 @@ uint32_t mfma_decode_workgroup_waves(uint32_t G, uint32_t d, uint32_t wk, uint32
 int launch_mfma_decode(const MfmaParams &p, uint32_t d, hipStream_t s)
 {
     const bool lloyd = p.k.alpha != nullptr;
+    if (d == 32) {
+        return lloyd ? launch_mfma_decode_d32_lloyd(p, s) : launch_mfma_decode_d32_uniform(p, s);
+    }
     if (d == 64) {
         return lloyd ? launch_mfma_decode_d64_lloyd(p, s) : launch_mfma_decode_d64_uniform(p, s);
+    }
+    if (d == 96) {
+        return lloyd ? launch_mfma_decode_d96_lloyd(p, s) : launch_mfma_decode_d96_uniform(p, s);
+    }
+    if (d == 160) {
+        return lloyd ? launch_mfma_decode_d160_lloyd(p, s) : launch_mfma_decode_d160_uniform(p, s);
+    }
+    if (d == 192) {
+        return lloyd ? launch_mfma_decode_d192_lloyd(p, s) : launch_mfma_decode_d192_uniform(p, s);
+    }
+    if (d == 224) {
+        return lloyd ? launch_mfma_decode_d224_lloyd(p, s) : launch_mfma_decode_d224_uniform(p, s);
     }
     if (d == 256) {
         return lloyd ? launch_mfma_decode_d256_lloyd(p, s) : launch_mfma_decode_d256_uniform(p, s);

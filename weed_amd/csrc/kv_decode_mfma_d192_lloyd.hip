@@ -1,0 +1,9 @@
+// Instantiates the matrix-core decode kernel for head_dim 192, Lloyd-Max coder (fields of 2..4 bits, groups up to 8).
+#include "kv_decode_mfma_kernel.h"
+
+namespace weedhip {
+int launch_mfma_decode_d192_lloyd(const MfmaParams &p, hipStream_t s)
+{
+    return weedhip_mfma::launch_d<192, true>(p, s);
+}
+} // namespace weedhip

@@ -30,7 +30,7 @@ typedef float float4v __attribute__((ext_vector_type(4)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
 
-// N dwords from a pointer aligned to 16 bytes when N % 4 == 0, else to 8 bytes (N is even for every supported shape).
+// N dwords from a pointer aligned to 16 bytes when N % 4 == 0, to 8 bytes when N is even, else to 4.
 // `base` is the same in every lane and `lane_off` a 32-bit byte offset, so the loads take the scalar-base form (one
 // offset register per lane instead of a 64-bit address).
 template <int N> __device__ __forceinline__ void load_dwords(const uint8_t *base, uint32_t lane_off, uint32_t (&x)[N])
@@ -45,13 +45,18 @@ template <int N> __device__ __forceinline__ void load_dwords(const uint8_t *base
             x[4 * i + 2] = v.z;
             x[4 * i + 3] = v.w;
         }
-    } else {
-        static_assert(N % 2 == 0, "lane runs are multiples of 8 bytes");
+    } else if constexpr (N % 2 == 0) {
 #pragma unroll
         for (int i = 0; i < N / 2; ++i) {
             const uint2v v = *reinterpret_cast<const uint2v *>(p + 8 * i);
             x[2 * i] = v.x;
             x[2 * i + 1] = v.y;
+        }
+    } else {
+        // odd runs (head_dim 96 with an odd field width): dword by dword
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            x[i] = *reinterpret_cast<const uint32_t *>(p + 4 * i);
         }
     }
 }

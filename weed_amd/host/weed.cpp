@@ -1316,20 +1316,20 @@ TensorPtr MultiHeadAttention::forward_quantized(TensorPtr Q, TensorPtr K, Tensor
 }
 
 // Query positions that one pass of the fused kernel serves: the (position, head) pairs of a KV head are the rows of
-// one matrix tile (16), which exists for head_dim 64 / 128 and fields of 2..5 bits or 8 + 8; any other shape goes through the
+// one matrix tile (16), which exists for head_dim 32 / 64 / 96 / 128 (256 with half the rows) and fields of 2..5 bits or 8 + 8; any other shape goes through the
 // generic kernel one position at a time.
 tcapint MultiHeadAttention::positions_per_pass() const
 {
     const tcapint G = num_heads / num_kv_heads;
     const int wk = (k_bits ? k_bits : kv_quant_bits) + ((kv_coder == KV_LLOYDMAX && k_sign) ? 1 : 0);
     const int wv = (v_bits ? v_bits : kv_quant_bits) + ((kv_coder == KV_LLOYDMAX && v_sign) ? 1 : 0);
-    if (head_dim == 256U) {
+    if (head_dim > 128) {
         // half the rows there: fields of 2..4 bits, at most 8 (position, head) pairs
         const bool narrow = wk >= 2 && wk <= 4 && wv >= 2 && wv <= 4;
         return (narrow && G <= 8U) ? std::max<tcapint>(1U, 8U / G) : 1U;
     }
     const bool widths = (wk >= 2 && wk <= 5 && wv >= 2 && wv <= 5) || (wk == 8 && wv == 8);
-    const bool tiles = G <= 16U && (head_dim == 64U || head_dim == 128U) && widths;
+    const bool tiles = G <= 16U && (head_dim == 32U || head_dim == 64U || head_dim == 96U || head_dim == 128U) && widths;
     return tiles ? std::max<tcapint>(1U, 16U / G) : 1U;
 }
 
