@@ -283,7 +283,7 @@ int weed_hip_kv_decode_attn_prefix(weed_hip_kv_cache *cache, const int32_t *lens
  * the chunk's own: position t attends to all but the last n_tokens - 1 - t of them.  q_dev / out_dev: logical
  * [n_seq, n_tokens, n_q_heads, d] with strides in elements.  The (position, head) pairs of a KV head are the rows of
  * one matrix tile, so n_tokens * (n_q_heads / n_kv_heads) may not exceed 16 and the fields must be 2..5 bits wide
- * (or 8 + 8 bits, uniform coder); head_dim above 128 allows 8 pairs and fields of 2..4 bits; callers
+ * (or of equal width 1, 6, 7 or 8); head_dim above 128 allows 8 pairs and fields of up to 4 bits; callers
  * with longer chunks split them (each part with its own lens_dev) or dequantise once and attend densely. */
 int weed_hip_kv_decode_attn_chunk(weed_hip_kv_cache *cache, const int32_t *lens_dev, int32_t n_tokens,
                                   int32_t n_q_heads, int32_t gqa_mapping, const float *q_dev, uint32_t q_off,

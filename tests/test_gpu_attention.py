@@ -341,13 +341,15 @@ def test_head_dims_above_128(gpu, oracle, d, wk, wv, Hq):
         cache.close()
 
 
-@pytest.mark.parametrize("kb,vb,d", [(8, 8, 128), (8, 8, 64), (8, 8, 96), (8, 8, 32), (5, 5, 128), (5, 4, 64),
-                                     (5, 6, 64), (8, 4, 128), (1, 7, 32)])
+@pytest.mark.parametrize("kb,vb,d", [(8, 8, 128), (8, 8, 64), (8, 8, 96), (8, 8, 32), (7, 7, 128), (7, 7, 32),
+                                     (6, 6, 64), (6, 6, 96), (1, 1, 128), (1, 1, 32), (1, 1, 256), (5, 5, 128),
+                                     (5, 4, 64), (5, 6, 64), (8, 4, 128), (1, 7, 32)])
 def test_uniform_widths_beyond_four_bits(gpu, oracle, kb, vb, d):
     """Weed's uniform coder at any width the reference's `kv_quant_bits` may take: attention equals the checker on the
-    same codes, with rotations and both GQA mappings.  8 + 8 bits (the common request) runs on the matrix cores, its
-    codes turned into fp16 arithmetically, also for a chunk of query positions and for 16 heads per KV head; 5-bit
-    codes use the single-value tables; the other widths go through the generic kernel."""
+    same codes, with rotations and both GQA mappings.  Equal widths of 6 to 8 bits (8 is the common request) run on the
+    matrix cores, their codes turned into fp16 arithmetically, also for a chunk of query positions and for 16 heads
+    per KV head; 5-bit codes use the single-value tables, 1-bit codes four-entry pair tables; unequal widths beyond
+    five bits go through the generic kernel."""
     import torch
     rng = np.random.default_rng(kb * 16 + vb + d)
     Hkv, Hq, lens = 2, 8, [300, 77, 64]
@@ -366,7 +368,7 @@ def test_uniform_widths_beyond_four_bits(gpu, oracle, kb, vb, d):
     # the codes really use the whole range
     kf, _ = export(cache, 0, 64)
     assert kf.max() == (1 << kb) - 1 and kf.min() == 0
-    if kb == 8 and vb == 8:
+    if kb == vb and kb >= 6:
         T = 2
         qc = rng.standard_normal((S, T, Hq, d), dtype=np.float32)
         out = torch.zeros((S, T, Hq, d), device="cuda")

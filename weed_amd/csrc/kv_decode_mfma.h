@@ -96,13 +96,14 @@ uint32_t mfma_decode_tile_rows(uint32_t d);
 // need too many registers for either and run single-buffered with two.
 constexpr bool mfma_decode_double_buffered(uint32_t gp, uint32_t d, uint32_t wk, uint32_t wv)
 {
-    return gp <= 8 && wk < 8 && d <= 128u && d * (wk + wv) >= 128u * 7u;
+    return gp <= 8 && wk < 6 && d <= 128u && d * (wk + wv) >= 128u * 7u;
 }
 // Wavefronts per workgroup; one workgroup fills a compute unit, so one copy of the lookup tables serves it.
 constexpr uint32_t mfma_decode_waves_per_wg(uint32_t gp, uint32_t d, uint32_t wk, uint32_t wv)
 {
-    // (8-bit fields: 64 registers of packed data per block and wavefront, so one buffer and two wavefronts per SIMD)
-    return (gp > 8 || wk == 8 || d > 128u || mfma_decode_double_buffered(gp, d, wk, wv)) ? 8u : 12u;
+    // (6- to 8-bit fields: up to 64 registers of packed data per block and wavefront, so one buffer and two wavefronts
+    // per SIMD)
+    return (gp > 8 || wk >= 6 || d > 128u || mfma_decode_double_buffered(gp, d, wk, wv)) ? 8u : 12u;
 }
 // Wavefronts per workgroup of the kernel instance that serves this shape (one workgroup fills a compute unit).
 uint32_t mfma_decode_workgroup_waves(uint32_t G, uint32_t d, uint32_t wk, uint32_t wv);

@@ -28,12 +28,14 @@ bool mfma_decode_supported(uint32_t d, uint32_t wk, uint32_t wv, uint32_t G)
     if (G < 1 || G > mfma_decode_tile_rows(d)) {
         return false;
     }
+    const bool one_bit = wk == 1 && wv == 1;
     if (d == 160 || d == 192 || d == 224 || d == 256) {
-        // up to 64 output registers per lane: fields of 2..4 bits only
-        return wk >= 2 && wk <= 4 && wv >= 2 && wv <= 4;
+        // up to 64 output registers per lane: fields of up to 4 bits only
+        return (wk >= 2 && wk <= 4 && wv >= 2 && wv <= 4) || one_bit;
     }
-    // fields of 2..5 bits through lookup tables, or the uniform coder's 8-bit codes on both sides
-    const bool widths = (wk >= 2 && wk <= 5 && wv >= 2 && wv <= 5) || (wk == 8 && wv == 8);
+    // fields of 2..5 bits through lookup tables (any pair of widths), or equal widths of 1 or 6..8 bits (the latter
+    // exist in the uniform coder only)
+    const bool widths = (wk >= 2 && wk <= 5 && wv >= 2 && wv <= 5) || one_bit || (wk == wv && wk >= 6 && wk <= 8);
     return (d == 32 || d == 64 || d == 96 || d == 128) && widths;
 }
 

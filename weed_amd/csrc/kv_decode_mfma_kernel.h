@@ -70,9 +70,9 @@ template <int N> __device__ __forceinline__ void load_dwords(const uint8_t *base
 constexpr uint32_t kTableRowBytes = 256;
 // Rows of one side's table: pair tables (2^(2W) entries) for fields of up to 4 bits; 5-bit fields (4-bit codes with
 // the residual sign) would need 1024 pairs, so they use a table of the 32 single values, each stored twice (both
-// halves of the word), and a pair is assembled from two lookups; 8-bit fields are turned into fp16 values
-// arithmetically and need no table.
-template <int W> constexpr uint32_t side_rows() { return W == 8 ? 0u : (W == 5 ? 32u : 1u << (2 * W)); }
+// halves of the word), and a pair is assembled from two lookups; fields of 6 to 8 bits (uniform coder only) are
+// turned into fp16 values arithmetically and need no table.
+template <int W> constexpr uint32_t side_rows() { return W >= 6 ? 0u : (W == 5 ? 32u : 1u << (2 * W)); }
 template <int WK, int WV> constexpr uint32_t table_rows()
 {
     return side_rows<WK>() > side_rows<WV>() ? side_rows<WK>() : side_rows<WV>();
@@ -151,11 +151,42 @@ template <int N, int P> __device__ __forceinline__ uint32_t pair_from_bytes(cons
     return __builtin_bit_cast(uint32_t, h);
 }
 
+// 6- and 7-bit fields (uniform coder only): the same arithmetic, with the two codes of a pair cut out of the run by
+// bit-field extracts (a funnel shift first where a code straddles two dwords).
+template <int W, int N, int F> __device__ __forceinline__ uint32_t field_bits(const uint32_t (&x)[N])
+{
+    constexpr int bit = W * F;
+    constexpr int dw = bit >> 5, sh = bit & 31;
+    uint32_t t;
+    if constexpr (sh + W <= 32) {
+        asm("v_bfe_u32 %0, %1, %2, %3" : "=v"(t) : "v"(x[dw]), "n"(sh), "n"(W));
+    } else {
+        uint32_t f;
+        asm("v_alignbit_b32 %0, %1, %2, %3" : "=v"(f) : "v"(x[dw + 1 < N ? dw + 1 : dw]), "v"(x[dw]), "n"(sh));
+        asm("v_bfe_u32 %0, %1, 0, %2" : "=v"(t) : "v"(f), "n"(W));
+    }
+    return t;
+}
+template <int W, int N, int P> __device__ __forceinline__ uint32_t pair_from_fields(const uint32_t (&x)[N])
+{
+    const uint32_t lo = field_bits<W, N, 2 * P>(x), hi = field_bits<W, N, 2 * P + 1>(x);
+    const uint32_t a = (lo | (hi << 16)) | 0x64006400u; // fp16 (1024 + code) twice
+    const half2v h = __builtin_bit_cast(half2v, a) + half2v{ (_Float16)-1023.5f, (_Float16)-1023.5f };
+    return __builtin_bit_cast(uint32_t, h);
+}
+
 // Item K (8 fields) of the lane's run -> 8 fp16 values in matrix-operand order.
 template <int W, int N, int K>
 __device__ __forceinline__ half8 dequant_item(const uint32_t (&x)[N], uint32_t lane_byte)
 {
     uint4v r;
+    if constexpr (W == 6 || W == 7) {
+        r.x = pair_from_fields<W, N, 4 * K>(x);
+        r.y = pair_from_fields<W, N, 4 * K + 1>(x);
+        r.z = pair_from_fields<W, N, 4 * K + 2>(x);
+        r.w = pair_from_fields<W, N, 4 * K + 3>(x);
+        return __builtin_bit_cast(half8, r);
+    }
     if constexpr (W == 8) {
         r.x = pair_from_bytes<N, 4 * K>(x);
         r.y = pair_from_bytes<N, 4 * K + 1>(x);
@@ -812,9 +843,13 @@ template <int D, bool LLOYD> int launch_d(const MfmaParams &p, hipStream_t s)
     WEED_CASE(3, 5)
     WEED_CASE(4, 5)
     if constexpr (!LLOYD) {
-        WEED_CASE(8, 8) // kv_quant_bits = 8 of the reference's uniform coder
+        // kv_quant_bits = 6, 7, 8 of the reference's uniform coder
+        WEED_CASE(6, 6)
+        WEED_CASE(7, 7)
+        WEED_CASE(8, 8)
     }
     }
+    WEED_CASE(1, 1) // one-bit codes (pair tables of four entries)
 #undef WEED_CASE
     return fail(WEED_HIP_EINVAL, "decode_mfma: unsupported field widths %u / %u", wk, wv);
 }

@@ -1325,10 +1325,10 @@ tcapint MultiHeadAttention::positions_per_pass() const
     const int wv = (v_bits ? v_bits : kv_quant_bits) + ((kv_coder == KV_LLOYDMAX && v_sign) ? 1 : 0);
     if (head_dim > 128) {
         // half the rows there: fields of 2..4 bits, at most 8 (position, head) pairs
-        const bool narrow = wk >= 2 && wk <= 4 && wv >= 2 && wv <= 4;
+        const bool narrow = (wk >= 2 && wk <= 4 && wv >= 2 && wv <= 4) || (wk == 1 && wv == 1);
         return (narrow && G <= 8U) ? std::max<tcapint>(1U, 8U / G) : 1U;
     }
-    const bool widths = (wk >= 2 && wk <= 5 && wv >= 2 && wv <= 5) || (wk == 8 && wv == 8);
+    const bool widths = (wk >= 2 && wk <= 5 && wv >= 2 && wv <= 5) || (wk == wv && (wk == 1 || (wk >= 6 && wk <= 8)));
     const bool tiles = G <= 16U && (head_dim == 32U || head_dim == 64U || head_dim == 96U || head_dim == 128U) && widths;
     return tiles ? std::max<tcapint>(1U, 16U / G) : 1U;
 }
