@@ -277,14 +277,14 @@ int weed_hip_kv_decode_attn_prefix(weed_hip_kv_cache *cache, const int32_t *lens
                                    int32_t gqa_mapping, const float *q_dev, uint32_t q_off, const uint32_t q_stride[3],
                                    float *out_dev, uint32_t o_off, const uint32_t o_stride[3], uint32_t flags);
 
-/* A chunk of n_tokens query positions per sequence in ONE pass over the packed cache (speculative or chunked
- * decoding; MultiHeadAttention::forward with 1 < T, multihead_attention.cpp:259-348 with the triangular mask of
+/* A chunk of n_tokens (1..64) query positions per sequence with the causal mask inside the kernel (speculative or
+ * chunked decoding; MultiHeadAttention::forward with 1 < T, multihead_attention.cpp:259-348 with the triangular mask of
  * 322-328).  The last n_tokens of the attended tokens (lens_dev[s], or the cached length when lens_dev is NULL) are
  * the chunk's own: position t attends to all but the last n_tokens - 1 - t of them.  q_dev / out_dev: logical
  * [n_seq, n_tokens, n_q_heads, d] with strides in elements.  The (position, head) pairs of a KV head are the rows of
- * one matrix tile, so n_tokens * (n_q_heads / n_kv_heads) may not exceed 16 and the fields must be 2..5 bits wide
- * (or of equal width 1, 6, 7 or 8); head_dim above 128 allows 8 pairs and fields of up to 4 bits; callers
- * with longer chunks split them (each part with its own lens_dev) or dequantise once and attend densely. */
+ * matrix tiles of 16 (8 above head_dim 128): up to that many pairs cost ONE pass over the packed cache, more pairs
+ * one pass per tile.  Needs a shape the matrix-core kernel serves: fields of 2..5 bits, or of equal width 1, 6, 7
+ * or 8 (up to 4 bits above head_dim 128). */
 int weed_hip_kv_decode_attn_chunk(weed_hip_kv_cache *cache, const int32_t *lens_dev, int32_t n_tokens,
                                   int32_t n_q_heads, int32_t gqa_mapping, const float *q_dev, uint32_t q_off,
                                   const uint32_t q_stride[4], float *out_dev, uint32_t o_off,

@@ -413,10 +413,12 @@ def test_prefix_lengths_override(gpu, oracle):
 @pytest.mark.parametrize("lloyd,d,Hkv,Hq,T,gqa_weed", [(False, 64, 2, 4, 3, True), (True, 128, 2, 8, 2, False),
                                                        (True, 128, 1, 4, 4, True), (False, 128, 2, 2, 5, False),
                                                        (True, 64, 2, 16, 2, True), (True, 128, 2, 8, 4, False),
-                                                       (True, 96, 2, 8, 3, True), (False, 32, 1, 4, 4, False)])
+                                                       (True, 96, 2, 8, 3, True), (False, 32, 1, 4, 4, False),
+                                                       (True, 128, 2, 8, 7, False), (False, 64, 1, 4, 11, True),
+                                                       (True, 256, 1, 4, 5, True)])
 def test_chunk_of_query_positions(gpu, oracle, lloyd, d, Hkv, Hq, T, gqa_weed):
-    """Several query positions per sequence in one pass over the cache: position t must equal the checker run over
-    all but the last T - 1 - t tokens.  The lengths put the chunk across a block boundary (a block whose tokens are
+    """Several query positions per sequence in one call (one pass over the cache per tile of (position, head) pairs;
+    the larger cases need two or three): position t must equal the checker run over all but the last T - 1 - t tokens.  The lengths put the chunk across a block boundary (a block whose tokens are
     all hidden from the early positions), inside one block, and far from any edge; both GQA mappings; column-major
     operands; rotations on; and the same with the attended lengths given explicitly."""
     import torch
@@ -459,8 +461,8 @@ def test_chunk_of_query_positions(gpu, oracle, lloyd, d, Hkv, Hq, T, gqa_weed):
     ref1 = torch.zeros_like(q1[:, 0])
     cache.decode_attn(q1[:, 0], ref1, gqa_mapping=gqa, flags=flags)
     assert torch.equal(out1[:, 0], ref1)
-    # more (position, head) pairs per KV head than a tile has rows
-    too_many = dev(np.zeros((S, 17, Hq, d), dtype=np.float32))
+    # more positions than the entry point takes
+    too_many = dev(np.zeros((S, 65, Hq, d), dtype=np.float32))
     with pytest.raises(gpu.WeedHipError):
         cache.decode_attn_chunk(too_many, torch.zeros_like(too_many), gqa_mapping=gqa)
     cache.close()

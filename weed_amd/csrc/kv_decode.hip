@@ -704,14 +704,14 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         max_len = std::max(max_len, (uint32_t)l);
     }
     const uint32_t G = Hq / Hkv;
-    // groups beyond a tile's rows take several passes of the matrix-core kernel (a chunk of positions must fit one)
+    // groups (or chunks: positions x heads) beyond a tile's rows take several passes of the matrix-core kernel
     const uint32_t tile_rows = mfma_decode_tile_rows(d);
-    const uint32_t passes = n_tokens == 1 ? (G + tile_rows - 1) / tile_rows : 1;
+    const uint32_t passes = (G + tile_rows - 1) / tile_rows;
     const uint32_t pass_heads = (G + passes - 1) / passes;
     const bool use_mfma = mfma_decode_supported(d, c->k.w, c->v.w, pass_heads);
     WEED_HIP_REQUIRE(n_tokens == 1 || use_mfma,
-                     "%s: %u positions x %u heads per KV head (at most 16 rows), head_dim %u: not served by the chunk kernel",
-                     fn, n_tokens, real_heads / Hkv, d);
+                     "%s: head_dim %u with fields of %u and %u bits is not served by the matrix-core kernel, which a "
+                     "chunk of positions needs", fn, d, c->k.w, c->v.w);
     uint32_t n_splits, split_tokens = 0;
     uint32_t total_blocks = 0;
     RunGeom runs = { 1, 0, 8 };
@@ -892,7 +892,7 @@ extern "C" int weed_hip_kv_decode_attn_chunk(weed_hip_kv_cache *c, const int32_t
 {
     const char *fn = "weed_hip_kv_decode_attn_chunk";
     WEED_HIP_REQUIRE(q_stride && o_stride, "%s: null pointer", fn);
-    WEED_HIP_REQUIRE(n_tokens >= 1 && n_tokens <= 16, "%s: %d positions outside [1, 16]", fn, n_tokens);
+    WEED_HIP_REQUIRE(n_tokens >= 1 && n_tokens <= 64, "%s: %d positions outside [1, 64]", fn, n_tokens);
     if (c && !lens_dev) {
         for (int32_t l : c->lens) {
             WEED_HIP_REQUIRE(l >= n_tokens, "%s: a sequence holds %d tokens, fewer than the chunk's %d", fn, l, n_tokens);

@@ -469,7 +469,8 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     // tokens at the end of the region that this lane's (position, head) pair does not see (0 unless the call is a
     // multi-token chunk), and the largest such count over the pairs
     const uint32_t hidden_max = p.q_tokens - 1U;
-    const uint32_t hidden = (hidden_max && head_ok) ? hidden_max - (p.blocked ? hc % p.q_tokens : hc / p.real_group) : 0U;
+    const uint32_t pair = p.head_first + hc; // index of the (position, head) pair among those of the KV head
+    const uint32_t hidden = (hidden_max && head_ok) ? hidden_max - (p.blocked ? pair % p.q_tokens : pair / p.real_group) : 0U;
     const uint32_t qh_c = head_ok ? q_head_of(p, kvh, hc) : 0;
     const float qscale = head_ok ? p.q_scale[(uint64_t)seq * p.Hq + qh_c] : 0.0f;
     const float betaq = head_ok ? p.k.beta * p.q_sum[(uint64_t)seq * p.Hq + qh_c] : 0.0f;

@@ -1295,10 +1295,10 @@ TensorPtr MultiHeadAttention::forward_quantized(TensorPtr Q, TensorPtr K, Tensor
     }
     HipDevice::check(weed_hip_sync()); // earlier launches may still read the previous call's lengths
     HipDevice::check(weed_hip_memcpy_h2d(lens_dev, lens.data(), need));
-    // The (position, head) pairs of a KV head are the rows of one tile of the fused kernel (16 at most), so a few
-    // positions go through the cache together: position t0 + i of a group attends to before + t0 + i + 1 tokens, which
-    // is "the group's last length minus the positions after it".
-    const tcapint per_call = positions_per_pass();
+    // The (position, head) pairs of a KV head are the rows of the fused kernel's tiles: one call serves up to 64
+    // positions (a pass over the cache per tile of pairs), each masking the tokens after its own position.  Shapes
+    // without matrix-core instances go position by position through the generic kernel.
+    const tcapint per_call = matrix_core_shape() ? 64U : 1U;
     const uint32_t q_str4[4] = { Q->stride[0U], Q->stride[1U], Q->stride[2U], Q->stride[3U] };
     const uint32_t o_str4[4] = { out->stride[0U], out->stride[1U], out->stride[2U], out->stride[3U] };
     for (tcapint t = 0U; t < uT; t += per_call) {
@@ -1315,22 +1315,18 @@ TensorPtr MultiHeadAttention::forward_quantized(TensorPtr Q, TensorPtr K, Tensor
     return out;
 }
 
-// Query positions that one pass of the fused kernel serves: the (position, head) pairs of a KV head are the rows of
-// one matrix tile (16), which exists for head_dim 32 / 64 / 96 / 128 (256 with half the rows) and fields of 2..5 bits or 8 + 8; any other shape goes through the
-// generic kernel one position at a time.
-tcapint MultiHeadAttention::positions_per_pass() const
+// Whether the fused kernel's matrix-core instances serve this module's cache: head_dim up to 128 with fields of
+// 2..5 bits (any pair) or of equal width 1, 6, 7 or 8; above 128 with fields of up to 4 bits.  Other shapes go
+// through the generic kernel, one query position at a time.
+bool MultiHeadAttention::matrix_core_shape() const
 {
-    const tcapint G = num_heads / num_kv_heads;
     const int wk = (k_bits ? k_bits : kv_quant_bits) + ((kv_coder == KV_LLOYDMAX && k_sign) ? 1 : 0);
     const int wv = (v_bits ? v_bits : kv_quant_bits) + ((kv_coder == KV_LLOYDMAX && v_sign) ? 1 : 0);
+    const bool narrow = (wk >= 2 && wk <= 4 && wv >= 2 && wv <= 4) || (wk == 1 && wv == 1);
     if (head_dim > 128) {
-        // half the rows there: fields of 2..4 bits, at most 8 (position, head) pairs
-        const bool narrow = (wk >= 2 && wk <= 4 && wv >= 2 && wv <= 4) || (wk == 1 && wv == 1);
-        return (narrow && G <= 8U) ? std::max<tcapint>(1U, 8U / G) : 1U;
+        return narrow;
     }
-    const bool widths = (wk >= 2 && wk <= 5 && wv >= 2 && wv <= 5) || (wk == wv && (wk == 1 || (wk >= 6 && wk <= 8)));
-    const bool tiles = G <= 16U && (head_dim == 32U || head_dim == 64U || head_dim == 96U || head_dim == 128U) && widths;
-    return tiles ? std::max<tcapint>(1U, 16U / G) : 1U;
+    return narrow || (wk >= 2 && wk <= 5 && wv >= 2 && wv <= 5) || (wk == wv && wk >= 6 && wk <= 8);
 }
 
 // Rough device times of the two ways to serve T new tokens against L cached ones (measured on MI355X: a pass of the
@@ -1343,9 +1339,12 @@ bool MultiHeadAttention::dense_is_cheaper(tcapint B, tcapint T, tcapint L) const
     const double kb = (double)(k_bits ? k_bits : kv_quant_bits) + (k_sign ? 1.0 : 0.0);
     const double vb = (double)(v_bits ? v_bits : kv_quant_bits) + (v_sign ? 1.0 : 0.0);
     const double packed = (double)B * Hkv * (double)L * (hd * (kb + vb) / 8.0 + 8.0);
-    const double per_call = (double)positions_per_pass();
-    const double passes = std::ceil((double)T / per_call);
-    const double fused_us = passes * (55.0 + packed / 5.0e6);
+    // a pass serves one tile of (position, head) pairs: 16 rows, 8 above head_dim 128; the generic kernel takes one
+    // position per pass at about a tenth of the rate
+    const bool tiles = matrix_core_shape();
+    const double tile_rows = head_dim > 128 ? 8.0 : 16.0;
+    const double passes = tiles ? std::ceil((double)T * (Hq / Hkv) / tile_rows) : (double)T;
+    const double fused_us = passes * (55.0 + packed / (tiles ? 5.0e6 : 0.5e6));
     const double deq_bytes = (double)B * Hkv * (double)L * hd * 4.0 * 2.0;
     const double flops = 2.0 * 2.0 * (double)B * Hq * (double)T * (double)L * hd;
     const double score_bytes = (double)B * Hq * (double)T * (double)L * 4.0 * 7.0;

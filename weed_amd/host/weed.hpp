@@ -419,7 +419,7 @@ struct MultiHeadAttention : public Module {
     // PREFILL_AUTO's rule for B sequences, T new tokens and L cached ones (the new ones included): true when
     // dequantising once and attending densely is estimated cheaper than the passes of the fused kernel
     bool dense_is_cheaper(tcapint B, tcapint T, tcapint L) const;
-    tcapint positions_per_pass() const; // query positions that one pass of the fused kernel serves for this module
+    bool matrix_core_shape() const; // whether the fused kernel's matrix-core instances serve this module's cache
 
 private:
     TensorPtr forward_quantized(TensorPtr Q, TensorPtr K, TensorPtr V, symint B, symint T);
