@@ -466,3 +466,60 @@ def test_chunk_of_query_positions(gpu, oracle, lloyd, d, Hkv, Hq, T, gqa_weed):
     with pytest.raises(gpu.WeedHipError):
         cache.decode_attn_chunk(too_many, torch.zeros_like(too_many), gqa_mapping=gqa)
     cache.close()
+
+
+def test_random_shapes_chunk_equals_single_positions(gpu):
+    """Sixty seeded random shapes -- head_dim, coder, field widths, group size (also beyond a tile), chunk length,
+    ragged lengths, GQA mapping: a chunk call must give what the single-position calls give (which the other tests
+    check against the CPU checker), so every instance family is exercised with every way the work is cut."""
+    import torch
+    rng = np.random.default_rng(2024)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(7)
+
+    def randn(*shape):
+        return torch.randn(shape, generator=gen, device="cuda")
+
+    for case in range(60):
+        d = int(rng.choice([32, 64, 96, 128, 160, 192, 224, 256]))
+        lloyd = bool(rng.integers(2))
+        if d > 128:
+            wk, wv = int(rng.integers(2, 5)), int(rng.integers(2, 5))
+        elif rng.random() < 0.25:
+            wk = wv = int(rng.choice([1, 6, 7, 8]))
+            lloyd = lloyd and wk == 1
+        else:
+            wk, wv = int(rng.integers(2, 6)), int(rng.integers(2, 6))
+
+        def split(w):
+            if not lloyd:
+                return w, 0
+            if w == 5:
+                return 4, 1
+            if w == 1:
+                return 1, 0
+            return (w - 1, 1) if rng.random() < 0.5 else (w, 0)
+
+        (kb, ks), (vb, vs) = split(wk), split(wv)
+        Hkv = int(rng.integers(1, 4))
+        G = int(rng.choice([1, 2, 3, 4, 7, 8, 12, 16, 20]))
+        T, S = int(rng.integers(1, 10)), int(rng.integers(1, 5))
+        lens = [int(rng.integers(T, 400)) for _ in range(S)]
+        cache = gpu.KVCache(gpu.KV_LLOYDMAX if lloyd else gpu.KV_UNIFORM, S, Hkv, d, max(lens) + 8, kb, vb, ks, vs)
+        if not lloyd:
+            cache.set_scales(1.0, 0.9)
+        for s, L in enumerate(lens):
+            cache.encode_append(randn(1, Hkv, L, d), randn(1, Hkv, L, d), seq_begin=s)
+        q = randn(S, T, Hkv * G, d)
+        out, ref = torch.zeros_like(q), torch.zeros_like(q)
+        mapping = gpu.GQA_BLOCKED if rng.integers(2) else gpu.GQA_WEED
+        cache.decode_attn_chunk(q, out, gqa_mapping=mapping)
+        for t in range(T):
+            lt = torch.tensor([L - (T - 1 - t) for L in lens], dtype=torch.int32, device="cuda")
+            cache.decode_attn_prefix(lt, q[:, t], ref[:, t], gqa_mapping=mapping)
+        gpu.sync()
+        what = "case %d: d %d, K %d+%d V %d+%d bits, %d x %d heads, %d positions, lengths %s" % (
+            case, d, kb, ks, vb, vs, Hkv, G, T, lens)
+        assert not torch.isnan(out).any(), what
+        assert (out - ref).abs().max().item() < 5e-5, what
+        cache.close()
