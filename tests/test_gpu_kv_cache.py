@@ -421,3 +421,63 @@ def test_cfg5a_encode_full_size(gpu, oracle):
         np.testing.assert_array_equal(got_a, exported[which][1])
     assert cache.seq_lens() == [T]
     cache.close()
+
+
+def test_random_append_sequences_give_the_same_cache(gpu):
+    """Forty seeded random append histories (chunk sizes around the 32-token half blocks, subsets of the sequences,
+    every head_dim family, both coders, all widths): the cache must equal, bit for bit, the one that a one-token
+    append followed by one append of the rest builds (which never takes the encoder's direct path), and attend
+    identically -- so the largest row scale kept per region agrees too."""
+    import torch
+    rng = np.random.default_rng(99)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(3)
+    for case in range(40):
+        d = int(rng.choice([32, 64, 96, 128, 256]))
+        lloyd = bool(rng.integers(2))
+        if lloyd:
+            kb, vb, ks, vs = int(rng.integers(1, 5)), int(rng.integers(1, 5)), int(rng.integers(2)), int(rng.integers(2))
+        else:
+            kb, vb, ks, vs = int(rng.integers(1, 9)), int(rng.integers(1, 9)), 0, 0
+        S, Hkv, cap = int(rng.integers(1, 5)), int(rng.integers(1, 4)), 320
+        mode = gpu.KV_LLOYDMAX if lloyd else gpu.KV_UNIFORM
+        a = gpu.KVCache(mode, S, Hkv, d, cap, kb, vb, ks, vs)
+        b = gpu.KVCache(mode, S, Hkv, d, cap, kb, vb, ks, vs)
+        if not lloyd:
+            a.set_scales(1.1, 0.7)
+            b.set_scales(1.1, 0.7)
+        K = torch.randn((S, Hkv, cap, d), generator=gen, device="cuda") * 2
+        V = torch.randn((S, Hkv, cap, d), generator=gen, device="cuda")
+        lens = [0] * S
+        for _ in range(int(rng.integers(2, 8))):
+            s0 = int(rng.integers(0, S))
+            n = int(rng.integers(1, S - s0 + 1))
+            T = int(rng.choice([1, 2, 5, 17, 31, 32, 33, 64, 96]))
+            if max(lens[s0:s0 + n]) + T > cap:
+                continue
+            a.encode_append(torch.stack([K[s, :, lens[s]:lens[s] + T] for s in range(s0, s0 + n)]),
+                            torch.stack([V[s, :, lens[s]:lens[s] + T] for s in range(s0, s0 + n)]), seq_begin=s0)
+            for s in range(s0, s0 + n):
+                lens[s] += T
+        for s in range(S):
+            if lens[s] >= 1:
+                b.encode_append(K[s:s + 1, :, :1], V[s:s + 1, :, :1], seq_begin=s)
+            if lens[s] > 1:
+                b.encode_append(K[s:s + 1, :, 1:lens[s]], V[s:s + 1, :, 1:lens[s]], seq_begin=s)
+        what = "case %d: d %d, K %d+%d V %d+%d bits, lengths %s" % (case, d, kb, ks, vb, vs, lens)
+        assert a.seq_lens() == lens and b.seq_lens() == lens, what
+        if max(lens):
+            for which in (0, 1):
+                fa, sa = export(a, which, max(lens))
+                fb, sb = export(b, which, max(lens))
+                for s in range(S):
+                    assert np.array_equal(fa[s, :, :lens[s]], fb[s, :, :lens[s]]), what
+                    assert np.array_equal(sa[s, :, :lens[s]], sb[s, :, :lens[s]]), what
+            q = torch.randn((S, Hkv * 2, d), generator=gen, device="cuda")
+            oa, ob = torch.zeros_like(q), torch.zeros_like(q)
+            a.decode_attn(q, oa)
+            b.decode_attn(q, ob)
+            gpu.sync()
+            assert torch.equal(oa, ob), what
+        a.close()
+        b.close()
