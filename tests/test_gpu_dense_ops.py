@@ -480,3 +480,57 @@ def test_degenerate_shapes(gpu):
         out = dev(np.zeros((7, d), dtype=np.float32))
         gpu.apply_rotation(dev(x), col_major(r), out)
         np.testing.assert_allclose(out.cpu().numpy(), x.astype(np.float64) @ r.astype(np.float64), rtol=1e-5, atol=1e-5)
+
+
+def test_random_shapes_and_layouts(gpu):
+    """Seeded random shapes, each operand row-major, column-major or a strided slice of a larger tensor: products
+    (with and without the fused bias: every kernel the dispatcher can pick), softmax, the three reductions and layout
+    changing copies against float64 numpy."""
+    import torch
+    rng = np.random.default_rng(5)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(11)
+
+    def view(shape, kind):
+        if kind == 0:
+            return torch.randn(shape, generator=gen, device="cuda")
+        if kind == 1:
+            return torch.randn(shape[::-1], generator=gen, device="cuda").permute(*reversed(range(len(shape))))
+        big = torch.randn(tuple(2 * n + 1 for n in shape), generator=gen, device="cuda")
+        return big[tuple(slice(1, 1 + 2 * n, 2) for n in shape)]
+
+    def f64(t):
+        return t.cpu().numpy().astype(np.float64)
+
+    for _ in range(80):
+        M = int(rng.choice([1, 2, 7, 16, 17, 33, 64, 65, 100, 128, 200, 256, 300]))
+        N = int(rng.choice([1, 5, 16, 17, 48, 100, 128, 250, 512, 640, 1024]))
+        K = int(rng.choice([1, 3, 8, 16, 33, 64, 100, 256, 260, 512, 1030, 2048, 4096]))
+        a, b = view((M, K), int(rng.integers(3))), view((K, N), int(rng.integers(3)))
+        out = view((M, N), int(rng.integers(3)))
+        bias = torch.randn(N, generator=gen, device="cuda") if rng.integers(2) else None
+        gpu.linear(a, b, bias, out)
+        want = f64(a) @ f64(b) + (f64(bias) if bias is not None else 0.0)
+        np.testing.assert_allclose(f64(out), want, rtol=2e-5, atol=1.2e-5 * np.sqrt(K),
+                                   err_msg="%d x %d x %d, strides %s %s %s" % (M, K, N, a.stride(), b.stride(), out.stride()))
+    for _ in range(80):
+        rank = int(rng.integers(1, 5))
+        shape = tuple(int(rng.choice([1, 2, 3, 5, 16, 33, 64, 130, 300])) for _ in range(rank))
+        if np.prod(shape) > 2_000_000:
+            continue
+        axis = int(rng.integers(rank))
+        x, out = view(shape, int(rng.integers(3))), view(shape, int(rng.integers(3)))
+        what = "shape %s axis %d, strides %s -> %s" % (shape, axis, x.stride(), out.stride())
+        gpu.softmax(x, out, axis)
+        x64 = f64(x)
+        e = np.exp(x64 - x64.max(axis=axis, keepdims=True))
+        np.testing.assert_allclose(f64(out), e / e.sum(axis=axis, keepdims=True), rtol=3e-5, atol=1e-9, err_msg=what)
+        if rank > 1:
+            r = view(tuple(n for i, n in enumerate(shape) if i != axis), int(rng.integers(3)))
+            for op, fn in ((gpu.REDUCE_SUM, np.sum), (gpu.REDUCE_MAX, np.max), (gpu.REDUCE_MIN, np.min)):
+                gpu.reduce(op, x, r, axis)
+                np.testing.assert_allclose(f64(r), fn(x64, axis=axis), rtol=2e-5, atol=2e-5 * np.sqrt(shape[axis]),
+                                           err_msg=what)
+        y = view(shape, int(rng.integers(3)))
+        gpu.elementwise(gpu.EW_COPY, x, None, y)
+        assert torch.equal(x, y), what
