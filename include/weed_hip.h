@@ -269,6 +269,18 @@ int weed_hip_kv_decode_attn(weed_hip_kv_cache *cache, int32_t n_q_heads, int32_t
                             uint32_t q_off, const uint32_t q_stride[3], float *out_dev, uint32_t o_off,
                             const uint32_t o_stride[3], uint32_t flags);
 
+/* weed_hip_kv_decode_attn for callers that cannot allocate device memory (code under HIP graph capture, serving loops
+ * and harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments, same kernels and
+ * bit-identical results; the workspace (rotated queries, split partials) is a 32 MiB array that is part of the
+ * library's device image and that every device the library was initialised on holds until the process ends.  Calls
+ * no hipMalloc / hipFree and creates no events (the library's timing scopes skip it).  Shapes whose workspace
+ * n_seq * n_q_heads * (d * 8 + 8 + slots * (d + 2) * 4) bytes (slots: context splits, at most a few dozen) exceeds the
+ * array return WEED_HIP_EINVAL.  All calls on one device share the array: calls that overlap on one device (two host
+ * threads, two streams) race; weed_hip_init must have run on the device. */
+int weed_hip_kv_decode_attn_noalloc(weed_hip_kv_cache *cache, int32_t n_q_heads, int32_t gqa_mapping,
+                                    const float *q_dev, uint32_t q_off, const uint32_t q_stride[3], float *out_dev,
+                                    uint32_t o_off, const uint32_t o_stride[3], uint32_t flags);
+
 /* The same, attending only over the first lens_dev[s] tokens of sequence s (device array of n_seq lengths, each at
  * most the cached length).  This is how a causal mask with a cache offset is expressed for one query position at a
  * time: the reference adds a triangular mask to a dense score matrix instead (multihead_attention.cpp:322-328,

@@ -92,6 +92,8 @@ SIGNATURES = {
     "weed_hip_kv_append_weed_words": (c_int, [c_void_p, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
     "weed_hip_kv_decode_attn": (c_int, [c_void_p, c_int32, c_int32, c_void_p, c_uint32, U32P, c_void_p, c_uint32, U32P,
                                         c_uint32]),
+    "weed_hip_kv_decode_attn_noalloc": (c_int, [c_void_p, c_int32, c_int32, c_void_p, c_uint32, U32P, c_void_p, c_uint32,
+                                                U32P, c_uint32]),
     "weed_hip_kv_decode_attn_prefix": (c_int, [c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_uint32, U32P, c_void_p,
                                                c_uint32, U32P, c_uint32]),
     "weed_hip_kv_decode_attn_chunk": (c_int, [c_void_p, c_void_p, c_int32, c_int32, c_int32, c_void_p, c_uint32, U32P,
@@ -226,6 +228,14 @@ class KVCache:
         qp, qo, qs = _geom(q)
         op, oo, os_ = _geom(out)
         check(self.lib.weed_hip_kv_decode_attn(self.handle, q.shape[1], gqa_mapping, qp, qo, qs, op, oo, os_, flags))
+
+    def decode_attn_noalloc(self, q, out, gqa_mapping=GQA_WEED, flags=0):
+        """decode_attn on the library's static workspace: allocates nothing, refuses shapes beyond 32 MiB of it."""
+        assert q.dim() == 3 and q.shape == out.shape
+        qp, qo, qs = _geom(q)
+        op, oo, os_ = _geom(out)
+        check(self.lib.weed_hip_kv_decode_attn_noalloc(self.handle, q.shape[1], gqa_mapping, qp, qo, qs, op, oo, os_,
+                                                       flags))
 
     def decode_attn_prefix(self, lens, q, out, gqa_mapping=GQA_WEED, flags=0):
         """As decode_attn, over the first lens[s] cached tokens only (lens: int32 torch tensor on the device)."""

@@ -22,9 +22,16 @@ hipStream_t stream();
 // Ensures weed_hip_init() ran (device 0 by default).  Returns a WEED_HIP_* status.
 int ensure_init();
 
+// Device weed_hip_init() selected last (-1 before the first call).
+int current_device();
+
+// Looks up this device's copy of the decode entry point's static scratch array (kv_decode.hip); weed_hip_init calls
+// it once per device with that device current.
+int decode_scratch_setup(int device_id);
+
 // RAII timing scope: when profiling is on, records events around the enclosed launches.
 struct ProfileScope {
-    explicit ProfileScope(const char *name);
+    explicit ProfileScope(const char *name, bool enabled = true);
     ~ProfileScope();
     ProfileScope(const ProfileScope &) = delete;
     ProfileScope &operator=(const ProfileScope &) = delete;

@@ -104,6 +104,8 @@ int fail(int code, const char *fmt, ...)
 
 hipStream_t stream() { return g_stream; }
 
+int current_device() { return g_initialised ? g_device : -1; }
+
 int ensure_init()
 {
     if (g_initialised) {
@@ -112,10 +114,10 @@ int ensure_init()
     return weed_hip_init(0);
 }
 
-ProfileScope::ProfileScope(const char *name)
+ProfileScope::ProfileScope(const char *name, bool enabled)
     : name_(name)
 {
-    if (!g_profile) {
+    if (!g_profile || !enabled) {
         return;
     }
     if (hipEventCreate(&start_) != hipSuccess || hipEventCreate(&stop_) != hipSuccess) {
@@ -158,6 +160,7 @@ int weed_hip_init(int device_id)
         return fail(WEED_HIP_EINVAL, "weed_hip_init: device %d out of range [0, %d)", device_id, count);
     }
     WEED_HIP_CHECK(hipSetDevice(device_id));
+    WEED_HIP_TRY(decode_scratch_setup(device_id));
     if (g_initialised && g_device == device_id) {
         return WEED_HIP_OK;
     }

@@ -18,6 +18,33 @@
 using namespace weedhip;
 using namespace weedkv;
 
+// Workspace of weed_hip_kv_decode_attn_noalloc: rotated queries, their fp16 halves, block offsets and the split
+// partials of one call.  Every device the library runs on holds its own copy until the process ends; in host code the
+// array's name is only a handle for hipGetSymbolAddress, the kernels get the address kept in g_scratch_dev.
+constexpr size_t kStaticScratchBytes = 32u << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+void *g_scratch_dev[kMaxDevices] = {};
+} // namespace
+
+namespace weedhip {
+// Called by weed_hip_init with `device_id` current: looks the device's copy of `scratch` up once.
+int decode_scratch_setup(int device_id)
+{
+    if (device_id < 0 || device_id >= kMaxDevices) {
+        return fail(WEED_HIP_EINVAL, "decode_scratch_setup: device %d outside [0, %d)", device_id, kMaxDevices);
+    }
+    if (!g_scratch_dev[device_id]) {
+        void *ptr = nullptr;
+        WEED_HIP_CHECK(hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)));
+        g_scratch_dev[device_id] = ptr;
+    }
+    return WEED_HIP_OK;
+}
+} // namespace weedhip
+
 namespace {
 
 constexpr int kGMax = 8;        // query heads of one kv head handled per pass
@@ -684,7 +711,7 @@ __global__ void __launch_bounds__(256) combine_rows_kernel(const float *__restri
 int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t gqa_mapping, const float *q_dev,
                 uint32_t q_off, const uint32_t q_stride[3], float *out_dev, uint32_t o_off, const uint32_t o_stride[3],
                 uint32_t flags, const int32_t *lens_dev, uint32_t n_tokens = 1, uint32_t q_tstride = 0,
-                uint32_t o_tstride = 0)
+                uint32_t o_tstride = 0, uint8_t *fixed_ws = nullptr, size_t fixed_ws_bytes = 0)
 {
     WEED_HIP_REQUIRE(c, "%s: null cache", fn);
     WEED_HIP_REQUIRE(q_dev && out_dev && q_stride && o_stride, "%s: null pointer", fn);
@@ -765,7 +792,12 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
     const size_t part_bytes = sizeof(float) * (size_t)S * Hq * n_splits * (d + 2);
     const size_t off_bytes = (sizeof(uint32_t) * ((size_t)S + 1) + 15) / 16 * 16;
     const size_t need = q_bytes + 2 * h_bytes + 2 * s_bytes + off_bytes + part_bytes;
-    if (need > c->dec_ws_bytes) {
+    if (fixed_ws) {
+        // the caller's workspace (the static scratch): nothing is allocated, larger shapes are refused
+        WEED_HIP_REQUIRE(need <= fixed_ws_bytes,
+                         "%s: this shape needs %zu bytes of workspace, the static scratch holds %zu (use "
+                         "weed_hip_kv_decode_attn)", fn, need, fixed_ws_bytes);
+    } else if (need > c->dec_ws_bytes) {
         WEED_HIP_CHECK(hipStreamSynchronize(stream()));
         (void)hipFree(c->dec_ws);
         c->dec_ws = nullptr;
@@ -775,7 +807,8 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         }
         c->dec_ws_bytes = need;
     }
-    uint8_t *wsp = reinterpret_cast<uint8_t *>(c->dec_ws);
+    uint8_t *wsp = fixed_ws ? fixed_ws : reinterpret_cast<uint8_t *>(c->dec_ws);
+    const bool timed = !fixed_ws; // the timing scopes create events, which the allocation-free entry point must not
     float *q_rot = reinterpret_cast<float *>(wsp);
     uint16_t *q_hi = reinterpret_cast<uint16_t *>(wsp + q_bytes);
     uint16_t *q_lo = reinterpret_cast<uint16_t *>(wsp + q_bytes + h_bytes);
@@ -824,7 +857,7 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         mp.max_slots = n_splits;
         mp.group_total = G;
         mp.tile_rows = pass_heads;
-        ProfileScope prof("kv_decode_attn");
+        ProfileScope prof("kv_decode_attn", timed);
         for (uint32_t first = 0; total_blocks && first < G; first += pass_heads) {
             mp.head_first = first;
             mp.G = std::min(pass_heads, G - first);
@@ -845,12 +878,12 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         p.partials = partials;
         p.n_splits = n_splits;
         p.split_tokens = split_tokens;
-        ProfileScope prof("kv_decode_attn");
+        ProfileScope prof("kv_decode_attn", timed);
         decode_generic_kernel<<<dim3(n_splits, Hkv, S), kThreads, 0, stream()>>>(p);
         WEED_HIP_LAUNCH_CHECK();
     }
     {
-        ProfileScope prof("kv_decode_combine");
+        ProfileScope prof("kv_decode_combine", timed);
         const SlotGeom sg = { use_mfma ? blk_off : nullptr, Hkv, G, runs,
                               gqa_mapping == WEED_HIP_GQA_BLOCKED ? 1 : 0 };
         if (many_rows && n_splits <= 64) {
@@ -873,6 +906,19 @@ extern "C" int weed_hip_kv_decode_attn(weed_hip_kv_cache *c, int32_t n_q_heads, 
 {
     return decode_impl("weed_hip_kv_decode_attn", c, n_q_heads, gqa_mapping, q_dev, q_off, q_stride, out_dev, o_off,
                        o_stride, flags, nullptr);
+}
+
+extern "C" int weed_hip_kv_decode_attn_noalloc(weed_hip_kv_cache *c, int32_t n_q_heads, int32_t gqa_mapping,
+                                               const float *q_dev, uint32_t q_off, const uint32_t q_stride[3],
+                                               float *out_dev, uint32_t o_off, const uint32_t o_stride[3],
+                                               uint32_t flags)
+{
+    const char *fn = "weed_hip_kv_decode_attn_noalloc";
+    const int dev = current_device();
+    WEED_HIP_REQUIRE(dev >= 0 && dev < kMaxDevices && g_scratch_dev[dev],
+                     "%s: weed_hip_init has not run on the current device", fn);
+    return decode_impl(fn, c, n_q_heads, gqa_mapping, q_dev, q_off, q_stride, out_dev, o_off, o_stride, flags, nullptr,
+                       1, 0, 0, static_cast<uint8_t *>(g_scratch_dev[dev]), kStaticScratchBytes);
 }
 
 extern "C" int weed_hip_kv_decode_attn_prefix(weed_hip_kv_cache *c, const int32_t *lens_dev, int32_t n_q_heads,
