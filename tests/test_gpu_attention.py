@@ -190,7 +190,7 @@ def test_one_long_region_keeps_within_the_slot_limit(gpu, oracle):
     cache.close()
 
 
-def test_run_geometry_knobs_do_not_change_the_answer(gpu, oracle, monkeypatch):
+def test_run_geometry_knobs_do_not_change_the_answer(gpu, oracle):
     """The launch cuts the block list into per-wavefront runs whose lengths are skewed by wavefront age; whatever
     the skew and the number of runs, every block must be attended exactly once: ragged batch (runs straddle regions,
     empty sequence in the middle) against the checker under several settings of the two tuning variables."""
@@ -204,12 +204,35 @@ def test_run_geometry_knobs_do_not_change_the_answer(gpu, oracle, monkeypatch):
     q = rng.standard_normal((S, Hq, d), dtype=np.float32)
     cache = build_cache(gpu, wl, gpu.KV_LLOYDMAX, K, V)
     want = checker_output(oracle, gpu, cache, wl, q, False)
-    for waves, skew in (("", ""), ("16", "0"), ("16", "45"), ("7", "90"), ("40", "30"), ("100000", "16")):
-        if waves:
-            monkeypatch.setenv("WEED_HIP_DECODE_WAVES", waves)
-            monkeypatch.setenv("WEED_HIP_DECODE_SKEW", skew)
-        got = run_decode(gpu, cache, q, gpu.GQA_BLOCKED, 0)
-        assert_attn_close(got, want, "waves=%s skew=%s" % (waves or "default", skew or "default"))
+    try:
+        for waves, skew in ((0, -1), (16, 0), (16, 45), (7, 90), (40, 30), (100000, 16)):
+            gpu.decode_tuning(waves, skew)
+            got = run_decode(gpu, cache, q, gpu.GQA_BLOCKED, 0)
+            assert_attn_close(got, want, "waves=%d skew=%d" % (waves, skew))
+    finally:
+        gpu.decode_tuning()
+    cache.close()
+
+
+def test_equal_contexts_with_and_without_the_region_search(gpu, oracle):
+    """A batch of equal contexts finds each wavefront's first region by division; the search used for ragged batches
+    must give the same bits."""
+    rng = np.random.default_rng(31)
+    d, Hkv, Hq, S, L = 128, 2, 8, 5, 1500
+    wl = workloads.Workload("equal", S, Hq, Hkv, d, [L] * S, 3, 4, 0, 0, 0)
+    K = rng.standard_normal((S, Hkv, L, d), dtype=np.float32)
+    V = rng.standard_normal((S, Hkv, L, d), dtype=np.float32)
+    q = rng.standard_normal((S, Hq, d), dtype=np.float32)
+    cache = build_cache(gpu, wl, gpu.KV_LLOYDMAX, K, V)
+    want = checker_output(oracle, gpu, cache, wl, q, False)
+    try:
+        fast = run_decode(gpu, cache, q, gpu.GQA_BLOCKED, 0)
+        gpu.decode_tuning(always_search=True)
+        searched = run_decode(gpu, cache, q, gpu.GQA_BLOCKED, 0)
+    finally:
+        gpu.decode_tuning()
+    assert_attn_close(fast, want, "equal contexts")
+    assert np.array_equal(fast, searched)
     cache.close()
 
 

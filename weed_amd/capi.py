@@ -92,6 +92,7 @@ SIGNATURES = {
     "weed_hip_kv_append_weed_words": (c_int, [c_void_p, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
     "weed_hip_kv_decode_attn": (c_int, [c_void_p, c_int32, c_int32, c_void_p, c_uint32, U32P, c_void_p, c_uint32, U32P,
                                         c_uint32]),
+    "weed_hip_kv_decode_tuning": (c_int, [c_int32, c_int32, c_int32]),
     "weed_hip_kv_decode_attn_noalloc": (c_int, [c_void_p, c_int32, c_int32, c_void_p, c_uint32, U32P, c_void_p, c_uint32,
                                                 U32P, c_uint32]),
     "weed_hip_kv_decode_attn_prefix": (c_int, [c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_uint32, U32P, c_void_p,
@@ -372,6 +373,11 @@ def block_scale(x, sequential=False):
     check(load().weed_hip_block_scale_f32(c_void_p(x.data_ptr()), 0, u32(x.shape), u32(x.stride()), int(sequential),
                                           byref(out)))
     return out.value
+
+
+def decode_tuning(wavefronts=0, skew_percent=-1, always_search=False):
+    """Work partition of the decode kernels (defaults: 0, -1, False); results do not depend on it."""
+    check(load().weed_hip_kv_decode_tuning(int(wavefronts), int(skew_percent), int(always_search)))
 
 
 def profile_enable(on):

@@ -54,9 +54,14 @@ struct weed_hip_kv_cache {
     // scratch for decode: rotated queries and split partials
     float *dec_ws = nullptr;
     size_t dec_ws_bytes = 0;
+    // LDS image of both sides' lookup tables for the matrix-core decode kernel (kMfmaTableImageBytes), rebuilt
+    // whenever the tables change
+    uint32_t *table_image = nullptr;
 };
 
 namespace weedhip {
 // Builds the kernel-side view of one tensor of the cache.
 SideParams side_params(const weed_hip_kv_cache *c, int which);
+// (Re)builds c->table_image from the current tables; a blocking copy, done when a cache is created or its tables set.
+int upload_table_image(weed_hip_kv_cache *c);
 } // namespace weedhip

@@ -4,6 +4,7 @@
 // MultiHeadAttention::forward (cpp:206-257).  Compiled with -ffp-contract=off: every multiply-add that must round
 // twice (as the reference's x86-64 build does) is written as separate operations, every fused one as fmaf().
 #include "kv_cache.h"
+#include "kv_decode_mfma.h"
 
 #include <algorithm>
 #include <cmath>
@@ -967,6 +968,29 @@ SideParams side_params(const weed_hip_kv_cache *c, int which)
     return sp;
 }
 
+int upload_table_image(weed_hip_kv_cache *c)
+{
+    const SideParams k = side_params(c, 0), v = side_params(c, 1);
+    uint16_t kl[32], vl[32];
+    for (int i = 0; i < 32; ++i) {
+        // the levels are exactly representable in binary16 (set_tables rounds them; the uniform coder's are code + 0.5)
+        kl[i] = __builtin_bit_cast(uint16_t, (_Float16)k.table[i]);
+        vl[i] = __builtin_bit_cast(uint16_t, (_Float16)v.table[i]);
+    }
+    const uint32_t words = mfma_table_rows(k.w, v.w) * (kMfmaTableRowBytes / 4);
+    if (!words) {
+        return WEED_HIP_OK;
+    }
+    std::vector<uint32_t> img(words);
+    for (uint32_t i = 0; i < words; ++i) {
+        img[i] = mfma_table_word(i, k.w, v.w, kl, vl);
+    }
+    // kernels already enqueued may still read the old image
+    WEED_HIP_CHECK(hipStreamSynchronize(stream()));
+    WEED_HIP_CHECK(hipMemcpy(c->table_image, img.data(), sizeof(uint32_t) * words, hipMemcpyHostToDevice));
+    return WEED_HIP_OK;
+}
+
 } // namespace weedhip
 
 extern "C" {
@@ -1040,6 +1064,15 @@ int weed_hip_kv_cache_create(weed_hip_kv_cache **cache, const weed_hip_kv_config
         weed_hip_kv_cache_destroy(c);
         return fail(WEED_HIP_ENOMEM, "weed_hip_kv_cache_create: device allocation failed: %s", hipGetErrorString(e));
     }
+    if (hipMalloc((void **)&c->table_image, kMfmaTableImageBytes) != hipSuccess) {
+        weed_hip_kv_cache_destroy(c);
+        return fail(WEED_HIP_ENOMEM, "weed_hip_kv_cache_create: device allocation failed");
+    }
+    const int st = upload_table_image(c);
+    if (st != WEED_HIP_OK) {
+        weed_hip_kv_cache_destroy(c);
+        return st;
+    }
     *cache = c;
     return WEED_HIP_OK;
 }
@@ -1056,6 +1089,7 @@ int weed_hip_kv_cache_destroy(weed_hip_kv_cache *c)
     (void)hipFree(c->enc_fields);
     (void)hipFree(c->enc_alpha);
     (void)hipFree(c->dec_ws);
+    (void)hipFree(c->table_image);
     delete c;
     return WEED_HIP_OK;
 }
@@ -1165,7 +1199,7 @@ int weed_hip_kv_cache_set_tables(weed_hip_kv_cache *c, int which, const float *b
             recon_rounded[i] = s.recon[i];
         }
     }
-    return WEED_HIP_OK;
+    return upload_table_image(c);
 }
 
 int weed_hip_kv_cache_get_tables(const weed_hip_kv_cache *c, int which, float *bounds, float *levels, float *recon)

@@ -463,6 +463,33 @@ constexpr uint32_t kMaxSlots = 1024; // partials per (sequence, head) that combi
 // Run-length skew between the wavefront age classes of a workgroup, in percent of the mean run (see RunGeom).
 constexpr uint32_t kRunSkewPercent = 16;
 
+// Tuning knobs of the work partition.  The defaults come from the environment, read ONCE per process (at the first
+// decode call or the first weed_hip_kv_decode_tuning): WEED_HIP_DECODE_WAVES (wavefronts the block list is cut for),
+// WEED_HIP_DECODE_SKEW (percent), WEED_HIP_DECODE_SEARCH=1 (always find a wavefront's first region by search, even in
+// a batch of equal contexts).
+struct DecodeTuning {
+    int wavefronts = 0;    // 0: as many as the device holds at once
+    int skew_percent = -1; // < 0: kRunSkewPercent
+    bool always_search = false;
+};
+DecodeTuning &decode_tuning()
+{
+    static DecodeTuning t = [] {
+        DecodeTuning v;
+        if (const char *env = std::getenv("WEED_HIP_DECODE_WAVES")) {
+            v.wavefronts = std::max(0, std::atoi(env));
+        }
+        if (const char *env = std::getenv("WEED_HIP_DECODE_SKEW")) {
+            v.skew_percent = std::atoi(env);
+        }
+        if (const char *env = std::getenv("WEED_HIP_DECODE_SEARCH")) {
+            v.always_search = std::atoi(env) != 0;
+        }
+        return v;
+    }();
+    return t;
+}
+
 struct SlotGeom {
     const uint32_t *blk_off; // null: every (sequence, head) has `max_slots` valid partials
     uint32_t Hkv, G;
@@ -753,15 +780,11 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         WEED_HIP_REQUIRE(blocks < (1ull << 32), "%s: too many cached tokens for one launch", fn);
         total_blocks = (uint32_t)blocks;
         runs.waves = mfma_decode_workgroup_waves(pass_heads, d, c->k.w, c->v.w);
-        uint32_t target_units = runs.waves * 256u; // one workgroup per compute unit
-        if (const char *env = std::getenv("WEED_HIP_DECODE_WAVES")) {
-            target_units = (uint32_t)std::max(1, std::atoi(env)); // tuning knob
-        }
+        const DecodeTuning &tune = decode_tuning();
+        // one workgroup per compute unit
+        const uint32_t target_units = tune.wavefronts > 0 ? (uint32_t)tune.wavefronts : runs.waves * 256u;
         runs.unit_blocks = std::max(1u, (total_blocks + target_units - 1) / target_units);
-        uint32_t skew_pct = kRunSkewPercent;
-        if (const char *env = std::getenv("WEED_HIP_DECODE_SKEW")) {
-            skew_pct = (uint32_t)std::min(90, std::max(0, std::atoi(env))); // tuning knob
-        }
+        const uint32_t skew_pct = tune.skew_percent >= 0 ? (uint32_t)std::min(90, tune.skew_percent) : kRunSkewPercent;
         const uint32_t nblk = (max_len + 63) / 64;
         for (;;) {
             runs.skew = std::min(runs.unit_blocks - 1, (runs.unit_blocks * skew_pct + 50) / 100);
@@ -835,8 +858,10 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
 
     if (use_mfma) {
         MfmaParams mp;
-        mp.k = side_params(c, 0);
-        mp.v = side_params(c, 1);
+        const SideParams ks = side_params(c, 0), vs = side_params(c, 1);
+        mp.k = MfmaSide{ ks.fields, ks.alpha, ks.region_bytes, ks.alpha_max, ks.alpha_const, ks.beta, ks.w };
+        mp.v = MfmaSide{ vs.fields, vs.alpha, vs.region_bytes, vs.alpha_max, vs.alpha_const, vs.beta, vs.w };
+        mp.table_image = c->table_image;
         mp.lens = lens_dev ? lens_dev : c->lens_dev;
         mp.padded = c->padded_tokens;
         mp.Hq = Hq;
@@ -853,6 +878,13 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         mp.blk_off = blk_off;
         mp.n_seq = S;
         mp.total_blocks = total_blocks;
+        mp.uniform_blocks = ((uint32_t)c->lens[0] + 63u) >> 6;
+        for (int32_t l : c->lens) {
+            if ((((uint32_t)l + 63u) >> 6) != mp.uniform_blocks || decode_tuning().always_search) {
+                mp.uniform_blocks = 0;
+                break;
+            }
+        }
         mp.runs = runs;
         mp.max_slots = n_splits;
         mp.group_total = G;
@@ -906,6 +938,15 @@ extern "C" int weed_hip_kv_decode_attn(weed_hip_kv_cache *c, int32_t n_q_heads, 
 {
     return decode_impl("weed_hip_kv_decode_attn", c, n_q_heads, gqa_mapping, q_dev, q_off, q_stride, out_dev, o_off,
                        o_stride, flags, nullptr);
+}
+
+extern "C" int weed_hip_kv_decode_tuning(int32_t wavefronts, int32_t skew_percent, int32_t always_search)
+{
+    DecodeTuning &t = decode_tuning();
+    t.wavefronts = std::max(0, wavefronts);
+    t.skew_percent = skew_percent;
+    t.always_search = always_search != 0;
+    return WEED_HIP_OK;
 }
 
 extern "C" int weed_hip_kv_decode_attn_noalloc(weed_hip_kv_cache *c, int32_t n_q_heads, int32_t gqa_mapping,

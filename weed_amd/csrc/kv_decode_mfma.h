@@ -60,11 +60,63 @@ __host__ __device__ inline uint32_t run_of_block(const RunGeom &rg, uint32_t b)
     return wg * rg.waves + group * classes + t;
 }
 
+// What the matrix-core kernel needs of one tensor of the cache (the reconstruction levels travel in the table image).
+struct MfmaSide {
+    const uint8_t *fields;     // packed items, one region per (sequence, kv head)
+    const float *alpha;        // [n_seq][n_kv_heads][padded_tokens] row scales, LLOYDMAX only
+    uint64_t region_bytes;
+    const uint32_t *alpha_max; // [n_seq][n_kv_heads] bit pattern of the largest row scale seen, LLOYDMAX only
+    float alpha_const;         // UNIFORM: step
+    float beta;                // UNIFORM: lo
+    uint32_t w;                // field width
+};
+
+// Rows of one side's lookup table in LDS (256 bytes each): pair tables (2^(2w) entries) for fields of up to 4 bits;
+// a table of the 32 single values for 5-bit fields; none for 6 to 8 bits, which are turned into numbers arithmetically.
+constexpr uint32_t mfma_side_rows(uint32_t w) { return w >= 6 ? 0u : (w == 5 ? 32u : 1u << (2 * w)); }
+constexpr uint32_t mfma_table_rows(uint32_t wk, uint32_t wv)
+{
+    return mfma_side_rows(wk) > mfma_side_rows(wv) ? mfma_side_rows(wk) : mfma_side_rows(wv);
+}
+constexpr uint32_t kMfmaTableRowBytes = 256;
+constexpr uint32_t kMfmaTableImageBytes = 256 * kMfmaTableRowBytes; // the largest image (4-bit pair tables)
+// Word i of the image a workgroup copies into LDS before its first block: entry e = i / 64 of the V table in the
+// first 32 words of row e (one replica per bank), of the K table in the last 32.  `k_levels` / `v_levels`: the fp16 bit
+// patterns of the 2^w reconstruction levels of each side.
+inline uint32_t mfma_table_word(uint32_t i, uint32_t wk, uint32_t wv, const uint16_t *k_levels, const uint16_t *v_levels)
+{
+    const uint32_t e = i >> 6, k_half = (i >> 5) & 1;
+    const uint32_t w = k_half ? wk : wv;
+    const uint16_t *lv = k_half ? k_levels : v_levels;
+    if (w >= 6) {
+        return 0;
+    }
+    if (w == 5) {
+        // the 32 single values, in both halves of the word
+        return e < 32u ? ((uint32_t)lv[e] | ((uint32_t)lv[e] << 16)) : 0u;
+    }
+    const uint32_t mask = (1u << w) - 1u;
+    return e < (1u << (2 * w)) ? ((uint32_t)lv[e & mask] | ((uint32_t)lv[(e >> w) & mask] << 16)) : 0u;
+}
+
+// Kernel arguments.  What a wavefront needs before it can request its first block comes first, so that it arrives
+// with the first kernel-argument fetches.
 struct MfmaParams {
-    SideParams k, v;
-    const int32_t *lens;
+    // Work partition: the 64-token blocks of all (sequence, kv head) regions form one list, region after region
+    // (sequence-major), cut into one run per wavefront (`runs`).
+    RunGeom runs;
+    uint32_t total_blocks;   // blk_off[n_seq] * Hkv
+    // Blocks per sequence when every sequence spans the same number (the common batch of equal contexts), else 0:
+    // a wavefront then finds its region by division instead of searching blk_off, and requests its first block
+    // without waiting for any other load.
+    uint32_t uniform_blocks;
+    uint32_t Hkv, n_seq;
     uint32_t padded;
-    uint32_t Hq, Hkv, G;
+    MfmaSide k, v;
+    const uint32_t *table_image; // mfma_table_rows(k.w, v.w) * 64 words, see mfma_table_word
+    const uint32_t *blk_off; // [n_seq + 1] prefix sums of the sequences' block counts (cached lengths)
+    const int32_t *lens;
+    uint32_t Hq, G;
     int blocked;            // 1: kv = h / G, 0: kv = h % Hkv (Weed)
     // multi-token chunks: the G "heads" of a KV head are (position, head) pairs, q_tokens positions x real_group
     // heads; pair hc stands for position hc % q_tokens (blocked) or hc / real_group (Weed mapping), and position t
@@ -73,18 +125,12 @@ struct MfmaParams {
     // groups larger than a tile has rows go through the cache in several launches: this one serves the heads
     // [head_first, head_first + G) of the group_total that share a KV head; tile_rows (0: G) picks the kernel instance
     uint32_t head_first, group_total, tile_rows;
+    uint32_t max_slots;      // partial slots per (sequence, head): most wavefronts that can touch one region
     const uint16_t *q_hi;   // [n_seq][Hq][d] fp16 bits: high half of the scaled, normalised query
     const uint16_t *q_lo;   // [n_seq][Hq][d] fp16 bits: what the high half misses
     const float *q_scale;   // [n_seq][Hq] power of two the query was divided by
     const float *q_sum;     // [n_seq][Hq] sum of the scaled query (for the uniform coder's offset term)
     float *partials;        // [n_seq][Hq][max_slots][d + 2]: m (log2 units), l, o[d]
-    // Work partition: the 64-token blocks of all (sequence, kv head) regions form one list, region after region
-    // (sequence-major), cut into one run per wavefront (`runs`).
-    const uint32_t *blk_off; // [n_seq + 1] prefix sums of the sequences' block counts (cached lengths)
-    uint32_t n_seq;
-    uint32_t total_blocks;   // blk_off[n_seq] * Hkv
-    RunGeom runs;
-    uint32_t max_slots;      // partial slots per (sequence, head): most wavefronts that can touch one region
 };
 
 bool mfma_decode_supported(uint32_t d, uint32_t wk, uint32_t wv, uint32_t G);

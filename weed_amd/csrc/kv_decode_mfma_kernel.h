@@ -67,16 +67,8 @@ template <int N> __device__ __forceinline__ void load_dwords(const uint8_t *base
 //      a lookup is  (entry << 8) | lane byte,  lane byte = (lane % 32) * 4 (+ 128 for K): the entry index lands in
 //      byte 1 of the address.  When a pair is a whole byte of the packed run (4-bit fields), ONE byte-permute builds
 //      the address from the run's dword and the lane byte; otherwise a bit-field extract and a shift-add do. ----
-constexpr uint32_t kTableRowBytes = 256;
-// Rows of one side's table: pair tables (2^(2W) entries) for fields of up to 4 bits; 5-bit fields (4-bit codes with
-// the residual sign) would need 1024 pairs, so they use a table of the 32 single values, each stored twice (both
-// halves of the word), and a pair is assembled from two lookups; fields of 6 to 8 bits (uniform coder only) are
-// turned into fp16 values arithmetically and need no table.
-template <int W> constexpr uint32_t side_rows() { return W >= 6 ? 0u : (W == 5 ? 32u : 1u << (2 * W)); }
-template <int WK, int WV> constexpr uint32_t table_rows()
-{
-    return side_rows<WK>() > side_rows<WV>() ? side_rows<WK>() : side_rows<WV>();
-}
+constexpr uint32_t kTableRowBytes = kMfmaTableRowBytes;
+template <int WK, int WV> constexpr uint32_t table_rows() { return mfma_table_rows(WK, WV); }
 
 template <int W, int N, int P> __device__ __forceinline__ uint32_t pair_addr(const uint32_t (&x)[N], uint32_t lane_byte)
 {
@@ -288,55 +280,37 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     constexpr int NSETS = 4 / TPS;   // register sets per 64-token block
     constexpr uint32_t ROWS = table_rows<WK, WV>();
 
-    extern __shared__ uint32_t lds[]; // the tables, then 64 staged fp16 levels
+    extern __shared__ uint32_t lds[]; // the lookup tables
 
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t c = lane & 15, g = lane >> 4;
     constexpr bool lloyd = LLOYD;
 
-    // ---- the pair tables.  The 2^w fp16 levels are staged in LDS first so that building the pairs needs no global
-    //      reads.  Every wavefront of the workgroup calls this exactly once (it contains barriers): wavefronts with
-    //      work after they have requested their first block and query, so that those loads travel meanwhile. ----
-    // the levels are requested first thing, so that they have arrived when the tables are built
-    float level_of_lane = 0.0f;
-    if (tid < 64) {
-        level_of_lane = (tid < 32) ? p.k.table[tid & 31] : p.v.table[tid & 31];
+    // ---- the lookup tables.  Their LDS image was built when the cache's tables were set; the workgroup copies it,
+    //      16 bytes per thread and step.  The image is requested first thing and stored after the wavefront has
+    //      requested its first block and query, so that those loads travel meanwhile.  Every wavefront of the
+    //      workgroup calls build_tables exactly once (it contains a barrier). ----
+    constexpr uint32_t kThreads = 64 * kWaves;
+    constexpr uint32_t kImgVecs = ROWS * (kTableRowBytes / 16);
+    constexpr uint32_t kImgLoads = (kImgVecs + kThreads - 1) / kThreads;
+    uint4v timg[kImgLoads ? kImgLoads : 1];
+    if constexpr (ROWS != 0) {
+        const uint4v *img = reinterpret_cast<const uint4v *>(p.table_image);
+#pragma unroll
+        for (uint32_t u = 0; u < kImgLoads; ++u) {
+            timg[u] = img[min(tid + u * kThreads, kImgVecs - 1)];
+        }
     }
     auto build_tables = [&]() {
         if constexpr (ROWS == 0) {
-            return; // no tables, hence no barriers either
+            return; // no tables, hence no barrier either
         }
-        uint16_t *levels_h = reinterpret_cast<uint16_t *>(lds + ROWS * (kTableRowBytes / 4)); // [2][32]
-        if (tid < 64) {
-            levels_h[tid] = __builtin_bit_cast(uint16_t, (_Float16)level_of_lane);
-        }
-        __syncthreads();
-        // eight table words per thread and pass: the reads of a pass are independent, so their latencies overlap
-        constexpr uint32_t kWords = ROWS * 64, kStep = 64 * kWaves, kBatch = 8;
-        for (uint32_t i0 = tid; i0 < kWords; i0 += kBatch * kStep) {
-            uint32_t val[kBatch];
+        uint4v *dst = reinterpret_cast<uint4v *>(lds);
 #pragma unroll
-            for (uint32_t u = 0; u < kBatch; ++u) {
-                const uint32_t i = min(i0 + u * kStep, kWords - 1);
-                const uint32_t e = i >> 6, half_row = (i >> 5) & 1; // 0: V table, 1: K table
-                const uint32_t w = half_row ? WK : WV;
-                const uint32_t base = half_row ? 0u : 32u;
-                if (w == 5u) {
-                    // the 32 single values, in both halves of the word
-                    const uint32_t lv = levels_h[base + (e & 31u)];
-                    val[u] = e < 32u ? (lv | (lv << 16)) : 0u;
-                    continue;
-                }
-                const uint32_t lo = levels_h[base + (e & ((1u << w) - 1u))];
-                const uint32_t hi = levels_h[base + ((e >> w) & ((1u << w) - 1u))];
-                val[u] = (e < (1u << (2 * w))) ? (lo | (hi << 16)) : 0u;
-            }
-#pragma unroll
-            for (uint32_t u = 0; u < kBatch; ++u) {
-                const uint32_t i = i0 + u * kStep;
-                if (i < kWords) {
-                    lds[i] = val[u];
-                }
+        for (uint32_t u = 0; u < kImgLoads; ++u) {
+            const uint32_t i = tid + u * kThreads;
+            if (i < kImgVecs) {
+                dst[i] = timg[u];
             }
         }
         __syncthreads();
@@ -358,7 +332,10 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
         return;
     }
     uint32_t seq;
-    {
+    const uint32_t uniform_nb = p.uniform_blocks;
+    if (uniform_nb) {
+        seq = g0 / (uniform_nb * p.Hkv);
+    } else {
         // largest s with blk_off[s] * Hkv <= g0 (sequences without tokens share their offset with the next one):
         // a 64-way search, one probe per lane and step
         uint32_t lo = 0, hi = p.n_seq;
@@ -373,8 +350,9 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
         seq = __builtin_amdgcn_readfirstlane(lo);
     }
     while (g0 < g1) {
-    const uint32_t seq_first = p.blk_off[seq];
-    const uint32_t nb_cap = p.blk_off[seq + 1] - seq_first; // blocks the cached length of this sequence spans
+    const uint32_t seq_first = uniform_nb ? seq * uniform_nb : p.blk_off[seq];
+    // blocks the cached length of this sequence spans
+    const uint32_t nb_cap = uniform_nb ? uniform_nb : p.blk_off[seq + 1] - seq_first;
     if (nb_cap == 0) {
         ++seq;
         continue;
@@ -782,7 +760,7 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
 
 template <int D, int WK, int WV, int GP, bool LLOYD> int launch_gp(const MfmaParams &p, hipStream_t s)
 {
-    constexpr size_t smem = (size_t)table_rows<WK, WV>() * kTableRowBytes + 64 * sizeof(uint16_t);
+    constexpr size_t smem = (size_t)table_rows<WK, WV>() * kTableRowBytes;
     constexpr uint32_t waves = mfma_decode_waves_per_wg(GP, D, WK, WV);
     static bool configured = false;
     if (!configured) {
