@@ -290,6 +290,10 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     //      16 bytes per thread and step.  The image is requested first thing and stored after the wavefront has
     //      requested its first block and query, so that those loads travel meanwhile.  Every wavefront of the
     //      workgroup calls build_tables exactly once (it contains a barrier). ----
+    // The arguments span four 64-byte lines of kernel-argument memory, each a miss of its own when first touched.
+    // Naming one value of every line here makes the compiler fetch all four at once instead of one after the other
+    // as the prologue gets to them.
+    asm volatile("" ::"s"(p.total_blocks), "s"(p.v.fields), "s"(p.table_image), "s"(p.q_hi));
     constexpr uint32_t kThreads = 64 * kWaves;
     constexpr uint32_t kImgVecs = ROWS * (kTableRowBytes / 16);
     constexpr uint32_t kImgLoads = (kImgVecs + kThreads - 1) / kThreads;
