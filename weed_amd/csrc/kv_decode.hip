@@ -212,6 +212,20 @@ __global__ void __launch_bounds__(256) prep_q_rows_kernel(const float *__restric
     __shared__ float qs[kRowsPerWg][256];
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t row0 = blockIdx.x * kRowsPerWg;
+    // The rotation does not depend on the query: its first 64 elements per thread are requested before anything else,
+    // so that they travel together with the query rows (one round trip to memory instead of two).  d is a multiple of
+    // 64 here (the host checks).
+    const bool rot_thread = rotate && tid < d;
+    float x0[64];
+    auto request = [&](float (&x)[64], uint32_t i0) {
+#pragma unroll
+        for (int u = 0; u < 64; ++u) {
+            x[u] = rot_t[tid + d * (i0 + u)];
+        }
+    };
+    if (rot_thread) {
+        request(x0, 0);
+    }
     if (blk_off && blockIdx.x == 0) {
         block_offsets(lens, n_seq, blk_off);
     }
@@ -231,19 +245,17 @@ __global__ void __launch_bounds__(256) prep_q_rows_kernel(const float *__restric
     for (int r = 0; r < kRowsPerWg; ++r) {
         acc[r] = rotate ? 0.0f : qs[r][tid];
     }
-    if (rotate && tid < d) {
-        // d is a multiple of 64 here (the host checks); sixty-four independent loads of the rotation are in flight at a time
+    if (rot_thread) {
+        // sixty-four elements at a time (same order of fused multiply-adds as the single-row kernel)
         for (uint32_t i0 = 0; i0 < d; i0 += 64) {
-            float x[64];
-#pragma unroll
-            for (int u = 0; u < 64; ++u) {
-                x[u] = rot_t[tid + d * (i0 + u)];
+            if (i0) {
+                request(x0, i0);
             }
 #pragma unroll
             for (int u = 0; u < 64; ++u) {
 #pragma unroll
                 for (int r = 0; r < kRowsPerWg; ++r) {
-                    acc[r] = fmaf(qs[r][i0 + u], x[u], acc[r]);
+                    acc[r] = fmaf(qs[r][i0 + u], x0[u], acc[r]);
                 }
             }
         }
@@ -600,6 +612,38 @@ __global__ void __launch_bounds__(256) combine_rows_kernel(const float *__restri
     const uint32_t tid = threadIdx.x;
     const uint32_t row0 = blockIdx.x * kRowsPerWg;
     const uint32_t PS = d + 2;
+    // The rotation does not depend on the partials: its first elements are requested before anything else, so that they
+    // travel together with the partials.  d is a multiple of 64 here (the host checks).
+    const bool rot_thread = unrotate && tid < d;
+    float x0[64];
+    auto request = [&](float (&x)[64], uint32_t j0) {
+#pragma unroll
+        for (int u = 0; u < 64; ++u) {
+            x[u] = rv[tid + d * (j0 + u)];
+        }
+    };
+    if (rot_thread) {
+        request(x0, 0);
+    }
+    // Thread groups of d2 (power of two >= d) threads take the partials in turn.  The first four partials of every
+    // group and row are requested here, before their weights are known (slots that turn out to be unused are read
+    // and dropped), so that they travel together with the partials' headers.
+    uint32_t d2 = 32;
+    while (d2 < d) {
+        d2 <<= 1;
+    }
+    const uint32_t grp = tid / d2, ngrp = 256 / d2, j = tid % d2;
+    const bool col_ok = j < d;
+    float x[kRowsPerWg][4];
+#pragma unroll
+    for (int r = 0; r < kRowsPerWg; ++r) {
+        const float *base = partials + (uint64_t)(row0 + r) * max_slots * PS + 2 + j;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const uint32_t k = grp + u * ngrp;
+            x[r][u] = (col_ok && row0 + r < n_rows && k < max_slots) ? base[(uint64_t)k * PS] : 0.0f;
+        }
+    }
     {
         // one wavefront per row, one lane per partial: weights of the row's partials
         static_assert(kRowsPerWg == 4, "one 64-lane wavefront per row");
@@ -629,26 +673,7 @@ __global__ void __launch_bounds__(256) combine_rows_kernel(const float *__restri
     }
     __syncthreads();
     {
-        // Thread groups of d2 (power of two >= d) threads take the partials in turn.  The first four partials of
-        // every group and row are fetched without branches, so that all loads of all rows are in flight together.
-        uint32_t d2 = 32;
-        while (d2 < d) {
-            d2 <<= 1;
-        }
-        const uint32_t grp = tid / d2, ngrp = 256 / d2, j = tid % d2;
-        const bool col_ok = j < d;
         float acc[kRowsPerWg];
-        float x[kRowsPerWg][4];
-#pragma unroll
-        for (int r = 0; r < kRowsPerWg; ++r) {
-            const float *base = partials + (uint64_t)(row0 + r) * max_slots * PS + 2 + j;
-            const uint32_t n = n_s[r];
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const uint32_t k = grp + u * ngrp;
-                x[r][u] = (col_ok && k < n) ? base[(uint64_t)k * PS] : 0.0f;
-            }
-        }
 #pragma unroll
         for (int r = 0; r < kRowsPerWg; ++r) {
             const float *base = partials + (uint64_t)(row0 + r) * max_slots * PS + 2 + j;
@@ -657,7 +682,8 @@ __global__ void __launch_bounds__(256) combine_rows_kernel(const float *__restri
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
                 const uint32_t k = grp + u * ngrp;
-                a = fmaf(k < n ? w_s[r][k] : 0.0f, x[r][u], a);
+                // (an unused slot may hold anything, so it is skipped rather than weighted with zero)
+                a = k < n ? fmaf(w_s[r][k], x[r][u], a) : a;
             }
             if (col_ok) {
                 for (uint32_t k = grp + 4 * ngrp; k < n; k += ngrp) {
@@ -701,18 +727,15 @@ __global__ void __launch_bounds__(256) combine_rows_kernel(const float *__restri
         for (int r = 0; r < kRowsPerWg; ++r) {
             res[r] = 0.0f;
         }
-        // d is a multiple of 64 here (the host checks); sixty-four independent loads of the rotation are in flight at a time
         for (uint32_t j0 = 0; j0 < d; j0 += 64) {
-            float x[64];
-#pragma unroll
-            for (int u = 0; u < 64; ++u) {
-                x[u] = rv[tid + d * (j0 + u)];
+            if (j0) {
+                request(x0, j0);
             }
 #pragma unroll
             for (int u = 0; u < 64; ++u) {
 #pragma unroll
                 for (int r = 0; r < kRowsPerWg; ++r) {
-                    res[r] = fmaf(o_sh[r][j0 + u], x[u], res[r]);
+                    res[r] = fmaf(o_sh[r][j0 + u], x0[u], res[r]);
                 }
             }
         }

@@ -74,25 +74,23 @@ template <int W, int N, int P> __device__ __forceinline__ uint32_t pair_addr(con
 {
     constexpr int bit = 2 * W * P;
     constexpr int dw = bit >> 5, sh = bit & 31;
-    uint32_t a;
     if constexpr (W == 4) {
         // result bytes (3..0) = (0, 0, byte sh/8 of the run's dword, lane byte); selector values 4..7 name the bytes of
         // the first source, 0..3 those of the second, 0x0c a zero byte
         constexpr uint32_t sel = 0x0c0c0000u | ((4u + sh / 8) << 8);
-        asm("v_perm_b32 %0, %1, %2, %3" : "=v"(a) : "v"(x[dw]), "v"(lane_byte), "s"(sel));
+        return __builtin_amdgcn_perm(x[dw], lane_byte, sel);
     } else {
+        // (builtins rather than inline assembly: the compiler then knows that no wait state is needed between the two
+        // instructions and may interleave the pairs)
         uint32_t t;
         if constexpr (sh + 2 * W <= 32) {
-            asm("v_bfe_u32 %0, %1, %2, %3" : "=v"(t) : "v"(x[dw]), "n"(sh), "n"(2 * W));
+            t = __builtin_amdgcn_ubfe(x[dw], sh, 2 * W);
         } else {
             // the pair straddles two dwords: funnel-shift it down first
-            uint32_t f;
-            asm("v_alignbit_b32 %0, %1, %2, %3" : "=v"(f) : "v"(x[dw + 1 < N ? dw + 1 : dw]), "v"(x[dw]), "n"(sh));
-            asm("v_bfe_u32 %0, %1, 0, %2" : "=v"(t) : "v"(f), "n"(2 * W));
+            t = __builtin_amdgcn_ubfe(__builtin_amdgcn_alignbit(x[dw + 1 < N ? dw + 1 : dw], x[dw], sh), 0, 2 * W);
         }
-        asm("v_lshl_add_u32 %0, %1, 8, %2" : "=v"(a) : "v"(t), "v"(lane_byte));
+        return (t << 8) + lane_byte;
     }
-    return a;
 }
 
 // LDS byte address of the single-value entry of field F (5-bit fields): (field << 8) | lane byte.
