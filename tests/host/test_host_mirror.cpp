@@ -146,6 +146,21 @@ TEST_CASE(test_reshape_rules, false)
     REQUIRE_THROWS_AS(std::make_shared<CpuRealStorage>(0U), std::invalid_argument);
 }
 
+TEST_CASE(test_shapes_beyond_32_bit_indices_are_refused, false)
+{
+    // 3 * 32 * 8192 * 8192 = 3 * 2^31 elements (the score tensor of a three-sequence 8192-token prefill at 32 heads)
+    // wraps to 2^31 in 32-bit arithmetic; 2 * ... wraps to 0.  Both must be refused before any storage exists.
+    const std::vector<tcapint> three{ 3U, 32U, 8192U, 8192U }, two{ 2U, 32U, 8192U, 8192U };
+    REQUIRE_THROWS_AS(Tensor::checked_elements(three), std::invalid_argument);
+    REQUIRE_THROWS_AS(Tensor::checked_elements(two), std::invalid_argument);
+    REQUIRE_THROWS_AS(Tensor::full_contiguous_stride(three), std::invalid_argument);
+    REQUIRE_THROWS_AS(Tensor::zeros(three, false, false, DType::REAL, DeviceTag::CPU), std::invalid_argument);
+    REQUIRE_THROWS_AS(Tensor::zeros(two, false, false, DType::REAL, DeviceTag::CPU), std::invalid_argument);
+    REQUIRE(Tensor::checked_elements({ 65535U, 65537U }) == 4294967295ULL); // the largest count that still fits
+    TensorPtr x = std::make_shared<Tensor>(std::vector<real1>{ 0, 1, 2, 3 }, std::vector<tcapint>{ 2, 2 }, false, DeviceTag::CPU);
+    REQUIRE_THROWS_AS(Tensor::reshape(x, { 65536, 65536 }), std::invalid_argument);
+}
+
 TEST_CASE(test_cpu_tensors_do_not_compute, false)
 {
     // there is no CPU arithmetic in this build: an op handed host tensors must say so, never fall back

@@ -604,6 +604,14 @@ int launch_matmul(const char *fn, const MatGeom &g, uint32_t batch, const float 
         return WEED_HIP_OK;
     }
     WEED_HIP_REQUIRE(batch <= 65535u, "%s: %u products in one call (at most 65535)", fn, batch);
+    if (batch > 1) {
+        // the kernels add a product's batch offsets to the operand offsets in 32 bits: refuse what would wrap
+        const uint64_t c0 = g.nb0 - 1, c1 = batch / g.nb0 - 1, lim = 0xffffffffull;
+        WEED_HIP_REQUIRE((uint64_t)g.a_off + c0 * g.a_bs[0] + c1 * g.a_bs[1] <= lim &&
+                             (uint64_t)g.b_off + c0 * g.b_bs[0] + c1 * g.b_bs[1] <= lim &&
+                             (uint64_t)g.o_off + c0 * g.o_bs[0] + c1 * g.o_bs[1] <= lim,
+                         "%s: a batch offset exceeds 32 bits", fn);
+    }
     const uint32_t M = g.M, N = g.N, K = g.K;
     ProfileScope prof("matmul");
     // few output tiles and a long k: the tiles' k ranges are split over more workgroups (guarded instances below)

@@ -4,6 +4,7 @@
 #include "weed_hip.h"
 
 #include <algorithm>
+#include <limits>
 #include <cmath>
 #include <random>
 
@@ -319,8 +320,24 @@ bool Tensor::is_contiguous(const std::vector<tcapint> &shp, const std::vector<tc
     return true;
 }
 
+// Number of elements of a shape, computed in 64 bits.  Sizes, strides and offsets are tcapint (32 bits, as in the
+// reference's default build, include/common/weed_types.hpp:48-66): a shape whose element count does not fit would
+// wrap silently and under-allocate, so it is refused here, before any storage exists or any kernel runs.
+uint64_t Tensor::checked_elements(const std::vector<tcapint> &shp)
+{
+    uint64_t n = 1U;
+    for (const tcapint &s : shp) {
+        n *= (uint64_t)s;
+        if (n > (uint64_t)std::numeric_limits<tcapint>::max()) {
+            throw std::invalid_argument("Tensor: shape has more elements than a 32-bit index can address");
+        }
+    }
+    return n;
+}
+
 std::vector<tcapint> Tensor::full_contiguous_stride(const std::vector<tcapint> &shp)
 {
+    (void)checked_elements(shp);
     std::vector<tcapint> str(shp.size());
     tcapint run = 1U;
     for (size_t i = 0U; i < shp.size(); ++i) {
@@ -376,11 +393,7 @@ Tensor::Tensor(const real1 &val, const bool &rg, const DeviceTag &dtag, const in
 
 tcapint Tensor::get_size() const
 {
-    tcapint n = 1U;
-    for (const tcapint &s : shape) {
-        n *= s;
-    }
-    return shape.empty() ? 0U : n;
+    return shape.empty() ? 0U : (tcapint)checked_elements(shape);
 }
 
 bool Tensor::is_scalar() const { return get_size() == 1U; }
@@ -466,7 +479,7 @@ TensorPtr Tensor::reshape(const TensorPtr a, const std::vector<symint> &s)
     const tcapint total = out->get_size();
     std::vector<tcapint> shp(s.size());
     symint infer = -1;
-    tcapint known = 1U;
+    uint64_t known = 1U;
     for (size_t i = 0U; i < s.size(); ++i) {
         if (s[i] < 0) {
             if (infer >= 0) {
@@ -475,14 +488,17 @@ TensorPtr Tensor::reshape(const TensorPtr a, const std::vector<symint> &s)
             infer = (symint)i;
         } else {
             shp[i] = (tcapint)s[i];
-            known *= (tcapint)s[i];
+            known *= (uint64_t)(tcapint)s[i];
+            if (known > (uint64_t)std::numeric_limits<tcapint>::max()) {
+                throw std::invalid_argument("Tensor::reshape(): sizes do not match");
+            }
         }
     }
     if (infer >= 0) {
         if (!known || (total % known)) {
             throw std::invalid_argument("Tensor::reshape(): cannot infer dimension size");
         }
-        shp[(size_t)infer] = total / known;
+        shp[(size_t)infer] = (tcapint)(total / known);
         known *= shp[(size_t)infer];
     }
     if (known != total || shp.empty()) {
@@ -1224,7 +1240,14 @@ TensorPtr MultiHeadAttention::forward_quantized(TensorPtr Q, TensorPtr K, Tensor
         HipDevice::check(weed_hip_kv_decode_attn(cache, num_heads, gqa, qp, Q->offset, q_str, op, 0U, q_str, flags));
         return out;
     }
-    if (prefill_path == PREFILL_DENSE || (prefill_path == PREFILL_AUTO && dense_is_cheaper(uB, uT, cache_len))) {
+    // the dense way builds [B, heads, T, L] score tensors, which 32-bit sizes and strides must be able to address
+    const bool dense_fits = (uint64_t)uB * Hq * uT * cache_len <= (uint64_t)std::numeric_limits<tcapint>::max()
+        && (uint64_t)uB * Hkv * cache_len * hd <= (uint64_t)std::numeric_limits<tcapint>::max();
+    if (prefill_path == PREFILL_DENSE && !dense_fits) {
+        throw std::invalid_argument("MultiHeadAttention::forward(): the dense prefill path would need score tensors of "
+                                    "more elements than a 32-bit index can address; use the fused path");
+    }
+    if (dense_fits && (prefill_path == PREFILL_DENSE || (prefill_path == PREFILL_AUTO && dense_is_cheaper(uB, uT, cache_len)))) {
         // Long multi-token calls (prefill): the fused kernel serves one query position per launch, so beyond a few
         // positions it is cheaper to do what the reference does -- dequantise the cache once (still in the rotated
         // basis) and run dense ops: rotate Q, product, / sqrt(d), + mask, softmax, product, un-rotate

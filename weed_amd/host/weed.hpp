@@ -190,6 +190,8 @@ struct Tensor {
 
     static bool is_contiguous(const std::vector<tcapint> &shp, const std::vector<tcapint> &s);
     static std::vector<tcapint> full_contiguous_stride(const std::vector<tcapint> &shp);
+    // element count in 64 bits; throws std::invalid_argument when it exceeds what tcapint can index
+    static uint64_t checked_elements(const std::vector<tcapint> &shp);
 
     static TensorPtr zeros(const std::vector<tcapint> &shape, const bool &rg = false, const bool &s = true,
         const DType &dtype = DType::REAL, const DeviceTag &dtag = DeviceTag::DEFAULT_DEVICE, const int64_t &did = -1);
