@@ -187,7 +187,8 @@ typedef struct {
     int32_t mode;          /* WEED_HIP_KV_UNIFORM or WEED_HIP_KV_LLOYDMAX                                      */
     int32_t n_seq;         /* B: sequences held side by side                                                  */
     int32_t n_kv_heads;    /* Hkv                                                                             */
-    int32_t head_dim;      /* d, a multiple of 32, at most 256                                                 */
+    int32_t head_dim;      /* d, any value in 1..256 as QuantizedKVCache::allocate takes (cpp:31-41); rows are
+                            * stored with d rounded up to a multiple of 32, zeros in the extra coordinates      */
     int32_t max_tokens;    /* capacity per sequence (Weed: max_seq_len)                                        */
     int32_t k_bits;        /* code bits for keys: 1..8 (UNIFORM, any kv_quant_bits of the reference), 1..4 (LLOYDMAX) */
     int32_t v_bits;        /* code bits for values, likewise                                                   */
@@ -221,8 +222,9 @@ int weed_hip_kv_cache_set_tables(weed_hip_kv_cache *cache, int which, const floa
 int weed_hip_kv_cache_get_tables(const weed_hip_kv_cache *cache, int which, float *bounds, float *levels, float *recon);
 
 /* sqrt(sum(x^2)/n + 1e-8) over a strided [n_seq, n_kv_heads, T, d] tensor (multihead_attention.cpp:226-241).
- * `sequential` != 0 reproduces the reference's one-thread fp32 summation order (flat column-major order of the
- * logical [rows, d] reshape of a CONTIGUOUS tensor) bit for bit; 0 uses a tree reduction. */
+ * `sequential` != 0 reproduces the reference's one-thread fp32 summation order bit for bit: the flat column-major
+ * index of the logical tensor (first dimension fastest, d slowest), whatever the strides of the view are; 0 uses a
+ * tree reduction. */
 int weed_hip_block_scale_f32(const float *x_dev, uint32_t off, const uint32_t shape[4], const uint32_t stride[4],
                              int sequential, float *scale_out /* host */);
 

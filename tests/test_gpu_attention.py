@@ -284,6 +284,49 @@ def test_head_dims_and_wide_groups(gpu, oracle):
         cache.close()
 
 
+@pytest.mark.parametrize("d", [8, 48, 80, 100, 250])
+@pytest.mark.parametrize("lloyd", [False, True])
+def test_any_head_dim(gpu, oracle, d, lloyd):
+    """QuantizedKVCache::allocate takes any d (multihead_attention.cpp:31-41; the reference's transformer example
+    runs head_dim 8): rows are stored with head_dim rounded up to a multiple of 32 and zeros in the extra coordinates.
+    The whole chain on the device (rotation in the reference's rounding order, coder, fused attention, un-rotation)
+    against the checker fed the raw inputs, the codes bit for bit, Weed's words included."""
+    import torch
+    rng = np.random.default_rng(7 * d + lloyd)
+    Hkv, Hq, lens = 2, 4, [150, 64, 1]
+    S, L = len(lens), max(lens)
+    bits = 4 if d <= 128 else 3
+    wl = workloads.Workload("any_d", S, Hq, Hkv, d, lens, bits, bits, 0, 0, 0)
+    K = rng.standard_normal((S, Hkv, L, d), dtype=np.float32)
+    V = rng.standard_normal((S, Hkv, L, d), dtype=np.float32)
+    q = rng.standard_normal((S, Hq, d), dtype=np.float32)
+    Rk, Rv = rotations(oracle, d, 500 + d)
+    Kr = oracle.apply_rotation(K.reshape(-1, d), Rk).reshape(K.shape)
+    Vr = oracle.apply_rotation(V.reshape(-1, d), Rv).reshape(V.shape)
+    mode = gpu.KV_LLOYDMAX if lloyd else gpu.KV_UNIFORM
+    scales = None if lloyd else (oracle.block_scale(Kr), oracle.block_scale(Vr))
+    cache = build_cache(gpu, wl, mode, K, V, rotations=(Rk, Rv), scales=scales, rotate=2)
+    kspec, vspec = coder_specs(oracle, cache)
+    for which, xr, spec in ((0, Kr, kspec), (1, Vr, vspec)):
+        for sq, n in enumerate(lens):
+            want_f, want_a = oracle.encode_rows(spec, xr[sq, :, :n].reshape(-1, d))
+            got_f, got_a = export(cache, which, n, seq_begin=sq, seq_count=1)
+            np.testing.assert_array_equal(got_f.reshape(-1, d), want_f)
+            if lloyd:
+                np.testing.assert_array_equal(got_a.reshape(-1), want_a)
+            else:
+                wpr = oracle.words_per_row(d, bits)
+                words = torch.zeros((1, Hkv, n, wpr), dtype=torch.int32, device="cuda")
+                cache.export_weed_words(which, words, seq_begin=sq)
+                want_w = oracle.uniform_write_rows(xr[sq, :, :n].reshape(-1, d), bits, spec.block_scale)
+                np.testing.assert_array_equal(words.cpu().numpy().reshape(-1, wpr), want_w)
+    flags = gpu.ATTN_ROTATE_Q | gpu.ATTN_UNROTATE_OUT
+    for gqa, weed in ((gpu.GQA_WEED, True), (gpu.GQA_BLOCKED, False)):
+        want = checker_output(oracle, gpu, cache, wl, q, weed, Rk=Rk, Rv=Rv)
+        assert_attn_close(run_decode(gpu, cache, q, gqa, flags), want, "head_dim %d" % d)
+    cache.close()
+
+
 @pytest.mark.parametrize("d", [32, 64, 96, 128])
 @pytest.mark.parametrize("wk", [2, 3, 4, 5])
 @pytest.mark.parametrize("wv", [2, 3, 4, 5])

@@ -118,7 +118,7 @@ def test_rows_in_weeds_word_packing_are_appended_as_they_are(gpu, oracle, kbits,
 
 
 @pytest.mark.parametrize("bits", [1, 2, 3, 4, 5, 6, 7, 8])
-@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("d", [64, 128, 8, 48, 80])  # 8: the reference's own transformer example; 48, 80: not multiples of 32
 def test_uniform_encode_bit_exact(gpu, oracle, bits, d):
     import torch
     rng = np.random.default_rng(100 * bits + d)
@@ -152,7 +152,7 @@ def test_uniform_encode_bit_exact(gpu, oracle, bits, d):
 
 @pytest.mark.parametrize("k_bits,k_sign,v_bits,v_sign", [(4, 1, 4, 1), (3, 1, 4, 0), (3, 0, 4, 0), (2, 1, 3, 0),
                                                          (1, 0, 2, 0)])
-@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("d", [64, 128, 8, 48, 80])
 def test_lloydmax_encode_bit_exact(gpu, oracle, k_bits, k_sign, v_bits, v_sign, d):
     import torch
     rng = np.random.default_rng(k_bits * 1000 + v_bits * 100 + d)
@@ -171,7 +171,8 @@ def test_lloydmax_encode_bit_exact(gpu, oracle, k_bits, k_sign, v_bits, v_sign, 
         out = torch.zeros((S, Hkv, T, d), dtype=torch.float32, device="cuda")
         cache.dequant(which, out)
         np.testing.assert_array_equal(out.cpu().numpy().reshape(-1, d), oracle.decode_rows(spec, want_f, want_a))
-    assert cache.row_bytes() == (d * (k_bits + k_sign) // 8 + 4, d * (v_bits + v_sign) // 8 + 4)
+    dp = (d + 31) // 32 * 32  # rows are stored with head_dim rounded up to a multiple of 32
+    assert cache.row_bytes() == (dp * (k_bits + k_sign) // 8 + 4, dp * (v_bits + v_sign) // 8 + 4)
     cache.close()
 
 
@@ -304,6 +305,16 @@ def test_block_scale(gpu, oracle):
     t = col_major(x)
     flat = np.transpose(x).reshape(-1)  # storage order of the column-major tensor
     assert gpu.block_scale(t, sequential=True) == np.float32(oracle.block_scale(flat))
+    # the same logical tensor laid out (B, T, heads, d) column-major, as a module hands its rotated K over: the sum
+    # still runs over the logical column-major index (b fastest, then head, token, coordinate), not over the storage
+    import torch
+    B, H, T, d = x.shape
+    store = dev(np.ascontiguousarray(np.transpose(x, (3, 1, 2, 0))))  # storage order: b fastest, then t, h, j
+    view = store.permute(3, 1, 2, 0)
+    assert tuple(view.stride()) == (1, B * T, B, B * T * H) and torch.equal(view, dev(x))
+    assert gpu.block_scale(view, sequential=True) == np.float32(oracle.block_scale(flat))
+    storage_order = store.cpu().numpy().reshape(-1)
+    assert not np.array_equal(storage_order, flat)
     want = np.sqrt(np.mean(x.astype(np.float64) ** 2) + 1e-8)
     assert abs(gpu.block_scale(t) - want) < 1e-6 * want
     assert abs(gpu.block_scale(dev(x)[:, 1:, ::2]) - np.sqrt(np.mean(x[:, 1:, ::2].astype(np.float64) ** 2) + 1e-8)) \
@@ -333,7 +344,7 @@ def test_rotation_on_device(gpu, oracle):
 def test_argument_errors_are_reported_not_faulted(gpu):
     import torch
     with pytest.raises(gpu.WeedHipError) as e:
-        gpu.KVCache(gpu.KV_LLOYDMAX, 1, 1, 48, 16, 3, 3)  # head_dim not a multiple of 32
+        gpu.KVCache(gpu.KV_LLOYDMAX, 1, 1, 300, 16, 3, 3)  # head_dim beyond 256
     assert e.value.code == gpu.EINVAL
     with pytest.raises(gpu.WeedHipError):
         gpu.KVCache(gpu.KV_UNIFORM, 1, 1, 64, 16, 3, 3, 1, 0)  # the uniform coder has no sign bit

@@ -42,6 +42,12 @@ struct Side {
 
 struct weed_hip_kv_cache {
     weed_hip_kv_config cfg;
+    // head_dim as stored: cfg.head_dim rounded up to a multiple of 32.  Rows are coded with zeros in the coordinates
+    // beyond cfg.head_dim (the query has zeros there too, so their key fields are inert; their value coordinates
+    // are never written out) and the rotations are kept as dp x dp matrices with an identity block for them.  Every
+    // layout, kernel instance and scratch size below goes by dp; cfg.head_dim bounds what is read from and written
+    // to the caller's tensors and enters the two scale factors sqrt(head_dim).
+    uint32_t dp = 0;
     uint32_t padded_tokens = 0;
     weedhip::Side k, v;
     bool has_rotations = false;

@@ -92,6 +92,17 @@ __global__ void transpose_square_kernel(const float *__restrict__ r, float *__re
     rt[j + d * i] = r[i + d * j];
 }
 
+// dst (column-major n x n) = src (column-major m x m, m <= n) in the leading block, identity in the rest.
+__global__ void embed_square_kernel(const float *__restrict__ src, uint32_t m, float *__restrict__ dst, uint32_t n)
+{
+    const uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= n * n) {
+        return;
+    }
+    const uint32_t i = idx % n, j = idx / n;
+    dst[idx] = (i < m && j < m) ? src[i + m * j] : (i == j ? 1.0f : 0.0f);
+}
+
 __global__ void bump_lens_kernel(int32_t *lens, int32_t seq_begin, int32_t seq_count, int32_t add)
 {
     const int32_t i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -196,10 +207,12 @@ __device__ __forceinline__ void write_half_block(const uint8_t *staged, const Di
 
 template <int PARTS>
 __device__ __forceinline__ void encode_rows_body(const float *__restrict__ x, const Geom4 &g, uint32_t Hkv, uint32_t T,
-                                                 uint32_t d, uint32_t rows, const float *__restrict__ rot_t, int rotate,
-                                                 const CoderParams &cp, uint8_t *__restrict__ fields,
-                                                 float *__restrict__ alpha_out, const DirectOut &direct, uint32_t block)
+                                                 uint32_t d, uint32_t d_real, uint32_t rows,
+                                                 const float *__restrict__ rot_t, int rotate, const CoderParams &cp,
+                                                 uint8_t *__restrict__ fields, float *__restrict__ alpha_out,
+                                                 const DirectOut &direct, uint32_t block)
 {
+    // d: head_dim as stored (a multiple of 32); d_real <= d: coordinates the caller's rows have, the rest are zeros
     extern __shared__ float smem[];
     const uint32_t pitch = d + 1;
     float *xs = smem;                   // [kEncRows][pitch]
@@ -229,7 +242,7 @@ __device__ __forceinline__ void encode_rows_body(const float *__restrict__ x, co
         for (uint32_t r = tid >> 5; r < kEncRows; r += kEncThreads / 32) {
             const unsigned long long base = row_base[r];
             for (uint32_t j = jl; j < d; j += 32) {
-                dst[r * pitch + j] = (base != ~0ull) ? x[base + (uint64_t)j * g.s[3]] : 0.0f;
+                dst[r * pitch + j] = (base != ~0ull && j < d_real) ? x[base + (uint64_t)j * g.s[3]] : 0.0f;
             }
         }
     }
@@ -347,7 +360,7 @@ __device__ __forceinline__ void encode_rows_body(const float *__restrict__ x, co
             }
         }
         const float norm = sqrtf(n2);
-        const float sqrt_d = sqrtf((float)d);
+        const float sqrt_d = sqrtf((float)d_real);
         float inv = 0.0f, a = 0.0f;
         if (norm > 1e-30f) {
             inv = sqrt_d / norm;
@@ -426,14 +439,14 @@ struct EncSide {
 template <int PARTS>
 __global__ void __launch_bounds__(kEncThreads)
     encode_rows_pair_kernel(EncSide k, EncSide v, uint32_t blocks_per_side, uint32_t Hkv, uint32_t T, uint32_t d,
-                            uint32_t rows, int rotate)
+                            uint32_t d_real, uint32_t rows, int rotate)
 {
     if (blockIdx.x < blocks_per_side) {
-        encode_rows_body<PARTS>(k.x, k.g, Hkv, T, d, rows, k.rot_t, rotate, k.cp, k.fields, k.alpha_out, k.direct,
-                                blockIdx.x);
+        encode_rows_body<PARTS>(k.x, k.g, Hkv, T, d, d_real, rows, k.rot_t, rotate, k.cp, k.fields, k.alpha_out,
+                                k.direct, blockIdx.x);
     } else {
-        encode_rows_body<PARTS>(v.x, v.g, Hkv, T, d, rows, v.rot_t, rotate, v.cp, v.fields, v.alpha_out, v.direct,
-                                blockIdx.x - blocks_per_side);
+        encode_rows_body<PARTS>(v.x, v.g, Hkv, T, d, d_real, rows, v.rot_t, rotate, v.cp, v.fields, v.alpha_out,
+                                v.direct, blockIdx.x - blocks_per_side);
     }
 }
 
@@ -587,8 +600,8 @@ __device__ __forceinline__ uint32_t load_field(const SideParams &sp, int which, 
 
 // mode 0: dense fp32 (read_row, multihead_attention.cpp:64-79: lo + (code + 0.5) * step, two roundings);
 // mode 1: one field per byte (+ row scales).
-__global__ void unpack_kernel(SideParams sp, int which, int kv_mode, uint32_t Hkv, uint32_t d, uint32_t padded,
-                              int32_t seq_begin, uint32_t S, uint32_t tok_begin, uint32_t T, int out_mode,
+__global__ void unpack_kernel(SideParams sp, int which, int kv_mode, uint32_t Hkv, uint32_t d, uint32_t d_stored,
+                              uint32_t padded, int32_t seq_begin, uint32_t S, uint32_t tok_begin, uint32_t T, int out_mode,
                               float *__restrict__ out_f, Geom4 og, uint8_t *__restrict__ out_b,
                               float *__restrict__ out_scale)
 {
@@ -603,7 +616,7 @@ __global__ void unpack_kernel(SideParams sp, int which, int kv_mode, uint32_t Hk
     const uint32_t s = (uint32_t)(idx / ((uint64_t)d * T * Hkv));
     const uint64_t region = (uint64_t)(seq_begin + s) * Hkv + h;
     const uint32_t n = tok_begin + t;
-    const uint32_t f = load_field(sp, which, region, n, j, d);
+    const uint32_t f = load_field(sp, which, region, n, j, d_stored);
     const float a = sp.alpha ? sp.alpha[region * padded + n] : 0.0f;
     if (out_mode == 1) {
         out_b[idx] = (uint8_t)f;
@@ -625,8 +638,9 @@ __global__ void unpack_kernel(SideParams sp, int which, int kv_mode, uint32_t Hk
 }
 
 // Rows in Weed's word packing: floor(32/bits) codes per int32 (multihead_attention.cpp:43-62).
-__global__ void weed_words_kernel(SideParams sp, int which, uint32_t Hkv, uint32_t d, int32_t seq_begin, uint32_t S,
-                                  uint32_t tok_begin, uint32_t T, uint32_t bits, int32_t *__restrict__ words)
+__global__ void weed_words_kernel(SideParams sp, int which, uint32_t Hkv, uint32_t d, uint32_t d_stored,
+                                  int32_t seq_begin, uint32_t S, uint32_t tok_begin, uint32_t T, uint32_t bits,
+                                  int32_t *__restrict__ words)
 {
     const uint32_t vpw = 32 / bits;
     const uint32_t wpr = (d + vpw - 1) / vpw;
@@ -644,26 +658,31 @@ __global__ void weed_words_kernel(SideParams sp, int which, uint32_t Hkv, uint32
     for (uint32_t k = 0; k < vpw; ++k) {
         const uint32_t j = wi * vpw + k;
         if (j < d) {
-            word |= load_field(sp, which, region, tok_begin + t, j, d) << (k * bits);
+            word |= load_field(sp, which, region, tok_begin + t, j, d_stored) << (k * bits);
         }
     }
     words[idx] = (int32_t)word;
 }
 
 // The reverse: rows in Weed's word packing become one code per byte, rows in (sequence, head, token) order.
-__global__ void fields_from_words_kernel(const int32_t *__restrict__ words, uint64_t rows, uint32_t d, uint32_t bits,
-                                         uint8_t *__restrict__ fields)
+__global__ void fields_from_words_kernel(const int32_t *__restrict__ words, uint64_t rows, uint32_t d,
+                                         uint32_t d_stored, uint32_t bits, uint8_t *__restrict__ fields)
 {
+    // rows of d codes in words; rows of d_stored >= d bytes out (zero codes in the coordinates beyond d)
     const uint32_t vpw = 32 / bits;
     const uint32_t wpr = (d + vpw - 1) / vpw;
     const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= rows * d) {
+    if (idx >= rows * d_stored) {
         return;
     }
-    const uint64_t row = idx / d;
-    const uint32_t j = (uint32_t)(idx - row * d);
-    const uint32_t word = (uint32_t)words[row * wpr + j / vpw];
-    fields[idx] = (uint8_t)((word >> ((j % vpw) * bits)) & ((1u << bits) - 1u));
+    const uint64_t row = idx / d_stored;
+    const uint32_t j = (uint32_t)(idx - row * d_stored);
+    uint32_t code = 0;
+    if (j < d) {
+        const uint32_t word = (uint32_t)words[row * wpr + j / vpw];
+        code = (word >> ((j % vpw) * bits)) & ((1u << bits) - 1u);
+    }
+    fields[idx] = (uint8_t)code;
 }
 
 // sum of squares: tree reduction (one partial per block, finished on the host in double)
@@ -695,16 +714,27 @@ __global__ void sumsq_kernel(const float *__restrict__ x, Geom4 g, uint32_t n1, 
     }
 }
 
-// The reference's order: one fp32 accumulator, storage order (multihead_attention.cpp:229-240).
-__global__ void sumsq_sequential_kernel(const float *__restrict__ x, uint64_t n, float *__restrict__ out)
+// The reference's order: one fp32 accumulator over the flat column-major index of the [B, heads, T, d] tensor
+// (multihead_attention.cpp:229-240 walks the contiguous reshape of it): the first dimension runs fastest, the last
+// slowest, whatever the strides of the view handed in are.
+__global__ void sumsq_sequential_kernel(const float *__restrict__ x, Geom4 g, uint32_t n0, uint32_t n1, uint32_t n2,
+                                        uint32_t n3, float *__restrict__ out)
 {
     if (blockIdx.x || threadIdx.x) {
         return;
     }
     float sum = 0.0f;
-    for (uint64_t i = 0; i < n; ++i) {
-        const float v = x[i];
-        sum = sum + v * v;
+    for (uint32_t i3 = 0; i3 < n3; ++i3) {
+        for (uint32_t i2 = 0; i2 < n2; ++i2) {
+            for (uint32_t i1 = 0; i1 < n1; ++i1) {
+                const uint64_t base =
+                    (uint64_t)g.off + (uint64_t)i1 * g.s[1] + (uint64_t)i2 * g.s[2] + (uint64_t)i3 * g.s[3];
+                for (uint32_t i0 = 0; i0 < n0; ++i0) {
+                    const float v = x[base + (uint64_t)i0 * g.s[0]];
+                    sum = sum + v * v;
+                }
+            }
+        }
     }
     out[0] = sum;
 }
@@ -770,7 +800,7 @@ int encode_both(weed_hip_kv_cache *c, int32_t seq_begin, int32_t seq_count, int3
                 uint32_t k_off, const uint32_t k_stride[4], const float *v_dev, uint32_t v_off,
                 const uint32_t v_stride[4], int rotate)
 {
-    const uint32_t d = (uint32_t)c->cfg.head_dim;
+    const uint32_t d = c->dp, d_real = (uint32_t)c->cfg.head_dim;
     const uint32_t Hkv = (uint32_t)c->cfg.n_kv_heads;
     const uint32_t rows = (uint32_t)seq_count * Hkv * (uint32_t)T_new;
     uint8_t *k_fields = c->enc_fields, *v_fields = c->enc_fields + (size_t)rows * d;
@@ -810,16 +840,16 @@ int encode_both(weed_hip_kv_cache *c, int32_t seq_begin, int32_t seq_count, int3
         const uint32_t T = (uint32_t)T_new;
         switch (parts) {
         case 8:
-            encode_rows_pair_kernel<8><<<2 * blocks, kEncThreads, smem, stream()>>>(ek, ev, blocks, Hkv, T, d, rows, rotate);
+            encode_rows_pair_kernel<8><<<2 * blocks, kEncThreads, smem, stream()>>>(ek, ev, blocks, Hkv, T, d, d_real, rows, rotate);
             break;
         case 4:
-            encode_rows_pair_kernel<4><<<2 * blocks, kEncThreads, smem, stream()>>>(ek, ev, blocks, Hkv, T, d, rows, rotate);
+            encode_rows_pair_kernel<4><<<2 * blocks, kEncThreads, smem, stream()>>>(ek, ev, blocks, Hkv, T, d, d_real, rows, rotate);
             break;
         case 2:
-            encode_rows_pair_kernel<2><<<2 * blocks, kEncThreads, smem, stream()>>>(ek, ev, blocks, Hkv, T, d, rows, rotate);
+            encode_rows_pair_kernel<2><<<2 * blocks, kEncThreads, smem, stream()>>>(ek, ev, blocks, Hkv, T, d, d_real, rows, rotate);
             break;
         default:
-            encode_rows_pair_kernel<1><<<2 * blocks, kEncThreads, smem, stream()>>>(ek, ev, blocks, Hkv, T, d, rows, rotate);
+            encode_rows_pair_kernel<1><<<2 * blocks, kEncThreads, smem, stream()>>>(ek, ev, blocks, Hkv, T, d, d_real, rows, rotate);
             break;
         }
         WEED_HIP_LAUNCH_CHECK();
@@ -831,7 +861,7 @@ int encode_both(weed_hip_kv_cache *c, int32_t seq_begin, int32_t seq_count, int3
 // (sequence, head, token) order) go into the block layout behind the tokens already cached.
 int pack_rows(weed_hip_kv_cache *c, int32_t seq_begin, int32_t seq_count, int32_t T_new)
 {
-    const uint32_t d = (uint32_t)c->cfg.head_dim;
+    const uint32_t d = c->dp;
     const uint32_t Hkv = (uint32_t)c->cfg.n_kv_heads;
     const uint32_t rows = (uint32_t)seq_count * Hkv * (uint32_t)T_new;
     uint8_t *k_fields = c->enc_fields, *v_fields = c->enc_fields + (size_t)rows * d;
@@ -876,7 +906,7 @@ int pack_rows(weed_hip_kv_cache *c, int32_t seq_begin, int32_t seq_count, int32_
 int reserve_append_scratch(weed_hip_kv_cache *c, const char *fn, int32_t seq_count, int32_t T_new)
 {
     const uint64_t rows64 = (uint64_t)seq_count * c->cfg.n_kv_heads * T_new;
-    WEED_HIP_REQUIRE(rows64 * c->cfg.head_dim < (1ull << 32), "%s: more than 2^32 elements in one call", fn);
+    WEED_HIP_REQUIRE(rows64 * c->dp < (1ull << 32), "%s: more than 2^32 elements in one call", fn);
     const size_t rows = (size_t)rows64;
     if (rows > c->enc_rows_cap) {
         WEED_HIP_CHECK(hipStreamSynchronize(stream()));
@@ -885,7 +915,7 @@ int reserve_append_scratch(weed_hip_kv_cache *c, const char *fn, int32_t seq_cou
         c->enc_fields = nullptr;
         c->enc_alpha = nullptr;
         c->enc_rows_cap = 0;
-        if (hipMalloc((void **)&c->enc_fields, 2 * rows * c->cfg.head_dim) != hipSuccess ||
+        if (hipMalloc((void **)&c->enc_fields, 2 * rows * c->dp) != hipSuccess ||
             hipMalloc((void **)&c->enc_alpha, 2 * rows * sizeof(float)) != hipSuccess) {
             return fail(WEED_HIP_ENOMEM, "%s: scratch allocation failed", fn);
         }
@@ -932,8 +962,8 @@ int launch_unpack(const weed_hip_kv_cache *c, int which, int32_t seq_begin, int3
     }
     const SideParams sp = side_params(c, which);
     unpack_kernel<<<(uint32_t)((total + 255) / 256), 256, 0, stream()>>>(
-        sp, which, c->cfg.mode, (uint32_t)c->cfg.n_kv_heads, (uint32_t)c->cfg.head_dim, c->padded_tokens, seq_begin,
-        (uint32_t)seq_count, (uint32_t)tok_begin, (uint32_t)T, out_mode, out_f, og, out_b, out_scale);
+        sp, which, c->cfg.mode, (uint32_t)c->cfg.n_kv_heads, (uint32_t)c->cfg.head_dim, c->dp, c->padded_tokens,
+        seq_begin, (uint32_t)seq_count, (uint32_t)tok_begin, (uint32_t)T, out_mode, out_f, og, out_b, out_scale);
     WEED_HIP_LAUNCH_CHECK();
     return WEED_HIP_OK;
 }
@@ -1004,8 +1034,8 @@ int weed_hip_kv_cache_create(weed_hip_kv_cache **cache, const weed_hip_kv_config
                      "weed_hip_kv_cache_create: unknown mode %d", cfg->mode);
     WEED_HIP_REQUIRE(cfg->n_seq > 0 && cfg->n_kv_heads > 0 && cfg->max_tokens > 0,
                      "weed_hip_kv_cache_create: n_seq, n_kv_heads and max_tokens must be positive");
-    WEED_HIP_REQUIRE(cfg->head_dim >= 32 && cfg->head_dim <= 256 && cfg->head_dim % 32 == 0,
-                     "weed_hip_kv_cache_create: head_dim %d must be a multiple of 32 in [32, 256]", cfg->head_dim);
+    WEED_HIP_REQUIRE(cfg->head_dim >= 1 && cfg->head_dim <= 256,
+                     "weed_hip_kv_cache_create: head_dim %d outside [1, 256]", cfg->head_dim);
     // Weed's uniform coder takes any width that divides into its 32-bit words sensibly; the Lloyd-Max tables exist
     // for 1..4 bits
     const int max_bits = cfg->mode == WEED_HIP_KV_UNIFORM ? 8 : 4;
@@ -1021,6 +1051,7 @@ int weed_hip_kv_cache_create(weed_hip_kv_cache **cache, const weed_hip_kv_config
         return fail(WEED_HIP_ENOMEM, "weed_hip_kv_cache_create: host allocation failed");
     }
     c->cfg = *cfg;
+    c->dp = ((uint32_t)cfg->head_dim + 31u) / 32u * 32u;
     c->padded_tokens = padded_tokens((uint32_t)cfg->max_tokens);
     c->lens.assign((size_t)cfg->n_seq, 0);
     const uint64_t regions = (uint64_t)cfg->n_seq * cfg->n_kv_heads;
@@ -1030,7 +1061,7 @@ int weed_hip_kv_cache_create(weed_hip_kv_cache **cache, const weed_hip_kv_config
         s.bits = which ? cfg->v_bits : cfg->k_bits;
         s.sign = which ? cfg->v_sign : cfg->k_sign;
         s.w = (uint32_t)(s.bits + s.sign);
-        s.region_bytes = region_bytes((uint32_t)cfg->max_tokens, (uint32_t)cfg->head_dim, s.w);
+        s.region_bytes = region_bytes((uint32_t)cfg->max_tokens, c->dp, s.w);
         load_builtin(s);
         const size_t fbytes = (size_t)(regions * s.region_bytes);
         hipError_t e = hipMalloc((void **)&s.fields, fbytes);
@@ -1118,10 +1149,10 @@ int weed_hip_kv_cache_row_bytes(const weed_hip_kv_cache *c, uint32_t *k_row_byte
     WEED_HIP_TRY(check_cache(c, "weed_hip_kv_cache_row_bytes"));
     const uint32_t extra = (c->cfg.mode == WEED_HIP_KV_LLOYDMAX) ? 4u : 0u;
     if (k_row_bytes) {
-        *k_row_bytes = (uint32_t)c->cfg.head_dim * c->k.w / 8 + extra;
+        *k_row_bytes = c->dp * c->k.w / 8 + extra;
     }
     if (v_row_bytes) {
-        *v_row_bytes = (uint32_t)c->cfg.head_dim * c->v.w / 8 + extra;
+        *v_row_bytes = c->dp * c->v.w / 8 + extra;
     }
     return WEED_HIP_OK;
 }
@@ -1138,7 +1169,8 @@ int weed_hip_kv_cache_set_rotations(weed_hip_kv_cache *c, const float *rk_dev, c
 {
     WEED_HIP_TRY(check_cache(c, "weed_hip_kv_cache_set_rotations"));
     WEED_HIP_REQUIRE(rk_dev && rv_dev, "weed_hip_kv_cache_set_rotations: null pointer");
-    const uint32_t d = (uint32_t)c->cfg.head_dim;
+    // kept as dp x dp: the caller's matrix in the leading block, an identity block for the coordinates beyond head_dim
+    const uint32_t d = c->dp, d_real = (uint32_t)c->cfg.head_dim;
     const size_t bytes = sizeof(float) * d * d;
     Side *sides[2] = { &c->k, &c->v };
     const float *src[2] = { rk_dev, rv_dev };
@@ -1149,7 +1181,8 @@ int weed_hip_kv_cache_set_rotations(weed_hip_kv_cache *c, const float *rk_dev, c
                 return fail(WEED_HIP_ENOMEM, "weed_hip_kv_cache_set_rotations: device allocation failed");
             }
         }
-        WEED_HIP_CHECK(hipMemcpyAsync(s.rot, src[which], bytes, hipMemcpyDeviceToDevice, stream()));
+        embed_square_kernel<<<(d * d + 255) / 256, 256, 0, stream()>>>(src[which], d_real, s.rot, d);
+        WEED_HIP_LAUNCH_CHECK();
         transpose_square_kernel<<<(d * d + 255) / 256, 256, 0, stream()>>>(s.rot, s.rot_t, d);
         WEED_HIP_LAUNCH_CHECK();
     }
@@ -1229,17 +1262,16 @@ int weed_hip_block_scale_f32(const float *x_dev, uint32_t off, const uint32_t sh
     const uint64_t total = (uint64_t)shape[0] * shape[1] * shape[2] * shape[3];
     WEED_HIP_REQUIRE(total > 0, "weed_hip_block_scale_f32: empty tensor");
     if (sequential) {
-        // the reference walks the flat buffer of a contiguous tensor, so the storage must be dense
-        uint64_t span = 1;
-        for (int i = 0; i < 4; ++i) {
-            span += (uint64_t)(shape[i] - 1) * stride[i];
-        }
-        WEED_HIP_REQUIRE(span == total, "weed_hip_block_scale_f32: sequential order needs a dense tensor");
         float *sum_dev = nullptr;
         if (hipMalloc((void **)&sum_dev, sizeof(float)) != hipSuccess) {
             return fail(WEED_HIP_ENOMEM, "weed_hip_block_scale_f32: device allocation failed");
         }
-        sumsq_sequential_kernel<<<1, 64, 0, stream()>>>(x_dev + off, total, sum_dev);
+        Geom4 gs;
+        gs.off = off;
+        for (int i = 0; i < 4; ++i) {
+            gs.s[i] = stride[i];
+        }
+        sumsq_sequential_kernel<<<1, 64, 0, stream()>>>(x_dev, gs, shape[0], shape[1], shape[2], shape[3], sum_dev);
         float sum = 0.0f;
         hipError_t e = hipMemcpyAsync(&sum, sum_dev, sizeof(float), hipMemcpyDeviceToHost, stream());
         if (e == hipSuccess) {
@@ -1321,13 +1353,13 @@ int weed_hip_kv_append_weed_words(weed_hip_kv_cache *c, int32_t seq_begin, int32
         }
     }
     WEED_HIP_TRY(reserve_append_scratch(c, fn, seq_count, T_new));
-    const uint32_t d = (uint32_t)c->cfg.head_dim;
+    const uint32_t d = (uint32_t)c->cfg.head_dim, dp = c->dp;
     const uint64_t rows = (uint64_t)seq_count * c->cfg.n_kv_heads * T_new;
-    const uint32_t blocks = (uint32_t)((rows * d + 255) / 256);
-    fields_from_words_kernel<<<blocks, 256, 0, stream()>>>(k_words_dev, rows, d, (uint32_t)c->k.bits, c->enc_fields);
+    const uint32_t blocks = (uint32_t)((rows * dp + 255) / 256);
+    fields_from_words_kernel<<<blocks, 256, 0, stream()>>>(k_words_dev, rows, d, dp, (uint32_t)c->k.bits, c->enc_fields);
     WEED_HIP_LAUNCH_CHECK();
-    fields_from_words_kernel<<<blocks, 256, 0, stream()>>>(v_words_dev, rows, d, (uint32_t)c->v.bits,
-                                                           c->enc_fields + rows * d);
+    fields_from_words_kernel<<<blocks, 256, 0, stream()>>>(v_words_dev, rows, d, dp, (uint32_t)c->v.bits,
+                                                           c->enc_fields + rows * dp);
     WEED_HIP_LAUNCH_CHECK();
     WEED_HIP_TRY(pack_rows(c, seq_begin, seq_count, T_new));
     return finish_append(c, seq_begin, seq_count, T_new);
@@ -1367,7 +1399,7 @@ int weed_hip_kv_export_weed_words(const weed_hip_kv_cache *c, int which, int32_t
     }
     const SideParams sp = side_params(c, which);
     weed_words_kernel<<<(uint32_t)((total + 255) / 256), 256, 0, stream()>>>(
-        sp, which, (uint32_t)c->cfg.n_kv_heads, (uint32_t)c->cfg.head_dim, seq_begin, (uint32_t)seq_count,
+        sp, which, (uint32_t)c->cfg.n_kv_heads, (uint32_t)c->cfg.head_dim, c->dp, seq_begin, (uint32_t)seq_count,
         (uint32_t)tok_begin, (uint32_t)T, (uint32_t)s.bits, words_dev);
     WEED_HIP_LAUNCH_CHECK();
     return WEED_HIP_OK;

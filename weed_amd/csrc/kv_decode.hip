@@ -76,7 +76,8 @@ struct DecodeParams {
     SideParams k, v;
     const int32_t *lens;
     uint32_t padded;
-    uint32_t d;
+    uint32_t d;      // head_dim as stored (a multiple of 32)
+    uint32_t d_real; // the caller's head_dim (the scores are divided by its square root)
     uint32_t Hq, Hkv, G;
     int blocked; // 1: kv = h / G, 0: kv = h % Hkv (Weed)
     const float *q_rot; // [n_seq][Hq][d]
@@ -123,8 +124,9 @@ __device__ void block_offsets(const int32_t *__restrict__ lens, uint32_t n_seq, 
 // q_rot[s][h][:] = q[s][h][:] . Rk  (multihead_attention.cpp:276), or a plain gather when rotate == 0.
 // For the matrix-core kernel the rotated query is also scaled by log2(e)/sqrt(d), divided by a power of two that
 // brings it into [-1, 1], and split into fp16 hi + lo halves.
+// `d`: head_dim as stored (a multiple of 32); `d_real` <= d: coordinates the caller's query has (zeros beyond them).
 __global__ void __launch_bounds__(256) prep_q_kernel(const float *__restrict__ q, Geom3 g, uint32_t Hq, uint32_t d,
-                                                     const float *__restrict__ rot_t, int rotate,
+                                                     uint32_t d_real, const float *__restrict__ rot_t, int rotate,
                                                      float *__restrict__ q_rot, uint16_t *__restrict__ q_hi,
                                                      uint16_t *__restrict__ q_lo, float *__restrict__ q_scale,
                                                      float *__restrict__ q_sum, const int32_t *__restrict__ lens,
@@ -139,7 +141,9 @@ __global__ void __launch_bounds__(256) prep_q_kernel(const float *__restrict__ q
         block_offsets(lens, n_seq, blk_off);
     }
     if (tid < d) {
-        qs[tid] = q[(uint64_t)g.off + (uint64_t)s * g.s[0] + head_offset(g, h) + (uint64_t)tid * g.s[2]];
+        qs[tid] = tid < d_real
+                      ? q[(uint64_t)g.off + (uint64_t)s * g.s[0] + head_offset(g, h) + (uint64_t)tid * g.s[2]]
+                      : 0.0f;
     }
     __syncthreads();
     float acc = 0.0f;
@@ -153,7 +157,7 @@ __global__ void __launch_bounds__(256) prep_q_kernel(const float *__restrict__ q
         }
         q_rot[((uint64_t)s * Hq + h) * d + tid] = acc;
     }
-    const float qc = acc * (1.4426950408889634f / sqrtf((float)d));
+    const float qc = acc * (1.4426950408889634f / sqrtf((float)d_real));
     red_max[tid] = fabsf(qc);
     red_sum[tid] = qc;
     __syncthreads();
@@ -203,7 +207,8 @@ constexpr int kRowsPerWg = 4;
 // every row, so each element of the rotation is read once per workgroup instead of once per row.  Used when there
 // are many rows (batched decode); results are identical (same order of fused multiply-adds).
 __global__ void __launch_bounds__(256) prep_q_rows_kernel(const float *__restrict__ q, Geom3 g, uint32_t Hq, uint32_t d,
-                                                          uint32_t n_rows, const float *__restrict__ rot_t, int rotate,
+                                                          uint32_t d_real, uint32_t n_rows,
+                                                          const float *__restrict__ rot_t, int rotate,
                                                           float *__restrict__ q_rot, uint16_t *__restrict__ q_hi,
                                                           uint16_t *__restrict__ q_lo, float *__restrict__ q_scale,
                                                           float *__restrict__ q_sum, const int32_t *__restrict__ lens,
@@ -233,7 +238,7 @@ __global__ void __launch_bounds__(256) prep_q_rows_kernel(const float *__restric
     for (int r = 0; r < kRowsPerWg; ++r) {
         const uint32_t row = row0 + r;
         float v = 0.0f;
-        if (row < n_rows && tid < d) {
+        if (row < n_rows && tid < d_real) {
             const uint32_t s = row / Hq, h = row % Hq;
             v = q[(uint64_t)g.off + (uint64_t)s * g.s[0] + head_offset(g, h) + (uint64_t)tid * g.s[2]];
         }
@@ -272,7 +277,7 @@ __global__ void __launch_bounds__(256) prep_q_rows_kernel(const float *__restric
         if (row >= n_rows) {
             break;
         }
-        const float k = 1.4426950408889634f / sqrtf((float)d);
+        const float k = 1.4426950408889634f / sqrtf((float)d_real);
         float mx = 0.0f, sum = 0.0f;
         for (uint32_t j = lane; j < d; j += 64) {
             const float qc = qs[r][j] * k;
@@ -319,7 +324,7 @@ __global__ void __launch_bounds__(kThreads) decode_generic_kernel(DecodeParams p
     const uint32_t n0 = split * p.split_tokens;
     const uint32_t n1 = min(L, n0 + p.split_tokens);
     const uint64_t region = (uint64_t)seq * p.Hkv + kvh;
-    const float sqrt_d = sqrtf((float)d);
+    const float sqrt_d = sqrtf((float)p.d_real);
     const uint32_t parts = kThreads / d ? kThreads / d : 1;
     const uint32_t part = tid / d, jj = tid % d;
     const bool pv_active = part < parts;
@@ -521,9 +526,9 @@ __device__ __forceinline__ uint32_t slots_of_row(const SlotGeom &sg, uint32_t s,
     return run_of_block(sg.runs, begin + nb - 1) - run_of_block(sg.runs, begin) + 1;
 }
 
-__global__ void combine_kernel(const float *__restrict__ partials, uint32_t Hq, uint32_t d, uint32_t max_slots,
-                               SlotGeom sg, const float *__restrict__ rv, int unrotate, int log2_domain,
-                               float *__restrict__ out, Geom3 og)
+__global__ void combine_kernel(const float *__restrict__ partials, uint32_t Hq, uint32_t d, uint32_t d_real,
+                               uint32_t max_slots, SlotGeom sg, const float *__restrict__ rv, int unrotate,
+                               int log2_domain, float *__restrict__ out, Geom3 og)
 {
     __shared__ float w_s[1024];
     __shared__ float o_sh[256];
@@ -595,13 +600,16 @@ __global__ void combine_kernel(const float *__restrict__ partials, uint32_t Hq, 
     } else {
         r = o_sh[tid];
     }
-    out[(uint64_t)og.off + (uint64_t)s * og.s[0] + head_offset(og, h) + (uint64_t)tid * og.s[2]] = r;
+    if (tid < d_real) {
+        out[(uint64_t)og.off + (uint64_t)s * og.s[0] + head_offset(og, h) + (uint64_t)tid * og.s[2]] = r;
+    }
 }
 
 // The same as combine_kernel for kRowsPerWg (sequence, head) rows per workgroup and at most 64 partials per row:
 // thread j owns coordinate j of every row, so the rotation is read once per workgroup.
 __global__ void __launch_bounds__(256) combine_rows_kernel(const float *__restrict__ partials, uint32_t Hq, uint32_t d,
-                                                           uint32_t max_slots, uint32_t n_rows, SlotGeom sg,
+                                                           uint32_t d_real, uint32_t max_slots, uint32_t n_rows,
+                                                           SlotGeom sg,
                                                            const float *__restrict__ rv, int unrotate, int log2_domain,
                                                            float *__restrict__ out, Geom3 og)
 {
@@ -748,7 +756,7 @@ __global__ void __launch_bounds__(256) combine_rows_kernel(const float *__restri
 #pragma unroll
     for (int r = 0; r < kRowsPerWg; ++r) {
         const uint32_t row = row0 + r;
-        if (row < n_rows) {
+        if (row < n_rows && tid < d_real) {
             const uint32_t s = row / Hq, h = row % Hq;
             out[(uint64_t)og.off + (uint64_t)s * og.s[0] + head_offset(og, h) + (uint64_t)tid * og.s[2]] = res[r];
         }
@@ -765,7 +773,9 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
 {
     WEED_HIP_REQUIRE(c, "%s: null cache", fn);
     WEED_HIP_REQUIRE(q_dev && out_dev && q_stride && o_stride, "%s: null pointer", fn);
-    const uint32_t Hkv = (uint32_t)c->cfg.n_kv_heads, d = (uint32_t)c->cfg.head_dim, S = (uint32_t)c->cfg.n_seq;
+    // d: head_dim as stored (a multiple of 32, see weed_hip_kv_cache::dp); d_real: the caller's
+    const uint32_t Hkv = (uint32_t)c->cfg.n_kv_heads, d = c->dp, S = (uint32_t)c->cfg.n_seq;
+    const uint32_t d_real = (uint32_t)c->cfg.head_dim;
     WEED_HIP_REQUIRE(n_q_heads > 0 && (uint32_t)n_q_heads % Hkv == 0,
                      "%s: n_q_heads %d must be a positive multiple of n_kv_heads %u", fn, n_q_heads, Hkv);
     WEED_HIP_REQUIRE(gqa_mapping == WEED_HIP_GQA_WEED || gqa_mapping == WEED_HIP_GQA_BLOCKED,
@@ -871,10 +881,10 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
     const bool many_rows = n_rows >= 512 && d % 64 == 0;
     if (many_rows) {
         prep_q_rows_kernel<<<(n_rows + kRowsPerWg - 1) / kRowsPerWg, 256, 0, stream()>>>(
-            q_dev, qg, Hq, d, n_rows, c->k.rot_t, rot_q ? 1 : 0, q_rot, q_hi, q_lo, q_scale, q_sum, c->lens_dev, S,
+            q_dev, qg, Hq, d, d_real, n_rows, c->k.rot_t, rot_q ? 1 : 0, q_rot, q_hi, q_lo, q_scale, q_sum, c->lens_dev, S,
             use_mfma ? blk_off : nullptr);
     } else {
-        prep_q_kernel<<<dim3(Hq, S), 256, 0, stream()>>>(q_dev, qg, Hq, d, c->k.rot_t, rot_q ? 1 : 0, q_rot, q_hi, q_lo,
+        prep_q_kernel<<<dim3(Hq, S), 256, 0, stream()>>>(q_dev, qg, Hq, d, d_real, c->k.rot_t, rot_q ? 1 : 0, q_rot, q_hi, q_lo,
                                                          q_scale, q_sum, c->lens_dev, S, use_mfma ? blk_off : nullptr);
     }
     WEED_HIP_LAUNCH_CHECK();
@@ -925,6 +935,7 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         p.lens = lens_dev ? lens_dev : c->lens_dev;
         p.padded = c->padded_tokens;
         p.d = d;
+        p.d_real = d_real;
         p.Hq = Hq;
         p.Hkv = Hkv;
         p.G = G;
@@ -943,10 +954,10 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
                               gqa_mapping == WEED_HIP_GQA_BLOCKED ? 1 : 0 };
         if (many_rows && n_splits <= 64) {
             combine_rows_kernel<<<(n_rows + kRowsPerWg - 1) / kRowsPerWg, 256, 0, stream()>>>(
-                partials, Hq, d, n_splits, n_rows, sg, c->v.rot, unrot ? 1 : 0, use_mfma ? 1 : 0, out_dev, og);
+                partials, Hq, d, d_real, n_splits, n_rows, sg, c->v.rot, unrot ? 1 : 0, use_mfma ? 1 : 0, out_dev, og);
         } else {
             combine_kernel<<<dim3(Hq, S), n_splits > 16 ? 1024 : 256, 0, stream()>>>(
-                partials, Hq, d, n_splits, sg, c->v.rot, unrot ? 1 : 0, use_mfma ? 1 : 0, out_dev, og);
+                partials, Hq, d, d_real, n_splits, sg, c->v.rot, unrot ? 1 : 0, use_mfma ? 1 : 0, out_dev, og);
         }
         WEED_HIP_LAUNCH_CHECK();
     }
