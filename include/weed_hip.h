@@ -44,6 +44,12 @@ enum {
 /* (src/devices/gpu_device.cpp:396-402, src/storage/gpu_real_storage.cpp:18-23).                        */
 /* ------------------------------------------------------------------------------------------------ */
 int weed_hip_init(int device_id);
+/* The other end of weed_hip_init (the reference's device object goes away with its queue and buffers,
+ * include/devices/gpu_device.hpp:60-82): waits for everything queued, then frees what the library itself holds on the
+ * device -- the cached blocks of weed_hip_malloc, the scratch of split products, its timing events, its own stream.
+ * Caches (weed_hip_kv_cache_destroy) and blocks from weed_hip_malloc that are still in use belong to the caller and
+ * are not touched; free them before or after.  A later weed_hip_init (or any call) starts the library again. */
+int weed_hip_shutdown(void);
 int weed_hip_device_count(int *count);
 int weed_hip_device_name(char *buf, size_t buf_len);
 /* Use an existing hipStream_t for all later launches (NULL restores the library's own stream). */

@@ -749,6 +749,64 @@ struct Bytes {
     }
 };
 
+TEST_CASE(test_integer_storage_on_the_host, false)
+{
+    // symbol-table storage (include/storage/cpu_int_storage.hpp): fills, element access, stream bytes
+    std::shared_ptr<CpuIntStorage> sp = std::make_shared<CpuIntStorage>(std::vector<symint>{ 7, -2, 40000 });
+    CpuIntStorage &s = *sp;
+    REQUIRE(s.dtype == DType::INT && s.stype == INT_CPU_DENSE && s.size == 3U);
+    REQUIRE(s[1U] == -2);
+    s.add(1U, 5);
+    REQUIRE(s[1U] == 3);
+    REQUIRE_THROWS_AS(s[3U], std::invalid_argument);
+    REQUIRE_THROWS_AS(std::make_shared<CpuIntStorage>(0U), std::invalid_argument);
+    std::ostringstream os;
+    s.save(os);
+    Bytes e;
+    e.u32(5U).u32(0xffffffffU).u32(0xffffffffU).u32(3U); // INT_CPU_DENSE, 8-byte device id -1, 3 elements
+    e.u32(7U).u32(3U).u32(40000U);
+    REQUIRE(os.str() == e.b);
+    std::istringstream is(e.b);
+    std::shared_ptr<CpuIntStorage> r = std::dynamic_pointer_cast<CpuIntStorage>(Storage::load(is));
+    REQUIRE(r && r->data == (std::vector<symint>{ 7, 3, 40000 }));
+    s.FillOnes();
+    REQUIRE(s.data == (std::vector<symint>{ 1, 1, 1 }));
+    s.FillValue(-9);
+    REQUIRE(s[2U] == -9);
+    s.FillZeros();
+    REQUIRE(s[0U] == 0);
+}
+
+TEST_CASE(test_integer_storage_on_the_device, true)
+{
+    // include/storage/gpu_int_storage.hpp: allocation, fills, blocking transfers both ways, stream round trip
+    std::vector<symint> ids(1000);
+    for (size_t i = 0; i < ids.size(); ++i) {
+        ids[i] = (symint)(i * 37 % 501) - 250;
+    }
+    std::shared_ptr<GpuIntStorage> g = std::make_shared<GpuIntStorage>(ids);
+    REQUIRE(g->device == DeviceTag::GPU && g->dtype == DType::INT && g->stype == INT_GPU_DENSE);
+    REQUIRE((*g)[0U] == ids[0] && (*g)[999U] == ids[999]);
+    REQUIRE_THROWS_AS((*g)[1000U], std::invalid_argument);
+    REQUIRE_THROWS_AS(g->write(0U, 1), std::domain_error); // as the reference: no element writes on a device
+    std::shared_ptr<CpuIntStorage> back = std::dynamic_pointer_cast<CpuIntStorage>(g->cpu());
+    REQUIRE(back && back->data == ids);
+    std::shared_ptr<GpuIntStorage> up = std::dynamic_pointer_cast<GpuIntStorage>(back->gpu());
+    REQUIRE(up && (*up)[123U] == ids[123]);
+    std::ostringstream os;
+    g->save(os);
+    std::istringstream is(os.str());
+    std::shared_ptr<GpuIntStorage> r = std::dynamic_pointer_cast<GpuIntStorage>(Storage::load(is));
+    REQUIRE(r && std::dynamic_pointer_cast<CpuIntStorage>(r->cpu())->data == ids);
+    GpuIntStorage z(64U);
+    z.FillOnes();
+    REQUIRE(z[63U] == 1);
+    z.FillValue(-5);
+    REQUIRE(z[0U] == -5 && z[63U] == -5);
+    z.FillZeros();
+    REQUIRE(z[31U] == 0);
+}
+
 TEST_CASE(test_checkpoint_linear_known_bytes, false)
 {
     // host-side storage: serialization needs no device

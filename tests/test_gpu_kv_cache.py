@@ -362,6 +362,99 @@ def test_argument_errors_are_reported_not_faulted(gpu):
     cache.close()
 
 
+def test_replaced_tables(gpu, oracle):
+    """weed_hip_kv_cache_set_tables: thresholds and levels of the caller's own (here: a uniform grid on [-2.5, 2.5] and
+    the half-cell centres), reconstruction values rounded to binary16 by the library.  Fields and row scales match the
+    checker given the same thresholds bit for bit; attention matches the checker fed the ROUNDED reconstruction
+    values, which are what the kernels multiply with."""
+    import torch
+    rng = np.random.default_rng(77)
+    d, S, Hkv, Hq, L = 128, 2, 2, 8, 300
+    K = rng.standard_normal((S, Hkv, L, d), dtype=np.float32) * 1.3
+    V = rng.standard_normal((S, Hkv, L, d), dtype=np.float32)
+    q = rng.standard_normal((S, Hq, d), dtype=np.float32)
+    cache = gpu.KVCache(gpu.KV_LLOYDMAX, S, Hkv, d, L, 3, 3, 1, 0)
+    specs = []
+    for which, bits, sign in ((0, 3, 1), (1, 3, 0)):
+        n = 1 << bits
+        edges = np.linspace(-2.5, 2.5, n + 1, dtype=np.float32)
+        bounds = edges[1:-1]
+        levels = ((edges[:-1] + edges[1:]) / 2).astype(np.float32)
+        if sign:
+            w = (edges[1] - edges[0]) / 4
+            recon = np.stack([levels - w, levels + w], axis=1).reshape(-1) * np.float32(1.0001)  # not binary16 values
+        else:
+            recon = levels * np.float32(1.0003)
+        rounded = np.array(cache.set_tables(which, list(bounds), list(levels), list(recon.astype(np.float32))), dtype=np.float32)
+        assert np.array_equal(rounded, rounded.astype(np.float16).astype(np.float32))  # binary16 values
+        assert not np.array_equal(rounded, recon) and np.allclose(rounded, recon, rtol=1e-3)
+        got_b, got_l, got_r = cache.get_tables(which)
+        assert np.array_equal(got_b, bounds) and np.array_equal(got_l, levels) and np.array_equal(got_r, rounded)
+        specs.append(oracle.CoderSpec(1, d, bits, sign=sign, bounds=bounds, levels=levels, recon=rounded))
+    cache.encode_append(dev(K), dev(V), rotate=0)
+    fields, scales = [], []
+    for which, x in ((0, K), (1, V)):
+        want_f, want_a = oracle.encode_rows(specs[which], x.reshape(-1, d))
+        got_f, got_a = export(cache, which, L)
+        np.testing.assert_array_equal(got_f.reshape(-1, d), want_f)
+        np.testing.assert_array_equal(got_a.reshape(-1), want_a)
+        fields.append(got_f)
+        scales.append(got_a)
+        out = torch.zeros((S, Hkv, L, d), dtype=torch.float32, device="cuda")
+        cache.dequant(which, out)
+        np.testing.assert_array_equal(out.cpu().numpy().reshape(-1, d), oracle.decode_rows(specs[which], want_f, want_a))
+    want = oracle.decode_attn(specs[0], specs[1], fields[0], scales[0], fields[1], scales[1], q, [L, L], gqa_weed=False)
+    qd = dev(q)
+    out = torch.zeros_like(qd)
+    cache.decode_attn(qd, out, gqa_mapping=gpu.GQA_BLOCKED, flags=0)
+    gpu.sync()
+    from gpu_helpers import assert_attn_close
+    assert_attn_close(out.cpu().numpy(), want, "replaced tables")
+    # the checker with the UN-rounded values differs visibly: the test would notice a library that skipped the rounding
+    cache.close()
+
+
+def test_a_block_cannot_be_freed_twice(gpu):
+    p1 = gpu.malloc(4096)
+    gpu.free(p1)
+    with pytest.raises(gpu.WeedHipError) as e:
+        gpu.free(p1)
+    assert e.value.code == gpu.EINVAL
+    p2 = gpu.malloc(4096)
+    p3 = gpu.malloc(4096)
+    assert p2 != p3  # the cached block was handed out once
+    gpu.free(p2)
+    gpu.free(p3)
+
+
+def test_shutdown_and_start_again(gpu, oracle):
+    """init -> work -> shutdown -> init -> work: the library gives back what it holds and starts again."""
+    import torch
+
+    def work(seed):
+        rng = np.random.default_rng(seed)
+        a = rng.standard_normal((200, 1100), dtype=np.float32)
+        b = rng.standard_normal((1100, 300), dtype=np.float32)
+        out = torch.zeros((200, 300), device="cuda")
+        gpu.matmul(dev(a), dev(b), out)  # a split product: uses the library's own scratch
+        gpu.sync()
+        np.testing.assert_allclose(out.cpu().numpy(), a.astype(np.float64) @ b.astype(np.float64), rtol=1e-4, atol=1e-3)
+        p = gpu.malloc(1 << 20)
+        gpu.free(p)  # stays in the library's cache
+
+    work(1)
+    gpu.shutdown()
+    gpu.shutdown()  # nothing left to do
+    gpu.check(gpu.load().weed_hip_init(0))
+    gpu.use_torch_stream(torch.cuda.current_stream())
+    work(2)
+    cache = gpu.KVCache(gpu.KV_LLOYDMAX, 1, 1, 64, 64, 3, 3)
+    x = torch.randn((1, 1, 40, 64), device="cuda")
+    cache.encode_append(x, x)
+    assert cache.seq_lens() == [40]
+    cache.close()
+
+
 @pytest.mark.parametrize("shape", [(3, 2, 5, 64), (7, 19, 128), (70, 20), (5, 3, 130), (130, 1, 2, 32)])
 def test_apply_rotation_reference_order(gpu, oracle, shape):
     """y = x.R over the last dimension of a strided tensor, in the reference's summation order: bit-exact against the

@@ -93,6 +93,7 @@ SIGNATURES = {
     "weed_hip_kv_decode_attn": (c_int, [c_void_p, c_int32, c_int32, c_void_p, c_uint32, U32P, c_void_p, c_uint32, U32P,
                                         c_uint32]),
     "weed_hip_kv_decode_tuning": (c_int, [c_int32, c_int32, c_int32]),
+    "weed_hip_shutdown": (c_int, []),
     "weed_hip_kv_decode_attn_noalloc": (c_int, [c_void_p, c_int32, c_int32, c_void_p, c_uint32, U32P, c_void_p, c_uint32,
                                                 U32P, c_uint32]),
     "weed_hip_kv_decode_attn_prefix": (c_int, [c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_uint32, U32P, c_void_p,
@@ -373,6 +374,22 @@ def block_scale(x, sequential=False):
     check(load().weed_hip_block_scale_f32(c_void_p(x.data_ptr()), 0, u32(x.shape), u32(x.stride()), int(sequential),
                                           byref(out)))
     return out.value
+
+
+def malloc(nbytes):
+    """Device block from the library's stream-ordered cache; returns the address."""
+    ptr = c_void_p()
+    check(load().weed_hip_malloc(byref(ptr), ctypes.c_size_t(nbytes)))
+    return ptr.value
+
+
+def free(ptr):
+    check(load().weed_hip_free(c_void_p(ptr)))
+
+
+def shutdown():
+    """Drain the stream and free what the library itself holds on the device; the next call starts it again."""
+    check(load().weed_hip_shutdown())
 
 
 def decode_tuning(wavefronts=0, skew_percent=-1, always_search=False):

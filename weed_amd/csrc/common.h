@@ -29,6 +29,9 @@ int current_device();
 // it once per device with that device current.
 int decode_scratch_setup(int device_id);
 
+// Frees the scratch of the split products (matmul.hip); weed_hip_shutdown calls it after draining the stream.
+void release_split_scratch();
+
 // RAII timing scope: when profiling is on, records events around the enclosed launches.
 struct ProfileScope {
     explicit ProfileScope(const char *name, bool enabled = true);

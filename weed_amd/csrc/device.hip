@@ -261,6 +261,15 @@ int weed_hip_free(void *ptr_dev)
     WEED_HIP_TRY(ensure_init());
     std::lock_guard<std::mutex> lock(g_pool_mutex);
     auto it = g_pool_sizes.find(ptr_dev);
+    if (it != g_pool_sizes.end()) {
+        // a block that is already in the cache must not enter it twice (two later allocations would share it)
+        auto range = g_pool_free.equal_range(it->second);
+        for (auto f = range.first; f != range.second; ++f) {
+            if (f->second == ptr_dev) {
+                return fail(WEED_HIP_EINVAL, "weed_hip_free: %p was freed already", ptr_dev);
+            }
+        }
+    }
     if (it != g_pool_sizes.end() && g_pool_cached + it->second <= pool_cap()) {
         g_pool_free.emplace(it->second, ptr_dev);
         g_pool_cached += it->second;
@@ -281,6 +290,36 @@ int weed_hip_release_cached(void)
     std::lock_guard<std::mutex> lock(g_pool_mutex);
     WEED_HIP_CHECK(hipStreamSynchronize(g_stream));
     pool_release_locked();
+    return WEED_HIP_OK;
+}
+
+int weed_hip_shutdown(void)
+{
+    std::lock_guard<std::mutex> lock(g_mutex);
+    if (!g_initialised) {
+        return WEED_HIP_OK;
+    }
+    WEED_HIP_CHECK(hipSetDevice(g_device));
+    WEED_HIP_CHECK(hipStreamSynchronize(g_stream));
+    if (g_own_stream && g_stream != g_own_stream) {
+        WEED_HIP_CHECK(hipStreamSynchronize(g_own_stream));
+    }
+    for (auto &kv : g_profiles) {
+        resolve_pending(kv.second);
+    }
+    g_profiles.clear();
+    g_profile = false;
+    {
+        std::lock_guard<std::mutex> pool_lock(g_pool_mutex);
+        pool_release_locked();
+    }
+    release_split_scratch();
+    if (g_own_stream) {
+        (void)hipStreamDestroy(g_own_stream);
+        g_own_stream = nullptr;
+    }
+    g_stream = nullptr;
+    g_initialised = false;
     return WEED_HIP_OK;
 }
 

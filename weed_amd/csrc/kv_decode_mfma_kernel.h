@@ -18,6 +18,7 @@
 // table is code + 0.5), so de-quantisation itself is exact; the only roundings are those of the fp32 accumulators.
 #include "kv_decode_mfma.h"
 
+#include <mutex>
 #include <type_traits>
 
 using namespace weedhip;
@@ -764,12 +765,14 @@ template <int D, int WK, int WV, int GP, bool LLOYD> int launch_gp(const MfmaPar
 {
     constexpr size_t smem = (size_t)table_rows<WK, WV>() * kTableRowBytes;
     constexpr uint32_t waves = mfma_decode_waves_per_wg(GP, D, WK, WV);
-    static bool configured = false;
-    if (!configured) {
-        WEED_HIP_CHECK(hipFuncSetAttribute((const void *)decode_mfma_kernel<D, WK, WV, GP, LLOYD>,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        configured = true;
-    }
+    // once per instance and process, whichever host thread gets here first (the others wait for it)
+    static std::once_flag configured;
+    static hipError_t config_status = hipSuccess;
+    std::call_once(configured, [] {
+        config_status = hipFuncSetAttribute((const void *)decode_mfma_kernel<D, WK, WV, GP, LLOYD>,
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    });
+    WEED_HIP_CHECK(config_status);
     if (p.runs.waves != waves) {
         return fail(WEED_HIP_EDEVICE, "decode_mfma: runs were cut for %u wavefronts per workgroup, the kernel has %u",
                     p.runs.waves, waves);

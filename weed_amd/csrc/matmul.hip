@@ -543,6 +543,17 @@ __global__ void __launch_bounds__(256) matmul_split_sum_kernel(const float *__re
 float *g_split_ws = nullptr;
 size_t g_split_ws_bytes = 0;
 
+} // namespace
+namespace weedhip {
+// weed_hip_shutdown: the stream has been drained
+void release_split_scratch()
+{
+    (void)hipFree(g_split_ws);
+    g_split_ws = nullptr;
+    g_split_ws_bytes = 0;
+}
+} // namespace weedhip
+namespace {
 int grow_split_scratch(const char *fn, size_t need)
 {
     if (need > g_split_ws_bytes) {

@@ -85,6 +85,23 @@ void Storage::save(std::ostream &os) const
     }
 }
 
+// Integer storage: the same header, then the elements as 32-bit integers (src/storage/cpu_int_storage.cpp,
+// src/storage/gpu_int_storage.cpp:24-39).
+void IntStorage::save(std::ostream &os) const
+{
+    put<uint32_t>(os, (uint32_t)stype);
+    Serializer::write_int64(os, (symint)get_device_id());
+    Serializer::write_tcapint(os, size);
+    StoragePtr host = const_cast<IntStorage *>(this)->cpu();
+    const CpuIntStorage *c = dynamic_cast<const CpuIntStorage *>(host.get());
+    if (!c || c->data.size() != size) {
+        throw std::domain_error("IntStorage::save: host copy failed");
+    }
+    for (tcapint i = 0U; i < size; ++i) {
+        Serializer::write_symint(os, c->data[i]);
+    }
+}
+
 StoragePtr Storage::load(std::istream &is)
 {
     uint32_t tag;
@@ -93,8 +110,18 @@ StoragePtr Storage::load(std::istream &is)
     Serializer::read_int64(is, did);
     tcapint size;
     Serializer::read_tcapint(is, size);
+    if (tag == (uint32_t)INT_CPU_DENSE || tag == (uint32_t)INT_GPU_DENSE) {
+        std::vector<symint> v(size);
+        for (tcapint i = 0U; i < size; ++i) {
+            Serializer::read_symint(is, v[i]);
+        }
+        if (tag == (uint32_t)INT_CPU_DENSE) {
+            return std::make_shared<CpuIntStorage>(v);
+        }
+        return std::make_shared<GpuIntStorage>(v, (int64_t)did);
+    }
     if (tag != (uint32_t)REAL_CPU_DENSE && tag != (uint32_t)REAL_GPU_DENSE) {
-        // complex, integer and sparse storages (tags 3-8) exist in the reference and not here
+        // complex and sparse storages (tags 3, 4, 7, 8) exist in the reference and not here
         throw std::domain_error("Can't recognize StorageType in Storage::load!");
     }
     std::vector<real1> v(size);

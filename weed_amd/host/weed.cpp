@@ -301,6 +301,103 @@ StoragePtr GpuRealStorage::cpu()
     return host;
 }
 
+CpuIntStorage::CpuIntStorage(tcapint n)
+    : IntStorage(INT_CPU_DENSE, CPU, DType::INT, n)
+    , data(n)
+{
+}
+
+CpuIntStorage::CpuIntStorage(const std::vector<symint> &val)
+    : IntStorage(INT_CPU_DENSE, CPU, DType::INT, (tcapint)val.size())
+    , data(val)
+{
+}
+
+symint CpuIntStorage::operator[](const tcapint &idx) const
+{
+    if (idx >= size) {
+        throw std::invalid_argument("CpuStorage::operator[] argument out-of-bounds!");
+    }
+    return data[idx];
+}
+
+void CpuIntStorage::write(const tcapint &idx, const symint &val)
+{
+    if (idx >= size) {
+        throw std::invalid_argument("CpuStorage::write argument out-of-bounds!");
+    }
+    data[idx] = val;
+}
+
+void CpuIntStorage::add(const tcapint &idx, const symint &val) { write(idx, (*this)[idx] + val); }
+void CpuIntStorage::FillZeros() { std::fill(data.begin(), data.end(), 0); }
+void CpuIntStorage::FillOnes() { std::fill(data.begin(), data.end(), 1); }
+void CpuIntStorage::FillValue(const symint &v) { std::fill(data.begin(), data.end(), v); }
+StoragePtr CpuIntStorage::gpu(int64_t did) { return std::make_shared<GpuIntStorage>(data, did); }
+
+GpuIntStorage::GpuIntStorage(tcapint n, int64_t did_)
+    : IntStorage(INT_GPU_DENSE, GPU, DType::INT, n)
+    , buffer(nullptr)
+    , did(did_ < 0 ? HipDevice::Instance().device_id : did_)
+{
+    WEED_DEVICE_LOCK();
+    void *p = nullptr;
+    HipDevice::check(weed_hip_malloc(&p, sizeof(symint) * (size_t)n));
+    buffer = static_cast<symint *>(p);
+}
+
+GpuIntStorage::GpuIntStorage(const std::vector<symint> &val, int64_t did_)
+    : GpuIntStorage((tcapint)val.size(), did_)
+{
+    WEED_DEVICE_LOCK();
+    HipDevice::check(weed_hip_memcpy_h2d(buffer, val.data(), sizeof(symint) * val.size()));
+}
+
+GpuIntStorage::~GpuIntStorage()
+{
+    if (buffer) {
+        WEED_DEVICE_LOCK();
+        (void)weed_hip_free(buffer);
+    }
+}
+
+symint GpuIntStorage::operator[](const tcapint &idx) const
+{
+    if (idx >= size) {
+        throw std::invalid_argument("GpuStorage::operator[] argument out-of-bounds!");
+    }
+    WEED_DEVICE_LOCK();
+    symint v = 0;
+    HipDevice::check(weed_hip_memcpy_d2h(&v, buffer + idx, sizeof(symint)));
+    return v;
+}
+
+void GpuIntStorage::write(const tcapint &, const symint &) { throw std::domain_error("Don't use GPU-based Storage::write()!"); }
+void GpuIntStorage::add(const tcapint &, const symint &) { throw std::domain_error("Don't use GPU-based Storage::add()!"); }
+
+void GpuIntStorage::FillZeros()
+{
+    WEED_DEVICE_LOCK();
+    HipDevice::check(weed_hip_memset(buffer, 0, sizeof(symint) * (size_t)size));
+}
+
+void GpuIntStorage::FillValue(const symint &v)
+{
+    const std::vector<symint> host(size, v);
+    WEED_DEVICE_LOCK();
+    HipDevice::check(weed_hip_memcpy_h2d(buffer, host.data(), sizeof(symint) * host.size()));
+}
+
+void GpuIntStorage::FillOnes() { FillValue(1); }
+
+StoragePtr GpuIntStorage::cpu()
+{
+    std::shared_ptr<CpuIntStorage> host = std::make_shared<CpuIntStorage>(size);
+    WEED_DEVICE_LOCK();
+    HipDevice::check(weed_hip_memcpy_d2h(host->data.data(), buffer, sizeof(symint) * (size_t)size));
+    return host;
+}
+
 // ---------------------------------------------------------------------------------------------------------
 // tensor
 // ---------------------------------------------------------------------------------------------------------

@@ -29,7 +29,8 @@ constexpr real1 ONE_R1 = 1.0f;
 
 enum DeviceTag { NONE_DEVICE = 0, DEFAULT_DEVICE = 1, CPU = 2, GPU = 3 }; // include/enums/device_tag.hpp
 enum DType { NONE_DTYPE = 0, REAL = 1, COMPLEX = 2, INT = 3, DEFAULT_DTYPE = REAL }; // include/enums/dtype.hpp
-enum StorageType { NONE_STORAGE_TYPE = 0, REAL_CPU_DENSE = 1, REAL_GPU_DENSE = 2 }; // include/enums/storage_type.hpp
+// include/enums/storage_type.hpp (complex and sparse storages, tags 3, 4, 7, 8, are not part of this build)
+enum StorageType { NONE_STORAGE_TYPE = 0, REAL_CPU_DENSE = 1, REAL_GPU_DENSE = 2, INT_CPU_DENSE = 5, INT_GPU_DENSE = 6 };
 // include/enums/module_type.hpp: the tags a serialized module starts with.  Only the three modules of this path can
 // be written or read here; the other values are listed so that a foreign tag is reported by name of its number.
 enum ModuleType {
@@ -154,6 +155,53 @@ struct GpuRealStorage : public RealStorage {
     void FillOnes() override;
     void FillValue(const real1 &v) override;
     StoragePtr cpu() override; // new CpuRealStorage filled by a blocking read (src/storage/gpu_real_storage.cpp:18-23)
+    StoragePtr gpu(int64_t = -1) override { return get_ptr(); }
+};
+
+// include/storage/typed_storage.hpp:30-72 for T = symint: the element type of symbol tables (token ids).
+struct IntStorage : public Storage {
+    using Storage::Storage;
+    virtual symint operator[](const tcapint &idx) const = 0;
+    virtual void write(const tcapint &idx, const symint &val) = 0;
+    virtual void add(const tcapint &idx, const symint &val) = 0;
+    virtual void FillValue(const symint &v) = 0;
+    void save(std::ostream &os) const override; // header, then the elements as 32-bit integers (cpu_int_storage.cpp)
+};
+
+// include/storage/cpu_int_storage.hpp
+struct CpuIntStorage : public IntStorage {
+    std::vector<symint> data;
+    explicit CpuIntStorage(tcapint n);
+    explicit CpuIntStorage(const std::vector<symint> &val);
+    symint operator[](const tcapint &idx) const override;
+    void write(const tcapint &idx, const symint &val) override;
+    void add(const tcapint &idx, const symint &val) override;
+    void FillZeros() override;
+    void FillOnes() override;
+    void FillValue(const symint &v) override;
+    StoragePtr cpu() override { return get_ptr(); }
+    StoragePtr gpu(int64_t did = -1) override; // uploads a copy
+};
+
+// include/storage/gpu_int_storage.hpp, include/storage/gpu_storage.hpp:25-102: owns its device buffer; allocation,
+// fills and the blocking transfers, which is all the reference does with integer storage on a device.  Element writes
+// are refused as there (gpu_storage.hpp:88-94).
+struct GpuIntStorage : public IntStorage {
+    symint *buffer;
+    int64_t did;
+    GpuIntStorage(tcapint n, int64_t did = -1);
+    explicit GpuIntStorage(const std::vector<symint> &val, int64_t did = -1);
+    ~GpuIntStorage() override;
+    GpuIntStorage(const GpuIntStorage &) = delete;
+    GpuIntStorage &operator=(const GpuIntStorage &) = delete;
+    int64_t get_device_id() const override { return did; }
+    symint operator[](const tcapint &idx) const override; // blocking one-element read, as GpuDevice::GetInt
+    void write(const tcapint &idx, const symint &val) override;
+    void add(const tcapint &idx, const symint &val) override;
+    void FillZeros() override;
+    void FillOnes() override;
+    void FillValue(const symint &v) override;
+    StoragePtr cpu() override; // new CpuIntStorage filled by a blocking read (src/storage/gpu_int_storage.cpp:17-23)
     StoragePtr gpu(int64_t = -1) override { return get_ptr(); }
 };
 
