@@ -46,8 +46,85 @@ def build_cache(capi, torch, wl, seed):
     return cache, q, rk, rv
 
 
-def cpu_baseline(capi, torch, cache, wl, q, rk, rv, budget_s=12.0):
-    """Time the CPU checker (reference cost structure, one core) on one sequence of the same workload."""
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def host_threads():
+    """Threads for the all-cores legs: the cores this process may run on, at most 16 (a GPU box's CPU share)."""
+    try:
+        n = len(os.sched_getaffinity(0))
+    except AttributeError:
+        n = os.cpu_count() or 1
+    return max(1, min(16, n))
+
+
+def run_threads(n, fn):
+    """fn(thread index) on n host threads (the checker's C functions release the interpreter lock); wall seconds."""
+    import threading
+    threads = [threading.Thread(target=fn, args=(i,)) for i in range(n)]
+    t0 = time.perf_counter()
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    return time.perf_counter() - t0
+
+
+def cpu_other_legs(np, n_threads):
+    """CPU legs of configurations 5a and 5b on bounded samples (a few seconds each)."""
+    from oracle import oracle as orc
+    out = {}
+    rng = np.random.default_rng(5)
+    d = 128
+    # 5a: rotation (naive product, multihead_attention.cpp:206-207 -> matmul.cpp:34-47) and the row coder
+    # (write_row loop, multihead_attention.cpp:244-257) over a sample of the 2 x 32768 rows, one core
+    rows = 2048
+    X = rng.standard_normal((rows, d), dtype=np.float32)
+    R = orc.orthonormalize_columns(rng.standard_normal(d * d).astype(np.float32))
+    t0 = time.perf_counter()
+    reps = 0
+    while time.perf_counter() - t0 < 3.0:
+        Y = orc.apply_rotation(X, R)
+        orc.uniform_write_rows(Y, 3, 1.0)
+        reps += 1
+    secs = time.perf_counter() - t0
+    # one token = 8 kv heads x (K row + V row) = 16 rows
+    out["cfg5a_encode"] = {
+        "value": reps * rows / 16.0 / secs, "unit": "tokens/s", "cores": 1, "kind": "port",
+        "sample": "%d x %d rows of 128 (of the 65536 rows of K and V of 4096 tokens x 8 heads): naive rotation "
+                  "product + write_row at 3 bits, %.1f s" % (reps, rows, secs)}
+    # 5b: naive fp32 product with sequential-k accumulation (matmul.cpp:34-47), column-major operands; the reference
+    # splits the 2^24 outputs over min(cores, 64) workers, so: a slab of rows per host thread
+    M, K, N = 4096, 1024, 4096
+    m_per = 32
+    A = rng.standard_normal(M * K).astype(np.float32)   # column-major [M, K]: element (i, k) at i + M*k
+    B = rng.standard_normal(K * N).astype(np.float32)   # column-major [K, N]
+    C = np.zeros(M * N, dtype=np.float32)
+
+    def slab(i):
+        orc.matmul(m_per, N, K, A, (i * m_per, 1, M), B, (0, 1, K), C, (i * m_per, 1, M))
+
+    secs = run_threads(n_threads, slab)
+    flops = 2.0 * n_threads * m_per * N * K
+    out["cfg5b_matmul"] = {
+        "value": flops / secs / 1e9, "unit": "GFLOP/s", "cores": n_threads, "kind": "port",
+        "sample": "%d of the 4096 output rows (%d per host thread), naive product with k ascending, %.1f s"
+                  % (n_threads * m_per, m_per, secs)}
+    return out
+
+
+def cpu_baseline(capi, torch, cache, wl, q, rk, rv, budget_s=10.0, n_threads=1):
+    """Time the CPU checker (reference cost structure) on one sequence of the same workload: one core (the
+    reference's own policy at this shape: workers = min(cores, items / 2^18) = 1, parallel_for.cpp:91-106), then one
+    sequence per host thread on all cores."""
     from oracle import oracle as orc
     d = wl.head_dim
     L = wl.lens[0]
@@ -74,7 +151,19 @@ def cpu_baseline(capi, torch, cache, wl, q, rk, rv, budget_s=12.0):
         elapsed = time.perf_counter() - t0
         if elapsed >= budget_s or steps >= 200:
             break
-    return steps / elapsed, steps, elapsed, out
+    # all cores: every host thread decodes the same sequence `per_thread` times (independent sequences in effect)
+    per_thread = max(1, int(round(0.5 * budget_s * steps / elapsed)))
+
+    def many(_):
+        for _i in range(per_thread):
+            orc.decode_attn(specs[0], specs[1], fields[0], scales[0], fields[1], scales[1], qh, [L], gqa_weed=False,
+                            Rk=rkh, Rv=rvh)
+
+    all_secs = run_threads(n_threads, many) if n_threads > 1 else elapsed * per_thread / steps
+    all_cores = {"value": n_threads * per_thread / all_secs, "unit": "tokens/s", "cores": n_threads,
+                 "sample": "%d decode steps of one sequence on each of %d host threads in %.1f s"
+                           % (per_thread, n_threads, all_secs)}
+    return steps / elapsed, steps, elapsed, out, all_cores
 
 
 def time_calls(torch, fn, steps, warmup):
@@ -158,11 +247,15 @@ def extras(capi, torch, workloads, steps, warmup):
         cache.reset()
         cache.encode_append(K, V, rotate=1)
 
-    secs = time_calls(torch, enc, steps, warmup)
+    secs, kernel_s = time_kernel(capi, torch, enc, "kv_encode", steps, warmup)
     in_bytes = 2 * K.numel() * 4
-    out["cfg5a_encode_4096x8x128_3bit"] = {"tokens_per_s": 4096 / secs, "ms": 1e3 * secs,
-                                           "input_gbs": in_bytes / secs / 1e9,
-                                           "rotation_tflops": 2 * 2.0 * K.numel() * d / secs / 1e12}
+    rot_flops = 2 * 2.0 * K.numel() * d  # K and V: rows x 2 d^2
+    out["cfg5a_encode_4096x8x128_3bit"] = {
+        "tokens_per_s": 4096 / secs, "ms": 1e3 * secs, "input_gbs": in_bytes / secs / 1e9,
+        "rotation_tflops": rot_flops / secs / 1e12, "kernel_ms": 1e3 * kernel_s,
+        "roofline": {"bound": "mfma", "achieved": rot_flops / kernel_s / 1e12, "peak": 157.3, "unit": "TFLOP/s",
+                     "frac": rot_flops / kernel_s / 1e12 / 157.3, "kernel": "encode_rows_pair_kernel (K and V)",
+                     "flops_per_launch": rot_flops}}
     cache.close()
     # configuration 4: 16 ragged sequences in [2048, 32768], K 2-bit + sign, V 3-bit, split-context merge
     wl4 = workloads.config(4)
@@ -180,8 +273,10 @@ def extras(capi, torch, workloads, steps, warmup):
         nbytes = wl4.bytes_per_step(True)
         out["cfg4_ragged16_hq%d" % hq] = {"tokens_per_s": wl4.n_seq / secs, "ms_per_step": 1e3 * secs,
                                           "packed_cache_bytes": nbytes, "kernel_ms": 1e3 * kernel_s,
-                                          "kernel_gbs": nbytes / kernel_s / 1e9,
-                                          "frac_of_hbm_peak": nbytes / kernel_s / 1e9 / HBM_PEAK_GBS}
+                                          "step_frac": nbytes / secs / 1e9 / HBM_PEAK_GBS,
+                                          "roofline": {"bound": "hbm", "achieved": nbytes / kernel_s / 1e9, "peak": HBM_PEAK_GBS,
+                                                       "unit": "GB/s", "frac": nbytes / kernel_s / 1e9 / HBM_PEAK_GBS,
+                                                       "algorithmic_bytes_per_launch": nbytes}}
     cache4.close()
     # Weed's own uniform coder at kv_quant_bits = 8 on the headline shape (64 x 8192 tokens x 8 heads, 256 B per token
     # and head): the matrix-core kernel with arithmetic de-quantisation instead of tables
@@ -200,8 +295,9 @@ def extras(capi, torch, workloads, steps, warmup):
     nbytes = sum(wl8.lens) * wl8.n_kv_heads * 2 * d
     out["uniform_8bit_64_sequences"] = {"tokens_per_s": wl8.n_seq / secs, "ms_per_step": 1e3 * secs,
                                         "packed_cache_bytes": nbytes, "kernel_ms": 1e3 * kernel_s,
-                                        "kernel_gbs": nbytes / kernel_s / 1e9,
-                                        "frac_of_hbm_peak": nbytes / kernel_s / 1e9 / HBM_PEAK_GBS}
+                                        "roofline": {"bound": "hbm", "achieved": nbytes / kernel_s / 1e9, "peak": HBM_PEAK_GBS,
+                                                       "unit": "GB/s", "frac": nbytes / kernel_s / 1e9 / HBM_PEAK_GBS,
+                                                       "algorithmic_bytes_per_launch": nbytes}}
     cache8.close()
     del q8, o8
     # configuration 3 again with 256 sequence caches per launch (2 GB of packed rows): what the per-launch fixed cost
@@ -215,8 +311,9 @@ def extras(capi, torch, workloads, steps, warmup):
     nbytes = wl3.bytes_per_step(lloydmax=True)
     out["cfg3_256_sequences"] = {"tokens_per_s": wl3.n_seq / secs, "ms_per_step": 1e3 * secs,
                                  "packed_cache_bytes": nbytes, "kernel_ms": 1e3 * kernel_s,
-                                 "kernel_gbs": nbytes / kernel_s / 1e9,
-                                 "frac_of_hbm_peak": nbytes / kernel_s / 1e9 / HBM_PEAK_GBS}
+                                 "roofline": {"bound": "hbm", "achieved": nbytes / kernel_s / 1e9, "peak": HBM_PEAK_GBS,
+                                                       "unit": "GB/s", "frac": nbytes / kernel_s / 1e9 / HBM_PEAK_GBS,
+                                                       "algorithmic_bytes_per_launch": nbytes}}
     cache3.close()
     return out
 
@@ -320,6 +417,9 @@ def main():
                         t[key.strip()] = int(val)
             if t.get("seqs") == args.seqs and t.get("ctx") == args.ctx:
                 traffic = t.get("hbm_bytes_per_launch")
+        traffic_source = ("replayed from profiles/%s (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, "
+                          "scaled by a copy kernel of known size); not measured in this run"
+                          % os.path.basename(traffic_file)) if traffic is not None else None
 
         result = {
             "metric": "quantized-KV decode attn tokens/sec + HBM GB/s (% roofline) at ctx 8192",
@@ -344,7 +444,7 @@ def main():
             },
             "roofline": {
                 "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+                "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "traffic_source": traffic_source,
                 "kernel": "decode attention main kernel", "kernel_ms": kernel_ms,
                 "algorithmic_bytes_per_launch": bytes_per_launch,
                 "combine_kernel_ms": c_ms / max(1, c_n),
@@ -365,11 +465,17 @@ def main():
             result["single_sequence"] = {"ms_per_step": single_ms, "tokens_per_s": 1e3 / single_ms,
                                          "gbs": wl1.bytes_per_step(True) / (single_ms * 1e-3) / 1e9}
         if not args.no_cpu_baseline:
-            tps, n, secs, cpu_out = cpu_baseline(capi, torch, cache, wl, q, rk, rv)
+            n_threads = host_threads()
+            tps, n, secs, cpu_out, all_cores = cpu_baseline(capi, torch, cache, wl, q, rk, rv, n_threads=n_threads)
             got = out[0:1].cpu().numpy()
             err = float(np.abs(got - cpu_out).max())
+            all_cores["gbs"] = wl1.bytes_per_step(True) * all_cores["value"] / 1e9
             result["cpu_baseline"] = {
                 "value": tps, "unit": "tokens/s", "cores": 1, "kind": "port",
+                "cpu_model": cpu_model(), "host_threads_available": n_threads,
+                "threading": "one core is the reference's own policy at this shape: workers = min(cores, items / 2^18)",
+                "all_cores": all_cores,
+                "other_configs": cpu_other_legs(np, n_threads),
                 "sample": "%d decode steps of ONE of the %d sequences (same shape, ctx %d) in %.1f s; scalar C "
                           "restatement of the reference's path: full dequantise, GQA replicate, K^T copy, naive dots, "
                           "divide, 3-pass softmax" % (n, wl.n_seq, args.ctx, secs),
