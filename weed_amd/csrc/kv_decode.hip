@@ -570,10 +570,20 @@ __global__ void combine_kernel(const float *__restrict__ partials, uint32_t Hq, 
         const uint32_t grp = tid / d2, ngrp = blockDim.x / d2, j = tid % d2;
         float acc = 0.0f;
         if (j < d) {
-            for (uint32_t k = grp; k < n_splits; k += ngrp) {
-                const float w = w_s[k];
-                if (w != 0.0f) {
-                    acc = fmaf(w, base[(uint64_t)k * (d + 2) + 2 + j], acc);
+            // eight partials at a time, so that their loads are in flight together
+            for (uint32_t k0 = grp; k0 < n_splits; k0 += 8 * ngrp) {
+                float y[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const uint32_t k = k0 + u * ngrp;
+                    y[u] = (k < n_splits && w_s[k] != 0.0f) ? base[(uint64_t)k * (d + 2) + 2 + j] : 0.0f;
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const uint32_t k = k0 + u * ngrp;
+                    if (k < n_splits && w_s[k] != 0.0f) {
+                        acc = fmaf(w_s[k], y[u], acc);
+                    }
                 }
             }
         }
@@ -694,8 +704,20 @@ __global__ void __launch_bounds__(256) combine_rows_kernel(const float *__restri
                 a = k < n ? fmaf(w_s[r][k], x[r][u], a) : a;
             }
             if (col_ok) {
-                for (uint32_t k = grp + 4 * ngrp; k < n; k += ngrp) {
-                    a = fmaf(w_s[r][k], base[(uint64_t)k * PS], a);
+                // further partials eight at a time, so that their loads are in flight together (ragged batches and
+                // long contexts leave dozens of partials per row)
+                for (uint32_t k0 = grp + 4 * ngrp; k0 < n; k0 += 8 * ngrp) {
+                    float y[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) {
+                        const uint32_t k = k0 + u * ngrp;
+                        y[u] = k < n ? base[(uint64_t)k * PS] : 0.0f;
+                    }
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) {
+                        const uint32_t k = k0 + u * ngrp;
+                        a = k < n ? fmaf(w_s[r][k], y[u], a) : a;
+                    }
                 }
             }
             acc[r] = a;
