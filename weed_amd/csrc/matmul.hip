@@ -127,8 +127,13 @@ __global__ void __launch_bounds__(256) matmul_mfma_kernel(const float *__restric
     if (EDGE && k_per_split) {
         g.K = min(g.K, k_first + k_per_split);
     }
-    __shared__ __attribute__((aligned(16))) float As[2][TK][PITCH];
-    __shared__ __attribute__((aligned(16))) float Bs[2][TK][PITCH];
+    // Row pitch of a staged slice.  An operand that arrives contiguous along its own index is stored with 16-byte
+    // writes (pitch 132: a multiple of 4).  One that arrives contiguous along k is stored transposed, element by
+    // element: thread (k4, j) writes rows 4 k4 .. 4 k4 + 3 of column j, and with pitch 130 the four k4 of 32
+    // neighbouring threads start 8 banks apart, so their writes hit 32 different banks (with 132 they pair up).
+    constexpr int PITCH_A = A_ICONTIG ? PITCH : PITCH - 2, PITCH_B = B_KCONTIG ? PITCH - 2 : PITCH;
+    __shared__ __attribute__((aligned(16))) float As[2][TK][PITCH_A];
+    __shared__ __attribute__((aligned(16))) float Bs[2][TK][PITCH_B];
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t wi = wave >> 1, wj = wave & 1;
     const uint32_t m0 = blockIdx.x * TM, n0 = blockIdx.y * TN;
@@ -293,8 +298,9 @@ __global__ void __launch_bounds__(256) matmul_mfma_kernel(const float *__restric
 //      A workgroup of 8 wavefronts owns 16 output columns; wavefront w takes the k range [w*k_per_wave, (w+1)*...).
 //      The products run on v_mfma_f32_16x16x4f32 (16 rows x 16 columns x 4 k per instruction).  The contraction
 //      index of an instruction may be any four k as long as both operands agree, so lane (column c = l % 16,
-//      group g = l / 16) keeps the sixteen consecutive k  kb + 16 g .. kb + 16 g + 15  of its column (four 16-byte
-//      loads) and instruction j of an iteration contracts over  { kb + 16 g + j : g = 0..3 }.  The few rows of `a`
+//      group g = l / 16) keeps the k  kb + 16 q + 4 g .. + 3  (q = 0..3) of its column -- four 16-byte loads, each of
+//      which reads 64 consecutive bytes per column across the four groups -- and instruction j = 4 q + i of an
+//      iteration contracts over  { kb + 16 q + 4 g + i : g = 0..3 }.  The few rows of `a`
 //      come from L2 (every workgroup reads all of them).  The eight partial tiles of a workgroup are added in LDS.
 constexpr int kSkinnyWaves = 8;
 
@@ -330,7 +336,7 @@ __global__ void __launch_bounds__(64 * kSkinnyWaves)
     auto load_w = [&](uint32_t kb, float4v (&w)[4]) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            const uint32_t k = kb + 16 * grp + 4 * q;
+            const uint32_t k = kb + 16 * q + 4 * grp; // the four lanes of a column read 64 consecutive bytes
             w[q] = (n_ok && k < kb1) ? *reinterpret_cast<const float4v *>(wcol + k) : float4v{ 0.0f, 0.0f, 0.0f, 0.0f };
         }
     };
@@ -342,7 +348,7 @@ __global__ void __launch_bounds__(64 * kSkinnyWaves)
             const uint32_t m = 16 * (mt0 + t) + c;
 #pragma unroll
             for (int j = 0; j < 16; ++j) {
-                const uint32_t k = kb + 16 * grp + j;
+                const uint32_t k = kb + 16 * (j / 4) + 4 * grp + (j % 4); // as the lane's element j of b
                 av[t][j] = (m < g.M && k < kb1)
                     ? a[(uint64_t)g.a_off + (uint64_t)m * g.a_s0 + (uint64_t)k * g.a_s1] : 0.0f;
             }
