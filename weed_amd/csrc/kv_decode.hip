@@ -137,8 +137,13 @@ __global__ void __launch_bounds__(256) prep_q_kernel(const float *__restrict__ q
     __shared__ float red_sum[256];
     const uint32_t h = blockIdx.x, s = blockIdx.y;
     const uint32_t tid = threadIdx.x;
-    if (blk_off && h == 0 && s == 0) {
-        block_offsets(lens, n_seq, blk_off);
+    if (s == n_seq) {
+        // the extra grid row: one of its workgroups builds the block offsets while the others rotate queries (as part
+        // of a query's workgroup the scan would be the kernel's longest chain)
+        if (blk_off && h == 0) {
+            block_offsets(lens, n_seq, blk_off);
+        }
+        return;
     }
     if (tid < d) {
         qs[tid] = tid < d_real
@@ -228,11 +233,16 @@ __global__ void __launch_bounds__(256) prep_q_rows_kernel(const float *__restric
             x[u] = rot_t[tid + d * (i0 + u)];
         }
     };
+    if (blockIdx.x * kRowsPerWg >= n_rows) {
+        // the extra workgroup behind the last rows: it builds the block offsets while the others rotate queries (as
+        // part of a query's workgroup the scan would be the kernel's longest chain)
+        if (blk_off) {
+            block_offsets(lens, n_seq, blk_off);
+        }
+        return;
+    }
     if (rot_thread) {
         request(x0, 0);
-    }
-    if (blk_off && blockIdx.x == 0) {
-        block_offsets(lens, n_seq, blk_off);
     }
 #pragma unroll
     for (int r = 0; r < kRowsPerWg; ++r) {
@@ -902,11 +912,11 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
     // the multi-row kernels pay off with many (sequence, head) rows; their rotation loops step by 64
     const bool many_rows = n_rows >= 512 && d % 64 == 0;
     if (many_rows) {
-        prep_q_rows_kernel<<<(n_rows + kRowsPerWg - 1) / kRowsPerWg, 256, 0, stream()>>>(
+        prep_q_rows_kernel<<<(n_rows + kRowsPerWg - 1) / kRowsPerWg + (use_mfma ? 1 : 0), 256, 0, stream()>>>(
             q_dev, qg, Hq, d, d_real, n_rows, c->k.rot_t, rot_q ? 1 : 0, q_rot, q_hi, q_lo, q_scale, q_sum, c->lens_dev, S,
             use_mfma ? blk_off : nullptr);
     } else {
-        prep_q_kernel<<<dim3(Hq, S), 256, 0, stream()>>>(q_dev, qg, Hq, d, d_real, c->k.rot_t, rot_q ? 1 : 0, q_rot, q_hi, q_lo,
+        prep_q_kernel<<<dim3(Hq, S + (use_mfma ? 1 : 0)), 256, 0, stream()>>>(q_dev, qg, Hq, d, d_real, c->k.rot_t, rot_q ? 1 : 0, q_rot, q_hi, q_lo,
                                                          q_scale, q_sum, c->lens_dev, S, use_mfma ? blk_off : nullptr);
     }
     WEED_HIP_LAUNCH_CHECK();
