@@ -280,8 +280,8 @@ int weed_hip_kv_decode_attn(weed_hip_kv_cache *cache, int32_t n_q_heads, int32_t
 /* How the decode kernels cut a launch's list of 64-token blocks into per-wavefront runs (no counterpart in the
  * reference; results do not depend on it, only speed).  wavefronts: number of runs, 0 = as many wavefronts as the
  * device holds at once; skew_percent: how much longer than the mean the runs of a workgroup's oldest wavefronts are
- * (and the youngest shorter), negative = the built-in 16; always_search != 0: find every run's first region by search
- * even when all sequences have equal lengths.  The process-wide defaults are read once from the environment variables
+ * (and the youngest shorter), negative = the built-in 16 (28 for kernel instances with three wavefronts per SIMD);
+ * always_search != 0: find every run's first region by search even when all sequences have equal lengths.  The process-wide defaults are read once from the environment variables
  * WEED_HIP_DECODE_WAVES, WEED_HIP_DECODE_SKEW and WEED_HIP_DECODE_SEARCH. */
 int weed_hip_kv_decode_tuning(int32_t wavefronts, int32_t skew_percent, int32_t always_search);
 

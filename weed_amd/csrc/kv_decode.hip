@@ -487,8 +487,10 @@ __global__ void __launch_bounds__(kThreads) decode_generic_kernel(DecodeParams p
 // v_rotation^T (multihead_attention.cpp:343-348): out_i = sum_j O_j Rv[i + d*j].
 constexpr uint32_t kMaxSlots = 1024; // partials per (sequence, head) that combine_kernel can weigh in one pass
 
-// Run-length skew between the wavefront age classes of a workgroup, in percent of the mean run (see RunGeom).
-constexpr uint32_t kRunSkewPercent = 16;
+// Run-length skew between the wavefront age classes of a workgroup, in percent of the mean run (see RunGeom): with
+// two wavefronts per SIMD the older one gets 16 % more than the mean; with three the spread between oldest and
+// youngest is wider (measured on the ragged batch: 16 % -> 47.8 us, 24-40 % -> 46.7-46.9 us, 48 % -> 48.2 us).
+constexpr uint32_t kRunSkewPercent = 16, kRunSkewPercent3 = 28;
 
 // Tuning knobs of the work partition.  The defaults come from the environment, read ONCE per process (at the first
 // decode call or the first weed_hip_kv_decode_tuning): WEED_HIP_DECODE_WAVES (wavefronts the block list is cut for),
@@ -849,7 +851,8 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         // one workgroup per compute unit
         const uint32_t target_units = tune.wavefronts > 0 ? (uint32_t)tune.wavefronts : runs.waves * 256u;
         runs.unit_blocks = std::max(1u, (total_blocks + target_units - 1) / target_units);
-        const uint32_t skew_pct = tune.skew_percent >= 0 ? (uint32_t)std::min(90, tune.skew_percent) : kRunSkewPercent;
+        const uint32_t skew_pct = tune.skew_percent >= 0 ? (uint32_t)std::min(90, tune.skew_percent)
+                                                         : (runs.waves == 12 ? kRunSkewPercent3 : kRunSkewPercent);
         const uint32_t nblk = (max_len + 63) / 64;
         for (;;) {
             runs.skew = std::min(runs.unit_blocks - 1, (runs.unit_blocks * skew_pct + 50) / 100);
