@@ -321,8 +321,10 @@ def extras(capi, torch, workloads, steps, warmup):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    # (a burst of a few dozen launches falls into the clock transient that follows the start of sustained load; a
+    # thousand steps are a tenth of a second and show the steady state)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--seqs", type=int, default=64, help="independent ctx-8192 sequence caches per launch")
     ap.add_argument("--ctx", type=int, default=8192)
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -386,6 +388,34 @@ def main():
         kernel_ms = k_ms / max(1, k_n)
         bytes_per_launch = wl.bytes_per_step(lloydmax=True)
         achieved = bytes_per_launch / (kernel_ms * 1e-3) / 1e9
+        one_kernel = c_n == 0  # the matrix-core kernel rotated the queries and merged its partials itself
+
+        # the same step as three kernels (query rotation, attention, merge), for comparison
+        separate = None
+        if one_kernel:
+            capi.decode_tuning(separate_merge=True)
+            try:
+                for _ in range(args.warmup):
+                    step()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(args.steps):
+                    step()
+                torch.cuda.synchronize()
+                sep_ms = 1e3 * (time.perf_counter() - t0) / args.steps
+                capi.profile_reset()
+                capi.profile_enable(True)
+                for _ in range(args.steps):
+                    step()
+                torch.cuda.synchronize()
+                sk_ms, sk_n = capi.profile_read("kv_decode_attn")
+                sc_ms, sc_n = capi.profile_read("kv_decode_combine")
+                capi.profile_enable(False)
+            finally:
+                capi.decode_tuning()
+            separate = {"ms_per_step": sep_ms, "attention_kernel_ms": sk_ms / max(1, sk_n),
+                        "attention_kernel_frac": bytes_per_launch / (sk_ms / max(1, sk_n) * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                        "merge_kernel_ms": sc_ms / max(1, sc_n)}
 
         # batch = 1 latency of the same shape (one sequence per launch: launch-latency bound); part of the extras, so
         # that a --no-extras run launches the main kernel at the headline shape only
@@ -445,9 +475,13 @@ def main():
             "roofline": {
                 "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "traffic_source": traffic_source,
-                "kernel": "decode attention main kernel", "kernel_ms": kernel_ms,
+                "kernel": ("decode attention kernel; the only kernel of the step: it rotates the queries and merges "
+                           "its partials itself") if one_kernel else "decode attention main kernel",
+                "kernels_per_step": 1 if one_kernel else 3,
+                "kernel_ms": kernel_ms,
                 "algorithmic_bytes_per_launch": bytes_per_launch,
                 "combine_kernel_ms": c_ms / max(1, c_n),
+                "same_step_as_three_kernels": separate,
             },
             "whole_step_gbs": bytes_per_launch / (ms_per_step * 1e-3) / 1e9,
         }

@@ -281,8 +281,13 @@ int weed_hip_kv_decode_attn(weed_hip_kv_cache *cache, int32_t n_q_heads, int32_t
  * reference; results do not depend on it, only speed).  wavefronts: number of runs, 0 = as many wavefronts as the
  * device holds at once; skew_percent: how much longer than the mean the runs of a workgroup's oldest wavefronts are
  * (and the youngest shorter), negative = the built-in 16 (28 for kernel instances with three wavefronts per SIMD);
- * always_search != 0: find every run's first region by search even when all sequences have equal lengths.  The process-wide defaults are read once from the environment variables
- * WEED_HIP_DECODE_WAVES, WEED_HIP_DECODE_SKEW and WEED_HIP_DECODE_SEARCH. */
+ * always_search: bit 0: find every run's first region by search even when all sequences have equal lengths;
+ * bit 1: never let the matrix-core kernel merge its partials itself; bit 2: never let it rotate the queries itself
+ * (when every workgroup's share of the launch is a whole number of (sequence, kv head) regions -- equal sequences in
+ * power-of-two batches, the common serving shape -- one kernel does the whole call; otherwise, or with these bits, a
+ * kernel ahead rotates the queries and one behind merges the partials; the two ways differ in the rounding of the
+ * last bits).  The process-wide defaults are read once from the environment variables WEED_HIP_DECODE_WAVES,
+ * WEED_HIP_DECODE_SKEW and WEED_HIP_DECODE_SEARCH. */
 int weed_hip_kv_decode_tuning(int32_t wavefronts, int32_t skew_percent, int32_t always_search);
 
 /* weed_hip_kv_decode_attn for callers that cannot allocate device memory (code under HIP graph capture, serving loops

@@ -236,6 +236,68 @@ def test_equal_contexts_with_and_without_the_region_search(gpu, oracle):
     cache.close()
 
 
+@pytest.mark.parametrize("lloyd,d,Hkv,Hq,S,L,kb,vb,waves,rot", [
+    (True, 128, 2, 8, 4, 1024, 3, 4, 32, True),     # two regions per workgroup, four wavefronts each
+    (True, 128, 1, 4, 5, 1024, 3, 4, 20, True),     # the last workgroup holds one region of its two
+    (True, 128, 2, 16, 2, 1024, 3, 4, 16, False),   # groups of 8, no rotations
+    (False, 64, 2, 16, 4, 768, 4, 4, 48, True),     # uniform coder, head_dim 64, groups of 8, three age classes
+    (True, 128, 2, 8, 2, 768, 2, 2, 24, True),      # three wavefronts per SIMD: three age classes
+    (True, 64, 4, 4, 8, 768, 3, 3, 96, True),       # groups of one, four regions per workgroup
+    (False, 128, 1, 2, 8, 2048, 8, 8, 64, True),    # 8-bit uniform codes (no lookup tables)
+])
+def test_workgroups_that_merge_their_own_regions(gpu, oracle, lloyd, d, Hkv, Hq, S, L, kb, vb, waves, rot):
+    """When every workgroup of the matrix-core kernel holds whole regions, it rotates its queries and merges its
+    partials itself and the call is a single kernel; the same call with the kernels ahead and behind must agree to
+    rounding, and both with the checker.  Also with per-sequence prefix lengths, zero among them."""
+    import torch
+    rng = np.random.default_rng(53)
+    wl = workloads.Workload("merge", S, Hq, Hkv, d, [L] * S, kb, vb, 0, 0, 0)
+    K = rng.standard_normal((S, Hkv, L, d), dtype=np.float32)
+    V = rng.standard_normal((S, Hkv, L, d), dtype=np.float32)
+    q = rng.standard_normal((S, Hq, d), dtype=np.float32)
+    Rk, Rv = rotations(oracle, d, 7) if rot else (None, None)
+    mode = gpu.KV_LLOYDMAX if lloyd else gpu.KV_UNIFORM
+    cache = build_cache(gpu, wl, mode, K, V, rotations=(Rk, Rv) if rot else None,
+                        scales=None if lloyd else (1.0, 1.0), rotate=1 if rot else 0)
+    flags = (gpu.ATTN_ROTATE_Q | gpu.ATTN_UNROTATE_OUT) if rot else 0
+    want = checker_output(oracle, gpu, cache, wl, q, False, Rk=Rk, Rv=Rv)
+    prefix = [L - 1 - 37 * s for s in range(S)]
+    prefix[S // 2] = 0
+    wl_p = workloads.Workload("merge", S, Hq, Hkv, d, prefix, kb, vb, 0, 0, 0)
+    want_p = checker_output(oracle, gpu, cache, wl_p, q, False, Rk=Rk, Rv=Rv)
+    lens_dev = torch.tensor(prefix, dtype=torch.int32, device="cuda")
+    try:
+        gpu.profile_reset()
+        gpu.profile_enable(True)
+        gpu.decode_tuning(waves)
+        one_kernel = run_decode(gpu, cache, q, gpu.GQA_BLOCKED, flags)
+        again = run_decode(gpu, cache, q, gpu.GQA_BLOCKED, flags)
+        qd = dev(q)
+        out = torch.zeros_like(qd)
+        cache.decode_attn_prefix(lens_dev, qd, out, gqa_mapping=gpu.GQA_BLOCKED, flags=flags)
+        gpu.sync()
+        one_kernel_p = out.cpu().numpy()
+        # the merging kernel ran: the timing scope of the second kernel saw no launch
+        assert gpu.profile_read("kv_decode_attn")[1] == 3 and gpu.profile_read("kv_decode_combine")[1] == 0
+        gpu.decode_tuning(waves, separate_query=True)
+        own_merge = run_decode(gpu, cache, q, gpu.GQA_BLOCKED, flags)
+        gpu.decode_tuning(waves, separate_merge=True)
+        three_kernels = run_decode(gpu, cache, q, gpu.GQA_BLOCKED, flags)
+        assert gpu.profile_read("kv_decode_combine")[1] == 1
+    finally:
+        gpu.profile_enable(False)
+        gpu.decode_tuning()
+    assert_attn_close(three_kernels, want, "three kernels")
+    assert_attn_close(own_merge, want, "own merge")
+    assert_attn_close(one_kernel, want, "one kernel")
+    assert_attn_close(one_kernel_p, want_p, "one kernel, prefix lengths")
+    np.testing.assert_allclose(one_kernel, three_kernels, rtol=2e-5, atol=2e-6)
+    assert np.all(one_kernel_p[S // 2] == 0.0)
+    # a second call gives the same bits (the order of every sum is fixed)
+    assert np.array_equal(again, one_kernel)
+    cache.close()
+
+
 def test_edge_lengths(gpu, oracle):
     """Empty sequences give zeros; lengths 1, 63, 64, 65 around the 64-token block; an appended token changes the
     result exactly as the checker says."""

@@ -51,27 +51,6 @@ constexpr int kGMax = 8;        // query heads of one kv head handled per pass
 constexpr int kThreads = 256;
 constexpr int kChunk = 256;     // tokens per inner iteration of the generic kernel
 
-// Strides of a (sequence, head, coordinate) tensor.  With `tokens` > 1 the "heads" the kernels see are (query
-// position, head) pairs of a multi-token chunk: virtual head hv stands for head hv / tokens at position hv % tokens
-// (blocked GQA: the pairs of one KV head stay together) or for head hv % heads at position hv / heads (Weed's
-// kv = h % Hkv, which the pairs then follow without change); `ts` is the stride between query positions.
-struct Geom3 {
-    uint32_t off;
-    uint32_t s[3];
-    uint32_t tokens, heads, ts;
-    int blocked;
-};
-
-__device__ __forceinline__ uint64_t head_offset(const Geom3 &g, uint32_t hv)
-{
-    if (g.tokens <= 1U) {
-        return (uint64_t)hv * g.s[1];
-    }
-    const uint32_t h = g.blocked ? hv / g.tokens : hv % g.heads;
-    const uint32_t t = g.blocked ? hv % g.tokens : hv / g.heads;
-    return (uint64_t)h * g.s[1] + (uint64_t)t * g.ts;
-}
-
 struct DecodeParams {
     SideParams k, v;
     const int32_t *lens;
@@ -500,6 +479,8 @@ struct DecodeTuning {
     int wavefronts = 0;    // 0: as many as the device holds at once
     int skew_percent = -1; // < 0: kRunSkewPercent
     bool always_search = false;
+    bool separate_merge = false; // always merge the partials with the second kernel
+    bool separate_query = false; // always rotate the queries with the kernel ahead
 };
 DecodeTuning &decode_tuning()
 {
@@ -512,7 +493,9 @@ DecodeTuning &decode_tuning()
             v.skew_percent = std::atoi(env);
         }
         if (const char *env = std::getenv("WEED_HIP_DECODE_SEARCH")) {
-            v.always_search = std::atoi(env) != 0;
+            v.always_search = (std::atoi(env) & 1) != 0;
+            v.separate_merge = (std::atoi(env) & 2) != 0;
+            v.separate_query = (std::atoi(env) & 4) != 0;
         }
         return v;
     }();
@@ -914,7 +897,36 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
     const uint32_t n_rows = S * Hq;
     // the multi-row kernels pay off with many (sequence, head) rows; their rotation loops step by 64
     const bool many_rows = n_rows >= 512 && d % 64 == 0;
-    if (many_rows) {
+
+    // Blocks per sequence when all sequences span the same number, else 0.
+    uint32_t uniform_blocks = 0;
+    // The workgroups of the matrix-core kernel merge their regions themselves (wg_regions regions each, else 0) when
+    // every workgroup's share of the block list is a whole number of regions and no run straddles a region boundary:
+    // equal sequences of nb blocks each, nb a multiple of one cycle of the age classes' runs, and a workgroup's blocks
+    // a multiple of nb.  They then also rotate their regions' queries themselves, and the call is ONE kernel.
+    uint32_t wg_regions = 0;
+    bool fused_query = false;
+    if (use_mfma && total_blocks) {
+        uniform_blocks = ((uint32_t)c->lens[0] + 63u) >> 6;
+        for (int32_t l : c->lens) {
+            if ((((uint32_t)l + 63u) >> 6) != uniform_blocks || decode_tuning().always_search) {
+                uniform_blocks = 0;
+                break;
+            }
+        }
+        const uint32_t gp = pass_heads <= 4 ? 4u : (pass_heads <= 8 ? 8u : 16u);
+        const uint32_t nb = uniform_blocks, cycle = run_classes(runs) * runs.unit_blocks;
+        const uint32_t wg_blocks = runs.waves * runs.unit_blocks;
+        if (mfma_decode_merges(gp, d) && nb != 0 && nb % cycle == 0 && wg_blocks % nb == 0 &&
+            !decode_tuning().separate_merge) {
+            wg_regions = wg_blocks / nb;
+            fused_query = wg_regions * pass_heads <= kMfmaQueryRows && !decode_tuning().separate_query;
+        }
+    }
+    const bool fused_merge = wg_regions != 0;
+    if (fused_query) {
+        // (nothing runs ahead of the matrix-core kernel)
+    } else if (many_rows) {
         prep_q_rows_kernel<<<(n_rows + kRowsPerWg - 1) / kRowsPerWg + (use_mfma ? 1 : 0), 256, 0, stream()>>>(
             q_dev, qg, Hq, d, d_real, n_rows, c->k.rot_t, rot_q ? 1 : 0, q_rot, q_hi, q_lo, q_scale, q_sum, c->lens_dev, S,
             use_mfma ? blk_off : nullptr);
@@ -946,13 +958,9 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         mp.blk_off = blk_off;
         mp.n_seq = S;
         mp.total_blocks = total_blocks;
-        mp.uniform_blocks = ((uint32_t)c->lens[0] + 63u) >> 6;
-        for (int32_t l : c->lens) {
-            if ((((uint32_t)l + 63u) >> 6) != mp.uniform_blocks || decode_tuning().always_search) {
-                mp.uniform_blocks = 0;
-                break;
-            }
-        }
+        mp.uniform_blocks = uniform_blocks;
+        mp.merge = MfmaMerge{ wg_regions, d_real, out_dev, og, c->v.rot, unrot ? 1 : 0 };
+        mp.query = MfmaQuery{ fused_query ? q_dev : nullptr, qg, c->k.rot_t, rot_q ? 1 : 0 };
         mp.runs = runs;
         mp.max_slots = n_splits;
         mp.group_total = G;
@@ -983,7 +991,7 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         decode_generic_kernel<<<dim3(n_splits, Hkv, S), kThreads, 0, stream()>>>(p);
         WEED_HIP_LAUNCH_CHECK();
     }
-    {
+    if (!fused_merge) {
         ProfileScope prof("kv_decode_combine", timed);
         const SlotGeom sg = { use_mfma ? blk_off : nullptr, Hkv, G, runs,
                               gqa_mapping == WEED_HIP_GQA_BLOCKED ? 1 : 0 };
@@ -1014,7 +1022,9 @@ extern "C" int weed_hip_kv_decode_tuning(int32_t wavefronts, int32_t skew_percen
     DecodeTuning &t = decode_tuning();
     t.wavefronts = std::max(0, wavefronts);
     t.skew_percent = skew_percent;
-    t.always_search = always_search != 0;
+    t.always_search = (always_search & 1) != 0;
+    t.separate_merge = (always_search & 2) != 0;
+    t.separate_query = (always_search & 4) != 0;
     return WEED_HIP_OK;
 }
 

@@ -99,6 +99,74 @@ inline uint32_t mfma_table_word(uint32_t i, uint32_t wk, uint32_t wv, const uint
     return e < (1u << (2 * w)) ? ((uint32_t)lv[e & mask] | ((uint32_t)lv[(e >> w) & mask] << 16)) : 0u;
 }
 
+// Strides of a (sequence, head, coordinate) tensor.  With `tokens` > 1 the "heads" the kernels see are (query
+// position, head) pairs of a multi-token chunk: virtual head hv stands for head hv / tokens at position hv % tokens
+// (blocked GQA: the pairs of one KV head stay together) or for head hv % heads at position hv / heads (Weed's
+// kv = h % Hkv, which the pairs then follow without change); `ts` is the stride between query positions.
+struct Geom3 {
+    uint32_t off;
+    uint32_t s[3];
+    uint32_t tokens, heads, ts;
+    int blocked;
+};
+
+__device__ __forceinline__ uint64_t head_offset(const Geom3 &g, uint32_t hv)
+{
+    if (g.tokens <= 1U) {
+        return (uint64_t)hv * g.s[1];
+    }
+    const uint32_t h = g.blocked ? hv / g.tokens : hv % g.heads;
+    const uint32_t t = g.blocked ? hv % g.tokens : hv / g.heads;
+    return (uint64_t)h * g.s[1] + (uint64_t)t * g.ts;
+}
+
+// Merge inside the matrix-core kernel.  When every workgroup's share of the block list is a whole number of regions
+// and no run straddles a region boundary (`wg_regions` regions per workgroup, each worked on by
+// waves / wg_regions wavefronts), the wavefronts leave their partials in LDS, and the workgroup merges them,
+// un-rotates the result and writes the output rows itself: no partials in memory, no second kernel.
+// `wg_regions` 0: the kernel writes the partials to memory and a second kernel merges them.
+struct MfmaMerge {
+    uint32_t wg_regions;
+    uint32_t d_real;   // coordinates the caller's rows have (<= the stored head_dim)
+    float *out;        // attention output
+    Geom3 og;          // its strides
+    const float *rv;   // V rotation, row-major [d][d]: out[t] = sum_j o[j] * rv[t + d * j]
+    int unrotate;
+};
+// Query rotation inside the matrix-core kernel, for launches whose workgroups merge (MfmaMerge): a workgroup rotates,
+// scales and splits the queries of its own regions' heads (at most kMfmaQueryRows rows) before its first block arrives,
+// so that no kernel runs ahead of this one.  `q` null: the kernel reads q_hi / q_lo / q_scale / q_sum from memory.
+struct MfmaQuery {
+    const float *q;      // the caller's queries
+    Geom3 qg;            // their strides
+    const float *rot_t;  // K rotation, transposed: q_rot[j] = sum_i q[i] * rot_t[j + d * i]
+    int rotate;          // 0: the queries are rotated already
+};
+constexpr uint32_t kMfmaQueryRows = 32;
+
+// Instances that can merge: groups of up to 8 heads at head_dim 64 or 128.
+constexpr bool mfma_decode_merges(uint32_t gp, uint32_t d) { return gp <= 8 && (d == 64u || d == 128u); }
+// Rows (region, head) that one pass of the merge takes, threads of its un-rotation, and its LDS behind the tables:
+// the wavefronts' partials [waves][gp][d + 2], the merged rows [rows][d], the un-rotation's partial sums
+// [threads / d][rows][d].
+constexpr uint32_t kMfmaMergeRows = 8;
+constexpr uint32_t kMfmaMergeThreads = 512;
+// The query rotation works in the same LDS before the first block: the raw queries [kMfmaQueryRows][d] and the
+// rotation's partial sums [threads / d][rows][d] where the partials will be, and its results (fp16 halves
+// [kMfmaQueryRows][d] each, a scale and a sum per row) where the merged rows and the un-rotation's sums will be.
+constexpr uint32_t mfma_merge_partials_words(uint32_t waves, uint32_t gp, uint32_t d)
+{
+    const uint32_t partials = waves * gp * (d + 2u), query = kMfmaQueryRows * d + kMfmaMergeThreads * kMfmaMergeRows;
+    return partials > query ? partials : query;
+}
+constexpr uint32_t mfma_merge_lds_bytes(uint32_t waves, uint32_t gp, uint32_t d)
+{
+    return 4u * (mfma_merge_partials_words(waves, gp, d) + kMfmaMergeRows * d + kMfmaMergeThreads * kMfmaMergeRows);
+}
+static_assert(kMfmaQueryRows * 128u + 2u * kMfmaQueryRows <= kMfmaMergeRows * 128u + kMfmaMergeThreads * kMfmaMergeRows &&
+                  kMfmaQueryRows * 64u + 2u * kMfmaQueryRows <= kMfmaMergeRows * 64u + kMfmaMergeThreads * kMfmaMergeRows,
+              "the query halves, scales and sums fit where the merged rows and the un-rotation's sums will be");
+
 // Kernel arguments.  What a wavefront needs before it can request its first block comes first, so that it arrives
 // with the first kernel-argument fetches.
 struct MfmaParams {
@@ -131,6 +199,8 @@ struct MfmaParams {
     const float *q_scale;   // [n_seq][Hq] power of two the query was divided by
     const float *q_sum;     // [n_seq][Hq] sum of the scaled query (for the uniform coder's offset term)
     float *partials;        // [n_seq][Hq][max_slots][d + 2]: m (log2 units), l, o[d]
+    MfmaMerge merge;
+    MfmaQuery query;
 };
 
 bool mfma_decode_supported(uint32_t d, uint32_t wk, uint32_t wv, uint32_t G);

@@ -261,13 +261,40 @@ __device__ __forceinline__ uint32_t q_head_of(const MfmaParams &p, uint32_t kvh,
     return p.blocked ? kvh * p.group_total + p.head_first + x : (p.head_first + x) * p.Hkv + kvh;
 }
 
+__device__ __forceinline__ float wave_max64(float v)
+{
+    for (int o = 32; o > 0; o >>= 1) {
+        v = fmaxf(v, __shfl_xor(v, o));
+    }
+    return v;
+}
+__device__ __forceinline__ float wave_sum64(float v)
+{
+    for (int o = 32; o > 0; o >>= 1) {
+        v += __shfl_xor(v, o);
+    }
+    return v;
+}
+
+// A load through a buffer descriptor: one descriptor, the lane's 32-bit byte offset and an offset that is the same in
+// every lane, so that a batch of loads needs no address register pair per load.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_of(const float *base, uint32_t bytes)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(base), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ float buffer_f32(__amdgpu_buffer_rsrc_t r, uint32_t lane_off, uint32_t uniform_off)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)lane_off, (int)uniform_off, 0));
+}
+
 // Bank mask (4-lane banks of a row) of the lanes [GP*i, GP*i + GP).
 template <int GP, int I> constexpr int bank_mask_of() { return ((1 << (GP / 4)) - 1) << (I * GP / 4); }
 
 // GP = number of query-head columns kept per score tile (the group size rounded up to 4, 8 or 16).  The Q.K^T
 // instruction always produces 16 columns; with GP < 16 the useful columns of 16/GP tiles are merged into one register
 // set before the softmax, so the exponentials and the fp16 splitting run on full registers.
-template <int D, int WK, int WV, int GP, bool LLOYD>
+// WGM: the workgroups merge their regions themselves (see MfmaMerge); every wavefront then has at most one segment.
+template <int D, int WK, int WV, int GP, bool LLOYD, bool WGM>
 __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) decode_mfma_kernel(MfmaParams p)
 {
     constexpr int kWaves = (int)mfma_decode_waves_per_wg(GP, D, WK, WV);
@@ -289,10 +316,11 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     //      16 bytes per thread and step.  The image is requested first thing and stored after the wavefront has
     //      requested its first block and query, so that those loads travel meanwhile.  Every wavefront of the
     //      workgroup calls build_tables exactly once (it contains a barrier). ----
-    // The arguments span four 64-byte lines of kernel-argument memory, each a miss of its own when first touched.
-    // Naming one value of every line here makes the compiler fetch all four at once instead of one after the other
+    // The arguments span six 64-byte lines of kernel-argument memory, each a miss of its own when first touched.
+    // Naming one value of every line here makes the compiler fetch all of them at once instead of one after the other
     // as the prologue gets to them.
-    asm volatile("" ::"s"(p.total_blocks), "s"(p.v.fields), "s"(p.table_image), "s"(p.q_hi));
+    asm volatile("" ::"s"(p.total_blocks), "s"(p.v.fields), "s"(p.table_image), "s"(p.q_hi), "s"(p.merge.out),
+                 "s"(p.query.q));
     constexpr uint32_t kThreads = 64 * kWaves;
     constexpr uint32_t kImgVecs = ROWS * (kTableRowBytes / 16);
     constexpr uint32_t kImgLoads = (kImgVecs + kThreads - 1) / kThreads;
@@ -330,13 +358,179 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
         __builtin_amdgcn_readfirstlane(blockIdx.x * kWaves + run_position_of_wave(p.runs, wave));
     uint32_t g0 = __builtin_amdgcn_readfirstlane(run_begin(p.runs, unit));
     const uint32_t g1 = min(g0 + run_len(p.runs, (unit % kWaves) % run_classes(p.runs)), p.total_blocks);
-    if (g0 >= g1) {
-        build_tables();
-        return;
+    // ---- merge inside the kernel (see MfmaMerge): LDS behind the tables, and this thread's share of the rotation ----
+    static_assert(!WGM || mfma_decode_merges(GP, D), "this instance cannot merge");
+    constexpr bool kCanMerge = WGM;
+    constexpr uint32_t NG = kMfmaMergeThreads / D; // groups of source coordinates of the un-rotation
+    constexpr uint32_t JPG = WGM ? D / (NG ? NG : 1) : 1; // source coordinates per group
+    float *const part_s = reinterpret_cast<float *>(lds) + ROWS * (kTableRowBytes / 4); // [position][GP][D + 2]
+    float xrot[kCanMerge ? JPG : 1];
+    auto request_rotation = [&]() {
+        // thread (group jg, coordinate t) of the first kMfmaMergeThreads takes rv[jg * JPG + u][t], u < JPG; the group
+        // is the same in all lanes of a wavefront
+        if constexpr (kCanMerge) {
+            if (p.merge.unrotate && tid < kMfmaMergeThreads) {
+                const __amdgpu_buffer_rsrc_t rot = buffer_of(p.merge.rv, 4 * D * D);
+                const uint32_t t = tid % D, jg = tid / D;
+#pragma unroll
+                for (uint32_t u = 0; u < JPG; ++u) {
+                    xrot[u] = buffer_f32(rot, 4 * (jg * JPG * D + t), 4 * D * u);
+                }
+            }
+        }
+    };
+    // With two wavefronts per SIMD the registers have room for the rotation elements all along: they are requested
+    // here; with three, when the wavefront is through with its blocks.
+    constexpr bool kEarlyRotation = WGM && kWaves == 8;
+    if constexpr (kEarlyRotation) {
+        request_rotation();
     }
-    uint32_t seq;
+    // ---- query rotation inside the kernel (see MfmaQuery).  Row (region ri of the workgroup, head slot hs) has index
+    //      ri * G + hs.  Requested here: this thread's share of the K rotation and of the raw queries. ----
+    constexpr uint32_t QPT = WGM ? (kMfmaQueryRows * D + kThreads - 1) / kThreads : 1; // raw query elements per thread
+    constexpr uint32_t PW = mfma_merge_partials_words(kWaves, GP, D);
+    float *const qraw_s = part_s;                              // [rows][D]
+    float *const qred_s = part_s + kMfmaQueryRows * D;         // [NG][kMfmaMergeRows][D]
+    uint16_t *const qh_s = reinterpret_cast<uint16_t *>(part_s + PW); // [rows][D] fp16 high halves
+    uint16_t *const ql_s = qh_s + kMfmaQueryRows * D;                 // [rows][D] low halves
+    float *const qscale_s = part_s + PW + kMfmaQueryRows * D;         // [rows]
+    float *const qsum_s = qscale_s + kMfmaQueryRows;                  // [rows]
+    const bool fused_q = WGM && p.query.q != nullptr;
+    const uint32_t wg_rows = WGM ? p.merge.wg_regions * p.G : 0;
+    const uint32_t wg_region0 = WGM ? blockIdx.x * p.merge.wg_regions : 0;
+    float xq[WGM ? JPG : 1], qr[QPT];
+    if constexpr (WGM) {
+        if (fused_q) {
+            if (p.query.rotate && tid < kMfmaMergeThreads) {
+                const __amdgpu_buffer_rsrc_t rot = buffer_of(p.query.rot_t, 4 * D * D);
+                const uint32_t t = tid % D, ig = tid / D;
+#pragma unroll
+                for (uint32_t u = 0; u < JPG; ++u) {
+                    xq[u] = buffer_f32(rot, 4 * (ig * JPG * D + t), 4 * D * u);
+                }
+            }
+            const uint32_t n_regions = p.n_seq * p.Hkv;
+            // element e = tid + i * kThreads of the rows: its row is the same in all lanes of a wavefront (kThreads is
+            // a multiple of D), so the row's address arithmetic is scalar
+            static_assert(kThreads % D == 0 && D % 64 == 0, "a wavefront stays inside one row");
+            const uint32_t row_of_wave = __builtin_amdgcn_readfirstlane(tid / D), j = tid % D;
+#pragma unroll
+            for (uint32_t i = 0; i < QPT; ++i) {
+                const uint32_t row = row_of_wave + i * (kThreads / D);
+                const uint32_t ri = row / p.G, hs = row - ri * p.G, region = wg_region0 + ri;
+                float v = 0.0f;
+                if (row < wg_rows && region < n_regions) {
+                    const uint32_t s_ = region / p.Hkv, kv_ = region - s_ * p.Hkv;
+                    const float *qrow = p.query.q + (uint64_t)p.query.qg.off + (uint64_t)s_ * p.query.qg.s[0] +
+                                        head_offset(p.query.qg, q_head_of(p, kv_, hs));
+                    if (j < p.merge.d_real) {
+                        v = qrow[(uint64_t)j * p.query.qg.s[2]];
+                    }
+                }
+                qr[i] = v;
+            }
+        }
+    }
+    // The workgroup's queries: rotated by all threads (thread (group ig, coordinate t) sums its JPG source coordinates
+    // for every row, the groups' sums are added in a fixed order), then one wavefront per row scales, normalises and
+    // splits the row as the stand-alone kernel does.  Contains the tables' barrier; every wavefront calls it once.
+    auto rotate_queries = [&]() {
+        if constexpr (WGM) {
+#pragma unroll
+            for (uint32_t i = 0; i < QPT; ++i) {
+                const uint32_t e = tid + i * kThreads;
+                if (e < kMfmaQueryRows * D) {
+                    qraw_s[e] = qr[i];
+                }
+            }
+            build_tables(); // (its barrier also makes the raw queries visible)
+            if constexpr (ROWS == 0) {
+                __syncthreads(); // (no tables, no barrier of theirs)
+            }
+            for (uint32_t r0 = 0; r0 < wg_rows; r0 += kMfmaMergeRows) {
+                if (p.query.rotate) {
+                    if (tid < kMfmaMergeThreads) {
+                        const uint32_t t = tid % D, ig = tid / D;
+#pragma unroll
+                        for (uint32_t rr = 0; rr < kMfmaMergeRows; ++rr) {
+                            float acc = 0.0f;
+                            const float4v *qrow = reinterpret_cast<const float4v *>(qraw_s + (r0 + rr) * D + ig * JPG);
+#pragma unroll
+                            for (uint32_t u4 = 0; u4 < JPG / 4; ++u4) {
+                                const float4v qv = qrow[u4];
+#pragma unroll
+                                for (uint32_t i = 0; i < 4; ++i) {
+                                    acc = fmaf(qv[i], xq[4 * u4 + i], acc);
+                                }
+                            }
+                            qred_s[(ig * kMfmaMergeRows + rr) * D + t] = acc;
+                        }
+                    }
+                    __syncthreads();
+                }
+                if (wave < kMfmaMergeRows && r0 + wave < wg_rows) {
+                    const uint32_t row = r0 + wave;
+                    constexpr uint32_t CPL = D / 64;
+                    float a[CPL];
+                    const float k = 1.4426950408889634f / sqrtf((float)p.merge.d_real);
+                    float mx = 0.0f, sum = 0.0f;
+#pragma unroll
+                    for (uint32_t cc = 0; cc < CPL; ++cc) {
+                        const uint32_t j = lane + 64 * cc;
+                        float v;
+                        if (p.query.rotate) {
+                            v = 0.0f;
+#pragma unroll
+                            for (uint32_t ig = 0; ig < NG; ++ig) {
+                                v += qred_s[(ig * kMfmaMergeRows + wave) * D + j];
+                            }
+                        } else {
+                            v = qraw_s[row * D + j];
+                        }
+                        a[cc] = v;
+                        const float qc = v * k;
+                        mx = fmaxf(mx, fabsf(qc));
+                        sum += qc;
+                    }
+                    mx = wave_max64(mx);
+                    sum = wave_sum64(sum);
+                    int e = 0;
+                    (void)frexpf(mx, &e);
+                    e = e < -100 ? -100 : (e > 100 ? 100 : e);
+                    const float inv = ldexpf(1.0f, -e);
+#pragma unroll
+                    for (uint32_t cc = 0; cc < CPL; ++cc) {
+                        const uint32_t j = lane + 64 * cc;
+                        const float qn = a[cc] * k * inv;
+                        const _Float16 hi = (_Float16)qn;
+                        const _Float16 lo = (_Float16)(qn - (float)hi);
+                        qh_s[row * D + j] = __builtin_bit_cast(uint16_t, hi);
+                        ql_s[row * D + j] = __builtin_bit_cast(uint16_t, lo);
+                    }
+                    if (lane == 0) {
+                        qscale_s[row] = ldexpf(1.0f, e);
+                        qsum_s[row] = sum;
+                    }
+                }
+                __syncthreads(); // the rows are there; the partial sums may be overwritten
+            }
+        }
+    };
+    const bool has_blocks = g0 < g1;
+    if (g0 >= g1 && !tables_ready) {
+        // a wavefront without blocks
+        if (fused_q) {
+            rotate_queries();
+        } else {
+            build_tables();
+        }
+        tables_ready = true;
+    }
+    uint32_t seq = 0;
     const uint32_t uniform_nb = p.uniform_blocks;
-    if (uniform_nb) {
+    if (g0 >= g1) {
+        // (nothing to find)
+    } else if (uniform_nb) {
         seq = g0 / (uniform_nb * p.Hkv);
     } else {
         // largest s with blk_off[s] * Hkv <= g0 (sequences without tokens share their offset with the next one):
@@ -356,9 +550,11 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     const uint32_t seq_first = uniform_nb ? seq * uniform_nb : p.blk_off[seq];
     // blocks the cached length of this sequence spans
     const uint32_t nb_cap = uniform_nb ? uniform_nb : p.blk_off[seq + 1] - seq_first;
-    if (nb_cap == 0) {
-        ++seq;
-        continue;
+    if constexpr (!WGM) {
+        if (nb_cap == 0) {
+            ++seq;
+            continue;
+        }
     }
     const uint32_t rel = g0 - seq_first * p.Hkv;
     const uint32_t kvh = rel / nb_cap;
@@ -425,7 +621,24 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     constexpr bool PACKED = GP <= 8;
     constexpr int NQ = PACKED ? 1 : 2;
     half8 qop[NQ][KS];
-    {
+    if (fused_q) {
+        if constexpr (WGM) {
+            rotate_queries(); // (with the tables' barrier)
+            tables_ready = true;
+            const uint32_t col_head = c % GP, col_part = c / GP; // (PACKED: merging instances have GP <= 8)
+            const bool col_ok = col_head < p.G && col_part < 2;
+            const uint32_t row = ((uint32_t)region - wg_region0) * p.G + (col_ok ? col_head : 0);
+            const uint16_t *src = (col_part ? ql_s : qh_s) + row * D + g * (D / 4);
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                uint4v v = { 0, 0, 0, 0 };
+                if (col_ok) {
+                    v = *reinterpret_cast<const uint4v *>(src + 8 * ks);
+                }
+                qop[0][ks] = __builtin_bit_cast(half8, v);
+            }
+        }
+    } else {
         const uint32_t col_head = PACKED ? c % GP : c;
         const uint32_t col_part = PACKED ? c / GP : 0; // 0: high half, 1: low half, above: unused column
         const bool col_ok = col_head < p.G && col_part < 2;
@@ -453,8 +666,17 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     const uint32_t pair = p.head_first + hc; // index of the (position, head) pair among those of the KV head
     const uint32_t hidden = (hidden_max && head_ok) ? hidden_max - (p.blocked ? pair % p.q_tokens : pair / p.real_group) : 0U;
     const uint32_t qh_c = head_ok ? q_head_of(p, kvh, hc) : 0;
-    const float qscale = head_ok ? p.q_scale[(uint64_t)seq * p.Hq + qh_c] : 0.0f;
-    const float betaq = head_ok ? p.k.beta * p.q_sum[(uint64_t)seq * p.Hq + qh_c] : 0.0f;
+    float qscale = 0.0f, betaq = 0.0f;
+    if (fused_q) {
+        const uint32_t row = ((uint32_t)region - wg_region0) * p.G + hc;
+        if (head_ok) {
+            qscale = qscale_s[row];
+            betaq = p.k.beta * qsum_s[row];
+        }
+    } else if (head_ok) {
+        qscale = p.q_scale[(uint64_t)seq * p.Hq + qh_c];
+        betaq = p.k.beta * p.q_sum[(uint64_t)seq * p.Hq + qh_c];
+    }
 
     // ---- The running maximum is only raised when a block exceeds it by more than 2^kSlack, so most blocks skip the
     //      rescaling of the output accumulators; probabilities may therefore reach 2^kSlack.  `ep` is the exponent
@@ -716,61 +938,169 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
         }
     }
 
-    // ---- this segment's un-normalised partial (m, l, o[d]) per query head, straight to global memory ----
-    const float l_head = head_sum<GP>(l_run) * unscale; // every lane of a head now holds its denominator
-    float lrow[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        lrow[r] = __shfl(l_head, (int)(4 * g + r));
-    }
+    // ---- this segment's un-normalised partial (m, l, o[d]) per query head: to LDS when the workgroup merges (every
+    //      wavefront then has one segment, and its position in the workgroup is its slot), else straight to global
+    //      memory ----
     constexpr int PS = D + 2;
-    const float o_mul = unscale * (lloyd ? 1.0f : p.v.alpha_const);
-    if constexpr (PACKED) {
-        // rows [GP, 2GP) hold the low-half products of heads [0, GP): they sit GP/4 lane rows further up
+    auto leave_partial = [&](auto to_lds) {
+        constexpr bool TO_LDS = decltype(to_lds)::value;
+        const float l_head = head_sum<GP>(l_run) * unscale; // every lane of a head now holds its denominator
+        float lrow[4];
 #pragma unroll
-        for (int jb = 0; jb < JB; ++jb) {
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                O[jb][r] += __shfl_down(O[jb][r], 4 * GP);
-            }
+        for (int r = 0; r < 4; ++r) {
+            lrow[r] = __shfl(l_head, (int)(4 * g + r));
         }
-    }
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const uint32_t hs = 4 * g + r;
-        if (hs < p.G) {
-            const uint32_t head = q_head_of(p, kvh, hs);
-            float *dst = p.partials + (((uint64_t)seq * p.Hq + head) * p.max_slots + slot) * PS;
+        const float o_mul = unscale * (lloyd ? 1.0f : p.v.alpha_const);
+        if constexpr (PACKED) {
+            // rows [GP, 2GP) hold the low-half products of heads [0, GP): they sit GP/4 lane rows further up
 #pragma unroll
             for (int jb = 0; jb < JB; ++jb) {
-                // uniform coder: value = step * (code + 0.5) + lo, so add lo * sum(p)
-                dst[2 + 16 * jb + c] = fmaf(O[jb][r], o_mul, p.v.beta * lrow[r]);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    O[jb][r] += __shfl_down(O[jb][r], 4 * GP);
+                }
             }
         }
-    }
-    if (g == 0 && c < p.G) {
-        // lane c of row 0 holds head c (c < GP)
-        const uint32_t head = q_head_of(p, kvh, c);
-        float *dst = p.partials + (((uint64_t)seq * p.Hq + head) * p.max_slots + slot) * PS;
-        dst[0] = m_run;
-        dst[1] = l_head;
+        float *const mine = part_s + run_position_of_wave(p.runs, wave) * (GP * PS);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const uint32_t hs = 4 * g + r;
+            if (hs < p.G) {
+                float *dst = TO_LDS ? mine + hs * PS
+                                    : p.partials + (((uint64_t)seq * p.Hq + q_head_of(p, kvh, hs)) * p.max_slots + slot) * PS;
+#pragma unroll
+                for (int jb = 0; jb < JB; ++jb) {
+                    // uniform coder: value = step * (code + 0.5) + lo, so add lo * sum(p)
+                    dst[2 + 16 * jb + c] = fmaf(O[jb][r], o_mul, p.v.beta * lrow[r]);
+                }
+            }
+        }
+        if (g == 0 && c < p.G) {
+            // lane c of row 0 holds head c (c < GP)
+            float *dst = TO_LDS ? mine + c * PS
+                                : p.partials + (((uint64_t)seq * p.Hq + q_head_of(p, kvh, c)) * p.max_slots + slot) * PS;
+            dst[0] = m_run;
+            dst[1] = l_head;
+        }
+    };
+    if constexpr (WGM) {
+        if constexpr (!kEarlyRotation) {
+            request_rotation(); // on its way while the partial is put together
+        }
+        leave_partial(std::true_type{});
+        break; // (the only segment: for the compiler this is no loop, so nothing is carried around it)
+    } else {
+        leave_partial(std::false_type{});
     }
     if (kvh + 1 == p.Hkv && b0 + seg == nb_cap) {
         ++seq;
     }
     } // segments
+
+    // ---- the workgroup's merge: rows (region, head) in passes of kMfmaMergeRows ----
+    if constexpr (WGM) {
+        if (!kEarlyRotation && !has_blocks) {
+            request_rotation(); // (the others did so before they left their partial)
+        }
+        constexpr int PS = D + 2;
+        constexpr uint32_t RP = kMfmaMergeRows;
+        float *const o_s = part_s + PW;               // [RP][D] merged, normalised rows
+        float *const red_s = o_s + RP * D;            // [NG][RP][D] partial sums of the un-rotation
+        const uint32_t slots = kWaves / p.merge.wg_regions;
+        const uint32_t rows = p.merge.wg_regions * p.G;
+        const uint32_t region0 = blockIdx.x * p.merge.wg_regions, n_regions = p.n_seq * p.Hkv;
+        __syncthreads(); // every wavefront's partial is in LDS (and nobody reads the tables any more)
+        for (uint32_t r0 = 0; r0 < rows; r0 += RP) {
+            // (the row of element e is the same in all lanes of a wavefront: kThreads is a multiple of D)
+            const uint32_t rr_of_wave = __builtin_amdgcn_readfirstlane(tid / D);
+            for (uint32_t rr = rr_of_wave; rr < RP; rr += kThreads / D) {
+                const uint32_t e = rr * D + tid % D, j = tid % D, row = r0 + rr;
+                float v = 0.0f;
+                if (row < rows) {
+                    const uint32_t ri = row / p.G, hs = row - ri * p.G;
+                    const float *first = part_s + (ri * slots * GP + hs) * PS; // slot k: + k * GP * PS
+                    float mx = -INFINITY;
+                    for (uint32_t k = 0; k < slots; ++k) {
+                        mx = fmaxf(mx, first[k * (GP * PS)]);
+                    }
+                    float den = 0.0f, acc = 0.0f;
+                    for (uint32_t k = 0; k < slots; ++k) {
+                        const float m = first[k * (GP * PS)];
+                        const float w = (m == -INFINITY) ? 0.0f : exp2f(m - mx);
+                        den = fmaf(w, first[k * (GP * PS) + 1], den);
+                        acc = fmaf(w, first[k * (GP * PS) + 2 + j], acc);
+                    }
+                    v = den > 0.0f ? acc / den : 0.0f;
+                }
+                o_s[e] = v;
+            }
+            __syncthreads();
+            if (p.merge.unrotate) {
+                if (tid < kMfmaMergeThreads) {
+                    const uint32_t t = tid % D, jg = tid / D;
+#pragma unroll
+                    for (uint32_t rr = 0; rr < RP; ++rr) {
+                        float acc = 0.0f;
+                        // (JPG is a multiple of 4; the merged row is read four coordinates at a time, every lane the
+                        // same address)
+                        const float4v *orow = reinterpret_cast<const float4v *>(o_s + rr * D + jg * JPG);
+#pragma unroll
+                        for (uint32_t u4 = 0; u4 < JPG / 4; ++u4) {
+                            const float4v ov = orow[u4];
+#pragma unroll
+                            for (uint32_t i = 0; i < 4; ++i) {
+                                acc = fmaf(ov[i], xrot[4 * u4 + i], acc);
+                            }
+                        }
+                        red_s[(jg * RP + rr) * D + t] = acc;
+                    }
+                }
+                __syncthreads();
+            }
+            for (uint32_t rr = rr_of_wave; rr < RP; rr += kThreads / D) {
+                const uint32_t e = rr * D + tid % D, t = tid % D, row = r0 + rr;
+                const uint32_t ri = row / p.G, hs = row - ri * p.G;
+                if (row < rows && region0 + ri < n_regions && t < p.merge.d_real) {
+                    float v;
+                    if (p.merge.unrotate) {
+                        v = 0.0f;
+#pragma unroll
+                        for (uint32_t jg = 0; jg < NG; ++jg) {
+                            v += red_s[(jg * RP + rr) * D + t];
+                        }
+                    } else {
+                        v = o_s[e];
+                    }
+                    const uint32_t region = region0 + ri;
+                    const uint32_t s_ = region / p.Hkv, kv_ = region - s_ * p.Hkv;
+                    p.merge.out[(uint64_t)p.merge.og.off + (uint64_t)s_ * p.merge.og.s[0] +
+                                head_offset(p.merge.og, q_head_of(p, kv_, hs)) + (uint64_t)t * p.merge.og.s[2]] = v;
+                }
+            }
+            __syncthreads(); // before the next pass overwrites the rows
+        }
+    }
 }
 
 template <int D, int WK, int WV, int GP, bool LLOYD> int launch_gp(const MfmaParams &p, hipStream_t s)
 {
-    constexpr size_t smem = (size_t)table_rows<WK, WV>() * kTableRowBytes;
     constexpr uint32_t waves = mfma_decode_waves_per_wg(GP, D, WK, WV);
+    constexpr size_t smem = (size_t)table_rows<WK, WV>() * kTableRowBytes;
+    constexpr size_t smem_merging = smem + (mfma_decode_merges(GP, D) ? mfma_merge_lds_bytes(waves, GP, D) : 0u);
+    static_assert(smem_merging <= 160u * 1024u, "tables and merge area exceed a compute unit's LDS");
     // once per instance and process, whichever host thread gets here first (the others wait for it)
     static std::once_flag configured;
     static hipError_t config_status = hipSuccess;
+    constexpr bool kMerges = mfma_decode_merges(GP, D);
     std::call_once(configured, [] {
-        config_status = hipFuncSetAttribute((const void *)decode_mfma_kernel<D, WK, WV, GP, LLOYD>,
+        config_status = hipFuncSetAttribute((const void *)decode_mfma_kernel<D, WK, WV, GP, LLOYD, false>,
                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if constexpr (kMerges) {
+            if (config_status == hipSuccess) {
+                config_status = hipFuncSetAttribute((const void *)decode_mfma_kernel<D, WK, WV, GP, LLOYD, true>,
+                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_merging);
+            }
+        }
     });
     WEED_HIP_CHECK(config_status);
     if (p.runs.waves != waves) {
@@ -778,7 +1108,16 @@ template <int D, int WK, int WV, int GP, bool LLOYD> int launch_gp(const MfmaPar
                     p.runs.waves, waves);
     }
     const uint32_t wg_blocks = waves * p.runs.unit_blocks;
-    decode_mfma_kernel<D, WK, WV, GP, LLOYD><<<(p.total_blocks + wg_blocks - 1) / wg_blocks, 64 * waves, smem, s>>>(p);
+    const uint32_t grid = (p.total_blocks + wg_blocks - 1) / wg_blocks;
+    if (p.merge.wg_regions != 0) {
+        if constexpr (kMerges) {
+            decode_mfma_kernel<D, WK, WV, GP, LLOYD, true><<<grid, 64 * waves, smem_merging, s>>>(p);
+        } else {
+            return fail(WEED_HIP_EDEVICE, "decode_mfma: this kernel instance cannot merge its partials itself");
+        }
+    } else {
+        decode_mfma_kernel<D, WK, WV, GP, LLOYD, false><<<grid, 64 * waves, smem, s>>>(p);
+    }
     WEED_HIP_LAUNCH_CHECK();
     return WEED_HIP_OK;
 }
