@@ -393,7 +393,7 @@ def main():
         # the same step as three kernels (query rotation, attention, merge), for comparison
         separate = None
         if one_kernel:
-            capi.decode_tuning(separate_merge=True)
+            capi.decode_tuning(separate_merge=True, separate_query=True)
             try:
                 for _ in range(args.warmup):
                     step()

@@ -282,13 +282,16 @@ def test_workgroups_that_merge_their_own_regions(gpu, oracle, lloyd, d, Hkv, Hq,
         gpu.decode_tuning(waves, separate_query=True)
         own_merge = run_decode(gpu, cache, q, gpu.GQA_BLOCKED, flags)
         gpu.decode_tuning(waves, separate_merge=True)
+        own_queries = run_decode(gpu, cache, q, gpu.GQA_BLOCKED, flags)
+        gpu.decode_tuning(waves, separate_merge=True, separate_query=True)
         three_kernels = run_decode(gpu, cache, q, gpu.GQA_BLOCKED, flags)
-        assert gpu.profile_read("kv_decode_combine")[1] == 1
+        assert gpu.profile_read("kv_decode_combine")[1] == 2
     finally:
         gpu.profile_enable(False)
         gpu.decode_tuning()
     assert_attn_close(three_kernels, want, "three kernels")
     assert_attn_close(own_merge, want, "own merge")
+    assert_attn_close(own_queries, want, "own queries")
     assert_attn_close(one_kernel, want, "one kernel")
     assert_attn_close(one_kernel_p, want_p, "one kernel, prefix lengths")
     np.testing.assert_allclose(one_kernel, three_kernels, rtol=2e-5, atol=2e-6)

@@ -507,12 +507,15 @@ struct SlotGeom {
     uint32_t Hkv, G;
     RunGeom runs; // matrix-core kernel: how the block list was cut into per-wavefront runs
     int blocked;
+    uint32_t uniform_blocks; // blocks per sequence when all sequences span the same number (blk_off is then not read:
+                             // nothing may have computed it), else 0
 };
 
 // Partial slots of head h of sequence s: the wavefronts whose runs intersect the head's region, in order.
 __device__ __forceinline__ uint32_t slots_of_row(const SlotGeom &sg, uint32_t s, uint32_t h)
 {
-    const uint32_t first_blk = sg.blk_off[s], nb = sg.blk_off[s + 1] - first_blk;
+    const uint32_t first_blk = sg.uniform_blocks ? s * sg.uniform_blocks : sg.blk_off[s];
+    const uint32_t nb = sg.uniform_blocks ? sg.uniform_blocks : sg.blk_off[s + 1] - first_blk;
     if (nb == 0) {
         return 0;
     }
@@ -834,6 +837,34 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         // one workgroup per compute unit
         const uint32_t target_units = tune.wavefronts > 0 ? (uint32_t)tune.wavefronts : runs.waves * 256u;
         runs.unit_blocks = std::max(1u, (total_blocks + target_units - 1) / target_units);
+        // Equal sequences of nb blocks: prefer a run length with which every workgroup holds whole regions (the
+        // kernel then does the whole call by itself, see below): nb / (classes * q) blocks with q = 1, 2 or 4, that
+        // is 4 / q regions per workgroup, provided the workgroups fill the compute units in at most two rounds.
+        {
+            uint32_t nb = ((uint32_t)c->lens[0] + 63u) >> 6;
+            for (int32_t l : c->lens) {
+                if ((((uint32_t)l + 63u) >> 6) != nb) {
+                    nb = 0;
+                    break;
+                }
+            }
+            const uint32_t gp = pass_heads <= 4 ? 4u : (pass_heads <= 8 ? 8u : 16u);
+            if (nb != 0 && mfma_decode_merges(gp, d) && tune.wavefronts == 0 && !tune.separate_merge &&
+                !tune.always_search) {
+                const uint32_t classes = run_classes(runs), regions = S * Hkv;
+                uint32_t best_rounds = 3;
+                for (uint32_t q = 1; q <= 4; q *= 2) {
+                    if (nb % (classes * q) != 0) {
+                        continue;
+                    }
+                    const uint32_t wgs = (regions * q + 3) / 4, rounds = (wgs + 255) / 256;
+                    if (rounds < best_rounds && wgs * 100 >= rounds * 256 * 95) {
+                        best_rounds = rounds;
+                        runs.unit_blocks = nb / (classes * q);
+                    }
+                }
+            }
+        }
         const uint32_t skew_pct = tune.skew_percent >= 0 ? (uint32_t)std::min(90, tune.skew_percent)
                                                          : (runs.waves == 12 ? kRunSkewPercent3 : kRunSkewPercent);
         const uint32_t nblk = (max_len + 63) / 64;
@@ -920,8 +951,12 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         if (mfma_decode_merges(gp, d) && nb != 0 && nb % cycle == 0 && wg_blocks % nb == 0 &&
             !decode_tuning().separate_merge) {
             wg_regions = wg_blocks / nb;
-            fused_query = wg_regions * pass_heads <= kMfmaQueryRows && !decode_tuning().separate_query;
         }
+        // Equal sequences: a workgroup's blocks lie in at most (wg_blocks - 1) / nb + 2 regions, whose queries it
+        // rotates itself when they are few enough for its LDS; nothing then runs ahead of the matrix-core kernel.
+        const uint32_t wg_most_regions = wg_regions ? wg_regions : (nb ? (wg_blocks - 1) / nb + 2 : 0);
+        fused_query = mfma_decode_merges(gp, d) && nb != 0 && wg_most_regions * pass_heads <= kMfmaQueryRows &&
+                      !decode_tuning().separate_query;
     }
     const bool fused_merge = wg_regions != 0;
     if (fused_query) {
@@ -994,7 +1029,7 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
     if (!fused_merge) {
         ProfileScope prof("kv_decode_combine", timed);
         const SlotGeom sg = { use_mfma ? blk_off : nullptr, Hkv, G, runs,
-                              gqa_mapping == WEED_HIP_GQA_BLOCKED ? 1 : 0 };
+                              gqa_mapping == WEED_HIP_GQA_BLOCKED ? 1 : 0, uniform_blocks };
         if (many_rows && n_splits <= 64) {
             combine_rows_kernel<<<(n_rows + kRowsPerWg - 1) / kRowsPerWg, 256, 0, stream()>>>(
                 partials, Hq, d, d_real, n_splits, n_rows, sg, c->v.rot, unrot ? 1 : 0, use_mfma ? 1 : 0, out_dev, og);

@@ -362,7 +362,8 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     static_assert(!WGM || mfma_decode_merges(GP, D), "this instance cannot merge");
     constexpr bool kCanMerge = WGM;
     constexpr uint32_t NG = kMfmaMergeThreads / D; // groups of source coordinates of the un-rotation
-    constexpr uint32_t JPG = WGM ? D / (NG ? NG : 1) : 1; // source coordinates per group
+    constexpr bool kQuery = mfma_decode_merges(GP, D);   // this instance can rotate its queries itself (MfmaQuery)
+    constexpr uint32_t JPG = kQuery ? D / (NG ? NG : 1) : 1; // source coordinates per group
     float *const part_s = reinterpret_cast<float *>(lds) + ROWS * (kTableRowBytes / 4); // [position][GP][D + 2]
     float xrot[kCanMerge ? JPG : 1];
     auto request_rotation = [&]() {
@@ -387,7 +388,7 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     }
     // ---- query rotation inside the kernel (see MfmaQuery).  Row (region ri of the workgroup, head slot hs) has index
     //      ri * G + hs.  Requested here: this thread's share of the K rotation and of the raw queries. ----
-    constexpr uint32_t QPT = WGM ? (kMfmaQueryRows * D + kThreads - 1) / kThreads : 1; // raw query elements per thread
+    constexpr uint32_t QPT = kQuery ? (kMfmaQueryRows * D + kThreads - 1) / kThreads : 1; // raw query elements per thread
     constexpr uint32_t PW = mfma_merge_partials_words(kWaves, GP, D);
     float *const qraw_s = part_s;                              // [rows][D]
     float *const qred_s = part_s + kMfmaQueryRows * D;         // [NG][kMfmaMergeRows][D]
@@ -395,11 +396,20 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     uint16_t *const ql_s = qh_s + kMfmaQueryRows * D;                 // [rows][D] low halves
     float *const qscale_s = part_s + PW + kMfmaQueryRows * D;         // [rows]
     float *const qsum_s = qscale_s + kMfmaQueryRows;                  // [rows]
-    const bool fused_q = WGM && p.query.q != nullptr;
-    const uint32_t wg_rows = WGM ? p.merge.wg_regions * p.G : 0;
-    const uint32_t wg_region0 = WGM ? blockIdx.x * p.merge.wg_regions : 0;
-    float xq[WGM ? JPG : 1], qr[QPT];
+    const bool fused_q = kQuery && p.query.q != nullptr;
+    // the regions this workgroup's blocks lie in (equal sequences of uniform_blocks blocks each)
+    uint32_t wg_region0 = 0, wg_rows = 0;
     if constexpr (WGM) {
+        wg_region0 = blockIdx.x * p.merge.wg_regions;
+        wg_rows = p.merge.wg_regions * p.G;
+    } else if (fused_q) {
+        const uint32_t wg_blocks = kWaves * p.runs.unit_blocks;
+        const uint32_t first = blockIdx.x * wg_blocks, last = min(first + wg_blocks, p.total_blocks) - 1;
+        wg_region0 = first / p.uniform_blocks;
+        wg_rows = (last / p.uniform_blocks - wg_region0 + 1) * p.G;
+    }
+    float xq[kQuery ? JPG : 1], qr[QPT];
+    if constexpr (kQuery) {
         if (fused_q) {
             if (p.query.rotate && tid < kMfmaMergeThreads) {
                 const __amdgpu_buffer_rsrc_t rot = buffer_of(p.query.rot_t, 4 * D * D);
@@ -435,7 +445,7 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     // for every row, the groups' sums are added in a fixed order), then one wavefront per row scales, normalises and
     // splits the row as the stand-alone kernel does.  Contains the tables' barrier; every wavefront calls it once.
     auto rotate_queries = [&]() {
-        if constexpr (WGM) {
+        if constexpr (kQuery) {
 #pragma unroll
             for (uint32_t i = 0; i < QPT; ++i) {
                 const uint32_t e = tid + i * kThreads;
@@ -546,6 +556,13 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
         }
         seq = __builtin_amdgcn_readfirstlane(lo);
     }
+    if constexpr (kQuery && !WGM) {
+        // (ahead of the loop over the segments, which must not carry the requested elements around)
+        if (fused_q && !tables_ready) {
+            rotate_queries();
+            tables_ready = true;
+        }
+    }
     while (g0 < g1) {
     const uint32_t seq_first = uniform_nb ? seq * uniform_nb : p.blk_off[seq];
     // blocks the cached length of this sequence spans
@@ -622,9 +639,12 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     constexpr int NQ = PACKED ? 1 : 2;
     half8 qop[NQ][KS];
     if (fused_q) {
-        if constexpr (WGM) {
-            rotate_queries(); // (with the tables' barrier)
-            tables_ready = true;
+        if constexpr (kQuery) {
+            if constexpr (WGM) {
+                // (the only segment: the first block is on its way meanwhile)
+                rotate_queries();
+                tables_ready = true;
+            }
             const uint32_t col_head = c % GP, col_part = c / GP; // (PACKED: merging instances have GP <= 8)
             const bool col_ok = col_head < p.G && col_part < 2;
             const uint32_t row = ((uint32_t)region - wg_region0) * p.G + (col_ok ? col_head : 0);
@@ -1094,7 +1114,7 @@ template <int D, int WK, int WV, int GP, bool LLOYD> int launch_gp(const MfmaPar
     constexpr bool kMerges = mfma_decode_merges(GP, D);
     std::call_once(configured, [] {
         config_status = hipFuncSetAttribute((const void *)decode_mfma_kernel<D, WK, WV, GP, LLOYD, false>,
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_merging);
         if constexpr (kMerges) {
             if (config_status == hipSuccess) {
                 config_status = hipFuncSetAttribute((const void *)decode_mfma_kernel<D, WK, WV, GP, LLOYD, true>,
@@ -1116,7 +1136,8 @@ template <int D, int WK, int WV, int GP, bool LLOYD> int launch_gp(const MfmaPar
             return fail(WEED_HIP_EDEVICE, "decode_mfma: this kernel instance cannot merge its partials itself");
         }
     } else {
-        decode_mfma_kernel<D, WK, WV, GP, LLOYD, false><<<grid, 64 * waves, smem, s>>>(p);
+        // (the area behind the tables is where a workgroup rotates its queries, when it does)
+        decode_mfma_kernel<D, WK, WV, GP, LLOYD, false><<<grid, 64 * waves, p.query.q ? smem_merging : smem, s>>>(p);
     }
     WEED_HIP_LAUNCH_CHECK();
     return WEED_HIP_OK;
