@@ -227,12 +227,16 @@ def test_equal_contexts_with_and_without_the_region_search(gpu, oracle):
     want = checker_output(oracle, gpu, cache, wl, q, False)
     try:
         fast = run_decode(gpu, cache, q, gpu.GQA_BLOCKED, 0)
+        # (with the merge left to the second kernel on both sides: the kernel's own merge adds in another order)
+        gpu.decode_tuning(separate_merge=True)
+        divided = run_decode(gpu, cache, q, gpu.GQA_BLOCKED, 0)
         gpu.decode_tuning(always_search=True)
         searched = run_decode(gpu, cache, q, gpu.GQA_BLOCKED, 0)
     finally:
         gpu.decode_tuning()
     assert_attn_close(fast, want, "equal contexts")
-    assert np.array_equal(fast, searched)
+    assert_attn_close(divided, want, "equal contexts, separate merge")
+    assert np.array_equal(divided, searched)
     cache.close()
 
 
@@ -244,11 +248,17 @@ def test_equal_contexts_with_and_without_the_region_search(gpu, oracle):
     (True, 128, 2, 8, 2, 768, 2, 2, 24, True),      # three wavefronts per SIMD: three age classes
     (True, 64, 4, 4, 8, 768, 3, 3, 96, True),       # groups of one, four regions per workgroup
     (False, 128, 1, 2, 8, 2048, 8, 8, 64, True),    # 8-bit uniform codes (no lookup tables)
+    # regions of several workgroups' shares: the workgroup that arrives last at a region merges it
+    (True, 128, 2, 8, 1, 2048, 3, 4, 32, True),     # two workgroups per region
+    (True, 128, 1, 4, 1, 8192, 3, 4, 128, True),    # sixteen workgroups per region
+    (True, 128, 2, 8, 2, 1536, 2, 2, 96, True),     # three wavefronts per SIMD
+    (False, 64, 2, 16, 3, 1536, 4, 4, 144, False),  # uniform coder, head_dim 64, groups of 8, no rotations
 ])
 def test_workgroups_that_merge_their_own_regions(gpu, oracle, lloyd, d, Hkv, Hq, S, L, kb, vb, waves, rot):
-    """When every workgroup of the matrix-core kernel holds whole regions, it rotates its queries and merges its
-    partials itself and the call is a single kernel; the same call with the kernels ahead and behind must agree to
-    rounding, and both with the checker.  Also with per-sequence prefix lengths, zero among them."""
+    """When every workgroup of the matrix-core kernel holds whole regions, or every region a whole number of
+    workgroups' shares, the kernel rotates its queries and merges its partials itself and the call is a single kernel;
+    the same call with the kernels ahead and behind must agree to rounding, and both with the checker.  Also with
+    per-sequence prefix lengths, zero among them, and twice in a row (the arrival counters are back at zero)."""
     import torch
     rng = np.random.default_rng(53)
     wl = workloads.Workload("merge", S, Hq, Hkv, d, [L] * S, kb, vb, 0, 0, 0)

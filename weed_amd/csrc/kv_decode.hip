@@ -896,7 +896,11 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
     const size_t s_bytes = (sizeof(float) * (size_t)S * Hq + 15) / 16 * 16;
     const size_t part_bytes = sizeof(float) * (size_t)S * Hq * n_splits * (d + 2);
     const size_t off_bytes = (sizeof(uint32_t) * ((size_t)S + 1) + 15) / 16 * 16;
-    const size_t need = q_bytes + 2 * h_bytes + 2 * s_bytes + off_bytes + part_bytes;
+    // (the arrival counters of the kernel's own merge come first, at the same place whatever the shape, because they
+    // have to be zero when a launch starts: they are cleared when the workspace is allocated and every launch leaves
+    // them at zero; the static scratch starts as zeros)
+    const size_t arrive_bytes = sizeof(uint32_t) * kMfmaMergeCounters;
+    const size_t need = arrive_bytes + q_bytes + 2 * h_bytes + 2 * s_bytes + off_bytes + part_bytes;
     if (fixed_ws) {
         // the caller's workspace (the static scratch): nothing is allocated, larger shapes are refused
         WEED_HIP_REQUIRE(need <= fixed_ws_bytes,
@@ -911,8 +915,11 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
             return fail(WEED_HIP_ENOMEM, "%s: workspace allocation of %zu bytes failed", fn, need);
         }
         c->dec_ws_bytes = need;
+        WEED_HIP_CHECK(hipMemsetAsync(c->dec_ws, 0, arrive_bytes, stream()));
     }
-    uint8_t *wsp = fixed_ws ? fixed_ws : reinterpret_cast<uint8_t *>(c->dec_ws);
+    uint8_t *ws0 = fixed_ws ? fixed_ws : reinterpret_cast<uint8_t *>(c->dec_ws);
+    uint32_t *arrive = reinterpret_cast<uint32_t *>(ws0);
+    uint8_t *wsp = ws0 + arrive_bytes;
     const bool timed = !fixed_ws; // the timing scopes create events, which the allocation-free entry point must not
     float *q_rot = reinterpret_cast<float *>(wsp);
     uint16_t *q_hi = reinterpret_cast<uint16_t *>(wsp + q_bytes);
@@ -935,7 +942,7 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
     // every workgroup's share of the block list is a whole number of regions and no run straddles a region boundary:
     // equal sequences of nb blocks each, nb a multiple of one cycle of the age classes' runs, and a workgroup's blocks
     // a multiple of nb.  They then also rotate their regions' queries themselves, and the call is ONE kernel.
-    uint32_t wg_regions = 0;
+    uint32_t wg_regions = 0, region_wgs = 0;
     bool fused_query = false;
     if (use_mfma && total_blocks) {
         uniform_blocks = ((uint32_t)c->lens[0] + 63u) >> 6;
@@ -951,6 +958,11 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         if (mfma_decode_merges(gp, d) && nb != 0 && nb % cycle == 0 && wg_blocks % nb == 0 &&
             !decode_tuning().separate_merge) {
             wg_regions = wg_blocks / nb;
+        } else if (mfma_decode_merges(gp, d) && nb != 0 && nb % wg_blocks == 0 && nb / wg_blocks >= 2 &&
+                   nb / wg_blocks <= std::min(n_splits, 64u) && (size_t)S * Hkv <= kMfmaMergeCounters &&
+                   !decode_tuning().separate_merge) {
+            // small batches of long sequences: every region is a whole number of workgroups' shares
+            region_wgs = nb / wg_blocks;
         }
         // Equal sequences: a workgroup's blocks lie in at most (wg_blocks - 1) / nb + 2 regions, whose queries it
         // rotates itself when they are few enough for its LDS; nothing then runs ahead of the matrix-core kernel.
@@ -958,7 +970,7 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         fused_query = mfma_decode_merges(gp, d) && nb != 0 && wg_most_regions * pass_heads <= kMfmaQueryRows &&
                       !decode_tuning().separate_query;
     }
-    const bool fused_merge = wg_regions != 0;
+    const bool fused_merge = wg_regions != 0 || region_wgs != 0;
     if (fused_query) {
         // (nothing runs ahead of the matrix-core kernel)
     } else if (many_rows) {
@@ -994,7 +1006,7 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         mp.n_seq = S;
         mp.total_blocks = total_blocks;
         mp.uniform_blocks = uniform_blocks;
-        mp.merge = MfmaMerge{ wg_regions, d_real, out_dev, og, c->v.rot, unrot ? 1 : 0 };
+        mp.merge = MfmaMerge{ wg_regions, region_wgs, arrive, d_real, out_dev, og, c->v.rot, unrot ? 1 : 0 };
         mp.query = MfmaQuery{ fused_query ? q_dev : nullptr, qg, c->k.rot_t, rot_q ? 1 : 0 };
         mp.runs = runs;
         mp.max_slots = n_splits;

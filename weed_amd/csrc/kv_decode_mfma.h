@@ -125,8 +125,15 @@ __device__ __forceinline__ uint64_t head_offset(const Geom3 &g, uint32_t hv)
 // waves / wg_regions wavefronts), the wavefronts leave their partials in LDS, and the workgroup merges them,
 // un-rotates the result and writes the output rows itself: no partials in memory, no second kernel.
 // `wg_regions` 0: the kernel writes the partials to memory and a second kernel merges them.
+// `region_wgs` >= 2 instead (wg_regions 0): every region is a whole number of workgroups' shares (small batches of long
+// sequences).  A workgroup then merges its wavefronts' partials into ONE partial of the region in memory and counts
+// itself in `arrive[region]`; the workgroup that completes the count merges the region's partials, un-rotates and
+// writes the output rows, and puts the counter back to zero (so the counters are zero between launches; whoever
+// allocates them clears them once).
 struct MfmaMerge {
     uint32_t wg_regions;
+    uint32_t region_wgs;
+    uint32_t *arrive;  // [n_seq * Hkv] arrival counters, zero when the launch starts
     uint32_t d_real;   // coordinates the caller's rows have (<= the stored head_dim)
     float *out;        // attention output
     Geom3 og;          // its strides
@@ -161,8 +168,11 @@ constexpr uint32_t mfma_merge_partials_words(uint32_t waves, uint32_t gp, uint32
 }
 constexpr uint32_t mfma_merge_lds_bytes(uint32_t waves, uint32_t gp, uint32_t d)
 {
-    return 4u * (mfma_merge_partials_words(waves, gp, d) + kMfmaMergeRows * d + kMfmaMergeThreads * kMfmaMergeRows);
+    // (+ 4 words at the end: the arrival count that one thread reads for the workgroup)
+    return 4u * (mfma_merge_partials_words(waves, gp, d) + kMfmaMergeRows * d + kMfmaMergeThreads * kMfmaMergeRows + 4u);
 }
+// Arrival counters that a workspace reserves.
+constexpr uint32_t kMfmaMergeCounters = 16384;
 static_assert(kMfmaQueryRows * 128u + 2u * kMfmaQueryRows <= kMfmaMergeRows * 128u + kMfmaMergeThreads * kMfmaMergeRows &&
                   kMfmaQueryRows * 64u + 2u * kMfmaQueryRows <= kMfmaMergeRows * 64u + kMfmaMergeThreads * kMfmaMergeRows,
               "the query halves, scales and sums fit where the merged rows and the un-rotation's sums will be");

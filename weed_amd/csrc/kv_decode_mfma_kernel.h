@@ -282,9 +282,18 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_of(const float *base, u
 {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(base), 0, (int)bytes, 0x00020000);
 }
+// COHERENT: the load is served at device scope (it does not hit a line that this XCD's L2 holds from before another
+// XCD wrote it), as a relaxed atomic load of device scope is.
+template <bool COHERENT = false>
 __device__ __forceinline__ float buffer_f32(__amdgpu_buffer_rsrc_t r, uint32_t lane_off, uint32_t uniform_off)
 {
-    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)lane_off, (int)uniform_off, 0));
+    constexpr int kDeviceScope = 16; // the sc1 bit of the cache policy
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)lane_off, (int)uniform_off,
+                                                                          COHERENT ? kDeviceScope : 0));
+}
+__device__ __forceinline__ float lane_value(float v, uint32_t l)
+{
+    return __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(v), (int)l));
 }
 
 // Bank mask (4-lane banks of a row) of the lanes [GP*i, GP*i + GP).
@@ -399,9 +408,12 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     const bool fused_q = kQuery && p.query.q != nullptr;
     // the regions this workgroup's blocks lie in (equal sequences of uniform_blocks blocks each)
     uint32_t wg_region0 = 0, wg_rows = 0;
-    if constexpr (WGM) {
+    if (WGM && p.merge.wg_regions != 0) {
         wg_region0 = blockIdx.x * p.merge.wg_regions;
         wg_rows = p.merge.wg_regions * p.G;
+    } else if (WGM) {
+        wg_region0 = (blockIdx.x * kWaves * p.runs.unit_blocks) / p.uniform_blocks; // a share of one region
+        wg_rows = p.G;
     } else if (fused_q) {
         const uint32_t wg_blocks = kWaves * p.runs.unit_blocks;
         const uint32_t first = blockIdx.x * wg_blocks, last = min(first + wg_blocks, p.total_blocks) - 1;
@@ -1026,34 +1038,44 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
         constexpr uint32_t RP = kMfmaMergeRows;
         float *const o_s = part_s + PW;               // [RP][D] merged, normalised rows
         float *const red_s = o_s + RP * D;            // [NG][RP][D] partial sums of the un-rotation
-        const uint32_t slots = kWaves / p.merge.wg_regions;
-        const uint32_t rows = p.merge.wg_regions * p.G;
-        const uint32_t region0 = blockIdx.x * p.merge.wg_regions, n_regions = p.n_seq * p.Hkv;
-        __syncthreads(); // every wavefront's partial is in LDS (and nobody reads the tables any more)
-        for (uint32_t r0 = 0; r0 < rows; r0 += RP) {
-            // (the row of element e is the same in all lanes of a wavefront: kThreads is a multiple of D)
-            const uint32_t rr_of_wave = __builtin_amdgcn_readfirstlane(tid / D);
+        uint32_t *const count_s = reinterpret_cast<uint32_t *>(red_s + kMfmaMergeThreads * RP);
+        const uint32_t n_regions = p.n_seq * p.Hkv;
+        // (the row of an element is the same in all lanes of a wavefront: kThreads is a multiple of D)
+        const uint32_t rr_of_wave = __builtin_amdgcn_readfirstlane(tid / D), col = tid % D;
+        // rows r0 .. r0 + RP - 1 of the workgroup (row = region index in the workgroup * G + head slot): o_s = the
+        // merge of the row's `slots` partials, which partial(ri, hs, k) finds; normalised, or with NORMALISE false
+        // left as the partial (m, l, o) that leave(rr, m, l, o) puts somewhere
+        auto merge_rows = [&](uint32_t r0, uint32_t rows, uint32_t slots, auto partial, auto normalise, auto leave) {
+            constexpr bool NORMALISE = decltype(normalise)::value;
             for (uint32_t rr = rr_of_wave; rr < RP; rr += kThreads / D) {
-                const uint32_t e = rr * D + tid % D, j = tid % D, row = r0 + rr;
+                const uint32_t row = r0 + rr;
                 float v = 0.0f;
                 if (row < rows) {
                     const uint32_t ri = row / p.G, hs = row - ri * p.G;
-                    const float *first = part_s + (ri * slots * GP + hs) * PS; // slot k: + k * GP * PS
                     float mx = -INFINITY;
                     for (uint32_t k = 0; k < slots; ++k) {
-                        mx = fmaxf(mx, first[k * (GP * PS)]);
+                        mx = fmaxf(mx, partial(ri, hs, k, 0u));
                     }
                     float den = 0.0f, acc = 0.0f;
                     for (uint32_t k = 0; k < slots; ++k) {
-                        const float m = first[k * (GP * PS)];
+                        const float m = partial(ri, hs, k, 0u);
                         const float w = (m == -INFINITY) ? 0.0f : exp2f(m - mx);
-                        den = fmaf(w, first[k * (GP * PS) + 1], den);
-                        acc = fmaf(w, first[k * (GP * PS) + 2 + j], acc);
+                        den = fmaf(w, partial(ri, hs, k, 1u), den);
+                        acc = fmaf(w, partial(ri, hs, k, 2u + col), acc);
                     }
-                    v = den > 0.0f ? acc / den : 0.0f;
+                    if constexpr (NORMALISE) {
+                        v = den > 0.0f ? acc / den : 0.0f;
+                    } else {
+                        leave(ri, hs, mx, den, acc);
+                    }
                 }
-                o_s[e] = v;
+                if constexpr (NORMALISE) {
+                    o_s[rr * D + col] = v;
+                }
             }
+        };
+        // un-rotation of the rows in o_s and the output rows of the regions region0 + ri
+        auto finish_rows = [&](uint32_t r0, uint32_t rows, uint32_t region0) {
             __syncthreads();
             if (p.merge.unrotate) {
                 if (tid < kMfmaMergeThreads) {
@@ -1078,26 +1100,121 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
                 __syncthreads();
             }
             for (uint32_t rr = rr_of_wave; rr < RP; rr += kThreads / D) {
-                const uint32_t e = rr * D + tid % D, t = tid % D, row = r0 + rr;
+                const uint32_t row = r0 + rr;
                 const uint32_t ri = row / p.G, hs = row - ri * p.G;
-                if (row < rows && region0 + ri < n_regions && t < p.merge.d_real) {
+                if (row < rows && region0 + ri < n_regions && col < p.merge.d_real) {
                     float v;
                     if (p.merge.unrotate) {
                         v = 0.0f;
 #pragma unroll
                         for (uint32_t jg = 0; jg < NG; ++jg) {
-                            v += red_s[(jg * RP + rr) * D + t];
+                            v += red_s[(jg * RP + rr) * D + col];
                         }
                     } else {
-                        v = o_s[e];
+                        v = o_s[rr * D + col];
                     }
                     const uint32_t region = region0 + ri;
                     const uint32_t s_ = region / p.Hkv, kv_ = region - s_ * p.Hkv;
                     p.merge.out[(uint64_t)p.merge.og.off + (uint64_t)s_ * p.merge.og.s[0] +
-                                head_offset(p.merge.og, q_head_of(p, kv_, hs)) + (uint64_t)t * p.merge.og.s[2]] = v;
+                                head_offset(p.merge.og, q_head_of(p, kv_, hs)) + (uint64_t)col * p.merge.og.s[2]] = v;
                 }
             }
             __syncthreads(); // before the next pass overwrites the rows
+        };
+        __syncthreads(); // every wavefront's partial is in LDS (and nobody reads the tables any more)
+        if (p.merge.wg_regions != 0) {
+            // whole regions: slots = wavefronts per region
+            const uint32_t slots = kWaves / p.merge.wg_regions, rows = p.merge.wg_regions * p.G;
+            auto in_lds = [&](uint32_t ri, uint32_t hs, uint32_t k, uint32_t word) {
+                return part_s[((ri * slots + k) * GP + hs) * PS + word];
+            };
+            for (uint32_t r0 = 0; r0 < rows; r0 += RP) {
+                merge_rows(r0, rows, slots, in_lds, std::true_type{}, [](uint32_t, uint32_t, float, float, float) {});
+                finish_rows(r0, rows, blockIdx.x * p.merge.wg_regions);
+            }
+        } else {
+            // A share of ONE region (p.G <= RP rows): the wavefronts' partials become one partial of the region in
+            // memory, stored through to device scope; when those stores have completed the workgroup counts itself,
+            // and the workgroup that completes the region's count reads all of the region's partials with loads of
+            // device scope and finishes the rows.  (No cache-wide write-back or invalidation: every wavefront issuing
+            // them costs more than the whole merge.)
+            const uint32_t wg_blocks = kWaves * p.runs.unit_blocks;
+            const uint32_t region = (blockIdx.x * wg_blocks) / p.uniform_blocks;
+            const uint32_t my_slot = blockIdx.x - (region * p.uniform_blocks) / wg_blocks;
+            const uint32_t s_ = region / p.Hkv, kv_ = region - s_ * p.Hkv;
+            auto in_lds = [&](uint32_t, uint32_t hs, uint32_t k, uint32_t word) {
+                return part_s[(k * GP + hs) * PS + word];
+            };
+            auto slot_of = [&](uint32_t hs, uint32_t k) {
+                return p.partials + (((uint64_t)s_ * p.Hq + q_head_of(p, kv_, hs)) * p.max_slots + k) * PS;
+            };
+            merge_rows(0, p.G, kWaves, in_lds, std::false_type{},
+                       [&](uint32_t, uint32_t hs, float m, float l, float o) {
+                           float *dst = slot_of(hs, my_slot);
+                           __hip_atomic_store(dst + 2 + col, o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                           if (col == 0) {
+                               __hip_atomic_store(dst, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                               __hip_atomic_store(dst + 1, l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                           }
+                       });
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (tid == 0) {
+                *count_s = __hip_atomic_fetch_add(p.merge.arrive + region, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            __syncthreads();
+            if (*count_s + 1 != p.merge.region_wgs) {
+                return;
+            }
+            if (tid == 0) {
+                __hip_atomic_store(p.merge.arrive + region, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            // The region's partials (at most 64, the host sees to that): lane k of every wavefront reads the header
+            // of partial k, the wavefront's 64 columns of the partials come eight partials at a time; all of these
+            // loads are independent of each other, so a row costs two trips to memory, not one per partial.
+            const uint32_t slots = p.merge.region_wgs;
+            for (uint32_t rr = rr_of_wave; rr < RP; rr += kThreads / D) {
+                float v = 0.0f;
+                if (rr < p.G) {
+                    const __amdgpu_buffer_rsrc_t src = buffer_of(slot_of(rr, 0), slots * (4 * PS));
+                    float m0 = buffer_f32<true>(src, lane * (4 * PS), 0), l0 = buffer_f32<true>(src, lane * (4 * PS), 4);
+                    float y[8];
+#pragma unroll
+                    for (uint32_t u = 0; u < 8; ++u) {
+                        y[u] = buffer_f32<true>(src, 4 * col, 4 * (min(u, slots - 1) * PS + 2));
+                    }
+                    if (lane >= slots) {
+                        m0 = -INFINITY;
+                        l0 = 0.0f;
+                    }
+                    const float mx = wave_max64(m0);
+                    const float w0 = (m0 == -INFINITY) ? 0.0f : exp2f(m0 - mx);
+                    const float den = wave_sum64(w0 * l0);
+                    float acc = 0.0f;
+                    for (uint32_t k0 = 0; k0 < slots; k0 += 8) {
+                        float z[8];
+                        if (k0 + 8 < slots) {
+#pragma unroll
+                            for (uint32_t u = 0; u < 8; ++u) {
+                                z[u] = buffer_f32<true>(src, 4 * col, 4 * (min(k0 + 8 + u, slots - 1) * PS + 2));
+                            }
+                        }
+#pragma unroll
+                        for (uint32_t u = 0; u < 8; ++u) {
+                            if (k0 + u < slots) {
+                                acc = fmaf(lane_value(w0, k0 + u), y[u], acc);
+                            }
+                        }
+#pragma unroll
+                        for (uint32_t u = 0; u < 8; ++u) {
+                            y[u] = z[u];
+                        }
+                    }
+                    v = den > 0.0f ? acc / den : 0.0f;
+                }
+                o_s[rr * D + col] = v;
+            }
+            finish_rows(0, p.G, region);
         }
     }
 }
@@ -1129,7 +1246,7 @@ template <int D, int WK, int WV, int GP, bool LLOYD> int launch_gp(const MfmaPar
     }
     const uint32_t wg_blocks = waves * p.runs.unit_blocks;
     const uint32_t grid = (p.total_blocks + wg_blocks - 1) / wg_blocks;
-    if (p.merge.wg_regions != 0) {
+    if (p.merge.wg_regions != 0 || p.merge.region_wgs != 0) {
         if constexpr (kMerges) {
             decode_mfma_kernel<D, WK, WV, GP, LLOYD, true><<<grid, 64 * waves, smem_merging, s>>>(p);
         } else {
