@@ -295,9 +295,11 @@ int weed_hip_kv_decode_tuning(int32_t wavefronts, int32_t skew_percent, int32_t 
  * bit-identical results; the workspace (rotated queries, split partials) is a 32 MiB array that is part of the
  * library's device image and that every device the library was initialised on holds until the process ends.  Calls
  * no hipMalloc / hipFree and creates no events (the library's timing scopes skip it).  Shapes whose workspace
- * n_seq * n_q_heads * (d * 8 + 8 + slots * (d + 2) * 4) bytes (slots: context splits, at most a few dozen) exceeds the
- * array return WEED_HIP_EINVAL.  All calls on one device share the array: calls that overlap on one device (two host
- * threads, two streams) race; weed_hip_init must have run on the device. */
+ * 64 KiB + n_seq * n_q_heads * (d * 8 + 8 + slots * (d + 2) * 4) bytes (slots: context splits, at most a few dozen)
+ * exceeds the array return WEED_HIP_EINVAL.  The first 64 KiB are arrival counters of the kernel's own merge: they start
+ * as zeros with the array and every launch that completes leaves them at zero.  All calls on one device share the
+ * array: calls that overlap on one device (two host threads, two streams) race; weed_hip_init must have run on the
+ * device. */
 int weed_hip_kv_decode_attn_noalloc(weed_hip_kv_cache *cache, int32_t n_q_heads, int32_t gqa_mapping,
                                     const float *q_dev, uint32_t q_off, const uint32_t q_stride[3], float *out_dev,
                                     uint32_t o_off, const uint32_t o_stride[3], uint32_t flags);
