@@ -1138,6 +1138,13 @@ int weed_hip_kv_cache_reset(weed_hip_kv_cache *c, int drop_rotations)
         fill_i32_kernel<<<(regions + 255) / 256, 256, 0, stream()>>>((int32_t *)c->v.alpha_max, 0, regions);
         WEED_HIP_LAUNCH_CHECK();
     }
+    if (c->dec_ws) {
+        // the arrival counters at the start of the decode workspace (zero between launches; cleared here too, so that
+        // a reset also recovers from a launch that the device aborted midway)
+        const uint32_t counters = std::min<size_t>(kMfmaMergeCounters, c->dec_ws_bytes / sizeof(int32_t));
+        fill_i32_kernel<<<(counters + 255) / 256, 256, 0, stream()>>>((int32_t *)c->dec_ws, 0, counters);
+        WEED_HIP_LAUNCH_CHECK();
+    }
     if (drop_rotations) {
         c->has_rotations = false;
     }

@@ -881,7 +881,7 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
     } else {
         // split the context so that the launch has a few workgroups per compute unit
         const uint32_t target_wgs = 2048;
-        uint32_t want = std::max(1u, target_wgs / (S * Hkv));
+        const uint32_t want = std::min((uint32_t)kMaxSlots, std::max(1u, target_wgs / (S * Hkv)));
         n_splits = std::max(1u, std::min((max_len + kChunk - 1) / kChunk, want));
         split_tokens = (max_len + n_splits - 1) / n_splits;
         split_tokens = std::max((uint32_t)kChunk, (split_tokens + kChunk - 1) / kChunk * kChunk);
@@ -971,6 +971,10 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
                       !decode_tuning().separate_query;
     }
     const bool fused_merge = wg_regions != 0 || region_wgs != 0;
+    // (the kernels that take one (sequence, head) row per workgroup have the sequence on a 16-bit grid dimension)
+    WEED_HIP_REQUIRE(S <= 65535u || (use_mfma && many_rows && n_splits <= 64),
+                     "%s: %u sequences in one call are served only for head_dims that are multiples of 64 with "
+                     "matrix-core instances; split the batch", fn, S);
     if (fused_query) {
         // (nothing runs ahead of the matrix-core kernel)
     } else if (many_rows) {

@@ -1398,6 +1398,23 @@ TensorPtr MultiHeadAttention::forward_quantized(TensorPtr Q, TensorPtr K, Tensor
         return out;
     }
     // causal attention: query position t sees the first before + t + 1 cached tokens of its sequence
+    // The (position, head) pairs of a KV head are the rows of the fused kernel's tiles: one call serves up to 64
+    // positions (a pass over the cache per tile of pairs), each masking the tokens after its own position.  Shapes
+    // without matrix-core instances go position by position through the generic kernel.
+    const tcapint per_call = matrix_core_shape() ? 64U : 1U;
+    const uint32_t q_str4[4] = { Q->stride[0U], Q->stride[1U], Q->stride[2U], Q->stride[3U] };
+    const uint32_t o_str4[4] = { out->stride[0U], out->stride[1U], out->stride[2U], out->stride[3U] };
+    if (uT <= per_call) {
+        // One call: its positions are the last uT cached tokens of every sequence, which is what the entry points
+        // assume without a length array (no host-built lengths, no transfer, no wait for earlier launches).
+        if (uT == 1U) {
+            HipDevice::check(weed_hip_kv_decode_attn(cache, num_heads, gqa, qp, Q->offset, q_str, op, 0U, q_str, flags));
+        } else {
+            HipDevice::check(weed_hip_kv_decode_attn_chunk(cache, nullptr, (int32_t)uT, num_heads, gqa, qp, Q->offset,
+                q_str4, op, 0U, o_str4, flags));
+        }
+        return out;
+    }
     const size_t need = sizeof(int32_t) * (size_t)uB * uT;
     if (need > lens_cap) {
         if (lens_dev) {
@@ -1415,12 +1432,6 @@ TensorPtr MultiHeadAttention::forward_quantized(TensorPtr Q, TensorPtr K, Tensor
     }
     HipDevice::check(weed_hip_sync()); // earlier launches may still read the previous call's lengths
     HipDevice::check(weed_hip_memcpy_h2d(lens_dev, lens.data(), need));
-    // The (position, head) pairs of a KV head are the rows of the fused kernel's tiles: one call serves up to 64
-    // positions (a pass over the cache per tile of pairs), each masking the tokens after its own position.  Shapes
-    // without matrix-core instances go position by position through the generic kernel.
-    const tcapint per_call = matrix_core_shape() ? 64U : 1U;
-    const uint32_t q_str4[4] = { Q->stride[0U], Q->stride[1U], Q->stride[2U], Q->stride[3U] };
-    const uint32_t o_str4[4] = { out->stride[0U], out->stride[1U], out->stride[2U], out->stride[3U] };
     for (tcapint t = 0U; t < uT; t += per_call) {
         const tcapint n = std::min(per_call, uT - t);
         const int32_t *lens_t = static_cast<const int32_t *>(lens_dev) + (size_t)(t + n - 1U) * uB;
