@@ -182,12 +182,34 @@ def time_kernel(capi, torch, fn, name, steps, warmup):
     one-off work of a shape's first launch (workspace growth, kernel attributes) stays out of both figures."""
     fn()
     torch.cuda.synchronize()
+    secs = time_calls(torch, fn, steps, warmup)  # (without the event pairs around the kernels)
     capi.profile_reset()
     capi.profile_enable(True)
-    secs = time_calls(torch, fn, steps, warmup)
+    time_calls(torch, fn, steps, 0)
     k_ms, k_n = capi.profile_read(name)
     capi.profile_enable(False)
     return secs, 1e-3 * k_ms / max(1, k_n)
+
+
+def decode_entry(capi, torch, fn, n_seq, nbytes, steps, warmup):
+    """One decode-attention configuration: step and kernel time, the kernel's roofline, and -- when the call is one
+    kernel (it rotated its queries and merged its partials itself) -- the same call as three kernels beside it."""
+    secs, kernel_s = time_kernel(capi, torch, fn, "kv_decode_attn", steps, warmup)
+    one_kernel = capi.profile_read("kv_decode_combine")[1] == 0
+    entry = {"tokens_per_s": n_seq / secs, "ms_per_step": 1e3 * secs, "packed_cache_bytes": nbytes,
+             "kernel_ms": 1e3 * kernel_s, "kernels_per_step": 1 if one_kernel else 3,
+             "step_frac": nbytes / secs / 1e9 / HBM_PEAK_GBS,
+             "roofline": {"bound": "hbm", "achieved": nbytes / kernel_s / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                          "frac": nbytes / kernel_s / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes_per_launch": nbytes}}
+    if one_kernel:
+        capi.decode_tuning(separate_merge=True, separate_query=True)
+        try:
+            secs3, kernel3_s = time_kernel(capi, torch, fn, "kv_decode_attn", steps, warmup)
+        finally:
+            capi.decode_tuning()
+        entry["same_step_as_three_kernels"] = {"ms_per_step": 1e3 * secs3, "attention_kernel_ms": 1e3 * kernel3_s,
+                                               "attention_kernel_frac": nbytes / kernel3_s / 1e9 / HBM_PEAK_GBS}
+    return entry
 
 
 def extras(capi, torch, workloads, steps, warmup):
@@ -268,15 +290,9 @@ def extras(capi, torch, workloads, steps, warmup):
     for hq in (8, 32):
         q = torch.randn((wl4.n_seq, hq, d), device="cuda")
         o = torch.zeros_like(q)
-        secs, kernel_s = time_kernel(capi, torch, lambda: cache4.decode_attn(q, o, capi.GQA_BLOCKED, 0),
-                                     "kv_decode_attn", steps, warmup)
-        nbytes = wl4.bytes_per_step(True)
-        out["cfg4_ragged16_hq%d" % hq] = {"tokens_per_s": wl4.n_seq / secs, "ms_per_step": 1e3 * secs,
-                                          "packed_cache_bytes": nbytes, "kernel_ms": 1e3 * kernel_s,
-                                          "step_frac": nbytes / secs / 1e9 / HBM_PEAK_GBS,
-                                          "roofline": {"bound": "hbm", "achieved": nbytes / kernel_s / 1e9, "peak": HBM_PEAK_GBS,
-                                                       "unit": "GB/s", "frac": nbytes / kernel_s / 1e9 / HBM_PEAK_GBS,
-                                                       "algorithmic_bytes_per_launch": nbytes}}
+        out["cfg4_ragged16_hq%d" % hq] = decode_entry(
+            capi, torch, lambda: cache4.decode_attn(q, o, capi.GQA_BLOCKED, 0), wl4.n_seq, wl4.bytes_per_step(True),
+            steps, warmup)
     cache4.close()
     # Weed's own uniform coder at kv_quant_bits = 8 on the headline shape (64 x 8192 tokens x 8 heads, 256 B per token
     # and head): the matrix-core kernel with arithmetic de-quantisation instead of tables
@@ -290,14 +306,9 @@ def extras(capi, torch, workloads, steps, warmup):
     del Ks, Vs
     q8 = torch.randn((wl8.n_seq, wl8.n_q_heads, d), device="cuda")
     o8 = torch.zeros_like(q8)
-    secs, kernel_s = time_kernel(capi, torch, lambda: cache8.decode_attn(q8, o8, capi.GQA_BLOCKED, 0),
-                                 "kv_decode_attn", steps, warmup)
-    nbytes = sum(wl8.lens) * wl8.n_kv_heads * 2 * d
-    out["uniform_8bit_64_sequences"] = {"tokens_per_s": wl8.n_seq / secs, "ms_per_step": 1e3 * secs,
-                                        "packed_cache_bytes": nbytes, "kernel_ms": 1e3 * kernel_s,
-                                        "roofline": {"bound": "hbm", "achieved": nbytes / kernel_s / 1e9, "peak": HBM_PEAK_GBS,
-                                                       "unit": "GB/s", "frac": nbytes / kernel_s / 1e9 / HBM_PEAK_GBS,
-                                                       "algorithmic_bytes_per_launch": nbytes}}
+    out["uniform_8bit_64_sequences"] = decode_entry(
+        capi, torch, lambda: cache8.decode_attn(q8, o8, capi.GQA_BLOCKED, 0), wl8.n_seq,
+        sum(wl8.lens) * wl8.n_kv_heads * 2 * d, steps, warmup)
     cache8.close()
     del q8, o8
     # configuration 3 again with 256 sequence caches per launch (2 GB of packed rows): what the per-launch fixed cost
@@ -306,14 +317,9 @@ def extras(capi, torch, workloads, steps, warmup):
     cache3, q3, _, _ = build_cache(capi, torch, wl3, seed=77)
     o3 = torch.zeros_like(q3)
     flags = capi.ATTN_ROTATE_Q | capi.ATTN_UNROTATE_OUT
-    secs, kernel_s = time_kernel(capi, torch, lambda: cache3.decode_attn(q3, o3, capi.GQA_BLOCKED, flags),
-                                 "kv_decode_attn", steps, warmup)
-    nbytes = wl3.bytes_per_step(lloydmax=True)
-    out["cfg3_256_sequences"] = {"tokens_per_s": wl3.n_seq / secs, "ms_per_step": 1e3 * secs,
-                                 "packed_cache_bytes": nbytes, "kernel_ms": 1e3 * kernel_s,
-                                 "roofline": {"bound": "hbm", "achieved": nbytes / kernel_s / 1e9, "peak": HBM_PEAK_GBS,
-                                                       "unit": "GB/s", "frac": nbytes / kernel_s / 1e9 / HBM_PEAK_GBS,
-                                                       "algorithmic_bytes_per_launch": nbytes}}
+    out["cfg3_256_sequences"] = decode_entry(
+        capi, torch, lambda: cache3.decode_attn(q3, o3, capi.GQA_BLOCKED, flags), wl3.n_seq,
+        wl3.bytes_per_step(lloydmax=True), steps, warmup)
     cache3.close()
     return out
 
@@ -520,7 +526,7 @@ def main():
         if not args.no_extras:
             # (short kernels need their own warm-up: after an idle stretch the first dozens of launches run at a lower
             # clock, 5 us slower on a 50 us kernel)
-            result["other_configs"] = extras(capi, torch, workloads, min(args.steps, 30), max(args.warmup, 30))
+            result["other_configs"] = extras(capi, torch, workloads, min(args.steps, 200), max(args.warmup, 50))
     print(json.dumps(result))
 
 

@@ -311,6 +311,65 @@ def test_workgroups_that_merge_their_own_regions(gpu, oracle, lloyd, d, Hkv, Hq,
     cache.close()
 
 
+@pytest.mark.parametrize("lloyd,d,Hkv,Hq,lens,kb,vb,waves", [
+    (True, 128, 2, 8, [700, 64, 3000, 129, 1, 2049], 3, 4, 0),      # ragged, runs straddle regions
+    (True, 128, 2, 8, [700, 64, 3000, 129, 1, 2049], 3, 4, 40),     # the same with few, long runs
+    (True, 128, 8, 8, [2048, 517, 8192, 1030, 4100], 3, 3, 300),    # groups of one, three wavefronts per SIMD
+    (False, 64, 2, 16, [1000, 333, 90, 2500], 4, 4, 0),             # uniform coder, head_dim 64, groups of 8
+    (True, 128, 2, 8, [1500] * 5, 3, 4, 0),                         # equal sequences that do not line up
+    (True, 128, 1, 4, [640] * 40, 3, 4, 0),                         # many short equal sequences per workgroup
+])
+def test_any_batch_as_one_kernel(gpu, oracle, lloyd, d, Hkv, Hq, lens, kb, vb, waves):
+    """Batches whose regions do not line up with the workgroups (ragged, or equal but unaligned): the wavefronts'
+    partials go through memory, the workgroup that arrives last at a region merges it, and the call is still one
+    kernel.  Against the checker and the three-kernel way, with prefix lengths, twice in a row."""
+    import torch
+    rng = np.random.default_rng(59)
+    S, L = len(lens), max(lens)
+    wl = workloads.Workload("any", S, Hq, Hkv, d, lens, kb, vb, 0, 0, 0)
+    K = rng.standard_normal((S, Hkv, L, d), dtype=np.float32)
+    V = rng.standard_normal((S, Hkv, L, d), dtype=np.float32)
+    q = rng.standard_normal((S, Hq, d), dtype=np.float32)
+    Rk, Rv = rotations(oracle, d, 11)
+    mode = gpu.KV_LLOYDMAX if lloyd else gpu.KV_UNIFORM
+    cache = build_cache(gpu, wl, mode, K, V, rotations=(Rk, Rv), scales=None if lloyd else (1.0, 1.0), rotate=1)
+    flags = gpu.ATTN_ROTATE_Q | gpu.ATTN_UNROTATE_OUT
+    want = checker_output(oracle, gpu, cache, wl, q, False, Rk=Rk, Rv=Rv)
+    prefix = [max(0, n - 1 - 13 * s) for s, n in enumerate(lens)]
+    prefix[S // 2] = 0
+    wl_p = workloads.Workload("any", S, Hq, Hkv, d, prefix, kb, vb, 0, 0, 0)
+    want_p = checker_output(oracle, gpu, cache, wl_p, q, False, Rk=Rk, Rv=Rv)
+    lens_dev = torch.tensor(prefix, dtype=torch.int32, device="cuda")
+    try:
+        gpu.profile_reset()
+        gpu.profile_enable(True)
+        gpu.decode_tuning(waves)
+        one_kernel = run_decode(gpu, cache, q, gpu.GQA_BLOCKED, flags)
+        again = run_decode(gpu, cache, q, gpu.GQA_BLOCKED, flags)
+        qd = dev(q)
+        out = torch.zeros_like(qd)
+        cache.decode_attn_prefix(lens_dev, qd, out, gqa_mapping=gpu.GQA_BLOCKED, flags=flags)
+        gpu.sync()
+        one_kernel_p = out.cpu().numpy()
+        assert gpu.profile_read("kv_decode_attn")[1] == 3 and gpu.profile_read("kv_decode_combine")[1] == 0
+        gpu.decode_tuning(waves, separate_query=True)
+        own_merge = run_decode(gpu, cache, q, gpu.GQA_BLOCKED, flags)
+        gpu.decode_tuning(waves, separate_merge=True, separate_query=True)
+        three_kernels = run_decode(gpu, cache, q, gpu.GQA_BLOCKED, flags)
+        assert gpu.profile_read("kv_decode_combine")[1] == 1
+    finally:
+        gpu.profile_enable(False)
+        gpu.decode_tuning()
+    assert_attn_close(three_kernels, want, "three kernels")
+    assert_attn_close(own_merge, want, "own merge")
+    assert_attn_close(one_kernel, want, "one kernel")
+    assert_attn_close(one_kernel_p, want_p, "one kernel, prefix lengths")
+    np.testing.assert_allclose(one_kernel, three_kernels, rtol=2e-5, atol=2e-6)
+    assert np.all(one_kernel_p[S // 2] == 0.0)
+    assert np.array_equal(again, one_kernel)
+    cache.close()
+
+
 def test_edge_lengths(gpu, oracle):
     """Empty sequences give zeros; lengths 1, 63, 64, 65 around the 64-token block; an appended token changes the
     result exactly as the checker says."""

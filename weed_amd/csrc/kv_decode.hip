@@ -943,6 +943,7 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
     // equal sequences of nb blocks each, nb a multiple of one cycle of the age classes' runs, and a workgroup's blocks
     // a multiple of nb.  They then also rotate their regions' queries themselves, and the call is ONE kernel.
     uint32_t wg_regions = 0, region_wgs = 0;
+    bool general_merge = false;
     bool fused_query = false;
     if (use_mfma && total_blocks) {
         uniform_blocks = ((uint32_t)c->lens[0] + 63u) >> 6;
@@ -964,13 +965,47 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
             // small batches of long sequences: every region is a whole number of workgroups' shares
             region_wgs = nb / wg_blocks;
         }
-        // Equal sequences: a workgroup's blocks lie in at most (wg_blocks - 1) / nb + 2 regions, whose queries it
-        // rotates itself when they are few enough for its LDS; nothing then runs ahead of the matrix-core kernel.
-        const uint32_t wg_most_regions = wg_regions ? wg_regions : (nb ? (wg_blocks - 1) / nb + 2 : 0);
-        fused_query = mfma_decode_merges(gp, d) && nb != 0 && wg_most_regions * pass_heads <= kMfmaQueryRows &&
-                      !decode_tuning().separate_query;
+        // Most regions that the blocks of one workgroup lie in (exact: the host knows the cached lengths).
+        uint32_t wg_most_regions = wg_regions;
+        bool every_sequence_has_tokens = true;
+        if (wg_regions == 0) {
+            std::vector<uint64_t> region_end; // blocks up to and including region r
+            region_end.reserve((size_t)S * Hkv);
+            uint64_t run = 0;
+            for (int32_t l : c->lens) {
+                const uint32_t b = ((uint32_t)l + 63u) >> 6;
+                every_sequence_has_tokens = every_sequence_has_tokens && b != 0;
+                for (uint32_t h = 0; h < Hkv; ++h) {
+                    run += b;
+                    region_end.push_back(run);
+                }
+            }
+            size_t r = 0;
+            for (uint64_t first = 0; first < total_blocks; first += wg_blocks) {
+                const uint64_t last = std::min<uint64_t>(first + wg_blocks, total_blocks) - 1;
+                while (region_end[r] <= first) {
+                    ++r;
+                }
+                size_t r1 = r;
+                while (region_end[r1] <= last) {
+                    ++r1;
+                }
+                wg_most_regions = std::max(wg_most_regions, (uint32_t)(r1 - r + 1));
+            }
+        }
+        // Anything else that the instance can merge: one slot per (run, region) in memory, an arrival counter per
+        // region (ragged batches: up to 63 sequences, whose block offsets a wavefront keeps in one register).
+        if (wg_regions == 0 && region_wgs == 0 && mfma_decode_merges(gp, d) && every_sequence_has_tokens &&
+            (nb != 0 || (S <= 63 && !decode_tuning().always_search)) && n_splits <= 64 && wg_most_regions <= 31 &&
+            (size_t)S * Hkv <= kMfmaMergeCounters && !decode_tuning().separate_merge) {
+            general_merge = true;
+        }
+        // A workgroup rotates the queries of the regions its blocks lie in itself when they are few enough for its
+        // LDS (equal sequences, or the ragged batches above); nothing then runs ahead of the matrix-core kernel.
+        fused_query = mfma_decode_merges(gp, d) && (nb != 0 || general_merge) &&
+                      wg_most_regions * pass_heads <= kMfmaQueryRows && !decode_tuning().separate_query;
     }
-    const bool fused_merge = wg_regions != 0 || region_wgs != 0;
+    const bool fused_merge = wg_regions != 0 || region_wgs != 0 || general_merge;
     // (the kernels that take one (sequence, head) row per workgroup have the sequence on a 16-bit grid dimension)
     WEED_HIP_REQUIRE(S <= 65535u || (use_mfma && many_rows && n_splits <= 64),
                      "%s: %u sequences in one call are served only for head_dims that are multiples of 64 with "
@@ -1010,7 +1045,9 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         mp.n_seq = S;
         mp.total_blocks = total_blocks;
         mp.uniform_blocks = uniform_blocks;
-        mp.merge = MfmaMerge{ wg_regions, region_wgs, arrive, d_real, out_dev, og, c->v.rot, unrot ? 1 : 0 };
+        mp.merge = MfmaMerge{ wg_regions, region_wgs, general_merge ? 1u : 0u, arrive, d_real, out_dev, og, c->v.rot,
+                              unrot ? 1 : 0 };
+        mp.cached_lens = c->lens_dev;
         mp.query = MfmaQuery{ fused_query ? q_dev : nullptr, qg, c->k.rot_t, rot_q ? 1 : 0 };
         mp.runs = runs;
         mp.max_slots = n_splits;

@@ -130,9 +130,15 @@ __device__ __forceinline__ uint64_t head_offset(const Geom3 &g, uint32_t hv)
 // itself in `arrive[region]`; the workgroup that completes the count merges the region's partials, un-rotates and
 // writes the output rows, and puts the counter back to zero (so the counters are zero between launches; whoever
 // allocates them clears them once).
+// `general` (wg_regions and region_wgs 0): anything else -- ragged batches (up to 63 sequences: a wavefront then
+// keeps the prefix sums of the sequences' block counts in a register), equal sequences that do not line up.  The
+// wavefronts store their partials through to device scope as one slot per (run, region); a workgroup that is done
+// counts itself in `arrive` of every region it has blocks of, and the workgroup that completes a region's count merges
+// that region's slots from memory.
 struct MfmaMerge {
     uint32_t wg_regions;
     uint32_t region_wgs;
+    uint32_t general;
     uint32_t *arrive;  // [n_seq * Hkv] arrival counters, zero when the launch starts
     uint32_t d_real;   // coordinates the caller's rows have (<= the stored head_dim)
     float *out;        // attention output
@@ -168,8 +174,8 @@ constexpr uint32_t mfma_merge_partials_words(uint32_t waves, uint32_t gp, uint32
 }
 constexpr uint32_t mfma_merge_lds_bytes(uint32_t waves, uint32_t gp, uint32_t d)
 {
-    // (+ 4 words at the end: the arrival count that one thread reads for the workgroup)
-    return 4u * (mfma_merge_partials_words(waves, gp, d) + kMfmaMergeRows * d + kMfmaMergeThreads * kMfmaMergeRows + 4u);
+    // (+ 64 words at the end: the arrival count that one thread reads for the workgroup, or one per region)
+    return 4u * (mfma_merge_partials_words(waves, gp, d) + kMfmaMergeRows * d + kMfmaMergeThreads * kMfmaMergeRows + 64u);
 }
 // Arrival counters that a workspace reserves.
 constexpr uint32_t kMfmaMergeCounters = 16384;
@@ -194,6 +200,7 @@ struct MfmaParams {
     const uint32_t *table_image; // mfma_table_rows(k.w, v.w) * 64 words, see mfma_table_word
     const uint32_t *blk_off; // [n_seq + 1] prefix sums of the sequences' block counts (cached lengths)
     const int32_t *lens;
+    const int32_t *cached_lens; // the lengths the block list was made from (lens may be shorter: prefix attention)
     uint32_t Hq, G;
     int blocked;            // 1: kv = h / G, 0: kv = h % Hkv (Weed)
     // multi-token chunks: the G "heads" of a KV head are (position, head) pairs, q_tokens positions x real_group

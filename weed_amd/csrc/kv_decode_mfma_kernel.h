@@ -369,7 +369,7 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     const uint32_t g1 = min(g0 + run_len(p.runs, (unit % kWaves) % run_classes(p.runs)), p.total_blocks);
     // ---- merge inside the kernel (see MfmaMerge): LDS behind the tables, and this thread's share of the rotation ----
     static_assert(!WGM || mfma_decode_merges(GP, D), "this instance cannot merge");
-    constexpr bool kCanMerge = WGM;
+    constexpr bool kCanMerge = mfma_decode_merges(GP, D);
     constexpr uint32_t NG = kMfmaMergeThreads / D; // groups of source coordinates of the un-rotation
     constexpr bool kQuery = mfma_decode_merges(GP, D);   // this instance can rotate its queries itself (MfmaQuery)
     constexpr uint32_t JPG = kQuery ? D / (NG ? NG : 1) : 1; // source coordinates per group
@@ -406,7 +406,61 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     float *const qscale_s = part_s + PW + kMfmaQueryRows * D;         // [rows]
     float *const qsum_s = qscale_s + kMfmaQueryRows;                  // [rows]
     const bool fused_q = kQuery && p.query.q != nullptr;
-    // the regions this workgroup's blocks lie in (equal sequences of uniform_blocks blocks each)
+    // ---- general merge (see MfmaMerge): in a ragged batch every wavefront keeps the prefix sums of the sequences'
+    //      block counts in a register, lane i the blocks ahead of sequence i (lanes from n_seq on: all blocks) ----
+    const bool general = kQuery && !WGM && p.merge.general != 0;
+    const bool own_offsets = general && p.uniform_blocks == 0;
+    uint32_t off_lane = 0;
+    if constexpr (kQuery && !WGM) {
+        if (own_offsets) {
+            const uint32_t nbl = lane < p.n_seq ? ((uint32_t)p.cached_lens[lane] + 63u) >> 6 : 0u;
+            uint32_t incl = nbl;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                const uint32_t t = __shfl_up(incl, o);
+                incl += lane >= (uint32_t)o ? t : 0u;
+            }
+            off_lane = incl - nbl;
+        }
+    }
+    // blocks ahead of sequence i (i the same in all lanes)
+    auto blk_off_at = [&](uint32_t i) -> uint32_t {
+        if (p.uniform_blocks) {
+            return i * p.uniform_blocks;
+        }
+        if (own_offsets) {
+            return (uint32_t)__builtin_amdgcn_readlane((int)off_lane, (int)i);
+        }
+        return p.blk_off[i];
+    };
+    // sequence that holds block b of the list (b the same in all lanes): the largest s with blk_off[s] * Hkv <= b
+    // (sequences without tokens share their offset with the next one)
+    auto seq_of_block = [&](uint32_t b) -> uint32_t {
+        if (p.uniform_blocks) {
+            return b / (p.uniform_blocks * p.Hkv);
+        }
+        if (own_offsets) {
+            const bool le = lane < p.n_seq && off_lane * p.Hkv <= b; // true for a prefix of the lanes, lane 0 included
+            return (uint32_t)__builtin_popcountll(__ballot(le)) - 1u;
+        }
+        // a 64-way search, one probe per lane and step
+        uint32_t lo = 0, hi = p.n_seq;
+        while (hi - lo > 1) {
+            const uint32_t stride = (hi - lo + 63) >> 6;
+            const uint32_t idx = lo + lane * stride;
+            const bool le = idx < hi && p.blk_off[idx] * p.Hkv <= b; // true for a prefix of the lanes, lane 0 included
+            const uint32_t n_le = (uint32_t)__builtin_popcountll(__ballot(le));
+            lo += (n_le - 1) * stride;
+            hi = min(lo + stride, hi);
+        }
+        return __builtin_amdgcn_readfirstlane(lo);
+    };
+    // region (sequence * Hkv + kv head) that holds block b
+    auto region_of_block = [&](uint32_t b) -> uint32_t {
+        const uint32_t s_ = seq_of_block(b), first = blk_off_at(s_), nb_ = blk_off_at(s_ + 1) - first;
+        return s_ * p.Hkv + (b - first * p.Hkv) / nb_;
+    };
+    // the regions this workgroup's blocks lie in
     uint32_t wg_region0 = 0, wg_rows = 0;
     if (WGM && p.merge.wg_regions != 0) {
         wg_region0 = blockIdx.x * p.merge.wg_regions;
@@ -414,11 +468,11 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     } else if (WGM) {
         wg_region0 = (blockIdx.x * kWaves * p.runs.unit_blocks) / p.uniform_blocks; // a share of one region
         wg_rows = p.G;
-    } else if (fused_q) {
+    } else if (fused_q || general) {
         const uint32_t wg_blocks = kWaves * p.runs.unit_blocks;
         const uint32_t first = blockIdx.x * wg_blocks, last = min(first + wg_blocks, p.total_blocks) - 1;
-        wg_region0 = first / p.uniform_blocks;
-        wg_rows = (last / p.uniform_blocks - wg_region0 + 1) * p.G;
+        wg_region0 = region_of_block(first);
+        wg_rows = (region_of_block(last) - wg_region0 + 1) * p.G;
     }
     float xq[kQuery ? JPG : 1], qr[QPT];
     if constexpr (kQuery) {
@@ -552,21 +606,8 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     const uint32_t uniform_nb = p.uniform_blocks;
     if (g0 >= g1) {
         // (nothing to find)
-    } else if (uniform_nb) {
-        seq = g0 / (uniform_nb * p.Hkv);
     } else {
-        // largest s with blk_off[s] * Hkv <= g0 (sequences without tokens share their offset with the next one):
-        // a 64-way search, one probe per lane and step
-        uint32_t lo = 0, hi = p.n_seq;
-        while (hi - lo > 1) {
-            const uint32_t stride = (hi - lo + 63) >> 6;
-            const uint32_t idx = lo + lane * stride;
-            const bool le = idx < hi && p.blk_off[idx] * p.Hkv <= g0; // true for a prefix of the lanes, lane 0 included
-            const uint32_t n_le = (uint32_t)__builtin_popcountll(__ballot(le));
-            lo += (n_le - 1) * stride;
-            hi = min(lo + stride, hi);
-        }
-        seq = __builtin_amdgcn_readfirstlane(lo);
+        seq = seq_of_block(g0);
     }
     if constexpr (kQuery && !WGM) {
         // (ahead of the loop over the segments, which must not carry the requested elements around)
@@ -576,9 +617,9 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
         }
     }
     while (g0 < g1) {
-    const uint32_t seq_first = uniform_nb ? seq * uniform_nb : p.blk_off[seq];
+    const uint32_t seq_first = blk_off_at(seq);
     // blocks the cached length of this sequence spans
-    const uint32_t nb_cap = uniform_nb ? uniform_nb : p.blk_off[seq + 1] - seq_first;
+    const uint32_t nb_cap = uniform_nb ? uniform_nb : blk_off_at(seq + 1) - seq_first;
     if constexpr (!WGM) {
         if (nb_cap == 0) {
             ++seq;
@@ -1003,7 +1044,8 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
 #pragma unroll
                 for (int jb = 0; jb < JB; ++jb) {
                     // uniform coder: value = step * (code + 0.5) + lo, so add lo * sum(p)
-                    dst[2 + 16 * jb + c] = fmaf(O[jb][r], o_mul, p.v.beta * lrow[r]);
+                    const float v = fmaf(O[jb][r], o_mul, p.v.beta * lrow[r]);
+                    dst[2 + 16 * jb + c] = v;
                 }
             }
         }
@@ -1030,9 +1072,16 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     } // segments
 
     // ---- the workgroup's merge: rows (region, head) in passes of kMfmaMergeRows ----
-    if constexpr (WGM) {
-        if (!kEarlyRotation && !has_blocks) {
-            request_rotation(); // (the others did so before they left their partial)
+    if constexpr (kQuery) {
+        if constexpr (WGM) {
+            if (!kEarlyRotation && !has_blocks) {
+                request_rotation(); // (the others did so before they left their partial)
+            }
+        } else {
+            if (!general) {
+                return; // a second kernel merges
+            }
+            request_rotation();
         }
         constexpr int PS = D + 2;
         constexpr uint32_t RP = kMfmaMergeRows;
@@ -1075,7 +1124,7 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
             }
         };
         // un-rotation of the rows in o_s and the output rows of the regions region0 + ri
-        auto finish_rows = [&](uint32_t r0, uint32_t rows, uint32_t region0) {
+        auto finish_rows = [&](uint32_t r0, uint32_t rows, auto region_of) {
             __syncthreads();
             if (p.merge.unrotate) {
                 if (tid < kMfmaMergeThreads) {
@@ -1102,7 +1151,7 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
             for (uint32_t rr = rr_of_wave; rr < RP; rr += kThreads / D) {
                 const uint32_t row = r0 + rr;
                 const uint32_t ri = row / p.G, hs = row - ri * p.G;
-                if (row < rows && region0 + ri < n_regions && col < p.merge.d_real) {
+                if (row < rows && region_of(ri) < n_regions && col < p.merge.d_real) {
                     float v;
                     if (p.merge.unrotate) {
                         v = 0.0f;
@@ -1113,7 +1162,7 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
                     } else {
                         v = o_s[rr * D + col];
                     }
-                    const uint32_t region = region0 + ri;
+                    const uint32_t region = region_of(ri);
                     const uint32_t s_ = region / p.Hkv, kv_ = region - s_ * p.Hkv;
                     p.merge.out[(uint64_t)p.merge.og.off + (uint64_t)s_ * p.merge.og.s[0] +
                                 head_offset(p.merge.og, q_head_of(p, kv_, hs)) + (uint64_t)col * p.merge.og.s[2]] = v;
@@ -1121,6 +1170,117 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
             }
             __syncthreads(); // before the next pass overwrites the rows
         };
+        // `count` regions, region_of(i) with slots_of(i) partials each (at most 64, the host sees to that), from memory,
+        // in passes of RP rows.  Lane k of every wavefront reads the header of its row's partial k, the wavefront's 64
+        // columns of the partials come eight partials at a time; all of these loads are independent of each other (and
+        // of device scope), so a pass costs two trips to memory, not one per partial.  Then the rows are finished.
+        auto finish_regions_from_memory = [&](uint32_t count, auto region_of, auto slots_of) {
+            const uint32_t rows = count * p.G;
+            for (uint32_t r0 = 0; r0 < rows; r0 += RP) {
+                for (uint32_t rr = rr_of_wave; rr < RP; rr += kThreads / D) {
+                    const uint32_t row = r0 + rr;
+                    float v = 0.0f;
+                    if (row < rows) {
+                        const uint32_t ri = row / p.G, hs = row - ri * p.G;
+                        const uint32_t region = region_of(ri), slots = slots_of(ri);
+                        const uint32_t s_ = region / p.Hkv, kv_ = region - s_ * p.Hkv;
+                        const float *first = p.partials + ((uint64_t)s_ * p.Hq + q_head_of(p, kv_, hs)) * p.max_slots * PS;
+                        const __amdgpu_buffer_rsrc_t src = buffer_of(first, slots * (4 * PS));
+                        float m0 = buffer_f32<true>(src, lane * (4 * PS), 0), l0 = buffer_f32<true>(src, lane * (4 * PS), 4);
+                        float y[8];
+#pragma unroll
+                        for (uint32_t u = 0; u < 8; ++u) {
+                            y[u] = buffer_f32<true>(src, 4 * col, 4 * (min(u, slots - 1) * PS + 2));
+                        }
+                        if (lane >= slots) {
+                            m0 = -INFINITY;
+                            l0 = 0.0f;
+                        }
+                        const float mx = wave_max64(m0);
+                        const float w0 = (m0 == -INFINITY) ? 0.0f : exp2f(m0 - mx);
+                        const float den = wave_sum64(w0 * l0);
+                        float acc = 0.0f;
+                        for (uint32_t k0 = 0; k0 < slots; k0 += 8) {
+                            float z[8];
+                            if (k0 + 8 < slots) {
+#pragma unroll
+                                for (uint32_t u = 0; u < 8; ++u) {
+                                    z[u] = buffer_f32<true>(src, 4 * col, 4 * (min(k0 + 8 + u, slots - 1) * PS + 2));
+                                }
+                            }
+#pragma unroll
+                            for (uint32_t u = 0; u < 8; ++u) {
+                                if (k0 + u < slots) {
+                                    acc = fmaf(lane_value(w0, k0 + u), y[u], acc);
+                                }
+                            }
+#pragma unroll
+                            for (uint32_t u = 0; u < 8; ++u) {
+                                y[u] = z[u];
+                            }
+                        }
+                        v = den > 0.0f ? acc / den : 0.0f;
+                    }
+                    o_s[rr * D + col] = v;
+                }
+                finish_rows(r0, rows, region_of);
+            }
+        };
+        if constexpr (!WGM) {
+            // General case: this wavefront's partials are stored; when every wavefront's are, the workgroup counts
+            // itself in every region it has blocks of (thread t: region wg_region0 + t), and merges those whose count
+            // it completes.
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            const uint32_t wg_regions_here = wg_rows / p.G, wg_blocks = kWaves * p.runs.unit_blocks;
+            if (wave == 0) {
+                // The partials were ordinary stores (stores of device scope between a wavefront's segments would hold
+                // up the loads of its next segment, which wait on the same counter): they sit in this XCD's L2, and ONE
+                // write-back per workgroup makes them visible to the others before the arrivals are counted.
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+                // (all lanes compute: the offsets travel between lanes)
+                const uint32_t region = min(wg_region0 + lane, n_regions - 1);
+                const uint32_t s_ = region / p.Hkv, kv_ = region - s_ * p.Hkv;
+                uint32_t first, nb_;
+                if (p.uniform_blocks) {
+                    first = s_ * p.uniform_blocks;
+                    nb_ = p.uniform_blocks;
+                } else {
+                    first = __shfl(off_lane, (int)s_);
+                    nb_ = __shfl(off_lane, (int)(s_ + 1)) - first;
+                }
+                const uint32_t begin = first * p.Hkv + kv_ * nb_, end = begin + nb_ - 1; // (the host refuses empty ones)
+                const uint32_t wgs = end / wg_blocks - begin / wg_blocks + 1;
+                const uint32_t slots = run_of_block(p.runs, end) - run_of_block(p.runs, begin) + 1;
+                uint32_t before_plus_one = 0;
+                if (lane < wg_regions_here) {
+                    uint32_t before = 0;
+                    if (wgs > 1) {
+                        before = __hip_atomic_fetch_add(p.merge.arrive + region, 1u, __ATOMIC_RELAXED,
+                                                        __HIP_MEMORY_SCOPE_AGENT);
+                        if (before + 1 == wgs) {
+                            __hip_atomic_store(p.merge.arrive + region, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        }
+                    }
+                    before_plus_one = before + 1;
+                }
+                // the regions to merge, packed: count_s[1 + 2 i] = region, count_s[2 + 2 i] = its slots, count_s[0] = how many
+                // (at most 31, the host sees to that)
+                const bool mine = lane < wg_regions_here && before_plus_one == wgs;
+                const uint64_t mask = __ballot(mine);
+                if (mine) {
+                    const uint32_t at = (uint32_t)__builtin_popcountll(mask & ((1ull << lane) - 1ull));
+                    count_s[1 + 2 * at] = region;
+                    count_s[2 + 2 * at] = slots;
+                }
+                if (lane == 0) {
+                    count_s[0] = (uint32_t)__builtin_popcountll(mask);
+                }
+            }
+            __syncthreads();
+            finish_regions_from_memory(
+                count_s[0], [&](uint32_t i) { return count_s[1 + 2 * i]; }, [&](uint32_t i) { return count_s[2 + 2 * i]; });
+        } else {
         __syncthreads(); // every wavefront's partial is in LDS (and nobody reads the tables any more)
         if (p.merge.wg_regions != 0) {
             // whole regions: slots = wavefronts per region
@@ -1130,7 +1290,7 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
             };
             for (uint32_t r0 = 0; r0 < rows; r0 += RP) {
                 merge_rows(r0, rows, slots, in_lds, std::true_type{}, [](uint32_t, uint32_t, float, float, float) {});
-                finish_rows(r0, rows, blockIdx.x * p.merge.wg_regions);
+                finish_rows(r0, rows, [&](uint32_t ri) { return blockIdx.x * p.merge.wg_regions + ri; });
             }
         } else {
             // A share of ONE region (p.G <= RP rows): the wavefronts' partials become one partial of the region in
@@ -1169,52 +1329,9 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
             if (tid == 0) {
                 __hip_atomic_store(p.merge.arrive + region, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
-            // The region's partials (at most 64, the host sees to that): lane k of every wavefront reads the header
-            // of partial k, the wavefront's 64 columns of the partials come eight partials at a time; all of these
-            // loads are independent of each other, so a row costs two trips to memory, not one per partial.
-            const uint32_t slots = p.merge.region_wgs;
-            for (uint32_t rr = rr_of_wave; rr < RP; rr += kThreads / D) {
-                float v = 0.0f;
-                if (rr < p.G) {
-                    const __amdgpu_buffer_rsrc_t src = buffer_of(slot_of(rr, 0), slots * (4 * PS));
-                    float m0 = buffer_f32<true>(src, lane * (4 * PS), 0), l0 = buffer_f32<true>(src, lane * (4 * PS), 4);
-                    float y[8];
-#pragma unroll
-                    for (uint32_t u = 0; u < 8; ++u) {
-                        y[u] = buffer_f32<true>(src, 4 * col, 4 * (min(u, slots - 1) * PS + 2));
-                    }
-                    if (lane >= slots) {
-                        m0 = -INFINITY;
-                        l0 = 0.0f;
-                    }
-                    const float mx = wave_max64(m0);
-                    const float w0 = (m0 == -INFINITY) ? 0.0f : exp2f(m0 - mx);
-                    const float den = wave_sum64(w0 * l0);
-                    float acc = 0.0f;
-                    for (uint32_t k0 = 0; k0 < slots; k0 += 8) {
-                        float z[8];
-                        if (k0 + 8 < slots) {
-#pragma unroll
-                            for (uint32_t u = 0; u < 8; ++u) {
-                                z[u] = buffer_f32<true>(src, 4 * col, 4 * (min(k0 + 8 + u, slots - 1) * PS + 2));
-                            }
-                        }
-#pragma unroll
-                        for (uint32_t u = 0; u < 8; ++u) {
-                            if (k0 + u < slots) {
-                                acc = fmaf(lane_value(w0, k0 + u), y[u], acc);
-                            }
-                        }
-#pragma unroll
-                        for (uint32_t u = 0; u < 8; ++u) {
-                            y[u] = z[u];
-                        }
-                    }
-                    v = den > 0.0f ? acc / den : 0.0f;
-                }
-                o_s[rr * D + col] = v;
-            }
-            finish_rows(0, p.G, region);
+            finish_regions_from_memory(
+                1, [&](uint32_t) { return region; }, [&](uint32_t) { return p.merge.region_wgs; });
+        }
         }
     }
 }
@@ -1254,7 +1371,8 @@ template <int D, int WK, int WV, int GP, bool LLOYD> int launch_gp(const MfmaPar
         }
     } else {
         // (the area behind the tables is where a workgroup rotates its queries, when it does)
-        decode_mfma_kernel<D, WK, WV, GP, LLOYD, false><<<grid, 64 * waves, p.query.q ? smem_merging : smem, s>>>(p);
+        decode_mfma_kernel<D, WK, WV, GP, LLOYD, false>
+            <<<grid, 64 * waves, (p.query.q || p.merge.general) ? smem_merging : smem, s>>>(p);
     }
     WEED_HIP_LAUNCH_CHECK();
     return WEED_HIP_OK;
