@@ -370,22 +370,52 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     // ---- merge inside the kernel (see MfmaMerge): LDS behind the tables, and this thread's share of the rotation ----
     static_assert(!WGM || mfma_decode_merges(GP, D), "this instance cannot merge");
     constexpr bool kCanMerge = mfma_decode_merges(GP, D);
-    constexpr uint32_t NG = kMfmaMergeThreads / D; // groups of source coordinates of the un-rotation
     constexpr bool kQuery = mfma_decode_merges(GP, D);   // this instance can rotate its queries itself (MfmaQuery)
-    constexpr uint32_t JPG = kQuery ? D / (NG ? NG : 1) : 1; // source coordinates per group
     float *const part_s = reinterpret_cast<float *>(lds) + ROWS * (kTableRowBytes / 4); // [position][GP][D + 2]
-    float xrot[kCanMerge ? JPG : 1];
-    auto request_rotation = [&]() {
-        // thread (group jg, coordinate t) of the first kMfmaMergeThreads takes rv[jg * JPG + u][t], u < JPG; the group
-        // is the same in all lanes of a wavefront
+    // The two small rotations (queries ahead of the loop, merged rows behind it) run on the fp32 matrix instruction
+    // v_mfma_f32_16x16x4f32: wavefront w < D / 16 owns the output columns [16 w, 16 w + 16) of up to 16 rows.  Step s of
+    // D / 4 contracts over the coordinates 4 s + g (g = lane / 16): lane (c, g) supplies row c's coordinate 4 s + g
+    // from LDS and the rotation's element [4 s + g][16 w + c], which it holds in a register.  The rows lie in LDS as
+    // [row][g][s] with a pitch of D + 4 floats, so that a lane's D / 4 values are contiguous (16-byte reads) and the
+    // sixteen rows' reads fall into different banks.
+    constexpr uint32_t SG = D / 4;       // steps = coordinates per lane
+    constexpr uint32_t RPITCH = D + 4;   // floats per staged row
+    auto staged_at = [](uint32_t row, uint32_t j) { return row * RPITCH + (j % 4) * SG + j / 4; };
+    // element s of the lane's share of a rotation matrix m (row-major [D][D], out[t] = sum_j in[j] * m[j][t])
+    auto request_matrix = [&](const float *m, float (&x)[kCanMerge ? SG : 1]) {
         if constexpr (kCanMerge) {
-            if (p.merge.unrotate && tid < kMfmaMergeThreads) {
-                const __amdgpu_buffer_rsrc_t rot = buffer_of(p.merge.rv, 4 * D * D);
-                const uint32_t t = tid % D, jg = tid / D;
+            if (wave < D / 16) {
+                const __amdgpu_buffer_rsrc_t rot = buffer_of(m, 4 * D * D);
 #pragma unroll
-                for (uint32_t u = 0; u < JPG; ++u) {
-                    xrot[u] = buffer_f32(rot, 4 * (jg * JPG * D + t), 4 * D * u);
+                for (uint32_t s_ = 0; s_ < SG; ++s_) {
+                    x[s_] = buffer_f32(rot, 4 * (g * D + 16 * wave + c), 16 * D * s_);
                 }
+            }
+        }
+    };
+    // rows r0 .. r0 + 15 of `staged` (staged_at layout) times the matrix whose elements the lane holds in x: lane
+    // (c, g), register v of the result = row r0 + 4 g + v, column 16 w + c
+    auto rotate_staged = [&](const float *staged, uint32_t r0, const float (&x)[kCanMerge ? SG : 1]) -> float4v {
+        float4v acc = { 0.0f, 0.0f, 0.0f, 0.0f };
+        if constexpr (kCanMerge) {
+            const float4v *mine = reinterpret_cast<const float4v *>(staged + (r0 + c) * RPITCH + g * SG);
+            float4v in[SG / 4];
+#pragma unroll
+            for (uint32_t u = 0; u < SG / 4; ++u) {
+                in[u] = mine[u];
+            }
+#pragma unroll
+            for (uint32_t s_ = 0; s_ < SG; ++s_) {
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(in[s_ / 4][s_ % 4], x[s_], acc, 0, 0, 0);
+            }
+        }
+        return acc;
+    };
+    float xrot[kCanMerge ? SG : 1];
+    auto request_rotation = [&]() {
+        if constexpr (kCanMerge) {
+            if (p.merge.unrotate) {
+                request_matrix(p.merge.rv, xrot);
             }
         }
     };
@@ -399,8 +429,8 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     //      ri * G + hs.  Requested here: this thread's share of the K rotation and of the raw queries. ----
     constexpr uint32_t QPT = kQuery ? (kMfmaQueryRows * D + kThreads - 1) / kThreads : 1; // raw query elements per thread
     constexpr uint32_t PW = mfma_merge_partials_words(kWaves, GP, D);
-    float *const qraw_s = part_s;                              // [rows][D]
-    float *const qred_s = part_s + kMfmaQueryRows * D;         // [NG][kMfmaMergeRows][D]
+    float *const qraw_s = part_s;                                       // [rows (+ 8 that a tile of 16 reaches into)] staged
+    float *const qrot_s = part_s + (kMfmaQueryRows + 8) * RPITCH;       // [kMfmaMergeRows][D] rotated rows of a pass
     uint16_t *const qh_s = reinterpret_cast<uint16_t *>(part_s + PW); // [rows][D] fp16 high halves
     uint16_t *const ql_s = qh_s + kMfmaQueryRows * D;                 // [rows][D] low halves
     float *const qscale_s = part_s + PW + kMfmaQueryRows * D;         // [rows]
@@ -474,16 +504,11 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
         wg_region0 = region_of_block(first);
         wg_rows = (region_of_block(last) - wg_region0 + 1) * p.G;
     }
-    float xq[kQuery ? JPG : 1], qr[QPT];
+    float xq[kQuery ? SG : 1], qr[QPT];
     if constexpr (kQuery) {
         if (fused_q) {
-            if (p.query.rotate && tid < kMfmaMergeThreads) {
-                const __amdgpu_buffer_rsrc_t rot = buffer_of(p.query.rot_t, 4 * D * D);
-                const uint32_t t = tid % D, ig = tid / D;
-#pragma unroll
-                for (uint32_t u = 0; u < JPG; ++u) {
-                    xq[u] = buffer_f32(rot, 4 * (ig * JPG * D + t), 4 * D * u);
-                }
+            if (p.query.rotate) {
+                request_matrix(p.query.rot_t, xq);
             }
             const uint32_t n_regions = p.n_seq * p.Hkv;
             // element e = tid + i * kThreads of the rows: its row is the same in all lanes of a wavefront (kThreads is
@@ -507,16 +532,15 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
             }
         }
     }
-    // The workgroup's queries: rotated by all threads (thread (group ig, coordinate t) sums its JPG source coordinates
-    // for every row, the groups' sums are added in a fixed order), then one wavefront per row scales, normalises and
-    // splits the row as the stand-alone kernel does.  Contains the tables' barrier; every wavefront calls it once.
+    // The workgroup's queries: rotated on the matrix instruction (see rotate_staged), then one wavefront per row scales,
+    // normalises and splits the row as the stand-alone kernel does.  Contains the tables' barrier; every wavefront calls it once.
     auto rotate_queries = [&]() {
         if constexpr (kQuery) {
 #pragma unroll
             for (uint32_t i = 0; i < QPT; ++i) {
                 const uint32_t e = tid + i * kThreads;
                 if (e < kMfmaQueryRows * D) {
-                    qraw_s[e] = qr[i];
+                    qraw_s[staged_at(e / D, e % D)] = qr[i];
                 }
             }
             build_tables(); // (its barrier also makes the raw queries visible)
@@ -525,21 +549,13 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
             }
             for (uint32_t r0 = 0; r0 < wg_rows; r0 += kMfmaMergeRows) {
                 if (p.query.rotate) {
-                    if (tid < kMfmaMergeThreads) {
-                        const uint32_t t = tid % D, ig = tid / D;
+                    if (wave < D / 16) {
+                        const float4v rot = rotate_staged(qraw_s, r0, xq);
+                        if (g < kMfmaMergeRows / 4) {
 #pragma unroll
-                        for (uint32_t rr = 0; rr < kMfmaMergeRows; ++rr) {
-                            float acc = 0.0f;
-                            const float4v *qrow = reinterpret_cast<const float4v *>(qraw_s + (r0 + rr) * D + ig * JPG);
-#pragma unroll
-                            for (uint32_t u4 = 0; u4 < JPG / 4; ++u4) {
-                                const float4v qv = qrow[u4];
-#pragma unroll
-                                for (uint32_t i = 0; i < 4; ++i) {
-                                    acc = fmaf(qv[i], xq[4 * u4 + i], acc);
-                                }
+                            for (uint32_t v = 0; v < 4; ++v) {
+                                qrot_s[(4 * g + v) * D + 16 * wave + c] = rot[v];
                             }
-                            qred_s[(ig * kMfmaMergeRows + rr) * D + t] = acc;
                         }
                     }
                     __syncthreads();
@@ -554,15 +570,7 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
                     for (uint32_t cc = 0; cc < CPL; ++cc) {
                         const uint32_t j = lane + 64 * cc;
                         float v;
-                        if (p.query.rotate) {
-                            v = 0.0f;
-#pragma unroll
-                            for (uint32_t ig = 0; ig < NG; ++ig) {
-                                v += qred_s[(ig * kMfmaMergeRows + wave) * D + j];
-                            }
-                        } else {
-                            v = qraw_s[row * D + j];
-                        }
+                        v = p.query.rotate ? qrot_s[wave * D + j] : qraw_s[staged_at(row, j)];
                         a[cc] = v;
                         const float qc = v * k;
                         mx = fmaxf(mx, fabsf(qc));
@@ -1085,9 +1093,8 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
         }
         constexpr int PS = D + 2;
         constexpr uint32_t RP = kMfmaMergeRows;
-        float *const o_s = part_s + PW;               // [RP][D] merged, normalised rows
-        float *const red_s = o_s + RP * D;            // [NG][RP][D] partial sums of the un-rotation
-        uint32_t *const count_s = reinterpret_cast<uint32_t *>(red_s + kMfmaMergeThreads * RP);
+        float *const o_s = part_s + PW;               // [RP (+ 8 that a tile of 16 reaches into)] merged, normalised rows, staged
+        uint32_t *const count_s = reinterpret_cast<uint32_t *>(o_s + RP * D + kMfmaMergeThreads * RP); // (the area's end)
         const uint32_t n_regions = p.n_seq * p.Hkv;
         // (the row of an element is the same in all lanes of a wavefront: kThreads is a multiple of D)
         const uint32_t rr_of_wave = __builtin_amdgcn_readfirstlane(tid / D), col = tid % D;
@@ -1096,21 +1103,32 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
         // left as the partial (m, l, o) that leave(rr, m, l, o) puts somewhere
         auto merge_rows = [&](uint32_t r0, uint32_t rows, uint32_t slots, auto partial, auto normalise, auto leave) {
             constexpr bool NORMALISE = decltype(normalise)::value;
+            constexpr uint32_t KS = kWaves; // most partials of a row (one per wavefront)
             for (uint32_t rr = rr_of_wave; rr < RP; rr += kThreads / D) {
                 const uint32_t row = r0 + rr;
                 float v = 0.0f;
                 if (row < rows) {
                     const uint32_t ri = row / p.G, hs = row - ri * p.G;
+                    // all reads first (slots that do not exist read the last one again), so that they travel together
+                    float m[KS], l[KS], o[KS];
+#pragma unroll
+                    for (uint32_t k = 0; k < KS; ++k) {
+                        const uint32_t kk = min(k, slots - 1);
+                        m[k] = partial(ri, hs, kk, 0u);
+                        l[k] = partial(ri, hs, kk, 1u);
+                        o[k] = partial(ri, hs, kk, 2u + col);
+                    }
                     float mx = -INFINITY;
-                    for (uint32_t k = 0; k < slots; ++k) {
-                        mx = fmaxf(mx, partial(ri, hs, k, 0u));
+#pragma unroll
+                    for (uint32_t k = 0; k < KS; ++k) {
+                        mx = k < slots ? fmaxf(mx, m[k]) : mx;
                     }
                     float den = 0.0f, acc = 0.0f;
-                    for (uint32_t k = 0; k < slots; ++k) {
-                        const float m = partial(ri, hs, k, 0u);
-                        const float w = (m == -INFINITY) ? 0.0f : exp2f(m - mx);
-                        den = fmaf(w, partial(ri, hs, k, 1u), den);
-                        acc = fmaf(w, partial(ri, hs, k, 2u + col), acc);
+#pragma unroll
+                    for (uint32_t k = 0; k < KS; ++k) {
+                        const float w = (k >= slots || m[k] == -INFINITY) ? 0.0f : exp2f(m[k] - mx);
+                        den = fmaf(w, l[k], den);
+                        acc = fmaf(w, o[k], acc);
                     }
                     if constexpr (NORMALISE) {
                         v = den > 0.0f ? acc / den : 0.0f;
@@ -1119,56 +1137,41 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
                     }
                 }
                 if constexpr (NORMALISE) {
-                    o_s[rr * D + col] = v;
+                    o_s[staged_at(rr, col)] = v;
                 }
             }
         };
-        // un-rotation of the rows in o_s and the output rows of the regions region0 + ri
-        auto finish_rows = [&](uint32_t r0, uint32_t rows, auto region_of) {
-            __syncthreads();
-            if (p.merge.unrotate) {
-                if (tid < kMfmaMergeThreads) {
-                    const uint32_t t = tid % D, jg = tid / D;
-#pragma unroll
-                    for (uint32_t rr = 0; rr < RP; ++rr) {
-                        float acc = 0.0f;
-                        // (JPG is a multiple of 4; the merged row is read four coordinates at a time, every lane the
-                        // same address)
-                        const float4v *orow = reinterpret_cast<const float4v *>(o_s + rr * D + jg * JPG);
-#pragma unroll
-                        for (uint32_t u4 = 0; u4 < JPG / 4; ++u4) {
-                            const float4v ov = orow[u4];
-#pragma unroll
-                            for (uint32_t i = 0; i < 4; ++i) {
-                                acc = fmaf(ov[i], xrot[4 * u4 + i], acc);
-                            }
-                        }
-                        red_s[(jg * RP + rr) * D + t] = acc;
-                    }
-                }
-                __syncthreads();
-            }
-            for (uint32_t rr = rr_of_wave; rr < RP; rr += kThreads / D) {
+        // un-rotation of the rows in o_s and the output rows of the regions region_of(ri); `more`: another pass follows
+        auto finish_rows = [&](uint32_t r0, uint32_t rows, auto region_of, bool more) {
+            __syncthreads(); // the merged rows are complete
+            auto store_row = [&](uint32_t rr, uint32_t column, float v) {
                 const uint32_t row = r0 + rr;
                 const uint32_t ri = row / p.G, hs = row - ri * p.G;
-                if (row < rows && region_of(ri) < n_regions && col < p.merge.d_real) {
-                    float v;
-                    if (p.merge.unrotate) {
-                        v = 0.0f;
-#pragma unroll
-                        for (uint32_t jg = 0; jg < NG; ++jg) {
-                            v += red_s[(jg * RP + rr) * D + col];
-                        }
-                    } else {
-                        v = o_s[rr * D + col];
-                    }
+                if (row < rows && region_of(ri) < n_regions && column < p.merge.d_real) {
                     const uint32_t region = region_of(ri);
                     const uint32_t s_ = region / p.Hkv, kv_ = region - s_ * p.Hkv;
                     p.merge.out[(uint64_t)p.merge.og.off + (uint64_t)s_ * p.merge.og.s[0] +
-                                head_offset(p.merge.og, q_head_of(p, kv_, hs)) + (uint64_t)col * p.merge.og.s[2]] = v;
+                                head_offset(p.merge.og, q_head_of(p, kv_, hs)) + (uint64_t)column * p.merge.og.s[2]] = v;
+                }
+            };
+            if (p.merge.unrotate) {
+                if (wave < D / 16) {
+                    const float4v out = rotate_staged(o_s, 0, xrot);
+                    if (g < RP / 4) {
+#pragma unroll
+                        for (uint32_t v = 0; v < 4; ++v) {
+                            store_row(4 * g + v, 16 * wave + c, out[v]);
+                        }
+                    }
+                }
+            } else {
+                for (uint32_t rr = rr_of_wave; rr < RP; rr += kThreads / D) {
+                    store_row(rr, col, o_s[staged_at(rr, col)]);
                 }
             }
-            __syncthreads(); // before the next pass overwrites the rows
+            if (more) {
+                __syncthreads(); // before the next pass overwrites the rows
+            }
         };
         // `count` regions, region_of(i) with slots_of(i) partials each (at most 64, the host sees to that), from memory,
         // in passes of RP rows.  Lane k of every wavefront reads the header of its row's partial k, the wavefront's 64
@@ -1221,9 +1224,9 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
                         }
                         v = den > 0.0f ? acc / den : 0.0f;
                     }
-                    o_s[rr * D + col] = v;
+                    o_s[staged_at(rr, col)] = v;
                 }
-                finish_rows(r0, rows, region_of);
+                finish_rows(r0, rows, region_of, r0 + RP < rows);
             }
         };
         if constexpr (!WGM) {
@@ -1290,7 +1293,7 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
             };
             for (uint32_t r0 = 0; r0 < rows; r0 += RP) {
                 merge_rows(r0, rows, slots, in_lds, std::true_type{}, [](uint32_t, uint32_t, float, float, float) {});
-                finish_rows(r0, rows, [&](uint32_t ri) { return blockIdx.x * p.merge.wg_regions + ri; });
+                finish_rows(r0, rows, [&](uint32_t ri) { return blockIdx.x * p.merge.wg_regions + ri; }, r0 + RP < rows);
             }
         } else {
             // A share of ONE region (p.G <= RP rows): the wavefronts' partials become one partial of the region in
