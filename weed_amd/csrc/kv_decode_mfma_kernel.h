@@ -419,12 +419,9 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
             }
         }
     };
-    // With two wavefronts per SIMD the registers have room for the rotation elements all along: they are requested
+    // With two wavefronts per SIMD the registers have room for the un-rotation's elements all along: they are requested
     // here; with three, when the wavefront is through with its blocks.
     constexpr bool kEarlyRotation = WGM && kWaves == 8;
-    if constexpr (kEarlyRotation) {
-        request_rotation();
-    }
     // ---- query rotation inside the kernel (see MfmaQuery).  Row (region ri of the workgroup, head slot hs) has index
     //      ri * G + hs.  Requested here: this thread's share of the K rotation and of the raw queries. ----
     constexpr uint32_t QPT = kQuery ? (kMfmaQueryRows * D + kThreads - 1) / kThreads : 1; // raw query elements per thread
@@ -505,7 +502,8 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
         wg_rows = (region_of_block(last) - wg_region0 + 1) * p.G;
     }
     float xq[kQuery ? SG : 1], qr[QPT];
-    if constexpr (kQuery) {
+    auto request_queries = [&]() {
+      if constexpr (kQuery) {
         if (fused_q) {
             if (p.query.rotate) {
                 request_matrix(p.query.rot_t, xq);
@@ -531,6 +529,13 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
                 qr[i] = v;
             }
         }
+      }
+    };
+    // (Asking for the first block of packed data before these requests gets that block on its way 2 us earlier and the
+    // loop going 0.7 us earlier, and the kernel 0.6 us slower: measured, not kept.)
+    request_queries();
+    if constexpr (kEarlyRotation) {
+        request_rotation();
     }
     // The workgroup's queries: rotated on the matrix instruction (see rotate_staged), then one wavefront per row scales,
     // normalises and splits the row as the stand-alone kernel does.  Contains the tables' barrier; every wavefront calls it once.
@@ -1095,6 +1100,9 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
         constexpr uint32_t RP = kMfmaMergeRows;
         float *const o_s = part_s + PW;               // [RP (+ 8 that a tile of 16 reaches into)] merged, normalised rows, staged
         uint32_t *const count_s = reinterpret_cast<uint32_t *>(o_s + RP * D + kMfmaMergeThreads * RP); // (the area's end)
+        // where the pass's rows go: element offset of row rr's first coordinate in the output (~0: no such row), found
+        // once per row while the rows are merged
+        unsigned long long *const rowbase_s = reinterpret_cast<unsigned long long *>(o_s + 16 * RPITCH);
         const uint32_t n_regions = p.n_seq * p.Hkv;
         // (the row of an element is the same in all lanes of a wavefront: kThreads is a multiple of D)
         const uint32_t rr_of_wave = __builtin_amdgcn_readfirstlane(tid / D), col = tid % D;
@@ -1126,12 +1134,13 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
                     float den = 0.0f, acc = 0.0f;
 #pragma unroll
                     for (uint32_t k = 0; k < KS; ++k) {
-                        const float w = (k >= slots || m[k] == -INFINITY) ? 0.0f : exp2f(m[k] - mx);
+                        // (the bare instruction, as in the main loop: arguments are <= 0, and a weight below 2^-126 is none)
+                        const float w = (k >= slots || m[k] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(m[k] - mx);
                         den = fmaf(w, l[k], den);
                         acc = fmaf(w, o[k], acc);
                     }
                     if constexpr (NORMALISE) {
-                        v = den > 0.0f ? acc / den : 0.0f;
+                        v = den > 0.0f ? acc * __builtin_amdgcn_rcpf(den) : 0.0f;
                     } else {
                         leave(ri, hs, mx, den, acc);
                     }
@@ -1143,15 +1152,23 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
         };
         // un-rotation of the rows in o_s and the output rows of the regions region_of(ri); `more`: another pass follows
         auto finish_rows = [&](uint32_t r0, uint32_t rows, auto region_of, bool more) {
-            __syncthreads(); // the merged rows are complete
-            auto store_row = [&](uint32_t rr, uint32_t column, float v) {
-                const uint32_t row = r0 + rr;
+            if (tid < RP) {
+                const uint32_t row = r0 + tid;
                 const uint32_t ri = row / p.G, hs = row - ri * p.G;
-                if (row < rows && region_of(ri) < n_regions && column < p.merge.d_real) {
+                unsigned long long base = ~0ull;
+                if (row < rows && region_of(ri) < n_regions) {
                     const uint32_t region = region_of(ri);
                     const uint32_t s_ = region / p.Hkv, kv_ = region - s_ * p.Hkv;
-                    p.merge.out[(uint64_t)p.merge.og.off + (uint64_t)s_ * p.merge.og.s[0] +
-                                head_offset(p.merge.og, q_head_of(p, kv_, hs)) + (uint64_t)column * p.merge.og.s[2]] = v;
+                    base = (uint64_t)p.merge.og.off + (uint64_t)s_ * p.merge.og.s[0] +
+                           head_offset(p.merge.og, q_head_of(p, kv_, hs));
+                }
+                rowbase_s[tid] = base;
+            }
+            __syncthreads(); // the merged rows are complete
+            auto store_row = [&](uint32_t rr, uint32_t column, float v) {
+                const unsigned long long base = rowbase_s[rr];
+                if (base != ~0ull && column < p.merge.d_real) {
+                    p.merge.out[base + (uint64_t)column * p.merge.og.s[2]] = v;
                 }
             };
             if (p.merge.unrotate) {
