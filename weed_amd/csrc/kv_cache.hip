@@ -1011,13 +1011,14 @@ int upload_table_image(weed_hip_kv_cache *c)
     if (!words) {
         return WEED_HIP_OK;
     }
-    std::vector<uint32_t> img(words);
-    for (uint32_t i = 0; i < words; ++i) {
-        img[i] = mfma_table_word(i, k.w, v.w, kl, vl);
+    // what the kernel reads: one word per 32 equal words of the LDS image (an entry's replicas over the banks)
+    std::vector<uint32_t> img(words / 32);
+    for (uint32_t i = 0; i < words / 32; ++i) {
+        img[i] = mfma_table_word(32 * i, k.w, v.w, kl, vl);
     }
     // kernels already enqueued may still read the old image
     WEED_HIP_CHECK(hipStreamSynchronize(stream()));
-    WEED_HIP_CHECK(hipMemcpy(c->table_image, img.data(), sizeof(uint32_t) * words, hipMemcpyHostToDevice));
+    WEED_HIP_CHECK(hipMemcpy(c->table_image, img.data(), sizeof(uint32_t) * img.size(), hipMemcpyHostToDevice));
     return WEED_HIP_OK;
 }
 

@@ -80,7 +80,7 @@ constexpr uint32_t mfma_table_rows(uint32_t wk, uint32_t wv)
 }
 constexpr uint32_t kMfmaTableRowBytes = 256;
 constexpr uint32_t kMfmaTableImageBytes = 256 * kMfmaTableRowBytes; // the largest image (4-bit pair tables)
-// Word i of the image a workgroup copies into LDS before its first block: entry e = i / 64 of the V table in the
+// Word i of the image a workgroup builds in LDS before its first block (32 equal words in a row, held once in memory): entry e = i / 64 of the V table in the
 // first 32 words of row e (one replica per bank), of the K table in the last 32.  `k_levels` / `v_levels`: the fp16 bit
 // patterns of the 2^w reconstruction levels of each side.
 inline uint32_t mfma_table_word(uint32_t i, uint32_t wk, uint32_t wv, const uint16_t *k_levels, const uint16_t *v_levels)
@@ -197,7 +197,7 @@ struct MfmaParams {
     uint32_t Hkv, n_seq;
     uint32_t padded;
     MfmaSide k, v;
-    const uint32_t *table_image; // mfma_table_rows(k.w, v.w) * 64 words, see mfma_table_word
+    const uint32_t *table_image; // mfma_table_rows(k.w, v.w) * 2 words: word j = word 32 j of the LDS image (mfma_table_word)
     const uint32_t *blk_off; // [n_seq + 1] prefix sums of the sequences' block counts (cached lengths)
     const int32_t *lens;
     const int32_t *cached_lens; // the lengths the block list was made from (lens may be shorter: prefix attention)

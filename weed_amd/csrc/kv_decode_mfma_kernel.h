@@ -335,10 +335,12 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     constexpr uint32_t kImgLoads = (kImgVecs + kThreads - 1) / kThreads;
     uint4v timg[kImgLoads ? kImgLoads : 1];
     if constexpr (ROWS != 0) {
-        const uint4v *img = reinterpret_cast<const uint4v *>(p.table_image);
+        // (the image in memory holds every entry once; its 32 replicas over the banks are made here: 16-byte piece i
+        // of the LDS image is four times word i / 8)
 #pragma unroll
         for (uint32_t u = 0; u < kImgLoads; ++u) {
-            timg[u] = img[min(tid + u * kThreads, kImgVecs - 1)];
+            const uint32_t w = p.table_image[min(tid + u * kThreads, kImgVecs - 1) / 8];
+            timg[u] = uint4v{ w, w, w, w };
         }
     }
     auto build_tables = [&]() {
