@@ -421,9 +421,9 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
             }
         }
     };
-    // With two wavefronts per SIMD the registers have room for the un-rotation's elements all along: they are requested
-    // here; with three, when the wavefront is through with its blocks.
-    constexpr bool kEarlyRotation = WGM && kWaves == 8;
+    // (The un-rotation's elements are requested when the wavefront is through with its blocks.  Requesting them at the
+    // start, where two wavefronts per SIMD have the registers for them, adds 16 MB of L2 traffic to the start of the
+    // launch and made the kernel 0.4 us slower.)
     // ---- query rotation inside the kernel (see MfmaQuery).  Row (region ri of the workgroup, head slot hs) has index
     //      ri * G + hs.  Requested here: this thread's share of the K rotation and of the raw queries. ----
     constexpr uint32_t QPT = kQuery ? (kMfmaQueryRows * D + kThreads - 1) / kThreads : 1; // raw query elements per thread
@@ -536,9 +536,6 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     // (Asking for the first block of packed data before these requests gets that block on its way 2 us earlier and the
     // loop going 0.7 us earlier, and the kernel 0.6 us slower: measured, not kept.)
     request_queries();
-    if constexpr (kEarlyRotation) {
-        request_rotation();
-    }
     // The workgroup's queries: rotated on the matrix instruction (see rotate_staged), then one wavefront per row scales,
     // normalises and splits the row as the stand-alone kernel does.  Contains the tables' barrier; every wavefront calls it once.
     auto rotate_queries = [&]() {
@@ -1073,9 +1070,7 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
         }
     };
     if constexpr (WGM) {
-        if constexpr (!kEarlyRotation) {
-            request_rotation(); // on its way while the partial is put together
-        }
+        request_rotation(); // on its way while the partial is put together
         leave_partial(std::true_type{});
         break; // (the only segment: for the compiler this is no loop, so nothing is carried around it)
     } else {
@@ -1089,7 +1084,7 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     // ---- the workgroup's merge: rows (region, head) in passes of kMfmaMergeRows ----
     if constexpr (kQuery) {
         if constexpr (WGM) {
-            if (!kEarlyRotation && !has_blocks) {
+            if (!has_blocks) {
                 request_rotation(); // (the others did so before they left their partial)
             }
         } else {
