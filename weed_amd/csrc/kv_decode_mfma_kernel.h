@@ -11,8 +11,12 @@
 //      log2(e) are folded into the query),
 //   4. splits the probabilities (times the V row scales) into fp16 hi + lo, which are already in A-operand order,
 //      and multiplies them with the looked-up V items: out[head][coordinate] accumulates in 4*(d/16) registers.
-// The wavefronts of a workgroup share the lookup tables and nothing else; every wavefront writes one un-normalised
-// partial (m, l, o[d]) per query head and region segment, and a second kernel merges the partials.
+// The wavefronts of a workgroup share the lookup tables; every wavefront leaves one un-normalised partial (m, l, o[d])
+// per query head and region segment.  Where the instance allows it (groups of up to 8 heads at head_dim 64 or 128) the
+// kernel is the whole decode call: the workgroup rotates, scales and splits the queries of its regions before its first
+// block arrives (MfmaQuery), and the partials are merged, un-rotated and stored by the workgroup itself -- through LDS
+// when it holds whole regions, through memory and an arrival counter per region otherwise (MfmaMerge).  Else a kernel
+// ahead prepares the queries and one behind merges the partials.
 //
 // Table values are exactly representable in fp16 (the Lloyd-Max tables are generated that way; the uniform coder's
 // table is code + 0.5), so de-quantisation itself is exact; the only roundings are those of the fp32 accumulators.
@@ -321,9 +325,9 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     const uint32_t c = lane & 15, g = lane >> 4;
     constexpr bool lloyd = LLOYD;
 
-    // ---- the lookup tables.  Their LDS image was built when the cache's tables were set; the workgroup copies it,
-    //      16 bytes per thread and step.  The image is requested first thing and stored after the wavefront has
-    //      requested its first block and query, so that those loads travel meanwhile.  Every wavefront of the
+    // ---- the lookup tables.  Their words were put together when the cache's tables were set; the workgroup spreads
+    //      them over the LDS banks, 16 bytes per thread and step.  The words are requested first thing and stored after
+    //      the wavefront has requested its first block and query, so that those loads travel meanwhile.  Every wavefront of the
     //      workgroup calls build_tables exactly once (it contains a barrier). ----
     // The arguments span six 64-byte lines of kernel-argument memory, each a miss of its own when first touched.
     // Naming one value of every line here makes the compiler fetch all of them at once instead of one after the other
