@@ -248,7 +248,10 @@ def test_equal_contexts_with_and_without_the_region_search(gpu, oracle):
     (True, 128, 2, 8, 2, 768, 2, 2, 24, True),      # three wavefronts per SIMD: three age classes
     (True, 64, 4, 4, 8, 768, 3, 3, 96, True),       # groups of one, four regions per workgroup
     (False, 128, 1, 2, 8, 2048, 8, 8, 64, True),    # 8-bit uniform codes (no lookup tables)
+    (True, 128, 2, 32, 4, 1024, 3, 4, 32, True),    # groups of 16 (the sixteen-column instance), 32 rows per workgroup
+    (False, 64, 1, 16, 6, 768, 4, 4, 0, True),      # groups of 16 at head_dim 64, whatever the natural geometry gives
     # regions of several workgroups' shares: the workgroup that arrives last at a region merges it
+    (True, 128, 1, 16, 1, 2048, 3, 4, 16, True),    # groups of 16, two workgroups per region
     (True, 128, 2, 8, 1, 2048, 3, 4, 32, True),     # two workgroups per region
     (True, 128, 1, 4, 1, 8192, 3, 4, 128, True),    # sixteen workgroups per region
     (True, 128, 2, 8, 2, 1536, 2, 2, 96, True),     # three wavefronts per SIMD
@@ -318,6 +321,7 @@ def test_workgroups_that_merge_their_own_regions(gpu, oracle, lloyd, d, Hkv, Hq,
     (False, 64, 2, 16, [1000, 333, 90, 2500], 4, 4, 0),             # uniform coder, head_dim 64, groups of 8
     (True, 128, 2, 8, [1500] * 5, 3, 4, 0),                         # equal sequences that do not line up
     (True, 128, 1, 4, [640] * 40, 3, 4, 0),                         # many short equal sequences per workgroup
+    (True, 128, 1, 16, [3000, 700, 1300], 3, 4, 0),                 # groups of 16, ragged
 ])
 def test_any_batch_as_one_kernel(gpu, oracle, lloyd, d, Hkv, Hq, lens, kb, vb, waves):
     """Batches whose regions do not line up with the workgroups (ragged, or equal but unaligned): the wavefronts'

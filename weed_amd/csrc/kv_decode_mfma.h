@@ -157,8 +157,8 @@ struct MfmaQuery {
 };
 constexpr uint32_t kMfmaQueryRows = 32;
 
-// Instances that can merge: groups of up to 8 heads at head_dim 64 or 128.
-constexpr bool mfma_decode_merges(uint32_t gp, uint32_t d) { return gp <= 8 && (d == 64u || d == 128u); }
+// Instances that can merge: head_dim 64 or 128.
+constexpr bool mfma_decode_merges(uint32_t gp, uint32_t d) { return gp <= 16 && (d == 64u || d == 128u); }
 // Rows (region, head) that one pass of the merge takes, threads of its un-rotation, and its LDS behind the tables:
 // the wavefronts' partials [waves][gp][d + 2], the merged rows [rows][d], the un-rotation's partial sums
 // [threads / d][rows][d].

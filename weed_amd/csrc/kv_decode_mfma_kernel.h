@@ -714,17 +714,27 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
                 rotate_queries();
                 tables_ready = true;
             }
-            const uint32_t col_head = c % GP, col_part = c / GP; // (PACKED: merging instances have GP <= 8)
+            const uint32_t col_head = PACKED ? c % GP : c;
+            const uint32_t col_part = PACKED ? c / GP : 0; // 0: high half, 1: low half, above: unused column
             const bool col_ok = col_head < p.G && col_part < 2;
-            const uint32_t row = ((uint32_t)region - wg_region0) * p.G + (col_ok ? col_head : 0);
-            const uint16_t *src = (col_part ? ql_s : qh_s) + row * D + g * (D / 4);
+            const uint32_t at = (((uint32_t)region - wg_region0) * p.G + (col_ok ? col_head : 0)) * D + g * (D / 4);
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                uint4v v = { 0, 0, 0, 0 };
+                uint4v hi = { 0, 0, 0, 0 }, lo = { 0, 0, 0, 0 };
                 if (col_ok) {
-                    v = *reinterpret_cast<const uint4v *>(src + 8 * ks);
+                    if (!PACKED || col_part == 0) {
+                        hi = *reinterpret_cast<const uint4v *>(qh_s + at + 8 * ks);
+                    }
+                    if (!PACKED || col_part == 1) {
+                        lo = *reinterpret_cast<const uint4v *>(ql_s + at + 8 * ks);
+                    }
                 }
-                qop[0][ks] = __builtin_bit_cast(half8, v);
+                if constexpr (PACKED) {
+                    qop[0][ks] = __builtin_bit_cast(half8, col_part ? lo : hi);
+                } else {
+                    qop[0][ks] = __builtin_bit_cast(half8, hi);
+                    qop[NQ - 1][ks] = __builtin_bit_cast(half8, lo);
+                }
             }
         }
     } else {
@@ -1314,7 +1324,7 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
                 finish_rows(r0, rows, [&](uint32_t ri) { return blockIdx.x * p.merge.wg_regions + ri; }, r0 + RP < rows);
             }
         } else {
-            // A share of ONE region (p.G <= RP rows): the wavefronts' partials become one partial of the region in
+            // A share of ONE region: the wavefronts' partials become one partial of the region in
             // memory, stored through to device scope; when those stores have completed the workgroup counts itself,
             // and the workgroup that completes the region's count reads all of the region's partials with loads of
             // device scope and finishes the rows.  (No cache-wide write-back or invalidation: every wavefront issuing
@@ -1329,7 +1339,8 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
             auto slot_of = [&](uint32_t hs, uint32_t k) {
                 return p.partials + (((uint64_t)s_ * p.Hq + q_head_of(p, kv_, hs)) * p.max_slots + k) * PS;
             };
-            merge_rows(0, p.G, kWaves, in_lds, std::false_type{},
+            for (uint32_t r0 = 0; r0 < p.G; r0 += RP)
+            merge_rows(r0, p.G, kWaves, in_lds, std::false_type{},
                        [&](uint32_t, uint32_t hs, float m, float l, float o) {
                            float *dst = slot_of(hs, my_slot);
                            __hip_atomic_store(dst + 2 + col, o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
