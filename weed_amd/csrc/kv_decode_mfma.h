@@ -159,29 +159,33 @@ constexpr uint32_t kMfmaQueryRows = 32;
 
 // Instances that can merge: head_dim 64 or 128.
 constexpr bool mfma_decode_merges(uint32_t gp, uint32_t d) { return gp <= 16 && (d == 64u || d == 128u); }
-// Rows (region, head) that one pass of the merge takes, threads of its un-rotation, and its LDS behind the tables:
-// the wavefronts' partials [waves][gp][d + 2], the merged rows [rows][d], the un-rotation's partial sums
-// [threads / d][rows][d].
+// Rows (region, head) that one pass of the merge or of the query rotation takes (the matrix instruction behind both
+// has 16 rows, so a pass reads 8 rows beyond its own), and the LDS of both behind the lookup tables, in words.
+// Rows are staged for the matrix instruction with a pitch of d + 4 words.
+//   Area A: the wavefronts' partials [waves][gp][d + 2] at the end of the kernel; at its start the staged raw queries
+//           [kMfmaQueryRows + 8][d + 4] and the rotated rows of a pass [kMfmaMergeRows][d].
+//   Area B: at the end the staged merged rows of a pass [kMfmaMergeRows + 8][d + 4], the pass's output row addresses
+//           (2 words each) and 64 words of arrival counts; at the start the queries' fp16 halves
+//           [kMfmaQueryRows][d] each (d words per row together), a scale and a sum per row.
 constexpr uint32_t kMfmaMergeRows = 8;
-constexpr uint32_t kMfmaMergeThreads = 512;
-// The query rotation works in the same LDS before the first block: the raw queries [kMfmaQueryRows][d] and the
-// rotation's partial sums [threads / d][rows][d] where the partials will be, and its results (fp16 halves
-// [kMfmaQueryRows][d] each, a scale and a sum per row) where the merged rows and the un-rotation's sums will be.
 constexpr uint32_t mfma_merge_partials_words(uint32_t waves, uint32_t gp, uint32_t d)
 {
-    const uint32_t partials = waves * gp * (d + 2u), query = kMfmaQueryRows * d + kMfmaMergeThreads * kMfmaMergeRows;
+    const uint32_t partials = waves * gp * (d + 2u);
+    const uint32_t query = (kMfmaQueryRows + 8u) * (d + 4u) + kMfmaMergeRows * d;
     return partials > query ? partials : query;
+}
+constexpr uint32_t mfma_merge_rows_words(uint32_t d)
+{
+    const uint32_t merged = (kMfmaMergeRows + 8u) * (d + 4u) + 2u * kMfmaMergeRows;
+    const uint32_t query = kMfmaQueryRows * d + 2u * kMfmaQueryRows;
+    return (merged > query ? merged : query) + 64u;
 }
 constexpr uint32_t mfma_merge_lds_bytes(uint32_t waves, uint32_t gp, uint32_t d)
 {
-    // (+ 64 words at the end: the arrival count that one thread reads for the workgroup, or one per region)
-    return 4u * (mfma_merge_partials_words(waves, gp, d) + kMfmaMergeRows * d + kMfmaMergeThreads * kMfmaMergeRows + 64u);
+    return 4u * (mfma_merge_partials_words(waves, gp, d) + mfma_merge_rows_words(d));
 }
 // Arrival counters that a workspace reserves.
 constexpr uint32_t kMfmaMergeCounters = 16384;
-static_assert(kMfmaQueryRows * 128u + 2u * kMfmaQueryRows <= kMfmaMergeRows * 128u + kMfmaMergeThreads * kMfmaMergeRows &&
-                  kMfmaQueryRows * 64u + 2u * kMfmaQueryRows <= kMfmaMergeRows * 64u + kMfmaMergeThreads * kMfmaMergeRows,
-              "the query halves, scales and sums fit where the merged rows and the un-rotation's sums will be");
 
 // Kernel arguments.  What a wavefront needs before it can request its first block comes first, so that it arrives
 // with the first kernel-argument fetches.

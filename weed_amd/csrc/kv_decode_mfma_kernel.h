@@ -1110,7 +1110,7 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
         constexpr int PS = D + 2;
         constexpr uint32_t RP = kMfmaMergeRows;
         float *const o_s = part_s + PW;               // [RP (+ 8 that a tile of 16 reaches into)] merged, normalised rows, staged
-        uint32_t *const count_s = reinterpret_cast<uint32_t *>(o_s + RP * D + kMfmaMergeThreads * RP); // (the area's end)
+        uint32_t *const count_s = reinterpret_cast<uint32_t *>(o_s + mfma_merge_rows_words(D) - 64); // (the area's end)
         // where the pass's rows go: element offset of row rr's first coordinate in the output (~0: no such row), found
         // once per row while the rows are merged
         unsigned long long *const rowbase_s = reinterpret_cast<unsigned long long *>(o_s + 16 * RPITCH);
