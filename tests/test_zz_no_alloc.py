@@ -83,3 +83,34 @@ def test_noalloc_refuses_shapes_beyond_its_workspace(gpu):
     gpu.sync()
     assert bool(torch.isfinite(out).all())
     cache.close()
+
+
+@pytest.mark.parametrize("n_seq,ctx", [(1, 2048), (8, 1024), (3, 1000)])
+def test_noalloc_call_replayed_from_a_graph(gpu, oracle, n_seq, ctx):
+    """The allocation-free entry point under graph capture: the captured call is one kernel whose workgroups count
+    their arrivals per region and leave the counters at zero, so every replay must give the bits of the eager call,
+    also with eager calls of another shape in between."""
+    import torch
+    flags = gpu.ATTN_ROTATE_Q | gpu.ATTN_UNROTATE_OUT
+    wl = workloads.Workload("graph", n_seq, 8, 2, 128, [ctx] * n_seq, 3, 4, 0, 0, 31)
+    cache, q, _, _ = _cache(gpu, oracle, wl, 9)
+    other = workloads.Workload("graph_b", 2, 4, 2, 64, [130, 37], 2, 3, 1, 0, 32)
+    cache_b, q_b, _, _ = _cache(gpu, oracle, other, 10)
+    qd, qb = dev(q), dev(q_b)
+    eager = torch.zeros_like(qd)
+    cache.decode_attn_noalloc(qd, eager, gqa_mapping=gpu.GQA_BLOCKED, flags=flags)
+    gpu.sync()
+    out = torch.full_like(qd, float("nan"))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=torch.cuda.current_stream()):
+        cache.decode_attn_noalloc(qd, out, gqa_mapping=gpu.GQA_BLOCKED, flags=flags)
+    for _ in range(4):
+        out.fill_(float("nan"))
+        graph.replay()
+        gpu.sync()
+        assert np.array_equal(out.cpu().numpy(), eager.cpu().numpy())
+        ob = torch.zeros_like(qb)
+        cache_b.decode_attn_noalloc(qb, ob, gqa_mapping=gpu.GQA_BLOCKED, flags=flags)
+        gpu.sync()
+    cache.close()
+    cache_b.close()
