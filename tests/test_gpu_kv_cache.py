@@ -527,11 +527,80 @@ def test_cfg5a_encode_full_size(gpu, oracle):
     cache.close()
 
 
+@pytest.mark.parametrize("lloyd,kw,vw,d,rotate", [(True, (3, 1), (3, 0), 128, 1), (True, (2, 0), (4, 1), 96, 0),
+                                                  (True, (4, 1), (1, 0), 256, 1), (False, (8, 0), (8, 0), 64, 0),
+                                                  (False, (5, 0), (3, 0), 32, 1), (False, (1, 0), (7, 0), 160, 0)])
+def test_one_token_appends_are_finished_by_the_encoder(gpu, lloyd, kw, vw, d, rotate):
+    """A decode step's append (one token for each of a run of sequences) is one kernel: the encoder puts the new
+    fields into their items itself, next to the fields of the tokens already cached, and the last workgroup moves
+    the lengths.  Seventy such steps over sequences of different lengths (every place a token can have in a 64-token
+    block, more rows than one workgroup takes, a last workgroup that is not full, runs that leave sequences out)
+    must give, bit for bit, the cache that one append per sequence gives, and the same attention."""
+    import torch
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(d + kw[0])
+    S, Hkv, cap = 5, 9, 160
+    mode = gpu.KV_LLOYDMAX if lloyd else gpu.KV_UNIFORM
+    a = gpu.KVCache(mode, S, Hkv, d, cap, kw[0], vw[0], kw[1], vw[1])
+    b = gpu.KVCache(mode, S, Hkv, d, cap, kw[0], vw[0], kw[1], vw[1])
+    rk, rv = torch.zeros(d * d, device="cuda"), torch.zeros(d * d, device="cuda")
+    gpu.make_rotation(3, d, rk)
+    gpu.make_rotation(4, d, rv)
+    for c in (a, b):
+        if not lloyd:
+            c.set_scales(1.3, 0.9)
+        c.set_rotations(rk, rv)
+    K = torch.randn((S, Hkv, cap, d), generator=gen, device="cuda") * 2
+    V = torch.randn((S, Hkv, cap, d), generator=gen, device="cuda")
+    lens = [0, 3, 31, 64, 70]
+    for s in range(S):
+        if lens[s]:
+            a.encode_append(K[s:s + 1, :, :lens[s]], V[s:s + 1, :, :lens[s]], seq_begin=s, rotate=rotate)
+    for step in range(70):
+        s0, n = (0, S) if step % 3 else (step % 4, min(2, S - step % 4))
+        k1 = torch.stack([K[s, :, lens[s]:lens[s] + 1] for s in range(s0, s0 + n)])
+        v1 = torch.stack([V[s, :, lens[s]:lens[s] + 1] for s in range(s0, s0 + n)])
+        a.encode_append(k1, v1, seq_begin=s0, rotate=rotate)
+        for s in range(s0, s0 + n):
+            lens[s] += 1
+    assert a.seq_lens() == lens
+    for s in range(S):
+        b.encode_append(K[s:s + 1, :, :lens[s]], V[s:s + 1, :, :lens[s]], seq_begin=s, rotate=rotate)
+    for which in (0, 1):
+        fa, sa = export(a, which, max(lens))
+        fb, sb = export(b, which, max(lens))
+        for s in range(S):
+            assert np.array_equal(fa[s, :, :lens[s]], fb[s, :, :lens[s]]), (which, s)
+            assert np.array_equal(sa[s, :, :lens[s]], sb[s, :, :lens[s]]), (which, s)
+    q = torch.randn((S, Hkv * 2, d), generator=gen, device="cuda")
+    oa, ob = torch.zeros_like(q), torch.zeros_like(q)
+    a.decode_attn(q, oa)
+    b.decode_attn(q, ob)
+    gpu.sync()
+    assert torch.equal(oa, ob)
+    # a cache that is reset starts over: items that still hold the old tokens' fields are rebuilt from their first field
+    a.reset()
+    b.reset()
+    for t in range(3):
+        a.encode_append(V[:, :, t:t + 1], K[:, :, t:t + 1], rotate=rotate)
+    b.encode_append(V[:, :, :3], K[:, :, :3], rotate=rotate)
+    for which in (0, 1):
+        fa, sa = export(a, which, 3)
+        fb, sb = export(b, which, 3)
+        assert np.array_equal(fa, fb) and np.array_equal(sa, sb), which
+    a.decode_attn(q, oa)
+    b.decode_attn(q, ob)
+    gpu.sync()
+    assert torch.equal(oa, ob)
+    a.close()
+    b.close()
+
+
 def test_random_append_sequences_give_the_same_cache(gpu):
     """Forty seeded random append histories (chunk sizes around the 32-token half blocks, subsets of the sequences,
     every head_dim family, both coders, all widths): the cache must equal, bit for bit, the one that a one-token
-    append followed by one append of the rest builds (which never takes the encoder's direct path), and attend
-    identically -- so the largest row scale kept per region agrees too."""
+    append followed by one append of the rest builds (the rest starts inside a half block, so it goes through the
+    packing kernel), and attend identically -- so the largest row scale kept per region agrees too."""
     import torch
     rng = np.random.default_rng(99)
     gen = torch.Generator(device="cuda")

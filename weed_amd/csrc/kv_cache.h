@@ -53,6 +53,7 @@ struct weed_hip_kv_cache {
     bool has_rotations = false;
     std::vector<int32_t> lens; // host mirror of lens_dev
     int32_t *lens_dev = nullptr;
+    uint32_t *append_done = nullptr; // behind lens_dev: workgroups of the append under way that are through
     // scratch for encode: one field per byte + row scales for the tokens being appended
     uint8_t *enc_fields = nullptr;
     float *enc_alpha = nullptr;

@@ -111,6 +111,40 @@ __global__ void bump_lens_kernel(int32_t *lens, int32_t seq_begin, int32_t seq_c
     }
 }
 
+// The last step of a small append, done by whichever workgroup of its last kernel finishes last: every workgroup of that
+// kernel reads the lengths as they were before the append, so they may only move once all of them are through.
+// `done` counts the workgroups that are (zero between appends: the last one puts it back).  Only for kernels of at
+// most kBumpWorkgroups workgroups: the additions to one counter come in one after the other, and two thousand of
+// them doubled the time of a prefill's encoder.  Larger appends end with bump_lens_kernel.
+constexpr uint32_t kBumpWorkgroups = 128;
+struct LensBump {
+    uint32_t *done; // null: a later kernel of this append moves the lengths
+    int32_t *lens;
+    int32_t seq_begin, seq_count, add;
+    uint32_t workgroups;
+};
+__device__ __forceinline__ void bump_lens_when_last(const LensBump &b)
+{
+    if (!b.done) {
+        return;
+    }
+    __shared__ uint32_t arrived;
+    __syncthreads(); // the loads of lens by this workgroup have returned: their values were used above
+    if (threadIdx.x == 0) {
+        arrived = __hip_atomic_fetch_add(b.done, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (arrived + 1 != b.workgroups) {
+        return;
+    }
+    for (int32_t i = (int32_t)threadIdx.x; i < b.seq_count; i += (int32_t)blockDim.x) {
+        b.lens[b.seq_begin + i] += b.add;
+    }
+    if (threadIdx.x == 0) {
+        __hip_atomic_store(b.done, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
 __global__ void fill_i32_kernel(int32_t *p, int32_t v, uint32_t n)
 {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -151,8 +185,9 @@ constexpr int kEncThreads = 256;
 //   rounding (multiply, then add, i ascending: src/ops/matmul.cpp:40-44).
 // PARTS = number of row slices the 256 threads are split into (each thread owns one output column of its slice).
 // `block` = index of the workgroup among those that work on this tensor.
-// Where an append whose rows fill whole 32-token half blocks goes directly (see encode_rows_body): the cache side's
-// own arrays.  `out` null: the rows go to the scratch arrays and a second kernel packs them.
+// Where an append whose rows fill whole 32-token half blocks, or one that adds one token per sequence, goes directly
+// (see encode_rows_body): the cache side's own arrays.  `out` null: the rows go to the scratch arrays and a second
+// kernel packs them.
 struct DirectOut {
     uint8_t *out;        // packed fields of the side
     uint64_t region_bytes;
@@ -205,7 +240,91 @@ __device__ __forceinline__ void write_half_block(const uint8_t *staged, const Di
     }
 }
 
-template <int PARTS>
+// What a thread of a V-side workgroup knows of the items its fields will join, asked for as soon as the lengths are
+// there (the rotation runs while these loads are under way): where each run of items starts, the bit its field
+// starts at, and the byte of every item that the field starts in.  A task is a row and a coordinate mod 16: the
+// items of its d / 16 coordinates follow each other in memory, w bytes each.
+struct ScatterV {
+    static constexpr uint32_t kPasses = kEncRows * 16 / kEncThreads; // tasks per thread
+    static_assert(kEncRows * 16 % kEncThreads == 0, "whole passes over (row, coordinate mod 16)");
+    uint8_t *dst[kPasses]; // null: no such row
+    uint32_t bit[kPasses];
+    uint32_t old[kPasses][16]; // head_dim <= 256: at most 16 items per run
+};
+__device__ __forceinline__ void request_scattered_v(ScatterV &pre, const uint32_t *tok_s, const DirectOut &o,
+                                                    uint32_t Hkv, uint32_t d, uint32_t row0, uint32_t rows)
+{
+    const uint32_t w = o.w, per = d / 16;
+    const uint64_t region0 = (uint64_t)o.seq_begin * Hkv + row0; // T = 1: one row per region, in region order
+#pragma unroll
+    for (uint32_t pass = 0; pass < ScatterV::kPasses; ++pass) {
+        const uint32_t idx = threadIdx.x + pass * kEncThreads;
+        const uint32_t r = idx >> 4, c = idx & 15;
+        pre.dst[pass] = nullptr;
+        if (row0 + r < rows) {
+            const FieldPos p = v_field_pos(tok_s[r], c, d, w);
+            pre.dst[pass] = o.out + (region0 + r) * o.region_bytes + p.byte;
+            pre.bit[pass] = p.bit;
+#pragma unroll
+            for (uint32_t jb = 0; jb < 16; ++jb) {
+                pre.old[pass][jb] = ((p.bit & 7) && jb < per) ? pre.dst[pass][jb * w + (p.bit >> 3)] : 0u;
+            }
+        }
+    }
+}
+
+// One new token per sequence (T = 1): staged row r is token tok_s[r] (the sequence's length so far) of region
+// row0 + r.  Its K items are whole (8 coordinates of the token).  Each of its V fields joins the item of its
+// coordinate: the bytes below the field stay as they are (the tokens already cached sit below it in the item), the
+// byte the field starts in keeps its low bits, and what lies above becomes the field and zeros.  No two rows share
+// an item.
+__device__ __forceinline__ void write_scattered(const uint8_t *staged, const uint32_t *tok_s, const ScatterV &pre,
+                                                const DirectOut &o, uint32_t Hkv, uint32_t d, uint32_t row0,
+                                                uint32_t rows)
+{
+    const uint32_t w = o.w;
+    const uint64_t region0 = (uint64_t)o.seq_begin * Hkv + row0; // T = 1: one row per region, in region order
+    if (!o.is_v) {
+        const uint32_t items = d / 8;
+        for (uint32_t idx = threadIdx.x; idx < kEncRows * items; idx += kEncThreads) {
+            const uint32_t r = idx / items, it = idx - r * items;
+            if (row0 + r >= rows) {
+                break;
+            }
+            uint8_t bytes[8];
+            item_build(staged + (uint64_t)r * d + it * 8, w, bytes);
+            uint8_t *dst = o.out + (region0 + r) * o.region_bytes + k_field_pos(tok_s[r], it * 8, d, w).byte;
+            for (uint32_t b = 0; b < w; ++b) {
+                dst[b] = bytes[b];
+            }
+        }
+        return;
+    }
+    const uint32_t per = d / 16;
+#pragma unroll
+    for (uint32_t pass = 0; pass < ScatterV::kPasses; ++pass) {
+        if (!pre.dst[pass]) {
+            break;
+        }
+        const uint32_t idx = threadIdx.x + pass * kEncThreads;
+        const uint32_t r = idx >> 4, c = idx & 15;
+        const uint32_t b0 = pre.bit[pass] >> 3, low = pre.bit[pass] & 7;
+#pragma unroll
+        for (uint32_t jb = 0; jb < 16; ++jb) {
+            if (jb < per) {
+                const uint32_t f = staged[(uint64_t)r * d + 16 * jb + c];
+                uint32_t bits = (pre.old[pass][jb] & ((1u << low) - 1u)) | (f << low); // w <= 8: at most 15 bits
+                for (uint32_t b = b0; b < w; ++b) {
+                    pre.dst[pass][jb * w + b] = (uint8_t)bits;
+                    bits >>= 8;
+                }
+            }
+        }
+    }
+}
+
+// ONE: an append of one token per sequence, which this kernel finishes itself (write_scattered).
+template <int PARTS, bool ONE>
 __device__ __forceinline__ void encode_rows_body(const float *__restrict__ x, const Geom4 &g, uint32_t Hkv, uint32_t T,
                                                  uint32_t d, uint32_t d_real, uint32_t rows,
                                                  const float *__restrict__ rot_t, int rotate, const CoderParams &cp,
@@ -224,6 +343,18 @@ __device__ __forceinline__ void encode_rows_body(const float *__restrict__ x, co
     // gather the rows (logical row = (s*Hkv + h)*T + t): the first 32 threads work out where their row starts, then
     // thread (tid / 32, tid % 32) walks rows tid / 32, +8, ... and columns tid % 32, +32, ... (no divisions per element)
     unsigned long long *row_base = reinterpret_cast<unsigned long long *>(inv_s + kEncRows); // [kEncRows], 8-byte aligned
+    uint32_t *tok_s = reinterpret_cast<uint32_t *>(row_base + kEncRows); // [kEncRows] tokens cached so far (T = 1 appends)
+    // the first 128 steps of the rotation's columns for this wavefront's first tile, in flight during the gather
+    float bpre[64];
+    const bool prefetched = ONE && rotate == 1 && d >= 128 && (tid >> 6) < d / 32;
+    if (prefetched) {
+        const float *bcol = rot_t + 32 * (tid >> 6) + (tid & 31);
+#pragma unroll
+        for (int u = 0; u < 64; ++u) {
+            bpre[u] = bcol[(uint64_t)d * (2 * u + ((tid & 63) >> 5))];
+        }
+    }
+    uint32_t cached = 0;
     if (tid < kEncRows) {
         const uint32_t row = row0 + tid;
         unsigned long long base = ~0ull;
@@ -234,6 +365,9 @@ __device__ __forceinline__ void encode_rows_body(const float *__restrict__ x, co
             base = (uint64_t)g.off + (uint64_t)s * g.s[0] + (uint64_t)h * g.s[1] + (uint64_t)t * g.s[2];
         }
         row_base[tid] = base;
+        if (ONE && row < rows) {
+            cached = (uint32_t)direct.lens[direct.seq_begin + (int32_t)(row / Hkv)]; // in flight during the gather
+        }
     }
     __syncthreads();
     {
@@ -246,7 +380,16 @@ __device__ __forceinline__ void encode_rows_body(const float *__restrict__ x, co
             }
         }
     }
+    if (ONE && tid < kEncRows) {
+        tok_s[tid] = cached;
+    }
     __syncthreads();
+    [[maybe_unused]] ScatterV pre;
+    if constexpr (ONE) {
+        if (direct.is_v) {
+            request_scattered_v(pre, tok_s, direct, Hkv, d, row0, rows);
+        }
+    }
 
     if (rotate == 1) {
         // y = x . R on the matrix cores: each wavefront owns 32-column tiles of the 32 x d result and walks the
@@ -268,9 +411,16 @@ __device__ __forceinline__ void encode_rows_body(const float *__restrict__ x, co
             uint32_t k0 = 0;
             for (; k0 + 128 <= d; k0 += 128) {
                 float b[64];
+                if (prefetched && tile == wave && k0 == 0) {
 #pragma unroll
-                for (int u = 0; u < 64; ++u) {
-                    b[u] = bcol[(uint64_t)d * (k0 + 2 * u + khalf)];
+                    for (int u = 0; u < 64; ++u) {
+                        b[u] = bpre[u];
+                    }
+                } else {
+#pragma unroll
+                    for (int u = 0; u < 64; ++u) {
+                        b[u] = bcol[(uint64_t)d * (k0 + 2 * u + khalf)];
+                    }
                 }
 #pragma unroll
                 for (int u = 0; u < 64; ++u) {
@@ -340,7 +490,11 @@ __device__ __forceinline__ void encode_rows_body(const float *__restrict__ x, co
         }
         if (direct.out) {
             __syncthreads();
-            write_half_block(staged, direct, Hkv, T, d, row0);
+            if constexpr (ONE) {
+                write_scattered(staged, tok_s, pre, direct, Hkv, d, row0, rows);
+            } else {
+                write_half_block(staged, direct, Hkv, T, d, row0);
+            }
         }
         return;
     }
@@ -367,7 +521,16 @@ __device__ __forceinline__ void encode_rows_body(const float *__restrict__ x, co
             a = norm / sqrt_d;
         }
         inv_s[tid] = inv;
-        if (direct.out) {
+        if (ONE) {
+            // one row per (sequence, head): scale to its token slot, and into the region's largest scale
+            if (row0 + tid < rows) {
+                const uint32_t region = (uint32_t)direct.seq_begin * Hkv + row0 + tid;
+                direct.alpha[(uint64_t)region * direct.padded + tok_s[tid]] = a;
+                if (direct.alpha_max) {
+                    atomicMax(direct.alpha_max + region, __float_as_uint(fabsf(a)));
+                }
+            }
+        } else if (direct.out) {
             // all kEncRows rows belong to one (sequence, head): scale to its token slot, largest scale to the region
             const uint32_t h = (row0 / T) % Hkv, sq = row0 / (T * Hkv);
             const uint32_t region = (uint32_t)(direct.seq_begin + (int32_t)sq) * Hkv + h;
@@ -421,7 +584,11 @@ __device__ __forceinline__ void encode_rows_body(const float *__restrict__ x, co
     }
     if (direct.out) {
         __syncthreads();
-        write_half_block(staged, direct, Hkv, T, d, row0);
+        if constexpr (ONE) {
+            write_scattered(staged, tok_s, pre, direct, Hkv, d, row0, rows);
+        } else {
+            write_half_block(staged, direct, Hkv, T, d, row0);
+        }
     }
 }
 
@@ -436,18 +603,19 @@ struct EncSide {
     float *alpha_out;
     DirectOut direct;
 };
-template <int PARTS>
+template <int PARTS, bool ONE>
 __global__ void __launch_bounds__(kEncThreads)
     encode_rows_pair_kernel(EncSide k, EncSide v, uint32_t blocks_per_side, uint32_t Hkv, uint32_t T, uint32_t d,
-                            uint32_t d_real, uint32_t rows, int rotate)
+                            uint32_t d_real, uint32_t rows, int rotate, LensBump bump)
 {
     if (blockIdx.x < blocks_per_side) {
-        encode_rows_body<PARTS>(k.x, k.g, Hkv, T, d, d_real, rows, k.rot_t, rotate, k.cp, k.fields, k.alpha_out,
+        encode_rows_body<PARTS, ONE>(k.x, k.g, Hkv, T, d, d_real, rows, k.rot_t, rotate, k.cp, k.fields, k.alpha_out,
                                 k.direct, blockIdx.x);
     } else {
-        encode_rows_body<PARTS>(v.x, v.g, Hkv, T, d, d_real, rows, v.rot_t, rotate, v.cp, v.fields, v.alpha_out,
+        encode_rows_body<PARTS, ONE>(v.x, v.g, Hkv, T, d, d_real, rows, v.rot_t, rotate, v.cp, v.fields, v.alpha_out,
                                 v.direct, blockIdx.x - blocks_per_side);
     }
+    bump_lens_when_last(bump);
 }
 
 // One thread per (new row, item of 8 coordinates): 8 bytes in, w bytes out.
@@ -575,6 +743,7 @@ struct PackArgs {
     float *k_alpha_out, *v_alpha_out; // null: the coder has no row scales
     uint32_t *v_alpha_max;
     uint32_t blocks_k, blocks_v;
+    LensBump bump;
 };
 __global__ void __launch_bounds__(256) pack_all_kernel(PackArgs a)
 {
@@ -588,6 +757,7 @@ __global__ void __launch_bounds__(256) pack_all_kernel(PackArgs a)
         scatter_v_scales_body(a.v_alpha_in, a.rows, a.Hkv, a.T, a.seq_begin, a.lens, a.v_alpha_out, a.v_alpha_max,
                               a.padded, blockIdx.x - a.blocks_k - a.blocks_v);
     }
+    bump_lens_when_last(a.bump);
 }
 
 __device__ __forceinline__ uint32_t load_field(const SideParams &sp, int which, uint64_t region, uint32_t n, uint32_t j,
@@ -792,9 +962,25 @@ EncSide enc_side_args(const weed_hip_kv_cache *c, const Side &side, const float 
     return e;
 }
 
-// Rotate, quantise and pack the new K and V rows: one launch for the two encoders, one for the three packing steps.
-// The scratch holds the K rows first, then the V rows.
+// Rotate, quantise and pack the new K and V rows, and move the lengths on.  One launch where the encoder can write
+// the items itself (whole half blocks, or one token per sequence), else one for the two encoders and one for the
+// three packing steps; a grid of more than kBumpWorkgroups is followed by one that moves the lengths.  The scratch
+// holds the K rows first, then the V rows.
 int pack_rows(weed_hip_kv_cache *c, int32_t seq_begin, int32_t seq_count, int32_t T_new);
+
+LensBump lens_bump(weed_hip_kv_cache *c, int32_t seq_begin, int32_t seq_count, int32_t T_new, uint32_t workgroups)
+{
+    return LensBump{ workgroups <= kBumpWorkgroups ? c->append_done : nullptr, c->lens_dev, seq_begin, seq_count, T_new,
+                     workgroups };
+}
+
+// After the last kernel of an append that was too large to move the lengths itself.
+int bump_lens(weed_hip_kv_cache *c, int32_t seq_begin, int32_t seq_count, int32_t T_new)
+{
+    bump_lens_kernel<<<((uint32_t)seq_count + 255) / 256, 256, 0, stream()>>>(c->lens_dev, seq_begin, seq_count, T_new);
+    WEED_HIP_LAUNCH_CHECK();
+    return WEED_HIP_OK;
+}
 
 int encode_both(weed_hip_kv_cache *c, int32_t seq_begin, int32_t seq_count, int32_t T_new, const float *k_dev,
                 uint32_t k_off, const uint32_t k_stride[4], const float *v_dev, uint32_t v_off,
@@ -814,6 +1000,10 @@ int encode_both(weed_hip_kv_cache *c, int32_t seq_begin, int32_t seq_count, int3
     for (int32_t sq = 0; direct && sq < seq_count; ++sq) {
         direct = c->lens[(size_t)(seq_begin + sq)] % 32 == 0;
     }
+    // A decode step's append (one token per sequence) is finished by the encoder too: a workgroup's 32 rows are the
+    // new tokens of 32 (sequence, head) pairs, and nothing else touches the items they go to.
+    const int scattered = !direct && T_new == 1;
+    direct = direct || scattered;
     if (direct) {
         const bool scales = c->cfg.mode == WEED_HIP_KV_LLOYDMAX;
         ek.direct = DirectOut{ c->k.fields, c->k.region_bytes, scales ? c->k.alpha : nullptr, nullptr, c->lens_dev,
@@ -821,38 +1011,37 @@ int encode_both(weed_hip_kv_cache *c, int32_t seq_begin, int32_t seq_count, int3
         ev.direct = DirectOut{ c->v.fields, c->v.region_bytes, scales ? c->v.alpha : nullptr,
                                scales ? c->v.alpha_max : nullptr, c->lens_dev, seq_begin, c->padded_tokens, c->v.w, 1 };
     }
-    const size_t smem = sizeof(float) * (2 * kEncRows * (d + 1) + kEncRows) + sizeof(unsigned long long) * kEncRows;
+    const size_t smem = sizeof(float) * (2 * kEncRows * (d + 1) + kEncRows) + sizeof(unsigned long long) * kEncRows +
+                        sizeof(uint32_t) * kEncRows;
     const uint32_t blocks = (rows + kEncRows - 1) / kEncRows;
     int parts = 1;
     while (parts * 2 * d <= (uint32_t)kEncThreads && parts < 8) {
         parts *= 2;
     }
+    typedef void (*EncKernel)(EncSide, EncSide, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, int, LensBump);
+    static const EncKernel kernels[2][4] = {
+        { encode_rows_pair_kernel<1, false>, encode_rows_pair_kernel<2, false>, encode_rows_pair_kernel<4, false>,
+          encode_rows_pair_kernel<8, false> },
+        { encode_rows_pair_kernel<1, true>, encode_rows_pair_kernel<2, true>, encode_rows_pair_kernel<4, true>,
+          encode_rows_pair_kernel<8, true> },
+    };
+    const EncKernel kernel = kernels[scattered][parts == 8 ? 3 : parts == 4 ? 2 : parts == 2 ? 1 : 0];
     if (smem > 48 * 1024) {
         // more than the default dynamic LDS limit (head_dim 256): opt in per kernel instance
-        const void *fns[4] = { (const void *)encode_rows_pair_kernel<1>, (const void *)encode_rows_pair_kernel<2>,
-                               (const void *)encode_rows_pair_kernel<4>, (const void *)encode_rows_pair_kernel<8> };
-        for (const void *fn : fns) {
-            WEED_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        }
+        WEED_HIP_CHECK(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
     }
     {
         ProfileScope prof("kv_encode");
-        const uint32_t T = (uint32_t)T_new;
-        switch (parts) {
-        case 8:
-            encode_rows_pair_kernel<8><<<2 * blocks, kEncThreads, smem, stream()>>>(ek, ev, blocks, Hkv, T, d, d_real, rows, rotate);
-            break;
-        case 4:
-            encode_rows_pair_kernel<4><<<2 * blocks, kEncThreads, smem, stream()>>>(ek, ev, blocks, Hkv, T, d, d_real, rows, rotate);
-            break;
-        case 2:
-            encode_rows_pair_kernel<2><<<2 * blocks, kEncThreads, smem, stream()>>>(ek, ev, blocks, Hkv, T, d, d_real, rows, rotate);
-            break;
-        default:
-            encode_rows_pair_kernel<1><<<2 * blocks, kEncThreads, smem, stream()>>>(ek, ev, blocks, Hkv, T, d, d_real, rows, rotate);
-            break;
+        LensBump bump = lens_bump(c, seq_begin, seq_count, T_new, 2 * blocks);
+        if (!direct) {
+            bump.done = nullptr; // the packing kernel reads the old lengths too
         }
+        kernel<<<2 * blocks, kEncThreads, smem, stream()>>>(ek, ev, blocks, Hkv, (uint32_t)T_new, d, d_real, rows, rotate,
+                                                           bump);
         WEED_HIP_LAUNCH_CHECK();
+        if (direct && !bump.done) {
+            WEED_HIP_TRY(bump_lens(c, seq_begin, seq_count, T_new));
+        }
     }
     return direct ? WEED_HIP_OK : pack_rows(c, seq_begin, seq_count, T_new);
 }
@@ -897,9 +1086,10 @@ int pack_rows(weed_hip_kv_cache *c, int32_t seq_begin, int32_t seq_count, int32_
     a.blocks_k = (uint32_t)((nk + 255) / 256);
     a.blocks_v = (uint32_t)((nv + 255) / 256);
     const uint32_t blocks_s = scales ? (rows + 255) / 256 : 0;
+    a.bump = lens_bump(c, seq_begin, seq_count, T_new, a.blocks_k + a.blocks_v + blocks_s);
     pack_all_kernel<<<a.blocks_k + a.blocks_v + blocks_s, 256, 0, stream()>>>(a);
     WEED_HIP_LAUNCH_CHECK();
-    return WEED_HIP_OK;
+    return a.bump.done ? WEED_HIP_OK : bump_lens(c, seq_begin, seq_count, T_new);
 }
 
 // Scratch for the rows of one append (K rows, then V rows): grows as needed.
@@ -924,11 +1114,9 @@ int reserve_append_scratch(weed_hip_kv_cache *c, const char *fn, int32_t seq_cou
     return WEED_HIP_OK;
 }
 
-// The appended tokens become visible: device and host copies of the lengths move on.
+// The host copy of the lengths follows the device's, which the last kernel of the append has moved.
 int finish_append(weed_hip_kv_cache *c, int32_t seq_begin, int32_t seq_count, int32_t T_new)
 {
-    bump_lens_kernel<<<((uint32_t)seq_count + 255) / 256, 256, 0, stream()>>>(c->lens_dev, seq_begin, seq_count, T_new);
-    WEED_HIP_LAUNCH_CHECK();
     for (int32_t s = 0; s < seq_count; ++s) {
         c->lens[(size_t)(seq_begin + s)] += T_new;
     }
@@ -1088,9 +1276,11 @@ int weed_hip_kv_cache_create(weed_hip_kv_cache **cache, const weed_hip_kv_config
                         hipGetErrorString(e));
         }
     }
-    hipError_t e = hipMalloc((void **)&c->lens_dev, sizeof(int32_t) * (size_t)cfg->n_seq);
+    // the lengths, and behind them the count of workgroups that are through with the append under way
+    hipError_t e = hipMalloc((void **)&c->lens_dev, sizeof(int32_t) * ((size_t)cfg->n_seq + 1));
     if (e == hipSuccess) {
-        e = hipMemsetAsync(c->lens_dev, 0, sizeof(int32_t) * (size_t)cfg->n_seq, stream());
+        e = hipMemsetAsync(c->lens_dev, 0, sizeof(int32_t) * ((size_t)cfg->n_seq + 1), stream());
+        c->append_done = reinterpret_cast<uint32_t *>(c->lens_dev + cfg->n_seq);
     }
     if (e != hipSuccess) {
         weed_hip_kv_cache_destroy(c);
@@ -1131,7 +1321,7 @@ int weed_hip_kv_cache_reset(weed_hip_kv_cache *c, int drop_rotations)
     WEED_HIP_TRY(check_cache(c, "weed_hip_kv_cache_reset"));
     std::fill(c->lens.begin(), c->lens.end(), 0);
     const uint32_t n = (uint32_t)c->cfg.n_seq;
-    fill_i32_kernel<<<(n + 255) / 256, 256, 0, stream()>>>(c->lens_dev, 0, n);
+    fill_i32_kernel<<<(n + 256) / 256, 256, 0, stream()>>>(c->lens_dev, 0, n + 1); // and the append's counter
     WEED_HIP_LAUNCH_CHECK();
     if (c->v.alpha_max) {
         const uint32_t regions = n * (uint32_t)c->cfg.n_kv_heads;
