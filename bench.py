@@ -279,6 +279,17 @@ def extras(capi, torch, workloads, steps, warmup):
                      "frac": rot_flops / kernel_s / 1e12 / 157.3, "kernel": "encode_rows_pair_kernel (K and V)",
                      "flops_per_launch": rot_flops}}
     cache.close()
+    # the append of a decode step: one new token for each of 64 sequences (one launch: the encoder writes the items
+    # and moves the lengths itself)
+    n_app = 1 + warmup + 2 * steps
+    cache1 = capi.KVCache(capi.KV_LLOYDMAX, 64, wl.n_kv_heads, d, n_app, 3, 3, 1, 0)
+    cache1.set_rotations(rk, rv)
+    k1 = torch.randn((64, wl.n_kv_heads, 1, d), device="cuda")
+    v1 = torch.randn((64, wl.n_kv_heads, 1, d), device="cuda")
+    secs, kernel_s = time_kernel(capi, torch, lambda: cache1.encode_append(k1, v1, rotate=1), "kv_encode", steps, warmup)
+    out["append_one_token_64_sequences"] = {"ms": 1e3 * secs, "kernel_ms": 1e3 * kernel_s, "kernels_per_append": 1,
+                                            "rows": 2 * 64 * wl.n_kv_heads}
+    cache1.close()
     # configuration 4: 16 ragged sequences in [2048, 32768], K 2-bit + sign, V 3-bit, split-context merge
     wl4 = workloads.config(4)
     cache4 = capi.KVCache(capi.KV_LLOYDMAX, wl4.n_seq, wl4.n_kv_heads, d, wl4.max_len, wl4.k_bits, wl4.v_bits,
