@@ -153,6 +153,17 @@ __global__ void fill_i32_kernel(int32_t *p, int32_t v, uint32_t n)
     }
 }
 
+// A load of a float through a buffer descriptor: the lane's 32-bit byte offset and one that is the same in every
+// lane, so that a batch of loads needs no address arithmetic per load.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_of(const float *base, uint32_t bytes)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(base), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ float buffer_f32(__amdgpu_buffer_rsrc_t r, uint32_t lane_off, uint32_t uniform_off)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)lane_off, (int)uniform_off, 0));
+}
+
 struct CoderParams {
     int mode;
     int bits;
@@ -323,6 +334,49 @@ __device__ __forceinline__ void write_scattered(const uint8_t *staged, const uin
     }
 }
 
+// Lloyd-Max fields of the staged rows: code = number of thresholds at or below the scaled coordinate (they ascend, so
+// the level of that code is the one behind the last threshold passed), then the sign bit against that level.  Four
+// consecutive coordinates per thread, stored as one 32-bit word (d is a multiple of 32, the destination is 4-byte
+// aligned and its rows are d bytes long).
+template <int BITS>
+__device__ __forceinline__ void lloyd_fields(const float *ys, uint32_t pitch, const float *inv_s, const CoderParams &cp,
+                                             uint8_t *fdst, uint32_t d, uint32_t row0, uint32_t rows)
+{
+    constexpr int NB = (1 << BITS) - 1;
+    float bound[NB], level[NB + 1];
+#pragma unroll
+    for (int k = 0; k < NB; ++k) {
+        bound[k] = cp.bounds[k];
+    }
+#pragma unroll
+    for (int k = 0; k <= NB; ++k) {
+        level[k] = cp.levels[k];
+    }
+    const bool sign = cp.sign != 0;
+    const uint32_t tid = threadIdx.x, jl = tid & 31;
+    for (uint32_t r = tid >> 5; r < kEncRows && row0 + r < rows; r += kEncThreads / 32) {
+        const float inv = inv_s[r];
+        for (uint32_t j = 4 * jl; j < d; j += 128) {
+            uint32_t word = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float u = ys[r * pitch + j + i] * inv;
+                uint32_t code = 0;
+                float lvl = level[0];
+#pragma unroll
+                for (int k = 0; k < NB; ++k) {
+                    const bool ge = u >= bound[k];
+                    code += ge ? 1u : 0u;
+                    lvl = ge ? level[k + 1] : lvl;
+                }
+                const uint32_t f = sign ? ((code << 1) | ((u >= lvl) ? 1u : 0u)) : code;
+                word |= f << (8 * i);
+            }
+            *reinterpret_cast<uint32_t *>(fdst + (uint64_t)r * d + j) = word;
+        }
+    }
+}
+
 // ONE: an append of one token per sequence, which this kernel finishes itself (write_scattered).
 template <int PARTS, bool ONE>
 __device__ __forceinline__ void encode_rows_body(const float *__restrict__ x, const Geom4 &g, uint32_t Hkv, uint32_t T,
@@ -348,10 +402,11 @@ __device__ __forceinline__ void encode_rows_body(const float *__restrict__ x, co
     float bpre[64];
     const bool prefetched = ONE && rotate == 1 && d >= 128 && (tid >> 6) < d / 32;
     if (prefetched) {
-        const float *bcol = rot_t + 32 * (tid >> 6) + (tid & 31);
+        const __amdgpu_buffer_rsrc_t rot = buffer_of(rot_t, 4 * d * d);
+        const uint32_t at = 4 * (32 * (tid >> 6) + (tid & 31) + d * ((tid & 63) >> 5));
 #pragma unroll
         for (int u = 0; u < 64; ++u) {
-            bpre[u] = bcol[(uint64_t)d * (2 * u + ((tid & 63) >> 5))];
+            bpre[u] = buffer_f32(rot, at, 8 * d * u);
         }
     }
     uint32_t cached = 0;
@@ -405,7 +460,10 @@ __device__ __forceinline__ void encode_rows_body(const float *__restrict__ x, co
             for (int i = 0; i < 16; ++i) {
                 acc[i] = 0.0f;
             }
-            const float *bcol = rot_t + 32 * tile + l32; // R[k][32*tile + l32] = rot_t[col + d*k]
+            // R[k][32*tile + l32] = rot_t[col + d*k]: the lane's part of the address is its column and its half of
+            // the step, the step itself is the same in every lane
+            const __amdgpu_buffer_rsrc_t rot = buffer_of(rot_t, 4 * d * d);
+            const uint32_t at = 4 * (32 * tile + l32 + d * khalf);
             // d is a multiple of 32: sixty-four steps at a time where d allows (the loads of the rotation come from
             // L2 and are the long pole: as many as possible are issued together), else sixteen
             uint32_t k0 = 0;
@@ -419,7 +477,7 @@ __device__ __forceinline__ void encode_rows_body(const float *__restrict__ x, co
                 } else {
 #pragma unroll
                     for (int u = 0; u < 64; ++u) {
-                        b[u] = bcol[(uint64_t)d * (k0 + 2 * u + khalf)];
+                        b[u] = buffer_f32(rot, at, 4 * d * (k0 + 2 * u));
                     }
                 }
 #pragma unroll
@@ -432,7 +490,7 @@ __device__ __forceinline__ void encode_rows_body(const float *__restrict__ x, co
 #pragma unroll
                 for (int u = 0; u < 16; ++u) {
                     a[u] = xs[l32 * pitch + k0 + 2 * u + khalf];
-                    b[u] = bcol[(uint64_t)d * (k0 + 2 * u + khalf)];
+                    b[u] = buffer_f32(rot, at, 4 * d * (k0 + 2 * u));
                 }
 #pragma unroll
                 for (int u = 0; u < 16; ++u) {
@@ -550,37 +608,21 @@ __device__ __forceinline__ void encode_rows_body(const float *__restrict__ x, co
         }
     }
     __syncthreads();
-    const int nb = (1 << cp.bits) - 1;
-    // all fifteen possible thresholds in registers (unused ones at +inf), so that the count below is branch- and
-    // load-free
-    float bound[15];
-#pragma unroll
-    for (int k = 0; k < 15; ++k) {
-        bound[k] = k < nb ? cp.bounds[k] : INFINITY;
-    }
-    // four consecutive coordinates per thread, stored as one 32-bit word (d is a multiple of 32, the field array is
-    // 4-byte aligned and rows are d bytes long)
-    const uint32_t jl = tid & 31;
-    for (uint32_t r = tid >> 5; r < kEncRows && row0 + r < rows; r += kEncThreads / 32) {
-        const float inv = inv_s[r];
-        for (uint32_t j = 4 * jl; j < d; j += 128) {
-            uint32_t word = 0;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const float u = ys[r * pitch + j + i] * inv;
-                int code = 0;
-#pragma unroll
-                for (int k = 0; k < 15; ++k) {
-                    code += (u >= bound[k]) ? 1 : 0;
-                }
-                uint32_t f = (uint32_t)code;
-                if (cp.sign) {
-                    f = (f << 1) | ((u >= cp.levels[code]) ? 1u : 0u);
-                }
-                word |= f << (8 * i);
-            }
-            *reinterpret_cast<uint32_t *>(fdst + (uint64_t)r * d + j) = word;
-        }
+    // one instance per code width: its thresholds (and, with a sign bit, its levels) sit in registers and nothing is
+    // compared against a threshold that the width does not have
+    switch (cp.bits) {
+    case 1:
+        lloyd_fields<1>(ys, pitch, inv_s, cp, fdst, d, row0, rows);
+        break;
+    case 2:
+        lloyd_fields<2>(ys, pitch, inv_s, cp, fdst, d, row0, rows);
+        break;
+    case 3:
+        lloyd_fields<3>(ys, pitch, inv_s, cp, fdst, d, row0, rows);
+        break;
+    default:
+        lloyd_fields<4>(ys, pitch, inv_s, cp, fdst, d, row0, rows);
+        break;
     }
     if (direct.out) {
         __syncthreads();
