@@ -428,10 +428,33 @@ __device__ __forceinline__ void encode_rows_body(const float *__restrict__ x, co
     {
         float *dst = rotate ? xs : ys;
         const uint32_t jl = tid & 31;
-        for (uint32_t r = tid >> 5; r < kEncRows; r += kEncThreads / 32) {
-            const unsigned long long base = row_base[r];
-            for (uint32_t j = jl; j < d; j += 32) {
-                dst[r * pitch + j] = (base != ~0ull && j < d_real) ? x[base + (uint64_t)j * g.s[3]] : 0.0f;
+        // rows that are contiguous and 16-byte aligned (the usual case) come in four coordinates per load
+        const bool wide = g.s[3] == 1 && d_real % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
+                          ((g.off | g.s[0] | g.s[1] | g.s[2]) & 3) == 0;
+        if (wide) {
+            float4 v[kEncRows / (kEncThreads / 32)];
+            for (uint32_t j = 4 * jl; j < d; j += 128) {
+#pragma unroll
+                for (uint32_t i = 0; i < kEncRows / (kEncThreads / 32); ++i) {
+                    const unsigned long long base = row_base[(tid >> 5) + i * (kEncThreads / 32)];
+                    v[i] = (base != ~0ull && j < d_real) ? *reinterpret_cast<const float4 *>(x + base + j)
+                                                         : float4{ 0.0f, 0.0f, 0.0f, 0.0f };
+                }
+#pragma unroll
+                for (uint32_t i = 0; i < kEncRows / (kEncThreads / 32); ++i) {
+                    float *at = dst + ((tid >> 5) + i * (kEncThreads / 32)) * pitch + j;
+                    at[0] = v[i].x;
+                    at[1] = v[i].y;
+                    at[2] = v[i].z;
+                    at[3] = v[i].w;
+                }
+            }
+        } else {
+            for (uint32_t r = tid >> 5; r < kEncRows; r += kEncThreads / 32) {
+                const unsigned long long base = row_base[r];
+                for (uint32_t j = jl; j < d; j += 32) {
+                    dst[r * pitch + j] = (base != ~0ull && j < d_real) ? x[base + (uint64_t)j * g.s[3]] : 0.0f;
+                }
             }
         }
     }
