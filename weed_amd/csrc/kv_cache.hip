@@ -352,8 +352,27 @@ __device__ __forceinline__ void lloyd_fields(const float *ys, uint32_t pitch, co
     for (int k = 0; k <= NB; ++k) {
         level[k] = cp.levels[k];
     }
-    const bool sign = cp.sign != 0;
     const uint32_t tid = threadIdx.x, jl = tid & 31;
+    if (!cp.sign) {
+        for (uint32_t r = tid >> 5; r < kEncRows && row0 + r < rows; r += kEncThreads / 32) {
+            const float inv = inv_s[r];
+            for (uint32_t j = 4 * jl; j < d; j += 128) {
+                uint32_t word = 0;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float u = ys[r * pitch + j + i] * inv;
+                    uint32_t code = 0;
+#pragma unroll
+                    for (int k = 0; k < NB; ++k) {
+                        code += (u >= bound[k]) ? 1u : 0u;
+                    }
+                    word |= code << (8 * i);
+                }
+                *reinterpret_cast<uint32_t *>(fdst + (uint64_t)r * d + j) = word;
+            }
+        }
+        return;
+    }
     for (uint32_t r = tid >> 5; r < kEncRows && row0 + r < rows; r += kEncThreads / 32) {
         const float inv = inv_s[r];
         for (uint32_t j = 4 * jl; j < d; j += 128) {
@@ -369,8 +388,7 @@ __device__ __forceinline__ void lloyd_fields(const float *ys, uint32_t pitch, co
                     code += ge ? 1u : 0u;
                     lvl = ge ? level[k + 1] : lvl;
                 }
-                const uint32_t f = sign ? ((code << 1) | ((u >= lvl) ? 1u : 0u)) : code;
-                word |= f << (8 * i);
+                word |= ((code << 1) | ((u >= lvl) ? 1u : 0u)) << (8 * i);
             }
             *reinterpret_cast<uint32_t *>(fdst + (uint64_t)r * d + j) = word;
         }
@@ -675,10 +693,10 @@ __global__ void __launch_bounds__(kEncThreads)
 {
     if (blockIdx.x < blocks_per_side) {
         encode_rows_body<PARTS, ONE>(k.x, k.g, Hkv, T, d, d_real, rows, k.rot_t, rotate, k.cp, k.fields, k.alpha_out,
-                                k.direct, blockIdx.x);
+                                     k.direct, blockIdx.x);
     } else {
         encode_rows_body<PARTS, ONE>(v.x, v.g, Hkv, T, d, d_real, rows, v.rot_t, rotate, v.cp, v.fields, v.alpha_out,
-                                v.direct, blockIdx.x - blocks_per_side);
+                                     v.direct, blockIdx.x - blocks_per_side);
     }
     bump_lens_when_last(bump);
 }
