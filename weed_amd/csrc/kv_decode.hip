@@ -822,24 +822,22 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
     uint32_t n_splits, split_tokens = 0;
     uint32_t total_blocks = 0;
     RunGeom runs = { 1, 0, 8 };
+    // Blocks per sequence as the partition counts them when that is more than the sequences have (see below), else 0.
+    uint32_t virtual_blocks = 0;
+    auto partition_blocks = [&](int32_t l) { return virtual_blocks ? virtual_blocks : ((uint32_t)l + 63u) >> 6; };
     if (use_mfma) {
         // every wavefront takes an equal run of 64-token blocks from the list of all regions' blocks; as many
         // wavefronts as the device holds at once
-        uint64_t blocks = 0;
-        for (int32_t l : c->lens) {
-            blocks += ((uint32_t)l + 63u) >> 6;
-        }
-        blocks *= Hkv;
-        WEED_HIP_REQUIRE(blocks < (1ull << 32), "%s: too many cached tokens for one launch", fn);
-        total_blocks = (uint32_t)blocks;
         runs.waves = mfma_decode_workgroup_waves(pass_heads, d, c->k.w, c->v.w);
         const DecodeTuning &tune = decode_tuning();
-        // one workgroup per compute unit
-        const uint32_t target_units = tune.wavefronts > 0 ? (uint32_t)tune.wavefronts : runs.waves * 256u;
-        runs.unit_blocks = std::max(1u, (total_blocks + target_units - 1) / target_units);
         // Equal sequences of nb blocks: prefer a run length with which every workgroup holds whole regions (the
         // kernel then does the whole call by itself, see below): nb / (classes * q) blocks with q = 1, 2 or 4, that
         // is 4 / q regions per workgroup, provided the workgroups fill the compute units in at most two rounds.
+        // A block count that no such run length divides is rounded up to the next one that one does (a few blocks,
+        // and only as far as the regions' memory reaches): the partition then counts blocks at the end of every
+        // region that hold no tokens, which the kernel skips as it skips those beyond a prefix length, and the
+        // wavefront they fall to has that much less to do -- far cheaper than runs that straddle regions.
+        uint32_t preferred_unit = 0;
         {
             uint32_t nb = ((uint32_t)c->lens[0] + 63u) >> 6;
             for (int32_t l : c->lens) {
@@ -852,22 +850,36 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
             if (nb != 0 && mfma_decode_merges(gp, d) && tune.wavefronts == 0 && !tune.separate_merge &&
                 !tune.always_search) {
                 const uint32_t classes = run_classes(runs), regions = S * Hkv;
-                uint32_t best_rounds = 3;
-                for (uint32_t q = 1; q <= 4; q *= 2) {
-                    if (nb % (classes * q) != 0) {
-                        continue;
-                    }
-                    const uint32_t wgs = (regions * q + 3) / 4, rounds = (wgs + 255) / 256;
-                    if (rounds < best_rounds && wgs * 100 >= rounds * 256 * 95) {
-                        best_rounds = rounds;
-                        runs.unit_blocks = nb / (classes * q);
+                const uint32_t reach = std::min(nb + std::max(1u, nb / 16), c->padded_tokens / 64);
+                for (uint32_t cand = nb; cand <= reach && !preferred_unit; ++cand) {
+                    uint32_t best_rounds = 3;
+                    for (uint32_t q = 1; q <= 4; q *= 2) {
+                        if (cand % (classes * q) != 0) {
+                            continue;
+                        }
+                        const uint32_t wgs = (regions * q + 3) / 4, rounds = (wgs + 255) / 256;
+                        if (rounds < best_rounds && wgs * 100 >= rounds * 256 * 95) {
+                            best_rounds = rounds;
+                            preferred_unit = cand / (classes * q);
+                            virtual_blocks = cand == nb ? 0 : cand;
+                        }
                     }
                 }
             }
         }
+        uint64_t blocks = 0;
+        for (int32_t l : c->lens) {
+            blocks += partition_blocks(l);
+        }
+        blocks *= Hkv;
+        WEED_HIP_REQUIRE(blocks < (1ull << 32), "%s: too many cached tokens for one launch", fn);
+        total_blocks = (uint32_t)blocks;
+        // one workgroup per compute unit
+        const uint32_t target_units = tune.wavefronts > 0 ? (uint32_t)tune.wavefronts : runs.waves * 256u;
+        runs.unit_blocks = preferred_unit ? preferred_unit : std::max(1u, (total_blocks + target_units - 1) / target_units);
         const uint32_t skew_pct = tune.skew_percent >= 0 ? (uint32_t)std::min(90, tune.skew_percent)
                                                          : (runs.waves == 12 ? kRunSkewPercent3 : kRunSkewPercent);
-        const uint32_t nblk = (max_len + 63) / 64;
+        const uint32_t nblk = virtual_blocks ? virtual_blocks : (max_len + 63) / 64;
         for (;;) {
             runs.skew = std::min(runs.unit_blocks - 1, (runs.unit_blocks * skew_pct + 50) / 100);
             const uint32_t shortest = runs.unit_blocks - runs.skew;
@@ -946,9 +958,9 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
     bool general_merge = false;
     bool fused_query = false;
     if (use_mfma && total_blocks) {
-        uniform_blocks = ((uint32_t)c->lens[0] + 63u) >> 6;
+        uniform_blocks = partition_blocks(c->lens[0]);
         for (int32_t l : c->lens) {
-            if ((((uint32_t)l + 63u) >> 6) != uniform_blocks || decode_tuning().always_search) {
+            if (partition_blocks(l) != uniform_blocks || decode_tuning().always_search) {
                 uniform_blocks = 0;
                 break;
             }
@@ -973,7 +985,7 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
             region_end.reserve((size_t)S * Hkv);
             uint64_t run = 0;
             for (int32_t l : c->lens) {
-                const uint32_t b = ((uint32_t)l + 63u) >> 6;
+                const uint32_t b = partition_blocks(l);
                 every_sequence_has_tokens = every_sequence_has_tokens && b != 0;
                 for (uint32_t h = 0; h < Hkv; ++h) {
                     run += b;
