@@ -322,6 +322,35 @@ def extras(capi, torch, workloads, steps, warmup):
         sum(wl8.lens) * wl8.n_kv_heads * 2 * d, steps, warmup)
     cache8.close()
     del q8, o8
+    # a decode loop as a server runs it on the headline shape: one new token for each of the 64 sequences, then the
+    # attention over everything cached (two launches per step), the contexts growing towards 8192 through every
+    # residue of the 64-token blocks
+    wlL = workloads.config(3, n_seq=64)
+    n_loop = warmup + steps
+    cacheL = capi.KVCache(capi.KV_LLOYDMAX, wlL.n_seq, wlL.n_kv_heads, d, wlL.max_len, wlL.k_bits, wlL.v_bits,
+                          wlL.k_sign, wlL.v_sign)
+    cacheL.set_rotations(rk, rv)
+    for s0 in range(0, wlL.n_seq, 8):
+        Ks = torch.randn((8, wlL.n_kv_heads, wlL.max_len - n_loop, d), device="cuda")
+        Vs = torch.randn((8, wlL.n_kv_heads, wlL.max_len - n_loop, d), device="cuda")
+        cacheL.encode_append(Ks, Vs, seq_begin=s0, rotate=1)
+    del Ks, Vs
+    qL = torch.randn((wlL.n_seq, wlL.n_q_heads, d), device="cuda")
+    oL = torch.zeros_like(qL)
+    kL = torch.randn((wlL.n_seq, wlL.n_kv_heads, 1, d), device="cuda")
+    vL = torch.randn((wlL.n_seq, wlL.n_kv_heads, 1, d), device="cuda")
+    flagsL = capi.ATTN_ROTATE_Q | capi.ATTN_UNROTATE_OUT
+
+    def loop_step():
+        cacheL.encode_append(kL, vL, rotate=1)
+        cacheL.decode_attn(qL, oL, capi.GQA_BLOCKED, flagsL)
+
+    secs = time_calls(torch, loop_step, steps, warmup)
+    out["decode_loop_64_sequences_towards_ctx8192"] = {"ms_per_step": 1e3 * secs, "tokens_per_s": wlL.n_seq / secs,
+                                                       "launches_per_step": 2,
+                                                       "ctx_from": wlL.max_len - steps, "ctx_to": wlL.max_len}
+    cacheL.close()
+    del qL, oL, kL, vL
     # configuration 3 again with 256 sequence caches per launch (2 GB of packed rows): what the per-launch fixed cost
     # (launch, table build, first-block latency, uneven finish) amortises to with four times the bytes
     wl3 = workloads.config(3, n_seq=256)
