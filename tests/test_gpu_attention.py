@@ -314,29 +314,32 @@ def test_workgroups_that_merge_their_own_regions(gpu, oracle, lloyd, d, Hkv, Hq,
     cache.close()
 
 
-@pytest.mark.parametrize("cap_blocks", [24, 23])
-def test_equal_sequences_whose_block_count_no_run_length_divides(gpu, oracle, cap_blocks):
-    """Equal sequences of 23 blocks on a full device: no run length divides them into whole regions per workgroup.
+@pytest.mark.parametrize("cap_blocks,top,step", [(24, 23 * 64 - 20, 0), (23, 23 * 64 - 20, 0), (24, 24 * 64 - 10, 30)])
+def test_block_counts_that_no_run_length_divides(gpu, oracle, cap_blocks, top, step):
+    """Sequences of 23 blocks on a full device: no run length divides them into whole regions per workgroup.
     Where the regions' memory reaches one block further (capacity of 24 blocks) the partition counts 24 blocks per
     region, the last one without tokens, and the call stays one kernel with whole regions per workgroup; with a
-    capacity of 23 blocks it cannot, and the runs straddle regions.  Both must agree with the checker, with the
-    three-kernel way, under prefix lengths (zero among them), and after a step's one-token append."""
+    capacity of 23 blocks it cannot, and the runs straddle regions.  The third case mixes sequences of 23 and 24
+    blocks, which are counted alike.  All must agree with the checker, with the three-kernel way, under prefix
+    lengths (zero among them), and after a step's one-token append."""
     import torch
-    S, Hkv, Hq, d, L = 32, 8, 16, 128, 23 * 64 - 20
+    S, Hkv, Hq, d = 32, 8, 16, 128
+    lens = [top - step * (s % 3) for s in range(S)]
     gen = torch.Generator(device="cuda")
     gen.manual_seed(77)
     rng = np.random.default_rng(78)
-    wl = workloads.Workload("rounded", S, Hq, Hkv, d, [L] * S, 3, 4, 0, 0, 0)
+    wl = workloads.Workload("rounded", S, Hq, Hkv, d, lens, 3, 4, 0, 0, 0)
     Rk, Rv = rotations(oracle, d, 9)
     cache = gpu.KVCache(gpu.KV_LLOYDMAX, S, Hkv, d, cap_blocks * 64, 3, 4, 0, 0)
     cache.set_rotations(dev(Rk), dev(Rv))
-    K = torch.randn((S, Hkv, L + 1, d), generator=gen, device="cuda")
-    V = torch.randn((S, Hkv, L + 1, d), generator=gen, device="cuda")
-    cache.encode_append(K[:, :, :L], V[:, :, :L], rotate=1)
+    K = torch.randn((S, Hkv, top + 1, d), generator=gen, device="cuda")
+    V = torch.randn((S, Hkv, top + 1, d), generator=gen, device="cuda")
+    for s in range(S):
+        cache.encode_append(K[s:s + 1, :, :lens[s]], V[s:s + 1, :, :lens[s]], seq_begin=s, rotate=1)
     q = rng.standard_normal((S, Hq, d), dtype=np.float32)
     flags = gpu.ATTN_ROTATE_Q | gpu.ATTN_UNROTATE_OUT
     want = checker_output(oracle, gpu, cache, wl, q, False, Rk=Rk, Rv=Rv)
-    prefix = [max(0, L - 1 - 45 * s) for s in range(S)]
+    prefix = [max(0, lens[s] - 1 - 45 * s) for s in range(S)]
     prefix[S // 2] = 0
     wl_p = workloads.Workload("rounded", S, Hq, Hkv, d, prefix, 3, 4, 0, 0, 0)
     want_p = checker_output(oracle, gpu, cache, wl_p, q, False, Rk=Rk, Rv=Rv)
@@ -362,9 +365,10 @@ def test_equal_sequences_whose_block_count_no_run_length_divides(gpu, oracle, ca
     assert_attn_close(got_p, want_p, "prefix lengths")
     assert np.all(got_p[S // 2] == 0.0)
     assert np.array_equal(again, got)
-    # the next step of a decode loop: one more token everywhere (still 23 blocks), attended again
-    cache.encode_append(K[:, :, L:L + 1], V[:, :, L:L + 1], rotate=1)
-    wl1 = workloads.Workload("rounded", S, Hq, Hkv, d, [L + 1] * S, 3, 4, 0, 0, 0)
+    # the next step of a decode loop: one more token everywhere (the block counts stay), attended again
+    cache.encode_append(torch.stack([K[s, :, lens[s]:lens[s] + 1] for s in range(S)]),
+                        torch.stack([V[s, :, lens[s]:lens[s] + 1] for s in range(S)]), rotate=1)
+    wl1 = workloads.Workload("rounded", S, Hq, Hkv, d, [n + 1 for n in lens], 3, 4, 0, 0, 0)
     want1 = checker_output(oracle, gpu, cache, wl1, q, False, Rk=Rk, Rv=Rv)
     assert_attn_close(run_decode(gpu, cache, q, gpu.GQA_BLOCKED, flags), want1, "after one more token")
     cache.close()

@@ -839,18 +839,17 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         // wavefront they fall to has that much less to do -- far cheaper than runs that straddle regions.
         uint32_t preferred_unit = 0;
         {
-            uint32_t nb = ((uint32_t)c->lens[0] + 63u) >> 6;
+            // (sequences whose block counts differ by as little are counted alike, as the longest of them)
+            uint32_t nb = 0, fewest = ~0u;
             for (int32_t l : c->lens) {
-                if ((((uint32_t)l + 63u) >> 6) != nb) {
-                    nb = 0;
-                    break;
-                }
+                nb = std::max(nb, ((uint32_t)l + 63u) >> 6);
+                fewest = std::min(fewest, ((uint32_t)l + 63u) >> 6);
             }
             const uint32_t gp = pass_heads <= 4 ? 4u : (pass_heads <= 8 ? 8u : 16u);
-            if (nb != 0 && mfma_decode_merges(gp, d) && tune.wavefronts == 0 && !tune.separate_merge &&
+            if (fewest != 0 && mfma_decode_merges(gp, d) && tune.wavefronts == 0 && !tune.separate_merge &&
                 !tune.always_search) {
                 const uint32_t classes = run_classes(runs), regions = S * Hkv;
-                const uint32_t reach = std::min(nb + std::max(1u, nb / 16), c->padded_tokens / 64);
+                const uint32_t reach = std::min(fewest + std::max(1u, fewest / 16), c->padded_tokens / 64);
                 for (uint32_t cand = nb; cand <= reach && !preferred_unit; ++cand) {
                     uint32_t best_rounds = 3;
                     for (uint32_t q = 1; q <= 4; q *= 2) {
@@ -861,7 +860,7 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
                         if (rounds < best_rounds && wgs * 100 >= rounds * 256 * 95) {
                             best_rounds = rounds;
                             preferred_unit = cand / (classes * q);
-                            virtual_blocks = cand == nb ? 0 : cand;
+                            virtual_blocks = cand == fewest ? 0 : cand;
                         }
                     }
                 }
