@@ -833,23 +833,24 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         // Equal sequences of nb blocks: prefer a run length with which every workgroup holds whole regions (the
         // kernel then does the whole call by itself, see below): nb / (classes * q) blocks with q = 1, 2 or 4, that
         // is 4 / q regions per workgroup, provided the workgroups fill the compute units in at most two rounds.
-        // A block count that no such run length divides is rounded up to the next one that one does (a few blocks,
-        // and only as far as the regions' memory reaches): the partition then counts blocks at the end of every
+        // A block count that no such run length divides is rounded up to the next one that one does (an eighth more
+        // at most, and only as far as the regions' memory reaches): the partition then counts blocks at the end of every
         // region that hold no tokens, which the kernel skips as it skips those beyond a prefix length, and the
         // wavefront they fall to has that much less to do -- far cheaper than runs that straddle regions.
         uint32_t preferred_unit = 0;
+        // (sequences whose block counts differ by as little are counted alike, as the longest of them)
+        uint32_t most = 0, fewest = ~0u;
+        for (int32_t l : c->lens) {
+            most = std::max(most, ((uint32_t)l + 63u) >> 6);
+            fewest = std::min(fewest, ((uint32_t)l + 63u) >> 6);
+        }
+        const uint32_t reach = std::min(fewest + std::max(1u, fewest / 8), c->padded_tokens / 64);
+        const bool may_round = fewest != 0 && mfma_decode_merges(pass_heads <= 4 ? 4u : (pass_heads <= 8 ? 8u : 16u), d) &&
+                               tune.wavefronts == 0 && !tune.separate_merge && !tune.always_search;
         {
-            // (sequences whose block counts differ by as little are counted alike, as the longest of them)
-            uint32_t nb = 0, fewest = ~0u;
-            for (int32_t l : c->lens) {
-                nb = std::max(nb, ((uint32_t)l + 63u) >> 6);
-                fewest = std::min(fewest, ((uint32_t)l + 63u) >> 6);
-            }
-            const uint32_t gp = pass_heads <= 4 ? 4u : (pass_heads <= 8 ? 8u : 16u);
-            if (fewest != 0 && mfma_decode_merges(gp, d) && tune.wavefronts == 0 && !tune.separate_merge &&
-                !tune.always_search) {
+            const uint32_t nb = most;
+            if (may_round) {
                 const uint32_t classes = run_classes(runs), regions = S * Hkv;
-                const uint32_t reach = std::min(fewest + std::max(1u, fewest / 16), c->padded_tokens / 64);
                 for (uint32_t cand = nb; cand <= reach && !preferred_unit; ++cand) {
                     uint32_t best_rounds = 3;
                     for (uint32_t q = 1; q <= 4; q *= 2) {
@@ -876,6 +877,16 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         // one workgroup per compute unit
         const uint32_t target_units = tune.wavefronts > 0 ? (uint32_t)tune.wavefronts : runs.waves * 256u;
         runs.unit_blocks = preferred_unit ? preferred_unit : std::max(1u, (total_blocks + target_units - 1) / target_units);
+        // Small batches of long sequences, where a region is several workgroups' shares: the same rounding, to a
+        // whole number of those shares.
+        if (!preferred_unit && may_round) {
+            const uint32_t wg_blocks = runs.waves * runs.unit_blocks;
+            const uint32_t cand = (most + wg_blocks - 1) / wg_blocks * wg_blocks;
+            if (cand != fewest && cand <= reach && cand / wg_blocks >= 2 && cand / wg_blocks <= 64) {
+                virtual_blocks = cand;
+                total_blocks = cand * S * Hkv;
+            }
+        }
         const uint32_t skew_pct = tune.skew_percent >= 0 ? (uint32_t)std::min(90, tune.skew_percent)
                                                          : (runs.waves == 12 ? kRunSkewPercent3 : kRunSkewPercent);
         const uint32_t nblk = virtual_blocks ? virtual_blocks : (max_len + 63) / 64;
