@@ -316,14 +316,15 @@ def test_workgroups_that_merge_their_own_regions(gpu, oracle, lloyd, d, Hkv, Hq,
 
 @pytest.mark.parametrize("cap_blocks,top,step,S,Hkv", [(24, 23 * 64 - 20, 0, 32, 8), (23, 23 * 64 - 20, 0, 32, 8),
                                                        (24, 24 * 64 - 10, 30, 32, 8), (128, 125 * 64 - 7, 0, 2, 2),
-                                                       (64, 61 * 64 - 1, 70, 3, 4)])
+                                                       (64, 61 * 64 - 1, 70, 3, 4), (128, 8000, 2500, 3, 2)])
 def test_block_counts_that_no_run_length_divides(gpu, oracle, cap_blocks, top, step, S, Hkv):
     """Sequences of 23 blocks on a full device: no run length divides them into whole regions per workgroup.
     Where the regions' memory reaches one block further (capacity of 24 blocks) the partition counts 24 blocks per
     region, the last one without tokens, and the call stays one kernel with whole regions per workgroup; with a
     capacity of 23 blocks it cannot, and the runs straddle regions.  The third case mixes sequences of 23 and 24
-    blocks, which are counted alike.  The last two are small batches, where a region is several workgroups' shares
-    and the count is rounded to a whole number of those.  All must agree with the checker, with the three-kernel
+    blocks, which are counted alike.  The last three are small batches, where a region is several workgroups' shares
+    and the count is rounded to a whole number of those; in the last one the sequences hold 8000, 5500 and 3000
+    tokens and are all counted as 128 blocks, so whole workgroups find no tokens in their share.  All must agree with the checker, with the three-kernel
     way, under prefix lengths (zero among them), and after a step's one-token append."""
     import torch
     Hq, d = 2 * Hkv, 128
