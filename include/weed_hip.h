@@ -283,10 +283,13 @@ int weed_hip_kv_decode_attn(weed_hip_kv_cache *cache, int32_t n_q_heads, int32_t
  * (and the youngest shorter), negative = the built-in 16 (28 for kernel instances with three wavefronts per SIMD);
  * always_search: bit 0: find every run's first region by search even when all sequences have equal lengths;
  * bit 1: never let the matrix-core kernel merge its partials itself; bit 2: never let it rotate the queries itself
- * (when every workgroup's share of the launch is a whole number of (sequence, kv head) regions -- equal sequences in
- * power-of-two batches, the common serving shape -- one kernel does the whole call; otherwise, or with these bits, a
- * kernel ahead rotates the queries and one behind merges the partials; the two ways differ in the rounding of the
- * last bits).  The process-wide defaults are read once from the environment variables WEED_HIP_DECODE_WAVES,
+ * (when every workgroup's share of the launch is a whole number of (sequence, kv head) regions, or every region a
+ * whole number of such shares, one kernel does the whole call: that is so for batches of 1 to 256 sequences whose
+ * lengths are equal or not too different -- sequences are counted as having as many blocks as the longest while that
+ * adds at most 3/4 to the blocks of the batch and the cache's capacity holds them; other batches of up to 63
+ * sequences are one kernel too, with partial results in memory; otherwise, or with these bits, a kernel ahead rotates
+ * the queries and one behind merges the partials; the ways differ in the rounding of the last bits).  A number of
+ * wavefronts other than 0 switches the choice of run lengths for whole regions off.  The process-wide defaults are read once from the environment variables WEED_HIP_DECODE_WAVES,
  * WEED_HIP_DECODE_SKEW and WEED_HIP_DECODE_SEARCH. */
 int weed_hip_kv_decode_tuning(int32_t wavefronts, int32_t skew_percent, int32_t always_search);
 
