@@ -219,35 +219,55 @@ __device__ __forceinline__ void write_half_block(const uint8_t *staged, const Di
     const uint32_t h = (row0 / T) % Hkv, sq = row0 / (T * Hkv);
     const uint64_t region = (uint64_t)(o.seq_begin + (int32_t)sq) * Hkv + h;
     const uint32_t n0 = (uint32_t)o.lens[o.seq_begin + (int32_t)sq] + row0 % T;
-    uint8_t *base = o.out + region * o.region_bytes;
     const uint32_t w = o.w;
-    uint8_t bytes[8];
-    if (!o.is_v) {
-        const uint32_t items = d / 8;
-        for (uint32_t idx = threadIdx.x; idx < kEncRows * items; idx += kEncThreads) {
-            const uint32_t r = idx / items, it = idx - r * items;
-            item_build(staged + (uint64_t)r * d + it * 8, w, bytes);
-            uint8_t *dst = base + k_field_pos(n0 + r, it * 8, d, w).byte;
+    // the half's block; items of w bytes are stored whole where w is a power of two, else byte by byte
+    uint8_t *base = o.out + region * o.region_bytes + (uint64_t)(n0 >> 6) * block_bytes(d, w);
+    auto store_item = [&](uint8_t *dst, uint32_t lo, uint32_t hi) { // fields 0..3 in lo, 4..7 in hi, 4 w bits each
+        const uint64_t bits = (uint64_t)lo | ((uint64_t)hi << (4 * w));
+        if (w == 4) {
+            *reinterpret_cast<uint32_t *>(dst) = (uint32_t)bits;
+        } else if (w == 8) {
+            *reinterpret_cast<uint2 *>(dst) = uint2{ lo, hi };
+        } else if (w == 2) {
+            *reinterpret_cast<uint16_t *>(dst) = (uint16_t)bits;
+        } else {
             for (uint32_t b = 0; b < w; ++b) {
-                dst[b] = bytes[b];
+                dst[b] = (uint8_t)(bits >> (8 * b));
             }
+        }
+    };
+    // (small quotients by multiplication with the rounded reciprocal: (x + 0.5) / n is never closer than 0.5 / n to an
+    // integer, and x stays below 1024)
+    if (!o.is_v) {
+        // item `it` of row r: coordinates 8 it .. 8 it + 7, which are item it % (d / 32) of lane group it / (d / 32)
+        const uint32_t ipl = d / 32, items = 4 * ipl;
+        const float inv_items = 1.0f / (float)items, inv_ipl = 1.0f / (float)ipl;
+        for (uint32_t idx = threadIdx.x; idx < kEncRows * items; idx += kEncThreads) {
+            const uint32_t r = (uint32_t)(((float)idx + 0.5f) * inv_items), it = idx - r * items;
+            const uint32_t gq = (uint32_t)(((float)it + 0.5f) * inv_ipl), ks = it - gq * ipl;
+            const uint2 f = *reinterpret_cast<const uint2 *>(staged + (uint64_t)r * d + it * 8); // 8-byte aligned
+            const uint32_t lo = (f.x & 0xffu) | (((f.x >> 8) & 0xffu) << w) | (((f.x >> 16) & 0xffu) << (2 * w)) |
+                                ((f.x >> 24) << (3 * w));
+            const uint32_t hi = (f.y & 0xffu) | (((f.y >> 8) & 0xffu) << w) | (((f.y >> 16) & 0xffu) << (2 * w)) |
+                                ((f.y >> 24) << (3 * w));
+            const uint32_t n = n0 + r, t = (n >> 4) & 3, r16 = n & 15;
+            store_item(base + (((gq * 16 + r16) * 4 + t) * ipl + ks) * w, lo, hi);
         }
         return;
     }
-    const uint32_t u = (n0 >> 5) & 1U, tok0 = n0 & ~63U;
+    // item of coordinate j and lane group gq: the tokens 4 gq .. 4 gq + 3 of the half's two 16-token tiles
+    const uint32_t u = (n0 >> 5) & 1U;
+    const float inv_d = 1.0f / (float)d;
     for (uint32_t idx = threadIdx.x; idx < 4 * d; idx += kEncThreads) {
-        const uint32_t j = idx % d, gq = idx / d;
-        uint8_t f8[8];
+        const uint32_t gq = (uint32_t)(((float)idx + 0.5f) * inv_d), j = idx - gq * d;
+        uint32_t lo = 0, hi = 0;
 #pragma unroll
-        for (uint32_t e = 0; e < 8; ++e) {
+        for (uint32_t e = 0; e < 4; ++e) {
             // token of field e inside this half: rows 4g .. 4g+3 of its first tile, then of its second
-            f8[e] = staged[(uint64_t)(16 * (e >> 2) + 4 * gq + (e & 3)) * d + j];
+            lo |= (uint32_t)staged[(uint64_t)(4 * gq + e) * d + j] << (e * w);
+            hi |= (uint32_t)staged[(uint64_t)(16 + 4 * gq + e) * d + j] << (e * w);
         }
-        item_build(f8, w, bytes);
-        uint8_t *dst = base + v_field_pos(tok0 + v_item_token(u, gq, 0), j, d, w).byte;
-        for (uint32_t b = 0; b < w; ++b) {
-            dst[b] = bytes[b];
-        }
+        store_item(base + (((gq * 16 + (j & 15)) * 2 + u) * (d / 16) + (j >> 4)) * w, lo, hi);
     }
 }
 
