@@ -177,6 +177,35 @@ def time_calls(torch, fn, steps, warmup):
     return (time.perf_counter() - t0) / steps
 
 
+def time_region(torch, fn, steps, warmup):
+    """Seconds per call on the device: two events on the launch stream around `steps` back-to-back calls."""
+    for _ in range(warmup):
+        fn()
+    stream = torch.cuda.current_stream()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record(stream)
+    for _ in range(steps):
+        fn()
+    ev1.record(stream)
+    ev1.synchronize()
+    return 1e-3 * ev0.elapsed_time(ev1) / steps
+
+
+def time_one_kernel_op(capi, torch, fn, name, steps, warmup):
+    """(seconds per call, seconds per launch, how the latter was taken) for an op that is one kernel per call: the
+    launch duration is the device time of a run of back-to-back calls divided by their number, as for the headline
+    (an event pair around every single launch adds the events' own 2-3 us to a kernel of a few dozen); an op that
+    turns out to take several launches per call keeps the event pairs."""
+    secs, pair_s = time_kernel(capi, torch, fn, name, steps, warmup)
+    launches = capi.profile_read(name)[1]
+    note = {"kernel_ms_event_pair_per_launch": 1e3 * pair_s}
+    if launches == steps:
+        note["kernel_ms_source"] = "device time of %d back-to-back calls (one kernel each) between two events, divided by their number" % steps
+        return secs, time_region(torch, fn, steps, warmup), note
+    note["kernel_ms_source"] = "event pairs around the launches"
+    return secs, pair_s, note
+
+
 def time_kernel(capi, torch, fn, name, steps, warmup):
     """(seconds per call, seconds per launch of the kernel recorded under `name`): one untimed call first, so that
     one-off work of a shape's first launch (workspace growth, kernel attributes) stays out of both figures."""
@@ -219,23 +248,25 @@ def extras(capi, torch, workloads, steps, warmup):
     A = torch.randn((1024, 4096), device="cuda").t()           # logical [4096, 1024], column-major
     W = (torch.randn((4096, 1024), device="cuda") * 0.02).t()  # logical [1024, 4096], column-major
     C = torch.empty((4096, 4096), device="cuda").t()
-    secs, kernel_s = time_kernel(capi, torch, lambda: capi.matmul(A, W, C), "matmul", steps, warmup)
+    secs, kernel_s, how = time_one_kernel_op(capi, torch, lambda: capi.matmul(A, W, C), "matmul", steps, warmup)
     flops = 2.0 * 4096 * 1024 * 4096
     out["cfg5b_matmul_f32_4096x1024x4096"] = {
         "tflops": flops / secs / 1e12, "kernel_ms": 1e3 * kernel_s, "kernel_tflops": flops / kernel_s / 1e12,
         "roofline": {"bound": "mfma", "achieved": flops / kernel_s / 1e12, "peak": 157.3, "unit": "TFLOP/s",
                      "frac": flops / kernel_s / 1e12 / 157.3}}
+    out["cfg5b_matmul_f32_4096x1024x4096"].update(how)
     del A, W, C
     # decode-time projection y = x.W: 8 rows against a [4096 x 4096] column-major weight (64 MiB streamed per call)
     X = torch.randn((4096, 8), device="cuda").t()               # logical [8, 4096], column-major
     Wp = (torch.randn((4096, 4096), device="cuda") * 0.02).t()  # logical [4096, 4096], column-major
     Y = torch.empty((4096, 8), device="cuda").t()
-    secs, kernel_s = time_kernel(capi, torch, lambda: capi.matmul(X, Wp, Y), "matmul", steps, warmup)
+    secs, kernel_s, how = time_one_kernel_op(capi, torch, lambda: capi.matmul(X, Wp, Y), "matmul", steps, warmup)
     wbytes = 4096 * 4096 * 4
     out["projection_8x4096x4096"] = {
         "ms": 1e3 * secs, "kernel_ms": 1e3 * kernel_s,
         "roofline": {"bound": "hbm", "achieved": wbytes / kernel_s / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": wbytes / kernel_s / 1e9 / HBM_PEAK_GBS}}
+    out["projection_8x4096x4096"].update(how)
     del X, Wp, Y
     # standalone softmax and sum over an [8192 x 8192] column-major matrix (256 MiB), along the contiguous axis and
     # along the strided one: 8 B per element (softmax) and 4 B per element (sum) of algorithmic traffic
@@ -246,11 +277,12 @@ def extras(capi, torch, workloads, steps, warmup):
     for axis, name in ((0, "contiguous_axis"), (1, "strided_axis")):
         for op, fn, bytes_per in (("softmax", lambda: capi.softmax(S, So, axis), 8),
                                   ("reduce", lambda: capi.reduce(capi.REDUCE_SUM, S, Sr, axis), 4)):
-            _, kernel_s = time_kernel(capi, torch, fn, op, steps, warmup)
+            _, kernel_s, how = time_one_kernel_op(capi, torch, fn, op, steps, warmup)
             gbs = S.numel() * bytes_per / kernel_s / 1e9
             dense["%s_%s" % (op, name)] = {"kernel_ms": 1e3 * kernel_s,
                                            "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS,
                                                         "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS}}
+            dense["%s_%s" % (op, name)].update(how)
     out["softmax_sum_f32_8192x8192"] = dense
     del S, So, Sr
     # configuration 5a: encode-and-append 4096 tokens x 8 kv heads x 128, 3-bit codes (rotate, quantise, pack)
@@ -277,18 +309,22 @@ def extras(capi, torch, workloads, steps, warmup):
         "rotation_tflops": rot_flops / secs / 1e12, "kernel_ms": 1e3 * kernel_s,
         "roofline": {"bound": "mfma", "achieved": rot_flops / kernel_s / 1e12, "peak": 157.3, "unit": "TFLOP/s",
                      "frac": rot_flops / kernel_s / 1e12 / 157.3, "kernel": "encode_rows_pair_kernel (K and V)",
-                     "flops_per_launch": rot_flops}}
+                     "flops_per_launch": rot_flops},
+        "kernel_ms_source": "event pairs around the launches (the call also resets the cache and moves the lengths, so "
+                            "a run of calls does not time the kernel alone; the events' own 2-3 us are in the figure)"}
     cache.close()
     # the append of a decode step: one new token for each of 64 sequences (one launch: the encoder writes the items
     # and moves the lengths itself)
-    n_app = 1 + warmup + 2 * steps
+    n_app = 1 + 2 * warmup + 3 * steps
     cache1 = capi.KVCache(capi.KV_LLOYDMAX, 64, wl.n_kv_heads, d, n_app, 3, 3, 1, 0)
     cache1.set_rotations(rk, rv)
     k1 = torch.randn((64, wl.n_kv_heads, 1, d), device="cuda")
     v1 = torch.randn((64, wl.n_kv_heads, 1, d), device="cuda")
-    secs, kernel_s = time_kernel(capi, torch, lambda: cache1.encode_append(k1, v1, rotate=1), "kv_encode", steps, warmup)
+    secs, kernel_s, how = time_one_kernel_op(capi, torch, lambda: cache1.encode_append(k1, v1, rotate=1), "kv_encode",
+                                             steps, warmup)
     out["append_one_token_64_sequences"] = {"ms": 1e3 * secs, "kernel_ms": 1e3 * kernel_s, "kernels_per_append": 1,
                                             "rows": 2 * 64 * wl.n_kv_heads}
+    out["append_one_token_64_sequences"].update(how)
     cache1.close()
     # configuration 4: 16 ragged sequences in [2048, 32768], K 2-bit + sign, V 3-bit, split-context merge
     wl4 = workloads.config(4)
