@@ -286,7 +286,7 @@ int weed_hip_kv_decode_attn(weed_hip_kv_cache *cache, int32_t n_q_heads, int32_t
  * (when every workgroup's share of the launch is a whole number of (sequence, kv head) regions, or every region a
  * whole number of such shares, one kernel does the whole call: that is so for batches of 1 to 256 sequences whose
  * lengths are equal or not too different -- sequences are counted as having as many blocks as the longest while that
- * adds at most 3/4 to the blocks of the batch and the cache's capacity holds them; other batches of up to 63
+ * adds at most 3/4 to the blocks of the batch; other batches of up to 63
  * sequences are one kernel too, with partial results in memory; otherwise, or with these bits, a kernel ahead rotates
  * the queries and one behind merges the partials; the ways differ in the rounding of the last bits).  A number of
  * wavefronts other than 0 switches the choice of run lengths for whole regions off.  The process-wide defaults are read once from the environment variables WEED_HIP_DECODE_WAVES,

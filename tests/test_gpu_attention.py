@@ -319,9 +319,9 @@ def test_workgroups_that_merge_their_own_regions(gpu, oracle, lloyd, d, Hkv, Hq,
                                                        (64, 61 * 64 - 1, 70, 3, 4), (128, 8000, 2500, 3, 2)])
 def test_block_counts_that_no_run_length_divides(gpu, oracle, cap_blocks, top, step, S, Hkv):
     """Sequences of 23 blocks on a full device: no run length divides them into whole regions per workgroup.
-    Where the regions' memory reaches one block further (capacity of 24 blocks) the partition counts 24 blocks per
-    region, the last one without tokens, and the call stays one kernel with whole regions per workgroup; with a
-    capacity of 23 blocks it cannot, and the runs straddle regions.  The third case mixes sequences of 23 and 24
+    The partition counts 24 blocks per region, the last one without tokens, and the call stays one kernel with whole
+    regions per workgroup -- also with a capacity of 23 blocks, where the 24th block of the last region would lie
+    behind the cache's memory and is never read.  The third case mixes sequences of 23 and 24
     blocks, which are counted alike.  The last three are small batches, where a region is several workgroups' shares
     and the count is rounded to a whole number of those; in the last one the sequences hold 8000, 5500 and 3000
     tokens and are all counted as 128 blocks, so whole workgroups find no tokens in their share.  All must agree with the checker, with the three-kernel

@@ -833,8 +833,7 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         // Equal sequences of nb blocks: prefer a run length with which every workgroup holds whole regions (the
         // kernel then does the whole call by itself, see below): nb / (classes * q) blocks with q = 1, 2 or 4, that
         // is 4 / q regions per workgroup, provided the workgroups fill the compute units in at most two rounds.
-        // A block count that no such run length divides is rounded up to the next one that one does (only as far as
-        // the regions' memory reaches, and see below): the partition then counts blocks at the end of every
+        // A block count that no such run length divides is rounded up to the next one that one does (see below): the partition then counts blocks at the end of every
         // region that hold no tokens, which the kernel skips as it skips those beyond a prefix length, and the
         // wavefront they fall to has that much less to do -- far cheaper than runs that straddle regions.
         uint32_t preferred_unit = 0;
@@ -855,8 +854,8 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         // Calls of less than a few dozen microseconds are all fixed cost, of which runs that straddle regions have
         // more: there the ratio may be four (16 sequences from [512, 8192]: 42 us against 33 us).
         const uint64_t most_counted = real_blocks * Hkv >= 32768 ? real_blocks * 7 / 4 : real_blocks * 4;
-        const uint32_t reach = (uint32_t)std::min<uint64_t>(std::max<uint64_t>(most_counted / S, fewest + 1),
-                                                            c->padded_tokens / 64);
+        // (counts beyond what a region's memory holds are fine: the kernel reads nothing behind a region's last block)
+        const uint32_t reach = (uint32_t)std::min<uint64_t>(std::max<uint64_t>(most_counted / S, fewest + 1), 1u << 24);
         const bool may_round = fewest != 0 && mfma_decode_merges(pass_heads <= 4 ? 4u : (pass_heads <= 8 ? 8u : 16u), d) &&
                                tune.wavefronts == 0 && !tune.separate_merge && !tune.always_search;
         {

@@ -697,9 +697,12 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
 
     // The first block of the segment is requested before anything else of the segment is read (the sequence's
     // attended length, the query): it exists whatever that length is, and its latency is the longest of the prologue.
+    // (A partition that counts more blocks per region than the cache holds may put b0 behind the region's memory:
+    // such a segment has no tokens and what is read for it is not used, but it is read from inside the region.)
     constexpr std::integral_constant<int, 0> p0{};
-    load_k(p0, b0);
-    load_v(p0, b0);
+    const uint32_t first_read = min(b0, (p.padded >> 6) - 1u);
+    load_k(p0, first_read);
+    load_v(p0, first_read);
 
     // ---- query operand.  The score instruction has 16 columns.  With GP <= 8 the fp16 high halves of the GP heads sit
     //      in columns [0, GP) and the low halves in [GP, 2GP), so ONE instruction per item yields both partial scores
