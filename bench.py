@@ -393,6 +393,27 @@ def extras(capi, torch, workloads, steps, warmup):
                                                        "ctx_from": wlL.max_len - steps, "ctx_to": wlL.max_len}
     cacheL.close()
     del qL, oL, kL, vL
+    # the headline shape with 64 sequences of different lengths, drawn uniformly from [4096, 8192] (seeded): what a
+    # serving batch looks like; the partition counts every sequence as the longest one
+    import random
+    rnd = random.Random(4096)
+    lens_r = [rnd.randint(4096, 8192) for _ in range(64)]
+    wlR = workloads.Workload("cfg3_ragged", 64, wlL.n_q_heads, wlL.n_kv_heads, d, lens_r, wlL.k_bits, wlL.v_bits,
+                             wlL.k_sign, wlL.v_sign, 0)
+    cacheR = capi.KVCache(capi.KV_LLOYDMAX, 64, wlR.n_kv_heads, d, 8192, wlR.k_bits, wlR.v_bits, wlR.k_sign, wlR.v_sign)
+    cacheR.set_rotations(rk, rv)
+    for s0, n in enumerate(lens_r):
+        Ks = torch.randn((1, wlR.n_kv_heads, n, d), device="cuda")
+        Vs = torch.randn((1, wlR.n_kv_heads, n, d), device="cuda")
+        cacheR.encode_append(Ks, Vs, seq_begin=s0, rotate=1)
+    del Ks, Vs
+    qR = torch.randn((64, wlR.n_q_heads, d), device="cuda")
+    oR = torch.zeros_like(qR)
+    out["cfg3_64_sequences_of_4096_to_8192_tokens"] = decode_entry(
+        capi, torch, lambda: cacheR.decode_attn(qR, oR, capi.GQA_BLOCKED, flagsL), 64, wlR.bytes_per_step(lloydmax=True),
+        steps, warmup)
+    cacheR.close()
+    del qR, oR
     # configuration 3 again with 256 sequence caches per launch (2 GB of packed rows): what the per-launch fixed cost
     # (launch, table build, first-block latency, uneven finish) amortises to with four times the bytes
     wl3 = workloads.config(3, n_seq=256)
