@@ -856,8 +856,8 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         const uint64_t most_counted = real_blocks * Hkv >= 32768 ? real_blocks * 7 / 4 : real_blocks * 4;
         // (counts beyond what a region's memory holds are fine: the kernel reads nothing behind a region's last block)
         const uint32_t reach = (uint32_t)std::min<uint64_t>(std::max<uint64_t>(most_counted / S, fewest + 1), 1u << 24);
-        const bool may_round = fewest != 0 && mfma_decode_merges(pass_heads <= 4 ? 4u : (pass_heads <= 8 ? 8u : 16u), d) &&
-                               tune.wavefronts == 0 && !tune.separate_merge && !tune.always_search;
+        // (instances that cannot merge their partials themselves gain from runs that stay inside regions as well)
+        const bool may_round = fewest != 0 && tune.wavefronts == 0 && !tune.separate_merge && !tune.always_search;
         {
             const uint32_t nb = most;
             if (may_round) {
