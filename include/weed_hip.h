@@ -241,7 +241,8 @@ int weed_hip_block_scale_f32(const float *x_dev, uint32_t off, const uint32_t sh
  * 2: rotate with the reference's order and rounding (src/ops/matmul.cpp:40-44), so that codes match a BLAS-less
  * reference build bit for bit.  Tokens are appended in logical order (token t of the call becomes token len+t).
  * An append of one token per sequence (a decode step's) and an append of whole 32-token half blocks behind whole half
- * blocks (a prefill, in chunks or not) are one kernel launch; other appends take two.  However the tokens arrive, the
+ * blocks (a prefill, in chunks or not) are one kernel launch (a large one is followed by a small kernel that moves
+ * the lengths); other appends take two.  However the tokens arrive, the
  * cache ends up with the same bits. */
 int weed_hip_kv_encode_append(weed_hip_kv_cache *cache, int32_t seq_begin, int32_t seq_count, int32_t T_new,
                               const float *k_dev, uint32_t k_off, const uint32_t k_stride[4], const float *v_dev,
