@@ -14,7 +14,7 @@ namespace weedhip {
 struct SideParams {
     const uint8_t *fields;  // packed items, one region per (sequence, kv head)
     const float *alpha;     // [n_seq][n_kv_heads][padded_tokens] row scales, LLOYDMAX only
-    const uint32_t *alpha_max; // [n_seq][n_kv_heads] bit pattern of the largest row scale seen, LLOYDMAX only
+    const uint32_t *alpha_max; // [n_seq][n_kv_heads][kScaleMaxSlots]: the largest of them is the bit pattern of the largest row scale seen, LLOYDMAX only
     uint64_t region_bytes;
     uint32_t w;             // field width
     float alpha_const;      // UNIFORM: step

@@ -203,7 +203,7 @@ struct DirectOut {
     uint8_t *out;        // packed fields of the side
     uint64_t region_bytes;
     float *alpha;        // [region][padded] row scales, null for the uniform coder
-    uint32_t *alpha_max; // [region] largest row scale (V side), or null
+    uint32_t *alpha_max; // [region][kScaleMaxSlots] largest row scale (V side), or null
     const int32_t *lens; // cached lengths BEFORE this append
     int32_t seq_begin;
     uint32_t padded, w;
@@ -646,7 +646,7 @@ __device__ __forceinline__ void encode_rows_body(const float *__restrict__ x, co
                 const uint32_t region = (uint32_t)direct.seq_begin * Hkv + row0 + tid;
                 direct.alpha[(uint64_t)region * direct.padded + tok_s[tid]] = a;
                 if (direct.alpha_max) {
-                    atomicMax(direct.alpha_max + region, __float_as_uint(fabsf(a)));
+                    atomicMax(direct.alpha_max + (uint64_t)region * kScaleMaxSlots, __float_as_uint(fabsf(a)));
                 }
             }
         } else if (direct.out) {
@@ -661,7 +661,8 @@ __device__ __forceinline__ void encode_rows_body(const float *__restrict__ x, co
                     bits = max(bits, (uint32_t)__shfl_xor((int)bits, o));
                 }
                 if (tid == 0) {
-                    atomicMax(direct.alpha_max + region, bits);
+                    // (the half blocks of a region take the words in turn)
+                    atomicMax(direct.alpha_max + (uint64_t)region * kScaleMaxSlots + (n >> 5) % kScaleMaxSlots, bits);
                 }
             }
         } else if (row0 + tid < rows) {
@@ -772,10 +773,12 @@ __device__ __forceinline__ void scatter_v_scales_body(const float *__restrict__ 
         mine = max(mine, (uint32_t)__shfl_xor((int)mine, o));
     }
     if (valid) {
+        // (the wavefronts take the region's words in turn)
+        const uint32_t slot = (row >> 6) % kScaleMaxSlots;
         if (region != lead) {
-            atomicMax(alpha_max + region, bits);
+            atomicMax(alpha_max + (uint64_t)region * kScaleMaxSlots + slot, bits);
         } else if ((threadIdx.x & 63) == (uint32_t)__builtin_ctzll(__ballot(valid && region == lead))) {
-            atomicMax(alpha_max + region, mine);
+            atomicMax(alpha_max + (uint64_t)region * kScaleMaxSlots + slot, mine);
         }
     }
 }
@@ -1367,10 +1370,10 @@ int weed_hip_kv_cache_create(weed_hip_kv_cache **cache, const weed_hip_kv_config
                 e = hipMemsetAsync(s.alpha, 0, abytes, stream());
             }
             if (e == hipSuccess) {
-                e = hipMalloc((void **)&s.alpha_max, regions * sizeof(uint32_t));
+                e = hipMalloc((void **)&s.alpha_max, regions * kScaleMaxSlots * sizeof(uint32_t));
             }
             if (e == hipSuccess) {
-                e = hipMemsetAsync(s.alpha_max, 0, regions * sizeof(uint32_t), stream());
+                e = hipMemsetAsync(s.alpha_max, 0, regions * kScaleMaxSlots * sizeof(uint32_t), stream());
             }
         }
         if (e != hipSuccess) {
@@ -1427,9 +1430,9 @@ int weed_hip_kv_cache_reset(weed_hip_kv_cache *c, int drop_rotations)
     fill_i32_kernel<<<(n + 256) / 256, 256, 0, stream()>>>(c->lens_dev, 0, n + 1); // and the append's counter
     WEED_HIP_LAUNCH_CHECK();
     if (c->v.alpha_max) {
-        const uint32_t regions = n * (uint32_t)c->cfg.n_kv_heads;
-        fill_i32_kernel<<<(regions + 255) / 256, 256, 0, stream()>>>((int32_t *)c->k.alpha_max, 0, regions);
-        fill_i32_kernel<<<(regions + 255) / 256, 256, 0, stream()>>>((int32_t *)c->v.alpha_max, 0, regions);
+        const uint32_t words = n * (uint32_t)c->cfg.n_kv_heads * kScaleMaxSlots;
+        fill_i32_kernel<<<(words + 255) / 256, 256, 0, stream()>>>((int32_t *)c->k.alpha_max, 0, words);
+        fill_i32_kernel<<<(words + 255) / 256, 256, 0, stream()>>>((int32_t *)c->v.alpha_max, 0, words);
         WEED_HIP_LAUNCH_CHECK();
     }
     if (c->dec_ws) {

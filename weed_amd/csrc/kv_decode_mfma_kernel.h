@@ -786,7 +786,11 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     constexpr float kSlack = 8.0f;
     int ep = 7;
     if (lloyd) {
-        const uint32_t bits = p.v.alpha_max[region];
+        uint32_t bits = 0; // (non-negative floats order like their bit patterns)
+#pragma unroll
+        for (uint32_t i = 0; i < kScaleMaxSlots; ++i) {
+            bits = max(bits, p.v.alpha_max[region * kScaleMaxSlots + i]);
+        }
         ep = bits ? 133 - (int)((bits >> 23) & 0xff) : 0;
         ep = ep > 100 ? 100 : (ep < -100 ? -100 : ep);
     }

@@ -32,6 +32,10 @@
 namespace weedkv {
 
 constexpr uint32_t kBlockTokens = 64;
+// The largest row scale of a region is kept as the maximum over this many words (64 bytes per region): the encoder's
+// workgroups raise different words, because raising ONE word from the 128 workgroups of a 4096-token prefill is served
+// one after the other (4 us of a 45 us encode); a reader takes the largest of them.
+constexpr uint32_t kScaleMaxSlots = 16;
 
 WK_HD uint32_t block_bytes(uint32_t d, uint32_t w) { return 8u * d * w; }
 
