@@ -855,7 +855,10 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         // more: there the ratio may be four (16 sequences from [512, 8192]: 42 us against 33 us).
         const uint64_t most_counted = real_blocks * Hkv >= 32768 ? real_blocks * 7 / 4 : real_blocks * 4;
         // (counts beyond what a region's memory holds are fine: the kernel reads nothing behind a region's last block)
-        const uint32_t reach = (uint32_t)std::min<uint64_t>(std::max<uint64_t>(most_counted / S, fewest + 1), 1u << 24);
+        // (and no further than 4096 blocks past the longest: the counts that qualify below recur every few hundred
+        // blocks at most, so a search that has found none by then finds none, and the host's time stays bounded)
+        const uint32_t reach = (uint32_t)std::min<uint64_t>(std::max<uint64_t>(most_counted / S, fewest + 1),
+                                                            std::min<uint64_t>((uint64_t)most + 4096, 1u << 24));
         // (instances that cannot merge their partials themselves gain from runs that stay inside regions as well)
         const bool may_round = fewest != 0 && tune.wavefronts == 0 && !tune.separate_merge && !tune.always_search;
         {
