@@ -833,9 +833,10 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         // Equal sequences of nb blocks: prefer a run length with which every workgroup holds whole regions (the
         // kernel then does the whole call by itself, see below): nb / (classes * q) blocks with q = 1, 2 or 4, that
         // is 4 / q regions per workgroup, provided the workgroups fill the compute units in at most two rounds.
-        // A block count that no such run length divides is rounded up to the next one that one does (see below): the partition then counts blocks at the end of every
-        // region that hold no tokens, which the kernel skips as it skips those beyond a prefix length, and the
-        // wavefront they fall to has that much less to do -- far cheaper than runs that straddle regions.
+        // A block count that no such run length divides is rounded up to the next one that one does (see below):
+        // the partition then counts blocks at the end of every region that hold no tokens, which the kernel skips
+        // as it skips those beyond a prefix length, and the wavefront they fall to has that much less to do -- far
+        // cheaper than runs that straddle regions.
         uint32_t preferred_unit = 0;
         // Sequences with different block counts are counted alike, as the longest of them, within the same bounds.
         uint32_t most = 0, fewest = ~0u;
