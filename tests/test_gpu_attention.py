@@ -442,6 +442,71 @@ def test_any_batch_as_one_kernel(gpu, oracle, lloyd, d, Hkv, Hq, lens, kb, vb, w
     cache.close()
 
 
+def test_random_batches_planned_against_plain(gpu):
+    """Sixty seeded random batches -- equal, nearly equal, mildly and widely different lengths, up to 128 sequences,
+    caches with and without room behind the longest sequence, both coders, head_dims with and without instances that
+    merge their own partials: what the default plan gives (block counts rounded up, sequences counted alike, one kernel
+    where it can) against the plain plan (real block counts, region search, three kernels), which the other tests
+    check against the CPU checker.  The bar is this file's."""
+    import torch
+    rng = np.random.default_rng(4242)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(11)
+
+    def randn(*shape):
+        return torch.randn(shape, generator=gen, device="cuda")
+
+    flags = gpu.ATTN_ROTATE_Q | gpu.ATTN_UNROTATE_OUT
+    try:
+        for case in range(60):
+            d = int(rng.choice([32, 96, 160, 256, 128, 64]))
+            Hkv = int(rng.choice([1, 2, 4, 8]))
+            G = int(rng.choice([1, 2, 4, 8]))
+            S = int(rng.choice([1, 2, 3, 5, 8, 16, 31, 40, 64, 70, 128]))
+            top = max(1, int(rng.integers(1, 50)) * 64 + int(rng.integers(-63, 1)))
+            kind = int(rng.integers(0, 4))
+            if kind == 0:
+                lens = [top] * S
+            elif kind == 1:
+                lens = [max(1, top - int(rng.integers(0, 130))) for _ in range(S)]
+            elif kind == 2:
+                lens = [max(1, int(top * rng.uniform(0.5, 1.0))) for _ in range(S)]
+            else:
+                lens = [max(1, int(top * rng.uniform(0.02, 1.0))) for _ in range(S)]
+            cap = max(lens) + int(rng.choice([0, 1, 64, 200, 1000]))
+            lloyd = bool(rng.integers(2))
+            if lloyd:
+                kb, vb = int(rng.choice([2, 3, 4])), int(rng.choice([2, 3, 4]))
+                ks, vs = int(rng.integers(2)), int(rng.integers(2))
+            else:
+                kb = vb = int(rng.choice([2, 3, 4, 5, 6, 8]))
+                ks = vs = 0
+            cache = gpu.KVCache(gpu.KV_LLOYDMAX if lloyd else gpu.KV_UNIFORM, S, Hkv, d, cap, kb, vb, ks, vs)
+            if not lloyd:
+                cache.set_scales(1.1, 0.9)
+            rk, rv = torch.zeros(d * d, device="cuda"), torch.zeros(d * d, device="cuda")
+            gpu.make_rotation(5, d, rk)
+            gpu.make_rotation(6, d, rv)
+            cache.set_rotations(rk, rv)
+            for s, n in enumerate(lens):
+                cache.encode_append(randn(1, Hkv, n, d), randn(1, Hkv, n, d), seq_begin=s, rotate=1)
+            q = randn(S, Hkv * G, d)
+            planned, plain = torch.zeros_like(q), torch.zeros_like(q)
+            gpu.decode_tuning()
+            cache.decode_attn(q, planned, gpu.GQA_BLOCKED, flags)
+            gpu.decode_tuning(always_search=True, separate_merge=True, separate_query=True)
+            cache.decode_attn(q, plain, gpu.GQA_BLOCKED, flags)
+            gpu.sync()
+            what = "case %d: d %d, K %d+%d V %d+%d bits, lloyd %d, %d x %d heads, capacity %d, lengths %s" % (
+                case, d, kb, ks, vb, vs, lloyd, Hkv, G, cap, lens)
+            assert not torch.isnan(planned).any(), what
+            excess = ((planned - plain).abs() - (1e-4 + 1e-3 * plain.abs())).max().item()
+            assert excess <= 0, what
+            cache.close()
+    finally:
+        gpu.decode_tuning()
+
+
 def test_edge_lengths(gpu, oracle):
     """Empty sequences give zeros; lengths 1, 63, 64, 65 around the 64-token block; an appended token changes the
     result exactly as the checker says."""
