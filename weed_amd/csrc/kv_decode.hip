@@ -470,6 +470,9 @@ constexpr uint32_t kMaxSlots = 1024; // partials per (sequence, head) that combi
 // two wavefronts per SIMD the older one gets 16 % more than the mean; with three the spread between oldest and
 // youngest is wider (measured on the ragged batch: 16 % -> 47.8 us, 24-40 % -> 46.7-46.9 us, 48 % -> 48.2 us).
 constexpr uint32_t kRunSkewPercent = 16, kRunSkewPercent3 = 28;
+// Most regions that the blocks of one workgroup may lie in for the workgroups to merge their regions themselves in the
+// general case (see decode_impl).
+constexpr uint32_t kMostRegionsMergedByWorkgroup = 6;
 
 // Tuning knobs of the work partition.  The defaults come from the environment, read ONCE per process (at the first
 // decode call or the first weed_hip_kv_decode_tuning): WEED_HIP_DECODE_WAVES (wavefronts the block list is cut for),
@@ -853,8 +856,10 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         // [4096, 8192]: 104.6 us with runs that straddle regions, 84.4 us counted alike; from [512, 8192], where the
         // partition would count 1.78 blocks per block with tokens: 76.3 against 73.9 us, a tie.)
         // Calls of less than a few dozen microseconds are all fixed cost, of which runs that straddle regions have
-        // more: there the ratio may be four (16 sequences from [512, 8192]: 42 us against 33 us).
-        const uint64_t most_counted = real_blocks * Hkv >= 32768 ? real_blocks * 7 / 4 : real_blocks * 4;
+        // more: there the ratio may be four (16 sequences from [512, 8192]: 42 us against 33 us).  What bounds such
+        // calls is the blocks as counted, which is what a wavefront of the longest sequence works through: 32
+        // sequences with up to 8192 tokens each gain 8 to 17 us counted alike, 48 such sequences lose 5 to 44 us.
+        const uint64_t most_counted = (uint64_t)most * S * Hkv > 32768 ? real_blocks * 7 / 4 : real_blocks * 4;
         // (counts beyond what a region's memory holds are fine: the kernel reads nothing behind a region's last block)
         // (and no further than 4096 blocks past the longest: the counts that qualify below recur every few hundred
         // blocks at most, so a search that has found none by then finds none, and the host's time stays bounded)
@@ -1040,8 +1045,13 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         }
         // Anything else that the instance can merge: one slot per (run, region) in memory, an arrival counter per
         // region (ragged batches: up to 63 sequences, whose block offsets a wavefront keeps in one register).
+        // A workgroup merges the regions that it completes one after the other, at its end, about 2 us each, where
+        // the separate kernel merges all regions at once for 10 to 12 us: measured on batches that are half long and
+        // half short sequences, the workgroups win up to 6 regions per workgroup, tie at 7 and lose from 8 on (5 to
+        // 30 us at 8 to 17).
         if (wg_regions == 0 && region_wgs == 0 && mfma_decode_merges(gp, d) && every_sequence_has_tokens &&
-            (nb != 0 || (S <= 63 && !decode_tuning().always_search)) && n_splits <= 64 && wg_most_regions <= 31 &&
+            (nb != 0 || (S <= 63 && !decode_tuning().always_search)) && n_splits <= 64 &&
+            wg_most_regions <= kMostRegionsMergedByWorkgroup &&
             (size_t)S * Hkv <= kMfmaMergeCounters && !decode_tuning().separate_merge) {
             general_merge = true;
         }
