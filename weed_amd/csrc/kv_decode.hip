@@ -869,7 +869,28 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         const bool may_round = fewest != 0 && tune.wavefronts == 0 && !tune.separate_merge && !tune.always_search;
         {
             const uint32_t nb = most;
-            if (may_round) {
+            // Fewer blocks than wavefronts and regions of no more blocks than a workgroup has wavefronts: the call is
+            // all fixed cost, of which the rows that a workgroup rotates and merges one pass after the other are the
+            // largest part, so as few regions per workgroup as one round of workgroups allows, however few of the
+            // compute units they fill (3 to 96 sequences of 100 tokens with groups of eight: 27 us with four regions
+            // per workgroup, 14 us with one).
+            const bool tiny = real_blocks * Hkv <= (uint64_t)runs.waves * 256u && nb <= runs.waves;
+            if (may_round && tiny) {
+                const uint32_t classes = run_classes(runs), regions = S * Hkv;
+                for (uint32_t q = 4; q >= 1 && !preferred_unit; q /= 2) {
+                    if ((regions * q + 3) / 4 > 256) {
+                        continue;
+                    }
+                    for (uint32_t cand = nb; cand <= reach; ++cand) {
+                        if (cand % (classes * q) == 0) {
+                            preferred_unit = cand / (classes * q);
+                            virtual_blocks = cand == fewest ? 0 : cand;
+                            break;
+                        }
+                    }
+                }
+            }
+            if (may_round && !preferred_unit) {
                 const uint32_t classes = run_classes(runs), regions = S * Hkv;
                 for (uint32_t cand = nb; cand <= reach && !preferred_unit; ++cand) {
                     uint32_t best_rounds = 3;
@@ -905,7 +926,7 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
                 const uint64_t all = (uint64_t)cand * S * Hkv;
                 const uint32_t unit = (uint32_t)std::max<uint64_t>(1, (all + target_units - 1) / target_units);
                 const uint32_t wg_blocks = runs.waves * unit;
-                if (cand % wg_blocks == 0 && cand / wg_blocks >= 2 && cand / wg_blocks <= 64 && all < (1ull << 32)) {
+                if (cand % wg_blocks == 0 && cand / wg_blocks <= 64 && all < (1ull << 32)) {
                     if (cand != fewest) {
                         virtual_blocks = cand;
                         total_blocks = (uint32_t)all;
@@ -1048,10 +1069,11 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         // A workgroup merges the regions that it completes one after the other, at its end, about 2 us each, where
         // the separate kernel merges all regions at once for 10 to 12 us: measured on batches that are half long and
         // half short sequences, the workgroups win up to 6 regions per workgroup, tie at 7 and lose from 8 on (5 to
-        // 30 us at 8 to 17).
+        // 30 us at 8 to 17).  Nor do they where they could not rotate their queries as well (a kernel ahead and the
+        // merges at the end: 3 to 200 sequences of 100 tokens with groups of eight, 27 us against 22 to 25).
         if (wg_regions == 0 && region_wgs == 0 && mfma_decode_merges(gp, d) && every_sequence_has_tokens &&
             (nb != 0 || (S <= 63 && !decode_tuning().always_search)) && n_splits <= 64 &&
-            wg_most_regions <= kMostRegionsMergedByWorkgroup &&
+            wg_most_regions <= kMostRegionsMergedByWorkgroup && wg_most_regions * pass_heads <= kMfmaQueryRows &&
             (size_t)S * Hkv <= kMfmaMergeCounters && !decode_tuning().separate_merge) {
             general_merge = true;
         }
