@@ -114,7 +114,7 @@ int weed_hip_copy_f32(uint64_t n, const float *a_dev, uint32_t a_off, uint32_t a
                       uint32_t o_stride);
 
 /* Broadcasting elementwise ops on tensors of one logical shape (rank <= 8, strides in elements, stride 0 repeats a
- * dimension): out = a (COPY; b may be NULL), a + b, a - b, a * b, a / b.  Replace Weed's add / mul
+ * dimension): out = a (COPY; b may be NULL), a + b, a - b, a * b, a / b, and the activations below.  Replace Weed's add / mul
  * (src/ops/commuting.cpp:17-25), sub (src/ops/sub.cpp), div with IEEE division (src/ops/div.cpp:17-20), add_in_place
  * (src/ops/in_place.cpp:17-25, out aliasing a) and the strided gather behind Tensor::contiguous
  * (include/tensors/tensor.hpp:319-331). */
@@ -123,7 +123,17 @@ enum {
     WEED_HIP_EW_ADD = 1,
     WEED_HIP_EW_SUB = 2,
     WEED_HIP_EW_MUL = 3,
-    WEED_HIP_EW_DIV = 4
+    WEED_HIP_EW_DIV = 4,
+    /* a * sigmoid(a) * b: the gate of SwiGLU::forward (include/modules/swiglu.hpp:71-77: `gate * Tensor::sigmoid(gate)
+     * * up`, three elementwise ops in the reference) as one pass */
+    WEED_HIP_EW_SILU_MUL = 5,
+    /* unary (b may be NULL): Weed::relu / sigmoid / tanh (src/ops/real_unary.cpp:80,135,191) and Tensor::gelu
+     * (src/tensors/tensor.cpp:841-851: 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))), eight elementwise ops in the
+     * reference) */
+    WEED_HIP_EW_RELU = 6,
+    WEED_HIP_EW_SIGMOID = 7,
+    WEED_HIP_EW_TANH = 8,
+    WEED_HIP_EW_GELU = 9
 };
 int weed_hip_elementwise_f32(int op, uint32_t rank, const uint32_t *shape, const float *a_dev, uint32_t a_off,
                              const uint32_t *a_stride, const float *b_dev, uint32_t b_off, const uint32_t *b_stride,
@@ -142,6 +152,20 @@ int weed_hip_triu_fill_f32(uint32_t rows, uint32_t cols, float val, uint32_t dia
 int weed_hip_rope_f32(const uint32_t shape[4], const float *x_dev, uint32_t x_off, const uint32_t x_stride[4],
                       const float *cos_dev, const float *sin_dev, uint32_t table_rows, uint32_t pos0, float *out_dev,
                       uint32_t o_off, const uint32_t o_stride[4]);
+
+/* RMSNorm::forward (include/modules/rms_norm.hpp:34-38: `x / ((mean(x * x, axis) + eps) ^ 0.5) * weight`, seven ops
+ * and an axis reduction in the reference) as one kernel: out = x / sqrt(mean(x^2 over axis) + eps) * w, with
+ * w[w_off + j * w_stride] for index j along the axis.  rank <= 8; x and out may be the same tensor. */
+int weed_hip_rms_norm_f32(uint32_t rank, const uint32_t *shape, uint32_t axis, const float *x_dev, uint32_t x_off,
+                          const uint32_t *x_stride, const float *w_dev, uint32_t w_off, uint32_t w_stride, float eps,
+                          float *out_dev, uint32_t o_off, const uint32_t *o_stride);
+
+/* LayerNorm::forward (src/modules/layernorm.cpp:29-42) as one kernel: xc = x - mean(x over axis),
+ * out = xc / sqrt(mean(xc^2) + eps) * gamma + beta, gamma and beta indexed along the axis like w above. */
+int weed_hip_layer_norm_f32(uint32_t rank, const uint32_t *shape, uint32_t axis, const float *x_dev, uint32_t x_off,
+                            const uint32_t *x_stride, const float *gamma_dev, uint32_t gamma_off, uint32_t gamma_stride,
+                            const float *beta_dev, uint32_t beta_off, uint32_t beta_stride, float eps, float *out_dev,
+                            uint32_t o_off, const uint32_t *o_stride);
 
 /* Numerically stable softmax along `axis`.  Replaces Weed::softmax (src/ops/softmax.cpp:276-287; OpenCL kernel
  * softmax_forward, qengine.cl:1001-1033).  rank <= 8. */

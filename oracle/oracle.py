@@ -206,6 +206,56 @@ def rope_forward(x, cos_t, sin_t, max_seq_len, pos0=0):
     return out
 
 
+# ---- activations and norms -----------------------------------------------------------------------
+
+RELU, SIGMOID, TANH, GELU = 0, 1, 2, 3
+
+
+def unary(op, x):
+    x = _f32(x)
+    out = np.empty_like(x)
+    fn = lib().wo_unary
+    fn.argtypes = [c_int, c_void_p, c_size_t, c_void_p]
+    fn(op, _p(x), x.size, _p(out))
+    return out
+
+
+def silu_mul(gate, up):
+    gate, up = _f32(gate), _f32(up)
+    out = np.empty_like(gate)
+    fn = lib().wo_silu_mul
+    fn.argtypes = [c_void_p, c_void_p, c_size_t, c_void_p]
+    fn(_p(gate), _p(up), gate.size, _p(out))
+    return out
+
+
+def norm_epsilon():
+    fn = lib().wo_norm_epsilon
+    fn.restype = c_float
+    return float(fn())
+
+
+def rms_norm(x, w, eps=None):
+    """x: [rows, n] (normalised along the last axis), w: [n]."""
+    x, w = _f32(x), _f32(w)
+    rows, n = x.shape
+    out = np.empty_like(x)
+    fn = lib().wo_rms_norm
+    fn.argtypes = [c_void_p, c_size_t, c_size_t, c_void_p, c_float, c_void_p]
+    fn(_p(x), rows, n, _p(w), c_float(norm_epsilon() if eps is None else eps), _p(out))
+    return out
+
+
+def layer_norm(x, gamma, beta, eps=None):
+    x, gamma, beta = _f32(x), _f32(gamma), _f32(beta)
+    rows, n = x.shape
+    out = np.empty_like(x)
+    fn = lib().wo_layer_norm
+    fn.argtypes = [c_void_p, c_size_t, c_size_t, c_void_p, c_void_p, c_float, c_void_p]
+    fn(_p(x), rows, n, _p(gamma), _p(beta), c_float(norm_epsilon() if eps is None else eps), _p(out))
+    return out
+
+
 # ---- decode attention ----------------------------------------------------------------------------
 
 def decode_attn(kspec, vspec, kf, ka, vf, va, q, seq_lens, gqa_weed=True, Rk=None, Rv=None, want_scores=False):

@@ -15,6 +15,13 @@
  *   wo_rope_tables / wo_rope_forward        : the reference has no test of RoPE -- PARITY UNPINNED against
  *       the reference; pinned by float64 closed forms of the tables, the identity at position 0 and the
  *       per-coordinate formula evaluated independently in numpy.
+ *   wo_unary, wo_silu_mul                   : the reference's unit tests (test/tests.cpp:230-244, 284-291,
+ *       314-321: relu(2) = 2, relu(-2) = 0, sigmoid(0) = 0.5, tanh(0) = 0) and float64 closed forms of every
+ *       function; gelu additionally against erf-free float64 evaluation of the same tanh formula.
+ *   wo_rms_norm, wo_layer_norm              : the reference has no test of either module -- PARITY UNPINNED
+ *       against the reference; pinned by float64 closed forms, by what the mathematics fixes (unit mean square /
+ *       zero mean and unit variance of the result before the affine step, scale invariance, a constant row) and by
+ *       the reference's test of the axis mean they are built from (test/tests.cpp:111-120: mean(1, 2, 3) = 2).
  *   wo_block_scale                          : float64 closed form (order-dependent in the last ulps).
  *   wo_orthonormalize_columns, wo_apply_rotation : invariants only (R^T R = I, y = x R, R R^T = I);
  *       the reference draws its Gaussian matrix from std::random_device, so no vector exists.
@@ -428,6 +435,109 @@ void wo_rope_forward(const float *x, uint32_t B, uint32_t H, uint32_t T, uint32_
             }
         }
     }
+}
+
+/* ------------------------------------------------------------------------------------------ */
+/* activations and norms                                                                       */
+/* ------------------------------------------------------------------------------------------ */
+
+/* include/common/weed_types.hpp:213-214: FP_NORM_EPSILON = epsilon / 4 of the real type */
+float wo_norm_epsilon(void) { return 1.1920928955078125e-07f / 4.0f; }
+
+/* src/ops/real_unary.cpp:80 (relu: std::max(x, 0)), :135 (sigmoid: 1 / (1 + exp(-x)), float exp), :191 (tanh);
+ * src/tensors/tensor.cpp:841-851 (gelu): x3 = x * x * x; inner = k2 * (x + k1 * x3); t = tanh(inner);
+ * k0 * x * (ones + t) -- every operator is a separate elementwise op, so every intermediate is rounded to float. */
+void wo_unary(int op, const float *x, size_t n, float *out)
+{
+    const float k0 = 0.5f, k1 = 0.044715f, k2 = 0.7978845608028654f;
+    for (size_t i = 0; i < n; ++i) {
+        const float v = x[i];
+        float r;
+        if (op == 0) {
+            r = (v > 0.0f) ? v : 0.0f;
+        } else if (op == 1) {
+            r = 1.0f / (1.0f + expf(-v));
+        } else if (op == 2) {
+            r = tanhf(v);
+        } else {
+            const float xx = v * v;
+            const float x3 = xx * v;
+            const float s = k1 * x3;
+            const float u = v + s;
+            const float inner = k2 * u;
+            const float t = tanhf(inner);
+            const float half_x = k0 * v;
+            const float one_t = 1.0f + t;
+            r = half_x * one_t;
+        }
+        out[i] = r;
+    }
+}
+
+/* include/modules/swiglu.hpp:75: gate * Tensor::sigmoid(gate) * up, left to right */
+void wo_silu_mul(const float *gate, const float *up, size_t n, float *out)
+{
+    for (size_t i = 0; i < n; ++i) {
+        const float sg = 1.0f / (1.0f + expf(-gate[i]));
+        const float a = gate[i] * sg;
+        out[i] = a * up[i];
+    }
+}
+
+/* Tensor::mean(a, axis) (src/tensors/tensor.cpp:682-693): Weed::reduce adds along the axis in index order
+ * (src/ops/reduce.cpp:33-38), then one division by the length */
+static float axis_mean(const float *v, size_t n)
+{
+    float sum = 0.0f;
+    for (size_t j = 0; j < n; ++j) {
+        sum += v[j];
+    }
+    return sum / (float)n;
+}
+
+/* include/modules/rms_norm.hpp:34-38: (x / ((mean(x * x, axis) + eps) ^ 0.5)) * weight; `^` is std::pow on floats
+ * (src/ops/pow.cpp:52-56) */
+void wo_rms_norm(const float *x, size_t rows, size_t n, const float *w, float eps, float *out)
+{
+    float *sq = (float *)malloc(sizeof(float) * n);
+    for (size_t r = 0; r < rows; ++r) {
+        const float *row = x + r * n;
+        for (size_t j = 0; j < n; ++j) {
+            sq[j] = row[j] * row[j];
+        }
+        const float t = axis_mean(sq, n) + eps;
+        const float root = powf(t, 0.5f);
+        for (size_t j = 0; j < n; ++j) {
+            const float q = row[j] / root;
+            out[r * n + j] = q * w[j];
+        }
+    }
+    free(sq);
+}
+
+/* src/modules/layernorm.cpp:29-42: xc = x - mean(x, -1); y = xc / ((mean(xc * xc, -1) + eps) ^ 0.5);
+ * y = y * gamma + beta */
+void wo_layer_norm(const float *x, size_t rows, size_t n, const float *gamma, const float *beta, float eps, float *out)
+{
+    float *xc = (float *)malloc(sizeof(float) * n);
+    float *sq = (float *)malloc(sizeof(float) * n);
+    for (size_t r = 0; r < rows; ++r) {
+        const float *row = x + r * n;
+        const float mu = axis_mean(row, n);
+        for (size_t j = 0; j < n; ++j) {
+            xc[j] = row[j] - mu;
+            sq[j] = xc[j] * xc[j];
+        }
+        const float t = axis_mean(sq, n) + eps;
+        const float root = powf(t, 0.5f);
+        for (size_t j = 0; j < n; ++j) {
+            const float q = xc[j] / root;
+            const float g = q * gamma[j];
+            out[r * n + j] = g + beta[j];
+        }
+    }
+    free(xc);
+    free(sq);
 }
 
 /* ------------------------------------------------------------------------------------------ */

@@ -74,6 +74,19 @@ void wo_reduce(int op, int rank, const uint32_t *shape, int axis, const float *a
 void wo_triu_fill(float *a, uint32_t off, uint32_t rows, uint32_t cols, uint32_t s0, uint32_t s1, float val,
                   uint32_t diagonal);
 
+/* ---- activations and norms of the attention module's two callers ---- */
+/* op 0 relu, 1 sigmoid, 2 tanh (src/ops/real_unary.cpp:80,135,191), 3 gelu as Tensor::gelu composes it from
+ * elementwise ops (src/tensors/tensor.cpp:841-851) */
+void wo_unary(int op, const float *x, size_t n, float *out);
+/* SwiGLU::forward's gate (include/modules/swiglu.hpp:71-77): (gate * sigmoid(gate)) * up */
+void wo_silu_mul(const float *gate, const float *up, size_t n, float *out);
+/* RMSNorm::forward (include/modules/rms_norm.hpp:34-38) over dense rows [rows][n]; w: [n] */
+void wo_rms_norm(const float *x, size_t rows, size_t n, const float *w, float eps, float *out);
+/* LayerNorm::forward (src/modules/layernorm.cpp:29-42) over dense rows [rows][n]; gamma, beta: [n] */
+void wo_layer_norm(const float *x, size_t rows, size_t n, const float *gamma, const float *beta, float eps, float *out);
+/* FP_NORM_EPSILON at fp32 (include/common/weed_types.hpp:213-214): the eps both norms default to */
+float wo_norm_epsilon(void);
+
 /* ---- single-query decode attention over a quantized cache, in the reference's cost structure
  * (multihead_attention.cpp:259-348): dequantise the whole cache to dense fp32, replicate KV heads,
  * materialise K^T, naive dots, divide by sqrt(d), three-pass softmax, naive P.V, un-rotate. ---- */

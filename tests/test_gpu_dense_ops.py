@@ -534,3 +534,88 @@ def test_random_shapes_and_layouts(gpu):
         y = view(shape, int(rng.integers(3)))
         gpu.elementwise(gpu.EW_COPY, x, None, y)
         assert torch.equal(x, y), what
+
+
+# ---- activations and norms of the attention module's callers ---------------------------------------------------
+
+def test_activations_reference_cases_and_checker(gpu, oracle):
+    """Weed::relu / sigmoid / tanh (src/ops/real_unary.cpp:80,135,191), Tensor::gelu (src/tensors/tensor.cpp:841-851)
+    and SwiGLU's gate (include/modules/swiglu.hpp:71-77).  The reference's own cases (test/tests.cpp:230-244, 284-291,
+    314-321) exactly, then seeded values against the CPU checker: relu bit for bit, the others to a few ulp (they go
+    through exp / tanh, whose last bit differs between math libraries)."""
+    import torch
+
+    def run(op, v, b=None):
+        a = dev(np.asarray(v, dtype=np.float32))
+        out = torch.zeros_like(a)
+        gpu.elementwise(op, a, dev(np.asarray(b, dtype=np.float32)) if b is not None else None, out)
+        return out.cpu().numpy()
+
+    assert run(gpu.EW_RELU, [2.0, -2.0]).tolist() == [2.0, 0.0]
+    assert run(gpu.EW_SIGMOID, [0.0])[0] == 0.5
+    assert run(gpu.EW_TANH, [0.0])[0] == 0.0
+    rng = np.random.default_rng(11)
+    x = np.concatenate([rng.standard_normal(100000) * 3, [0.0, -0.0, 30.0, -30.0, 88.0, -88.0]]).astype(np.float32)
+    up = rng.standard_normal(x.size).astype(np.float32)
+    np.testing.assert_array_equal(run(gpu.EW_RELU, x), oracle.unary(oracle.RELU, x))
+    np.testing.assert_allclose(run(gpu.EW_SIGMOID, x), oracle.unary(oracle.SIGMOID, x), rtol=1e-6, atol=1e-37)
+    np.testing.assert_allclose(run(gpu.EW_TANH, x), oracle.unary(oracle.TANH, x), rtol=1e-6, atol=1e-37)
+    np.testing.assert_allclose(run(gpu.EW_GELU, x), oracle.unary(oracle.GELU, x), rtol=2e-6, atol=3e-7)
+    np.testing.assert_allclose(run(gpu.EW_SILU_MUL, x, up), oracle.silu_mul(x, up), rtol=2e-6, atol=1e-37)
+    # strided and broadcast operands: a column-major (B, T, d_ff) gate against an `up` that repeats over T
+    g3 = rng.standard_normal((5, 3, 70)).astype(np.float32)
+    u3 = rng.standard_normal((5, 1, 70)).astype(np.float32)
+    gd, ud = col_major(g3), col_major(u3)
+    out = torch.zeros_like(gd)
+    gpu.elementwise(gpu.EW_SILU_MUL, gd, ud, out)
+    want = oracle.silu_mul(g3, np.broadcast_to(u3, g3.shape))
+    np.testing.assert_allclose(out.cpu().numpy(), want, rtol=2e-6, atol=1e-37)
+
+
+@pytest.mark.parametrize("shape,axis", [((3,), 0), ((64, 1, 4096), 2), ((4, 6, 8), 2), ((16, 6, 8), 2), ((3, 5, 4096), 2),
+                                        ((2, 700, 96), 2), ((4096, 3), 0), ((20000, 40), 1), ((7, 20000), 1),
+                                        ((33, 4, 5000), 2), ((5, 9, 11), 1)])
+def test_norms_against_checker(gpu, oracle, shape, axis):
+    """RMSNorm::forward (include/modules/rms_norm.hpp:34-38) and LayerNorm::forward (src/modules/layernorm.cpp:29-42)
+    as one kernel each, on column-major tensors (the layout the modules see: a decode step's (B, 1, d_model) has the
+    batch index fastest) and on row-major ones (the axis contiguous), against the CPU checker.  The checker adds a
+    row one element after the other in fp32 as the reference does; the kernels add as trees, so the comparison allows
+    the rounding of a sum of that length, and a float64 evaluation has to lie within the same distance."""
+    import torch
+    rng = np.random.default_rng(shape[0] * 7 + len(shape))
+    n = shape[axis]
+    x = (rng.standard_normal(shape) * rng.uniform(0.5, 8.0) + rng.uniform(-1, 1)).astype(np.float32)
+    w = rng.uniform(0.5, 2.0, n).astype(np.float32)
+    beta = rng.standard_normal(n).astype(np.float32)
+    eps = oracle.norm_epsilon()
+    rows = np.moveaxis(x, axis, -1).reshape(-1, n)
+    back = lambda y: np.moveaxis(y.reshape(np.moveaxis(x, axis, -1).shape), -1, axis)
+    want_rms, want_ln = back(oracle.rms_norm(rows, w)), back(oracle.layer_norm(rows, w, beta))
+    x64 = x.astype(np.float64)
+    bshape = [1] * len(shape)
+    bshape[axis] = n
+    w64, b64 = w.astype(np.float64).reshape(bshape), beta.astype(np.float64).reshape(bshape)
+    f64_rms = x64 / np.sqrt(np.mean(x64 * x64, axis=axis, keepdims=True) + eps) * w64
+    xc = x64 - x64.mean(axis=axis, keepdims=True)
+    f64_ln = xc / np.sqrt(np.mean(xc * xc, axis=axis, keepdims=True) + eps) * w64 + b64
+    tol = dict(rtol=2e-5, atol=2e-5)
+    wd, bd = dev(w), dev(beta)
+    for mk in (col_major, dev):
+        xd = mk(x)
+        out = torch.zeros_like(xd)
+        gpu.rms_norm(xd, wd, eps, out, axis)
+        np.testing.assert_allclose(out.cpu().numpy(), want_rms, **tol)
+        np.testing.assert_allclose(out.cpu().numpy(), f64_rms, **tol)
+        out2 = torch.zeros_like(xd)
+        gpu.layer_norm(xd, wd, bd, eps, out2, axis)
+        np.testing.assert_allclose(out2.cpu().numpy(), want_ln, **tol)
+        np.testing.assert_allclose(out2.cpu().numpy(), f64_ln, **tol)
+        # in place (the modules never do, the entry points allow it)
+        gpu.rms_norm(xd, wd, eps, xd, axis)
+        np.testing.assert_array_equal(xd.cpu().numpy(), out.cpu().numpy())
+    # a strided weight: every second element of a longer vector
+    w2 = dev(np.repeat(w, 2))[::2]
+    xd = col_major(x)
+    out = torch.zeros_like(xd)
+    gpu.rms_norm(xd, w2, eps, out, axis)
+    np.testing.assert_allclose(out.cpu().numpy(), want_rms, **tol)

@@ -16,6 +16,7 @@ KV_UNIFORM, KV_LLOYDMAX = 0, 1
 GQA_WEED, GQA_BLOCKED = 0, 1
 ATTN_ROTATE_Q, ATTN_UNROTATE_OUT = 1, 2
 REDUCE_SUM, REDUCE_MAX, REDUCE_MIN = 0, 1, 2
+EW_COPY, EW_ADD, EW_SUB, EW_MUL, EW_DIV, EW_SILU_MUL, EW_RELU, EW_SIGMOID, EW_TANH, EW_GELU = range(10)
 
 
 class KVConfig(ctypes.Structure):
@@ -65,6 +66,10 @@ SIGNATURES = {
     "weed_hip_triu_fill_f32": (c_int, [c_uint32, c_uint32, c_float, c_uint32, c_void_p, c_uint32, c_uint32, c_uint32]),
     "weed_hip_rope_f32": (c_int, [U32P, c_void_p, c_uint32, U32P, c_void_p, c_void_p, c_uint32, c_uint32, c_void_p,
                                   c_uint32, U32P]),
+    "weed_hip_rms_norm_f32": (c_int, [c_uint32, U32P, c_uint32, c_void_p, c_uint32, U32P, c_void_p, c_uint32, c_uint32,
+                                      c_float, c_void_p, c_uint32, U32P]),
+    "weed_hip_layer_norm_f32": (c_int, [c_uint32, U32P, c_uint32, c_void_p, c_uint32, U32P, c_void_p, c_uint32, c_uint32,
+                                        c_void_p, c_uint32, c_uint32, c_float, c_void_p, c_uint32, U32P]),
     "weed_hip_softmax_f32": (c_int, [c_uint32, U32P, c_uint32, c_void_p, c_uint32, U32P, c_void_p, c_uint32, U32P]),
     "weed_hip_reduce_f32": (c_int, [c_int, c_uint32, U32P, c_uint32, c_void_p, c_uint32, U32P, c_void_p, c_uint32,
                                     U32P]),
@@ -324,6 +329,21 @@ def elementwise(op, a, b, out):
         bp, bs = c_void_p(b.data_ptr()), u32(b.stride())
     check(load().weed_hip_elementwise_f32(op, out.dim(), u32(out.shape), c_void_p(a.data_ptr()), 0, u32(a.stride()),
                                           bp, 0, bs, c_void_p(out.data_ptr()), 0, u32(out.stride())))
+
+
+def rms_norm(x, w, eps, out, axis=-1):
+    """out = x / sqrt(mean(x^2 over axis) + eps) * w on torch views; w is a 1-D view along the axis."""
+    axis %= x.dim()
+    check(load().weed_hip_rms_norm_f32(x.dim(), u32(x.shape), axis, c_void_p(x.data_ptr()), 0, u32(x.stride()),
+                                       c_void_p(w.data_ptr()), 0, w.stride(0), eps, c_void_p(out.data_ptr()), 0,
+                                       u32(out.stride())))
+
+
+def layer_norm(x, gamma, beta, eps, out, axis=-1):
+    axis %= x.dim()
+    check(load().weed_hip_layer_norm_f32(x.dim(), u32(x.shape), axis, c_void_p(x.data_ptr()), 0, u32(x.stride()),
+                                         c_void_p(gamma.data_ptr()), 0, gamma.stride(0), c_void_p(beta.data_ptr()), 0,
+                                         beta.stride(0), eps, c_void_p(out.data_ptr()), 0, u32(out.stride())))
 
 
 def triu_fill(a, val, diagonal=1):

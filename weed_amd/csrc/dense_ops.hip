@@ -550,9 +550,27 @@ template <int OP> __global__ void __launch_bounds__(256) elementwise_kernel(cons
         float r;
         if (OP == 0) {
             r = x;
-        } else {
+        } else if (OP <= 5) {
             const float y = b[bi];
-            r = OP == 1 ? x + y : OP == 2 ? x - y : OP == 3 ? x * y : x / y;
+            if (OP == 5) {
+                // SwiGLU's gate (include/modules/swiglu.hpp:71-77): gate * sigmoid(gate) * up, left to right
+                const float sg = 1.0f / (1.0f + expf(-x));
+                r = (x * sg) * y;
+            } else {
+                r = OP == 1 ? x + y : OP == 2 ? x - y : OP == 3 ? x * y : x / y;
+            }
+        } else if (OP == 6) {
+            r = fmaxf(x, 0.0f); // src/ops/real_unary.cpp:80
+        } else if (OP == 7) {
+            r = 1.0f / (1.0f + expf(-x)); // src/ops/real_unary.cpp:135
+        } else if (OP == 8) {
+            r = tanhf(x); // src/ops/real_unary.cpp:191
+        } else {
+            // Tensor::gelu (src/tensors/tensor.cpp:841-851), one rounded operation after the other as the reference's
+            // chain of elementwise ops: x3 = x * x * x; inner = k2 * (x + k1 * x3); k0 * x * (1 + tanh(inner))
+            const float x3 = (x * x) * x;
+            const float inner = 0.7978845608028654f * (x + 0.044715f * x3);
+            r = (0.5f * x) * (1.0f + tanhf(inner));
         }
         out[oi] = r;
     }
@@ -741,9 +759,10 @@ int weed_hip_elementwise_f32(int op, uint32_t rank, const uint32_t *shape, const
                              float *out_dev, uint32_t o_off, const uint32_t *o_stride)
 {
     const char *fn = "weed_hip_elementwise_f32";
-    WEED_HIP_REQUIRE(op >= WEED_HIP_EW_COPY && op <= WEED_HIP_EW_DIV, "%s: unknown op %d", fn, op);
+    WEED_HIP_REQUIRE(op >= WEED_HIP_EW_COPY && op <= WEED_HIP_EW_GELU, "%s: unknown op %d", fn, op);
     WEED_HIP_REQUIRE(a_dev && out_dev && shape && a_stride && o_stride, "%s: null pointer", fn);
-    WEED_HIP_REQUIRE(op == WEED_HIP_EW_COPY || (b_dev && b_stride), "%s: null second operand", fn);
+    const bool unary = op == WEED_HIP_EW_COPY || op >= WEED_HIP_EW_RELU;
+    WEED_HIP_REQUIRE(unary || (b_dev && b_stride), "%s: null second operand", fn);
     WEED_HIP_REQUIRE(rank >= 1 && rank <= (uint32_t)kMaxRank, "%s: rank %u outside [1, %d]", fn, rank, kMaxRank);
     WEED_HIP_TRY(ensure_init());
     PointGeom g;
@@ -756,7 +775,7 @@ int weed_hip_elementwise_f32(int op, uint32_t rank, const uint32_t *shape, const
         WEED_HIP_REQUIRE(shape[i] > 0, "%s: dimension %u is empty", fn, i);
         g.shape[i] = shape[i];
         g.a_stride[i] = a_stride[i];
-        g.b_stride[i] = op == WEED_HIP_EW_COPY ? 0 : b_stride[i];
+        g.b_stride[i] = unary ? 0 : b_stride[i];
         g.o_stride[i] = o_stride[i];
         g.n *= shape[i];
     }
@@ -800,8 +819,23 @@ int weed_hip_elementwise_f32(int op, uint32_t rank, const uint32_t *shape, const
         }
     }
     const uint32_t blocks = (uint32_t)std::min<uint64_t>((g.n + 255) / 256, 256u * 64u);
-    const float *b = op == WEED_HIP_EW_COPY ? a_dev : b_dev;
+    const float *b = unary ? a_dev : b_dev;
     switch (op) {
+    case WEED_HIP_EW_SILU_MUL:
+        elementwise_kernel<5><<<blocks, 256, 0, stream()>>>(a_dev, b, out_dev, g);
+        break;
+    case WEED_HIP_EW_RELU:
+        elementwise_kernel<6><<<blocks, 256, 0, stream()>>>(a_dev, b, out_dev, g);
+        break;
+    case WEED_HIP_EW_SIGMOID:
+        elementwise_kernel<7><<<blocks, 256, 0, stream()>>>(a_dev, b, out_dev, g);
+        break;
+    case WEED_HIP_EW_TANH:
+        elementwise_kernel<8><<<blocks, 256, 0, stream()>>>(a_dev, b, out_dev, g);
+        break;
+    case WEED_HIP_EW_GELU:
+        elementwise_kernel<9><<<blocks, 256, 0, stream()>>>(a_dev, b, out_dev, g);
+        break;
     case WEED_HIP_EW_COPY:
         elementwise_kernel<0><<<blocks, 256, 0, stream()>>>(a_dev, b, out_dev, g);
         break;
