@@ -861,7 +861,7 @@ TEST_CASE(test_checkpoint_linear_known_bytes, false)
         REQUIRE_THROWS_AS(Module::load(is), std::runtime_error);
     }
     {
-        std::istringstream is(Bytes().u32(7U).b); // LAYERNORM_T in the reference
+        std::istringstream is(Bytes().u32(8U).b); // EMBEDDING_T in the reference: not a module of this path
         REQUIRE_THROWS_AS(Module::load(is), std::domain_error);
     }
     {
@@ -941,6 +941,527 @@ TEST_CASE(test_checkpoint_attention_round_trip, true)
     std::istringstream wrong(std::string(64, 'x'));
     b->reset_cache();
     REQUIRE_THROWS_AS(b->load_quantizer(wrong), std::runtime_error);
+}
+
+// --------------------------------------------------------------------------------------------------------------------
+// norms, activations, SwiGLU and the two modules that call the attention module
+// --------------------------------------------------------------------------------------------------------------------
+
+// float64 versions of the pieces (column-major (rows, n) arrays: element (r, j) at r + rows * j)
+std::vector<double> host_rms_norm(const std::vector<double> &x, size_t rows, tcapint n, const std::vector<real1> &w)
+{
+    std::vector<double> y(x.size());
+    for (size_t r = 0; r < rows; ++r) {
+        double sq = 0.0;
+        for (tcapint j = 0; j < n; ++j) {
+            sq += x[r + rows * j] * x[r + rows * j];
+        }
+        const double root = std::sqrt(sq / n + (double)FP_NORM_EPSILON);
+        for (tcapint j = 0; j < n; ++j) {
+            y[r + rows * j] = x[r + rows * j] / root * (double)w[j];
+        }
+    }
+    return y;
+}
+std::vector<double> host_layer_norm(const std::vector<double> &x, size_t rows, tcapint n, const std::vector<real1> &g,
+    const std::vector<real1> &b, double eps)
+{
+    std::vector<double> y(x.size());
+    for (size_t r = 0; r < rows; ++r) {
+        double mu = 0.0, var = 0.0;
+        for (tcapint j = 0; j < n; ++j) {
+            mu += x[r + rows * j];
+        }
+        mu /= n;
+        for (tcapint j = 0; j < n; ++j) {
+            var += (x[r + rows * j] - mu) * (x[r + rows * j] - mu);
+        }
+        const double root = std::sqrt(var / n + eps);
+        for (tcapint j = 0; j < n; ++j) {
+            y[r + rows * j] = (x[r + rows * j] - mu) / root * (double)g[j] + (double)b[j];
+        }
+    }
+    return y;
+}
+double host_gelu(double v) { return 0.5 * v * (1.0 + std::tanh(0.7978845608028654 * (v + 0.044715 * v * v * v))); }
+std::vector<double> plus(const std::vector<double> &a, const std::vector<double> &b)
+{
+    std::vector<double> y(a.size());
+    for (size_t i = 0; i < a.size(); ++i) {
+        y[i] = a[i] + b[i];
+    }
+    return y;
+}
+void set_param(const ParameterPtr &p, const std::vector<real1> &v, const std::vector<tcapint> &shape)
+{
+    Parameter fresh(v, shape, true, TEST_DTAG);
+    p->storage = fresh.storage;
+    p->shape = fresh.shape;
+    p->stride = fresh.stride;
+    p->offset = 0U;
+}
+
+// What MultiHeadAttention::forward returns for the (B, T, dm) input `xin` (float64) when `before` tokens were cached
+// ahead of the call: float64 attention over the rows the device cache holds AFTER the call (as the kernels see them,
+// rotated basis), so the coder's error is not part of the comparison.
+std::vector<double> host_mha(MultiHeadAttention &mha, const HostLinear &wq, const HostLinear &wo, const std::vector<double> &xin,
+    tcapint B, tcapint T, tcapint before)
+{
+    const tcapint H = (tcapint)mha.num_heads, Hkv = (tcapint)mha.num_kv_heads, hd = (tcapint)mha.head_dim;
+    const size_t rows = (size_t)B * T;
+    std::vector<double> Qd = host_linear(wq, xin, rows);
+    if (mha.rope) {
+        Qd = host_rope(Qd, B, T, H, hd, *mha.rope, before);
+    }
+    Qd = host_rotate(Qd, rows * H, hd, mha.k_rotation);
+    const tcapint cap = mha.max_seq_len, n_tok = before + T;
+    std::vector<real1> krows((size_t)B * Hkv * n_tok * hd), vrows(krows.size());
+    for (tcapint p = 0; p < B * Hkv; ++p) {
+        for (tcapint tok = 0; tok < n_tok; ++tok) {
+            mha.k_qcache.read_row(p * cap + tok, &krows[((size_t)p * n_tok + tok) * hd]);
+            mha.v_qcache.read_row(p * cap + tok, &vrows[((size_t)p * n_tok + tok) * hd]);
+        }
+    }
+    AttnCheck g{ B, H, Hkv, hd, mha.gqa_blocked,
+        [&](tcapint b, tcapint kvh, tcapint tok, tcapint j) { return (double)krows[(((size_t)(b * Hkv + kvh)) * n_tok + tok) * hd + j]; },
+        [&](tcapint b, tcapint kvh, tcapint tok, tcapint j) { return (double)vrows[(((size_t)(b * Hkv + kvh)) * n_tok + tok) * hd + j]; } };
+    std::vector<double> att = host_attention(g, Qd, T, before);
+    att = host_rotate(att, rows * H, hd, mha.v_rotation_trans);
+    return host_linear(wo, att, rows);
+}
+
+TEST_CASE(test_activation_modules_reference_cases, true)
+{
+    // test/tests.cpp:230-244 (relu), 284-291 (sigmoid), 314-321 (tanh), forward values
+    auto scalar = [](real1 v) { return std::make_shared<Tensor>(v, false, TEST_DTAG); };
+    REQUIRE(get_real(Tensor::relu(scalar(R(2)))) == R(2));
+    REQUIRE(get_real(Tensor::relu(scalar(R(-2)))) == R(0));
+    REQUIRE(get_real(Tensor::sigmoid(scalar(R(0)))) == R(0.5));
+    REQUIRE(get_real(Tensor::tanh(scalar(R(0)))) == R(0));
+    // test/tests.cpp:111-120 with an axis: mean(1, 2, 3) = 2, and the axis stays with extent 1
+    TensorPtr x = std::make_shared<Tensor>(std::vector<real1>{ R(1), R(4), R(2), R(5), R(3), R(6) }, std::vector<tcapint>{ 2, 3 },
+        false, TEST_DTAG);
+    TensorPtr m = Tensor::mean(x, 1);
+    REQUIRE(m->shape == (std::vector<tcapint>{ 2U, 1U }));
+    REQUIRE(m->to_vector() == (std::vector<real1>{ R(2), R(5) }));
+    // modules against the CPU checker on a (B, T, features) tensor; relu bit for bit
+    const std::vector<real1> v = gaussian(3U * 5U * 40U, 21U, 2.5f);
+    TensorPtr t = std::make_shared<Tensor>(v, std::vector<tcapint>{ 3U, 5U, 40U }, false, TEST_DTAG);
+    struct Act {
+        std::shared_ptr<Module> m;
+        int op;
+        ModuleType tag;
+    };
+    for (const Act &a : { Act{ std::make_shared<ReLU>(), 0, RELU_T }, Act{ std::make_shared<Sigmoid>(), 1, SIGMOID_T },
+             Act{ std::make_shared<Tanh>(), 2, TANH_T }, Act{ std::make_shared<GeLU>(), 3, GELU_T } }) {
+        std::vector<real1> want(v.size());
+        wo_unary(a.op, v.data(), v.size(), want.data());
+        const std::vector<real1> got = a.m->forward(t)->to_vector();
+        bool ok = got.size() == want.size();
+        for (size_t i = 0; ok && i < got.size(); ++i) {
+            ok = a.op == 0 ? got[i] == want[i] : std::fabs(got[i] - want[i]) <= 3e-7f + 2e-6f * std::fabs(want[i]);
+        }
+        REQUIRE(ok);
+        // their stream is the tag alone (module.cpp:53-56, 87-98)
+        std::ostringstream os;
+        a.m->save(os);
+        REQUIRE(os.str() == Bytes().u32((uint32_t)a.tag).b);
+        std::istringstream is(os.str());
+        std::shared_ptr<Module> r = Module::load(is);
+        REQUIRE(r && r->mtype == a.tag);
+    }
+    REQUIRE_THROWS_AS(Tensor::relu(std::make_shared<Tensor>(v, std::vector<tcapint>{ 3U, 5U, 40U }, false, DeviceTag::CPU)),
+        std::domain_error);
+}
+
+TEST_CASE(test_rms_norm_and_layer_norm_modules, true)
+{
+    // include/modules/rms_norm.hpp:34-38 and src/modules/layernorm.cpp:29-42 on (B, T, features) column-major tensors,
+    // against the CPU checker (rows gathered for it) and float64
+    const tcapint B = 3U, T = 4U, n = 96U;
+    const std::vector<real1> v = gaussian((size_t)B * T * n, 31U, 3.0f);
+    TensorPtr x = std::make_shared<Tensor>(v, std::vector<tcapint>{ B, T, n }, false, TEST_DTAG);
+    const size_t rows = (size_t)B * T;
+    std::vector<real1> dense(v.size()); // [row][n] for the checker
+    for (size_t r = 0; r < rows; ++r) {
+        for (tcapint j = 0; j < n; ++j) {
+            dense[r * n + j] = v[r + rows * j];
+        }
+    }
+    const std::vector<real1> w = gaussian(n, 32U, 0.3f), bt = gaussian(n, 33U);
+    RMSNorm rms(n, -1, TEST_DTAG);
+    REQUIRE(rms.weight->to_vector() == std::vector<real1>(n, ONE_R1)); // FillOnes (rms_norm.hpp:30)
+    REQUIRE(rms.parameters().size() == 1U);
+    set_param(rms.weight, w, { n });
+    std::vector<real1> want(v.size());
+    wo_rms_norm(dense.data(), rows, n, w.data(), wo_norm_epsilon(), want.data());
+    std::vector<real1> got = rms.forward(x)->to_vector();
+    std::vector<double> want64 = host_rms_norm(to_double(v), rows, n, w);
+    bool ok = true, ok64 = true;
+    for (size_t r = 0; r < rows; ++r) {
+        for (tcapint j = 0; j < n; ++j) {
+            ok = ok && std::fabs(got[r + rows * j] - want[r * n + j]) <= 2e-6f + 2e-6f * std::fabs(want[r * n + j]);
+            ok64 = ok64 && std::fabs((double)got[r + rows * j] - want64[r + rows * j]) <= 2e-6 + 2e-6 * std::fabs(want64[r + rows * j]);
+        }
+    }
+    REQUIRE(ok);
+    REQUIRE(ok64);
+    REQUIRE_THROWS_AS(RMSNorm(n + 1U, -1, TEST_DTAG).forward(x), std::invalid_argument);
+
+    LayerNorm ln(n, TEST_DTAG);
+    REQUIRE(ln.eps == FP_NORM_EPSILON && ln.gamma->shape == (std::vector<tcapint>{ 1U, 1U, n }));
+    REQUIRE(ln.gamma->to_vector() == std::vector<real1>(n, ONE_R1) && ln.beta->to_vector() == std::vector<real1>(n, ZERO_R1));
+    set_param(ln.gamma, w, { 1U, 1U, n });
+    set_param(ln.beta, bt, { 1U, 1U, n });
+    wo_layer_norm(dense.data(), rows, n, w.data(), bt.data(), ln.eps, want.data());
+    got = ln.forward(x)->to_vector();
+    want64 = host_layer_norm(to_double(v), rows, n, w, bt, (double)ln.eps);
+    ok = ok64 = true;
+    for (size_t r = 0; r < rows; ++r) {
+        for (tcapint j = 0; j < n; ++j) {
+            ok = ok && std::fabs(got[r + rows * j] - want[r * n + j]) <= 4e-6f + 4e-6f * std::fabs(want[r * n + j]);
+            ok64 = ok64 && std::fabs((double)got[r + rows * j] - want64[r + rows * j]) <= 4e-6 + 4e-6 * std::fabs(want64[r + rows * j]);
+        }
+    }
+    REQUIRE(ok);
+    REQUIRE(ok64);
+}
+
+TEST_CASE(test_checkpoint_norm_and_swiglu_known_bytes, false)
+{
+    // hand-assembled from the reference's writers: rms_norm.hpp:39-44, layernorm.cpp:44-50, swiglu.cpp:18-25
+    RMSNorm rms(3U, -1, DeviceTag::CPU);
+    std::ostringstream os;
+    rms.save(os);
+    Bytes e;
+    e.u32(30U).u32(0xffffffffU).u32(3U);            // RMS_NORM_T, axis -1, hidden_size
+    e.u32(0xffffffffU).u32(0U).u32(1U).u32(3U).u32(1U); // weight: device id -1, offset 0, rank 1, (3, stride 1)
+    e.u32(1U).u32(0xffffffffU).u32(0xffffffffU).u32(3U).f32(1.0f).f32(1.0f).f32(1.0f);
+    REQUIRE(os.str() == e.b);
+    {
+        std::istringstream is(e.b);
+        RMSNormPtr r = std::dynamic_pointer_cast<RMSNorm>(Module::load(is));
+        REQUIRE(r && r->axis == -1 && r->hidden_size == 3U && r->weight->to_vector() == std::vector<real1>(3, 1.0f));
+        REQUIRE(is.peek() == std::char_traits<char>::eof());
+    }
+    LayerNorm ln(2U, DeviceTag::CPU, 0.25f);
+    std::dynamic_pointer_cast<RealStorage>(ln.beta->storage)->write(1U, -3.0f);
+    std::ostringstream ol;
+    ln.save(ol);
+    Bytes l;
+    l.u32(7U).u32(2U).f32(0.25f); // LAYERNORM_T, features, eps
+    for (int which = 0; which < 2; ++which) {
+        l.u32(0xffffffffU).u32(0U).u32(3U).u32(1U).u32(0U).u32(1U).u32(0U).u32(2U).u32(1U); // (1, 1, 2), strides (0, 0, 1)
+        l.u32(1U).u32(0xffffffffU).u32(0xffffffffU).u32(2U);
+        if (which == 0) {
+            l.f32(1.0f).f32(1.0f);
+        } else {
+            l.f32(0.0f).f32(-3.0f);
+        }
+    }
+    REQUIRE(ol.str() == l.b);
+    {
+        std::istringstream is(l.b);
+        LayerNormPtr r = std::dynamic_pointer_cast<LayerNorm>(Module::load(is));
+        REQUIRE(r && r->features == 2U && r->eps == 0.25f && r->beta->to_vector() == (std::vector<real1>{ 0.0f, -3.0f }));
+        REQUIRE(r && r->gamma->shape == (std::vector<tcapint>{ 1U, 1U, 2U }));
+    }
+    // SwiGLU: tag, sizes, then three bias-free Linear records
+    SwiGLU g(2U, 3U, DeviceTag::CPU);
+    REQUIRE(g.parameters().size() == 3U);
+    std::ostringstream og;
+    g.save(og);
+    const std::string head = Bytes().u32(32U).u32(2U).u32(3U).u32(2U).u32(2U).u32(3U).b; // ..., LINEAR_T, in 2, out 3
+    REQUIRE(og.str().compare(0, head.size(), head) == 0);
+    const size_t lin = 4U * 3U + 4U * 7U + 4U * 4U + 4U * 6U + 1U; // tag + sizes, parameter header, storage header, 6 floats, no bias
+    REQUIRE(og.str().size() == 12U + 3U * lin);
+    {
+        std::istringstream is(og.str());
+        SwiGLUPtr r = std::dynamic_pointer_cast<SwiGLU>(Module::load(is));
+        REQUIRE(r && r->hidden_size == 2U && r->intermediate_size == 3U && r->parameters().size() == 3U);
+        REQUIRE(r && r->down_proj->in_features == 3U && r->down_proj->out_features == 2U && !r->down_proj->bias);
+        REQUIRE(r && r->gate_proj->weight->to_vector() == g.gate_proj->weight->to_vector());
+    }
+    // a record whose sub-module has the wrong type is refused
+    {
+        std::string bad = og.str();
+        bad[12] = 31; // the gate projection's tag becomes ROPE_T
+        std::istringstream is(bad);
+        REQUIRE_THROWS_AS(Module::load(is), std::runtime_error);
+    }
+    REQUIRE_THROWS_AS(SwiGLU().forward(nullptr), std::domain_error);
+}
+
+TEST_CASE(test_transformer_encoder_layer_example_sizes, true)
+{
+    // The sizes of the reference's own example (examples/binary_addition_transformer.cpp:91-104: d_model 8, d_ff 16,
+    // one head, 16 sequences of 6 tokens) through TransformerEncoderLayer::forward
+    // (src/modules/transformer_encoder_layer.cpp:63-125), with the stock 4-bit cache, against float64:
+    // x1 = x + attn(norm1(x)); out = x1 + ff2(gelu(ff1(norm2(x1)))).  A prefill and two decode steps.
+    const tcapint B = 16U, dm = 8U, dff = 16U, H = 1U;
+    TransformerEncoderLayer layer(dm, H, dff, TEST_DTAG, GELU_FN);
+    REQUIRE(layer.parameters().size() == 8U + 2U + 2U + 2U + 2U);
+    REQUIRE(layer.activation->mtype == GELU_T && layer.self_attn->head_dim == 8 && layer.self_attn->num_kv_heads == 1);
+    layer.self_attn->rotation_seed = 17U;
+    layer.set_max_kv_seq_len(16U);
+    MultiHeadAttention &mha = *layer.self_attn;
+    const HostLinear wq = install(mha.W_q, 101U), wk = install(mha.W_k, 102U), wv = install(mha.W_v, 103U), wo = install(mha.W_o, 104U);
+    (void)wk;
+    (void)wv;
+    const HostLinear f1 = install(layer.ff1, 105U), f2 = install(layer.ff2, 106U);
+    const std::vector<real1> g1 = gaussian(dm, 107U, 0.2f), b1 = gaussian(dm, 108U, 0.2f), g2 = gaussian(dm, 109U, 0.2f),
+                             b2 = gaussian(dm, 110U, 0.2f);
+    std::vector<real1> gamma1(dm), gamma2(dm);
+    for (tcapint j = 0; j < dm; ++j) {
+        gamma1[j] = 1.0f + g1[j];
+        gamma2[j] = 1.0f + g2[j];
+    }
+    set_param(layer.norm1->gamma, gamma1, { 1U, 1U, dm });
+    set_param(layer.norm1->beta, b1, { 1U, 1U, dm });
+    set_param(layer.norm2->gamma, gamma2, { 1U, 1U, dm });
+    set_param(layer.norm2->beta, b2, { 1U, 1U, dm });
+    tcapint before = 0U;
+    for (const tcapint T : { 6U, 1U, 1U }) {
+        const std::vector<real1> xv = gaussian((size_t)B * T * dm, 200U + before);
+        TensorPtr x = std::make_shared<Tensor>(xv, std::vector<tcapint>{ B, T, dm }, false, TEST_DTAG);
+        const std::vector<real1> got = layer.forward(x)->to_vector();
+        REQUIRE(mha.cache_len == before + T && mha.max_seq_len == 16U);
+        const size_t rows = (size_t)B * T;
+        const std::vector<double> xd = to_double(xv);
+        const std::vector<double> x1 = plus(xd, host_mha(mha, wq, wo, host_layer_norm(xd, rows, dm, gamma1, b1, FP_NORM_EPSILON), B, T, before));
+        std::vector<double> ff = host_linear(f1, host_layer_norm(x1, rows, dm, gamma2, b2, FP_NORM_EPSILON), rows);
+        for (double &v : ff) {
+            v = host_gelu(v);
+        }
+        const std::vector<double> want = plus(x1, host_linear(f2, ff, rows));
+        double worst = 0.0;
+        const bool ok = attn_close(got, want, &worst);
+        if (!ok) {
+            std::printf("    T %u before %u: worst abs err %.3e\n", T, before, worst);
+        }
+        REQUIRE(ok);
+        before += T;
+    }
+    layer.reset_cache();
+    REQUIRE(mha.cache_len == 0U && mha.k_rotation.empty());
+    // the other activations the constructor takes; the one it cannot run is refused
+    REQUIRE(TransformerEncoderLayer(dm, H, dff, TEST_DTAG, RELU_FN).activation->mtype == RELU_T);
+    REQUIRE(TransformerEncoderLayer(dm, H, dff, TEST_DTAG, SIGMOID_FN).activation->mtype == SIGMOID_T);
+    REQUIRE(TransformerEncoderLayer(dm, H, dff, TEST_DTAG, TANH_FN).activation->mtype == TANH_T);
+    REQUIRE_THROWS_AS(TransformerEncoderLayer(dm, H, dff, TEST_DTAG, SWIGLU_FN), std::invalid_argument);
+}
+
+TEST_CASE(test_qwen_decoder_layer_prefill_then_decode, true)
+{
+    // include/modules/qwen_decoder_layer.hpp:104-115: h = x + attn(rms1(x)); out = h + mlp(rms2(h)), grouped query
+    // heads, rotary positions that continue across calls, the Lloyd-Max cache; a prefill, two decode steps and a
+    // chunk against float64 (attention over the rows the device cache holds)
+    const tcapint B = 3U, dm = 256U, H = 4U, Hkv = 2U, dff = 384U, hd = 64U;
+    QwenDecoderLayer layer(dm, H, Hkv, dff, 48U);
+    REQUIRE(layer.self_attn->rope && layer.self_attn->rope->max_seq_len == 48U && layer.self_attn->head_dim == (symint)hd);
+    REQUIRE(layer.parameters().size() == 8U + 3U + 1U + 1U);
+    MultiHeadAttention &mha = *layer.self_attn;
+    mha.kv_coder = KV_LLOYDMAX;
+    mha.k_bits = 3;
+    mha.v_bits = 4;
+    mha.gqa_blocked = true;
+    mha.rotation_seed = 99U;
+    const HostLinear wq = install(mha.W_q, 301U), wk = install(mha.W_k, 302U), wv = install(mha.W_v, 303U), wo = install(mha.W_o, 304U);
+    (void)wk;
+    (void)wv;
+    HostLinear gate = install(layer.mlp->gate_proj, 305U), up = install(layer.mlp->up_proj, 307U), down = install(layer.mlp->down_proj, 309U);
+    for (HostLinear *l : { &gate, &up, &down }) {
+        std::fill(l->b.begin(), l->b.end(), 0.0f); // bias-free projections (swiglu.hpp:35-37)
+    }
+    REQUIRE(!layer.mlp->gate_proj->bias && !layer.mlp->down_proj->bias);
+    std::vector<real1> w1 = gaussian(dm, 311U, 0.2f), w2 = gaussian(dm, 312U, 0.2f);
+    for (tcapint j = 0; j < dm; ++j) {
+        w1[j] += 1.0f;
+        w2[j] += 1.0f;
+    }
+    set_param(layer.input_layernorm->weight, w1, { dm });
+    set_param(layer.post_attention_layernorm->weight, w2, { dm });
+    tcapint before = 0U;
+    for (const tcapint T : { 9U, 1U, 1U, 4U }) {
+        const std::vector<real1> xv = gaussian((size_t)B * T * dm, 400U + before);
+        TensorPtr x = std::make_shared<Tensor>(xv, std::vector<tcapint>{ B, T, dm }, false, TEST_DTAG);
+        const std::vector<real1> got = layer.forward(x)->to_vector();
+        REQUIRE(mha.cache_len == before + T && mha.max_seq_len == 48U);
+        const size_t rows = (size_t)B * T;
+        const std::vector<double> xd = to_double(xv);
+        const std::vector<double> h = plus(xd, host_mha(mha, wq, wo, host_rms_norm(xd, rows, dm, w1), B, T, before));
+        const std::vector<double> r2 = host_rms_norm(h, rows, dm, w2);
+        const std::vector<double> gd = host_linear(gate, r2, rows), ud = host_linear(up, r2, rows);
+        std::vector<double> act(gd.size());
+        for (size_t i = 0; i < gd.size(); ++i) {
+            act[i] = gd[i] / (1.0 + std::exp(-gd[i])) * ud[i];
+        }
+        const std::vector<double> want = plus(h, host_linear(down, act, rows));
+        double worst = 0.0;
+        const bool ok = attn_close(got, want, &worst);
+        if (!ok) {
+            std::printf("    T %u before %u: worst abs err %.3e\n", T, before, worst);
+        }
+        REQUIRE(ok);
+        before += T;
+    }
+    // lifecycle calls reach the attention module (qwen_decoder_layer.hpp:98-102)
+    layer.reset_cache();
+    REQUIRE(mha.cache_len == 0U && mha.max_seq_len == 0U);
+    layer.set_max_kv_seq_len(20U);
+    REQUIRE(mha.max_seq_len == 20U);
+}
+
+TEST_CASE(test_checkpoint_layers_round_trip, true)
+{
+    // save -> load of both layer modules (transformer_encoder_layer.cpp:126-138, qwen_decoder_layer.cpp:18-27,
+    // module.cpp:231-304) and bit-identical replay of a prefill and a decode step; the fixed-size head of each record
+    // against hand-assembled bytes
+    const tcapint B = 2U;
+    {
+        TransformerEncoderLayer a(32U, 2U, 48U, TEST_DTAG, TANH_FN);
+        a.self_attn->rotation_seed = 5U;
+        a.set_max_kv_seq_len(16U);
+        const std::vector<real1> x0 = gaussian((size_t)B * 5U * 32U, 1U), x1 = gaussian((size_t)B * 32U, 2U);
+        TensorPtr t0 = std::make_shared<Tensor>(x0, std::vector<tcapint>{ B, 5U, 32U }, false, TEST_DTAG);
+        TensorPtr t1 = std::make_shared<Tensor>(x1, std::vector<tcapint>{ B, 1U, 32U }, false, TEST_DTAG);
+        const std::vector<real1> y0 = a.forward(t0)->to_vector(), y1 = a.forward(t1)->to_vector();
+        std::stringstream ss;
+        a.save(ss);
+        a.self_attn->save_quantizer(ss);
+        const std::string head = Bytes().u32(18U).u32(32U).u32(48U).u32(2U).u32(17U).b; // tag, d_model, d_ff, heads, attention tag
+        REQUIRE(ss.str().compare(0, head.size(), head) == 0);
+        TransformerEncoderLayerPtr b = std::dynamic_pointer_cast<TransformerEncoderLayer>(Module::load(ss));
+        REQUIRE((bool)b);
+        if (b) {
+            b->self_attn->load_quantizer(ss);
+            REQUIRE(ss.peek() == std::char_traits<char>::eof());
+            REQUIRE(b->d_model == 32U && b->d_ff == 48U && b->num_heads == 2U && b->activation->mtype == TANH_T);
+            REQUIRE(b->parameters().size() == a.parameters().size());
+            REQUIRE(b->forward(t0)->to_vector() == y0);
+            REQUIRE(b->forward(t1)->to_vector() == y1);
+        }
+    }
+    {
+        QwenDecoderLayer a(64U, 2U, 1U, 96U, 24U);
+        a.self_attn->kv_coder = KV_LLOYDMAX;
+        a.self_attn->k_bits = 2;
+        a.self_attn->k_sign = true;
+        a.self_attn->v_bits = 3;
+        a.self_attn->rotation_seed = 6U;
+        const std::vector<real1> x0 = gaussian((size_t)B * 7U * 64U, 3U), x1 = gaussian((size_t)B * 64U, 4U);
+        TensorPtr t0 = std::make_shared<Tensor>(x0, std::vector<tcapint>{ B, 7U, 64U }, false, TEST_DTAG);
+        TensorPtr t1 = std::make_shared<Tensor>(x1, std::vector<tcapint>{ B, 1U, 64U }, false, TEST_DTAG);
+        const std::vector<real1> y0 = a.forward(t0)->to_vector(), y1 = a.forward(t1)->to_vector();
+        std::stringstream ss;
+        a.save(ss);
+        a.self_attn->save_quantizer(ss);
+        const std::string head = Bytes().u32(33U).u32(64U).u32(2U).u32(1U).u32(17U).b; // tag, d_model, heads, kv heads, attention tag
+        REQUIRE(ss.str().compare(0, head.size(), head) == 0);
+        QwenDecoderLayerPtr b = std::dynamic_pointer_cast<QwenDecoderLayer>(Module::load(ss));
+        REQUIRE((bool)b);
+        if (b) {
+            b->self_attn->load_quantizer(ss);
+            REQUIRE(ss.peek() == std::char_traits<char>::eof());
+            REQUIRE(b->d_model == 64U && b->num_heads == 2U && b->num_kv_heads == 1U && b->self_attn->rope &&
+                b->self_attn->rope->max_seq_len == 24U && b->mlp->intermediate_size == 96U);
+            REQUIRE(b->input_layernorm->hidden_size == 64U && b->post_attention_layernorm->axis == -1);
+            REQUIRE(b->parameters().size() == a.parameters().size());
+            REQUIRE(b->forward(t0)->to_vector() == y0);
+            REQUIRE(b->forward(t1)->to_vector() == y1);
+        }
+    }
+}
+
+TEST_CASE(test_replaced_tables_travel_in_the_quantizer_record, true)
+{
+    // MultiHeadAttention::set_tables forwards to weed_hip_kv_cache_set_tables; the tables are part of the quantizer
+    // record, so a reloaded module codes the same tokens into the same cache rows
+    const tcapint B = 2U, dm = 64U, H = 2U, Hkv = 2U, hd = 32U, T = 6U;
+    auto make = [&]() {
+        MultiHeadAttentionPtr m = std::make_shared<MultiHeadAttention>(dm, H, Hkv, hd, TEST_DTAG, nullptr, ZERO_R1, -1, true, 4);
+        m->kv_coder = KV_LLOYDMAX;
+        m->k_bits = 2;
+        m->k_sign = true;
+        m->v_bits = 3;
+        m->rotation_seed = 77U;
+        m->set_max_kv_seq_len(16U);
+        return m;
+    };
+    // the caller's own tables: uniform grids instead of the Lloyd-Max levels (values exactly representable in binary16)
+    const std::vector<real1> kb{ -1.0f, 0.0f, 1.0f }, kl{ -1.5f, -0.5f, 0.5f, 1.5f },
+        kr{ -1.75f, -1.25f, -0.75f, -0.25f, 0.25f, 0.75f, 1.25f, 1.75f };
+    std::vector<real1> vb, vl;
+    for (int i = 0; i < 8; ++i) {
+        vl.push_back(-1.75f + 0.5f * (real1)i);
+        if (i) {
+            vb.push_back(-2.0f + 0.5f * (real1)i);
+        }
+    }
+    MultiHeadAttentionPtr a = make(), stock = make();
+    REQUIRE_THROWS_AS(a->set_tables(0, kb, kl, kl), std::invalid_argument); // 2 bits + sign needs 8 reconstruction values
+    REQUIRE_THROWS_AS(a->set_tables(2, kb, kl, kr), std::invalid_argument);
+    a->set_tables(0, kb, kl, kr);
+    a->set_tables(1, vb, vl, vl);
+    for (const MultiHeadAttentionPtr &m : { a, stock }) {
+        install(m->W_q, 1U);
+        install(m->W_k, 2U);
+        install(m->W_v, 3U);
+        install(m->W_o, 4U);
+    }
+    const std::vector<real1> xv = gaussian((size_t)B * T * dm, 9U);
+    TensorPtr x = std::make_shared<Tensor>(xv, std::vector<tcapint>{ B, T, dm }, false, TEST_DTAG);
+    const std::vector<real1> ya = a->forward(x)->to_vector(), ys = stock->forward(x)->to_vector();
+    REQUIRE(ya != ys);
+    REQUIRE_THROWS_AS(a->set_tables(0, kb, kl, kr), std::logic_error); // tokens are cached
+    auto rows_of = [&](MultiHeadAttention &m) {
+        std::vector<real1> r((size_t)2U * B * Hkv * T * hd);
+        size_t at = 0;
+        for (QuantizedKVCache *qc : { &m.k_qcache, &m.v_qcache }) {
+            for (tcapint p = 0; p < B * Hkv; ++p) {
+                for (tcapint tok = 0; tok < T; ++tok, at += hd) {
+                    qc->read_row(p * m.max_seq_len + tok, &r[at]);
+                }
+            }
+        }
+        return r;
+    };
+    const std::vector<real1> rows_a = rows_of(*a);
+    // every dequantised coordinate is row scale times one of the caller's values: ratios of a row are ratios of table entries
+    REQUIRE(rows_a != rows_of(*stock));
+    std::stringstream ss;
+    a->save(ss);
+    a->save_quantizer(ss);
+    MultiHeadAttentionPtr b = std::dynamic_pointer_cast<MultiHeadAttention>(Module::load(ss));
+    REQUIRE((bool)b);
+    if (!b) {
+        return;
+    }
+    b->load_quantizer(ss);
+    REQUIRE(ss.peek() == std::char_traits<char>::eof());
+    REQUIRE(b->custom_tables[0].bounds == kb && b->custom_tables[0].recon == kr && b->custom_tables[1].levels == vl);
+    REQUIRE(b->forward(x)->to_vector() == ya);
+    REQUIRE(rows_of(*b) == rows_a);
+    // the tables survive reset_cache(), as the weights do
+    b->reset_cache();
+    b->rotation_seed = 77U;
+    b->set_max_kv_seq_len(16U);
+    REQUIRE(b->forward(x)->to_vector() == ya);
+    // a version-1 record (no tables) still loads: built-in tables
+    std::stringstream s1;
+    stock->save_quantizer(s1);
+    std::string v1 = s1.str();
+    REQUIRE(v1.size() > 24U && v1[3] == '2');
+    v1[3] = '1';
+    v1.resize(v1.size() - 24U); // six empty lists
+    std::istringstream is1(v1);
+    MultiHeadAttentionPtr c = make();
+    c->load_quantizer(is1);
+    REQUIRE(is1.peek() == std::char_traits<char>::eof());
+    REQUIRE(c->custom_tables[0].bounds.empty() && c->k_rotation == stock->k_rotation);
+    // the uniform coder has no tables
+    MultiHeadAttention u(dm, H, Hkv, hd, TEST_DTAG, nullptr, ZERO_R1, -1, true, 4);
+    REQUIRE_THROWS_AS(u.set_tables(0, kb, kl, kr), std::invalid_argument);
 }
 
 } // namespace

@@ -34,7 +34,9 @@ def test_host_library_loads_and_exports_the_mirror():
                  "Weed::MultiHeadAttention::forward(", "Weed::MultiHeadAttention::reset_cache()",
                  "Weed::QuantizedKVCache::write_row(unsigned int, float const*)",
                  "Weed::QuantizedKVCache::read_row(unsigned int, float*) const",
-                 "Weed::Linear::forward("):
+                 "Weed::Linear::forward(", "Weed::RMSNorm::forward(", "Weed::LayerNorm::forward(", "Weed::SwiGLU::forward(",
+                 "Weed::QwenDecoderLayer::forward(", "Weed::TransformerEncoderLayer::forward(",
+                 "Weed::MultiHeadAttention::set_tables("):
         assert name in out, name
     assert lib is not None
 
@@ -47,4 +49,4 @@ def test_host_logic_without_a_device():
 @pytest.mark.gpu
 def test_host_mirror_on_device():
     out = _run([])
-    assert "0 failed" in out and "test_attention_lloydmax" in out
+    assert "0 failed" in out and "test_attention_lloydmax" in out and "test_qwen_decoder_layer_prefill_then_decode" in out

@@ -1,14 +1,25 @@
-// Checkpoint streams of the attention path: Storage, Parameter, Linear, RoPE, MultiHeadAttention.
+// Checkpoint streams of the attention path: Storage, Parameter, Linear, RoPE, MultiHeadAttention, the norms and
+// activations, SwiGLU, TransformerEncoderLayer, QwenDecoderLayer.
 //
 // The byte layout is the reference's at its default build widths (include/common/serializer.hpp,
 // src/storage/storage.cpp:25-119, src/tensors/parameter.cpp:16-56, src/modules/module.cpp:53-260,
-// src/modules/linear.cpp:109-118, src/modules/rope.cpp:100-106, src/modules/multihead_attention.cpp:358-375):
+// src/modules/linear.cpp:109-118, src/modules/rope.cpp:100-106, src/modules/multihead_attention.cpp:358-375,
+// include/modules/rms_norm.hpp:39-44, src/modules/layernorm.cpp:44-50, src/modules/swiglu.cpp:18-25,
+// src/modules/transformer_encoder_layer.cpp:126-138, src/modules/qwen_decoder_layer.cpp:18-27):
 //
 //   Module      u32 module type
 //   Linear      Module, u32 in_features, u32 out_features, Parameter weight, u8 has_bias, [Parameter bias]
 //   RoPE        Module, u32 head_dim, u32 max_seq_len, f32 base
 //   Attention   Module, f32 mask_val, i32 d_model, i32 num_heads, i32 num_kv_heads, i32 head_dim, u8 use_kv_cache,
 //               i32 kv_quant_bits, Linear W_q, W_k, W_v, W_o, u8 has_rope, [RoPE]
+//   ReLU, Sigmoid, Tanh, GeLU   Module (the tag alone)
+//   RMSNorm     Module, i32 axis, u32 hidden_size, Parameter weight
+//   LayerNorm   Module, u32 features, f32 eps, Parameter gamma, Parameter beta
+//   SwiGLU      Module, u32 hidden_size, u32 intermediate_size, Linear gate_proj, up_proj, down_proj
+//   Encoder layer   Module, u32 d_model, u32 d_ff, u32 num_heads, Attention, Linear ff1, ff2, LayerNorm norm1, norm2,
+//               activation module
+//   Qwen layer  Module, u32 d_model, u32 num_heads, u32 num_kv_heads, Attention, SwiGLU, RMSNorm input_layernorm,
+//               RMSNorm post_attention_layernorm
 //   Parameter   i32 device id, u32 offset, u32 rank, rank x (u32 shape, u32 stride), Storage
 //   Storage     u32 storage type, 8 bytes device id (low four defined), u32 size, size x f32
 //
@@ -231,15 +242,70 @@ void MultiHeadAttention::save(std::ostream &os) const
     }
 }
 
-namespace {
-LinearPtr load_linear(std::istream &is)
+void RMSNorm::save(std::ostream &os) const
 {
-    LinearPtr l = std::dynamic_pointer_cast<Linear>(Module::load(is));
-    if (!l) {
-        throw std::runtime_error("MultiHeadAttention record: a projection is not a Linear module");
-    }
-    return l;
+    Module::save(os);
+    Serializer::write_symint(os, axis);
+    Serializer::write_tcapint(os, hidden_size);
+    weight->save(os);
 }
+
+void LayerNorm::save(std::ostream &os) const
+{
+    Module::save(os);
+    Serializer::write_tcapint(os, features);
+    Serializer::write_real(os, eps);
+    gamma->save(os);
+    beta->save(os);
+}
+
+void SwiGLU::save(std::ostream &os) const
+{
+    Module::save(os);
+    Serializer::write_tcapint(os, hidden_size);
+    Serializer::write_tcapint(os, intermediate_size);
+    gate_proj->save(os);
+    up_proj->save(os);
+    down_proj->save(os);
+}
+
+void TransformerEncoderLayer::save(std::ostream &os) const
+{
+    Module::save(os);
+    Serializer::write_tcapint(os, d_model);
+    Serializer::write_tcapint(os, d_ff);
+    Serializer::write_tcapint(os, num_heads);
+    self_attn->save(os);
+    ff1->save(os);
+    ff2->save(os);
+    norm1->save(os);
+    norm2->save(os);
+    activation->save(os);
+}
+
+void QwenDecoderLayer::save(std::ostream &os) const
+{
+    Module::save(os);
+    Serializer::write_tcapint(os, d_model);
+    Serializer::write_tcapint(os, num_heads);
+    Serializer::write_tcapint(os, num_kv_heads);
+    self_attn->save(os);
+    mlp->save(os);
+    input_layernorm->save(os);
+    post_attention_layernorm->save(os);
+}
+
+namespace {
+// the sub-module a record names next, which must be of type T
+template <typename T> std::shared_ptr<T> load_as(std::istream &is, const char *what)
+{
+    std::shared_ptr<T> m = std::dynamic_pointer_cast<T>(Module::load(is));
+    if (!m) {
+        throw std::runtime_error(std::string("module record: ") + what + " is not of the expected module type");
+    }
+    return m;
+}
+LinearPtr load_linear(std::istream &is) { return load_as<Linear>(is, "a projection"); }
 } // namespace
 
 std::shared_ptr<Module> Module::load(std::istream &is)
@@ -296,6 +362,65 @@ std::shared_ptr<Module> Module::load(std::istream &is)
         }
         return m;
     }
+    case RELU_T:
+        return std::make_shared<ReLU>();
+    case SIGMOID_T:
+        return std::make_shared<Sigmoid>();
+    case TANH_T:
+        return std::make_shared<Tanh>();
+    case GELU_T:
+        return std::make_shared<GeLU>();
+    case RMS_NORM_T: {
+        RMSNormPtr r = std::make_shared<RMSNorm>();
+        Serializer::read_symint(is, r->axis);
+        Serializer::read_tcapint(is, r->hidden_size);
+        r->weight = Parameter::load(is);
+        return r;
+    }
+    case LAYERNORM_T: {
+        LayerNormPtr l = std::make_shared<LayerNorm>();
+        Serializer::read_tcapint(is, l->features);
+        Serializer::read_real(is, l->eps);
+        l->gamma = Parameter::load(is);
+        l->beta = Parameter::load(is);
+        return l;
+    }
+    case SWIGLU_T: {
+        SwiGLUPtr g = std::make_shared<SwiGLU>();
+        Serializer::read_tcapint(is, g->hidden_size);
+        Serializer::read_tcapint(is, g->intermediate_size);
+        g->gate_proj = load_linear(is);
+        g->up_proj = load_linear(is);
+        g->down_proj = load_linear(is);
+        g->_register_params();
+        return g;
+    }
+    case TRANSFORMER_ENCODER_LAYER_T: {
+        TransformerEncoderLayerPtr t = std::make_shared<TransformerEncoderLayer>();
+        Serializer::read_tcapint(is, t->d_model);
+        Serializer::read_tcapint(is, t->d_ff);
+        Serializer::read_tcapint(is, t->num_heads);
+        t->self_attn = load_as<MultiHeadAttention>(is, "the attention of an encoder layer");
+        t->ff1 = load_linear(is);
+        t->ff2 = load_linear(is);
+        t->norm1 = load_as<LayerNorm>(is, "norm1 of an encoder layer");
+        t->norm2 = load_as<LayerNorm>(is, "norm2 of an encoder layer");
+        t->activation = Module::load(is);
+        t->_register_params();
+        return t;
+    }
+    case QWEN_DECODER_LAYER_T: {
+        QwenDecoderLayerPtr q = std::make_shared<QwenDecoderLayer>();
+        Serializer::read_tcapint(is, q->d_model);
+        Serializer::read_tcapint(is, q->num_heads);
+        Serializer::read_tcapint(is, q->num_kv_heads);
+        q->self_attn = load_as<MultiHeadAttention>(is, "the attention of a decoder layer");
+        q->mlp = load_as<SwiGLU>(is, "the feed-forward block of a decoder layer");
+        q->input_layernorm = load_as<RMSNorm>(is, "input_layernorm");
+        q->post_attention_layernorm = load_as<RMSNorm>(is, "post_attention_layernorm");
+        q->_register_params();
+        return q;
+    }
     default:
         throw std::domain_error("Module::load: module type " + std::to_string(tag) + " is not part of this build");
     }
@@ -303,7 +428,27 @@ std::shared_ptr<Module> Module::load(std::istream &is)
 
 // ---- the quantizer record (extension) ----
 namespace {
-constexpr uint32_t kQuantizerMagic = 0x31515a57U; // "WZQ1"
+constexpr uint32_t kQuantizerMagicV1 = 0x31515a57U; // "WZQ1": no tables
+constexpr uint32_t kQuantizerMagic = 0x32515a57U;   // "WZQ2": the record below
+void put_floats(std::ostream &os, const std::vector<real1> &v)
+{
+    Serializer::write_tcapint(os, (tcapint)v.size());
+    for (const real1 &x : v) {
+        Serializer::write_real(os, x);
+    }
+}
+void get_floats(std::istream &is, std::vector<real1> &v, size_t most)
+{
+    tcapint n;
+    Serializer::read_tcapint(is, n);
+    if (n > most) {
+        throw std::runtime_error("MultiHeadAttention::load_quantizer: implausible table size");
+    }
+    v.resize(n);
+    for (real1 &x : v) {
+        Serializer::read_real(is, x);
+    }
+}
 }
 
 void MultiHeadAttention::save_quantizer(std::ostream &os) const
@@ -320,10 +465,14 @@ void MultiHeadAttention::save_quantizer(std::ostream &os) const
     Serializer::write_real(os, k_qcache.block_scale);
     Serializer::write_real(os, v_qcache.block_scale);
     for (const std::vector<real1> *r : { &k_rotation, &v_rotation }) {
-        Serializer::write_tcapint(os, (tcapint)r->size());
-        for (const real1 &x : *r) {
-            Serializer::write_real(os, x);
-        }
+        put_floats(os, *r);
+    }
+    // the Lloyd-Max tables that set_tables() installed, K side then V side: thresholds, levels, reconstruction
+    // values; three empty lists stand for the built-in tables
+    for (const CoderTables &t : custom_tables) {
+        put_floats(os, t.bounds);
+        put_floats(os, t.levels);
+        put_floats(os, t.recon);
     }
 }
 
@@ -331,11 +480,15 @@ void MultiHeadAttention::load_quantizer(std::istream &is)
 {
     uint32_t magic;
     get(is, magic);
-    if (magic != kQuantizerMagic) {
+    if (magic != kQuantizerMagic && magic != kQuantizerMagicV1) {
         throw std::runtime_error("MultiHeadAttention::load_quantizer: not a quantizer record");
     }
     if (cache_len) {
         throw std::logic_error("MultiHeadAttention::load_quantizer: the cache already holds tokens; reset_cache() first");
+    }
+    if (k_qcache.dev) {
+        // a live (still empty) device cache was made with the old settings: the next forward() makes a new one
+        reset_cache();
     }
     symint coder, kb, vb;
     Serializer::read_symint(is, coder);
@@ -364,6 +517,20 @@ void MultiHeadAttention::load_quantizer(std::istream &is)
         r->resize(n);
         for (real1 &x : *r) {
             Serializer::read_real(is, x);
+        }
+    }
+    for (CoderTables &t : custom_tables) {
+        t = CoderTables{};
+    }
+    if (magic == kQuantizerMagic) {
+        for (int which = 0; which < 2; ++which) {
+            CoderTables t;
+            get_floats(is, t.bounds, 255U);
+            get_floats(is, t.levels, 256U);
+            get_floats(is, t.recon, 512U);
+            if (!t.bounds.empty() || !t.levels.empty() || !t.recon.empty()) {
+                set_tables(which, t.bounds, t.levels, t.recon); // checks the sizes against the code widths just read
+            }
         }
     }
 }

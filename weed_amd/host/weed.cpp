@@ -684,6 +684,45 @@ TensorPtr Tensor::sub(TensorPtr a, TensorPtr b) { return binary(WEED_HIP_EW_SUB,
 TensorPtr Tensor::mul(TensorPtr a, TensorPtr b) { return binary(WEED_HIP_EW_MUL, a, b, "Tensor::mul"); }
 TensorPtr Tensor::div(TensorPtr a, TensorPtr b) { return binary(WEED_HIP_EW_DIV, a, b, "Tensor::div"); }
 
+TensorPtr Tensor::mean(TensorPtr a, symint axis)
+{
+    axis = wrap_axis(axis, a->shape.size(), "Tensor::mean");
+    TensorPtr tmp = sum(a, axis) / (real1)(a->shape[(size_t)axis]);
+    // the axis comes back with extent 1 (tensor.cpp:689-691)
+    std::vector<symint> shp(a->shape.begin(), a->shape.end());
+    shp[(size_t)axis] = 1;
+    return reshape(tmp, shp);
+}
+
+namespace {
+TensorPtr unary(void (*op)(const Tensor &, Tensor &), const TensorPtr &a)
+{
+    TensorPtr out = allocate(a->shape, *a);
+    op(*a, *out);
+    return out;
+}
+void unary_op(int op, const Tensor &a, Tensor &out, const char *who)
+{
+    validate_all_same_device({ &a, &out }, who);
+    if (a.get_size() != out.get_size()) {
+        throw std::invalid_argument(std::string("In Weed::") + who + "(a, out), out size does not match input size!");
+    }
+    elementwise(op, a, nullptr, out, who);
+}
+} // namespace
+
+TensorPtr Tensor::relu(TensorPtr a) { return unary(Weed::relu, a); }
+TensorPtr Tensor::sigmoid(TensorPtr a) { return unary(Weed::sigmoid, a); }
+TensorPtr Tensor::tanh(TensorPtr a) { return unary(Weed::tanh, a); }
+TensorPtr Tensor::gelu(const TensorPtr x)
+{
+    // the reference's chain x3 = x * x * x; inner = k2 * (x + k1 * x3); k0 * x * (1 + tanh(inner))
+    // (tensor.cpp:841-851) as one kernel that rounds after every operation as the chain does
+    TensorPtr out = allocate(x->shape, *x);
+    unary_op(WEED_HIP_EW_GELU, *x, *out, "gelu");
+    return out;
+}
+
 TensorPtr Tensor::matmul(TensorPtr a, TensorPtr b)
 {
     if (a->shape.size() < 2U) {
@@ -879,6 +918,10 @@ void add_in_place(Tensor &a, const Tensor &b)
     validate_all_same_device({ &a, &b }, "InPlaceKernel::in_place");
     elementwise(WEED_HIP_EW_ADD, a, &b, a, "add_in_place");
 }
+
+void relu(const Tensor &a, Tensor &out) { unary_op(WEED_HIP_EW_RELU, a, out, "relu"); }
+void sigmoid(const Tensor &a, Tensor &out) { unary_op(WEED_HIP_EW_SIGMOID, a, out, "sigmoid"); }
+void tanh(const Tensor &a, Tensor &out) { unary_op(WEED_HIP_EW_TANH, a, out, "tanh"); }
 
 void triu_fill(Tensor &a, const real1 &val, const tcapint diagonal)
 {
@@ -1212,6 +1255,33 @@ void MultiHeadAttention::reset_cache()
     v_qcache = QuantizedKVCache{};
 }
 
+void MultiHeadAttention::set_tables(int which, const std::vector<real1> &bounds, const std::vector<real1> &levels,
+    const std::vector<real1> &recon)
+{
+    if (which != 0 && which != 1) {
+        throw std::invalid_argument("MultiHeadAttention::set_tables(): which must be 0 (keys) or 1 (values)");
+    }
+    if (kv_coder != KV_LLOYDMAX) {
+        throw std::invalid_argument("MultiHeadAttention::set_tables(): the uniform coder has no tables");
+    }
+    const int bits = which ? (v_bits ? v_bits : kv_quant_bits) : (k_bits ? k_bits : kv_quant_bits);
+    const bool sign = which ? v_sign : k_sign;
+    if (bits < 1 || bits > 4 || bounds.size() != (size_t)(1 << bits) - 1U || levels.size() != (size_t)1 << bits
+        || recon.size() != (size_t)1 << (bits + (sign ? 1 : 0))) {
+        throw std::invalid_argument("MultiHeadAttention::set_tables(): table sizes do not match the code width");
+    }
+    if (cache_len) {
+        throw std::logic_error("MultiHeadAttention::set_tables(): the cache already holds tokens; reset_cache() first");
+    }
+    custom_tables[which] = CoderTables{ bounds, levels, recon };
+    if (k_qcache.dev) {
+        WEED_DEVICE_LOCK();
+        std::vector<real1> rounded(recon.size());
+        HipDevice::check(weed_hip_kv_cache_set_tables(k_qcache.dev->handle, which, bounds.data(), levels.data(), recon.data(),
+            rounded.data()));
+    }
+}
+
 TensorPtr MultiHeadAttention::forward(const TensorPtr x)
 {
     // x: (B, T, d_model)
@@ -1289,6 +1359,14 @@ TensorPtr MultiHeadAttention::forward_quantized(TensorPtr Q, TensorPtr K, Tensor
             }
         }
         HipDevice::check(weed_hip_kv_cache_set_rotations(dev->handle, k_rot_dev->buffer, v_rot_dev->buffer));
+        for (int which = 0; which < 2; ++which) {
+            const CoderTables &t = custom_tables[which];
+            if (!t.bounds.empty()) {
+                std::vector<real1> rounded(t.recon.size());
+                HipDevice::check(weed_hip_kv_cache_set_tables(dev->handle, which, t.bounds.data(), t.levels.data(),
+                    t.recon.data(), rounded.data()));
+            }
+        }
         for (QuantizedKVCache *qc : { &k_qcache, &v_qcache }) {
             qc->dev = dev;
             qc->which = (qc == &v_qcache) ? 1 : 0;
@@ -1554,6 +1632,177 @@ TensorPtr MultiHeadAttention::attend_dense(TensorPtr Q, TensorPtr K, TensorPtr V
     }
     TensorPtr weights = Tensor::softmax(scores, -1);
     return weights >> V;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// norms, SwiGLU and the two modules that call the attention module
+// ---------------------------------------------------------------------------------------------------------
+
+RMSNorm::RMSNorm(const tcapint &hidden_size_, const symint &axis_, DeviceTag dtag)
+    : Module(RMS_NORM_T)
+    , axis(axis_)
+    , hidden_size(hidden_size_)
+{
+    weight = std::make_shared<Parameter>(std::vector<real1>(hidden_size_, ONE_R1), std::vector<tcapint>{ hidden_size_ }, false, dtag);
+}
+
+TensorPtr RMSNorm::forward(const TensorPtr x)
+{
+    const symint ax = wrap_axis(axis, x->shape.size(), "RMSNorm::forward");
+    if (x->shape[(size_t)ax] != hidden_size || weight->get_size() != hidden_size) {
+        throw std::invalid_argument("Tensor shape mismatch in mul!"); // what the reference's `* weight` reports
+    }
+    validate_all_same_device({ x.get(), weight.get() }, "RMSNorm::forward");
+    TensorPtr out = allocate(x->shape, *x);
+    real1 *xp = device_ptr(*x, "RMSNorm::forward"), *wp = device_ptr(*weight, "RMSNorm::forward");
+    real1 *op = device_ptr(*out, "RMSNorm::forward");
+    WEED_DEVICE_LOCK();
+    HipDevice::check(weed_hip_rms_norm_f32((uint32_t)x->shape.size(), x->shape.data(), (uint32_t)ax, xp, x->offset,
+        x->stride.data(), wp, weight->offset, weight->stride.back(), FP_NORM_EPSILON, op, out->offset, out->stride.data()));
+    return out;
+}
+
+LayerNorm::LayerNorm(const tcapint &f, const DeviceTag &dtag, const real1 &e, const int64_t &did)
+    : Module(LAYERNORM_T)
+    , features(f)
+    , eps(e)
+{
+    gamma = std::make_shared<Parameter>(std::vector<real1>(f, ONE_R1), std::vector<tcapint>{ 1U, 1U, f }, true, dtag, did);
+    beta = std::make_shared<Parameter>(std::vector<real1>(f, ZERO_R1), std::vector<tcapint>{ 1U, 1U, f }, true, dtag, did);
+}
+
+TensorPtr LayerNorm::forward(const TensorPtr x)
+{
+    if (x->shape.empty() || x->shape.back() != features || gamma->get_size() != features || beta->get_size() != features) {
+        throw std::invalid_argument("Tensor shape mismatch in mul!");
+    }
+    validate_all_same_device({ x.get(), gamma.get(), beta.get() }, "LayerNorm::forward");
+    TensorPtr out = allocate(x->shape, *x);
+    real1 *xp = device_ptr(*x, "LayerNorm::forward"), *gp = device_ptr(*gamma, "LayerNorm::forward");
+    real1 *bp = device_ptr(*beta, "LayerNorm::forward"), *op = device_ptr(*out, "LayerNorm::forward");
+    WEED_DEVICE_LOCK();
+    HipDevice::check(weed_hip_layer_norm_f32((uint32_t)x->shape.size(), x->shape.data(), (uint32_t)x->shape.size() - 1U, xp,
+        x->offset, x->stride.data(), gp, gamma->offset, gamma->stride.back(), bp, beta->offset, beta->stride.back(), eps, op,
+        out->offset, out->stride.data()));
+    return out;
+}
+
+SwiGLU::SwiGLU(const tcapint &hidden_size_, const tcapint &intermediate_size_, DeviceTag dtag)
+    : Module(SWIGLU_T)
+    , hidden_size(hidden_size_)
+    , intermediate_size(intermediate_size_)
+{
+    gate_proj = std::make_shared<Linear>(hidden_size, intermediate_size, false, true, DType::REAL, dtag);
+    up_proj = std::make_shared<Linear>(hidden_size, intermediate_size, false, true, DType::REAL, dtag);
+    down_proj = std::make_shared<Linear>(intermediate_size, hidden_size, false, true, DType::REAL, dtag);
+    _register_params();
+}
+
+void SwiGLU::_register_params()
+{
+    param_vector.clear();
+    for (const LinearPtr &l : { gate_proj, up_proj, down_proj }) {
+        const std::vector<ParameterPtr> p = l->parameters();
+        param_vector.insert(param_vector.end(), p.begin(), p.end());
+    }
+}
+
+TensorPtr SwiGLU::forward(const TensorPtr x)
+{
+    if (!gate_proj || !up_proj || !down_proj) {
+        throw std::domain_error("SwiGLU::forward(): the module has no projections (default-constructed)");
+    }
+    TensorPtr gate = gate_proj->forward(x);
+    TensorPtr up = up_proj->forward(x);
+    // SiLU(gate) * up
+    TensorPtr activated = allocate(gate->shape, *gate);
+    elementwise(WEED_HIP_EW_SILU_MUL, *gate, up.get(), *activated, "SwiGLU::forward");
+    return down_proj->forward(activated);
+}
+
+TransformerEncoderLayer::TransformerEncoderLayer(const tcapint &d_model_, const tcapint &num_heads_, const tcapint &d_ff_,
+    const DeviceTag &dtag, const ActivationFunctionType &afn, const int64_t &did)
+    : Module(TRANSFORMER_ENCODER_LAYER_T)
+    , d_model(d_model_)
+    , d_ff(d_ff_)
+    , num_heads(num_heads_)
+    , self_attn(std::make_shared<MultiHeadAttention>(d_model_, num_heads_, num_heads_, 0U, dtag, nullptr, ZERO_R1, did))
+    , ff1(std::make_shared<Linear>(d_model_, d_ff_, true, true, DType::REAL, dtag, did))
+    , ff2(std::make_shared<Linear>(d_ff_, d_model_, true, true, DType::REAL, dtag, did))
+    , norm1(std::make_shared<LayerNorm>(d_model_, dtag, FP_NORM_EPSILON, did))
+    , norm2(std::make_shared<LayerNorm>(d_model_, dtag, FP_NORM_EPSILON, did))
+{
+    switch (afn) {
+    case SIGMOID_FN:
+        activation = std::make_shared<Sigmoid>();
+        break;
+    case TANH_FN:
+        activation = std::make_shared<Tanh>();
+        break;
+    case RELU_FN:
+        activation = std::make_shared<ReLU>();
+        break;
+    case SWIGLU_FN:
+        // the reference puts a SwiGLU without projections here (transformer_encoder_layer.cpp:50-52), which cannot run
+        throw std::invalid_argument("TransformerEncoderLayer: SWIGLU_FN has no projections to run between ff1 and ff2");
+    case GELU_FN:
+    default:
+        activation = std::make_shared<GeLU>();
+    }
+    _register_params();
+}
+
+void TransformerEncoderLayer::_register_params()
+{
+    param_vector = self_attn->parameters();
+    for (const std::vector<ParameterPtr> &q : { ff1->parameters(), ff2->parameters(), norm1->parameters(), norm2->parameters() }) {
+        param_vector.insert(param_vector.end(), q.begin(), q.end());
+    }
+}
+
+TensorPtr TransformerEncoderLayer::forward(const TensorPtr x)
+{
+    TensorPtr x1 = self_attn->forward(norm1->forward(x));
+    x1 = x + x1;
+    TensorPtr ff = ff2->forward(activation->forward(ff1->forward(norm2->forward(x1))));
+    return x1 + ff;
+}
+
+QwenDecoderLayer::QwenDecoderLayer(const tcapint &d_model_, const tcapint &num_heads_, const tcapint &num_kv_heads_,
+    const tcapint &d_ff_, const tcapint &max_seq_len, const real1_f &rope_base, const real1_f &, const int64_t &did)
+    : Module(QWEN_DECODER_LAYER_T)
+    , d_model(d_model_)
+    , num_heads(num_heads_)
+    , num_kv_heads(num_kv_heads_)
+{
+    // (the reference takes `eps` and never hands it on: RMSNorm always uses FP_NORM_EPSILON, rms_norm.hpp:35)
+    const tcapint head_dim = d_model_ / num_heads_;
+    RoPEPtr rope = std::make_shared<RoPE>(head_dim, max_seq_len, rope_base);
+    self_attn = std::make_shared<MultiHeadAttention>(d_model_, num_heads_, num_kv_heads_, head_dim, DEFAULT_DEVICE, rope,
+        ZERO_R1, did);
+    mlp = std::make_shared<SwiGLU>(d_model_, d_ff_);
+    input_layernorm = std::make_shared<RMSNorm>(d_model_, -1);
+    post_attention_layernorm = std::make_shared<RMSNorm>(d_model_, -1);
+    _register_params();
+}
+
+void QwenDecoderLayer::_register_params()
+{
+    param_vector.clear();
+    for (const std::vector<ParameterPtr> &q : { self_attn->parameters(), mlp->parameters(), input_layernorm->parameters(),
+             post_attention_layernorm->parameters() }) {
+        param_vector.insert(param_vector.end(), q.begin(), q.end());
+    }
+}
+
+TensorPtr QwenDecoderLayer::forward(const TensorPtr x)
+{
+    // pre-norm + attention + residual
+    TensorPtr h = self_attn->forward(input_layernorm->forward(x));
+    h = h + x;
+    // pre-norm + feed-forward + residual
+    TensorPtr f = mlp->forward(post_attention_layernorm->forward(h));
+    return f + h;
 }
 
 } // namespace Weed

@@ -1,8 +1,9 @@
 // Host-side mirror of the part of Weed's C++ interface that sits on the quantized-KV attention path:
 // Storage / Tensor (real, dense, forward only), the op entry points with their device switch, Linear,
-// QuantizedKVCache and MultiHeadAttention.  Names, argument meaning and exception types follow the reference
-// (include/tensors/tensor.hpp, include/storage/*.hpp, include/ops/*.hpp, include/modules/linear.hpp,
-// include/modules/multihead_attention.hpp); every computation goes to the device library behind
+// QuantizedKVCache and MultiHeadAttention, and the two modules that call it -- TransformerEncoderLayer and
+// QwenDecoderLayer -- with the norms and activations they are made of.  Names, argument meaning and exception types
+// follow the reference (include/tensors/tensor.hpp, include/storage/*.hpp, include/ops/*.hpp, include/modules/*.hpp);
+// every computation goes to the device library behind
 // include/weed_hip.h.  There is no CPU arithmetic here: a CPU-tagged tensor is a host container that can be filled,
 // read and moved to the device, and an op handed one throws std::domain_error.
 #pragma once
@@ -31,14 +32,27 @@ enum DeviceTag { NONE_DEVICE = 0, DEFAULT_DEVICE = 1, CPU = 2, GPU = 3 }; // inc
 enum DType { NONE_DTYPE = 0, REAL = 1, COMPLEX = 2, INT = 3, DEFAULT_DTYPE = REAL }; // include/enums/dtype.hpp
 // include/enums/storage_type.hpp (complex and sparse storages, tags 3, 4, 7, 8, are not part of this build)
 enum StorageType { NONE_STORAGE_TYPE = 0, REAL_CPU_DENSE = 1, REAL_GPU_DENSE = 2, INT_CPU_DENSE = 5, INT_GPU_DENSE = 6 };
-// include/enums/module_type.hpp: the tags a serialized module starts with.  Only the three modules of this path can
-// be written or read here; the other values are listed so that a foreign tag is reported by name of its number.
+// include/enums/module_type.hpp: the tags a serialized module starts with.  Only the modules of this path can be
+// written or read here; any other tag is reported by its number.
 enum ModuleType {
     NONE_MODULE_TYPE = 0,
     LINEAR_T = 2,
+    RELU_T = 3,
+    SIGMOID_T = 4,
+    TANH_T = 5,
+    LAYERNORM_T = 7,
     MULTIHEAD_ATTENTION_T = 17,
+    TRANSFORMER_ENCODER_LAYER_T = 18,
+    GELU_T = 19,
+    RMS_NORM_T = 30,
     ROPE_T = 31,
+    SWIGLU_T = 32,
+    QWEN_DECODER_LAYER_T = 33,
 };
+// include/enums/activation_function_type.hpp
+enum ActivationFunctionType { NONE_FN = 0, SIGMOID_FN = 1, TANH_FN = 2, RELU_FN = 3, GELU_FN = 4, SWIGLU_FN = 5 };
+// include/common/weed_types.hpp:213-214 at fp32: the epsilon both norms default to
+constexpr real1 FP_NORM_EPSILON = 1.1920928955078125e-07f / 4.0f;
 
 // include/common/serializer.hpp: fixed-width little-endian fields, written as the reference's default build writes
 // them (tcapint and symint 32 bits, real1 and real1_f IEEE single, bool one byte, enums 32 bits).
@@ -258,6 +272,13 @@ struct Tensor {
     static TensorPtr mul(TensorPtr a, TensorPtr b);
     static TensorPtr div(TensorPtr a, TensorPtr b);
     static TensorPtr matmul(TensorPtr a, TensorPtr b);
+    // src/tensors/tensor.cpp:682-693: sum along the axis, divided by its length; the axis stays with extent 1
+    static TensorPtr mean(TensorPtr a, symint axis);
+    // src/tensors/tensor.cpp:841-935: one elementwise kernel each (the reference composes gelu from eight ops)
+    static TensorPtr relu(TensorPtr a);
+    static TensorPtr sigmoid(TensorPtr a);
+    static TensorPtr tanh(TensorPtr a);
+    static TensorPtr gelu(const TensorPtr x);
 };
 
 TensorPtr operator+(TensorPtr left, TensorPtr right);
@@ -282,6 +303,9 @@ void sub(const Tensor &a, const Tensor &b, Tensor &out); // src/ops/sub.cpp
 void div(const Tensor &a, const Tensor &b, Tensor &out); // src/ops/div.cpp:17-20
 void add_in_place(Tensor &a, const Tensor &b); // src/ops/in_place.cpp:17-25
 void triu_fill(Tensor &a, const real1 &val, const tcapint diagonal = 1); // src/ops/triu_fill.cpp:42-59
+void relu(const Tensor &a, Tensor &out); // src/ops/real_unary.cpp:485-497
+void sigmoid(const Tensor &a, Tensor &out);
+void tanh(const Tensor &a, Tensor &out);
 
 struct Parameter : public Tensor { // include/tensors/parameter.hpp
     using Tensor::Tensor;
@@ -302,8 +326,7 @@ struct Module {
     virtual ~Module() {}
     // src/modules/module.cpp:53-56: the type tag; the inheriting struct writes the rest.
     virtual void save(std::ostream &os) const;
-    // src/modules/module.cpp:58-260 for LINEAR_T, ROPE_T and MULTIHEAD_ATTENTION_T; any other tag throws
-    // std::domain_error.
+    // src/modules/module.cpp:58-304 for the tags of ModuleType above; any other tag throws std::domain_error.
     static std::shared_ptr<Module> load(std::istream &is);
     virtual TensorPtr forward(const TensorPtr x) = 0;
     virtual std::vector<ParameterPtr> parameters() { return {}; }
@@ -459,8 +482,19 @@ struct MultiHeadAttention : public Module {
     // Extension, a separate record that a caller may write after save(): what the stream above lacks to make a
     // reloaded module encode and decode identically -- coder, bit widths, sign bits, head mapping, rotation seed,
     // max_seq_len, the two block scales and the two rotations (empty before the first forward()).
+    // Since version 2 of the record also the Lloyd-Max tables of either side when set_tables() replaced them.
     void save_quantizer(std::ostream &os) const;
     void load_quantizer(std::istream &is);
+    // Replace the built-in Lloyd-Max tables of the K side (which = 0) or the V side (1): 2^bits - 1 thresholds, 2^bits
+    // levels, 2^(bits + sign) reconstruction values (weed_hip_kv_cache_set_tables).  Takes effect for the tokens coded
+    // afterwards: call it before the first forward(), or after reset_cache().  The tables survive reset_cache() and
+    // travel in the quantizer record.
+    void set_tables(int which, const std::vector<real1> &bounds, const std::vector<real1> &levels,
+        const std::vector<real1> &recon);
+    struct CoderTables {
+        std::vector<real1> bounds, levels, recon;
+    };
+    CoderTables custom_tables[2]; // empty vectors: the built-in tables
 
     std::vector<ParameterPtr> parameters() override { return param_vector; }
     void set_max_kv_seq_len(tcapint m) override { max_seq_len = m; }
@@ -483,5 +517,167 @@ public:
     ~MultiHeadAttention() override;
 };
 typedef std::shared_ptr<MultiHeadAttention> MultiHeadAttentionPtr;
+
+// include/modules/relu.hpp, sigmoid.hpp, tanh.hpp, gelu.hpp: activation functions as modules (their stream is the tag
+// alone).
+struct ReLU : public Module {
+    ReLU()
+        : Module(RELU_T)
+    {
+    }
+    TensorPtr forward(const TensorPtr x) override { return Tensor::relu(x); }
+};
+struct Sigmoid : public Module {
+    Sigmoid()
+        : Module(SIGMOID_T)
+    {
+    }
+    TensorPtr forward(const TensorPtr x) override { return Tensor::sigmoid(x); }
+};
+struct Tanh : public Module {
+    Tanh()
+        : Module(TANH_T)
+    {
+    }
+    TensorPtr forward(const TensorPtr x) override { return Tensor::tanh(x); }
+};
+struct GeLU : public Module {
+    GeLU()
+        : Module(GELU_T)
+    {
+    }
+    TensorPtr forward(const TensorPtr x) override { return Tensor::gelu(x); }
+};
+
+// include/modules/rms_norm.hpp: x / sqrt(mean(x^2, axis) + eps) * weight.  forward() is one kernel
+// (weed_hip_rms_norm_f32) where the reference chains seven elementwise ops and an axis sum.
+struct RMSNorm : public Module {
+    symint axis;
+    tcapint hidden_size;
+    ParameterPtr weight; // (hidden_size), ones
+
+    RMSNorm()
+        : Module(RMS_NORM_T)
+        , axis(-1)
+        , hidden_size(0U)
+    {
+    }
+    RMSNorm(const tcapint &hidden_size_, const symint &axis_ = -1, DeviceTag dtag = DEFAULT_DEVICE);
+    std::vector<ParameterPtr> parameters() override { return { weight }; }
+    TensorPtr forward(const TensorPtr x) override;
+    void save(std::ostream &os) const override; // rms_norm.hpp:39-44
+};
+typedef std::shared_ptr<RMSNorm> RMSNormPtr;
+
+// include/modules/layernorm.hpp, src/modules/layernorm.cpp:29-50: normalisation over the last dimension, then
+// gamma (ones) and beta (zeros), both of shape (1, 1, features).  forward() is one kernel (weed_hip_layer_norm_f32).
+struct LayerNorm : public Module {
+    tcapint features;
+    real1 eps;
+    ParameterPtr gamma;
+    ParameterPtr beta;
+
+    LayerNorm()
+        : Module(LAYERNORM_T)
+        , features(0U)
+        , eps(FP_NORM_EPSILON)
+    {
+    }
+    LayerNorm(const tcapint &f, const DeviceTag &dtag = DeviceTag::DEFAULT_DEVICE, const real1 &e = FP_NORM_EPSILON,
+        const int64_t &did = -1);
+    TensorPtr forward(const TensorPtr x) override;
+    std::vector<ParameterPtr> parameters() override { return { gamma, beta }; }
+    void save(std::ostream &os) const override;
+};
+typedef std::shared_ptr<LayerNorm> LayerNormPtr;
+
+// include/modules/swiglu.hpp: down_proj(gate_proj(x) * sigmoid(gate_proj(x)) * up_proj(x)), three bias-free Linear
+// modules.  The gate is one elementwise kernel (WEED_HIP_EW_SILU_MUL).  Unlike the reference's constructor, this one
+// registers the projections' parameters right away (the reference only does so when a module is loaded).
+struct SwiGLU : public Module {
+    tcapint hidden_size;
+    tcapint intermediate_size;
+    LinearPtr gate_proj;
+    LinearPtr up_proj;
+    LinearPtr down_proj;
+    std::vector<ParameterPtr> param_vector;
+
+    SwiGLU()
+        : Module(SWIGLU_T)
+        , hidden_size(0U)
+        , intermediate_size(0U)
+    {
+    }
+    SwiGLU(const tcapint &hidden_size_, const tcapint &intermediate_size_, DeviceTag dtag = DEFAULT_DEVICE);
+    void _register_params();
+    std::vector<ParameterPtr> parameters() override { return param_vector; }
+    TensorPtr forward(const TensorPtr x) override;
+    void save(std::ostream &os) const override; // src/modules/swiglu.cpp:18-25
+};
+typedef std::shared_ptr<SwiGLU> SwiGLUPtr;
+
+// include/modules/transformer_encoder_layer.hpp, src/modules/transformer_encoder_layer.cpp:24-139: pre-norm block
+// x1 = x + attn(norm1(x)); out = x1 + ff2(act(ff1(norm2(x1)))).  The reference's forward() also moves its sub-modules
+// between host and device around every step (cpp:64-121); here everything lives on the device, so that is left out.
+struct TransformerEncoderLayer : public Module {
+    tcapint d_model;
+    tcapint d_ff;
+    tcapint num_heads;
+    MultiHeadAttentionPtr self_attn;
+    LinearPtr ff1;
+    LinearPtr ff2;
+    LayerNormPtr norm1;
+    LayerNormPtr norm2;
+    std::shared_ptr<Module> activation;
+    std::vector<ParameterPtr> param_vector;
+
+    TransformerEncoderLayer()
+        : Module(TRANSFORMER_ENCODER_LAYER_T)
+        , d_model(0U)
+        , d_ff(0U)
+        , num_heads(0U)
+    {
+    }
+    TransformerEncoderLayer(const tcapint &d_model_, const tcapint &num_heads_, const tcapint &d_ff_,
+        const DeviceTag &dtag = DEFAULT_DEVICE, const ActivationFunctionType &afn = GELU_FN, const int64_t &did = -1);
+    void _register_params();
+    std::vector<ParameterPtr> parameters() override { return param_vector; }
+    void set_max_kv_seq_len(tcapint m) override { self_attn->set_max_kv_seq_len(m); }
+    void reset_cache() override { self_attn->reset_cache(); }
+    TensorPtr forward(const TensorPtr x) override;
+    void save(std::ostream &os) const override;
+};
+typedef std::shared_ptr<TransformerEncoderLayer> TransformerEncoderLayerPtr;
+
+// include/modules/qwen_decoder_layer.hpp: h = x + attn(rms1(x)); out = h + mlp(rms2(h)), with rotary positions, grouped
+// query heads and bias-carrying projections in the attention as the reference's constructor builds them (hpp:37-50).
+struct QwenDecoderLayer : public Module {
+    tcapint d_model;
+    tcapint num_heads;
+    tcapint num_kv_heads;
+    MultiHeadAttentionPtr self_attn;
+    SwiGLUPtr mlp;
+    RMSNormPtr input_layernorm;
+    RMSNormPtr post_attention_layernorm;
+    std::vector<ParameterPtr> param_vector;
+
+    QwenDecoderLayer()
+        : Module(QWEN_DECODER_LAYER_T)
+        , d_model(0U)
+        , num_heads(0U)
+        , num_kv_heads(0U)
+    {
+    }
+    QwenDecoderLayer(const tcapint &d_model_, const tcapint &num_heads_, const tcapint &num_kv_heads_, const tcapint &d_ff_,
+        const tcapint &max_seq_len = 2048U, const real1_f &rope_base = 10000.0f, const real1_f &eps = 1e-6f,
+        const int64_t &did = -1);
+    void _register_params();
+    std::vector<ParameterPtr> parameters() override { return param_vector; }
+    void set_max_kv_seq_len(tcapint m) override { self_attn->set_max_kv_seq_len(m); }
+    void reset_cache() override { self_attn->reset_cache(); }
+    TensorPtr forward(const TensorPtr x) override;
+    void save(std::ostream &os) const override; // src/modules/qwen_decoder_layer.cpp:18-27
+};
+typedef std::shared_ptr<QwenDecoderLayer> QwenDecoderLayerPtr;
 
 } // namespace Weed
