@@ -20,6 +20,10 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+# Launches that run ahead of every timed region whatever --warmup says: the first dozens of launches after an idle
+# stretch sit in a clock transient (a burst of 25 launches of the headline kernel reads 3-4 % slower than a thousand).
+WARMUP_FLOOR_HEADLINE = 150
+WARMUP_FLOOR_EXTRA = 50
 
 
 def build_cache(capi, torch, wl, seed):
@@ -247,6 +251,94 @@ def decode_entry(capi, torch, fn, n_seq, nbytes, steps, warmup):
     return entry
 
 
+def streaming_read(capi, torch, nbytes, steps, warmup):
+    """What merely reading `nbytes` costs on this part: a buffer of that size swept by the library's read-only kernel,
+    in the decode kernel's launch shape (one contiguous run per wavefront) and as a plain sweep; ms per launch from two
+    events around `steps` back-to-back launches."""
+    buf = torch.empty((nbytes + 3) // 4, dtype=torch.int32, device="cuda")
+    buf.fill_(1)
+    sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+    runs_s = time_region(torch, lambda: capi.read_sweep(buf, nbytes, 1, sink), steps, warmup)
+    sweep_s = time_region(torch, lambda: capi.read_sweep(buf, nbytes, 0, sink), steps, warmup)
+    del buf
+    return {"bytes": nbytes, "per_wavefront_runs_ms": 1e3 * runs_s, "per_wavefront_runs_gbs": nbytes / runs_s / 1e9,
+            "plain_sweep_ms": 1e3 * sweep_s, "plain_sweep_gbs": nbytes / sweep_s / 1e9, "launches": steps,
+            "kernel": "weed_hip_read_sweep: 16-byte loads, nothing written; 256 workgroups x 8 wavefronts with one "
+                      "contiguous run each (the decode kernel's shape), and a grid-stride sweep"}
+
+
+def layer_decode_step(capi, torch, np, n_calls, n_seq=64, ctx=8192, d_model=4096, n_heads=32, n_kv=8, d_ff=14336):
+    """One decode step of one Qwen-style decoder layer (include/modules/qwen_decoder_layer.hpp:104-115) through the C
+    ABI, launch for launch what the host mirror's QwenDecoderLayer::forward issues for a (B, 1, d_model) input:
+    RMSNorm, the Q / K / V projections (with bias), RoPE on Q and K at position ctx, append, fused attention over the
+    packed cache, the output projection, residual, RMSNorm, gate / up projections, SiLU gate, down projection,
+    residual.  Activations are column-major (batch index fastest) as Weed lays them out; weights are random.  The
+    cache starts n_calls tokens short of ctx and every call of the returned step appends one token per sequence."""
+    B, D, H, Hkv, hd = n_seq, d_model, n_heads, n_kv, d_model // n_heads
+    dev = "cuda"
+    g = torch.Generator(device=dev)
+    g.manual_seed(31)
+
+    def cm(rows, cols, scale=1.0):  # logical [rows, cols], column-major
+        return (torch.randn((cols, rows), generator=g, device=dev) * scale).t()
+
+    x = cm(B, D)
+    w_q, w_k, w_v, w_o = cm(D, H * hd, 0.02), cm(D, Hkv * hd, 0.02), cm(D, Hkv * hd, 0.02), cm(H * hd, D, 0.02)
+    b_q, b_k, b_v, b_o = (torch.zeros(n, device=dev) for n in (H * hd, Hkv * hd, Hkv * hd, D))
+    w_gate, w_up, w_down = cm(D, d_ff, 0.02), cm(D, d_ff, 0.02), cm(d_ff, D, 0.02)
+    ln1, ln2 = torch.ones(D, device=dev), torch.ones(D, device=dev)
+    # RoPE tables, column-major [rows, head_dim] (src/modules/rope.cpp:18-51); only row `ctx - 1` is used
+    rows = ctx + 1
+    i = np.arange(hd // 2, dtype=np.float32)
+    theta = np.power(np.float32(10000.0), -2.0 * i / np.float32(hd)).astype(np.float32)
+    ang = np.arange(rows, dtype=np.float32)[:, None] * np.repeat(theta, 2)[None, :]
+    cos_t = torch.from_numpy(np.ascontiguousarray(np.cos(ang).T.astype(np.float32))).to(dev).reshape(-1)
+    sin_t = torch.from_numpy(np.ascontiguousarray(np.sin(ang).T.astype(np.float32))).to(dev).reshape(-1)
+    cache = capi.KVCache(capi.KV_LLOYDMAX, B, Hkv, hd, ctx, 3, 4)
+    rk, rv = torch.zeros(hd * hd, device=dev), torch.zeros(hd * hd, device=dev)
+    capi.make_rotation(41, hd, rk)
+    capi.make_rotation(42, hd, rv)
+    cache.set_rotations(rk, rv)
+    for s0 in range(0, B, 8):
+        Ks = torch.randn((8, Hkv, ctx - n_calls, hd), generator=g, device=dev)
+        Vs = torch.randn((8, Hkv, ctx - n_calls, hd), generator=g, device=dev)
+        cache.encode_append(Ks, Vs, seq_begin=s0, rotate=1)
+    del Ks, Vs
+
+    def buf(cols):
+        return torch.empty((cols, B), device=dev).t()  # logical [B, cols], column-major
+
+    h1, q, k, v, qr, kr, att, o, res1, h2, gate, up, act, down, out = (
+        buf(D), buf(H * hd), buf(Hkv * hd), buf(Hkv * hd), buf(H * hd), buf(Hkv * hd), buf(H * hd), buf(D), buf(D),
+        buf(D), buf(d_ff), buf(d_ff), buf(d_ff), buf(D), buf(D))
+    eps = float(np.float32(np.finfo(np.float32).eps / 4))
+
+    def heads(t, n):  # the (B, heads, T = 1, head_dim) view of a (B, 1, heads * head_dim) activation: feature = h + n * j
+        return torch.as_strided(t, (B, n, 1, hd), (1, B, B, B * n))
+
+    flags = capi.ATTN_ROTATE_Q | capi.ATTN_UNROTATE_OUT
+
+    def step():
+        capi.rms_norm(x, ln1, eps, h1)
+        capi.linear(h1, w_q, b_q, q)
+        capi.linear(h1, w_k, b_k, k)
+        capi.linear(h1, w_v, b_v, v)
+        capi.rope(heads(q, H), cos_t, sin_t, rows, heads(qr, H), pos0=ctx - 1)
+        capi.rope(heads(k, Hkv), cos_t, sin_t, rows, heads(kr, Hkv), pos0=ctx - 1)
+        cache.encode_append(heads(kr, Hkv), heads(v, Hkv), rotate=1)
+        cache.decode_attn(heads(qr, H)[:, :, 0], heads(att, H)[:, :, 0], capi.GQA_BLOCKED, flags)
+        capi.linear(att, w_o, b_o, o)
+        capi.elementwise(capi.EW_ADD, o, x, res1)
+        capi.rms_norm(res1, ln2, eps, h2)
+        capi.linear(h2, w_gate, None, gate)
+        capi.linear(h2, w_up, None, up)
+        capi.elementwise(capi.EW_SILU_MUL, gate, up, act)
+        capi.linear(act, w_down, None, down)
+        capi.elementwise(capi.EW_ADD, down, res1, out)
+
+    return cache, step
+
+
 def extras(capi, torch, workloads, steps, warmup):
     """The other configurations, measured the same way (reported beside the headline, not as `value`)."""
     out = {}
@@ -274,23 +366,33 @@ def extras(capi, torch, workloads, steps, warmup):
                      "frac": wbytes / kernel_s / 1e9 / HBM_PEAK_GBS}}
     out["projection_8x4096x4096"].update(how)
     del X, Wp, Y
-    # standalone softmax and sum over an [8192 x 8192] column-major matrix (256 MiB), along the contiguous axis and
-    # along the strided one: 8 B per element (softmax) and 4 B per element (sum) of algorithmic traffic
-    S = torch.randn((8192, 8192), device="cuda").t()
-    So = torch.empty((8192, 8192), device="cuda").t()
-    Sr = torch.empty(8192, device="cuda")
+    # standalone softmax and sum over an [8192 x 16384] column-major matrix (512 MiB, twice the Infinity Cache, so
+    # that back-to-back launches read from HBM), along the contiguous axis and along the strided one: 8 B per element
+    # (softmax) and 4 B per element (sum) of algorithmic traffic.  Along the strided axis a column block of 32 rows
+    # x 16384 does not fit a compute unit, so that softmax reads the data twice: 12 B per element actually moved
+    # (`bytes_model`); its fraction by the 8 B the metric counts is the one in `roofline.frac`.
+    S = torch.randn((16384, 8192), device="cuda").t()
+    So = torch.empty((16384, 8192), device="cuda").t()
     dense = {}
     for axis, name in ((0, "contiguous_axis"), (1, "strided_axis")):
+        Sr = torch.empty(S.shape[1 - axis], device="cuda")
         for op, fn, bytes_per in (("softmax", lambda: capi.softmax(S, So, axis), 8),
                                   ("reduce", lambda: capi.reduce(capi.REDUCE_SUM, S, Sr, axis), 4)):
             _, kernel_s, how = time_one_kernel_op(capi, torch, fn, op, steps, warmup)
             gbs = S.numel() * bytes_per / kernel_s / 1e9
-            dense["%s_%s" % (op, name)] = {"kernel_ms": 1e3 * kernel_s,
-                                           "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS,
-                                                        "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS}}
-            dense["%s_%s" % (op, name)].update(how)
-    out["softmax_sum_f32_8192x8192"] = dense
-    del S, So, Sr
+            e = {"kernel_ms": 1e3 * kernel_s, "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS,
+                                                           "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS}}
+            if op == "softmax" and axis == 1:
+                moved = S.numel() * 12 / kernel_s / 1e9
+                e["roofline"]["bytes_model"] = {"bytes_per_element_moved": 12, "gbs_moved": moved,
+                                                "frac_moved": moved / HBM_PEAK_GBS,
+                                                "why": "a 32-row column block of this length exceeds a compute unit's "
+                                                       "registers and LDS: one pass for (max, sum), one to normalise"}
+            e.update(how)
+            dense["%s_%s" % (op, name)] = e
+        del Sr
+    out["softmax_sum_f32_8192x16384"] = dense
+    del S, So
     # configuration 5a: encode-and-append 4096 tokens x 8 kv heads x 128, 3-bit codes (rotate, quantise, pack)
     wl = workloads.config(5)
     d = wl.head_dim
@@ -307,17 +409,28 @@ def extras(capi, torch, workloads, steps, warmup):
         cache.reset()
         cache.encode_append(K, V, rotate=1)
 
-    secs, kernel_s = time_kernel(capi, torch, enc, "kv_encode", steps, warmup)
+    secs, pair_s = time_kernel(capi, torch, enc, "kv_encode", steps, warmup)
+    # the kernel alone: a run of back-to-back appends of 4096 tokens into a cache that holds them all, no reset in
+    # between (every append after the first is the same launch: whole half blocks behind whole half blocks, followed by
+    # the small kernel that moves the lengths), two events around the run
+    n_run = min(steps, 40)
+    n_warm = WARMUP_FLOOR_EXTRA
+    big = capi.KVCache(capi.KV_LLOYDMAX, 1, wl.n_kv_heads, d, 4096 * (n_run + n_warm), 3, 3)
+    big.set_rotations(rk, rv)
+    kernel_s = time_region(torch, lambda: big.encode_append(K, V, rotate=1), n_run, n_warm)
+    big.close()
     in_bytes = 2 * K.numel() * 4
     rot_flops = 2 * 2.0 * K.numel() * d  # K and V: rows x 2 d^2
     out["cfg5a_encode_4096x8x128_3bit"] = {
         "tokens_per_s": 4096 / secs, "ms": 1e3 * secs, "input_gbs": in_bytes / secs / 1e9,
         "rotation_tflops": rot_flops / secs / 1e12, "kernel_ms": 1e3 * kernel_s,
+        "kernel_ms_event_pair_per_launch": 1e3 * pair_s,
         "roofline": {"bound": "mfma", "achieved": rot_flops / kernel_s / 1e12, "peak": 157.3, "unit": "TFLOP/s",
                      "frac": rot_flops / kernel_s / 1e12 / 157.3, "kernel": "encode_rows_pair_kernel (K and V)",
                      "flops_per_launch": rot_flops},
-        "kernel_ms_source": "event pairs around the launches (the call also resets the cache and moves the lengths, so "
-                            "a run of calls does not time the kernel alone; the events' own 2-3 us are in the figure)"}
+        "kernel_ms_source": "device time of %d back-to-back appends of 4096 tokens (encoder kernel + the kernel that "
+                            "moves the lengths, no cache reset) between two events, divided by their number; `ms` is "
+                            "the call with the reset that a benchmark loop needs" % n_run}
     cache.close()
     # the append of a decode step: one new token for each of 64 sequences (one launch: the encoder writes the items
     # and moves the lengths itself)
@@ -424,6 +537,33 @@ def extras(capi, torch, workloads, steps, warmup):
         capi, torch, lambda: cache3.decode_attn(q3, o3, capi.GQA_BLOCKED, flags), wl3.n_seq,
         wl3.bytes_per_step(lloydmax=True), steps, warmup)
     cache3.close()
+    del q3, o3
+    # one decode step of one Qwen-style decoder layer on the headline shape (64 sequences near ctx 8192)
+    import numpy as np
+    n_l = min(steps, 50)
+    cacheQ, layer_step = layer_decode_step(capi, torch, np, n_calls=WARMUP_FLOOR_EXTRA + 3 * n_l + 1)
+    layer_step()
+    torch.cuda.synchronize()
+    host_s = time_calls(torch, layer_step, n_l, WARMUP_FLOOR_EXTRA)
+    dev_s = time_region(torch, layer_step, n_l, 0)
+    capi.profile_reset()
+    capi.profile_enable(True)
+    time_calls(torch, layer_step, n_l, 0)
+    parts = {}
+    for name in ("kv_decode_attn", "kv_encode", "matmul", "rms_norm", "elementwise", "rope"):
+        ms, n = capi.profile_read(name)
+        parts[name] = {"ms_per_step": ms / n_l, "launches_per_step": n / n_l}
+    capi.profile_enable(False)
+    out["qwen_layer_decode_step_64_sequences_ctx8192"] = {
+        "ms_per_step": 1e3 * host_s, "device_ms_per_step": 1e3 * dev_s, "tokens_per_s": 64 / host_s,
+        "launches_per_step": sum(p["launches_per_step"] for p in parts.values()),
+        "attention_share": parts["kv_decode_attn"]["ms_per_step"] / (1e3 * dev_s),
+        "by_kernel_family_event_pairs": parts,
+        "shape": "d_model 4096, 32 / 8 heads of 128, d_ff 14336, fp32 weights (0.97 GB per layer), K 3-bit + V 4-bit "
+                 "cache; RMSNorm, Q/K/V projections, RoPE x2, append, attention, output projection, residual, RMSNorm, "
+                 "gate/up projections, SiLU gate, down projection, residual",
+        "weight_bytes": 4 * (2 * 4096 * 4096 + 2 * 4096 * 1024 + 3 * 4096 * 14336)}
+    cacheQ.close()
     return out
 
 
@@ -438,6 +578,9 @@ def main():
     ap.add_argument("--ctx", type=int, default=8192)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the other configurations (4, 5a, 5b)")
+    ap.add_argument("--calibrate-read", action="store_true",
+                    help="only launch the library's read-only sweeps over as many bytes as the headline step reads "
+                         "(the practical ceiling of a read stream on this part), for a rocprofv3 kernel trace")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="only launch the library's plain copy kernel on MIB mebibytes (5 launches): the known-size "
                          "reference against which rocprofv3's FETCH_SIZE / WRITE_SIZE readings are scaled")
@@ -465,6 +608,12 @@ def main():
             torch.cuda.synchronize()
         print(json.dumps({"calibrate_copy_bytes_read": 4 * n, "calibrate_copy_bytes_written": 4 * n, "launches": 5}))
         return
+    if args.calibrate_read:
+        with torch.cuda.stream(stream):
+            wl = workloads.config(3, n_seq=args.seqs, scale=args.ctx / 8192.0)
+            r = streaming_read(capi, torch, wl.bytes_per_step(lloydmax=True), max(args.steps, 200), WARMUP_FLOOR_HEADLINE)
+        print(json.dumps({"streaming_read": r}))
+        return
     with torch.cuda.stream(stream):
         wl = workloads.config(3, n_seq=args.seqs, scale=args.ctx / 8192.0)
         cache, q, rk, rv = build_cache(capi, torch, wl, seed=1234)
@@ -474,7 +623,8 @@ def main():
         def step():
             cache.decode_attn(q, out, capi.GQA_BLOCKED, flags)
 
-        for _ in range(args.warmup):
+        warm = max(args.warmup, WARMUP_FLOOR_HEADLINE)
+        for _ in range(warm):
             step()
         torch.cuda.synchronize()
         # (two HIP events on the launch stream around the timed region, beside the host clock)
@@ -512,7 +662,7 @@ def main():
         if one_kernel:
             capi.decode_tuning(separate_merge=True, separate_query=True)
             try:
-                for _ in range(args.warmup):
+                for _ in range(max(args.warmup, WARMUP_FLOOR_EXTRA)):
                     step()
                 torch.cuda.synchronize()
                 t0 = time.perf_counter()
@@ -534,6 +684,17 @@ def main():
                         "attention_kernel_frac": bytes_per_launch / (sk_ms / max(1, sk_n) * 1e-3) / 1e9 / HBM_PEAK_GBS,
                         "merge_kernel_ms": sc_ms / max(1, sc_n)}
 
+        # The same step for a module whose projections have the rotations folded in (no RoPE between W_q and the cache:
+        # R_k goes into W_q offline; R_v^T into W_o with or without RoPE): flags = 0, nothing rotated in the kernel
+        def step_folded():
+            cache.decode_attn(q, out, capi.GQA_BLOCKED, 0)
+
+        folded_s = time_region(torch, step_folded, args.steps, max(args.warmup, WARMUP_FLOOR_EXTRA))
+        for _ in range(WARMUP_FLOOR_EXTRA):
+            step()  # (leaves `out` as the full call computes it, for the CPU cross-check below)
+        # what merely reading the step's bytes costs
+        read_ceiling = streaming_read(capi, torch, bytes_per_launch, min(max(args.steps, 50), 200), WARMUP_FLOOR_EXTRA)
+
         # batch = 1 latency of the same shape (one sequence per launch: launch-latency bound); part of the extras, so
         # that a --no-extras run launches the main kernel at the headline shape only
         wl1 = workloads.config(3, n_seq=1, scale=args.ctx / 8192.0)
@@ -541,7 +702,7 @@ def main():
         if not args.no_extras:
             cache1, q1, _, _ = build_cache(capi, torch, wl1, seed=99)
             out1 = torch.zeros_like(q1)
-            for _ in range(args.warmup):
+            for _ in range(max(args.warmup, WARMUP_FLOOR_EXTRA)):
                 cache1.decode_attn(q1, out1, capi.GQA_BLOCKED, flags)
             torch.cuda.synchronize()
             t0 = time.perf_counter()
@@ -575,6 +736,7 @@ def main():
             "n_gpus": 1,
             "steps": args.steps,
             "warmup": args.warmup,
+            "warmup_floor_launches": WARMUP_FLOOR_HEADLINE,
             "ms_per_step": ms_per_step,
             "higher_is_better": True,
             "scaling": "weak",
@@ -603,6 +765,13 @@ def main():
                 "algorithmic_bytes_per_launch": bytes_per_launch,
                 "combine_kernel_ms": c_ms / max(1, c_n),
                 "same_step_as_three_kernels": separate,
+                "streaming_read_ms": read_ceiling["per_wavefront_runs_ms"],
+                "streaming_read": read_ceiling,
+                "frac_of_streaming_read": read_ceiling["per_wavefront_runs_ms"] / kernel_ms,
+                "rotations_folded_into_projections": {
+                    "kernel_ms": 1e3 * folded_s, "frac": bytes_per_launch / folded_s / 1e9 / HBM_PEAK_GBS,
+                    "what": "the same call with flags = 0: queries arrive in the K basis and the result stays in the V "
+                            "basis, as for a module that folds R_k into W_q (no RoPE) and R_v^T into W_o offline"},
             },
             "whole_step_gbs": bytes_per_launch / (ms_per_step * 1e-3) / 1e9,
         }
@@ -612,7 +781,7 @@ def main():
             qc = torch.randn((S_, 4, Hq_, d_), device="cuda")
             oc = torch.zeros_like(qc)
             chunk_s = time_calls(torch, lambda: cache.decode_attn_chunk(qc, oc, None, capi.GQA_BLOCKED, flags),
-                                 min(args.steps, 20), min(args.warmup, 3))
+                                 min(args.steps, 200), max(args.warmup, WARMUP_FLOOR_EXTRA))
             result["chunk_of_4_positions"] = {"ms_per_call": 1e3 * chunk_s, "positions_per_s": 4 * wl.n_seq / chunk_s,
                                               "vs_4_single_position_calls": 4 * ms_per_step * 1e-3 / chunk_s}
             del qc, oc
@@ -641,7 +810,7 @@ def main():
         if not args.no_extras:
             # (short kernels need their own warm-up: after an idle stretch the first dozens of launches run at a lower
             # clock, 5 us slower on a 50 us kernel)
-            result["other_configs"] = extras(capi, torch, workloads, min(args.steps, 200), max(args.warmup, 50))
+            result["other_configs"] = extras(capi, torch, workloads, min(args.steps, 200), max(args.warmup, WARMUP_FLOOR_EXTRA))
     print(json.dumps(result))
 
 

@@ -61,6 +61,7 @@ SIGNATURES = {
                                     c_uint32, c_uint32, c_uint32, c_void_p, c_uint32, c_uint32, c_void_p, c_uint32,
                                     c_uint32, c_uint32]),
     "weed_hip_copy_f32": (c_int, [c_uint64, c_void_p, c_uint32, c_uint32, c_void_p, c_uint32, c_uint32]),
+    "weed_hip_read_sweep": (c_int, [c_void_p, c_uint64, c_int, c_void_p]),
     "weed_hip_elementwise_f32": (c_int, [c_int, c_uint32, U32P, c_void_p, c_uint32, U32P, c_void_p, c_uint32, U32P,
                                          c_void_p, c_uint32, U32P]),
     "weed_hip_triu_fill_f32": (c_int, [c_uint32, c_uint32, c_float, c_uint32, c_void_p, c_uint32, c_uint32, c_uint32]),
@@ -318,6 +319,11 @@ def copy(a, out):
 
 
 EW_COPY, EW_ADD, EW_SUB, EW_MUL, EW_DIV = range(5)
+
+
+def read_sweep(buf, nbytes, per_wavefront_runs, sink):
+    """Read the first nbytes of the torch tensor `buf` once (calibration); sink: a one-element int32 device tensor."""
+    check(load().weed_hip_read_sweep(c_void_p(buf.data_ptr()), nbytes, int(per_wavefront_runs), c_void_p(sink.data_ptr())))
 
 
 def elementwise(op, a, b, out):
