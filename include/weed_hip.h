@@ -335,7 +335,8 @@ int weed_hip_kv_decode_tuning(int32_t wavefronts, int32_t skew_percent, int32_t 
  * no hipMalloc / hipFree and creates no events (the library's timing scopes skip it).  Shapes whose workspace
  * 64 KiB + n_seq * n_q_heads * (d * 8 + 8 + slots * (d + 2) * 4) bytes (slots: context splits, at most a few dozen)
  * exceeds the array return WEED_HIP_EINVAL.  The first 64 KiB are arrival counters of the kernel's own merge: they start
- * as zeros with the array and every launch that completes leaves them at zero.  All calls on one device share the
+ * as zeros with the array and every launch that completes leaves them at zero; weed_hip_kv_cache_reset (of any cache)
+ * and weed_hip_shutdown clear them too, which is how a process recovers them after a launch the device aborted.  All calls on one device share the
  * array: calls that overlap on one device (two host threads, two streams) race; weed_hip_init must have run on the
  * device. */
 int weed_hip_kv_decode_attn_noalloc(weed_hip_kv_cache *cache, int32_t n_q_heads, int32_t gqa_mapping,

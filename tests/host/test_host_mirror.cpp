@@ -83,7 +83,7 @@ std::vector<real1> gaussian(size_t n, uint32_t seed, real1 scale = 1.0f)
     return v;
 }
 
-// The attention tolerance: |got - want| <= 1e-4 + 1e-3 |want|
+// The attention tolerance: |got - want| <= max(1e-4, 1e-3 |want|)
 bool attn_close(const std::vector<real1> &got, const std::vector<double> &want, double *worst = nullptr)
 {
     bool ok = got.size() == want.size();
@@ -91,7 +91,7 @@ bool attn_close(const std::vector<real1> &got, const std::vector<double> &want, 
     for (size_t i = 0; ok && i < got.size(); ++i) {
         const double err = std::fabs((double)got[i] - want[i]);
         w = std::max(w, err);
-        if (!(err <= 1e-4 + 1e-3 * std::fabs(want[i]))) {
+        if (!(err <= std::max(1e-4, 1e-3 * std::fabs(want[i])))) {
             ok = false;
         }
     }

@@ -442,6 +442,54 @@ def test_any_batch_as_one_kernel(gpu, oracle, lloyd, d, Hkv, Hq, lens, kb, vb, w
     cache.close()
 
 
+@pytest.mark.parametrize("which", ["cfg4_reduced", "equal_24", "small_4"])
+def test_merges_through_memory_repeat_bit_for_bit(gpu, oracle, which):
+    """The merges that go through memory and an arrival counter per region -- ragged batches (configuration 4 at a
+    sixteenth of its lengths), equal sequences whose regions do not line up with the workgroups (24 sequences), and a
+    small batch whose regions are several workgroups' shares (4 sequences) -- run 300 times back to back through the
+    one-kernel path: every output must equal the first one bit for bit (the order of the additions is fixed, so any
+    difference would be a partial read before its writer's store was visible), and the first must match the
+    checker.  The counters' release / acquire pair is what this leans on."""
+    import torch
+    rng = np.random.default_rng(7)
+    if which == "cfg4_reduced":
+        wl = workloads.config(4, scale=1.0 / 16)
+        Hq = 32
+    else:
+        n = 24 if which == "equal_24" else 4
+        wl = workloads.Workload(which, n, 32, 8, 128, [1984 if n == 24 else 8192] * n, 3, 4, 0, 0, 0)
+        Hq = 32
+    S, Hkv, d, L = wl.n_seq, wl.n_kv_heads, wl.head_dim, wl.max_len
+    cache = gpu.KVCache(gpu.KV_LLOYDMAX, S, Hkv, d, L, wl.k_bits, wl.v_bits, wl.k_sign, wl.v_sign)
+    for s0, n_tok in enumerate(wl.lens):
+        Ks = torch.randn((1, Hkv, n_tok, d), device="cuda")
+        Vs = torch.randn((1, Hkv, n_tok, d), device="cuda")
+        cache.encode_append(Ks, Vs, seq_begin=s0)
+    q = rng.standard_normal((S, Hq, d), dtype=np.float32)
+    qd = dev(q)
+    outs = [torch.zeros_like(qd) for _ in range(4)]
+    try:
+        gpu.profile_reset()
+        gpu.profile_enable(True)
+        cache.decode_attn(qd, outs[0], gpu.GQA_BLOCKED, 0)
+        gpu.sync()
+        assert gpu.profile_read("kv_decode_attn")[1] == 1 and gpu.profile_read("kv_decode_combine")[1] == 0
+    finally:
+        gpu.profile_enable(False)
+    first = outs[0].clone()
+    wl_q = workloads.Workload(which, S, Hq, Hkv, d, wl.lens, wl.k_bits, wl.v_bits, wl.k_sign, wl.v_sign, 0)
+    if which != "small_4":  # (the scalar checker takes seconds per thousand tokens and head)
+        assert_attn_close(first.cpu().numpy(), checker_output(oracle, gpu, cache, wl_q, q, False), which)
+    # launches back to back, three outputs in flight between comparisons so that the device never idles between them
+    for rep in range(100):
+        for o in outs[1:]:
+            cache.decode_attn(qd, o, gpu.GQA_BLOCKED, 0)
+        gpu.sync()
+        for i, o in enumerate(outs[1:]):
+            assert torch.equal(o, first), "%s: repeat %d differs from the first result" % (which, 3 * rep + i + 1)
+    cache.close()
+
+
 def test_random_batches_planned_against_plain(gpu):
     """Sixty seeded random batches -- equal, nearly equal, mildly and widely different lengths, up to 128 sequences,
     caches with and without room behind the longest sequence, both coders, head_dims with and without instances that

@@ -29,6 +29,11 @@ int current_device();
 // it once per device with that device current.
 int decode_scratch_setup(int device_id);
 
+// Puts the arrival counters at the start of the current device's static decode scratch back to zero (a fill kernel
+// on the library's stream).  Every launch that completes leaves them at zero; this is for a launch that the device
+// aborted midway.  weed_hip_kv_cache_reset and weed_hip_shutdown call it.
+int decode_scratch_clear_counters();
+
 // Frees the scratch of the split products (matmul.hip); weed_hip_shutdown calls it after draining the stream.
 void release_split_scratch();
 

@@ -300,6 +300,8 @@ int weed_hip_shutdown(void)
         return WEED_HIP_OK;
     }
     WEED_HIP_CHECK(hipSetDevice(g_device));
+    // (the static decode scratch outlives the library's state: leave its arrival counters at zero for a later start)
+    WEED_HIP_TRY(decode_scratch_clear_counters());
     WEED_HIP_CHECK(hipStreamSynchronize(g_stream));
     if (g_own_stream && g_stream != g_own_stream) {
         WEED_HIP_CHECK(hipStreamSynchronize(g_own_stream));

@@ -52,6 +52,7 @@ struct weed_hip_kv_cache {
     weedhip::Side k, v;
     bool has_rotations = false;
     std::vector<int32_t> lens; // host mirror of lens_dev
+    std::vector<uint64_t> plan_region_end; // host scratch of the decode planner, kept between calls
     int32_t *lens_dev = nullptr;
     uint32_t *append_done = nullptr; // behind lens_dev: workgroups of the append under way that are through
     // scratch for encode: one field per byte + row scales for the tokens being appended

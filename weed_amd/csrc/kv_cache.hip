@@ -1442,6 +1442,8 @@ int weed_hip_kv_cache_reset(weed_hip_kv_cache *c, int drop_rotations)
         fill_i32_kernel<<<(counters + 255) / 256, 256, 0, stream()>>>((int32_t *)c->dec_ws, 0, counters);
         WEED_HIP_LAUNCH_CHECK();
     }
+    // ... and those at the start of the device's static scratch (weed_hip_kv_decode_attn_noalloc), which no cache owns
+    WEED_HIP_TRY(decode_scratch_clear_counters());
     if (drop_rotations) {
         c->has_rotations = false;
     }

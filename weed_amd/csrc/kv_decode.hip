@@ -27,6 +27,13 @@ static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 namespace {
 constexpr int kMaxDevices = 64;
 void *g_scratch_dev[kMaxDevices] = {};
+__global__ void __launch_bounds__(256) clear_words_kernel(uint32_t *p, uint32_t n)
+{
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) {
+        p[i] = 0u;
+    }
+}
 } // namespace
 
 namespace weedhip {
@@ -41,6 +48,17 @@ int decode_scratch_setup(int device_id)
         WEED_HIP_CHECK(hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)));
         g_scratch_dev[device_id] = ptr;
     }
+    return WEED_HIP_OK;
+}
+int decode_scratch_clear_counters()
+{
+    const int dev = current_device();
+    if (dev < 0 || dev >= kMaxDevices || !g_scratch_dev[dev]) {
+        return WEED_HIP_OK; // the library has not been started on this device: nothing to clear
+    }
+    clear_words_kernel<<<(kMfmaMergeCounters + 255) / 256, 256, 0, stream()>>>(static_cast<uint32_t *>(g_scratch_dev[dev]),
+                                                                              kMfmaMergeCounters);
+    WEED_HIP_LAUNCH_CHECK();
     return WEED_HIP_OK;
 }
 } // namespace weedhip
@@ -822,6 +840,9 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
     WEED_HIP_REQUIRE(n_tokens == 1 || use_mfma,
                      "%s: head_dim %u with fields of %u and %u bits is not served by the matrix-core kernel, which a "
                      "chunk of positions needs", fn, d, c->k.w, c->v.w);
+    // ONE copy of the process-wide tuning for the whole plan: weed_hip_kv_decode_tuning may change it from another host
+    // thread at any time, and a plan must not pair a block count chosen under one setting with a search mode of another.
+    const DecodeTuning tune = decode_tuning();
     uint32_t n_splits, split_tokens = 0;
     uint32_t total_blocks = 0;
     RunGeom runs = { 1, 0, 8 };
@@ -832,7 +853,6 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         // every wavefront takes an equal run of 64-token blocks from the list of all regions' blocks; as many
         // wavefronts as the device holds at once
         runs.waves = mfma_decode_workgroup_waves(pass_heads, d, c->k.w, c->v.w);
-        const DecodeTuning &tune = decode_tuning();
         // Equal sequences of nb blocks: prefer a run length with which every workgroup holds whole regions (the
         // kernel then does the whole call by itself, see below): nb / (classes * q) blocks with q = 1, 2 or 4, that
         // is 4 / q regions per workgroup, provided the workgroups fill the compute units in at most two rounds.
@@ -1019,7 +1039,7 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
     if (use_mfma && total_blocks) {
         uniform_blocks = partition_blocks(c->lens[0]);
         for (int32_t l : c->lens) {
-            if (partition_blocks(l) != uniform_blocks || decode_tuning().always_search) {
+            if (partition_blocks(l) != uniform_blocks || tune.always_search) {
                 uniform_blocks = 0;
                 break;
             }
@@ -1028,11 +1048,11 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         const uint32_t nb = uniform_blocks, cycle = run_classes(runs) * runs.unit_blocks;
         const uint32_t wg_blocks = runs.waves * runs.unit_blocks;
         if (mfma_decode_merges(gp, d) && nb != 0 && nb % cycle == 0 && wg_blocks % nb == 0 &&
-            !decode_tuning().separate_merge) {
+            !tune.separate_merge) {
             wg_regions = wg_blocks / nb;
         } else if (mfma_decode_merges(gp, d) && nb != 0 && nb % wg_blocks == 0 && nb / wg_blocks >= 2 &&
                    nb / wg_blocks <= std::min(n_splits, 64u) && (size_t)S * Hkv <= kMfmaMergeCounters &&
-                   !decode_tuning().separate_merge) {
+                   !tune.separate_merge) {
             // small batches of long sequences: every region is a whole number of workgroups' shares
             region_wgs = nb / wg_blocks;
         }
@@ -1040,7 +1060,9 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         uint32_t wg_most_regions = wg_regions;
         bool every_sequence_has_tokens = true;
         if (wg_regions == 0) {
-            std::vector<uint64_t> region_end; // blocks up to and including region r
+            // (a buffer of the cache object, so that a decode call allocates nothing on the host either)
+            std::vector<uint64_t> &region_end = c->plan_region_end; // blocks up to and including region r
+            region_end.clear();
             region_end.reserve((size_t)S * Hkv);
             uint64_t run = 0;
             for (int32_t l : c->lens) {
@@ -1072,19 +1094,20 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         // 30 us at 8 to 17).  Nor do they where they could not rotate their queries as well (a kernel ahead and the
         // merges at the end: 3 to 200 sequences of 100 tokens with groups of eight, 27 us against 22 to 25).
         if (wg_regions == 0 && region_wgs == 0 && mfma_decode_merges(gp, d) && every_sequence_has_tokens &&
-            (nb != 0 || (S <= 63 && !decode_tuning().always_search)) && n_splits <= 64 &&
+            (nb != 0 || (S <= 63 && !tune.always_search)) && n_splits <= 64 &&
             wg_most_regions <= kMostRegionsMergedByWorkgroup && wg_most_regions * pass_heads <= kMfmaQueryRows &&
-            (size_t)S * Hkv <= kMfmaMergeCounters && !decode_tuning().separate_merge) {
+            (size_t)S * Hkv <= kMfmaMergeCounters && !tune.separate_merge) {
             general_merge = true;
         }
         // A workgroup rotates the queries of the regions its blocks lie in itself when they are few enough for its
         // LDS (equal sequences, or the ragged batches above); nothing then runs ahead of the matrix-core kernel.
         fused_query = mfma_decode_merges(gp, d) && (nb != 0 || general_merge) &&
-                      wg_most_regions * pass_heads <= kMfmaQueryRows && !decode_tuning().separate_query;
+                      wg_most_regions * pass_heads <= kMfmaQueryRows && !tune.separate_query;
     }
     const bool fused_merge = wg_regions != 0 || region_wgs != 0 || general_merge;
     // (the kernels that take one (sequence, head) row per workgroup have the sequence on a 16-bit grid dimension)
-    WEED_HIP_REQUIRE(S <= 65535u || (use_mfma && many_rows && n_splits <= 64),
+    // (prep_q_kernel puts one more row on that dimension when it also builds the block offsets)
+    WEED_HIP_REQUIRE(S + ((use_mfma && !fused_query && !many_rows) ? 1u : 0u) <= 65535u || (use_mfma && many_rows && n_splits <= 64),
                      "%s: %u sequences in one call are served only for head_dims that are multiples of 64 with "
                      "matrix-core instances; split the batch", fn, S);
     if (fused_query) {

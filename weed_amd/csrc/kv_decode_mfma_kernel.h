@@ -1273,9 +1273,11 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
             const uint32_t wg_regions_here = wg_rows / p.G, wg_blocks = kWaves * p.runs.unit_blocks;
             if (wave == 0) {
                 // The partials were ordinary stores (stores of device scope between a wavefront's segments would hold
-                // up the loads of its next segment, which wait on the same counter): they sit in this XCD's L2, and ONE
-                // write-back per workgroup makes them visible to the others before the arrivals are counted.
-                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+                // up the loads of its next segment, which wait on the same counter): they sit in this XCD's L2.  The
+                // arrival below is a RELEASE of device scope -- one L2 write-back per workgroup, ordered after every
+                // wavefront's stores by the barrier above -- and the workgroup that completes a count takes an ACQUIRE
+                // fence of device scope before it reads the region's partials: release / acquire on the counter is what
+                // makes the other workgroups' partials visible, not the timing of the caches.
                 // (all lanes compute: the offsets travel between lanes)
                 const uint32_t region = min(wg_region0 + lane, n_regions - 1);
                 const uint32_t s_ = region / p.Hkv, kv_ = region - s_ * p.Hkv;
@@ -1294,7 +1296,7 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
                 if (lane < wg_regions_here) {
                     uint32_t before = 0;
                     if (wgs > 1) {
-                        before = __hip_atomic_fetch_add(p.merge.arrive + region, 1u, __ATOMIC_RELAXED,
+                        before = __hip_atomic_fetch_add(p.merge.arrive + region, 1u, __ATOMIC_RELEASE,
                                                         __HIP_MEMORY_SCOPE_AGENT);
                         if (before + 1 == wgs) {
                             __hip_atomic_store(p.merge.arrive + region, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -1306,6 +1308,9 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
                 // (at most 31, the host sees to that)
                 const bool mine = lane < wg_regions_here && before_plus_one == wgs;
                 const uint64_t mask = __ballot(mine);
+                if (mask) {
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+                }
                 if (mine) {
                     const uint32_t at = (uint32_t)__builtin_popcountll(mask & ((1ull << lane) - 1ull));
                     count_s[1 + 2 * at] = region;
@@ -1332,10 +1337,10 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
             }
         } else {
             // A share of ONE region: the wavefronts' partials become one partial of the region in
-            // memory, stored through to device scope; when those stores have completed the workgroup counts itself,
-            // and the workgroup that completes the region's count reads all of the region's partials with loads of
-            // device scope and finishes the rows.  (No cache-wide write-back or invalidation: every wavefront issuing
-            // them costs more than the whole merge.)
+            // memory; behind a barrier ONE thread counts the workgroup with a RELEASE of device scope, and the
+            // workgroup that completes the region's count takes an ACQUIRE fence of device scope, then reads all of
+            // the region's partials and finishes the rows.  (One write-back per workgroup and one invalidation per
+            // region: every wavefront issuing them costs more than the whole merge.)
             const uint32_t wg_blocks = kWaves * p.runs.unit_blocks;
             const uint32_t region = (blockIdx.x * wg_blocks) / p.uniform_blocks;
             const uint32_t my_slot = blockIdx.x - (region * p.uniform_blocks) / wg_blocks;
@@ -1359,7 +1364,11 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __syncthreads();
             if (tid == 0) {
-                *count_s = __hip_atomic_fetch_add(p.merge.arrive + region, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                const uint32_t before = __hip_atomic_fetch_add(p.merge.arrive + region, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+                if (before + 1 == p.merge.region_wgs) {
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+                }
+                *count_s = before;
             }
             __syncthreads();
             if (*count_s + 1 != p.merge.region_wgs) {
