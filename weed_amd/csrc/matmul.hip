@@ -433,25 +433,71 @@ __global__ void __launch_bounds__(64 * kSkinnyWaves)
 }
 
 
-// ---- Seventeen to 64 rows: the same streaming of b, but the rows of a no longer come cheaply from L2 if every
-//      16-column workgroup reads all of them (64 rows x K floats per workgroup, four times the bytes of b in total).
-//      Here a workgroup owns 128 columns (16 per wavefront), all its wavefronts walk the same k range and share the
-//      rows of a through LDS ([k][row], two buffers, one barrier per 64-k step), and the k ranges are split over
-//      gridDim.y workgroups whose partial results a small second kernel adds up in a fixed order.
+// ---- Seventeen to 64 rows: the same streaming of b, but at this many rows the fp32 matrix instruction would bound
+//      the product (128 flop per byte of b against the part's 20), and the rows of a no longer come cheaply from L2 if
+//      every 16-column workgroup reads all of them.  So the products run on the bfloat16 matrix instruction
+//      v_mfma_f32_16x16x32_bf16 (sixteen times the fp32 rate) with BOTH operands split exactly into three bfloat16
+//      parts: a float's 24-bit significand is three 8-bit pieces, x = x1 + x2 + x3 with every part a bfloat16, so
+//      x.w is the sum of nine exact products of which the six with i + j <= 4 carry everything above 2^-24 of the
+//      result; they accumulate in fp32 inside the instruction.  The outcome has the quality of an fp32 product
+//      (measured: error below 1.2e-7 of the sum of the terms' magnitudes), not the bits of a sequential fp32 sum.
+//      A workgroup owns 128 columns (16 per wavefront); all its wavefronts walk the same k range and share the rows
+//      of `a`, which the workgroup splits step by step into LDS ([part][row][k], rows padded to 144 bytes so that
+//      sixteen rows' 16-byte reads cover all banks once; two buffers, one barrier per 64-k step); the k ranges are
+//      split over gridDim.y workgroups whose partial results a small kernel behind adds up in a fixed order.
+//      64 rows: 4096 x 4096 weights 39 -> 33 us per product, 4096 x 14336 125 -> 76 us, 14336 x 4096 105 -> 72 us.
+//      What bounds it now is the SIMDs' issue slots: per 32 KB of b a compute unit issues 384 matrix instructions,
+//      ~1500 vector instructions (the splits) and 192 16-byte LDS reads, and the three kinds add up rather than
+//      overlap (every piece switched off in turn: the loads and splits alone run at 4.8 TB/s, the whole at 3.3).
+//      Measured and dropped: the rows split once by a kernel ahead and copied into LDS as an image (more L2 traffic
+//      than the fp32 rows: 84 us), two column tiles per wavefront (72 us), sixteen wavefronts per workgroup (78 us),
+//      four wavefronts per workgroup (73 us), three to six register sets of b instead of two (98 us).
 constexpr int kWideWaves = 8;
-constexpr int kWidePitch = 65; // floats per k row of the staged block of a: two-way bank conflicts at worst
+constexpr int kWidePitchH = 72; // halves per staged row: 64 k + 8 of padding
+
+typedef uint32_t uint4w __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+// w = p1 + p2 + p3 exactly, every part a bfloat16 (the upper halves of the returned words): the top 8 bits of the
+// significand, the top 8 bits of what is left, and the rest (at most 8 bits)
+__device__ __forceinline__ void split_bf16x3(float w, uint32_t &p1, uint32_t &p2, uint32_t &p3)
+{
+    p1 = __float_as_uint(w) & 0xffff0000u;
+    const float r1 = w - __uint_as_float(p1);
+    p2 = __float_as_uint(r1) & 0xffff0000u;
+    const float r2 = r1 - __uint_as_float(p2);
+    p3 = __float_as_uint(r2);
+}
+// the upper halves of (lo, hi) as one word, `lo` in the low half
+__device__ __forceinline__ uint32_t pack_upper_halves(uint32_t lo, uint32_t hi)
+{
+    return __builtin_amdgcn_perm(hi, lo, 0x07060302u);
+}
+// eight consecutive values -> three operands of the matrix instruction (one per part)
+__device__ __forceinline__ void split_eight(const float (&v)[8], uint4w (&part)[3])
+{
+    uint32_t p[3][8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        split_bf16x3(v[e], p[0][e], p[1][e], p[2][e]);
+    }
+#pragma unroll
+    for (int pl = 0; pl < 3; ++pl) {
+        part[pl] = uint4w{ pack_upper_halves(p[pl][0], p[pl][1]), pack_upper_halves(p[pl][2], p[pl][3]),
+                           pack_upper_halves(p[pl][4], p[pl][5]), pack_upper_halves(p[pl][6], p[pl][7]) };
+    }
+}
 
 template <int MT>
 __global__ void __launch_bounds__(64 * kWideWaves)
     matmul_skinny_wide_kernel(const float *__restrict__ a, const float *__restrict__ b, float *__restrict__ part,
-                              MatGeom g_launch, uint32_t k_per_split)
+                              MatGeom g, uint32_t k_per_split)
 {
     typedef float float4v __attribute__((ext_vector_type(4)));
-    const MatGeom g = batch_geom(g_launch);
-    __shared__ float As[2][64][kWidePitch];
+    __shared__ __attribute__((aligned(16))) uint16_t xs[2][3][16 * MT][kWidePitchH];
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t c = lane & 15, grp = lane >> 4;
-    const uint32_t n = blockIdx.x * 128 + wave * 16 + c;
+    const uint32_t n = blockIdx.x * (16 * kWideWaves) + wave * 16 + c;
     const bool n_ok = n < g.N;
     const float *wcol = b + (uint64_t)g.b_off + (uint64_t)(n_ok ? n : 0) * g.b_s1;
     const uint32_t kb0 = blockIdx.y * k_per_split;
@@ -461,6 +507,7 @@ __global__ void __launch_bounds__(64 * kWideWaves)
     for (int mt = 0; mt < MT; ++mt) {
         acc[mt] = float4v{ 0.0f, 0.0f, 0.0f, 0.0f };
     }
+    // this lane's sixteen consecutive k of its column, kb + 16 grp .., zero beyond the range (K is a multiple of 4)
     auto load_w = [&](uint32_t kb, float4v (&w)[4]) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
@@ -468,53 +515,88 @@ __global__ void __launch_bounds__(64 * kWideWaves)
             w[q] = (n_ok && k < kb1) ? *reinterpret_cast<const float4v *>(wcol + k) : float4v{ 0.0f, 0.0f, 0.0f, 0.0f };
         }
     };
-    // the 16*MT x 64 block of a for one step: thread t fetches rows (t % 16) + 16 i of k column t / 16 + 32 j
-    constexpr int kStage = MT * 2; // elements per thread: 16*MT rows x 64 k over 512 threads
-    auto fetch_a = [&](uint32_t kb, float (&v)[kStage]) {
+    // the rows of a for one 64-k step: thread (row = tid % (16 MT), octet = tid / (16 MT)) fetches a[row][kb + 8 octet
+    // .. + 7], splits the eight values and stores one 16-byte piece per part
+    constexpr uint32_t kRows = 16 * MT;
+    const uint32_t srow = tid % kRows, soct = tid / kRows;
+    const bool stager = soct < 8;
+    const float *arow = a + (uint64_t)g.a_off + (uint64_t)(srow < g.M ? srow : 0) * g.a_s0;
+    auto fetch_rows = [&](uint32_t kb, float (&v)[8]) {
 #pragma unroll
-        for (int e = 0; e < kStage; ++e) {
-            const uint32_t m = (tid & 15) + 16 * (e % MT);
-            const uint32_t k = kb + (tid >> 4) + 32 * (e / MT);
-            v[e] = (m < g.M && k < kb1) ? a[(uint64_t)g.a_off + (uint64_t)m * g.a_s0 + (uint64_t)k * g.a_s1] : 0.0f;
+        for (int e = 0; e < 8; ++e) {
+            const uint32_t k = kb + 8 * soct + e;
+            v[e] = (stager && srow < g.M && k < kb1) ? arow[(uint64_t)k * g.a_s1] : 0.0f;
         }
     };
-    auto store_a = [&](int buf, const float (&v)[kStage]) {
+    auto store_rows = [&](int buf, const float (&v)[8]) {
+        if (stager) {
+            uint4w part3[3];
+            split_eight(v, part3);
 #pragma unroll
-        for (int e = 0; e < kStage; ++e) {
-            As[buf][(tid >> 4) + 32 * (e / MT)][(tid & 15) + 16 * (e % MT)] = v[e];
-        }
-    };
-    float4v w[2][4];
-    float stage[kStage];
-    if (kb0 < kb1) {
-        load_w(kb0, w[0]);
-        fetch_a(kb0, stage);
-        store_a(0, stage);
-    }
-    __syncthreads();
-    auto iterate = [&](auto pc, uint32_t kb) {
-        constexpr int P = decltype(pc)::value;
-        load_w(kb + 64, w[1 - P]);
-        fetch_a(kb + 64, stage); // lands in registers while this step is multiplied
-#pragma unroll
-        for (int j = 0; j < 16; ++j) {
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(As[P][16 * grp + j][16 * mt + c], w[P][j / 4][j % 4],
-                                                               acc[mt], 0, 0, 0);
+            for (int pl = 0; pl < 3; ++pl) {
+                *reinterpret_cast<uint4w *>(&xs[buf][pl][srow][8 * soct]) = part3[pl];
             }
         }
-        store_a(1 - P, stage);
+    };
+    constexpr int kDepth = 2; // register sets of b: the columns of the next step travel while one is multiplied (more sets: slower)
+    float4v w[kDepth][4];
+    float stage[8];
+    if (kb0 < kb1) {
+#pragma unroll
+        for (int i = 0; i < kDepth - 1; ++i) {
+            load_w(kb0 + 64 * i, w[i]);
+        }
+        fetch_rows(kb0, stage);
+        store_rows(0, stage);
+    }
+    __syncthreads();
+    auto iterate = [&](auto pc, auto xc, uint32_t kb) {
+        constexpr int P = decltype(pc)::value; // register set of this step
+        constexpr int X = decltype(xc)::value; // LDS buffer of this step
+        load_w(kb + 64 * (kDepth - 1), w[(P + kDepth - 1) % kDepth]);
+        fetch_rows(kb + 64, stage); // lands in registers while this step is multiplied
+        // the two halves of this lane's sixteen k: instruction j contracts over { kb + 16 grp + 8 j .. + 7 : grp }
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const float v[8] = { w[P][2 * j][0], w[P][2 * j][1], w[P][2 * j][2], w[P][2 * j][3],
+                                 w[P][2 * j + 1][0], w[P][2 * j + 1][1], w[P][2 * j + 1][2], w[P][2 * j + 1][3] };
+            uint4w bw[3];
+            split_eight(v, bw);
+            const bf16x8 B0 = __builtin_bit_cast(bf16x8, bw[0]), B1 = __builtin_bit_cast(bf16x8, bw[1]),
+                         B2 = __builtin_bit_cast(bf16x8, bw[2]);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                bf16x8 A[3];
+#pragma unroll
+                for (int pl = 0; pl < 3; ++pl) {
+                    A[pl] = __builtin_bit_cast(
+                        bf16x8, *reinterpret_cast<const uint4w *>(&xs[X][pl][16 * mt + c][16 * grp + 8 * j]));
+                }
+                // the small terms first
+                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A[2], B0, acc[mt], 0, 0, 0);
+                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A[1], B1, acc[mt], 0, 0, 0);
+                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A[0], B2, acc[mt], 0, 0, 0);
+                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A[1], B0, acc[mt], 0, 0, 0);
+                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A[0], B1, acc[mt], 0, 0, 0);
+                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A[0], B0, acc[mt], 0, 0, 0);
+            }
+        }
+        store_rows(1 - X, stage);
         __syncthreads(); // the other buffer is complete, and nobody reads this one any more
     };
-    for (uint32_t kb = kb0; kb < kb1; kb += 128) {
-        iterate(std::integral_constant<int, 0>{}, kb);
-        if (kb + 64 < kb1) {
-            iterate(std::integral_constant<int, 1>{}, kb + 64);
-        }
+    // rounds of 2 kDepth steps so that register set and LDS buffer are compile-time constants
+    uint32_t kb = kb0;
+    while (kb < kb1) {
+        static_for_sets<0, 2 * kDepth>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            if (kb < kb1) {
+                iterate(std::integral_constant<int, i % kDepth>{}, std::integral_constant<int, i % 2>{}, kb);
+                kb += 64;
+            }
+        });
     }
     // partial result of this k range: part[split][row][column] (dense, row-major in columns)
-    float *dst = part + ((uint64_t)blockIdx.z * gridDim.y + blockIdx.y) * g.M * g.N;
+    float *dst = part + (uint64_t)blockIdx.y * g.M * g.N;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
@@ -654,25 +736,21 @@ int launch_matmul(const char *fn, const MatGeom &g, uint32_t batch, const float 
         // every wavefront of a workgroup takes a whole number of 64-k iterations
         const uint32_t k_per_wave = ((K + kSkinnyWaves - 1) / kSkinnyWaves + 63) / 64 * 64;
         const dim3 wgs((N + 15) / 16, 1, batch);
-        if (M > 16 && N >= 512) {
-            // shared rows, k split over workgroups (about one workgroup per compute unit), second pass adds the splits
-            const uint32_t col_wgs = (N + 127) / 128;
-            uint32_t splits = std::max(1u, std::min((256u + col_wgs - 1) / col_wgs, K / 256u));
+        if (M > 16 && N >= 512 && batch == 1) {
+            // shared rows, k split over workgroups (about 450 workgroups in all), a second pass adds the splits
+            const uint32_t col_wgs = (N + 16 * kWideWaves - 1) / (16 * kWideWaves);
+            uint32_t splits = std::max(1u, std::min((448u + col_wgs / 2) / col_wgs, K / 256u));
             const uint32_t k_per_split = ((K + splits - 1) / splits + 63) / 64 * 64;
             splits = (K + k_per_split - 1) / k_per_split;
-            const size_t need = sizeof(float) * (size_t)batch * splits * M * N;
-            WEED_HIP_TRY(grow_split_scratch(fn, need));
-            const dim3 wide(col_wgs, splits, batch);
+            WEED_HIP_TRY(grow_split_scratch(fn, sizeof(float) * (size_t)splits * M * N));
+            const dim3 wide(col_wgs, splits, 1);
             if (M <= 32) {
-                matmul_skinny_wide_kernel<2><<<wide, 64 * kWideWaves, 0, stream()>>>(a_dev, b_dev, g_split_ws, g,
-                                                                                   k_per_split);
+                matmul_skinny_wide_kernel<2><<<wide, 64 * kWideWaves, 0, stream()>>>(a_dev, b_dev, g_split_ws, g, k_per_split);
             } else {
-                matmul_skinny_wide_kernel<4><<<wide, 64 * kWideWaves, 0, stream()>>>(a_dev, b_dev, g_split_ws, g,
-                                                                                   k_per_split);
+                matmul_skinny_wide_kernel<4><<<wide, 64 * kWideWaves, 0, stream()>>>(a_dev, b_dev, g_split_ws, g, k_per_split);
             }
             WEED_HIP_LAUNCH_CHECK();
-            matmul_split_sum_kernel<<<dim3((M * N + 255) / 256, 1, batch), 256, 0, stream()>>>(g_split_ws, out_dev, g,
-                                                                                             splits);
+            matmul_split_sum_kernel<<<dim3((M * N + 255) / 256, 1, 1), 256, 0, stream()>>>(g_split_ws, out_dev, g, splits);
             WEED_HIP_LAUNCH_CHECK();
             return WEED_HIP_OK;
         }

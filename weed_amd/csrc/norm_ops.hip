@@ -163,6 +163,64 @@ __global__ void __launch_bounds__(THREADS) norm_kernel(const float *__restrict__
     }
 }
 
+// Few rows along a strided axis (a decode step's (B, 1, d_model) activations: the batch index is the contiguous one):
+// a workgroup takes 16 neighbouring rows and adds up the WHOLE axis for them, but finishes only its own slice of the
+// axis (gridDim.y slices).  The sums are computed once per slice -- redundant reads of a tensor that sits in L2 -- so
+// that the per-element work (a correctly rounded division among it) spreads over enough compute units.
+template <bool LAYER> __global__ void __launch_bounds__(1024) norm_sliced_kernel(const float *__restrict__ x,
+                                                                               const float *__restrict__ w,
+                                                                               const float *__restrict__ beta,
+                                                                               float *__restrict__ out, NormGeom g)
+{
+    constexpr int RT = 16, THREADS = 1024, NY = THREADS / RT, U = 8;
+    __shared__ float red[(THREADS / 64) * RT];
+    const uint32_t tx = threadIdx.x % RT, ty = threadIdx.x / RT;
+    const uint32_t row = blockIdx.x * RT + tx;
+    const bool valid = row < g.rows;
+    uint64_t x_base = g.x_off, o_base = g.o_off;
+    if (valid) {
+        row_bases(g, row, x_base, o_base);
+    }
+    const uint32_t xs = g.x_stride[g.axis], os = g.o_stride[g.axis];
+    const uint32_t len = valid ? g.axis_len : 0U;
+    const float *xp = x + x_base;
+    float *op = out + o_base;
+    const float n = (float)g.axis_len;
+    // sum of f(element) over the thread's share of the row, U loads in flight
+    auto share = [&](auto f) {
+        float s = 0.0f;
+        for (uint32_t j0 = ty; j0 < len; j0 += NY * U) {
+            float v[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const uint32_t j = j0 + u * NY;
+                v[u] = j < len ? xp[(uint64_t)j * xs] : 0.0f;
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                s += (j0 + u * NY < len) ? f(v[u]) : 0.0f;
+            }
+        }
+        return s;
+    };
+    float mu = 0.0f;
+    if constexpr (LAYER) {
+        mu = row_sum<RT, THREADS>(share([](float v) { return v; }), red) / n;
+    }
+    const float mean_sq = row_sum<RT, THREADS>(share([mu](float v) { return (v - mu) * (v - mu); }), red) / n;
+    const float r = sqrtf(mean_sq + g.eps);
+    const uint32_t per = (g.axis_len + gridDim.y - 1) / gridDim.y;
+    const uint32_t j_end = min(len, (blockIdx.y + 1) * per);
+    for (uint32_t j = blockIdx.y * per + ty; j < j_end; j += NY) {
+        const float xc = xp[(uint64_t)j * xs] - mu;
+        float y = (xc / r) * w[(uint64_t)g.w_off + (uint64_t)j * g.w_stride];
+        if constexpr (LAYER) {
+            y = y + beta[(uint64_t)g.b_off + (uint64_t)j * g.b_stride];
+        }
+        op[(uint64_t)j * os] = y;
+    }
+}
+
 template <bool LAYER, int RT, int THREADS>
 void launch_cached(const float *x, const float *w, const float *b, float *out, const NormGeom &g, hipStream_t s)
 {
@@ -221,9 +279,14 @@ int norm_impl(const char *fn, uint32_t rank, const uint32_t *shape, uint32_t axi
         launch_cached<LAYER, 1, 256>(x_dev, w_dev, b_dev, out_dev, g, s);
     } else if (g.rows >= 32U * 512U) {
         launch_cached<LAYER, 32, 256>(x_dev, w_dev, b_dev, out_dev, g, s);
-    } else {
-        // few rows, strided axis (a decode step's activations): 16 neighbouring rows and 64 threads along the axis
+    } else if (x_dev == out_dev) {
+        // in place: the whole row must be summed before any of it is overwritten, so one workgroup does both
         launch_cached<LAYER, 16, 1024>(x_dev, w_dev, b_dev, out_dev, g, s);
+    } else {
+        // few rows, strided axis (a decode step's activations): see norm_sliced_kernel
+        const uint32_t row_tiles = (g.rows + 15U) / 16U;
+        const uint32_t slices = std::max(1U, std::min((128U + row_tiles - 1U) / row_tiles, (g.axis_len + 63U) / 64U));
+        norm_sliced_kernel<LAYER><<<dim3(row_tiles, slices), 1024, 0, s>>>(x_dev, w_dev, b_dev, out_dev, g);
     }
     WEED_HIP_LAUNCH_CHECK();
     return WEED_HIP_OK;
