@@ -339,6 +339,73 @@ def layer_decode_step(capi, torch, np, n_calls, n_seq=64, ctx=8192, d_model=4096
     return cache, step
 
 
+def plan_scan(capi, torch, steps=100, warmup=WARMUP_FLOOR_EXTRA):
+    """The decode planner's default plan against the plain three-kernel plan (query kernel, attention, merge) over a
+    grid of batch sizes, context lengths, group sizes and ragged batches: microseconds per call by two events around
+    `steps` back-to-back calls.  A record to check changes of the planner's thresholds against: `behind` lists the
+    shapes where the default is more than 3 us slower than three kernels."""
+    import random
+    flags = capi.ATTN_ROTATE_Q | capi.ATTN_UNROTATE_OUT
+    d = 128
+    rk, rv = torch.zeros(d * d, device="cuda"), torch.zeros(d * d, device="cuda")
+    capi.make_rotation(5, d, rk)
+    capi.make_rotation(6, d, rv)
+    shapes = []
+    for Hkv, Hq in ((8, 32), (2, 16)):
+        for S in (3, 12, 24, 50, 96, 200, 512):
+            for ctx in (100, 300, 1000, 2100, 5000):
+                shapes.append(("equal", Hkv, Hq, [ctx] * S))
+    for S in (1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128):
+        shapes.append(("equal", 8, 32, [8192] * S))
+    for ctx in (7744, 8000, 8129):
+        shapes.append(("equal", 8, 32, [ctx] * 64))
+    rnd = random.Random(17)
+    for S in (4, 16, 48, 64, 128):
+        shapes.append(("ragged 4096..8192", 8, 32, [rnd.randint(4096, 8192) for _ in range(S)]))
+        shapes.append(("ragged 512..8192", 8, 32, [rnd.randint(512, 8192) for _ in range(S)]))
+        shapes.append(("half 8192 half 1024", 8, 32, [8192 if i % 2 == 0 else 1024 for i in range(S)]))
+    rows, behind = [], []
+    for kind, Hkv, Hq, lens in shapes:
+        S = len(lens)
+        cache = capi.KVCache(capi.KV_LLOYDMAX, S, Hkv, d, max(lens), 3, 4, 0, 0)
+        cache.set_rotations(rk, rv)
+        if len(set(lens)) == 1:
+            K = torch.randn((min(S, 64), Hkv, lens[0], d), device="cuda")
+            for s0 in range(0, S, 64):
+                n = min(64, S - s0)
+                cache.encode_append(K[:n], K[:n], seq_begin=s0, rotate=1)
+        else:
+            K = torch.randn((1, Hkv, max(lens), d), device="cuda")
+            for s0, n in enumerate(lens):
+                cache.encode_append(K[:, :, :n], K[:, :, :n], seq_begin=s0, rotate=1)
+        del K
+        q = torch.randn((S, Hq, d), device="cuda")
+        out = torch.zeros_like(q)
+        us = []
+        kernels = None
+        for kw in ({}, dict(separate_merge=True, separate_query=True)):
+            capi.decode_tuning(**kw)
+            try:
+                if not kw:
+                    capi.profile_reset()
+                    capi.profile_enable(True)
+                    cache.decode_attn(q, out, capi.GQA_BLOCKED, flags)
+                    torch.cuda.synchronize()
+                    kernels = 1 if capi.profile_read("kv_decode_combine")[1] == 0 else 3
+                    capi.profile_enable(False)
+                us.append(1e6 * time_region(torch, lambda: cache.decode_attn(q, out, capi.GQA_BLOCKED, flags), steps, warmup))
+            finally:
+                capi.decode_tuning()
+        row = {"kind": kind, "n_seq": S, "kv_heads": Hkv, "q_heads": Hq,
+               "ctx": lens[0] if len(set(lens)) == 1 else [min(lens), max(lens)], "default_us": round(us[0], 2),
+               "default_kernels": kernels, "three_kernels_us": round(us[1], 2)}
+        rows.append(row)
+        if us[0] > us[1] + 3.0:
+            behind.append(row)
+        cache.close()
+    return {"plan_scan": rows, "behind_three_kernels_by_more_than_3us": behind, "steps": steps, "warmup": warmup}
+
+
 def extras(capi, torch, workloads, steps, warmup):
     """The other configurations, measured the same way (reported beside the headline, not as `value`)."""
     out = {}
@@ -365,7 +432,12 @@ def extras(capi, torch, workloads, steps, warmup):
         "roofline": {"bound": "hbm", "achieved": wbytes / kernel_s / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": wbytes / kernel_s / 1e9 / HBM_PEAK_GBS}}
     out["projection_8x4096x4096"].update(how)
-    del X, Wp, Y
+    sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+    read_s = time_region(torch, lambda: capi.read_sweep(Wp, wbytes, 0, sink), steps, warmup)
+    out["projection_8x4096x4096"]["roofline"]["streaming_read_ms"] = 1e3 * read_s
+    out["projection_8x4096x4096"]["roofline"]["streaming_read_what"] = (
+        "the library's read-only sweep over the same 64 MiB weight: what a launch that only reads the bytes takes")
+    del X, Wp, Y, sink
     # standalone softmax and sum over an [8192 x 16384] column-major matrix (512 MiB, twice the Infinity Cache, so
     # that back-to-back launches read from HBM), along the contiguous axis and along the strided one: 8 B per element
     # (softmax) and 4 B per element (sum) of algorithmic traffic.  Along the strided axis a column block of 32 rows
@@ -581,6 +653,9 @@ def main():
     ap.add_argument("--calibrate-read", action="store_true",
                     help="only launch the library's read-only sweeps over as many bytes as the headline step reads "
                          "(the practical ceiling of a read stream on this part), for a rocprofv3 kernel trace")
+    ap.add_argument("--plan-scan", action="store_true",
+                    help="only scan the decode planner: its default plan against three kernels over a grid of batch "
+                         "sizes, contexts, group sizes and ragged batches (about a minute)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="only launch the library's plain copy kernel on MIB mebibytes (5 launches): the known-size "
                          "reference against which rocprofv3's FETCH_SIZE / WRITE_SIZE readings are scaled")
@@ -607,6 +682,10 @@ def main():
                 capi.copy(src, dst)
             torch.cuda.synchronize()
         print(json.dumps({"calibrate_copy_bytes_read": 4 * n, "calibrate_copy_bytes_written": 4 * n, "launches": 5}))
+        return
+    if args.plan_scan:
+        with torch.cuda.stream(stream):
+            print(json.dumps(plan_scan(capi, torch)))
         return
     if args.calibrate_read:
         with torch.cuda.stream(stream):
