@@ -317,7 +317,9 @@ int weed_hip_kv_decode_attn(weed_hip_kv_cache *cache, int32_t n_q_heads, int32_t
  * device holds at once; skew_percent: how much longer than the mean the runs of a workgroup's oldest wavefronts are
  * (and the youngest shorter), negative = the built-in 16 (28 for kernel instances with three wavefronts per SIMD);
  * always_search: bit 0: find every run's first region by search even when all sequences have equal lengths;
- * bit 1: never let the matrix-core kernel merge its partials itself; bit 2: never let it rotate the queries itself
+ * bit 1: never let the matrix-core kernel merge its partials itself; bit 2: never let it rotate the queries itself;
+ * bit 3: every wavefront takes one contiguous piece of the cache (otherwise, in batches of equal sequences,
+ * neighbouring wavefronts take the blocks of their common piece in turns)
  * (when every workgroup's share of the launch is a whole number of (sequence, kv head) regions, or every region a
  * whole number of such shares, one kernel does the whole call: that is so for batches of 1 to 256 sequences whose
  * lengths are equal or not too different -- sequences are counted as having as many blocks as the longest while that

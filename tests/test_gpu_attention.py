@@ -227,8 +227,9 @@ def test_equal_contexts_with_and_without_the_region_search(gpu, oracle):
     want = checker_output(oracle, gpu, cache, wl, q, False)
     try:
         fast = run_decode(gpu, cache, q, gpu.GQA_BLOCKED, 0)
-        # (with the merge left to the second kernel on both sides: the kernel's own merge adds in another order)
-        gpu.decode_tuning(separate_merge=True)
+        # (with the merge left to the second kernel and one contiguous piece per wavefront on both sides: the kernel's
+        # own merge, and wavefronts that take their blocks in turns, add in another order)
+        gpu.decode_tuning(separate_merge=True, contiguous_runs=True)
         divided = run_decode(gpu, cache, q, gpu.GQA_BLOCKED, 0)
         gpu.decode_tuning(always_search=True)
         searched = run_decode(gpu, cache, q, gpu.GQA_BLOCKED, 0)
@@ -256,6 +257,12 @@ def test_equal_contexts_with_and_without_the_region_search(gpu, oracle):
     (True, 128, 1, 4, 1, 8192, 3, 4, 128, True),    # sixteen workgroups per region
     (True, 128, 2, 8, 2, 1536, 2, 2, 96, True),     # three wavefronts per SIMD
     (False, 64, 2, 16, 3, 1536, 4, 4, 144, False),  # uniform coder, head_dim 64, groups of 8, no rotations
+    # longer runs, which neighbouring wavefronts work through in turns
+    (True, 128, 2, 8, 4, 4096, 3, 4, 64, True),     # runs of 8 +- 1 blocks, all eight of a workgroup's region in turns
+    (True, 128, 2, 8, 2, 4096, 3, 4, 64, True),     # runs of 4 +- 1, two workgroups per region
+    (True, 128, 2, 8, 4, 2048, 3, 4, 16, True),     # runs of 16 +- 3, four regions of one cycle per workgroup
+    (True, 64, 2, 4, 2, 3072, 3, 4, 48, True),      # three age classes: runs of 5, 4 and 3, twelve in turns
+    (True, 64, 2, 4, 4, 1536, 3, 4, 48, True),      # three age classes, two regions per workgroup, six in turns
 ])
 def test_workgroups_that_merge_their_own_regions(gpu, oracle, lloyd, d, Hkv, Hq, S, L, kb, vb, waves, rot):
     """When every workgroup of the matrix-core kernel holds whole regions, or every region a whole number of
@@ -311,6 +318,32 @@ def test_workgroups_that_merge_their_own_regions(gpu, oracle, lloyd, d, Hkv, Hq,
     assert np.all(one_kernel_p[S // 2] == 0.0)
     # a second call gives the same bits (the order of every sum is fixed)
     assert np.array_equal(again, one_kernel)
+    cache.close()
+
+
+@pytest.mark.parametrize("d,Hkv,Hq,S,L,waves", [(128, 2, 8, 4, 4096, 64), (128, 2, 8, 2, 4096, 64), (64, 2, 4, 2, 3072, 48)])
+def test_runs_that_take_turns(gpu, oracle, d, Hkv, Hq, S, L, waves):
+    """In batches of equal sequences the wavefronts of neighbouring runs take the blocks of their common piece in turns
+    (each keeps its number of blocks); with one contiguous piece per wavefront instead, the call adds the same blocks
+    in another grouping: both agree with the checker, and they differ in the last bits (so the turns were taken)."""
+    rng = np.random.default_rng(59)
+    wl = workloads.Workload("turns", S, Hq, Hkv, d, [L] * S, 3, 4, 0, 0, 0)
+    K = rng.standard_normal((S, Hkv, L, d), dtype=np.float32)
+    V = rng.standard_normal((S, Hkv, L, d), dtype=np.float32)
+    q = rng.standard_normal((S, Hq, d), dtype=np.float32)
+    cache = build_cache(gpu, wl, gpu.KV_LLOYDMAX, K, V)
+    want = checker_output(oracle, gpu, cache, wl, q, False)
+    try:
+        gpu.decode_tuning(waves)
+        turns = run_decode(gpu, cache, q, gpu.GQA_BLOCKED, 0)
+        gpu.decode_tuning(waves, contiguous_runs=True)
+        pieces = run_decode(gpu, cache, q, gpu.GQA_BLOCKED, 0)
+    finally:
+        gpu.decode_tuning()
+    assert_attn_close(turns, want, "turns")
+    assert_attn_close(pieces, want, "contiguous pieces")
+    np.testing.assert_allclose(turns, pieces, rtol=2e-5, atol=2e-6)
+    assert not np.array_equal(turns, pieces)
     cache.close()
 
 

@@ -418,11 +418,13 @@ def shutdown():
     check(load().weed_hip_shutdown())
 
 
-def decode_tuning(wavefronts=0, skew_percent=-1, always_search=False, separate_merge=False, separate_query=False):
+def decode_tuning(wavefronts=0, skew_percent=-1, always_search=False, separate_merge=False, separate_query=False,
+                  contiguous_runs=False):
     """Work partition of the decode kernels (defaults: 0, -1, False); results do not depend on it beyond the
     rounding of the last bits.  separate_merge / separate_query: never let the matrix-core kernel merge its partials /
     rotate its queries itself."""
-    flags = int(bool(always_search)) | 2 * int(bool(separate_merge)) | 4 * int(bool(separate_query))
+    flags = (int(bool(always_search)) | 2 * int(bool(separate_merge)) | 4 * int(bool(separate_query)) |
+             8 * int(bool(contiguous_runs)))
     check(load().weed_hip_kv_decode_tuning(int(wavefronts), int(skew_percent), flags))
 
 

@@ -13,10 +13,17 @@ namespace weedhip {
 // Positions cycle through the classes (position p belongs to class p % classes, and is worked on by wavefront
 // (p % classes) * 4 + p / classes), so every group of `classes` consecutive runs spans classes * unit_blocks blocks:
 // regions whose boundaries fall on multiples of that (equal sequences, the common case) are never straddled by a run.
+// `group_cycles` > 0 (1, 2 or 4): the runs of that many consecutive cycles share their blocks in turns instead of
+// taking one contiguous piece each: the group's blocks go round the runs one by one (the runs of the oldest class
+// first) until the youngest class has its share, then round the remaining classes, and so on.  Each run keeps its
+// length, so the partition into regions, slots and workgroups is the same; what changes is that neighbouring
+// wavefronts read neighbouring blocks at about the same time.  Only for launches whose workgroups merge and in which
+// no group crosses a region boundary (equal sequences whose block count is a multiple of the group's).
 struct RunGeom {
-    uint32_t unit_blocks; // mean run length
-    uint32_t skew;        // < unit_blocks
-    uint32_t waves;       // wavefronts per workgroup: 8 or 12
+    uint32_t unit_blocks;  // mean run length
+    uint32_t skew;         // < unit_blocks
+    uint32_t waves;        // wavefronts per workgroup: 8 or 12
+    uint32_t group_cycles; // 0: every run is one contiguous piece
 };
 __host__ __device__ inline uint32_t run_classes(const RunGeom &rg) { return rg.waves / 4; } // 2 or 3
 __host__ __device__ inline uint32_t run_len(const RunGeom &rg, uint32_t age_class)
@@ -40,7 +47,8 @@ __host__ __device__ inline uint32_t run_begin(const RunGeom &rg, uint32_t P)
     }
     return b;
 }
-// Position index of the run that holds block b.
+// Position index of the run that holds block b (contiguous runs; with runs that take turns: the same for the first
+// block of a group).
 __host__ __device__ inline uint32_t run_of_block(const RunGeom &rg, uint32_t b)
 {
     const uint32_t classes = run_classes(rg);

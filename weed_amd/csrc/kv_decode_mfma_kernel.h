@@ -371,8 +371,25 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     // `unit`: position index of this wavefront's run (runs are numbered along the block list)
     const uint32_t unit =
         __builtin_amdgcn_readfirstlane(blockIdx.x * kWaves + run_position_of_wave(p.runs, wave));
-    uint32_t g0 = __builtin_amdgcn_readfirstlane(run_begin(p.runs, unit));
-    const uint32_t g1 = min(g0 + run_len(p.runs, (unit % kWaves) % run_classes(p.runs)), p.total_blocks);
+    // Runs that take turns (RunGeom::group_cycles; instances whose workgroups merge only): g0 .. g1 are then the blocks
+    // of the run's whole group, of which this wavefront takes its `turn_count` blocks -- one segment, since no group
+    // crosses a region boundary.  In turn i the runs that are still short of their length take one block each, ordered
+    // by (class, cycle); the youngest class drops out after u0 turns, the middle one (three classes) after u1.  Block
+    // number i of a run, counted from the group's first block, is therefore
+    // turn_at + turn_cycles * (i + min(i, u0) + min(i, u1))   (u1 = 0 with two classes).
+    constexpr uint32_t kClasses = kWaves / 4;
+    const uint32_t turn_cycles = WGM ? p.runs.group_cycles : 0u; // 0, 1, 2 or 4
+    const uint32_t wave_s = __builtin_amdgcn_readfirstlane(wave); // (the same in all lanes: block indices stay scalar)
+    const uint32_t age_class = wave_s >> 2, cycle_in_group = (wave_s & 3) & (turn_cycles - 1u);
+    const uint32_t turn_at = age_class * turn_cycles + cycle_in_group;
+    const uint32_t turn_count =
+        (uint32_t)((int)p.runs.unit_blocks + (int)p.runs.skew * ((int)kClasses - 1 - 2 * (int)age_class) / ((int)kClasses - 1));
+    const uint32_t turn_u0 = p.runs.unit_blocks - p.runs.skew, turn_u1 = kClasses == 3 ? p.runs.unit_blocks : 0u;
+    uint32_t g0 = __builtin_amdgcn_readfirstlane(
+        turn_cycles ? (unit - (cycle_in_group * kClasses + age_class)) * p.runs.unit_blocks : run_begin(p.runs, unit));
+    const uint32_t g1 = min(g0 + (turn_cycles ? turn_cycles * kClasses * p.runs.unit_blocks
+                                              : run_len(p.runs, (unit % kWaves) % run_classes(p.runs))),
+                            p.total_blocks);
     // ---- merge inside the kernel (see MfmaMerge): LDS behind the tables, and this thread's share of the rotation ----
     static_assert(!WGM || mfma_decode_merges(GP, D), "this instance cannot merge");
     constexpr bool kCanMerge = mfma_decode_merges(GP, D);
@@ -700,7 +717,11 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     // (A partition that counts more blocks per region than the cache holds may put b0 behind the region's memory:
     // such a segment has no tokens and what is read for it is not used, but it is read from inside the region.)
     constexpr std::integral_constant<int, 0> p0{};
-    const uint32_t first_read = min(b0, (p.padded >> 6) - 1u);
+    // block number i of this wavefront in the segment (an index into the region); ~0 behind its last one
+    auto nth_block = [&](uint32_t i) -> uint32_t {
+        return i < turn_count ? b0 + turn_at + turn_cycles * (i + min(i, turn_u0) + min(i, turn_u1)) : ~0u;
+    };
+    const uint32_t first_read = min(turn_cycles ? b0 + turn_at : b0, (p.padded >> 6) - 1u);
     load_k(p0, first_read);
     load_v(p0, first_read);
 
@@ -1023,7 +1044,8 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
 
     // ---- main loop.  The refills are unconditional (the next block index is clamped to the last block of the
     //      segment) so that the loop body has no branch around loads and outstanding loads can be counted exactly. ----
-    {
+    if (!WGM || turn_cycles == 0) {
+        // contiguous runs
         uint32_t blk = b0;
         if (blk < b1) {
             const uint32_t last = b1 - 1;
@@ -1040,6 +1062,30 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
                 for (; blk < b1; ++blk) {
                     process_block(p0, blk, min(blk + 1, last));
                 }
+            }
+        }
+    } else {
+        // runs that take turns (the wavefront's blocks ascend, so the first one at or behind b1 ends the segment)
+        uint32_t i = 0, blk = nth_block(0);
+        const uint32_t last = b1 - 1; // (only used while blk < b1, so b1 >= 1)
+        if constexpr (NB == 2) {
+            constexpr std::integral_constant<int, 1> p1{};
+            while (blk < b1) {
+                const uint32_t second = nth_block(i + 1);
+                process_block(p0, blk, min(second, last));
+                if (second >= b1) {
+                    break;
+                }
+                const uint32_t third = nth_block(i + 2);
+                process_block(p1, second, min(third, last));
+                blk = third;
+                i += 2;
+            }
+        } else {
+            while (blk < b1) {
+                const uint32_t next = nth_block(++i);
+                process_block(p0, blk, min(next, last));
+                blk = next;
             }
         }
     }
