@@ -264,7 +264,7 @@ def streaming_read(capi, torch, nbytes, steps, warmup):
     return {"bytes": nbytes, "per_wavefront_runs_ms": 1e3 * runs_s, "per_wavefront_runs_gbs": nbytes / runs_s / 1e9,
             "plain_sweep_ms": 1e3 * sweep_s, "plain_sweep_gbs": nbytes / sweep_s / 1e9, "launches": steps,
             "kernel": "weed_hip_read_sweep: 16-byte loads, nothing written; 256 workgroups x 8 wavefronts with one "
-                      "contiguous run each (the decode kernel's shape), and a grid-stride sweep"}
+                      "contiguous run each (the decode kernel's shape), and the same wavefronts taking the 8 KB units in turns"}
 
 
 def layer_decode_step(capi, torch, np, n_calls, n_seq=64, ctx=8192, d_model=4096, n_heads=32, n_kv=8, d_ff=14336):

@@ -114,10 +114,11 @@ int weed_hip_copy_f32(uint64_t n, const float *a_dev, uint32_t a_off, uint32_t a
                       uint32_t o_stride);
 
 /* Calibration, no counterpart in the reference: read `bytes` of device memory once with 16-byte loads and write
- * nothing.  per_wavefront_runs = 0: a plain sweep (consecutive workgroups read consecutive pieces); 1: the decode
- * kernel's launch shape -- 256 workgroups of 8 wavefronts, every wavefront walks one contiguous run in 8 KB units with
- * the next unit in flight (a tail below 8 KB is not read).  The time of such a launch is what merely reading the
- * bytes of a decode step costs on this part.  sink_dev: one word that is (practically) never written. */
+ * nothing, by 256 workgroups of 8 wavefronts in units of 8 KB with the next unit in flight (a tail below 8 KB is not
+ * read).  per_wavefront_runs = 1: every wavefront walks one contiguous run, the decode kernel's launch shape; 0: the
+ * device's wavefronts take the units in turns, so that the device reads one contiguous stretch at any moment.  The
+ * time of such a launch is what merely reading the bytes of a decode step costs on this part.  sink_dev: one word that
+ * is (practically) never written. */
 int weed_hip_read_sweep(const void *src_dev, uint64_t bytes, int per_wavefront_runs, uint32_t *sink_dev);
 
 /* Broadcasting elementwise ops on tensors of one logical shape (rank <= 8, strides in elements, stride 0 repeats a

@@ -508,33 +508,20 @@ __global__ void __launch_bounds__(256) copy_kernel(const float *__restrict__ a, 
 // 16 bytes per load; the xor of everything read is stored only if it equals a value it cannot be expected to have, so
 // the reads cannot be optimised away and nothing is written.
 typedef uint32_t sweep_u4 __attribute__((ext_vector_type(4)));
-// plain sweep: consecutive workgroups read consecutive 4 KB pieces, grid-stride
-__global__ void __launch_bounds__(256) read_sweep_kernel(const sweep_u4 *__restrict__ src, uint64_t n_vec, uint32_t *sink)
-{
-    sweep_u4 acc = { 0, 0, 0, 0 };
-    const uint64_t step = (uint64_t)gridDim.x * blockDim.x;
-    uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    for (; i + 3 * step < n_vec; i += 4 * step) {
-        const sweep_u4 a = src[i], b = src[i + step], c = src[i + 2 * step], d = src[i + 3 * step];
-        acc ^= a ^ b ^ c ^ d;
-    }
-    for (; i < n_vec; i += step) {
-        acc ^= src[i];
-    }
-    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u) {
-        sink[0] = acc.x;
-    }
-}
-// The decode kernel's launch shape: one workgroup of 8 wavefronts per compute unit, every wavefront walks ONE
-// contiguous run of the buffer in units of 8 KB (eight 16-byte loads per lane), the next unit requested before the
-// current one is consumed.
+// The decode kernel's launch shape: one workgroup of 8 wavefronts per compute unit; a wavefront reads units of 8 KB
+// (eight 16-byte loads per lane), the next unit requested before the current one is consumed.  RUNS: every wavefront
+// walks ONE contiguous run of the buffer, as the decode kernel's wavefronts do; otherwise the wavefronts of the device
+// take the units in turns (unit u goes to wavefront u mod 2048), so that at any moment the device reads one
+// contiguous stretch of the buffer -- the fastest order found for this part.
 constexpr uint32_t kRunUnitVecs = 512; // 16-byte vectors per unit
+template <bool RUNS>
 __global__ void __launch_bounds__(512) read_runs_kernel(const sweep_u4 *__restrict__ src, uint64_t n_units,
                                                         uint32_t units_per_run, uint32_t *sink)
 {
     const uint32_t lane = threadIdx.x & 63, run = blockIdx.x * 8 + (threadIdx.x >> 6);
-    const uint64_t u0 = (uint64_t)run * units_per_run;
-    const uint64_t u1 = u0 + units_per_run < n_units ? u0 + units_per_run : n_units;
+    const uint64_t stride = RUNS ? 1u : gridDim.x * 8u;
+    const uint64_t u0 = RUNS ? (uint64_t)run * units_per_run : run;
+    const uint64_t u1 = RUNS ? (u0 + units_per_run < n_units ? u0 + units_per_run : n_units) : n_units;
     sweep_u4 acc = { 0, 0, 0, 0 };
     if (u0 < u1) {
         sweep_u4 cur[8], nxt[8];
@@ -543,8 +530,8 @@ __global__ void __launch_bounds__(512) read_runs_kernel(const sweep_u4 *__restri
         for (int k = 0; k < 8; ++k) {
             cur[k] = p[64 * k];
         }
-        for (uint64_t u = u0; u < u1; ++u) {
-            const sweep_u4 *q = src + (u + 1 < u1 ? u + 1 : u) * kRunUnitVecs + lane;
+        for (uint64_t u = u0; u < u1; u += stride) {
+            const sweep_u4 *q = src + (u + stride < u1 ? u + stride : u) * kRunUnitVecs + lane;
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
                 nxt[k] = q[64 * k];
@@ -819,21 +806,16 @@ int weed_hip_read_sweep(const void *src_dev, uint64_t bytes, int per_wavefront_r
     WEED_HIP_REQUIRE(reinterpret_cast<uintptr_t>(src_dev) % 16U == 0U, "%s: the buffer must be 16-byte aligned", fn);
     WEED_HIP_TRY(ensure_init());
     ProfileScope prof("read_sweep");
-    if (per_wavefront_runs) {
-        const uint64_t n_units = bytes / (16ull * kRunUnitVecs); // (a tail below one unit is not read)
-        const uint32_t runs = 256u * 8u;
-        const uint64_t per = (n_units + runs - 1) / runs;
-        WEED_HIP_REQUIRE(per < (1ull << 32), "%s: buffer too large", fn);
-        if (n_units) {
-            read_runs_kernel<<<256, 512, 0, stream()>>>(static_cast<const sweep_u4 *>(src_dev), n_units, (uint32_t)per,
-                                                        sink_dev);
-        }
-    } else {
-        const uint64_t n_vec = bytes / 16ull;
-        if (n_vec) {
-            const uint32_t blocks = (uint32_t)std::min<uint64_t>((n_vec + 255) / 256, 256u * 16u);
-            read_sweep_kernel<<<blocks, 256, 0, stream()>>>(static_cast<const sweep_u4 *>(src_dev), n_vec, sink_dev);
-        }
+    const uint64_t n_units = bytes / (16ull * kRunUnitVecs); // (a tail below one unit is not read)
+    const uint32_t runs = 256u * 8u;
+    const uint64_t per = (n_units + runs - 1) / runs;
+    WEED_HIP_REQUIRE(per < (1ull << 32), "%s: buffer too large", fn);
+    if (n_units && per_wavefront_runs) {
+        read_runs_kernel<true><<<256, 512, 0, stream()>>>(static_cast<const sweep_u4 *>(src_dev), n_units, (uint32_t)per,
+                                                          sink_dev);
+    } else if (n_units) {
+        read_runs_kernel<false><<<256, 512, 0, stream()>>>(static_cast<const sweep_u4 *>(src_dev), n_units, (uint32_t)per,
+                                                           sink_dev);
     }
     WEED_HIP_LAUNCH_CHECK();
     return WEED_HIP_OK;
