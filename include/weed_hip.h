@@ -74,7 +74,8 @@ int weed_hip_memcpy_d2d(void *dst_dev, const void *src_dev, size_t bytes);
  * point brackets its dominant kernel with events; weed_hip_profile_read returns the accumulated time. */
 int weed_hip_profile_enable(int on);
 int weed_hip_profile_reset(void);
-/* name: "kv_decode_attn", "kv_decode_combine", "kv_encode", "kv_pack", "matmul", "softmax", "reduce" */
+/* name: "kv_decode_attn", "kv_decode_combine", "kv_encode", "kv_pack", "matmul", "softmax", "reduce", "elementwise",
+ * "copy", "rope", "rms_norm", "layer_norm", "read_sweep" */
 int weed_hip_profile_read(const char *name, double *total_ms, uint64_t *launches);
 
 /* ------------------------------------------------------------------------------------------------ */
