@@ -456,6 +456,7 @@ constexpr int kWideWaves = 8;
 constexpr int kWidePitchH = 72; // halves per staged row: 64 k + 8 of padding
 
 typedef uint32_t uint4w __attribute__((ext_vector_type(4)));
+typedef uint32_t uint2w __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
 // w = p1 + p2 + p3 exactly, every part a bfloat16 (the upper halves of the returned words): the top 8 bits of the
@@ -507,16 +508,22 @@ __global__ void __launch_bounds__(64 * kWideWaves)
     for (int mt = 0; mt < MT; ++mt) {
         acc[mt] = float4v{ 0.0f, 0.0f, 0.0f, 0.0f };
     }
-    // this lane's sixteen consecutive k of its column, kb + 16 grp .., zero beyond the range (K is a multiple of 4)
+    // Sixteen k of this lane's column per 64-k step, zero beyond the range (K is a multiple of 4): load q takes
+    // kb + 16 q + 4 grp .. + 3, so that the four lanes of a column read 64 consecutive bytes per instruction and every
+    // cache line a load touches is used up by that load (with the lane's sixteen k consecutive, each of the four
+    // loads touched every line of the step, and the lines had to survive in the first-level cache between them).
     auto load_w = [&](uint32_t kb, float4v (&w)[4]) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            const uint32_t k = kb + 16 * grp + 4 * q;
+            const uint32_t k = kb + 16 * q + 4 * grp;
             w[q] = (n_ok && k < kb1) ? *reinterpret_cast<const float4v *>(wcol + k) : float4v{ 0.0f, 0.0f, 0.0f, 0.0f };
         }
     };
     // the rows of a for one 64-k step: thread (row = tid % (16 MT), octet = tid / (16 MT)) fetches a[row][kb + 8 octet
-    // .. + 7], splits the eight values and stores one 16-byte piece per part
+    // .. + 7], splits the eight values and stores two 8-byte pieces per part.  A row lies in LDS in the order in which
+    // the matrix instructions contract: instruction j of a step contracts, in lane group grp, over the k
+    // 32 j + 4 grp .. + 3 and 32 j + 16 + 4 grp .. + 3 (what the lane's loads 2 j and 2 j + 1 of b hold), so k =
+    // 32 j + 16 h + 4 grp + e sits at position 32 j + 8 grp + 4 h + e and a lane's eight values are one 16-byte read.
     constexpr uint32_t kRows = 16 * MT;
     const uint32_t srow = tid % kRows, soct = tid / kRows;
     const bool stager = soct < 8;
@@ -532,9 +539,12 @@ __global__ void __launch_bounds__(64 * kWideWaves)
         if (stager) {
             uint4w part3[3];
             split_eight(v, part3);
+            // the thread's k = 8 soct + e': j = soct / 4, h = (soct % 4) / 2, grp = 2 (soct % 2) + e' / 4
+            const uint32_t at = 32 * (soct / 4) + 16 * (soct % 2) + 4 * ((soct % 4) / 2);
 #pragma unroll
             for (int pl = 0; pl < 3; ++pl) {
-                *reinterpret_cast<uint4w *>(&xs[buf][pl][srow][8 * soct]) = part3[pl];
+                *reinterpret_cast<uint2w *>(&xs[buf][pl][srow][at]) = uint2w{ part3[pl][0], part3[pl][1] };
+                *reinterpret_cast<uint2w *>(&xs[buf][pl][srow][at + 8]) = uint2w{ part3[pl][2], part3[pl][3] };
             }
         }
     };
@@ -553,9 +563,11 @@ __global__ void __launch_bounds__(64 * kWideWaves)
     auto iterate = [&](auto pc, auto xc, uint32_t kb) {
         constexpr int P = decltype(pc)::value; // register set of this step
         constexpr int X = decltype(xc)::value; // LDS buffer of this step
-        load_w(kb + 64 * (kDepth - 1), w[(P + kDepth - 1) % kDepth]);
+        // (the rows first: loads return in order, so waiting for the rows at the end of the step must not mean waiting
+        // for the columns requested behind them, which are not needed before a later step)
         fetch_rows(kb + 64, stage); // lands in registers while this step is multiplied
-        // the two halves of this lane's sixteen k: instruction j contracts over { kb + 16 grp + 8 j .. + 7 : grp }
+        load_w(kb + 64 * (kDepth - 1), w[(P + kDepth - 1) % kDepth]);
+        // the two halves of this lane's sixteen k: instruction j contracts over what the loads 2 j and 2 j + 1 hold
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const float v[8] = { w[P][2 * j][0], w[P][2 * j][1], w[P][2 * j][2], w[P][2 * j][3],
@@ -570,7 +582,7 @@ __global__ void __launch_bounds__(64 * kWideWaves)
 #pragma unroll
                 for (int pl = 0; pl < 3; ++pl) {
                     A[pl] = __builtin_bit_cast(
-                        bf16x8, *reinterpret_cast<const uint4w *>(&xs[X][pl][16 * mt + c][16 * grp + 8 * j]));
+                        bf16x8, *reinterpret_cast<const uint4w *>(&xs[X][pl][16 * mt + c][32 * j + 8 * grp]));
                 }
                 // the small terms first
                 acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A[2], B0, acc[mt], 0, 0, 0);
