@@ -437,7 +437,39 @@ def extras(capi, torch, workloads, steps, warmup):
     out["projection_8x4096x4096"]["roofline"]["streaming_read_ms"] = 1e3 * read_s
     out["projection_8x4096x4096"]["roofline"]["streaming_read_what"] = (
         "the library's read-only sweep over the same 64 MiB weight: what a launch that only reads the bytes takes")
-    del X, Wp, Y, sink
+    # The same product over six weights in turn (384 MiB, more than the 256 MB Infinity Cache holds): back-to-back
+    # calls on ONE 64 MiB weight are served in part by that cache; a model's step reads every weight once.
+    Wr = [Wp] + [(torch.randn((4096, 4096), device="cuda") * 0.02).t() for _ in range(5)]
+    turn = [0]
+
+    def in_turn():
+        capi.matmul(X, Wr[turn[0] % 6], Y)
+        turn[0] += 1
+    rot_s = time_region(torch, in_turn, steps, warmup)
+    out["projection_8x4096x4096"]["six_weights_in_turn"] = {
+        "kernel_ms": 1e3 * rot_s, "gbs": wbytes / rot_s / 1e9, "frac": wbytes / rot_s / 1e9 / HBM_PEAK_GBS,
+        "what": "the same call over six different weights in turn, so that every call reads its weight from HBM"}
+    del X, Wr, Wp, Y, sink
+    # 64 rows (a decode step of 64 sequences) against [4096 x 14336] weights (235 MB each), four in turn: the
+    # matrix-core kernel for 17 to 64 rows (bfloat16 products of exactly split operands) and the kernel that adds its
+    # k ranges, two launches per call
+    X = torch.randn((4096, 64), device="cuda").t()               # logical [64, 4096], column-major
+    Wg = [(torch.randn((14336, 4096), device="cuda") * 0.02).t() for _ in range(4)]  # logical [4096, 14336], column-major
+    Y = torch.empty((14336, 64), device="cuda").t()
+    turn[0] = 0
+
+    def wide_in_turn():
+        capi.matmul(X, Wg[turn[0] % 4], Y)
+        turn[0] += 1
+    wide_s = time_region(torch, wide_in_turn, steps, warmup)
+    wide_bytes = 4096 * 14336 * 4
+    out["projection_64x4096x14336"] = {
+        "ms": 1e3 * wide_s, "launches_per_call": 2,
+        "roofline": {"bound": "hbm", "achieved": wide_bytes / wide_s / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": wide_bytes / wide_s / 1e9 / HBM_PEAK_GBS},
+        "what": "64 rows, four weights in turn (0.94 GB); the time is the whole call: the product's kernel and the sum "
+                "over its k ranges"}
+    del X, Wg, Y
     # standalone softmax and sum over an [8192 x 16384] column-major matrix (512 MiB, twice the Infinity Cache, so
     # that back-to-back launches read from HBM), along the contiguous axis and along the strided one: 8 B per element
     # (softmax) and 4 B per element (sum) of algorithmic traffic.  Along the strided axis a column block of 32 rows
