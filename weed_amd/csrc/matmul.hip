@@ -445,13 +445,18 @@ __global__ void __launch_bounds__(64 * kSkinnyWaves)
 //      of `a`, which the workgroup splits step by step into LDS ([part][row][k], rows padded to 144 bytes so that
 //      sixteen rows' 16-byte reads cover all banks once; two buffers, one barrier per 64-k step); the k ranges are
 //      split over gridDim.y workgroups whose partial results a small kernel behind adds up in a fixed order.
-//      64 rows: 4096 x 4096 weights 39 -> 33 us per product, 4096 x 14336 125 -> 76 us, 14336 x 4096 105 -> 72 us.
-//      What bounds it now is the SIMDs' issue slots: per 32 KB of b a compute unit issues 384 matrix instructions,
-//      ~1500 vector instructions (the splits) and 192 16-byte LDS reads, and the three kinds add up rather than
-//      overlap (every piece switched off in turn: the loads and splits alone run at 4.8 TB/s, the whole at 3.3).
+//      64 rows, back to back on one weight (which the 256 MB memory-side cache then holds in part): 4096 x 4096
+//      weights 39 -> 33 us per product, 4096 x 14336 125 -> 76 us, 14336 x 4096 105 -> 72 us.  Over four 4096 x 14336
+//      weights in turn, so that every product reads HBM: 94 us, then 82 with the two changes noted at load_w and
+//      in iterate() below (whole cache lines per load instruction; the rows requested ahead of the columns).
+//      Counters: matrix pipe 27 % busy, vector issue 41 % (the splits), LDS 34 %, wavefronts waiting for memory 35 %
+//      of their time: nothing is saturated, the phases of a step follow each other in every wavefront.
 //      Measured and dropped: the rows split once by a kernel ahead and copied into LDS as an image (more L2 traffic
 //      than the fp32 rows: 84 us), two column tiles per wavefront (72 us), sixteen wavefronts per workgroup (78 us),
-//      four wavefronts per workgroup (73 us), three to six register sets of b instead of two (98 us).
+//      four wavefronts per workgroup (73 us), three or four register sets of b instead of two (86 and 101 us against
+//      82), 224 to 896 workgroups instead of about 448 (87 to 94 us), the sum over the k ranges by the last
+//      workgroup of a column tile instead of a kernel behind (32 workgroups then read 458 KB each at the very end:
+//      a layer's seven products 416 -> 731 us).
 constexpr int kWideWaves = 8;
 constexpr int kWidePitchH = 72; // halves per staged row: 64 k + 8 of padding
 
