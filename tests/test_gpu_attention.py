@@ -263,6 +263,11 @@ def test_equal_contexts_with_and_without_the_region_search(gpu, oracle):
     (True, 128, 2, 8, 4, 2048, 3, 4, 16, True),     # runs of 16 +- 3, four regions of one cycle per workgroup
     (True, 64, 2, 4, 2, 3072, 3, 4, 48, True),      # three age classes: runs of 5, 4 and 3, twelve in turns
     (True, 64, 2, 4, 4, 1536, 3, 4, 48, True),      # three age classes, two regions per workgroup, six in turns
+    # head_dim 96 (and 80, which is stored as 96): a workgroup's 768 threads are eight rows of 96
+    (True, 96, 2, 8, 4, 768, 3, 4, 48, True),       # two regions per workgroup
+    (True, 96, 2, 16, 4, 1536, 4, 4, 96, False),    # groups of 8, one region per workgroup, no rotations
+    (True, 80, 2, 8, 4, 768, 3, 4, 48, True),       # head_dim 80
+    (False, 96, 1, 4, 8, 768, 4, 4, 96, True),      # uniform coder, four regions per workgroup
 ])
 def test_workgroups_that_merge_their_own_regions(gpu, oracle, lloyd, d, Hkv, Hq, S, L, kb, vb, waves, rot):
     """When every workgroup of the matrix-core kernel holds whole regions, or every region a whole number of
@@ -358,8 +363,9 @@ def test_block_counts_that_no_run_length_divides(gpu, oracle, cap_blocks, top, s
     behind the cache's memory and is never read.  The third case mixes sequences of 23 and 24
     blocks, which are counted alike.  Three cases are small batches, where a region is several workgroups' shares
     and the count is rounded to a whole number of those; in the last of them the sequences hold 8000, 5500 and 3000
-    tokens and are all counted as 128 blocks, so whole workgroups find no tokens in their share.  The head_dims 256
-    and 96 have no instance that merges its partials itself: the same partitions, three kernels per call.  All must
+    tokens and are all counted as 128 blocks, so whole workgroups find no tokens in their share.  Head_dim 256
+    has no instance that merges its partials itself: the same partition, three kernels per call; head_dim 96 merges
+    whole regions like 128 (its workgroups of twelve wavefronts are eight rows of 96 threads).  All must
     agree with the checker, with the three-kernel way, under prefix lengths (zero among them), and after a step's
     one-token append."""
     import torch
@@ -395,7 +401,7 @@ def test_block_counts_that_no_run_length_divides(gpu, oracle, cap_blocks, top, s
         gpu.sync()
         got_p = out.cpu().numpy()
         assert gpu.profile_read("kv_decode_attn")[1] == 3
-        assert gpu.profile_read("kv_decode_combine")[1] == (0 if d == 128 else 3)
+        assert gpu.profile_read("kv_decode_combine")[1] == (0 if d in (128, 96) else 3)
         gpu.decode_tuning(separate_merge=True, separate_query=True)
         three_kernels = run_decode(gpu, cache, q, gpu.GQA_BLOCKED, flags)
     finally:

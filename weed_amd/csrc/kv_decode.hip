@@ -1051,7 +1051,7 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         const uint32_t gp = pass_heads <= 4 ? 4u : (pass_heads <= 8 ? 8u : 16u);
         const uint32_t nb = uniform_blocks, cycle = run_classes(runs) * runs.unit_blocks;
         const uint32_t wg_blocks = runs.waves * runs.unit_blocks;
-        if (mfma_decode_merges(gp, d) && nb != 0 && nb % cycle == 0 && wg_blocks % nb == 0 &&
+        if (mfma_decode_merges_whole_regions(gp, d, runs.waves) && nb != 0 && nb % cycle == 0 && wg_blocks % nb == 0 &&
             !tune.separate_merge) {
             wg_regions = wg_blocks / nb;
         } else if (mfma_decode_merges(gp, d) && nb != 0 && nb % wg_blocks == 0 && nb / wg_blocks >= 2 &&
@@ -1105,7 +1105,7 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         }
         // A workgroup rotates the queries of the regions its blocks lie in itself when they are few enough for its
         // LDS (equal sequences, or the ragged batches above); nothing then runs ahead of the matrix-core kernel.
-        fused_query = mfma_decode_merges(gp, d) && (nb != 0 || general_merge) &&
+        fused_query = (wg_regions != 0 || mfma_decode_merges(gp, d)) && (nb != 0 || general_merge) &&
                       wg_most_regions * pass_heads <= kMfmaQueryRows && !tune.separate_query;
     }
     // Workgroups that merge whole regions or whole shares of a region: neighbouring runs take their blocks in turns

@@ -167,6 +167,13 @@ constexpr uint32_t kMfmaQueryRows = 32;
 
 // Instances that can merge: head_dim 64 or 128.
 constexpr bool mfma_decode_merges(uint32_t gp, uint32_t d) { return gp <= 16 && (d == 64u || d == 128u); }
+// Instances whose workgroups can merge WHOLE regions in LDS and rotate their queries (MfmaMerge::wg_regions; not the
+// merges through memory, in which a wavefront works on one row at a time): the above, and head_dim 96 where a
+// workgroup has twelve wavefronts, so that its 768 threads are eight rows of 96.  (`waves`: mfma_decode_waves_per_wg.)
+constexpr bool mfma_decode_merges_whole_regions(uint32_t gp, uint32_t d, uint32_t waves)
+{
+    return mfma_decode_merges(gp, d) || (gp <= 16 && d == 96u && waves == 12u);
+}
 // Rows (region, head) that one pass of the merge or of the query rotation takes (the matrix instruction behind both
 // has 16 rows, so a pass reads 8 rows beyond its own), and the LDS of both behind the lookup tables, in words.
 // Rows are staged for the matrix instruction with a pitch of d + 4 words.

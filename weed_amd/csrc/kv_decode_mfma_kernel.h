@@ -391,9 +391,11 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
                                               : run_len(p.runs, (unit % kWaves) % run_classes(p.runs))),
                             p.total_blocks);
     // ---- merge inside the kernel (see MfmaMerge): LDS behind the tables, and this thread's share of the rotation ----
-    static_assert(!WGM || mfma_decode_merges(GP, D), "this instance cannot merge");
-    constexpr bool kCanMerge = mfma_decode_merges(GP, D);
-    constexpr bool kQuery = mfma_decode_merges(GP, D);   // this instance can rotate its queries itself (MfmaQuery)
+    static_assert(!WGM || mfma_decode_merges_whole_regions(GP, D, kWaves), "this instance cannot merge");
+    constexpr bool kCanMerge = WGM ? mfma_decode_merges_whole_regions(GP, D, kWaves) : mfma_decode_merges(GP, D);
+    constexpr bool kQuery = kCanMerge;   // this instance can rotate its queries itself (MfmaQuery)
+    // (head_dim 96: a wavefront's 64 threads are not all in one row; what is a scalar elsewhere is per thread there)
+    constexpr bool kRowPerWave = D % 64 == 0;
     float *const part_s = reinterpret_cast<float *>(lds) + ROWS * (kTableRowBytes / 4); // [position][GP][D + 2]
     // The two small rotations (queries ahead of the loop, merged rows behind it) run on the fp32 matrix instruction
     // v_mfma_f32_16x16x4f32: wavefront w < D / 16 owns the output columns [16 w, 16 w + 16) of up to 16 rows.  Step s of
@@ -534,8 +536,8 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
             const uint32_t n_regions = p.n_seq * p.Hkv;
             // element e = tid + i * kThreads of the rows: its row is the same in all lanes of a wavefront (kThreads is
             // a multiple of D), so the row's address arithmetic is scalar
-            static_assert(kThreads % D == 0 && D % 64 == 0, "a wavefront stays inside one row");
-            const uint32_t row_of_wave = __builtin_amdgcn_readfirstlane(tid / D), j = tid % D;
+            static_assert(kThreads % D == 0, "the workgroup's threads are whole rows");
+            const uint32_t row_of_wave = kRowPerWave ? __builtin_amdgcn_readfirstlane(tid / D) : tid / D, j = tid % D;
 #pragma unroll
             for (uint32_t i = 0; i < QPT; ++i) {
                 const uint32_t row = row_of_wave + i * (kThreads / D);
@@ -587,15 +589,17 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
                 }
                 if (wave < kMfmaMergeRows && r0 + wave < wg_rows) {
                     const uint32_t row = r0 + wave;
-                    constexpr uint32_t CPL = D / 64;
+                    constexpr uint32_t CPL = (D + 63) / 64;
                     float a[CPL];
                     const float k = 1.4426950408889634f / sqrtf((float)p.merge.d_real);
                     float mx = 0.0f, sum = 0.0f;
 #pragma unroll
                     for (uint32_t cc = 0; cc < CPL; ++cc) {
                         const uint32_t j = lane + 64 * cc;
-                        float v;
-                        v = p.query.rotate ? qrot_s[wave * D + j] : qraw_s[staged_at(row, j)];
+                        float v = 0.0f;
+                        if (D % 64 == 0 || j < D) {
+                            v = p.query.rotate ? qrot_s[wave * D + j] : qraw_s[staged_at(row, j)];
+                        }
                         a[cc] = v;
                         const float qc = v * k;
                         mx = fmaxf(mx, fabsf(qc));
@@ -613,8 +617,10 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
                         const float qn = a[cc] * k * inv;
                         const _Float16 hi = (_Float16)qn;
                         const _Float16 lo = (_Float16)(qn - (float)hi);
-                        qh_s[row * D + j] = __builtin_bit_cast(uint16_t, hi);
-                        ql_s[row * D + j] = __builtin_bit_cast(uint16_t, lo);
+                        if (D % 64 == 0 || j < D) {
+                            qh_s[row * D + j] = __builtin_bit_cast(uint16_t, hi);
+                            ql_s[row * D + j] = __builtin_bit_cast(uint16_t, lo);
+                        }
                     }
                     if (lane == 0) {
                         qscale_s[row] = ldexpf(1.0f, e);
@@ -1169,7 +1175,7 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
         unsigned long long *const rowbase_s = reinterpret_cast<unsigned long long *>(o_s + 16 * RPITCH);
         const uint32_t n_regions = p.n_seq * p.Hkv;
         // (the row of an element is the same in all lanes of a wavefront: kThreads is a multiple of D)
-        const uint32_t rr_of_wave = __builtin_amdgcn_readfirstlane(tid / D), col = tid % D;
+        const uint32_t rr_of_wave = kRowPerWave ? __builtin_amdgcn_readfirstlane(tid / D) : tid / D, col = tid % D;
         // rows r0 .. r0 + RP - 1 of the workgroup (row = region index in the workgroup * G + head slot): o_s = the
         // merge of the row's `slots` partials, which partial(ri, hs, k) finds; normalised, or with NORMALISE false
         // left as the partial (m, l, o) that leave(rr, m, l, o) puts somewhere
@@ -1434,12 +1440,13 @@ template <int D, int WK, int WV, int GP, bool LLOYD> int launch_gp(const MfmaPar
 {
     constexpr uint32_t waves = mfma_decode_waves_per_wg(GP, D, WK, WV);
     constexpr size_t smem = (size_t)table_rows<WK, WV>() * kTableRowBytes;
-    constexpr size_t smem_merging = smem + (mfma_decode_merges(GP, D) ? mfma_merge_lds_bytes(waves, GP, D) : 0u);
+    constexpr size_t smem_merging =
+        smem + (mfma_decode_merges_whole_regions(GP, D, waves) ? mfma_merge_lds_bytes(waves, GP, D) : 0u);
     static_assert(smem_merging <= 160u * 1024u, "tables and merge area exceed a compute unit's LDS");
     // once per instance and process, whichever host thread gets here first (the others wait for it)
     static std::once_flag configured;
     static hipError_t config_status = hipSuccess;
-    constexpr bool kMerges = mfma_decode_merges(GP, D);
+    constexpr bool kMerges = mfma_decode_merges_whole_regions(GP, D, waves);
     std::call_once(configured, [] {
         config_status = hipFuncSetAttribute((const void *)decode_mfma_kernel<D, WK, WV, GP, LLOYD, false>,
                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_merging);
@@ -1457,6 +1464,9 @@ template <int D, int WK, int WV, int GP, bool LLOYD> int launch_gp(const MfmaPar
     }
     const uint32_t wg_blocks = waves * p.runs.unit_blocks;
     const uint32_t grid = (p.total_blocks + wg_blocks - 1) / wg_blocks;
+    if (p.merge.region_wgs != 0 && !mfma_decode_merges(GP, D)) {
+        return fail(WEED_HIP_EDEVICE, "decode_mfma: this kernel instance cannot merge partials through memory");
+    }
     if (p.merge.wg_regions != 0 || p.merge.region_wgs != 0) {
         if constexpr (kMerges) {
             decode_mfma_kernel<D, WK, WV, GP, LLOYD, true><<<grid, 64 * waves, smem_merging, s>>>(p);
