@@ -268,6 +268,9 @@ def test_equal_contexts_with_and_without_the_region_search(gpu, oracle):
     (True, 96, 2, 16, 4, 1536, 4, 4, 96, False),    # groups of 8, one region per workgroup, no rotations
     (True, 80, 2, 8, 4, 768, 3, 4, 48, True),       # head_dim 80
     (False, 96, 1, 4, 8, 768, 4, 4, 96, True),      # uniform coder, four regions per workgroup
+    (True, 96, 2, 8, 1, 3072, 3, 4, 48, True),      # head_dim 96, two workgroups per region
+    (True, 96, 1, 4, 1, 6144, 3, 4, 96, True),      # head_dim 96, eight workgroups per region
+    (True, 80, 2, 16, 2, 3072, 3, 4, 96, False),    # head_dim 80, groups of 8, two workgroups per region, no rotations
 ])
 def test_workgroups_that_merge_their_own_regions(gpu, oracle, lloyd, d, Hkv, Hq, S, L, kb, vb, waves, rot):
     """When every workgroup of the matrix-core kernel holds whole regions, or every region a whole number of

@@ -1054,7 +1054,7 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         if (mfma_decode_merges_whole_regions(gp, d, runs.waves) && nb != 0 && nb % cycle == 0 && wg_blocks % nb == 0 &&
             !tune.separate_merge) {
             wg_regions = wg_blocks / nb;
-        } else if (mfma_decode_merges(gp, d) && nb != 0 && nb % wg_blocks == 0 && nb / wg_blocks >= 2 &&
+        } else if (mfma_decode_merges_whole_regions(gp, d, runs.waves) && nb != 0 && nb % wg_blocks == 0 && nb / wg_blocks >= 2 &&
                    nb / wg_blocks <= std::min(n_splits, 64u) && (size_t)S * Hkv <= kMfmaMergeCounters &&
                    !tune.separate_merge) {
             // small batches of long sequences: every region is a whole number of workgroups' shares
@@ -1105,7 +1105,7 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         }
         // A workgroup rotates the queries of the regions its blocks lie in itself when they are few enough for its
         // LDS (equal sequences, or the ragged batches above); nothing then runs ahead of the matrix-core kernel.
-        fused_query = (wg_regions != 0 || mfma_decode_merges(gp, d)) && (nb != 0 || general_merge) &&
+        fused_query = (wg_regions != 0 || region_wgs != 0 || mfma_decode_merges(gp, d)) && (nb != 0 || general_merge) &&
                       wg_most_regions * pass_heads <= kMfmaQueryRows && !tune.separate_query;
     }
     // Workgroups that merge whole regions or whole shares of a region: neighbouring runs take their blocks in turns

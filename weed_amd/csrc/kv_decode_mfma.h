@@ -167,9 +167,10 @@ constexpr uint32_t kMfmaQueryRows = 32;
 
 // Instances that can merge: head_dim 64 or 128.
 constexpr bool mfma_decode_merges(uint32_t gp, uint32_t d) { return gp <= 16 && (d == 64u || d == 128u); }
-// Instances whose workgroups can merge WHOLE regions in LDS and rotate their queries (MfmaMerge::wg_regions; not the
-// merges through memory, in which a wavefront works on one row at a time): the above, and head_dim 96 where a
-// workgroup has twelve wavefronts, so that its 768 threads are eight rows of 96.  (`waves`: mfma_decode_waves_per_wg.)
+// Instances whose workgroups can merge whole regions, or whole shares of one region, and rotate their queries
+// (MfmaMerge::wg_regions and region_wgs; not the general case, which is compiled into the other variant of an
+// instance): the above, and head_dim 96 where a workgroup has twelve wavefronts, so that its 768 threads are eight
+// rows of 96.  (`waves`: mfma_decode_waves_per_wg.)
 constexpr bool mfma_decode_merges_whole_regions(uint32_t gp, uint32_t d, uint32_t waves)
 {
     return mfma_decode_merges(gp, d) || (gp <= 16 && d == 96u && waves == 12u);

@@ -1266,52 +1266,69 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
         // of device scope), so a pass costs two trips to memory, not one per partial.  Then the rows are finished.
         auto finish_regions_from_memory = [&](uint32_t count, auto region_of, auto slots_of) {
             const uint32_t rows = count * p.G;
-            for (uint32_t r0 = 0; r0 < rows; r0 += RP) {
-                for (uint32_t rr = rr_of_wave; rr < RP; rr += kThreads / D) {
-                    const uint32_t row = r0 + rr;
-                    float v = 0.0f;
-                    if (row < rows) {
-                        const uint32_t ri = row / p.G, hs = row - ri * p.G;
-                        const uint32_t region = region_of(ri), slots = slots_of(ri);
-                        const uint32_t s_ = region / p.Hkv, kv_ = region - s_ * p.Hkv;
-                        const float *first = p.partials + ((uint64_t)s_ * p.Hq + q_head_of(p, kv_, hs)) * p.max_slots * PS;
-                        const __amdgpu_buffer_rsrc_t src = buffer_of(first, slots * (4 * PS));
-                        float m0 = buffer_f32<true>(src, lane * (4 * PS), 0), l0 = buffer_f32<true>(src, lane * (4 * PS), 4);
-                        float y[8];
+            // row rr of the pass (the same in all lanes of the wavefront), this lane's column of it (col_ok: it has one)
+            auto one_row = [&](uint32_t r0, uint32_t rr, uint32_t column, bool col_ok) {
+                const uint32_t row = r0 + rr;
+                float v = 0.0f;
+                if (row < rows) {
+                    const uint32_t ri = row / p.G, hs = row - ri * p.G;
+                    const uint32_t region = region_of(ri), slots = slots_of(ri);
+                    const uint32_t s_ = region / p.Hkv, kv_ = region - s_ * p.Hkv;
+                    const float *first = p.partials + ((uint64_t)s_ * p.Hq + q_head_of(p, kv_, hs)) * p.max_slots * PS;
+                    const __amdgpu_buffer_rsrc_t src = buffer_of(first, slots * (4 * PS));
+                    const uint32_t cb = 4 * (col_ok ? column : 0u);
+                    float m0 = buffer_f32<true>(src, lane * (4 * PS), 0), l0 = buffer_f32<true>(src, lane * (4 * PS), 4);
+                    float y[8];
+#pragma unroll
+                    for (uint32_t u = 0; u < 8; ++u) {
+                        y[u] = buffer_f32<true>(src, cb, 4 * (min(u, slots - 1) * PS + 2));
+                    }
+                    if (lane >= slots) {
+                        m0 = -INFINITY;
+                        l0 = 0.0f;
+                    }
+                    const float mx = wave_max64(m0);
+                    const float w0 = (m0 == -INFINITY) ? 0.0f : exp2f(m0 - mx);
+                    const float den = wave_sum64(w0 * l0);
+                    float acc = 0.0f;
+                    for (uint32_t k0 = 0; k0 < slots; k0 += 8) {
+                        float z[8];
+                        if (k0 + 8 < slots) {
+#pragma unroll
+                            for (uint32_t u = 0; u < 8; ++u) {
+                                z[u] = buffer_f32<true>(src, cb, 4 * (min(k0 + 8 + u, slots - 1) * PS + 2));
+                            }
+                        }
 #pragma unroll
                         for (uint32_t u = 0; u < 8; ++u) {
-                            y[u] = buffer_f32<true>(src, 4 * col, 4 * (min(u, slots - 1) * PS + 2));
-                        }
-                        if (lane >= slots) {
-                            m0 = -INFINITY;
-                            l0 = 0.0f;
-                        }
-                        const float mx = wave_max64(m0);
-                        const float w0 = (m0 == -INFINITY) ? 0.0f : exp2f(m0 - mx);
-                        const float den = wave_sum64(w0 * l0);
-                        float acc = 0.0f;
-                        for (uint32_t k0 = 0; k0 < slots; k0 += 8) {
-                            float z[8];
-                            if (k0 + 8 < slots) {
-#pragma unroll
-                                for (uint32_t u = 0; u < 8; ++u) {
-                                    z[u] = buffer_f32<true>(src, 4 * col, 4 * (min(k0 + 8 + u, slots - 1) * PS + 2));
-                                }
-                            }
-#pragma unroll
-                            for (uint32_t u = 0; u < 8; ++u) {
-                                if (k0 + u < slots) {
-                                    acc = fmaf(lane_value(w0, k0 + u), y[u], acc);
-                                }
-                            }
-#pragma unroll
-                            for (uint32_t u = 0; u < 8; ++u) {
-                                y[u] = z[u];
+                            if (k0 + u < slots) {
+                                acc = fmaf(lane_value(w0, k0 + u), y[u], acc);
                             }
                         }
-                        v = den > 0.0f ? acc / den : 0.0f;
+#pragma unroll
+                        for (uint32_t u = 0; u < 8; ++u) {
+                            y[u] = z[u];
+                        }
                     }
-                    o_s[staged_at(rr, col)] = v;
+                    v = den > 0.0f ? acc / den : 0.0f;
+                }
+                if (col_ok) {
+                    o_s[staged_at(rr, column)] = v;
+                }
+            };
+            for (uint32_t r0 = 0; r0 < rows; r0 += RP) {
+                if constexpr (kRowPerWave) {
+                    for (uint32_t rr = rr_of_wave; rr < RP; rr += kThreads / D) {
+                        one_row(r0, rr, col, true);
+                    }
+                } else {
+                    // (a wavefront's threads are not all in one row: wavefront w takes row w, 64 columns at a time)
+                    if (wave < RP) {
+#pragma unroll
+                        for (uint32_t cc = 0; cc < (D + 63) / 64; ++cc) {
+                            one_row(r0, wave, lane + 64 * cc, lane + 64 * cc < D);
+                        }
+                    }
                 }
                 finish_rows(r0, rows, region_of, r0 + RP < rows);
             }
@@ -1464,9 +1481,6 @@ template <int D, int WK, int WV, int GP, bool LLOYD> int launch_gp(const MfmaPar
     }
     const uint32_t wg_blocks = waves * p.runs.unit_blocks;
     const uint32_t grid = (p.total_blocks + wg_blocks - 1) / wg_blocks;
-    if (p.merge.region_wgs != 0 && !mfma_decode_merges(GP, D)) {
-        return fail(WEED_HIP_EDEVICE, "decode_mfma: this kernel instance cannot merge partials through memory");
-    }
     if (p.merge.wg_regions != 0 || p.merge.region_wgs != 0) {
         if constexpr (kMerges) {
             decode_mfma_kernel<D, WK, WV, GP, LLOYD, true><<<grid, 64 * waves, smem_merging, s>>>(p);
