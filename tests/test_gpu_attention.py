@@ -271,6 +271,11 @@ def test_equal_contexts_with_and_without_the_region_search(gpu, oracle):
     (True, 96, 2, 8, 1, 3072, 3, 4, 48, True),      # head_dim 96, two workgroups per region
     (True, 96, 1, 4, 1, 6144, 3, 4, 96, True),      # head_dim 96, eight workgroups per region
     (True, 80, 2, 16, 2, 3072, 3, 4, 96, False),    # head_dim 80, groups of 8, two workgroups per region, no rotations
+    # head_dim 32 (and below, stored as 32): two rows per wavefront
+    (True, 32, 2, 8, 4, 768, 3, 4, 48, True),       # two regions per workgroup
+    (True, 8, 1, 1, 8, 1536, 4, 4, 96, True),       # head_dim 8 (the reference example's), one head
+    (False, 32, 2, 16, 1, 3072, 4, 4, 48, True),    # uniform coder, groups of 8, two workgroups per region
+    (True, 24, 1, 4, 1, 6144, 2, 2, 96, False),     # head_dim 24, eight workgroups per region, no rotations
 ])
 def test_workgroups_that_merge_their_own_regions(gpu, oracle, lloyd, d, Hkv, Hq, S, L, kb, vb, waves, rot):
     """When every workgroup of the matrix-core kernel holds whole regions, or every region a whole number of

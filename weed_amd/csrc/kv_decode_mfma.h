@@ -169,11 +169,11 @@ constexpr uint32_t kMfmaQueryRows = 32;
 constexpr bool mfma_decode_merges(uint32_t gp, uint32_t d) { return gp <= 16 && (d == 64u || d == 128u); }
 // Instances whose workgroups can merge whole regions, or whole shares of one region, and rotate their queries
 // (MfmaMerge::wg_regions and region_wgs; not the general case, which is compiled into the other variant of an
-// instance): the above, and head_dim 96 where a workgroup has twelve wavefronts, so that its 768 threads are eight
-// rows of 96.  (`waves`: mfma_decode_waves_per_wg.)
+// instance): the above, head_dim 96 where a workgroup has twelve wavefronts, so that its 768 threads are eight
+// rows of 96, and head_dim 32 (two rows per wavefront).  (`waves`: mfma_decode_waves_per_wg.)
 constexpr bool mfma_decode_merges_whole_regions(uint32_t gp, uint32_t d, uint32_t waves)
 {
-    return mfma_decode_merges(gp, d) || (gp <= 16 && d == 96u && waves == 12u);
+    return mfma_decode_merges(gp, d) || (gp <= 16 && ((d == 96u && waves == 12u) || d == 32u));
 }
 // Rows (region, head) that one pass of the merge or of the query rotation takes (the matrix instruction behind both
 // has 16 rows, so a pass reads 8 rows beyond its own), and the LDS of both behind the lookup tables, in words.
