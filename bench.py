@@ -267,13 +267,16 @@ def streaming_read(capi, torch, nbytes, steps, warmup):
                       "contiguous run each (the decode kernel's shape), and the same wavefronts taking the 8 KB units in turns"}
 
 
-def layer_decode_step(capi, torch, np, n_calls, n_seq=64, ctx=8192, d_model=4096, n_heads=32, n_kv=8, d_ff=14336):
+def layer_decode_step(capi, torch, np, n_calls, n_seq=64, ctx=8192, d_model=4096, n_heads=32, n_kv=8, d_ff=14336,
+                      side_by_side=False):
     """One decode step of one Qwen-style decoder layer (include/modules/qwen_decoder_layer.hpp:104-115) through the C
     ABI, launch for launch what the host mirror's QwenDecoderLayer::forward issues for a (B, 1, d_model) input:
     RMSNorm, the Q / K / V projections (with bias), RoPE on Q and K at position ctx, append, fused attention over the
     packed cache, the output projection, residual, RMSNorm, gate / up projections, SiLU gate, down projection,
     residual.  Activations are column-major (batch index fastest) as Weed lays them out; weights are random.  The
-    cache starts n_calls tokens short of ctx and every call of the returned step appends one token per sequence."""
+    cache starts n_calls tokens short of ctx and every call of the returned step appends one token per sequence.
+    side_by_side: the weights of Q, K, V lie side by side in one buffer, and so do gate and up, as after the host
+    mirror's fuse_projections(); the projections that share their input are then one product each (13 launches)."""
     B, D, H, Hkv, hd = n_seq, d_model, n_heads, n_kv, d_model // n_heads
     dev = "cuda"
     g = torch.Generator(device=dev)
@@ -283,9 +286,17 @@ def layer_decode_step(capi, torch, np, n_calls, n_seq=64, ctx=8192, d_model=4096
         return (torch.randn((cols, rows), generator=g, device=dev) * scale).t()
 
     x = cm(B, D)
-    w_q, w_k, w_v, w_o = cm(D, H * hd, 0.02), cm(D, Hkv * hd, 0.02), cm(D, Hkv * hd, 0.02), cm(H * hd, D, 0.02)
-    b_q, b_k, b_v, b_o = (torch.zeros(n, device=dev) for n in (H * hd, Hkv * hd, Hkv * hd, D))
-    w_gate, w_up, w_down = cm(D, d_ff, 0.02), cm(D, d_ff, 0.02), cm(d_ff, D, 0.02)
+    nq, nkv = H * hd, Hkv * hd
+    if side_by_side:
+        w_qkv, b_qkv, w_gu = cm(D, nq + 2 * nkv, 0.02), torch.zeros(nq + 2 * nkv, device=dev), cm(D, 2 * d_ff, 0.02)
+        w_q, w_k, w_v = w_qkv[:, :nq], w_qkv[:, nq:nq + nkv], w_qkv[:, nq + nkv:]
+        b_q, b_k, b_v = b_qkv[:nq], b_qkv[nq:nq + nkv], b_qkv[nq + nkv:]
+        w_gate, w_up = w_gu[:, :d_ff], w_gu[:, d_ff:]
+        w_o, b_o, w_down = cm(nq, D, 0.02), torch.zeros(D, device=dev), cm(d_ff, D, 0.02)
+    else:
+        w_q, w_k, w_v, w_o = cm(D, nq, 0.02), cm(D, nkv, 0.02), cm(D, nkv, 0.02), cm(nq, D, 0.02)
+        b_q, b_k, b_v, b_o = (torch.zeros(n, device=dev) for n in (nq, nkv, nkv, D))
+        w_gate, w_up, w_down = cm(D, d_ff, 0.02), cm(D, d_ff, 0.02), cm(d_ff, D, 0.02)
     ln1, ln2 = torch.ones(D, device=dev), torch.ones(D, device=dev)
     # RoPE tables, column-major [rows, head_dim] (src/modules/rope.cpp:18-51); only row `ctx - 1` is used
     rows = ctx + 1
@@ -308,9 +319,13 @@ def layer_decode_step(capi, torch, np, n_calls, n_seq=64, ctx=8192, d_model=4096
     def buf(cols):
         return torch.empty((cols, B), device=dev).t()  # logical [B, cols], column-major
 
-    h1, q, k, v, qr, kr, att, o, res1, h2, gate, up, act, down, out = (
-        buf(D), buf(H * hd), buf(Hkv * hd), buf(Hkv * hd), buf(H * hd), buf(Hkv * hd), buf(H * hd), buf(D), buf(D),
-        buf(D), buf(d_ff), buf(d_ff), buf(d_ff), buf(D), buf(D))
+    h1, qr, kr, att, o, res1, h2, act, down, out = (
+        buf(D), buf(nq), buf(nkv), buf(nq), buf(D), buf(D), buf(D), buf(d_ff), buf(D), buf(D))
+    if side_by_side:
+        qkv, gu = buf(nq + 2 * nkv), buf(2 * d_ff)
+        q, k, v, gate, up = qkv[:, :nq], qkv[:, nq:nq + nkv], qkv[:, nq + nkv:], gu[:, :d_ff], gu[:, d_ff:]
+    else:
+        q, k, v, gate, up = buf(nq), buf(nkv), buf(nkv), buf(d_ff), buf(d_ff)
     eps = float(np.float32(np.finfo(np.float32).eps / 4))
 
     def heads(t, n):  # the (B, heads, T = 1, head_dim) view of a (B, 1, heads * head_dim) activation: feature = h + n * j
@@ -320,9 +335,12 @@ def layer_decode_step(capi, torch, np, n_calls, n_seq=64, ctx=8192, d_model=4096
 
     def step():
         capi.rms_norm(x, ln1, eps, h1)
-        capi.linear(h1, w_q, b_q, q)
-        capi.linear(h1, w_k, b_k, k)
-        capi.linear(h1, w_v, b_v, v)
+        if side_by_side:
+            capi.linear(h1, w_qkv, b_qkv, qkv)
+        else:
+            capi.linear(h1, w_q, b_q, q)
+            capi.linear(h1, w_k, b_k, k)
+            capi.linear(h1, w_v, b_v, v)
         capi.rope(heads(q, H), cos_t, sin_t, rows, heads(qr, H), pos0=ctx - 1)
         capi.rope(heads(k, Hkv), cos_t, sin_t, rows, heads(kr, Hkv), pos0=ctx - 1)
         cache.encode_append(heads(kr, Hkv), heads(v, Hkv), rotate=1)
@@ -330,8 +348,11 @@ def layer_decode_step(capi, torch, np, n_calls, n_seq=64, ctx=8192, d_model=4096
         capi.linear(att, w_o, b_o, o)
         capi.elementwise(capi.EW_ADD, o, x, res1)
         capi.rms_norm(res1, ln2, eps, h2)
-        capi.linear(h2, w_gate, None, gate)
-        capi.linear(h2, w_up, None, up)
+        if side_by_side:
+            capi.linear(h2, w_gu, None, gu)
+        else:
+            capi.linear(h2, w_gate, None, gate)
+            capi.linear(h2, w_up, None, up)
         capi.elementwise(capi.EW_SILU_MUL, gate, up, act)
         capi.linear(act, w_down, None, down)
         capi.elementwise(capi.EW_ADD, down, res1, out)
@@ -668,6 +689,19 @@ def extras(capi, torch, workloads, steps, warmup):
                  "gate/up projections, SiLU gate, down projection, residual",
         "weight_bytes": 4 * (2 * 4096 * 4096 + 2 * 4096 * 1024 + 3 * 4096 * 14336)}
     cacheQ.close()
+    del cacheQ, layer_step
+    # the same step with the weights of the projections that share their input side by side (the host mirror's
+    # fuse_projections()): Q, K, V are one product, gate and up another
+    cacheF, fused_step = layer_decode_step(capi, torch, np, n_calls=WARMUP_FLOOR_EXTRA + 2 * n_l + 1, side_by_side=True)
+    fused_step()
+    torch.cuda.synchronize()
+    fused_host_s = time_calls(torch, fused_step, n_l, WARMUP_FLOOR_EXTRA)
+    fused_dev_s = time_region(torch, fused_step, n_l, 0)
+    out["qwen_layer_decode_step_64_sequences_ctx8192"]["projections_side_by_side"] = {
+        "ms_per_step": 1e3 * fused_host_s, "device_ms_per_step": 1e3 * fused_dev_s, "launches_per_step": 13,
+        "what": "the weights of Q, K, V in one buffer and those of gate and up in another, as after "
+                "fuse_projections() of the host mirror's layer: one product for each group"}
+    cacheF.close()
     return out
 
 

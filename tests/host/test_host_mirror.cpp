@@ -1312,6 +1312,113 @@ TEST_CASE(test_qwen_decoder_layer_prefill_then_decode, true)
     REQUIRE(mha.max_seq_len == 20U);
 }
 
+TEST_CASE(test_projections_side_by_side, true)
+{
+    // fuse_projections() moves the weights of the projections that share their input (Q, K, V; gate, up) side by side
+    // and runs them as one product: the same parameters, the same stream on save, results equal to those of the
+    // separate products up to the rounding of a differently cut sum
+    const tcapint B = 3U;
+    auto close_to = [](const std::vector<real1> &a, const std::vector<real1> &b) {
+        if (a.size() != b.size()) {
+            return false;
+        }
+        for (size_t i = 0; i < a.size(); ++i) {
+            if (std::fabs((double)a[i] - (double)b[i]) > std::max(1e-4, 1e-3 * std::fabs((double)b[i]))) {
+                return false;
+            }
+        }
+        return true;
+    };
+    {
+        QwenDecoderLayer a(128U, 4U, 2U, 192U, 24U);
+        a.self_attn->kv_coder = KV_LLOYDMAX;
+        a.self_attn->k_bits = 3;
+        a.self_attn->v_bits = 4;
+        a.self_attn->rotation_seed = 8U;
+        std::stringstream ss;
+        a.save(ss);
+        a.self_attn->save_quantizer(ss);
+        const std::string before = ss.str();
+        QwenDecoderLayerPtr b = std::dynamic_pointer_cast<QwenDecoderLayer>(Module::load(ss));
+        REQUIRE((bool)b);
+        if (!b) {
+            return;
+        }
+        b->self_attn->load_quantizer(ss);
+        std::vector<std::vector<real1>> values;
+        for (const ParameterPtr &p : b->parameters()) {
+            values.push_back(p->to_vector());
+        }
+        const std::vector<ParameterPtr> held = b->parameters();
+        b->fuse_projections();
+        b->fuse_projections(); // (a second call finds them in place)
+        // one storage under Q, K, V and one under gate, up; the parameter objects are the ones held before
+        REQUIRE(b->self_attn->W_q->weight->storage == b->self_attn->W_k->weight->storage);
+        REQUIRE(b->self_attn->W_k->weight->storage == b->self_attn->W_v->weight->storage);
+        REQUIRE(b->self_attn->W_q->weight->storage != b->self_attn->W_o->weight->storage);
+        REQUIRE(b->mlp->gate_proj->weight->storage == b->mlp->up_proj->weight->storage);
+        REQUIRE(b->self_attn->W_k->weight->offset == 128U * 128U && b->self_attn->W_v->weight->offset == 128U * (128U + 64U));
+        const std::vector<ParameterPtr> now = b->parameters();
+        REQUIRE(now.size() == held.size());
+        for (size_t i = 0; i < now.size() && i < held.size(); ++i) {
+            REQUIRE(now[i] == held[i]);
+            REQUIRE(now[i]->to_vector() == values[i]);
+        }
+        // the stream of the moved module is the stream of the original
+        std::stringstream after;
+        b->save(after);
+        b->self_attn->save_quantizer(after);
+        REQUIRE(after.str() == before);
+        tcapint seen = 0U;
+        for (const tcapint T : { 6U, 1U, 1U, 3U }) {
+            const std::vector<real1> xv = gaussian((size_t)B * T * 128U, 700U + seen);
+            TensorPtr x = std::make_shared<Tensor>(xv, std::vector<tcapint>{ B, T, 128U }, false, TEST_DTAG);
+            const std::vector<real1> ya = a.forward(x)->to_vector(), yb = b->forward(x)->to_vector();
+            REQUIRE(close_to(yb, ya));
+            seen += T;
+        }
+    }
+    {
+        // with biases (the encoder layer's attention), and a module whose projections differ in width
+        TransformerEncoderLayer a(64U, 4U, 96U, TEST_DTAG, GELU_FN);
+        a.self_attn->rotation_seed = 3U;
+        a.set_max_kv_seq_len(16U);
+        std::stringstream ss;
+        a.save(ss);
+        TransformerEncoderLayerPtr b = std::dynamic_pointer_cast<TransformerEncoderLayer>(Module::load(ss));
+        REQUIRE((bool)b);
+        if (!b) {
+            return;
+        }
+        b->self_attn->rotation_seed = 3U;
+        b->set_max_kv_seq_len(16U);
+        b->fuse_projections();
+        REQUIRE(b->self_attn->W_q->bias && b->self_attn->W_q->bias->storage == b->self_attn->W_v->bias->storage);
+        for (const tcapint T : { 5U, 1U }) {
+            const std::vector<real1> xv = gaussian((size_t)B * T * 64U, 800U + T);
+            TensorPtr x = std::make_shared<Tensor>(xv, std::vector<tcapint>{ B, T, 64U }, false, TEST_DTAG);
+            REQUIRE(close_to(b->forward(x)->to_vector(), a.forward(x)->to_vector()));
+        }
+        // modules that cannot lie side by side are refused
+        LinearPtr p = std::make_shared<Linear>(8U, 4U, true, true, DType::REAL, TEST_DTAG);
+        LinearPtr q = std::make_shared<Linear>(16U, 4U, true, true, DType::REAL, TEST_DTAG);
+        LinearPtr r = std::make_shared<Linear>(8U, 6U, false, true, DType::REAL, TEST_DTAG);
+        REQUIRE_THROWS_AS(place_side_by_side({ p, q }), std::invalid_argument);
+        REQUIRE_THROWS_AS(place_side_by_side({ p, r }), std::invalid_argument);
+        // ... and ones that do not (yet) are applied one by one
+        LinearPtr s2 = std::make_shared<Linear>(8U, 6U, true, true, DType::REAL, TEST_DTAG);
+        const std::vector<real1> xv = gaussian(5U * 8U, 9U);
+        TensorPtr x = std::make_shared<Tensor>(xv, std::vector<tcapint>{ 5U, 8U }, false, TEST_DTAG);
+        const std::vector<TensorPtr> apart = forward_side_by_side({ p, s2 }, x);
+        REQUIRE(apart.size() == 2U && apart[0]->to_vector() == p->forward(x)->to_vector());
+        place_side_by_side({ p, s2 });
+        const std::vector<TensorPtr> together = forward_side_by_side({ p, s2 }, x);
+        REQUIRE(together.size() == 2U && together[1]->shape == std::vector<tcapint>({ 5U, 6U }));
+        REQUIRE(close_to(together[0]->to_vector(), apart[0]->to_vector()));
+        REQUIRE(close_to(together[1]->to_vector(), apart[1]->to_vector()));
+    }
+}
+
 TEST_CASE(test_checkpoint_layers_round_trip, true)
 {
     // save -> load of both layer modules (transformer_encoder_layer.cpp:126-138, qwen_decoder_layer.cpp:18-27,

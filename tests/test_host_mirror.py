@@ -36,7 +36,8 @@ def test_host_library_loads_and_exports_the_mirror():
                  "Weed::QuantizedKVCache::read_row(unsigned int, float*) const",
                  "Weed::Linear::forward(", "Weed::RMSNorm::forward(", "Weed::LayerNorm::forward(", "Weed::SwiGLU::forward(",
                  "Weed::QwenDecoderLayer::forward(", "Weed::TransformerEncoderLayer::forward(",
-                 "Weed::MultiHeadAttention::set_tables("):
+                 "Weed::MultiHeadAttention::set_tables(", "Weed::place_side_by_side(", "Weed::forward_side_by_side(",
+                 "Weed::QwenDecoderLayer::fuse_projections()"):
         assert name in out, name
     assert lib is not None
 
@@ -50,3 +51,4 @@ def test_host_logic_without_a_device():
 def test_host_mirror_on_device():
     out = _run([])
     assert "0 failed" in out and "test_attention_lloydmax" in out and "test_qwen_decoder_layer_prefill_then_decode" in out
+    assert "test_projections_side_by_side" in out

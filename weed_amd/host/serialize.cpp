@@ -148,6 +148,20 @@ StoragePtr Storage::load(std::istream &is)
 // ---- Parameter ----
 void Parameter::save(std::ostream &out)
 {
+    // A parameter that is a view of a larger storage (projections laid side by side, place_side_by_side) is written
+    // as a compact copy of its own elements: the stream is the one the module wrote before it was moved.
+    tcapint span = 1U;
+    for (size_t i = 0U; i < shape.size(); ++i) {
+        span += (shape[i] - 1U) * stride[i];
+    }
+    if (offset != 0U || storage->size != span) {
+        std::shared_ptr<Tensor> self = std::make_shared<Tensor>(static_cast<const Tensor &>(*this));
+        const TensorPtr own = Tensor::compact(self);
+        Parameter copy;
+        static_cast<Tensor &>(copy) = *own;
+        copy.save(out);
+        return;
+    }
     Serializer::write_symint(out, (symint)storage->get_device_id());
     for (size_t i = 0U; i < stride.size(); ++i) {
         if (!stride[i]) {

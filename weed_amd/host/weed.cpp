@@ -570,6 +570,16 @@ TensorPtr Tensor::contiguous(const TensorPtr a)
     return out;
 }
 
+TensorPtr Tensor::compact(const TensorPtr a)
+{
+    if (a->is_contiguous() && a->offset == 0U && a->storage->size == a->get_size()) {
+        return a;
+    }
+    TensorPtr out = allocate(a->shape, *a);
+    elementwise(WEED_HIP_EW_COPY, *a, nullptr, *out, "Tensor::compact");
+    return out;
+}
+
 TensorPtr Tensor::reshape(const TensorPtr a, const std::vector<symint> &s)
 {
     TensorPtr out = a->is_contiguous() ? std::make_shared<Tensor>(*a) : contiguous(a);
@@ -1001,6 +1011,113 @@ TensorPtr Linear::forward(const TensorPtr x)
     return out;
 }
 
+namespace {
+// weights (in, out) with a column per output, k contiguous; biases (1, out)
+bool plain_linear(const Linear &l)
+{
+    const Parameter *w = l.weight.get(), *b = l.bias.get();
+    return w && w->shape.size() == 2U && w->shape[0U] == l.in_features && w->shape[1U] == l.out_features &&
+        (w->stride[0U] == 1U || l.in_features == 1U) && (w->stride[1U] == l.in_features || l.out_features == 1U) &&
+        (!b || (b->shape.size() == 2U && b->shape[0U] == 1U && b->shape[1U] == l.out_features &&
+                (b->stride[1U] == 1U || l.out_features == 1U)));
+}
+bool lie_side_by_side(const std::vector<LinearPtr> &ls)
+{
+    if (ls.size() < 2U || !ls[0U] || !plain_linear(*ls[0U])) {
+        return false;
+    }
+    const Linear &first = *ls[0U];
+    tcapint cols = 0U;
+    for (const LinearPtr &l : ls) {
+        if (!l || !plain_linear(*l) || l->in_features != first.in_features || !l->bias != !first.bias ||
+            l->weight->storage != first.weight->storage ||
+            l->weight->offset != first.weight->offset + cols * first.in_features ||
+            (l->bias && (l->bias->storage != first.bias->storage || l->bias->offset != first.bias->offset + cols))) {
+            return false;
+        }
+        cols += l->out_features;
+    }
+    return true;
+}
+} // namespace
+
+void place_side_by_side(const std::vector<LinearPtr> &ls)
+{
+    if (ls.size() < 2U) {
+        return;
+    }
+    tcapint cols = 0U;
+    for (const LinearPtr &l : ls) {
+        if (!l || !l->weight || !plain_linear(*l) || l->in_features != ls[0U]->in_features || !l->bias != !ls[0U]->bias) {
+            throw std::invalid_argument("place_side_by_side(): the modules need plain (in, out) weights of the same "
+                                        "in_features, and biases all or none");
+        }
+        cols += l->out_features;
+    }
+    if (lie_side_by_side(ls)) {
+        return;
+    }
+    const tcapint in = ls[0U]->in_features;
+    for (const LinearPtr &l : ls) {
+        validate_all_same_device({ ls[0U]->weight.get(), l->weight.get() }, "place_side_by_side");
+        if (l->bias) {
+            validate_all_same_device({ ls[0U]->weight.get(), l->bias.get() }, "place_side_by_side");
+        }
+    }
+    TensorPtr w = allocate({ in, cols }, *ls[0U]->weight);
+    TensorPtr b = ls[0U]->bias ? allocate({ 1U, cols }, *ls[0U]->bias) : nullptr;
+    tcapint at = 0U;
+    for (const LinearPtr &l : ls) {
+        TensorPtr wv = Tensor::slice(w, 1, at, l->out_features);
+        elementwise(WEED_HIP_EW_COPY, *l->weight, nullptr, *wv, "place_side_by_side");
+        l->weight->storage = wv->storage;
+        l->weight->offset = wv->offset;
+        l->weight->stride = wv->stride;
+        if (b) {
+            TensorPtr bv = Tensor::slice(b, 1, at, l->out_features);
+            elementwise(WEED_HIP_EW_COPY, *l->bias, nullptr, *bv, "place_side_by_side");
+            l->bias->storage = bv->storage;
+            l->bias->offset = bv->offset;
+            l->bias->stride = bv->stride;
+        }
+        at += l->out_features;
+    }
+}
+
+std::vector<TensorPtr> forward_side_by_side(const std::vector<LinearPtr> &ls, const TensorPtr x)
+{
+    std::vector<TensorPtr> out;
+    if (!lie_side_by_side(ls)) {
+        for (const LinearPtr &l : ls) {
+            out.push_back(l->forward(x));
+        }
+        return out;
+    }
+    tcapint cols = 0U;
+    for (const LinearPtr &l : ls) {
+        cols += l->out_features;
+    }
+    // one module over all the columns: views of the shared storages
+    Linear all;
+    all.in_features = ls[0U]->in_features;
+    all.out_features = cols;
+    all.weight = std::make_shared<Parameter>();
+    static_cast<Tensor &>(*all.weight) = static_cast<const Tensor &>(*ls[0U]->weight);
+    all.weight->shape = { all.in_features, cols };
+    if (ls[0U]->bias) {
+        all.bias = std::make_shared<Parameter>();
+        static_cast<Tensor &>(*all.bias) = static_cast<const Tensor &>(*ls[0U]->bias);
+        all.bias->shape = { 1U, cols };
+    }
+    TensorPtr y = all.forward(x);
+    tcapint at = 0U;
+    for (const LinearPtr &l : ls) {
+        out.push_back(Tensor::slice(y, -1, at, l->out_features));
+        at += l->out_features;
+    }
+    return out;
+}
+
 std::vector<ParameterPtr> Linear::parameters()
 {
     std::vector<ParameterPtr> p{ weight };
@@ -1282,6 +1399,8 @@ void MultiHeadAttention::set_tables(int which, const std::vector<real1> &bounds,
     }
 }
 
+void MultiHeadAttention::fuse_projections() { place_side_by_side({ W_q, W_k, W_v }); }
+
 TensorPtr MultiHeadAttention::forward(const TensorPtr x)
 {
     // x: (B, T, d_model)
@@ -1290,9 +1409,9 @@ TensorPtr MultiHeadAttention::forward(const TensorPtr x)
     }
     const symint B = (symint)x->shape[0U], T = (symint)x->shape[1U];
 
-    TensorPtr Q = W_q->forward(x);
-    TensorPtr K = W_k->forward(x);
-    TensorPtr V = W_v->forward(x);
+    // (one product when fuse_projections() laid the three weights side by side)
+    const std::vector<TensorPtr> qkv = forward_side_by_side({ W_q, W_k, W_v }, x);
+    TensorPtr Q = qkv[0U], K = qkv[1U], V = qkv[2U];
 
     Q = Tensor::reshape(Q, { B, T, num_heads, head_dim });
     K = Tensor::reshape(K, { B, T, num_kv_heads, head_dim });
@@ -1707,13 +1826,20 @@ void SwiGLU::_register_params()
     }
 }
 
+void SwiGLU::fuse_projections()
+{
+    if (gate_proj && up_proj) {
+        place_side_by_side({ gate_proj, up_proj });
+    }
+}
+
 TensorPtr SwiGLU::forward(const TensorPtr x)
 {
     if (!gate_proj || !up_proj || !down_proj) {
         throw std::domain_error("SwiGLU::forward(): the module has no projections (default-constructed)");
     }
-    TensorPtr gate = gate_proj->forward(x);
-    TensorPtr up = up_proj->forward(x);
+    const std::vector<TensorPtr> gu = forward_side_by_side({ gate_proj, up_proj }, x);
+    TensorPtr gate = gu[0U], up = gu[1U];
     // SiLU(gate) * up
     TensorPtr activated = allocate(gate->shape, *gate);
     elementwise(WEED_HIP_EW_SILU_MUL, *gate, up.get(), *activated, "SwiGLU::forward");
@@ -1760,6 +1886,8 @@ void TransformerEncoderLayer::_register_params()
     }
 }
 
+void TransformerEncoderLayer::fuse_projections() { self_attn->fuse_projections(); }
+
 TensorPtr TransformerEncoderLayer::forward(const TensorPtr x)
 {
     TensorPtr x1 = self_attn->forward(norm1->forward(x));
@@ -1793,6 +1921,12 @@ void QwenDecoderLayer::_register_params()
              post_attention_layernorm->parameters() }) {
         param_vector.insert(param_vector.end(), q.begin(), q.end());
     }
+}
+
+void QwenDecoderLayer::fuse_projections()
+{
+    self_attn->fuse_projections();
+    mlp->fuse_projections();
 }
 
 TensorPtr QwenDecoderLayer::forward(const TensorPtr x)

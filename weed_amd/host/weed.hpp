@@ -258,6 +258,8 @@ struct Tensor {
     static TensorPtr zeros(const std::vector<tcapint> &shape, const bool &rg = false, const bool &s = true,
         const DType &dtype = DType::REAL, const DeviceTag &dtag = DeviceTag::DEFAULT_DEVICE, const int64_t &did = -1);
     static TensorPtr contiguous(const TensorPtr a);
+    // `a` itself when its storage holds exactly its elements in order, else a copy that does
+    static TensorPtr compact(const TensorPtr a);
     static TensorPtr reshape(const TensorPtr a, const std::vector<symint> &s);
     static TensorPtr transpose(const TensorPtr a);
     static TensorPtr transpose(const TensorPtr a, symint i, symint j);
@@ -356,6 +358,19 @@ struct Linear : public Module {
     void save(std::ostream &os) const override; // src/modules/linear.cpp:109-118
 };
 typedef std::shared_ptr<Linear> LinearPtr;
+
+// Linear modules that read the same input and whose weights (in_features x out_features, a column per output) lie
+// side by side in one storage, their biases in another, are applied with ONE product: the outputs of the first
+// module, then those of the second, ... are consecutive columns of one result.  No counterpart in the reference,
+// whose attention and SwiGLU modules launch one product per projection (Q, K, V; gate, up); at decode time the
+// small ones cost a launch and a pass over half-empty compute units each.
+// place_side_by_side(): moves the modules' weights and biases into such storages.  The Parameter objects stay the
+//   same (lists of parameters held elsewhere remain valid), the values are copied; all modules need the same
+//   in_features, device and bias-or-not.  A module saved afterwards writes a compact copy of its own weight, so the
+//   stream is the same as before.
+// forward_side_by_side(): the modules' outputs for x, in one launch when they lie side by side, else one by one.
+void place_side_by_side(const std::vector<LinearPtr> &linears);
+std::vector<TensorPtr> forward_side_by_side(const std::vector<LinearPtr> &linears, const TensorPtr x);
 
 // The packed K and V rows of one attention module live in ONE device object (include/weed_hip.h); the two
 // QuantizedKVCache members of the module are views of its two halves.
@@ -500,6 +515,8 @@ struct MultiHeadAttention : public Module {
     void set_max_kv_seq_len(tcapint m) override { max_seq_len = m; }
     void reset_cache() override;
     TensorPtr forward(const TensorPtr x) override;
+    // The Q, K and V projections as one product from now on (place_side_by_side; results agree to rounding).
+    void fuse_projections();
     // PREFILL_AUTO's rule for B sequences, T new tokens and L cached ones (the new ones included): true when
     // dequantising once and attending densely is estimated cheaper than the passes of the fused kernel
     bool dense_is_cheaper(tcapint B, tcapint T, tcapint L) const;
@@ -612,6 +629,8 @@ struct SwiGLU : public Module {
     void _register_params();
     std::vector<ParameterPtr> parameters() override { return param_vector; }
     TensorPtr forward(const TensorPtr x) override;
+    // The gate and up projections as one product from now on (place_side_by_side).
+    void fuse_projections();
     void save(std::ostream &os) const override; // src/modules/swiglu.cpp:18-25
 };
 typedef std::shared_ptr<SwiGLU> SwiGLUPtr;
@@ -645,6 +664,7 @@ struct TransformerEncoderLayer : public Module {
     void set_max_kv_seq_len(tcapint m) override { self_attn->set_max_kv_seq_len(m); }
     void reset_cache() override { self_attn->reset_cache(); }
     TensorPtr forward(const TensorPtr x) override;
+    void fuse_projections(); // the attention module's
     void save(std::ostream &os) const override;
 };
 typedef std::shared_ptr<TransformerEncoderLayer> TransformerEncoderLayerPtr;
@@ -676,6 +696,7 @@ struct QwenDecoderLayer : public Module {
     void set_max_kv_seq_len(tcapint m) override { self_attn->set_max_kv_seq_len(m); }
     void reset_cache() override { self_attn->reset_cache(); }
     TensorPtr forward(const TensorPtr x) override;
+    void fuse_projections(); // the attention module's and the SwiGLU's
     void save(std::ostream &os) const override; // src/modules/qwen_decoder_layer.cpp:18-27
 };
 typedef std::shared_ptr<QwenDecoderLayer> QwenDecoderLayerPtr;
