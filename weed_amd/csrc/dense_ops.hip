@@ -559,6 +559,67 @@ struct PointGeom {
     uint64_t n;
 };
 
+// The operation of an elementwise op on one pair of operands (unary ops ignore y).
+template <int OP> __device__ __forceinline__ float elementwise_apply(float x, float y)
+{
+    if (OP == 0) {
+        return x;
+    } else if (OP == 5) {
+        // SwiGLU's gate (include/modules/swiglu.hpp:71-77): gate * sigmoid(gate) * up, left to right
+        const float sg = 1.0f / (1.0f + expf(-x));
+        return (x * sg) * y;
+    } else if (OP <= 4) {
+        return OP == 1 ? x + y : OP == 2 ? x - y : OP == 3 ? x * y : x / y;
+    } else if (OP == 6) {
+        return fmaxf(x, 0.0f); // src/ops/real_unary.cpp:80
+    } else if (OP == 7) {
+        return 1.0f / (1.0f + expf(-x)); // src/ops/real_unary.cpp:135
+    } else if (OP == 8) {
+        return tanhf(x); // src/ops/real_unary.cpp:191
+    }
+    // Tensor::gelu (src/tensors/tensor.cpp:841-851), one rounded operation after the other as the reference's
+    // chain of elementwise ops: x3 = x * x * x; inner = k2 * (x + k1 * x3); k0 * x * (1 + tanh(inner))
+    const float x3 = (x * x) * x;
+    const float inner = 0.7978845608028654f * (x + 0.044715f * x3);
+    return (0.5f * x) * (1.0f + tanhf(inner));
+}
+
+// All operands dense in the same order of dimensions, 16-byte aligned, a multiple of four elements: 16-byte accesses,
+// four of them in flight per thread and operand, no index arithmetic per element.
+typedef float ew_f4 __attribute__((ext_vector_type(4)));
+template <int OP> __global__ void __launch_bounds__(256) elementwise_flat_kernel(const ew_f4 *__restrict__ a,
+                                                                                 const ew_f4 *__restrict__ b, ew_f4 *out,
+                                                                                 uint64_t n4)
+{
+    constexpr bool kBinary = OP >= 1 && OP <= 5;
+    auto one = [](const ew_f4 &x, const ew_f4 &y) {
+        return ew_f4{ elementwise_apply<OP>(x[0], y[0]), elementwise_apply<OP>(x[1], y[1]),
+                      elementwise_apply<OP>(x[2], y[2]), elementwise_apply<OP>(x[3], y[3]) };
+    };
+    // a workgroup takes whole pieces of 16 KB (its 256 threads x four 16-byte accesses, consecutive in memory), piece
+    // number blockIdx.x + k * gridDim.x: the workgroups that run at one time work through one contiguous stretch of
+    // every operand
+    const uint64_t pieces = n4 / 1024U;
+    for (uint64_t pc = blockIdx.x; pc < pieces; pc += gridDim.x) {
+        const uint64_t i = pc * 1024U + threadIdx.x;
+        ew_f4 x[4], y[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            x[u] = a[i + 256 * u];
+            y[u] = kBinary ? b[i + 256 * u] : x[u];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            out[i + 256 * u] = one(x[u], y[u]);
+        }
+    }
+    // what is left behind the last whole piece
+    for (uint64_t i = pieces * 1024U + (uint64_t)blockIdx.x * 256U + threadIdx.x; i < n4; i += (uint64_t)gridDim.x * 256U) {
+        const ew_f4 x = a[i];
+        out[i] = one(x, kBinary ? b[i] : x);
+    }
+}
+
 // One thread per logical element, dimension 0 fastest (the host orders the dimensions so that this is the direction
 // in which the output is most contiguous).
 template <int OP> __global__ void __launch_bounds__(256) elementwise_kernel(const float *__restrict__ a,
@@ -592,32 +653,7 @@ template <int OP> __global__ void __launch_bounds__(256) elementwise_kernel(cons
             }
         }
         const float x = a[ai];
-        float r;
-        if (OP == 0) {
-            r = x;
-        } else if (OP <= 5) {
-            const float y = b[bi];
-            if (OP == 5) {
-                // SwiGLU's gate (include/modules/swiglu.hpp:71-77): gate * sigmoid(gate) * up, left to right
-                const float sg = 1.0f / (1.0f + expf(-x));
-                r = (x * sg) * y;
-            } else {
-                r = OP == 1 ? x + y : OP == 2 ? x - y : OP == 3 ? x * y : x / y;
-            }
-        } else if (OP == 6) {
-            r = fmaxf(x, 0.0f); // src/ops/real_unary.cpp:80
-        } else if (OP == 7) {
-            r = 1.0f / (1.0f + expf(-x)); // src/ops/real_unary.cpp:135
-        } else if (OP == 8) {
-            r = tanhf(x); // src/ops/real_unary.cpp:191
-        } else {
-            // Tensor::gelu (src/tensors/tensor.cpp:841-851), one rounded operation after the other as the reference's
-            // chain of elementwise ops: x3 = x * x * x; inner = k2 * (x + k1 * x3); k0 * x * (1 + tanh(inner))
-            const float x3 = (x * x) * x;
-            const float inner = 0.7978845608028654f * (x + 0.044715f * x3);
-            r = (0.5f * x) * (1.0f + tanhf(inner));
-        }
-        out[oi] = r;
+        out[oi] = elementwise_apply<OP>(x, (OP >= 1 && OP <= 5) ? b[bi] : x);
     }
 }
 
@@ -887,6 +923,39 @@ int weed_hip_elementwise_f32(int op, uint32_t rank, const uint32_t *shape, const
     }
     const uint32_t blocks = (uint32_t)std::min<uint64_t>((g.n + 255) / 256, 256u * 64u);
     const float *b = unary ? a_dev : b_dev;
+    // every operand dense in the same order of dimensions, aligned, whole 16-byte pieces: the flat kernel
+    bool flat = g.n % 4U == 0U && g.n >= 4096U;
+    uint64_t dense = 1;
+    for (uint32_t dd = 0; dd < g.rank && flat; ++dd) {
+        if (g.shape[dd] == 1U) {
+            continue;
+        }
+        flat = g.o_stride[dd] == dense && g.a_stride[dd] == dense && (unary || g.b_stride[dd] == dense);
+        dense *= g.shape[dd];
+    }
+    auto aligned = [](const float *p, uint32_t off) { return ((reinterpret_cast<uintptr_t>(p) + 4ull * off) & 15U) == 0U; };
+    flat = flat && aligned(a_dev, a_off) && aligned(out_dev, o_off) && (unary || aligned(b_dev, b_off));
+    if (flat) {
+        const uint64_t n4 = g.n / 4U;
+        const uint32_t fb = (uint32_t)std::min<uint64_t>((n4 + 1023) / 1024, 256u * 16u);
+        const ew_f4 *a4 = reinterpret_cast<const ew_f4 *>(a_dev + a_off);
+        const ew_f4 *b4 = reinterpret_cast<const ew_f4 *>(unary ? a_dev + a_off : b_dev + b_off);
+        ew_f4 *o4 = reinterpret_cast<ew_f4 *>(out_dev + o_off);
+        switch (op) {
+        case WEED_HIP_EW_COPY: elementwise_flat_kernel<0><<<fb, 256, 0, stream()>>>(a4, b4, o4, n4); break;
+        case WEED_HIP_EW_ADD: elementwise_flat_kernel<1><<<fb, 256, 0, stream()>>>(a4, b4, o4, n4); break;
+        case WEED_HIP_EW_SUB: elementwise_flat_kernel<2><<<fb, 256, 0, stream()>>>(a4, b4, o4, n4); break;
+        case WEED_HIP_EW_MUL: elementwise_flat_kernel<3><<<fb, 256, 0, stream()>>>(a4, b4, o4, n4); break;
+        case WEED_HIP_EW_DIV: elementwise_flat_kernel<4><<<fb, 256, 0, stream()>>>(a4, b4, o4, n4); break;
+        case WEED_HIP_EW_SILU_MUL: elementwise_flat_kernel<5><<<fb, 256, 0, stream()>>>(a4, b4, o4, n4); break;
+        case WEED_HIP_EW_RELU: elementwise_flat_kernel<6><<<fb, 256, 0, stream()>>>(a4, b4, o4, n4); break;
+        case WEED_HIP_EW_SIGMOID: elementwise_flat_kernel<7><<<fb, 256, 0, stream()>>>(a4, b4, o4, n4); break;
+        case WEED_HIP_EW_TANH: elementwise_flat_kernel<8><<<fb, 256, 0, stream()>>>(a4, b4, o4, n4); break;
+        default: elementwise_flat_kernel<9><<<fb, 256, 0, stream()>>>(a4, b4, o4, n4); break;
+        }
+        WEED_HIP_LAUNCH_CHECK();
+        return WEED_HIP_OK;
+    }
     switch (op) {
     case WEED_HIP_EW_SILU_MUL:
         elementwise_kernel<5><<<blocks, 256, 0, stream()>>>(a_dev, b, out_dev, g);
