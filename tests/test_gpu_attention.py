@@ -276,6 +276,12 @@ def test_equal_contexts_with_and_without_the_region_search(gpu, oracle):
     (True, 8, 1, 1, 8, 1536, 4, 4, 96, True),       # head_dim 8 (the reference example's), one head
     (False, 32, 2, 16, 1, 3072, 4, 4, 48, True),    # uniform coder, groups of 8, two workgroups per region
     (True, 24, 1, 4, 1, 6144, 2, 2, 96, False),     # head_dim 24, eight workgroups per region, no rotations
+    # head_dim 256: a wavefront takes two of the sixteen tiles of the small rotations; at most 16 rows per workgroup
+    (True, 256, 2, 8, 4, 1024, 3, 4, 32, True),     # two regions per workgroup
+    (False, 256, 2, 16, 2, 1024, 4, 4, 16, False),  # uniform coder, groups of 8, two regions = 16 rows, no rotations
+    (False, 256, 2, 16, 2, 1024, 4, 4, 16, True),   # ... with rotations: two passes of eight rows each
+    (True, 256, 1, 4, 1, 4096, 3, 4, 64, True),     # eight workgroups per region
+    (True, 240, 2, 16, 1, 2048, 3, 4, 32, True),    # head_dim 240, groups of 8, two workgroups per region
 ])
 def test_workgroups_that_merge_their_own_regions(gpu, oracle, lloyd, d, Hkv, Hq, S, L, kb, vb, waves, rot):
     """When every workgroup of the matrix-core kernel holds whole regions, or every region a whole number of
@@ -371,9 +377,9 @@ def test_block_counts_that_no_run_length_divides(gpu, oracle, cap_blocks, top, s
     behind the cache's memory and is never read.  The third case mixes sequences of 23 and 24
     blocks, which are counted alike.  Three cases are small batches, where a region is several workgroups' shares
     and the count is rounded to a whole number of those; in the last of them the sequences hold 8000, 5500 and 3000
-    tokens and are all counted as 128 blocks, so whole workgroups find no tokens in their share.  Head_dim 256
-    has no instance that merges its partials itself: the same partition, three kernels per call; head_dim 96 merges
-    whole regions like 128 (its workgroups of twelve wavefronts are eight rows of 96 threads).  All must
+    tokens and are all counted as 128 blocks, so whole workgroups find no tokens in their share.  Head_dims 256
+    and 96 merge whole regions like 128 (at 96 a workgroup of twelve wavefronts is eight rows of 96 threads, at 256
+    one of eight wavefronts is two rows).  All must
     agree with the checker, with the three-kernel way, under prefix lengths (zero among them), and after a step's
     one-token append."""
     import torch
@@ -409,7 +415,7 @@ def test_block_counts_that_no_run_length_divides(gpu, oracle, cap_blocks, top, s
         gpu.sync()
         got_p = out.cpu().numpy()
         assert gpu.profile_read("kv_decode_attn")[1] == 3
-        assert gpu.profile_read("kv_decode_combine")[1] == (0 if d in (128, 96) else 3)
+        assert gpu.profile_read("kv_decode_combine")[1] == 0
         gpu.decode_tuning(separate_merge=True, separate_query=True)
         three_kernels = run_decode(gpu, cache, q, gpu.GQA_BLOCKED, flags)
     finally:

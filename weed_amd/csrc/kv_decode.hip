@@ -1099,21 +1099,22 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         // merges at the end: 3 to 200 sequences of 100 tokens with groups of eight, 27 us against 22 to 25).
         if (wg_regions == 0 && region_wgs == 0 && mfma_decode_merges(gp, d) && every_sequence_has_tokens &&
             (nb != 0 || (S <= 63 && !tune.always_search)) && n_splits <= 64 &&
-            wg_most_regions <= kMostRegionsMergedByWorkgroup && wg_most_regions * pass_heads <= kMfmaQueryRows &&
+            wg_most_regions <= kMostRegionsMergedByWorkgroup && wg_most_regions * pass_heads <= mfma_query_rows(d) &&
             (size_t)S * Hkv <= kMfmaMergeCounters && !tune.separate_merge) {
             general_merge = true;
         }
         // A workgroup rotates the queries of the regions its blocks lie in itself when they are few enough for its
         // LDS (equal sequences, or the ragged batches above); nothing then runs ahead of the matrix-core kernel.
         fused_query = (wg_regions != 0 || region_wgs != 0 || mfma_decode_merges(gp, d)) && (nb != 0 || general_merge) &&
-                      wg_most_regions * pass_heads <= kMfmaQueryRows && !tune.separate_query;
+                      wg_most_regions * pass_heads <= mfma_query_rows(d) && !tune.separate_query;
     }
     // Workgroups that merge whole regions or whole shares of a region: neighbouring runs take their blocks in turns
     // (see RunGeom), as many cycles' runs together as divide both a workgroup's share and a region, so that no group
     // crosses a region boundary.  (Measured on 1 to 256 sequences of 1024 to 16384 tokens: 1 to 6 % faster with runs
-    // of 4 to 32 blocks, nothing with shorter ones, 1 to 1.5 % slower with runs of 64.)
+    // of 4 to 32 blocks, nothing with shorter ones, 1 to 1.5 % slower with runs of 64.  Not at head_dim 256, where
+    // a block is twice the bytes: 64 sequences of 8192 tokens took 267 us with turns and 232 us without.)
     if ((wg_regions != 0 || region_wgs != 0) && runs.unit_blocks >= kFewestBlocksOfRunsInTurns &&
-        runs.unit_blocks <= kMostBlocksOfRunsInTurns && !tune.contiguous_runs) {
+        runs.unit_blocks <= kMostBlocksOfRunsInTurns && !tune.contiguous_runs && d <= 128) {
         const uint32_t cycle = run_classes(runs) * runs.unit_blocks;
         uint32_t cycles = runs.waves / run_classes(runs);
         while (uniform_blocks % (cycles * cycle) != 0) {

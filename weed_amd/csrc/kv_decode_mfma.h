@@ -164,16 +164,22 @@ struct MfmaQuery {
     int rotate;          // 0: the queries are rotated already
 };
 constexpr uint32_t kMfmaQueryRows = 32;
+// ... of which head_dims above 128 use 16 (their rows are twice as long, and the area is shared with the partials)
+constexpr uint32_t mfma_query_rows(uint32_t d) { return d > 128u ? 16u : kMfmaQueryRows; }
+// Query rows that the kernel rotates in one go: a pass's eight, or (head_dims above 128) all sixteen
+constexpr uint32_t mfma_rotated_query_rows(uint32_t d) { return d > 128u ? 16u : 8u; }
 
 // Instances that can merge: head_dim 64 or 128.
 constexpr bool mfma_decode_merges(uint32_t gp, uint32_t d) { return gp <= 16 && (d == 64u || d == 128u); }
 // Instances whose workgroups can merge whole regions, or whole shares of one region, and rotate their queries
 // (MfmaMerge::wg_regions and region_wgs; not the general case, which is compiled into the other variant of an
 // instance): the above, head_dim 96 where a workgroup has twelve wavefronts, so that its 768 threads are eight
-// rows of 96, and head_dim 32 (two rows per wavefront).  (`waves`: mfma_decode_waves_per_wg.)
+// rows of 96, head_dim 32 (two rows per wavefront), and head_dim 256 with groups of up to eight (a wavefront then
+// takes two of the sixteen 16-column tiles of the small rotations).  (`waves`: mfma_decode_waves_per_wg.)
 constexpr bool mfma_decode_merges_whole_regions(uint32_t gp, uint32_t d, uint32_t waves)
 {
-    return mfma_decode_merges(gp, d) || (gp <= 16 && ((d == 96u && waves == 12u) || d == 32u));
+    return mfma_decode_merges(gp, d) || (gp <= 16 && ((d == 96u && waves == 12u) || d == 32u)) ||
+        (gp <= 8 && d == 256u && waves == 8u);
 }
 // Rows (region, head) that one pass of the merge or of the query rotation takes (the matrix instruction behind both
 // has 16 rows, so a pass reads 8 rows beyond its own), and the LDS of both behind the lookup tables, in words.
@@ -187,13 +193,13 @@ constexpr uint32_t kMfmaMergeRows = 8;
 constexpr uint32_t mfma_merge_partials_words(uint32_t waves, uint32_t gp, uint32_t d)
 {
     const uint32_t partials = waves * gp * (d + 2u);
-    const uint32_t query = (kMfmaQueryRows + 8u) * (d + 4u) + kMfmaMergeRows * d;
+    const uint32_t query = (mfma_query_rows(d) + 8u) * (d + 4u) + mfma_rotated_query_rows(d) * d;
     return partials > query ? partials : query;
 }
 constexpr uint32_t mfma_merge_rows_words(uint32_t d)
 {
     const uint32_t merged = (kMfmaMergeRows + 8u) * (d + 4u) + 2u * kMfmaMergeRows;
-    const uint32_t query = kMfmaQueryRows * d + 2u * kMfmaQueryRows;
+    const uint32_t query = mfma_query_rows(d) * d + 2u * mfma_query_rows(d);
     return (merged > query ? merged : query) + 64u;
 }
 constexpr uint32_t mfma_merge_lds_bytes(uint32_t waves, uint32_t gp, uint32_t d)

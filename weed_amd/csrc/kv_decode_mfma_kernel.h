@@ -398,28 +398,33 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     constexpr bool kRowPerWave = D % 64 == 0;
     float *const part_s = reinterpret_cast<float *>(lds) + ROWS * (kTableRowBytes / 4); // [position][GP][D + 2]
     // The two small rotations (queries ahead of the loop, merged rows behind it) run on the fp32 matrix instruction
-    // v_mfma_f32_16x16x4f32: wavefront w < D / 16 owns the output columns [16 w, 16 w + 16) of up to 16 rows.  Step s of
+    // v_mfma_f32_16x16x4f32: tile w < D / 16 is the output columns [16 w, 16 w + 16) of up to 16 rows.  Step s of
     // D / 4 contracts over the coordinates 4 s + g (g = lane / 16): lane (c, g) supplies row c's coordinate 4 s + g
     // from LDS and the rotation's element [4 s + g][16 w + c], which it holds in a register.  The rows lie in LDS as
     // [row][g][s] with a pitch of D + 4 floats, so that a lane's D / 4 values are contiguous (16-byte reads) and the
     // sixteen rows' reads fall into different banks.
     constexpr uint32_t SG = D / 4;       // steps = coordinates per lane
+    constexpr uint32_t NT = (D / 16 + kWaves - 1) / kWaves; // tiles per wavefront: tile wave + t * kWaves, t < NT
+    constexpr uint32_t kQRows = mfma_query_rows(D);
     constexpr uint32_t RPITCH = D + 4;   // floats per staged row
     auto staged_at = [](uint32_t row, uint32_t j) { return row * RPITCH + (j % 4) * SG + j / 4; };
     // element s of the lane's share of a rotation matrix m (row-major [D][D], out[t] = sum_j in[j] * m[j][t])
-    auto request_matrix = [&](const float *m, float (&x)[kCanMerge ? SG : 1]) {
+    // (Where a wavefront has two tiles, at head_dim 256, it holds one at a time: both together are half of its
+    // registers, and the loop's state lies in the others.)
+    auto request_matrix = [&](const float *m, float (&x)[kCanMerge ? SG : 1], uint32_t t) {
         if constexpr (kCanMerge) {
-            if (wave < D / 16) {
+            const uint32_t tile = wave + t * kWaves;
+            if (tile < D / 16) {
                 const __amdgpu_buffer_rsrc_t rot = buffer_of(m, 4 * D * D);
 #pragma unroll
                 for (uint32_t s_ = 0; s_ < SG; ++s_) {
-                    x[s_] = buffer_f32(rot, 4 * (g * D + 16 * wave + c), 16 * D * s_);
+                    x[s_] = buffer_f32(rot, 4 * (g * D + 16 * tile + c), 16 * D * s_);
                 }
             }
         }
     };
     // rows r0 .. r0 + 15 of `staged` (staged_at layout) times the matrix whose elements the lane holds in x: lane
-    // (c, g), register v of the result = row r0 + 4 g + v, column 16 w + c
+    // (c, g), register v of the result = row r0 + 4 g + v, column 16 * tile + c
     auto rotate_staged = [&](const float *staged, uint32_t r0, const float (&x)[kCanMerge ? SG : 1]) -> float4v {
         float4v acc = { 0.0f, 0.0f, 0.0f, 0.0f };
         if constexpr (kCanMerge) {
@@ -440,7 +445,7 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     auto request_rotation = [&]() {
         if constexpr (kCanMerge) {
             if (p.merge.unrotate) {
-                request_matrix(p.merge.rv, xrot);
+                request_matrix(p.merge.rv, xrot, 0);
             }
         }
     };
@@ -449,14 +454,15 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     // launch and made the kernel 0.4 us slower.)
     // ---- query rotation inside the kernel (see MfmaQuery).  Row (region ri of the workgroup, head slot hs) has index
     //      ri * G + hs.  Requested here: this thread's share of the K rotation and of the raw queries. ----
-    constexpr uint32_t QPT = kQuery ? (kMfmaQueryRows * D + kThreads - 1) / kThreads : 1; // raw query elements per thread
+    constexpr uint32_t QPT = kQuery ? (kQRows * D + kThreads - 1) / kThreads : 1; // raw query elements per thread
     constexpr uint32_t PW = mfma_merge_partials_words(kWaves, GP, D);
     float *const qraw_s = part_s;                                       // [rows (+ 8 that a tile of 16 reaches into)] staged
-    float *const qrot_s = part_s + (kMfmaQueryRows + 8) * RPITCH;       // [kMfmaMergeRows][D] rotated rows of a pass
+    constexpr uint32_t kRotatedRows = mfma_rotated_query_rows(D);
+    float *const qrot_s = part_s + (kQRows + 8) * RPITCH;       // [kRotatedRows][D] rotated rows of a pass
     uint16_t *const qh_s = reinterpret_cast<uint16_t *>(part_s + PW); // [rows][D] fp16 high halves
-    uint16_t *const ql_s = qh_s + kMfmaQueryRows * D;                 // [rows][D] low halves
-    float *const qscale_s = part_s + PW + kMfmaQueryRows * D;         // [rows]
-    float *const qsum_s = qscale_s + kMfmaQueryRows;                  // [rows]
+    uint16_t *const ql_s = qh_s + kQRows * D;                 // [rows][D] low halves
+    float *const qscale_s = part_s + PW + kQRows * D;         // [rows]
+    float *const qsum_s = qscale_s + kQRows;                  // [rows]
     const bool fused_q = kQuery && p.query.q != nullptr;
     // ---- general merge (see MfmaMerge): in a ragged batch every wavefront keeps the prefix sums of the sequences'
     //      block counts in a register, lane i the blocks ahead of sequence i (lanes from n_seq on: all blocks) ----
@@ -531,7 +537,7 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
       if constexpr (kQuery) {
         if (fused_q) {
             if (p.query.rotate) {
-                request_matrix(p.query.rot_t, xq);
+                request_matrix(p.query.rot_t, xq, 0);
             }
             const uint32_t n_regions = p.n_seq * p.Hkv;
             // element e = tid + i * kThreads of the rows: its row is the same in all lanes of a wavefront (kThreads is
@@ -566,7 +572,7 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
 #pragma unroll
             for (uint32_t i = 0; i < QPT; ++i) {
                 const uint32_t e = tid + i * kThreads;
-                if (e < kMfmaQueryRows * D) {
+                if (e < kQRows * D) {
                     qraw_s[staged_at(e / D, e % D)] = qr[i];
                 }
             }
@@ -576,12 +582,22 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
             }
             for (uint32_t r0 = 0; r0 < wg_rows; r0 += kMfmaMergeRows) {
                 if (p.query.rotate) {
-                    if (wave < D / 16) {
-                        const float4v rot = rotate_staged(qraw_s, r0, xq);
-                        if (g < kMfmaMergeRows / 4) {
+                    // (with two tiles per wavefront: all sixteen rows in the first pass, tile after tile)
+                    if (NT == 1 || r0 == 0) {
 #pragma unroll
-                            for (uint32_t v = 0; v < 4; ++v) {
-                                qrot_s[(4 * g + v) * D + 16 * wave + c] = rot[v];
+                        for (uint32_t t = 0; t < NT; ++t) {
+                            const uint32_t tile = wave + t * kWaves;
+                            if (t > 0) {
+                                request_matrix(p.query.rot_t, xq, t);
+                            }
+                            if (tile < D / 16) {
+                                const float4v rot = rotate_staged(qraw_s, r0, xq);
+                                if (g < kRotatedRows / 4) {
+#pragma unroll
+                                    for (uint32_t v = 0; v < 4; ++v) {
+                                        qrot_s[(4 * g + v) * D + 16 * tile + c] = rot[v];
+                                    }
+                                }
                             }
                         }
                     }
@@ -598,7 +614,7 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
                         const uint32_t j = lane + 64 * cc;
                         float v = 0.0f;
                         if (D % 64 == 0 || j < D) {
-                            v = p.query.rotate ? qrot_s[wave * D + j] : qraw_s[staged_at(row, j)];
+                            v = p.query.rotate ? qrot_s[(NT == 1 ? wave : row) * D + j] : qraw_s[staged_at(row, j)];
                         }
                         a[cc] = v;
                         const float qc = v * k;
@@ -1242,12 +1258,19 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
                 }
             };
             if (p.merge.unrotate) {
-                if (wave < D / 16) {
-                    const float4v out = rotate_staged(o_s, 0, xrot);
-                    if (g < RP / 4) {
 #pragma unroll
-                        for (uint32_t v = 0; v < 4; ++v) {
-                            store_row(4 * g + v, 16 * wave + c, out[v]);
+                for (uint32_t t = 0; t < NT; ++t) {
+                    const uint32_t tile = wave + t * kWaves;
+                    if (NT > 1 && (t > 0 || r0 > 0)) {
+                        request_matrix(p.merge.rv, xrot, t); // (the first pass's first tile is there, see request_rotation)
+                    }
+                    if (tile < D / 16) {
+                        const float4v out = rotate_staged(o_s, 0, xrot);
+                        if (g < RP / 4) {
+#pragma unroll
+                            for (uint32_t v = 0; v < 4; ++v) {
+                                store_row(4 * g + v, 16 * tile + c, out[v]);
+                            }
                         }
                     }
                 }
