@@ -158,20 +158,24 @@ template <int RT, int THREADS> __global__ void __launch_bounds__(THREADS) softma
     }
 }
 
-// Softmax along a strided axis of at most kStridedCached * (kStridedThreads / RT) elements: RT neighbouring rows per
+// Softmax along a strided axis of at most kStridedCached * (THREADS / RT) elements: RT neighbouring rows per
 // workgroup, every thread keeps its share of a row in registers (all loads in flight at once), so the data is read
 // once and each element costs one exponential.
 constexpr int kStridedCached = 64;
 constexpr int kStridedThreads = 512;
+constexpr int kStridedThreadsLong = 1024; // (few rows of up to 8192 or 16384 elements: 8 or 4 rows per workgroup)
 
-template <int RT>
-__global__ void __launch_bounds__(kStridedThreads) softmax_strided_cached_kernel(const float *__restrict__ a,
+// (SPREAD, for tiles narrower than a 128-byte line: the grid is eight equal shares and workgroup b takes tile b / 8 of
+// share b % 8, so that the workgroups which complete each other's lines run at the same time behind the same L2.)
+template <int RT, int THREADS = 512, bool SPREAD = false>
+__global__ void __launch_bounds__(THREADS) softmax_strided_cached_kernel(const float *__restrict__ a,
                                                                       float *__restrict__ out, AxisGeom g)
 {
-    __shared__ float red[kStridedThreads];
-    constexpr int NY = kStridedThreads / RT;
+    __shared__ float red[THREADS];
+    constexpr int NY = THREADS / RT;
     const uint32_t tx = threadIdx.x % RT, ty = threadIdx.x / RT;
-    const uint32_t row = blockIdx.x * RT + tx;
+    const uint32_t tile = SPREAD ? (blockIdx.x % 8U) * (gridDim.x / 8U) + blockIdx.x / 8U : blockIdx.x;
+    const uint32_t row = tile * RT + tx;
     const bool valid = row < g.rows;
     uint64_t a_base = 0, o_base = 0;
     if (valid) {
@@ -200,13 +204,13 @@ __global__ void __launch_bounds__(kStridedThreads) softmax_strided_cached_kernel
     for (int c = 0; c < kStridedCached; ++c) {
         m = fmaxf(m, x[c]);
     }
-    m = block_reduce<1, RT, kStridedThreads>(m, red);
+    m = block_reduce<1, RT, THREADS>(m, red);
 #pragma unroll
     for (int c = 0; c < kStridedCached; ++c) {
         x[c] = expf(x[c] - m);
         s += x[c];
     }
-    s = block_reduce<0, RT, kStridedThreads>(s, red);
+    s = block_reduce<0, RT, THREADS>(s, red);
 #pragma unroll
     for (int c = 0; c < kStridedCached; ++c) {
         const uint32_t j = ty + c * NY;
@@ -1072,6 +1076,15 @@ int weed_hip_softmax_f32(uint32_t rank, const uint32_t *shape, uint32_t axis, co
         softmax_strided_cached_kernel<32><<<(g.rows + 31) / 32, kStridedThreads, 0, stream()>>>(a_dev, out_dev, g);
     } else if (g.axis_len <= (uint32_t)(kStridedCached * kStridedThreads / 16)) {
         softmax_strided_cached_kernel<16><<<(g.rows + 15) / 16, kStridedThreads, 0, stream()>>>(a_dev, out_dev, g);
+    } else if (g.rows < 2048U && g.axis_len <= (uint32_t)(kStridedCached * kStridedThreadsLong / 4)) {
+        // few long rows (scores of a decode step): narrow tiles, so that there are workgroups enough, and one pass
+        // (64 to 1024 rows of 8192: 22 to 42 us, where 16 rows per workgroup and two passes take 60 to 70)
+        softmax_strided_cached_kernel<4, kStridedThreadsLong, true>
+            <<<8 * ((g.rows + 31) / 32), kStridedThreadsLong, 0, stream()>>>(a_dev, out_dev, g);
+    } else if (g.rows < 3072U && g.axis_len <= (uint32_t)(kStridedCached * kStridedThreadsLong / 8)) {
+        // (2048 rows of 8192: 49 us against 75; from 3072 rows on the two passes over 16 or 32 rows are as fast or faster)
+        softmax_strided_cached_kernel<8, kStridedThreadsLong, true>
+            <<<8 * ((g.rows + 63) / 64), kStridedThreadsLong, 0, stream()>>>(a_dev, out_dev, g);
     } else if (how == AXIS_ROWS32) {
         softmax_kernel<32, 256><<<(g.rows + 31) / 32, 256, 0, stream()>>>(a_dev, out_dev, g);
     } else if (how == AXIS_ROWS32_WIDE) {
