@@ -263,12 +263,14 @@ def test_softmax_and_reduce_strided_against_checker(gpu, oracle, shape):
 
 @pytest.mark.parametrize("shape,axis", [((9004, 40), 0), ((40000, 24), 1), ((64, 8, 1, 700), 3), ((260, 3, 5), 0),
                                         ((192, 1100), 0), ((2044, 1030), 0), ((67, 1500), 0), ((1101, 1200), 0),
-                                        ((300, 9000), 1), ((2060, 5000), 1)])
+                                        ((300, 9000), 1), ((2060, 5000), 1),
+                                        ((8200, 300), 1), ((12300, 1100), 1)])
 def test_softmax_and_reduce_launch_shapes(gpu, shape, axis):
     """One case per way the threads are spread: a contiguous row longer than what the registers keep between the
     passes, enough rows for 32 per workgroup, few long strided rows (decode-time scores), a short aligned row, and
     many short contiguous rows (one wavefront each: aligned, longer than a wavefront's registers, unaligned lengths),
-    and few strided rows of 9000 and 5000 elements, which 4 and 8 neighbouring rows per workgroup keep in registers.
+    few strided rows of 9000 and 5000 elements, which 4 and 8 neighbouring rows per workgroup keep in registers,
+    and many strided rows of 300 (kept in 32 registers per thread) and of 1100 elements (two passes).
     Some positions are masked with -inf, one row of the decode case entirely (its softmax is NaN, as in numpy)."""
     import torch
     rng = np.random.default_rng(shape[0] + axis)

@@ -167,7 +167,7 @@ constexpr int kStridedThreadsLong = 1024; // (few rows of up to 8192 or 16384 el
 
 // (SPREAD, for tiles narrower than a 128-byte line: the grid is eight equal shares and workgroup b takes tile b / 8 of
 // share b % 8, so that the workgroups which complete each other's lines run at the same time behind the same L2.)
-template <int RT, int THREADS = 512, bool SPREAD = false>
+template <int RT, int THREADS = 512, bool SPREAD = false, int CACHED = kStridedCached>
 __global__ void __launch_bounds__(THREADS) softmax_strided_cached_kernel(const float *__restrict__ a,
                                                                       float *__restrict__ out, AxisGeom g)
 {
@@ -186,33 +186,33 @@ __global__ void __launch_bounds__(THREADS) softmax_strided_cached_kernel(const f
     // rows past the end read row 0's first element (any readable address) and are discarded
     const float *ap = a + (valid ? a_base : (uint64_t)g.a_off);
     float *op = out + o_base;
-    float x[kStridedCached];
+    float x[CACHED];
     // unconditional loads of clamped positions (the host checks that the row's span fits 32 bits), then the select
     const uint32_t last = len ? len - 1U : 0U;
 #pragma unroll
-    for (int c = 0; c < kStridedCached; ++c) {
+    for (int c = 0; c < CACHED; ++c) {
         const uint32_t j = ty + c * NY;
         x[c] = ap[min(j, last) * as];
     }
 #pragma unroll
-    for (int c = 0; c < kStridedCached; ++c) {
+    for (int c = 0; c < CACHED; ++c) {
         const uint32_t j = ty + c * NY;
         x[c] = j < len ? x[c] : -INFINITY;
     }
     float m = -INFINITY, s = 0.0f;
 #pragma unroll
-    for (int c = 0; c < kStridedCached; ++c) {
+    for (int c = 0; c < CACHED; ++c) {
         m = fmaxf(m, x[c]);
     }
     m = block_reduce<1, RT, THREADS>(m, red);
 #pragma unroll
-    for (int c = 0; c < kStridedCached; ++c) {
+    for (int c = 0; c < CACHED; ++c) {
         x[c] = expf(x[c] - m);
         s += x[c];
     }
     s = block_reduce<0, RT, THREADS>(s, red);
 #pragma unroll
-    for (int c = 0; c < kStridedCached; ++c) {
+    for (int c = 0; c < CACHED; ++c) {
         const uint32_t j = ty + c * NY;
         if (j < len) {
             op[(uint64_t)j * os] = x[c] / s;
@@ -1072,9 +1072,20 @@ int weed_hip_softmax_f32(uint32_t rank, const uint32_t *shape, uint32_t axis, co
         softmax_kernel<1, 256><<<g.rows, 256, 0, stream()>>>(a_dev, out_dev, g);
     } else if ((uint64_t)g.axis_len * g.a_stride[axis] >= (1ull << 32)) {
         softmax_kernel<16, 1024><<<(g.rows + 15) / 16, 1024, 0, stream()>>>(a_dev, out_dev, g);
+    } else if (g.axis_len <= 16U * kStridedThreads / 32 && g.rows >= 32U * 256U) {
+        // (short axes keep fewer registers per thread, so that more workgroups share a compute unit and their
+        // loads, sums and stores overlap: 2^18 rows of 512 at 4.2 TB/s of algorithmic bytes with 32 registers,
+        // 2.9 with 64; 2^19 rows of 256 at 4.1 with 16)
+        softmax_strided_cached_kernel<32, kStridedThreads, false, 16>
+            <<<(g.rows + 31) / 32, kStridedThreads, 0, stream()>>>(a_dev, out_dev, g);
+    } else if (g.axis_len <= 32U * kStridedThreads / 32 && g.rows >= 32U * 256U) {
+        softmax_strided_cached_kernel<32, kStridedThreads, false, 32>
+            <<<(g.rows + 31) / 32, kStridedThreads, 0, stream()>>>(a_dev, out_dev, g);
     } else if (g.axis_len <= (uint32_t)(kStridedCached * kStridedThreads / 32) && g.rows >= 32U * 256U) {
         softmax_strided_cached_kernel<32><<<(g.rows + 31) / 32, kStridedThreads, 0, stream()>>>(a_dev, out_dev, g);
-    } else if (g.axis_len <= (uint32_t)(kStridedCached * kStridedThreads / 16)) {
+    } else if (g.axis_len <= (uint32_t)(kStridedCached * kStridedThreads / 16) && g.rows < 12288U) {
+        // (with more rows the two passes over 32 rows per workgroup are faster: 16-row tiles are half lines.
+        // 4096 rows of 2048: 22 us against 35; 16384 rows: 83 against 72; 65536 rows: 427 against 369)
         softmax_strided_cached_kernel<16><<<(g.rows + 15) / 16, kStridedThreads, 0, stream()>>>(a_dev, out_dev, g);
     } else if (g.rows < 2048U && g.axis_len <= (uint32_t)(kStridedCached * kStridedThreadsLong / 4)) {
         // few long rows (scores of a decode step): narrow tiles, so that there are workgroups enough, and one pass
