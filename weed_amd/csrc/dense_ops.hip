@@ -16,7 +16,6 @@ using namespace weedhip;
 namespace {
 
 constexpr int kMaxRank = 8;
-constexpr int kThreads = 256;
 
 struct AxisGeom {
     uint32_t rank;
@@ -96,6 +95,27 @@ __device__ __forceinline__ void softmax_accumulate(float &m, float &s, float x)
     }
 }
 
+// The same for N elements at once: their maximum first, then one exponential per element (and one more where the
+// running maximum rises), instead of a branch with an exponential on either side per element.
+template <int N> __device__ __forceinline__ void softmax_accumulate(float &m, float &s, const float (&x)[N])
+{
+    float top = x[0];
+#pragma unroll
+    for (int u = 1; u < N; ++u) {
+        top = fmaxf(top, x[u]);
+    }
+    if (top > m) {
+        s *= expf(m - top); // (m = -inf: s is 0 and stays 0)
+        m = top;
+    }
+    if (m > -INFINITY) {
+#pragma unroll
+        for (int u = 0; u < N; ++u) {
+            s += expf(x[u] - m);
+        }
+    }
+}
+
 // Merge the per-thread (m, s) pairs of the threads that share a row; returns the row's (max, sum) in every thread.
 template <int RT, int THREADS> __device__ __forceinline__ void softmax_merge(float &m, float &s, float *red)
 {
@@ -135,12 +155,10 @@ template <int RT, int THREADS> __global__ void __launch_bounds__(THREADS) softma
             const uint32_t j = j0 + u * NY;
             x[u] = j < len ? ap[(uint64_t)j * as] : -INFINITY;
         }
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            softmax_accumulate(m, s, x[u]);
-        }
+        softmax_accumulate(m, s, x);
     }
     softmax_merge<RT, THREADS>(m, s, red);
+    const float inv = 1.0f / s; // (s >= 1 wherever the row has a finite element)
     for (uint32_t j0 = ty; j0 < len; j0 += NY * U) {
         float x[U];
 #pragma unroll
@@ -152,7 +170,7 @@ template <int RT, int THREADS> __global__ void __launch_bounds__(THREADS) softma
         for (int u = 0; u < U; ++u) {
             const uint32_t j = j0 + u * NY;
             if (j < len) {
-                op[(uint64_t)j * os] = expf(x[u] - m) / s;
+                op[(uint64_t)j * os] = expf(x[u] - m) * inv;
             }
         }
     }
@@ -211,11 +229,12 @@ __global__ void __launch_bounds__(THREADS) softmax_strided_cached_kernel(const f
         s += x[c];
     }
     s = block_reduce<0, RT, THREADS>(s, red);
+    const float inv = 1.0f / s;
 #pragma unroll
     for (int c = 0; c < CACHED; ++c) {
         const uint32_t j = ty + c * NY;
         if (j < len) {
-            op[(uint64_t)j * os] = x[c] / s;
+            op[(uint64_t)j * os] = x[c] * inv;
         }
     }
 }
@@ -254,41 +273,39 @@ __global__ void __launch_bounds__(THREADS) softmax_contiguous_kernel(const float
             s += (cache[c].x + cache[c].y) + (cache[c].z + cache[c].w);
         }
         s = block_reduce<0, 1, THREADS>(s, red);
+        const float inv = 1.0f / s;
 #pragma unroll
         for (int c = 0; c < CACHED; ++c) {
             const uint32_t idx = threadIdx.x + c * THREADS;
             if (idx < n4) {
-                op[idx] = make_float4(cache[c].x / s, cache[c].y / s, cache[c].z / s, cache[c].w / s);
+                op[idx] = make_float4(cache[c].x * inv, cache[c].y * inv, cache[c].z * inv, cache[c].w * inv);
             }
         }
         return;
     }
 #pragma unroll
     for (int c = 0; c < CACHED; ++c) {
-        softmax_accumulate(m, s, cache[c].x);
-        softmax_accumulate(m, s, cache[c].y);
-        softmax_accumulate(m, s, cache[c].z);
-        softmax_accumulate(m, s, cache[c].w);
+        const float v4[4] = { cache[c].x, cache[c].y, cache[c].z, cache[c].w };
+        softmax_accumulate(m, s, v4);
     }
     for (uint32_t idx = threadIdx.x + CACHED * THREADS; idx < n4; idx += THREADS) {
         const float4 v = ap[idx];
-        softmax_accumulate(m, s, v.x);
-        softmax_accumulate(m, s, v.y);
-        softmax_accumulate(m, s, v.z);
-        softmax_accumulate(m, s, v.w);
+        const float v4[4] = { v.x, v.y, v.z, v.w };
+        softmax_accumulate(m, s, v4);
     }
     softmax_merge<1, THREADS>(m, s, red);
+    const float inv = 1.0f / s;
 #pragma unroll
     for (int c = 0; c < CACHED; ++c) {
         const uint32_t idx = threadIdx.x + c * THREADS;
         if (idx < n4) {
             const float4 v = cache[c];
-            op[idx] = make_float4(expf(v.x - m) / s, expf(v.y - m) / s, expf(v.z - m) / s, expf(v.w - m) / s);
+            op[idx] = make_float4(expf(v.x - m) * inv, expf(v.y - m) * inv, expf(v.z - m) * inv, expf(v.w - m) * inv);
         }
     }
     for (uint32_t idx = threadIdx.x + CACHED * THREADS; idx < n4; idx += THREADS) {
         const float4 v = ap[idx];
-        op[idx] = make_float4(expf(v.x - m) / s, expf(v.y - m) / s, expf(v.z - m) / s, expf(v.w - m) / s);
+        op[idx] = make_float4(expf(v.x - m) * inv, expf(v.y - m) * inv, expf(v.z - m) * inv, expf(v.w - m) * inv);
     }
 }
 
@@ -352,16 +369,17 @@ __global__ void __launch_bounds__(256) softmax_wave_rows_kernel(const float *__r
                 }
             }
             s = wave_reduce<0>(s);
+            const float inv = 1.0f / s;
 #pragma unroll
             for (int c = 0; c < CACHED; ++c) {
                 const uint32_t idx = lane + 64U * c;
                 if (idx < nvec) {
                     if (V == 4) {
-                        reinterpret_cast<float4 *>(op)[idx] = make_float4(cache[c][0] / s, cache[c][V > 1 ? 1 : 0] / s,
-                                                                          cache[c][V > 2 ? 2 : 0] / s,
-                                                                          cache[c][V > 3 ? 3 : 0] / s);
+                        reinterpret_cast<float4 *>(op)[idx] = make_float4(cache[c][0] * inv, cache[c][V > 1 ? 1 : 0] * inv,
+                                                                          cache[c][V > 2 ? 2 : 0] * inv,
+                                                                          cache[c][V > 3 ? 3 : 0] * inv);
                     } else {
-                        op[idx] = cache[c][0] / s;
+                        op[idx] = cache[c][0] * inv;
                     }
                 }
             }
@@ -369,37 +387,37 @@ __global__ void __launch_bounds__(256) softmax_wave_rows_kernel(const float *__r
         }
 #pragma unroll
         for (int c = 0; c < CACHED; ++c) {
-#pragma unroll
-            for (int e = 0; e < V; ++e) {
-                softmax_accumulate(m, s, cache[c][e]);
-            }
+            softmax_accumulate(m, s, cache[c]);
         }
         for (uint32_t idx = lane + 64U * CACHED; idx < nvec; idx += 64U) {
+            float v[V];
 #pragma unroll
             for (int e = 0; e < V; ++e) {
-                softmax_accumulate(m, s, ap[(uint64_t)idx * V + e]);
+                v[e] = ap[(uint64_t)idx * V + e];
             }
+            softmax_accumulate(m, s, v);
         }
         const float row_max = wave_reduce<1>(m);
         const float total = wave_reduce<0>((m > -INFINITY) ? s * expf(m - row_max) : 0.0f);
+        const float inv = 1.0f / total;
 #pragma unroll
         for (int c = 0; c < CACHED; ++c) {
             const uint32_t idx = lane + 64U * c;
             if (idx < nvec) {
                 if (V == 4) {
                     reinterpret_cast<float4 *>(op)[idx] =
-                        make_float4(expf(cache[c][0] - row_max) / total, expf(cache[c][V > 1 ? 1 : 0] - row_max) / total,
-                                    expf(cache[c][V > 2 ? 2 : 0] - row_max) / total,
-                                    expf(cache[c][V > 3 ? 3 : 0] - row_max) / total);
+                        make_float4(expf(cache[c][0] - row_max) * inv, expf(cache[c][V > 1 ? 1 : 0] - row_max) * inv,
+                                    expf(cache[c][V > 2 ? 2 : 0] - row_max) * inv,
+                                    expf(cache[c][V > 3 ? 3 : 0] - row_max) * inv);
                 } else {
-                    op[idx] = expf(cache[c][0] - row_max) / total;
+                    op[idx] = expf(cache[c][0] - row_max) * inv;
                 }
             }
         }
         for (uint32_t idx = lane + 64U * CACHED; idx < nvec; idx += 64U) {
 #pragma unroll
             for (int e = 0; e < V; ++e) {
-                op[(uint64_t)idx * V + e] = expf(ap[(uint64_t)idx * V + e] - row_max) / total;
+                op[(uint64_t)idx * V + e] = expf(ap[(uint64_t)idx * V + e] - row_max) * inv;
             }
         }
     }
