@@ -282,6 +282,8 @@ def test_equal_contexts_with_and_without_the_region_search(gpu, oracle):
     (False, 256, 2, 16, 2, 1024, 4, 4, 16, True),   # ... with rotations: two passes of eight rows each
     (True, 256, 1, 4, 1, 4096, 3, 4, 64, True),     # eight workgroups per region
     (True, 240, 2, 16, 1, 2048, 3, 4, 32, True),    # head_dim 240, groups of 8, two workgroups per region
+    (True, 256, 2, 8, 2, 1024, 2, 2, 16, True),     # head_dim 256, 2-bit codes on both sides
+    (False, 256, 2, 4, 2, 2048, 4, 2, 32, False),   # head_dim 256, uniform 4-bit K and 2-bit V, no rotations
 ])
 def test_workgroups_that_merge_their_own_regions(gpu, oracle, lloyd, d, Hkv, Hq, S, L, kb, vb, waves, rot):
     """When every workgroup of the matrix-core kernel holds whole regions, or every region a whole number of
