@@ -68,6 +68,26 @@ def test_noalloc_matches_decode_attn_on_two_calls_in_a_row(gpu, oracle):
     cache_b.close()
 
 
+def test_noalloc_head_dim_256_whole_regions_per_workgroup(gpu, oracle):
+    """A batch of equal sequences at head_dim 256, which is one kernel (the workgroups rotate their queries and merge
+    their partials themselves): the same bits from both entry points, and the checker's values."""
+    flags = gpu.ATTN_ROTATE_Q | gpu.ATTN_UNROTATE_OUT
+    wl = workloads.Workload("noalloc_256", 4, 8, 2, 256, [1024] * 4, 3, 4, 0, 0, 23)
+    cache, q, Rk, Rv = _cache(gpu, oracle, wl, 7)
+    try:
+        gpu.decode_tuning(32)
+        ref, out = _both(gpu, cache, q, flags)
+    finally:
+        gpu.decode_tuning()
+    assert np.array_equal(ref, out)
+    kspec, vspec = coder_specs(oracle, cache)
+    kf, ka = export(cache, 0, wl.max_len)
+    vf, va = export(cache, 1, wl.max_len)
+    want = oracle.decode_attn(kspec, vspec, kf, ka, vf, va, q, wl.lens, gqa_weed=False, Rk=Rk, Rv=Rv)
+    assert_attn_close(out, want, "noalloc at head_dim 256 vs checker")
+    cache.close()
+
+
 def test_noalloc_refuses_shapes_beyond_its_workspace(gpu):
     import torch
     # 1024 sequences x 64 heads x 128: the rotated queries alone are 32 MiB, the size of the static workspace
