@@ -76,7 +76,7 @@ def test_matmul_matrix_core_layouts(gpu, oracle, a_col, b_col, o_col):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (1, 100, 260), (5, 33, 1000), (16, 48, 256), (17, 16, 4100),
-                                   (33, 250, 516), (64, 512, 1024)])
+                                   (33, 250, 516), (64, 512, 1024), (24, 600, 1100), (50, 1040, 772)])
 def test_matmul_decode_projections(gpu, oracle, M, N, K):
     """Few rows against a tall column-major weight (y = x.W at decode time, the matrix-core streaming kernel):
     row counts on both sides of the 16-row tiles, column counts that are not multiples of 16, k ranges that do not

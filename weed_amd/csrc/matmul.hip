@@ -494,7 +494,7 @@ __device__ __forceinline__ void split_eight(const float (&v)[8], uint4w (&part)[
     }
 }
 
-template <int MT>
+template <int MT, bool AK = false> // AK: the rows of a are contiguous along k (a_s1 == 1), 16-byte aligned
 __global__ void __launch_bounds__(64 * kWideWaves)
     matmul_skinny_wide_kernel(const float *__restrict__ a, const float *__restrict__ b, float *__restrict__ part,
                               MatGeom g, uint32_t k_per_split)
@@ -529,15 +529,27 @@ __global__ void __launch_bounds__(64 * kWideWaves)
     // the matrix instructions contract: instruction j of a step contracts, in lane group grp, over the k
     // 32 j + 4 grp .. + 3 and 32 j + 16 + 4 grp .. + 3 (what the lane's loads 2 j and 2 j + 1 of b hold), so k =
     // 32 j + 16 h + 4 grp + e sits at position 32 j + 8 grp + 4 h + e and a lane's eight values are one 16-byte read.
+    // (With rows that are contiguous along k the eight lanes of a row's octets are neighbours and fetch 256 consecutive
+    // bytes with two 16-byte loads each; else the lanes of an octet are 64 neighbouring rows, eight 4-byte loads each.)
     constexpr uint32_t kRows = 16 * MT;
-    const uint32_t srow = tid % kRows, soct = tid / kRows;
-    const bool stager = soct < 8;
+    const uint32_t srow = AK ? tid / 8 : tid % kRows, soct = AK ? tid % 8 : tid / kRows;
+    const bool stager = AK ? srow < kRows : soct < 8;
     const float *arow = a + (uint64_t)g.a_off + (uint64_t)(srow < g.M ? srow : 0) * g.a_s0;
     auto fetch_rows = [&](uint32_t kb, float (&v)[8]) {
+        if constexpr (AK) {
+            const uint32_t k = kb + 8 * soct;
+            const bool ok = stager && srow < g.M && k < kb1; // (K is a multiple of 4; a range ends on a multiple of 64 or at K)
+            const float4v lo = ok ? *reinterpret_cast<const float4v *>(arow + k) : float4v{ 0.0f, 0.0f, 0.0f, 0.0f };
+            const float4v hi = (ok && k + 4 < kb1) ? *reinterpret_cast<const float4v *>(arow + k + 4)
+                                                    : float4v{ 0.0f, 0.0f, 0.0f, 0.0f };
+            v[0] = lo[0], v[1] = lo[1], v[2] = lo[2], v[3] = lo[3];
+            v[4] = hi[0], v[5] = hi[1], v[6] = hi[2], v[7] = hi[3];
+        } else {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const uint32_t k = kb + 8 * soct + e;
-            v[e] = (stager && srow < g.M && k < kb1) ? arow[(uint64_t)k * g.a_s1] : 0.0f;
+            for (int e = 0; e < 8; ++e) {
+                const uint32_t k = kb + 8 * soct + e;
+                v[e] = (stager && srow < g.M && k < kb1) ? arow[(uint64_t)k * g.a_s1] : 0.0f;
+            }
         }
     };
     auto store_rows = [&](int buf, const float (&v)[8]) {
@@ -773,8 +785,15 @@ int launch_matmul(const char *fn, const MatGeom &g, uint32_t batch, const float 
             splits = (K + k_per_split - 1) / k_per_split;
             WEED_HIP_TRY(grow_split_scratch(fn, sizeof(float) * (size_t)splits * M * N));
             const dim3 wide(col_wgs, splits, 1);
+            const bool a_k = g.a_s1 == 1 && (g.a_s0 & 3) == 0 && aligned16(a_dev, g.a_off);
             if (M <= 32) {
-                matmul_skinny_wide_kernel<2><<<wide, 64 * kWideWaves, 0, stream()>>>(a_dev, b_dev, g_split_ws, g, k_per_split);
+                if (a_k) {
+                    matmul_skinny_wide_kernel<2, true><<<wide, 64 * kWideWaves, 0, stream()>>>(a_dev, b_dev, g_split_ws, g, k_per_split);
+                } else {
+                    matmul_skinny_wide_kernel<2><<<wide, 64 * kWideWaves, 0, stream()>>>(a_dev, b_dev, g_split_ws, g, k_per_split);
+                }
+            } else if (a_k) {
+                matmul_skinny_wide_kernel<4, true><<<wide, 64 * kWideWaves, 0, stream()>>>(a_dev, b_dev, g_split_ws, g, k_per_split);
             } else {
                 matmul_skinny_wide_kernel<4><<<wide, 64 * kWideWaves, 0, stream()>>>(a_dev, b_dev, g_split_ws, g, k_per_split);
             }
