@@ -282,6 +282,12 @@ def test_equal_contexts_with_and_without_the_region_search(gpu, oracle):
     (False, 256, 2, 16, 2, 1024, 4, 4, 16, True),   # ... with rotations: two passes of eight rows each
     (True, 256, 1, 4, 1, 4096, 3, 4, 64, True),     # eight workgroups per region
     (True, 240, 2, 16, 1, 2048, 3, 4, 32, True),    # head_dim 240, groups of 8, two workgroups per region
+    # head_dims 160, 192 and 224: the workgroup's 512 threads are not whole rows, those behind the last whole row idle
+    (True, 192, 2, 8, 4, 1024, 3, 4, 32, True),     # head_dim 192, two regions per workgroup
+    (True, 160, 2, 16, 2, 1024, 3, 4, 16, True),    # head_dim 160, groups of 8, 16 rows per workgroup
+    (False, 224, 1, 4, 1, 4096, 4, 4, 64, True),    # head_dim 224, uniform coder, eight workgroups per region
+    (True, 200, 2, 8, 1, 2048, 3, 4, 32, False),    # head_dim 200 (stored as 224), two workgroups per region, no rotations
+    (True, 176, 1, 4, 5, 1024, 2, 3, 40, True),     # head_dim 176 (stored as 192), the last workgroup holds one region of its two
     (True, 256, 2, 8, 2, 1024, 2, 2, 16, True),     # head_dim 256, 2-bit codes on both sides
     (False, 256, 2, 4, 2, 2048, 4, 2, 32, False),   # head_dim 256, uniform 4-bit K and 2-bit V, no rotations
 ])

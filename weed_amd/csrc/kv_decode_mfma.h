@@ -174,12 +174,13 @@ constexpr bool mfma_decode_merges(uint32_t gp, uint32_t d) { return gp <= 16 && 
 // Instances whose workgroups can merge whole regions, or whole shares of one region, and rotate their queries
 // (MfmaMerge::wg_regions and region_wgs; not the general case, which is compiled into the other variant of an
 // instance): the above, head_dim 96 where a workgroup has twelve wavefronts, so that its 768 threads are eight
-// rows of 96, head_dim 32 (two rows per wavefront), and head_dim 256 with groups of up to eight (a wavefront then
-// takes two of the sixteen 16-column tiles of the small rotations).  (`waves`: mfma_decode_waves_per_wg.)
+// rows of 96, head_dim 32 (two rows per wavefront), and head_dims 160 to 256 with groups of up to eight (a wavefront
+// then takes two of the ten to sixteen 16-column tiles of the small rotations; at 160, 192 and 224 the threads
+// behind the last whole row idle where a thread is a column).  (`waves`: mfma_decode_waves_per_wg.)
 constexpr bool mfma_decode_merges_whole_regions(uint32_t gp, uint32_t d, uint32_t waves)
 {
     return mfma_decode_merges(gp, d) || (gp <= 16 && ((d == 96u && waves == 12u) || d == 32u)) ||
-        (gp <= 8 && d == 256u && waves == 8u);
+        (gp <= 8 && d > 128u && d <= 256u && waves == 8u);
 }
 // Rows (region, head) that one pass of the merge or of the query rotation takes (the matrix instruction behind both
 // has 16 rows, so a pass reads 8 rows beyond its own), and the LDS of both behind the lookup tables, in words.

@@ -454,7 +454,11 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     // launch and made the kernel 0.4 us slower.)
     // ---- query rotation inside the kernel (see MfmaQuery).  Row (region ri of the workgroup, head slot hs) has index
     //      ri * G + hs.  Requested here: this thread's share of the K rotation and of the raw queries. ----
-    constexpr uint32_t QPT = kQuery ? (kQRows * D + kThreads - 1) / kThreads : 1; // raw query elements per thread
+    // Where a thread is a column of a row (the raw queries, the merged rows), the workgroup's first kRowsAtOnce * D
+    // threads are kRowsAtOnce whole rows; at head_dims that do not divide the threads (160, 192, 224) the rest idle.
+    constexpr uint32_t kRowsAtOnce = kThreads / D;
+    const bool row_thread = tid < kRowsAtOnce * D;
+    constexpr uint32_t QPT = kQuery ? (kQRows + kRowsAtOnce - 1) / kRowsAtOnce : 1; // raw query elements per thread
     constexpr uint32_t PW = mfma_merge_partials_words(kWaves, GP, D);
     float *const qraw_s = part_s;                                       // [rows (+ 8 that a tile of 16 reaches into)] staged
     constexpr uint32_t kRotatedRows = mfma_rotated_query_rows(D);
@@ -540,16 +544,16 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
                 request_matrix(p.query.rot_t, xq, 0);
             }
             const uint32_t n_regions = p.n_seq * p.Hkv;
-            // element e = tid + i * kThreads of the rows: its row is the same in all lanes of a wavefront (kThreads is
-            // a multiple of D), so the row's address arithmetic is scalar
-            static_assert(kThreads % D == 0, "the workgroup's threads are whole rows");
+            // thread (row tid / D + i * kRowsAtOnce, column tid % D): where D is a multiple of 64 the row is the same in
+            // all lanes of a wavefront, so the row's address arithmetic is scalar
+            static_assert(kRowsAtOnce >= 1, "the workgroup's threads are at least one row");
             const uint32_t row_of_wave = kRowPerWave ? __builtin_amdgcn_readfirstlane(tid / D) : tid / D, j = tid % D;
 #pragma unroll
             for (uint32_t i = 0; i < QPT; ++i) {
-                const uint32_t row = row_of_wave + i * (kThreads / D);
+                const uint32_t row = row_of_wave + i * kRowsAtOnce;
                 const uint32_t ri = row / p.G, hs = row - ri * p.G, region = wg_region0 + ri;
                 float v = 0.0f;
-                if (row < wg_rows && region < n_regions) {
+                if (row_thread && row < wg_rows && region < n_regions) {
                     const uint32_t s_ = region / p.Hkv, kv_ = region - s_ * p.Hkv;
                     const float *qrow = p.query.q + (uint64_t)p.query.qg.off + (uint64_t)s_ * p.query.qg.s[0] +
                                         head_offset(p.query.qg, q_head_of(p, kv_, hs));
@@ -571,9 +575,9 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
         if constexpr (kQuery) {
 #pragma unroll
             for (uint32_t i = 0; i < QPT; ++i) {
-                const uint32_t e = tid + i * kThreads;
-                if (e < kQRows * D) {
-                    qraw_s[staged_at(e / D, e % D)] = qr[i];
+                const uint32_t row = tid / D + i * kRowsAtOnce;
+                if (row_thread && row < kQRows) {
+                    qraw_s[staged_at(row, tid % D)] = qr[i];
                 }
             }
             build_tables(); // (its barrier also makes the raw queries visible)
@@ -1190,15 +1194,17 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
         // once per row while the rows are merged
         unsigned long long *const rowbase_s = reinterpret_cast<unsigned long long *>(o_s + 16 * RPITCH);
         const uint32_t n_regions = p.n_seq * p.Hkv;
-        // (the row of an element is the same in all lanes of a wavefront: kThreads is a multiple of D)
-        const uint32_t rr_of_wave = kRowPerWave ? __builtin_amdgcn_readfirstlane(tid / D) : tid / D, col = tid % D;
+        // (the row of an element is the same in all lanes of a wavefront where D is a multiple of 64; threads that are
+        // not part of a whole row start behind the pass's rows)
+        const uint32_t rr_of_wave = !row_thread ? RP : kRowPerWave ? __builtin_amdgcn_readfirstlane(tid / D) : tid / D;
+        const uint32_t col = tid % D;
         // rows r0 .. r0 + RP - 1 of the workgroup (row = region index in the workgroup * G + head slot): o_s = the
         // merge of the row's `slots` partials, which partial(ri, hs, k) finds; normalised, or with NORMALISE false
         // left as the partial (m, l, o) that leave(rr, m, l, o) puts somewhere
         auto merge_rows = [&](uint32_t r0, uint32_t rows, uint32_t slots, auto partial, auto normalise, auto leave) {
             constexpr bool NORMALISE = decltype(normalise)::value;
             constexpr uint32_t KS = kWaves; // most partials of a row (one per wavefront)
-            for (uint32_t rr = rr_of_wave; rr < RP; rr += kThreads / D) {
+            for (uint32_t rr = rr_of_wave; rr < RP; rr += kRowsAtOnce) {
                 const uint32_t row = r0 + rr;
                 float v = 0.0f;
                 if (row < rows) {
@@ -1275,7 +1281,7 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
                     }
                 }
             } else {
-                for (uint32_t rr = rr_of_wave; rr < RP; rr += kThreads / D) {
+                for (uint32_t rr = rr_of_wave; rr < RP; rr += kRowsAtOnce) {
                     store_row(rr, col, o_s[staged_at(rr, col)]);
                 }
             }
@@ -1341,7 +1347,7 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
             };
             for (uint32_t r0 = 0; r0 < rows; r0 += RP) {
                 if constexpr (kRowPerWave) {
-                    for (uint32_t rr = rr_of_wave; rr < RP; rr += kThreads / D) {
+                    for (uint32_t rr = rr_of_wave; rr < RP; rr += kRowsAtOnce) {
                         one_row(r0, rr, col, true);
                     }
                 } else {
