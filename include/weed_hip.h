@@ -326,9 +326,9 @@ int weed_hip_kv_decode_attn(weed_hip_kv_cache *cache, int32_t n_q_heads, int32_t
  * whole number of such shares, one kernel does the whole call: that is so for batches of 1 to 256 sequences whose
  * lengths are equal or not too different -- sequences are counted as having as many blocks as the longest while that
  * adds at most 3/4 to the blocks of the batch; other batches of up to 63
- * sequences are one kernel too, with partial results in memory -- all of this at head_dims 33 to 64 and 97 to 128; up
- * to 32, at 65 to 96 and at 129 to 256 (there with at most eight query heads per kv head) only the first two cases;
- * otherwise, or with these bits, a kernel ahead rotates
+ * sequences are one kernel too, with partial results in memory -- all of this at head_dims up to 128 (65 to 96 with at
+ * most eight query heads per kv head and fields of at most 5 bits); at 129 to 256 (with at most eight query heads per
+ * kv head) only the first two cases; otherwise, or with these bits, a kernel ahead rotates
  * the queries and one behind merges the partials; the ways differ in the rounding of the last bits).  A number of
  * wavefronts other than 0 switches the choice of run lengths for whole regions off.  The process-wide defaults are read once from the environment variables WEED_HIP_DECODE_WAVES,
  * WEED_HIP_DECODE_SKEW and WEED_HIP_DECODE_SEARCH. */

@@ -451,6 +451,12 @@ def test_block_counts_that_no_run_length_divides(gpu, oracle, cap_blocks, top, s
     (True, 128, 2, 8, [1500] * 5, 3, 4, 0),                         # equal sequences that do not line up
     (True, 128, 1, 4, [640] * 40, 3, 4, 0),                         # many short equal sequences per workgroup
     (True, 128, 1, 16, [3000, 700, 1300], 3, 4, 0),                 # groups of 16, ragged
+    # head_dims 96 and 32: the third variant of their instances
+    (True, 96, 2, 8, [700, 64, 3000, 129, 1, 2049], 3, 4, 0),       # head_dim 96, ragged
+    (True, 80, 2, 16, [1000, 333, 90, 2500], 3, 4, 0),              # head_dim 80, groups of 8
+    (True, 96, 8, 8, [2048, 517, 4096, 1030], 3, 3, 0),             # head_dim 96, groups of one
+    (True, 32, 2, 8, [700, 64, 3000, 129, 1, 2049], 3, 4, 0),       # head_dim 32, ragged
+    (False, 24, 1, 4, [1500] * 5, 4, 4, 0),                         # head_dim 24, uniform coder, equal sequences that do not line up
 ])
 def test_any_batch_as_one_kernel(gpu, oracle, lloyd, d, Hkv, Hq, lens, kb, vb, waves):
     """Batches whose regions do not line up with the workgroups (ragged, or equal but unaligned): the wavefronts'

@@ -1097,7 +1097,7 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         // half short sequences, the workgroups win up to 6 regions per workgroup, tie at 7 and lose from 8 on (5 to
         // 30 us at 8 to 17).  Nor do they where they could not rotate their queries as well (a kernel ahead and the
         // merges at the end: 3 to 200 sequences of 100 tokens with groups of eight, 27 us against 22 to 25).
-        if (wg_regions == 0 && region_wgs == 0 && mfma_decode_merges(gp, d) && every_sequence_has_tokens &&
+        if (wg_regions == 0 && region_wgs == 0 && mfma_decode_merges_in_general(gp, d, runs.waves) && every_sequence_has_tokens &&
             (nb != 0 || (S <= 63 && !tune.always_search)) && n_splits <= 64 &&
             wg_most_regions <= kMostRegionsMergedByWorkgroup && wg_most_regions * pass_heads <= mfma_query_rows(d) &&
             (size_t)S * Hkv <= kMfmaMergeCounters && !tune.separate_merge) {
@@ -1105,7 +1105,8 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         }
         // A workgroup rotates the queries of the regions its blocks lie in itself when they are few enough for its
         // LDS (equal sequences, or the ragged batches above); nothing then runs ahead of the matrix-core kernel.
-        fused_query = (wg_regions != 0 || region_wgs != 0 || mfma_decode_merges(gp, d)) && (nb != 0 || general_merge) &&
+        fused_query = (wg_regions != 0 || region_wgs != 0 || mfma_decode_merges_in_general(gp, d, runs.waves)) &&
+                      (nb != 0 || general_merge) &&
                       wg_most_regions * pass_heads <= mfma_query_rows(d) && !tune.separate_query;
     }
     // Workgroups that merge whole regions or whole shares of a region: neighbouring runs take their blocks in turns

@@ -182,6 +182,18 @@ constexpr bool mfma_decode_merges_whole_regions(uint32_t gp, uint32_t d, uint32_
     return mfma_decode_merges(gp, d) || (gp <= 16 && ((d == 96u && waves == 12u) || d == 32u)) ||
         (gp <= 8 && d > 128u && d <= 256u && waves == 8u);
 }
+// Head_dims whose instances have a third variant that merges in the general case and rotates its queries (ragged
+// batches; see decode_mfma_kernel's MODE): 96 and 32, where the workgroups merge whole regions.  Above 128 the
+// instances have no registers for it.
+constexpr bool mfma_decode_general_variant(uint32_t gp, uint32_t d, uint32_t waves)
+{
+    return !mfma_decode_merges(gp, d) && (d == 96u || d == 32u) && mfma_decode_merges_whole_regions(gp, d, waves);
+}
+// ... so the general case is served by these instances:
+constexpr bool mfma_decode_merges_in_general(uint32_t gp, uint32_t d, uint32_t waves)
+{
+    return mfma_decode_merges(gp, d) || mfma_decode_general_variant(gp, d, waves);
+}
 // Rows (region, head) that one pass of the merge or of the query rotation takes (the matrix instruction behind both
 // has 16 rows, so a pass reads 8 rows beyond its own), and the LDS of both behind the lookup tables, in words.
 // Rows are staged for the matrix instruction with a pitch of d + 4 words.

@@ -306,10 +306,14 @@ template <int GP, int I> constexpr int bank_mask_of() { return ((1 << (GP / 4)) 
 // GP = number of query-head columns kept per score tile (the group size rounded up to 4, 8 or 16).  The Q.K^T
 // instruction always produces 16 columns; with GP < 16 the useful columns of 16/GP tiles are merged into one register
 // set before the softmax, so the exponentials and the fp16 splitting run on full registers.
-// WGM: the workgroups merge their regions themselves (see MfmaMerge); every wavefront then has at most one segment.
-template <int D, int WK, int WV, int GP, bool LLOYD, bool WGM>
+// MODE 1 (WGM): the workgroups merge their regions themselves (see MfmaMerge); every wavefront then has at most one
+// segment.  MODE 0: any partition; it merges in the general case (ragged batches) and rotates its queries where
+// mfma_decode_merges(GP, D) says so.  MODE 2: as MODE 0 with both of these, for the head_dims whose MODE 0 leaves them
+// out because they cost it registers that every other launch would pay for (mfma_decode_general_variant).
+template <int D, int WK, int WV, int GP, bool LLOYD, int MODE>
 __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) decode_mfma_kernel(MfmaParams p)
 {
+    constexpr bool WGM = MODE == 1;
     constexpr int kWaves = (int)mfma_decode_waves_per_wg(GP, D, WK, WV);
     constexpr int KS = D / 32;       // Q.K^T k-steps (32 coordinates each); also K items per tile per lane
     constexpr int JB = D / 16;       // 16-coordinate column blocks of the output
@@ -392,7 +396,8 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
                             p.total_blocks);
     // ---- merge inside the kernel (see MfmaMerge): LDS behind the tables, and this thread's share of the rotation ----
     static_assert(!WGM || mfma_decode_merges_whole_regions(GP, D, kWaves), "this instance cannot merge");
-    constexpr bool kCanMerge = WGM ? mfma_decode_merges_whole_regions(GP, D, kWaves) : mfma_decode_merges(GP, D);
+    static_assert(MODE != 2 || mfma_decode_general_variant(GP, D, kWaves), "there is no such variant of this instance");
+    constexpr bool kCanMerge = MODE != 0 ? mfma_decode_merges_whole_regions(GP, D, kWaves) : mfma_decode_merges(GP, D);
     constexpr bool kQuery = kCanMerge;   // this instance can rotate its queries itself (MfmaQuery)
     // (head_dim 96: a wavefront's 64 threads are not all in one row; what is a scalar elsewhere is per thread there)
     constexpr bool kRowPerWave = D % 64 == 0;
@@ -1493,12 +1498,19 @@ template <int D, int WK, int WV, int GP, bool LLOYD> int launch_gp(const MfmaPar
     static std::once_flag configured;
     static hipError_t config_status = hipSuccess;
     constexpr bool kMerges = mfma_decode_merges_whole_regions(GP, D, waves);
+    constexpr bool kGeneralVariant = mfma_decode_general_variant(GP, D, waves);
     std::call_once(configured, [] {
-        config_status = hipFuncSetAttribute((const void *)decode_mfma_kernel<D, WK, WV, GP, LLOYD, false>,
+        config_status = hipFuncSetAttribute((const void *)decode_mfma_kernel<D, WK, WV, GP, LLOYD, 0>,
                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_merging);
         if constexpr (kMerges) {
             if (config_status == hipSuccess) {
-                config_status = hipFuncSetAttribute((const void *)decode_mfma_kernel<D, WK, WV, GP, LLOYD, true>,
+                config_status = hipFuncSetAttribute((const void *)decode_mfma_kernel<D, WK, WV, GP, LLOYD, 1>,
+                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_merging);
+            }
+        }
+        if constexpr (kGeneralVariant) {
+            if (config_status == hipSuccess) {
+                config_status = hipFuncSetAttribute((const void *)decode_mfma_kernel<D, WK, WV, GP, LLOYD, 2>,
                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_merging);
             }
         }
@@ -1512,13 +1524,20 @@ template <int D, int WK, int WV, int GP, bool LLOYD> int launch_gp(const MfmaPar
     const uint32_t grid = (p.total_blocks + wg_blocks - 1) / wg_blocks;
     if (p.merge.wg_regions != 0 || p.merge.region_wgs != 0) {
         if constexpr (kMerges) {
-            decode_mfma_kernel<D, WK, WV, GP, LLOYD, true><<<grid, 64 * waves, smem_merging, s>>>(p);
+            decode_mfma_kernel<D, WK, WV, GP, LLOYD, 1><<<grid, 64 * waves, smem_merging, s>>>(p);
         } else {
             return fail(WEED_HIP_EDEVICE, "decode_mfma: this kernel instance cannot merge its partials itself");
         }
     } else {
         // (the area behind the tables is where a workgroup rotates its queries, when it does)
-        decode_mfma_kernel<D, WK, WV, GP, LLOYD, false>
+        if constexpr (kGeneralVariant) {
+            if (p.query.q || p.merge.general) {
+                decode_mfma_kernel<D, WK, WV, GP, LLOYD, 2><<<grid, 64 * waves, smem_merging, s>>>(p);
+                WEED_HIP_LAUNCH_CHECK();
+                return WEED_HIP_OK;
+            }
+        }
+        decode_mfma_kernel<D, WK, WV, GP, LLOYD, 0>
             <<<grid, 64 * waves, (p.query.q || p.merge.general) ? smem_merging : smem, s>>>(p);
     }
     WEED_HIP_LAUNCH_CHECK();
