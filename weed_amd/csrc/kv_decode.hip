@@ -1051,10 +1051,13 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         const uint32_t gp = pass_heads <= 4 ? 4u : (pass_heads <= 8 ? 8u : 16u);
         const uint32_t nb = uniform_blocks, cycle = run_classes(runs) * runs.unit_blocks;
         const uint32_t wg_blocks = runs.waves * runs.unit_blocks;
-        if (mfma_decode_merges_whole_regions(gp, d, runs.waves) && nb != 0 && nb % cycle == 0 && wg_blocks % nb == 0 &&
-            !tune.separate_merge) {
+        // (groups that take several passes at head_dims above 128: every pass would rotate and merge at the end of
+        // its workgroups, which measured 2 to 4 us behind one kernel ahead and one behind all passes -- 16 sequences of
+        // 8192 tokens, sixteen heads per kv head: 88.1 against 85.7 us at head_dim 256, 83.5 against 79.4 at 192)
+        const bool may_merge = mfma_decode_merges_whole_regions(gp, d, runs.waves) && (d <= 128 || passes == 1);
+        if (may_merge && nb != 0 && nb % cycle == 0 && wg_blocks % nb == 0 && !tune.separate_merge) {
             wg_regions = wg_blocks / nb;
-        } else if (mfma_decode_merges_whole_regions(gp, d, runs.waves) && nb != 0 && nb % wg_blocks == 0 && nb / wg_blocks >= 2 &&
+        } else if (may_merge && nb != 0 && nb % wg_blocks == 0 && nb / wg_blocks >= 2 &&
                    nb / wg_blocks <= std::min(n_splits, 64u) && (size_t)S * Hkv <= kMfmaMergeCounters &&
                    !tune.separate_merge) {
             // small batches of long sequences: every region is a whole number of workgroups' shares
