@@ -377,6 +377,8 @@ def plan_scan(capi, torch, steps=100, warmup=WARMUP_FLOOR_EXTRA, d=128):
                 shapes.append(("equal", Hkv, Hq, [ctx] * S))
     for S in (1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128):
         shapes.append(("equal", 8, 32, [8192] * S))
+    for S, ctx in ((1, 1000), (1, 8192), (16, 8192), (64, 2100)):
+        shapes.append(("equal, groups of 32", 2, 64, [ctx] * S))  # (two passes of sixteen heads)
     for ctx in (7744, 8000, 8129):
         shapes.append(("equal", 8, 32, [ctx] * 64))
     rnd = random.Random(17)

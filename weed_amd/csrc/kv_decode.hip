@@ -1051,10 +1051,12 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         const uint32_t gp = pass_heads <= 4 ? 4u : (pass_heads <= 8 ? 8u : 16u);
         const uint32_t nb = uniform_blocks, cycle = run_classes(runs) * runs.unit_blocks;
         const uint32_t wg_blocks = runs.waves * runs.unit_blocks;
-        // (groups that take several passes at head_dims above 128: every pass would rotate and merge at the end of
-        // its workgroups, which measured 2 to 4 us behind one kernel ahead and one behind all passes -- 16 sequences of
-        // 8192 tokens, sixteen heads per kv head: 88.1 against 85.7 us at head_dim 256, 83.5 against 79.4 at 192)
-        const bool may_merge = mfma_decode_merges_whole_regions(gp, d, runs.waves) && (d <= 128 || passes == 1);
+        // (Groups that take several passes of the kernel -- more than sixteen heads per kv head, more than eight at
+        // head_dims above 128 -- go the three-kernel way: every pass would rotate its queries and merge at the end of
+        // its workgroups, where one kernel ahead and one behind serve all passes.  Measured, 64 heads on 2 kv heads
+        // of 128: 16 sequences of 8192 tokens 63.4 against 59.5 us, one sequence 57.7 against 37.2, two of 30000
+        // tokens 105 against 58; 96 heads on 2: 91 against 61.)
+        const bool may_merge = mfma_decode_merges_whole_regions(gp, d, runs.waves) && passes == 1;
         if (may_merge && nb != 0 && nb % cycle == 0 && wg_blocks % nb == 0 && !tune.separate_merge) {
             wg_regions = wg_blocks / nb;
         } else if (may_merge && nb != 0 && nb % wg_blocks == 0 && nb / wg_blocks >= 2 &&
@@ -1100,7 +1102,7 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         // half short sequences, the workgroups win up to 6 regions per workgroup, tie at 7 and lose from 8 on (5 to
         // 30 us at 8 to 17).  Nor do they where they could not rotate their queries as well (a kernel ahead and the
         // merges at the end: 3 to 200 sequences of 100 tokens with groups of eight, 27 us against 22 to 25).
-        if (wg_regions == 0 && region_wgs == 0 && mfma_decode_merges_in_general(gp, d, runs.waves) && every_sequence_has_tokens &&
+        if (wg_regions == 0 && region_wgs == 0 && passes == 1 && mfma_decode_merges_in_general(gp, d, runs.waves) && every_sequence_has_tokens &&
             (nb != 0 || (S <= 63 && !tune.always_search)) && n_splits <= 64 &&
             wg_most_regions <= kMostRegionsMergedByWorkgroup && wg_most_regions * pass_heads <= mfma_query_rows(d) &&
             (size_t)S * Hkv <= kMfmaMergeCounters && !tune.separate_merge) {
@@ -1108,7 +1110,7 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         }
         // A workgroup rotates the queries of the regions its blocks lie in itself when they are few enough for its
         // LDS (equal sequences, or the ragged batches above); nothing then runs ahead of the matrix-core kernel.
-        fused_query = (wg_regions != 0 || region_wgs != 0 || mfma_decode_merges_in_general(gp, d, runs.waves)) &&
+        fused_query = passes == 1 && (wg_regions != 0 || region_wgs != 0 || mfma_decode_merges_in_general(gp, d, runs.waves)) &&
                       (nb != 0 || general_merge) &&
                       wg_most_regions * pass_heads <= mfma_query_rows(d) && !tune.separate_query;
     }

@@ -461,8 +461,11 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     //      ri * G + hs.  Requested here: this thread's share of the K rotation and of the raw queries. ----
     // Where a thread is a column of a row (the raw queries, the merged rows), the workgroup's first kRowsAtOnce * D
     // threads are kRowsAtOnce whole rows; at head_dims that do not divide the threads (160, 192, 224) the rest idle.
+    // (Known at compile time where the threads are whole rows, and the same in all lanes of a wavefront where D is a
+    // multiple of 64: what depends on it stays scalar, as the rows' address arithmetic must.)
     constexpr uint32_t kRowsAtOnce = kThreads / D;
-    const bool row_thread = tid < kRowsAtOnce * D;
+    const bool row_thread = kRowsAtOnce * D == kThreads ||
+        (D % 64 == 0 ? (uint32_t)__builtin_amdgcn_readfirstlane((int)tid) : tid) < kRowsAtOnce * D;
     constexpr uint32_t QPT = kQuery ? (kQRows + kRowsAtOnce - 1) / kRowsAtOnce : 1; // raw query elements per thread
     constexpr uint32_t PW = mfma_merge_partials_words(kWaves, GP, D);
     float *const qraw_s = part_s;                                       // [rows (+ 8 that a tile of 16 reaches into)] staged
