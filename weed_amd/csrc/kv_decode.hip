@@ -921,7 +921,9 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
             if (may_round && !preferred_unit) {
                 const uint32_t classes = run_classes(runs), regions = S * Hkv;
                 for (uint32_t cand = nb; cand <= reach && !preferred_unit; ++cand) {
-                    uint32_t best_rounds = 3;
+                    // (one or two rounds of workgroups; above head_dim 128, where a workgroup's queries and merges
+                    // take longer and a compute unit holds one workgroup, one round only)
+                    uint32_t best_rounds = d > 128 ? 2 : 3;
                     for (uint32_t q = 1; q <= 4; q *= 2) {
                         if (cand % (classes * q) != 0) {
                             continue;
@@ -1061,7 +1063,10 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         // of 128: 16 sequences of 8192 tokens 63.4 against 59.5 us, one sequence 57.7 against 37.2, two of 30000
         // tokens 105 against 58; 96 heads on 2: 91 against 61.)
         const bool may_merge = mfma_decode_merges_whole_regions(gp, d, runs.waves) && passes == 1;
-        if (may_merge && nb != 0 && nb % cycle == 0 && wg_blocks % nb == 0 && !tune.separate_merge) {
+        // (above head_dim 128 in one round of workgroups only: 64 sequences of 300 or 2100 tokens on 32 kv heads of
+        // 256 in two rounds took 69 and 224 us against 61 and 216 with three kernels, where one round is 13 us ahead)
+        if (may_merge && nb != 0 && nb % cycle == 0 && wg_blocks % nb == 0 && !tune.separate_merge &&
+            (d <= 128 || (total_blocks + wg_blocks - 1) / wg_blocks <= 256)) {
             wg_regions = wg_blocks / nb;
         } else if (may_merge && nb != 0 && nb % wg_blocks == 0 && nb / wg_blocks >= 2 &&
                    nb / wg_blocks <= std::min(n_splits, 64u) && (size_t)S * Hkv <= kMfmaMergeCounters &&
