@@ -331,7 +331,8 @@ int weed_hip_kv_decode_attn(weed_hip_kv_cache *cache, int32_t n_q_heads, int32_t
  * kv head) only the first two cases; otherwise, or with these bits, a kernel ahead rotates
  * the queries and one behind merges the partials; the ways differ in the rounding of the last bits).  A number of
  * wavefronts other than 0 switches the choice of run lengths for whole regions off.  The process-wide defaults are read once from the environment variables WEED_HIP_DECODE_WAVES,
- * WEED_HIP_DECODE_SKEW and WEED_HIP_DECODE_SEARCH. */
+ * WEED_HIP_DECODE_SKEW and WEED_HIP_DECODE_SEARCH; with WEED_HIP_DECODE_PLAN=1 every decode call writes the partition
+ * it chose (run length, wavefronts, which of the cases above) to stderr. */
 int weed_hip_kv_decode_tuning(int32_t wavefronts, int32_t skew_percent, int32_t always_search);
 
 /* weed_hip_kv_decode_attn for callers that cannot allocate device memory (code under HIP graph capture, serving loops

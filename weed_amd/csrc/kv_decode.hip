@@ -505,6 +505,7 @@ struct DecodeTuning {
     bool separate_merge = false; // always merge the partials with the second kernel
     bool separate_query = false; // always rotate the queries with the kernel ahead
     bool contiguous_runs = false; // never let neighbouring runs take turns (RunGeom::group_cycles)
+    bool print_plan = false;      // WEED_HIP_DECODE_PLAN=1: every call writes its partition to stderr
 };
 DecodeTuning &decode_tuning()
 {
@@ -521,6 +522,9 @@ DecodeTuning &decode_tuning()
             v.separate_merge = (std::atoi(env) & 2) != 0;
             v.separate_query = (std::atoi(env) & 4) != 0;
             v.contiguous_runs = (std::atoi(env) & 8) != 0;
+        }
+        if (const char *env = std::getenv("WEED_HIP_DECODE_PLAN")) {
+            v.print_plan = std::atoi(env) != 0;
         }
         return v;
     }();
@@ -883,7 +887,10 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         // more: there the ratio may be four (16 sequences from [512, 8192]: 42 us against 33 us).  What bounds such
         // calls is the blocks as counted, which is what a wavefront of the longest sequence works through: 32
         // sequences with up to 8192 tokens each gain 8 to 17 us counted alike, 48 such sequences lose 5 to 44 us.
-        const uint64_t most_counted = (uint64_t)most * S * Hkv > 32768 ? real_blocks * 7 / 4 : real_blocks * 4;
+        const uint64_t counted_alike = (uint64_t)most * S * Hkv;
+        const uint64_t most_counted = counted_alike > 32768 ? real_blocks * 7 / 4
+            : counted_alike > 16384                         ? real_blocks * 5 / 2
+                                                            : real_blocks * 4;
         // (counts beyond what a region's memory holds are fine: the kernel reads nothing behind a region's last block)
         // (and no further than 4096 blocks past the longest: the counts that qualify below recur every few hundred
         // blocks at most, so a search that has found none by then finds none, and the host's time stays bounded)
@@ -1112,7 +1119,7 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         // 30 us at 8 to 17).  Nor do they where they could not rotate their queries as well (a kernel ahead and the
         // merges at the end: 3 to 200 sequences of 100 tokens with groups of eight, 27 us against 22 to 25).
         if (wg_regions == 0 && region_wgs == 0 && passes == 1 && mfma_decode_merges_in_general(gp, d, runs.waves) && every_sequence_has_tokens &&
-            (nb != 0 || (S <= 63 && !tune.always_search)) && n_splits <= 64 &&
+            (nb != 0 || (S <= 63 && !tune.always_search)) && n_splits <= (d % 64 == 0 ? 64u : 24u) &&
             wg_most_regions <= kMostRegionsMergedByWorkgroup && wg_most_regions * pass_heads <= mfma_query_rows(d) &&
             (size_t)S * Hkv <= kMfmaMergeCounters && !tune.separate_merge) {
             general_merge = true;
@@ -1138,6 +1145,14 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         runs.group_cycles = cycles;
     }
     const bool fused_merge = wg_regions != 0 || region_wgs != 0 || general_merge;
+    if (tune.print_plan) {
+        std::fprintf(stderr,
+                     "%s: S %u Hkv %u G %u d %u bits %u/%u  matrix cores %d  passes %u  blocks %u  run %u (skew %u, in turns %u) "
+                     "x %u wavefronts  whole regions per workgroup %u  workgroups per region %u  general merge %d  "
+                     "queries in the kernel %d  slots %u\n",
+                     fn, S, Hkv, G, d, c->k.w, c->v.w, (int)use_mfma, passes, total_blocks, runs.unit_blocks, runs.skew,
+                     runs.group_cycles, runs.waves, wg_regions, region_wgs, (int)general_merge, (int)fused_query, n_splits);
+    }
     // (the kernels that take one (sequence, head) row per workgroup have the sequence on a 16-bit grid dimension)
     // (prep_q_kernel puts one more row on that dimension when it also builds the block offsets)
     WEED_HIP_REQUIRE(S + ((use_mfma && !fused_query && !many_rows) ? 1u : 0u) <= 65535u || (use_mfma && many_rows && n_splits <= 64),
