@@ -445,7 +445,7 @@ def test_block_counts_that_no_run_length_divides(gpu, oracle, cap_blocks, top, s
 
 @pytest.mark.parametrize("lloyd,d,Hkv,Hq,lens,kb,vb,waves", [
     (True, 128, 2, 8, [700, 64, 3000, 129, 1, 2049], 3, 4, 0),      # ragged, runs straddle regions
-    (True, 128, 2, 8, [700, 64, 3000, 129, 1, 2049], 3, 4, 40),     # the same with few, long runs
+    (True, 128, 2, 4, [700, 64, 3000, 129, 1, 2049], 3, 4, 40),     # few, long runs: up to six regions (twelve rows) per workgroup
     (True, 128, 8, 8, [2048, 517, 8192, 1030, 4100], 3, 3, 400),    # groups of one, three wavefronts per SIMD
     (False, 64, 2, 16, [1000, 333, 90, 2500], 4, 4, 0),             # uniform coder, head_dim 64, groups of 8
     (True, 128, 2, 8, [1500] * 5, 3, 4, 0),                         # equal sequences that do not line up

@@ -491,6 +491,9 @@ constexpr uint32_t kRunSkewPercent = 16, kRunSkewPercent3 = 28;
 // Most regions that the blocks of one workgroup may lie in for the workgroups to merge their regions themselves in the
 // general case (see decode_impl).
 constexpr uint32_t kMostRegionsMergedByWorkgroup = 6;
+// ... and most rows (region, head) of them: two passes of the merge (96 sequences of 2100 or 5000 tokens with four heads
+// per kv head, five regions = 20 rows per workgroup: 59.2 and 116.8 us, against 51.2 and 111.9 with the merge kernel)
+constexpr uint32_t kMostRowsMergedByWorkgroup = 16;
 
 // Tuning knobs of the work partition.  The defaults come from the environment, read ONCE per process (at the first
 // decode call or the first weed_hip_kv_decode_tuning): WEED_HIP_DECODE_WAVES (wavefronts the block list is cut for),
@@ -1120,7 +1123,8 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         // merges at the end: 3 to 200 sequences of 100 tokens with groups of eight, 27 us against 22 to 25).
         if (wg_regions == 0 && region_wgs == 0 && passes == 1 && mfma_decode_merges_in_general(gp, d, runs.waves) && every_sequence_has_tokens &&
             (nb != 0 || (S <= 63 && !tune.always_search)) && n_splits <= (d % 64 == 0 ? 64u : 24u) &&
-            wg_most_regions <= kMostRegionsMergedByWorkgroup && wg_most_regions * pass_heads <= mfma_query_rows(d) &&
+            wg_most_regions <= kMostRegionsMergedByWorkgroup &&
+            wg_most_regions * pass_heads <= std::min(kMostRowsMergedByWorkgroup, mfma_query_rows(d)) &&
             (size_t)S * Hkv <= kMfmaMergeCounters && !tune.separate_merge) {
             general_merge = true;
         }
