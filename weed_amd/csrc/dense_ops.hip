@@ -239,6 +239,153 @@ __global__ void __launch_bounds__(THREADS) softmax_strided_cached_kernel(const f
     }
 }
 
+// ---- Few rows, long strided axis (the scores of a decode step as the reference lays them out: [B * heads] rows whose
+//      elements are B * heads apart): 64 rows per workgroup would be a handful of workgroups, so the axis is cut into
+//      bands.  Workgroup (row group x, band y) = 64 rows x 4 lanes of the band's positions; three small launches:
+//      every band's (max, sum) per row, their merge per row, exp(x - max) / sum per band.  The partial results live
+//      in a static array (the library serves one stream per device: calls do not overlap).
+constexpr uint32_t kBandRows = 4096, kMostBands = 128, kBandPartials = 65536; // (about 512 workgroups: bands x rows <= 32768 + a row group)
+__device__ float2 g_band_part[kBandPartials]; // [band][pitch]
+__device__ float2 g_band_final[kBandRows];
+
+struct BandGeom {
+    uint32_t bands, band_len, pitch; // pitch: the rows, rounded up to whole row groups
+};
+
+template <int OP> // 0 sum, 1 max, 2 min, 3 softmax's (max, sum)
+__global__ void __launch_bounds__(256) band_partial_kernel(const float *__restrict__ a, AxisGeom g, BandGeom bg)
+{
+    __shared__ float2 red[256];
+    constexpr int U = kAxisUnroll;
+    const uint32_t rr = threadIdx.x % 64U, jj = threadIdx.x / 64U;
+    const uint32_t row = blockIdx.x * 64U + rr;
+    const bool valid = row < g.rows;
+    uint64_t a_base = g.a_off, o_base = 0;
+    if (valid) {
+        row_bases(g, row, a_base, o_base);
+    }
+    const uint32_t as = g.a_stride[g.axis];
+    const uint32_t j0 = blockIdx.y * bg.band_len, j1 = valid ? min(j0 + bg.band_len, g.axis_len) : 0U;
+    const float *ap = a + a_base;
+    float m = OP == 3 ? -INFINITY : identity<OP == 3 ? 1 : OP>(), s = 0.0f;
+    for (uint32_t j = j0 + jj; j < j1; j += 4U * U) {
+        float x[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint32_t k = j + 4U * u;
+            x[u] = k < j1 ? ap[(uint64_t)k * as] : (OP == 3 ? -INFINITY : identity<OP == 3 ? 1 : OP>());
+        }
+        if constexpr (OP == 3) {
+            softmax_accumulate(m, s, x);
+        } else {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                m = combine<OP == 3 ? 1 : OP>(m, x[u]);
+            }
+        }
+    }
+    red[threadIdx.x] = make_float2(m, s);
+    __syncthreads();
+    if (jj == 0U && valid) {
+#pragma unroll
+        for (uint32_t k = 1; k < 4U; ++k) {
+            const float2 o = red[64U * k + rr];
+            if constexpr (OP == 3) {
+                const float top = fmaxf(m, o.x);
+                s = (m > -INFINITY ? s * expf(m - top) : 0.0f) + (o.x > -INFINITY ? o.y * expf(o.x - top) : 0.0f);
+                m = top;
+            } else {
+                m = combine<OP == 3 ? 1 : OP>(m, o.x);
+            }
+        }
+        g_band_part[blockIdx.y * bg.pitch + row] = make_float2(m, s);
+    }
+}
+
+// 64 rows per workgroup, four lanes per row that take every fourth band (all of a lane's partial results are requested
+// before the first is used: one thread per row walking 128 bands one after the other took 35 us), then the four lanes'
+// results in lane order
+template <int OP>
+__global__ void __launch_bounds__(256) band_merge_kernel(float *__restrict__ out, AxisGeom g, BandGeom bg)
+{
+    __shared__ float2 red[256];
+    const uint32_t rr = threadIdx.x % 64U, jj = threadIdx.x / 64U;
+    const uint32_t row = blockIdx.x * 64U + rr;
+    const bool valid = row < g.rows;
+    auto merge = [](float2 &acc, const float2 o) {
+        if constexpr (OP == 3) {
+            const float top = fmaxf(acc.x, o.x);
+            acc.y = (acc.x > -INFINITY ? acc.y * expf(acc.x - top) : 0.0f) + (o.x > -INFINITY ? o.y * expf(o.x - top) : 0.0f);
+            acc.x = top;
+        } else {
+            acc.x = combine<OP == 3 ? 1 : OP>(acc.x, o.x);
+        }
+    };
+    float2 acc = make_float2(OP == 3 ? -INFINITY : identity<OP == 3 ? 1 : OP>(), 0.0f);
+    constexpr uint32_t kMine = kMostBands / 4U; // bands jj, jj + 4, ...
+    float2 mine[kMine];
+#pragma unroll
+    for (uint32_t k = 0; k < kMine; ++k) {
+        const uint32_t b = jj + 4U * k;
+        mine[k] = (valid && b < bg.bands) ? g_band_part[b * bg.pitch + row] : acc;
+    }
+#pragma unroll
+    for (uint32_t k = 0; k < kMine; ++k) {
+        if (jj + 4U * k < bg.bands) {
+            merge(acc, mine[k]);
+        }
+    }
+    red[threadIdx.x] = acc;
+    __syncthreads();
+    if (jj != 0U || !valid) {
+        return;
+    }
+#pragma unroll
+    for (uint32_t k = 1; k < 4U; ++k) {
+        merge(acc, red[64U * k + rr]);
+    }
+    if constexpr (OP == 3) {
+        g_band_final[row] = make_float2(acc.x, 1.0f / acc.y);
+    } else {
+        uint64_t a_base, o_base;
+        row_bases(g, row, a_base, o_base);
+        out[o_base] = acc.x;
+    }
+}
+
+__global__ void __launch_bounds__(256) band_softmax_finish_kernel(const float *__restrict__ a, float *__restrict__ out,
+                                                                  AxisGeom g, BandGeom bg)
+{
+    constexpr int U = kAxisUnroll;
+    const uint32_t rr = threadIdx.x % 64U, jj = threadIdx.x / 64U;
+    const uint32_t row = blockIdx.x * 64U + rr;
+    if (row >= g.rows) {
+        return;
+    }
+    uint64_t a_base, o_base;
+    row_bases(g, row, a_base, o_base);
+    const uint32_t as = g.a_stride[g.axis], os = g.o_stride[g.axis];
+    const uint32_t j0 = blockIdx.y * bg.band_len, j1 = min(j0 + bg.band_len, g.axis_len);
+    const float2 ms = g_band_final[row];
+    const float *ap = a + a_base;
+    float *op = out + o_base;
+    for (uint32_t j = j0 + jj; j < j1; j += 4U * U) {
+        float x[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint32_t k = j + 4U * u;
+            x[u] = k < j1 ? ap[(uint64_t)k * as] : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint32_t k = j + 4U * u;
+            if (k < j1) {
+                op[(uint64_t)k * os] = expf(x[u] - ms.x) * ms.y;
+            }
+        }
+    }
+}
+
 // Softmax along a contiguous, 16-byte aligned axis: one workgroup per row, float4 accesses, and the first
 // CACHED * 4 * THREADS elements of the row stay in registers between the passes.  Rows up to that length (FITS) are
 // read once and cost one exponential per element; longer rows keep a running (max, sum) and are read twice.
@@ -423,6 +570,81 @@ __global__ void __launch_bounds__(256) softmax_wave_rows_kernel(const float *__r
     }
 }
 
+// Rows of up to CACHED * LPR * V elements, LPR lanes per row (a power of two below 64): 64 / LPR rows per wavefront, so
+// that a wavefront's loads are whole contiguous stretches of memory also where a row is a few dozen elements (a
+// wavefront per row would leave most lanes idle there: 262144 rows of 16 took 209 us, 65536 rows of 128 54 us).
+template <int V, int CACHED, int LPR>
+__global__ void __launch_bounds__(256) softmax_short_rows_kernel(const float *__restrict__ a, float *__restrict__ out,
+                                                                 AxisGeom g)
+{
+    constexpr uint32_t RPW = 64U / LPR; // rows per wavefront
+    const uint32_t lane = threadIdx.x & 63U, sub = lane % LPR;
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t nvec = g.axis_len / V;
+    // (every lane of a wavefront makes the same number of trips, so that the exchanges between lanes are whole)
+    for (uint32_t row0 = (blockIdx.x * 4U + wave) * RPW; row0 < g.rows; row0 += gridDim.x * 4U * RPW) {
+        const uint32_t row = row0 + lane / LPR;
+        const bool valid = row < g.rows;
+        uint64_t a_base = g.a_off, o_base = g.o_off;
+        if (valid) {
+            row_bases(g, row, a_base, o_base);
+        }
+        const float *ap = a + a_base;
+        float *op = out + o_base;
+        float cache[CACHED][V];
+        float m = -INFINITY, s = 0.0f;
+#pragma unroll
+        for (int c = 0; c < CACHED; ++c) {
+            const uint32_t idx = sub + LPR * c;
+            const bool ok = valid && idx < nvec;
+            if (V == 4) {
+                const float4 v = ok ? reinterpret_cast<const float4 *>(ap)[idx]
+                                    : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+                cache[c][0] = v.x;
+                cache[c][V > 1 ? 1 : 0] = v.y;
+                cache[c][V > 2 ? 2 : 0] = v.z;
+                cache[c][V > 3 ? 3 : 0] = v.w;
+            } else {
+                cache[c][0] = ok ? ap[idx] : -INFINITY;
+            }
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                m = fmaxf(m, cache[c][e]);
+            }
+        }
+#pragma unroll
+        for (int off = LPR / 2; off > 0; off >>= 1) {
+            m = fmaxf(m, __shfl_xor(m, off, 64));
+        }
+#pragma unroll
+        for (int c = 0; c < CACHED; ++c) {
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                cache[c][e] = expf(cache[c][e] - m);
+                s += cache[c][e];
+            }
+        }
+#pragma unroll
+        for (int off = LPR / 2; off > 0; off >>= 1) {
+            s += __shfl_xor(s, off, 64);
+        }
+        const float inv = 1.0f / s;
+#pragma unroll
+        for (int c = 0; c < CACHED; ++c) {
+            const uint32_t idx = sub + LPR * c;
+            if (valid && idx < nvec) {
+                if (V == 4) {
+                    reinterpret_cast<float4 *>(op)[idx] = make_float4(cache[c][0] * inv, cache[c][V > 1 ? 1 : 0] * inv,
+                                                                      cache[c][V > 2 ? 2 : 0] * inv,
+                                                                      cache[c][V > 3 ? 3 : 0] * inv);
+                } else {
+                    op[idx] = cache[c][0] * inv;
+                }
+            }
+        }
+    }
+}
+
 template <int OP, int V>
 __global__ void __launch_bounds__(256) reduce_wave_rows_kernel(const float *__restrict__ a, float *__restrict__ out,
                                                                AxisGeom g)
@@ -445,6 +667,42 @@ __global__ void __launch_bounds__(256) reduce_wave_rows_kernel(const float *__re
         }
         v = wave_reduce<OP>(v);
         if (lane == 0U) {
+            out[o_base] = v;
+        }
+    }
+}
+
+// Short contiguous rows, LPR lanes per row (see softmax_short_rows_kernel): 64 / LPR rows per wavefront.
+template <int OP, int V, int LPR>
+__global__ void __launch_bounds__(256) reduce_short_rows_kernel(const float *__restrict__ a, float *__restrict__ out,
+                                                                AxisGeom g)
+{
+    constexpr uint32_t RPW = 64U / LPR;
+    const uint32_t lane = threadIdx.x & 63U, sub = lane % LPR;
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t nvec = g.axis_len / V;
+    for (uint32_t row0 = (blockIdx.x * 4U + wave) * RPW; row0 < g.rows; row0 += gridDim.x * 4U * RPW) {
+        const uint32_t row = row0 + lane / LPR;
+        const bool valid = row < g.rows;
+        uint64_t a_base = g.a_off, o_base = g.o_off;
+        if (valid) {
+            row_bases(g, row, a_base, o_base);
+        }
+        const float *ap = a + a_base;
+        float v = identity<OP>();
+        for (uint32_t idx = sub; valid && idx < nvec; idx += LPR) {
+            if (V == 4) {
+                const float4 x = reinterpret_cast<const float4 *>(ap)[idx];
+                v = combine<OP>(v, combine<OP>(combine<OP>(x.x, x.y), combine<OP>(x.z, x.w)));
+            } else {
+                v = combine<OP>(v, ap[idx]);
+            }
+        }
+#pragma unroll
+        for (int off = LPR / 2; off > 0; off >>= 1) {
+            v = combine<OP>(v, __shfl_xor(v, off, 64));
+        }
+        if (valid && sub == 0U) {
             out[o_base] = v;
         }
     }
@@ -835,8 +1093,34 @@ AxisLaunch choose_axis_launch(const AxisGeom &g, const float *a_dev, const float
     return g.rows >= 32U * 1024U ? AXIS_ROWS32 : g.rows >= 32U * 128U ? AXIS_ROWS32_WIDE : AXIS_ROWS16;
 }
 
+// Few rows and a long strided axis: bands of the axis (see band_partial_kernel); bands == 0: not this way.
+BandGeom choose_bands(const AxisGeom &g, uint32_t most_rows)
+{
+    BandGeom bg = { 0U, 0U, 0U };
+    if (g.a_stride[g.axis] <= 1U || g.rows < 16U || g.rows > std::min(most_rows, kBandRows) || g.axis_len < 4096U ||
+        (uint64_t)g.axis_len * g.a_stride[g.axis] >= (1ull << 32)) {
+        return bg;
+    }
+    const uint32_t row_groups = (g.rows + 63U) / 64U;
+    const uint32_t want = std::max(1U, std::min(kMostBands, 512U / row_groups));
+    bg.band_len = std::max(32U, (g.axis_len + want - 1U) / want);
+    bg.band_len = (bg.band_len + 31U) / 32U * 32U;
+    bg.bands = (g.axis_len + bg.band_len - 1U) / bg.band_len;
+    bg.pitch = row_groups * 64U;
+    if ((uint64_t)bg.bands * bg.pitch > kBandPartials) {
+        bg.bands = 0U;
+    }
+    return bg;
+}
+
 // Four rows per workgroup; beyond 16 workgroups per compute unit the wavefronts loop over rows.
 uint32_t wave_row_blocks(uint32_t rows) { return std::min<uint32_t>((rows + 3U) / 4U, 256U * 16U); }
+// ... with 64 / lanes_per_row rows per wavefront
+uint32_t short_row_blocks(uint32_t rows, uint32_t lanes_per_row)
+{
+    const uint32_t per_wg = 4U * (64U / lanes_per_row);
+    return std::min<uint32_t>((rows + per_wg - 1U) / per_wg, 256U * 16U);
+}
 
 } // namespace
 
@@ -1077,9 +1361,36 @@ int weed_hip_softmax_f32(uint32_t rank, const uint32_t *shape, uint32_t axis, co
         } else {
             softmax_contiguous_kernel<8, 256, false><<<g.rows, 256, 0, stream()>>>(a_dev, out_dev, g);
         }
+    } else if (how == AXIS_WAVE_VEC && g.axis_len <= 512U) {
+        // short rows: as few lanes per row as keep a lane's share at one or two 16-byte pieces
+        const uint32_t n4 = g.axis_len / 4U;
+#define WEED_SHORT_ROWS(V, C, LPR)                                                                                     \
+    softmax_short_rows_kernel<V, C, LPR><<<short_row_blocks(g.rows, LPR), 256, 0, stream()>>>(a_dev, out_dev, g)
+        if (n4 <= 4U) {
+            WEED_SHORT_ROWS(4, 1, 4);
+        } else if (n4 <= 8U) {
+            WEED_SHORT_ROWS(4, 2, 4);
+        } else if (n4 <= 16U) {
+            WEED_SHORT_ROWS(4, 1, 16);
+        } else if (n4 <= 32U) {
+            WEED_SHORT_ROWS(4, 2, 16);
+        } else if (n4 <= 64U) {
+            WEED_SHORT_ROWS(4, 4, 16);
+        } else {
+            WEED_SHORT_ROWS(4, 4, 32);
+        }
     } else if (how == AXIS_WAVE_VEC) {
         // (kWaveRowMax = 8 * 4 * 64: such a row always fits a wavefront's registers)
         softmax_wave_rows_kernel<4, 8, true><<<wave_row_blocks(g.rows), 256, 0, stream()>>>(a_dev, out_dev, g);
+    } else if (how == AXIS_WAVE && g.axis_len <= 128U) {
+        if (g.axis_len <= 8U) {
+            WEED_SHORT_ROWS(1, 2, 4);
+        } else if (g.axis_len <= 32U) {
+            WEED_SHORT_ROWS(1, 2, 16);
+        } else {
+            WEED_SHORT_ROWS(1, 4, 32);
+        }
+#undef WEED_SHORT_ROWS
     } else if (how == AXIS_WAVE) {
         if (g.axis_len <= 16U * 64U) {
             softmax_wave_rows_kernel<1, 16, true><<<wave_row_blocks(g.rows), 256, 0, stream()>>>(a_dev, out_dev, g);
@@ -1105,13 +1416,20 @@ int weed_hip_softmax_f32(uint32_t rank, const uint32_t *shape, uint32_t axis, co
         // (with more rows the two passes over 32 rows per workgroup are faster: 16-row tiles are half lines.
         // 4096 rows of 2048: 22 us against 35; 16384 rows: 83 against 72; 65536 rows: 427 against 369)
         softmax_strided_cached_kernel<16><<<(g.rows + 15) / 16, kStridedThreads, 0, stream()>>>(a_dev, out_dev, g);
+    } else if (const BandGeom bg = choose_bands(g, 4096U); bg.bands != 0U) {
+        // (up to 4096 rows of at least 4096 strided elements -- with 8192 rows and more the walks over 32 rows per
+        // workgroup are as fast or faster: 8192 x 8192 174 against 187 us; 4096 x 32768 372 us here against 525 --: 64 rows of 32768 25 us, where 16 rows per workgroup took
+        // 166; 256 rows of 8192 16 us against 25 with the narrow tiles below; 2048 rows of 16384 83 against 127)
+        const dim3 grid((g.rows + 63U) / 64U, bg.bands);
+        band_partial_kernel<3><<<grid, 256, 0, stream()>>>(a_dev, g, bg);
+        band_merge_kernel<3><<<(g.rows + 63U) / 64U, 256, 0, stream()>>>(out_dev, g, bg);
+        band_softmax_finish_kernel<<<grid, 256, 0, stream()>>>(a_dev, out_dev, g, bg);
     } else if (g.rows < 2048U && g.axis_len <= (uint32_t)(kStridedCached * kStridedThreadsLong / 4)) {
-        // few long rows (scores of a decode step): narrow tiles, so that there are workgroups enough, and one pass
-        // (64 to 1024 rows of 8192: 22 to 42 us, where 16 rows per workgroup and two passes take 60 to 70)
+        // few rows of 2049 to 4095 elements: narrow tiles, so that there are workgroups enough, and one pass
         softmax_strided_cached_kernel<4, kStridedThreadsLong, true>
             <<<8 * ((g.rows + 31) / 32), kStridedThreadsLong, 0, stream()>>>(a_dev, out_dev, g);
     } else if (g.rows < 3072U && g.axis_len <= (uint32_t)(kStridedCached * kStridedThreadsLong / 8)) {
-        // (2048 rows of 8192: 49 us against 75; from 3072 rows on the two passes over 16 or 32 rows are as fast or faster)
+        // (2049 to 3071 rows; from 3072 rows on the two passes over 16 or 32 rows are as fast or faster)
         softmax_strided_cached_kernel<8, kStridedThreadsLong, true>
             <<<8 * ((g.rows + 63) / 64), kStridedThreadsLong, 0, stream()>>>(a_dev, out_dev, g);
     } else if (how == AXIS_ROWS32) {
@@ -1136,11 +1454,21 @@ int weed_hip_reduce_f32(int op, uint32_t rank, const uint32_t *shape, uint32_t a
     WEED_HIP_TRY(make_geom(fn, rank, shape, axis, a_off, a_stride, o_off, o_stride, false, g));
     ProfileScope prof("reduce");
     const AxisLaunch how = choose_axis_launch(g, a_dev, out_dev, false);
+    const BandGeom bands = choose_bands(g, 3072U); // (4096 rows of 4096 to 8192: 13 and 23 us without bands, 16 and 26 with)
 #define WEED_LAUNCH_REDUCE(OP)                                                                                         \
-    if (how == AXIS_CONTIGUOUS) {                                                                                      \
+    if (bands.bands != 0U && how != AXIS_CONTIGUOUS && how != AXIS_ROW && how != AXIS_WAVE && how != AXIS_WAVE_VEC) {  \
+        band_partial_kernel<OP><<<dim3((g.rows + 63U) / 64U, bands.bands), 256, 0, stream()>>>(a_dev, g, bands);       \
+        band_merge_kernel<OP><<<(g.rows + 63U) / 64U, 256, 0, stream()>>>(out_dev, g, bands);                         \
+    } else if (how == AXIS_CONTIGUOUS) {                                                                               \
         reduce_contiguous_kernel<OP, 256><<<g.rows, 256, 0, stream()>>>(a_dev, out_dev, g);                            \
+    } else if (how == AXIS_WAVE_VEC && g.axis_len <= 64U) {                                                            \
+        reduce_short_rows_kernel<OP, 4, 4><<<short_row_blocks(g.rows, 4), 256, 0, stream()>>>(a_dev, out_dev, g);      \
+    } else if (how == AXIS_WAVE_VEC && g.axis_len <= 256U) {                                                           \
+        reduce_short_rows_kernel<OP, 4, 16><<<short_row_blocks(g.rows, 16), 256, 0, stream()>>>(a_dev, out_dev, g);    \
     } else if (how == AXIS_WAVE_VEC) {                                                                                 \
         reduce_wave_rows_kernel<OP, 4><<<wave_row_blocks(g.rows), 256, 0, stream()>>>(a_dev, out_dev, g);              \
+    } else if (how == AXIS_WAVE && g.axis_len <= 64U) {                                                                \
+        reduce_short_rows_kernel<OP, 1, 16><<<short_row_blocks(g.rows, 16), 256, 0, stream()>>>(a_dev, out_dev, g);    \
     } else if (how == AXIS_WAVE) {                                                                                     \
         reduce_wave_rows_kernel<OP, 1><<<wave_row_blocks(g.rows), 256, 0, stream()>>>(a_dev, out_dev, g);              \
     } else if (how == AXIS_ROW) {                                                                                      \
