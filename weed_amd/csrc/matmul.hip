@@ -115,16 +115,16 @@ typedef float float4v __attribute__((ext_vector_type(4)));
 
 constexpr int TM = 128, TN = 128, TK = 16, PITCH = 132;
 
-template <bool A_ICONTIG, bool B_KCONTIG, bool EDGE = false>
+template <bool A_ICONTIG, bool B_KCONTIG, bool EDGE = false, bool SPLIT = EDGE>
 __global__ void __launch_bounds__(256) matmul_mfma_kernel(const float *__restrict__ a, const float *__restrict__ b,
                                                           float *__restrict__ out, MatGeom g_launch,
                                                           uint32_t k_per_split = 0)
 {
-    // EDGE instances may split k over blockIdx.z (unbatched products only, so batch_geom adds nothing then):
+    // EDGE and SPLIT instances may split k over blockIdx.z (unbatched products only, so batch_geom adds nothing then):
     // k_per_split != 0 means `out` is the dense scratch part[split][row][column] and a second kernel adds the splits
     MatGeom g = batch_geom(g_launch);
-    const uint32_t k_first = (EDGE && k_per_split) ? blockIdx.z * k_per_split : 0U;
-    if (EDGE && k_per_split) {
+    const uint32_t k_first = (SPLIT && k_per_split) ? blockIdx.z * k_per_split : 0U;
+    if (SPLIT && k_per_split) {
         g.K = min(g.K, k_first + k_per_split);
     }
     // Row pitch of a staged slice.  An operand that arrives contiguous along its own index is stored with 16-byte
@@ -262,7 +262,7 @@ __global__ void __launch_bounds__(256) matmul_mfma_kernel(const float *__restric
                 for (int e = 0; e < 4; ++e) {
                     v[e] = (!EDGE || col < g.N) ? with_bias(g, acc[x][y][4 * r4 + e], col) : 0.0f;
                 }
-                if (EDGE && k_per_split) {
+                if (SPLIT && k_per_split) {
                     float *part = out + ((uint64_t)blockIdx.z * g.M + row) * g.N + col;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
@@ -736,6 +736,8 @@ bool mfma_eligible(const MatGeom &g, const float *a, const float *b, const float
 
 namespace {
 
+int launch_matmul_body(const char *fn, const MatGeom &g, uint32_t batch, const float *a_dev, const float *b_dev, float *out_dev);
+
 int launch_matmul(const char *fn, const MatGeom &g, uint32_t batch, const float *a_dev, const float *b_dev, float *out_dev)
 {
     WEED_HIP_REQUIRE(a_dev && b_dev && out_dev, "%s: null pointer", fn);
@@ -743,6 +745,12 @@ int launch_matmul(const char *fn, const MatGeom &g, uint32_t batch, const float 
     if (!g.M || !g.N || !batch) {
         return WEED_HIP_OK;
     }
+    ProfileScope prof("matmul");
+    return launch_matmul_body(fn, g, batch, a_dev, b_dev, out_dev);
+}
+
+int launch_matmul_body(const char *fn, const MatGeom &g, uint32_t batch, const float *a_dev, const float *b_dev, float *out_dev)
+{
     WEED_HIP_REQUIRE(batch <= 65535u, "%s: %u products in one call (at most 65535)", fn, batch);
     if (batch > 1) {
         // the kernels add a product's batch offsets to the operand offsets in 32 bits: refuse what would wrap
@@ -753,10 +761,34 @@ int launch_matmul(const char *fn, const MatGeom &g, uint32_t batch, const float 
                          "%s: a batch offset exceeds 32 bits", fn);
     }
     const uint32_t M = g.M, N = g.N, K = g.K;
-    ProfileScope prof("matmul");
     // few output tiles and a long k: the tiles' k ranges are split over more workgroups (guarded instances below)
     const uint64_t out_tiles = (uint64_t)((M + TM - 1) / TM) * ((N + TN - 1) / TN) * batch;
     const bool split_k = batch == 1 && M > 16 && N > 16 && out_tiles < 128 && K >= 1024;
+    if (split_k && mfma_eligible(g, a_dev, b_dev, out_dev) && !skinny_eligible(g, b_dev)) {
+        // few whole tiles and a long k: the unguarded kernel over k ranges, a second kernel adds them
+        uint32_t splits = std::min<uint32_t>((uint32_t)(256 / out_tiles), K / 256);
+        const uint32_t k_per_split = ((K + splits - 1) / splits + TK - 1) / TK * TK;
+        splits = (K + k_per_split - 1) / k_per_split;
+        if (splits >= 2) {
+            WEED_HIP_TRY(grow_split_scratch(fn, sizeof(float) * (size_t)splits * M * N));
+            const dim3 grid(M / TM, N / TN, splits);
+            WEED_HIP_REQUIRE(grid.y <= 65535u, "%s: N = %u too large", fn, N);
+            const bool a_i = g.a_s0 == 1, b_k = g.b_s0 == 1;
+            if (a_i && b_k) {
+                matmul_mfma_kernel<true, true, false, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, g_split_ws, g, k_per_split);
+            } else if (a_i) {
+                matmul_mfma_kernel<true, false, false, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, g_split_ws, g, k_per_split);
+            } else if (b_k) {
+                matmul_mfma_kernel<false, true, false, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, g_split_ws, g, k_per_split);
+            } else {
+                matmul_mfma_kernel<false, false, false, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, g_split_ws, g, k_per_split);
+            }
+            WEED_HIP_LAUNCH_CHECK();
+            matmul_split_sum_kernel<<<dim3((M * N + 255) / 256, 1, 1), 256, 0, stream()>>>(g_split_ws, out_dev, g, splits);
+            WEED_HIP_LAUNCH_CHECK();
+            return WEED_HIP_OK;
+        }
+    }
     if (!split_k && mfma_eligible(g, a_dev, b_dev, out_dev)) {
         const dim3 grid(M / TM, N / TN, batch);
         WEED_HIP_REQUIRE(grid.y <= 65535u, "%s: N = %u too large", fn, N);
@@ -811,6 +843,38 @@ int launch_matmul(const char *fn, const MatGeom &g, uint32_t batch, const float 
         }
         WEED_HIP_LAUNCH_CHECK();
         return WEED_HIP_OK;
+    }
+    // Ragged sizes around an interior of whole 128 x 128 tiles (a prefill of 1000 tokens): the unguarded kernel takes the
+    // interior, the strips behind it go the way their own shapes call for (1000 x 4096 x 4096: 379 us, 469 with every
+    // tile guarded; not below 2^32 multiply-adds, where the extra launches cost more than the guards).
+    if (batch == 1 && M >= TM && N >= TN && (M % TM || N % TN) && (uint64_t)M * N * K >= (1ull << 32)) {
+        MatGeom in = g;
+        in.M = M / TM * TM;
+        in.N = N / TN * TN;
+        const uint64_t lim = 0xffffffffull;
+        const bool fits = (uint64_t)g.a_off + (uint64_t)in.M * g.a_s0 <= lim && (uint64_t)g.o_off + (uint64_t)in.M * g.o_s0 <= lim &&
+            (uint64_t)g.b_off + (uint64_t)in.N * g.b_s1 <= lim && (uint64_t)g.o_off + (uint64_t)in.N * g.o_s1 <= lim &&
+            (uint64_t)g.bias_off + (uint64_t)in.N * g.bias_s <= lim;
+        if (fits && mfma_eligible(in, a_dev, b_dev, out_dev)) {
+            WEED_HIP_TRY(launch_matmul_body(fn, in, 1, a_dev, b_dev, out_dev));
+            if (in.M < M) { // the rows behind, all columns
+                MatGeom e = g;
+                e.M = M - in.M;
+                e.a_off += in.M * g.a_s0;
+                e.o_off += in.M * g.o_s0;
+                WEED_HIP_TRY(launch_matmul_body(fn, e, 1, a_dev, b_dev, out_dev));
+            }
+            if (in.N < N) { // the columns behind, the interior's rows
+                MatGeom e = g;
+                e.M = in.M;
+                e.N = N - in.N;
+                e.b_off += in.N * g.b_s1;
+                e.o_off += in.N * g.o_s1;
+                e.bias_off += in.N * g.bias_s;
+                WEED_HIP_TRY(launch_matmul_body(fn, e, 1, a_dev, b_dev, out_dev));
+            }
+            return WEED_HIP_OK;
+        }
     }
     if (M > 16 && N > 16 && K >= 8) {
         // ragged, unaligned or doubly strided: matrix-core tiles with guarded loads and stores
