@@ -106,7 +106,8 @@ def test_matmul_decode_projections(gpu, oracle, M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(200, 300, 4096), (128, 128, 2048), (130, 70, 1030), (17, 17, 8), (257, 129, 33),
-                                   (1000, 1000, 100), (1000, 1100, 512), (300, 4136, 1024), (129, 128, 2048)])
+                                   (1000, 1000, 100), (1000, 1100, 512), (300, 4136, 1024), (129, 128, 2048),
+                                   (260, 4100, 4096)])
 def test_matmul_matrix_core_edges(gpu, M, N, K):
     """Shapes that are not multiples of the 128 x 128 x 16 tiles, unaligned and doubly strided views, and few tiles with
     a long k (split over workgroups, summed by a second kernel): against float64, and nothing outside the output view

@@ -846,11 +846,15 @@ int launch_matmul_body(const char *fn, const MatGeom &g, uint32_t batch, const f
     }
     // Ragged sizes around an interior of whole 128 x 128 tiles (a prefill of 1000 tokens): the unguarded kernel takes the
     // interior, the strips behind it go the way their own shapes call for (1000 x 4096 x 4096: 379 us, 469 with every
-    // tile guarded; not below 2^32 multiply-adds, where the extra launches cost more than the guards).
-    if (batch == 1 && M >= TM && N >= TN && (M % TM || N % TN) && (uint64_t)M * N * K >= (1ull << 32)) {
+    // tile guarded; not below 2^32 multiply-adds, where the extra launches cost more than the guards).  (Guarded
+    // instances that read the tiles inside the matrix with the unguarded loads, one launch for everything, were
+    // measured too: 579 us for the same product -- the instance's registers and address arithmetic slow every tile.)
+    if (batch == 1 && M >= TM && N >= 2 * TN && (M % TM || N % TN) && (uint64_t)M * N * K >= (1ull << 32)) {
         MatGeom in = g;
         in.M = M / TM * TM;
         in.N = N / TN * TN;
+        if (N % TN && N % TN <= 16) in.N -= TN; // a strip of under 17 columns has no matrix-core kernel: one more tile goes with it
+                                                // (a strip of under 17 rows is the skinny kernels' own shape)
         const uint64_t lim = 0xffffffffull;
         const bool fits = (uint64_t)g.a_off + (uint64_t)in.M * g.a_s0 <= lim && (uint64_t)g.o_off + (uint64_t)in.M * g.o_s0 <= lim &&
             (uint64_t)g.b_off + (uint64_t)in.N * g.b_s1 <= lim && (uint64_t)g.o_off + (uint64_t)in.N * g.o_s1 <= lim &&
