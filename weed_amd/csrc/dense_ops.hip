@@ -1345,6 +1345,10 @@ int weed_hip_rope_f32(const uint32_t shape[4], const float *x_dev, uint32_t x_of
     return WEED_HIP_OK;
 }
 
+// Up to this many contiguous rows beyond 8192 elements get sixteen wavefronts each instead of four (one workgroup per
+// row either way; with more rows the compute units are full of four-wavefront workgroups anyway).
+constexpr uint32_t kFewLongRows = 512U;
+
 int weed_hip_softmax_f32(uint32_t rank, const uint32_t *shape, uint32_t axis, const float *a_dev, uint32_t a_off,
                          const uint32_t *a_stride, float *out_dev, uint32_t o_off, const uint32_t *o_stride)
 {
@@ -1358,6 +1362,11 @@ int weed_hip_softmax_f32(uint32_t rank, const uint32_t *shape, uint32_t axis, co
     if (how == AXIS_CONTIGUOUS) {
         if (g.axis_len <= 8U * 4U * 256U) {
             softmax_contiguous_kernel<8, 256, true><<<g.rows, 256, 0, stream()>>>(a_dev, out_dev, g);
+        } else if (g.rows <= kFewLongRows && g.axis_len <= 8U * 4U * 1024U) {
+            // few rows, each a workgroup's: sixteen wavefronts keep up to 32768 elements in registers and read once
+            softmax_contiguous_kernel<8, 1024, true><<<g.rows, 1024, 0, stream()>>>(a_dev, out_dev, g);
+        } else if (g.rows <= kFewLongRows) {
+            softmax_contiguous_kernel<8, 1024, false><<<g.rows, 1024, 0, stream()>>>(a_dev, out_dev, g);
         } else {
             softmax_contiguous_kernel<8, 256, false><<<g.rows, 256, 0, stream()>>>(a_dev, out_dev, g);
         }
