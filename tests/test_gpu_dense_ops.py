@@ -107,11 +107,12 @@ def test_matmul_decode_projections(gpu, oracle, M, N, K):
 
 @pytest.mark.parametrize("M,N,K", [(200, 300, 4096), (128, 128, 2048), (130, 70, 1030), (17, 17, 8), (257, 129, 33),
                                    (1000, 1000, 100), (1000, 1100, 512), (300, 4136, 1024), (129, 128, 2048),
-                                   (260, 4100, 4096)])
+                                   (260, 4100, 4096), (512, 4096, 1024), (760, 4096, 1024), (1000, 1000, 1028)])
 def test_matmul_matrix_core_edges(gpu, M, N, K):
     """Shapes that are not multiples of the 128 x 128 x 16 tiles, unaligned and doubly strided views, and few tiles with
-    a long k (split over workgroups, summed by a second kernel): against float64, and nothing outside the output view
-    may be written."""
+    a long k (split over workgroups, summed by a second kernel), also 128 and 192 tiles, which split in two and four:
+    against float64, and nothing outside the output view may be written.  Sizes that are multiples of 4 run the
+    instances whose 16-byte loads are checked as a whole, the others the element-wise ones."""
     import torch
     rng = np.random.default_rng(M + 2 * N + 3 * K)
     A = rng.standard_normal((M, K), dtype=np.float32)

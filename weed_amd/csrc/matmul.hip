@@ -2,6 +2,7 @@
 // src/ops/matmul.cpp:95-122).  Replaces the OpenCL kernel matmul_real (src/common/qengine.cl:598-640).
 #include "common.h"
 
+#include <cmath>
 #include <algorithm>
 #include <type_traits>
 
@@ -108,18 +109,24 @@ __global__ void __launch_bounds__(256) matmul_tiled_kernel(const float *__restri
 // are); the four combinations are template instances.  Shapes that are not multiples of the tile, operands strided
 // in both dimensions and unaligned views use the EDGE instances: the same tiles and instructions, with element-wise
 // guarded loads (zeros beyond the edges) and guarded stores; there the two flags only choose which way the threads
-// walk an operand.  Products with fewer than 17 rows or columns use the generic kernel above.
+// walk an operand.  Sizes that are not multiples of the tile in the unguarded kernel's layout (contiguous dimensions
+// of a multiple of 4 elements, 16-byte aligned) use the QUAD instances: the unguarded kernel's 16-byte loads, each
+// checked as a whole.  Products with fewer than 17 rows or columns use the generic kernel above.
 // ------------------------------------------------------------------------------------------------
 typedef float float16v __attribute__((ext_vector_type(16)));
 typedef float float4v __attribute__((ext_vector_type(4)));
 
 constexpr int TM = 128, TN = 128, TK = 16, PITCH = 132;
 
-template <bool A_ICONTIG, bool B_KCONTIG, bool EDGE = false, bool SPLIT = EDGE>
+template <bool A_ICONTIG, bool B_KCONTIG, int GUARD = 0, bool SPLIT = GUARD == 1>
 __global__ void __launch_bounds__(256) matmul_mfma_kernel(const float *__restrict__ a, const float *__restrict__ b,
                                                           float *__restrict__ out, MatGeom g_launch,
                                                           uint32_t k_per_split = 0)
 {
+    // GUARD: 0 whole tiles, nothing checked; 1 (EDGE) any shape and strides, element by element; 2 (QUAD) the layout of
+    // 0 -- one contiguous dimension per operand, 16-byte aligned, its extent a multiple of 4 -- with sizes that are not
+    // multiples of the tile: 16-byte loads, each checked as a whole.
+    constexpr bool EDGE = GUARD == 1, QUAD = GUARD == 2;
     // EDGE and SPLIT instances may split k over blockIdx.z (unbatched products only, so batch_geom adds nothing then):
     // k_per_split != 0 means `out` is the dense scratch part[split][row][column] and a second kernel adds the splits
     MatGeom g = batch_geom(g_launch);
@@ -152,6 +159,9 @@ __global__ void __launch_bounds__(256) matmul_mfma_kernel(const float *__restric
     }
 
     // two float4 per operand per thread and K slice
+    // (Guarded loads sit in branches of their own.  Issuing every load from an address clamped into the operand
+    // instead was measured twice and was slower both times: zeroed right behind the load, 1000 x 4099 x 4096 took 1076
+    // us against 488; with a bit per load kept and the zeroing left to the staging, a slice later, 543.)
     float4v ra[2], rb[2];
     auto fetch = [&](uint32_t k0) {
 #pragma unroll
@@ -174,23 +184,32 @@ __global__ void __launch_bounds__(256) matmul_mfma_kernel(const float *__restric
                 }
                 continue;
             }
+            const float4v zero4 = { 0.0f, 0.0f, 0.0f, 0.0f }; // (QUAD: each 16-byte load checked as a whole)
             if (A_ICONTIG) {
                 const uint32_t i4 = idx & 31, k = idx >> 5;
-                ra[q] = *reinterpret_cast<const float4v *>(a + (uint64_t)g.a_off + (m0 + 4 * i4) +
-                                                           (uint64_t)(k0 + k) * g.a_s1);
+                const bool in = !QUAD || (m0 + 4 * i4 < g.M && k0 + k < g.K);
+                ra[q] = in ? *reinterpret_cast<const float4v *>(a + (uint64_t)g.a_off + (m0 + 4 * i4) +
+                                                                (uint64_t)(k0 + k) * g.a_s1)
+                           : zero4;
             } else {
                 const uint32_t k4 = idx & 3, i = idx >> 2;
-                ra[q] = *reinterpret_cast<const float4v *>(a + (uint64_t)g.a_off + (uint64_t)(m0 + i) * g.a_s0 +
-                                                           (k0 + 4 * k4));
+                const bool in = !QUAD || (m0 + i < g.M && k0 + 4 * k4 < g.K);
+                ra[q] = in ? *reinterpret_cast<const float4v *>(a + (uint64_t)g.a_off + (uint64_t)(m0 + i) * g.a_s0 +
+                                                                (k0 + 4 * k4))
+                           : zero4;
             }
             if (B_KCONTIG) {
                 const uint32_t k4 = idx & 3, j = idx >> 2;
-                rb[q] = *reinterpret_cast<const float4v *>(b + (uint64_t)g.b_off + (k0 + 4 * k4) +
-                                                           (uint64_t)(n0 + j) * g.b_s1);
+                const bool in = !QUAD || (n0 + j < g.N && k0 + 4 * k4 < g.K);
+                rb[q] = in ? *reinterpret_cast<const float4v *>(b + (uint64_t)g.b_off + (k0 + 4 * k4) +
+                                                                (uint64_t)(n0 + j) * g.b_s1)
+                           : zero4;
             } else {
                 const uint32_t j4 = idx & 31, k = idx >> 5;
-                rb[q] = *reinterpret_cast<const float4v *>(b + (uint64_t)g.b_off + (uint64_t)(k0 + k) * g.b_s0 +
-                                                           (n0 + 4 * j4));
+                const bool in = !QUAD || (n0 + 4 * j4 < g.N && k0 + k < g.K);
+                rb[q] = in ? *reinterpret_cast<const float4v *>(b + (uint64_t)g.b_off + (uint64_t)(k0 + k) * g.b_s0 +
+                                                                (n0 + 4 * j4))
+                           : zero4;
             }
         }
     };
@@ -260,7 +279,7 @@ __global__ void __launch_bounds__(256) matmul_mfma_kernel(const float *__restric
                 float v[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    v[e] = (!EDGE || col < g.N) ? with_bias(g, acc[x][y][4 * r4 + e], col) : 0.0f;
+                    v[e] = (GUARD == 0 || col < g.N) ? with_bias(g, acc[x][y][4 * r4 + e], col) : 0.0f;
                 }
                 if (SPLIT && k_per_split) {
                     float *part = out + ((uint64_t)blockIdx.z * g.M + row) * g.N + col;
@@ -270,12 +289,16 @@ __global__ void __launch_bounds__(256) matmul_mfma_kernel(const float *__restric
                             part[(uint64_t)e * g.N] = acc[x][y][4 * r4 + e];
                         }
                     }
-                } else if (EDGE) {
+                } else if (EDGE || (QUAD && (g.o_s0 != 1 || row + 3 >= g.M))) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         if (row + e < g.M && col < g.N) {
                             dst[(uint64_t)e * g.o_s0] = v[e];
                         }
+                    }
+                } else if (QUAD) {
+                    if (col < g.N) {
+                        *reinterpret_cast<float4v *>(dst) = float4v{ v[0], v[1], v[2], v[3] };
                     }
                 } else if (g.o_s0 == 1) {
                     *reinterpret_cast<float4v *>(dst) = float4v{ v[0], v[1], v[2], v[3] };
@@ -708,10 +731,19 @@ bool skinny_eligible(const MatGeom &g, const float *b)
 bool aligned16(const float *p, uint64_t elem_off) { return (((uintptr_t)p + 4 * elem_off) & 15) == 0; }
 
 // The matrix-core kernel needs full tiles, one contiguous dimension per operand and 16-byte aligned vector accesses.
-bool mfma_eligible(const MatGeom &g, const float *a, const float *b, const float *out)
+bool mfma_eligible(const MatGeom &g, const float *a, const float *b, const float *out, bool whole_tiles = true)
 {
-    if (g.M % TM || g.N % TN || g.K % TK || !g.K) {
+    if (whole_tiles && (g.M % TM || g.N % TN || g.K % TK)) {
         return false;
+    }
+    if (!g.K) {
+        return false;
+    }
+    if (!whole_tiles) {
+        // 16-byte loads checked as a whole: the contiguous dimension's extent is a multiple of 4
+        if ((g.a_s0 == 1 ? g.M : g.K) % 4 || (g.b_s0 == 1 ? g.K : g.N) % 4) {
+            return false;
+        }
     }
     const bool a_i = g.a_s0 == 1, a_k = g.a_s1 == 1;
     const bool b_k = g.b_s0 == 1, b_j = g.b_s1 == 1;
@@ -730,6 +762,31 @@ bool mfma_eligible(const MatGeom &g, const float *a, const float *b, const float
     }
     // every product of a batch keeps the alignment
     return !((g.a_bs[0] | g.a_bs[1] | g.b_bs[0] | g.b_bs[1] | g.o_bs[0] | g.o_bs[1]) & 3);
+}
+
+// Into how many ranges to split k over workgroups (1: not at all).  The tiles run in rounds of one per compute unit,
+// each of k / splits slices plus a fixed part per workgroup (prologue, write-out: about 128 slices' worth), and a second
+// kernel adds the ranges.  So 128 tiles gain from two ranges (512 x 4096 x 4096: 308 -> 184 us: one launch of 128
+// workgroups leaves half the part idle), 192 from four (three rounds of a quarter each: 313 -> 253), 384 from two
+// (three rounds of a half instead of two whole ones: 567 -> 454), and 256 or 512 tiles from none.
+uint32_t choose_k_splits(uint64_t out_tiles, uint32_t K)
+{
+    if (out_tiles > 512) {
+        return 1;
+    }
+    const auto cost = [&](uint32_t s) {
+        const double rounds = std::ceil((double)(out_tiles * s) / 256.0);
+        return rounds * ((double)K / s + 128.0) + (s > 1 ? 40.0 + 0.3 * (double)(s * out_tiles) : 0.0);
+    };
+    uint32_t best = 1;
+    double best_cost = cost(1) * 0.92; // (a split has to gain something beyond what two measurements differ by)
+    for (uint32_t s = 2; s <= std::min(64U, K / 256U); ++s) {
+        if (cost(s) < best_cost) {
+            best_cost = cost(s);
+            best = s;
+        }
+    }
+    return best;
 }
 
 } // namespace
@@ -763,10 +820,11 @@ int launch_matmul_body(const char *fn, const MatGeom &g, uint32_t batch, const f
     const uint32_t M = g.M, N = g.N, K = g.K;
     // few output tiles and a long k: the tiles' k ranges are split over more workgroups (guarded instances below)
     const uint64_t out_tiles = (uint64_t)((M + TM - 1) / TM) * ((N + TN - 1) / TN) * batch;
-    const bool split_k = batch == 1 && M > 16 && N > 16 && out_tiles < 128 && K >= 1024;
+    const uint32_t want_splits = (batch == 1 && M > 16 && N > 16 && K >= 1024) ? choose_k_splits(out_tiles, K) : 1U;
+    const bool split_k = want_splits >= 2;
     if (split_k && mfma_eligible(g, a_dev, b_dev, out_dev) && !skinny_eligible(g, b_dev)) {
         // few whole tiles and a long k: the unguarded kernel over k ranges, a second kernel adds them
-        uint32_t splits = std::min<uint32_t>((uint32_t)(256 / out_tiles), K / 256);
+        uint32_t splits = want_splits;
         const uint32_t k_per_split = ((K + splits - 1) / splits + TK - 1) / TK * TK;
         splits = (K + k_per_split - 1) / k_per_split;
         if (splits >= 2) {
@@ -775,13 +833,13 @@ int launch_matmul_body(const char *fn, const MatGeom &g, uint32_t batch, const f
             WEED_HIP_REQUIRE(grid.y <= 65535u, "%s: N = %u too large", fn, N);
             const bool a_i = g.a_s0 == 1, b_k = g.b_s0 == 1;
             if (a_i && b_k) {
-                matmul_mfma_kernel<true, true, false, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, g_split_ws, g, k_per_split);
+                matmul_mfma_kernel<true, true, 0, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, g_split_ws, g, k_per_split);
             } else if (a_i) {
-                matmul_mfma_kernel<true, false, false, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, g_split_ws, g, k_per_split);
+                matmul_mfma_kernel<true, false, 0, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, g_split_ws, g, k_per_split);
             } else if (b_k) {
-                matmul_mfma_kernel<false, true, false, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, g_split_ws, g, k_per_split);
+                matmul_mfma_kernel<false, true, 0, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, g_split_ws, g, k_per_split);
             } else {
-                matmul_mfma_kernel<false, false, false, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, g_split_ws, g, k_per_split);
+                matmul_mfma_kernel<false, false, 0, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, g_split_ws, g, k_per_split);
             }
             WEED_HIP_LAUNCH_CHECK();
             matmul_split_sum_kernel<<<dim3((M * N + 255) / 256, 1, 1), 256, 0, stream()>>>(g_split_ws, out_dev, g, splits);
@@ -844,22 +902,37 @@ int launch_matmul_body(const char *fn, const MatGeom &g, uint32_t batch, const f
         WEED_HIP_LAUNCH_CHECK();
         return WEED_HIP_OK;
     }
-    // Ragged sizes around an interior of whole 128 x 128 tiles (a prefill of 1000 tokens): the unguarded kernel takes the
-    // interior, the strips behind it go the way their own shapes call for (1000 x 4096 x 4096: 379 us, 469 with every
-    // tile guarded; not below 2^32 multiply-adds, where the extra launches cost more than the guards).  (Guarded
+    // Ragged sizes around an interior of whole 128 x 128 tiles (a prefill of 1000 tokens): one launch takes the interior,
+    // the strips behind it go the way their own shapes call for.  Two things can pay for the extra launches (never below
+    // 2^32 multiply-adds).  Where the whole product would need the element-wise guards (a row count that is not a
+    // multiple of 4, an unaligned view), the interior does not: 1000 x 4096 x 4096 took 379 us so, 469 with every tile
+    // guarded element by element.  And where the loads are checked 16 bytes at a time anyway, the tiles run in rounds of
+    // one per compute unit, so a few tiles beyond a whole number of rounds cost a whole round: 1000 x 4096 x 4100 is
+    // 8 x 33 = 264 tiles, 582 us in one launch against 365 for N = 4096, and 407 us as an interior of 7 x 31 tiles with
+    // its two strips; 1000 x 4096 x 4096 itself is 256 tiles and stays one launch (365 us either way).  (Guarded
     // instances that read the tiles inside the matrix with the unguarded loads, one launch for everything, were
-    // measured too: 579 us for the same product -- the instance's registers and address arithmetic slow every tile.)
+    // measured too: 579 us for that product -- the instance's registers and address arithmetic slow every tile.)
     if (batch == 1 && M >= TM && N >= 2 * TN && (M % TM || N % TN) && (uint64_t)M * N * K >= (1ull << 32)) {
         MatGeom in = g;
         in.M = M / TM * TM;
         in.N = N / TN * TN;
         if (N % TN && N % TN <= 16) in.N -= TN; // a strip of under 17 columns has no matrix-core kernel: one more tile goes with it
                                                 // (a strip of under 17 rows is the skinny kernels' own shape)
+        bool strips_pay = true;
+        if (mfma_eligible(g, a_dev, b_dev, out_dev, false)) {
+            // in rounds of 256 tiles; a strip's few tiles split k and fill the part, plus what its launch costs
+            const auto tiles = [](uint32_t m, uint32_t n) { return (double)((m + TM - 1) / TM) * ((n + TN - 1) / TN); };
+            const double whole = std::ceil(tiles(M, N) / 256.0);
+            double split = std::ceil(tiles(in.M, in.N) / 256.0);
+            if (in.M < M) split += tiles(M - in.M, N) / 256.0 + 0.15;
+            if (in.N < N) split += tiles(in.M, N - in.N) / 256.0 + 0.15;
+            strips_pay = split < whole;
+        }
         const uint64_t lim = 0xffffffffull;
         const bool fits = (uint64_t)g.a_off + (uint64_t)in.M * g.a_s0 <= lim && (uint64_t)g.o_off + (uint64_t)in.M * g.o_s0 <= lim &&
             (uint64_t)g.b_off + (uint64_t)in.N * g.b_s1 <= lim && (uint64_t)g.o_off + (uint64_t)in.N * g.o_s1 <= lim &&
             (uint64_t)g.bias_off + (uint64_t)in.N * g.bias_s <= lim;
-        if (fits && mfma_eligible(in, a_dev, b_dev, out_dev)) {
+        if (strips_pay && fits && mfma_eligible(in, a_dev, b_dev, out_dev, false)) { // (k not a multiple of 16: the interior is checked per load)
             WEED_HIP_TRY(launch_matmul_body(fn, in, 1, a_dev, b_dev, out_dev));
             if (in.M < M) { // the rows behind, all columns
                 MatGeom e = g;
@@ -884,7 +957,7 @@ int launch_matmul_body(const char *fn, const MatGeom &g, uint32_t batch, const f
         // ragged, unaligned or doubly strided: matrix-core tiles with guarded loads and stores
         uint32_t splits = 1, k_per_split = 0;
         if (split_k) {
-            splits = std::min<uint32_t>((uint32_t)(256 / out_tiles), K / 256);
+            splits = want_splits;
             k_per_split = ((K + splits - 1) / splits + TK - 1) / TK * TK;
             splits = (K + k_per_split - 1) / k_per_split;
             if (splits < 2) {
@@ -898,15 +971,34 @@ int launch_matmul_body(const char *fn, const MatGeom &g, uint32_t batch, const f
         }
         const dim3 grid((M + TM - 1) / TM, (N + TN - 1) / TN, k_per_split ? splits : batch);
         WEED_HIP_REQUIRE(grid.y <= 65535u, "%s: N = %u too large", fn, N);
+        if (mfma_eligible(g, a_dev, b_dev, out_dev, false)) {
+            // the unguarded kernel's layout, sizes that are not multiples of the tile: 16-byte loads checked as a whole
+            const bool a_i = g.a_s0 == 1, b_k = g.b_s0 == 1;
+            if (a_i && b_k) {
+                matmul_mfma_kernel<true, true, 2, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, dst, g, k_per_split);
+            } else if (a_i) {
+                matmul_mfma_kernel<true, false, 2, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, dst, g, k_per_split);
+            } else if (b_k) {
+                matmul_mfma_kernel<false, true, 2, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, dst, g, k_per_split);
+            } else {
+                matmul_mfma_kernel<false, false, 2, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, dst, g, k_per_split);
+            }
+            WEED_HIP_LAUNCH_CHECK();
+            if (k_per_split) {
+                matmul_split_sum_kernel<<<dim3((M * N + 255) / 256, 1, 1), 256, 0, stream()>>>(g_split_ws, out_dev, g, splits);
+                WEED_HIP_LAUNCH_CHECK();
+            }
+            return WEED_HIP_OK;
+        }
         const bool a_i = g.a_s0 <= g.a_s1, b_k = g.b_s0 <= g.b_s1;
         if (a_i && b_k) {
-            matmul_mfma_kernel<true, true, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, dst, g, k_per_split);
+            matmul_mfma_kernel<true, true, 1><<<grid, 256, 0, stream()>>>(a_dev, b_dev, dst, g, k_per_split);
         } else if (a_i) {
-            matmul_mfma_kernel<true, false, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, dst, g, k_per_split);
+            matmul_mfma_kernel<true, false, 1><<<grid, 256, 0, stream()>>>(a_dev, b_dev, dst, g, k_per_split);
         } else if (b_k) {
-            matmul_mfma_kernel<false, true, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, dst, g, k_per_split);
+            matmul_mfma_kernel<false, true, 1><<<grid, 256, 0, stream()>>>(a_dev, b_dev, dst, g, k_per_split);
         } else {
-            matmul_mfma_kernel<false, false, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, dst, g, k_per_split);
+            matmul_mfma_kernel<false, false, 1><<<grid, 256, 0, stream()>>>(a_dev, b_dev, dst, g, k_per_split);
         }
         WEED_HIP_LAUNCH_CHECK();
         if (k_per_split) {
