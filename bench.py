@@ -364,7 +364,8 @@ def plan_scan(capi, torch, steps=100, warmup=WARMUP_FLOOR_EXTRA, d=128):
     """The decode planner's default plan against the plain three-kernel plan (query kernel, attention, merge) over a
     grid of batch sizes, context lengths, group sizes and ragged batches: microseconds per call by two events around
     `steps` back-to-back calls (the better of two such measurements per plan).  A record to check changes of the planner's thresholds against: `behind` lists the
-    shapes where the default is more than 3 us slower than three kernels."""
+    shapes where the default is more than 3 us slower than three kernels, `differ` those where the two plans' results
+    are further apart than the GPU tests allow (2e-5 relative + 2e-6)."""
     import random
     flags = capi.ATTN_ROTATE_Q | capi.ATTN_UNROTATE_OUT
     rk, rv = torch.zeros(d * d, device="cuda"), torch.zeros(d * d, device="cuda")
@@ -386,7 +387,7 @@ def plan_scan(capi, torch, steps=100, warmup=WARMUP_FLOOR_EXTRA, d=128):
         shapes.append(("ragged 4096..8192", 8, 32, [rnd.randint(4096, 8192) for _ in range(S)]))
         shapes.append(("ragged 512..8192", 8, 32, [rnd.randint(512, 8192) for _ in range(S)]))
         shapes.append(("half 8192 half 1024", 8, 32, [8192 if i % 2 == 0 else 1024 for i in range(S)]))
-    rows, behind = [], []
+    rows, behind, differ = [], [], []
     for kind, Hkv, Hq, lens in shapes:
         S = len(lens)
         cache = capi.KVCache(capi.KV_LLOYDMAX, S, Hkv, d, max(lens), 3, 4, 0, 0)
@@ -421,14 +422,31 @@ def plan_scan(capi, torch, steps=100, warmup=WARMUP_FLOOR_EXTRA, d=128):
                 us[i % 2] = min(us[i % 2], t)
             finally:
                 capi.decode_tuning()
+        # the two plans' results, element by element (they add the same partial results in different places)
+        results = []
+        for kw in ({}, dict(separate_merge=True, separate_query=True)):
+            capi.decode_tuning(**kw)
+            try:
+                out.zero_()
+                cache.decode_attn(q, out, capi.GQA_BLOCKED, flags)
+                torch.cuda.synchronize()
+                results.append(out.clone())
+            finally:
+                capi.decode_tuning()
+        diff = (results[0] - results[1]).abs()
         row = {"kind": kind, "n_seq": S, "kv_heads": Hkv, "q_heads": Hq,
                "ctx": lens[0] if len(set(lens)) == 1 else [min(lens), max(lens)], "default_us": round(us[0], 2),
-               "default_kernels": kernels, "three_kernels_us": round(us[1], 2)}
+               "default_kernels": kernels, "three_kernels_us": round(us[1], 2),
+               "max_abs_difference": float(diff.max())}
         rows.append(row)
         if us[0] > us[1] + 3.0:
             behind.append(row)
+        if bool((diff > 2e-5 * results[1].abs() + 2e-6).any()) or not bool(torch.isfinite(results[0]).all()):
+            differ.append(row)
+        del results, diff
         cache.close()
-    return {"plan_scan": rows, "behind_three_kernels_by_more_than_3us": behind, "steps": steps, "warmup": warmup,
+    return {"plan_scan": rows, "behind_three_kernels_by_more_than_3us": behind,
+            "results_differ_by_more_than_2e-5_relative_plus_2e-6": differ, "steps": steps, "warmup": warmup,
             "head_dim": d}
 
 
