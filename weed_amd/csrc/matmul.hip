@@ -661,6 +661,241 @@ __global__ void __launch_bounds__(64 * kWideWaves)
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Whole tiles on the bfloat16 matrix instruction without giving up fp32 results: both operands are split exactly into
+// three bfloat16 parts (split_bf16x3 above) and six of the nine products of parts -- all but the three smallest, which
+// lie below 2^-24 of the terms -- are accumulated in fp32 by v_mfma_f32_32x32x16_bf16.  Six instructions of 32 cycles
+// do the work of eight fp32 instructions of 64, so the matrix pipe has 3/8 of the cycles to spend.  The error against
+// the exact product is that of a chain of fp32 additions (about 1.2e-7 of the sum of |a.b|).  An operand that is not
+// finite gives NaN where a plain fp32 product would give an infinity (inf - inf in the split).
+//   workgroup = 4 wavefronts, tile 128 x 128, each wavefront a 64 x 64 quadrant = 2 x 2 instruction tiles;
+//   k in slices of 32: the slice is fetched as fp32 (16 values per thread and operand) while the previous one is
+//   multiplied, split by the thread that fetched it and staged in LDS as [part][row][k] bfloat16 (80 bytes per row, so
+//   the 16-byte operand reads of 16 neighbouring rows fall on different banks); one LDS buffer, two barriers per slice,
+//   two workgroups per compute unit to overlap them.
+// ------------------------------------------------------------------------------------------------
+constexpr int SK = 32;     // k per slice
+constexpr int SPITCH = 40; // bfloat16 per staged row: 32 k + 8 of padding
+
+// Which (row, k) of the 128 x 32 slice a thread fetches and stages.
+//  ALONG_ROWS (the operand is contiguous along its row index): thread = (k quad kq = lane % 8, row quad i4 = 8 wave +
+//    lane / 8): four 16-byte loads, rows 4 i4 .. + 3 at k = 4 kq + e; a wavefront reads eight k, 128 contiguous bytes
+//    each.  It stores 8 bytes (four k) per row and part: 32 neighbouring lanes hit 32 different pairs of banks.
+//  else (contiguous along k): two units u = tid + 256 q of (row, k octet kg = u % 4): two 16-byte loads each, four
+//    lanes read a row's 128 bytes; rows are permuted inside groups of 16 so that the 16-byte stores of 16 neighbouring
+//    lanes hit different banks.
+// GUARD: sizes that are not multiples of the tile (the contiguous dimension's extent a multiple of 4): every 16-byte
+// load is checked as a whole against the operand's `rows` and `k_end`, zeros beyond.
+template <bool ALONG_ROWS, bool GUARD>
+__device__ __forceinline__ void split_fetch(const float *__restrict__ p, uint64_t off, uint32_t s_row, uint32_t s_k,
+                                            uint32_t row0, uint32_t k0, uint32_t rows, uint32_t k_end, float4v (&r)[4])
+{
+    const uint32_t tid = threadIdx.x;
+    const float4v zero4 = { 0.0f, 0.0f, 0.0f, 0.0f };
+    if constexpr (ALONG_ROWS) {
+        const uint32_t kq = tid & 7, i4 = tid >> 3;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const bool in = !GUARD || (row0 + 4 * i4 < rows && k0 + 4 * kq + e < k_end);
+            r[e] = in ? *reinterpret_cast<const float4v *>(p + off + (row0 + 4 * i4) + (uint64_t)(k0 + 4 * kq + e) * s_k)
+                      : zero4;
+        }
+    } else {
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const uint32_t u = tid + 256 * q, kg = u & 3;
+            const uint32_t row = (u >> 6) * 16 + 4 * ((u >> 2) & 3) + ((u >> 4) & 3);
+            const float *src = p + off + (uint64_t)(row0 + row) * s_row + (k0 + 8 * kg);
+            const bool in0 = !GUARD || (row0 + row < rows && k0 + 8 * kg < k_end);
+            const bool in1 = !GUARD || (row0 + row < rows && k0 + 8 * kg + 4 < k_end);
+            r[2 * q] = in0 ? *reinterpret_cast<const float4v *>(src) : zero4;
+            r[2 * q + 1] = in1 ? *reinterpret_cast<const float4v *>(src + 4) : zero4;
+        }
+    }
+}
+
+template <bool ALONG_ROWS>
+__device__ __forceinline__ void split_stage(uint16_t (*S)[TM][SPITCH], const float4v (&r)[4])
+{
+    const uint32_t tid = threadIdx.x;
+    if constexpr (ALONG_ROWS) {
+        const uint32_t kq = tid & 7, i4 = tid >> 3;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            uint32_t part[3][4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                split_bf16x3(r[e][x], part[0][e], part[1][e], part[2][e]);
+            }
+#pragma unroll
+            for (int pl = 0; pl < 3; ++pl) {
+                *reinterpret_cast<uint2w *>(&S[pl][4 * i4 + x][4 * kq]) =
+                    uint2w{ pack_upper_halves(part[pl][0], part[pl][1]), pack_upper_halves(part[pl][2], part[pl][3]) };
+            }
+        }
+    } else {
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const uint32_t u = tid + 256 * q, kg = u & 3;
+            const uint32_t row = (u >> 6) * 16 + 4 * ((u >> 2) & 3) + ((u >> 4) & 3);
+            const float v[8] = { r[2 * q][0],     r[2 * q][1],     r[2 * q][2],     r[2 * q][3],
+                                 r[2 * q + 1][0], r[2 * q + 1][1], r[2 * q + 1][2], r[2 * q + 1][3] };
+            uint4w part[3];
+            split_eight(v, part);
+#pragma unroll
+            for (int pl = 0; pl < 3; ++pl) {
+                *reinterpret_cast<uint4w *>(&S[pl][row][8 * kg]) = part[pl];
+            }
+        }
+    }
+}
+
+// k_per_split != 0 (unbatched products): blockIdx.z takes the k range [z k_per_split, ...) and `out` is the dense
+// scratch part[split][row][column], which a second kernel adds up.
+template <bool A_ICONTIG, bool B_KCONTIG, bool GUARD>
+__global__ void __launch_bounds__(256) matmul_split_mfma_kernel(const float *__restrict__ a, const float *__restrict__ b,
+                                                                float *__restrict__ out, MatGeom g_launch,
+                                                                uint32_t k_per_split)
+{
+    const MatGeom g = batch_geom(g_launch);
+    const uint32_t k_first = k_per_split ? blockIdx.z * k_per_split : 0U;
+    const uint32_t k_end = k_per_split ? min(g.K, k_first + k_per_split) : g.K;
+    __shared__ __attribute__((aligned(16))) uint16_t As[3][TM][SPITCH];
+    __shared__ __attribute__((aligned(16))) uint16_t Bs[3][TN][SPITCH];
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t wi = wave >> 1, wj = wave & 1;
+    const uint32_t m0 = blockIdx.x * TM, n0 = blockIdx.y * TN;
+    const uint32_t l32 = lane & 31, lk = lane >> 5;
+
+    float16v acc[2][2];
+#pragma unroll
+    for (int x = 0; x < 2; ++x) {
+#pragma unroll
+        for (int y = 0; y < 2; ++y) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                acc[x][y][r] = 0.0f;
+            }
+        }
+    }
+
+    float4v ra[4], rb[4];
+    auto fetch = [&](uint32_t k0) {
+        // a: rows are the row index i (stride a_s0), k has stride a_s1; b: "rows" are the columns j (stride b_s1)
+        split_fetch<A_ICONTIG, GUARD>(a, g.a_off, g.a_s0, g.a_s1, m0, k0, g.M, k_end, ra);
+        split_fetch<!B_KCONTIG, GUARD>(b, g.b_off, g.b_s1, g.b_s0, n0, k0, g.N, k_end, rb);
+    };
+    auto stage = [&]() {
+        split_stage<A_ICONTIG>(As, ra);
+        split_stage<!B_KCONTIG>(Bs, rb);
+    };
+
+    const uint32_t n_slices = (k_end - k_first + SK - 1) / SK;
+    fetch(k_first);
+    stage();
+    __syncthreads();
+    for (uint32_t kt = 0; kt < n_slices; ++kt) {
+        if (kt + 1 < n_slices) {
+            fetch(k_first + (kt + 1) * SK);
+        }
+#pragma unroll
+        for (int ks = 0; ks < SK / 16; ++ks) {
+            // lane (row or column l32, k octet lk) of an instruction tile
+            bf16x8 A[2][3], B[2][3];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+#pragma unroll
+                for (int pl = 0; pl < 3; ++pl) {
+                    A[t][pl] = __builtin_bit_cast(
+                        bf16x8, *reinterpret_cast<const uint4w *>(&As[pl][64 * wi + 32 * t + l32][16 * ks + 8 * lk]));
+                    B[t][pl] = __builtin_bit_cast(
+                        bf16x8, *reinterpret_cast<const uint4w *>(&Bs[pl][64 * wj + 32 * t + l32][16 * ks + 8 * lk]));
+                }
+            }
+            // the small products first
+#pragma unroll
+            for (int x = 0; x < 2; ++x) {
+#pragma unroll
+                for (int y = 0; y < 2; ++y) {
+                    acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A[x][2], B[y][0], acc[x][y], 0, 0, 0);
+                    acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A[x][1], B[y][1], acc[x][y], 0, 0, 0);
+                    acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A[x][0], B[y][2], acc[x][y], 0, 0, 0);
+                    acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A[x][1], B[y][0], acc[x][y], 0, 0, 0);
+                    acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A[x][0], B[y][1], acc[x][y], 0, 0, 0);
+                    acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A[x][0], B[y][0], acc[x][y], 0, 0, 0);
+                }
+            }
+        }
+        __syncthreads(); // everybody has read the slice
+        if (kt + 1 < n_slices) {
+            stage();
+        }
+        __syncthreads();
+    }
+
+    // register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its 32 x 32 tile
+#pragma unroll
+    for (int x = 0; x < 2; ++x) {
+#pragma unroll
+        for (int y = 0; y < 2; ++y) {
+            const uint32_t col = n0 + 64 * wj + 32 * y + l32;
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                const uint32_t row = m0 + 64 * wi + 32 * x + 8 * r4 + 4 * lk;
+                float *dst = out + (uint64_t)g.o_off + (uint64_t)row * g.o_s0 + (uint64_t)col * g.o_s1;
+                if (k_per_split) {
+                    float *part = out + ((uint64_t)blockIdx.z * g.M + row) * g.N + col;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if (!GUARD || (row + e < g.M && col < g.N)) {
+                            part[(uint64_t)e * g.N] = acc[x][y][4 * r4 + e];
+                        }
+                    }
+                    continue;
+                }
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    v[e] = (!GUARD || col < g.N) ? with_bias(g, acc[x][y][4 * r4 + e], col) : 0.0f;
+                }
+                if (GUARD && (g.o_s0 != 1 || row + 3 >= g.M)) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if (row + e < g.M && col < g.N) {
+                            dst[(uint64_t)e * g.o_s0] = v[e];
+                        }
+                    }
+                } else if (g.o_s0 == 1) {
+                    if (!GUARD || col < g.N) {
+                        *reinterpret_cast<float4v *>(dst) = float4v{ v[0], v[1], v[2], v[3] };
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        dst[(uint64_t)e * g.o_s0] = v[e];
+                    }
+                }
+            }
+        }
+    }
+}
+
+// Launches the instance for the operands' layouts (a contiguous along i or k, b along k or j).
+template <bool GUARD>
+void launch_split_mfma(dim3 grid, const float *a_dev, const float *b_dev, float *dst, const MatGeom &g, uint32_t k_per_split)
+{
+    const bool a_i = g.a_s0 == 1, b_k = g.b_s0 == 1;
+    if (a_i && b_k) {
+        matmul_split_mfma_kernel<true, true, GUARD><<<grid, 256, 0, stream()>>>(a_dev, b_dev, dst, g, k_per_split);
+    } else if (a_i) {
+        matmul_split_mfma_kernel<true, false, GUARD><<<grid, 256, 0, stream()>>>(a_dev, b_dev, dst, g, k_per_split);
+    } else if (b_k) {
+        matmul_split_mfma_kernel<false, true, GUARD><<<grid, 256, 0, stream()>>>(a_dev, b_dev, dst, g, k_per_split);
+    } else {
+        matmul_split_mfma_kernel<false, false, GUARD><<<grid, 256, 0, stream()>>>(a_dev, b_dev, dst, g, k_per_split);
+    }
+}
+
 // out = sum over the k splits, in rising split order.
 __global__ void __launch_bounds__(256) matmul_split_sum_kernel(const float *__restrict__ part, float *__restrict__ out,
                                                               MatGeom g_launch, uint32_t splits)
@@ -825,14 +1060,17 @@ int launch_matmul_body(const char *fn, const MatGeom &g, uint32_t batch, const f
     if (split_k && mfma_eligible(g, a_dev, b_dev, out_dev) && !skinny_eligible(g, b_dev)) {
         // few whole tiles and a long k: the unguarded kernel over k ranges, a second kernel adds them
         uint32_t splits = want_splits;
-        const uint32_t k_per_split = ((K + splits - 1) / splits + TK - 1) / TK * TK;
+        const uint32_t k_unit = K % SK == 0 ? SK : TK; // (whole slices of the kernel that takes the ranges)
+        const uint32_t k_per_split = ((K + splits - 1) / splits + k_unit - 1) / k_unit * k_unit;
         splits = (K + k_per_split - 1) / k_per_split;
         if (splits >= 2) {
             WEED_HIP_TRY(grow_split_scratch(fn, sizeof(float) * (size_t)splits * M * N));
             const dim3 grid(M / TM, N / TN, splits);
             WEED_HIP_REQUIRE(grid.y <= 65535u, "%s: N = %u too large", fn, N);
             const bool a_i = g.a_s0 == 1, b_k = g.b_s0 == 1;
-            if (a_i && b_k) {
+            if (k_per_split % SK == 0) {
+                launch_split_mfma<false>(grid, a_dev, b_dev, g_split_ws, g, k_per_split);
+            } else if (a_i && b_k) {
                 matmul_mfma_kernel<true, true, 0, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, g_split_ws, g, k_per_split);
             } else if (a_i) {
                 matmul_mfma_kernel<true, false, 0, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, g_split_ws, g, k_per_split);
@@ -851,6 +1089,12 @@ int launch_matmul_body(const char *fn, const MatGeom &g, uint32_t batch, const f
         const dim3 grid(M / TM, N / TN, batch);
         WEED_HIP_REQUIRE(grid.y <= 65535u, "%s: N = %u too large", fn, N);
         const bool a_i = g.a_s0 == 1, b_k = g.b_s0 == 1;
+        if (K % SK == 0) {
+            // six bfloat16 products of exactly split operands in place of the fp32 instruction
+            launch_split_mfma<false>(grid, a_dev, b_dev, out_dev, g, 0);
+            WEED_HIP_LAUNCH_CHECK();
+            return WEED_HIP_OK;
+        }
         if (a_i && b_k) {
             matmul_mfma_kernel<true, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, out_dev, g);
         } else if (a_i) {
@@ -973,16 +1217,7 @@ int launch_matmul_body(const char *fn, const MatGeom &g, uint32_t batch, const f
         WEED_HIP_REQUIRE(grid.y <= 65535u, "%s: N = %u too large", fn, N);
         if (mfma_eligible(g, a_dev, b_dev, out_dev, false)) {
             // the unguarded kernel's layout, sizes that are not multiples of the tile: 16-byte loads checked as a whole
-            const bool a_i = g.a_s0 == 1, b_k = g.b_s0 == 1;
-            if (a_i && b_k) {
-                matmul_mfma_kernel<true, true, 2, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, dst, g, k_per_split);
-            } else if (a_i) {
-                matmul_mfma_kernel<true, false, 2, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, dst, g, k_per_split);
-            } else if (b_k) {
-                matmul_mfma_kernel<false, true, 2, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, dst, g, k_per_split);
-            } else {
-                matmul_mfma_kernel<false, false, 2, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, dst, g, k_per_split);
-            }
+            launch_split_mfma<true>(grid, a_dev, b_dev, dst, g, k_per_split);
             WEED_HIP_LAUNCH_CHECK();
             if (k_per_split) {
                 matmul_split_sum_kernel<<<dim3((M * N + 255) / 256, 1, 1), 256, 0, stream()>>>(g_split_ws, out_dev, g, splits);
