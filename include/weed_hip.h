@@ -89,6 +89,18 @@ int weed_hip_matmul_f32(uint32_t M, uint32_t N, uint32_t K, const float *a_dev, 
                         uint32_t a_s1, const float *b_dev, uint32_t b_off, uint32_t b_s0, uint32_t b_s1, float *out_dev,
                         uint32_t o_off, uint32_t o_s0, uint32_t o_s1);
 
+/* Which matrix instruction the large products run on (no counterpart in the reference; process-wide, takes effect
+ * with the next call).  0, the default: products whose operands are contiguous along one dimension and 16-byte aligned,
+ * with more than 64 rows, run on the bfloat16 instruction with both operands split exactly into three bfloat16 parts and
+ * six of the nine products of parts accumulated in fp32 -- 1.5 times the fp32 instruction's speed and more.  The error
+ * against the exact product is the fp32 instruction's own: relative to sum_k |a_ik| |b_kj| per element, at k = 1028 over
+ * operands spanning 2^-20 .. 2^20, largest 7.1e-7 against 5.9e-7 and mean 5.8e-8 against 5.1e-8; for operands of one
+ * magnitude 8.0e-8 against 1.0e-7 and 9.1e-9 against 1.1e-8 (a sequential fp32 sum: 3.4e-7 and 2.0e-8).  An operand that
+ * is not finite gives NaN where the fp32 instruction would give an infinity.  1: the fp32 instruction everywhere (v_mfma_f32_32x32x2_f32: every product
+ * exact, sums rounded to fp32 in ascending k per 16-k slice).  Products with at most 64 rows against a k-contiguous
+ * weight, and unaligned or doubly strided operands, do not depend on it. */
+int weed_hip_matmul_tuning(int32_t fp32_instruction);
+
 /* batch[0] * batch[1] independent products in one launch: product (c0, c1) uses the offsets
  * off + c0 * bs[0] + c1 * bs[1] of each operand.  The reference has no device entry for this: Tensor::matmul loops
  * over the leading dimensions on the host and calls the 2-D product once per index (src/tensors/tensor.cpp:1213-1272);

@@ -61,18 +61,57 @@ def test_matmul_strided_against_checker(gpu, oracle, M, N, K):
 
 @pytest.mark.parametrize("a_col,b_col,o_col", [(True, True, True), (True, False, False), (False, True, True),
                                                  (False, False, False), (True, True, False)])
-def test_matmul_matrix_core_layouts(gpu, oracle, a_col, b_col, o_col):
-    """Full 128 x 128 x 16 tiles with every combination of contiguous dimension (the matrix-core kernel's four
-    instances) against the checker's sequential fp32 sums."""
-    M, N, K = 256, 384, 160
+@pytest.mark.parametrize("fp32_instruction,K", [(False, 160), (True, 160), (False, 144)])
+def test_matmul_matrix_core_layouts(gpu, oracle, a_col, b_col, o_col, fp32_instruction, K):
+    """Full 128 x 128 tiles with every combination of contiguous dimension (the four instances of the kernel on the
+    bfloat16 instruction with split operands, of the one on the fp32 instruction when that is asked for, and of the
+    latter for a k that is a multiple of 16 but not of 32) against the checker's sequential fp32 sums."""
+    M, N = 256, 384
     rng = np.random.default_rng(M + N + K + a_col * 4 + b_col * 2 + o_col)
     A = rng.standard_normal((M, K), dtype=np.float32)
     B = rng.standard_normal((K, N), dtype=np.float32)
     want = np.zeros(M * N, dtype=np.float32)
     oracle.matmul(M, N, K, A.reshape(-1), (0, K, 1), B.reshape(-1), (0, N, 1), want, (0, N, 1))
     C = (col_major if o_col else dev)(np.zeros((M, N), dtype=np.float32))
-    gpu.matmul((col_major if a_col else dev)(A), (col_major if b_col else dev)(B), C)
+    gpu.matmul_tuning(fp32_instruction)
+    try:
+        gpu.matmul((col_major if a_col else dev)(A), (col_major if b_col else dev)(B), C)
+    finally:
+        gpu.matmul_tuning(False)
     np.testing.assert_allclose(C.cpu().numpy(), want.reshape(M, N), rtol=2e-5, atol=2e-5 * np.sqrt(K))
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 128, 32), (256, 384, 64), (132, 136, 36), (128, 256, 2048), (1000, 260, 1028)])
+@pytest.mark.parametrize("wide_range", [False, True])
+def test_matmul_split_products_keep_fp32_accuracy(gpu, M, N, K, wide_range):
+    """Products that run on the bfloat16 matrix instruction (both operands split exactly into three parts, six of
+    the nine products of parts kept) are as accurate as the same products on the fp32 instruction: against float64
+    and relative to sum |a||b| per element, the largest error is at most 1.5 times the fp32 instruction's (+ 5e-8) and
+    the mean error at most 1.25 times, for whole tiles, ragged sizes and k ranges, every layout, and operands whose
+    magnitudes span 2^-20 .. 2^20.  A part's product left out or mis-paired would show as 2^-16 of a term: at k = 32
+    and 64 that is ten times the errors seen."""
+    rng = np.random.default_rng(M + 3 * N + 7 * K + wide_range)
+    A = rng.standard_normal((M, K), dtype=np.float32)
+    B = rng.standard_normal((K, N), dtype=np.float32)
+    if wide_range:
+        A = (A * np.exp2(rng.integers(-20, 21, size=A.shape))).astype(np.float32)
+        B = (B * np.exp2(rng.integers(-20, 21, size=B.shape))).astype(np.float32)
+    A64, B64 = A.astype(np.float64), B.astype(np.float64)
+    want = A64 @ B64
+    scale = np.abs(A64) @ np.abs(B64)
+    for mk_a, mk_b in ((col_major, col_major), (dev, dev), (col_major, dev), (dev, col_major)):
+        err = {}
+        for fp32_instruction in (True, False):
+            C = col_major(np.zeros((M, N), dtype=np.float32))
+            gpu.matmul_tuning(fp32_instruction)
+            try:
+                gpu.matmul(mk_a(A), mk_b(B), C)
+            finally:
+                gpu.matmul_tuning(False)
+            err[fp32_instruction] = np.abs(C.cpu().numpy().astype(np.float64) - want) / scale
+        assert err[True].max() <= 1.5e-6  # (the yardstick itself is sane)
+        assert err[False].max() <= 1.5 * err[True].max() + 5e-8, (mk_a.__name__, mk_b.__name__, err[False].max(), err[True].max())
+        assert err[False].mean() <= 1.25 * err[True].mean(), (mk_a.__name__, mk_b.__name__, err[False].mean(), err[True].mean())
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (1, 100, 260), (5, 33, 1000), (16, 48, 256), (17, 16, 4100),
@@ -108,7 +147,8 @@ def test_matmul_decode_projections(gpu, oracle, M, N, K):
 @pytest.mark.parametrize("M,N,K", [(200, 300, 4096), (128, 128, 2048), (130, 70, 1030), (17, 17, 8), (257, 129, 33),
                                    (1000, 1000, 100), (1000, 1100, 512), (300, 4136, 1024), (129, 128, 2048),
                                    (260, 4100, 4096), (512, 4096, 1024), (760, 4096, 1024), (1000, 1000, 1028)])
-def test_matmul_matrix_core_edges(gpu, M, N, K):
+@pytest.mark.parametrize("fp32_instruction", [False, True])
+def test_matmul_matrix_core_edges(gpu, M, N, K, fp32_instruction):
     """Shapes that are not multiples of the 128 x 128 x 16 tiles, unaligned and doubly strided views, and few tiles with
     a long k (split over workgroups, summed by a second kernel), also 128 and 192 tiles, which split in two and four:
     against float64, and nothing outside the output view may be written.  Sizes that are multiples of 4 run the
@@ -119,6 +159,15 @@ def test_matmul_matrix_core_edges(gpu, M, N, K):
     B = rng.standard_normal((K, N), dtype=np.float32)
     want = A.astype(np.float64) @ B.astype(np.float64)
     tol = dict(rtol=2e-5, atol=4e-6 * np.sqrt(K) * 3)
+    gpu.matmul_tuning(fp32_instruction)
+    try:
+        _matrix_core_edges(gpu, M, N, K, A, B, want, tol)
+    finally:
+        gpu.matmul_tuning(False)
+
+
+def _matrix_core_edges(gpu, M, N, K, A, B, want, tol):
+    import torch
     for mk_a, mk_b in ((col_major, col_major), (dev, dev), (col_major, dev), (dev, col_major)):
         C = col_major(np.zeros((M, N), dtype=np.float32))
         gpu.matmul(mk_a(A), mk_b(B), C)
@@ -138,7 +187,7 @@ def test_matmul_matrix_core_edges(gpu, M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(3, 5, 7), (8, 4096, 1024), (16, 100, 260), (40, 640, 1024), (64, 250, 516),
-                                   (128, 256, 64), (70, 33, 19)])
+                                   (128, 256, 64), (70, 33, 19), (132, 260, 68), (256, 256, 2048)])
 def test_linear_equals_product_then_broadcast_add(gpu, M, N, K):
     """The bias added in the product's last step gives the bits of the two separate ops of Linear::forward
     (matmul, then the broadcast add), on every product kernel (generic, matrix-core tiles, both streaming kernels);

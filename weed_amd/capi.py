@@ -99,6 +99,7 @@ SIGNATURES = {
     "weed_hip_kv_decode_attn": (c_int, [c_void_p, c_int32, c_int32, c_void_p, c_uint32, U32P, c_void_p, c_uint32, U32P,
                                         c_uint32]),
     "weed_hip_kv_decode_tuning": (c_int, [c_int32, c_int32, c_int32]),
+    "weed_hip_matmul_tuning": (c_int, [c_int32]),
     "weed_hip_shutdown": (c_int, []),
     "weed_hip_kv_decode_attn_noalloc": (c_int, [c_void_p, c_int32, c_int32, c_void_p, c_uint32, U32P, c_void_p, c_uint32,
                                                 U32P, c_uint32]),
@@ -286,6 +287,11 @@ def matmul(a, b, out):
     check(load().weed_hip_matmul_f32(M, N, K, c_void_p(a.data_ptr()), 0, a.stride(0), a.stride(1),
                                      c_void_p(b.data_ptr()), 0, b.stride(0), b.stride(1), c_void_p(out.data_ptr()), 0,
                                      out.stride(0), out.stride(1)))
+
+
+def matmul_tuning(fp32_instruction=False):
+    """Large products on the fp32 matrix instruction (True) or as six bfloat16 products of split operands (default)."""
+    check(load().weed_hip_matmul_tuning(1 if fp32_instruction else 0))
 
 
 def matmul_batched(a, b, out):

@@ -2,6 +2,7 @@
 // src/ops/matmul.cpp:95-122).  Replaces the OpenCL kernel matmul_real (src/common/qengine.cl:598-640).
 #include "common.h"
 
+#include <atomic>
 #include <cmath>
 #include <algorithm>
 #include <type_traits>
@@ -487,13 +488,16 @@ typedef uint32_t uint4w __attribute__((ext_vector_type(4)));
 typedef uint32_t uint2w __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
-// w = p1 + p2 + p3 exactly, every part a bfloat16 (the upper halves of the returned words): the top 8 bits of the
-// significand, the top 8 bits of what is left, and the rest (at most 8 bits)
+// w = p1 + p2 + p3 exactly, every part a bfloat16 (the upper halves of the returned words): w rounded to 8 significant
+// bits, what is left rounded to 8 bits, and the rest (at most 8 bits).  Rounding to nearest (ties away from zero: half a
+// unit added to the bits before they are cut) keeps the second part below 2^-8 and the third below 2^-16 of w, so the
+// three products of parts that the kernels leave out stay below 2^-23 of a term; cutting the bits instead would let
+// them reach 2^-21, and all with the term's sign.  (|w| within 2^-9 of the largest float rounds up to infinity.)
 __device__ __forceinline__ void split_bf16x3(float w, uint32_t &p1, uint32_t &p2, uint32_t &p3)
 {
-    p1 = __float_as_uint(w) & 0xffff0000u;
+    p1 = (__float_as_uint(w) + 0x8000u) & 0xffff0000u;
     const float r1 = w - __uint_as_float(p1);
-    p2 = __float_as_uint(r1) & 0xffff0000u;
+    p2 = (__float_as_uint(r1) + 0x8000u) & 0xffff0000u;
     const float r2 = r1 - __uint_as_float(p2);
     p3 = __float_as_uint(r2);
 }
@@ -1030,6 +1034,10 @@ namespace {
 
 int launch_matmul_body(const char *fn, const MatGeom &g, uint32_t batch, const float *a_dev, const float *b_dev, float *out_dev);
 
+// weed_hip_matmul_tuning: the fp32 matrix instruction for every product (false: six bfloat16 products of split operands
+// where the layout allows)
+std::atomic<bool> g_fp32_instruction{ false };
+
 int launch_matmul(const char *fn, const MatGeom &g, uint32_t batch, const float *a_dev, const float *b_dev, float *out_dev)
 {
     WEED_HIP_REQUIRE(a_dev && b_dev && out_dev, "%s: null pointer", fn);
@@ -1053,6 +1061,7 @@ int launch_matmul_body(const char *fn, const MatGeom &g, uint32_t batch, const f
                          "%s: a batch offset exceeds 32 bits", fn);
     }
     const uint32_t M = g.M, N = g.N, K = g.K;
+    const bool split_parts = !g_fp32_instruction.load(std::memory_order_relaxed);
     // few output tiles and a long k: the tiles' k ranges are split over more workgroups (guarded instances below)
     const uint64_t out_tiles = (uint64_t)((M + TM - 1) / TM) * ((N + TN - 1) / TN) * batch;
     const uint32_t want_splits = (batch == 1 && M > 16 && N > 16 && K >= 1024) ? choose_k_splits(out_tiles, K) : 1U;
@@ -1060,7 +1069,7 @@ int launch_matmul_body(const char *fn, const MatGeom &g, uint32_t batch, const f
     if (split_k && mfma_eligible(g, a_dev, b_dev, out_dev) && !skinny_eligible(g, b_dev)) {
         // few whole tiles and a long k: the unguarded kernel over k ranges, a second kernel adds them
         uint32_t splits = want_splits;
-        const uint32_t k_unit = K % SK == 0 ? SK : TK; // (whole slices of the kernel that takes the ranges)
+        const uint32_t k_unit = (split_parts && K % SK == 0) ? SK : TK; // (whole slices of the kernel that takes the ranges)
         const uint32_t k_per_split = ((K + splits - 1) / splits + k_unit - 1) / k_unit * k_unit;
         splits = (K + k_per_split - 1) / k_per_split;
         if (splits >= 2) {
@@ -1068,7 +1077,7 @@ int launch_matmul_body(const char *fn, const MatGeom &g, uint32_t batch, const f
             const dim3 grid(M / TM, N / TN, splits);
             WEED_HIP_REQUIRE(grid.y <= 65535u, "%s: N = %u too large", fn, N);
             const bool a_i = g.a_s0 == 1, b_k = g.b_s0 == 1;
-            if (k_per_split % SK == 0) {
+            if (split_parts && k_per_split % SK == 0) {
                 launch_split_mfma<false>(grid, a_dev, b_dev, g_split_ws, g, k_per_split);
             } else if (a_i && b_k) {
                 matmul_mfma_kernel<true, true, 0, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, g_split_ws, g, k_per_split);
@@ -1089,7 +1098,7 @@ int launch_matmul_body(const char *fn, const MatGeom &g, uint32_t batch, const f
         const dim3 grid(M / TM, N / TN, batch);
         WEED_HIP_REQUIRE(grid.y <= 65535u, "%s: N = %u too large", fn, N);
         const bool a_i = g.a_s0 == 1, b_k = g.b_s0 == 1;
-        if (K % SK == 0) {
+        if (split_parts && K % SK == 0) {
             // six bfloat16 products of exactly split operands in place of the fp32 instruction
             launch_split_mfma<false>(grid, a_dev, b_dev, out_dev, g, 0);
             WEED_HIP_LAUNCH_CHECK();
@@ -1216,8 +1225,19 @@ int launch_matmul_body(const char *fn, const MatGeom &g, uint32_t batch, const f
         const dim3 grid((M + TM - 1) / TM, (N + TN - 1) / TN, k_per_split ? splits : batch);
         WEED_HIP_REQUIRE(grid.y <= 65535u, "%s: N = %u too large", fn, N);
         if (mfma_eligible(g, a_dev, b_dev, out_dev, false)) {
-            // the unguarded kernel's layout, sizes that are not multiples of the tile: 16-byte loads checked as a whole
-            launch_split_mfma<true>(grid, a_dev, b_dev, dst, g, k_per_split);
+            // the unguarded kernels' layout, sizes that are not multiples of the tile: 16-byte loads checked as a whole
+            const bool a_i = g.a_s0 == 1, b_k = g.b_s0 == 1;
+            if (split_parts) {
+                launch_split_mfma<true>(grid, a_dev, b_dev, dst, g, k_per_split);
+            } else if (a_i && b_k) {
+                matmul_mfma_kernel<true, true, 2, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, dst, g, k_per_split);
+            } else if (a_i) {
+                matmul_mfma_kernel<true, false, 2, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, dst, g, k_per_split);
+            } else if (b_k) {
+                matmul_mfma_kernel<false, true, 2, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, dst, g, k_per_split);
+            } else {
+                matmul_mfma_kernel<false, false, 2, true><<<grid, 256, 0, stream()>>>(a_dev, b_dev, dst, g, k_per_split);
+            }
             WEED_HIP_LAUNCH_CHECK();
             if (k_per_split) {
                 matmul_split_sum_kernel<<<dim3((M * N + 255) / 256, 1, 1), 256, 0, stream()>>>(g_split_ws, out_dev, g, splits);
@@ -1250,6 +1270,12 @@ int launch_matmul_body(const char *fn, const MatGeom &g, uint32_t batch, const f
 }
 
 } // namespace
+
+extern "C" int weed_hip_matmul_tuning(int32_t fp32_instruction)
+{
+    g_fp32_instruction.store(fp32_instruction != 0, std::memory_order_relaxed);
+    return WEED_HIP_OK;
+}
 
 extern "C" int weed_hip_matmul_f32(uint32_t M, uint32_t N, uint32_t K, const float *a_dev, uint32_t a_off,
                                    uint32_t a_s0, uint32_t a_s1, const float *b_dev, uint32_t b_off, uint32_t b_s0,
