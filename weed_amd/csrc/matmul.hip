@@ -1003,19 +1003,22 @@ bool mfma_eligible(const MatGeom &g, const float *a, const float *b, const float
     return !((g.a_bs[0] | g.a_bs[1] | g.b_bs[0] | g.b_bs[1] | g.o_bs[0] | g.o_bs[1]) & 3);
 }
 
-// Into how many ranges to split k over workgroups (1: not at all).  The tiles run in rounds of one per compute unit,
+// Into how many ranges to split k over workgroups (1: not at all).  The tiles run in rounds of two per compute unit,
 // each of k / splits slices plus a fixed part per workgroup (prologue, write-out: about 128 slices' worth), and a second
-// kernel adds the ranges.  So 128 tiles gain from two ranges (512 x 4096 x 4096: 308 -> 184 us: one launch of 128
-// workgroups leaves half the part idle), 192 from four (three rounds of a quarter each: 313 -> 253), 384 from two
-// (three rounds of a half instead of two whole ones: 567 -> 454), and 256 or 512 tiles from none.
+// kernel adds the ranges.  So 128 tiles gain from four ranges (512 x 4096 x 4096: 308 us whole on the fp32
+// instruction, 184 in two ranges; with split operands 143 in two and 108 in four), 256 tiles from two (1024 x 4096 x
+// 4096: 235 -> 204 us), and 512 tiles from none.
 uint32_t choose_k_splits(uint64_t out_tiles, uint32_t K)
 {
     if (out_tiles > 512) {
         return 1;
     }
     const auto cost = [&](uint32_t s) {
-        const double rounds = std::ceil((double)(out_tiles * s) / 256.0);
-        return rounds * ((double)K / s + 128.0) + (s > 1 ? 40.0 + 0.3 * (double)(s * out_tiles) : 0.0);
+        // (two workgroups share a compute unit and fill each other's barrier waits: together they take 1.5 times
+        // what one alone takes -- 1024 x 4096 x 4096, 256 tiles: 235 us whole, 204 in two ranges)
+        const double wgs = (double)(out_tiles * s);
+        const double rounds = std::ceil(wgs / 512.0), crowd = wgs <= 256.0 ? 1.0 : 1.5;
+        return rounds * crowd * ((double)K / s + 128.0) + (s > 1 ? 40.0 + 0.3 * (double)(s * out_tiles) : 0.0);
     };
     uint32_t best = 1;
     double best_cost = cost(1) * 0.92; // (a split has to gain something beyond what two measurements differ by)
