@@ -802,6 +802,11 @@ __global__ void __launch_bounds__(256) matmul_split_mfma_kernel(const float *__r
         if (kt + 1 < n_slices) {
             fetch(k_first + (kt + 1) * SK);
         }
+        // (a wavefront that multiplies goes ahead of one that splits and stages: the two workgroups of a compute unit
+        // start together and would otherwise stay in step, all multiplying, then all splitting; 4096^3: 187 -> 194
+        // TFLOP/s, 2048 x 4096 x 4096: 190 -> 200; the kernel on the fp32 instruction, with three workgroups per compute
+        // unit, does not gain from it: 122 against 126)
+        __builtin_amdgcn_s_setprio(1);
 #pragma unroll
         for (int ks = 0; ks < SK / 16; ++ks) {
             // lane (row or column l32, k octet lk) of an instruction tile
@@ -830,6 +835,7 @@ __global__ void __launch_bounds__(256) matmul_split_mfma_kernel(const float *__r
                 }
             }
         }
+        __builtin_amdgcn_s_setprio(0);
         __syncthreads(); // everybody has read the slice
         if (kt + 1 < n_slices) {
             stage();
