@@ -95,10 +95,14 @@ int weed_hip_matmul_f32(uint32_t M, uint32_t N, uint32_t K, const float *a_dev, 
  * six of the nine products of parts accumulated in fp32 -- 1.5 times the fp32 instruction's speed and more.  The error
  * against the exact product is the fp32 instruction's own: relative to sum_k |a_ik| |b_kj| per element, at k = 1028 over
  * operands spanning 2^-20 .. 2^20, largest 7.1e-7 against 5.9e-7 and mean 5.8e-8 against 5.1e-8; for operands of one
- * magnitude 8.0e-8 against 1.0e-7 and 9.1e-9 against 1.1e-8 (a sequential fp32 sum: 3.4e-7 and 2.0e-8).  An operand that
- * is not finite gives NaN where the fp32 instruction would give an infinity.  1: the fp32 instruction everywhere (v_mfma_f32_32x32x2_f32: every product
- * exact, sums rounded to fp32 in ascending k per 16-k slice).  Products with at most 64 rows against a k-contiguous
- * weight, and unaligned or doubly strided operands, do not depend on it. */
+ * magnitude 8.0e-8 against 1.0e-7 and 9.1e-9 against 1.1e-8 (a sequential fp32 sum: 3.4e-7 and 2.0e-8).  Two things are
+ * not kept: an operand that is not finite gives NaN where the fp32 instruction would give an infinity, and operand
+ * values below 2^-112 in magnitude lose accuracy, because their second and third parts fall below bfloat16's normal
+ * range and the instruction takes them as zeros (largest error 1.3e-6 for values around 2^-115, 3e-5 around 2^-120,
+ * 9e-4 around 2^-125; fp32 denormals count as zero), where the fp32 instruction keeps 2e-7 down to the denormals.  1: the fp32 instruction everywhere (v_mfma_f32_32x32x2_f32: every product
+ * exact, sums rounded to fp32 in ascending k per 16-k slice), also for the products of 17 to 64 rows against a
+ * k-contiguous weight, which otherwise split their operands the same way.  Products with at most 16 rows, and unaligned
+ * or doubly strided operands, do not depend on it. */
 int weed_hip_matmul_tuning(int32_t fp32_instruction);
 
 /* batch[0] * batch[1] independent products in one launch: product (c0, c1) uses the offsets

@@ -114,6 +114,27 @@ def test_matmul_split_products_keep_fp32_accuracy(gpu, M, N, K, wide_range):
         assert err[False].mean() <= 1.25 * err[True].mean(), (mk_a.__name__, mk_b.__name__, err[False].mean(), err[True].mean())
 
 
+@pytest.mark.parametrize("M,N,K", [(128, 128, 64), (40, 640, 1024), (132, 260, 68)])
+def test_matmul_on_the_fp32_instruction_keeps_tiny_operands(gpu, M, N, K):
+    """What weed_hip_matmul_tuning(1) is for: operands around 2^-120 against operands around 2^120.  On the fp32
+    instruction the product keeps fp32 accuracy (whole tiles, the 17-64-row projection, ragged sizes); split into
+    bfloat16 parts, the small operands' second and third parts would fall below bfloat16's normal range."""
+    rng = np.random.default_rng(M + N + K)
+    A = (rng.standard_normal((M, K)) * 2.0 ** -120).astype(np.float32)
+    B = (rng.standard_normal((K, N)) * 2.0 ** 120).astype(np.float32)
+    A64, B64 = A.astype(np.float64), B.astype(np.float64)
+    want = A64 @ B64
+    scale = np.abs(A64) @ np.abs(B64)
+    C = col_major(np.zeros((M, N), dtype=np.float32))
+    gpu.matmul_tuning(True)
+    try:
+        gpu.matmul(col_major(A), col_major(B), C)
+    finally:
+        gpu.matmul_tuning(False)
+    err = np.abs(C.cpu().numpy().astype(np.float64) - want) / scale
+    assert err.max() <= 1e-6, err.max()
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (1, 100, 260), (5, 33, 1000), (16, 48, 256), (17, 16, 4100),
                                    (33, 250, 516), (64, 512, 1024), (24, 600, 1100), (50, 1040, 772)])
 def test_matmul_decode_projections(gpu, oracle, M, N, K):

@@ -1129,7 +1129,7 @@ int launch_matmul_body(const char *fn, const MatGeom &g, uint32_t batch, const f
         // every wavefront of a workgroup takes a whole number of 64-k iterations
         const uint32_t k_per_wave = ((K + kSkinnyWaves - 1) / kSkinnyWaves + 63) / 64 * 64;
         const dim3 wgs((N + 15) / 16, 1, batch);
-        if (M > 16 && N >= 512 && batch == 1) {
+        if (M > 16 && N >= 512 && batch == 1 && split_parts) {
             // shared rows, k split over workgroups (about 450 workgroups in all), a second pass adds the splits
             const uint32_t col_wgs = (N + 16 * kWideWaves - 1) / (16 * kWideWaves);
             uint32_t splits = std::max(1u, std::min((448u + col_wgs / 2) / col_wgs, K / 256u));
