@@ -114,6 +114,68 @@ def test_matmul_split_products_keep_fp32_accuracy(gpu, M, N, K, wide_range):
         assert err[False].mean() <= 1.25 * err[True].mean(), (mk_a.__name__, mk_b.__name__, err[False].mean(), err[True].mean())
 
 
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_matmul_random_shapes_through_the_dispatch(gpu, seed):
+    """Forty random products per seed -- sizes that are and are not multiples of the tile or of 4, few and many rows,
+    short and long k, either contiguous dimension per operand, padded (and so unaligned) views, with and without a
+    bias, on either matrix instruction -- against the float64 product: the error stays below 2e-6 of sum |a||b| per
+    element, and nothing outside a padded output view is written.  (What the launch code chooses between: whole
+    tiles, checked 16-byte loads, element-wise guards, an interior with strips, k ranges, the streaming kernels.)"""
+    import random
+    import torch
+    rnd = random.Random(seed)
+
+    def dim():
+        c = rnd.random()
+        if c < 0.3:
+            return rnd.choice([128, 256, 384, 512, 1024])
+        if c < 0.6:
+            return 4 * rnd.randint(5, 400)
+        return rnd.randint(17, 1500)
+
+    for _ in range(40):
+        M, N = dim(), dim()
+        K = rnd.choice([32, 64, 96, 128, 1024, 2048, 4096, 4100, 1000, 36, 999, 8 * rnd.randint(1, 300)])
+        if M * N * K > 2 ** 32:
+            K = max(8, K // 8)
+        if rnd.random() < 0.15:
+            M = rnd.randint(1, 70)
+        la, lb, lo = rnd.choice("ik"), rnd.choice("kj"), rnd.choice("ij")
+        pad = rnd.choice([0, 0, 4, 1])
+
+        def view(rows, cols, contiguous_rows):
+            if contiguous_rows:
+                base = torch.randn((cols, rows + pad), device="cuda")
+                return (base[:, :rows].t() if pad else base.t()), base
+            base = torch.randn((rows, cols + pad), device="cuda")
+            return (base[:, :cols] if pad else base), base
+
+        A, _ = view(M, K, la == "i")
+        B, _ = view(K, N, lb == "k")
+        C, c_base = view(M, N, lo == "i")
+        c_base.fill_(-7.0)
+        bias = torch.randn(N, device="cuda") if rnd.random() < 0.3 else None
+        fp32_instruction = rnd.random() < 0.3
+        case = (M, N, K, la, lb, lo, pad, bias is not None, fp32_instruction)
+        gpu.matmul_tuning(fp32_instruction)
+        try:
+            if bias is not None:
+                gpu.linear(A, B, bias, C)
+            else:
+                gpu.matmul(A, B, C)
+        finally:
+            gpu.matmul_tuning(False)
+        want = A.double() @ B.double()
+        scale = A.double().abs() @ B.double().abs()
+        if bias is not None:
+            want = want + bias.double()
+            scale = scale + bias.double().abs()
+        err = ((C.double() - want).abs() / scale).max().item()
+        assert err < 2e-6, (case, err)
+        if pad:
+            assert bool((c_base[:, (M if lo == "i" else N):] == -7.0).all()), case
+
+
 @pytest.mark.parametrize("M,N,K", [(128, 128, 64), (40, 640, 1024), (132, 260, 68)])
 def test_matmul_on_the_fp32_instruction_keeps_tiny_operands(gpu, M, N, K):
     """What weed_hip_matmul_tuning(1) is for: operands around 2^-120 against operands around 2^120.  On the fp32
