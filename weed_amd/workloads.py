@@ -51,7 +51,7 @@ class Workload:
 
 
 def config(index, seed=1234, scale=1.0, n_seq=None):
-    """The BASELINE configurations 1..5 (index 5 returns the encode half; see matmul_config for the dense half).
+    """The five benchmark configurations, 1..5 (index 5 returns the encode half; see matmul_config for the dense half).
 
     `scale` < 1 shrinks context lengths (for tests that run the scalar CPU checker), `n_seq` overrides the number of
     side-by-side sequences for configurations 1-3 (the bench times many distinct caches per launch)."""
