@@ -268,7 +268,7 @@ def streaming_read(capi, torch, nbytes, steps, warmup):
 
 
 def layer_decode_step(capi, torch, np, n_calls, n_seq=64, ctx=8192, d_model=4096, n_heads=32, n_kv=8, d_ff=14336,
-                      side_by_side=False):
+                      side_by_side=False, n_tokens=1):
     """One decode step of one Qwen-style decoder layer (include/modules/qwen_decoder_layer.hpp:104-115) through the C
     ABI, launch for launch what the host mirror's QwenDecoderLayer::forward issues for a (B, 1, d_model) input:
     RMSNorm, the Q / K / V projections (with bias), RoPE on Q and K at position ctx, append, fused attention over the
@@ -276,8 +276,11 @@ def layer_decode_step(capi, torch, np, n_calls, n_seq=64, ctx=8192, d_model=4096
     residual.  Activations are column-major (batch index fastest) as Weed lays them out; weights are random.  The
     cache starts n_calls tokens short of ctx and every call of the returned step appends one token per sequence.
     side_by_side: the weights of Q, K, V lie side by side in one buffer, and so do gate and up, as after the host
-    mirror's fuse_projections(); the projections that share their input are then one product each (13 launches)."""
+    mirror's fuse_projections(); the projections that share their input are then one product each (13 launches).
+    n_tokens > 1: a prefill chunk instead, (B, n_tokens, d_model): the same launches over B * n_tokens rows, every call
+    appends n_tokens per sequence and attends with the chunk's causal mask over the packed cache."""
     B, D, H, Hkv, hd = n_seq, d_model, n_heads, n_kv, d_model // n_heads
+    T, R = n_tokens, n_seq * n_tokens  # rows of an activation: r = b + B * t (column-major (B, T, features))
     dev = "cuda"
     g = torch.Generator(device=dev)
     g.manual_seed(31)
@@ -285,7 +288,7 @@ def layer_decode_step(capi, torch, np, n_calls, n_seq=64, ctx=8192, d_model=4096
     def cm(rows, cols, scale=1.0):  # logical [rows, cols], column-major
         return (torch.randn((cols, rows), generator=g, device=dev) * scale).t()
 
-    x = cm(B, D)
+    x = cm(R, D)
     nq, nkv = H * hd, Hkv * hd
     if side_by_side:
         w_qkv, b_qkv, w_gu = cm(D, nq + 2 * nkv, 0.02), torch.zeros(nq + 2 * nkv, device=dev), cm(D, 2 * d_ff, 0.02)
@@ -311,13 +314,13 @@ def layer_decode_step(capi, torch, np, n_calls, n_seq=64, ctx=8192, d_model=4096
     capi.make_rotation(42, hd, rv)
     cache.set_rotations(rk, rv)
     for s0 in range(0, B, 8):
-        Ks = torch.randn((8, Hkv, ctx - n_calls, hd), generator=g, device=dev)
-        Vs = torch.randn((8, Hkv, ctx - n_calls, hd), generator=g, device=dev)
+        Ks = torch.randn((8, Hkv, ctx - n_calls * T, hd), generator=g, device=dev)
+        Vs = torch.randn((8, Hkv, ctx - n_calls * T, hd), generator=g, device=dev)
         cache.encode_append(Ks, Vs, seq_begin=s0, rotate=1)
     del Ks, Vs
 
     def buf(cols):
-        return torch.empty((cols, B), device=dev).t()  # logical [B, cols], column-major
+        return torch.empty((cols, R), device=dev).t()  # logical [B * T, cols], column-major
 
     h1, qr, kr, att, o, res1, h2, act, down, out = (
         buf(D), buf(nq), buf(nkv), buf(nq), buf(D), buf(D), buf(D), buf(d_ff), buf(D), buf(D))
@@ -328,8 +331,8 @@ def layer_decode_step(capi, torch, np, n_calls, n_seq=64, ctx=8192, d_model=4096
         q, k, v, gate, up = buf(nq), buf(nkv), buf(nkv), buf(d_ff), buf(d_ff)
     eps = float(np.float32(np.finfo(np.float32).eps / 4))
 
-    def heads(t, n):  # the (B, heads, T = 1, head_dim) view of a (B, 1, heads * head_dim) activation: feature = h + n * j
-        return torch.as_strided(t, (B, n, 1, hd), (1, B, B, B * n))
+    def heads(t, n):  # the (B, heads, T, head_dim) view of a (B, T, heads * head_dim) activation: feature = h + n * j
+        return torch.as_strided(t, (B, n, T, hd), (1, R, B, R * n))
 
     flags = capi.ATTN_ROTATE_Q | capi.ATTN_UNROTATE_OUT
 
@@ -341,10 +344,14 @@ def layer_decode_step(capi, torch, np, n_calls, n_seq=64, ctx=8192, d_model=4096
             capi.linear(h1, w_q, b_q, q)
             capi.linear(h1, w_k, b_k, k)
             capi.linear(h1, w_v, b_v, v)
-        capi.rope(heads(q, H), cos_t, sin_t, rows, heads(qr, H), pos0=ctx - 1)
-        capi.rope(heads(k, Hkv), cos_t, sin_t, rows, heads(kr, Hkv), pos0=ctx - 1)
+        capi.rope(heads(q, H), cos_t, sin_t, rows, heads(qr, H), pos0=ctx - T)
+        capi.rope(heads(k, Hkv), cos_t, sin_t, rows, heads(kr, Hkv), pos0=ctx - T)
         cache.encode_append(heads(kr, Hkv), heads(v, Hkv), rotate=1)
-        cache.decode_attn(heads(qr, H)[:, :, 0], heads(att, H)[:, :, 0], capi.GQA_BLOCKED, flags)
+        if T == 1:
+            cache.decode_attn(heads(qr, H)[:, :, 0], heads(att, H)[:, :, 0], capi.GQA_BLOCKED, flags)
+        else:
+            cache.decode_attn_chunk(heads(qr, H).permute(0, 2, 1, 3), heads(att, H).permute(0, 2, 1, 3), None,
+                                    capi.GQA_BLOCKED, flags)
         capi.linear(att, w_o, b_o, o)
         capi.elementwise(capi.EW_ADD, o, x, res1)
         capi.rms_norm(res1, ln2, eps, h2)
@@ -740,6 +747,42 @@ def extras(capi, torch, workloads, steps, warmup):
         "what": "the weights of Q, K, V in one buffer and those of gate and up in another, as after "
                 "fuse_projections() of the host mirror's layer: one product for each group"}
     cacheF.close()
+    del cacheF, fused_step
+    # a prefill chunk through the same layer: 64 tokens for each of the 64 sequences (4096 rows per product), appended
+    # behind ctx ~ 7700 and attended with the chunk's causal mask over the packed cache
+    n_c = 4
+    cacheP, chunk_step = layer_decode_step(capi, torch, np, n_calls=2 * n_c + 3, n_tokens=64)
+    chunk_step()
+    torch.cuda.synchronize()
+    chunk_host_s = time_calls(torch, chunk_step, n_c, 2)
+    capi.profile_reset()
+    capi.profile_enable(True)
+    time_calls(torch, chunk_step, n_c, 0)
+    partsP = {}
+    for name in ("kv_decode_attn", "kv_encode", "matmul", "rms_norm", "elementwise", "rope"):
+        ms, n = capi.profile_read(name)
+        partsP[name] = {"ms_per_step": ms / n_c, "launches_per_step": n / n_c}
+    capi.profile_enable(False)
+    chunk_flops = 2.0 * 4096 * 4096 * (2 * 4096 + 2 * 1024 + 3 * 14336)
+    out["qwen_layer_prefill_chunk_64_tokens_64_sequences"] = {
+        "ms_per_step": 1e3 * chunk_host_s, "tokens_per_s": 4096 / chunk_host_s,
+        "by_kernel_family_event_pairs": partsP,
+        "projection_tflops": chunk_flops / (1e-3 * partsP["matmul"]["ms_per_step"]) / 1e12,
+        "shape": "the layer of qwen_layer_decode_step on (64, 64, 4096) activations: seven products of 4096 rows "
+                 "(1.79 TFLOP), append of 64 tokens per sequence, attention of the 64 positions over ~7700 cached tokens"}
+    cacheP.close()
+    del cacheP, chunk_step
+    # the same chunk with every product on the fp32 matrix instruction (weed_hip_matmul_tuning)
+    capi.matmul_tuning(True)
+    try:
+        cache32, chunk32 = layer_decode_step(capi, torch, np, n_calls=n_c + 3, n_tokens=64)
+        chunk32()
+        torch.cuda.synchronize()
+        out["qwen_layer_prefill_chunk_64_tokens_64_sequences"]["on_the_fp32_instruction_ms_per_step"] = \
+            1e3 * time_calls(torch, chunk32, n_c, 2)
+        cache32.close()
+    finally:
+        capi.matmul_tuning(False)
     return out
 
 
