@@ -759,6 +759,28 @@ def test_groups_larger_than_a_tile(gpu, oracle, d, Hkv, G):
     cache.close()
 
 
+def test_passes_of_a_large_group_share_one_launch(gpu, oracle):
+    """40 query heads per KV head are three passes of the matrix-core kernel, and they are ONE launch whose workgroups
+    find their pass from their index (those of a pass are rounded up to a multiple of eight, the extra ones leave at
+    once): enough sequences for several octets of workgroups per pass, ragged lengths, one sequence without tokens;
+    against the checker."""
+    rng = np.random.default_rng(40)
+    d, Hkv, G = 128, 2, 40
+    lens = [int(x) for x in rng.integers(1, 700, size=24)]
+    lens[5] = 0
+    S, Hq = len(lens), Hkv * G
+    K = rng.standard_normal((S, Hkv, max(lens), d), dtype=np.float32)
+    V = rng.standard_normal((S, Hkv, max(lens), d), dtype=np.float32)
+    q = rng.standard_normal((S, Hq, d), dtype=np.float32)
+    wl = workloads.Workload("mqa", S, Hq, Hkv, d, lens, 3, 4, 1, 0, 0)
+    cache = build_cache(gpu, wl, gpu.KV_LLOYDMAX, K, V)
+    want = checker_output(oracle, gpu, cache, wl, q, False)
+    got = run_decode(gpu, cache, q, gpu.GQA_BLOCKED, 0)
+    assert_attn_close(got, want, "three passes in one launch")
+    assert np.all(got[5] == 0.0)
+    cache.close()
+
+
 @pytest.mark.parametrize("d", [160, 192, 224, 256])
 @pytest.mark.parametrize("wk,wv,Hq", [(2, 2, 2), (3, 4, 8), (4, 4, 16), (4, 3, 4), (4, 2, 32)])
 def test_head_dims_above_128(gpu, oracle, d, wk, wv, Hq):

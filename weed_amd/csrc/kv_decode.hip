@@ -1206,10 +1206,20 @@ int decode_impl(const char *fn, weed_hip_kv_cache *c, int32_t n_q_heads, int32_t
         mp.group_total = G;
         mp.tile_rows = pass_heads;
         ProfileScope prof("kv_decode_attn", timed);
-        for (uint32_t first = 0; total_blocks && first < G; first += pass_heads) {
-            mp.head_first = first;
-            mp.G = std::min(pass_heads, G - first);
+        mp.grid_passes = 0;
+        if (passes > 1 && total_blocks && !fused_merge && !fused_query) {
+            // every pass in ONE launch: the passes' workgroups that read the same blocks run next to each other on one
+            // XCD, so the cache is fetched from memory once instead of once per pass
+            mp.grid_passes = passes;
+            mp.head_first = 0;
+            mp.G = pass_heads;
             WEED_HIP_TRY(launch_mfma_decode(mp, d, stream()));
+        } else {
+            for (uint32_t first = 0; total_blocks && first < G; first += pass_heads) {
+                mp.head_first = first;
+                mp.G = std::min(pass_heads, G - first);
+                WEED_HIP_TRY(launch_mfma_decode(mp, d, stream()));
+            }
         }
     } else {
         DecodeParams p;

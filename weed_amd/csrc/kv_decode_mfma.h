@@ -249,6 +249,11 @@ struct MfmaParams {
     // groups larger than a tile has rows go through the cache in several launches: this one serves the heads
     // [head_first, head_first + G) of the group_total that share a KV head; tile_rows (0: G) picks the kernel instance
     uint32_t head_first, group_total, tile_rows;
+    // grid_passes > 1 (instances that do not merge): ONE launch holds that many such passes, tile_rows heads each, and
+    // a workgroup finds its pass and its place in it from its index: launch index = ((w / 8) * grid_passes + pass) * 8
+    // + w % 8, so that the workgroups that read the same blocks for different heads are dispatched next to each other
+    // and onto the same XCD (launch index % 8), whose L2 then serves all but the first of them
+    uint32_t grid_passes;
     uint32_t max_slots;      // partial slots per (sequence, head): most wavefronts that can touch one region
     const uint16_t *q_hi;   // [n_seq][Hq][d] fp16 bits: high half of the scaled, normalised query
     const uint16_t *q_lo;   // [n_seq][Hq][d] fp16 bits: what the high half misses

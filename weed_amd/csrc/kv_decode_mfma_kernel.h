@@ -311,10 +311,24 @@ template <int GP, int I> constexpr int bank_mask_of() { return ((1 << (GP / 4)) 
 // mfma_decode_merges(GP, D) says so.  MODE 2: as MODE 0 with both of these, for the head_dims whose MODE 0 leaves them
 // out because they cost it registers that every other launch would pay for (mfma_decode_general_variant).
 template <int D, int WK, int WV, int GP, bool LLOYD, int MODE>
-__global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) decode_mfma_kernel(MfmaParams p)
+__global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) decode_mfma_kernel(MfmaParams launch)
 {
     constexpr bool WGM = MODE == 1;
     constexpr int kWaves = (int)mfma_decode_waves_per_wg(GP, D, WK, WV);
+    MfmaParams p = launch;
+    uint32_t wg_index = blockIdx.x; // this workgroup's place among those of its pass
+    if constexpr (MODE == 0) {
+        if (launch.grid_passes > 1) {
+            const uint32_t octet = blockIdx.x >> 3, pass = octet % launch.grid_passes;
+            wg_index = (octet / launch.grid_passes) * 8 + (blockIdx.x & 7);
+            const uint32_t wg_blocks = kWaves * launch.runs.unit_blocks;
+            if (wg_index >= (launch.total_blocks + wg_blocks - 1) / wg_blocks) {
+                return; // (the workgroups of a pass were rounded up to a multiple of eight)
+            }
+            p.head_first = pass * launch.tile_rows;
+            p.G = min(launch.tile_rows, launch.group_total - p.head_first);
+        }
+    }
     constexpr int KS = D / 32;       // Q.K^T k-steps (32 coordinates each); also K items per tile per lane
     constexpr int JB = D / 16;       // 16-coordinate column blocks of the output
     constexpr int NK = KS * WK;      // dwords of packed K per lane per block
@@ -374,7 +388,7 @@ __global__ void __launch_bounds__(64 * mfma_decode_waves_per_wg(GP, D, WK, WV)) 
     //      boundaries; every segment leaves one partial in the slot `unit - first unit of the region`. ----
     // `unit`: position index of this wavefront's run (runs are numbered along the block list)
     const uint32_t unit =
-        __builtin_amdgcn_readfirstlane(blockIdx.x * kWaves + run_position_of_wave(p.runs, wave));
+        __builtin_amdgcn_readfirstlane(wg_index * kWaves + run_position_of_wave(p.runs, wave));
     // Runs that take turns (RunGeom::group_cycles; instances whose workgroups merge only): g0 .. g1 are then the blocks
     // of the run's whole group, of which this wavefront takes its `turn_count` blocks -- one segment, since no group
     // crosses a region boundary.  In turn i the runs that are still short of their length take one block each, ordered
@@ -1524,7 +1538,13 @@ template <int D, int WK, int WV, int GP, bool LLOYD> int launch_gp(const MfmaPar
                     p.runs.waves, waves);
     }
     const uint32_t wg_blocks = waves * p.runs.unit_blocks;
-    const uint32_t grid = (p.total_blocks + wg_blocks - 1) / wg_blocks;
+    uint32_t grid = (p.total_blocks + wg_blocks - 1) / wg_blocks;
+    if (p.grid_passes > 1) {
+        if (p.merge.wg_regions != 0 || p.merge.region_wgs != 0 || p.merge.general || p.query.q) {
+            return fail(WEED_HIP_EDEVICE, "decode_mfma: several passes in one launch neither merge nor rotate queries");
+        }
+        grid = (grid + 7) / 8 * 8 * p.grid_passes;
+    }
     if (p.merge.wg_regions != 0 || p.merge.region_wgs != 0) {
         if constexpr (kMerges) {
             decode_mfma_kernel<D, WK, WV, GP, LLOYD, 1><<<grid, 64 * waves, smem_merging, s>>>(p);
