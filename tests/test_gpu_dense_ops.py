@@ -401,7 +401,8 @@ def test_softmax_and_reduce_strided_against_checker(gpu, oracle, shape):
                                         ((8200, 300), 1), ((12300, 1100), 1),
                                         ((16, 5000), 0), ((40, 3000), 0), ((7, 2000), 0), ((500, 1100), 0), ((29, 1500), 0),
                                         ((256, 1030), 0), ((64, 40000), 1), ((300, 20000), 1), ((2048, 4100), 1), ((4000, 4200), 1),
-                                        ((32768, 5), 0), ((20000, 4), 0), ((40004, 3), 0)])
+                                        ((32768, 5), 0), ((20000, 4), 0), ((40004, 3), 0),
+                                        ((15, 100000), 1), ((8, 32768), 1), ((5, 40000), 1), ((3600, 16400), 1)])
 def test_softmax_and_reduce_launch_shapes(gpu, shape, axis):
     """One case per way the threads are spread: a contiguous row longer than what the registers keep between the
     passes, enough rows for 32 per workgroup, few long strided rows (decode-time scores), a short aligned row, and
@@ -410,7 +411,8 @@ def test_softmax_and_reduce_launch_shapes(gpu, shape, axis):
     and many strided rows of 300 (kept in 32 registers per thread) and of 1100 elements (two passes); many contiguous
     rows of 7 to 500 elements, which share a wavefront (4 to 32 lanes per row); few rows with a strided axis of 20000
     and 40000 elements, which is cut into bands (three launches); few contiguous rows of 20000 to 40004 elements
-    (sixteen wavefronts per row, one pass up to 32768 elements).
+    (sixteen wavefronts per row, one pass up to 32768 elements); fewer than 16 long strided rows and 3600 rows of 16400,
+    which go by bands as well (the sums from 2^18 elements on).
     Some positions are masked with -inf, one row of the decode case entirely (its softmax is NaN, as in numpy)."""
     import torch
     rng = np.random.default_rng(shape[0] + axis)

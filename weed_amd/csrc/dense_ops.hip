@@ -1094,10 +1094,16 @@ AxisLaunch choose_axis_launch(const AxisGeom &g, const float *a_dev, const float
 }
 
 // Few rows and a long strided axis: bands of the axis (see band_partial_kernel); bands == 0: not this way.
-BandGeom choose_bands(const AxisGeom &g, uint32_t most_rows)
+// (Fewer than 16 rows fill an eighth of a band workgroup's lanes or less, and the launches have a floor of their own:
+// they only go this way from `few_rows_least` elements on -- 15 strided rows of 100000: softmax 155 -> 54 us, sum 53 -> 15;
+// 8 rows of 32768: 43 -> 38 and 17 -> 10; 8 rows of 8192 stay with one workgroup per row, 15 and 6 us against 18 and 8.)
+BandGeom choose_bands(const AxisGeom &g, uint32_t most_rows, uint64_t few_rows_least)
 {
     BandGeom bg = { 0U, 0U, 0U };
-    if (g.a_stride[g.axis] <= 1U || g.rows < 16U || g.rows > std::min(most_rows, kBandRows) || g.axis_len < 4096U ||
+    if (g.rows < 16U && (uint64_t)g.rows * g.axis_len < few_rows_least) {
+        return bg;
+    }
+    if (g.a_stride[g.axis] <= 1U || g.rows > std::min(most_rows, kBandRows) || g.axis_len < 4096U ||
         (uint64_t)g.axis_len * g.a_stride[g.axis] >= (1ull << 32)) {
         return bg;
     }
@@ -1406,7 +1412,7 @@ int weed_hip_softmax_f32(uint32_t rank, const uint32_t *shape, uint32_t axis, co
         } else {
             softmax_wave_rows_kernel<1, 16, false><<<wave_row_blocks(g.rows), 256, 0, stream()>>>(a_dev, out_dev, g);
         }
-    } else if (how == AXIS_ROW) {
+    } else if (how == AXIS_ROW && choose_bands(g, 4096U, 3U << 16).bands == 0U) { // (fewer than 16 long strided rows go by bands)
         softmax_kernel<1, 256><<<g.rows, 256, 0, stream()>>>(a_dev, out_dev, g);
     } else if ((uint64_t)g.axis_len * g.a_stride[axis] >= (1ull << 32)) {
         softmax_kernel<16, 1024><<<(g.rows + 15) / 16, 1024, 0, stream()>>>(a_dev, out_dev, g);
@@ -1425,7 +1431,7 @@ int weed_hip_softmax_f32(uint32_t rank, const uint32_t *shape, uint32_t axis, co
         // (with more rows the two passes over 32 rows per workgroup are faster: 16-row tiles are half lines.
         // 4096 rows of 2048: 22 us against 35; 16384 rows: 83 against 72; 65536 rows: 427 against 369)
         softmax_strided_cached_kernel<16><<<(g.rows + 15) / 16, kStridedThreads, 0, stream()>>>(a_dev, out_dev, g);
-    } else if (const BandGeom bg = choose_bands(g, 4096U); bg.bands != 0U) {
+    } else if (const BandGeom bg = choose_bands(g, 4096U, 3U << 16); bg.bands != 0U) {
         // (up to 4096 rows of at least 4096 strided elements -- with 8192 rows and more the walks over 32 rows per
         // workgroup are as fast or faster: 8192 x 8192 174 against 187 us; 4096 x 32768 372 us here against 525 --: 64 rows of 32768 25 us, where 16 rows per workgroup took
         // 166; 256 rows of 8192 16 us against 25 with the narrow tiles below; 2048 rows of 16384 83 against 127)
@@ -1463,9 +1469,9 @@ int weed_hip_reduce_f32(int op, uint32_t rank, const uint32_t *shape, uint32_t a
     WEED_HIP_TRY(make_geom(fn, rank, shape, axis, a_off, a_stride, o_off, o_stride, false, g));
     ProfileScope prof("reduce");
     const AxisLaunch how = choose_axis_launch(g, a_dev, out_dev, false);
-    const BandGeom bands = choose_bands(g, 3072U); // (4096 rows of 4096 to 8192: 13 and 23 us without bands, 16 and 26 with)
+    const BandGeom bands = choose_bands(g, g.axis_len >= 16384U ? 4096U : 3072U, 1U << 18); // (4096 rows of 4096 to 8192: 13 and 23 us without bands, 16 and 26 with)
 #define WEED_LAUNCH_REDUCE(OP)                                                                                         \
-    if (bands.bands != 0U && how != AXIS_CONTIGUOUS && how != AXIS_ROW && how != AXIS_WAVE && how != AXIS_WAVE_VEC) {  \
+    if (bands.bands != 0U && how != AXIS_CONTIGUOUS && how != AXIS_WAVE && how != AXIS_WAVE_VEC) {                     \
         band_partial_kernel<OP><<<dim3((g.rows + 63U) / 64U, bands.bands), 256, 0, stream()>>>(a_dev, g, bands);       \
         band_merge_kernel<OP><<<(g.rows + 63U) / 64U, 256, 0, stream()>>>(out_dev, g, bands);                         \
     } else if (how == AXIS_CONTIGUOUS) {                                                                               \
