@@ -102,7 +102,8 @@ int weed_hip_matmul_f32(uint32_t M, uint32_t N, uint32_t K, const float *a_dev, 
  * 9e-4 around 2^-125; fp32 denormals count as zero), where the fp32 instruction keeps 2e-7 down to the denormals.  1: the fp32 instruction everywhere (v_mfma_f32_32x32x2_f32: every product
  * exact, sums rounded to fp32 in ascending k per 16-k slice), also for the products of 17 to 64 rows against a
  * k-contiguous weight, which otherwise split their operands the same way.  Products with at most 16 rows, and unaligned
- * or doubly strided operands, do not depend on it. */
+ * or doubly strided operands, do not depend on it.  The process-wide default is read once from the environment
+ * variable WEED_HIP_MATMUL_FP32 (1 = the fp32 instruction). */
 int weed_hip_matmul_tuning(int32_t fp32_instruction);
 
 /* batch[0] * batch[1] independent products in one launch: product (c0, c1) uses the offsets

@@ -3,6 +3,7 @@
 #include "common.h"
 
 #include <atomic>
+#include <cstdlib>
 #include <cmath>
 #include <algorithm>
 #include <type_traits>
@@ -1045,7 +1046,11 @@ int launch_matmul_body(const char *fn, const MatGeom &g, uint32_t batch, const f
 
 // weed_hip_matmul_tuning: the fp32 matrix instruction for every product (false: six bfloat16 products of split operands
 // where the layout allows)
-std::atomic<bool> g_fp32_instruction{ false };
+// (the process-wide default comes from the environment variable WEED_HIP_MATMUL_FP32, read once: 1 = the fp32 instruction)
+std::atomic<bool> g_fp32_instruction{ [] {
+    const char *e = std::getenv("WEED_HIP_MATMUL_FP32");
+    return e != nullptr && e[0] == '1';
+}() };
 
 int launch_matmul(const char *fn, const MatGeom &g, uint32_t batch, const float *a_dev, const float *b_dev, float *out_dev)
 {
